@@ -1,0 +1,247 @@
+"""ctypes bindings for the CPU oracle (oracle/liboracle.so) and, where it has been built, the
+compiled reference sampler (oracle/_ref/libgeist_ref_sampler.so).
+
+Test infrastructure only: the shipped library never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+
+c_float_p = C.POINTER(C.c_float)
+c_int32_p = C.POINTER(C.c_int32)
+
+
+class OracleRng(C.Structure):
+    _fields_ = [("state", C.c_uint64)]
+
+
+class DrawInfo(C.Structure):
+    _fields_ = [("boundary_dist", C.c_double), ("mass", C.c_double), ("n_keep", C.c_size_t),
+                ("draws", C.c_int)]
+
+
+class ChainParams(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_int), ("top_p", C.c_float),
+                ("min_p", C.c_float)]
+
+
+class SessionSampler(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("top_k", C.c_int),
+                ("rng", OracleRng)]
+
+
+def _fp(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(c_float_p)
+
+
+def _ip(a):
+    assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(c_int32_p)
+
+
+def build_oracle():
+    subprocess.run(["make", "-C", ORACLE_DIR, "-s"], check=True)
+
+
+def load_oracle(fast=False):
+    name = "liboracle_fast.so" if fast else "liboracle.so"
+    path = os.path.join(ORACLE_DIR, name)
+    if not os.path.exists(path):
+        build_oracle()
+    lib = C.CDLL(path)
+    lib.oracle_rng_next_u64.restype = C.c_uint64
+    lib.oracle_rng_next_unit.restype = C.c_float
+    lib.oracle_argmax.restype = C.c_int32
+    lib.oracle_argmax.argtypes = [C.c_size_t, c_float_p]
+    lib.oracle_softmax_into.restype = C.c_double
+    lib.oracle_softmax_into.argtypes = [C.c_size_t, c_float_p, C.c_float, c_float_p]
+    lib.oracle_softmax_normalised.restype = C.c_double
+    lib.oracle_softmax_normalised.argtypes = [C.c_size_t, c_float_p, C.c_float, c_float_p]
+    lib.oracle_temperature_u.restype = C.c_int32
+    lib.oracle_temperature_u.argtypes = [C.c_size_t, c_float_p, C.c_float, C.c_float,
+                                         C.POINTER(DrawInfo)]
+    lib.oracle_top_k_u.restype = C.c_int32
+    lib.oracle_top_k_u.argtypes = [C.c_size_t, c_float_p, C.c_int, C.c_float, C.c_float,
+                                   C.POINTER(DrawInfo)]
+    lib.oracle_top_p_u.restype = C.c_int32
+    lib.oracle_top_p_u.argtypes = [C.c_size_t, c_float_p, C.c_float, C.c_float, C.c_float,
+                                   C.POINTER(DrawInfo)]
+    lib.oracle_temperature.restype = C.c_int32
+    lib.oracle_temperature.argtypes = [C.c_size_t, c_float_p, C.c_float, C.POINTER(OracleRng)]
+    lib.oracle_top_k.restype = C.c_int32
+    lib.oracle_top_k.argtypes = [C.c_size_t, c_float_p, C.c_int, C.c_float, C.POINTER(OracleRng)]
+    lib.oracle_top_p.restype = C.c_int32
+    lib.oracle_top_p.argtypes = [C.c_size_t, c_float_p, C.c_float, C.c_float, C.POINTER(OracleRng)]
+    lib.oracle_session_apply_opts.argtypes = [C.POINTER(SessionSampler), C.c_float, C.c_float,
+                                              C.c_int, C.c_uint64]
+    lib.oracle_session_draws.argtypes = [C.POINTER(SessionSampler), C.c_size_t]
+    lib.oracle_softcap_inplace.argtypes = [C.c_size_t, c_float_p, C.c_float]
+    lib.oracle_finalize_row.restype = C.c_int32
+    lib.oracle_finalize_row.argtypes = [C.POINTER(SessionSampler), C.c_size_t, c_float_p, C.c_float]
+    lib.oracle_finalize_batch.argtypes = [C.POINTER(SessionSampler), C.c_size_t, C.c_size_t,
+                                          c_float_p, C.c_float, c_int32_p]
+    lib.oracle_apply_penalties.argtypes = [C.c_size_t, c_float_p, c_int32_p, C.c_size_t, C.c_float,
+                                           C.c_float, C.c_float]
+    lib.oracle_sample_chain_u.restype = C.c_int32
+    lib.oracle_sample_chain_u.argtypes = [C.c_size_t, c_float_p, C.POINTER(ChainParams), C.c_float,
+                                          C.POINTER(DrawInfo)]
+    lib.oracle_spec_verify.restype = C.c_int32
+    lib.oracle_spec_verify.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_size_t, c_float_p,
+                                       C.c_size_t, c_int32_p, c_float_p, C.c_float, c_int32_p]
+    lib.oracle_batch_top_k_u.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_size_t, C.c_int,
+                                         C.c_float, c_float_p, c_int32_p, C.c_int]
+    lib.oracle_batch_chain_u.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_size_t,
+                                         C.POINTER(ChainParams), c_int32_p, C.c_size_t, c_int32_p,
+                                         C.c_float, C.c_float, C.c_float, c_float_p, c_int32_p,
+                                         C.c_int]
+    lib.oracle_max_threads.restype = C.c_int
+    return lib
+
+
+class Oracle:
+    """Thin numpy-facing wrapper."""
+
+    def __init__(self, fast=False):
+        self.lib = load_oracle(fast)
+
+    # -- rng
+    def rng(self, seed):
+        r = OracleRng()
+        self.lib.oracle_rng_seed(C.byref(r), C.c_uint64(seed))
+        return r
+
+    def next_u64(self, r):
+        return int(self.lib.oracle_rng_next_u64(C.byref(r)))
+
+    def next_unit(self, r):
+        return float(self.lib.oracle_rng_next_unit(C.byref(r)))
+
+    # -- modes
+    def argmax(self, row):
+        return int(self.lib.oracle_argmax(row.size, _fp(row)))
+
+    def softmax_into(self, row, t):
+        out = np.empty_like(row)
+        s = self.lib.oracle_softmax_into(row.size, _fp(row), t, _fp(out))
+        return out, float(s)
+
+    def softmax_normalised(self, row, t):
+        out = np.empty_like(row)
+        s = self.lib.oracle_softmax_normalised(row.size, _fp(row), t, _fp(out))
+        return out, float(s)
+
+    def temperature_u(self, row, t, u):
+        info = DrawInfo()
+        tok = self.lib.oracle_temperature_u(row.size, _fp(row), t, u, C.byref(info))
+        return int(tok), info
+
+    def top_k_u(self, row, k, t, u):
+        info = DrawInfo()
+        tok = self.lib.oracle_top_k_u(row.size, _fp(row), k, t, u, C.byref(info))
+        return int(tok), info
+
+    def top_p_u(self, row, p, t, u):
+        info = DrawInfo()
+        tok = self.lib.oracle_top_p_u(row.size, _fp(row), p, t, u, C.byref(info))
+        return int(tok), info
+
+    def chain_u(self, row, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0):
+        info = DrawInfo()
+        prm = ChainParams(temperature, top_k, top_p, min_p)
+        tok = self.lib.oracle_sample_chain_u(row.size, _fp(row), C.byref(prm), u, C.byref(info))
+        return int(tok), info
+
+    def penalties(self, row, hist, rep, freq, pres):
+        out = row.copy()
+        hist = np.ascontiguousarray(hist, dtype=np.int32)
+        self.lib.oracle_apply_penalties(out.size, _fp(out), _ip(hist), hist.size, rep, freq, pres)
+        return out
+
+    def softcap(self, row, cap):
+        out = row.copy()
+        self.lib.oracle_softcap_inplace(out.size, _fp(out), cap)
+        return out
+
+    def session(self, temperature=0.0, top_p=1.0, top_k=0, seed=0):
+        s = SessionSampler()
+        self.lib.oracle_session_defaults(C.byref(s))
+        self.lib.oracle_session_apply_opts(C.byref(s), temperature, top_p, top_k, C.c_uint64(seed))
+        return s
+
+    def finalize_row(self, sess, row, softcap=0.0):
+        tmp = row.copy()
+        return int(self.lib.oracle_finalize_row(C.byref(sess), tmp.size, _fp(tmp), softcap))
+
+    def finalize_batch(self, sess, rows, softcap=0.0):
+        tmp = np.ascontiguousarray(rows, dtype=np.float32).copy()
+        k, n = tmp.shape
+        out = np.empty(k, dtype=np.int32)
+        self.lib.oracle_finalize_batch(C.byref(sess), k, n, _fp(tmp), softcap, _ip(out))
+        return out
+
+    def spec_verify(self, target, q, draft, u, temperature):
+        target = np.ascontiguousarray(target, dtype=np.float32)
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        draft = np.ascontiguousarray(draft, dtype=np.int32)
+        u = np.ascontiguousarray(u, dtype=np.float32)
+        L = draft.size
+        n = target.shape[1]
+        assert target.shape[0] == L + 1 and q.shape == (L, n) and u.size == L + 1
+        out = np.full(L + 1, -1, dtype=np.int32)
+        nacc = self.lib.oracle_spec_verify(L, n, _fp(target), n, _fp(q), n, _ip(draft), _fp(u),
+                                           temperature, _ip(out))
+        return int(nacc), out
+
+    def batch_chain_u(self, logits, u, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, hist=None,
+                      hist_len=None, rep=1.0, freq=0.0, pres=0.0, threads=1):
+        rows, n = logits.shape
+        out = np.empty(rows, dtype=np.int32)
+        prm = ChainParams(temperature, top_k, top_p, min_p)
+        hp = _ip(hist) if hist is not None else None
+        hl = _ip(hist_len) if hist_len is not None else None
+        hld = hist.shape[1] if hist is not None else 0
+        self.lib.oracle_batch_chain_u(rows, n, _fp(logits), n, C.byref(prm), hp, hld, hl, rep, freq,
+                                      pres, _fp(u), _ip(out), threads)
+        return out
+
+
+# ---------------------------------------------------------------------------------------------
+# The compiled reference (built from the reference's own sources by `make -C oracle ref`).
+# ---------------------------------------------------------------------------------------------
+class RefWorkspace(C.Structure):
+    _fields_ = [("probs", c_float_p), ("n_vocab", C.c_size_t)]
+
+
+def ref_path(fast=False):
+    return os.path.join(ORACLE_DIR, "_ref",
+                        "libgeist_ref_sampler_fast.so" if fast else "libgeist_ref_sampler.so")
+
+
+def load_ref(fast=False):
+    """Returns the compiled reference library, or None where it has not been built."""
+    path = ref_path(fast)
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path)
+    lib.geist_rng_next_u64.restype = C.c_uint64
+    lib.geist_rng_next_unit.restype = C.c_float
+    lib.geist_sampler_argmax.restype = C.c_int32
+    lib.geist_sampler_argmax.argtypes = [C.c_size_t, c_float_p]
+    lib.geist_sampler_temperature.restype = C.c_int32
+    lib.geist_sampler_temperature.argtypes = [C.c_size_t, c_float_p, C.c_float,
+                                              C.POINTER(OracleRng)]
+    lib.geist_sampler_workspace_init.argtypes = [C.POINTER(RefWorkspace), C.c_size_t]
+    lib.geist_sampler_workspace_destroy.argtypes = [C.POINTER(RefWorkspace)]
+    lib.geist_sampler_top_k_ws.restype = C.c_int32
+    lib.geist_sampler_top_k_ws.argtypes = [C.POINTER(RefWorkspace), c_float_p, C.c_int, C.c_float,
+                                           C.POINTER(OracleRng)]
+    lib.geist_sampler_top_p_ws.restype = C.c_int32
+    lib.geist_sampler_top_p_ws.argtypes = [C.POINTER(RefWorkspace), c_float_p, C.c_float, C.c_float,
+                                           C.POINTER(OracleRng)]
+    return lib
