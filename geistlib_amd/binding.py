@@ -1,0 +1,176 @@
+"""ctypes binding of include/geist_sampler_hip.h. Device memory comes from torch tensors
+(`tensor.data_ptr()`); nothing here computes on logits."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+GEIST_HIP_OK = 0
+PRECEDENCE_REFERENCE = 0
+PRECEDENCE_CHAIN = 1
+
+_STATUS = {0: "OK", 1: "E_OOM", 2: "E_INVALID_ARG", 3: "E_INTERNAL", 7: "E_UNSUPPORTED",
+           9: "E_BACKEND"}
+
+
+class GeistHipError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"{_STATUS.get(code, code)}: {text}")
+        self.code = code
+
+
+class Rows(C.Structure):
+    _fields_ = [("d_logits", C.c_void_p), ("ld", C.c_size_t), ("rows", C.c_size_t),
+                ("n_vocab", C.c_size_t), ("d_history", C.c_void_p), ("history_ld", C.c_size_t),
+                ("d_history_len", C.c_void_p)]
+
+
+class SampleParams(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("top_k", C.c_int),
+                ("min_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("frequency_penalty", C.c_float), ("presence_penalty", C.c_float),
+                ("logit_softcap", C.c_float), ("precedence", C.c_int)]
+
+    @classmethod
+    def make(cls, temperature=0.0, top_p=1.0, top_k=0, min_p=0.0, rep=1.0, freq=0.0, pres=0.0,
+             softcap=0.0, precedence=PRECEDENCE_CHAIN):
+        return cls(temperature, top_p, top_k, min_p, rep, freq, pres, softcap, precedence)
+
+
+def library_path(name="libgeist_sampler_hip.so"):
+    return os.path.join(HERE, "lib", name)
+
+
+_LIB = None
+
+
+def load_library():
+    """Loads the built HIP library. There is no fallback: a missing library is an error."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `make -C geistlib_amd` "
+                           "(or __graft_entry__.build()); the sampling path has no CPU fallback")
+    lib = C.CDLL(path)
+    vp, sz, i32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_float
+    lib.geist_hip_sampler_create.argtypes = [i32, sz, sz, vp, C.POINTER(vp)]
+    lib.geist_hip_sampler_destroy.argtypes = [vp]
+    lib.geist_hip_sampler_destroy.restype = None
+    lib.geist_hip_sampler_last_error.argtypes = [vp]
+    lib.geist_hip_sampler_last_error.restype = C.c_char_p
+    lib.geist_hip_sampler_sync.argtypes = [vp]
+    lib.geist_hip_sampler_set_stream.argtypes = [vp, vp]
+    lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
+    lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
+                                              vp]
+    lib.geist_hip_argmax_f32.argtypes = [vp, vp, sz, C.POINTER(C.c_int32)]
+    lib.geist_hip_apply_penalties.argtypes = [vp, vp, sz, sz, sz, vp, sz, vp, f32, f32, f32]
+    lib.geist_hip_softmax_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, sz]
+    lib.geist_hip_spec_verify.argtypes = [vp, vp, sz, vp, sz, vp, vp, sz, sz, sz, f32, vp, vp]
+    lib.geist_hip_malloc.argtypes = [vp, sz, C.POINTER(vp)]
+    lib.geist_hip_free.argtypes = [vp, vp]
+    lib.geist_hip_upload.argtypes = [vp, vp, vp, sz]
+    lib.geist_hip_download.argtypes = [vp, vp, vp, sz]
+    lib.geist_hip_sampler_timing_enable.argtypes = [vp, i32]
+    lib.geist_hip_sampler_timing_read.argtypes = [vp, C.POINTER(C.c_double), C.POINTER(C.c_long),
+                                                  i32]
+    _LIB = lib
+    return lib
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+class HipSampler:
+    """One device workspace + stream, as one sampler workspace per session in the reference."""
+
+    def __init__(self, max_rows, max_vocab, device=0, stream=None):
+        self.lib = load_library()
+        self.h = C.c_void_p()
+        rc = self.lib.geist_hip_sampler_create(device, max_rows, max_vocab, stream, C.byref(self.h))
+        if rc != GEIST_HIP_OK:
+            raise GeistHipError(rc, "geist_hip_sampler_create failed")
+
+    def close(self):
+        if self.h:
+            self.lib.geist_hip_sampler_destroy(self.h)
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc):
+        if rc != GEIST_HIP_OK:
+            raise GeistHipError(rc, self.lib.geist_hip_sampler_last_error(self.h).decode())
+
+    def set_stream(self, stream_ptr):
+        self._check(self.lib.geist_hip_sampler_set_stream(self.h, stream_ptr))
+
+    def sync(self):
+        self._check(self.lib.geist_hip_sampler_sync(self.h))
+
+    @staticmethod
+    def rows(logits, history=None, history_len=None, n_vocab=None):
+        """logits: 2-D float32 device tensor (row stride = logits.stride(0))."""
+        assert logits.dim() == 2 and logits.stride(1) == 1
+        r = Rows()
+        r.d_logits = logits.data_ptr()
+        r.ld = logits.stride(0) if logits.shape[0] > 1 else max(logits.stride(0), logits.shape[1])
+        r.rows = logits.shape[0]
+        r.n_vocab = n_vocab if n_vocab is not None else logits.shape[1]
+        if history is not None:
+            assert history.dim() == 2 and history.stride(1) == 1
+            r.d_history = history.data_ptr()
+            r.history_ld = history.stride(0) if history.shape[0] > 1 else history.shape[1]
+            r.d_history_len = history_len.data_ptr()
+        return r
+
+    def sample(self, rows, params, uniforms, out):
+        self._check(self.lib.geist_hip_sample_rows(self.h, C.byref(rows), C.byref(params),
+                                                   _ptr(uniforms), _ptr(out)))
+
+    def sample_rng(self, rows, params, states, shared, out):
+        self._check(self.lib.geist_hip_sample_rows_rng(self.h, C.byref(rows), C.byref(params),
+                                                       _ptr(states), int(shared), _ptr(out)))
+
+    def argmax_f32(self, logits_row):
+        idx = C.c_int32(-1)
+        self._check(self.lib.geist_hip_argmax_f32(self.h, _ptr(logits_row), logits_row.numel(),
+                                                  C.byref(idx)))
+        return idx.value
+
+    def apply_penalties(self, logits, history, history_len, rep, freq, pres):
+        ld = logits.stride(0) if logits.shape[0] > 1 else logits.shape[1]
+        hld = history.stride(0) if history.shape[0] > 1 else history.shape[1]
+        self._check(self.lib.geist_hip_apply_penalties(self.h, _ptr(logits), ld, logits.shape[0],
+                                                       logits.shape[1], _ptr(history), hld,
+                                                       _ptr(history_len), rep, freq, pres))
+
+    def softmax(self, rows, params, probs):
+        ld = probs.stride(0) if probs.shape[0] > 1 else probs.shape[1]
+        self._check(self.lib.geist_hip_softmax_rows(self.h, C.byref(rows), C.byref(params),
+                                                    _ptr(probs), ld))
+
+    def spec_verify(self, target, q, draft, uniforms, temperature, out_tokens, n_accepted):
+        n_seq, lp1, n = target.shape
+        L = lp1 - 1
+        assert q.shape == (n_seq, L, n) and draft.shape == (n_seq, L)
+        assert target.is_contiguous() and q.is_contiguous()
+        self._check(self.lib.geist_hip_spec_verify(self.h, _ptr(target), n, _ptr(q), n, _ptr(draft),
+                                                   _ptr(uniforms), n_seq, L, n, temperature,
+                                                   _ptr(out_tokens), _ptr(n_accepted)))
+
+    def timing_enable(self, on=True):
+        self._check(self.lib.geist_hip_sampler_timing_enable(self.h, int(on)))
+
+    def timing_read(self, reset=True):
+        ms, n = C.c_double(), C.c_long()
+        self._check(self.lib.geist_hip_sampler_timing_read(self.h, C.byref(ms), C.byref(n),
+                                                           int(reset)))
+        return ms.value, n.value

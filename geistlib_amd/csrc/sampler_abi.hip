@@ -1,0 +1,520 @@
+/*
+ * sampler_abi.hip -- the C ABI declared in include/geist_sampler_hip.h: argument checks, launch
+ * geometry and the order of kernels for each sampling configuration. No arithmetic on logits
+ * happens on the host.
+ */
+#include "../../include/geist_sampler_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "sampler_kernels.h"
+
+using namespace gs;
+
+struct geist_hip_sampler {
+    int         device     = 0;
+    hipStream_t stream     = nullptr;
+    size_t      max_rows   = 0;
+    size_t      max_vocab  = 0;
+    int         max_chunks = 0;
+
+    /* device workspace */
+    uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
+    double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
+    uint32_t *cand_key   = nullptr; /* [max_rows][max_chunks][TOPK_CAND_CAP] */
+    int32_t  *cand_idx   = nullptr;
+    int32_t  *cand_cnt   = nullptr; /* [max_rows][max_chunks] */
+    int32_t  *row_flag   = nullptr; /* [max_rows] */
+    float    *uniforms   = nullptr; /* [max_rows] */
+    float    *probe_p    = nullptr; /* [max_rows] */
+    int32_t  *scalar_out = nullptr; /* [max_rows] */
+    int32_t  *h_scalar   = nullptr; /* pinned */
+
+    /* timing of the dominant kernel */
+    bool                    timing = false;
+    std::vector<hipEvent_t> ev_start, ev_stop;
+    size_t                  ev_used = 0;
+
+    char err[512] = {0};
+};
+
+static int fail(geist_hip_sampler *s, int code, const char *fmt, ...) {
+    if (s) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(s->err, sizeof s->err, fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
+#define HIPCHK(s, call)                                                                        \
+    do {                                                                                       \
+        hipError_t e_ = (call);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return fail((s), e_ == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND, \
+                        "%s: %s", #call, hipGetErrorString(e_));                               \
+    } while (0)
+
+static int after_launch(geist_hip_sampler *s, const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(s, GEIST_HIP_E_BACKEND, "launch of %s failed: %s", what, hipGetErrorString(e));
+    return GEIST_HIP_OK;
+}
+
+/* ---- launch geometry ---------------------------------------------------------------------- */
+static bool plan_chunks(size_t rows, size_t n_vocab, int &nv, int &per_chunk, int &n_chunks) {
+    const size_t big   = (n_vocab + 8191) / 8192;
+    const size_t small = (n_vocab + 2047) / 2048;
+    if (big > (size_t) MAX_CHUNKS)
+        return false;
+    /* fewer than two workgroups per compute unit: cut the rows finer */
+    nv                 = (rows * big < 512 && small <= (size_t) MAX_CHUNKS) ? 2 : 8;
+    const size_t cap   = (size_t) 1024 * nv;
+    const size_t c0    = (n_vocab + cap - 1) / cap;
+    size_t       per   = (n_vocab + c0 - 1) / c0;
+    per                = (per + 63) / 64 * 64;
+    per_chunk          = (int) per;
+    n_chunks           = (int) ((n_vocab + per - 1) / per);
+    return true;
+}
+
+static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
+                       const struct geist_hip_sample_params *p, bool stochastic, Launch &L) {
+    if (!s || !r || !r->d_logits)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null sampler, rows or logits");
+    if (r->rows == 0 || r->n_vocab == 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "empty batch (rows=%zu, n_vocab=%zu)", r->rows,
+                    r->n_vocab);
+    if (r->rows > s->max_rows || r->n_vocab > s->max_vocab)
+        return fail(s, GEIST_HIP_E_INVALID_ARG,
+                    "batch %zu x %zu exceeds the workspace (%zu x %zu)", r->rows, r->n_vocab,
+                    s->max_rows, s->max_vocab);
+    if (r->ld < r->n_vocab)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "row stride %zu < n_vocab %zu", r->ld, r->n_vocab);
+    if (r->n_vocab > 0x7fffff00u)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "n_vocab too large");
+    int nv, per, nc;
+    if (!plan_chunks(r->rows, r->n_vocab, nv, per, nc) || nc > s->max_chunks)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "n_vocab %zu needs more than %d chunks",
+                    r->n_vocab, s->max_chunks);
+    const bool pen = p && r->d_history && r->d_history_len &&
+                     (p->repetition_penalty != 1.0f || p->frequency_penalty != 0.0f ||
+                      p->presence_penalty != 0.0f);
+    if (pen && r->history_ld > (size_t) HISTORY_MAX)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "history_ld %zu exceeds %d", r->history_ld,
+                    HISTORY_MAX);
+    if (pen && !(p->repetition_penalty > 0.0f))
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "repetition_penalty must be > 0");
+    L.rv.logits    = r->d_logits;
+    L.rv.ld        = (long) r->ld;
+    L.rv.n_vocab   = (int) r->n_vocab;
+    L.rv.per_chunk = per;
+    L.rv.n_chunks  = nc;
+    L.rv.vec_ok    = (((uintptr_t) r->d_logits) % 16 == 0) && (r->ld % 4 == 0);
+    L.rv.hist      = pen ? r->d_history : nullptr;
+    L.rv.hist_ld   = (long) r->history_ld;
+    L.rv.hist_len  = pen ? r->d_history_len : nullptr;
+    L.rv.rep       = pen ? p->repetition_penalty : 1.0f;
+    L.rv.freq      = pen ? p->frequency_penalty : 0.0f;
+    L.rv.pres      = pen ? p->presence_penalty : 0.0f;
+    /* the soft-cap is monotone, so greedy rows skip it (head.c:145-149) */
+    L.rv.softcap   = (p && stochastic && p->logit_softcap > 0.0f) ? p->logit_softcap : 0.0f;
+    L.rows         = (int) r->rows;
+    L.nv           = nv;
+    L.pen          = pen;
+    L.stream       = s->stream;
+    return GEIST_HIP_OK;
+}
+
+/* ---- timing brackets ---------------------------------------------------------------------- */
+static void mark_start(geist_hip_sampler *s) {
+    if (!s->timing)
+        return;
+    if (s->ev_used == s->ev_start.size()) {
+        hipEvent_t a, b;
+        if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess)
+            return;
+        s->ev_start.push_back(a);
+        s->ev_stop.push_back(b);
+    }
+    (void) hipEventRecord(s->ev_start[s->ev_used], s->stream);
+}
+static void mark_stop(geist_hip_sampler *s) {
+    if (!s->timing || s->ev_used >= s->ev_start.size())
+        return;
+    (void) hipEventRecord(s->ev_stop[s->ev_used], s->stream);
+    s->ev_used++;
+}
+
+/* ============================================================================================ */
+extern "C" {
+
+int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void *stream,
+                             geist_hip_sampler **out) {
+    if (!out || max_rows == 0 || max_vocab == 0)
+        return GEIST_HIP_E_INVALID_ARG; /* sampler.c:138-140 */
+    *out = nullptr;
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || device < 0 || device >= n_dev)
+        return GEIST_HIP_E_BACKEND;
+    geist_hip_sampler *s = new (std::nothrow) geist_hip_sampler();
+    if (!s)
+        return GEIST_HIP_E_OOM;
+    s->device    = device;
+    s->stream    = (hipStream_t) stream;
+    s->max_rows  = max_rows;
+    s->max_vocab = max_vocab;
+    size_t mc    = (max_vocab + 2047) / 2048;
+    if (mc > (size_t) MAX_CHUNKS)
+        mc = MAX_CHUNKS;
+    if ((max_vocab + 8191) / 8192 > (size_t) MAX_CHUNKS) {
+        delete s;
+        return GEIST_HIP_E_UNSUPPORTED;
+    }
+    s->max_chunks = (int) mc;
+    const size_t rc = max_rows * mc;
+    hipError_t   e  = hipSetDevice(device);
+    if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_key, rc * TOPK_CAND_CAP * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_idx, rc * TOPK_CAND_CAP * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_cnt, rc * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->probe_p, max_rows * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->scalar_out, max_rows * sizeof(int32_t));
+    if (e == hipSuccess) e = hipHostMalloc((void **) &s->h_scalar, 64 * sizeof(int32_t), hipHostMallocDefault);
+    if (e != hipSuccess) {
+        const int code = e == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND;
+        geist_hip_sampler_destroy(s);
+        return code; /* sampler.c:142-145 */
+    }
+    *out = s;
+    return GEIST_HIP_OK;
+}
+
+void geist_hip_sampler_destroy(geist_hip_sampler *s) {
+    if (!s)
+        return;
+    (void) hipSetDevice(s->device);
+    (void) hipStreamSynchronize(s->stream);
+    (void) hipFree(s->chunk_best);
+    (void) hipFree(s->chunk_sum);
+    (void) hipFree(s->cand_key);
+    (void) hipFree(s->cand_idx);
+    (void) hipFree(s->cand_cnt);
+    (void) hipFree(s->row_flag);
+    (void) hipFree(s->uniforms);
+    (void) hipFree(s->probe_p);
+    (void) hipFree(s->scalar_out);
+    if (s->h_scalar)
+        (void) hipHostFree(s->h_scalar);
+    for (hipEvent_t e : s->ev_start)
+        (void) hipEventDestroy(e);
+    for (hipEvent_t e : s->ev_stop)
+        (void) hipEventDestroy(e);
+    delete s;
+}
+
+const char *geist_hip_sampler_last_error(const geist_hip_sampler *s) { return s ? s->err : ""; }
+
+int geist_hip_sampler_sync(geist_hip_sampler *s) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipStreamSynchronize(s->stream));
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_set_stream(geist_hip_sampler *s, void *stream) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->stream = (hipStream_t) stream;
+    return GEIST_HIP_OK;
+}
+
+/* What the configuration asks for after the precedence rules. */
+struct Resolved {
+    bool  greedy;
+    bool  use_k, use_p, use_m;
+    int   k;
+    float top_p, min_p, inv_t;
+};
+
+static int resolve(geist_hip_sampler *s, const struct geist_hip_sample_params *p, size_t n_vocab,
+                   Resolved &r) {
+    if (!p)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null params");
+    const float T = p->temperature;
+    r             = Resolved{};
+    if (!(T > 0.0f)) { /* T == 0 in the dispatch, T < 0 inside each sampler: argmax, no draw */
+        r.greedy = true;
+        return GEIST_HIP_OK;
+    }
+    r.inv_t = 1.0f / T; /* sampler.c:77 */
+    const bool p_set = p->top_p > 0.0f && p->top_p < 1.0f;
+    if (p->precedence == GEIST_HIP_PRECEDENCE_REFERENCE) {
+        if (p->min_p != 0.0f)
+            return fail(s, GEIST_HIP_E_INVALID_ARG,
+                        "min_p needs GEIST_HIP_PRECEDENCE_CHAIN (the reference has no min-p)");
+        if (p->top_k > 1) { /* head.c:174-176: top-k wins, top_p is not consulted */
+            r.use_k = (size_t) p->top_k < n_vocab; /* sampler.c:187-189 */
+        } else if (p_set) {
+            r.use_p = true;
+        }
+    } else if (p->precedence == GEIST_HIP_PRECEDENCE_CHAIN) {
+        r.use_k = p->top_k > 1 && (size_t) p->top_k < n_vocab;
+        r.use_p = p_set;
+        r.use_m = p->min_p > 0.0f;
+    } else {
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown precedence %d", p->precedence);
+    }
+    r.k     = r.use_k ? (p->top_k > 8192 ? 8192 : p->top_k) : 0; /* sampler.c:213-215 */
+    r.top_p = r.use_p ? p->top_p : 1.0f;
+    r.min_p = r.use_m ? p->min_p : 0.0f;
+    return GEIST_HIP_OK;
+}
+
+static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                       const struct geist_hip_sample_params *params, const float *d_uniforms,
+                       geist_hip_token_t *d_out) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null output");
+    Resolved rs;
+    int      rc = resolve(s, params, rows ? rows->n_vocab : 0, rs);
+    if (rc)
+        return rc;
+    Launch L;
+    rc = make_launch(s, rows, params, !rs.greedy, L);
+    if (rc)
+        return rc;
+    if (!rs.greedy && !d_uniforms)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic configuration without uniforms");
+    HIPCHK(s, hipSetDevice(s->device));
+
+    FinalLaunch f{};
+    f.inv_t      = rs.inv_t;
+    f.top_p      = rs.top_p;
+    f.min_p      = rs.min_p;
+    f.uniforms   = d_uniforms;
+    f.chunk_best = s->chunk_best;
+    f.chunk_sum  = s->chunk_sum;
+    f.cand_key   = s->cand_key;
+    f.cand_idx   = s->cand_idx;
+    f.cand_cnt   = s->cand_cnt;
+    f.out        = d_out;
+    f.cap        = TOPK_CAND_CAP;
+
+    if (rs.greedy) {
+        mark_start(s);
+        launch_chunk_best(L, s->chunk_best);
+        mark_stop(s);
+        f.mode = FINAL_ARGMAX;
+        launch_row_final(L, f);
+        return after_launch(s, "argmax");
+    }
+    if (rs.use_k) {
+        if (rs.k > TOPK_FAST_MAX) {
+            f.mode = FINAL_TOPK;
+            f.k    = rs.k;
+            mark_start(s);
+            const int e = launch_topk_general(L, f);
+            mark_stop(s);
+            if (e != 0)
+                return fail(s, GEIST_HIP_E_BACKEND, "top-k (general) launch: %s",
+                            hipGetErrorString((hipError_t) e));
+            return after_launch(s, "top-k (general)");
+        }
+        mark_start(s);
+        launch_topk_scan(L, rs.k, TOPK_CAND_CAP, s->cand_key, s->cand_idx, s->cand_cnt);
+        mark_stop(s);
+        f.mode = FINAL_TOPK;
+        f.k    = rs.k;
+        launch_row_final(L, f);
+        return after_launch(s, "top-k");
+    }
+    if (!rs.use_p && !rs.use_m) {
+        launch_chunk_best(L, s->chunk_best);
+        mark_start(s);
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+        mark_stop(s);
+        f.mode = FINAL_TEMPERATURE;
+        launch_row_final(L, f);
+        return after_launch(s, "temperature");
+    }
+    return fail(s, GEIST_HIP_E_UNSUPPORTED, "full-vocabulary top-p / min-p is not built yet");
+}
+
+int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                          const struct geist_hip_sample_params *params, const float *d_uniforms,
+                          geist_hip_token_t *d_out_tokens) {
+    return sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+}
+
+int geist_hip_sample_rows_rng(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                              const struct geist_hip_sample_params *params,
+                              uint64_t *d_rng_states, int shared,
+                              geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!rows || !params)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null rows or params");
+    if (rows->rows > s->max_rows)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "too many rows");
+    const bool greedy = !(params->temperature > 0.0f);
+    if (!greedy) {
+        if (!d_rng_states)
+            return fail(s, GEIST_HIP_E_INVALID_ARG, "null rng states");
+        HIPCHK(s, hipSetDevice(s->device));
+        launch_rng_units(s->stream, d_rng_states, shared, (int) rows->rows, s->uniforms);
+    }
+    return sample_impl(s, rows, params, greedy ? nullptr : s->uniforms, d_out_tokens);
+}
+
+int geist_hip_argmax_f32(geist_hip_sampler *s, const float *d_logits, size_t n,
+                         int32_t *out_index) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!out_index)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null out_index");
+    struct geist_hip_rows r{};
+    r.d_logits = d_logits;
+    r.ld       = n;
+    r.rows     = 1;
+    r.n_vocab  = n;
+    struct geist_hip_sample_params p{};
+    p.repetition_penalty = 1.0f;
+    int rc = sample_impl(s, &r, &p, nullptr, s->scalar_out);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipMemcpyAsync(s->h_scalar, s->scalar_out, sizeof(int32_t), hipMemcpyDeviceToHost,
+                             s->stream));
+    HIPCHK(s, hipStreamSynchronize(s->stream));
+    *out_index = s->h_scalar[0];
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_apply_penalties(geist_hip_sampler *s, float *d_logits, size_t ld, size_t rows,
+                              size_t n_vocab, const int32_t *d_history, size_t history_ld,
+                              const int32_t *d_history_len, float rep, float freq, float pres) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_history || !d_history_len)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null history");
+    struct geist_hip_rows r{};
+    r.d_logits      = d_logits;
+    r.ld            = ld;
+    r.rows          = rows;
+    r.n_vocab       = n_vocab;
+    r.d_history     = d_history;
+    r.history_ld    = history_ld;
+    r.d_history_len = d_history_len;
+    struct geist_hip_sample_params p{};
+    p.repetition_penalty = rep;
+    p.frequency_penalty  = freq;
+    p.presence_penalty   = pres;
+    Launch L;
+    int    rc = make_launch(s, &r, &p, false, L);
+    if (rc)
+        return rc;
+    if (!L.pen)
+        return GEIST_HIP_OK; /* neutral parameters: nothing to do */
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_penalties(L, d_logits);
+    return after_launch(s, "penalties");
+}
+
+int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                           const struct geist_hip_sample_params *params, float *d_probs,
+                           size_t ld_probs) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!params || !d_probs)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null params or output");
+    if (!(params->temperature > 0.0f))
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "softmax needs temperature > 0");
+    Launch L;
+    int    rc = make_launch(s, rows, params, true, L);
+    if (rc)
+        return rc;
+    if (ld_probs < rows->n_vocab)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_probs < n_vocab");
+    const float inv_t = 1.0f / params->temperature;
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_chunk_best(L, s->chunk_best);
+    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+    launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs);
+    return after_launch(s, "softmax");
+}
+
+int geist_hip_spec_verify(geist_hip_sampler *s, const float *, size_t, const float *, size_t,
+                          const int32_t *, const float *, size_t, size_t, size_t, float,
+                          geist_hip_token_t *, int32_t *) {
+    return fail(s, GEIST_HIP_E_UNSUPPORTED, "speculative verification is not built yet");
+}
+
+/* ---- device-memory helpers ----------------------------------------------------------------- */
+int geist_hip_malloc(geist_hip_sampler *s, size_t bytes, void **d_ptr) {
+    if (!s || !d_ptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipSetDevice(s->device));
+    HIPCHK(s, hipMalloc(d_ptr, bytes ? bytes : 1));
+    return GEIST_HIP_OK;
+}
+int geist_hip_free(geist_hip_sampler *s, void *d_ptr) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipFree(d_ptr));
+    return GEIST_HIP_OK;
+}
+int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, s->stream));
+    HIPCHK(s, hipStreamSynchronize(s->stream));
+    return GEIST_HIP_OK;
+}
+int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, size_t bytes) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, s->stream));
+    HIPCHK(s, hipStreamSynchronize(s->stream));
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_timing_enable(geist_hip_sampler *s, int on) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->timing = on != 0;
+    return GEIST_HIP_OK;
+}
+int geist_hip_sampler_timing_read(geist_hip_sampler *s, double *ms_total, long *launches,
+                                  int reset) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipStreamSynchronize(s->stream));
+    double tot = 0.0;
+    for (size_t i = 0; i < s->ev_used; ++i) {
+        float ms = 0.0f;
+        HIPCHK(s, hipEventElapsedTime(&ms, s->ev_start[i], s->ev_stop[i]));
+        tot += ms;
+    }
+    if (ms_total)
+        *ms_total = tot;
+    if (launches)
+        *launches = (long) s->ev_used;
+    if (reset)
+        s->ev_used = 0;
+    return GEIST_HIP_OK;
+}
+
+} /* extern "C" */

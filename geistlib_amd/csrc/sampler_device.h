@@ -1,0 +1,261 @@
+/*
+ * sampler_device.h -- device-side building blocks shared by the sampling kernels (gfx950,
+ * wavefront 64, 256-thread workgroups).
+ *
+ * Layout of a logit row in a launch: the row is cut into n_chunks pieces of `per_chunk`
+ * elements (a multiple of 64 floats, so every chunk starts on a 256-byte boundary of the row).
+ * One workgroup owns one (row, chunk) pair and holds the whole chunk in registers: thread t
+ * owns the float4 groups f = j * 256 + t, j = 0 .. NV-1, i.e. a wavefront reads 1 KiB of
+ * consecutive addresses per load instruction.
+ */
+#ifndef GEIST_SAMPLER_DEVICE_H
+#define GEIST_SAMPLER_DEVICE_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "glibc_expf.h"
+#include "sampler_kernels.h"
+
+namespace gs {
+
+constexpr int TPB    = 256;
+constexpr int WAVE   = 64;
+constexpr int NWAVES = TPB / WAVE;
+
+/* Order-preserving map fp32 -> u32 used for every comparison on this path. It restates the
+ * reference's comparisons (src/engine/sampler.c:56, 72, 171-174): -0 and +0 are equal, and a
+ * NaN never compares greater, so it takes the lowest key. */
+__device__ __forceinline__ uint32_t f2key(float x) {
+    uint32_t b = __float_as_uint(x);
+    if (x != x)
+        return 0u;
+    if ((b << 1) == 0u)
+        b = 0u;
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float key2f(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+/* (key, index) packed so that an unsigned max picks the greater key and, among equal keys,
+ * the LOWER index (src/engine/sampler.c:56: strict '>' keeps the first maximum). */
+__device__ __forceinline__ uint64_t pack_best(uint32_t key, uint32_t idx) {
+    return ((uint64_t) key << 32) | (uint64_t) (0xffffffffu - idx);
+}
+__device__ __forceinline__ uint32_t best_idx(uint64_t p) { return 0xffffffffu - (uint32_t) p; }
+__device__ __forceinline__ uint32_t best_key(uint64_t p) { return (uint32_t) (p >> 32); }
+
+/* ---- wavefront-64 reductions -------------------------------------------------------------- */
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
+    uint32_t lo = (uint32_t) v, hi = (uint32_t) (v >> 32);
+    lo = (uint32_t) __shfl_xor((int) lo, m, WAVE);
+    hi = (uint32_t) __shfl_xor((int) hi, m, WAVE);
+    return ((uint64_t) hi << 32) | lo;
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const uint64_t o = shfl_xor_u64(v, m);
+        v                = o > v ? o : v;
+    }
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const uint32_t o = (uint32_t) __shfl_xor((int) v, m, WAVE);
+        v                = o > v ? o : v;
+    }
+    return v;
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        v += __shfl_xor(v, m, WAVE);
+    return v;
+}
+/* inclusive prefix sum over the lanes of a wavefront, lane order */
+__device__ __forceinline__ double wave_scan_f64(double v) {
+    const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const double o = __shfl_up(v, d, WAVE);
+        if (lane >= d)
+            v += o;
+    }
+    return v;
+}
+__device__ __forceinline__ int wave_scan_i32(int v) {
+    const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int o = __shfl_up(v, d, WAVE);
+        if (lane >= d)
+            v += o;
+    }
+    return v;
+}
+
+/* ---- workgroup combines through LDS -------------------------------------------------------- */
+/* All 256 threads call; every thread receives the maximum. `scratch` holds NWAVES entries. */
+__device__ __forceinline__ uint64_t block_max_u64(uint64_t v, uint64_t *scratch) {
+    v = wave_max_u64(v);
+    if ((threadIdx.x & (WAVE - 1)) == 0)
+        scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    uint64_t r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NWAVES; ++w)
+        r = scratch[w] > r ? scratch[w] : r;
+    __syncthreads();
+    return r;
+}
+/* Sum over the workgroup in a fixed order (lanes by butterfly, then waves 0..3). */
+__device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
+    v = wave_sum_f64(v);
+    if ((threadIdx.x & (WAVE - 1)) == 0)
+        scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    double r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NWAVES; ++w)
+        r += scratch[w];
+    __syncthreads();
+    return r;
+}
+/* Inclusive prefix sum over the 256 threads in thread order; *total receives the sum. */
+__device__ __forceinline__ double block_scan_f64(double v, double *scratch, double *total) {
+    const int w    = threadIdx.x / WAVE;
+    const int lane = threadIdx.x & (WAVE - 1);
+    v              = wave_scan_f64(v);
+    if (lane == WAVE - 1)
+        scratch[w] = v;
+    __syncthreads();
+    double off = 0.0, all = 0.0;
+#pragma unroll
+    for (int i = 0; i < NWAVES; ++i) {
+        if (i < w)
+            off += scratch[i];
+        all += scratch[i];
+    }
+    __syncthreads();
+    if (total)
+        *total = all;
+    return v + off;
+}
+__device__ __forceinline__ int block_scan_i32(int v, int *scratch, int *total) {
+    const int w    = threadIdx.x / WAVE;
+    const int lane = threadIdx.x & (WAVE - 1);
+    v              = wave_scan_i32(v);
+    if (lane == WAVE - 1)
+        scratch[w] = v;
+    __syncthreads();
+    int off = 0, all = 0;
+#pragma unroll
+    for (int i = 0; i < NWAVES; ++i) {
+        if (i < w)
+            off += scratch[i];
+        all += scratch[i];
+    }
+    __syncthreads();
+    if (total)
+        *total = all;
+    return v + off;
+}
+
+/* ---- the logit transform applied while a chunk is read ------------------------------------ */
+
+/* Penalty arithmetic; every step rounds once, matching the CPU statement of the same rule. */
+__device__ __forceinline__ float penalise(float l, uint32_t count, float rep, float freq,
+                                          float pres) {
+    l = l > 0.0f ? __fdiv_rn(l, rep) : __fmul_rn(l, rep);
+    l = __fsub_rn(l, __fmul_rn(freq, (float) count));
+    l = __fsub_rn(l, pres);
+    return l;
+}
+
+/* Counts the occurrences of each vocabulary id of [base, end) in the row's history (end - base
+ * <= CHUNK; ids outside the row's vocabulary fall outside every chunk and are ignored).
+ * cnt16 packs two 16-bit counters per word (histories are capped at 65535 entries). */
+template <int CHUNK>
+__device__ __forceinline__ void history_counts(const RowView &rv, int row, int base, int end,
+                                               uint32_t *cnt16) {
+    for (int i = threadIdx.x; i < CHUNK / 2; i += TPB)
+        cnt16[i] = 0u;
+    __syncthreads();
+    int len = rv.hist_len ? rv.hist_len[row] : 0;
+    if (len > rv.hist_ld)
+        len = (int) rv.hist_ld;
+    const int32_t *h   = rv.hist + (long) row * rv.hist_ld;
+    for (int i = threadIdx.x; i < len; i += TPB) {
+        const int t   = h[i];
+        const int off = t - base;
+        if (off >= 0 && t < end)
+            atomicAdd(&cnt16[off >> 1], 1u << (16 * (off & 1)));
+    }
+    __syncthreads();
+}
+
+/* Loads the chunk [base, end) of a row into registers (layout in the file header), applying
+ * penalties (when cnt16 != NULL) and the soft-cap. Positions at or beyond `end` hold -inf. */
+template <int NV>
+__device__ __forceinline__ void load_chunk(const RowView &rv, const float *__restrict__ row,
+                                           int base, int end, const uint32_t *cnt16,
+                                           float4 (&v)[NV]) {
+    const int   tid  = threadIdx.x;
+    const float ninf = -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+        if (rv.vec_ok && e + 3 < end) {
+            v[j] = *reinterpret_cast<const float4 *>(row + e);
+        } else {
+            v[j].x = e + 0 < end ? row[e + 0] : ninf;
+            v[j].y = e + 1 < end ? row[e + 1] : ninf;
+            v[j].z = e + 2 < end ? row[e + 2] : ninf;
+            v[j].w = e + 3 < end ? row[e + 3] : ninf;
+        }
+    }
+    if (cnt16) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int      off = 4 * (j * TPB + tid); /* even, so two words cover the float4 */
+            const uint32_t w0  = cnt16[(off >> 1) + 0];
+            const uint32_t w1  = cnt16[(off >> 1) + 1];
+            if (w0 | w1) {
+                if (w0 & 0xffffu)
+                    v[j].x = penalise(v[j].x, w0 & 0xffffu, rv.rep, rv.freq, rv.pres);
+                if (w0 >> 16)
+                    v[j].y = penalise(v[j].y, w0 >> 16, rv.rep, rv.freq, rv.pres);
+                if (w1 & 0xffffu)
+                    v[j].z = penalise(v[j].z, w1 & 0xffffu, rv.rep, rv.freq, rv.pres);
+                if (w1 >> 16)
+                    v[j].w = penalise(v[j].w, w1 >> 16, rv.rep, rv.freq, rv.pres);
+            }
+        }
+    }
+    if (rv.softcap > 0.0f) {
+        const float c = rv.softcap;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            v[j].x = __fmul_rn(tanhf(__fdiv_rn(v[j].x, c)), c);
+            v[j].y = __fmul_rn(tanhf(__fdiv_rn(v[j].y, c)), c);
+            v[j].z = __fmul_rn(tanhf(__fdiv_rn(v[j].z, c)), c);
+            v[j].w = __fmul_rn(tanhf(__fdiv_rn(v[j].w, c)), c);
+        }
+    }
+}
+
+__device__ __forceinline__ float f4_get(const float4 &q, int c) {
+    return c == 0 ? q.x : c == 1 ? q.y : c == 2 ? q.z : q.w;
+}
+
+/* fp32 steps of the reference's softmax argument, (l - max) * inv_t (sampler.c:80), kept as
+ * two separately rounded operations. */
+__device__ __forceinline__ float softmax_arg(float l, float mx, float inv_t) {
+    return __fmul_rn(__fsub_rn(l, mx), inv_t);
+}
+
+} // namespace gs
+#endif

@@ -1,0 +1,70 @@
+/*
+ * sampler_kernels.h -- host-visible launch interface of the sampling kernels.
+ */
+#ifndef GEIST_SAMPLER_KERNELS_H
+#define GEIST_SAMPLER_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gs {
+
+constexpr int MAX_CHUNKS     = 128;  /* chunks per row */
+constexpr int TOPK_CAND_CAP  = 256;  /* candidates one chunk may hand on */
+constexpr int TOPK_FAST_MAX  = 128;  /* largest k served by the candidate path */
+constexpr int TOPK_MAX       = 8192; /* the reference caps top_k here (sampler.c:213-215) */
+constexpr int FINAL_CAND_MAX = 4096; /* candidates one row may merge in LDS */
+constexpr int HISTORY_MAX    = 65535;
+
+enum { FINAL_ARGMAX = 0, FINAL_TEMPERATURE = 1, FINAL_TOPK = 2 };
+
+/* One batch of logit rows as the kernels see it, with the transform applied while reading. */
+struct RowView {
+    const float   *logits; /* row 0 */
+    long           ld;
+    int            n_vocab;
+    int            per_chunk;
+    int            n_chunks;
+    int            vec_ok; /* rows are 16-byte aligned: float4 loads allowed */
+    const int32_t *hist;   /* NULL = no penalties */
+    long           hist_ld;
+    const int32_t *hist_len;
+    float          rep, freq, pres;
+    float          softcap; /* 0 = off */
+};
+
+struct Launch {
+    RowView     rv;
+    int         rows;
+    int         nv;  /* float4 groups per thread: 2 or 8 */
+    bool        pen; /* history lookup on */
+    hipStream_t stream;
+};
+
+struct FinalLaunch {
+    int             mode, k, cap;
+    float           inv_t, top_p, min_p;
+    const float    *uniforms;
+    const uint64_t *chunk_best;
+    const double   *chunk_sum;
+    const uint32_t *cand_key;
+    const int32_t  *cand_idx;
+    const int32_t  *cand_cnt;
+    int32_t        *out;
+};
+
+void launch_chunk_best(const Launch &L, uint64_t *chunk_best);
+void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
+                         double *chunk_sum, const int32_t *probe_token, float *probe_p);
+void launch_topk_scan(const Launch &L, int k, int cap, uint32_t *cand_key, int32_t *cand_idx,
+                      int32_t *cand_cnt);
+void launch_row_final(const Launch &L, const FinalLaunch &f);
+/* returns a hipError_t value */
+int  launch_topk_general(const Launch &L, const FinalLaunch &f);
+void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
+                        const double *chunk_sum, float *probs, long ld_probs);
+void launch_penalties(const Launch &L, float *logits_rw);
+void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
+
+} // namespace gs
+#endif

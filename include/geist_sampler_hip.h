@@ -1,0 +1,169 @@
+/*
+ * geist_sampler_hip.h -- C ABI of the MI355X (gfx950) token-sampling path.
+ *
+ * Plain C: pointers and sizes only. Logit rows [rows x n_vocab] fp32 stay resident in device
+ * memory; every entry point enqueues hand-written HIP kernels on the sampler's stream and
+ * returns (asynchronous unless stated otherwise). There is no CPU fallback: when no device
+ * or no kernel image for it is available the calls fail with GEIST_E_BACKEND.
+ *
+ * Each declaration cites the interface of the reference (geistlib 0.9.0, paths relative to
+ * its tree) that it replaces or extends.
+ */
+#ifndef GEIST_SAMPLER_HIP_H
+#define GEIST_SAMPLER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes: numerically identical to `enum geist_status` (include/geist.h:46-67), so a
+ * caller compiled against the reference header can return them unchanged. */
+#define GEIST_HIP_OK 0
+#define GEIST_HIP_E_OOM 1
+#define GEIST_HIP_E_INVALID_ARG 2
+#define GEIST_HIP_E_INTERNAL 3
+#define GEIST_HIP_E_UNSUPPORTED 7
+#define GEIST_HIP_E_BACKEND 9
+
+/* geist_token_t (include/geist.h:190) */
+typedef int32_t geist_hip_token_t;
+
+typedef struct geist_hip_sampler geist_hip_sampler;
+
+/* Replaces geist_sampler_workspace_init (src/engine/sampler.h:50-57, sampler.c:136-148): the
+ * caller-owned scratch of the reference becomes a device workspace sized once for
+ * `max_rows` rows of up to `max_vocab` logits. `stream` is a hipStream_t (NULL = the
+ * device's default stream). All later calls on this object run on that stream; one object
+ * per host thread, as one workspace per session in the reference. */
+int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void *stream,
+                             geist_hip_sampler **out);
+/* Replaces geist_sampler_workspace_destroy (sampler.c:150-157). NULL is a no-op. */
+void geist_hip_sampler_destroy(geist_hip_sampler *s);
+/* Text of the last failure on this object (the reference keeps such text in per-handle
+ * error slots, src/base/error.h:34-39). Never NULL. */
+const char *geist_hip_sampler_last_error(const geist_hip_sampler *s);
+/* Blocks until everything enqueued on the sampler's stream has finished. */
+int geist_hip_sampler_sync(geist_hip_sampler *s);
+/* Rebinds the stream later calls are enqueued on (NULL = default stream). */
+int geist_hip_sampler_set_stream(geist_hip_sampler *s, void *stream);
+
+/* A batch of logit rows in device memory. Row r starts at d_logits + r * ld.
+ * The optional token history drives the penalties: row r owns d_history[r * history_ld ..
+ * + d_history_len[r]) ; ids outside [0, n_vocab) are ignored. */
+struct geist_hip_rows {
+    const float   *d_logits;
+    size_t         ld;
+    size_t         rows;
+    size_t         n_vocab;
+    const int32_t *d_history;     /* NULL = no history */
+    size_t         history_ld;
+    const int32_t *d_history_len; /* rows entries */
+};
+
+/* Sampling configuration for one call. The first four fields are the sampler fields of
+ * `struct geist_session_opts` (include/geist.h:213-229) after
+ * transformer_session_apply_opts (src/archs/transformer/forward/step.c:385-411).
+ *
+ * precedence:
+ *   GEIST_HIP_PRECEDENCE_REFERENCE  the reference's dispatch (head.c:172-183): T == 0 -> argmax;
+ *                                   top_k > 1 -> top-k (top_p ignored); 0 < top_p < 1 -> top-p;
+ *                                   else temperature. min_p must be 0.
+ *   GEIST_HIP_PRECEDENCE_CHAIN      temperature -> top-k -> top-p -> min-p composed, each filter
+ *                                   acting on the survivors of the previous one. With a single
+ *                                   filter set it gives the same token as the reference mode.
+ * Penalties (history present and any of the three non-neutral) and the soft-cap
+ * (tanhf(x / cap) * cap, head.c:148-159; applied only when T > 0) act on the logits before
+ * either precedence, without writing to d_logits. */
+#define GEIST_HIP_PRECEDENCE_REFERENCE 0
+#define GEIST_HIP_PRECEDENCE_CHAIN 1
+struct geist_hip_sample_params {
+    float temperature;
+    float top_p;
+    int   top_k;
+    float min_p;
+    float repetition_penalty; /* 1 = neutral */
+    float frequency_penalty;  /* 0 = neutral */
+    float presence_penalty;   /* 0 = neutral */
+    float logit_softcap;      /* 0 = off */
+    int   precedence;
+};
+
+/* Replaces the sampler dispatch of finalize_logits_batch (head.c:274-304) for `rows` rows at
+ * once: d_out_tokens[r] = token sampled from row r with the uniform d_uniforms[r] (the value
+ * geist_rng_next_unit would have returned for that row). d_uniforms may be NULL when the
+ * configuration is greedy. */
+int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                          const struct geist_hip_sample_params *params, const float *d_uniforms,
+                          geist_hip_token_t *d_out_tokens);
+
+/* Same, drawing the uniforms on the device from xorshift64* states (struct geist_rng,
+ * src/engine/sampler.h:28-32; sampler.c:35-48) held in device memory.
+ *   shared != 0: one state for the whole batch, row r takes the (r+1)-th draw and the state
+ *                advances by `rows` draws -- the reference's batch order (head.c:274-304).
+ *   shared == 0: d_rng_states[r] belongs to row r and advances by one draw.
+ * Greedy configurations leave the states untouched (sampler.c:110-112, 184-186, 238-240). */
+int geist_hip_sample_rows_rng(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                              const struct geist_hip_sample_params *params,
+                              uint64_t *d_rng_states, int shared,
+                              geist_hip_token_t *d_out_tokens);
+
+/* Fills the backend slot `argmax_f32` (include/geist_backend.h:414-421): greedy argmax over one
+ * fp32 row of n logits in device memory, lowest index wins ties; synchronous, only the 4-byte
+ * index crosses to the host. */
+int geist_hip_argmax_f32(geist_hip_sampler *s, const float *d_logits, size_t n,
+                         int32_t *out_index);
+
+/* Penalties applied IN PLACE to the rows (the caller-side mutation the reference performs for
+ * its soft-cap, head.c:148-159). For each distinct history id t of a row with count c:
+ *   l = logits[t]; l = l > 0 ? l / rep : l * rep; l -= freq * c; l -= pres.
+ * No reference counterpart (the reference has no penalties). */
+int geist_hip_apply_penalties(geist_hip_sampler *s, float *d_logits, size_t ld, size_t rows,
+                              size_t n_vocab, const int32_t *d_history, size_t history_ld,
+                              const int32_t *d_history_len, float rep, float freq, float pres);
+
+/* Normalised probabilities of each row after penalties, soft-cap and temperature, the values
+ * the reference's top-p path holds in ws->probs after sampler.c:246-253:
+ *   d_probs[r * ld_probs + i] = (float)((double)expf((l_i - max) / T) / sum). */
+int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                           const struct geist_hip_sample_params *params, float *d_probs,
+                           size_t ld_probs);
+
+/* Speculative-decode verification for n_seq sequences with draft length L (no reference
+ * counterpart: include/geist_util.h:233-240 documents that the reference's speculative loop
+ * omits rejection sampling; the batch shape is that of verify_forward,
+ * src/archs/transformer/arch_ops.c:176-270).
+ *   d_target   [n_seq][L+1][n_vocab] logits, sequence stride (L+1)*ld_t, row stride ld_t
+ *   d_draft_q  [n_seq][L][n_vocab] draft probabilities, row stride ld_q
+ *   d_draft    [n_seq][L] draft token ids,  d_uniforms [n_seq][L+1]
+ * T > 0: position j accepted iff u_j * q_j(x_j) < p_j(x_j); at the first rejection the token is
+ * drawn with u_L from max(0, p_j - q_j) renormalised; if all are accepted the bonus token is a
+ * temperature draw from row L with u_L. T <= 0: exact-match against the row argmax.
+ *   d_out_tokens [n_seq][L+1]: accepted draft ids, then the emitted token; rest untouched.
+ *   d_n_accepted [n_seq]. */
+int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
+                          const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
+                          const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,
+                          float temperature, geist_hip_token_t *d_out_tokens,
+                          int32_t *d_n_accepted);
+
+/* ---- small device-memory helpers so that a plain-C host needs no HIP headers -------------- */
+int geist_hip_malloc(geist_hip_sampler *s, size_t bytes, void **d_ptr);
+int geist_hip_free(geist_hip_sampler *s, void *d_ptr);
+int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes);   /* sync */
+int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, size_t bytes); /* sync */
+
+/* Timing of the kernels this object enqueues, for benchmarks: when enabled, each sampling call
+ * brackets its dominant (logit-streaming) kernel with events on the sampler's stream.
+ * geist_hip_sampler_timing_read synchronises and returns the accumulated milliseconds and the
+ * number of bracketed launches since the last reset. */
+int geist_hip_sampler_timing_enable(geist_hip_sampler *s, int on);
+int geist_hip_sampler_timing_read(geist_hip_sampler *s, double *ms_total, long *launches,
+                                  int reset);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GEIST_SAMPLER_HIP_H */

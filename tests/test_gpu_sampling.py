@@ -1,0 +1,300 @@
+"""GPU parity tests proper: the HIP path, called through the C ABI, against the CPU oracle on
+identical logits and identical uniforms. Token ids are bit-exact (lowest index wins ties) except
+draws within 1e-6 of a CDF boundary, which are counted and printed."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from gpu_util import compare_ids, run_rows, to_dev  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def hs():
+    from geistlib_amd import HipSampler
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a device; the sampling path has no CPU fallback")
+    s = HipSampler(max_rows=512, max_vocab=262144)
+    yield s
+    s.close()
+
+
+def P(**kw):
+    from geistlib_amd import SampleParams
+    return SampleParams.make(**kw)
+
+
+def rows_rng(seed, rows, n, scale=2.0, ties=False):
+    g = np.random.default_rng(seed)
+    x = (g.standard_normal((rows, n)) * scale).astype(np.float32)
+    if ties:
+        x = (np.round(x * 4) / 4).astype(np.float32)
+    u = (g.integers(0, 1 << 24, rows).astype(np.float32) / np.float32(1 << 24)).astype(np.float32)
+    return x, u
+
+
+# ----------------------------------------------------------------------------------- argmax
+@pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 256, 1000, 2048, 2049, 8191, 8192, 8193, 50000,
+                               128256, 262144])
+def test_argmax_matches_oracle(hs, oracle, n):
+    print(f"argmax n={n}", flush=True)
+    x, _ = rows_rng(n, 7, n)
+    x[3, :] = np.round(x[3, :])            # many exact ties
+    x[4, :] = 1.5                          # all equal -> index 0
+    x[5, n // 2:] = x[5].max() + 1         # tie of the maximum: first of the upper half
+    got = run_rows(hs, torch, x, None, P(temperature=0.0))
+    want = [oracle.argmax(x[r]) for r in range(x.shape[0])]
+    assert got.tolist() == want
+
+
+def test_argmax_reference_vectors(hs):
+    # tests/test_sampler_unit.c:33-37 of the reference -> 3
+    x = np.array([[-1, 2, .5, 3, 3, -.5]], dtype=np.float32)
+    assert run_rows(hs, torch, x, None, P(temperature=0.0)).tolist() == [3]
+    # tests/test_fused_probe_agreement_unit.c:147-157 -> 77, through the backend-slot entry point
+    p = np.array([100.0 if i == 77 else i % 7 for i in range(256)], dtype=np.float32)
+    assert hs.argmax_f32(to_dev(p, torch)) == 77
+
+
+def test_argmax_special_values(hs, oracle):
+    n = 5000
+    x, _ = rows_rng(1, 6, n)
+    x[0, 10] = np.nan                      # NaN elsewhere never wins
+    x[1, 0] = np.nan                       # NaN at index 0 is never displaced
+    x[2, :] = -np.inf
+    x[2, 4000] = -1e30
+    x[3, :] = -np.inf                      # all -inf -> 0
+    x[4, 77] = np.inf
+    x[4, 99] = np.inf
+    x[5, :] = 0.0
+    x[5, 7] = -0.0                         # -0 == +0: index 0 stays
+    got = run_rows(hs, torch, x, None, P(temperature=0.0))
+    want = [oracle.argmax(x[r]) for r in range(6)]
+    assert got.tolist() == want
+    assert want[1] == 0 and want[3] == 0 and want[4] == 77 and want[5] == 0
+
+
+# ------------------------------------------------------------------------------ temperature
+@pytest.mark.parametrize("n,T", [(5, 1.0), (64, 0.8), (1000, 0.1), (8192, 0.8), (8193, 1.7),
+                                 (50000, 0.8), (128256, 0.8), (151936, 1.0)])
+def test_temperature_matches_oracle(hs, oracle, n, T):
+    print(f"temperature n={n} T={T}", flush=True)
+    x, u = rows_rng(n + 1, 24, n, scale=3.0)
+    x[1] = 0.25                            # uniform row: id == floor(u * n)
+    got = run_rows(hs, torch, x, u, P(temperature=T))
+    res = [oracle.temperature_u(x[r], T, float(u[r])) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"temperature n={n}")
+    assert got[1] == int(np.floor(float(u[1]) * n))
+    print(f"  rows within 1e-6 of a CDF boundary: {near}")
+    assert near <= 1
+
+
+# ------------------------------------------------------------------------------------ top-k
+@pytest.mark.parametrize("n,k,T", [(8, 2, 1.0), (300, 3, 1.0), (1000, 40, 0.7), (5000, 64, 0.6),
+                                   (8192, 128, 1.0), (8193, 5, 0.9), (50000, 40, 0.7),
+                                   (128256, 40, 0.7), (262144, 64, 0.6)])
+def test_top_k_matches_oracle(hs, oracle, n, k, T):
+    print(f"top-k n={n} k={k}", flush=True)
+    x, u = rows_rng(n + k, 16, n)
+    x[2] = np.round(x[2] * 2) / 2          # ties straddling the cutoff
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_k=k, precedence=0))
+    res = [oracle.top_k_u(x[r], k, T, float(u[r])) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-k n={n} k={k}")
+    print(f"  rows within 1e-6 of a CDF boundary: {near}")
+    assert near <= 1
+
+
+@pytest.mark.parametrize("n,k,T", [(3000, 200, 10.0), (20000, 129, 1.0), (20000, 1000, 0.9),
+                                   (20000, 8192, 1.2), (20000, 9000, 1.2), (128256, 4096, 1.0)])
+def test_top_k_large_k_general_path(hs, oracle, n, k, T):
+    """k above the candidate path (the reference caps k at 8192, sampler.c:213-215)."""
+    print(f"top-k general n={n} k={k}", flush=True)
+    x, u = rows_rng(n + k, 6, n)
+    x[2] = np.round(x[2] * 2) / 2
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_k=k, precedence=0))
+    res = [oracle.top_k_u(x[r], k, T, float(u[r])) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-k n={n} k={k}")
+    assert near <= 1
+
+
+def test_top_k_degenerate_rows(hs, oracle):
+    """Rows that overflow the per-chunk candidate lists: all-equal logits, a masked row where only
+    a few logits are finite, two-valued rows. Equal logits keep ascending index order."""
+    n, k = 30000, 40
+    x, u = rows_rng(12, 8, n)
+    x[0] = 0.5
+    x[1] = -np.inf
+    x[1, [17, 2900, 29999]] = [1.0, 2.0, 0.5]
+    x[2] = np.where(np.arange(n) % 2 == 0, 1.0, -1.0)
+    x[3] = np.round(x[3])
+    x[4, :] = 3.0
+    x[4, 100:200] = 3.5
+    u[5] = 0.0
+    u[6] = np.float32(1.0 - 2.0 ** -24)
+    for T, kk, p in [(1.0, k, 1.0), (0.7, k, 0.9), (1.0, 128, 1.0)]:
+        got = run_rows(hs, torch, x, u, P(temperature=T, top_k=kk, top_p=p))
+        res = [oracle.chain_u(x[r], float(u[r]), temperature=T, top_k=kk, top_p=p)
+               for r in range(x.shape[0])]
+        compare_ids(got, [t for t, _ in res], [i for _, i in res], "degenerate rows")
+
+
+def test_top_k_reference_unit_vector(hs, oracle):
+    # tests/test_sampler_unit.c:92-112: top-2 of 8 logits only ever yields ids {2, 4}
+    from geistlib_amd.workloads import xorshift_units
+    row = np.array([0, 1, 4, 2, 5, 1.5, 0, .5], dtype=np.float32)
+    u, _ = xorshift_units(11, 256)
+    x = np.tile(row, (256, 1))
+    got = run_rows(hs, torch, x, u, P(temperature=1.0, top_k=2, precedence=0))
+    want = [oracle.top_k_u(row, 2, 1.0, float(v))[0] for v in u]
+    assert got.tolist() == want and set(got.tolist()) == {2, 4}
+
+
+@pytest.mark.parametrize("n,k,p,m", [(1000, 40, 0.9, 0.0), (128256, 40, 0.9, 0.0),
+                                     (128256, 40, 0.9, 0.05), (50000, 64, 0.5, 0.0),
+                                     (50000, 100, 1.0, 0.1), (262144, 64, 0.9, 0.0)])
+def test_chain_top_k_top_p_min_p(hs, oracle, n, k, p, m):
+    print(f"chain n={n} k={k} p={p} m={m}", flush=True)
+    x, u = rows_rng(n * 3 + k, 16, n)
+    got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=p, min_p=m))
+    res = [oracle.chain_u(x[r], float(u[r]), temperature=0.7, top_k=k, top_p=p, min_p=m)
+           for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "chain")
+    print(f"  rows within 1e-6 of a CDF boundary: {near}")
+    assert near <= 1
+
+
+def test_reference_precedence_ignores_top_p_when_top_k_set(hs, oracle):
+    x, u = rows_rng(99, 8, 20000)
+    got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=40, top_p=0.5, precedence=0))
+    want = [oracle.top_k_u(x[r], 40, 0.7, float(u[r]))[0] for r in range(8)]
+    assert got.tolist() == want
+
+
+# ------------------------------------------------------------------------------ penalties
+def test_penalties_in_place_match_oracle(hs, oracle):
+    g = np.random.default_rng(5)
+    rows, n, H = 6, 30000, 700
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    hist = g.integers(0, n, (rows, H)).astype(np.int32)
+    hist[:, :50] = hist[:, 50:100]         # duplicates
+    hist[0, :10] = [-1, n, n + 5, -7, 0, 0, 0, n - 1, n - 1, 2**31 - 1]
+    hl = np.array([H, H, 0, 1, 333, H], dtype=np.int32)
+    d = to_dev(x, torch)
+    hs.apply_penalties(d, to_dev(hist, torch), to_dev(hl, torch), 1.1, 0.5, 0.3)
+    hs.sync()
+    got = d.cpu().numpy()
+    for r in range(rows):
+        want = oracle.penalties(x[r], hist[r, :hl[r]], 1.1, 0.5, 0.3)
+        assert np.array_equal(got[r], want), f"row {r}"
+
+
+def test_penalties_fused_into_sampling(hs, oracle):
+    g = np.random.default_rng(6)
+    rows, n, H = 16, 40000, 512
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    hist = g.integers(0, 2000, (rows, H)).astype(np.int32)   # concentrated -> many repeats
+    top = np.argsort(-x, axis=1)[:, :20].astype(np.int32)
+    hist[:, :20] = top                     # the leaders are penalised, so the outcome changes
+    hl = np.full(rows, H, dtype=np.int32)
+    u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
+    before = x.copy()
+    for params, kw in [(P(temperature=0.7, top_k=40, top_p=0.9, rep=1.3, freq=0.5, pres=0.3),
+                        dict(temperature=0.7, top_k=40, top_p=0.9)),
+                       (P(temperature=0.0, rep=1.3, freq=0.5, pres=0.3), dict(temperature=0.0)),
+                       (P(temperature=0.9, rep=1.3, freq=0.5, pres=0.3), dict(temperature=0.9))]:
+        got = run_rows(hs, torch, x, u, params, hist, hl)
+        res = []
+        for r in range(rows):
+            pen = oracle.penalties(x[r], hist[r], 1.3, 0.5, 0.3)
+            res.append(oracle.chain_u(pen, float(u[r]), **kw))
+        compare_ids(got, [t for t, _ in res], [i for _, i in res], "fused penalties")
+    assert np.array_equal(x, before)
+
+
+# ------------------------------------------------------------------------------ softmax
+@pytest.mark.parametrize("n,T", [(1000, 1.0), (128256, 0.7)])
+def test_normalised_probabilities(hs, oracle, n, T):
+    from geistlib_amd import HipSampler
+    x, _ = rows_rng(n, 4, n)
+    d = to_dev(x, torch)
+    probs = torch.empty_like(d)
+    hs.softmax(HipSampler.rows(d), P(temperature=T), probs)
+    hs.sync()
+    got = probs.cpu().numpy()
+    for r in range(4):
+        want, _ = oracle.softmax_normalised(x[r], T)
+        # north-star bound: 1e-5 relative in fp32 (observed: identical up to 1 ulp)
+        assert np.allclose(got[r], want, rtol=1e-5, atol=0)
+        assert np.max(np.abs(got[r] - want) / np.maximum(want, 1e-38)) < 2e-7
+
+
+# ---------------------------------------------------------------------------------- rng
+def test_device_rng_matches_reference_stream(hs, oracle):
+    from geistlib_amd import HipSampler
+    from geistlib_amd.workloads import xorshift_units
+    rows, n = 12, 20000
+    x, _ = rows_rng(17, rows, n)
+    d = to_dev(x, torch)
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    # shared state: row r takes draw r + 1 (finalize_logits_batch order)
+    st = torch.tensor([0xC0FFEE], dtype=torch.int64, device="cuda")
+    hs.sample_rng(HipSampler.rows(d), P(temperature=0.8, top_k=40, precedence=0), st, True, out)
+    hs.sync()
+    u, state_after = xorshift_units(0xC0FFEE, rows)
+    want = [oracle.top_k_u(x[r], 40, 0.8, float(u[r]))[0] for r in range(rows)]
+    assert out.cpu().tolist() == want
+    assert int(st.cpu().numpy().view(np.uint64)[0]) == state_after
+    # greedy leaves the state alone
+    hs.sample_rng(HipSampler.rows(d), P(temperature=0.0), st, True, out)
+    hs.sync()
+    assert int(st.cpu().numpy().view(np.uint64)[0]) == state_after
+    # per-row states
+    seeds = np.arange(1, rows + 1, dtype=np.uint64) * np.uint64(7919)
+    st = torch.from_numpy(seeds.view(np.int64)).cuda()
+    hs.sample_rng(HipSampler.rows(d), P(temperature=0.8), st, False, out)
+    hs.sync()
+    want = []
+    for r in range(rows):
+        ur, _ = xorshift_units(int(seeds[r]), 1)
+        want.append(oracle.temperature_u(x[r], 0.8, float(ur[0]))[0])
+    assert out.cpu().tolist() == want
+
+
+# ------------------------------------------------------------------- strided / unaligned
+def test_row_stride_and_unaligned_rows(hs, oracle):
+    g = np.random.default_rng(3)
+    rows, n, ld = 5, 10001, 10007          # odd stride: rows are not 16-byte aligned
+    buf = (g.standard_normal((rows, ld)) * 2).astype(np.float32)
+    d = to_dev(buf, torch)
+    view = d[:, :n]
+    u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
+    from geistlib_amd import HipSampler
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    r = HipSampler.rows(view)
+    assert r.ld == ld and r.n_vocab == n
+    hs.sample(r, P(temperature=0.7, top_k=10, precedence=0), to_dev(u, torch), out)
+    hs.sync()
+    want = [oracle.top_k_u(np.ascontiguousarray(buf[i, :n]), 10, 0.7, float(u[i]))[0]
+            for i in range(rows)]
+    assert out.cpu().tolist() == want
+
+
+def test_argument_errors(hs):
+    from geistlib_amd import HipSampler
+    from geistlib_amd.binding import GeistHipError
+    d = torch.zeros((2, 100), dtype=torch.float32, device="cuda")
+    out = torch.empty(2, dtype=torch.int32, device="cuda")
+    with pytest.raises(GeistHipError):     # stochastic without uniforms
+        hs.sample(HipSampler.rows(d), P(temperature=0.7), None, out)
+    with pytest.raises(GeistHipError):     # min_p under the reference precedence
+        hs.sample(HipSampler.rows(d), P(temperature=0.7, min_p=0.1, precedence=0), out, out)
+    big = HipSampler.rows(d)
+    big.rows = 100000
+    with pytest.raises(GeistHipError):     # beyond the workspace
+        hs.sample(big, P(temperature=0.0), None, out)
