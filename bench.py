@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X token-sampling path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the sampling path over one batch of synthetic logit rows that already
+sit in HBM: penalties + temperature + top-k + top-p + draw for the default workload
+(B = 64 x V = 128256 fp32, T = 0.7, top-k 40, top-p 0.9, one seeded uniform per row, history of
+2048 Zipf ids per row with repetition 1.1 / frequency 0.5 / presence 0.3). Prints ONE JSON line.
+
+value      rows sampled per second over the timed K steps (whole job, one GPU)
+roofline   the logit-streaming kernel: algorithmic bytes per launch / its mean duration, the
+           duration taken with HIP events on the sampler's stream around every launch of that
+           kernel during a second pass of K steps
+cpu_baseline  the CPU restatement of the same step (oracle, reference build flags) timed on
+           this host's cores on a bounded sample; reported, not the optimisation target
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def build_workload(name):
+    from geistlib_amd import workloads as W
+    if name == "cfg2_pen":
+        return W.config2(with_penalties=True)
+    if name == "cfg2":
+        return W.config2(with_penalties=False)
+    if name == "cfg3":
+        return W.config3()
+    if name == "cfg4":
+        return W.config4()
+    if name == "cfg1":
+        return W.config1()
+    raise SystemExit(f"unknown workload {name}")
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """Times the oracle (built with the reference's release flags) on this host."""
+    from oracle_lib import Oracle
+    try:
+        o = Oracle(fast=True)
+    except Exception as e:  # the oracle objects are test infrastructure; absence is not fatal
+        return {"value": None, "unit": "rows/s", "cores": 0, "kind": "port",
+                "sample": f"oracle unavailable: {e}"}, None
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 10 ** 6,
+                o.lib.oracle_max_threads())
+    kw = dict(temperature=w.temperature, top_k=w.top_k, top_p=w.top_p, min_p=w.min_p,
+              hist=w.history, hist_len=w.history_len, rep=w.rep, freq=w.freq, pres=w.pres)
+    out = {}
+    for label, threads in (("1", 1), ("all", cores)):
+        o.batch_chain_u(w.logits[:min(4, w.rows)], w.uniforms, threads=threads, **{
+            **kw, "hist": None if w.history is None else w.history[:4],
+            "hist_len": None if w.history_len is None else w.history_len[:4]})  # warm-up
+        reps, t_used = 0, 0.0
+        while reps < 10 and t_used < budget_s / 2:
+            t0 = time.perf_counter()
+            ids = o.batch_chain_u(w.logits, w.uniforms, threads=threads, **kw)
+            t_used += time.perf_counter() - t0
+            reps += 1
+        out[label] = (w.rows * reps / t_used, reps, ids)
+    v_all, reps_all, ids = out["all"]
+    v_1, reps_1, _ = out["1"]
+    return {"value": round(v_all, 2), "unit": "rows/s", "cores": cores, "kind": "port",
+            "single_core_rows_per_s": round(v_1, 2),
+            "sample": f"whole batch of {w.rows} rows x {reps_all} repeats on {cores} threads "
+                      f"(one row per thread) and x {reps_1} repeats on 1 thread; oracle built with "
+                      "-O3 -ffast-math -march=x86-64-v3 -fopenmp"}, ids
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="cfg2_pen")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: rows are independent and this build has no "
+                         "multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from geistlib_amd import HipSampler, SampleParams
+    if not torch.cuda.is_available():
+        raise SystemExit("no GPU visible: the sampling path has no CPU fallback")
+
+    w = build_workload(args.workload)
+    dev = torch.device("cuda:0")
+    d_logits = torch.from_numpy(w.logits).to(dev)
+    d_u = torch.from_numpy(w.uniforms).to(dev)
+    d_h = torch.from_numpy(w.history).to(dev) if w.history is not None else None
+    d_hl = torch.from_numpy(w.history_len).to(dev) if w.history is not None else None
+    d_out = torch.empty(w.rows, dtype=torch.int32, device=dev)
+    hs = HipSampler(max_rows=w.rows, max_vocab=w.n_vocab)
+    rows = HipSampler.rows(d_logits, d_h, d_hl)
+    prm = SampleParams.make(temperature=w.temperature, top_k=w.top_k, top_p=w.top_p,
+                            min_p=w.min_p, rep=w.rep, freq=w.freq, pres=w.pres)
+
+    def step():
+        hs.sample(rows, prm, d_u, d_out)
+
+    for _ in range(args.warmup):
+        step()
+    hs.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    hs.sync()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    ids_gpu = d_out.cpu().numpy()
+
+    # second pass: events around every launch of the logit-streaming kernel
+    hs.timing_enable(True)
+    hs.timing_read(reset=True)
+    for _ in range(args.steps):
+        step()
+    k_ms, k_n = hs.timing_read(reset=True)
+    hs.timing_enable(False)
+    kernel_us = k_ms * 1e3 / max(k_n, 1)
+
+    # one-step latency: enqueue + wait, median
+    lat = []
+    for _ in range(200):
+        t1 = time.perf_counter()
+        step()
+        hs.sync()
+        lat.append((time.perf_counter() - t1) * 1e6)
+    lat.sort()
+
+    alg_bytes = w.algorithmic_bytes()
+    achieved = alg_bytes / (kernel_us * 1e-6) / 1e9
+    result = {
+        "metric": "sampled rows/s",
+        "value": round(w.rows * args.steps / elapsed, 1),
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": w.name, "rows": w.rows, "n_vocab": w.n_vocab,
+                   "temperature": w.temperature, "top_k": w.top_k, "top_p": w.top_p,
+                   "min_p": w.min_p, "penalties": [w.rep, w.freq, w.pres],
+                   "history_per_row": 0 if w.history is None else int(w.history.shape[1])},
+        "us_per_step": round(ms_per_step * 1e3, 3),
+        "step_latency_us_median": round(lat[len(lat) // 2], 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_topk_scan" if w.top_k > 1 else "k_chunk_expsum",
+                     "kernel_us": round(kernel_us, 3), "algorithmic_bytes": alg_bytes,
+                     "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_cpu:
+        base, ids_cpu = cpu_baseline(w)
+        result["cpu_baseline"] = base
+        if ids_cpu is not None:
+            result["parity"] = {"rows": int(w.rows),
+                                "ids_differ": int(np.sum(ids_cpu != ids_gpu))}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -27,8 +27,7 @@ struct geist_hip_sampler {
     /* device workspace */
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
-    uint32_t *cand_key   = nullptr; /* [max_rows][max_chunks][TOPK_CAND_CAP] */
-    int32_t  *cand_idx   = nullptr;
+    uint64_t *cand_pack  = nullptr; /* [max_rows][max_chunks][TOPK_CAND_CAP] */
     int32_t  *cand_cnt   = nullptr; /* [max_rows][max_chunks] */
     int32_t  *row_flag   = nullptr; /* [max_rows] */
     float    *uniforms   = nullptr; /* [max_rows] */
@@ -184,8 +183,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     hipError_t   e  = hipSetDevice(device);
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
-    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_key, rc * TOPK_CAND_CAP * sizeof(uint32_t));
-    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_idx, rc * TOPK_CAND_CAP * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_pack, rc * TOPK_CAND_CAP * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->cand_cnt, rc * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
@@ -208,8 +206,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipStreamSynchronize(s->stream);
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
-    (void) hipFree(s->cand_key);
-    (void) hipFree(s->cand_idx);
+    (void) hipFree(s->cand_pack);
     (void) hipFree(s->cand_cnt);
     (void) hipFree(s->row_flag);
     (void) hipFree(s->uniforms);
@@ -308,8 +305,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     f.uniforms   = d_uniforms;
     f.chunk_best = s->chunk_best;
     f.chunk_sum  = s->chunk_sum;
-    f.cand_key   = s->cand_key;
-    f.cand_idx   = s->cand_idx;
+    f.cand_pack  = s->cand_pack;
     f.cand_cnt   = s->cand_cnt;
     f.out        = d_out;
     f.cap        = TOPK_CAND_CAP;
@@ -335,7 +331,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
             return after_launch(s, "top-k (general)");
         }
         mark_start(s);
-        launch_topk_scan(L, rs.k, TOPK_CAND_CAP, s->cand_key, s->cand_idx, s->cand_cnt);
+        launch_topk_scan(L, rs.k, TOPK_CAND_CAP, s->cand_pack, s->cand_cnt);
         mark_stop(s);
         f.mode = FINAL_TOPK;
         f.k    = rs.k;

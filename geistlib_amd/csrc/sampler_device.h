@@ -175,19 +175,24 @@ __device__ __forceinline__ float penalise(float l, uint32_t count, float rep, fl
     return l;
 }
 
-/* Counts the occurrences of each vocabulary id of [base, end) in the row's history (end - base
- * <= CHUNK; ids outside the row's vocabulary fall outside every chunk and are ignored).
- * cnt16 packs two 16-bit counters per word (histories are capped at 65535 entries). */
+/* The history lookup of one chunk, in two steps so that the logit loads can be in flight while
+ * the history is read: history_clear() zeroes the table (ends with a barrier), history_count()
+ * adds the occurrences of each vocabulary id of [base, end) in the row's history (ends with a
+ * barrier). cnt16 packs two 16-bit counters per word: histories are capped at 65535 entries.
+ * Ids outside the row's vocabulary fall outside every chunk and are ignored. */
 template <int CHUNK>
-__device__ __forceinline__ void history_counts(const RowView &rv, int row, int base, int end,
-                                               uint32_t *cnt16) {
-    for (int i = threadIdx.x; i < CHUNK / 2; i += TPB)
-        cnt16[i] = 0u;
+__device__ __forceinline__ void history_clear(uint32_t *cnt16) {
+    uint4 *p = reinterpret_cast<uint4 *>(cnt16);
+    for (int i = threadIdx.x; i < CHUNK / 8; i += TPB)
+        p[i] = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();
+}
+__device__ __forceinline__ void history_count(const RowView &rv, int row, int base, int end,
+                                              uint32_t *cnt16) {
     int len = rv.hist_len ? rv.hist_len[row] : 0;
     if (len > rv.hist_ld)
         len = (int) rv.hist_ld;
-    const int32_t *h   = rv.hist + (long) row * rv.hist_ld;
+    const int32_t *h = rv.hist + (long) row * rv.hist_ld;
     for (int i = threadIdx.x; i < len; i += TPB) {
         const int t   = h[i];
         const int off = t - base;
@@ -197,12 +202,11 @@ __device__ __forceinline__ void history_counts(const RowView &rv, int row, int b
     __syncthreads();
 }
 
-/* Loads the chunk [base, end) of a row into registers (layout in the file header), applying
- * penalties (when cnt16 != NULL) and the soft-cap. Positions at or beyond `end` hold -inf. */
+/* Issues the loads of the chunk [base, end) of a row into registers (layout in the file
+ * header). Positions at or beyond `end` hold -inf. */
 template <int NV>
-__device__ __forceinline__ void load_chunk(const RowView &rv, const float *__restrict__ row,
-                                           int base, int end, const uint32_t *cnt16,
-                                           float4 (&v)[NV]) {
+__device__ __forceinline__ void load_raw(const RowView &rv, const float *__restrict__ row,
+                                         int base, int end, float4 (&v)[NV]) {
     const int   tid  = threadIdx.x;
     const float ninf = -__builtin_inff();
 #pragma unroll
@@ -217,21 +221,27 @@ __device__ __forceinline__ void load_chunk(const RowView &rv, const float *__res
             v[j].w = e + 3 < end ? row[e + 3] : ninf;
         }
     }
+}
+
+/* Penalties (when cnt16 != NULL) and the soft-cap on a chunk held in registers. */
+template <int NV>
+__device__ __forceinline__ void apply_transform(const RowView &rv, const uint32_t *cnt16,
+                                                float4 (&v)[NV]) {
+    const int tid = threadIdx.x;
     if (cnt16) {
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            const int      off = 4 * (j * TPB + tid); /* even, so two words cover the float4 */
-            const uint32_t w0  = cnt16[(off >> 1) + 0];
-            const uint32_t w1  = cnt16[(off >> 1) + 1];
-            if (w0 | w1) {
-                if (w0 & 0xffffu)
-                    v[j].x = penalise(v[j].x, w0 & 0xffffu, rv.rep, rv.freq, rv.pres);
-                if (w0 >> 16)
-                    v[j].y = penalise(v[j].y, w0 >> 16, rv.rep, rv.freq, rv.pres);
-                if (w1 & 0xffffu)
-                    v[j].z = penalise(v[j].z, w1 & 0xffffu, rv.rep, rv.freq, rv.pres);
-                if (w1 >> 16)
-                    v[j].w = penalise(v[j].w, w1 >> 16, rv.rep, rv.freq, rv.pres);
+            const int   off = 4 * (j * TPB + tid); /* even, so two words cover the float4 */
+            const uint2 w   = *reinterpret_cast<const uint2 *>(cnt16 + (off >> 1));
+            if (w.x | w.y) {
+                if (w.x & 0xffffu)
+                    v[j].x = penalise(v[j].x, w.x & 0xffffu, rv.rep, rv.freq, rv.pres);
+                if (w.x >> 16)
+                    v[j].y = penalise(v[j].y, w.x >> 16, rv.rep, rv.freq, rv.pres);
+                if (w.y & 0xffffu)
+                    v[j].z = penalise(v[j].z, w.y & 0xffffu, rv.rep, rv.freq, rv.pres);
+                if (w.y >> 16)
+                    v[j].w = penalise(v[j].w, w.y >> 16, rv.rep, rv.freq, rv.pres);
             }
         }
     }
@@ -246,6 +256,16 @@ __device__ __forceinline__ void load_chunk(const RowView &rv, const float *__res
         }
     }
 }
+
+/* max of three floats in one instruction. Unlike fmaxf() no canonicalising self-max is emitted
+ * per operand; a quiet NaN operand is ignored (a signalling NaN may come back quieted, which
+ * only makes the caller keep more candidates). */
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float f4_max(const float4 &q) { return max3f(max3f(q.x, q.y, q.z), q.w, q.w); }
 
 __device__ __forceinline__ float f4_get(const float4 &q, int c) {
     return c == 0 ? q.x : c == 1 ? q.y : c == 2 ? q.z : q.w;

@@ -47,8 +47,7 @@ struct FinalLaunch {
     const float    *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
-    const uint32_t *cand_key;
-    const int32_t  *cand_idx;
+    const uint64_t *cand_pack;
     const int32_t  *cand_cnt;
     int32_t        *out;
 };
@@ -56,8 +55,7 @@ struct FinalLaunch {
 void launch_chunk_best(const Launch &L, uint64_t *chunk_best);
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, float *probe_p);
-void launch_topk_scan(const Launch &L, int k, int cap, uint32_t *cand_key, int32_t *cand_idx,
-                      int32_t *cand_cnt);
+void launch_topk_scan(const Launch &L, int k, int cap, uint64_t *cand_pack, int32_t *cand_cnt);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);

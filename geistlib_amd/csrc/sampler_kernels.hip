@@ -24,6 +24,18 @@ namespace gs {
 
 __device__ const uint64_t g_expf_tab[32] = GEIST_EXPF_TABLE_INIT;
 
+/* Phase timestamps for kernel tuning; compiled in only by the tuning probe. */
+#ifdef GS_PHASES
+__device__ long long g_phase[16384 * 8];
+#define GS_MARK(i)                                                                             \
+    do {                                                                                       \
+        if (threadIdx.x == 0)                                                                  \
+            g_phase[((long) blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = wall_clock64();   \
+    } while (0)
+#else
+#define GS_MARK(i) ((void) 0)
+#endif
+
 /* number of leading key bits the per-chunk threshold search resolves */
 constexpr int THR_BITS = 16;
 
@@ -35,17 +47,21 @@ __device__ __forceinline__ void chunk_bounds(const RowView &rv, int chunk, int &
         end = rv.n_vocab;
 }
 
-/* Loads and transforms the chunk of (row, chunk); PEN selects the history lookup. `cnt16` is
- * an LDS table of NV*512 words when PEN, else unused. */
+/* Loads and transforms the chunk [base, end) of a row; PEN selects the history lookup. `cnt16`
+ * is an LDS table of NV*512 words when PEN, else unused. The logit loads are issued before the
+ * history is read so that both are in flight together. */
 template <int NV, bool PEN>
 __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int base, int end,
                                             uint32_t *cnt16, float4 (&v)[NV]) {
     const float *rowp = rv.logits + (long) row * rv.ld;
     if (PEN) {
-        history_counts<NV * TPB * 4>(rv, row, base, end, cnt16);
-        load_chunk<NV>(rv, rowp, base, end, cnt16, v);
+        history_clear<NV * TPB * 4>(cnt16);
+        load_raw<NV>(rv, rowp, base, end, v);
+        history_count(rv, row, base, end, cnt16);
+        apply_transform<NV>(rv, cnt16, v);
     } else {
-        load_chunk<NV>(rv, rowp, base, end, nullptr, v);
+        load_raw<NV>(rv, rowp, base, end, v);
+        apply_transform<NV>(rv, nullptr, v);
     }
 }
 
@@ -54,7 +70,7 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int base
  * ========================================================================================== */
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_chunk_best(RowView rv, uint64_t *__restrict__ chunk_best) {
-    __shared__ uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     int                 base, end;
@@ -100,7 +116,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       double *__restrict__ chunk_sum,
                                                       const int32_t *__restrict__ probe_token,
                                                       float *__restrict__ probe_p) {
-    __shared__ uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
     __shared__ uint64_t s_tab[32];
@@ -136,82 +152,102 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
 /* ============================================================================================
  * k_topk_scan: every element of the chunk that can belong to the row's top k.
  *
- * The k-th largest of the 256 per-thread maxima is a lower bound of the chunk's k-th largest
- * element, so every element at or above it is kept; the bound is found on the leading
- * THR_BITS of the key by a bitwise search with wavefront ballots. A chunk that yields more
- * than `cap` candidates reports its true count and the row takes the general path.
+ * The workgroup's 256 per-thread maxima are folded into G = 64, 128 or 256 group maxima; the
+ * k-th largest of them is a lower bound of the chunk's k-th largest element, so every element
+ * at or above it is kept (about -G ln(1 - k/G) of them). The bound is found on the leading
+ * THR_BITS of the order-preserving key by a bitwise search with wavefront ballots. Comparisons
+ * on the elements themselves stay in fp32: max ignores NaN and `!(x < bound)` keeps it, which
+ * is what the key order prescribes. A chunk that yields more than `cap` candidates reports its
+ * true count and the row takes the general path.
  * ========================================================================================== */
+template <int VPL>
+__device__ __forceinline__ uint32_t kth_group_max(uint32_t q0, uint32_t q1, uint32_t q2,
+                                                  uint32_t q3, int kk) {
+    uint32_t tau = 0;
+#pragma unroll
+    for (int bit = 31; bit >= 32 - THR_BITS; --bit) {
+        const uint32_t t   = tau | (1u << bit);
+        int            cnt = __popcll(__ballot(q0 >= t));
+        if (VPL >= 2)
+            cnt += __popcll(__ballot(q1 >= t));
+        if (VPL >= 4)
+            cnt += __popcll(__ballot(q2 >= t)) + __popcll(__ballot(q3 >= t));
+        if (cnt >= kk)
+            tau = t;
+    }
+    return tau;
+}
+
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_topk_scan(RowView rv, int k, int cap,
-                                                   uint32_t *__restrict__ cand_key,
-                                                   int32_t *__restrict__ cand_idx,
+                                                   uint64_t *__restrict__ cand_pack,
                                                    int32_t *__restrict__ cand_cnt) {
-    __shared__ uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ uint32_t s_tmax[TPB];
-    __shared__ uint32_t s_ckey[TOPK_CAND_CAP];
-    __shared__ int32_t  s_cidx[TOPK_CAND_CAP];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ float    s_tmax[TPB];
+    __shared__ uint64_t s_cand[TOPK_CAND_CAP];
     __shared__ int      s_n;
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     const int           lane = tid & (WAVE - 1);
     int                 base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
+    GS_MARK(0);
     float4 v[NV];
     fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
 
-    uint32_t key[NV][4];
-    uint32_t tm = 0;
+    float tm = -__builtin_inff();
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            key[j][c] = f2key(f4_get(v[j], c));
-            tm        = key[j][c] > tm ? key[j][c] : tm;
-        }
-    }
+    for (int j = 0; j < NV; ++j)
+        tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
     s_tmax[tid] = tm;
     if (tid == 0)
         s_n = 0;
+    GS_MARK(1);
     __syncthreads();
+    GS_MARK(2);
 
-    const uint32_t q0 = s_tmax[lane], q1 = s_tmax[lane + 64], q2 = s_tmax[lane + 128],
-                   q3 = s_tmax[lane + 192];
-    const int kk  = k < TPB ? k : TPB;
-    uint32_t  tau = 0;
-#pragma unroll
-    for (int bit = 31; bit >= 32 - THR_BITS; --bit) {
-        const uint32_t t   = tau | (1u << bit);
-        const int      cnt = __popcll(__ballot(q0 >= t)) + __popcll(__ballot(q1 >= t)) +
-                        __popcll(__ballot(q2 >= t)) + __popcll(__ballot(q3 >= t));
-        if (cnt >= kk)
-            tau = t;
+    const float g0 = s_tmax[lane], g1 = s_tmax[lane + 64], g2 = s_tmax[lane + 128],
+                g3 = s_tmax[lane + 192];
+    uint32_t tau;
+    if (k <= 24) {
+        tau = kth_group_max<1>(f2key(max3f(max3f(g0, g1, g2), g3, g3)), 0, 0, 0, k);
+    } else if (k <= 64) {
+        tau = kth_group_max<2>(f2key(max3f(g0, g2, g2)), f2key(max3f(g1, g3, g3)), 0, 0, k);
+    } else {
+        tau = kth_group_max<4>(f2key(g0), f2key(g1), f2key(g2), f2key(g3), k < TPB ? k : TPB);
     }
+    const float bound = key2f(tau); /* tau == 0 maps to NaN: nothing is below it */
+    GS_MARK(3);
 
-    if (tm >= tau) {
+    /* Padding holds -inf, so with a finite bound no index test is needed on the hot path. */
+    const bool check_idx = !(bound > -__builtin_inff());
+    if (!(tm < bound)) {
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            const int e = base + 4 * (j * TPB + tid);
+            const float m4 = f4_max(v[j]);
+            if (!(m4 < bound) || check_idx) {
+                const int e = base + 4 * (j * TPB + tid);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (key[j][c] >= tau && e + c < end) {
-                    const int pos = atomicAdd(&s_n, 1);
-                    if (pos < cap) {
-                        s_ckey[pos] = key[j][c];
-                        s_cidx[pos] = e + c;
+                for (int c = 0; c < 4; ++c) {
+                    const float x = f4_get(v[j], c);
+                    if (!(x < bound) && (!check_idx || e + c < end)) {
+                        const int pos = atomicAdd(&s_n, 1);
+                        if (pos < cap)
+                            s_cand[pos] = pack_best(f2key(x), (uint32_t) (e + c));
                     }
                 }
             }
         }
     }
+    GS_MARK(4);
     __syncthreads();
     const int  n = s_n;
     const long o = (long) row * rv.n_chunks + chunk;
     if (tid == 0)
         cand_cnt[o] = n;
     const int m = n < cap ? n : cap;
-    for (int i = tid; i < m; i += TPB) {
-        cand_key[o * cap + i] = s_ckey[i];
-        cand_idx[o * cap + i] = s_cidx[i];
-    }
+    for (int i = tid; i < m; i += TPB)
+        cand_pack[o * cap + i] = s_cand[i];
+    GS_MARK(5);
 }
 
 /* ============================================================================================
@@ -326,6 +362,66 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
     return (int) best_idx(spack[at]);
 }
 
+/* finish_sorted for n <= 128 survivors on ONE wavefront (call with all 64 lanes of a single
+ * wave): lane l owns entries 2l and 2l+1, the prefix sums are wavefront scans, no barrier.
+ * `tab` is the expf table in LDS. */
+__device__ int finish_sorted_wave(int n, const uint64_t *spack, float inv_t, float top_p,
+                                  float min_p, float u, const uint64_t *tab) {
+    const int  lane  = threadIdx.x & (WAVE - 1);
+    const bool use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool use_m = min_p > 0.0f;
+    const bool norm  = use_p || use_m;
+    const int  i0 = 2 * lane, i1 = 2 * lane + 1;
+    const float l0 = key2f(best_key(spack[0]));
+    float w0 = i0 < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i0])), l0, inv_t), tab)
+                      : 0.0f;
+    float w1 = i1 < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i1])), l0, inv_t), tab)
+                      : 0.0f;
+    double part = (double) w0 + (double) w1;
+    double incl = wave_scan_f64(part);
+    if (norm) {
+        const double sum = __shfl(incl, WAVE - 1, WAVE);
+        w0   = i0 < n ? (float) ((double) w0 / sum) : 0.0f;
+        w1   = i1 < n ? (float) ((double) w1 / sum) : 0.0f;
+        part = (double) w0 + (double) w1;
+        incl = wave_scan_f64(part);
+    }
+    const double c0 = (incl - part) + (double) w0; /* inclusive prefix at entry i0 */
+    const double c1 = c0 + (double) w1;            /* ... at entry i1 */
+    int keep = n;
+    if (use_p) {
+        const uint64_t m0 = __ballot(i0 < n && c0 >= (double) top_p);
+        const uint64_t m1 = __ballot(i1 < n && c1 >= (double) top_p);
+        int first = n - 1;
+        if (m0) first = 2 * (__ffsll((long long) m0) - 1);
+        if (m1) {
+            const int f1 = 2 * (__ffsll((long long) m1) - 1) + 1;
+            first = (m0 && first < f1) ? first : f1;
+        }
+        keep = (m0 | m1) ? first + 1 : n;
+    }
+    if (use_m) {
+        const float floor_w = __fmul_rn(min_p, __shfl(w0, 0, WAVE));
+        int m = __popcll(__ballot(i0 < n && w0 >= floor_w)) +
+                __popcll(__ballot(i1 < n && w1 >= floor_w));
+        if (m < 1) m = 1;
+        keep = m < keep ? m : keep;
+    }
+    if (keep < 1) keep = 1;
+    const double   at_keep = ((keep - 1) & 1) ? c1 : c0;
+    const double   mass    = __shfl(at_keep, (keep - 1) >> 1, WAVE);
+    const double   target  = (double) u * mass;
+    const uint64_t h0 = __ballot(i0 < keep && target < c0);
+    const uint64_t h1 = __ballot(i1 < keep && target < c1);
+    int at = keep - 1;
+    if (h0 | h1) {
+        const int f0 = h0 ? 2 * (__ffsll((long long) h0) - 1) : 0x7fffffff;
+        const int f1 = h1 ? 2 * (__ffsll((long long) h1) - 1) + 1 : 0x7fffffff;
+        at = f0 < f1 ? f0 : f1;
+    }
+    return (int) best_idx(spack[at]);
+}
+
 /* Workgroup-wide choice of one radix digit: hist[256] holds the counts of the current digit
  * among the keys that match the prefix; returns the digit that contains the `remaining`-th
  * largest key and updates `remaining` to the rank inside that digit. */
@@ -345,9 +441,9 @@ __device__ __forceinline__ int radix_pick_digit(const int *hist, int &remaining,
     return digit;
 }
 
-/* LDS radix select: the k-th largest of n keys held in LDS (1 <= k <= n). Returns the key and
- * how many of the entries equal to it are needed. */
-__device__ uint32_t lds_kth_largest(const uint32_t *keys, int n, int k, int *hist, int *s_scan,
+/* LDS radix select: the k-th largest key of n packed entries held in LDS (1 <= k <= n). Returns
+ * the key and how many of the entries equal to it are needed. */
+__device__ uint32_t lds_kth_largest(const uint64_t *packs, int n, int k, int *hist, int *s_scan,
                                     int *s_sel, int &need_ties) {
     const int tid    = threadIdx.x;
     uint32_t  prefix = 0, mask = 0;
@@ -356,7 +452,7 @@ __device__ uint32_t lds_kth_largest(const uint32_t *keys, int n, int k, int *his
         hist[tid] = 0;
         __syncthreads();
         for (int i = tid; i < n; i += TPB) {
-            const uint32_t key = keys[i];
+            const uint32_t key = best_key(packs[i]);
             if ((key & mask) == prefix)
                 atomicAdd(&hist[(key >> shift) & 255u], 1);
         }
@@ -518,8 +614,7 @@ struct FinalArgs {
     const float   *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
-    const uint32_t *cand_key;
-    const int32_t  *cand_idx;
+    const uint64_t *cand_pack;
     const int32_t  *cand_cnt;
     int32_t        *out;
 };
@@ -529,10 +624,12 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     __shared__ uint64_t      s_red[NWAVES];
     __shared__ FinishShared  s_fs;
     __shared__ GeneralShared s_gs;
-    __shared__ uint32_t      s_key[FINAL_CAND_MAX];
-    __shared__ int32_t       s_idx[FINAL_CAND_MAX];
+    __shared__ uint64_t      s_cpack[FINAL_CAND_MAX];
+    __shared__ uint64_t      s_m[TPB];
     __shared__ uint64_t      s_pack[TOPK_FAST_MAX];
-    __shared__ uint32_t      s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ double        s_csum[MAX_CHUNKS];
+    __shared__ uint32_t      s_kmin, s_kmax;
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ int           s_off[MAX_CHUNKS + 1];
     __shared__ int           s_n, s_nt, s_chunk;
     __shared__ double        s_before;
@@ -555,15 +652,21 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     if (a.mode == FINAL_TEMPERATURE) {
         /* sampler.c:90-102 over all n in index order: locate the chunk from the per-chunk sums,
          * then scan that chunk. */
+        if (tid < C)
+            s_csum[tid] = a.chunk_sum[(long) row * C + tid];
+        if (tid < 32)
+            s_fs.tab[tid] = g_expf_tab[tid];
+        const float u_row = a.uniforms[row];
+        __syncthreads();
         if (tid == 0) {
             double tot = 0.0;
             for (int c = 0; c < C; ++c)
-                tot += a.chunk_sum[(long) row * C + c];
-            const double target = (double) a.uniforms[row] * tot;
+                tot += s_csum[c];
+            const double target = (double) u_row * tot;
             double       run    = 0.0;
             int          at     = C - 1;
             for (int c = 0; c < C; ++c) {
-                const double nxt = run + a.chunk_sum[(long) row * C + c];
+                const double nxt = run + s_csum[c];
                 if (target < nxt || c == C - 1) {
                     at = c;
                     break;
@@ -574,8 +677,6 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
             s_before  = run;
             s_fs.mass = target;
         }
-        if (tid < 32)
-            s_fs.tab[tid] = g_expf_tab[tid];
         const float mx = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
         /* (row_best_from_chunks ends with a barrier: s_chunk, s_before, tab are visible) */
         const int chunk = s_chunk;
@@ -621,89 +722,143 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     }
 
     /* ---- FINAL_TOPK: merge the per-chunk candidates ---------------------------------------- */
-    if (tid == 0) {
-        int  run  = 0;
-        bool over = false;
-        for (int c = 0; c < C; ++c) {
-            const int n_c = a.cand_cnt[(long) row * C + c];
-            s_off[c]      = run;
-            if (n_c > a.cap)
-                over = true;
-            run += n_c < a.cap ? n_c : a.cap;
-        }
-        s_off[C] = run;
-        if (run > FINAL_CAND_MAX)
-            over = true;
-        s_n  = over ? -1 : run;
-        s_nt = 0;
+    if (tid < 32)
+        s_fs.tab[tid] = g_expf_tab[tid];
+    const float u_row = a.uniforms[row];
+    int         n_c   = 0;
+    bool        over  = false;
+    if (tid < C) {
+        const int raw = a.cand_cnt[(long) row * C + tid];
+        over          = raw > a.cap;
+        n_c           = over ? a.cap : raw;
     }
-    __syncthreads();
-    const int N = s_n;
-    int       k;
-    if (N < 0) {
+    int       N;
+    const int incl = block_scan_i32(n_c, s_gs.scan, &N);
+    if (tid < C)
+        s_off[tid] = incl - n_c;
+    if (tid == 0) {
+        s_off[C] = N;
+        s_n      = 0;
+        s_nt     = 0;
+        s_kmin   = 0xffffffffu;
+        s_kmax   = 0u;
+    }
+    const bool general = __syncthreads_or(over) || N > FINAL_CAND_MAX;
+    int        k;
+    if (general) {
         /* some chunk had more candidates than it may hand on (long runs of equal values,
          * masked rows): select over the whole row instead */
         k = topk_row_general<NV, PEN>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
     } else {
-        const int w = tid / WAVE, lane = tid & (WAVE - 1);
-        for (int c = w; c < C; c += NWAVES) {
-            const int  o0  = s_off[c];
-            const int  n_c = s_off[c + 1] - o0;
-            const long src = ((long) row * C + c) * a.cap;
-            for (int i = lane; i < n_c; i += WAVE) {
-                s_key[o0 + i] = a.cand_key[src + i];
-                s_idx[o0 + i] = a.cand_idx[src + i];
+        /* gather every candidate of the row into LDS; one global round trip */
+        uint32_t kmin = 0xffffffffu, kmax = 0u;
+        for (int i = tid; i < N; i += TPB) {
+            int lo = 0, hi = C; /* s_off[lo] <= i < s_off[hi] */
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (s_off[mid] <= i)
+                    lo = mid;
+                else
+                    hi = mid;
             }
+            const uint64_t p = a.cand_pack[((long) row * C + lo) * a.cap + (i - s_off[lo])];
+            s_cpack[i]       = p;
+            const uint32_t key = best_key(p);
+            kmin = key < kmin ? key : kmin;
+            kmax = key > kmax ? key : kmax;
         }
+        kmax = wave_max_u32(kmax);
+        kmin = ~wave_max_u32(~kmin);
+        if ((tid & (WAVE - 1)) == 0) {
+            atomicMax(&s_kmax, kmax);
+            atomicMin(&s_kmin, kmin);
+        }
+        s_gs.hist[tid] = 0;
         __syncthreads();
         k = a.k < N ? a.k : N;
-        int            need_ties;
-        const uint32_t kth =
-            lds_kth_largest(s_key, N, k, s_gs.hist, s_gs.scan, s_gs.sel, need_ties);
-
-        /* survivors: everything above the k-th key, plus the `need_ties` lowest-index ties */
-        if (tid == 0)
-            s_n = 0;
+        /* one 8-bit radix step on the highest bits in which the candidates differ */
+        const uint32_t diff = s_kmin ^ s_kmax;
+        int            sh   = diff ? (31 - __clz((int) diff)) - 7 : 0;
+        if (sh < 0)
+            sh = 0;
         for (int i = tid; i < N; i += TPB)
-            if (s_key[i] == kth)
-                atomicAdd(&s_nt, 1);
+            atomicAdd(&s_gs.hist[(best_key(s_cpack[i]) >> sh) & 255u], 1);
         __syncthreads();
-        const int n_ties = s_nt;
+        int            remaining = k;
+        const int      digit     = radix_pick_digit(s_gs.hist, remaining, s_gs.scan, s_gs.sel);
+        const uint32_t low       = ((s_kmax >> sh) & ~255u) | (uint32_t) digit;
+        /* everything in or above the digit that holds the k-th largest */
         for (int i = tid; i < N; i += TPB) {
-            const uint32_t key  = s_key[i];
-            bool           take = key > kth;
-            if (key == kth) {
-                take = true;
-                if (n_ties > need_ties) { /* only the lowest-index ties survive */
-                    const int me   = s_idx[i];
-                    int       rank = 0;
-                    for (int j = 0; j < N; ++j)
-                        rank += (s_key[j] == kth) && (s_idx[j] < me);
-                    take = rank < need_ties;
+            const uint64_t p = s_cpack[i];
+            if ((best_key(p) >> sh) >= low) {
+                const int pos = atomicAdd(&s_n, 1);
+                if (pos < TPB)
+                    s_m[pos] = p;
+            }
+        }
+        __syncthreads();
+        const int m = s_n;
+        if (m <= TPB) {
+            /* order them by counting (entries are distinct); the first k are the survivors */
+            uint64_t me   = 0;
+            int      rank = 0;
+            if (tid < m) {
+                me = s_m[tid];
+                for (int j = 0; j < m; ++j)
+                    rank += s_m[j] > me;
+                if (rank < k)
+                    s_pack[rank] = me;
+            }
+            __syncthreads();
+        } else {
+            /* crowded digit (many near-equal candidates): full radix select in LDS */
+            if (tid == 0)
+                s_n = 0;
+            int            need_ties;
+            const uint32_t kth =
+                lds_kth_largest(s_cpack, N, k, s_gs.hist, s_gs.scan, s_gs.sel, need_ties);
+            for (int i = tid; i < N; i += TPB)
+                if (best_key(s_cpack[i]) == kth)
+                    atomicAdd(&s_nt, 1);
+            __syncthreads();
+            const int n_ties = s_nt;
+            for (int i = tid; i < N; i += TPB) {
+                const uint64_t p    = s_cpack[i];
+                const uint32_t key  = best_key(p);
+                bool           take = key > kth;
+                if (key == kth) {
+                    take = true;
+                    if (n_ties > need_ties) { /* only the lowest-index ties survive */
+                        int rank = 0;
+                        for (int j = 0; j < N; ++j)
+                            rank += (best_key(s_cpack[j]) == kth) && (s_cpack[j] > p);
+                        take = rank < need_ties;
+                    }
+                }
+                if (take) {
+                    const int pos = atomicAdd(&s_n, 1);
+                    s_m[pos]      = p; /* k <= TOPK_FAST_MAX <= TPB entries */
                 }
             }
-            if (take) {
-                const int pos = atomicAdd(&s_n, 1);
-                s_pack[pos]   = pack_best(key, (uint32_t) s_idx[i]);
+            __syncthreads();
+            uint64_t me   = 0;
+            int      rank = 0;
+            if (tid < k) {
+                me = s_m[tid];
+                for (int j = 0; j < k; ++j)
+                    rank += s_m[j] > me;
+                s_pack[rank] = me;
             }
+            __syncthreads();
         }
-        __syncthreads();
-        /* order the k survivors: rank by counting (entries are distinct) */
-        uint64_t me   = 0;
-        int      rank = 0;
-        if (tid < k) {
-            me = s_pack[tid];
-            for (int j = 0; j < k; ++j)
-                rank += s_pack[j] > me;
-        }
-        __syncthreads();
-        if (tid < k)
-            s_pack[rank] = me;
-        __syncthreads();
     }
-    const int tok = finish_sorted(k, s_pack, a.inv_t, a.top_p, a.min_p, a.uniforms[row], s_fs);
-    if (tid == 0)
-        a.out[row] = tok;
+    /* k <= TOPK_FAST_MAX = 128: the tail runs on one wavefront without barriers */
+    if (tid < WAVE) {
+        const int tok =
+            finish_sorted_wave(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab);
+        if (tid == 0)
+            a.out[row] = tok;
+    }
 }
 
 /* ============================================================================================
@@ -715,7 +870,7 @@ __global__ __launch_bounds__(TPB) void k_topk_general(RowView rv, FinalArgs a, i
     extern __shared__ uint64_t s_dyn_pack[];
     __shared__ FinishShared    s_fs;
     __shared__ GeneralShared   s_gs;
-    __shared__ uint32_t        s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     const int                  row = blockIdx.x;
     const int k = topk_row_general<NV, PEN>(rv, row, a.k, s_dyn_pack, spack_cap, s_cnt16, s_gs);
     const int tok =
@@ -732,7 +887,7 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
                                                      const uint64_t *__restrict__ chunk_best,
                                                      const double *__restrict__ chunk_sum,
                                                      float *__restrict__ probs, long ld_probs) {
-    __shared__ uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ double   s_total;
@@ -770,11 +925,12 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
  * ========================================================================================== */
 template <int NV>
 __global__ __launch_bounds__(TPB) void k_penalties(RowView rv, float *__restrict__ logits_rw) {
-    __shared__ uint32_t s_cnt16[NV * TPB * 2];
+    __shared__ __align__(16) uint32_t s_cnt16[NV * TPB * 2];
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     int                 base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
-    history_counts<NV * TPB * 4>(rv, row, base, end, s_cnt16);
+    history_clear<NV * TPB * 4>(s_cnt16);
+    history_count(rv, row, base, end, s_cnt16);
     float *rowp = logits_rw + (long) row * rv.ld;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -859,12 +1015,10 @@ void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_bes
     });
 }
 
-void launch_topk_scan(const Launch &L, int k, int cap, uint32_t *cand_key, int32_t *cand_idx,
-                      int32_t *cand_cnt) {
+void launch_topk_scan(const Launch &L, int k, int cap, uint64_t *cand_pack, int32_t *cand_cnt) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_topk_scan<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, k, cap, cand_key, cand_idx,
-                                                                 cand_cnt);
+        k_topk_scan<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, k, cap, cand_pack, cand_cnt);
     });
 }
 
@@ -879,8 +1033,7 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.uniforms   = f.uniforms;
     a.chunk_best = f.chunk_best;
     a.chunk_sum  = f.chunk_sum;
-    a.cand_key   = f.cand_key;
-    a.cand_idx   = f.cand_idx;
+    a.cand_pack  = f.cand_pack;
     a.cand_cnt   = f.cand_cnt;
     a.out        = f.out;
     const dim3 grid(L.rows), block(TPB);
