@@ -27,8 +27,7 @@ struct geist_hip_sampler {
     /* device workspace */
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
-    uint64_t *cand_pack  = nullptr; /* [max_rows][max_chunks][TOPK_CAND_CAP] */
-    int32_t  *cand_cnt   = nullptr; /* [max_rows][max_chunks] */
+    float    *tmax       = nullptr; /* [max_rows][max_chunks][256] per-thread maxima */
     int32_t  *row_flag   = nullptr; /* [max_rows] */
     float    *uniforms   = nullptr; /* [max_rows] */
     float    *probe_p    = nullptr; /* [max_rows] */
@@ -76,12 +75,9 @@ static bool plan_chunks(size_t rows, size_t n_vocab, int &nv, int &per_chunk, in
         return false;
     /* fewer than two workgroups per compute unit: cut the rows finer */
     nv                 = (rows * big < 512 && small <= (size_t) MAX_CHUNKS) ? 2 : 8;
-    const size_t cap   = (size_t) 1024 * nv;
-    const size_t c0    = (n_vocab + cap - 1) / cap;
-    size_t       per   = (n_vocab + c0 - 1) / c0;
-    per                = (per + 63) / 64 * 64;
-    per_chunk          = (int) per;
-    n_chunks           = (int) ((n_vocab + per - 1) / per);
+    /* every chunk but the last is exactly what one workgroup holds in registers */
+    per_chunk = 1024 * nv;
+    n_chunks  = (int) ((n_vocab + per_chunk - 1) / per_chunk);
     return true;
 }
 
@@ -183,8 +179,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     hipError_t   e  = hipSetDevice(device);
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
-    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_pack, rc * TOPK_CAND_CAP * sizeof(uint64_t));
-    if (e == hipSuccess) e = hipMalloc((void **) &s->cand_cnt, rc * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->tmax, rc * 256 * sizeof(float));
     if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
     if (e == hipSuccess) e = hipMalloc((void **) &s->probe_p, max_rows * sizeof(float));
@@ -206,8 +201,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipStreamSynchronize(s->stream);
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
-    (void) hipFree(s->cand_pack);
-    (void) hipFree(s->cand_cnt);
+    (void) hipFree(s->tmax);
     (void) hipFree(s->row_flag);
     (void) hipFree(s->uniforms);
     (void) hipFree(s->probe_p);
@@ -305,10 +299,8 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     f.uniforms   = d_uniforms;
     f.chunk_best = s->chunk_best;
     f.chunk_sum  = s->chunk_sum;
-    f.cand_pack  = s->cand_pack;
-    f.cand_cnt   = s->cand_cnt;
+    f.tmax       = s->tmax;
     f.out        = d_out;
-    f.cap        = TOPK_CAND_CAP;
 
     if (rs.greedy) {
         mark_start(s);
@@ -330,8 +322,29 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                             hipGetErrorString((hipError_t) e));
             return after_launch(s, "top-k (general)");
         }
+        /* the thread-maxima path wants the large chunks whatever the batch size: the final
+         * kernel holds one key per scanning thread in LDS */
+        L.nv           = 8;
+        L.rv.per_chunk = 8192;
+        L.rv.n_chunks  = (int) ((rows->n_vocab + 8191) / 8192);
+        /* Penalties that can only lower a logit (rep >= 1, freq >= 0, pres >= 0) need not be
+         * applied while scanning: the raw thread maxima then bound the penalised ones from
+         * above, the final kernel penalises the elements it re-reads and checks that k of them
+         * still reach the bound -- which proves that no element outside the re-read threads can
+         * belong to the top k. A margin on the rank of the bound keeps that check from failing
+         * when several leading logits are penalised away; a row that still fails takes the
+         * general path. */
+        Launch scan = L;
+        f.k_sel     = rs.k;
+        if (L.pen && L.rv.rep >= 1.0f && L.rv.freq >= 0.0f && L.rv.pres >= 0.0f) {
+            scan.pen         = false;
+            scan.rv.hist     = nullptr;
+            scan.rv.hist_len = nullptr;
+            const int margin = rs.k / 2 > 8 ? rs.k / 2 : 8;
+            f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
+        }
         mark_start(s);
-        launch_topk_scan(L, rs.k, TOPK_CAND_CAP, s->cand_pack, s->cand_cnt);
+        launch_tmax_scan(scan, s->tmax);
         mark_stop(s);
         f.mode = FINAL_TOPK;
         f.k    = rs.k;

@@ -46,6 +46,16 @@ __device__ __forceinline__ uint64_t pack_best(uint32_t key, uint32_t idx) {
 __device__ __forceinline__ uint32_t best_idx(uint64_t p) { return 0xffffffffu - (uint32_t) p; }
 __device__ __forceinline__ uint32_t best_key(uint64_t p) { return (uint32_t) (p >> 32); }
 
+/* Workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global
+ * load in flight (its fence covers all address spaces); where loads should stay outstanding
+ * across the barrier -- the chunk's logits while the history table is built -- this one waits
+ * for the LDS counter alone. */
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 /* ---- wavefront-64 reductions -------------------------------------------------------------- */
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
     uint32_t lo = (uint32_t) v, hi = (uint32_t) (v >> 32);
@@ -95,6 +105,48 @@ __device__ __forceinline__ int wave_scan_i32(int v) {
             v += o;
     }
     return v;
+}
+
+/* Inclusive prefix sum over the wavefront with DPP moves: shifts inside each row of 16 lanes,
+ * then the row totals are broadcast into the following rows. */
+__device__ __forceinline__ int wave_scan_i32_dpp(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false); /* row_shr:1 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false); /* row_shr:2 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false); /* row_shr:4 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false); /* row_shr:8 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false); /* row_bcast:15 -> rows 1, 3 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); /* row_bcast:31 -> rows 2, 3 */
+    return v;
+}
+/* The same for doubles: both halves travel by DPP, lanes without a source add 0.0. */
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_fetch_f64(double v) {
+    const uint64_t u  = (uint64_t) __double_as_longlong(v);
+    const int      lo = __builtin_amdgcn_update_dpp(0, (int) (uint32_t) u, CTRL, ROW_MASK, 0xf, false);
+    const int      hi =
+        __builtin_amdgcn_update_dpp(0, (int) (uint32_t) (u >> 32), CTRL, ROW_MASK, 0xf, false);
+    return __longlong_as_double((long long) (((uint64_t) (uint32_t) hi << 32) | (uint32_t) lo));
+}
+__device__ __forceinline__ double wave_scan_f64_dpp(double v) {
+    v += dpp_fetch_f64<0x111, 0xf>(v);
+    v += dpp_fetch_f64<0x112, 0xf>(v);
+    v += dpp_fetch_f64<0x114, 0xf>(v);
+    v += dpp_fetch_f64<0x118, 0xf>(v);
+    v += dpp_fetch_f64<0x142, 0xa>(v);
+    v += dpp_fetch_f64<0x143, 0xc>(v);
+    return v;
+}
+
+/* Each lane asks for `cnt` consecutive places in a list whose length lives in LDS; one atomic
+ * per wavefront. Returns the lane's first place. All 64 lanes must call. */
+__device__ __forceinline__ int wave_reserve(int cnt, int *counter) {
+    const int incl  = wave_scan_i32_dpp(cnt);
+    const int total = __shfl(incl, WAVE - 1, WAVE);
+    int       base  = 0;
+    if ((threadIdx.x & (WAVE - 1)) == WAVE - 1 && total)
+        base = atomicAdd(counter, total);
+    base = __shfl(base, WAVE - 1, WAVE);
+    return base + incl - cnt;
 }
 
 /* ---- workgroup combines through LDS -------------------------------------------------------- */
@@ -185,21 +237,89 @@ __device__ __forceinline__ void history_clear(uint32_t *cnt16) {
     uint4 *p = reinterpret_cast<uint4 *>(cnt16);
     for (int i = threadIdx.x; i < CHUNK / 8; i += TPB)
         p[i] = make_uint4(0u, 0u, 0u, 0u);
-    __syncthreads();
+    lds_barrier();
 }
-__device__ __forceinline__ void history_count(const RowView &rv, int row, int base, int end,
-                                              uint32_t *cnt16) {
-    int len = rv.hist_len ? rv.hist_len[row] : 0;
+/* Reading a row's history in two steps so that its loads are in flight early:
+ * history_prefetch() issues the loads of the row's length and of the first 8 ids per thread
+ * (4 ids per load; an unaligned history is read id by id later), history_for_each() then
+ * calls f(id) for every entry, the workgroup's threads sharing the entries. */
+struct HistPrefetch {
+    int4 a, b;
+    int  len;
+    bool vec;
+};
+/* `n_rows` is the number of rows of the launch. The row's length is fetched with a vector load
+ * (each lane reads the length of a following row, lane 0 its own): a scalar load here would
+ * sit in the same counter as the LDS traffic and stall the first barrier until it returns. */
+__device__ __forceinline__ HistPrefetch history_prefetch(const RowView &rv, int row, int n_rows) {
+    HistPrefetch   pf;
+    const int32_t *h   = rv.hist + (long) row * rv.hist_ld;
+    const int      ld4 = (int) (rv.hist_ld >> 2);
+    const int      g   = threadIdx.x;
+    {
+        int r = row + (int) (threadIdx.x & (WAVE - 1));
+        r     = r < n_rows ? r : n_rows - 1;
+        pf.len = rv.hist_len[r]; /* lane 0 holds this row's length; broadcast when consumed */
+    }
+    pf.vec             = (((uintptr_t) h) & 15) == 0;
+    const int4 *h4     = reinterpret_cast<const int4 *>(h);
+    pf.a               = make_int4(-1, -1, -1, -1);
+    pf.b               = make_int4(-1, -1, -1, -1);
+    if (pf.vec && g < ld4)
+        pf.a = h4[g];
+    if (pf.vec && g + TPB < ld4)
+        pf.b = h4[g + TPB];
+    return pf;
+}
+template <typename F>
+__device__ __forceinline__ void history_for_each(const RowView &rv, int row,
+                                                 const HistPrefetch &pf, F &&f) {
+    int len = __builtin_amdgcn_readfirstlane(pf.len);
     if (len > rv.hist_ld)
         len = (int) rv.hist_ld;
-    const int32_t *h = rv.hist + (long) row * rv.hist_ld;
-    for (int i = threadIdx.x; i < len; i += TPB) {
-        const int t   = h[i];
+    const int32_t *h  = rv.hist + (long) row * rv.hist_ld;
+    int            i0 = 0;
+    if (pf.vec) {
+        const int4 *h4 = reinterpret_cast<const int4 *>(h);
+        const int   n4 = len >> 2;
+        const int   g  = threadIdx.x;
+        if (g < n4) {
+            f(pf.a.x);
+            f(pf.a.y);
+            f(pf.a.z);
+            f(pf.a.w);
+        }
+        if (g + TPB < n4) {
+            f(pf.b.x);
+            f(pf.b.y);
+            f(pf.b.z);
+            f(pf.b.w);
+        }
+        for (int g2 = g + 2 * TPB; g2 < n4; g2 += 2 * TPB) {
+            const int4 a = h4[g2];
+            const int4 b = g2 + TPB < n4 ? h4[g2 + TPB] : make_int4(-1, -1, -1, -1);
+            f(a.x);
+            f(a.y);
+            f(a.z);
+            f(a.w);
+            f(b.x);
+            f(b.y);
+            f(b.z);
+            f(b.w);
+        }
+        i0 = n4 << 2;
+    }
+    for (int i = i0 + threadIdx.x; i < len; i += TPB)
+        f(h[i]);
+}
+__device__ __forceinline__ void history_count(const RowView &rv, int row, const HistPrefetch &pf,
+                                              int base, int end, uint32_t *cnt16) {
+    history_for_each(rv, row, pf, [&](int t) {
         const int off = t - base;
         if (off >= 0 && t < end)
             atomicAdd(&cnt16[off >> 1], 1u << (16 * (off & 1)));
-    }
-    __syncthreads();
+    });
+    lds_barrier();
 }
 
 /* Issues the loads of the chunk [base, end) of a row into registers (layout in the file
@@ -209,6 +329,13 @@ __device__ __forceinline__ void load_raw(const RowView &rv, const float *__restr
                                          int base, int end, float4 (&v)[NV]) {
     const int   tid  = threadIdx.x;
     const float ninf = -__builtin_inff();
+    if (rv.vec_ok && end - base == NV * TPB * 4) { /* full chunk: no per-element tests */
+        const float4 *p = reinterpret_cast<const float4 *>(row + base) + tid;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            v[j] = p[j * TPB];
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int e = base + 4 * (j * TPB + tid);

@@ -10,10 +10,10 @@
 namespace gs {
 
 constexpr int MAX_CHUNKS     = 128;  /* chunks per row */
-constexpr int TOPK_CAND_CAP  = 256;  /* candidates one chunk may hand on */
+constexpr int TMAX_LDS       = 8192; /* thread maxima of one row the final kernel holds in LDS */
+constexpr int SEL_MAX        = 192;  /* threads whose elements the final kernel re-reads */
 constexpr int TOPK_FAST_MAX  = 128;  /* largest k served by the candidate path */
 constexpr int TOPK_MAX       = 8192; /* the reference caps top_k here (sampler.c:213-215) */
-constexpr int FINAL_CAND_MAX = 4096; /* candidates one row may merge in LDS */
 constexpr int HISTORY_MAX    = 65535;
 
 enum { FINAL_ARGMAX = 0, FINAL_TEMPERATURE = 1, FINAL_TOPK = 2 };
@@ -42,20 +42,19 @@ struct Launch {
 };
 
 struct FinalLaunch {
-    int             mode, k, cap;
+    int             mode, k, k_sel;
     float           inv_t, top_p, min_p;
     const float    *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
-    const uint64_t *cand_pack;
-    const int32_t  *cand_cnt;
+    const float    *tmax;
     int32_t        *out;
 };
 
 void launch_chunk_best(const Launch &L, uint64_t *chunk_best);
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, float *probe_p);
-void launch_topk_scan(const Launch &L, int k, int cap, uint64_t *cand_pack, int32_t *cand_cnt);
+void launch_tmax_scan(const Launch &L, float *tmax);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);

@@ -4,7 +4,7 @@
  * Kernel map (reference lines the arithmetic follows are cited at each kernel):
  *   k_chunk_best     per-(row, chunk) maximum with lowest-index tie-break     sampler.c:52-62, 70-75
  *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t)          sampler.c:77-83
- *   k_topk_scan      per-(row, chunk) candidates that can be in the top k     sampler.c:202-207
+ *   k_tmax_scan      per-thread maxima: the single pass of the top-k path       sampler.c:202-207
  *   k_row_final      per-row combine: argmax / index-order CDF draw / top-k
  *                    select, sorted softmax, top-p, min-p, draw               sampler.c:90-102, 209-222, 272-299
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
@@ -36,9 +36,6 @@ __device__ long long g_phase[16384 * 8];
 #define GS_MARK(i) ((void) 0)
 #endif
 
-/* number of leading key bits the per-chunk threshold search resolves */
-constexpr int THR_BITS = 16;
-
 template <int NV>
 __device__ __forceinline__ void chunk_bounds(const RowView &rv, int chunk, int &base, int &end) {
     base = chunk * rv.per_chunk;
@@ -51,14 +48,18 @@ __device__ __forceinline__ void chunk_bounds(const RowView &rv, int chunk, int &
  * is an LDS table of NV*512 words when PEN, else unused. The logit loads are issued before the
  * history is read so that both are in flight together. */
 template <int NV, bool PEN>
-__device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int base, int end,
-                                            uint32_t *cnt16, float4 (&v)[NV]) {
+__device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_rows, int base,
+                                            int end, uint32_t *cnt16, float4 (&v)[NV]) {
     const float *rowp = rv.logits + (long) row * rv.ld;
     if (PEN) {
-        history_clear<NV * TPB * 4>(cnt16);
+        const HistPrefetch pf = history_prefetch(rv, row, n_rows);
         load_raw<NV>(rv, rowp, base, end, v);
-        history_count(rv, row, base, end, cnt16);
+        history_clear<NV * TPB * 4>(cnt16);
+        GS_MARK(3);
+        history_count(rv, row, pf, base, end, cnt16);
+        GS_MARK(4);
         apply_transform<NV>(rv, cnt16, v);
+        GS_MARK(5);
     } else {
         load_raw<NV>(rv, rowp, base, end, v);
         apply_transform<NV>(rv, nullptr, v);
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_best(RowView rv, uint64_t *__rest
     int                 base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
 
     uint64_t best = 0;
 #pragma unroll
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
     const float mx = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
 
     const int tok = probe_token ? probe_token[row] : -1;
@@ -150,104 +151,32 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
 }
 
 /* ============================================================================================
- * k_topk_scan: every element of the chunk that can belong to the row's top k.
- *
- * The workgroup's 256 per-thread maxima are folded into G = 64, 128 or 256 group maxima; the
- * k-th largest of them is a lower bound of the chunk's k-th largest element, so every element
- * at or above it is kept (about -G ln(1 - k/G) of them). The bound is found on the leading
- * THR_BITS of the order-preserving key by a bitwise search with wavefront ballots. Comparisons
- * on the elements themselves stay in fp32: max ignores NaN and `!(x < bound)` keeps it, which
- * is what the key order prescribes. A chunk that yields more than `cap` candidates reports its
- * true count and the row takes the general path.
+ * k_tmax_scan: the one pass over the logits of the top-k path. Each thread keeps only the
+ * maximum of the 4*NV elements it read (after penalties and soft-cap) and stores it; nothing
+ * else leaves the workgroup. The row-final kernel picks the k-th largest of a row's thread
+ * maxima -- a lower bound of the row's k-th largest element, because k different threads hold
+ * an element at or above it -- and re-reads only the elements of the threads at or above that
+ * bound (about k of them, 4*NV elements each).
+ * max ignores NaN; a thread with no element of the row stores NaN and is never chosen.
  * ========================================================================================== */
-template <int VPL>
-__device__ __forceinline__ uint32_t kth_group_max(uint32_t q0, uint32_t q1, uint32_t q2,
-                                                  uint32_t q3, int kk) {
-    uint32_t tau = 0;
-#pragma unroll
-    for (int bit = 31; bit >= 32 - THR_BITS; --bit) {
-        const uint32_t t   = tau | (1u << bit);
-        int            cnt = __popcll(__ballot(q0 >= t));
-        if (VPL >= 2)
-            cnt += __popcll(__ballot(q1 >= t));
-        if (VPL >= 4)
-            cnt += __popcll(__ballot(q2 >= t)) + __popcll(__ballot(q3 >= t));
-        if (cnt >= kk)
-            tau = t;
-    }
-    return tau;
-}
-
 template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_topk_scan(RowView rv, int k, int cap,
-                                                   uint64_t *__restrict__ cand_pack,
-                                                   int32_t *__restrict__ cand_cnt) {
+__global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict__ tmax) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ float    s_tmax[TPB];
-    __shared__ uint64_t s_cand[TOPK_CAND_CAP];
-    __shared__ int      s_n;
-    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
-    const int           lane = tid & (WAVE - 1);
-    int                 base, end;
+    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    int       base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     GS_MARK(0);
     float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
-
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
     float tm = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < NV; ++j)
         tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
-    s_tmax[tid] = tm;
-    if (tid == 0)
-        s_n = 0;
+    if (base + 4 * tid >= end)
+        tm = __builtin_nanf("");
     GS_MARK(1);
-    __syncthreads();
+    tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
     GS_MARK(2);
-
-    const float g0 = s_tmax[lane], g1 = s_tmax[lane + 64], g2 = s_tmax[lane + 128],
-                g3 = s_tmax[lane + 192];
-    uint32_t tau;
-    if (k <= 24) {
-        tau = kth_group_max<1>(f2key(max3f(max3f(g0, g1, g2), g3, g3)), 0, 0, 0, k);
-    } else if (k <= 64) {
-        tau = kth_group_max<2>(f2key(max3f(g0, g2, g2)), f2key(max3f(g1, g3, g3)), 0, 0, k);
-    } else {
-        tau = kth_group_max<4>(f2key(g0), f2key(g1), f2key(g2), f2key(g3), k < TPB ? k : TPB);
-    }
-    const float bound = key2f(tau); /* tau == 0 maps to NaN: nothing is below it */
-    GS_MARK(3);
-
-    /* Padding holds -inf, so with a finite bound no index test is needed on the hot path. */
-    const bool check_idx = !(bound > -__builtin_inff());
-    if (!(tm < bound)) {
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const float m4 = f4_max(v[j]);
-            if (!(m4 < bound) || check_idx) {
-                const int e = base + 4 * (j * TPB + tid);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float x = f4_get(v[j], c);
-                    if (!(x < bound) && (!check_idx || e + c < end)) {
-                        const int pos = atomicAdd(&s_n, 1);
-                        if (pos < cap)
-                            s_cand[pos] = pack_best(f2key(x), (uint32_t) (e + c));
-                    }
-                }
-            }
-        }
-    }
-    GS_MARK(4);
-    __syncthreads();
-    const int  n = s_n;
-    const long o = (long) row * rv.n_chunks + chunk;
-    if (tid == 0)
-        cand_cnt[o] = n;
-    const int m = n < cap ? n : cap;
-    for (int i = tid; i < m; i += TPB)
-        cand_pack[o * cap + i] = s_cand[i];
-    GS_MARK(5);
 }
 
 /* ============================================================================================
@@ -362,63 +291,91 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
     return (int) best_idx(spack[at]);
 }
 
-/* finish_sorted for n <= 128 survivors on ONE wavefront (call with all 64 lanes of a single
- * wave): lane l owns entries 2l and 2l+1, the prefix sums are wavefront scans, no barrier.
- * `tab` is the expf table in LDS. */
+/* finish_sorted for n <= 64 * IPT survivors on ONE wavefront (call with all 64 lanes of a
+ * single wave): lane l owns entries IPT*l .. IPT*l + IPT-1, the prefix sums are wavefront scans,
+ * no barrier. `tab` is the expf table in LDS. */
+template <int IPT>
 __device__ int finish_sorted_wave(int n, const uint64_t *spack, float inv_t, float top_p,
                                   float min_p, float u, const uint64_t *tab) {
-    const int  lane  = threadIdx.x & (WAVE - 1);
-    const bool use_p = top_p > 0.0f && top_p < 1.0f;
-    const bool use_m = min_p > 0.0f;
-    const bool norm  = use_p || use_m;
-    const int  i0 = 2 * lane, i1 = 2 * lane + 1;
-    const float l0 = key2f(best_key(spack[0]));
-    float w0 = i0 < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i0])), l0, inv_t), tab)
-                      : 0.0f;
-    float w1 = i1 < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i1])), l0, inv_t), tab)
-                      : 0.0f;
-    double part = (double) w0 + (double) w1;
-    double incl = wave_scan_f64(part);
+    const int   lane  = threadIdx.x & (WAVE - 1);
+    const bool  use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool  use_m = min_p > 0.0f;
+    const bool  norm  = use_p || use_m;
+    const float l0    = key2f(best_key(spack[0]));
+    float       w[IPT];
+    double      part = 0.0;
+#pragma unroll
+    for (int t = 0; t < IPT; ++t) {
+        const int i = IPT * lane + t;
+        w[t] = i < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), tab)
+                     : 0.0f;
+        part += (double) w[t];
+    }
+    double incl = wave_scan_f64_dpp(part);
     if (norm) {
         const double sum = __shfl(incl, WAVE - 1, WAVE);
-        w0   = i0 < n ? (float) ((double) w0 / sum) : 0.0f;
-        w1   = i1 < n ? (float) ((double) w1 / sum) : 0.0f;
-        part = (double) w0 + (double) w1;
-        incl = wave_scan_f64(part);
+        part             = 0.0;
+#pragma unroll
+        for (int t = 0; t < IPT; ++t) {
+            const int i = IPT * lane + t;
+            w[t]        = i < n ? (float) ((double) w[t] / sum) : 0.0f;
+            part += (double) w[t];
+        }
+        incl = wave_scan_f64_dpp(part);
     }
-    const double c0 = (incl - part) + (double) w0; /* inclusive prefix at entry i0 */
-    const double c1 = c0 + (double) w1;            /* ... at entry i1 */
+    double c[IPT]; /* inclusive prefix at each owned entry */
+    {
+        double run = incl - part;
+#pragma unroll
+        for (int t = 0; t < IPT; ++t) {
+            run += (double) w[t];
+            c[t] = run;
+        }
+    }
     int keep = n;
     if (use_p) {
-        const uint64_t m0 = __ballot(i0 < n && c0 >= (double) top_p);
-        const uint64_t m1 = __ballot(i1 < n && c1 >= (double) top_p);
-        int first = n - 1;
-        if (m0) first = 2 * (__ffsll((long long) m0) - 1);
-        if (m1) {
-            const int f1 = 2 * (__ffsll((long long) m1) - 1) + 1;
-            first = (m0 && first < f1) ? first : f1;
+        int first = 0x7fffffff;
+#pragma unroll
+        for (int t = IPT - 1; t >= 0; --t) {
+            const uint64_t mk = __ballot(IPT * lane + t < n && c[t] >= (double) top_p);
+            if (mk) {
+                const int f = IPT * (__ffsll((long long) mk) - 1) + t;
+                first       = f < first ? f : first;
+            }
         }
-        keep = (m0 | m1) ? first + 1 : n;
+        if (first != 0x7fffffff)
+            keep = first + 1;
     }
     if (use_m) {
-        const float floor_w = __fmul_rn(min_p, __shfl(w0, 0, WAVE));
-        int m = __popcll(__ballot(i0 < n && w0 >= floor_w)) +
-                __popcll(__ballot(i1 < n && w1 >= floor_w));
-        if (m < 1) m = 1;
+        const float floor_w = __fmul_rn(min_p, __shfl(w[0], 0, WAVE));
+        int         m       = 0;
+#pragma unroll
+        for (int t = 0; t < IPT; ++t)
+            m += __popcll(__ballot(IPT * lane + t < n && w[t] >= floor_w));
+        if (m < 1)
+            m = 1;
         keep = m < keep ? m : keep;
     }
-    if (keep < 1) keep = 1;
-    const double   at_keep = ((keep - 1) & 1) ? c1 : c0;
-    const double   mass    = __shfl(at_keep, (keep - 1) >> 1, WAVE);
-    const double   target  = (double) u * mass;
-    const uint64_t h0 = __ballot(i0 < keep && target < c0);
-    const uint64_t h1 = __ballot(i1 < keep && target < c1);
-    int at = keep - 1;
-    if (h0 | h1) {
-        const int f0 = h0 ? 2 * (__ffsll((long long) h0) - 1) : 0x7fffffff;
-        const int f1 = h1 ? 2 * (__ffsll((long long) h1) - 1) + 1 : 0x7fffffff;
-        at = f0 < f1 ? f0 : f1;
+    if (keep < 1)
+        keep = 1;
+    double at_keep = c[0];
+#pragma unroll
+    for (int t = 1; t < IPT; ++t)
+        if (((keep - 1) % IPT) == t)
+            at_keep = c[t];
+    const double mass   = __shfl(at_keep, (keep - 1) / IPT, WAVE);
+    const double target = (double) u * mass;
+    int          at     = 0x7fffffff;
+#pragma unroll
+    for (int t = IPT - 1; t >= 0; --t) {
+        const uint64_t hk = __ballot(IPT * lane + t < keep && target < c[t]);
+        if (hk) {
+            const int f = IPT * (__ffsll((long long) hk) - 1) + t;
+            at          = f < at ? f : at;
+        }
     }
+    if (at == 0x7fffffff)
+        at = keep - 1;
     return (int) best_idx(spack[at]);
 }
 
@@ -515,7 +472,7 @@ __device__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t
         __syncthreads();
         for (int base = 0; base < n; base += TILE) {
             const int end = base + TILE < n ? base + TILE : n;
-            fetch_chunk<NV, PEN>(rv, row, base, end, cnt16, v);
+            fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, cnt16, v);
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
                 const int e = base + 4 * (j * TPB + tid);
@@ -543,7 +500,7 @@ __device__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t
     int ties_before = 0;
     for (int base = 0; base < n; base += TILE) {
         const int end = base + TILE < n ? base + TILE : n;
-        fetch_chunk<NV, PEN>(rv, row, base, end, cnt16, v);
+        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, cnt16, v);
         int ties_here = 0;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
@@ -601,37 +558,255 @@ __device__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t
     return k;
 }
 
-/* ============================================================================================
- * k_row_final: one workgroup per row.
- * ========================================================================================== */
 struct FinalArgs {
     int   mode; /* FINAL_ARGMAX, FINAL_TEMPERATURE, FINAL_TOPK */
     int   k;
-    int   cap;
+    int   k_sel; /* rank of the thread maximum used as the bound (>= k) */
     float inv_t;
     float top_p;
     float min_p;
     const float   *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
-    const uint64_t *cand_pack;
-    const int32_t  *cand_cnt;
+    const float    *tmax;
     int32_t        *out;
 };
+
+/* ============================================================================================
+ * topk_from_tmax: the row-final side of the thread-maxima path (see k_tmax_scan).
+ *   1. each thread of this workgroup takes KPT of the row's thread maxima (entry q*256 + tid
+ *      belongs to chunk q, scanning thread tid) and keeps their maximum;
+ *   2. the k-th largest of 128 pairwise maxima of those bounds the k-th largest thread maximum,
+ *      hence the row's k-th largest element, from below; every wavefront finds it on the
+ *      leading 20 key bits by a bitwise search with ballots;
+ *   3. the scanning threads at or above the bound are listed (about k ln-ish many);
+ *   4. their 4*NV elements each are read again, penalised from the history counts of exactly
+ *      those elements, soft-capped, and those reaching the bound are kept;
+ *   5. the kept entries are ordered by counting and the first k are the row's top k, equal
+ *      logits in ascending index order (sampler.c:207).
+ * Returns true when the row has to take the general path instead (fewer than k real maxima,
+ * long runs of equal values); otherwise k_out entries lie sorted in s_pack.
+ * ========================================================================================== */
+template <int NV, bool PEN, int KPT>
+__device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArgs &a, int row,
+                                               uint8_t *slot, uint32_t *s_mx, int *s_selid,
+                                               uint32_t *s_pcnt, uint64_t *s_m, uint64_t *s_pack,
+                                               int *s_n, int *s_n2, int &k_out) {
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int C   = rv.n_chunks;
+    HistPrefetch pf;
+    if (PEN)
+        pf = history_prefetch(rv, row, (int) gridDim.x);
+    /* 1 */
+    const float *tm = a.tmax + (long) row * C * TPB + tid;
+    float        raw[KPT];
+#pragma unroll
+    for (int q = 0; q < KPT; ++q)
+        raw[q] = q < C ? tm[q * TPB] : __builtin_nanf("");
+    {
+        uint4 *z = reinterpret_cast<uint4 *>(slot);
+        for (int i = tid; i < KPT * TPB / 16; i += TPB)
+            z[i] = make_uint4(0u, 0u, 0u, 0u);
+        if (PEN) {
+            for (int i = tid; i < SEL_MAX * 4 * NV; i += TPB)
+                s_pcnt[i] = 0u;
+        }
+        if (tid == 0) {
+            *s_n  = 0;
+            *s_n2 = 0;
+        }
+    }
+    float mxf = __builtin_nanf("");
+#pragma unroll
+    for (int q = 0; q + 1 < KPT; q += 2)
+        mxf = max3f(mxf, raw[q], raw[q + 1]);
+    s_mx[tid] = f2key(mxf); /* 0 when the thread saw no real maximum */
+    __syncthreads();
+    GS_MARK(1);
+    /* 2 */
+    const uint32_t a0 = s_mx[lane], a1 = s_mx[lane + 64], a2 = s_mx[lane + 128],
+                   a3 = s_mx[lane + 192];
+    int      real;
+    uint32_t tau = 0u;
+    if (a.k_sel <= 48) {
+        /* 128 pairwise maxima: about -128 ln(1 - k/128) threads end up selected */
+        const uint32_t m0 = a0 > a2 ? a0 : a2, m1 = a1 > a3 ? a1 : a3;
+        real = __popcll(__ballot(m0 != 0u)) + __popcll(__ballot(m1 != 0u));
+#pragma unroll
+        for (int bit = 31; bit >= 12; --bit) {
+            const uint32_t t   = tau | (1u << bit);
+            const int      cnt = __popcll(__ballot(m0 >= t)) + __popcll(__ballot(m1 >= t));
+            if (cnt >= a.k_sel)
+                tau = t;
+        }
+    } else {
+        /* all 256 maxima: about -256 ln(1 - k/256) threads */
+        real = __popcll(__ballot(a0 != 0u)) + __popcll(__ballot(a1 != 0u)) +
+               __popcll(__ballot(a2 != 0u)) + __popcll(__ballot(a3 != 0u));
+#pragma unroll
+        for (int bit = 31; bit >= 12; --bit) {
+            const uint32_t t   = tau | (1u << bit);
+            const int      cnt = __popcll(__ballot(a0 >= t)) + __popcll(__ballot(a1 >= t)) +
+                            __popcll(__ballot(a2 >= t)) + __popcll(__ballot(a3 >= t));
+            if (cnt >= a.k_sel)
+                tau = t;
+        }
+    }
+    GS_MARK(2);
+    /* keys at or below that of -inf: the bound says nothing (masked rows) */
+    if (real < a.k_sel || tau < 0x00800000u)
+        return true;
+    const float bound = key2f(tau);
+    /* 3 */
+    int cnt = 0;
+#pragma unroll
+    for (int q = 0; q < KPT; ++q)
+        cnt += raw[q] >= bound;
+    int pos = wave_reserve(cnt, s_n);
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+        if (raw[q] >= bound) {
+            if (pos < SEL_MAX) {
+                s_selid[pos]        = q * TPB + tid;
+                slot[q * TPB + tid] = (uint8_t) (pos + 1);
+            }
+            ++pos;
+        }
+    }
+    __syncthreads();
+    const int n_sel = *s_n;
+    if (n_sel > SEL_MAX)
+        return true; /* long runs of equal maxima */
+    /* 4 */
+    constexpr int TASKS = SEL_MAX * NV / TPB;
+    float4        r[TASKS];
+    int           e0[TASKS], e1[TASKS];
+    const float  *rowp = rv.logits + (long) row * rv.ld;
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+        const int t = tid + q * TPB;
+        const int s = t / NV, j = t % NV;
+        e0[q] = 0;
+        e1[q] = 0;
+        r[q]  = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (s < n_sel) {
+            const int L = s_selid[s];
+            const int chunk = L / TPB, tt = L % TPB;
+            int       base, end;
+            chunk_bounds<NV>(rv, chunk, base, end);
+            const int e = base + 4 * (j * TPB + tt);
+            e0[q] = e;
+            e1[q] = end;
+            if (rv.vec_ok && e + 3 < end) {
+                r[q] = *reinterpret_cast<const float4 *>(rowp + e);
+            } else {
+                r[q].x = e + 0 < end ? rowp[e + 0] : 0.f;
+                r[q].y = e + 1 < end ? rowp[e + 1] : 0.f;
+                r[q].z = e + 2 < end ? rowp[e + 2] : 0.f;
+                r[q].w = e + 3 < end ? rowp[e + 3] : 0.f;
+            }
+        }
+    }
+    GS_MARK(3);
+    if (PEN) {
+        const int shift = 31 - __clz(rv.per_chunk); /* per_chunk = 1024 * NV */
+        history_for_each(rv, row, pf, [&](int t) {
+            if (t < 0 || t >= rv.n_vocab)
+                return;
+            const int off = t & (rv.per_chunk - 1);
+            const int f   = off >> 2;
+            const int s   = slot[(t >> shift) * TPB + (f % TPB)];
+            if (s)
+                atomicAdd(&s_pcnt[((s - 1) * NV + f / TPB) * 4 + (off & 3)], 1u);
+        });
+        __syncthreads();
+    }
+    GS_MARK(4);
+    uint32_t ck[TASKS][4];
+    int      keep = 0;
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+        const int t = tid + q * TPB;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            ck[q][c] = 0u;
+            if (e0[q] + c < e1[q]) {
+                float x = f4_get(r[q], c);
+                if (PEN) {
+                    const uint32_t n_hist = s_pcnt[t * 4 + c];
+                    if (n_hist)
+                        x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
+                }
+                if (rv.softcap > 0.0f)
+                    x = __fmul_rn(tanhf(__fdiv_rn(x, rv.softcap)), rv.softcap);
+                if (x >= bound) {
+                    ck[q][c] = f2key(x);
+                    ++keep;
+                }
+            }
+        }
+    }
+    pos = wave_reserve(keep, s_n2);
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (ck[q][c]) {
+                if (pos < TPB)
+                    s_m[pos] = pack_best(ck[q][c], (uint32_t) (e0[q] + c));
+                ++pos;
+            }
+        }
+    }
+    __syncthreads();
+    const int m = *s_n2;
+    GS_MARK(5);
+    /* m > 256: long runs of equal values at the bound. m < k can only happen when the thread
+     * maxima were taken before the penalties (see the launch code): then too many of the
+     * leading logits were penalised below the bound and it certifies nothing. */
+    if (m > TPB || m < a.k)
+        return true;
+    const int k = a.k;
+    /* 5: entry i is compared with the others by P = 256 / m2 <= 64 neighbouring lanes */
+    int m2 = 4;
+    while (m2 < m)
+        m2 <<= 1;
+    const int P = TPB / m2, i = tid / P, part = tid % P;
+    uint64_t  me   = 0;
+    int       rank = 0;
+    if (i < m) {
+        me = s_m[i];
+#pragma unroll 4
+        for (int j = part; j < m; j += P)
+            rank += s_m[j] > me;
+    }
+    for (int d = 1; d < P; d <<= 1)
+        rank += __shfl_xor(rank, d, WAVE);
+    if (i < m && part == 0 && rank < k)
+        s_pack[rank] = me;
+    __syncthreads();
+    k_out = k;
+    return false;
+}
+
+/* ============================================================================================
+ * k_row_final: one workgroup per row.
+ * ========================================================================================== */
 
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     __shared__ uint64_t      s_red[NWAVES];
     __shared__ FinishShared  s_fs;
     __shared__ GeneralShared s_gs;
-    __shared__ uint64_t      s_cpack[FINAL_CAND_MAX];
+    __shared__ __align__(16) uint8_t s_big[TMAX_LDS];
+    __shared__ uint32_t      s_bitmap[TPB];
+    __shared__ int           s_selid[SEL_MAX];
+    __shared__ uint32_t      s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
     __shared__ uint64_t      s_m[TPB];
     __shared__ uint64_t      s_pack[TOPK_FAST_MAX];
     __shared__ double        s_csum[MAX_CHUNKS];
-    __shared__ uint32_t      s_kmin, s_kmax;
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ int           s_off[MAX_CHUNKS + 1];
-    __shared__ int           s_n, s_nt, s_chunk;
+    __shared__ int           s_n, s_n2, s_chunk;
     __shared__ double        s_before;
 
     const int row = blockIdx.x, tid = threadIdx.x;
@@ -683,7 +858,7 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
         int       base, end;
         chunk_bounds<NV>(rv, chunk, base, end);
         float4 v[NV];
-        fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
+        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
         /* index order inside the chunk is (j, thread, component): scan one j-slab at a time */
         double       carry  = s_before;
         const double target = s_fs.mass;
@@ -721,144 +896,35 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
         return;
     }
 
-    /* ---- FINAL_TOPK: merge the per-chunk candidates ---------------------------------------- */
+    /* ---- FINAL_TOPK: select from the row's thread maxima, then gather ------------------------ */
+    GS_MARK(0);
     if (tid < 32)
         s_fs.tab[tid] = g_expf_tab[tid];
-    const float u_row = a.uniforms[row];
-    int         n_c   = 0;
-    bool        over  = false;
-    if (tid < C) {
-        const int raw = a.cand_cnt[(long) row * C + tid];
-        over          = raw > a.cap;
-        n_c           = over ? a.cap : raw;
-    }
-    int       N;
-    const int incl = block_scan_i32(n_c, s_gs.scan, &N);
-    if (tid < C)
-        s_off[tid] = incl - n_c;
-    if (tid == 0) {
-        s_off[C] = N;
-        s_n      = 0;
-        s_nt     = 0;
-        s_kmin   = 0xffffffffu;
-        s_kmax   = 0u;
-    }
-    const bool general = __syncthreads_or(over) || N > FINAL_CAND_MAX;
-    int        k;
+    const float u_row   = a.uniforms[row];
+    int         k       = 0;
+    bool        general = true;
+    if (C <= 16)
+        general = topk_from_tmax<NV, PEN, 16>(rv, a, row, s_big, s_bitmap, s_selid, s_pcnt, s_m,
+                                              s_pack, &s_n, &s_n2, k);
+    else if (C <= TMAX_LDS / TPB)
+        general = topk_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, s_big, s_bitmap, s_selid,
+                                                          s_pcnt, s_m, s_pack, &s_n, &s_n2, k);
     if (general) {
-        /* some chunk had more candidates than it may hand on (long runs of equal values,
-         * masked rows): select over the whole row instead */
+        /* rows this shortcut cannot serve (masked rows full of -inf, all-equal rows, tiny or
+         * huge vocabularies): exact selection over the whole row */
+        __syncthreads();
         k = topk_row_general<NV, PEN>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
-    } else {
-        /* gather every candidate of the row into LDS; one global round trip */
-        uint32_t kmin = 0xffffffffu, kmax = 0u;
-        for (int i = tid; i < N; i += TPB) {
-            int lo = 0, hi = C; /* s_off[lo] <= i < s_off[hi] */
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (s_off[mid] <= i)
-                    lo = mid;
-                else
-                    hi = mid;
-            }
-            const uint64_t p = a.cand_pack[((long) row * C + lo) * a.cap + (i - s_off[lo])];
-            s_cpack[i]       = p;
-            const uint32_t key = best_key(p);
-            kmin = key < kmin ? key : kmin;
-            kmax = key > kmax ? key : kmax;
-        }
-        kmax = wave_max_u32(kmax);
-        kmin = ~wave_max_u32(~kmin);
-        if ((tid & (WAVE - 1)) == 0) {
-            atomicMax(&s_kmax, kmax);
-            atomicMin(&s_kmin, kmin);
-        }
-        s_gs.hist[tid] = 0;
-        __syncthreads();
-        k = a.k < N ? a.k : N;
-        /* one 8-bit radix step on the highest bits in which the candidates differ */
-        const uint32_t diff = s_kmin ^ s_kmax;
-        int            sh   = diff ? (31 - __clz((int) diff)) - 7 : 0;
-        if (sh < 0)
-            sh = 0;
-        for (int i = tid; i < N; i += TPB)
-            atomicAdd(&s_gs.hist[(best_key(s_cpack[i]) >> sh) & 255u], 1);
-        __syncthreads();
-        int            remaining = k;
-        const int      digit     = radix_pick_digit(s_gs.hist, remaining, s_gs.scan, s_gs.sel);
-        const uint32_t low       = ((s_kmax >> sh) & ~255u) | (uint32_t) digit;
-        /* everything in or above the digit that holds the k-th largest */
-        for (int i = tid; i < N; i += TPB) {
-            const uint64_t p = s_cpack[i];
-            if ((best_key(p) >> sh) >= low) {
-                const int pos = atomicAdd(&s_n, 1);
-                if (pos < TPB)
-                    s_m[pos] = p;
-            }
-        }
-        __syncthreads();
-        const int m = s_n;
-        if (m <= TPB) {
-            /* order them by counting (entries are distinct); the first k are the survivors */
-            uint64_t me   = 0;
-            int      rank = 0;
-            if (tid < m) {
-                me = s_m[tid];
-                for (int j = 0; j < m; ++j)
-                    rank += s_m[j] > me;
-                if (rank < k)
-                    s_pack[rank] = me;
-            }
-            __syncthreads();
-        } else {
-            /* crowded digit (many near-equal candidates): full radix select in LDS */
-            if (tid == 0)
-                s_n = 0;
-            int            need_ties;
-            const uint32_t kth =
-                lds_kth_largest(s_cpack, N, k, s_gs.hist, s_gs.scan, s_gs.sel, need_ties);
-            for (int i = tid; i < N; i += TPB)
-                if (best_key(s_cpack[i]) == kth)
-                    atomicAdd(&s_nt, 1);
-            __syncthreads();
-            const int n_ties = s_nt;
-            for (int i = tid; i < N; i += TPB) {
-                const uint64_t p    = s_cpack[i];
-                const uint32_t key  = best_key(p);
-                bool           take = key > kth;
-                if (key == kth) {
-                    take = true;
-                    if (n_ties > need_ties) { /* only the lowest-index ties survive */
-                        int rank = 0;
-                        for (int j = 0; j < N; ++j)
-                            rank += (best_key(s_cpack[j]) == kth) && (s_cpack[j] > p);
-                        take = rank < need_ties;
-                    }
-                }
-                if (take) {
-                    const int pos = atomicAdd(&s_n, 1);
-                    s_m[pos]      = p; /* k <= TOPK_FAST_MAX <= TPB entries */
-                }
-            }
-            __syncthreads();
-            uint64_t me   = 0;
-            int      rank = 0;
-            if (tid < k) {
-                me = s_m[tid];
-                for (int j = 0; j < k; ++j)
-                    rank += s_m[j] > me;
-                s_pack[rank] = me;
-            }
-            __syncthreads();
-        }
     }
+    GS_MARK(6);
     /* k <= TOPK_FAST_MAX = 128: the tail runs on one wavefront without barriers */
     if (tid < WAVE) {
         const int tok =
-            finish_sorted_wave(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab);
+            k <= WAVE ? finish_sorted_wave<1>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab)
+                      : finish_sorted_wave<2>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab);
         if (tid == 0)
             a.out[row] = tok;
     }
+    GS_MARK(7);
 }
 
 /* ============================================================================================
@@ -903,7 +969,7 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, base, end, s_cnt16, v);
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
     const float  mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
     const double tot = s_total;
     float       *out = probs + (long) row * ld_probs;
@@ -929,8 +995,9 @@ __global__ __launch_bounds__(TPB) void k_penalties(RowView rv, float *__restrict
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     int                 base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
+    const HistPrefetch pf = history_prefetch(rv, row, (int) gridDim.y);
     history_clear<NV * TPB * 4>(s_cnt16);
-    history_count(rv, row, base, end, s_cnt16);
+    history_count(rv, row, pf, base, end, s_cnt16);
     float *rowp = logits_rw + (long) row * rv.ld;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -1015,10 +1082,10 @@ void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_bes
     });
 }
 
-void launch_topk_scan(const Launch &L, int k, int cap, uint64_t *cand_pack, int32_t *cand_cnt) {
+void launch_tmax_scan(const Launch &L, float *tmax) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_topk_scan<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, k, cap, cand_pack, cand_cnt);
+        k_tmax_scan<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, tmax);
     });
 }
 
@@ -1026,15 +1093,14 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     FinalArgs a;
     a.mode       = f.mode;
     a.k          = f.k;
-    a.cap        = f.cap;
+    a.k_sel      = f.k_sel > f.k ? f.k_sel : f.k;
     a.inv_t      = f.inv_t;
     a.top_p      = f.top_p;
     a.min_p      = f.min_p;
     a.uniforms   = f.uniforms;
     a.chunk_best = f.chunk_best;
     a.chunk_sum  = f.chunk_sum;
-    a.cand_pack  = f.cand_pack;
-    a.cand_cnt   = f.cand_cnt;
+    a.tmax       = f.tmax;
     a.out        = f.out;
     const dim3 grid(L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {

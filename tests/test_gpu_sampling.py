@@ -217,6 +217,28 @@ def test_penalties_fused_into_sampling(hs, oracle):
     assert np.array_equal(x, before)
 
 
+def test_penalties_that_push_the_leaders_out(hs, oracle):
+    """Most of the leading logits are penalised far down, so the thread maxima taken before the
+    penalties promise too much: the row must still come out exact (it re-selects over the whole
+    row), also when a penalty RAISES logits (rep < 1, negative frequency / presence)."""
+    g = np.random.default_rng(16)
+    rows, n, H = 8, 60000, 400
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    lead = np.argsort(-x, axis=1)[:, :H].astype(np.int32)
+    hist = lead.copy()
+    hist[4:, 200:] = g.integers(0, n, (4, 200))
+    hl = np.full(rows, H, dtype=np.int32)
+    u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
+    for rep, freq, pres in [(1.0, 0.0, 6.0), (2.5, 1.0, 0.0), (0.7, -0.4, -0.3), (1.0, -2.0, 0.0)]:
+        got = run_rows(hs, torch, x, u, P(temperature=0.8, top_k=40, top_p=0.95, rep=rep, freq=freq,
+                                          pres=pres), hist, hl)
+        res = []
+        for r in range(rows):
+            pen = oracle.penalties(x[r], hist[r], rep, freq, pres)
+            res.append(oracle.chain_u(pen, float(u[r]), temperature=0.8, top_k=40, top_p=0.95))
+        compare_ids(got, [t for t, _ in res], [i for _, i in res], f"penalties {rep} {freq} {pres}")
+
+
 # ------------------------------------------------------------------------------ softmax
 @pytest.mark.parametrize("n,T", [(1000, 1.0), (128256, 0.7)])
 def test_normalised_probabilities(hs, oracle, n, T):
