@@ -33,6 +33,8 @@ struct geist_hip_sampler {
     float    *probe_p    = nullptr; /* [max_rows] */
     int32_t  *scalar_out = nullptr; /* [max_rows] */
     int32_t  *h_scalar   = nullptr; /* pinned */
+    float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
+                                     * full-vocabulary top-p / min-p path */
 
     /* timing of the dominant kernel */
     bool                    timing = false;
@@ -206,6 +208,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->uniforms);
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
+    (void) hipFree(s->probs);
     if (s->h_scalar)
         (void) hipHostFree(s->h_scalar);
     for (hipEvent_t e : s->ev_start)
@@ -304,7 +307,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
 
     if (rs.greedy) {
         mark_start(s);
-        launch_chunk_best(L, s->chunk_best);
+        launch_tmax_scan(L, s->tmax, s->chunk_best);
         mark_stop(s);
         f.mode = FINAL_ARGMAX;
         launch_row_final(L, f);
@@ -344,7 +347,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
             f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
         }
         mark_start(s);
-        launch_tmax_scan(scan, s->tmax);
+        launch_tmax_scan(scan, s->tmax, nullptr);
         mark_stop(s);
         f.mode = FINAL_TOPK;
         f.k    = rs.k;
@@ -352,7 +355,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         return after_launch(s, "top-k");
     }
     if (!rs.use_p && !rs.use_m) {
-        launch_chunk_best(L, s->chunk_best);
+        launch_tmax_scan(L, s->tmax, s->chunk_best);
         mark_start(s);
         launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
         mark_stop(s);
@@ -360,7 +363,29 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         launch_row_final(L, f);
         return after_launch(s, "temperature");
     }
-    return fail(s, GEIST_HIP_E_UNSUPPORTED, "full-vocabulary top-p / min-p is not built yet");
+    /* top-p and/or min-p over the whole vocabulary */
+    if (!s->probs)
+        HIPCHK(s, hipMalloc((void **) &s->probs, s->max_rows * s->max_vocab * sizeof(float)));
+    L.nv           = 8;
+    L.rv.per_chunk = 8192;
+    L.rv.n_chunks  = (int) ((rows->n_vocab + 8191) / 8192);
+    if (L.rv.n_chunks > s->max_chunks)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "n_vocab %zu needs more than %d chunks",
+                    rows->n_vocab, s->max_chunks);
+    launch_tmax_scan(L, s->tmax, s->chunk_best);
+    mark_start(s);
+    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+    mark_stop(s);
+    f.mode     = FINAL_SORTED;
+    f.row_flag = s->row_flag;
+    launch_row_final(L, f);
+    /* rows whose kept prefix is too wide for the shortcut flagged themselves; the next two
+     * kernels return at once for every other row */
+    launch_write_probs(L, rs.inv_t, s->chunk_best, s->chunk_sum, s->probs, (long) s->max_vocab,
+                       s->row_flag);
+    launch_sorted_general(L, s->probs, (long) s->max_vocab, rs.top_p, rs.min_p, d_uniforms,
+                          s->row_flag, d_out);
+    return after_launch(s, "top-p / min-p");
 }
 
 int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
@@ -459,9 +484,9 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
         return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_probs < n_vocab");
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
-    launch_chunk_best(L, s->chunk_best);
+    launch_tmax_scan(L, s->tmax, s->chunk_best);
     launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
-    launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs);
+    launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
 }
 

@@ -16,7 +16,7 @@ constexpr int TOPK_FAST_MAX  = 128;  /* largest k served by the candidate path *
 constexpr int TOPK_MAX       = 8192; /* the reference caps top_k here (sampler.c:213-215) */
 constexpr int HISTORY_MAX    = 65535;
 
-enum { FINAL_ARGMAX = 0, FINAL_TEMPERATURE = 1, FINAL_TOPK = 2 };
+enum { FINAL_ARGMAX = 0, FINAL_TEMPERATURE = 1, FINAL_TOPK = 2, FINAL_SORTED = 3 };
 
 /* One batch of logit rows as the kernels see it, with the transform applied while reading. */
 struct RowView {
@@ -49,17 +49,23 @@ struct FinalLaunch {
     const double   *chunk_sum;
     const float    *tmax;
     int32_t        *out;
+    int32_t        *row_flag;
 };
 
-void launch_chunk_best(const Launch &L, uint64_t *chunk_best);
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, float *probe_p);
-void launch_tmax_scan(const Launch &L, float *tmax);
+/* chunk_best may be NULL when only the thread maxima are wanted */
+void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
+/* row_flag != NULL: only rows with a non-zero flag are written */
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                        const double *chunk_sum, float *probs, long ld_probs);
+                        const double *chunk_sum, float *probs, long ld_probs,
+                        const int32_t *row_flag);
+void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
+                           float min_p, const float *uniforms, const int32_t *row_flag,
+                           int32_t *out);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

@@ -2,11 +2,12 @@
  * sampler_kernels.hip -- the HIP kernels of the token-sampling path (gfx950).
  *
  * Kernel map (reference lines the arithmetic follows are cited at each kernel):
- *   k_chunk_best     per-(row, chunk) maximum with lowest-index tie-break     sampler.c:52-62, 70-75
  *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t)          sampler.c:77-83
- *   k_tmax_scan      per-thread maxima: the single pass of the top-k path       sampler.c:202-207
+ *   k_tmax_scan      per-thread maxima (the single pass of the top-k path) and,
+ *                    on request, the per-chunk maximum with its first index       sampler.c:52-62, 202-207
  *   k_row_final      per-row combine: argmax / index-order CDF draw / top-k
  *                    select, sorted softmax, top-p, min-p, draw               sampler.c:90-102, 209-222, 272-299
+ *   k_sorted_general full-vocabulary top-p / min-p by mass-weighted radix descent sampler.c:246-304
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
  *   k_penalties      in-place penalties                                       (no reference counterpart)
  *   k_rng_units      xorshift64* uniforms                                     sampler.c:35-48
@@ -64,36 +65,6 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_ro
         load_raw<NV>(rv, rowp, base, end, v);
         apply_transform<NV>(rv, nullptr, v);
     }
-}
-
-/* ============================================================================================
- * k_chunk_best: the maximum of each chunk and where it first occurs.
- * ========================================================================================== */
-template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_chunk_best(RowView rv, uint64_t *__restrict__ chunk_best) {
-    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ uint64_t s_red[NWAVES];
-    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
-    int                 base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
-
-    uint64_t best = 0;
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (e + c < end) {
-                const uint64_t p = pack_best(f2key(f4_get(v[j], c)), (uint32_t) (e + c));
-                best             = p > best ? p : best;
-            }
-        }
-    }
-    best = block_max_u64(best, s_red);
-    if (tid == 0)
-        chunk_best[(long) row * rv.n_chunks + chunk] = best;
 }
 
 /* Row maximum from the per-chunk results; every thread returns the same packed value. */
@@ -159,9 +130,11 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
  * bound (about k of them, 4*NV elements each).
  * max ignores NaN; a thread with no element of the row stores NaN and is never chosen.
  * ========================================================================================== */
-template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict__ tmax) {
+template <int NV, bool PEN, bool BEST>
+__global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict__ tmax,
+                                                   uint64_t *__restrict__ chunk_best) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ uint64_t s_red[NWAVES];
     const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     int       base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
@@ -177,6 +150,31 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
     GS_MARK(1);
     tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
     GS_MARK(2);
+    if (BEST) {
+        /* the chunk's maximum and the first index holding it (sampler.c:52-62): only threads
+         * whose own maximum equals the chunk's look for the index */
+        const uint32_t mykey = f2key(tm);
+        uint32_t       bk    = wave_max_u32(mykey);
+        bk = (uint32_t) (block_max_u64((uint64_t) bk, s_red));
+        uint64_t best = 0;
+        if (mykey == bk) {
+            int first = 0x7fffffff;
+#pragma unroll
+            for (int j = NV - 1; j >= 0; --j) {
+                const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+                for (int c = 3; c >= 0; --c)
+                    if (e + c < end && f2key(f4_get(v[j], c)) == bk)
+                        first = e + c;
+            }
+            if (first != 0x7fffffff)
+                best = pack_best(bk, (uint32_t) first);
+        }
+        best = block_max_u64(best, s_red);
+        if (tid == 0) /* an all-NaN chunk reports key 0 at its first index */
+            chunk_best[(long) row * rv.n_chunks + chunk] =
+                best ? best : pack_best(0u, (uint32_t) base);
+    }
 }
 
 /* ============================================================================================
@@ -570,6 +568,7 @@ struct FinalArgs {
     const double   *chunk_sum;
     const float    *tmax;
     int32_t        *out;
+    int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to k_sorted_general */
 };
 
 /* ============================================================================================
@@ -789,6 +788,10 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
     return false;
 }
 
+} // namespace gs
+#include "sampler_sorted_prob.h"
+namespace gs {
+
 /* ============================================================================================
  * k_row_final: one workgroup per row.
  * ========================================================================================== */
@@ -803,6 +806,8 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     __shared__ int           s_selid[SEL_MAX];
     __shared__ uint32_t      s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
     __shared__ uint64_t      s_m[TPB];
+    __shared__ uint64_t      s_srt[TPB];
+    __shared__ float         s_wt[TPB];
     __shared__ uint64_t      s_pack[TOPK_FAST_MAX];
     __shared__ double        s_csum[MAX_CHUNKS];
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
@@ -896,6 +901,37 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
         return;
     }
 
+    if (a.mode == FINAL_SORTED) {
+        /* top-p / min-p over the whole vocabulary (sampler.c:232-305) */
+        if (tid < 32)
+            s_fs.tab[tid] = g_expf_tab[tid];
+        if (tid < C)
+            s_csum[tid] = a.chunk_sum[(long) row * C + tid];
+        const float u_row = a.uniforms[row];
+        const float mx    = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
+        if (tid == 0) {
+            double tot = 0.0;
+            for (int c = 0; c < C; ++c)
+                tot += s_csum[c];
+            s_before = tot;
+        }
+        __syncthreads();
+        const double sum = s_before;
+        int          tok = -1;
+        if (C <= 16)
+            tok = sorted_from_tmax<NV, PEN, 16>(rv, a, row, mx, sum, u_row, s_big, s_bitmap, s_wt,
+                                                s_selid, s_pcnt, s_m, s_srt, &s_n, &s_n2, s_fs.tab);
+        else if (C <= TMAX_LDS / TPB)
+            tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big,
+                                                            s_bitmap, s_wt, s_selid, s_pcnt, s_m,
+                                                            s_srt, &s_n, &s_n2, s_fs.tab);
+        if (tid == 0) {
+            a.row_flag[row] = tok < 0 ? 1 : 0;
+            a.out[row]      = tok;
+        }
+        return;
+    }
+
     /* ---- FINAL_TOPK: select from the row's thread maxima, then gather ------------------------ */
     GS_MARK(0);
     if (tid < 32)
@@ -952,12 +988,15 @@ template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
                                                      const uint64_t *__restrict__ chunk_best,
                                                      const double *__restrict__ chunk_sum,
-                                                     float *__restrict__ probs, long ld_probs) {
+                                                     float *__restrict__ probs, long ld_probs,
+                                                     const int32_t *__restrict__ row_flag) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ double   s_total;
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    if (row_flag && !row_flag[row])
+        return; /* only the rows that asked for their probabilities */
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid == 0) {
@@ -1066,13 +1105,6 @@ static void dispatch(int nv, bool pen, F &&f) {
 #define GS_NV decltype(nv)::value
 #define GS_PEN decltype(pen)::value
 
-void launch_chunk_best(const Launch &L, uint64_t *chunk_best) {
-    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
-    dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_chunk_best<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, chunk_best);
-    });
-}
-
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, float *probe_p) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
@@ -1082,10 +1114,13 @@ void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_bes
     });
 }
 
-void launch_tmax_scan(const Launch &L, float *tmax) {
+void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_tmax_scan<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, tmax);
+        if (chunk_best)
+            k_tmax_scan<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(L.rv, tmax, chunk_best);
+        else
+            k_tmax_scan<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(L.rv, tmax, nullptr);
     });
 }
 
@@ -1101,6 +1136,7 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.chunk_best = f.chunk_best;
     a.chunk_sum  = f.chunk_sum;
     a.tmax       = f.tmax;
+    a.row_flag   = f.row_flag;
     a.out        = f.out;
     const dim3 grid(L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
@@ -1138,12 +1174,20 @@ int launch_topk_general(const Launch &L, const FinalLaunch &f) {
 }
 
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                        const double *chunk_sum, float *probs, long ld_probs) {
+                        const double *chunk_sum, float *probs, long ld_probs,
+                        const int32_t *row_flag) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_write_probs<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, inv_t, chunk_best,
-                                                                   chunk_sum, probs, ld_probs);
+        k_write_probs<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
+            L.rv, inv_t, chunk_best, chunk_sum, probs, ld_probs, row_flag);
     });
+}
+
+void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
+                           float min_p, const float *uniforms, const int32_t *row_flag,
+                           int32_t *out) {
+    k_sorted_general<<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(probs, ld_probs, L.rv.n_vocab, top_p,
+                                                               min_p, uniforms, row_flag, out);
 }
 
 void launch_penalties(const Launch &L, float *logits_rw) {

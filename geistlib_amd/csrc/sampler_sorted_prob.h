@@ -1,0 +1,630 @@
+/*
+ * sampler_sorted_prob.h -- the full-vocabulary probability-ordered modes: top-p (the
+ * reference's geist_sampler_top_p_ws, src/engine/sampler.c:232-305) and min-p, without a
+ * top-k in front. Included by sampler_kernels.hip.
+ *
+ * The reference normalises every probability, sorts all of them and walks the sorted list.
+ * Here nothing is sorted but the few entries that can matter:
+ *   fast path (in k_row_final)  thread maxima -> a logit bound below which nothing of the kept
+ *                               prefix can lie -> re-read the threads above it -> order those
+ *                               entries -> walk. Serves rows whose kept prefix is small.
+ *   general path (k_sorted_general)  for rows the fast path hands on: the normalised
+ *                               probabilities of the row are written once (k_write_probs), then
+ *                               a mass-weighted radix descent over their bit patterns finds the
+ *                               nucleus edge and the drawn entry without ordering anything.
+ */
+#ifndef GEIST_SAMPLER_SORTED_PROB_H
+#define GEIST_SAMPLER_SORTED_PROB_H
+
+namespace gs {
+
+/* Walk over n <= 64 * IPT entries already in walk order, on ONE wavefront: entry i carries
+ * its weight pn_i as the high word of spack[i] (fp32 bits; positive floats order like their
+ * bits) and its vocabulary id in the low word (complemented, as pack_best()).
+ * Nucleus: sampler.c:273-283; min-p: pn >= min_p * pn_0; draw: sampler.c:286-299.
+ * Returns the vocabulary id, or -1 when top_p is set, min_p is not, and the n entries do not
+ * reach top_p (the caller's bound was too tight). */
+template <int IPT>
+__device__ int finish_weights_wave(int n, const uint64_t *spack, float top_p, float min_p,
+                                   float u) {
+    const int  lane  = threadIdx.x & (WAVE - 1);
+    const bool use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool use_m = min_p > 0.0f;
+    float      w[IPT];
+    double     part = 0.0;
+#pragma unroll
+    for (int t = 0; t < IPT; ++t) {
+        const int i = IPT * lane + t;
+        w[t]        = i < n ? __uint_as_float(best_key(spack[i])) : 0.0f;
+        part += (double) w[t];
+    }
+    const double incl = wave_scan_f64_dpp(part);
+    double       c[IPT];
+    {
+        double run = incl - part;
+#pragma unroll
+        for (int t = 0; t < IPT; ++t) {
+            run += (double) w[t];
+            c[t] = run;
+        }
+    }
+    int keep = n;
+    if (use_p) {
+        int first = 0x7fffffff;
+#pragma unroll
+        for (int t = IPT - 1; t >= 0; --t) {
+            const uint64_t mk = __ballot(IPT * lane + t < n && c[t] >= (double) top_p);
+            if (mk) {
+                const int f = IPT * (__ffsll((long long) mk) - 1) + t;
+                first       = f < first ? f : first;
+            }
+        }
+        if (first != 0x7fffffff)
+            keep = first + 1;
+        else if (!use_m)
+            return -1;
+    }
+    if (use_m) {
+        const float floor_w = __fmul_rn(min_p, __shfl(w[0], 0, WAVE));
+        int         m       = 0;
+#pragma unroll
+        for (int t = 0; t < IPT; ++t)
+            m += __popcll(__ballot(IPT * lane + t < n && w[t] >= floor_w));
+        if (m < 1)
+            m = 1;
+        keep = m < keep ? m : keep;
+    }
+    if (keep < 1)
+        keep = 1;
+    double at_keep = c[0];
+#pragma unroll
+    for (int t = 1; t < IPT; ++t)
+        if (((keep - 1) % IPT) == t)
+            at_keep = c[t];
+    const double mass   = __shfl(at_keep, (keep - 1) / IPT, WAVE);
+    const double target = (double) u * mass;
+    int          at     = 0x7fffffff;
+#pragma unroll
+    for (int t = IPT - 1; t >= 0; --t) {
+        const uint64_t hk = __ballot(IPT * lane + t < keep && target < c[t]);
+        if (hk) {
+            const int f = IPT * (__ffsll((long long) hk) - 1) + t;
+            at          = f < at ? f : at;
+        }
+    }
+    if (at == 0x7fffffff)
+        at = keep - 1;
+    return (int) best_idx(spack[at]);
+}
+
+/* ============================================================================================
+ * sorted_from_tmax: fast path. `mx` is the row maximum, `sum` the row's double sum of
+ * expf((l - mx) * inv_t) (both from the streaming kernels). Steps:
+ *   1. thread maxima -> each thread of this workgroup keeps the largest of its KPT and its
+ *      normalised probability w;
+ *   2. top-p: the elements at or above a logit t weigh at least the sum of w over the threads
+ *      whose maximum is >= t (one distinct element each), so the largest t for which that sum
+ *      reaches top_p bounds the nucleus from below; found by a bitwise search on the key.
+ *      min-p: pn_i >= min_p * pn_0 needs (l_i - mx) * inv_t >= ln(min_p), a bound in closed
+ *      form (taken with slack). Both set: the kept prefix is the shorter one, so the larger
+ *      bound serves;
+ *   3. re-read the threads at or above the bound, transform, keep the entries above it with
+ *      their exact pn = (float)((double)p / sum) (sampler.c:251-253);
+ *   4. order by (pn descending, index ascending) (sampler.c:270) and walk.
+ * Returns the vocabulary id, or -1 when the row has to take the general path.
+ * ========================================================================================== */
+template <int NV, bool PEN, int KPT>
+__device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalArgs &a, int row,
+                                                float mx, double sum, float u_row, uint8_t *slot,
+                                                uint32_t *s_mx, float *s_wt, int *s_selid,
+                                                uint32_t *s_pcnt, uint64_t *s_m, uint64_t *s_srt,
+                                                int *s_n, int *s_n2, const uint64_t *tab) {
+    const int  tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int  C     = rv.n_chunks;
+    const bool use_p = a.top_p > 0.0f && a.top_p < 1.0f;
+    const bool use_m = a.min_p > 0.0f;
+    HistPrefetch pf;
+    if (PEN)
+        pf = history_prefetch(rv, row, (int) gridDim.x);
+    /* 1 */
+    const float *tm = a.tmax + (long) row * C * TPB + tid;
+    float        raw[KPT];
+#pragma unroll
+    for (int q = 0; q < KPT; ++q)
+        raw[q] = q < C ? tm[q * TPB] : __builtin_nanf("");
+    {
+        uint4 *z = reinterpret_cast<uint4 *>(slot);
+        for (int i = tid; i < KPT * TPB / 16; i += TPB)
+            z[i] = make_uint4(0u, 0u, 0u, 0u);
+        if (PEN) {
+            for (int i = tid; i < SEL_MAX * 4 * NV; i += TPB)
+                s_pcnt[i] = 0u;
+        }
+        if (tid == 0) {
+            *s_n  = 0;
+            *s_n2 = 0;
+        }
+    }
+    float mxf = __builtin_nanf("");
+#pragma unroll
+    for (int q = 0; q + 1 < KPT; q += 2)
+        mxf = max3f(mxf, raw[q], raw[q + 1]);
+    const uint32_t mkey = f2key(mxf);
+    float          wt   = 0.0f;
+    if (mkey)
+        wt = (float) ((double) geist_expf_glibc(softmax_arg(mxf, mx, a.inv_t), tab) / sum);
+    s_mx[tid] = mkey;
+    s_wt[tid] = wt;
+    __syncthreads();
+    /* 2 */
+    uint32_t key_lo = 0u;
+    if (use_p) {
+        const uint32_t k0 = s_mx[lane], k1 = s_mx[lane + 64], k2 = s_mx[lane + 128],
+                       k3 = s_mx[lane + 192];
+        const float w0 = s_wt[lane], w1 = s_wt[lane + 64], w2 = s_wt[lane + 128],
+                    w3 = s_wt[lane + 192];
+        /* fp32 sums of at most 256 terms: ask for a little more than top_p */
+        const float need = a.top_p * 1.0001f;
+        uint32_t    tau  = 0u;
+#pragma unroll 1
+        for (int bit = 31; bit >= 14; --bit) {
+            const uint32_t t = tau | (1u << bit);
+            float acc = (k0 >= t ? w0 : 0.f) + (k1 >= t ? w1 : 0.f) + (k2 >= t ? w2 : 0.f) +
+                        (k3 >= t ? w3 : 0.f);
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1)
+                acc += __shfl_xor(acc, m, WAVE);
+            if (acc >= need)
+                tau = t;
+        }
+        if (tau < 0x00800000u && !use_m)
+            return -1; /* the thread maxima alone do not weigh top_p: a wide nucleus */
+        key_lo = tau;
+    }
+    if (use_m) {
+        /* (l - mx) * inv_t >= ln(min_p) - slack  <=>  l >= mx + (ln(min_p) - slack) / inv_t */
+        const double   lg  = log((double) a.min_p) - 1e-3;
+        const float    t_m = (float) ((double) mx + lg / (double) a.inv_t - 1e-3 * fabs((double) mx));
+        const uint32_t km  = f2key(t_m);
+        key_lo             = km > key_lo ? km : key_lo;
+    }
+    if (key_lo < 0x00800000u)
+        return -1;
+    const float bound = key2f(key_lo);
+    /* 3 */
+    int cnt = 0;
+#pragma unroll
+    for (int q = 0; q < KPT; ++q)
+        cnt += raw[q] >= bound;
+    int pos = wave_reserve(cnt, s_n);
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+        if (raw[q] >= bound) {
+            if (pos < SEL_MAX) {
+                s_selid[pos]        = q * TPB + tid;
+                slot[q * TPB + tid] = (uint8_t) (pos + 1);
+            }
+            ++pos;
+        }
+    }
+    __syncthreads();
+    const int n_sel = *s_n;
+    if (n_sel > SEL_MAX)
+        return -1;
+    constexpr int TASKS = SEL_MAX * NV / TPB;
+    float4        r[TASKS];
+    int           e0[TASKS], e1[TASKS];
+    const float  *rowp = rv.logits + (long) row * rv.ld;
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+        const int t = tid + q * TPB;
+        const int s = t / NV, j = t % NV;
+        e0[q] = 0;
+        e1[q] = 0;
+        r[q]  = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (s < n_sel) {
+            const int L = s_selid[s];
+            const int chunk = L / TPB, tt = L % TPB;
+            int       base, end;
+            chunk_bounds<NV>(rv, chunk, base, end);
+            const int e = base + 4 * (j * TPB + tt);
+            e0[q] = e;
+            e1[q] = end;
+            if (rv.vec_ok && e + 3 < end) {
+                r[q] = *reinterpret_cast<const float4 *>(rowp + e);
+            } else {
+                r[q].x = e + 0 < end ? rowp[e + 0] : 0.f;
+                r[q].y = e + 1 < end ? rowp[e + 1] : 0.f;
+                r[q].z = e + 2 < end ? rowp[e + 2] : 0.f;
+                r[q].w = e + 3 < end ? rowp[e + 3] : 0.f;
+            }
+        }
+    }
+    if (PEN) {
+        const int shift = 31 - __clz(rv.per_chunk);
+        history_for_each(rv, row, pf, [&](int t) {
+            if (t < 0 || t >= rv.n_vocab)
+                return;
+            const int off = t & (rv.per_chunk - 1);
+            const int f   = off >> 2;
+            const int s   = slot[(t >> shift) * TPB + (f % TPB)];
+            if (s)
+                atomicAdd(&s_pcnt[((s - 1) * NV + f / TPB) * 4 + (off & 3)], 1u);
+        });
+        __syncthreads();
+    }
+    uint32_t ck[TASKS][4];
+    int      keep = 0;
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+        const int t = tid + q * TPB;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            ck[q][c] = 0u;
+            if (e0[q] + c < e1[q]) {
+                float x = f4_get(r[q], c);
+                if (PEN) {
+                    const uint32_t n_hist = s_pcnt[t * 4 + c];
+                    if (n_hist)
+                        x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
+                }
+                if (rv.softcap > 0.0f)
+                    x = __fmul_rn(tanhf(__fdiv_rn(x, rv.softcap)), rv.softcap);
+                if (x >= bound) {
+                    const float pn =
+                        (float) ((double) geist_expf_glibc(softmax_arg(x, mx, a.inv_t), tab) / sum);
+                    /* bit 31 marks the slot as taken even when pn underflows to 0 */
+                    ck[q][c] = __float_as_uint(pn) | 0x80000000u;
+                    ++keep;
+                }
+            }
+        }
+    }
+    pos = wave_reserve(keep, s_n2);
+#pragma unroll
+    for (int q = 0; q < TASKS; ++q) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (ck[q][c]) {
+                if (pos < TPB)
+                    s_m[pos] = pack_best(ck[q][c] & 0x7fffffffu, (uint32_t) (e0[q] + c));
+                ++pos;
+            }
+        }
+    }
+    __syncthreads();
+    const int m = *s_n2;
+    if (m > TPB || m < 1)
+        return -1;
+    /* 4: order by counting, entry i compared by P = 256 / m2 <= 64 neighbouring lanes */
+    int m2 = 4;
+    while (m2 < m)
+        m2 <<= 1;
+    const int P = TPB / m2, i = tid / P, part = tid % P;
+    uint64_t  me   = 0;
+    int       rank = 0;
+    if (i < m) {
+        me = s_m[i];
+#pragma unroll 4
+        for (int j = part; j < m; j += P)
+            rank += s_m[j] > me;
+    }
+    for (int d = 1; d < P; d <<= 1)
+        rank += __shfl_xor(rank, d, WAVE);
+    if (i < m && part == 0)
+        s_srt[rank] = me;
+    __syncthreads();
+    int tok = 0;
+    if (tid < WAVE) {
+        if (m <= WAVE)
+            tok = finish_weights_wave<1>(m, s_srt, a.top_p, a.min_p, u_row);
+        else if (m <= 2 * WAVE)
+            tok = finish_weights_wave<2>(m, s_srt, a.top_p, a.min_p, u_row);
+        else
+            tok = finish_weights_wave<4>(m, s_srt, a.top_p, a.min_p, u_row);
+    }
+    if (tid == 0)
+        *s_n = tok;
+    __syncthreads();
+    tok = *s_n;
+    __syncthreads();
+    return tok;
+}
+
+/* ============================================================================================
+ * k_sorted_general: rows the fast path handed on (row_flag != 0). One workgroup per row works
+ * on the row's normalised probabilities pn (written by k_write_probs).
+ *
+ * The sorted order of the reference (pn descending, equal pn by ascending index) is never
+ * materialised. A descent over the bit pattern of pn -- 11, 11 and 10 bits per level, each
+ * level one pass building a histogram of entry counts and of mass per digit -- finds the value
+ * kappa at which the running mass of the sorted list first reaches a target, the mass and count
+ * strictly above kappa, and how many of the entries equal to kappa are needed. Mass is summed
+ * in 2^-62 fixed point, so the result does not depend on the order of the atomic additions.
+ * Two descents: the nucleus edge (target top_p), then the draw (target u * kept mass). A last
+ * pass in index order finds the j-th entry equal to the drawn value.
+ * ========================================================================================== */
+constexpr int SG_BINS = 2048;
+
+struct SortedGenShared {
+    uint32_t cnt[SG_BINS];
+    uint64_t mass[SG_BINS];
+    uint64_t scan64[NWAVES];
+    uint32_t scan32[NWAVES];
+    uint64_t res_mass_above;
+    uint32_t res_cnt_above;
+    int      res_digit;
+    uint64_t red64[NWAVES];
+};
+
+__device__ __forceinline__ uint64_t pn_fx(float pn) {
+    return (uint64_t) __double2ull_rz((double) pn * 0x1p62);
+}
+
+__device__ __forceinline__ uint64_t block_sum_u64(uint64_t v, uint64_t *scratch) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        v += shfl_xor_u64(v, m);
+    if ((threadIdx.x & (WAVE - 1)) == 0)
+        scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    uint64_t r = 0;
+#pragma unroll
+    for (int w = 0; w < NWAVES; ++w)
+        r += scratch[w];
+    __syncthreads();
+    return r;
+}
+
+/* One descent. `limit_key`/`limit_ties`: only entries that precede the (limit_key, limit_ties)
+ * edge of a previous descent take part -- entries with key > limit_key, plus the first
+ * limit_ties (by index) of those equal to it, whose mass is limit_ties * fx(limit_key); pass
+ * limit_key = 0, limit_ties = 0 with `limited` false for no restriction.
+ * Out: kappa (key bits), cnt_above / mass_above (strictly greater keys), ties_total.
+ * Returns false when the whole (restricted) list weighs less than the target. */
+__device__ bool sg_descent(const float *pn, int n, uint64_t target, bool limited,
+                           uint32_t limit_key, uint32_t limit_ties, SortedGenShared &sh,
+                           uint32_t &kappa, uint32_t &cnt_above, uint64_t &mass_above,
+                           uint32_t &ties_total) {
+    const int tid    = threadIdx.x;
+    uint32_t  prefix = 0u, mask = 0u;
+    cnt_above  = 0u;
+    mass_above = 0ull;
+    ties_total = 0u;
+    const int shifts[3] = {21, 10, 0};
+    const int widths[3] = {11, 11, 10};
+    for (int lv = 0; lv < 3; ++lv) {
+        const int      shf = shifts[lv];
+        const uint32_t dm  = (1u << widths[lv]) - 1u;
+        for (int i = tid; i < SG_BINS; i += TPB) {
+            sh.cnt[i]  = 0u;
+            sh.mass[i] = 0ull;
+        }
+        __syncthreads();
+        for (int i = tid; i < n; i += TPB) {
+            const float    p   = pn[i];
+            const uint32_t key = __float_as_uint(p);
+            if ((key & mask) != prefix)
+                continue;
+            if (limited && key <= limit_key)
+                continue; /* entries equal to the limit are added below, as a block */
+            const uint32_t d = (key >> shf) & dm;
+            atomicAdd(&sh.cnt[d], 1u);
+            atomicAdd((unsigned long long *) &sh.mass[d], (unsigned long long) pn_fx(p));
+        }
+        if (limited && tid == 0 && limit_ties && (limit_key & mask) == prefix) {
+            const uint32_t d = (limit_key >> shf) & dm;
+            atomicAdd(&sh.cnt[d], limit_ties);
+            atomicAdd((unsigned long long *) &sh.mass[d],
+                      (unsigned long long) (pn_fx(__uint_as_float(limit_key)) * limit_ties));
+        }
+        __syncthreads();
+        /* thread t owns the 8 digits SG_BINS-1-8t .. SG_BINS-8-8t, i.e. descending order */
+        uint64_t lm = 0;
+        uint32_t lc = 0;
+#pragma unroll
+        for (int q = 0; q < SG_BINS / TPB; ++q) {
+            const int d = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
+            lm += sh.mass[d];
+            lc += sh.cnt[d];
+        }
+        /* exclusive prefix over threads (descending digits) */
+        uint64_t im = lm;
+        uint32_t ic = lc;
+        {
+            const int lane = tid & (WAVE - 1), w = tid / WAVE;
+#pragma unroll
+            for (int d = 1; d < WAVE; d <<= 1) {
+                const uint64_t om = ((uint64_t) (uint32_t) __shfl_up((int) (im >> 32), d, WAVE) << 32) |
+                                    (uint32_t) __shfl_up((int) (uint32_t) im, d, WAVE);
+                const uint32_t oc = (uint32_t) __shfl_up((int) ic, d, WAVE);
+                if (lane >= d) {
+                    im += om;
+                    ic += oc;
+                }
+            }
+            if (lane == WAVE - 1) {
+                sh.scan64[w] = im;
+                sh.scan32[w] = ic;
+            }
+            if (tid == 0)
+                sh.res_digit = -1;
+            __syncthreads();
+            for (int x = 0; x < w; ++x) {
+                im += sh.scan64[x];
+                ic += sh.scan32[x];
+            }
+        }
+        uint64_t run_m = mass_above + (im - lm);
+        uint32_t run_c = cnt_above + (ic - lc);
+#pragma unroll
+        for (int q = 0; q < SG_BINS / TPB; ++q) {
+            const int      d  = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
+            const uint64_t bm = sh.mass[d];
+            if (sh.cnt[d] && run_m < target && run_m + bm >= target) {
+                sh.res_digit      = d;
+                sh.res_mass_above = run_m;
+                sh.res_cnt_above  = run_c;
+            }
+            run_m += bm;
+            run_c += sh.cnt[d];
+        }
+        __syncthreads();
+        const int d = sh.res_digit;
+        if (d < 0)
+            return false;
+        mass_above = sh.res_mass_above;
+        cnt_above  = sh.res_cnt_above;
+        ties_total = sh.cnt[d];
+        prefix |= (uint32_t) d << shf;
+        mask |= dm << shf;
+        __syncthreads();
+    }
+    kappa = prefix;
+    return true;
+}
+
+__global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict__ probs,
+                                                        long ld_probs, int n, float top_p,
+                                                        float min_p,
+                                                        const float *__restrict__ uniforms,
+                                                        const int32_t *__restrict__ row_flag,
+                                                        int32_t *__restrict__ out) {
+    __shared__ SortedGenShared sh;
+    __shared__ int             s_scan[NWAVES];
+    __shared__ int             s_pick;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    if (!row_flag[row])
+        return;
+    const float *pn    = probs + (long) row * ld_probs;
+    const bool   use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool   use_m = min_p > 0.0f;
+
+    /* largest probability, then the min-p prefix: count and mass of pn >= min_p * pn_0 */
+    uint32_t kmax = 0u;
+    for (int i = tid; i < n; i += TPB) {
+        const uint32_t key = __float_as_uint(pn[i]);
+        kmax               = key > kmax ? key : kmax;
+    }
+    kmax = (uint32_t) block_max_u64((uint64_t) wave_max_u32(kmax), sh.red64);
+    uint32_t n_m    = (uint32_t) n;
+    uint64_t mass_m = 0;
+    if (use_m) {
+        const float floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
+        uint64_t    lm      = 0;
+        uint64_t    lc      = 0;
+        for (int i = tid; i < n; i += TPB) {
+            const float p = pn[i];
+            if (p >= floor_w) {
+                lm += pn_fx(p);
+                ++lc;
+            }
+        }
+        mass_m = block_sum_u64(lm, sh.red64);
+        n_m    = (uint32_t) block_sum_u64(lc, sh.red64);
+        if (n_m < 1u) { /* cannot happen (pn_0 >= min_p * pn_0 for min_p <= 1); keep the max */
+            n_m    = 1u;
+            mass_m = pn_fx(__uint_as_float(kmax));
+        }
+    }
+    /* nucleus edge */
+    bool     limited   = false;
+    uint32_t edge_key  = 0u, edge_ties = 0u;
+    uint64_t mass_keep = 0;
+    uint32_t n_keep    = (uint32_t) n;
+    bool     have_p    = false;
+    if (use_p) {
+        const uint64_t target = (uint64_t) __double2ull_ru((double) top_p * 0x1p62);
+        uint32_t       kappa, cnt_above, ties;
+        uint64_t       mass_above;
+        if (sg_descent(pn, n, target, false, 0u, 0u, sh, kappa, cnt_above, mass_above, ties)) {
+            const uint64_t each = pn_fx(__uint_as_float(kappa));
+            uint64_t       j    = each ? (target - mass_above + each - 1) / each : 1;
+            if (j < 1)
+                j = 1;
+            if (j > ties)
+                j = ties;
+            have_p    = true;
+            limited   = true;
+            edge_key  = kappa;
+            edge_ties = (uint32_t) j;
+            n_keep    = cnt_above + (uint32_t) j;
+            mass_keep = mass_above + each * j;
+        }
+    }
+    if (use_m && (!have_p || n_m < n_keep)) {
+        /* the min-p prefix is the shorter one: every entry with pn >= floor, ties included */
+        const float floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
+        limited   = true;
+        n_keep    = n_m;
+        mass_keep = mass_m;
+        /* as an edge: keys >= floor, i.e. key > floor_bits - 1 with no ties taken from there */
+        edge_key  = __float_as_uint(floor_w) ? __float_as_uint(floor_w) - 1u : 0u;
+        edge_ties = 0u;
+        if (__float_as_uint(floor_w) == 0u)
+            limited = false;
+    } else if (!have_p) {
+        /* neither filter bites (top_p not reached by the whole row): the whole row is kept */
+        uint64_t lm = 0;
+        for (int i = tid; i < n; i += TPB)
+            lm += pn_fx(pn[i]);
+        mass_keep = block_sum_u64(lm, sh.red64);
+        limited   = false;
+    }
+    /* the draw: first entry of the kept prefix at which the running mass exceeds u * mass */
+    /* running mass > u * mass  <=>  running mass >= floor(u * mass) + 1 in integers */
+    const uint64_t target2 =
+        (uint64_t) __double2ull_rd((double) uniforms[row] * (double) mass_keep) + 1ull;
+    uint32_t       kd, cnt_above_d, ties_d;
+    uint64_t       mass_above_d;
+    int32_t        tok = -1;
+    if (sg_descent(pn, n, target2, limited, edge_key, edge_ties, sh, kd, cnt_above_d,
+                   mass_above_d, ties_d)) {
+        const uint64_t each = pn_fx(__uint_as_float(kd));
+        uint64_t       j    = each ? (target2 - mass_above_d + each - 1) / each : 1;
+        if (j < 1)
+            j = 1;
+        if (j > ties_d)
+            j = ties_d;
+        /* the j-th entry (index order) with pn == kd: each thread takes a contiguous range */
+        const int span = (n + TPB - 1) / TPB;
+        const int lo   = tid * span < n ? tid * span : n;
+        const int hi   = lo + span < n ? lo + span : n;
+        int       mine = 0;
+        for (int i = lo; i < hi; ++i)
+            mine += __float_as_uint(pn[i]) == kd;
+        const int incl = block_scan_i32(mine, s_scan, nullptr);
+        if (tid == 0)
+            s_pick = -1;
+        __syncthreads();
+        if (incl >= (int) j && incl - mine < (int) j) {
+            int seen = incl - mine;
+            for (int i = lo; i < hi; ++i) {
+                if (__float_as_uint(pn[i]) == kd && ++seen == (int) j) {
+                    s_pick = i;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        tok = s_pick;
+    }
+    if (tok < 0) {
+        /* not reachable with exact integer masses (the target never exceeds the kept mass);
+         * kept as a defined outcome: the most probable entry */
+        if (tid == 0)
+            s_pick = 0x7fffffff;
+        __syncthreads();
+        for (int i = tid; i < n; i += TPB)
+            if (__float_as_uint(pn[i]) == kmax)
+                atomicMin(&s_pick, i);
+        __syncthreads();
+        tok = s_pick == 0x7fffffff ? 0 : s_pick;
+    }
+    if (tid == 0)
+        out[row] = tok;
+    (void) n_keep;
+}
+
+} // namespace gs
+#endif

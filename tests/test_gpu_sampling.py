@@ -176,6 +176,67 @@ def test_reference_precedence_ignores_top_p_when_top_k_set(hs, oracle):
     assert got.tolist() == want
 
 
+# ------------------------------------------------------------ top-p / min-p, whole vocabulary
+def test_top_p_reference_unit_vector(hs, oracle):
+    # tests/test_sampler_unit.c:115-131: top_p = 0.5 on {10, 0, 0, 0, 0} -> index 0 nearly always
+    from geistlib_amd.workloads import xorshift_units
+    row = np.array([10, 0, 0, 0, 0], dtype=np.float32)
+    u, _ = xorshift_units(13, 128)
+    got = run_rows(hs, torch, np.tile(row, (128, 1)), u, P(temperature=1.0, top_p=0.5, precedence=0))
+    want = [oracle.top_p_u(row, 0.5, 1.0, float(v))[0] for v in u]
+    assert got.tolist() == want and got.tolist().count(0) > 120
+
+
+@pytest.mark.parametrize("n,scale,T,p", [(5, 3.0, 1.0, 0.5), (300, 6.0, 0.7, 0.9),
+                                         (5000, 6.0, 0.7, 0.9), (128256, 5.0, 0.7, 0.9),
+                                         (128256, 6.0, 0.7, 0.95), (262144, 6.0, 0.6, 0.9)])
+def test_top_p_peaked_rows(hs, oracle, n, scale, T, p):
+    """Small nuclei: served from the thread maxima."""
+    print(f"top-p peaked n={n} p={p}", flush=True)
+    x, u = rows_rng(n + 7, 12, n, scale=scale)
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_p=p, precedence=0))
+    res = [oracle.top_p_u(x[r], p, T, float(u[r])) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-p n={n}")
+    assert near <= 1
+
+
+@pytest.mark.parametrize("n,scale,T,p", [(64, 1.0, 1.0, 0.9), (5000, 1.0, 1.0, 0.9),
+                                         (40000, 2.0, 1.0, 0.95), (128256, 2.0, 0.7, 0.9),
+                                         (151936, 2.0, 1.0, 0.3), (9000, 0.0, 1.0, 0.37)])
+def test_top_p_wide_nucleus_general_path(hs, oracle, n, scale, T, p):
+    """Nuclei of thousands of entries (flat rows, the all-equal row): the radix descent."""
+    print(f"top-p wide n={n} p={p}", flush=True)
+    x, u = rows_rng(n + 11, 6, n, scale=scale)
+    x[1] = np.round(x[1] * 8) / 8          # many equal probabilities: index order among them
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_p=p, precedence=0))
+    res = [oracle.top_p_u(x[r], p, T, float(u[r])) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-p wide n={n}")
+    assert near <= 1
+
+
+@pytest.mark.parametrize("n,scale,T,p,m", [(2000, 2.0, 1.0, 1.0, 0.05), (128256, 2.0, 1.0, 0.95, 0.05),
+                                           (151936, 2.0, 1.0, 0.95, 0.05), (50000, 1.0, 1.0, 1.0, 0.5),
+                                           (50000, 2.0, 0.8, 0.5, 0.001), (50000, 1.0, 1.0, 0.9, 1e-6)])
+def test_min_p_and_top_p_chain(hs, oracle, n, scale, T, p, m):
+    print(f"min-p n={n} p={p} m={m}", flush=True)
+    x, u = rows_rng(n + 13, 8, n, scale=scale)
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_p=p, min_p=m))
+    res = [oracle.chain_u(x[r], float(u[r]), temperature=T, top_p=p, min_p=m)
+           for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"min-p n={n}")
+    assert near <= 1
+
+
+def test_top_p_limits_match_reference_dispatch(hs, oracle):
+    x, u = rows_rng(5, 6, 3000)
+    for p in (0.0, -1.0, 1.0, 1.5):        # sampler.c:238-243: <= 0 -> argmax... but the session
+        got = run_rows(hs, torch, x, u, P(temperature=0.8, top_p=p, precedence=0))
+        # ...maps top_p <= 0 to 1.0 (step.c:391) and the dispatch (head.c:177) sends p >= 1 to the
+        # temperature sampler; the C ABI takes the session's view
+        want = [oracle.temperature_u(x[r], 0.8, float(u[r]))[0] for r in range(6)]
+        assert got.tolist() == want
+
+
 # ------------------------------------------------------------------------------ penalties
 def test_penalties_in_place_match_oracle(hs, oracle):
     g = np.random.default_rng(5)
