@@ -27,6 +27,7 @@ struct geist_hip_sampler {
     /* device workspace */
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
+    double   *resid_sum  = nullptr; /* [max_rows][max_chunks] spec verification */
     float    *tmax       = nullptr; /* [max_rows][max_chunks][256] per-thread maxima */
     int32_t  *row_flag   = nullptr; /* [max_rows] */
     float    *uniforms   = nullptr; /* [max_rows] */
@@ -181,6 +182,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     hipError_t   e  = hipSetDevice(device);
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->tmax, rc * 256 * sizeof(float));
     if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
@@ -203,6 +205,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipStreamSynchronize(s->stream);
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
+    (void) hipFree(s->resid_sum);
     (void) hipFree(s->tmax);
     (void) hipFree(s->row_flag);
     (void) hipFree(s->uniforms);
@@ -357,7 +360,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (!rs.use_p && !rs.use_m) {
         launch_tmax_scan(L, s->tmax, s->chunk_best);
         mark_start(s);
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
         mark_stop(s);
         f.mode = FINAL_TEMPERATURE;
         launch_row_final(L, f);
@@ -374,7 +377,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                     rows->n_vocab, s->max_chunks);
     launch_tmax_scan(L, s->tmax, s->chunk_best);
     mark_start(s);
-    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
     mark_stop(s);
     f.mode     = FINAL_SORTED;
     f.row_flag = s->row_flag;
@@ -485,15 +488,64 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
     launch_tmax_scan(L, s->tmax, s->chunk_best);
-    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, nullptr);
+    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
 }
 
-int geist_hip_spec_verify(geist_hip_sampler *s, const float *, size_t, const float *, size_t,
-                          const int32_t *, const float *, size_t, size_t, size_t, float,
-                          geist_hip_token_t *, int32_t *) {
-    return fail(s, GEIST_HIP_E_UNSUPPORTED, "speculative verification is not built yet");
+int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
+                          const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
+                          const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,
+                          float temperature, geist_hip_token_t *d_out_tokens,
+                          int32_t *d_n_accepted) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_target || !d_draft || !d_out_tokens || !d_n_accepted)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_seq == 0 || L == 0 || L > (size_t) SPEC_DRAFT_MAX)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "n_seq %zu, draft length %zu (1..%d)", n_seq, L,
+                    SPEC_DRAFT_MAX);
+    const bool greedy = !(temperature > 0.0f);
+    if (!greedy && (!d_draft_q || !d_uniforms))
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic verification needs q and uniforms");
+    if (!greedy && ld_q < n_vocab)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_q < n_vocab");
+    struct geist_hip_rows r{};
+    r.d_logits = d_target;
+    r.ld       = ld_t;
+    r.rows     = n_seq * (L + 1);
+    r.n_vocab  = n_vocab;
+    struct geist_hip_sample_params p{};
+    p.temperature        = temperature;
+    p.repetition_penalty = 1.0f;
+    Launch La;
+    int    rc = make_launch(s, &r, &p, false, La);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    const float inv_t = greedy ? 1.0f : 1.0f / temperature;
+    mark_start(s);
+    launch_tmax_scan(La, s->tmax, s->chunk_best);
+    mark_stop(s);
+    if (!greedy)
+        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p);
+    SpecLaunch sp{};
+    sp.n_seq      = (int) n_seq;
+    sp.L          = (int) L;
+    sp.greedy     = greedy ? 1 : 0;
+    sp.inv_t      = inv_t;
+    sp.q          = d_draft_q;
+    sp.ld_q       = (long) ld_q;
+    sp.draft      = d_draft;
+    sp.uniforms   = d_uniforms;
+    sp.chunk_best = s->chunk_best;
+    sp.chunk_sum  = s->chunk_sum;
+    sp.probe_p    = s->probe_p;
+    sp.resid_sum  = s->resid_sum;
+    sp.out_tokens = d_out_tokens;
+    sp.n_accepted = d_n_accepted;
+    launch_spec(La, sp);
+    return after_launch(s, "spec verification");
 }
 
 /* ---- device-memory helpers ----------------------------------------------------------------- */

@@ -52,8 +52,28 @@ struct FinalLaunch {
     int32_t        *row_flag;
 };
 
+/* probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
+ * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                         double *chunk_sum, const int32_t *probe_token, float *probe_p);
+                         double *chunk_sum, const int32_t *probe_token, int probe_L,
+                         float *probe_p);
+
+struct SpecLaunch {
+    int             n_seq, L, greedy;
+    float           inv_t;
+    const float    *q;
+    long            ld_q;
+    const int32_t  *draft;
+    const float    *uniforms;
+    const uint64_t *chunk_best;
+    const double   *chunk_sum;
+    const float    *probe_p;
+    double         *resid_sum;
+    int32_t        *out_tokens;
+    int32_t        *n_accepted;
+};
+constexpr int SPEC_DRAFT_MAX = 63;
+void launch_spec(const Launch &L, const SpecLaunch &sp);
 /* chunk_best may be NULL when only the thread maxima are wanted */
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best);
 void launch_row_final(const Launch &L, const FinalLaunch &f);

@@ -10,6 +10,7 @@
  *   k_sorted_general full-vocabulary top-p / min-p by mass-weighted radix descent sampler.c:246-304
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
  *   k_penalties      in-place penalties                                       (no reference counterpart)
+ *   k_spec_resid, k_spec_final   speculative-decode verification              (no reference counterpart)
  *   k_rng_units      xorshift64* uniforms                                     sampler.c:35-48
  *
  * All streaming kernels use a (n_chunks, rows) grid of 256-thread workgroups and read each
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       const uint64_t *__restrict__ chunk_best,
                                                       double *__restrict__ chunk_sum,
                                                       const int32_t *__restrict__ probe_token,
-                                                      float *__restrict__ probe_p) {
+                                                      int probe_L, float *__restrict__ probe_p) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
@@ -101,7 +102,13 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
     const float mx = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
 
-    const int tok = probe_token ? probe_token[row] : -1;
+    /* spec verification: target row s*(L+1)+j is probed at draft token j of sequence s */
+    int tok = -1;
+    if (probe_token) {
+        const int j = row % (probe_L + 1);
+        if (j < probe_L)
+            tok = probe_token[(long) (row / (probe_L + 1)) * probe_L + j];
+    }
     double    acc = 0.0;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -790,6 +797,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 
 } // namespace gs
 #include "sampler_sorted_prob.h"
+#include "sampler_spec.h"
 namespace gs {
 
 /* ============================================================================================
@@ -1106,12 +1114,42 @@ static void dispatch(int nv, bool pen, F &&f) {
 #define GS_PEN decltype(pen)::value
 
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                         double *chunk_sum, const int32_t *probe_token, float *probe_p) {
+                         double *chunk_sum, const int32_t *probe_token, int probe_L,
+                         float *probe_p) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_chunk_expsum<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, inv_t, chunk_best,
-                                                                    chunk_sum, probe_token, probe_p);
+        k_chunk_expsum<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
+            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p);
     });
+}
+
+void launch_spec(const Launch &L, const SpecLaunch &sp) {
+    SpecArgs a;
+    a.L          = sp.L;
+    a.greedy     = sp.greedy;
+    a.inv_t      = sp.inv_t;
+    a.q          = sp.q;
+    a.ld_q       = sp.ld_q;
+    a.draft      = sp.draft;
+    a.uniforms   = sp.uniforms;
+    a.chunk_best = sp.chunk_best;
+    a.chunk_sum  = sp.chunk_sum;
+    a.probe_p    = sp.probe_p;
+    a.resid_sum  = sp.resid_sum;
+    a.out_tokens = sp.out_tokens;
+    a.n_accepted = sp.n_accepted;
+    const dim3 block(TPB);
+    if (!sp.greedy) {
+        const dim3 grid(L.rv.n_chunks, sp.n_seq);
+        if (L.nv == 8)
+            k_spec_resid<8><<<grid, block, 0, L.stream>>>(L.rv, a);
+        else
+            k_spec_resid<2><<<grid, block, 0, L.stream>>>(L.rv, a);
+    }
+    if (L.nv == 8)
+        k_spec_final<8><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a);
+    else
+        k_spec_final<2><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a);
 }
 
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best) {

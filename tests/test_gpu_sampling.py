@@ -317,6 +317,85 @@ def test_normalised_probabilities(hs, oracle, n, T):
         assert np.max(np.abs(got[r] - want) / np.maximum(want, 1e-38)) < 2e-7
 
 
+# ------------------------------------------------------------------- speculative verify
+def _spec_case(seed, n_seq, L, n, sigma=0.5):
+    g = np.random.default_rng(seed)
+    target = (g.standard_normal((n_seq, L + 1, n)) * 2).astype(np.float32)
+    noisy = target[:, :L, :].astype(np.float64) + g.standard_normal((n_seq, L, n)) * sigma
+    noisy -= noisy.max(axis=-1, keepdims=True)
+    e = np.exp(noisy)
+    q = (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+    cdf = np.cumsum(q.astype(np.float64), axis=-1)
+    pick = g.random((n_seq, L, 1)) * cdf[..., -1:]
+    draft = np.minimum((cdf < pick).sum(axis=-1), n - 1).astype(np.int32)
+    u = (g.integers(0, 1 << 24, (n_seq, L + 1)) / np.float32(1 << 24)).astype(np.float32)
+    return target, q, draft, u
+
+
+def _run_spec(hs, target, q, draft, u, T):
+    n_seq, lp1, n = target.shape
+    out = torch.full((n_seq, lp1), -9, dtype=torch.int32, device="cuda")
+    nacc = torch.full((n_seq,), -9, dtype=torch.int32, device="cuda")
+    hs.spec_verify(to_dev(target, torch), to_dev(q, torch), to_dev(draft, torch), to_dev(u, torch),
+                   T, out, nacc)
+    hs.sync()
+    return nacc.cpu().numpy(), out.cpu().numpy()
+
+
+@pytest.mark.parametrize("n_seq,L,n,T", [(6, 4, 5000, 1.0), (5, 8, 20000, 0.8), (4, 8, 128256, 1.0),
+                                         (3, 1, 300, 1.3), (8, 3, 8193, 1.0)])
+def test_spec_verify_matches_oracle(hs, oracle, n_seq, L, n, T):
+    print(f"spec n_seq={n_seq} L={L} n={n}", flush=True)
+    target, q, draft, u = _spec_case(n_seq * 100 + L, n_seq, L, n)
+    nacc, out = _run_spec(hs, target, q, draft, u, T)
+    seen = set()
+    for s in range(n_seq):
+        want_n, want = oracle.spec_verify(target[s], q[s], draft[s], u[s], T)
+        assert nacc[s] == want_n, (s, nacc[s], want_n)
+        assert out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), (s, out[s], want)
+        assert np.all(out[s, want_n + 1:] == -9)       # the rest stays untouched
+        seen.add(want_n)
+    print("  accepted lengths seen:", sorted(seen))
+
+
+def test_spec_verify_special_cases(hs, oracle):
+    n_seq, L, n = 4, 5, 7000
+    target, q, draft, u = _spec_case(77, n_seq, L, n)
+    # q == p: everything is accepted whatever the uniforms; the bonus is a temperature draw
+    pn = np.stack([[oracle.softmax_normalised(target[s, j], 1.0)[0] for j in range(L)]
+                   for s in range(n_seq)]).astype(np.float32)
+    u_hi = np.full_like(u, np.float32(1 - 2.0 ** -24))
+    u_hi[:, L] = u[:, L]
+    nacc, out = _run_spec(hs, target, pn, draft, u_hi, 1.0)
+    assert nacc.tolist() == [L] * n_seq
+    for s in range(n_seq):
+        assert out[s, :L].tolist() == draft[s].tolist()
+        assert out[s, L] == oracle.temperature_u(target[s, L], 1.0, float(u[s, L]))[0]
+    # a draft that put all its mass on a token the target gives nothing: reject at once,
+    # and the residual is the target distribution itself
+    q2 = np.zeros_like(q)
+    t2 = target.copy()
+    t2[:, 0, 11] = -300.0
+    q2[:, :, 11] = 1.0
+    d2 = np.full_like(draft, 11)
+    nacc, out = _run_spec(hs, t2, q2, d2, u, 1.0)
+    assert nacc.tolist() == [0] * n_seq
+    for s in range(n_seq):
+        want_n, want = oracle.spec_verify(t2[s], q2[s], d2[s], u[s], 1.0)
+        assert want_n == 0 and out[s, 0] == want[0]
+    # greedy: exact-match prefix (src/engine/session.c:599-606 of the reference)
+    am = np.array([[oracle.argmax(target[s, j]) for j in range(L + 1)] for s in range(n_seq)],
+                  dtype=np.int32)
+    d3 = am[:, :L].copy()
+    d3[1, 2] = (d3[1, 2] + 1) % n
+    d3[2, 0] = (d3[2, 0] + 1) % n
+    nacc, out = _run_spec(hs, target, q, d3, u, 0.0)
+    assert nacc.tolist() == [L, 2, 0, L]
+    for s in range(n_seq):
+        k = nacc[s]
+        assert out[s, :k].tolist() == d3[s, :k].tolist() and out[s, k] == am[s, k]
+
+
 # ---------------------------------------------------------------------------------- rng
 def test_device_rng_matches_reference_stream(hs, oracle):
     from geistlib_amd import HipSampler
