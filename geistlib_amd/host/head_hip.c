@@ -1,0 +1,152 @@
+/*
+ * head_hip.c -- sampler state of a session and the sampler dispatch of the output head, for
+ * logits resident in device memory (C23). See include/geist_head_hip.h for the map onto the
+ * reference's functions.
+ */
+#include "geist_head_hip.h"
+#include "geist_sampler_hip.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+struct geist_hip_head {
+    /* src/archs/transformer/arch_state.h:287-294 */
+    float    temperature;
+    float    top_p;
+    int      top_k;
+    float    logit_softcap;
+    size_t   vocab;
+    size_t   m_max;
+    geist_hip_sampler *hs;
+    uint64_t *d_rng;   /* the session's struct geist_rng, in device memory */
+    int32_t  *d_tokens; /* m_max */
+    char      err[256];
+};
+
+static int head_fail(struct geist_hip_head *h, int code, const char *what) {
+    if (h != nullptr)
+        snprintf(h->err, sizeof h->err, "%s: %s", what,
+                 h->hs != nullptr ? geist_hip_sampler_last_error(h->hs) : "");
+    return code;
+}
+
+static int seed_rng(struct geist_hip_head *h, uint64_t seed) {
+    /* geist_rng_seed, src/engine/sampler.c:27-33 */
+    const uint64_t state = seed != 0 ? seed : UINT64_C(0x9E3779B97F4A7C15);
+    return geist_hip_upload(h->hs, h->d_rng, &state, sizeof state);
+}
+
+int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_softcap,
+                          void *stream, struct geist_hip_head **out) {
+    if (out == nullptr || vocab == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    *out                     = nullptr;
+    struct geist_hip_head *h = calloc(1, sizeof *h);
+    if (h == nullptr)
+        return GEIST_HIP_E_OOM;
+    h->vocab         = vocab;
+    h->m_max         = m_max != 0 ? m_max : 64; /* include/geist.h:244-246 */
+    h->logit_softcap = logit_softcap;
+    /* sampler defaults: greedy (arch_state.c:1168-1171) */
+    h->temperature = 0.0f;
+    h->top_p       = 1.0f;
+    h->top_k       = 0;
+    int rc         = geist_hip_sampler_create(device, h->m_max, vocab, stream, &h->hs);
+    void *p        = nullptr;
+    if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(h->hs, sizeof(uint64_t), &p)) == GEIST_HIP_OK)
+        h->d_rng = p;
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        h->d_tokens = p;
+    /* arch_state.c:1173: the default seed */
+    if (rc == GEIST_HIP_OK)
+        rc = seed_rng(h, UINT64_C(0xCAFEBABE1234));
+    if (rc != GEIST_HIP_OK) {
+        geist_hip_head_destroy(h);
+        return rc;
+    }
+    *out = h;
+    return GEIST_HIP_OK;
+}
+
+void geist_hip_head_destroy(struct geist_hip_head *h) {
+    if (h == nullptr)
+        return;
+    if (h->hs != nullptr) {
+        geist_hip_free(h->hs, h->d_rng);
+        geist_hip_free(h->hs, h->d_tokens);
+        geist_hip_sampler_destroy(h->hs);
+    }
+    free(h);
+}
+
+const char *geist_hip_head_errmsg(const struct geist_hip_head *h) { return h ? h->err : ""; }
+
+int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_session_opts *opts) {
+    if (h == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (opts == nullptr)
+        return GEIST_HIP_OK; /* geist_session_create with NULL opts: greedy defaults stay */
+    /* step.c:390-396 */
+    h->temperature = opts->temperature;
+    h->top_p       = opts->top_p > 0.0f ? opts->top_p : 1.0f;
+    h->top_k       = opts->top_k;
+    if (opts->random_seed != 0 && seed_rng(h, opts->random_seed) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "seeding the device RNG");
+    /* step.c:398-409 sizes the host workspace here; the device workspace was sized at create */
+    return GEIST_HIP_OK;
+}
+
+static int finalize(struct geist_hip_head *h, const float *d_logits, size_t k, int32_t *out) {
+    if (h == nullptr || d_logits == nullptr || out == nullptr || k == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (k > h->m_max)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
+    const struct geist_hip_rows rows = {
+        .d_logits = d_logits, .ld = h->vocab, .rows = k, .n_vocab = h->vocab};
+    /* head.c:172-183 / 291-302: T == 0 -> argmax; top_k > 1 -> top-k; 0 < top_p < 1 -> top-p;
+     * else temperature. Rows in order, one shared RNG (head.c:274-304). */
+    const struct geist_hip_sample_params prm = {.temperature        = h->temperature,
+                                                .top_p              = h->top_p,
+                                                .top_k              = h->top_k,
+                                                .repetition_penalty = 1.0f,
+                                                .logit_softcap      = h->logit_softcap,
+                                                .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
+    if (geist_hip_sample_rows_rng(h->hs, &rows, &prm, h->d_rng, /*shared=*/1, h->d_tokens) !=
+        GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "sampling");
+    if (geist_hip_download(h->hs, out, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
+    for (size_t r = 0; r < k; r++) /* head.c:137-139: an id outside the vocabulary is an error */
+        if (out[r] < 0 || (size_t) out[r] >= h->vocab)
+            return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_finalize_one_row(struct geist_hip_head *h, const float *d_logits,
+                                    int32_t *out_token) {
+    return finalize(h, d_logits, 1, out_token);
+}
+
+int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logits, size_t k,
+                                  int32_t *out_tokens) {
+    return finalize(h, d_logits, k, out_tokens);
+}
+
+int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,
+                              int32_t *out_index) {
+    if (h == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (n > h->vocab) /* geist_backend.h:322-326: outside the probed geometry */
+        return head_fail(h, GEIST_HIP_E_UNSUPPORTED, "row longer than the probed vocabulary");
+    if (geist_hip_argmax_f32(h->hs, d_logits, n, out_index) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "argmax");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_rng_state(struct geist_hip_head *h, uint64_t *state) {
+    if (h == nullptr || state == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    return geist_hip_download(h->hs, state, h->d_rng, sizeof *state);
+}

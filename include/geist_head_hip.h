@@ -1,0 +1,69 @@
+/*
+ * geist_head_hip.h -- the sampler side of the reference's output head, for logits that stay on
+ * the device. Mirrors, function for function, what src/archs/transformer/forward/head.c and
+ * step.c do between "the lm_head wrote [k, vocab] logits into scratch_logits" and "token ids":
+ *
+ *   geist_hip_head_create          sampler defaults of transformer_session_alloc
+ *                                  (src/archs/transformer/arch_state.c:1168-1173)
+ *   geist_hip_head_apply_opts      transformer_session_apply_opts (forward/step.c:385-411)
+ *   geist_hip_head_finalize_one_row   sampler part of finalize_logits_one_row (head.c:131-188)
+ *   geist_hip_head_finalize_batch     sampler part of finalize_logits_batch (head.c:274-304)
+ *   geist_hip_head_argmax_f32      the backend slot fused->argmax_f32
+ *                                  (include/geist_backend.h:414-421)
+ *
+ * The RNG state of the session lives in device memory and advances there, one draw per
+ * stochastic row in row order, exactly as the reference's single host RNG does.
+ */
+#ifndef GEIST_HEAD_HIP_H
+#define GEIST_HEAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef GEIST_VERSION_MAJOR /* the reference's <geist.h> is not in this translation unit */
+/* Layout of struct geist_session_opts, include/geist.h:209-247. */
+struct geist_session_opts {
+    size_t      max_seq_len;
+    float       temperature;
+    float       top_p;
+    int         top_k;
+    uint64_t    random_seed;
+    const char *awq_scales_path;
+    int         kv_mode; /* enum geist_kv_mode */
+    size_t      m_max;
+};
+#endif
+
+struct geist_hip_head;
+
+/* `vocab` logits per row, at most `m_max` rows per batch call (0 = 64, the reference's default,
+ * include/geist.h:244-246). `logit_softcap` is the model's soft-cap (0 = none), applied only
+ * when temperature > 0 (head.c:148-149). Returns a geist_status value. */
+int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_softcap,
+                          void *stream, struct geist_hip_head **out);
+void geist_hip_head_destroy(struct geist_hip_head *h);
+const char *geist_hip_head_errmsg(const struct geist_hip_head *h);
+
+/* opts == NULL keeps the greedy defaults (geist_session_create's NULL opts). */
+int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_session_opts *opts);
+
+/* d_logits: [1, vocab] / [k, vocab] fp32 in device memory, row stride vocab. Synchronous: the
+ * token ids are in host memory on return, as in the reference. */
+int geist_hip_head_finalize_one_row(struct geist_hip_head *h, const float *d_logits,
+                                    int32_t *out_token);
+int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logits, size_t k,
+                                  int32_t *out_tokens);
+int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,
+                              int32_t *out_index);
+
+/* Current RNG state (for tests and for handing a session over). */
+int geist_hip_head_rng_state(struct geist_hip_head *h, uint64_t *state);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GEIST_HEAD_HIP_H */

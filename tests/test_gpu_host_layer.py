@@ -1,0 +1,259 @@
+"""The C23 host layer on a GPU: the reference's sampler symbols served by the HIP path, and the
+session/head mirror. The checks restate the reference's tests/test_sampler_unit.c (eight checks)
+and the model-free part of its session sampling tests; where the reference's own unit-test binary
+was built against this library (oracle/_ref/test_sampler_unit_hip) it is run as well."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+c_float_p = C.POINTER(C.c_float)
+
+
+class Rng(C.Structure):
+    _fields_ = [("state", C.c_uint64)]
+
+
+class Ws(C.Structure):
+    _fields_ = [("probs", c_float_p), ("n_vocab", C.c_size_t)]
+
+
+class SessionOpts(C.Structure):
+    _fields_ = [("max_seq_len", C.c_size_t), ("temperature", C.c_float), ("top_p", C.c_float),
+                ("top_k", C.c_int), ("random_seed", C.c_uint64), ("awq_scales_path", C.c_char_p),
+                ("kv_mode", C.c_int), ("m_max", C.c_size_t)]
+
+
+@pytest.fixture(scope="module")
+def host():
+    lib = C.CDLL(os.path.join(ROOT, "geistlib_amd", "lib", "libgeist_sampler_host.so"))
+    lib.geist_rng_next_u64.restype = C.c_uint64
+    lib.geist_rng_next_unit.restype = C.c_float
+    lib.geist_sampler_argmax.argtypes = [C.c_size_t, c_float_p]
+    lib.geist_sampler_temperature.argtypes = [C.c_size_t, c_float_p, C.c_float, C.POINTER(Rng)]
+    lib.geist_sampler_workspace_init.argtypes = [C.POINTER(Ws), C.c_size_t]
+    lib.geist_sampler_workspace_destroy.argtypes = [C.POINTER(Ws)]
+    lib.geist_sampler_top_k_ws.argtypes = [C.POINTER(Ws), c_float_p, C.c_int, C.c_float,
+                                           C.POINTER(Rng)]
+    lib.geist_sampler_top_p_ws.argtypes = [C.POINTER(Ws), c_float_p, C.c_float, C.c_float,
+                                           C.POINTER(Rng)]
+    lib.geist_hip_head_create.argtypes = [C.c_int, C.c_size_t, C.c_size_t, C.c_float, C.c_void_p,
+                                          C.POINTER(C.c_void_p)]
+    lib.geist_hip_head_destroy.argtypes = [C.c_void_p]
+    lib.geist_hip_head_errmsg.restype = C.c_char_p
+    lib.geist_hip_head_errmsg.argtypes = [C.c_void_p]
+    lib.geist_hip_head_apply_opts.argtypes = [C.c_void_p, C.POINTER(SessionOpts)]
+    lib.geist_hip_head_finalize_one_row.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int32)]
+    lib.geist_hip_head_finalize_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
+                                                  C.POINTER(C.c_int32)]
+    lib.geist_hip_head_argmax_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
+                                              C.POINTER(C.c_int32)]
+    lib.geist_hip_head_rng_state.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
+    return lib
+
+
+def fp(a):
+    return a.ctypes.data_as(c_float_p)
+
+
+def f32(*v):
+    return np.array(v, dtype=np.float32)
+
+
+def test_reference_unit_test_binary_on_the_hip_path():
+    exe = os.path.join(ROOT, "oracle", "_ref", "test_sampler_unit_hip")
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is mounted (make -C oracle ref)")
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "PASS: all 8 sampler checks" in r.stdout
+    # check 4 is bit-deterministic (expf(0) == 1): the counts the reference prints
+    assert "[997 1055 979 999 970]" in r.stdout
+
+
+def test_eight_reference_checks(host, oracle):
+    # 1 (tests/test_sampler_unit.c:33-37)
+    x = f32(-1, 2, .5, 3, 3, -.5)
+    assert host.geist_sampler_argmax(6, fp(x)) == 3
+    # 2 (40-51)
+    rng = Rng()
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(42))
+    x = f32(0, 0, 0, 10, 0)
+    hits = sum(host.geist_sampler_temperature(5, fp(x), 0.1, C.byref(rng)) == 3 for _ in range(1000))
+    assert hits > 990
+    # 3 (54-60): greedy, and no draw consumed
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(1))
+    x = f32(1, 2, 3, .5)
+    assert host.geist_sampler_temperature(4, fp(x), 0.0, C.byref(rng)) == 2
+    assert rng.state == 1
+    # 4 (63-89): exact counts
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(7))
+    x = np.zeros(5, dtype=np.float32)
+    counts = [0] * 5
+    for _ in range(5000):
+        counts[host.geist_sampler_temperature(5, fp(x), 1.0, C.byref(rng))] += 1
+    assert counts == [997, 1055, 979, 999, 970]
+    # 5 (92-112)
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(11))
+    x = f32(0, 1, 4, 2, 5, 1.5, 0, .5)
+    ws = Ws()
+    assert host.geist_sampler_workspace_init(C.byref(ws), 8) == 0
+    seen = set(host.geist_sampler_top_k_ws(C.byref(ws), fp(x), 2, 1.0, C.byref(rng))
+               for _ in range(1000))
+    host.geist_sampler_workspace_destroy(C.byref(ws))
+    assert seen == {2, 4}
+    # 6 (115-131)
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(13))
+    x = f32(10, 0, 0, 0, 0)
+    assert host.geist_sampler_workspace_init(C.byref(ws), 5) == 0
+    hits = sum(host.geist_sampler_top_p_ws(C.byref(ws), fp(x), 0.5, 1.0, C.byref(rng)) == 0
+               for _ in range(1000))
+    host.geist_sampler_workspace_destroy(C.byref(ws))
+    assert hits > 990
+    # 7 (134-148): workspace reuse, destroy is idempotent and NULL-safe
+    assert host.geist_sampler_workspace_init(C.byref(ws), 8) == 0
+    host.geist_rng_seed(C.byref(rng), C.c_uint64(17))
+    x = f32(.1, .2, .3, 5, .1, 0, 0, 0)
+    for _ in range(100):
+        host.geist_sampler_top_k_ws(C.byref(ws), fp(x), 3, 1.0, C.byref(rng))
+    host.geist_sampler_workspace_destroy(C.byref(ws))
+    host.geist_sampler_workspace_destroy(C.byref(ws))
+    host.geist_sampler_workspace_destroy(None)
+    assert ws.n_vocab == 0 and not ws.probs
+    # workspace_init argument errors (sampler.c:138-140): GEIST_E_INVALID_ARG == 2
+    assert host.geist_sampler_workspace_init(None, 8) == 2
+    assert host.geist_sampler_workspace_init(C.byref(ws), 0) == 2
+
+
+def test_symbols_follow_the_oracle_draw_for_draw(host, oracle):
+    g = np.random.default_rng(9)
+    n = 20000
+    x = (g.standard_normal(n) * 2).astype(np.float32)
+    ws = Ws()
+    assert host.geist_sampler_workspace_init(C.byref(ws), n) == 0
+    cases = [("temperature", (0.8,)), ("top_k", (40, 0.7)), ("top_k", (1, 0.7)),
+             ("top_k", (n + 5, 0.9)), ("top_k", (300, 1.1)), ("top_p", (0.9, 0.7)),
+             ("top_p", (1.0, 0.7)), ("top_p", (0.0, 0.7)), ("temperature", (0.0,))]
+    for mode, prm in cases:
+        rng = Rng()
+        host.geist_rng_seed(C.byref(rng), C.c_uint64(0xC0FFEE))
+        r = oracle.rng(0xC0FFEE)
+        for _ in range(6):
+            if mode == "temperature":
+                got = host.geist_sampler_temperature(n, fp(x), prm[0], C.byref(rng))
+                want = oracle.lib.oracle_temperature(n, fp(x), prm[0], C.byref(r))
+            elif mode == "top_k":
+                got = host.geist_sampler_top_k_ws(C.byref(ws), fp(x), prm[0], prm[1], C.byref(rng))
+                want = oracle.lib.oracle_top_k(n, fp(x), prm[0], prm[1], C.byref(r))
+            else:
+                got = host.geist_sampler_top_p_ws(C.byref(ws), fp(x), prm[0], prm[1], C.byref(rng))
+                want = oracle.lib.oracle_top_p(n, fp(x), prm[0], prm[1], C.byref(r))
+            assert got == want, (mode, prm)
+        assert rng.state == int(r.state), "draw count differs from the reference"
+    host.geist_sampler_workspace_destroy(C.byref(ws))
+
+
+# ------------------------------------------------------------------ session / head mirror
+def make_head(host, vocab, m_max=0, softcap=0.0):
+    h = C.c_void_p()
+    assert host.geist_hip_head_create(0, vocab, m_max, softcap, None, C.byref(h)) == 0
+    return h
+
+
+def test_head_dispatch_precedence_and_rng(host, oracle):
+    """Model-free statement of tests/test_session_sampling_int.c: greedy is repeatable, a seeded
+    stochastic run differs from greedy and repeats with the same seed; plus the dispatch table of
+    head.c:172-183 and the draw count per mode."""
+    g = np.random.default_rng(31)
+    vocab = 32000
+    x = (g.standard_normal((8, vocab)) * 2).astype(np.float32)
+    d = torch.from_numpy(x).cuda()
+    table = [(0.0, 1.0, 0), (0.0, 0.9, 40), (0.7, 0.9, 40), (0.7, 1.0, 40), (0.7, 0.9, 1),
+             (0.7, 0.9, 0), (0.7, 1.0, 0), (0.7, 0.0, 0), (0.7, -2.0, 0), (10.0, 1.0, 200)]
+    for T, p, k in table:
+        h = make_head(host, vocab)
+        opts = SessionOpts(0, T, p, k, 0xDEADBEEF, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        sess = oracle.session(T, p, k, seed=0xDEADBEEF)
+        # one row at a time (decode_step cadence) ...
+        for r in range(3):
+            tok = C.c_int32(-1)
+            assert host.geist_hip_head_finalize_one_row(h, C.c_void_p(d[r].data_ptr()),
+                                                        C.byref(tok)) == 0
+            assert tok.value == oracle.finalize_row(sess, x[r]), (T, p, k, r)
+        # ... then a batch of rows with the shared RNG (verify_forward cadence)
+        out = (C.c_int32 * 5)()
+        assert host.geist_hip_head_finalize_batch(h, C.c_void_p(d[3].data_ptr()), 5, out) == 0
+        assert list(out) == oracle.finalize_batch(sess, x[3:8]).tolist(), (T, p, k)
+        st = C.c_uint64(0)
+        assert host.geist_hip_head_rng_state(h, C.byref(st)) == 0
+        assert st.value == int(sess.rng.state), "RNG consumption differs"
+        host.geist_hip_head_destroy(h)
+
+
+def test_head_defaults_and_null_opts(host, oracle):
+    vocab = 5000
+    g = np.random.default_rng(2)
+    x = (g.standard_normal((1, vocab)) * 2).astype(np.float32)
+    d = torch.from_numpy(x).cuda()
+    h = make_head(host, vocab)
+    assert host.geist_hip_head_apply_opts(h, None) == 0          # NULL opts = greedy
+    st = C.c_uint64(0)
+    host.geist_hip_head_rng_state(h, C.byref(st))
+    assert st.value == 0xCAFEBABE1234                              # arch_state.c:1173
+    tok = C.c_int32(-1)
+    assert host.geist_hip_head_finalize_one_row(h, C.c_void_p(d.data_ptr()), C.byref(tok)) == 0
+    assert tok.value == oracle.argmax(x[0])
+    host.geist_hip_head_rng_state(h, C.byref(st))
+    assert st.value == 0xCAFEBABE1234                              # greedy draws nothing
+    # random_seed == 0 keeps the default seed (step.c:393-395)
+    opts = SessionOpts(0, 0.8, 1.0, 0, 0, None, 0, 0)
+    host.geist_hip_head_apply_opts(h, C.byref(opts))
+    host.geist_hip_head_rng_state(h, C.byref(st))
+    assert st.value == 0xCAFEBABE1234
+    # more rows than m_max is refused
+    out = (C.c_int32 * 100)()
+    assert host.geist_hip_head_finalize_batch(h, C.c_void_p(d.data_ptr()), 100, out) != 0
+    assert b"m_max" in host.geist_hip_head_errmsg(h)
+    host.geist_hip_head_destroy(h)
+
+
+def test_head_argmax_slot(host):
+    # tests/test_fused_probe_agreement_unit.c:147-157: p[i] = (i == 77 ? 100 : i % 7) -> 77
+    p = np.array([100.0 if i == 77 else i % 7 for i in range(256)], dtype=np.float32)
+    d = torch.from_numpy(p).cuda()
+    h = make_head(host, 256)
+    idx = C.c_int32(-1)
+    assert host.geist_hip_head_argmax_f32(h, C.c_void_p(d.data_ptr()), 256, C.byref(idx)) == 0
+    assert idx.value == 77
+    assert host.geist_hip_head_argmax_f32(h, C.c_void_p(d.data_ptr()), 999, C.byref(idx)) == 7
+    host.geist_hip_head_destroy(h)
+
+
+def test_head_softcap_only_when_sampling(host, oracle):
+    """head.c:148-159: tanhf(x / c) * c in front of the stochastic samplers, skipped when greedy.
+    The device tanhf is not glibc's, so capped logits agree to a few ulp, not bit for bit: the
+    token ids are compared on rows whose draw is not at a CDF boundary."""
+    g = np.random.default_rng(5)
+    vocab, cap = 20000, 30.0
+    x = (g.standard_normal((6, vocab)) * 12).astype(np.float32)
+    d = torch.from_numpy(x).cuda()
+    h = make_head(host, vocab, 0, cap)
+    opts = SessionOpts(0, 0.9, 1.0, 50, 77, None, 0, 0)
+    host.geist_hip_head_apply_opts(h, C.byref(opts))
+    out = (C.c_int32 * 6)()
+    assert host.geist_hip_head_finalize_batch(h, C.c_void_p(d.data_ptr()), 6, out) == 0
+    r = oracle.rng(77)
+    agree = 0
+    for i in range(6):
+        u = oracle.next_unit(r)
+        want, info = oracle.top_k_u(oracle.softcap(x[i], cap), 50, 0.9, u)
+        agree += (out[i] == want) or info.boundary_dist < 1e-4
+    assert agree == 6
+    host.geist_hip_head_destroy(h)
