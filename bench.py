@@ -10,8 +10,8 @@ sit in HBM: penalties + temperature + top-k + top-p + draw for the default workl
 
 value      rows sampled per second over the timed K steps (whole job, one GPU)
 roofline   the logit-streaming kernel: algorithmic bytes per launch / its mean duration, the
-           duration taken with HIP events on the sampler's stream around every launch of that
-           kernel during a second pass of K steps
+           duration taken with HIP events on the sampler's stream around K back-to-back launches
+           of that kernel alone, right after the timed region
 cpu_baseline  the CPU restatement of the same step (oracle, reference build flags) timed on
            this host's cores on a bounded sample; reported, not the optimisation target
 """
@@ -124,14 +124,9 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     ids_gpu = d_out.cpu().numpy()
 
-    # second pass: events around every launch of the logit-streaming kernel
-    hs.timing_enable(True)
-    hs.timing_read(reset=True)
-    for _ in range(args.steps):
-        step()
-    k_ms, k_n = hs.timing_read(reset=True)
-    hs.timing_enable(False)
-    kernel_us = k_ms * 1e3 / max(k_n, 1)
+    # the logit-streaming kernel on its own: HIP events on the sampler's stream around K
+    # back-to-back launches of that kernel (same rows, same configuration)
+    kernel_us = hs.time_stream_kernel(rows, prm, d_u, d_out, args.steps)
 
     # one-step latency: enqueue + wait, median
     lat = []
@@ -165,7 +160,7 @@ def main():
         "step_latency_us_median": round(lat[len(lat) // 2], 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_topk_scan" if w.top_k > 1 else "k_chunk_expsum",
+                     "kernel": "k_tmax_scan" if (w.top_k > 1 or w.temperature <= 0) else "k_chunk_expsum",
                      "kernel_us": round(kernel_us, 3), "algorithmic_bytes": alg_bytes,
                      "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }

@@ -73,9 +73,9 @@ def load_library():
     lib.geist_hip_free.argtypes = [vp, vp]
     lib.geist_hip_upload.argtypes = [vp, vp, vp, sz]
     lib.geist_hip_download.argtypes = [vp, vp, vp, sz]
-    lib.geist_hip_sampler_timing_enable.argtypes = [vp, i32]
-    lib.geist_hip_sampler_timing_read.argtypes = [vp, C.POINTER(C.c_double), C.POINTER(C.c_long),
-                                                  i32]
+    lib.geist_hip_sampler_time_stream_kernel.argtypes = [vp, C.POINTER(Rows),
+                                                         C.POINTER(SampleParams), vp, vp, i32,
+                                                         C.POINTER(C.c_double)]
     _LIB = lib
     return lib
 
@@ -166,11 +166,11 @@ class HipSampler:
                                                    _ptr(uniforms), n_seq, L, n, temperature,
                                                    _ptr(out_tokens), _ptr(n_accepted)))
 
-    def timing_enable(self, on=True):
-        self._check(self.lib.geist_hip_sampler_timing_enable(self.h, int(on)))
-
-    def timing_read(self, reset=True):
-        ms, n = C.c_double(), C.c_long()
-        self._check(self.lib.geist_hip_sampler_timing_read(self.h, C.byref(ms), C.byref(n),
-                                                           int(reset)))
-        return ms.value, n.value
+    def time_stream_kernel(self, rows, params, uniforms, out, launches):
+        """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around
+        `launches` back-to-back launches on the sampler's stream)."""
+        ms = C.c_double()
+        self._check(self.lib.geist_hip_sampler_time_stream_kernel(
+            self.h, C.byref(rows), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
+            C.byref(ms)))
+        return ms.value * 1e3 / launches

@@ -155,13 +155,15 @@ int geist_hip_free(geist_hip_sampler *s, void *d_ptr);
 int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes);   /* sync */
 int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, size_t bytes); /* sync */
 
-/* Timing of the kernels this object enqueues, for benchmarks: when enabled, each sampling call
- * brackets its dominant (logit-streaming) kernel with events on the sampler's stream.
- * geist_hip_sampler_timing_read synchronises and returns the accumulated milliseconds and the
- * number of bracketed launches since the last reset. */
-int geist_hip_sampler_timing_enable(geist_hip_sampler *s, int on);
-int geist_hip_sampler_timing_read(geist_hip_sampler *s, double *ms_total, long *launches,
-                                  int reset);
+/* For benchmarks (no reference counterpart): enqueues ONLY the logit-streaming kernel of the given
+ * configuration `launches` times back to back on the sampler's stream, between two HIP events
+ * recorded on that stream, waits, and returns the elapsed milliseconds. Dividing by `launches`
+ * gives the mean duration of that kernel (thread-maxima scan for top-k and argmax, exp-sum scan
+ * for temperature / top-p / min-p). One complete sampling call is made first. */
+int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                                         const struct geist_hip_sample_params *params,
+                                         const float *d_uniforms, geist_hip_token_t *d_out_tokens,
+                                         int launches, double *ms_total);
 
 #ifdef __cplusplus
 }
