@@ -86,6 +86,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg2_pen")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of sampling, run a plain device copy of the logit buffer "
+                         "(a kernel of known traffic, for scaling rocprof's FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: rows are independent and this build has no "
@@ -107,6 +110,16 @@ def main():
     rows = HipSampler.rows(d_logits, d_h, d_hl)
     prm = SampleParams.make(temperature=w.temperature, top_k=w.top_k, top_p=w.top_p,
                             min_p=w.min_p, rep=w.rep, freq=w.freq, pres=w.pres)
+
+    if args.calibrate_copy:
+        dst = torch.empty_like(d_logits)
+        for _ in range(args.steps):
+            dst.copy_(d_logits)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": d_logits.numel() * 4,
+                          "calibrate_copy_bytes_written": d_logits.numel() * 4,
+                          "launches": args.steps}))
+        return
 
     def step():
         hs.sample(rows, prm, d_u, d_out)

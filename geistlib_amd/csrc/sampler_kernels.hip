@@ -5,8 +5,9 @@
  *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t)          sampler.c:77-83
  *   k_tmax_scan      per-thread maxima (the single pass of the top-k path) and,
  *                    on request, the per-chunk maximum with its first index       sampler.c:52-62, 202-207
- *   k_row_final      per-row combine: argmax / index-order CDF draw / top-k
- *                    select, sorted softmax, top-p, min-p, draw               sampler.c:90-102, 209-222, 272-299
+ *   k_final_argmax / _temperature / _topk / _sorted   per-row combine of each mode: argmax,
+ *                    index-order CDF draw, top-k select + sorted softmax + top-p + min-p +
+ *                    draw, top-p / min-p shortcut                             sampler.c:90-102, 209-222, 272-299
  *   k_sorted_general full-vocabulary top-p / min-p by mass-weighted radix descent sampler.c:246-304
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
  *   k_penalties      in-place penalties                                       (no reference counterpart)
@@ -462,7 +463,7 @@ struct GeneralShared {
 };
 
 template <int NV, bool PEN>
-__device__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t *spack,
+__device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t *spack,
                                 int spack_cap, uint32_t *cnt16, GeneralShared &gs_) {
     constexpr int TILE = NV * TPB * 4;
     const int     tid  = threadIdx.x;
@@ -801,161 +802,175 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 namespace gs {
 
 /* ============================================================================================
- * k_row_final: one workgroup per row.
+ * Row-final kernels: one workgroup per row, one kernel per sampling mode.
  * ========================================================================================== */
 
+/* argmax: sampler.c:52-62 */
+__global__ __launch_bounds__(TPB) void k_final_argmax(RowView rv, FinalArgs a) {
+    __shared__ uint64_t s_red[NWAVES];
+    const int           row = blockIdx.x;
+    const uint64_t      b   = row_best_from_chunks(a.chunk_best, row, rv.n_chunks, s_red);
+    if (threadIdx.x == 0) {
+        const float first = rv.logits[(long) row * rv.ld];
+        /* a NaN at index 0 is never displaced by the strict '>' of the reference; after the
+         * transforms it stays NaN, so the raw value decides */
+        a.out[row] = (first != first) ? 0 : (int32_t) best_idx(b);
+    }
+}
+
+/* temperature: sampler.c:90-102 over all n in index order: locate the chunk from the per-chunk
+ * sums, then scan that chunk. */
 template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
-    __shared__ uint64_t      s_red[NWAVES];
-    __shared__ FinishShared  s_fs;
+__global__ __launch_bounds__(TPB) void k_final_temperature(RowView rv, FinalArgs a) {
+    __shared__ uint64_t     s_red[NWAVES];
+    __shared__ FinishShared s_fs;
+    __shared__ double       s_csum[MAX_CHUNKS];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ int          s_chunk;
+    __shared__ double       s_before;
+    const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
+    if (tid < C)
+        s_csum[tid] = a.chunk_sum[(long) row * C + tid];
+    if (tid < 32)
+        s_fs.tab[tid] = g_expf_tab[tid];
+    const float u_row = a.uniforms[row];
+    __syncthreads();
+    if (tid == 0) {
+        double tot = 0.0;
+        for (int c = 0; c < C; ++c)
+            tot += s_csum[c];
+        const double target = (double) u_row * tot;
+        double       run    = 0.0;
+        int          at     = C - 1;
+        for (int c = 0; c < C; ++c) {
+            const double nxt = run + s_csum[c];
+            if (target < nxt || c == C - 1) {
+                at = c;
+                break;
+            }
+            run = nxt;
+        }
+        s_chunk   = at;
+        s_before  = run;
+        s_fs.mass = target;
+    }
+    const float mx = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
+    /* (row_best_from_chunks ends with a barrier: s_chunk, s_before, tab are visible) */
+    const int chunk = s_chunk;
+    int       base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    float4 v[NV];
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
+    /* index order inside the chunk is (j, thread, component): scan one j-slab at a time */
+    double       carry  = s_before;
+    const double target = s_fs.mass;
+    if (tid == 0)
+        s_fs.pick = 0x7fffffff;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+        float     p[4];
+        double    part = 0.0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            p[c] = (e + c < end)
+                       ? geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, a.inv_t), s_fs.tab)
+                       : 0.0f;
+            part += (double) p[c];
+        }
+        double       slab;
+        const double incl = block_scan_f64(part, s_fs.scan, &slab);
+        double       run  = carry + (incl - part);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            run += (double) p[c];
+            if (e + c < end && target < run) {
+                atomicMin(&s_fs.pick, e + c);
+                break;
+            }
+        }
+        carry += slab;
+    }
+    __syncthreads();
+    if (tid == 0)
+        a.out[row] = s_fs.pick == 0x7fffffff ? end - 1 : s_fs.pick;
+}
+
+/* top-p / min-p over the whole vocabulary (sampler.c:232-305): the thread-maxima shortcut; a
+ * row it cannot serve raises its flag for k_sorted_general. */
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
+    __shared__ uint64_t s_red[NWAVES];
+    __shared__ uint64_t s_tab[32];
+    __shared__ __align__(16) uint8_t s_big[TMAX_LDS];
+    __shared__ uint32_t s_mx[TPB];
+    __shared__ int      s_selid[SEL_MAX];
+    __shared__ uint32_t s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
+    __shared__ uint64_t s_m[TPB];
+    __shared__ uint64_t s_srt[TPB];
+    __shared__ float    s_wt[TPB];
+    __shared__ double   s_csum[MAX_CHUNKS];
+    __shared__ int      s_n, s_n2;
+    __shared__ double   s_sum;
+    const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    if (tid < C)
+        s_csum[tid] = a.chunk_sum[(long) row * C + tid];
+    const float u_row = a.uniforms[row];
+    const float mx    = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
+    if (tid == 0) {
+        double tot = 0.0;
+        for (int c = 0; c < C; ++c)
+            tot += s_csum[c];
+        s_sum = tot;
+    }
+    __syncthreads();
+    const double sum = s_sum;
+    int          tok = -1;
+    if (C <= 16)
+        tok = sorted_from_tmax<NV, PEN, 16>(rv, a, row, mx, sum, u_row, s_big, s_mx, s_wt, s_selid,
+                                            s_pcnt, s_m, s_srt, &s_n, &s_n2, s_tab);
+    else if (C <= TMAX_LDS / TPB)
+        tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big, s_mx,
+                                                        s_wt, s_selid, s_pcnt, s_m, s_srt, &s_n,
+                                                        &s_n2, s_tab);
+    if (tid == 0) {
+        a.row_flag[row] = tok < 0 ? 1 : 0;
+        a.out[row]      = tok;
+    }
+}
+
+/* top-k (sampler.c:178-228) and the chain behind it: select from the row's thread maxima, then
+ * gather; rows the shortcut cannot serve (masked rows full of -inf, all-equal rows, tiny or huge
+ * vocabularies) select over the whole row in place. */
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
+    __shared__ uint64_t      s_tab[32];
     __shared__ GeneralShared s_gs;
     __shared__ __align__(16) uint8_t s_big[TMAX_LDS];
-    __shared__ uint32_t      s_bitmap[TPB];
+    __shared__ uint32_t      s_mx[TPB];
     __shared__ int           s_selid[SEL_MAX];
     __shared__ uint32_t      s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
     __shared__ uint64_t      s_m[TPB];
-    __shared__ uint64_t      s_srt[TPB];
-    __shared__ float         s_wt[TPB];
     __shared__ uint64_t      s_pack[TOPK_FAST_MAX];
-    __shared__ double        s_csum[MAX_CHUNKS];
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ int           s_n, s_n2, s_chunk;
-    __shared__ double        s_before;
-
-    const int row = blockIdx.x, tid = threadIdx.x;
-    const int C = rv.n_chunks;
-
-    if (a.mode == FINAL_ARGMAX) {
-        /* sampler.c:52-62 */
-        const uint64_t b = row_best_from_chunks(a.chunk_best, row, C, s_red);
-        if (tid == 0) {
-            const float first = rv.logits[(long) row * rv.ld];
-            /* a NaN at index 0 is never displaced by the strict '>' of the reference; after the
-             * transforms it stays NaN, so the raw value decides */
-            a.out[row] = (first != first) ? 0 : (int32_t) best_idx(b);
-        }
-        return;
-    }
-
-    if (a.mode == FINAL_TEMPERATURE) {
-        /* sampler.c:90-102 over all n in index order: locate the chunk from the per-chunk sums,
-         * then scan that chunk. */
-        if (tid < C)
-            s_csum[tid] = a.chunk_sum[(long) row * C + tid];
-        if (tid < 32)
-            s_fs.tab[tid] = g_expf_tab[tid];
-        const float u_row = a.uniforms[row];
-        __syncthreads();
-        if (tid == 0) {
-            double tot = 0.0;
-            for (int c = 0; c < C; ++c)
-                tot += s_csum[c];
-            const double target = (double) u_row * tot;
-            double       run    = 0.0;
-            int          at     = C - 1;
-            for (int c = 0; c < C; ++c) {
-                const double nxt = run + s_csum[c];
-                if (target < nxt || c == C - 1) {
-                    at = c;
-                    break;
-                }
-                run = nxt;
-            }
-            s_chunk   = at;
-            s_before  = run;
-            s_fs.mass = target;
-        }
-        const float mx = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
-        /* (row_best_from_chunks ends with a barrier: s_chunk, s_before, tab are visible) */
-        const int chunk = s_chunk;
-        int       base, end;
-        chunk_bounds<NV>(rv, chunk, base, end);
-        float4 v[NV];
-        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
-        /* index order inside the chunk is (j, thread, component): scan one j-slab at a time */
-        double       carry  = s_before;
-        const double target = s_fs.mass;
-        if (tid == 0)
-            s_fs.pick = 0x7fffffff;
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int e = base + 4 * (j * TPB + tid);
-            float     p[4];
-            double    part = 0.0;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                p[c] = (e + c < end)
-                           ? geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, a.inv_t), s_fs.tab)
-                           : 0.0f;
-                part += (double) p[c];
-            }
-            double       slab;
-            const double incl = block_scan_f64(part, s_fs.scan, &slab);
-            double       run  = carry + (incl - part);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                run += (double) p[c];
-                if (e + c < end && target < run) {
-                    atomicMin(&s_fs.pick, e + c);
-                    break;
-                }
-            }
-            carry += slab;
-        }
-        __syncthreads();
-        if (tid == 0)
-            a.out[row] = s_fs.pick == 0x7fffffff ? end - 1 : s_fs.pick;
-        return;
-    }
-
-    if (a.mode == FINAL_SORTED) {
-        /* top-p / min-p over the whole vocabulary (sampler.c:232-305) */
-        if (tid < 32)
-            s_fs.tab[tid] = g_expf_tab[tid];
-        if (tid < C)
-            s_csum[tid] = a.chunk_sum[(long) row * C + tid];
-        const float u_row = a.uniforms[row];
-        const float mx    = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
-        if (tid == 0) {
-            double tot = 0.0;
-            for (int c = 0; c < C; ++c)
-                tot += s_csum[c];
-            s_before = tot;
-        }
-        __syncthreads();
-        const double sum = s_before;
-        int          tok = -1;
-        if (C <= 16)
-            tok = sorted_from_tmax<NV, PEN, 16>(rv, a, row, mx, sum, u_row, s_big, s_bitmap, s_wt,
-                                                s_selid, s_pcnt, s_m, s_srt, &s_n, &s_n2, s_fs.tab);
-        else if (C <= TMAX_LDS / TPB)
-            tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big,
-                                                            s_bitmap, s_wt, s_selid, s_pcnt, s_m,
-                                                            s_srt, &s_n, &s_n2, s_fs.tab);
-        if (tid == 0) {
-            a.row_flag[row] = tok < 0 ? 1 : 0;
-            a.out[row]      = tok;
-        }
-        return;
-    }
-
-    /* ---- FINAL_TOPK: select from the row's thread maxima, then gather ------------------------ */
+    __shared__ int           s_n, s_n2;
+    const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
     GS_MARK(0);
     if (tid < 32)
-        s_fs.tab[tid] = g_expf_tab[tid];
+        s_tab[tid] = g_expf_tab[tid];
     const float u_row   = a.uniforms[row];
     int         k       = 0;
     bool        general = true;
     if (C <= 16)
-        general = topk_from_tmax<NV, PEN, 16>(rv, a, row, s_big, s_bitmap, s_selid, s_pcnt, s_m,
+        general = topk_from_tmax<NV, PEN, 16>(rv, a, row, s_big, s_mx, s_selid, s_pcnt, s_m,
                                               s_pack, &s_n, &s_n2, k);
     else if (C <= TMAX_LDS / TPB)
-        general = topk_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, s_big, s_bitmap, s_selid,
-                                                          s_pcnt, s_m, s_pack, &s_n, &s_n2, k);
+        general = topk_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, s_big, s_mx, s_selid, s_pcnt,
+                                                          s_m, s_pack, &s_n, &s_n2, k);
     if (general) {
-        /* rows this shortcut cannot serve (masked rows full of -inf, all-equal rows, tiny or
-         * huge vocabularies): exact selection over the whole row */
         __syncthreads();
         k = topk_row_general<NV, PEN>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
     }
@@ -963,8 +978,8 @@ __global__ __launch_bounds__(TPB) void k_row_final(RowView rv, FinalArgs a) {
     /* k <= TOPK_FAST_MAX = 128: the tail runs on one wavefront without barriers */
     if (tid < WAVE) {
         const int tok =
-            k <= WAVE ? finish_sorted_wave<1>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab)
-                      : finish_sorted_wave<2>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_fs.tab);
+            k <= WAVE ? finish_sorted_wave<1>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_tab)
+                      : finish_sorted_wave<2>(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_tab);
         if (tid == 0)
             a.out[row] = tok;
     }
@@ -1177,8 +1192,17 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.row_flag   = f.row_flag;
     a.out        = f.out;
     const dim3 grid(L.rows), block(TPB);
+    if (f.mode == FINAL_ARGMAX) {
+        k_final_argmax<<<grid, block, 0, L.stream>>>(L.rv, a);
+        return;
+    }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_row_final<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
+        if (f.mode == FINAL_TEMPERATURE)
+            k_final_temperature<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
+        else if (f.mode == FINAL_SORTED)
+            k_final_sorted<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
+        else
+            k_final_topk<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
     });
 }
 

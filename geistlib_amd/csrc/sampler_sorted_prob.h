@@ -5,7 +5,7 @@
  *
  * The reference normalises every probability, sorts all of them and walks the sorted list.
  * Here nothing is sorted but the few entries that can matter:
- *   fast path (in k_row_final)  thread maxima -> a logit bound below which nothing of the kept
+ *   fast path (k_final_sorted)   thread maxima -> a logit bound below which nothing of the kept
  *                               prefix can lie -> re-read the threads above it -> order those
  *                               entries -> walk. Serves rows whose kept prefix is small.
  *   general path (k_sorted_general)  for rows the fast path hands on: the normalised
