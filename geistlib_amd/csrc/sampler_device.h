@@ -312,6 +312,44 @@ __device__ __forceinline__ void history_for_each(const RowView &rv, int row,
     for (int i = i0 + threadIdx.x; i < len; i += TPB)
         f(h[i]);
 }
+/* Two-phase variant for lookups that go through LDS: look(id) is evaluated for up to eight
+ * entries before apply(code) runs for each of them, so the eight LDS reads are in flight together
+ * instead of each waiting behind the previous entry's atomic. */
+template <typename L, typename A>
+__device__ __forceinline__ void history_for_each_batched(const RowView &rv, int row,
+                                                         const HistPrefetch &pf, L &&look,
+                                                         A &&apply) {
+    int len = __builtin_amdgcn_readfirstlane(pf.len);
+    if (len > rv.hist_ld)
+        len = (int) rv.hist_ld;
+    const int32_t *h  = rv.hist + (long) row * rv.hist_ld;
+    int            i0 = 0;
+    auto           eight = [&](const int4 &a, const int4 &b) {
+        const int c0 = look(a.x), c1 = look(a.y), c2 = look(a.z), c3 = look(a.w);
+        const int c4 = look(b.x), c5 = look(b.y), c6 = look(b.z), c7 = look(b.w);
+        apply(c0);
+        apply(c1);
+        apply(c2);
+        apply(c3);
+        apply(c4);
+        apply(c5);
+        apply(c6);
+        apply(c7);
+    };
+    if (pf.vec) {
+        const int4 *h4   = reinterpret_cast<const int4 *>(h);
+        const int   n4   = len >> 2;
+        const int   g    = threadIdx.x;
+        const int4  none = make_int4(-1, -1, -1, -1);
+        if (g < n4)
+            eight(pf.a, g + TPB < n4 ? pf.b : none);
+        for (int g2 = g + 2 * TPB; g2 < n4; g2 += 2 * TPB)
+            eight(h4[g2], g2 + TPB < n4 ? h4[g2 + TPB] : none);
+        i0 = n4 << 2;
+    }
+    for (int i = i0 + threadIdx.x; i < len; i += TPB)
+        apply(look(h[i]));
+}
 __device__ __forceinline__ void history_count(const RowView &rv, int row, const HistPrefetch &pf,
                                               int base, int end, uint32_t *cnt16) {
     history_for_each(rv, row, pf, [&](int t) {

@@ -29,11 +29,11 @@ __device__ const uint64_t g_expf_tab[32] = GEIST_EXPF_TABLE_INIT;
 
 /* Phase timestamps for kernel tuning; compiled in only by the tuning probe. */
 #ifdef GS_PHASES
-__device__ long long g_phase[16384 * 8];
+__device__ long long g_phase[16384 * 16];
 #define GS_MARK(i)                                                                             \
     do {                                                                                       \
         if (threadIdx.x == 0)                                                                  \
-            g_phase[((long) blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = wall_clock64();   \
+            g_phase[((long) blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();   \
     } while (0)
 #else
 #define GS_MARK(i) ((void) 0)
@@ -615,8 +615,9 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         for (int i = tid; i < KPT * TPB / 16; i += TPB)
             z[i] = make_uint4(0u, 0u, 0u, 0u);
         if (PEN) {
-            for (int i = tid; i < SEL_MAX * 4 * NV; i += TPB)
-                s_pcnt[i] = 0u;
+            uint4 *zc = reinterpret_cast<uint4 *>(s_pcnt);
+            for (int i = tid; i < SEL_MAX * NV; i += TPB)
+                zc[i] = make_uint4(0u, 0u, 0u, 0u);
         }
         if (tid == 0) {
             *s_n  = 0;
@@ -635,7 +636,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
                    a3 = s_mx[lane + 192];
     int      real;
     uint32_t tau = 0u;
-    if (a.k_sel <= 48) {
+    if (a.k_sel <= 64) {
         /* 128 pairwise maxima: about -128 ln(1 - k/128) threads end up selected */
         const uint32_t m0 = a0 > a2 ? a0 : a2, m1 = a1 > a3 ? a1 : a3;
         real = __popcll(__ballot(m0 != 0u)) + __popcll(__ballot(m1 != 0u));
@@ -665,23 +666,26 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         return true;
     const float bound = key2f(tau);
     /* 3 */
-    int cnt = 0;
+    uint32_t selmask = 0u;
 #pragma unroll
     for (int q = 0; q < KPT; ++q)
-        cnt += raw[q] >= bound;
-    int pos = wave_reserve(cnt, s_n);
-#pragma unroll
-    for (int q = 0; q < KPT; ++q) {
-        if (raw[q] >= bound) {
-            if (pos < SEL_MAX) {
-                s_selid[pos]        = q * TPB + tid;
-                slot[q * TPB + tid] = (uint8_t) (pos + 1);
-            }
-            ++pos;
+        selmask |= (uint32_t) (raw[q] >= bound) << q;
+    GS_MARK(8);
+    int pos = wave_reserve(__popc(selmask), s_n);
+    GS_MARK(9);
+    while (selmask) { /* a few rounds: the selected maxima are spread over the threads */
+        const int q = __ffs(selmask) - 1;
+        selmask &= selmask - 1u;
+        if (pos < SEL_MAX) {
+            s_selid[pos]        = q * TPB + tid;
+            slot[q * TPB + tid] = (uint8_t) (pos + 1);
         }
+        ++pos;
     }
+    GS_MARK(10);
     __syncthreads();
     const int n_sel = *s_n;
+    GS_MARK(11);
     if (n_sel > SEL_MAX)
         return true; /* long runs of equal maxima */
     /* 4 */
@@ -717,54 +721,52 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
     GS_MARK(3);
     if (PEN) {
         const int shift = 31 - __clz(rv.per_chunk); /* per_chunk = 1024 * NV */
-        history_for_each(rv, row, pf, [&](int t) {
-            if (t < 0 || t >= rv.n_vocab)
-                return;
-            const int off = t & (rv.per_chunk - 1);
-            const int f   = off >> 2;
-            const int s   = slot[(t >> shift) * TPB + (f % TPB)];
-            if (s)
-                atomicAdd(&s_pcnt[((s - 1) * NV + f / TPB) * 4 + (off & 3)], 1u);
-        });
+        history_for_each_batched(
+            rv, row, pf,
+            [&](int t) -> int { /* 1 + index of the element's counter, 0 = not gathered */
+                if (t < 0 || t >= rv.n_vocab)
+                    return 0;
+                const int off = t & (rv.per_chunk - 1);
+                const int f   = off >> 2;
+                const int s   = slot[(t >> shift) * TPB + (f % TPB)];
+                return s ? 1 + ((s - 1) * NV + f / TPB) * 4 + (off & 3) : 0;
+            },
+            [&](int code) {
+                if (code)
+                    atomicAdd(&s_pcnt[code - 1], 1u);
+            });
         __syncthreads();
     }
     GS_MARK(4);
-    uint32_t ck[TASKS][4];
-    int      keep = 0;
+    /* survivors are appended in any order: the ranking below orders them */
 #pragma unroll
     for (int q = 0; q < TASKS; ++q) {
         const int t = tid + q * TPB;
+        if (e0[q] >= e1[q])
+            continue; /* no task (whole wavefronts beyond the list skip the block) */
+        uint4 hc = make_uint4(0u, 0u, 0u, 0u);
+        if (PEN)
+            hc = *reinterpret_cast<const uint4 *>(&s_pcnt[t * 4]);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            ck[q][c] = 0u;
             if (e0[q] + c < e1[q]) {
                 float x = f4_get(r[q], c);
                 if (PEN) {
-                    const uint32_t n_hist = s_pcnt[t * 4 + c];
+                    const uint32_t n_hist = c == 0 ? hc.x : c == 1 ? hc.y : c == 2 ? hc.z : hc.w;
                     if (n_hist)
                         x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
                 }
                 if (rv.softcap > 0.0f)
                     x = __fmul_rn(tanhf(__fdiv_rn(x, rv.softcap)), rv.softcap);
                 if (x >= bound) {
-                    ck[q][c] = f2key(x);
-                    ++keep;
+                    const int at = atomicAdd(s_n2, 1);
+                    if (at < TPB)
+                        s_m[at] = pack_best(f2key(x), (uint32_t) (e0[q] + c));
                 }
             }
         }
     }
-    pos = wave_reserve(keep, s_n2);
-#pragma unroll
-    for (int q = 0; q < TASKS; ++q) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (ck[q][c]) {
-                if (pos < TPB)
-                    s_m[pos] = pack_best(ck[q][c], (uint32_t) (e0[q] + c));
-                ++pos;
-            }
-        }
-    }
+    GS_MARK(12);
     __syncthreads();
     const int m = *s_n2;
     GS_MARK(5);
@@ -906,7 +908,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __shared__ __align__(16) uint8_t s_big[TMAX_LDS];
     __shared__ uint32_t s_mx[TPB];
     __shared__ int      s_selid[SEL_MAX];
-    __shared__ uint32_t s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
+    __shared__ __align__(16) uint32_t s_pcnt[PEN ? SEL_MAX * 4 * NV : 4];
     __shared__ uint64_t s_m[TPB];
     __shared__ uint64_t s_srt[TPB];
     __shared__ float    s_wt[TPB];
@@ -952,7 +954,7 @@ __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
     __shared__ __align__(16) uint8_t s_big[TMAX_LDS];
     __shared__ uint32_t      s_mx[TPB];
     __shared__ int           s_selid[SEL_MAX];
-    __shared__ uint32_t      s_pcnt[PEN ? SEL_MAX * 4 * NV : 1];
+    __shared__ __align__(16) uint32_t s_pcnt[PEN ? SEL_MAX * 4 * NV : 4];
     __shared__ uint64_t      s_m[TPB];
     __shared__ uint64_t      s_pack[TOPK_FAST_MAX];
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
