@@ -30,6 +30,15 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes moved by one launch of the streaming kernel, from rocprofv3's FETCH_SIZE and
+# WRITE_SIZE scaled by what the same counters read for a plain copy of the logit buffer
+# (fetch x 1.9985, write x 1.0000); the summaries are profiles/k_tmax_scan_k_final_topk__*.md.
+# A counter run cannot happen inside a timed benchmark, so the figure is carried here.
+PROFILED_TRAFFIC = {
+    "cfg2_b64_v128256_pen2048": 33922495,
+    "cfg2_b64_v128256": 33922491,
+}
+
 
 def build_workload(name):
     from geistlib_amd import workloads as W
@@ -151,7 +160,9 @@ def main():
     lat.sort()
 
     alg_bytes = w.algorithmic_bytes()
-    achieved = alg_bytes / (kernel_us * 1e-6) / 1e9
+    # the streaming kernel's own share of those bytes: every logit once
+    kernel_bytes = w.rows * w.n_vocab * 4
+    achieved = kernel_bytes / (kernel_us * 1e-6) / 1e9
     result = {
         "metric": "sampled rows/s",
         "value": round(w.rows * args.steps / elapsed, 1),
@@ -172,9 +183,11 @@ def main():
         "us_per_step": round(ms_per_step * 1e3, 3),
         "step_latency_us_median": round(lat[len(lat) // 2], 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": PROFILED_TRAFFIC.get(w.name),
                      "kernel": "k_tmax_scan" if (w.top_k > 1 or w.temperature <= 0) else "k_chunk_expsum",
-                     "kernel_us": round(kernel_us, 3), "algorithmic_bytes": alg_bytes,
+                     "kernel_us": round(kernel_us, 3), "kernel_algorithmic_bytes": kernel_bytes,
+                     "step_algorithmic_bytes": alg_bytes,
                      "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }
     if not args.no_cpu:
