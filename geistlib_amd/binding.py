@@ -76,6 +76,7 @@ def load_library():
     lib.geist_hip_sampler_time_stream_kernel.argtypes = [vp, C.POINTER(Rows),
                                                          C.POINTER(SampleParams), vp, vp, i32,
                                                          C.POINTER(C.c_double)]
+    lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     _LIB = lib
     return lib
 
@@ -174,3 +175,12 @@ class HipSampler:
             self.h, C.byref(rows), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
             C.byref(ms)))
         return ms.value * 1e3 / launches
+
+    def row_paths(self, rows):
+        """Which walk served each row of the last full-vocabulary top-p / min-p call
+        (1 shortcut, 2 candidate list, 3 whole row)."""
+        import numpy as np
+        out = np.zeros(int(rows), dtype=np.int32)
+        self._check(self.lib.geist_hip_sampler_row_paths(self.h, out.ctypes.data_as(C.c_void_p),
+                                                         int(rows)))
+        return out

@@ -36,6 +36,7 @@ struct geist_hip_sampler {
     int32_t  *h_scalar   = nullptr; /* pinned */
     float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
                                      * full-vocabulary top-p / min-p path */
+    gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
 
@@ -193,6 +194,13 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
+    (void) hipFree(s->cand.zhist);
+    (void) hipFree(s->cand.row_bound);
+    (void) hipFree(s->cand.out_key);
+    (void) hipFree(s->cand.key);
+    (void) hipFree(s->cand.idx);
+    (void) hipFree(s->cand.count);
+    (void) hipFree(s->cand.path);
     if (s->h_scalar)
         (void) hipHostFree(s->h_scalar);
     delete s;
@@ -335,7 +343,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (!rs.use_p && !rs.use_m) {
         if (!stream_only(s))
             launch_tmax_scan(L, s->tmax, s->chunk_best);
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr);
         if (stream_only(s))
             return after_launch(s, "exp-sum scan");
         f.mode = FINAL_TEMPERATURE;
@@ -343,8 +351,17 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         return after_launch(s, "temperature");
     }
     /* top-p and/or min-p over the whole vocabulary */
-    if (!s->probs)
-        HIPCHK(s, hipMalloc((void **) &s->probs, s->max_rows * s->max_vocab * sizeof(float)));
+    if (!s->probs) {
+        const size_t R = s->max_rows;
+        HIPCHK(s, hipMalloc((void **) &s->cand.zhist, R * s->max_chunks * ZBINS * sizeof(float)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.row_bound, R * sizeof(int32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.out_key, R * sizeof(uint32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.key, R * CAND_CAP * sizeof(uint32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.idx, R * CAND_CAP * sizeof(uint32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.count, R * sizeof(int32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.path, R * sizeof(int32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->probs, R * s->max_vocab * sizeof(float)));
+    }
     L.nv           = 8;
     L.rv.per_chunk = 8192;
     L.rv.n_chunks  = (int) ((rows->n_vocab + 8191) / 8192);
@@ -353,18 +370,23 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                     rows->n_vocab, s->max_chunks);
     if (!stream_only(s))
         launch_tmax_scan(L, s->tmax, s->chunk_best);
-    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+    f.cand = s->cand;
+    if (!rs.use_p)
+        f.cand.zhist = nullptr; /* the min-p bound needs no binned mass */
+    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, f.cand.zhist);
     if (stream_only(s))
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;
     f.row_flag = s->row_flag;
     launch_row_final(L, f);
-    /* rows whose kept prefix is too wide for the shortcut flagged themselves; the next two
-     * kernels return at once for every other row */
+    /* rows whose kept prefix is too wide for the shortcut flagged themselves 1: their candidates
+     * are listed and walked; what that cannot serve either is flagged 2 for the last two kernels.
+     * Each of these kernels returns at once for every row not flagged for it. */
+    launch_candidates(L, f);
     launch_write_probs(L, rs.inv_t, s->chunk_best, s->chunk_sum, s->probs, (long) s->max_vocab,
                        s->row_flag);
     launch_sorted_general(L, s->probs, (long) s->max_vocab, rs.top_p, rs.min_p, d_uniforms,
-                          s->row_flag, d_out);
+                          s->row_flag, d_out, s->cand.path);
     return after_launch(s, "top-p / min-p");
 }
 
@@ -465,7 +487,7 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
     launch_tmax_scan(L, s->tmax, s->chunk_best);
-    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr);
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
 }
@@ -503,7 +525,7 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     const float inv_t = greedy ? 1.0f : 1.0f / temperature;
     launch_tmax_scan(La, s->tmax, s->chunk_best);
     if (!greedy)
-        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p);
+        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p, nullptr);
     SpecLaunch sp{};
     sp.n_seq      = (int) n_seq;
     sp.L          = (int) L;
@@ -582,6 +604,16 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
     (void) hipEventDestroy(b);
     *ms_total = ms;
     return rc;
+}
+
+int geist_hip_sampler_row_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows) {
+    if (!s || !h_paths)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (rows > s->max_rows)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "rows %zu > max_rows %zu", rows, s->max_rows);
+    if (!s->cand.path)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "no full-vocabulary top-p / min-p call was made yet");
+    return geist_hip_download(s, h_paths, s->cand.path, rows * sizeof(int32_t));
 }
 
 } /* extern "C" */

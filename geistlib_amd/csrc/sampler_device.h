@@ -442,5 +442,13 @@ __device__ __forceinline__ float softmax_arg(float l, float mx, float inv_t) {
     return __fmul_rn(__fsub_rn(l, mx), inv_t);
 }
 
+/* z bin of an element: z = -(softmax argument) >= 0 in steps of 1/ZBIN_PER_NAT, truncated;
+ * -inf and everything past the last bin land in ZBINS - 1 or above (callers clamp or skip). The
+ * exp-sum pass and the candidate pass must agree on it bit for bit, hence one function. */
+__device__ __forceinline__ int zbin(float arg) {
+    const float z = __fmul_rn(arg, -(float) ZBIN_PER_NAT);
+    return z < (float) (ZBINS - 1) ? (int) z : ZBINS - 1;
+}
+
 } // namespace gs
 #endif

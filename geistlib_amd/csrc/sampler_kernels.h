@@ -41,7 +41,29 @@ struct Launch {
     hipStream_t stream;
 };
 
+/* Workspace of the candidate path of the full-vocabulary top-p / min-p modes. The exp-sum pass
+ * leaves, per chunk, the mass of the chunk's elements binned by z = (max - l) * inv_t in steps
+ * of 1/ZBIN_PER_NAT; a row the thread-maxima shortcut cannot serve derives from those (and from
+ * min_p) the last bin that can hold an element of its kept prefix, a third pass over the row
+ * lists the elements up to that bin with their normalised probabilities, and a row-final kernel
+ * works on the list. */
+constexpr int ZBINS        = 128;
+constexpr int ZBIN_PER_NAT = 4;
+constexpr int CAND_CAP     = 16384; /* list entries per row */
+constexpr int CAND_LDS     = 4096;  /* lists up to this length are staged in LDS */
+struct CandSpace {
+    float    *zhist;     /* [rows][chunks][ZBINS], NULL when top_p is off */
+    int32_t  *row_bound; /* [rows] last z bin listed */
+    uint32_t *out_key;   /* [rows] bits of a pn no element past that bin can exceed */
+    uint32_t *key;       /* [rows][CAND_CAP] bits of pn */
+    uint32_t *idx;       /* [rows][CAND_CAP] vocabulary ids */
+    int32_t  *count;     /* [rows] */
+    int32_t  *path;      /* [rows] which walk served the row: 1 thread-maxima shortcut, 2 list,
+                          * 3 whole row */
+};
+
 struct FinalLaunch {
+    CandSpace       cand;
     int             mode, k, k_sel;
     float           inv_t, top_p, min_p;
     const float    *uniforms;
@@ -54,9 +76,10 @@ struct FinalLaunch {
 
 /* probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
  * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
+/* zhist != NULL: also the per-chunk mass by z bin (see CandSpace) */
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p);
+                         float *probe_p, float *zhist);
 
 struct SpecLaunch {
     int             n_seq, L, greedy;
@@ -79,13 +102,16 @@ void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
-/* row_flag != NULL: only rows with a non-zero flag are written */
+/* rows flagged 1 by the sorted row-final kernel: list their candidates, then draw from the
+ * list; rows the list cannot serve are flagged 2 for the two kernels below */
+void launch_candidates(const Launch &L, const FinalLaunch &f);
+/* row_flag != NULL: only rows flagged 2 are written */
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
                         const double *chunk_sum, float *probs, long ld_probs,
                         const int32_t *row_flag);
 void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
                            float min_p, const float *uniforms, const int32_t *row_flag,
-                           int32_t *out);
+                           int32_t *out, int32_t *path);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

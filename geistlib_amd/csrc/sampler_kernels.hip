@@ -84,19 +84,23 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
  * Optionally records p at one token of the row (spec verification needs p(x_j)).
  * ========================================================================================== */
-template <int NV, bool PEN>
+template <int NV, bool PEN, bool HIST>
 __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       const uint64_t *__restrict__ chunk_best,
                                                       double *__restrict__ chunk_sum,
                                                       const int32_t *__restrict__ probe_token,
-                                                      int probe_L, float *__restrict__ probe_p) {
+                                                      int probe_L, float *__restrict__ probe_p,
+                                                      float *__restrict__ zhist) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
     __shared__ uint64_t s_tab[32];
+    __shared__ float    s_zh[HIST ? ZBINS : 1];
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
+    if (HIST && tid < ZBINS)
+        s_zh[tid] = 0.0f; /* visible after the barrier inside row_best_from_chunks() */
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
@@ -117,16 +121,26 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
-                const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
+                const float p   = geist_expf_glibc(arg, s_tab);
                 acc += (double) p;
                 if (e + c == tok)
                     probe_p[row] = p;
+                if (HIST) {
+                    /* the last bin and everything beyond weigh less than V * e^-31: left out,
+                     * and the bins only ever serve as a bound taken with a margin */
+                    const int zb = zbin(arg);
+                    if (zb < ZBINS - 1)
+                        atomicAdd(&s_zh[zb], p);
+                }
             }
         }
     }
-    acc = block_sum_f64(acc, s_sum);
+    acc = block_sum_f64(acc, s_sum); /* (its barriers also complete s_zh) */
     if (tid == 0)
         chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+    if (HIST && tid < ZBINS)
+        zhist[((long) row * rv.n_chunks + chunk) * ZBINS + tid] = s_zh[tid];
 }
 
 /* ============================================================================================
@@ -576,7 +590,9 @@ struct FinalArgs {
     const double   *chunk_sum;
     const float    *tmax;
     int32_t        *out;
-    int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to k_sorted_general */
+    int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to the candidate list,
+                               * 2 = to k_sorted_general */
+    CandSpace       cand;
 };
 
 /* ============================================================================================
@@ -938,9 +954,57 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big, s_mx,
                                                         s_wt, s_selid, s_pcnt, s_m, s_srt, &s_n,
                                                         &s_n2, s_tab);
+    if (tok >= 0) {
+        if (tid == 0) {
+            a.row_flag[row]  = 0;
+            a.out[row]       = tok;
+            a.cand.path[row] = 1;
+        }
+        return;
+    }
+    /* The shortcut could not serve the row. Last z bin that can hold an element of the kept
+     * prefix: top-p from the binned mass of the exp-sum pass (a little more than top_p of the
+     * sum must lie at or before it), min-p in closed form (pn_i >= min_p * pn_0 needs
+     * z_i <= -ln(min_p), taken with slack); both set: the shorter prefix, so the smaller bin. */
+    __syncthreads();
+    float *s_zh = s_wt; /* TPB floats, free again */
+    if (a.cand.zhist && tid < ZBINS) {
+        const float *zh = a.cand.zhist + (long) row * C * ZBINS + tid;
+        float        h  = 0.0f;
+        for (int c = 0; c < C; ++c)
+            h += zh[(long) c * ZBINS];
+        s_zh[tid] = h;
+    }
+    __syncthreads();
     if (tid == 0) {
-        a.row_flag[row] = tok < 0 ? 1 : 0;
-        a.out[row]      = tok;
+        int B = ZBINS - 1;
+        if (a.top_p > 0.0f && a.top_p < 1.0f && a.cand.zhist) {
+            const double need = (double) a.top_p * sum * 1.0002;
+            double       cum  = 0.0;
+            for (int b = 0; b < ZBINS - 1; ++b) {
+                cum += (double) s_zh[b];
+                if (cum >= need) {
+                    B = b;
+                    break;
+                }
+            }
+        }
+        if (a.min_p > 0.0f) {
+            const double z_m = -log((double) a.min_p) + 2e-3;
+            const int    b_m = z_m * ZBIN_PER_NAT < (double) (ZBINS - 1) ? (int) (z_m * ZBIN_PER_NAT)
+                                                                         : ZBINS - 1;
+            B = b_m < B ? b_m : B;
+        }
+        /* an element outside the list has z >= (B + 1) / ZBIN_PER_NAT (the product in zbin() is
+         * exact), so its p is at most expf of minus that; one step up covers any non-monotonic
+         * last bit of expf or of the division */
+        const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+        const float pn_out = (float) ((double) p_out / sum);
+        a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
+        a.cand.row_bound[row] = B;
+        a.cand.count[row]     = 0;
+        a.row_flag[row]       = B < ZBINS - 1 ? 1 : 2;
+        a.out[row]            = -1;
     }
 }
 
@@ -1020,7 +1084,7 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
     __shared__ uint64_t s_tab[32];
     __shared__ double   s_total;
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
-    if (row_flag && !row_flag[row])
+    if (row_flag && row_flag[row] != 2)
         return; /* only the rows that asked for their probabilities */
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
@@ -1132,11 +1196,15 @@ static void dispatch(int nv, bool pen, F &&f) {
 
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p) {
+                         float *probe_p, float *zhist) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_chunk_expsum<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
-            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p);
+        if (zhist)
+            k_chunk_expsum<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, zhist);
+        else
+            k_chunk_expsum<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, nullptr);
     });
 }
 
@@ -1193,6 +1261,7 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.tmax       = f.tmax;
     a.row_flag   = f.row_flag;
     a.out        = f.out;
+    a.cand       = f.cand;
     const dim3 grid(L.rows), block(TPB);
     if (f.mode == FINAL_ARGMAX) {
         k_final_argmax<<<grid, block, 0, L.stream>>>(L.rv, a);
@@ -1247,11 +1316,21 @@ void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best
     });
 }
 
+void launch_candidates(const Launch &L, const FinalLaunch &f) {
+    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
+        k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
+            L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
+    });
+    k_sorted_candidates<<<dim3(L.rows), block, 0, L.stream>>>(f.cand, f.top_p, f.min_p, f.uniforms,
+                                                             f.row_flag, f.out);
+}
+
 void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
                            float min_p, const float *uniforms, const int32_t *row_flag,
-                           int32_t *out) {
-    k_sorted_general<<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(probs, ld_probs, L.rv.n_vocab, top_p,
-                                                               min_p, uniforms, row_flag, out);
+                           int32_t *out, int32_t *path) {
+    k_sorted_general<<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(
+        probs, ld_probs, L.rv.n_vocab, top_p, min_p, uniforms, row_flag, out, path);
 }
 
 void launch_penalties(const Launch &L, float *logits_rw) {

@@ -484,21 +484,73 @@ __device__ bool sg_descent(const float *pn, int n, uint64_t target, bool limited
     return true;
 }
 
-__global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict__ probs,
-                                                        long ld_probs, int n, float top_p,
-                                                        float min_p,
-                                                        const float *__restrict__ uniforms,
-                                                        const int32_t *__restrict__ row_flag,
-                                                        int32_t *__restrict__ out) {
-    __shared__ SortedGenShared sh;
-    __shared__ int             s_scan[NWAVES];
-    __shared__ int             s_pick;
-    const int row = blockIdx.x, tid = threadIdx.x;
-    if (!row_flag[row])
-        return;
-    const float *pn    = probs + (long) row * ld_probs;
-    const bool   use_p = top_p > 0.0f && top_p < 1.0f;
-    const bool   use_m = min_p > 0.0f;
+/* The j-th smallest id among the list entries whose key equals `key`, ids < 2^21: two counting
+ * passes over the bits of the id (the list is in no particular order). */
+__device__ int list_jth_id(const float *pn, const uint32_t *ids, int n, uint32_t key, int j,
+                           SortedGenShared &sh, int *s_scan, int *s_pick) {
+    const int tid    = threadIdx.x;
+    uint32_t  prefix = 0u;
+    int       want   = j; /* 1-based rank inside the current digit range */
+    for (int lv = 0; lv < 2; ++lv) {
+        const int shf = lv == 0 ? 10 : 0;
+        for (int i = tid; i < SG_BINS; i += TPB)
+            sh.cnt[i] = 0u;
+        if (tid == 0)
+            *s_pick = -1;
+        __syncthreads();
+        for (int i = tid; i < n; i += TPB) {
+            if (__float_as_uint(pn[i]) != key)
+                continue;
+            const uint32_t id = ids[i];
+            if (lv == 1 && (id >> 10) != prefix)
+                continue;
+            atomicAdd(&sh.cnt[lv == 0 ? (id >> 10) & (SG_BINS - 1) : id & 1023u], 1u);
+        }
+        __syncthreads();
+        constexpr int PER = SG_BINS / TPB; /* ascending digits */
+        int           mine = 0;
+#pragma unroll
+        for (int q = 0; q < PER; ++q)
+            mine += (int) sh.cnt[tid * PER + q];
+        const int incl = block_scan_i32(mine, s_scan, nullptr);
+        int       run  = incl - mine;
+        if (run < want && incl >= want) {
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const int c = (int) sh.cnt[tid * PER + q];
+                if (run < want && run + c >= want) {
+                    *s_pick       = tid * PER + q;
+                    sh.res_digit  = run;
+                }
+                run += c;
+            }
+        }
+        __syncthreads();
+        const int d = *s_pick;
+        if (d < 0)
+            return -1;
+        want -= sh.res_digit;
+        if (lv == 0)
+            prefix = (uint32_t) d;
+        else
+            prefix = (prefix << 10) | (uint32_t) d;
+        __syncthreads();
+    }
+    return (int) prefix;
+}
+
+/* The walk of sampler.c:270-299 (plus min-p) over n normalised probabilities without sorting
+ * them. LIST = false: pn[] is a whole row in index order. LIST = true: pn[]/ids[] list, in any
+ * order, every entry of the row up to some z bin; no entry outside the list has a pn whose bits
+ * exceed `kout`, so the walk is exact as long as the kept prefix ends strictly above kout --
+ * otherwise -1 is returned and the row is walked in full. */
+template <bool LIST>
+__device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float top_p, float min_p,
+                              float u, uint32_t kout, SortedGenShared &sh, int *s_scan,
+                              int *s_pick) {
+    const int  tid   = threadIdx.x;
+    const bool use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool use_m = min_p > 0.0f;
 
     /* largest probability, then the min-p prefix: count and mass of pn >= min_p * pn_0 */
     uint32_t kmax = 0u;
@@ -555,6 +607,8 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict_
     if (use_m && (!have_p || n_m < n_keep)) {
         /* the min-p prefix is the shorter one: every entry with pn >= floor, ties included */
         const float floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
+        if (LIST && __float_as_uint(floor_w) <= kout)
+            return -1; /* entries outside the list may pass the floor too */
         limited   = true;
         n_keep    = n_m;
         mass_keep = mass_m;
@@ -563,8 +617,13 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict_
         edge_ties = 0u;
         if (__float_as_uint(floor_w) == 0u)
             limited = false;
-    } else if (!have_p) {
-        /* neither filter bites (top_p not reached by the whole row): the whole row is kept */
+    } else if (have_p) {
+        if (LIST && edge_key <= kout)
+            return -1; /* the nucleus may end among entries outside the list */
+    } else {
+        /* neither filter bites (top_p not reached by all n entries) */
+        if (LIST)
+            return -1;
         uint64_t lm = 0;
         for (int i = tid; i < n; i += TPB)
             lm += pn_fx(pn[i]);
@@ -573,8 +632,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict_
     }
     /* the draw: first entry of the kept prefix at which the running mass exceeds u * mass */
     /* running mass > u * mass  <=>  running mass >= floor(u * mass) + 1 in integers */
-    const uint64_t target2 =
-        (uint64_t) __double2ull_rd((double) uniforms[row] * (double) mass_keep) + 1ull;
+    const uint64_t target2 = (uint64_t) __double2ull_rd((double) u * (double) mass_keep) + 1ull;
     uint32_t       kd, cnt_above_d, ties_d;
     uint64_t       mass_above_d;
     int32_t        tok = -1;
@@ -586,44 +644,174 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict_
             j = 1;
         if (j > ties_d)
             j = ties_d;
-        /* the j-th entry (index order) with pn == kd: each thread takes a contiguous range */
-        const int span = (n + TPB - 1) / TPB;
-        const int lo   = tid * span < n ? tid * span : n;
-        const int hi   = lo + span < n ? lo + span : n;
-        int       mine = 0;
-        for (int i = lo; i < hi; ++i)
-            mine += __float_as_uint(pn[i]) == kd;
-        const int incl = block_scan_i32(mine, s_scan, nullptr);
-        if (tid == 0)
-            s_pick = -1;
-        __syncthreads();
-        if (incl >= (int) j && incl - mine < (int) j) {
-            int seen = incl - mine;
-            for (int i = lo; i < hi; ++i) {
-                if (__float_as_uint(pn[i]) == kd && ++seen == (int) j) {
-                    s_pick = i;
-                    break;
+        if (LIST) {
+            tok = list_jth_id(pn, ids, n, kd, (int) j, sh, s_scan, s_pick);
+        } else {
+            /* the j-th entry (index order) with pn == kd: each thread takes a contiguous range */
+            const int span = (n + TPB - 1) / TPB;
+            const int lo   = tid * span < n ? tid * span : n;
+            const int hi   = lo + span < n ? lo + span : n;
+            int       mine = 0;
+            for (int i = lo; i < hi; ++i)
+                mine += __float_as_uint(pn[i]) == kd;
+            const int incl = block_scan_i32(mine, s_scan, nullptr);
+            if (tid == 0)
+                *s_pick = -1;
+            __syncthreads();
+            if (incl >= (int) j && incl - mine < (int) j) {
+                int seen = incl - mine;
+                for (int i = lo; i < hi; ++i) {
+                    if (__float_as_uint(pn[i]) == kd && ++seen == (int) j) {
+                        *s_pick = i;
+                        break;
+                    }
                 }
             }
+            __syncthreads();
+            tok = *s_pick;
+            __syncthreads();
         }
-        __syncthreads();
-        tok = s_pick;
     }
-    if (tok < 0) {
+    if (tok < 0 && !LIST) {
         /* not reachable with exact integer masses (the target never exceeds the kept mass);
          * kept as a defined outcome: the most probable entry */
         if (tid == 0)
-            s_pick = 0x7fffffff;
+            *s_pick = 0x7fffffff;
         __syncthreads();
         for (int i = tid; i < n; i += TPB)
             if (__float_as_uint(pn[i]) == kmax)
-                atomicMin(&s_pick, i);
+                atomicMin(s_pick, i);
         __syncthreads();
-        tok = s_pick == 0x7fffffff ? 0 : s_pick;
+        tok = *s_pick == 0x7fffffff ? 0 : *s_pick;
     }
-    if (tid == 0)
-        out[row] = tok;
     (void) n_keep;
+    return tok;
+}
+
+__global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict__ probs,
+                                                        long ld_probs, int n, float top_p,
+                                                        float min_p,
+                                                        const float *__restrict__ uniforms,
+                                                        const int32_t *__restrict__ row_flag,
+                                                        int32_t *__restrict__ out,
+                                                        int32_t *__restrict__ path) {
+    __shared__ SortedGenShared sh;
+    __shared__ int             s_scan[NWAVES];
+    __shared__ int             s_pick;
+    const int row = blockIdx.x;
+    if (row_flag[row] != 2)
+        return;
+    const int tok = sorted_descend<false>(probs + (long) row * ld_probs, nullptr, n, top_p, min_p,
+                                          uniforms[row], 0u, sh, s_scan, &s_pick);
+    if (threadIdx.x == 0) {
+        out[row]  = tok;
+        path[row] = 3;
+    }
+}
+
+/* ============================================================================================
+ * k_list_candidates: third pass over the rows flagged 1. Every element whose z bin is at or
+ * before the row's bound is appended, in no particular order, to the row's list as (bits of its
+ * normalised probability pn = (float)((double)p / sum), vocabulary id). A list longer than
+ * CAND_CAP keeps counting; the row-final kernel then hands the row on.
+ * ========================================================================================== */
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t,
+                                                         const uint64_t *__restrict__ chunk_best,
+                                                         const double *__restrict__ chunk_sum,
+                                                         const int32_t *__restrict__ row_flag,
+                                                         CandSpace cand) {
+    static_assert(4 * NV <= 32, "one mask bit per element of a thread");
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ uint64_t s_red[NWAVES];
+    __shared__ uint64_t s_tab[32];
+    __shared__ double   s_total;
+    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    if (row_flag[row] != 1)
+        return;
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    if (tid == 0) {
+        double t = 0.0;
+        for (int c = 0; c < rv.n_chunks; ++c)
+            t += chunk_sum[(long) row * rv.n_chunks + c];
+        s_total = t;
+    }
+    int base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    float4 v[NV];
+    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
+    const float  mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
+    const double tot = s_total;
+    const int    B   = cand.row_bound[row];
+    uint32_t     mask = 0u;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const bool in = e + c < end && zbin(softmax_arg(f4_get(v[j], c), mx, inv_t)) <= B;
+            mask |= (uint32_t) in << (4 * j + c);
+        }
+    }
+    int       pos = wave_reserve(__popc(mask), &cand.count[row]);
+    uint32_t *ck  = cand.key + (long) row * CAND_CAP;
+    uint32_t *ci  = cand.idx + (long) row * CAND_CAP;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if ((mask >> (4 * j + c)) & 1u) {
+                if (pos < CAND_CAP) {
+                    const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                    ck[pos]       = __float_as_uint((float) ((double) p / tot));
+                    ci[pos]       = (uint32_t) (e + c);
+                }
+                ++pos;
+            }
+        }
+    }
+}
+
+/* k_sorted_candidates: one workgroup per row flagged 1 walks the row's list (staged in LDS when
+ * it fits). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
+ * prefix that may reach past the list -- is flagged 2 for k_sorted_general. */
+__global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float top_p, float min_p,
+                                                           const float *__restrict__ uniforms,
+                                                           int32_t *__restrict__ row_flag,
+                                                           int32_t *__restrict__ out) {
+    __shared__ SortedGenShared sh;
+    __shared__ int             s_scan[NWAVES];
+    __shared__ int             s_pick;
+    __shared__ uint32_t        s_key[CAND_LDS];
+    __shared__ uint32_t        s_idx[CAND_LDS];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    if (row_flag[row] != 1)
+        return;
+    const int n   = cand.count[row];
+    int       tok = -1;
+    if (n >= 1 && n <= CAND_CAP) {
+        const uint32_t *gk = cand.key + (long) row * CAND_CAP;
+        const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
+        if (n <= CAND_LDS) {
+            for (int i = tid; i < n; i += TPB) {
+                s_key[i] = gk[i];
+                s_idx[i] = gi[i];
+            }
+            __syncthreads();
+            gk = s_key;
+            gi = s_idx;
+        }
+        tok = sorted_descend<true>(reinterpret_cast<const float *>(gk), gi, n, top_p, min_p,
+                                   uniforms[row], cand.out_key[row], sh, s_scan, &s_pick);
+    }
+    if (tid == 0) {
+        row_flag[row] = tok < 0 ? 2 : 0;
+        out[row]      = tok;
+        if (tok >= 0)
+            cand.path[row] = 2;
+    }
 }
 
 } // namespace gs

@@ -165,6 +165,11 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
                                          const float *d_uniforms, geist_hip_token_t *d_out_tokens,
                                          int launches, double *ms_total);
 
+/* Diagnostics (no reference counterpart): after a full-vocabulary top-p / min-p call, which walk
+ * served each row: 1 = shortcut over the per-thread maxima, 2 = candidate list, 3 = the whole
+ * row. Synchronous; h_paths receives `rows` entries. */
+int geist_hip_sampler_row_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -227,6 +227,64 @@ def test_min_p_and_top_p_chain(hs, oracle, n, scale, T, p, m):
     assert near <= 1
 
 
+@pytest.mark.parametrize("n,scale,T,p,m", [(128256, 3.0, 1.0, 0.9, 0.0), (151936, 2.0, 1.0, 0.95, 0.05),
+                                           (50000, 2.5, 1.0, 0.8, 0.0), (262144, 3.0, 1.0, 0.9, 0.0),
+                                           (128256, 2.0, 1.0, 1.0, 0.02), (20000, 2.0, 1.0, 0.6, 0.0)])
+def test_top_p_candidate_list_path(hs, oracle, n, scale, T, p, m):
+    """Kept prefixes of hundreds to thousands of entries: too many for the thread-maxima shortcut,
+    few enough to be listed by a third pass and walked from the list. Row 1 is quantised, so
+    many list entries share one probability and the draw has to respect index order among them."""
+    print(f"top-p list n={n} p={p} m={m}", flush=True)
+    x, u = rows_rng(n + 17, 10, n, scale=scale)
+    x[1] = np.round(x[1] * 4) / 4
+    got = run_rows(hs, torch, x, u, P(temperature=T, top_p=p, min_p=m))
+    paths = hs.row_paths(x.shape[0])
+    res = [oracle.chain_u(x[r], float(u[r]), temperature=T, top_p=p, min_p=m)
+           for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-p list n={n}")
+    assert near <= 1
+    assert set(paths.tolist()) <= {1, 2, 3}
+    assert (paths == 2).sum() >= 6, f"paths {paths.tolist()}, kept {[i.n_keep for _, i in res]}"
+
+
+def test_top_p_vocabulary_beyond_the_shortcut(oracle):
+    """More than 32 chunks of 8192: the thread-maxima shortcut is not attempted at all."""
+    from geistlib_amd import HipSampler
+    n = 300000
+    big = HipSampler(max_rows=4, max_vocab=n)
+    try:
+        x, u = rows_rng(321, 4, n, scale=3.0)
+        x[3] *= 0.1
+        got = run_rows(big, torch, x, u, P(temperature=1.0, top_p=0.9, precedence=0))
+        paths = big.row_paths(4).tolist()
+    finally:
+        big.close()
+    res = [oracle.top_p_u(x[r], 0.9, 1.0, float(u[r])) for r in range(4)]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "top-p n=300000")
+    assert near <= 1
+    assert paths == [2, 2, 2, 3], paths
+
+
+def test_sorted_paths_all_three_in_one_batch(hs, oracle):
+    """One batch whose rows need the shortcut, the list and the whole-row walk."""
+    n = 100000
+    g = np.random.default_rng(99)
+    x = np.empty((6, n), dtype=np.float32)
+    x[0] = g.standard_normal(n) * 6            # peaked: shortcut
+    x[1] = g.standard_normal(n) * 6
+    x[2] = g.standard_normal(n) * 3            # hundreds kept: list
+    x[3] = g.standard_normal(n) * 3
+    x[4] = g.standard_normal(n) * 0.5          # tens of thousands kept: whole row
+    x[5] = 1.0                                 # all equal
+    u = g.random(6).astype(np.float32)
+    got = run_rows(hs, torch, x, u, P(temperature=1.0, top_p=0.9, precedence=0))
+    paths = hs.row_paths(6).tolist()
+    res = [oracle.top_p_u(x[r], 0.9, 1.0, float(u[r])) for r in range(6)]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "three paths")
+    assert near <= 1
+    assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
+
+
 def test_top_p_limits_match_reference_dispatch(hs, oracle):
     x, u = rows_rng(5, 6, 3000)
     for p in (0.0, -1.0, 1.0, 1.5):        # sampler.c:238-243: <= 0 -> argmax... but the session
