@@ -194,7 +194,6 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
-    (void) hipFree(s->cand.zhist);
     (void) hipFree(s->cand.row_bound);
     (void) hipFree(s->cand.out_key);
     (void) hipFree(s->cand.key);
@@ -343,7 +342,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (!rs.use_p && !rs.use_m) {
         if (!stream_only(s))
             launch_tmax_scan(L, s->tmax, s->chunk_best);
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr);
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
         if (stream_only(s))
             return after_launch(s, "exp-sum scan");
         f.mode = FINAL_TEMPERATURE;
@@ -353,7 +352,6 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     /* top-p and/or min-p over the whole vocabulary */
     if (!s->probs) {
         const size_t R = s->max_rows;
-        HIPCHK(s, hipMalloc((void **) &s->cand.zhist, R * s->max_chunks * ZBINS * sizeof(float)));
         HIPCHK(s, hipMalloc((void **) &s->cand.row_bound, R * sizeof(int32_t)));
         HIPCHK(s, hipMalloc((void **) &s->cand.out_key, R * sizeof(uint32_t)));
         HIPCHK(s, hipMalloc((void **) &s->cand.key, R * CAND_CAP * sizeof(uint32_t)));
@@ -371,9 +369,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (!stream_only(s))
         launch_tmax_scan(L, s->tmax, s->chunk_best);
     f.cand = s->cand;
-    if (!rs.use_p)
-        f.cand.zhist = nullptr; /* the min-p bound needs no binned mass */
-    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, f.cand.zhist);
+    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
     if (stream_only(s))
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;
@@ -487,7 +483,7 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
     launch_tmax_scan(L, s->tmax, s->chunk_best);
-    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr);
+    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
 }
@@ -525,7 +521,7 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     const float inv_t = greedy ? 1.0f : 1.0f / temperature;
     launch_tmax_scan(La, s->tmax, s->chunk_best);
     if (!greedy)
-        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p, nullptr);
+        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p);
     SpecLaunch sp{};
     sp.n_seq      = (int) n_seq;
     sp.L          = (int) L;

@@ -41,18 +41,16 @@ struct Launch {
     hipStream_t stream;
 };
 
-/* Workspace of the candidate path of the full-vocabulary top-p / min-p modes. The exp-sum pass
- * leaves, per chunk, the mass of the chunk's elements binned by z = (max - l) * inv_t in steps
- * of 1/ZBIN_PER_NAT; a row the thread-maxima shortcut cannot serve derives from those (and from
- * min_p) the last bin that can hold an element of its kept prefix, a third pass over the row
- * lists the elements up to that bin with their normalised probabilities, and a row-final kernel
- * works on the list. */
+/* Workspace of the candidate path of the full-vocabulary top-p / min-p modes. Elements are
+ * binned by z = (max - l) * inv_t in steps of 1/ZBIN_PER_NAT; a row the thread-maxima shortcut
+ * cannot serve derives (from the binned mass of its thread maxima and from min_p) the last bin
+ * that can hold an element of its kept prefix, a third pass over the row lists the elements up
+ * to that bin with their normalised probabilities, and a row-final kernel works on the list. */
 constexpr int ZBINS        = 128;
 constexpr int ZBIN_PER_NAT = 4;
 constexpr int CAND_CAP     = 16384; /* list entries per row */
 constexpr int CAND_LDS     = 4096;  /* lists up to this length are staged in LDS */
 struct CandSpace {
-    float    *zhist;     /* [rows][chunks][ZBINS], NULL when top_p is off */
     int32_t  *row_bound; /* [rows] last z bin listed */
     uint32_t *out_key;   /* [rows] bits of a pn no element past that bin can exceed */
     uint32_t *key;       /* [rows][CAND_CAP] bits of pn */
@@ -76,10 +74,9 @@ struct FinalLaunch {
 
 /* probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
  * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
-/* zhist != NULL: also the per-chunk mass by z bin (see CandSpace) */
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, float *zhist);
+                         float *probe_p);
 
 struct SpecLaunch {
     int             n_seq, L, greedy;

@@ -84,23 +84,19 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
  * Optionally records p at one token of the row (spec verification needs p(x_j)).
  * ========================================================================================== */
-template <int NV, bool PEN, bool HIST>
+template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       const uint64_t *__restrict__ chunk_best,
                                                       double *__restrict__ chunk_sum,
                                                       const int32_t *__restrict__ probe_token,
-                                                      int probe_L, float *__restrict__ probe_p,
-                                                      float *__restrict__ zhist) {
+                                                      int probe_L, float *__restrict__ probe_p) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
     __shared__ uint64_t s_tab[32];
-    __shared__ float    s_zh[HIST ? ZBINS : 1];
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
-    if (HIST && tid < ZBINS)
-        s_zh[tid] = 0.0f; /* visible after the barrier inside row_best_from_chunks() */
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
@@ -121,26 +117,16 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
-                const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
-                const float p   = geist_expf_glibc(arg, s_tab);
+                const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
                 acc += (double) p;
                 if (e + c == tok)
                     probe_p[row] = p;
-                if (HIST) {
-                    /* the last bin and everything beyond weigh less than V * e^-31: left out,
-                     * and the bins only ever serve as a bound taken with a margin */
-                    const int zb = zbin(arg);
-                    if (zb < ZBINS - 1)
-                        atomicAdd(&s_zh[zb], p);
-                }
             }
         }
     }
-    acc = block_sum_f64(acc, s_sum); /* (its barriers also complete s_zh) */
+    acc = block_sum_f64(acc, s_sum);
     if (tid == 0)
         chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
-    if (HIST && tid < ZBINS)
-        zhist[((long) row * rv.n_chunks + chunk) * ZBINS + tid] = s_zh[tid];
 }
 
 /* ============================================================================================
@@ -962,29 +948,57 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         }
         return;
     }
-    /* The shortcut could not serve the row. Last z bin that can hold an element of the kept
-     * prefix: top-p from the binned mass of the exp-sum pass (a little more than top_p of the
-     * sum must lie at or before it), min-p in closed form (pn_i >= min_p * pn_0 needs
-     * z_i <= -ln(min_p), taken with slack); both set: the shorter prefix, so the smaller bin. */
+    /* The shortcut could not serve the row. Last z bin (z = (max - l) * inv_t) that can hold an
+     * element of the kept prefix.
+     *   top-p: estimated from ALL the row's thread maxima, binned by z with fast exponentials as
+     *   weights. Where M of the T scanning threads have their maximum above a value, about
+     *   -T ln(1 - M/T) elements lie above it if the vocabulary order is unrelated to the logits
+     *   (each element beyond a thread's first hides behind that thread's maximum), so a bin's
+     *   mass is scaled by 1 / (1 - M/T) at the bin. The first bin at which the scaled mass
+     *   passes top_p plus a quarter of the rest, and one more bin, is taken. It is an estimate:
+     *   the walk over the list sums the listed mass exactly and hands the row on to the
+     *   whole-row walk when the kept prefix is not certainly inside the list.
+     *   min-p: pn_i >= min_p * pn_0 needs z_i <= -ln(min_p), in closed form, taken with slack.
+     *   Both set: the shorter prefix, so the smaller bin. */
     __syncthreads();
-    float *s_zh = s_wt; /* TPB floats, free again */
-    if (a.cand.zhist && tid < ZBINS) {
-        const float *zh = a.cand.zhist + (long) row * C * ZBINS + tid;
-        float        h  = 0.0f;
-        for (int c = 0; c < C; ++c)
-            h += zh[(long) c * ZBINS];
-        s_zh[tid] = h;
+    float     *s_zh   = s_wt;                           /* TPB floats, free again */
+    int       *s_zc   = reinterpret_cast<int *>(s_mx);  /* TPB words, free again */
+    const bool want_p = a.top_p > 0.0f && a.top_p < 1.0f;
+    if (tid < ZBINS) {
+        s_zh[tid] = 0.0f;
+        s_zc[tid] = 0;
+    }
+    __syncthreads();
+    if (want_p) {
+        const float *tm = a.tmax + (long) row * C * TPB + tid;
+        for (int q = 0; q < C; ++q) {
+            const float t = tm[(long) q * TPB];
+            if (t != t)
+                continue; /* a thread without an element of the row */
+            const float arg = softmax_arg(t, mx, a.inv_t);
+            const int   zb  = zbin(arg);
+            atomicAdd(&s_zc[zb], 1);
+            if (zb < ZBINS - 1)
+                unsafeAtomicAdd(&s_zh[zb], __expf(arg));
+        }
     }
     __syncthreads();
     if (tid == 0) {
         int B = ZBINS - 1;
-        if (a.top_p > 0.0f && a.top_p < 1.0f && a.cand.zhist) {
-            const double need = (double) a.top_p * sum * 1.0002;
+        if (want_p) {
+            int T = 0;
+            for (int b = 0; b < ZBINS; ++b)
+                T += s_zc[b];
+            const double need = ((double) a.top_p + 0.25 * (1.0 - (double) a.top_p)) * sum;
             double       cum  = 0.0;
+            int          M    = 0;
             for (int b = 0; b < ZBINS - 1; ++b) {
-                cum += (double) s_zh[b];
+                const double mid  = (double) M + 0.5 * (double) s_zc[b];
+                const double left = 1.0 - mid / (double) (T > 0 ? T : 1);
+                cum += (double) s_zh[b] / (left > 0.05 ? left : 0.05);
+                M += s_zc[b];
                 if (cum >= need) {
-                    B = b;
+                    B = b + 1 < ZBINS - 1 ? b + 1 : b;
                     break;
                 }
             }
@@ -1196,15 +1210,11 @@ static void dispatch(int nv, bool pen, F &&f) {
 
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, float *zhist) {
+                         float *probe_p) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        if (zhist)
-            k_chunk_expsum<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, zhist);
-        else
-            k_chunk_expsum<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, nullptr);
+        k_chunk_expsum<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
+            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p);
     });
 }
 

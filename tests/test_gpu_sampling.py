@@ -228,7 +228,7 @@ def test_min_p_and_top_p_chain(hs, oracle, n, scale, T, p, m):
 
 
 @pytest.mark.parametrize("n,scale,T,p,m", [(128256, 3.0, 1.0, 0.9, 0.0), (151936, 2.0, 1.0, 0.95, 0.05),
-                                           (50000, 2.5, 1.0, 0.8, 0.0), (262144, 3.0, 1.0, 0.9, 0.0),
+                                           (50000, 2.5, 1.0, 0.8, 0.0), (262144, 3.6, 1.0, 0.9, 0.0),
                                            (128256, 2.0, 1.0, 1.0, 0.02), (20000, 2.0, 1.0, 0.6, 0.0)])
 def test_top_p_candidate_list_path(hs, oracle, n, scale, T, p, m):
     """Kept prefixes of hundreds to thousands of entries: too many for the thread-maxima shortcut,
@@ -253,7 +253,7 @@ def test_top_p_vocabulary_beyond_the_shortcut(oracle):
     n = 300000
     big = HipSampler(max_rows=4, max_vocab=n)
     try:
-        x, u = rows_rng(321, 4, n, scale=3.0)
+        x, u = rows_rng(321, 4, n, scale=4.0)
         x[3] *= 0.1
         got = run_rows(big, torch, x, u, P(temperature=1.0, top_p=0.9, precedence=0))
         paths = big.row_paths(4).tolist()
