@@ -199,6 +199,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->cand.key);
     (void) hipFree(s->cand.idx);
     (void) hipFree(s->cand.count);
+    (void) hipFree(s->cand.row_sum);
     (void) hipFree(s->cand.path);
     if (s->h_scalar)
         (void) hipHostFree(s->h_scalar);
@@ -357,6 +358,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         HIPCHK(s, hipMalloc((void **) &s->cand.key, R * CAND_CAP * sizeof(uint32_t)));
         HIPCHK(s, hipMalloc((void **) &s->cand.idx, R * CAND_CAP * sizeof(uint32_t)));
         HIPCHK(s, hipMalloc((void **) &s->cand.count, R * sizeof(int32_t)));
+        HIPCHK(s, hipMalloc((void **) &s->cand.row_sum, R * sizeof(double)));
         HIPCHK(s, hipMalloc((void **) &s->cand.path, R * sizeof(int32_t)));
         HIPCHK(s, hipMalloc((void **) &s->probs, R * s->max_vocab * sizeof(float)));
     }
@@ -366,10 +368,16 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (L.rv.n_chunks > s->max_chunks)
         return fail(s, GEIST_HIP_E_UNSUPPORTED, "n_vocab %zu needs more than %d chunks",
                     rows->n_vocab, s->max_chunks);
+    /* min-p bounds the kept prefix by the row maximum alone, so the exp-sum pass can list the
+     * candidates on its way; rows whose list overflows fall back to the bound of the row-final
+     * kernel and a third pass */
+    const int zb_m    = zbin_of_min_p(rs.min_p);
+    f.cand            = s->cand;
+    f.minp_listed     = rs.use_m && zb_m < ZBINS - 1;
     if (!stream_only(s))
-        launch_tmax_scan(L, s->tmax, s->chunk_best);
-    f.cand = s->cand;
-    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+        launch_tmax_scan(L, s->tmax, s->chunk_best, f.minp_listed ? s->cand.count : nullptr);
+    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
+                        f.minp_listed && !stream_only(s) ? &f.cand : nullptr, zb_m);
     if (stream_only(s))
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;

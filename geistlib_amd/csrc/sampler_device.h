@@ -118,6 +118,20 @@ __device__ __forceinline__ int wave_scan_i32_dpp(int v) {
     v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); /* row_bcast:31 -> rows 2, 3 */
     return v;
 }
+/* Sum of a float over the wavefront by the same DPP steps; every lane receives the total
+ * (the order of the additions is fixed, so equal inputs give equal sums). */
+__device__ __forceinline__ float wave_sum_f32_dpp(float v) {
+#define GS_DPP_F32(ctrl, rows) \
+    __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rows, 0xf, false))
+    v += GS_DPP_F32(0x111, 0xf);
+    v += GS_DPP_F32(0x112, 0xf);
+    v += GS_DPP_F32(0x114, 0xf);
+    v += GS_DPP_F32(0x118, 0xf);
+    v += GS_DPP_F32(0x142, 0xa);
+    v += GS_DPP_F32(0x143, 0xc);
+#undef GS_DPP_F32
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), WAVE - 1));
+}
 /* The same for doubles: both halves travel by DPP, lanes without a source add 0.0. */
 template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ double dpp_fetch_f64(double v) {

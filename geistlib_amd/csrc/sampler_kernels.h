@@ -56,12 +56,14 @@ struct CandSpace {
     uint32_t *key;       /* [rows][CAND_CAP] bits of pn */
     uint32_t *idx;       /* [rows][CAND_CAP] vocabulary ids */
     int32_t  *count;     /* [rows] */
+    double   *row_sum;   /* [rows] the row's exp-sum, for lists that hold p instead of pn */
     int32_t  *path;      /* [rows] which walk served the row: 1 thread-maxima shortcut, 2 list,
                           * 3 whole row */
 };
 
 struct FinalLaunch {
     CandSpace       cand;
+    bool            minp_listed; /* the exp-sum pass already listed the rows under the min-p bound */
     int             mode, k, k_sel;
     float           inv_t, top_p, min_p;
     const float    *uniforms;
@@ -74,9 +76,15 @@ struct FinalLaunch {
 
 /* probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
  * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
+/* list != NULL (min-p set): the pass also lists, per row, every element up to z bin zb_list with
+ * its unnormalised p -- the min-p bound needs nothing but the row maximum. list->count must be
+ * zero on entry (launch_tmax_scan can clear it). */
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p);
+                         float *probe_p, const CandSpace *list = nullptr, int zb_list = 0);
+/* last z bin that can hold an entry passing min_p (with slack); ZBINS - 1 when min_p is off or
+ * that deep */
+int zbin_of_min_p(float min_p);
 
 struct SpecLaunch {
     int             n_seq, L, greedy;
@@ -95,7 +103,8 @@ struct SpecLaunch {
 constexpr int SPEC_DRAFT_MAX = 63;
 void launch_spec(const Launch &L, const SpecLaunch &sp);
 /* chunk_best may be NULL when only the thread maxima are wanted */
-void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best);
+void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best,
+                      int32_t *zero_per_row = nullptr);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);

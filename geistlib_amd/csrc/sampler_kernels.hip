@@ -21,6 +21,7 @@
 
 #include "sampler_device.h"
 
+#include <cmath>
 #include <type_traits>
 
 namespace gs {
@@ -84,16 +85,19 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
  * Optionally records p at one token of the row (spec verification needs p(x_j)).
  * ========================================================================================== */
-template <int NV, bool PEN>
+template <int NV, bool PEN, bool LISTM>
 __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       const uint64_t *__restrict__ chunk_best,
                                                       double *__restrict__ chunk_sum,
                                                       const int32_t *__restrict__ probe_token,
-                                                      int probe_L, float *__restrict__ probe_p) {
+                                                      int probe_L, float *__restrict__ probe_p,
+                                                      CandSpace list, int zb_list) {
+    static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
     __shared__ uint64_t s_tab[32];
+    __shared__ int      s_listed, s_base;
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
@@ -110,23 +114,55 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
         if (j < probe_L)
             tok = probe_token[(long) (row / (probe_L + 1)) * probe_L + j];
     }
-    double    acc = 0.0;
+    if (LISTM && tid == 0)
+        s_listed = 0;
+    double    acc  = 0.0;
+    uint32_t  mask = 0u;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int e = base + 4 * (j * TPB + tid);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
-                const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
+                const float p   = geist_expf_glibc(arg, s_tab);
                 acc += (double) p;
                 if (e + c == tok)
                     probe_p[row] = p;
+                if (LISTM)
+                    mask |= (uint32_t) (zbin(arg) <= zb_list) << (4 * j + c);
             }
         }
     }
-    acc = block_sum_f64(acc, s_sum);
+    acc = block_sum_f64(acc, s_sum); /* (its barriers publish s_listed = 0) */
     if (tid == 0)
         chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+    if (LISTM) {
+        /* places in the row's list: one LDS counter for the workgroup, one global add for all */
+        int pos = wave_reserve(__popc(mask), &s_listed);
+        __syncthreads();
+        if (tid == 0)
+            s_base = s_listed ? atomicAdd(&list.count[row], s_listed) : 0;
+        __syncthreads();
+        pos += s_base;
+        uint32_t *ck = list.key + (long) row * CAND_CAP;
+        uint32_t *ci = list.idx + (long) row * CAND_CAP;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if ((mask >> (4 * j + c)) & 1u) {
+                    if (pos < CAND_CAP) {
+                        ck[pos] = __float_as_uint(
+                            geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab));
+                        ci[pos] = (uint32_t) (e + c);
+                    }
+                    ++pos;
+                }
+            }
+        }
+    }
 }
 
 /* ============================================================================================
@@ -140,10 +176,13 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
  * ========================================================================================== */
 template <int NV, bool PEN, bool BEST>
 __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict__ tmax,
-                                                   uint64_t *__restrict__ chunk_best) {
+                                                   uint64_t *__restrict__ chunk_best,
+                                                   int32_t *__restrict__ zero_per_row) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
     const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    if (BEST && zero_per_row && chunk == 0 && tid == 0)
+        zero_per_row[row] = 0; /* a counter the following pass adds to */
     int       base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     GS_MARK(0);
@@ -579,6 +618,10 @@ struct FinalArgs {
     int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to the candidate list,
                                * 2 = to k_sorted_general */
     CandSpace       cand;
+    double          ln_min_p; /* log(min_p), taken on the host */
+    int             zb_min_p; /* last z bin that can hold an entry passing min_p (with slack);
+                               * ZBINS - 1 when min_p is off or that deep */
+    bool            minp_listed; /* the exp-sum pass listed every row up to that bin */
 };
 
 /* ============================================================================================
@@ -918,6 +961,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __shared__ int      s_n, s_n2;
     __shared__ double   s_sum;
     const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
+    GS_MARK(0);
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid < C)
@@ -933,6 +977,22 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __syncthreads();
     const double sum = s_sum;
     int          tok = -1;
+    GS_MARK(1);
+    if (a.minp_listed && a.cand.count[row] <= CAND_CAP) {
+        /* the exp-sum pass listed the row under the min-p bound (holding p, not pn): the list
+         * walk serves it, top-p included -- the kept prefix is the shorter of the two */
+        if (tid == 0) {
+            const int   B      = a.zb_min_p;
+            const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float pn_out = (float) ((double) p_out / sum);
+            a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
+            a.cand.row_bound[row] = B;
+            a.cand.row_sum[row]   = sum;
+            a.row_flag[row]       = 4;
+            a.out[row]            = -1;
+        }
+        return;
+    }
     if (C <= 16)
         tok = sorted_from_tmax<NV, PEN, 16>(rv, a, row, mx, sum, u_row, s_big, s_mx, s_wt, s_selid,
                                             s_pcnt, s_m, s_srt, &s_n, &s_n2, s_tab);
@@ -940,6 +1000,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big, s_mx,
                                                         s_wt, s_selid, s_pcnt, s_m, s_srt, &s_n,
                                                         &s_n2, s_tab);
+    GS_MARK(6);
     if (tok >= 0) {
         if (tid == 0) {
             a.row_flag[row]  = 0;
@@ -961,65 +1022,80 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
      *   min-p: pn_i >= min_p * pn_0 needs z_i <= -ln(min_p), in closed form, taken with slack.
      *   Both set: the shorter prefix, so the smaller bin. */
     __syncthreads();
-    float     *s_zh   = s_wt;                           /* TPB floats, free again */
-    int       *s_zc   = reinterpret_cast<int *>(s_mx);  /* TPB words, free again */
+    constexpr int COPIES = 8; /* lanes spread over copies of the bins: fewer same-address adds */
+    float        *s_zh   = reinterpret_cast<float *>(s_big);                      /* [COPIES][ZBINS] */
+    int          *s_zc   = reinterpret_cast<int *>(s_big + COPIES * ZBINS * 4);   /* [COPIES][ZBINS] */
+    static_assert(COPIES * ZBINS * 8 <= TMAX_LDS, "bins live in the slot table's space");
     const bool want_p = a.top_p > 0.0f && a.top_p < 1.0f;
-    if (tid < ZBINS) {
-        s_zh[tid] = 0.0f;
-        s_zc[tid] = 0;
-    }
+    for (int i = tid; i < COPIES * ZBINS * 2; i += TPB)
+        reinterpret_cast<uint32_t *>(s_big)[i] = 0u;
     __syncthreads();
     if (want_p) {
-        const float *tm = a.tmax + (long) row * C * TPB + tid;
+        const float *tm   = a.tmax + (long) row * C * TPB + tid;
+        const int    copy = (tid & (COPIES - 1)) * ZBINS;
+        const int    last = a.zb_min_p < ZBINS - 2 ? a.zb_min_p + 1 : ZBINS - 2; /* deeper bins cannot matter */
         for (int q = 0; q < C; ++q) {
-            const float t = tm[(long) q * TPB];
-            if (t != t)
-                continue; /* a thread without an element of the row */
-            const float arg = softmax_arg(t, mx, a.inv_t);
-            const int   zb  = zbin(arg);
-            atomicAdd(&s_zc[zb], 1);
-            if (zb < ZBINS - 1)
-                unsafeAtomicAdd(&s_zh[zb], __expf(arg));
+            const float arg = softmax_arg(tm[(long) q * TPB], mx, a.inv_t);
+            const int   zb  = zbin(arg); /* NaN (a thread without an element) lands past `last` */
+            if (zb <= last) {
+                atomicAdd(&s_zc[copy + zb], 1);
+                unsafeAtomicAdd(&s_zh[copy + zb], __expf(arg));
+            }
         }
     }
     __syncthreads();
-    if (tid == 0) {
+    GS_MARK(7);
+    if (tid < WAVE) {
         int B = ZBINS - 1;
         if (want_p) {
-            int T = 0;
-            for (int b = 0; b < ZBINS; ++b)
-                T += s_zc[b];
-            const double need = ((double) a.top_p + 0.25 * (1.0 - (double) a.top_p)) * sum;
-            double       cum  = 0.0;
-            int          M    = 0;
-            for (int b = 0; b < ZBINS - 1; ++b) {
-                const double mid  = (double) M + 0.5 * (double) s_zc[b];
-                const double left = 1.0 - mid / (double) (T > 0 ? T : 1);
-                cum += (double) s_zh[b] / (left > 0.05 ? left : 0.05);
-                M += s_zc[b];
-                if (cum >= need) {
-                    B = b + 1 < ZBINS - 1 ? b + 1 : b;
-                    break;
-                }
+            /* scanning threads that hold at least one element of the row */
+            const int rem  = rv.n_vocab - (C - 1) * rv.per_chunk;
+            const int T    = (C - 1) * TPB + ((rem + 3) / 4 < TPB ? (rem + 3) / 4 : TPB);
+            const int b0   = 2 * tid, b1 = 2 * tid + 1;
+            int       c0 = 0, c1 = 0;
+            float     w0 = 0.f, w1 = 0.f;
+#pragma unroll
+            for (int k = 0; k < COPIES; ++k) {
+                c0 += s_zc[k * ZBINS + b0];
+                c1 += s_zc[k * ZBINS + b1];
+                w0 += s_zh[k * ZBINS + b0];
+                w1 += s_zh[k * ZBINS + b1];
             }
+            const int    before = wave_scan_i32_dpp(c0 + c1) - c0 - c1;
+            const double invT   = 1.0 / (double) (T > 0 ? T : 1);
+            const double l0     = 1.0 - ((double) before + 0.5 * (double) c0) * invT;
+            const double l1     = 1.0 - ((double) (before + c0) + 0.5 * (double) c1) * invT;
+            const double s0     = (double) w0 / (l0 > 0.05 ? l0 : 0.05);
+            const double s1     = (double) w1 / (l1 > 0.05 ? l1 : 0.05);
+            const double incl   = wave_scan_f64_dpp(s0 + s1);
+            const double need   = ((double) a.top_p + 0.25 * (1.0 - (double) a.top_p)) * sum;
+            const uint64_t h0   = __ballot(incl - s1 >= need && b0 < ZBINS - 1);
+            const uint64_t h1   = __ballot(incl >= need && b1 < ZBINS - 1);
+            int            first = ZBINS;
+            if (h0)
+                first = 2 * (__ffsll((long long) h0) - 1);
+            if (h1) {
+                const int f1 = 2 * (__ffsll((long long) h1) - 1) + 1;
+                first        = f1 < first ? f1 : first;
+            }
+            if (first < ZBINS - 1)
+                B = first + 1 < ZBINS - 1 ? first + 1 : first; /* one more bin for the estimate */
         }
-        if (a.min_p > 0.0f) {
-            const double z_m = -log((double) a.min_p) + 2e-3;
-            const int    b_m = z_m * ZBIN_PER_NAT < (double) (ZBINS - 1) ? (int) (z_m * ZBIN_PER_NAT)
-                                                                         : ZBINS - 1;
-            B = b_m < B ? b_m : B;
+        B = a.zb_min_p < B ? a.zb_min_p : B;
+        if (tid == 0) {
+            /* an element outside the list has z >= (B + 1) / ZBIN_PER_NAT (the product in zbin()
+             * is exact), so its p is at most expf of minus that; one step up covers any
+             * non-monotonic last bit of expf or of the division */
+            const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float pn_out = (float) ((double) p_out / sum);
+            a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
+            a.cand.row_bound[row] = B;
+            a.cand.count[row]     = 0;
+            a.row_flag[row]       = B < ZBINS - 1 ? 1 : 2;
+            a.out[row]            = -1;
         }
-        /* an element outside the list has z >= (B + 1) / ZBIN_PER_NAT (the product in zbin() is
-         * exact), so its p is at most expf of minus that; one step up covers any non-monotonic
-         * last bit of expf or of the division */
-        const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
-        const float pn_out = (float) ((double) p_out / sum);
-        a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
-        a.cand.row_bound[row] = B;
-        a.cand.count[row]     = 0;
-        a.row_flag[row]       = B < ZBINS - 1 ? 1 : 2;
-        a.out[row]            = -1;
     }
+    GS_MARK(8);
 }
 
 /* top-k (sampler.c:178-228) and the chain behind it: select from the row's thread maxima, then
@@ -1210,12 +1286,29 @@ static void dispatch(int nv, bool pen, F &&f) {
 
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p) {
+                         float *probe_p, const CandSpace *list, int zb_list) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    if (list && L.nv == 8) {
+        if (L.pen)
+            k_chunk_expsum<8, true, true><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, *list, zb_list);
+        else
+            k_chunk_expsum<8, false, true><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, *list, zb_list);
+        return;
+    }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_chunk_expsum<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
-            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p);
+        k_chunk_expsum<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(
+            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, CandSpace{}, 0);
     });
+}
+
+int zbin_of_min_p(float min_p) {
+    if (!(min_p > 0.0f))
+        return ZBINS - 1;
+    /* pn_i >= min_p * pn_0 needs z_i <= -ln(min_p); slack for the fp32 steps in between */
+    const double z_m = -std::log((double) min_p) + 2e-3;
+    return z_m * ZBIN_PER_NAT < (double) (ZBINS - 1) ? (int) (z_m * ZBIN_PER_NAT) : ZBINS - 1;
 }
 
 void launch_spec(const Launch &L, const SpecLaunch &sp) {
@@ -1247,13 +1340,15 @@ void launch_spec(const Launch &L, const SpecLaunch &sp) {
         k_spec_final<2><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a);
 }
 
-void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best) {
+void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best, int32_t *zero_per_row) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         if (chunk_best)
-            k_tmax_scan<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(L.rv, tmax, chunk_best);
+            k_tmax_scan<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(L.rv, tmax, chunk_best,
+                                                                          zero_per_row);
         else
-            k_tmax_scan<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(L.rv, tmax, nullptr);
+            k_tmax_scan<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(L.rv, tmax, nullptr,
+                                                                           nullptr);
     });
 }
 
@@ -1272,6 +1367,9 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.row_flag   = f.row_flag;
     a.out        = f.out;
     a.cand       = f.cand;
+    a.ln_min_p   = f.min_p > 0.0f ? std::log((double) f.min_p) : 0.0;
+    a.zb_min_p    = zbin_of_min_p(f.min_p);
+    a.minp_listed = f.minp_listed;
     const dim3 grid(L.rows), block(TPB);
     if (f.mode == FINAL_ARGMAX) {
         k_final_argmax<<<grid, block, 0, L.stream>>>(L.rv, a);

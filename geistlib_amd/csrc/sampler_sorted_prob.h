@@ -137,8 +137,9 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
         for (int i = tid; i < KPT * TPB / 16; i += TPB)
             z[i] = make_uint4(0u, 0u, 0u, 0u);
         if (PEN) {
-            for (int i = tid; i < SEL_MAX * 4 * NV; i += TPB)
-                s_pcnt[i] = 0u;
+            uint4 *zc = reinterpret_cast<uint4 *>(s_pcnt);
+            for (int i = tid; i < SEL_MAX * NV; i += TPB)
+                zc[i] = make_uint4(0u, 0u, 0u, 0u);
         }
         if (tid == 0) {
             *s_n  = 0;
@@ -156,6 +157,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     s_mx[tid] = mkey;
     s_wt[tid] = wt;
     __syncthreads();
+    GS_MARK(2);
     /* 2 */
     uint32_t key_lo = 0u;
     if (use_p) {
@@ -171,9 +173,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
             const uint32_t t = tau | (1u << bit);
             float acc = (k0 >= t ? w0 : 0.f) + (k1 >= t ? w1 : 0.f) + (k2 >= t ? w2 : 0.f) +
                         (k3 >= t ? w3 : 0.f);
-#pragma unroll
-            for (int m = 32; m >= 1; m >>= 1)
-                acc += __shfl_xor(acc, m, WAVE);
+            acc = wave_sum_f32_dpp(acc);
             if (acc >= need)
                 tau = t;
         }
@@ -183,7 +183,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     }
     if (use_m) {
         /* (l - mx) * inv_t >= ln(min_p) - slack  <=>  l >= mx + (ln(min_p) - slack) / inv_t */
-        const double   lg  = log((double) a.min_p) - 1e-3;
+        const double   lg  = a.ln_min_p - 1e-3;
         const float    t_m = (float) ((double) mx + lg / (double) a.inv_t - 1e-3 * fabs((double) mx));
         const uint32_t km  = f2key(t_m);
         key_lo             = km > key_lo ? km : key_lo;
@@ -191,24 +191,25 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     if (key_lo < 0x00800000u)
         return -1;
     const float bound = key2f(key_lo);
+    GS_MARK(3);
     /* 3 */
-    int cnt = 0;
+    uint32_t selmask = 0u;
 #pragma unroll
     for (int q = 0; q < KPT; ++q)
-        cnt += raw[q] >= bound;
-    int pos = wave_reserve(cnt, s_n);
-#pragma unroll
-    for (int q = 0; q < KPT; ++q) {
-        if (raw[q] >= bound) {
-            if (pos < SEL_MAX) {
-                s_selid[pos]        = q * TPB + tid;
-                slot[q * TPB + tid] = (uint8_t) (pos + 1);
-            }
-            ++pos;
+        selmask |= (uint32_t) (raw[q] >= bound) << q;
+    int pos = wave_reserve(__popc(selmask), s_n);
+    while (selmask) {
+        const int q = __ffs(selmask) - 1;
+        selmask &= selmask - 1u;
+        if (pos < SEL_MAX) {
+            s_selid[pos]        = q * TPB + tid;
+            slot[q * TPB + tid] = (uint8_t) (pos + 1);
         }
+        ++pos;
     }
     __syncthreads();
     const int n_sel = *s_n;
+    GS_MARK(4);
     if (n_sel > SEL_MAX)
         return -1;
     constexpr int TASKS = SEL_MAX * NV / TPB;
@@ -242,29 +243,37 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     }
     if (PEN) {
         const int shift = 31 - __clz(rv.per_chunk);
-        history_for_each(rv, row, pf, [&](int t) {
-            if (t < 0 || t >= rv.n_vocab)
-                return;
-            const int off = t & (rv.per_chunk - 1);
-            const int f   = off >> 2;
-            const int s   = slot[(t >> shift) * TPB + (f % TPB)];
-            if (s)
-                atomicAdd(&s_pcnt[((s - 1) * NV + f / TPB) * 4 + (off & 3)], 1u);
-        });
+        history_for_each_batched(
+            rv, row, pf,
+            [&](int t) -> int { /* 1 + index of the element's counter, 0 = not gathered */
+                if (t < 0 || t >= rv.n_vocab)
+                    return 0;
+                const int off = t & (rv.per_chunk - 1);
+                const int f   = off >> 2;
+                const int s   = slot[(t >> shift) * TPB + (f % TPB)];
+                return s ? 1 + ((s - 1) * NV + f / TPB) * 4 + (off & 3) : 0;
+            },
+            [&](int code) {
+                if (code)
+                    atomicAdd(&s_pcnt[code - 1], 1u);
+            });
         __syncthreads();
     }
-    uint32_t ck[TASKS][4];
-    int      keep = 0;
+    /* survivors are appended in any order: the ranking below orders them */
 #pragma unroll
     for (int q = 0; q < TASKS; ++q) {
         const int t = tid + q * TPB;
+        if (e0[q] >= e1[q])
+            continue;
+        uint4 hc = make_uint4(0u, 0u, 0u, 0u);
+        if (PEN)
+            hc = *reinterpret_cast<const uint4 *>(&s_pcnt[t * 4]);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            ck[q][c] = 0u;
             if (e0[q] + c < e1[q]) {
                 float x = f4_get(r[q], c);
                 if (PEN) {
-                    const uint32_t n_hist = s_pcnt[t * 4 + c];
+                    const uint32_t n_hist = c == 0 ? hc.x : c == 1 ? hc.y : c == 2 ? hc.z : hc.w;
                     if (n_hist)
                         x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
                 }
@@ -273,27 +282,16 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
                 if (x >= bound) {
                     const float pn =
                         (float) ((double) geist_expf_glibc(softmax_arg(x, mx, a.inv_t), tab) / sum);
-                    /* bit 31 marks the slot as taken even when pn underflows to 0 */
-                    ck[q][c] = __float_as_uint(pn) | 0x80000000u;
-                    ++keep;
+                    const int at = atomicAdd(s_n2, 1);
+                    if (at < TPB)
+                        s_m[at] = pack_best(__float_as_uint(pn), (uint32_t) (e0[q] + c));
                 }
-            }
-        }
-    }
-    pos = wave_reserve(keep, s_n2);
-#pragma unroll
-    for (int q = 0; q < TASKS; ++q) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (ck[q][c]) {
-                if (pos < TPB)
-                    s_m[pos] = pack_best(ck[q][c] & 0x7fffffffu, (uint32_t) (e0[q] + c));
-                ++pos;
             }
         }
     }
     __syncthreads();
     const int m = *s_n2;
+    GS_MARK(5);
     if (m > TPB || m < 1)
         return -1;
     /* 4: order by counting, entry i compared by P = 256 / m2 <= 64 neighbouring lanes */
@@ -579,6 +577,7 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
             mass_m = pn_fx(__uint_as_float(kmax));
         }
     }
+    GS_MARK(2);
     /* nucleus edge */
     bool     limited   = false;
     uint32_t edge_key  = 0u, edge_ties = 0u;
@@ -630,6 +629,7 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
         mass_keep = block_sum_u64(lm, sh.red64);
         limited   = false;
     }
+    GS_MARK(3);
     /* the draw: first entry of the kept prefix at which the running mass exceeds u * mass */
     /* running mass > u * mass  <=>  running mass >= floor(u * mass) + 1 in integers */
     const uint64_t target2 = (uint64_t) __double2ull_rd((double) u * (double) mass_keep) + 1ull;
@@ -644,6 +644,7 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
             j = 1;
         if (j > ties_d)
             j = ties_d;
+        GS_MARK(4);
         if (LIST) {
             tok = list_jth_id(pn, ids, n, kd, (int) j, sh, s_scan, s_pick);
         } else {
@@ -729,6 +730,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (row_flag[row] != 1)
         return;
+    GS_MARK(0);
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid == 0) {
@@ -741,9 +743,11 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
     fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
+    GS_MARK(1);
     const float  mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
     const double tot = s_total;
     const int    B   = cand.row_bound[row];
+    GS_MARK(2);
     uint32_t     mask = 0u;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -754,7 +758,9 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
             mask |= (uint32_t) in << (4 * j + c);
         }
     }
+    GS_MARK(6);
     int       pos = wave_reserve(__popc(mask), &cand.count[row]);
+    GS_MARK(7);
     uint32_t *ck  = cand.key + (long) row * CAND_CAP;
     uint32_t *ci  = cand.idx + (long) row * CAND_CAP;
 #pragma unroll
@@ -772,9 +778,10 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
             }
         }
     }
+    GS_MARK(8);
 }
 
-/* k_sorted_candidates: one workgroup per row flagged 1 walks the row's list (staged in LDS when
+/* k_sorted_candidates: one workgroup per row flagged 1 or 4 walks the row's list (staged in LDS when
  * it fits). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
  * prefix that may reach past the list -- is flagged 2 for k_sorted_general. */
 __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float top_p, float min_p,
@@ -787,25 +794,37 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
     __shared__ uint32_t        s_key[CAND_LDS];
     __shared__ uint32_t        s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
-    if (row_flag[row] != 1)
+    const int flag = row_flag[row];
+    if (flag != 1 && flag != 4)
         return;
     const int n   = cand.count[row];
     int       tok = -1;
+    GS_MARK(0);
     if (n >= 1 && n <= CAND_CAP) {
-        const uint32_t *gk = cand.key + (long) row * CAND_CAP;
+        uint32_t       *wk = cand.key + (long) row * CAND_CAP;
+        const uint32_t *gk = wk;
         const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
+        /* flag 4: the list holds p; pn = (float)((double)p / sum), sampler.c:251-253 */
+        const double sum = flag == 4 ? cand.row_sum[row] : 1.0;
         if (n <= CAND_LDS) {
             for (int i = tid; i < n; i += TPB) {
-                s_key[i] = gk[i];
+                const uint32_t k = gk[i];
+                s_key[i] = flag == 4 ? __float_as_uint((float) ((double) __uint_as_float(k) / sum)) : k;
                 s_idx[i] = gi[i];
             }
             __syncthreads();
             gk = s_key;
             gi = s_idx;
+        } else if (flag == 4) {
+            for (int i = tid; i < n; i += TPB)
+                wk[i] = __float_as_uint((float) ((double) __uint_as_float(wk[i]) / sum));
+            __syncthreads();
         }
+        GS_MARK(1);
         tok = sorted_descend<true>(reinterpret_cast<const float *>(gk), gi, n, top_p, min_p,
                                    uniforms[row], cand.out_key[row], sh, s_scan, &s_pick);
     }
+    GS_MARK(7);
     if (tid == 0) {
         row_flag[row] = tok < 0 ? 2 : 0;
         out[row]      = tok;
