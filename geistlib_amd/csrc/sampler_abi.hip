@@ -387,10 +387,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
      * are listed and walked; what that cannot serve either is flagged 2 for the last two kernels.
      * Each of these kernels returns at once for every row not flagged for it. */
     launch_candidates(L, f);
-    launch_write_probs(L, rs.inv_t, s->chunk_best, s->chunk_sum, s->probs, (long) s->max_vocab,
-                       s->row_flag);
-    launch_sorted_general(L, s->probs, (long) s->max_vocab, rs.top_p, rs.min_p, d_uniforms,
-                          s->row_flag, d_out, s->cand.path);
+    launch_sorted_general(L, f, s->probs, (long) s->max_vocab);
     return after_launch(s, "top-p / min-p");
 }
 

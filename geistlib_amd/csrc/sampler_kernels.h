@@ -115,9 +115,8 @@ void launch_candidates(const Launch &L, const FinalLaunch &f);
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
                         const double *chunk_sum, float *probs, long ld_probs,
                         const int32_t *row_flag);
-void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
-                           float min_p, const float *uniforms, const int32_t *row_flag,
-                           int32_t *out, int32_t *path);
+/* rows flagged 2: probabilities of the whole row into `probs`, then the walk over them */
+void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

@@ -1434,11 +1434,12 @@ void launch_candidates(const Launch &L, const FinalLaunch &f) {
                                                              f.row_flag, f.out);
 }
 
-void launch_sorted_general(const Launch &L, const float *probs, long ld_probs, float top_p,
-                           float min_p, const float *uniforms, const int32_t *row_flag,
-                           int32_t *out, int32_t *path) {
-    k_sorted_general<<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(
-        probs, ld_probs, L.rv.n_vocab, top_p, min_p, uniforms, row_flag, out, path);
+void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {
+    dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
+        k_sorted_general<GS_NV, GS_PEN><<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(
+            L.rv, f.inv_t, f.chunk_best, f.chunk_sum, probs, ld_probs, f.top_p, f.min_p, f.uniforms,
+            f.row_flag, f.out, f.cand.path);
+    });
 }
 
 void launch_penalties(const Launch &L, float *logits_rw) {

@@ -689,22 +689,63 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
     return tok;
 }
 
-__global__ __launch_bounds__(TPB) void k_sorted_general(const float *__restrict__ probs,
-                                                        long ld_probs, int n, float top_p,
-                                                        float min_p,
+/* k_sorted_general: rows flagged 2. One workgroup per row first writes the row's normalised
+ * probabilities pn_i = (float)((double)p_i / sum) (sampler.c:246-253) into the probs workspace,
+ * chunk by chunk, then walks them. The rows that get here are rare (kept prefixes of tens of
+ * thousands of entries, rows of equal values), so the row is not spread over more workgroups. */
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB) void k_sorted_general(RowView rv, float inv_t,
+                                                        const uint64_t *__restrict__ chunk_best,
+                                                        const double *__restrict__ chunk_sum,
+                                                        float *__restrict__ probs, long ld_probs,
+                                                        float top_p, float min_p,
                                                         const float *__restrict__ uniforms,
                                                         const int32_t *__restrict__ row_flag,
                                                         int32_t *__restrict__ out,
                                                         int32_t *__restrict__ path) {
     __shared__ SortedGenShared sh;
-    __shared__ int             s_scan[NWAVES];
-    __shared__ int             s_pick;
-    const int row = blockIdx.x;
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ uint64_t s_tab[32];
+    __shared__ int      s_scan[NWAVES];
+    __shared__ int      s_pick;
+    __shared__ double   s_total;
+    const int row = blockIdx.x, tid = threadIdx.x;
     if (row_flag[row] != 2)
         return;
-    const int tok = sorted_descend<false>(probs + (long) row * ld_probs, nullptr, n, top_p, min_p,
-                                          uniforms[row], 0u, sh, s_scan, &s_pick);
-    if (threadIdx.x == 0) {
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    if (tid == 0) {
+        double t = 0.0;
+        for (int c = 0; c < rv.n_chunks; ++c)
+            t += chunk_sum[(long) row * rv.n_chunks + c];
+        s_total = t;
+    }
+    const float  mx = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, sh.red64)));
+    const double tot = s_total;
+    float       *pn  = probs + (long) row * ld_probs;
+    for (int chunk = 0; chunk < rv.n_chunks; ++chunk) {
+        int base, end;
+        chunk_bounds<NV>(rv, chunk, base, end);
+        float4 v[NV];
+        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (e + c < end) {
+                    const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                    pn[e + c]     = (float) ((double) p / tot);
+                }
+            }
+        }
+        __syncthreads(); /* the history table is rebuilt for the next chunk */
+    }
+    __threadfence_block();
+    __syncthreads();
+    const int tok = sorted_descend<false>(pn, nullptr, rv.n_vocab, top_p, min_p, uniforms[row], 0u,
+                                          sh, s_scan, &s_pick);
+    if (tid == 0) {
         out[row]  = tok;
         path[row] = 3;
     }
@@ -781,6 +822,194 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     GS_MARK(8);
 }
 
+/* ============================================================================================
+ * list_walk_fast: the walk over a candidate list with ONE histogram. The keys that can matter lie
+ * in (kout, kmax]; that range is cut into SG_BINS bins of equal width in key space, descending,
+ * and the mass per bin is accumulated once (2^-62 fixed point, so exact and order-independent).
+ * Prefix sums over the bins locate the bin in which the running mass of the sorted order reaches
+ * a target; the handful of entries of that bin are ordered by counting and walked by one thread.
+ * That is done for the nucleus edge (target top_p) and for the draw (target u * kept mass, bins
+ * beyond the edge cut off), with the kept set described by one packed (key, id) threshold.
+ * Returns the token, -1 when the list cannot certify the kept prefix (see sorted_descend), -2
+ * when a bin holds more than TPB entries (long runs of equal values): the radix descent then
+ * serves the list.
+ * ========================================================================================== */
+struct ListWalkShared {
+    uint64_t mass[SG_BINS];
+    uint64_t small[TPB];
+    uint64_t srt[TPB];
+    uint64_t red64[NWAVES];
+    uint64_t scan64[NWAVES];
+    uint64_t res_before, res_before_edge, out_pack, out_mass;
+    int      res_bin, n_small;
+};
+
+__device__ __forceinline__ uint64_t wave_scan_u64(uint64_t v) {
+    const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const uint64_t o = ((uint64_t) (uint32_t) __shfl_up((int) (v >> 32), d, WAVE) << 32) |
+                           (uint32_t) __shfl_up((int) (uint32_t) v, d, WAVE);
+        if (lane >= d)
+            v += o;
+    }
+    return v;
+}
+
+/* Orders and walks the entries of bin `b` that belong to the kept set (pack >= edge_pack): the
+ * first one at which `before` plus the running mass reaches `target` goes to sh.out_pack, the
+ * running mass including it to sh.out_mass. Returns false when the bin holds too many. */
+__device__ bool list_resolve_bin(const float *pn, const uint32_t *ids, int n, uint32_t kout,
+                                 uint32_t kmax, int shift, int b, uint64_t before, uint64_t target,
+                                 uint64_t edge_pack, ListWalkShared &sh) {
+    const int tid = threadIdx.x;
+    if (tid == 0)
+        sh.n_small = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += TPB) {
+        const uint32_t key = __float_as_uint(pn[i]);
+        if (key <= kout || (int) ((kmax - key) >> shift) != b)
+            continue;
+        const uint64_t pk = pack_best(key, ids[i]);
+        if (pk < edge_pack)
+            continue;
+        const int at = atomicAdd(&sh.n_small, 1);
+        if (at < TPB)
+            sh.small[at] = pk;
+    }
+    __syncthreads();
+    const int c = sh.n_small;
+    if (c > TPB)
+        return false;
+    if (tid < c) {
+        const uint64_t me   = sh.small[tid];
+        int            rank = 0;
+        for (int j = 0; j < c; ++j)
+            rank += sh.small[j] > me;
+        sh.srt[rank] = me;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint64_t run = before;
+        int      at  = c - 1;
+        for (int i = 0; i < c; ++i) {
+            run += pn_fx(__uint_as_float(best_key(sh.srt[i])));
+            if (run >= target) {
+                at = i;
+                break;
+            }
+        }
+        sh.out_pack = c > 0 ? sh.srt[at] : 0ull;
+        sh.out_mass = run;
+    }
+    __syncthreads();
+    return true;
+}
+
+__device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float top_p, float min_p,
+                              float u, uint32_t kout, ListWalkShared &sh) {
+    const int  tid   = threadIdx.x;
+    const bool use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool use_m = min_p > 0.0f;
+    uint32_t   kmax  = 0u;
+    for (int i = tid; i < n; i += TPB) {
+        const uint32_t key = __float_as_uint(pn[i]);
+        kmax               = key > kmax ? key : kmax;
+    }
+    kmax = (uint32_t) block_max_u64((uint64_t) wave_max_u32(kmax), sh.red64);
+    if (kmax <= kout)
+        return -1;
+    const int   bits    = 32 - __clz((int) (kmax - kout));
+    const int   shift   = bits > 11 ? bits - 11 : 0;
+    const float floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
+    for (int i = tid; i < SG_BINS; i += TPB)
+        sh.mass[i] = 0ull;
+    __syncthreads();
+    uint64_t lm = 0;
+    for (int i = tid; i < n; i += TPB) {
+        const float    p   = pn[i];
+        const uint32_t key = __float_as_uint(p);
+        if (key <= kout)
+            continue;
+        const uint64_t fx = pn_fx(p);
+        atomicAdd((unsigned long long *) &sh.mass[(kmax - key) >> shift], (unsigned long long) fx);
+        if (use_m && p >= floor_w)
+            lm += fx;
+    }
+    __syncthreads();
+    const uint64_t mass_m = use_m ? block_sum_u64(lm, sh.red64) : 0ull;
+    /* exclusive prefix of the bins: thread t owns bins 8t .. 8t+7 */
+    constexpr int PER = SG_BINS / TPB;
+    uint64_t      own = 0;
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+        own += sh.mass[tid * PER + q];
+    uint64_t excl = wave_scan_u64(own);
+    if ((tid & (WAVE - 1)) == WAVE - 1)
+        sh.scan64[tid / WAVE] = excl;
+    __syncthreads();
+    for (int w = 0; w < tid / WAVE; ++w)
+        excl += sh.scan64[w];
+    excl -= own;
+    /* the bin at which the running mass reaches `target`; optionally the mass before bin `be` */
+    auto locate = [&](uint64_t target, int be) {
+        if (tid == 0)
+            sh.res_bin = -1;
+        __syncthreads();
+        uint64_t run = excl;
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int      b = tid * PER + q;
+            const uint64_t m = sh.mass[b];
+            if (b == be)
+                sh.res_before_edge = run;
+            if (m && run < target && run + m >= target) {
+                sh.res_bin    = b;
+                sh.res_before = run;
+            }
+            run += m;
+        }
+        __syncthreads();
+    };
+
+    uint64_t edge_pack = 0ull, mass_keep = 0ull;
+    bool     have_p    = false;
+    if (use_p) {
+        const uint64_t target = (uint64_t) __double2ull_ru((double) top_p * 0x1p62);
+        locate(target, -1);
+        const int b = sh.res_bin;
+        if (b >= 0) {
+            if (!list_resolve_bin(pn, ids, n, kout, kmax, shift, b, sh.res_before, target, 0ull, sh))
+                return -2;
+            have_p    = true;
+            edge_pack = sh.out_pack;
+            mass_keep = sh.out_mass;
+        }
+    }
+    const uint32_t kf = __float_as_uint(floor_w);
+    if (use_m && (!have_p || kf > best_key(edge_pack))) {
+        if (kf <= kout)
+            return -1; /* entries outside the list may pass the floor too */
+        edge_pack = (uint64_t) kf << 32; /* every id with a key at or above the floor */
+        mass_keep = mass_m;
+    } else if (!have_p || best_key(edge_pack) <= kout) {
+        return -1; /* the nucleus may reach past the list */
+    }
+    /* the draw: running mass > u * kept mass  <=>  running mass >= floor(u * kept mass) + 1 */
+    const uint64_t target2 = (uint64_t) __double2ull_rd((double) u * (double) mass_keep) + 1ull;
+    const int      be      = (int) ((kmax - best_key(edge_pack)) >> shift);
+    locate(target2, be);
+    int      bd     = sh.res_bin;
+    uint64_t before = sh.res_before;
+    if (bd < 0 || bd >= be) { /* inside the partly kept bin of the edge */
+        bd     = be;
+        before = sh.res_before_edge;
+    }
+    if (!list_resolve_bin(pn, ids, n, kout, kmax, shift, bd, before, target2, edge_pack, sh))
+        return -2;
+    return (int) best_idx(sh.out_pack);
+}
+
 /* k_sorted_candidates: one workgroup per row flagged 1 or 4 walks the row's list (staged in LDS when
  * it fits). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
  * prefix that may reach past the list -- is flagged 2 for k_sorted_general. */
@@ -788,11 +1017,14 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
                                                            const float *__restrict__ uniforms,
                                                            int32_t *__restrict__ row_flag,
                                                            int32_t *__restrict__ out) {
-    __shared__ SortedGenShared sh;
-    __shared__ int             s_scan[NWAVES];
-    __shared__ int             s_pick;
-    __shared__ uint32_t        s_key[CAND_LDS];
-    __shared__ uint32_t        s_idx[CAND_LDS];
+    __shared__ union {
+        SortedGenShared gen;
+        ListWalkShared  fast;
+    } sh;
+    __shared__ int      s_scan[NWAVES];
+    __shared__ int      s_pick;
+    __shared__ uint32_t s_key[CAND_LDS];
+    __shared__ uint32_t s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int flag = row_flag[row];
     if (flag != 1 && flag != 4)
@@ -821,8 +1053,13 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
             __syncthreads();
         }
         GS_MARK(1);
-        tok = sorted_descend<true>(reinterpret_cast<const float *>(gk), gi, n, top_p, min_p,
-                                   uniforms[row], cand.out_key[row], sh, s_scan, &s_pick);
+        const float *keys = reinterpret_cast<const float *>(gk);
+        tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], cand.out_key[row], sh.fast);
+        if (tok == -2) {
+            __syncthreads();
+            tok = sorted_descend<true>(keys, gi, n, top_p, min_p, uniforms[row], cand.out_key[row],
+                                       sh.gen, s_scan, &s_pick);
+        }
     }
     GS_MARK(7);
     if (tid == 0) {
