@@ -28,6 +28,9 @@ struct geist_hip_sampler {
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
     double   *resid_sum  = nullptr; /* [max_rows][max_chunks] spec verification */
+    double   *slab_sum   = nullptr; /* [max_rows][max_chunks][8] slab sums of the exp-sum pass */
+    double   *resid_slab = nullptr; /* [max_rows][max_chunks][8] spec verification */
+    void     *verdict    = nullptr; /* [max_rows] acceptance results of spec verification */
     float    *tmax       = nullptr; /* [max_rows][max_chunks][256] per-thread maxima */
     int32_t  *row_flag   = nullptr; /* [max_rows] */
     float    *uniforms   = nullptr; /* [max_rows] */
@@ -165,7 +168,10 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->slab_sum, rc * 8 * sizeof(double));
+    if (e == hipSuccess) e = hipMalloc((void **) &s->resid_slab, rc * 8 * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->tmax, rc * 256 * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(&s->verdict, max_rows * SPEC_VERDICT_BYTES);
     if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
     if (e == hipSuccess) e = hipMalloc((void **) &s->probe_p, max_rows * sizeof(float));
@@ -188,7 +194,10 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
     (void) hipFree(s->resid_sum);
+    (void) hipFree(s->slab_sum);
+    (void) hipFree(s->resid_slab);
     (void) hipFree(s->tmax);
+    (void) hipFree(s->verdict);
     (void) hipFree(s->row_flag);
     (void) hipFree(s->uniforms);
     (void) hipFree(s->probe_p);
@@ -343,10 +352,12 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     if (!rs.use_p && !rs.use_m) {
         if (!stream_only(s))
             launch_tmax_scan(L, s->tmax, s->chunk_best);
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr, 0,
+                            s->slab_sum);
         if (stream_only(s))
             return after_launch(s, "exp-sum scan");
-        f.mode = FINAL_TEMPERATURE;
+        f.mode     = FINAL_TEMPERATURE;
+        f.slab_sum = s->slab_sum;
         launch_row_final(L, f);
         return after_launch(s, "temperature");
     }
@@ -526,7 +537,8 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     const float inv_t = greedy ? 1.0f : 1.0f / temperature;
     launch_tmax_scan(La, s->tmax, s->chunk_best);
     if (!greedy)
-        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p);
+        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p,
+                            nullptr, 0, s->slab_sum);
     SpecLaunch sp{};
     sp.n_seq      = (int) n_seq;
     sp.L          = (int) L;
@@ -540,6 +552,9 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     sp.chunk_sum  = s->chunk_sum;
     sp.probe_p    = s->probe_p;
     sp.resid_sum  = s->resid_sum;
+    sp.resid_slab = s->resid_slab;
+    sp.slab_sum   = s->slab_sum;
+    sp.verdict    = s->verdict;
     sp.out_tokens = d_out_tokens;
     sp.n_accepted = d_n_accepted;
     launch_spec(La, sp);

@@ -190,6 +190,28 @@ __device__ __forceinline__ double block_sum_f64(double v, double *scratch) {
     __syncthreads();
     return r;
 }
+/* NV sums over the workgroup at once (wavefront totals by DPP steps, then the four waves in
+ * order): every thread receives all NV totals. `scratch` holds NWAVES * NV entries. */
+template <int NV>
+__device__ __forceinline__ void block_sum_f64_multi(double (&v)[NV], double *scratch) {
+    const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const double t = wave_scan_f64_dpp(v[j]); /* lane 63 holds the wavefront's total */
+        if (lane == WAVE - 1)
+            scratch[w * NV + j] = t;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        double r = scratch[j];
+#pragma unroll
+        for (int x = 1; x < NWAVES; ++x)
+            r += scratch[x * NV + j];
+        v[j] = r;
+    }
+    __syncthreads();
+}
 /* Inclusive prefix sum over the 256 threads in thread order; *total receives the sum. */
 __device__ __forceinline__ double block_scan_f64(double v, double *scratch, double *total) {
     const int w    = threadIdx.x / WAVE;

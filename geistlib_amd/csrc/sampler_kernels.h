@@ -69,6 +69,7 @@ struct FinalLaunch {
     const float    *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
+    const double   *slab_sum;
     const float    *tmax;
     int32_t        *out;
     int32_t        *row_flag;
@@ -78,10 +79,13 @@ struct FinalLaunch {
  * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
 /* list != NULL (min-p set): the pass also lists, per row, every element up to z bin zb_list with
  * its unnormalised p -- the min-p bound needs nothing but the row maximum. list->count must be
- * zero on entry (launch_tmax_scan can clear it). */
+ * zero on entry (launch_tmax_scan can clear it).
+ * slab_sum != NULL (and no list): also the sums of the chunk's slabs of 1024 elements,
+ * [rows][chunks][8], which the index-order walks locate their starting point with. */
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, const CandSpace *list = nullptr, int zb_list = 0);
+                         float *probe_p, const CandSpace *list = nullptr, int zb_list = 0,
+                         double *slab_sum = nullptr);
 /* last z bin that can hold an entry passing min_p (with slack); ZBINS - 1 when min_p is off or
  * that deep */
 int zbin_of_min_p(float min_p);
@@ -97,10 +101,15 @@ struct SpecLaunch {
     const double   *chunk_sum;
     const float    *probe_p;
     double         *resid_sum;
+    double         *resid_slab; /* [n_seq][chunks][8] */
+    const double   *slab_sum;   /* [rows][chunks][8] from the exp-sum pass */
+    void           *verdict; /* [n_seq] x SPEC_VERDICT_BYTES, written by the acceptance kernel */
     int32_t        *out_tokens;
     int32_t        *n_accepted;
 };
-constexpr int SPEC_DRAFT_MAX = 63;
+constexpr int SLABS_MAX         = 8; /* slab sums are stored 8 per chunk whatever NV is */
+constexpr int SPEC_DRAFT_MAX      = 63;
+constexpr int SPEC_VERDICT_BYTES = 24;
 void launch_spec(const Launch &L, const SpecLaunch &sp);
 /* chunk_best may be NULL when only the thread maxima are wanted */
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best,

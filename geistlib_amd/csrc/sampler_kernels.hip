@@ -85,17 +85,18 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
  * Optionally records p at one token of the row (spec verification needs p(x_j)).
  * ========================================================================================== */
-template <int NV, bool PEN, bool LISTM>
+template <int NV, bool PEN, bool LISTM, bool SLABS>
 __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                                                       const uint64_t *__restrict__ chunk_best,
                                                       double *__restrict__ chunk_sum,
+                                                      double *__restrict__ slab_sum,
                                                       const int32_t *__restrict__ probe_token,
                                                       int probe_L, float *__restrict__ probe_p,
                                                       CandSpace list, int zb_list) {
     static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
-    __shared__ double   s_sum[NWAVES];
+    __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ int      s_listed, s_base;
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
@@ -117,16 +118,22 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     if (LISTM && tid == 0)
         s_listed = 0;
     double    acc  = 0.0;
+    double    accs[SLABS ? NV : 1];
     uint32_t  mask = 0u;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int e = base + 4 * (j * TPB + tid);
+        if (SLABS)
+            accs[j] = 0.0;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
                 const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
                 const float p   = geist_expf_glibc(arg, s_tab);
-                acc += (double) p;
+                if (SLABS)
+                    accs[j] += (double) p;
+                else
+                    acc += (double) p;
                 if (e + c == tok)
                     probe_p[row] = p;
                 if (LISTM)
@@ -134,9 +141,23 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             }
         }
     }
-    acc = block_sum_f64(acc, s_sum); /* (its barriers publish s_listed = 0) */
-    if (tid == 0)
-        chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+    if (SLABS) {
+        /* the chunk's sum is the sum of its slab sums, in slab order */
+        block_sum_f64_multi<SLABS ? NV : 1>(accs, s_sum);
+        if (tid == 0) {
+            const long at = (long) row * rv.n_chunks + chunk;
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                slab_sum[at * SLABS_MAX + j] = accs[j];
+                acc += accs[j];
+            }
+            chunk_sum[at] = acc;
+        }
+    } else {
+        acc = block_sum_f64(acc, s_sum); /* (its barriers publish s_listed = 0) */
+        if (tid == 0)
+            chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+    }
     if (LISTM) {
         /* places in the row's list: one LDS counter for the workgroup, one global add for all */
         int pos = wave_reserve(__popc(mask), &s_listed);
@@ -613,6 +634,7 @@ struct FinalArgs {
     const float   *uniforms;
     const uint64_t *chunk_best;
     const double   *chunk_sum;
+    const double   *slab_sum; /* FINAL_TEMPERATURE: [rows][chunks][SLABS_MAX] */
     const float    *tmax;
     int32_t        *out;
     int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to the candidate list,
@@ -844,6 +866,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 }
 
 } // namespace gs
+#include "sampler_walk.h"
 #include "sampler_sorted_prob.h"
 #include "sampler_spec.h"
 namespace gs {
@@ -869,79 +892,24 @@ __global__ __launch_bounds__(TPB) void k_final_argmax(RowView rv, FinalArgs a) {
  * sums, then scan that chunk. */
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_final_temperature(RowView rv, FinalArgs a) {
-    __shared__ uint64_t     s_red[NWAVES];
-    __shared__ FinishShared s_fs;
-    __shared__ double       s_csum[MAX_CHUNKS];
-    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ int          s_chunk;
-    __shared__ double       s_before;
+    __shared__ uint64_t   s_red[NWAVES];
+    __shared__ uint64_t   s_tab[32];
+    __shared__ WalkShared s_walk;
+    __shared__ double     s_csum[MAX_CHUNKS];
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? TPB * 2 : 1];
     const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
     if (tid < C)
         s_csum[tid] = a.chunk_sum[(long) row * C + tid];
     if (tid < 32)
-        s_fs.tab[tid] = g_expf_tab[tid];
+        s_tab[tid] = g_expf_tab[tid];
     const float u_row = a.uniforms[row];
-    __syncthreads();
-    if (tid == 0) {
-        double tot = 0.0;
-        for (int c = 0; c < C; ++c)
-            tot += s_csum[c];
-        const double target = (double) u_row * tot;
-        double       run    = 0.0;
-        int          at     = C - 1;
-        for (int c = 0; c < C; ++c) {
-            const double nxt = run + s_csum[c];
-            if (target < nxt || c == C - 1) {
-                at = c;
-                break;
-            }
-            run = nxt;
-        }
-        s_chunk   = at;
-        s_before  = run;
-        s_fs.mass = target;
-    }
-    const float mx = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
-    /* (row_best_from_chunks ends with a barrier: s_chunk, s_before, tab are visible) */
-    const int chunk = s_chunk;
-    int       base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
-    /* index order inside the chunk is (j, thread, component): scan one j-slab at a time */
-    double       carry  = s_before;
-    const double target = s_fs.mass;
+    const float mx    = key2f(best_key(row_best_from_chunks(a.chunk_best, row, C, s_red)));
+    /* (row_best_from_chunks ends with a barrier: s_csum and the table are visible) */
+    const int tok = index_order_walk<NV, PEN, false>(
+        rv, row, (int) gridDim.x, s_csum, a.slab_sum + (long) row * C * SLABS_MAX, C, u_row, mx,
+        a.inv_t, 0.0, nullptr, false, s_tab, s_cnt16, s_walk);
     if (tid == 0)
-        s_fs.pick = 0x7fffffff;
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
-        float     p[4];
-        double    part = 0.0;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            p[c] = (e + c < end)
-                       ? geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, a.inv_t), s_fs.tab)
-                       : 0.0f;
-            part += (double) p[c];
-        }
-        double       slab;
-        const double incl = block_scan_f64(part, s_fs.scan, &slab);
-        double       run  = carry + (incl - part);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            run += (double) p[c];
-            if (e + c < end && target < run) {
-                atomicMin(&s_fs.pick, e + c);
-                break;
-            }
-        }
-        carry += slab;
-    }
-    __syncthreads();
-    if (tid == 0)
-        a.out[row] = s_fs.pick == 0x7fffffff ? end - 1 : s_fs.pick;
+        a.out[row] = tok;
 }
 
 /* top-p / min-p over the whole vocabulary (sampler.c:232-305): the thread-maxima shortcut; a
@@ -1286,20 +1254,28 @@ static void dispatch(int nv, bool pen, F &&f) {
 
 void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
                          double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, const CandSpace *list, int zb_list) {
+                         float *probe_p, const CandSpace *list, int zb_list, double *slab_sum) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     if (list && L.nv == 8) {
         if (L.pen)
-            k_chunk_expsum<8, true, true><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, *list, zb_list);
+            k_chunk_expsum<8, true, true, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p, *list,
+                zb_list);
         else
-            k_chunk_expsum<8, false, true><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, *list, zb_list);
+            k_chunk_expsum<8, false, true, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p, *list,
+                zb_list);
         return;
     }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_chunk_expsum<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(
-            L.rv, inv_t, chunk_best, chunk_sum, probe_token, probe_L, probe_p, CandSpace{}, 0);
+        if (slab_sum)
+            k_chunk_expsum<GS_NV, GS_PEN, false, true><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, slab_sum, probe_token, probe_L, probe_p,
+                CandSpace{}, 0);
+        else
+            k_chunk_expsum<GS_NV, GS_PEN, false, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
+                CandSpace{}, 0);
     });
 }
 
@@ -1324,20 +1300,24 @@ void launch_spec(const Launch &L, const SpecLaunch &sp) {
     a.chunk_sum  = sp.chunk_sum;
     a.probe_p    = sp.probe_p;
     a.resid_sum  = sp.resid_sum;
+    a.resid_slab = sp.resid_slab;
+    a.slab_sum   = sp.slab_sum;
     a.out_tokens = sp.out_tokens;
     a.n_accepted = sp.n_accepted;
-    const dim3 block(TPB);
+    const dim3   block(TPB);
+    SpecVerdict *vd = static_cast<SpecVerdict *>(sp.verdict);
+    k_spec_accept<<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
     if (!sp.greedy) {
         const dim3 grid(L.rv.n_chunks, sp.n_seq);
         if (L.nv == 8)
-            k_spec_resid<8><<<grid, block, 0, L.stream>>>(L.rv, a);
+            k_spec_resid<8><<<grid, block, 0, L.stream>>>(L.rv, a, vd);
         else
-            k_spec_resid<2><<<grid, block, 0, L.stream>>>(L.rv, a);
+            k_spec_resid<2><<<grid, block, 0, L.stream>>>(L.rv, a, vd);
     }
     if (L.nv == 8)
-        k_spec_final<8><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a);
+        k_spec_final<8><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
     else
-        k_spec_final<2><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a);
+        k_spec_final<2><<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
 }
 
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best, int32_t *zero_per_row) {
@@ -1363,6 +1343,7 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.uniforms   = f.uniforms;
     a.chunk_best = f.chunk_best;
     a.chunk_sum  = f.chunk_sum;
+    a.slab_sum   = f.slab_sum;
     a.tmax       = f.tmax;
     a.row_flag   = f.row_flag;
     a.out        = f.out;

@@ -490,7 +490,6 @@ __device__ int list_jth_id(const float *pn, const uint32_t *ids, int n, uint32_t
     uint32_t  prefix = 0u;
     int       want   = j; /* 1-based rank inside the current digit range */
     for (int lv = 0; lv < 2; ++lv) {
-        const int shf = lv == 0 ? 10 : 0;
         for (int i = tid; i < SG_BINS; i += TPB)
             sh.cnt[i] = 0u;
         if (tid == 0)

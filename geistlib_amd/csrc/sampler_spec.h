@@ -12,8 +12,9 @@
  *   j* = L : token ~ p_L, the temperature sampler's walk (sampler.c:90-102) with u_L.
  *
  * Kernels (after k_tmax_scan + k_chunk_expsum over all n_seq * (L+1) target rows):
- *   k_spec_resid   grid (chunks, n_seq): finds j* and sums max(0, p - q) over its chunk of row j*
- *   k_spec_final   grid (n_seq): finds j* again, writes the accepted ids, draws the last token
+ *   k_spec_accept  grid (n_seq): row sums and maxima, j*, the accepted ids and their count
+ *   k_spec_resid   grid (chunks, n_seq): sums max(0, p - q) over its chunk of row j*
+ *   k_spec_final   grid (n_seq): draws the last token
  */
 #ifndef GEIST_SAMPLER_SPEC_H
 #define GEIST_SAMPLER_SPEC_H
@@ -32,129 +33,122 @@ struct SpecArgs {
     const double   *chunk_sum;
     const float    *probe_p; /* unnormalised p_j(x_j) per target row */
     double         *resid_sum; /* [n_seq][chunks] */
+    double         *resid_slab; /* [n_seq][chunks][SLABS_MAX] */
+    const double   *slab_sum;  /* [rows][chunks][SLABS_MAX] of the exp-sum pass */
     int32_t        *out_tokens; /* [n_seq][L+1] */
     int32_t        *n_accepted; /* [n_seq] */
 };
 
 constexpr int SPEC_L_MAX = 63;
 
-struct SpecShared {
-    double   row_sum[SPEC_L_MAX + 1];
-    uint64_t row_best[SPEC_L_MAX + 1];
-    float    q_tok[SPEC_L_MAX + 1];
-    int      first_reject;
+/* What k_spec_accept leaves per sequence for the two kernels behind it. */
+struct SpecVerdict {
+    double sum;   /* exp-sum of target row j* */
+    float  mx;    /* its maximum */
+    int    js;    /* j*: first rejected position, L when every draft token is accepted */
+    int    amax;  /* argmax of row j* (greedy mode) */
+    int    pad;
 };
+static_assert(sizeof(SpecVerdict) == SPEC_VERDICT_BYTES, "workspace is sized by the constant");
 
-/* Sums of every target row of the sequence (chunk order), the row maxima, q_j(x_j), then the
- * first rejected position. Every thread returns j* (L when all drafts are accepted). */
-__device__ __forceinline__ int spec_first_reject(const RowView &rv, const SpecArgs &a, int seq,
-                                                 SpecShared &sh) {
-    const int tid = threadIdx.x, C = rv.n_chunks, L = a.L;
-    if (tid <= L) {
-        const long row = (long) seq * (L + 1) + tid;
+/* ---- k_spec_accept --------------------------------------------------------------------------- */
+/* One workgroup per sequence. Groups of 16 lanes each take one target row: the lanes share the
+ * row's chunks, partial maxima / sums are combined inside the group in a fixed order (DPP row
+ * steps). Then lane j of the first wavefront tests position j and a ballot gives j*. */
+__global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, SpecVerdict *verdict) {
+    __shared__ double   s_sum[SPEC_L_MAX + 1];
+    __shared__ uint64_t s_best[SPEC_L_MAX + 1];
+    const int seq = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks, L = a.L;
+    const int part = tid & 15;
+    for (int j = tid >> 4; j <= L; j += TPB / 16) {
+        const long row = (long) seq * (L + 1) + j;
         uint64_t   b   = 0;
-        for (int c = 0; c < C; ++c) {
+        double     t   = 0.0;
+        for (int c = part; c < C; c += 16) {
             const uint64_t p = a.chunk_best[row * C + c];
             b                = p > b ? p : b;
+            if (!a.greedy)
+                t += a.chunk_sum[row * C + c];
         }
-        sh.row_best[tid] = b;
-        if (!a.greedy) {
-            double tot = 0.0;
-            for (int c = 0; c < C; ++c)
-                tot += a.chunk_sum[row * C + c];
-            sh.row_sum[tid] = tot;
-            float qt        = 0.0f;
-            if (tid < L) {
-                const int x = a.draft[(long) seq * L + tid];
-                if (x >= 0 && x < rv.n_vocab)
-                    qt = a.q[((long) seq * L + tid) * a.ld_q + x];
-            }
-            sh.q_tok[tid] = qt;
+        /* combine the 16 lanes of the group (one DPP row): lane 15 of the row ends with all */
+#define GS_DPP_MAX_U64(ctrl)                                                                    \
+    {                                                                                          \
+        const uint64_t ob =                                                                    \
+            ((uint64_t) (uint32_t) __builtin_amdgcn_update_dpp(0, (int) (b >> 32), ctrl, 0xf, 0xf, \
+                                                               false)                          \
+             << 32) |                                                                          \
+            (uint32_t) __builtin_amdgcn_update_dpp(0, (int) (uint32_t) b, ctrl, 0xf, 0xf, false); \
+        b = ob > b ? ob : b;                                                                   \
+    }
+        GS_DPP_MAX_U64(0x111) /* row_shr:1 */
+        GS_DPP_MAX_U64(0x112)
+        GS_DPP_MAX_U64(0x114)
+        GS_DPP_MAX_U64(0x118)
+#undef GS_DPP_MAX_U64
+        t += dpp_fetch_f64<0x111, 0xf>(t);
+        t += dpp_fetch_f64<0x112, 0xf>(t);
+        t += dpp_fetch_f64<0x114, 0xf>(t);
+        t += dpp_fetch_f64<0x118, 0xf>(t);
+        if (part == 15) {
+            s_best[j] = b;
+            s_sum[j]  = t;
         }
     }
     __syncthreads();
-    if (tid == 0) {
-        int j = 0;
-        for (; j < L; ++j) {
-            const long row = (long) seq * (L + 1) + j;
-            const int  x   = a.draft[(long) seq * L + j];
-            bool       ok;
-            if (a.greedy) {
-                /* a NaN at index 0 keeps the argmax at 0 (sampler.c:52-62) */
-                const float first = rv.logits[row * rv.ld];
-                const int   am    = (first != first) ? 0 : (int) best_idx(sh.row_best[j]);
-                ok                = x == am;
-            } else {
-                float pn = 0.0f;
-                if (x >= 0 && x < rv.n_vocab)
-                    pn = (float) ((double) a.probe_p[row] / sh.row_sum[j]);
-                ok = (double) a.uniforms[(long) seq * (L + 1) + j] * (double) sh.q_tok[j] <
-                     (double) pn;
-            }
-            if (!ok)
-                break;
-        }
-        sh.first_reject = j;
-    }
-    __syncthreads();
-    return sh.first_reject;
-}
-
-/* The four weights thread `tid` owns in slab j of a chunk: p_i (temperature walk) or
- * max(0, pn_i - q_i) (residual walk). Positions at or beyond `end` weigh 0. */
-template <bool RESID>
-__device__ __forceinline__ void slab_weights(const float4 &v, const float4 &qv, int e, int end,
-                                             float mx, float inv_t, double sum,
-                                             const uint64_t *tab, float (&w)[4]) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        float x = 0.0f;
-        if (e + c < end) {
-            const float p = geist_expf_glibc(softmax_arg(f4_get(v, c), mx, inv_t), tab);
-            if (RESID) {
-                const float r = __fsub_rn((float) ((double) p / sum), f4_get(qv, c));
-                x             = r > 0.0f ? r : 0.0f;
-            } else {
-                x = p;
-            }
-        }
-        w[c] = x;
-    }
-}
-
-template <int NV>
-__device__ __forceinline__ void load_q_chunk(const float *qrow, bool vec, int base, int end,
-                                             float4 (&qv)[NV]) {
-    const int tid = threadIdx.x;
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
-        if (vec && e + 3 < end) {
-            qv[j] = *reinterpret_cast<const float4 *>(qrow + e);
+    if (tid >= WAVE)
+        return;
+    bool ok = true; /* lanes at or beyond L never reject */
+    if (tid < L) {
+        const long row = (long) seq * (L + 1) + tid;
+        const int  x   = a.draft[(long) seq * L + tid];
+        if (a.greedy) {
+            /* a NaN at index 0 keeps the argmax at 0 (sampler.c:52-62) */
+            const float first = rv.logits[row * rv.ld];
+            ok                = x == ((first != first) ? 0 : (int) best_idx(s_best[tid]));
         } else {
-            qv[j].x = e + 0 < end ? qrow[e + 0] : 0.f;
-            qv[j].y = e + 1 < end ? qrow[e + 1] : 0.f;
-            qv[j].z = e + 2 < end ? qrow[e + 2] : 0.f;
-            qv[j].w = e + 3 < end ? qrow[e + 3] : 0.f;
+            float pn = 0.0f, qt = 0.0f;
+            if (x >= 0 && x < rv.n_vocab) {
+                pn = (float) ((double) a.probe_p[row] / s_sum[tid]);
+                qt = a.q[((long) seq * L + tid) * a.ld_q + x];
+            }
+            ok = (double) a.uniforms[(long) seq * (L + 1) + tid] * (double) qt < (double) pn;
         }
+    }
+    const uint64_t rej = __ballot(!ok);
+    const int      js  = rej ? __ffsll((long long) rej) - 1 : L;
+    if (tid < js)
+        a.out_tokens[(long) seq * (L + 1) + tid] = a.draft[(long) seq * L + tid];
+    if (tid == 0) {
+        const long  row   = (long) seq * (L + 1) + js;
+        const float first = rv.logits[row * rv.ld];
+        SpecVerdict v;
+        v.sum  = a.greedy ? 0.0 : s_sum[js];
+        v.mx   = key2f(best_key(s_best[js]));
+        v.js   = js;
+        v.amax = (first != first) ? 0 : (int) best_idx(s_best[js]);
+        v.pad  = 0;
+        verdict[seq]      = v;
+        a.n_accepted[seq] = js;
     }
 }
 
 /* ---- k_spec_resid ---------------------------------------------------------------------------- */
 template <int NV>
-__global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a) {
-    __shared__ SpecShared sh;
-    __shared__ double     s_sum[NWAVES];
-    __shared__ uint64_t   s_tab[32];
+__global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a,
+                                                    const SpecVerdict *__restrict__ verdict) {
+    __shared__ double   s_sum[NWAVES * NV];
+    __shared__ uint64_t s_tab[32];
     const int seq = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
-    const int js = spec_first_reject(rv, a, seq, sh);
+    const SpecVerdict vd = verdict[seq];
+    const int         js = vd.js;
     if (a.greedy || js >= a.L)
         return; /* nothing to resample from */
     const long   row = (long) seq * (a.L + 1) + js;
-    const float  mx  = key2f(best_key(sh.row_best[js]));
-    const double sum = sh.row_sum[js];
+    const float  mx  = vd.mx;
+    const double sum = vd.sum;
+    __syncthreads();
     int          base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4       v[NV], qv[NV];
@@ -162,121 +156,52 @@ __global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a) {
     const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
     load_raw<NV>(rv, rv.logits + row * rv.ld, base, end, v);
     load_q_chunk<NV>(qrow, qvec, base, end, qv);
-    double acc = 0.0;
+    double acc[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         float w[4];
         slab_weights<true>(v[j], qv[j], base + 4 * (j * TPB + tid), end, mx, a.inv_t, sum, s_tab, w);
-        acc += (double) w[0];
-        acc += (double) w[1];
-        acc += (double) w[2];
-        acc += (double) w[3];
+        acc[j] = (double) w[0];
+        acc[j] += (double) w[1];
+        acc[j] += (double) w[2];
+        acc[j] += (double) w[3];
     }
-    acc = block_sum_f64(acc, s_sum);
-    if (tid == 0)
-        a.resid_sum[(long) seq * rv.n_chunks + chunk] = acc;
-}
-
-/* Index-order walk over one row: locates the chunk from the per-chunk weights, then scans that
- * chunk slab by slab (index order inside a chunk is (slab, thread, component)). Returns the id
- * to every thread; when rounding leaves the target beyond the last weight, the last entry of
- * that chunk with a positive weight (the reference returns the last index, sampler.c:100-101). */
-template <int NV, bool RESID>
-__device__ int index_order_walk(const RowView &rv, long row, const double *chunk_w, int C,
-                                float u, float mx, float inv_t, double sum, const float *qrow,
-                                bool qvec, const uint64_t *tab, double *s_scan, int *s_i2,
-                                double *s_d2) {
-    const int tid = threadIdx.x;
+    block_sum_f64_multi<NV>(acc, s_sum);
     if (tid == 0) {
-        double tot = 0.0;
-        for (int c = 0; c < C; ++c)
-            tot += chunk_w[c];
-        const double target = (double) u * tot;
-        double       run    = 0.0;
-        int          at     = C - 1;
-        for (int c = 0; c < C; ++c) {
-            const double nxt = run + chunk_w[c];
-            if (target < nxt || c == C - 1) {
-                at = c;
-                break;
-            }
-            run = nxt;
-        }
-        s_i2[0] = at;
-        s_i2[1] = 0x7fffffff; /* pick */
-        s_i2[2] = -1;         /* last positive */
-        s_d2[0] = run;
-        s_d2[1] = target;
-    }
-    __syncthreads();
-    const int    chunk  = s_i2[0];
-    double       carry  = s_d2[0];
-    const double target = s_d2[1];
-    int          base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    float4 v[NV], qv[NV];
-    load_raw<NV>(rv, rv.logits + row * rv.ld, base, end, v);
-    if (RESID)
-        load_q_chunk<NV>(qrow, qvec, base, end, qv);
+        const long at  = (long) seq * rv.n_chunks + chunk;
+        double     tot = 0.0;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
-        float     w[4];
-        slab_weights<RESID>(v[j], RESID ? qv[j] : v[j], e, end, mx, inv_t, sum, tab, w);
-        const double part = (double) w[0] + (double) w[1] + (double) w[2] + (double) w[3];
-        double       slab;
-        const double incl = block_scan_f64(part, s_scan, &slab);
-        double       run  = carry + (incl - part);
-        int          lastpos = -1;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            run += (double) w[c];
-            if (w[c] > 0.0f)
-                lastpos = e + c;
-            if (e + c < end && w[c] > 0.0f && target < run) {
-                atomicMin(&s_i2[1], e + c);
-                break;
-            }
+        for (int j = 0; j < NV; ++j) {
+            a.resid_slab[at * SLABS_MAX + j] = acc[j];
+            tot += acc[j];
         }
-        if (lastpos >= 0)
-            atomicMax(&s_i2[2], lastpos);
-        carry += slab;
+        a.resid_sum[at] = tot;
     }
-    __syncthreads();
-    int tok = s_i2[1];
-    if (tok == 0x7fffffff)
-        tok = s_i2[2] >= 0 ? s_i2[2] : end - 1;
-    __syncthreads();
-    return tok;
 }
 
 /* ---- k_spec_final ---------------------------------------------------------------------------- */
 template <int NV>
-__global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a) {
-    __shared__ SpecShared sh;
-    __shared__ double     s_scan[NWAVES];
+__global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a,
+                                                    const SpecVerdict *__restrict__ verdict) {
+    __shared__ WalkShared s_walk;
     __shared__ double     s_w[MAX_CHUNKS];
     __shared__ uint64_t   s_tab[32];
-    __shared__ int        s_i2[4];
-    __shared__ double     s_d2[2];
     const int seq = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks, L = a.L;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
-    const int js = spec_first_reject(rv, a, seq, sh);
-    if (tid < js)
-        a.out_tokens[(long) seq * (L + 1) + tid] = a.draft[(long) seq * L + tid];
-    if (tid == 0)
-        a.n_accepted[seq] = js;
-    const long  row = (long) seq * (L + 1) + js;
-    const float u   = a.uniforms[(long) seq * (L + 1) + L];
-    int         tok;
+    GS_MARK(0);
+    const SpecVerdict vd  = verdict[seq];
+    const int         js  = vd.js;
+    const long        row = (long) seq * (L + 1) + js;
+    const float       u   = a.uniforms[(long) seq * (L + 1) + L];
+    int               tok;
     if (a.greedy) {
-        const float first = rv.logits[row * rv.ld];
-        tok               = (first != first) ? 0 : (int) best_idx(sh.row_best[js]);
+        tok = vd.amax;
     } else {
-        const float  mx   = key2f(best_key(sh.row_best[js]));
-        const double sum  = sh.row_sum[js];
+        const float  mx    = vd.mx;
+        const double sum   = vd.sum;
         bool         resid = js < L;
+        GS_MARK(1);
         if (resid) {
             if (tid < C)
                 s_w[tid] = a.resid_sum[(long) seq * C + tid];
@@ -290,14 +215,18 @@ __global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a) {
         if (resid) {
             const float *qrow = a.q + ((long) seq * L + js) * a.ld_q;
             const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
-            tok = index_order_walk<NV, true>(rv, row, s_w, C, u, mx, a.inv_t, sum, qrow, qvec,
-                                             s_tab, s_scan, s_i2, s_d2);
+            tok = index_order_walk<NV, false, true>(rv, (int) row, 0, s_w,
+                                                    a.resid_slab + (long) seq * C * SLABS_MAX, C, u,
+                                                    mx, a.inv_t, sum, qrow, qvec, s_tab, nullptr,
+                                                    s_walk);
         } else {
             if (tid < C)
                 s_w[tid] = a.chunk_sum[row * C + tid];
             __syncthreads();
-            tok = index_order_walk<NV, false>(rv, row, s_w, C, u, mx, a.inv_t, sum, nullptr, false,
-                                              s_tab, s_scan, s_i2, s_d2);
+            tok = index_order_walk<NV, false, false>(rv, (int) row, 0, s_w,
+                                                     a.slab_sum + row * C * SLABS_MAX, C, u, mx,
+                                                     a.inv_t, sum, nullptr, false, s_tab, nullptr,
+                                                     s_walk);
         }
     }
     if (tid == 0)

@@ -1,0 +1,160 @@
+/*
+ * sampler_walk.h -- the index-order walk the temperature sampler (src/engine/sampler.c:90-102),
+ * the bonus token and the residual resampling of speculative verification share. Included by
+ * sampler_kernels.hip.
+ *
+ * A row is never walked from its start. The streaming pass leaves, per chunk, the sum of the
+ * weights and the sums of the chunk's slabs: slab j of a chunk is the 1024 consecutive elements
+ * the threads t = 0..255 hold as their j-th float4, positions base + 4 * (j * 256 + t) + c.
+ * Index order inside a chunk is (slab, thread, component), so the chunk is located from the chunk
+ * sums, the slab from the slab sums, and only that slab is read again: 4 elements per thread,
+ * one workgroup scan.
+ */
+#ifndef GEIST_SAMPLER_WALK_H
+#define GEIST_SAMPLER_WALK_H
+
+namespace gs {
+
+
+/* The four weights thread `tid` owns in a slab: p_i (temperature walk) or max(0, pn_i - q_i)
+ * (residual walk). Positions at or beyond `end` weigh 0. */
+template <bool RESID>
+__device__ __forceinline__ void slab_weights(const float4 &v, const float4 &qv, int e, int end,
+                                             float mx, float inv_t, double sum,
+                                             const uint64_t *tab, float (&w)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float x = 0.0f;
+        if (e + c < end) {
+            const float p = geist_expf_glibc(softmax_arg(f4_get(v, c), mx, inv_t), tab);
+            if (RESID) {
+                const float r = __fsub_rn((float) ((double) p / sum), f4_get(qv, c));
+                x             = r > 0.0f ? r : 0.0f;
+            } else {
+                x = p;
+            }
+        }
+        w[c] = x;
+    }
+}
+
+template <int NV>
+__device__ __forceinline__ void load_q_chunk(const float *qrow, bool vec, int base, int end,
+                                             float4 (&qv)[NV]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+        if (vec && e + 3 < end) {
+            qv[j] = *reinterpret_cast<const float4 *>(qrow + e);
+        } else {
+            qv[j].x = e + 0 < end ? qrow[e + 0] : 0.f;
+            qv[j].y = e + 1 < end ? qrow[e + 1] : 0.f;
+            qv[j].z = e + 2 < end ? qrow[e + 2] : 0.f;
+            qv[j].w = e + 3 < end ? qrow[e + 3] : 0.f;
+        }
+    }
+}
+
+struct WalkShared {
+    double scan[NWAVES];
+    double before, target;
+    int    chunk, slab, pick, last_pos;
+};
+
+/* Walks row `row` in index order for the first element at which the running weight exceeds
+ * u * (sum of chunk_w). chunk_w: C per-chunk weights in LDS; slab_w: the row's C * SLABS_MAX slab
+ * weights in global memory; NV: slabs per chunk of the pass that wrote them. Returns the id to
+ * every thread. Should rounding leave the target beyond the located slab, the following slabs of
+ * the chunk are walked too; beyond those the chunk's last index (the reference returns the last
+ * index of the row, sampler.c:100-101; the located chunk is then the last one), for the residual
+ * walk the last element seen with a positive weight. */
+template <int NV, bool PEN, bool RESID>
+__device__ int index_order_walk(const RowView &rv, int row, int n_rows, const double *chunk_w,
+                                const double *__restrict__ slab_w, int C, float u, float mx,
+                                float inv_t, double sum, const float *qrow, bool qvec,
+                                const uint64_t *tab, uint32_t *s_cnt16, WalkShared &sh) {
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        double tot = 0.0;
+        for (int c = 0; c < C; ++c)
+            tot += chunk_w[c];
+        const double target = (double) u * tot;
+        double       run    = 0.0;
+        int          at     = C - 1;
+        for (int c = 0; c < C; ++c) {
+            const double nxt = run + chunk_w[c];
+            if (target < nxt || c == C - 1) {
+                at = c;
+                break;
+            }
+            run = nxt;
+        }
+        int js = NV - 1;
+        for (int j = 0; j < NV; ++j) {
+            const double nxt = run + slab_w[at * SLABS_MAX + j];
+            if (target < nxt || j == NV - 1) {
+                js = j;
+                break;
+            }
+            run = nxt;
+        }
+        sh.chunk    = at;
+        sh.slab     = js;
+        sh.before   = run;
+        sh.target   = target;
+        sh.pick     = 0x7fffffff;
+        sh.last_pos = -1;
+    }
+    __syncthreads();
+    const int    chunk  = sh.chunk;
+    double       carry  = sh.before;
+    const double target = sh.target;
+    int          base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    for (int j = sh.slab; j < NV; ++j) {
+        const int sbase = base + j * 4 * TPB;
+        if (sbase >= end)
+            break;
+        const int send = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
+        float4    v[1], qv[1];
+        fetch_chunk<1, PEN>(rv, row, n_rows, sbase, send, s_cnt16, v); /* a slab is a chunk of 1024 */
+        qv[0] = v[0];
+        if (RESID)
+            load_q_chunk<1>(qrow, qvec, sbase, send, qv);
+        const int e = sbase + 4 * tid;
+        float     w[4];
+        slab_weights<RESID>(v[0], qv[0], e, send, mx, inv_t, sum, tab, w);
+        const double part = (double) w[0] + (double) w[1] + (double) w[2] + (double) w[3];
+        double       slab;
+        const double incl = block_scan_f64(part, sh.scan, &slab);
+        double       run  = carry + (incl - part);
+        int          lastpos = -1;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            run += (double) w[c];
+            if (w[c] > 0.0f)
+                lastpos = e + c;
+            if (e + c < send && w[c] > 0.0f && target < run) {
+                atomicMin(&sh.pick, e + c);
+                break;
+            }
+        }
+        if (RESID && lastpos >= 0)
+            atomicMax(&sh.last_pos, lastpos);
+        __syncthreads();
+        if (sh.pick != 0x7fffffff)
+            break;
+        carry += slab;
+        __syncthreads();
+    }
+    __syncthreads();
+    int tok = sh.pick;
+    if (tok == 0x7fffffff)
+        tok = RESID && sh.last_pos >= 0 ? sh.last_pos : end - 1;
+    __syncthreads();
+    return tok;
+}
+
+} // namespace gs
+#endif
