@@ -1411,8 +1411,15 @@ void launch_candidates(const Launch &L, const FinalLaunch &f) {
         k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
             L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
     });
-    k_sorted_candidates<<<dim3(L.rows), block, 0, L.stream>>>(f.cand, f.top_p, f.min_p, f.uniforms,
-                                                             f.row_flag, f.out);
+    static bool lds_set = false; /* once per process: the kernel's LDS beyond the static part */
+    const int   dyn     = CAND_CAP * (int) sizeof(uint32_t);
+    if (!lds_set) {
+        (void) hipFuncSetAttribute((const void *) k_sorted_candidates,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
+        lds_set = true;
+    }
+    k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(f.cand, f.top_p, f.min_p, f.uniforms,
+                                                               f.row_flag, f.out);
 }
 
 void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {

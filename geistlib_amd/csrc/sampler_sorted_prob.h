@@ -279,12 +279,10 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
                 }
                 if (rv.softcap > 0.0f)
                     x = __fmul_rn(tanhf(__fdiv_rn(x, rv.softcap)), rv.softcap);
-                if (x >= bound) {
-                    const float pn =
-                        (float) ((double) geist_expf_glibc(softmax_arg(x, mx, a.inv_t), tab) / sum);
+                if (x >= bound) { /* the logit for now; its probability below, one per thread */
                     const int at = atomicAdd(s_n2, 1);
                     if (at < TPB)
-                        s_m[at] = pack_best(__float_as_uint(pn), (uint32_t) (e0[q] + c));
+                        s_m[at] = ((uint64_t) __float_as_uint(x) << 32) | (uint32_t) (e0[q] + c);
                 }
             }
         }
@@ -294,6 +292,14 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     GS_MARK(5);
     if (m > TPB || m < 1)
         return -1;
+    if (tid < m) {
+        const uint64_t ent = s_m[tid];
+        const float    x   = __uint_as_float((uint32_t) (ent >> 32));
+        const float    pn  =
+            (float) ((double) geist_expf_glibc(softmax_arg(x, mx, a.inv_t), tab) / sum);
+        s_m[tid] = pack_best(__float_as_uint(pn), (uint32_t) ent);
+    }
+    __syncthreads();
     /* 4: order by counting, entry i compared by P = 256 / m2 <= 64 neighbouring lanes */
     int m2 = 4;
     while (m2 < m)
@@ -756,6 +762,8 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(RowView rv, float inv_t,
  * normalised probability pn = (float)((double)p / sum), vocabulary id). A list longer than
  * CAND_CAP keeps counting; the row-final kernel then hands the row on.
  * ========================================================================================== */
+constexpr int LIST_STAGE = 2048; /* candidates of one chunk staged in LDS */
+
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t,
                                                          const uint64_t *__restrict__ chunk_best,
@@ -767,6 +775,9 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     __shared__ uint64_t s_red[NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ double   s_total;
+    __shared__ int      s_count, s_base;
+    __shared__ float    s_arg[LIST_STAGE];
+    __shared__ uint32_t s_id[LIST_STAGE];
     const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (row_flag[row] != 1)
         return;
@@ -778,6 +789,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
         for (int c = 0; c < rv.n_chunks; ++c)
             t += chunk_sum[(long) row * rv.n_chunks + c];
         s_total = t;
+        s_count = 0;
     }
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
@@ -799,22 +811,55 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
         }
     }
     GS_MARK(6);
-    int       pos = wave_reserve(__popc(mask), &cand.count[row]);
+    /* places: inside the workgroup through LDS, one global add for the workgroup */
+    int pos = wave_reserve(__popc(mask), &s_count);
+    __syncthreads();
+    const int n_blk = s_count;
+    if (tid == 0)
+        s_base = n_blk ? atomicAdd(&cand.count[row], n_blk) : 0;
     GS_MARK(7);
-    uint32_t *ck  = cand.key + (long) row * CAND_CAP;
-    uint32_t *ci  = cand.idx + (long) row * CAND_CAP;
+    uint32_t *ck = cand.key + (long) row * CAND_CAP;
+    uint32_t *ci = cand.idx + (long) row * CAND_CAP;
+    if (n_blk <= LIST_STAGE) {
+        /* stage (softmax argument, id) densely, then one exponential per staged entry */
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + tid);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if ((mask >> (4 * j + c)) & 1u) {
-                if (pos < CAND_CAP) {
-                    const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
-                    ck[pos]       = __float_as_uint((float) ((double) p / tot));
-                    ci[pos]       = (uint32_t) (e + c);
+            for (int c = 0; c < 4; ++c) {
+                if ((mask >> (4 * j + c)) & 1u) {
+                    s_arg[pos] = softmax_arg(f4_get(v[j], c), mx, inv_t);
+                    s_id[pos]  = (uint32_t) (e + c);
+                    ++pos;
                 }
-                ++pos;
+            }
+        }
+        __syncthreads();
+        const int gbase = s_base;
+        for (int i = tid; i < n_blk; i += TPB) {
+            if (gbase + i < CAND_CAP) {
+                const float p   = geist_expf_glibc(s_arg[i], s_tab);
+                ck[gbase + i]   = __float_as_uint((float) ((double) p / tot));
+                ci[gbase + i]   = s_id[i];
+            }
+        }
+    } else {
+        __syncthreads();
+        pos += s_base;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if ((mask >> (4 * j + c)) & 1u) {
+                    if (pos < CAND_CAP) {
+                        const float p =
+                            geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                        ck[pos] = __float_as_uint((float) ((double) p / tot));
+                        ci[pos] = (uint32_t) (e + c);
+                    }
+                    ++pos;
+                }
             }
         }
     }
@@ -1016,13 +1061,13 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
                                                            const float *__restrict__ uniforms,
                                                            int32_t *__restrict__ row_flag,
                                                            int32_t *__restrict__ out) {
+    extern __shared__ uint32_t s_key[]; /* CAND_CAP keys: every list is walked from LDS */
     __shared__ union {
         SortedGenShared gen;
         ListWalkShared  fast;
     } sh;
     __shared__ int      s_scan[NWAVES];
     __shared__ int      s_pick;
-    __shared__ uint32_t s_key[CAND_LDS];
     __shared__ uint32_t s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int flag = row_flag[row];
@@ -1032,25 +1077,30 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
     int       tok = -1;
     GS_MARK(0);
     if (n >= 1 && n <= CAND_CAP) {
-        uint32_t       *wk = cand.key + (long) row * CAND_CAP;
-        const uint32_t *gk = wk;
+        const uint32_t *gk = cand.key + (long) row * CAND_CAP;
         const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
         /* flag 4: the list holds p; pn = (float)((double)p / sum), sampler.c:251-253 */
         const double sum = flag == 4 ? cand.row_sum[row] : 1.0;
-        if (n <= CAND_LDS) {
-            for (int i = tid; i < n; i += TPB) {
-                const uint32_t k = gk[i];
-                s_key[i] = flag == 4 ? __float_as_uint((float) ((double) __uint_as_float(k) / sum)) : k;
-                s_idx[i] = gi[i];
+        for (int i0 = 0; i0 < n; i0 += 4 * TPB) { /* four independent loads in flight per thread */
+            uint32_t k[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                k[q] = i0 + q * TPB + tid < n ? gk[i0 + q * TPB + tid] : 0u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = i0 + q * TPB + tid;
+                if (i < n)
+                    s_key[i] = flag == 4 ? __float_as_uint((float) ((double) __uint_as_float(k[q]) / sum))
+                                         : k[q];
             }
-            __syncthreads();
-            gk = s_key;
-            gi = s_idx;
-        } else if (flag == 4) {
-            for (int i = tid; i < n; i += TPB)
-                wk[i] = __float_as_uint((float) ((double) __uint_as_float(wk[i]) / sum));
-            __syncthreads();
         }
+        if (n <= CAND_LDS) {
+            for (int i = tid; i < n; i += TPB)
+                s_idx[i] = gi[i];
+            gi = s_idx;
+        }
+        __syncthreads();
+        gk = s_key;
         GS_MARK(1);
         const float *keys = reinterpret_cast<const float *>(gk);
         tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], cand.out_key[row], sh.fast);
