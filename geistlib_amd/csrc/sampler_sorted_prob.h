@@ -903,23 +903,30 @@ __device__ __forceinline__ uint64_t wave_scan_u64(uint64_t v) {
 /* Orders and walks the entries of bin `b` that belong to the kept set (pack >= edge_pack): the
  * first one at which `before` plus the running mass reaches `target` goes to sh.out_pack, the
  * running mass including it to sh.out_mass. Returns false when the bin holds too many. */
-__device__ bool list_resolve_bin(const float *pn, const uint32_t *ids, int n, uint32_t kout,
+__device__ __forceinline__ bool list_resolve_bin(const float *pn, const uint32_t *ids, int n, uint32_t kout,
                                  uint32_t kmax, int shift, int b, uint64_t before, uint64_t target,
                                  uint64_t edge_pack, ListWalkShared &sh) {
     const int tid = threadIdx.x;
     if (tid == 0)
         sh.n_small = 0;
     __syncthreads();
-    for (int i = tid; i < n; i += TPB) {
-        const uint32_t key = __float_as_uint(pn[i]);
-        if (key <= kout || (int) ((kmax - key) >> shift) != b)
-            continue;
-        const uint64_t pk = pack_best(key, ids[i]);
-        if (pk < edge_pack)
-            continue;
-        const int at = atomicAdd(&sh.n_small, 1);
-        if (at < TPB)
-            sh.small[at] = pk;
+    for (int i0 = tid; i0 < n; i0 += 4 * TPB) {
+        uint32_t k[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            k[q] = i0 + q * TPB < n ? __float_as_uint(pn[i0 + q * TPB]) : 0u;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t key = k[q];
+            if (key <= kout || (int) ((kmax - key) >> shift) != b)
+                continue;
+            const uint64_t pk = pack_best(key, ids[i0 + q * TPB]);
+            if (pk < edge_pack)
+                continue;
+            const int at = atomicAdd(&sh.n_small, 1);
+            if (at < TPB)
+                sh.small[at] = pk;
+        }
     }
     __syncthreads();
     const int c = sh.n_small;
@@ -933,34 +940,59 @@ __device__ bool list_resolve_bin(const float *pn, const uint32_t *ids, int n, ui
         sh.srt[rank] = me;
     }
     __syncthreads();
-    if (tid == 0) {
-        uint64_t run = before;
-        int      at  = c - 1;
-        for (int i = 0; i < c; ++i) {
-            run += pn_fx(__uint_as_float(best_key(sh.srt[i])));
-            if (run >= target) {
-                at = i;
-                break;
+    if (tid < WAVE) { /* lane l walks entries 4l .. 4l+3 behind the lanes before it */
+        uint64_t f[4], tot = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int i = 4 * tid + q;
+            f[q]        = i < c ? pn_fx(__uint_as_float(best_key(sh.srt[i]))) : 0ull;
+            tot += f[q];
+        }
+        uint64_t run = before + wave_scan_u64(tot) - tot;
+        int      at  = 0x7fffffff;
+        uint64_t at_mass = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            run += f[q];
+            if (at == 0x7fffffff && 4 * tid + q < c && run >= target) {
+                at      = 4 * tid + q;
+                at_mass = run;
             }
         }
-        sh.out_pack = c > 0 ? sh.srt[at] : 0ull;
-        sh.out_mass = run;
+        const uint64_t hit = __ballot(at != 0x7fffffff);
+        if (hit) {
+            if (tid == __ffsll((long long) hit) - 1) {
+                sh.out_pack = sh.srt[at];
+                sh.out_mass = at_mass;
+            }
+        } else if (tid == (c > 0 ? (c - 1) / 4 : 0)) {
+            /* not reached inside the bin (cannot happen with exact masses): its last entry */
+            sh.out_pack = c > 0 ? sh.srt[c - 1] : 0ull;
+            sh.out_mass = run;
+        }
     }
     __syncthreads();
     return true;
 }
 
-__device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float top_p, float min_p,
-                              float u, uint32_t kout, ListWalkShared &sh) {
+__device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *ids, int n,
+                                              float top_p, float min_p, float u, uint32_t kout,
+                                              ListWalkShared &sh) {
     const int  tid   = threadIdx.x;
     const bool use_p = top_p > 0.0f && top_p < 1.0f;
     const bool use_m = min_p > 0.0f;
     uint32_t   kmax  = 0u;
-    for (int i = tid; i < n; i += TPB) {
-        const uint32_t key = __float_as_uint(pn[i]);
-        kmax               = key > kmax ? key : kmax;
+    for (int i0 = tid; i0 < n; i0 += 4 * TPB) {
+        uint32_t k[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            k[q] = i0 + q * TPB < n ? __float_as_uint(pn[i0 + q * TPB]) : 0u;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            kmax = k[q] > kmax ? k[q] : kmax;
     }
     kmax = (uint32_t) block_max_u64((uint64_t) wave_max_u32(kmax), sh.red64);
+    GS_MARK(8);
     if (kmax <= kout)
         return -1;
     const int   bits    = 32 - __clz((int) (kmax - kout));
@@ -970,17 +1002,26 @@ __device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float
         sh.mass[i] = 0ull;
     __syncthreads();
     uint64_t lm = 0;
-    for (int i = tid; i < n; i += TPB) {
-        const float    p   = pn[i];
-        const uint32_t key = __float_as_uint(p);
-        if (key <= kout)
-            continue;
-        const uint64_t fx = pn_fx(p);
-        atomicAdd((unsigned long long *) &sh.mass[(kmax - key) >> shift], (unsigned long long) fx);
-        if (use_m && p >= floor_w)
-            lm += fx;
+    for (int i0 = tid; i0 < n; i0 += 4 * TPB) { /* the loads first: the adds below may alias them */
+        float p4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            p4[q] = i0 + q * TPB < n ? pn[i0 + q * TPB] : 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float    p   = p4[q];
+            const uint32_t key = __float_as_uint(p);
+            if (key <= kout) /* also the padding: kout >= 1 */
+                continue;
+            const uint64_t fx = pn_fx(p);
+            atomicAdd((unsigned long long *) &sh.mass[(kmax - key) >> shift],
+                      (unsigned long long) fx);
+            if (use_m && p >= floor_w)
+                lm += fx;
+        }
     }
     __syncthreads();
+    GS_MARK(9);
     const uint64_t mass_m = use_m ? block_sum_u64(lm, sh.red64) : 0ull;
     /* exclusive prefix of the bins: thread t owns bins 8t .. 8t+7 */
     constexpr int PER = SG_BINS / TPB;
@@ -995,6 +1036,7 @@ __device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float
     for (int w = 0; w < tid / WAVE; ++w)
         excl += sh.scan64[w];
     excl -= own;
+    GS_MARK(10);
     /* the bin at which the running mass reaches `target`; optionally the mass before bin `be` */
     auto locate = [&](uint64_t target, int be) {
         if (tid == 0)
@@ -1030,6 +1072,7 @@ __device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float
             mass_keep = sh.out_mass;
         }
     }
+    GS_MARK(11);
     const uint32_t kf = __float_as_uint(floor_w);
     if (use_m && (!have_p || kf > best_key(edge_pack))) {
         if (kf <= kout)
@@ -1045,6 +1088,7 @@ __device__ int list_walk_fast(const float *pn, const uint32_t *ids, int n, float
     locate(target2, be);
     int      bd     = sh.res_bin;
     uint64_t before = sh.res_before;
+    GS_MARK(12);
     if (bd < 0 || bd >= be) { /* inside the partly kept bin of the edge */
         bd     = be;
         before = sh.res_before_edge;
@@ -1081,13 +1125,13 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
         const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
         /* flag 4: the list holds p; pn = (float)((double)p / sum), sampler.c:251-253 */
         const double sum = flag == 4 ? cand.row_sum[row] : 1.0;
-        for (int i0 = 0; i0 < n; i0 += 4 * TPB) { /* four independent loads in flight per thread */
-            uint32_t k[4];
+        for (int i0 = 0; i0 < n; i0 += 8 * TPB) { /* eight independent loads in flight per thread */
+            uint32_t k[8];
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int q = 0; q < 8; ++q)
                 k[q] = i0 + q * TPB + tid < n ? gk[i0 + q * TPB + tid] : 0u;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int q = 0; q < 8; ++q) {
                 const int i = i0 + q * TPB + tid;
                 if (i < n)
                     s_key[i] = flag == 4 ? __float_as_uint((float) ((double) __uint_as_float(k[q]) / sum))
