@@ -77,6 +77,7 @@ def load_library():
                                                          C.POINTER(SampleParams), vp, vp, i32,
                                                          C.POINTER(C.c_double)]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
+    lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
     _LIB = lib
     return lib
 
@@ -175,6 +176,15 @@ class HipSampler:
             self.h, C.byref(rows), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
             C.byref(ms)))
         return ms.value * 1e3 / launches
+
+    def logprob(self, logits, tokens, out, softcap=0.0):
+        """out[r, j] = log_softmax(logits[r])[tokens[r, j]] (float64), logits soft-capped first
+        when softcap > 0."""
+        rows, n = logits.shape
+        assert tokens.shape == out.shape and tokens.shape[0] == rows
+        self._check(self.lib.geist_hip_logprob_rows(
+            self.h, _ptr(logits), logits.stride(0), rows, n, softcap, _ptr(tokens),
+            tokens.stride(0), tokens.shape[1], _ptr(out), out.stride(0)))
 
     def row_paths(self, rows):
         """Which walk served each row of the last full-vocabulary top-p / min-p call

@@ -504,6 +504,34 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     return after_launch(s, "softmax");
 }
 
+int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t ld, size_t rows,
+                           size_t n_vocab, float logit_softcap, const int32_t *d_tokens,
+                           size_t tokens_ld, size_t k_per_row, double *d_out, size_t out_ld) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_tokens || !d_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null tokens or output");
+    if (k_per_row == 0 || tokens_ld < k_per_row || out_ld < k_per_row)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "k_per_row %zu with strides %zu / %zu", k_per_row,
+                    tokens_ld, out_ld);
+    if (k_per_row > 0x7fffffffu)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "k_per_row too large");
+    struct geist_hip_rows          r = {d_logits, ld, rows, n_vocab, nullptr, 0, nullptr};
+    struct geist_hip_sample_params p = {};
+    p.temperature        = 1.0f;
+    p.repetition_penalty = 1.0f;
+    p.logit_softcap      = logit_softcap;
+    Launch L;
+    int    rc = make_launch(s, &r, &p, true, L);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_tmax_scan(L, s->tmax, s->chunk_best);
+    launch_logprob(L, s->chunk_best, s->chunk_sum, d_tokens, (long) tokens_ld, (int) k_per_row,
+                   d_out, (long) out_ld);
+    return after_launch(s, "log-probabilities");
+}
+
 int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
                           const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
                           const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,

@@ -15,6 +15,7 @@
 #include <stdint.h>
 
 #include "glibc_expf.h"
+#include "glibc_tanhf.h"
 #include "sampler_kernels.h"
 
 namespace gs {
@@ -450,10 +451,10 @@ __device__ __forceinline__ void apply_transform(const RowView &rv, const uint32_
         const float c = rv.softcap;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            v[j].x = __fmul_rn(tanhf(__fdiv_rn(v[j].x, c)), c);
-            v[j].y = __fmul_rn(tanhf(__fdiv_rn(v[j].y, c)), c);
-            v[j].z = __fmul_rn(tanhf(__fdiv_rn(v[j].z, c)), c);
-            v[j].w = __fmul_rn(tanhf(__fdiv_rn(v[j].w, c)), c);
+            v[j].x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].x, c)), c);
+            v[j].y = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].y, c)), c);
+            v[j].z = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].z, c)), c);
+            v[j].w = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].w, c)), c);
         }
     }
 }

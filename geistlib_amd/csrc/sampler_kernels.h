@@ -126,6 +126,9 @@ void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best
                         const int32_t *row_flag);
 /* rows flagged 2: probabilities of the whole row into `probs`, then the walk over them */
 void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs);
+/* after launch_tmax_scan(L, tmax, chunk_best): out[row][j] = log_softmax(row)[tokens[row][j]] */
+void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,
+                    const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

@@ -824,7 +824,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
                         x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
                 }
                 if (rv.softcap > 0.0f)
-                    x = __fmul_rn(tanhf(__fdiv_rn(x, rv.softcap)), rv.softcap);
+                    x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);
                 if (x >= bound) {
                     const int at = atomicAdd(s_n2, 1);
                     if (at < TPB)
@@ -1173,6 +1173,71 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
 }
 
 /* ============================================================================================
+ * Log-probability scoring: log_softmax(row)[token] for K tokens per row, as the reference's
+ * evaluation tool computes it from peeked logits (tools/eval_geist.c:63-73 over
+ * geist_session_peek_logits, src/archs/transformer/arch.c:167-197, which hands out the soft-capped
+ * values): fp32 max, double exp of the fp32 difference, double sum, then
+ * (double)(l[token] - max) - log(sum). Only K doubles per row leave the device.
+ *   k_chunk_lse      grid (chunks, rows): sum of exp((double)(l - max)) over the chunk
+ *   k_final_logprob  grid (rows): log of the row's sum, then the K values
+ * ========================================================================================== */
+template <int NV>
+__global__ __launch_bounds__(TPB) void k_chunk_lse(RowView rv, const uint64_t *__restrict__ chunk_best,
+                                                   double *__restrict__ chunk_sum) {
+    __shared__ uint64_t s_red[NWAVES];
+    __shared__ double   s_sum[NWAVES];
+    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    int                 base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    float4 v[NV];
+    fetch_chunk<NV, false>(rv, row, (int) gridDim.y, base, end, nullptr, v);
+    const float mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
+    double      acc = 0.0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (e + c < end)
+                acc += exp((double) __fsub_rn(f4_get(v[j], c), mx));
+    }
+    acc = block_sum_f64(acc, s_sum);
+    if (tid == 0)
+        chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+}
+
+__global__ __launch_bounds__(TPB) void k_final_logprob(RowView rv,
+                                                       const uint64_t *__restrict__ chunk_best,
+                                                       const double *__restrict__ chunk_sum,
+                                                       const int32_t *__restrict__ tokens,
+                                                       long tokens_ld, int k_per_row,
+                                                       double *__restrict__ out, long out_ld) {
+    __shared__ uint64_t s_red[NWAVES];
+    __shared__ double   s_lse;
+    const int           row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
+    const float mx = key2f(best_key(row_best_from_chunks(chunk_best, row, C, s_red)));
+    if (tid == 0) {
+        double tot = 0.0;
+        for (int c = 0; c < C; ++c)
+            tot += chunk_sum[(long) row * C + c];
+        s_lse = log(tot);
+    }
+    __syncthreads();
+    const double lse = s_lse;
+    for (int j = tid; j < k_per_row; j += TPB) {
+        const int t = tokens[(long) row * tokens_ld + j];
+        double    r = __builtin_nan("");
+        if (t >= 0 && t < rv.n_vocab) {
+            float x = rv.logits[(long) row * rv.ld + t];
+            if (rv.softcap > 0.0f)
+                x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);
+            r = (double) __fsub_rn(x, mx) - lse;
+        }
+        out[(long) row * out_ld + j] = r;
+    }
+}
+
+/* ============================================================================================
  * k_penalties: in-place penalties; only the penalised positions are written back.
  * ========================================================================================== */
 template <int NV>
@@ -1428,6 +1493,17 @@ void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, 
             L.rv, f.inv_t, f.chunk_best, f.chunk_sum, probs, ld_probs, f.top_p, f.min_p, f.uniforms,
             f.row_flag, f.out, f.cand.path);
     });
+}
+
+void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,
+                    const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld) {
+    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    if (L.nv == 8)
+        k_chunk_lse<8><<<grid, block, 0, L.stream>>>(L.rv, chunk_best, chunk_sum);
+    else
+        k_chunk_lse<2><<<grid, block, 0, L.stream>>>(L.rv, chunk_best, chunk_sum);
+    k_final_logprob<<<dim3(L.rows), block, 0, L.stream>>>(L.rv, chunk_best, chunk_sum, tokens,
+                                                         tokens_ld, k_per_row, out, out_ld);
 }
 
 void launch_penalties(const Launch &L, float *logits_rw) {

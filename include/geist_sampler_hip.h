@@ -131,6 +131,19 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
                            const struct geist_hip_sample_params *params, float *d_probs,
                            size_t ld_probs);
 
+/* Scoring without moving logits to the host. Replaces geist_session_peek_logits
+ * (include/geist_util.h:195-211; src/archs/transformer/arch.c:167-197, which hands out the
+ * soft-capped values) followed by the log-softmax lookup of the reference's evaluation tool
+ * (logprob_at, tools/eval_geist.c:63-73), for k_per_row candidate tokens of each row:
+ *   d_out[r * out_ld + j] = (double)(l[t] - max) - log(sum_i exp((double)(l_i - max))),
+ *   t = d_tokens[r * tokens_ld + j], l = the row after tanhf(x / cap) * cap when cap > 0.
+ * Token ids outside [0, n_vocab) give NaN. No penalties, no temperature: peek_logits exposes the
+ * model's values. Double results; against the CPU statement they differ only by the order of the
+ * double sum and the last bit of exp/log (bound 1e-9 absolute in the tests). */
+int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t ld, size_t rows,
+                           size_t n_vocab, float logit_softcap, const int32_t *d_tokens,
+                           size_t tokens_ld, size_t k_per_row, double *d_out, size_t out_ld);
+
 /* Speculative-decode verification for n_seq sequences with draft length L (no reference
  * counterpart: include/geist_util.h:233-240 documents that the reference's speculative loop
  * omits rejection sampling; the batch shape is that of verify_forward,

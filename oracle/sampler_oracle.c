@@ -641,3 +641,15 @@ void oracle_batch_chain_u(size_t rows, size_t n, const float *logits, size_t ld,
         free(tmp);
     }
 }
+
+/* tools/eval_geist.c:63-73 */
+double oracle_logprob_at(size_t n, const float *logits, int32_t token) {
+    float maxv = logits[0];
+    for (size_t i = 1; i < n; i++)
+        if (logits[i] > maxv)
+            maxv = logits[i];
+    double sum = 0.0;
+    for (size_t i = 0; i < n; i++)
+        sum += exp((double) (logits[i] - maxv));
+    return (double) (logits[token] - maxv) - log(sum);
+}

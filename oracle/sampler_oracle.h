@@ -155,6 +155,11 @@ void oracle_batch_chain_u(size_t rows, size_t n, const float *logits, size_t ld,
                           const float *u, int32_t *out, int threads);
 int  oracle_max_threads(void);
 
+/* log_softmax(logits)[token] as the reference's evaluation tool computes it from peeked
+ * logits (tools/eval_geist.c:63-73): fp32 max, double exp of the fp32 difference, sequential
+ * double sum, (double)(logits[token] - max) - log(sum). */
+double oracle_logprob_at(size_t n, const float *logits, int32_t token);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,6 +82,8 @@ def load_oracle(fast=False):
                                               C.c_int, C.c_uint64]
     lib.oracle_session_draws.argtypes = [C.POINTER(SessionSampler), C.c_size_t]
     lib.oracle_softcap_inplace.argtypes = [C.c_size_t, c_float_p, C.c_float]
+    lib.oracle_logprob_at.argtypes = [C.c_size_t, c_float_p, C.c_int32]
+    lib.oracle_logprob_at.restype = C.c_double
     lib.oracle_finalize_row.restype = C.c_int32
     lib.oracle_finalize_row.argtypes = [C.POINTER(SessionSampler), C.c_size_t, c_float_p, C.c_float]
     lib.oracle_finalize_batch.argtypes = [C.POINTER(SessionSampler), C.c_size_t, C.c_size_t,
@@ -162,6 +164,10 @@ class Oracle:
         hist = np.ascontiguousarray(hist, dtype=np.int32)
         self.lib.oracle_apply_penalties(out.size, _fp(out), _ip(hist), hist.size, rep, freq, pres)
         return out
+
+    def logprob_at(self, row, token):
+        row = np.ascontiguousarray(row, dtype=np.float32)
+        return float(self.lib.oracle_logprob_at(row.size, _fp(row), int(token)))
 
     def softcap(self, row, cap):
         out = row.copy()

@@ -296,7 +296,10 @@ def test_top_p_limits_match_reference_dispatch(hs, oracle):
 
 
 # ------------------------------------------------------------------------------ penalties
-def test_penalties_in_place_match_oracle(hs, oracle):
+@pytest.mark.parametrize("rep,freq,pres", [(1.1, 0.5, 0.3), (1.3, 0.3, 0.7), (0.9, 0.07, 0.011)])
+def test_penalties_in_place_match_oracle(hs, oracle, rep, freq, pres):
+    """Bit-exact: every step of the penalty rounds on its own (freq * count is not exact for
+    most freq, so a fused multiply-subtract would show here)."""
     g = np.random.default_rng(5)
     rows, n, H = 6, 30000, 700
     x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
@@ -305,11 +308,11 @@ def test_penalties_in_place_match_oracle(hs, oracle):
     hist[0, :10] = [-1, n, n + 5, -7, 0, 0, 0, n - 1, n - 1, 2**31 - 1]
     hl = np.array([H, H, 0, 1, 333, H], dtype=np.int32)
     d = to_dev(x, torch)
-    hs.apply_penalties(d, to_dev(hist, torch), to_dev(hl, torch), 1.1, 0.5, 0.3)
+    hs.apply_penalties(d, to_dev(hist, torch), to_dev(hl, torch), rep, freq, pres)
     hs.sync()
     got = d.cpu().numpy()
     for r in range(rows):
-        want = oracle.penalties(x[r], hist[r, :hl[r]], 1.1, 0.5, 0.3)
+        want = oracle.penalties(x[r], hist[r, :hl[r]], rep, freq, pres)
         assert np.array_equal(got[r], want), f"row {r}"
 
 
@@ -373,6 +376,59 @@ def test_normalised_probabilities(hs, oracle, n, T):
         # north-star bound: 1e-5 relative in fp32 (observed: identical up to 1 ulp)
         assert np.allclose(got[r], want, rtol=1e-5, atol=0)
         assert np.max(np.abs(got[r] - want) / np.maximum(want, 1e-38)) < 2e-7
+
+
+# ------------------------------------------------------------------------------ soft-cap
+@pytest.mark.parametrize("mode", ["temperature", "top_k", "top_p", "min_p"])
+def test_softcap_fused_matches_libm_tanhf(hs, oracle, mode):
+    """head.c:148-159: tanhf(x / cap) * cap before sampling. The device evaluates glibc's tanhf
+    (geistlib_amd/csrc/glibc_tanhf.h), so ids are compared as in every other mode and the
+    probabilities of capped rows agree to the last bit wherever the exp-sum does."""
+    from geistlib_amd import HipSampler
+    cap, n = 30.0, 60000
+    x, u = rows_rng(77, 12, n, scale=25.0)            # most logits are bent by the cap
+    x[3, :100] = [np.float32(v) for v in np.linspace(-1e-20, 1e-20, 100)]   # tiny arguments
+    x[4, :4] = [np.inf, -np.inf, 700.0, -700.0]
+    kw = dict(temperature=0.9, top_k=50 if mode == "top_k" else 0,
+              top_p=0.9 if mode == "top_p" else 1.0, min_p=0.02 if mode == "min_p" else 0.0)
+    got = run_rows(hs, torch, x, u, P(softcap=cap, **kw))
+    res = [oracle.chain_u(oracle.softcap(x[r], cap), float(u[r]), **kw) for r in range(x.shape[0])]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"softcap {mode}")
+    assert near <= 1
+    if mode == "temperature":
+        d = to_dev(x[:3], torch)
+        probs = torch.empty_like(d)
+        hs.softmax(HipSampler.rows(d), P(temperature=0.9, softcap=cap), probs)
+        hs.sync()
+        got_p = probs.cpu().numpy()
+        for r in range(3):
+            want, _ = oracle.softmax_normalised(oracle.softcap(x[r], cap), 0.9)
+            assert np.max(np.abs(got_p[r] - want) / np.maximum(want, 1e-38)) < 2e-7
+            assert np.mean(got_p[r].view(np.uint32) == want.view(np.uint32)) > 0.999
+
+
+# ------------------------------------------------------------------------------ scoring
+@pytest.mark.parametrize("n,cap", [(1000, 0.0), (128256, 0.0), (128256, 30.0), (262144, 50.0)])
+def test_logprob_rows_match_oracle(hs, oracle, n, cap):
+    """geist_session_peek_logits + logprob_at (tools/eval_geist.c:63-73) without the copy to the
+    host; tolerance 1e-9 absolute on doubles (order of the sum, last bits of exp and log)."""
+    rows, K = 5, 7
+    x, _ = rows_rng(n + 3, rows, n, scale=6.0)
+    g = np.random.default_rng(n)
+    tok = g.integers(0, n, (rows, K)).astype(np.int32)
+    tok[:, 0] = np.argmax(x, axis=1)
+    tok[0, 1], tok[0, 2] = -1, n                      # outside the vocabulary -> NaN
+    out = torch.full((rows, K), 7.0, dtype=torch.float64, device="cuda")
+    hs.logprob(to_dev(x, torch), to_dev(tok, torch), out, softcap=cap)
+    hs.sync()
+    got = out.cpu().numpy()
+    for r in range(rows):
+        row = oracle.softcap(x[r], cap) if cap > 0 else x[r]
+        for j in range(K):
+            if 0 <= tok[r, j] < n:
+                assert abs(got[r, j] - oracle.logprob_at(row, tok[r, j])) < 1e-9, (r, j)
+            else:
+                assert np.isnan(got[r, j])
 
 
 # ------------------------------------------------------------------- speculative verify

@@ -287,3 +287,29 @@ def test_spec_verify_preserves_target_distribution(oracle, n):
                     _, o2 = oracle.spec_verify(target, q, draft, np.array([ua, ur], np.float32), 1.0)
                     out_mass[o2[0]] += q[0, x] / (G * G)
     assert np.allclose(out_mass, p, atol=3.0 / G), (out_mass, p)
+
+
+# ------------------------------------------------------------------ log-probability scoring
+def test_logprob_at_closed_forms_and_library(oracle):
+    """tools/eval_geist.c:63-73. Pins: uniform logits -> -log(n) for every token; two-point rows;
+    shift invariance; scipy's float64 log_softmax of the same fp32 values."""
+    from scipy.special import log_softmax
+    n = 1000
+    assert oracle.logprob_at(np.full(n, 3.25, np.float32), 17) == pytest.approx(-np.log(n), abs=1e-13)
+    row = np.array([0.0, np.log(3.0)], dtype=np.float32)      # probabilities 1/4 and 3/4
+    d = float(row[1]) - float(row[0])
+    assert oracle.logprob_at(row, 1) == pytest.approx(-np.log1p(np.exp(-d)), abs=1e-14)
+    assert oracle.logprob_at(row, 0) == pytest.approx(-d - np.log1p(np.exp(-d)), abs=1e-14)
+    g = np.random.default_rng(3)
+    x = (g.standard_normal(5000) * 4).astype(np.float32)
+    want = log_softmax(x.astype(np.float64))
+    # the reference subtracts the maximum in fp32 before widening, so against an all-float64
+    # library the differences carry fp32 rounding (~1e-7 each); with the same fp32 differences
+    # fed to numpy's own exp / sum / log the agreement is to the last few bits
+    d32 = (x - x.max()).astype(np.float32).astype(np.float64)
+    same = d32 - np.log(np.sum(np.exp(d32)))
+    for t in (0, 1, 4999, int(np.argmax(x)), int(np.argmin(x))):
+        assert oracle.logprob_at(x, t) == pytest.approx(want[t], abs=2e-6)
+        assert oracle.logprob_at(x, t) == pytest.approx(same[t], abs=1e-12)
+    probs = np.exp([oracle.logprob_at(x[:50], t) for t in range(50)])
+    assert probs.sum() == pytest.approx(1.0, abs=1e-12)
