@@ -68,7 +68,8 @@ def load_library():
     lib.geist_hip_argmax_f32.argtypes = [vp, vp, sz, C.POINTER(C.c_int32)]
     lib.geist_hip_apply_penalties.argtypes = [vp, vp, sz, sz, sz, vp, sz, vp, f32, f32, f32]
     lib.geist_hip_softmax_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, sz]
-    lib.geist_hip_spec_verify.argtypes = [vp, vp, sz, vp, sz, vp, vp, sz, sz, sz, f32, vp, vp]
+    lib.geist_hip_spec_verify.argtypes = [vp, vp, sz, vp, sz, vp, vp, sz, sz, sz, f32, f32, vp, vp]
+    lib.geist_hip_rng_draw_units.argtypes = [vp, vp, sz, vp]
     lib.geist_hip_malloc.argtypes = [vp, sz, C.POINTER(vp)]
     lib.geist_hip_free.argtypes = [vp, vp]
     lib.geist_hip_upload.argtypes = [vp, vp, vp, sz]
@@ -159,14 +160,16 @@ class HipSampler:
         self._check(self.lib.geist_hip_softmax_rows(self.h, C.byref(rows), C.byref(params),
                                                     _ptr(probs), ld))
 
-    def spec_verify(self, target, q, draft, uniforms, temperature, out_tokens, n_accepted):
+    def spec_verify(self, target, q, draft, uniforms, temperature, out_tokens, n_accepted,
+                    softcap=0.0):
+        """q = None: point-mass drafts (the drafter proposed each token with certainty)."""
         n_seq, lp1, n = target.shape
         L = lp1 - 1
-        assert q.shape == (n_seq, L, n) and draft.shape == (n_seq, L)
-        assert target.is_contiguous() and q.is_contiguous()
+        assert draft.shape == (n_seq, L) and target.is_contiguous()
+        assert q is None or (q.shape == (n_seq, L, n) and q.is_contiguous())
         self._check(self.lib.geist_hip_spec_verify(self.h, _ptr(target), n, _ptr(q), n, _ptr(draft),
                                                    _ptr(uniforms), n_seq, L, n, temperature,
-                                                   _ptr(out_tokens), _ptr(n_accepted)))
+                                                   softcap, _ptr(out_tokens), _ptr(n_accepted)))
 
     def time_stream_kernel(self, rows, params, uniforms, out, launches):
         """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around

@@ -535,8 +535,8 @@ int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t l
 int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
                           const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
                           const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,
-                          float temperature, geist_hip_token_t *d_out_tokens,
-                          int32_t *d_n_accepted) {
+                          float temperature, float logit_softcap,
+                          geist_hip_token_t *d_out_tokens, int32_t *d_n_accepted) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     if (!d_target || !d_draft || !d_out_tokens || !d_n_accepted)
@@ -545,9 +545,9 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
         return fail(s, GEIST_HIP_E_INVALID_ARG, "n_seq %zu, draft length %zu (1..%d)", n_seq, L,
                     SPEC_DRAFT_MAX);
     const bool greedy = !(temperature > 0.0f);
-    if (!greedy && (!d_draft_q || !d_uniforms))
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic verification needs q and uniforms");
-    if (!greedy && ld_q < n_vocab)
+    if (!greedy && !d_uniforms)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic verification needs uniforms");
+    if (!greedy && d_draft_q && ld_q < n_vocab)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_q < n_vocab");
     struct geist_hip_rows r{};
     r.d_logits = d_target;
@@ -557,8 +557,9 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     struct geist_hip_sample_params p{};
     p.temperature        = temperature;
     p.repetition_penalty = 1.0f;
+    p.logit_softcap      = logit_softcap;
     Launch La;
-    int    rc = make_launch(s, &r, &p, false, La);
+    int    rc = make_launch(s, &r, &p, !greedy, La); /* greedy rows skip the monotone cap */
     if (rc)
         return rc;
     HIPCHK(s, hipSetDevice(s->device));
@@ -648,6 +649,17 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
     (void) hipEventDestroy(b);
     *ms_total = ms;
     return rc;
+}
+
+int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,
+                             float *d_out_units) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_rng_state || !d_out_units || n == 0 || n > 0x7fffffffu)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null state or output, or n out of range");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_rng_units(s->stream, d_rng_state, /*shared=*/1, (int) n, d_out_units);
+    return after_launch(s, "rng draws");
 }
 
 int geist_hip_sampler_row_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows) {

@@ -907,7 +907,7 @@ __global__ __launch_bounds__(TPB) void k_final_temperature(RowView rv, FinalArgs
     /* (row_best_from_chunks ends with a barrier: s_csum and the table are visible) */
     const int tok = index_order_walk<NV, PEN, false>(
         rv, row, (int) gridDim.x, s_csum, a.slab_sum + (long) row * C * SLABS_MAX, C, u_row, mx,
-        a.inv_t, 0.0, nullptr, false, s_tab, s_cnt16, s_walk);
+        a.inv_t, 0.0, nullptr, false, -1, s_tab, s_cnt16, s_walk);
     if (tid == 0)
         a.out[row] = tok;
 }

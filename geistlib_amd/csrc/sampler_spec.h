@@ -25,7 +25,7 @@ struct SpecArgs {
     int             L;       /* draft length */
     int             greedy;  /* T <= 0: exact match against the row argmax */
     float           inv_t;
-    const float    *q;       /* [n_seq][L][n_vocab], row stride ld_q */
+    const float    *q;       /* [n_seq][L][n_vocab], row stride ld_q; NULL = point-mass drafts */
     long            ld_q;
     const int32_t  *draft;   /* [n_seq][L] */
     const float    *uniforms; /* [n_seq][L+1] */
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, Spe
             float pn = 0.0f, qt = 0.0f;
             if (x >= 0 && x < rv.n_vocab) {
                 pn = (float) ((double) a.probe_p[row] / s_sum[tid]);
-                qt = a.q[((long) seq * L + tid) * a.ld_q + x];
+                qt = a.q ? a.q[((long) seq * L + tid) * a.ld_q + x] : 1.0f; /* NULL: point mass */
             }
             ok = (double) a.uniforms[(long) seq * (L + 1) + tid] * (double) qt < (double) pn;
         }
@@ -152,10 +152,12 @@ __global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a,
     int          base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4       v[NV], qv[NV];
-    const float *qrow = a.q + ((long) seq * a.L + js) * a.ld_q;
+    const float *qrow = a.q ? a.q + ((long) seq * a.L + js) * a.ld_q : nullptr;
     const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
+    const int    qx   = a.draft[(long) seq * a.L + js];
     load_raw<NV>(rv, rv.logits + row * rv.ld, base, end, v);
-    load_q_chunk<NV>(qrow, qvec, base, end, qv);
+    load_q_chunk<NV>(qrow, qvec, qx, base, end, qv);
+    apply_transform<NV>(rv, nullptr, v); /* the soft-cap, as in the passes before */
     double acc[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -213,20 +215,21 @@ __global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a,
             __syncthreads();
         }
         if (resid) {
-            const float *qrow = a.q + ((long) seq * L + js) * a.ld_q;
+            const float *qrow = a.q ? a.q + ((long) seq * L + js) * a.ld_q : nullptr;
             const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
+            const int    qx   = a.draft[(long) seq * L + js];
             tok = index_order_walk<NV, false, true>(rv, (int) row, 0, s_w,
                                                     a.resid_slab + (long) seq * C * SLABS_MAX, C, u,
-                                                    mx, a.inv_t, sum, qrow, qvec, s_tab, nullptr,
-                                                    s_walk);
+                                                    mx, a.inv_t, sum, qrow, qvec, qx, s_tab,
+                                                    nullptr, s_walk);
         } else {
             if (tid < C)
                 s_w[tid] = a.chunk_sum[row * C + tid];
             __syncthreads();
             tok = index_order_walk<NV, false, false>(rv, (int) row, 0, s_w,
                                                      a.slab_sum + row * C * SLABS_MAX, C, u, mx,
-                                                     a.inv_t, sum, nullptr, false, s_tab, nullptr,
-                                                     s_walk);
+                                                     a.inv_t, sum, nullptr, false, -1, s_tab,
+                                                     nullptr, s_walk);
         }
     }
     if (tid == 0)

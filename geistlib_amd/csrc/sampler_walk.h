@@ -38,14 +38,21 @@ __device__ __forceinline__ void slab_weights(const float4 &v, const float4 &qv, 
     }
 }
 
+/* Draft probabilities of a chunk. qrow == NULL: the drafter proposed its token with certainty
+ * (an n-gram lookup, src/engine/session.c:437-513), q is 1 at `x` and 0 elsewhere. */
 template <int NV>
-__device__ __forceinline__ void load_q_chunk(const float *qrow, bool vec, int base, int end,
+__device__ __forceinline__ void load_q_chunk(const float *qrow, bool vec, int x, int base, int end,
                                              float4 (&qv)[NV]) {
     const int tid = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         const int e = base + 4 * (j * TPB + tid);
-        if (vec && e + 3 < end) {
+        if (qrow == nullptr) {
+            qv[j].x = e + 0 == x ? 1.f : 0.f;
+            qv[j].y = e + 1 == x ? 1.f : 0.f;
+            qv[j].z = e + 2 == x ? 1.f : 0.f;
+            qv[j].w = e + 3 == x ? 1.f : 0.f;
+        } else if (vec && e + 3 < end) {
             qv[j] = *reinterpret_cast<const float4 *>(qrow + e);
         } else {
             qv[j].x = e + 0 < end ? qrow[e + 0] : 0.f;
@@ -64,7 +71,8 @@ struct WalkShared {
 
 /* Walks row `row` in index order for the first element at which the running weight exceeds
  * u * (sum of chunk_w). chunk_w: C per-chunk weights in LDS; slab_w: the row's C * SLABS_MAX slab
- * weights in global memory; NV: slabs per chunk of the pass that wrote them. Returns the id to
+ * weights in global memory; NV: slabs per chunk of the pass that wrote them; qrow / qx: the
+ * draft probabilities of the residual walk (see load_q_chunk). Returns the id to
  * every thread. Should rounding leave the target beyond the located slab, the following slabs of
  * the chunk are walked too; beyond those the chunk's last index (the reference returns the last
  * index of the row, sampler.c:100-101; the located chunk is then the last one), for the residual
@@ -72,7 +80,7 @@ struct WalkShared {
 template <int NV, bool PEN, bool RESID>
 __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const double *chunk_w,
                                 const double *__restrict__ slab_w, int C, float u, float mx,
-                                float inv_t, double sum, const float *qrow, bool qvec,
+                                float inv_t, double sum, const float *qrow, bool qvec, int qx,
                                 const uint64_t *tab, uint32_t *s_cnt16, WalkShared &sh) {
     const int tid = threadIdx.x;
     if (tid == 0) {
@@ -121,7 +129,7 @@ __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const do
         fetch_chunk<1, PEN>(rv, row, n_rows, sbase, send, s_cnt16, v); /* a slab is a chunk of 1024 */
         qv[0] = v[0];
         if (RESID)
-            load_q_chunk<1>(qrow, qvec, sbase, send, qv);
+            load_q_chunk<1>(qrow, qvec, qx, sbase, send, qv);
         const int e = sbase + 4 * tid;
         float     w[4];
         slab_weights<RESID>(v[0], qv[0], e, send, mx, inv_t, sum, tab, w);

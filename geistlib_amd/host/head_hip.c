@@ -21,6 +21,9 @@ struct geist_hip_head {
     geist_hip_sampler *hs;
     uint64_t *d_rng;   /* the session's struct geist_rng, in device memory */
     int32_t  *d_tokens; /* m_max */
+    float    *d_units;  /* m_max uniforms of one speculative round */
+    int32_t  *d_drafts; /* m_max */
+    int32_t  *d_nacc;
     char      err[256];
 };
 
@@ -59,6 +62,14 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
     if (rc == GEIST_HIP_OK &&
         (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_tokens = p;
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(float), &p)) == GEIST_HIP_OK)
+        h->d_units = p;
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        h->d_drafts = p;
+    if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(h->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        h->d_nacc = p;
     /* arch_state.c:1173: the default seed */
     if (rc == GEIST_HIP_OK)
         rc = seed_rng(h, UINT64_C(0xCAFEBABE1234));
@@ -76,6 +87,9 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
     if (h->hs != nullptr) {
         geist_hip_free(h->hs, h->d_rng);
         geist_hip_free(h->hs, h->d_tokens);
+        geist_hip_free(h->hs, h->d_units);
+        geist_hip_free(h->hs, h->d_drafts);
+        geist_hip_free(h->hs, h->d_nacc);
         geist_hip_sampler_destroy(h->hs);
     }
     free(h);
@@ -142,6 +156,67 @@ int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, s
         return head_fail(h, GEIST_HIP_E_UNSUPPORTED, "row longer than the probed vocabulary");
     if (geist_hip_argmax_f32(h->hs, d_logits, n, out_index) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "argmax");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_spec_accept(struct geist_hip_head *h, const float *d_logits, size_t k,
+                               const int32_t *drafts, int mode, size_t out_capacity,
+                               int32_t *out_tokens, size_t *n_out) {
+    if (h == nullptr || d_logits == nullptr || drafts == nullptr || out_tokens == nullptr ||
+        n_out == nullptr || k == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    *n_out = 0;
+    if (k > h->m_max)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
+    if (out_capacity < k + 1)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "out_capacity below k + 1");
+    const bool greedy   = !(h->temperature > 0.0f);
+    const bool filtered = h->top_k > 1 || (h->top_p > 0.0f && h->top_p < 1.0f);
+    if (mode == GEIST_HIP_SPEC_REJECTION && !greedy && filtered)
+        return head_fail(h, GEIST_HIP_E_UNSUPPORTED,
+                         "rejection sampling against a top-k / top-p filtered target");
+    if (mode != GEIST_HIP_SPEC_REJECTION || greedy || k == 1) {
+        /* session.c:599-625: sample every row, accept the longest matching prefix */
+        int32_t   sampled[64];
+        int32_t  *v  = k <= 64 ? sampled : malloc(k * sizeof *v);
+        if (v == nullptr)
+            return GEIST_HIP_E_OOM;
+        const int rc = finalize(h, d_logits, k, v);
+        if (rc == GEIST_HIP_OK) {
+            size_t accepted = 0;
+            for (size_t i = 0; i + 1 < k; i++) {
+                if (v[i] != drafts[i + 1])
+                    break;
+                accepted++;
+            }
+            memcpy(out_tokens, drafts, (accepted + 1) * sizeof *out_tokens);
+            out_tokens[accepted + 1] = v[accepted];
+            *n_out                   = accepted + 2;
+        }
+        if (v != sampled)
+            free(v);
+        return rc;
+    }
+    /* rejection sampling: L = k - 1 drafts (drafts[1..k)) against rows 0..L-1, bonus from row L */
+    const size_t L = k - 1;
+    if (geist_hip_upload(h->hs, h->d_drafts, drafts + 1, L * sizeof(int32_t)) != GEIST_HIP_OK ||
+        geist_hip_rng_draw_units(h->hs, h->d_rng, k, h->d_units) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "staging the drafts");
+    if (geist_hip_spec_verify(h->hs, d_logits, h->vocab, nullptr, 0, h->d_drafts, h->d_units, 1, L,
+                              h->vocab, h->temperature, h->logit_softcap, h->d_tokens,
+                              h->d_nacc) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "verification");
+    int32_t n_acc = 0;
+    if (geist_hip_download(h->hs, &n_acc, h->d_nacc, sizeof n_acc) != GEIST_HIP_OK ||
+        n_acc < 0 || (size_t) n_acc > L ||
+        geist_hip_download(h->hs, out_tokens + 1, h->d_tokens,
+                           ((size_t) n_acc + 1) * sizeof(int32_t)) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the verdict");
+    out_tokens[0] = drafts[0];
+    *n_out        = (size_t) n_acc + 2;
+    for (size_t i = 0; i < *n_out; i++)
+        if (out_tokens[i] < 0 || (size_t) out_tokens[i] >= h->vocab)
+            return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
     return GEIST_HIP_OK;
 }
 

@@ -10,6 +10,9 @@
  *   geist_hip_head_finalize_batch     sampler part of finalize_logits_batch (head.c:274-304)
  *   geist_hip_head_argmax_f32      the backend slot fused->argmax_f32
  *                                  (include/geist_backend.h:414-421)
+ *   geist_hip_head_spec_accept     the accept loop of geist_session_decode_speculative
+ *                                  (src/engine/session.c:599-625) over the rows verify_forward
+ *                                  produced (src/archs/transformer/arch_ops.c:176-270)
  *
  * The RNG state of the session lives in device memory and advances there, one draw per
  * stochastic row in row order, exactly as the reference's single host RNG does.
@@ -59,6 +62,30 @@ int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logit
                                   int32_t *out_tokens);
 int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,
                               int32_t *out_index);
+
+/* The accept step of one speculative round. drafts[0..k) are the tokens fed to verify_forward
+ * (drafts[0] is the already-sampled next token, session.c:563-568), d_logits the [k, vocab] rows
+ * it produced: row i holds the logits for the position after drafts[i].
+ *   GEIST_HIP_SPEC_REFERENCE  the reference's loop: every row is sampled with the session's
+ *       sampler (one shared RNG, row order, as finalize_logits_batch), the longest prefix with
+ *       sampled[i] == drafts[i + 1] is accepted and sampled[accepted] is the correction
+ *       (session.c:599-625). Under T > 0 the stream is valid but not distribution-preserving
+ *       (include/geist_util.h:233-240).
+ *   GEIST_HIP_SPEC_REJECTION  T > 0 with no top-k / top-p filter: rejection sampling against the
+ *       n-gram drafter's point-mass proposals -- draft i+1 is accepted with probability
+ *       p_i(drafts[i+1]); at the first rejection the correction is drawn from p_i with that
+ *       token struck out; if all are accepted the bonus is a temperature draw from row k-1. The
+ *       emitted stream then has the distribution of k decode_step calls. Consumes k draws of
+ *       the session's RNG, like the reference mode. T == 0 behaves as the reference mode;
+ *       a filter set with T > 0 returns GEIST_E_UNSUPPORTED (7).
+ * Writes drafts[0..accepted], then the correction: n_out = accepted + 2 tokens in all,
+ * out_capacity >= k + 1 (include/geist_util.h:226). The caller truncates its KV cache to the
+ * accepted prefix and prefills the correction as the reference does (session.c:611-632). */
+#define GEIST_HIP_SPEC_REFERENCE 0
+#define GEIST_HIP_SPEC_REJECTION 1
+int geist_hip_head_spec_accept(struct geist_hip_head *h, const float *d_logits, size_t k,
+                               const int32_t *drafts, int mode, size_t out_capacity,
+                               int32_t *out_tokens, size_t *n_out);
 
 /* Current RNG state (for tests and for handing a session over). */
 int geist_hip_head_rng_state(struct geist_hip_head *h, uint64_t *state);

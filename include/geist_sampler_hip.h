@@ -149,18 +149,28 @@ int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t l
  * omits rejection sampling; the batch shape is that of verify_forward,
  * src/archs/transformer/arch_ops.c:176-270).
  *   d_target   [n_seq][L+1][n_vocab] logits, sequence stride (L+1)*ld_t, row stride ld_t
- *   d_draft_q  [n_seq][L][n_vocab] draft probabilities, row stride ld_q
+ *   d_draft_q  [n_seq][L][n_vocab] draft probabilities, row stride ld_q; NULL when the drafter
+ *              proposes with certainty (the reference's n-gram lookup, session.c:437-513):
+ *              q_j is then 1 at the draft token, a draft is accepted with probability p_j(x_j)
+ *              and the resample is p_j with x_j struck out
  *   d_draft    [n_seq][L] draft token ids,  d_uniforms [n_seq][L+1]
  * T > 0: position j accepted iff u_j * q_j(x_j) < p_j(x_j); at the first rejection the token is
  * drawn with u_L from max(0, p_j - q_j) renormalised; if all are accepted the bonus token is a
  * temperature draw from row L with u_L. T <= 0: exact-match against the row argmax.
+ * logit_softcap > 0: the target rows are capped (tanhf(x / cap) * cap, head.c:148-159) before
+ * anything else when T > 0, as the reference caps them before it samples.
  *   d_out_tokens [n_seq][L+1]: accepted draft ids, then the emitted token; rest untouched.
  *   d_n_accepted [n_seq]. */
 int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
                           const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
                           const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,
-                          float temperature, geist_hip_token_t *d_out_tokens,
-                          int32_t *d_n_accepted);
+                          float temperature, float logit_softcap,
+                          geist_hip_token_t *d_out_tokens, int32_t *d_n_accepted);
+
+/* n consecutive geist_rng_next_unit values (sampler.c:44-48) from the state at d_rng_state (a
+ * struct geist_rng in device memory), written to d_out_units; the state advances by n draws. */
+int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,
+                             float *d_out_units);
 
 /* ---- small device-memory helpers so that a plain-C host needs no HIP headers -------------- */
 int geist_hip_malloc(geist_hip_sampler *s, size_t bytes, void **d_ptr);

@@ -55,6 +55,9 @@ def host():
     lib.geist_hip_head_argmax_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
                                               C.POINTER(C.c_int32)]
     lib.geist_hip_head_rng_state.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
+    lib.geist_hip_head_spec_accept.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
+                                               C.POINTER(C.c_int32), C.c_int, C.c_size_t,
+                                               C.POINTER(C.c_int32), C.POINTER(C.c_size_t)]
     return lib
 
 
@@ -256,4 +259,81 @@ def test_head_softcap_only_when_sampling(host, oracle):
         want, info = oracle.top_k_u(oracle.softcap(x[i], cap), 50, 0.9, u)
         agree += (out[i] == want) or info.boundary_dist < 1e-4
     assert agree == 6
+    host.geist_hip_head_destroy(h)
+
+
+# ------------------------------------------------------------------ speculative accept step
+def _accept(host, h, d, drafts, mode):
+    k = len(drafts)
+    dr = (C.c_int32 * k)(*drafts)
+    out = (C.c_int32 * (k + 1))(*([-1] * (k + 1)))
+    n_out = C.c_size_t(0)
+    rc = host.geist_hip_head_spec_accept(h, C.c_void_p(d.data_ptr()), k, dr, mode, k + 1, out,
+                                         C.byref(n_out))
+    return rc, list(out)[:n_out.value]
+
+
+@pytest.mark.parametrize("T,p,k_top", [(0.0, 1.0, 0), (0.8, 1.0, 0), (0.8, 0.9, 40), (0.7, 0.92, 0)])
+def test_spec_accept_reference_loop(host, oracle, T, p, k_top):
+    """src/engine/session.c:599-625 restated: sample every verify row with the session's
+    sampler (shared RNG, row order), accept the longest prefix with sampled[i] == drafts[i+1],
+    emit drafts[0..accepted] and the correction sampled[accepted]."""
+    g = np.random.default_rng(41)
+    vocab, k = 20000, 6
+    x = (g.standard_normal((k, vocab)) * 3).astype(np.float32)
+    x[np.arange(k), [11, 22, 33, 44, 55, 66]] += 30.0        # rows 0..5 all but surely pick these
+    d = torch.from_numpy(x).cuda()
+    for drafts in ([7, 11, 22, 33, 44, 55], [7, 11, 22, 99, 44, 55], [7, 5, 22, 33, 44, 55]):
+        h = make_head(host, vocab)
+        opts = SessionOpts(0, T, p, k_top, 1234, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        sess = oracle.session(T, p, k_top, seed=1234)
+        sampled = oracle.finalize_batch(sess, x).tolist()
+        acc = 0
+        for i in range(k - 1):
+            if sampled[i] != drafts[i + 1]:
+                break
+            acc += 1
+        want = drafts[:acc + 1] + [sampled[acc]]
+        rc, got = _accept(host, h, d, drafts, 0)
+        assert rc == 0 and got == want, (T, drafts, got, want)
+        st = C.c_uint64(0)
+        host.geist_hip_head_rng_state(h, C.byref(st))
+        assert st.value == int(sess.rng.state)
+        host.geist_hip_head_destroy(h)
+
+
+def test_spec_accept_rejection_sampling_point_mass(host, oracle):
+    """Rejection sampling against the n-gram drafter's certain proposals: the oracle's verify with
+    one-hot draft probabilities, fed the same k uniforms the session's RNG yields."""
+    g = np.random.default_rng(43)
+    vocab, k = 5000, 5
+    L = k - 1
+    for trial in range(12):
+        x = (g.standard_normal((k, vocab)) * 2).astype(np.float32)
+        drafts = [3] + [int(t) for t in g.integers(0, vocab, L)]
+        for j in range(L):                                  # make acceptance likely but not sure
+            x[j, drafts[j + 1]] += np.float32(g.choice([4.0, 8.0, 12.0]))
+        d = torch.from_numpy(x).cuda()
+        h = make_head(host, vocab)
+        opts = SessionOpts(0, 0.9, 1.0, 0, 77 + trial, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        r = oracle.rng(77 + trial)
+        u = np.array([oracle.next_unit(r) for _ in range(k)], dtype=np.float32)
+        q = np.zeros((L, vocab), dtype=np.float32)
+        q[np.arange(L), drafts[1:]] = 1.0
+        n_acc, toks = oracle.spec_verify(x, q, np.array(drafts[1:], np.int32), u, 0.9)
+        want = [drafts[0]] + toks[:n_acc + 1].tolist()
+        rc, got = _accept(host, h, d, drafts, 1)
+        assert rc == 0 and got == want, (trial, got, want)
+        st = C.c_uint64(0)
+        host.geist_hip_head_rng_state(h, C.byref(st))
+        assert st.value == int(r.state), "k draws per round"
+        host.geist_hip_head_destroy(h)
+    # a filtered target is refused in this mode, the greedy session falls back to exact match
+    h = make_head(host, vocab)
+    opts = SessionOpts(0, 0.9, 0.9, 0, 1, None, 0, 0)
+    host.geist_hip_head_apply_opts(h, C.byref(opts))
+    rc, _ = _accept(host, h, d, drafts, 1)
+    assert rc == 7
     host.geist_hip_head_destroy(h)

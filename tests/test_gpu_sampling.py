@@ -472,6 +472,34 @@ def test_spec_verify_matches_oracle(hs, oracle, n_seq, L, n, T):
     print("  accepted lengths seen:", sorted(seen))
 
 
+def test_spec_verify_point_mass_drafts_and_softcap(hs, oracle):
+    """d_draft_q = NULL is q = one-hot at the draft token; the soft-cap is applied to the target
+    rows before anything else."""
+    n_seq, L, n, cap = 6, 5, 30000, 20.0
+    g = np.random.default_rng(8)
+    target = (g.standard_normal((n_seq, L + 1, n)) * 3).astype(np.float32)
+    draft = g.integers(0, n, (n_seq, L)).astype(np.int32)
+    for s in range(n_seq):
+        for j in range(L):
+            target[s, j, draft[s, j]] += np.float32(25.0 if (s + j) % 3 else 0.0)
+    u = (g.integers(0, 1 << 24, (n_seq, L + 1)) / np.float32(1 << 24)).astype(np.float32)
+    out = torch.full((n_seq, L + 1), -9, dtype=torch.int32, device="cuda")
+    nacc = torch.full((n_seq,), -9, dtype=torch.int32, device="cuda")
+    hs.spec_verify(to_dev(target, torch), None, to_dev(draft, torch), to_dev(u, torch), 0.8, out,
+                   nacc, softcap=cap)
+    hs.sync()
+    out, nacc = out.cpu().numpy(), nacc.cpu().numpy()
+    seen = set()
+    for s in range(n_seq):
+        capped = np.stack([oracle.softcap(target[s, j], cap) for j in range(L + 1)])
+        q = np.zeros((L, n), dtype=np.float32)
+        q[np.arange(L), draft[s]] = 1.0
+        want_n, want = oracle.spec_verify(capped, q, draft[s], u[s], 0.8)
+        assert nacc[s] == want_n and out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), s
+        seen.add(want_n)
+    assert len(seen) >= 2
+
+
 def test_spec_verify_special_cases(hs, oracle):
     n_seq, L, n = 4, 5, 7000
     target, q, draft, u = _spec_case(77, n_seq, L, n)
