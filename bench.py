@@ -52,6 +52,8 @@ def build_workload(name):
         return W.config4()
     if name == "cfg1":
         return W.config1()
+    if name == "cfg5":
+        return W.config5()
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -88,6 +90,56 @@ def cpu_baseline(w, budget_s=20.0):
                       "-O3 -ffast-math -march=x86-64-v3 -fopenmp"}, ids
 
 
+def bench_spec(w, args):
+    """Configuration 5: speculative verification of n_seq sequences x (L + 1) target rows. A step
+    is one geist_hip_spec_verify call; rows/s counts target rows."""
+    import torch
+    from geistlib_amd import HipSampler
+    x = w.extra
+    n_seq, L = x["n_seq"], x["draft_len"]
+    dev = torch.device("cuda:0")
+    t = torch.from_numpy(x["target"]).to(dev)
+    q = torch.from_numpy(x["q"]).to(dev)
+    d = torch.from_numpy(x["draft"]).to(dev)
+    u = torch.from_numpy(x["uniforms"]).to(dev)
+    out = torch.full((n_seq, L + 1), -1, dtype=torch.int32, device=dev)
+    nacc = torch.full((n_seq,), -1, dtype=torch.int32, device=dev)
+    hs = HipSampler(max_rows=n_seq * (L + 1), max_vocab=w.n_vocab)
+
+    def step():
+        hs.spec_verify(t, q, d, u, w.temperature, out, nacc)
+
+    for _ in range(args.warmup):
+        step()
+    hs.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    hs.sync()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed * 1e3 / args.steps
+    rows = n_seq * (L + 1)
+    # every target logit once, one row of draft probabilities per sequence (the rejected
+    # position's), uniforms in, ids and counts out
+    alg = rows * w.n_vocab * 4 + n_seq * w.n_vocab * 4 + rows * 4 + rows * 4 + n_seq * 4
+    achieved = alg / (ms * 1e-3) / 1e9
+    result = {
+        "metric": "sampled rows/s", "value": round(rows * args.steps / elapsed, 1),
+        "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w.name, "sequences": n_seq, "draft_len": L, "n_vocab": w.n_vocab,
+                   "temperature": w.temperature},
+        "us_per_step": round(ms * 1e3, 3),
+        "sequences_per_s": round(n_seq * args.steps / elapsed, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "whole step (five kernels)", "step_algorithmic_bytes": alg},
+        "accepted_lengths": sorted(nacc.cpu().numpy().tolist()),
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +161,8 @@ def main():
         raise SystemExit("no GPU visible: the sampling path has no CPU fallback")
 
     w = build_workload(args.workload)
+    if args.workload == "cfg5":
+        return bench_spec(w, args)
     dev = torch.device("cuda:0")
     d_logits = torch.from_numpy(w.logits).to(dev)
     d_u = torch.from_numpy(w.uniforms).to(dev)

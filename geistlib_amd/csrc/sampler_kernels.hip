@@ -120,25 +120,34 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     double    acc  = 0.0;
     double    accs[SLABS ? NV : 1];
     uint32_t  mask = 0u;
+    /* positions at or beyond `end` hold -inf (load_raw): they weigh exactly 0 and land in no
+     * bin, so the loop carries no bound tests */
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        const int e = base + 4 * (j * TPB + tid);
-        if (SLABS)
-            accs[j] = 0.0;
+        double a4 = 0.0;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            if (e + c < end) {
-                const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
-                const float p   = geist_expf_glibc(arg, s_tab);
-                if (SLABS)
-                    accs[j] += (double) p;
-                else
-                    acc += (double) p;
-                if (e + c == tok)
-                    probe_p[row] = p;
-                if (LISTM)
-                    mask |= (uint32_t) (zbin(arg) <= zb_list) << (4 * j + c);
-            }
+            const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
+            a4 += (double) geist_expf_glibc_nonpos(arg, s_tab);
+            if (LISTM)
+                mask |= (uint32_t) (zbin(arg) <= zb_list) << (4 * j + c);
+        }
+        if (SLABS)
+            accs[j] = a4;
+        else
+            acc += a4;
+    }
+    if (tok >= base && tok < end) {
+        /* the thread that holds the probed element evaluates it once more */
+        const int off = tok - base, f = off >> 2;
+        if ((f & (TPB - 1)) == tid) {
+            const int j = f / TPB;
+            float     x = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < NV; ++jj)
+                if (jj == j)
+                    x = f4_get(v[jj], off & 3);
+            probe_p[row] = geist_expf_glibc_nonpos(softmax_arg(x, mx, inv_t), s_tab);
         }
     }
     if (SLABS) {
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
                 if ((mask >> (4 * j + c)) & 1u) {
                     if (pos < CAND_CAP) {
                         ck[pos] = __float_as_uint(
-                            geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab));
+                            geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab));
                         ci[pos] = (uint32_t) (e + c);
                     }
                     ++pos;
@@ -284,7 +293,7 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
     }
     __syncthreads();
     const float l0 = key2f(best_key(spack[0]));
-#define GS_P(i) geist_expf_glibc(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), fs.tab)
+#define GS_P(i) geist_expf_glibc_nonpos(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), fs.tab)
 
     double part = 0.0;
     for (int i = lo; i < hi; ++i)
@@ -373,7 +382,7 @@ __device__ int finish_sorted_wave(int n, const uint64_t *spack, float inv_t, flo
 #pragma unroll
     for (int t = 0; t < IPT; ++t) {
         const int i = IPT * lane + t;
-        w[t] = i < n ? geist_expf_glibc(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), tab)
+        w[t] = i < n ? geist_expf_glibc_nonpos(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), tab)
                      : 0.0f;
         part += (double) w[t];
     }
@@ -951,7 +960,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */
         if (tid == 0) {
             const int   B      = a.zb_min_p;
-            const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float p_out  = geist_expf_glibc_nonpos(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
             const float pn_out = (float) ((double) p_out / sum);
             a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
             a.cand.row_bound[row] = B;
@@ -1054,7 +1063,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
             /* an element outside the list has z >= (B + 1) / ZBIN_PER_NAT (the product in zbin()
              * is exact), so its p is at most expf of minus that; one step up covers any
              * non-monotonic last bit of expf or of the division */
-            const float p_out  = geist_expf_glibc(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float p_out  = geist_expf_glibc_nonpos(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
             const float pn_out = (float) ((double) p_out / sum);
             a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
             a.cand.row_bound[row] = B;
@@ -1165,7 +1174,7 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
-                const float p = geist_expf_glibc(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                const float p = geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
                 out[e + c]    = (float) ((double) p / tot);
             }
         }

@@ -19,13 +19,16 @@ int main(int argc, char **argv) {
         const uint32_t u = (uint32_t) b;
         float          x;
         memcpy(&x, &u, 4);
-        const float want = expf(x), got = geist_expf_glibc(x, TAB);
-        uint32_t    uw, ug;
+        const float want = expf(x), got = geist_expf_glibc(x, TAB),
+                    got2 = geist_expf_glibc_nonpos(x, TAB); /* the branch-free variant */
+        uint32_t    uw, ug, ug2;
         memcpy(&uw, &want, 4);
         memcpy(&ug, &got, 4);
-        const bool both_nan = want != want && got != got;
+        memcpy(&ug2, &got2, 4);
+        const bool both_nan  = want != want && got != got;
+        const bool both_nan2 = want != want && got2 != got2;
         ++total;
-        if (uw != ug && !both_nan)
+        if ((uw != ug && !both_nan) || (uw != ug2 && !both_nan2))
             ++bad;
     }
     printf("%ld %ld\n", bad, total);
