@@ -165,6 +165,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     s->max_chunks = (int) mc;
     const size_t rc = max_rows * mc;
     hipError_t   e  = hipSetDevice(device);
+    if (e == hipSuccess) e = (hipError_t) configure_device_kernels();
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));

@@ -117,6 +117,8 @@ void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best,
 void launch_row_final(const Launch &L, const FinalLaunch &f);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
+/* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */
+int configure_device_kernels();
 /* rows flagged 1 by the sorted row-final kernel: list their candidates, then draw from the
  * list; rows the list cannot serve are flagged 2 for the two kernels below */
 void launch_candidates(const Launch &L, const FinalLaunch &f);

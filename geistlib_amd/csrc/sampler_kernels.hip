@@ -1479,19 +1479,20 @@ void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best
     });
 }
 
+int configure_device_kernels() {
+    /* k_sorted_candidates keeps a whole candidate list in LDS: more than the static limit */
+    return (int) hipFuncSetAttribute((const void *) k_sorted_candidates,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     CAND_CAP * (int) sizeof(uint32_t));
+}
+
 void launch_candidates(const Launch &L, const FinalLaunch &f) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
             L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
     });
-    static bool lds_set = false; /* once per process: the kernel's LDS beyond the static part */
-    const int   dyn     = CAND_CAP * (int) sizeof(uint32_t);
-    if (!lds_set) {
-        (void) hipFuncSetAttribute((const void *) k_sorted_candidates,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
-        lds_set = true;
-    }
+    const int dyn = CAND_CAP * (int) sizeof(uint32_t); /* see configure_device_kernels() */
     k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(f.cand, f.top_p, f.min_p, f.uniforms,
                                                                f.row_flag, f.out);
 }

@@ -285,6 +285,24 @@ def test_sorted_paths_all_three_in_one_batch(hs, oracle):
     assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
 
 
+def test_sorted_modes_many_rows_and_one_row(hs, oracle):
+    """More rows than compute units share the list walk (one workgroup per row, 100 KB of LDS
+    each), and the single-row call of decode_step."""
+    n = 20000
+    g = np.random.default_rng(123)
+    x = (g.standard_normal((400, n)) * g.choice([0.7, 2.5, 6.0], (400, 1))).astype(np.float32)
+    u = g.random(400).astype(np.float32)
+    got = run_rows(hs, torch, x, u, P(temperature=1.0, top_p=0.9, min_p=0.001))
+    paths = hs.row_paths(400)
+    res = [oracle.chain_u(x[r], float(u[r]), temperature=1.0, top_p=0.9, min_p=0.001)
+           for r in range(400)]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "400 rows")
+    assert near <= 2 and 2 in paths and set(paths.tolist()) <= {1, 2, 3}
+    for r in (0, 1, 2):
+        one = run_rows(hs, torch, x[r:r + 1], u[r:r + 1], P(temperature=1.0, top_p=0.9, min_p=0.001))
+        assert one[0] == got[r]
+
+
 def test_top_p_limits_match_reference_dispatch(hs, oracle):
     x, u = rows_rng(5, 6, 3000)
     for p in (0.0, -1.0, 1.0, 1.5):        # sampler.c:238-243: <= 0 -> argmax... but the session
