@@ -2,16 +2,22 @@
  * sampler_kernels.hip -- the HIP kernels of the token-sampling path (gfx950).
  *
  * Kernel map (reference lines the arithmetic follows are cited at each kernel):
- *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t)          sampler.c:77-83
  *   k_tmax_scan      per-thread maxima (the single pass of the top-k path) and,
  *                    on request, the per-chunk maximum with its first index       sampler.c:52-62, 202-207
+ *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t); on request the sums of
+ *                    the chunk's slabs, or the min-p candidates of the row        sampler.c:77-83
  *   k_final_argmax / _temperature / _topk / _sorted   per-row combine of each mode: argmax,
  *                    index-order CDF draw, top-k select + sorted softmax + top-p + min-p +
  *                    draw, top-p / min-p shortcut                             sampler.c:90-102, 209-222, 272-299
- *   k_sorted_general full-vocabulary top-p / min-p by mass-weighted radix descent sampler.c:246-304
+ *   k_topk_general   top-k for k above 128 and degenerate rows                 sampler.c:178-228
+ *   k_list_candidates, k_sorted_candidates, k_sorted_general (sampler_sorted_prob.h)
+ *                    full-vocabulary top-p / min-p for kept prefixes the shortcut cannot
+ *                    serve: candidate list, then the whole row                 sampler.c:246-304
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
+ *   k_chunk_lse, k_final_logprob   log-softmax of chosen tokens               tools/eval_geist.c:63-73
  *   k_penalties      in-place penalties                                       (no reference counterpart)
- *   k_spec_resid, k_spec_final   speculative-decode verification              (no reference counterpart)
+ *   k_spec_accept, k_spec_resid, k_spec_final (sampler_spec.h)
+ *                    speculative-decode verification                          (no reference counterpart)
  *   k_rng_units      xorshift64* uniforms                                     sampler.c:35-48
  *
  * All streaming kernels use a (n_chunks, rows) grid of 256-thread workgroups and read each

@@ -4,14 +4,18 @@
  * top-k in front. Included by sampler_kernels.hip.
  *
  * The reference normalises every probability, sorts all of them and walks the sorted list.
- * Here nothing is sorted but the few entries that can matter:
- *   fast path (k_final_sorted)   thread maxima -> a logit bound below which nothing of the kept
- *                               prefix can lie -> re-read the threads above it -> order those
- *                               entries -> walk. Serves rows whose kept prefix is small.
- *   general path (k_sorted_general)  for rows the fast path hands on: the normalised
- *                               probabilities of the row are written once (k_write_probs), then
- *                               a mass-weighted radix descent over their bit patterns finds the
- *                               nucleus edge and the drawn entry without ordering anything.
+ * Here nothing is sorted but the few entries that can matter; a row takes the cheapest of three
+ * walks that can certify its result, decided on the device through the row's flag:
+ *   shortcut (k_final_sorted)    thread maxima -> a logit bound below which nothing of the kept
+ *                                prefix can lie -> re-read the threads above it -> order those
+ *                                entries -> walk. Kept prefixes of up to about a hundred.
+ *   list (flag 1 or 4: k_list_candidates / the exp-sum pass, k_sorted_candidates)
+ *                                every element up to a z bin is listed with its normalised
+ *                                probability; one mass histogram over the list locates the
+ *                                nucleus edge and the draw. Kept prefixes of thousands.
+ *   whole row (flag 2: k_sorted_general)   the row's probabilities are written once, then a
+ *                                mass-weighted radix descent over their bit patterns finds the
+ *                                edge and the drawn entry. Anything else.
  */
 #ifndef GEIST_SAMPLER_SORTED_PROB_H
 #define GEIST_SAMPLER_SORTED_PROB_H
