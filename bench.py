@@ -8,10 +8,13 @@ sit in HBM: penalties + temperature + top-k + top-p + draw for the default workl
 (B = 64 x V = 128256 fp32, T = 0.7, top-k 40, top-p 0.9, one seeded uniform per row, history of
 2048 Zipf ids per row with repetition 1.1 / frequency 0.5 / presence 0.3). Prints ONE JSON line.
 
-value      rows sampled per second over the timed K steps (whole job, one GPU)
+value      rows sampled per second over the timed K steps (whole job, one GPU). The steps rotate
+           over copies of the batch that together exceed the caches, so every step streams its
+           logits from HBM; `rows_per_s_cache_resident` is the same loop on one buffer, whose
+           logits the 256 MB Infinity Cache keeps between steps
 roofline   the logit-streaming kernel: algorithmic bytes per launch / its mean duration, the
            duration taken with HIP events on the sampler's stream around K back-to-back launches
-           of that kernel alone, right after the timed region
+           of that kernel alone over the same rotating copies, right after the timed region
 cpu_baseline  the CPU restatement of the same step (oracle, reference build flags) timed on
            this host's cores on a bounded sample; reported, not the optimisation target
 """
@@ -29,6 +32,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+COLD_WORKING_SET = 640 * 1024 * 1024   # bytes of logits the timed loops cycle through
 
 # HBM bytes moved by one launch of the streaming kernel, from rocprofv3's FETCH_SIZE and
 # WRITE_SIZE scaled by what the same counters read for a plain copy of the logit buffer
@@ -147,6 +151,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg2_pen")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="skip the cache-resident legs and the latency probe, so that every launch "
+                         "of the run streams its logits from HBM (for rocprofv3 runs whose "
+                         "per-kernel averages are to be compared with roofline.kernel_us)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of sampling, run a plain device copy of the logit buffer "
                          "(a kernel of known traffic, for scaling rocprof's FETCH_SIZE/WRITE_SIZE)")
@@ -184,31 +192,51 @@ def main():
                           "launches": args.steps}))
         return
 
-    def step():
-        hs.sample(rows, prm, d_u, d_out)
+    # Inputs resident in HBM, not in the caches: the steps rotate over copies of the batch that
+    # together exceed the 256 MB Infinity Cache (plus the L2s) more than twice, so every step
+    # streams its logits from HBM. One buffer used over and over would stay cache-resident and
+    # the streaming kernel would run above the HBM rate.
+    n_copies = max(2, -(-COLD_WORKING_SET // (d_logits.numel() * 4)))
+    copies = [d_logits] + [d_logits.clone() for _ in range(n_copies - 1)]
+    rows_cold = [HipSampler.rows(c, d_h, d_hl) for c in copies]
 
-    for _ in range(args.warmup):
-        step()
+    def step(i=0):
+        hs.sample(rows_cold[i % n_copies], prm, d_u, d_out)
+
+    for i in range(args.warmup):
+        step(i)
     hs.sync()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(i)
     hs.sync()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
     ids_gpu = d_out.cpu().numpy()
 
+    # the same with one buffer: logits that the caches still hold from the step before (in a
+    # decoder the lm_head has just written them)
+    ms_resident = None
+    if not args.cold_only:
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step(0)
+        hs.sync()
+        ms_resident = (time.perf_counter() - t1) * 1e3 / args.steps
+
     # the logit-streaming kernel on its own: HIP events on the sampler's stream around K
-    # back-to-back launches of that kernel (same rows, same configuration)
-    kernel_us = hs.time_stream_kernel(rows, prm, d_u, d_out, args.steps)
+    # back-to-back launches of that kernel (same configuration), again over the rotating copies
+    kernel_us = hs.time_stream_kernel_multi(rows_cold, prm, d_u, d_out, args.steps)
+    kernel_us_resident = (None if args.cold_only
+                          else hs.time_stream_kernel(rows, prm, d_u, d_out, args.steps))
 
     # one-step latency: enqueue + wait, median
     lat = []
-    for _ in range(200):
+    for i in range(0 if args.cold_only else 200):
         t1 = time.perf_counter()
-        step()
+        step(i)
         hs.sync()
         lat.append((time.perf_counter() - t1) * 1e6)
     lat.sort()
@@ -235,12 +263,19 @@ def main():
                    "min_p": w.min_p, "penalties": [w.rep, w.freq, w.pres],
                    "history_per_row": 0 if w.history is None else int(w.history.shape[1])},
         "us_per_step": round(ms_per_step * 1e3, 3),
-        "step_latency_us_median": round(lat[len(lat) // 2], 2),
+        "us_per_step_cache_resident": None if ms_resident is None else round(ms_resident * 1e3, 3),
+        "rows_per_s_cache_resident": None if ms_resident is None else round(
+            w.rows / (ms_resident * 1e-3), 1),
+        "input_copies_rotated": n_copies,
+        "step_latency_us_median": round(lat[len(lat) // 2], 2) if lat else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": PROFILED_TRAFFIC.get(w.name),
                      "kernel": "k_tmax_scan" if (w.top_k > 1 or w.temperature <= 0) else "k_chunk_expsum",
-                     "kernel_us": round(kernel_us, 3), "kernel_algorithmic_bytes": kernel_bytes,
+                     "kernel_us": round(kernel_us, 3),
+                     "kernel_us_cache_resident": None if kernel_us_resident is None else round(
+                         kernel_us_resident, 3),
+                     "kernel_algorithmic_bytes": kernel_bytes,
                      "step_algorithmic_bytes": alg_bytes,
                      "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }

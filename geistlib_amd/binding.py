@@ -77,6 +77,9 @@ def load_library():
     lib.geist_hip_sampler_time_stream_kernel.argtypes = [vp, C.POINTER(Rows),
                                                          C.POINTER(SampleParams), vp, vp, i32,
                                                          C.POINTER(C.c_double)]
+    lib.geist_hip_sampler_time_stream_kernel_multi.argtypes = [vp, C.POINTER(Rows), sz,
+                                                               C.POINTER(SampleParams), vp, vp, i32,
+                                                               C.POINTER(C.c_double)]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
     _LIB = lib
@@ -177,6 +180,15 @@ class HipSampler:
         ms = C.c_double()
         self._check(self.lib.geist_hip_sampler_time_stream_kernel(
             self.h, C.byref(rows), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
+            C.byref(ms)))
+        return ms.value * 1e3 / launches
+
+    def time_stream_kernel_multi(self, rows_list, params, uniforms, out, launches):
+        """As time_stream_kernel, launch i reading rows_list[i % len(rows_list)]."""
+        arr = (Rows * len(rows_list))(*rows_list)
+        ms = C.c_double()
+        self._check(self.lib.geist_hip_sampler_time_stream_kernel_multi(
+            self.h, arr, len(rows_list), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
             C.byref(ms)))
         return ms.value * 1e3 / launches
 

@@ -122,6 +122,7 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
     L.rv.hist_ld   = (long) r->history_ld;
     L.rv.hist_len  = pen ? r->d_history_len : nullptr;
     L.rv.rep       = pen ? p->repetition_penalty : 1.0f;
+    L.rv.inv_rep   = 1.0 / (double) L.rv.rep;
     L.rv.freq      = pen ? p->frequency_penalty : 0.0f;
     L.rv.pres      = pen ? p->presence_penalty : 0.0f;
     /* the soft-cap is monotone, so greedy rows skip it (head.c:145-149) */
@@ -620,27 +621,31 @@ int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, siz
     return GEIST_HIP_OK;
 }
 
-int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geist_hip_rows *rows,
-                                         const struct geist_hip_sample_params *params,
-                                         const float *d_uniforms, geist_hip_token_t *d_out_tokens,
-                                         int launches, double *ms_total) {
+int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
+                                               const struct geist_hip_rows *rows, size_t n_batches,
+                                               const struct geist_hip_sample_params *params,
+                                               const float *d_uniforms,
+                                               geist_hip_token_t *d_out_tokens, int launches,
+                                               double *ms_total) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
-    if (launches < 1 || !ms_total)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1 or null result");
+    if (launches < 1 || !ms_total || !rows || n_batches < 1)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
     hipEvent_t a, b;
     HIPCHK(s, hipSetDevice(s->device));
     HIPCHK(s, hipEventCreate(&a));
     HIPCHK(s, hipEventCreate(&b));
     /* a complete call first, so that the kernel finds the inputs an earlier stage leaves it */
-    int rc = sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+    int rc = 0;
+    for (size_t i = 0; i < n_batches && !rc; ++i)
+        rc = sample_impl(s, &rows[i], params, d_uniforms, d_out_tokens);
     s->stream_kernel_only = true;
-    if (!rc)
-        rc = sample_impl(s, rows, params, d_uniforms, d_out_tokens); /* warm the code object */
+    for (size_t i = 0; i < n_batches && !rc; ++i) /* warm the code object, cycle the caches */
+        rc = sample_impl(s, &rows[i], params, d_uniforms, d_out_tokens);
     if (!rc)
         rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
     for (int i = 0; i < launches && !rc; ++i)
-        rc = sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+        rc = sample_impl(s, &rows[(size_t) i % n_batches], params, d_uniforms, d_out_tokens);
     s->stream_kernel_only = false;
     float ms = 0.0f;
     if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
@@ -650,6 +655,14 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
     (void) hipEventDestroy(b);
     *ms_total = ms;
     return rc;
+}
+
+int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                                         const struct geist_hip_sample_params *params,
+                                         const float *d_uniforms, geist_hip_token_t *d_out_tokens,
+                                         int launches, double *ms_total) {
+    return geist_hip_sampler_time_stream_kernel_multi(s, rows, 1, params, d_uniforms, d_out_tokens,
+                                                      launches, ms_total);
 }
 
 int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,

@@ -30,6 +30,7 @@ struct RowView {
     long           hist_ld;
     const int32_t *hist_len;
     float          rep, freq, pres;
+    double         inv_rep; /* 1.0 / (double) rep, see penalise() */
     float          softcap; /* 0 = off */
 };
 

@@ -24,6 +24,9 @@
  * logit exactly once per kernel; the logits are never written (k_penalties excepted).
  */
 #include "sampler_kernels.h"
+#ifndef GS_XCD_REMAP
+#define GS_XCD_REMAP 1
+#endif
 
 #include "sampler_device.h"
 
@@ -216,7 +219,17 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
                                                    int32_t *__restrict__ zero_per_row) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
-    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    /* Workgroups go to the eight XCDs round-robin by their linear id, and each XCD has its own
+     * L2. The row-final kernel runs one workgroup per row (row r on XCD r mod 8) and reads the
+     * row's thread maxima and some of its logits again: with the rows dealt out so that all
+     * chunks of row r are scanned on XCD r mod 8, those reads find the lines in the local L2. */
+    int       row = blockIdx.y, chunk = blockIdx.x;
+    const int tid = threadIdx.x;
+    if ((gridDim.y & 7) == 0 && GS_XCD_REMAP) {
+        const int lin = blockIdx.y * gridDim.x + blockIdx.x, slot = lin >> 3;
+        row           = (lin & 7) + 8 * (slot / (int) gridDim.x);
+        chunk         = slot % (int) gridDim.x;
+    }
     if (BEST && zero_per_row && chunk == 0 && tid == 0)
         zero_per_row[row] = 0; /* a counter the following pass adds to */
     int       base, end;
@@ -820,30 +833,61 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         __syncthreads();
     }
     GS_MARK(4);
-    /* survivors are appended in any order: the ranking below orders them */
+    /* survivors are appended in any order (the ranking below orders them): their keys wait in
+     * registers until the lane has seen all its tasks, so that it asks for places once -- every
+     * LDS atomic that returns a value costs the wavefront a round trip */
+#ifdef GS_PHASES
+    __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): when have the gathered values arrived? */
+    GS_MARK(14);
+#endif
+    uint32_t ck[TASKS][4];
+    int      n_keep = 0;
 #pragma unroll
     for (int q = 0; q < TASKS; ++q) {
         const int t = tid + q * TPB;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            ck[q][c] = 0u;
         if (e0[q] >= e1[q])
             continue; /* no task (whole wavefronts beyond the list skip the block) */
-        uint4 hc = make_uint4(0u, 0u, 0u, 0u);
-        if (PEN)
-            hc = *reinterpret_cast<const uint4 *>(&s_pcnt[t * 4]);
+        float x4[4] = {r[q].x, r[q].y, r[q].z, r[q].w};
+#ifdef GS_EXP_NOPEN_TRANSFORM
+        if (false) {
+#else
+        if (PEN) {
+#endif
+            const uint4 hc = *reinterpret_cast<const uint4 *>(&s_pcnt[t * 4]);
+            if (hc.x | hc.y | hc.z | hc.w) { /* few float4 groups hold a history token */
+                x4[0] = hc.x ? penalise(x4[0], hc.x, rv.rep, rv.inv_rep, rv.freq, rv.pres) : x4[0];
+                x4[1] = hc.y ? penalise(x4[1], hc.y, rv.rep, rv.inv_rep, rv.freq, rv.pres) : x4[1];
+                x4[2] = hc.z ? penalise(x4[2], hc.z, rv.rep, rv.inv_rep, rv.freq, rv.pres) : x4[2];
+                x4[3] = hc.w ? penalise(x4[3], hc.w, rv.rep, rv.inv_rep, rv.freq, rv.pres) : x4[3];
+            }
+        }
+        if (rv.softcap > 0.0f) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                x4[c] = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x4[c], rv.softcap)), rv.softcap);
+        }
+        const int nvalid = e1[q] - e0[q]; /* 4 but at the row's end */
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            if (e0[q] + c < e1[q]) {
-                float x = f4_get(r[q], c);
-                if (PEN) {
-                    const uint32_t n_hist = c == 0 ? hc.x : c == 1 ? hc.y : c == 2 ? hc.z : hc.w;
-                    if (n_hist)
-                        x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
-                }
-                if (rv.softcap > 0.0f)
-                    x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);
-                if (x >= bound) {
-                    const int at = atomicAdd(s_n2, 1);
+            if (x4[c] >= bound && c < nvalid) { /* (a NaN fails the comparison: keys are > 0) */
+                ck[q][c] = f2key(x4[c]);
+                ++n_keep;
+            }
+        }
+    }
+    if (n_keep) {
+        int at = atomicAdd(s_n2, n_keep);
+#pragma unroll
+        for (int q = 0; q < TASKS; ++q) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (ck[q][c]) {
                     if (at < TPB)
-                        s_m[at] = pack_best(f2key(x), (uint32_t) (e0[q] + c));
+                        s_m[at] = pack_best(ck[q][c], (uint32_t) (e0[q] + c));
+                    ++at;
                 }
             }
         }
@@ -1275,7 +1319,7 @@ __global__ __launch_bounds__(TPB) void k_penalties(RowView rv, float *__restrict
             for (int c = 0; c < 4; ++c) {
                 const int e = base + off + c;
                 if (cnt[c] && e < end)
-                    rowp[e] = penalise(rowp[e], cnt[c], rv.rep, rv.freq, rv.pres);
+                    rowp[e] = penalise(rowp[e], cnt[c], rv.rep, rv.inv_rep, rv.freq, rv.pres);
             }
         }
     }

@@ -279,7 +279,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
                 if (PEN) {
                     const uint32_t n_hist = c == 0 ? hc.x : c == 1 ? hc.y : c == 2 ? hc.z : hc.w;
                     if (n_hist)
-                        x = penalise(x, n_hist, rv.rep, rv.freq, rv.pres);
+                        x = penalise(x, n_hist, rv.rep, rv.inv_rep, rv.freq, rv.pres);
                 }
                 if (rv.softcap > 0.0f)
                     x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);

@@ -188,6 +188,16 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
                                          const float *d_uniforms, geist_hip_token_t *d_out_tokens,
                                          int launches, double *ms_total);
 
+/* The same over n_batches batches of equal shape, launch i reading rows[i % n_batches]: with
+ * enough batches to exceed the caches (256 MB of Infinity Cache on an MI355X) every launch streams
+ * its logits from HBM, which is what a roofline against the HBM rate has to time. */
+int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
+                                               const struct geist_hip_rows *rows, size_t n_batches,
+                                               const struct geist_hip_sample_params *params,
+                                               const float *d_uniforms,
+                                               geist_hip_token_t *d_out_tokens, int launches,
+                                               double *ms_total);
+
 /* Diagnostics (no reference counterpart): after a full-vocabulary top-p / min-p call, which walk
  * served each row: 1 = shortcut over the per-thread maxima, 2 = candidate list, 3 = the whole
  * row. Synchronous; h_paths receives `rows` entries. */
