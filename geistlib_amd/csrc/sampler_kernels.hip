@@ -49,6 +49,21 @@ __device__ long long g_phase[16384 * 16];
 #define GS_MARK(i) ((void) 0)
 #endif
 
+/* Which (row, chunk) a workgroup of a (chunks, rows) grid works on. Workgroups go to the eight
+ * XCDs round-robin by their linear id, and each XCD has its own L2. With the rows dealt out so
+ * that every chunk of row r is handled on XCD r mod 8 -- in every pass, and the one-workgroup-
+ * per-row kernels put row r there as well -- a later pass or the row-final kernel finds the
+ * lines an earlier pass touched in the local L2. Needs a row count that is a multiple of 8. */
+__device__ __forceinline__ void xcd_row_chunk(int &row, int &chunk) {
+    row   = blockIdx.y;
+    chunk = blockIdx.x;
+    if ((gridDim.y & 7) == 0 && GS_XCD_REMAP) {
+        const int lin = blockIdx.y * gridDim.x + blockIdx.x, slot = lin >> 3;
+        row           = (lin & 7) + 8 * (slot / (int) gridDim.x);
+        chunk         = slot % (int) gridDim.x;
+    }
+}
+
 template <int NV>
 __device__ __forceinline__ void chunk_bounds(const RowView &rv, int chunk, int &base, int &end) {
     base = chunk * rv.per_chunk;
@@ -108,7 +123,9 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ int      s_listed, s_base;
-    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    int                 row, chunk;
+    xcd_row_chunk(row, chunk);
+    const int tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     int base, end;
@@ -219,17 +236,9 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
                                                    int32_t *__restrict__ zero_per_row) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ uint64_t s_red[NWAVES];
-    /* Workgroups go to the eight XCDs round-robin by their linear id, and each XCD has its own
-     * L2. The row-final kernel runs one workgroup per row (row r on XCD r mod 8) and reads the
-     * row's thread maxima and some of its logits again: with the rows dealt out so that all
-     * chunks of row r are scanned on XCD r mod 8, those reads find the lines in the local L2. */
-    int       row = blockIdx.y, chunk = blockIdx.x;
+    int row, chunk;
+    xcd_row_chunk(row, chunk);
     const int tid = threadIdx.x;
-    if ((gridDim.y & 7) == 0 && GS_XCD_REMAP) {
-        const int lin = blockIdx.y * gridDim.x + blockIdx.x, slot = lin >> 3;
-        row           = (lin & 7) + 8 * (slot / (int) gridDim.x);
-        chunk         = slot % (int) gridDim.x;
-    }
     if (BEST && zero_per_row && chunk == 0 && tid == 0)
         zero_per_row[row] = 0; /* a counter the following pass adds to */
     int       base, end;
@@ -1245,8 +1254,10 @@ __global__ __launch_bounds__(TPB) void k_chunk_lse(RowView rv, const uint64_t *_
                                                    double *__restrict__ chunk_sum) {
     __shared__ uint64_t s_red[NWAVES];
     __shared__ double   s_sum[NWAVES];
-    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
-    int                 base, end;
+    int                 row, chunk;
+    xcd_row_chunk(row, chunk);
+    const int tid = threadIdx.x;
+    int       base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
     fetch_chunk<NV, false>(rv, row, (int) gridDim.y, base, end, nullptr, v);

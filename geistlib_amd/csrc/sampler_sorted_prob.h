@@ -782,7 +782,9 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     __shared__ int      s_count, s_base;
     __shared__ float    s_arg[LIST_STAGE];
     __shared__ uint32_t s_id[LIST_STAGE];
-    const int           row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    int                 row, chunk;
+    xcd_row_chunk(row, chunk);
+    const int tid = threadIdx.x;
     if (row_flag[row] != 1)
         return;
     GS_MARK(0);
