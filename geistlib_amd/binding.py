@@ -80,6 +80,8 @@ def load_library():
     lib.geist_hip_sampler_time_stream_kernel_multi.argtypes = [vp, C.POINTER(Rows), sz,
                                                                C.POINTER(SampleParams), vp, vp, i32,
                                                                C.POINTER(C.c_double)]
+    lib.geist_hip_sampler_time_plain_read.argtypes = [vp, C.POINTER(Rows), sz, i32,
+                                                      C.POINTER(C.c_double)]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
     _LIB = lib
@@ -190,6 +192,14 @@ class HipSampler:
         self._check(self.lib.geist_hip_sampler_time_stream_kernel_multi(
             self.h, arr, len(rows_list), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
             C.byref(ms)))
+        return ms.value * 1e3 / launches
+
+    def time_plain_read(self, rows_list, launches):
+        """Mean duration in microseconds of a kernel that only reads the rows (calibration)."""
+        arr = (Rows * len(rows_list))(*rows_list)
+        ms = C.c_double()
+        self._check(self.lib.geist_hip_sampler_time_plain_read(self.h, arr, len(rows_list),
+                                                               int(launches), C.byref(ms)))
         return ms.value * 1e3 / launches
 
     def logprob(self, logits, tokens, out, softcap=0.0):

@@ -665,6 +665,40 @@ int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geis
                                                       launches, ms_total);
 }
 
+int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                                      size_t n_batches, int launches, double *ms_total) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (launches < 1 || !ms_total || !rows || n_batches < 1)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
+    std::vector<Launch> L(n_batches);
+    for (size_t i = 0; i < n_batches; ++i) {
+        const int rc = make_launch(s, &rows[i], nullptr, false, L[i]);
+        if (rc)
+            return rc;
+        L[i].nv           = 8; /* the geometry of the top-k scan */
+        L[i].rv.per_chunk = 8192;
+        L[i].rv.n_chunks  = (int) ((rows[i].n_vocab + 8191) / 8192);
+    }
+    hipEvent_t a, b;
+    HIPCHK(s, hipSetDevice(s->device));
+    HIPCHK(s, hipEventCreate(&a));
+    HIPCHK(s, hipEventCreate(&b));
+    for (size_t i = 0; i < n_batches; ++i)
+        launch_plain_read(L[i], s->uniforms);
+    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
+    for (int i = 0; i < launches && !rc; ++i)
+        launch_plain_read(L[(size_t) i % n_batches], s->uniforms);
+    float ms = 0.0f;
+    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
+                hipEventElapsedTime(&ms, a, b) != hipSuccess))
+        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
+    (void) hipEventDestroy(a);
+    (void) hipEventDestroy(b);
+    *ms_total = ms;
+    return rc ? rc : after_launch(s, "plain read");
+}
+
 int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,
                              float *d_out_units) {
     if (!s)

@@ -132,6 +132,8 @@ void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, 
 /* after launch_tmax_scan(L, tmax, chunk_best): out[row][j] = log_softmax(row)[tokens[row][j]] */
 void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,
                     const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld);
+/* calibration: reads the rows as the streaming kernels do and stores nothing */
+void launch_plain_read(const Launch &L, float *sink);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

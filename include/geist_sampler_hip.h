@@ -198,6 +198,12 @@ int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
                                                geist_hip_token_t *d_out_tokens, int launches,
                                                double *ms_total);
 
+/* Calibration for benchmarks (no reference counterpart): the same timing loop around a kernel
+ * that only reads the rows, with the launch geometry of the top-k scan, and stores nothing. Its
+ * mean duration is the floor of any one-pass kernel over these bytes on this device. */
+int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                                      size_t n_batches, int launches, double *ms_total);
+
 /* Diagnostics (no reference counterpart): after a full-vocabulary top-p / min-p call, which walk
  * served each row: 1 = shortcut over the per-thread maxima, 2 = candidate list, 3 = the whole
  * row. Synchronous; h_paths receives `rows` entries. */
