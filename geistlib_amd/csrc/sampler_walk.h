@@ -83,36 +83,44 @@ __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const do
                                 float inv_t, double sum, const float *qrow, bool qvec, int qx,
                                 const uint64_t *tab, uint32_t *s_cnt16, WalkShared &sh) {
     const int tid = threadIdx.x;
-    if (tid == 0) {
-        double tot = 0.0;
-        for (int c = 0; c < C; ++c)
-            tot += chunk_w[c];
+    if (tid < WAVE) {
+        /* chunk, then slab, by prefix sums on one wavefront: lane l holds chunks l and l + 64
+         * (MAX_CHUNKS = 128), the running sums come from DPP scans, the first chunk whose
+         * running sum exceeds the target from a ballot */
+        static_assert(MAX_CHUNKS <= 2 * WAVE, "two chunks per lane");
+        const double w0 = tid < C ? chunk_w[tid] : 0.0;
+        const double w1 = tid + WAVE < C ? chunk_w[tid + WAVE] : 0.0;
+        const double i0 = wave_scan_f64_dpp(w0);
+        const double h0 = __shfl(i0, WAVE - 1, WAVE);
+        const double i1 = h0 + wave_scan_f64_dpp(w1);
+        const double tot    = __shfl(i1, WAVE - 1, WAVE);
         const double target = (double) u * tot;
-        double       run    = 0.0;
-        int          at     = C - 1;
-        for (int c = 0; c < C; ++c) {
-            const double nxt = run + chunk_w[c];
-            if (target < nxt || c == C - 1) {
-                at = c;
-                break;
-            }
-            run = nxt;
+        const uint64_t b0 = __ballot(tid < C && target < i0);
+        const uint64_t b1 = __ballot(tid + WAVE < C && target < i1);
+        int            at = C - 1;
+        if (b0)
+            at = __ffsll((long long) b0) - 1;
+        else if (b1)
+            at = WAVE + __ffsll((long long) b1) - 1;
+        /* running sum before chunk `at`: the inclusive sum of the lane before it */
+        const double p0  = __shfl_up(i0, 1, WAVE), p1 = __shfl_up(i1, 1, WAVE);
+        const double e0  = tid ? p0 : 0.0, e1 = tid ? p1 : h0;
+        double       run = at < WAVE ? __shfl(e0, at, WAVE) : __shfl(e1, at - WAVE, WAVE);
+        /* slabs of that chunk: lane j holds slab j */
+        const double sw = tid < NV ? slab_w[at * SLABS_MAX + tid] : 0.0;
+        const double si = run + wave_scan_f64_dpp(sw);
+        const uint64_t bs = __ballot(tid < NV && target < si);
+        const int      js = bs ? __ffsll((long long) bs) - 1 : NV - 1;
+        const double ps   = __shfl_up(si, 1, WAVE);
+        run               = __shfl(tid ? ps : run, js, WAVE);
+        if (tid == 0) {
+            sh.chunk    = at;
+            sh.slab     = js;
+            sh.before   = run;
+            sh.target   = target;
+            sh.pick     = 0x7fffffff;
+            sh.last_pos = -1;
         }
-        int js = NV - 1;
-        for (int j = 0; j < NV; ++j) {
-            const double nxt = run + slab_w[at * SLABS_MAX + j];
-            if (target < nxt || j == NV - 1) {
-                js = j;
-                break;
-            }
-            run = nxt;
-        }
-        sh.chunk    = at;
-        sh.slab     = js;
-        sh.before   = run;
-        sh.target   = target;
-        sh.pick     = 0x7fffffff;
-        sh.last_pos = -1;
     }
     __syncthreads();
     const int    chunk  = sh.chunk;
