@@ -499,5 +499,12 @@ __device__ __forceinline__ int zbin(float arg) {
     return z < (float) (ZBINS - 1) ? (int) z : ZBINS - 1;
 }
 
+/* zbin(arg) <= b, as one comparison: the scaling in zbin() is by a power of two, hence exact,
+ * and truncation keeps z < b + 1, so the test is arg > -(b + 1) / ZBIN_PER_NAT (false for NaN,
+ * as zbin's last bin is). */
+__device__ __forceinline__ float zbin_threshold(int b) {
+    return -(float) (b + 1) / (float) ZBIN_PER_NAT;
+}
+
 } // namespace gs
 #endif

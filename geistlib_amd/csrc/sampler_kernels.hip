@@ -143,9 +143,10 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
     }
     if (LISTM && tid == 0)
         s_listed = 0;
-    double    acc  = 0.0;
-    double    accs[SLABS ? NV : 1];
-    uint32_t  mask = 0u;
+    double      acc  = 0.0;
+    double      accs[SLABS ? NV : 1];
+    uint32_t    mask = 0u;
+    const float list_thr = zbin_threshold(zb_list); /* zbin(arg) <= zb_list */
     /* positions at or beyond `end` hold -inf (load_raw): they weigh exactly 0 and land in no
      * bin, so the loop carries no bound tests */
 #pragma unroll
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
             a4 += (double) geist_expf_glibc_nonpos(arg, s_tab);
             if (LISTM)
-                mask |= (uint32_t) (zbin(arg) <= zb_list) << (4 * j + c);
+                mask |= (uint32_t) (arg > list_thr) << (4 * j + c);
         }
         if (SLABS)
             accs[j] = a4;

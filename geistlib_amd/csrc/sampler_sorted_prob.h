@@ -805,6 +805,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     const float  mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
     const double tot = s_total;
     const int    B   = cand.row_bound[row];
+    const float  thr = zbin_threshold(B); /* zbin(arg) <= B */
     GS_MARK(2);
     uint32_t     mask = 0u;
 #pragma unroll
@@ -812,7 +813,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
         const int e = base + 4 * (j * TPB + tid);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const bool in = e + c < end && zbin(softmax_arg(f4_get(v[j], c), mx, inv_t)) <= B;
+            const bool in = e + c < end && softmax_arg(f4_get(v[j], c), mx, inv_t) > thr;
             mask |= (uint32_t) in << (4 * j + c);
         }
     }
