@@ -58,55 +58,61 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 /* ---- wavefront-64 reductions -------------------------------------------------------------- */
+/* All by DPP moves (shifts inside each row of 16 lanes, then the row results are broadcast into
+ * the following rows), so that lane 63 ends with the result over all 64 lanes; a readlane hands
+ * it to every lane. No LDS crossbar traffic, and a fixed order of combination. Lanes without a
+ * source receive 0, the neutral element of every reduction here. */
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
     uint32_t lo = (uint32_t) v, hi = (uint32_t) (v >> 32);
     lo = (uint32_t) __shfl_xor((int) lo, m, WAVE);
     hi = (uint32_t) __shfl_xor((int) hi, m, WAVE);
     return ((uint64_t) hi << 32) | lo;
 }
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_fetch_u32(uint32_t v) {
+    return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, CTRL, ROW_MASK, 0xf, false);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint64_t dpp_fetch_u64(uint64_t v) {
+    return ((uint64_t) dpp_fetch_u32<CTRL, ROW_MASK>((uint32_t) (v >> 32)) << 32) |
+           dpp_fetch_u32<CTRL, ROW_MASK>((uint32_t) v);
+}
+__device__ __forceinline__ uint32_t readlane_u32(uint32_t v, int lane) {
+    return (uint32_t) __builtin_amdgcn_readlane((int) v, lane);
+}
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        const uint64_t o = shfl_xor_u64(v, m);
-        v                = o > v ? o : v;
+#define GS_STEP(ctrl, rows)                                                                    \
+    {                                                                                          \
+        const uint64_t o = dpp_fetch_u64<ctrl, rows>(v);                                       \
+        v                = o > v ? o : v;                                                      \
     }
-    return v;
+    GS_STEP(0x111, 0xf) GS_STEP(0x112, 0xf) GS_STEP(0x114, 0xf) GS_STEP(0x118, 0xf)
+    GS_STEP(0x142, 0xa) GS_STEP(0x143, 0xc)
+#undef GS_STEP
+    return ((uint64_t) readlane_u32((uint32_t) (v >> 32), WAVE - 1) << 32) |
+           readlane_u32((uint32_t) v, WAVE - 1);
 }
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        const uint32_t o = (uint32_t) __shfl_xor((int) v, m, WAVE);
-        v                = o > v ? o : v;
+#define GS_STEP(ctrl, rows)                                                                    \
+    {                                                                                          \
+        const uint32_t o = dpp_fetch_u32<ctrl, rows>(v);                                       \
+        v                = o > v ? o : v;                                                      \
     }
-    return v;
+    GS_STEP(0x111, 0xf) GS_STEP(0x112, 0xf) GS_STEP(0x114, 0xf) GS_STEP(0x118, 0xf)
+    GS_STEP(0x142, 0xa) GS_STEP(0x143, 0xc)
+#undef GS_STEP
+    return readlane_u32(v, WAVE - 1);
 }
+__device__ __forceinline__ double wave_scan_f64_dpp(double v);
+__device__ __forceinline__ int    wave_scan_i32_dpp(int v);
 __device__ __forceinline__ double wave_sum_f64(double v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1)
-        v += __shfl_xor(v, m, WAVE);
-    return v;
+    const uint64_t t = (uint64_t) __double_as_longlong(wave_scan_f64_dpp(v));
+    return __longlong_as_double((long long) (((uint64_t) readlane_u32((uint32_t) (t >> 32), WAVE - 1) << 32) |
+                                             readlane_u32((uint32_t) t, WAVE - 1)));
 }
-/* inclusive prefix sum over the lanes of a wavefront, lane order */
-__device__ __forceinline__ double wave_scan_f64(double v) {
-    const int lane = threadIdx.x & (WAVE - 1);
-#pragma unroll
-    for (int d = 1; d < WAVE; d <<= 1) {
-        const double o = __shfl_up(v, d, WAVE);
-        if (lane >= d)
-            v += o;
-    }
-    return v;
-}
-__device__ __forceinline__ int wave_scan_i32(int v) {
-    const int lane = threadIdx.x & (WAVE - 1);
-#pragma unroll
-    for (int d = 1; d < WAVE; d <<= 1) {
-        const int o = __shfl_up(v, d, WAVE);
-        if (lane >= d)
-            v += o;
-    }
-    return v;
-}
+/* inclusive prefix sums over the lanes of a wavefront, lane order */
+__device__ __forceinline__ double wave_scan_f64(double v) { return wave_scan_f64_dpp(v); }
+__device__ __forceinline__ int    wave_scan_i32(int v) { return wave_scan_i32_dpp(v); }
 
 /* Inclusive prefix sum over the wavefront with DPP moves: shifts inside each row of 16 lanes,
  * then the row totals are broadcast into the following rows. */
