@@ -443,6 +443,21 @@ __device__ __forceinline__ void load_raw(const RowView &rv, const float *__restr
     }
 }
 
+/* The logit soft-cap, tanhf(x / cap) * cap (head.c:148-159), kept out of line: few models have
+ * one, and glibc's tanhf is some two hundred instructions per element -- inlined at every site
+ * it would multiply the size of every kernel and evict the code that does run from the
+ * instruction cache. Arguments and results travel in registers. */
+__device__ __noinline__ float softcap1(float x, float cap) {
+    return __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, cap)), cap);
+}
+__device__ __noinline__ float4 softcap4(float4 v, float cap) {
+    v.x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v.x, cap)), cap);
+    v.y = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v.y, cap)), cap);
+    v.z = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v.z, cap)), cap);
+    v.w = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v.w, cap)), cap);
+    return v;
+}
+
 /* Penalties (when cnt16 != NULL) and the soft-cap on a chunk held in registers. */
 template <int NV>
 __device__ __forceinline__ void apply_transform(const RowView &rv, const uint32_t *cnt16,
@@ -469,10 +484,7 @@ __device__ __forceinline__ void apply_transform(const RowView &rv, const uint32_
         const float c = rv.softcap;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            v[j].x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].x, c)), c);
-            v[j].y = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].y, c)), c);
-            v[j].z = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].z, c)), c);
-            v[j].w = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(v[j].w, c)), c);
+            v[j] = softcap4(v[j], c);
         }
     }
 }

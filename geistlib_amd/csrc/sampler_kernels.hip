@@ -877,7 +877,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         if (rv.softcap > 0.0f) {
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                x4[c] = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x4[c], rv.softcap)), rv.softcap);
+                x4[c] = softcap1(x4[c], rv.softcap);
         }
         const int nvalid = e1[q] - e0[q]; /* 4 but at the row's end */
 #pragma unroll
@@ -1301,7 +1301,7 @@ __global__ __launch_bounds__(TPB) void k_final_logprob(RowView rv,
         if (t >= 0 && t < rv.n_vocab) {
             float x = rv.logits[(long) row * rv.ld + t];
             if (rv.softcap > 0.0f)
-                x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);
+                x = softcap1(x, rv.softcap);
             r = (double) __fsub_rn(x, mx) - lse;
         }
         out[(long) row * out_ld + j] = r;

@@ -282,7 +282,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
                         x = penalise(x, n_hist, rv.rep, rv.inv_rep, rv.freq, rv.pres);
                 }
                 if (rv.softcap > 0.0f)
-                    x = __fmul_rn(geist_tanhf_glibc(__fdiv_rn(x, rv.softcap)), rv.softcap);
+                    x = softcap1(x, rv.softcap);
                 if (x >= bound) { /* the logit for now; its probability below, one per thread */
                     const int at = atomicAdd(s_n2, 1);
                     if (at < TPB)
