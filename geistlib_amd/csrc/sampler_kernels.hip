@@ -75,6 +75,25 @@ __device__ __forceinline__ void chunk_bounds(const RowView &rv, int chunk, int &
 /* Loads and transforms the chunk [base, end) of a row; PEN selects the history lookup. `cnt16`
  * is an LDS table of NV*512 words when PEN, else unused. The logit loads are issued before the
  * history is read so that both are in flight together. */
+/* The soft-cap maps the -inf that pads a partial chunk to -cap, a finite logit with weight in
+ * every sum.  Positions at or beyond `end` are set back to -inf, so that consumers may keep
+ * treating them as weightless without a bound test of their own.  (A -inf INSIDE the row does
+ * become -cap, as it does in the reference: src/engine/sampler.c:95-99.) */
+template <int NV>
+__device__ __forceinline__ void remask_padding(const RowView &rv, int base, int end,
+                                               float4 (&v)[NV]) {
+    if (rv.softcap > 0.0f && end - base < NV * TPB * 4) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + (int) threadIdx.x);
+            if (e + 0 >= end) v[j].x = -INFINITY;
+            if (e + 1 >= end) v[j].y = -INFINITY;
+            if (e + 2 >= end) v[j].z = -INFINITY;
+            if (e + 3 >= end) v[j].w = -INFINITY;
+        }
+    }
+}
+
 template <int NV, bool PEN>
 __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_rows, int base,
                                             int end, uint32_t *cnt16, float4 (&v)[NV]) {
@@ -92,6 +111,7 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_ro
         load_raw<NV>(rv, rowp, base, end, v);
         apply_transform<NV>(rv, nullptr, v);
     }
+    remask_padding<NV>(rv, base, end, v);
 }
 
 /* Row maximum from the per-chunk results; every thread returns the same packed value. */

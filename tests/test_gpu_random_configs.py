@@ -1,0 +1,94 @@
+"""Differential test over random configurations: batch shape, vocabulary, sampling mode, penalties,
+history, soft-cap and logit distribution are all drawn from a seeded generator and every token id
+is compared with the oracle (penalties -> soft-cap -> chain), under the counted-exception rule of
+the other parity tests."""
+import numpy as np
+import pytest
+
+from gpu_util import compare_ids, run_rows
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hs():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=24, max_vocab=70000)
+    yield s
+    s.close()
+
+
+def _case(g):
+    rows = int(g.integers(1, 25))
+    n = int(g.choice([1, 2, 3, 7, 64, 255, 256, 257, 1000, 1024, 4097, 8192, 8193, 20000, 50257,
+                      65536, 70000]))
+    kind = g.choice(["normal", "wide", "peaked", "quantised", "ties", "student"])
+    if kind == "normal":
+        x = g.standard_normal((rows, n)) * 2
+    elif kind == "wide":
+        x = g.standard_normal((rows, n)) * 0.3
+    elif kind == "peaked":
+        x = g.standard_normal((rows, n)) * 7
+    elif kind == "quantised":
+        x = np.round(g.standard_normal((rows, n)) * 3 * 4) / 4
+    elif kind == "ties":
+        x = g.integers(-3, 4, (rows, n)).astype(np.float64)
+    else:
+        x = g.standard_t(3, (rows, n)) * 2.5
+    x = x.astype(np.float32)
+    mode = g.choice(["argmax", "temperature", "top_k", "top_p", "min_p", "chain", "k_p"])
+    prm = dict(temperature=float(g.choice([0.5, 0.7, 1.0, 1.3])), top_k=0, top_p=1.0, min_p=0.0)
+    if mode == "argmax":
+        prm["temperature"] = 0.0
+    if mode in ("top_k", "chain", "k_p"):
+        prm["top_k"] = int(g.choice([2, 5, 40, 64, 128, 129, 300, 1000]))
+    if mode in ("top_p", "chain", "k_p"):
+        prm["top_p"] = float(g.choice([0.3, 0.8, 0.9, 0.95, 0.99]))
+    if mode in ("min_p", "chain"):
+        prm["min_p"] = float(g.choice([0.001, 0.02, 0.05, 0.3]))
+    pen = None
+    if g.random() < 0.5 and n > 1:
+        H = int(g.choice([1, 17, 300, 2048]))
+        hist = g.integers(0, n, (rows, H)).astype(np.int32)
+        hl = g.integers(0, H + 1, rows).astype(np.int32)
+        lowering = g.random() < 0.7            # the common case has its own (lazy) code path
+        pen = dict(hist=hist, hl=hl,
+                   rep=float(g.choice([1.0, 1.1, 1.5]) if lowering else g.choice([0.8, 1.2])),
+                   freq=float(g.choice([0.0, 0.3, 0.5]) if lowering else g.choice([-0.2, 0.4])),
+                   pres=float(g.choice([0.0, 0.3]) if lowering else g.choice([-0.1, 0.2])))
+    cap = float(g.choice([0.0, 0.0, 30.0, 5.0]))
+    u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
+    return x, u, prm, pen, cap, f"{kind} rows={rows} n={n} {mode} {prm} pen={pen is not None} cap={cap}"
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations_match_oracle(hs, oracle, seed):
+    from geistlib_amd import SampleParams
+    g = np.random.default_rng(1000 + seed)
+    near_total = 0
+    for case in range(14):
+        x, u, prm, pen, cap, what = _case(g)
+        print(f"seed {seed} case {case}: {what}", flush=True)
+        kw = dict(prm)
+        if pen is not None:
+            kw.update(rep=pen["rep"], freq=pen["freq"], pres=pen["pres"])
+        p = SampleParams.make(softcap=cap, **kw)
+        got = run_rows(hs, torch, x, u, p, None if pen is None else pen["hist"],
+                       None if pen is None else pen["hl"])
+        res = []
+        for r in range(x.shape[0]):
+            row = x[r]
+            if pen is not None:
+                row = oracle.penalties(row, pen["hist"][r, :pen["hl"][r]], pen["rep"], pen["freq"],
+                                       pen["pres"])
+            if cap > 0 and prm["temperature"] > 0:
+                row = oracle.softcap(row, cap)
+            if prm["temperature"] <= 0:
+                res.append((oracle.argmax(row), None))
+            else:
+                res.append(oracle.chain_u(row, float(u[r]), **prm))
+        near_total += compare_ids(got, [t for t, _ in res], [i for _, i in res], what)
+    assert near_total <= 2

@@ -425,6 +425,35 @@ def test_softcap_fused_matches_libm_tanhf(hs, oracle, mode):
             assert np.mean(got_p[r].view(np.uint32) == want.view(np.uint32)) > 0.999
 
 
+@pytest.mark.parametrize("n", [64, 4097, 20000])
+@pytest.mark.parametrize("mode", ["temperature", "top_k", "top_p", "min_p"])
+def test_softcap_small_cap_ragged_row(hs, oracle, mode, n):
+    """A small cap on a row that ends inside a chunk: the -inf that pads the chunk must stay
+    weightless after the cap (tanhf(-inf) * cap = -cap is a finite logit, and with cap = 5 a few
+    thousand of them outweigh the row). Probabilities are compared too."""
+    from geistlib_amd import HipSampler
+    cap = 5.0
+    g = np.random.default_rng(n)
+    x = (g.standard_t(3, (8, n)) * 4.0).astype(np.float32)
+    x[1, n // 2] = -np.inf                            # inside the row -inf does become -cap
+    u = g.random(8).astype(np.float32)
+    kw = dict(temperature=1.0, top_k=40 if mode == "top_k" else 0,
+              top_p=0.9 if mode == "top_p" else 1.0, min_p=0.01 if mode == "min_p" else 0.0)
+    got = run_rows(hs, torch, x, u, P(softcap=cap, **kw))
+    res = [oracle.chain_u(oracle.softcap(x[r], cap), float(u[r]), **kw) for r in range(8)]
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"small cap {mode} n={n}")
+    assert near <= 1
+    if mode == "temperature":
+        d = to_dev(x, torch)
+        probs = torch.empty_like(d)
+        hs.softmax(HipSampler.rows(d), P(temperature=1.0, softcap=cap), probs)
+        hs.sync()
+        got_p = probs.cpu().numpy()
+        for r in range(8):
+            want, _ = oracle.softmax_normalised(oracle.softcap(x[r], cap), 1.0)
+            assert np.max(np.abs(got_p[r] - want) / np.maximum(want, 1e-38)) < 2e-7
+
+
 # ------------------------------------------------------------------------------ scoring
 @pytest.mark.parametrize("n,cap", [(1000, 0.0), (128256, 0.0), (128256, 30.0), (262144, 50.0)])
 def test_logprob_rows_match_oracle(hs, oracle, n, cap):
