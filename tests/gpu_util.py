@@ -11,9 +11,20 @@ def to_dev(a, torch):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_rows(sampler, torch, logits, uniforms, params, history=None, history_len=None):
+def run_rows(sampler, torch, logits, uniforms, params, history=None, history_len=None,
+             pad=0, lead=0):
+    """pad: extra elements between rows; lead: elements before the first row (an unaligned base).
+    Both gaps hold a huge logit, so a read outside a row changes the result."""
     from geistlib_amd import HipSampler
-    d_logits = to_dev(logits, torch)
+    if pad or lead:
+        rows, n = logits.shape
+        flat = np.full(lead + rows * (n + pad), 3e38, dtype=np.float32)
+        body = flat[lead:].reshape(rows, n + pad)
+        body[:, :n] = logits
+        d_flat = to_dev(flat, torch)
+        d_logits = d_flat[lead:].view(rows, n + pad)[:, :n]
+    else:
+        d_logits = to_dev(logits, torch)
     d_u = to_dev(uniforms, torch) if uniforms is not None else None
     d_h = to_dev(history, torch) if history is not None else None
     d_hl = to_dev(history_len, torch) if history_len is not None else None

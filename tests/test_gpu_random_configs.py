@@ -39,6 +39,9 @@ def _case(g):
     else:
         x = g.standard_t(3, (rows, n)) * 2.5
     x = x.astype(np.float32)
+    if g.random() < 0.25 and n > 8:               # banned tokens: -inf inside the row
+        x[g.random((rows, n)) < 0.1] = -np.inf
+        x[:, int(g.integers(0, n))] = 1.0         # at least one finite logit per row
     mode = g.choice(["argmax", "temperature", "top_k", "top_p", "min_p", "chain", "k_p"])
     prm = dict(temperature=float(g.choice([0.5, 0.7, 1.0, 1.3])), top_k=0, top_p=1.0, min_p=0.0)
     if mode == "argmax":
@@ -61,23 +64,25 @@ def _case(g):
                    pres=float(g.choice([0.0, 0.3]) if lowering else g.choice([-0.1, 0.2])))
     cap = float(g.choice([0.0, 0.0, 30.0, 5.0]))
     u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
-    return x, u, prm, pen, cap, f"{kind} rows={rows} n={n} {mode} {prm} pen={pen is not None} cap={cap}"
+    pad, lead = int(g.choice([0, 0, 1, 3, 4, 64])), int(g.choice([0, 0, 1, 2, 4]))
+    return x, u, prm, pen, cap, pad, lead, (f"{kind} rows={rows} n={n} {mode} {prm} "
+                                            f"pen={pen is not None} cap={cap} pad={pad} lead={lead}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(16))
 def test_random_configurations_match_oracle(hs, oracle, seed):
     from geistlib_amd import SampleParams
     g = np.random.default_rng(1000 + seed)
     near_total = 0
     for case in range(14):
-        x, u, prm, pen, cap, what = _case(g)
+        x, u, prm, pen, cap, pad, lead, what = _case(g)
         print(f"seed {seed} case {case}: {what}", flush=True)
         kw = dict(prm)
         if pen is not None:
             kw.update(rep=pen["rep"], freq=pen["freq"], pres=pen["pres"])
         p = SampleParams.make(softcap=cap, **kw)
         got = run_rows(hs, torch, x, u, p, None if pen is None else pen["hist"],
-                       None if pen is None else pen["hl"])
+                       None if pen is None else pen["hl"], pad=pad, lead=lead)
         res = []
         for r in range(x.shape[0]):
             row = x[r]
@@ -92,3 +97,71 @@ def test_random_configurations_match_oracle(hs, oracle, seed):
                 res.append(oracle.chain_u(row, float(u[r]), **prm))
         near_total += compare_ids(got, [t for t, _ in res], [i for _, i in res], what)
     assert near_total <= 2
+
+
+# ------------------------------------------------------------------- speculative verify
+@pytest.fixture(scope="module")
+def hs_spec():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=72, max_vocab=50257)
+    yield s
+    s.close()
+
+
+def _spec_matches(oracle, target, q, draft, u, T, nacc, out):
+    want_n, want = oracle.spec_verify(target, q, draft, u, T)
+    return nacc == want_n and out[:want_n + 1].tolist() == want[:want_n + 1].tolist()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_spec_verify_matches_oracle(hs_spec, oracle, seed):
+    """Random draft length, batch, vocabulary, temperature, soft-cap and draft quality, dense and
+    point-mass drafts. A sequence that differs must be explained by a uniform within 2e-6 of a
+    decision boundary (found by nudging each uniform of that sequence); those are counted."""
+    from gpu_util import to_dev
+    g = np.random.default_rng(5000 + seed)
+    near = 0
+    for case in range(6):
+        n_seq, L = int(g.integers(1, 9)), int(g.integers(1, 9))
+        n = int(g.choice([2, 64, 257, 1000, 4097, 8193, 20000, 50257]))
+        T = float(g.choice([0.0, 0.7, 1.0, 1.3]))
+        cap = float(g.choice([0.0, 0.0, 5.0, 30.0]))
+        dense = g.random() < 0.6
+        sigma = float(g.choice([0.05, 0.5, 2.0]))
+        what = f"seed {seed} case {case}: n_seq={n_seq} L={L} n={n} T={T} cap={cap} dense={dense}"
+        print(what, flush=True)
+        target = (g.standard_normal((n_seq, L + 1, n)) * 2.5).astype(np.float32)
+        noisy = target[:, :L, :].astype(np.float64) + g.standard_normal((n_seq, L, n)) * sigma
+        noisy -= noisy.max(axis=-1, keepdims=True)
+        e = np.exp(noisy)
+        q = (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+        cdf = np.cumsum(q.astype(np.float64), axis=-1)
+        pick = g.random((n_seq, L, 1)) * cdf[..., -1:]
+        draft = np.minimum((cdf < pick).sum(axis=-1), n - 1).astype(np.int32)
+        if not dense:
+            q = np.zeros_like(q)
+            np.put_along_axis(q, draft[..., None].astype(np.int64), 1.0, axis=-1)
+        u = (g.integers(0, 1 << 24, (n_seq, L + 1)) / np.float32(1 << 24)).astype(np.float32)
+        out = torch.full((n_seq, L + 1), -9, dtype=torch.int32, device="cuda")
+        nacc = torch.full((n_seq,), -9, dtype=torch.int32, device="cuda")
+        hs_spec.spec_verify(to_dev(target, torch), to_dev(q, torch) if dense else None,
+                            to_dev(draft, torch), to_dev(u, torch), T, out, nacc, softcap=cap)
+        hs_spec.sync()
+        out, nacc = out.cpu().numpy(), nacc.cpu().numpy()
+        for s in range(n_seq):
+            tg = target[s]
+            if cap > 0 and T > 0:
+                tg = np.stack([oracle.softcap(tg[j], cap) for j in range(L + 1)])
+            if _spec_matches(oracle, tg, q[s], draft[s], u[s], T, nacc[s], out[s]):
+                continue
+            explained = False
+            for j in range(L + 1):
+                for d in (-2e-6, 2e-6):
+                    u2 = u[s].copy()
+                    u2[j] = np.float32(min(max(float(u2[j]) + d, 0.0), 1 - 2.0 ** -24))
+                    explained |= _spec_matches(oracle, tg, q[s], draft[s], u2, T, nacc[s], out[s])
+            assert explained, (what, s, nacc[s], out[s])
+            near += 1
+    assert near <= 2
