@@ -165,3 +165,59 @@ def test_random_spec_verify_matches_oracle(hs_spec, oracle, seed):
             assert explained, (what, s, nacc[s], out[s])
             near += 1
     assert near <= 2
+
+
+# --------------------------------------------------------- probabilities and log-probabilities
+@pytest.mark.parametrize("seed", range(6))
+def test_random_softmax_and_logprob_rows(hs, oracle, seed):
+    """geist_hip_softmax_rows and geist_hip_logprob_rows over random shapes, strides, penalties,
+    temperatures and caps: probabilities within 2e-7 relative of the oracle's (the contract is
+    1e-5), log-probabilities within 1e-9 absolute."""
+    from geistlib_amd import HipSampler, SampleParams
+    from gpu_util import to_dev
+    g = np.random.default_rng(9000 + seed)
+    for case in range(8):
+        rows = int(g.integers(1, 13))
+        n = int(g.choice([1, 2, 5, 64, 257, 1000, 4097, 8193, 20000, 65536, 70000]))
+        pad = int(g.choice([0, 0, 1, 4, 7]))
+        T = float(g.choice([0.5, 1.0, 1.7]))
+        cap = float(g.choice([0.0, 0.0, 5.0, 30.0]))
+        scale = float(g.choice([0.3, 2.0, 8.0]))
+        with_pen = g.random() < 0.4 and n > 1
+        what = f"seed {seed} case {case}: rows={rows} n={n} pad={pad} T={T} cap={cap} pen={with_pen}"
+        print(what, flush=True)
+        x = (g.standard_normal((rows, n)) * scale).astype(np.float32)
+        buf = np.full((rows, n + pad), 3e38, dtype=np.float32)
+        buf[:, :n] = x
+        d = to_dev(buf, torch)[:, :n]
+        kw, hist, hl, d_h, d_hl = {}, None, None, None, None
+        if with_pen:
+            H = int(g.choice([3, 200, 2048]))
+            hist = g.integers(0, n, (rows, H)).astype(np.int32)
+            hl = g.integers(0, H + 1, rows).astype(np.int32)
+            d_h, d_hl = to_dev(hist, torch), to_dev(hl, torch)
+            kw = dict(rep=1.2, freq=0.25, pres=0.5)
+        probs = torch.full((rows, n + pad), -1.0, dtype=torch.float32, device="cuda")
+        hs.softmax(HipSampler.rows(d, d_h, d_hl), SampleParams.make(temperature=T, softcap=cap, **kw),
+                   probs[:, :n])
+        hs.sync()
+        got = probs.cpu().numpy()
+        assert np.all(got[:, n:] == -1.0), what        # nothing written between the rows
+        K = 5
+        tok = g.integers(0, n, (rows, K)).astype(np.int32)
+        lp = torch.zeros((rows, K), dtype=torch.float64, device="cuda")
+        hs.logprob(d, to_dev(tok, torch), lp, softcap=cap)
+        hs.sync()
+        lp = lp.cpu().numpy()
+        for r in range(rows):
+            row = x[r]
+            if with_pen:
+                row = oracle.penalties(row, hist[r, :hl[r]], 1.2, 0.25, 0.5)
+            if cap > 0:
+                row = oracle.softcap(row, cap)
+            want, _ = oracle.softmax_normalised(row, T)
+            err = np.max(np.abs(got[r, :n] - want) / np.maximum(want, 1e-38))
+            assert err < 2e-7, (what, r, err)
+            plain = oracle.softcap(x[r], cap) if cap > 0 else x[r]
+            for j in range(K):
+                assert abs(lp[r, j] - oracle.logprob_at(plain, int(tok[r, j]))) < 1e-9, (what, r, j)
