@@ -84,6 +84,7 @@ def load_library():
                                                       C.POINTER(C.c_double)]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
+    lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     _LIB = lib
     return lib
 
@@ -175,6 +176,17 @@ class HipSampler:
         self._check(self.lib.geist_hip_spec_verify(self.h, _ptr(target), n, _ptr(q), n, _ptr(draft),
                                                    _ptr(uniforms), n_seq, L, n, temperature,
                                                    softcap, _ptr(out_tokens), _ptr(n_accepted)))
+
+    def propose_drafts_ngram(self, history, history_len, seeds, k_max, max_suffix, out_drafts,
+                             out_count, out_match_len):
+        """N-gram drafts for every sequence: history [n_seq, H] int32 with history_len [n_seq],
+        seeds [n_seq]; out_drafts [n_seq, >= k_max], out_count and out_match_len [n_seq]."""
+        n_seq = history.shape[0]
+        hld = history.stride(0) if n_seq > 1 else history.shape[1]
+        old = out_drafts.stride(0) if n_seq > 1 else out_drafts.shape[1]
+        self._check(self.lib.geist_hip_propose_drafts_ngram(
+            self.h, _ptr(history), hld, _ptr(history_len), _ptr(seeds), n_seq, int(k_max),
+            int(max_suffix), _ptr(out_drafts), old, _ptr(out_count), _ptr(out_match_len)))
 
     def time_stream_kernel(self, rows, params, uniforms, out, launches):
         """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around

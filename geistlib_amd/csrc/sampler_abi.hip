@@ -534,6 +534,29 @@ int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t l
     return after_launch(s, "log-probabilities");
 }
 
+int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,
+                                   size_t history_ld, const int32_t *d_history_len,
+                                   const geist_hip_token_t *d_seed, size_t n_seq, size_t k_max,
+                                   size_t max_suffix, geist_hip_token_t *d_out_drafts,
+                                   size_t out_ld, int32_t *d_out_count, int32_t *d_out_match_len) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_history || !d_history_len || !d_seed || !d_out_drafts || !d_out_count ||
+        !d_out_match_len)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_seq == 0 || n_seq > 0x7fffffffu)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "n_seq %zu", n_seq);
+    if (k_max == 0 || k_max > (size_t) NGRAM_DRAFT_MAX)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "k_max %zu (1..%d)", k_max, NGRAM_DRAFT_MAX);
+    if (out_ld < k_max)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "out_ld %zu < k_max %zu", out_ld, k_max);
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_ngram_draft(s->stream, d_history, (long) history_ld, d_history_len, d_seed, (int) n_seq,
+                       (int) k_max, max_suffix > 64 ? 64 : (int) max_suffix, d_out_drafts,
+                       (long) out_ld, d_out_count, d_out_match_len);
+    return after_launch(s, "n-gram drafts");
+}
+
 int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld_t,
                           const float *d_draft_q, size_t ld_q, const int32_t *d_draft,
                           const float *d_uniforms, size_t n_seq, size_t L, size_t n_vocab,

@@ -110,6 +110,8 @@ struct SpecLaunch {
 };
 constexpr int SLABS_MAX         = 8; /* slab sums are stored 8 per chunk whatever NV is */
 constexpr int SPEC_DRAFT_MAX      = 63;
+constexpr int NGRAM_SUFFIX_MAX    = 8;  /* session.c:455-456 */
+constexpr int NGRAM_DRAFT_MAX     = 16; /* GEIST_SPEC_KMAX_HARDCAP, session.c:515 */
 constexpr int SPEC_VERDICT_BYTES = 24;
 void launch_spec(const Launch &L, const SpecLaunch &sp);
 /* chunk_best may be NULL when only the thread maxima are wanted */
@@ -134,6 +136,10 @@ void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_s
                     const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld);
 /* calibration: reads the rows as the streaming kernels do and stores nothing */
 void launch_plain_read(const Launch &L, float *sink);
+void launch_ngram_draft(hipStream_t stream, const int32_t *history, long history_ld,
+                        const int32_t *history_len, const int32_t *seeds, int n_seq, int k_max,
+                        int max_suffix, int32_t *out, long out_ld, int32_t *out_count,
+                        int32_t *out_match);
 void launch_penalties(const Launch &L, float *logits_rw);
 void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows, float *uniforms);
 

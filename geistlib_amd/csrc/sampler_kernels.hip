@@ -958,6 +958,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #include "sampler_walk.h"
 #include "sampler_sorted_prob.h"
 #include "sampler_spec.h"
+#include "sampler_draft.h"
 namespace gs {
 
 /* ============================================================================================
@@ -1617,6 +1618,15 @@ void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_s
         k_chunk_lse<2><<<grid, block, 0, L.stream>>>(L.rv, chunk_best, chunk_sum);
     k_final_logprob<<<dim3(L.rows), block, 0, L.stream>>>(L.rv, chunk_best, chunk_sum, tokens,
                                                          tokens_ld, k_per_row, out, out_ld);
+}
+
+void launch_ngram_draft(hipStream_t stream, const int32_t *history, long history_ld,
+                        const int32_t *history_len, const int32_t *seeds, int n_seq, int k_max,
+                        int max_suffix, int32_t *out, long out_ld, int32_t *out_count,
+                        int32_t *out_match) {
+    k_ngram_draft<<<dim3(n_seq), dim3(TPB), 0, stream>>>(history, history_ld, history_len, seeds,
+                                                         k_max, max_suffix, out, out_ld, out_count,
+                                                         out_match);
 }
 
 void launch_plain_read(const Launch &L, float *sink) {

@@ -24,6 +24,7 @@ struct geist_hip_head {
     float    *d_units;  /* m_max uniforms of one speculative round */
     int32_t  *d_drafts; /* m_max */
     int32_t  *d_nacc;
+    int32_t  *d_ngram;  /* seed, history length, count, matched length, 16 drafts */
     char      err[256];
 };
 
@@ -70,6 +71,9 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
         h->d_drafts = p;
     if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(h->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_nacc = p;
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_malloc(h->hs, 20 * sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        h->d_ngram = p;
     /* arch_state.c:1173: the default seed */
     if (rc == GEIST_HIP_OK)
         rc = seed_rng(h, UINT64_C(0xCAFEBABE1234));
@@ -90,6 +94,7 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         geist_hip_free(h->hs, h->d_units);
         geist_hip_free(h->hs, h->d_drafts);
         geist_hip_free(h->hs, h->d_nacc);
+        geist_hip_free(h->hs, h->d_ngram);
         geist_hip_sampler_destroy(h->hs);
     }
     free(h);
@@ -156,6 +161,41 @@ int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, s
         return head_fail(h, GEIST_HIP_E_UNSUPPORTED, "row longer than the probed vocabulary");
     if (geist_hip_argmax_f32(h->hs, d_logits, n, out_index) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "argmax");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_propose_drafts(struct geist_hip_head *h, const int32_t *d_history,
+                                  size_t history_n, int32_t seed, size_t k_max,
+                                  int32_t *out_drafts, size_t *n_drafts, size_t *match_len) {
+    if (h == nullptr || out_drafts == nullptr || n_drafts == nullptr ||
+        (history_n > 0 && d_history == nullptr))
+        return GEIST_HIP_E_INVALID_ARG;
+    *n_drafts = 0;
+    if (match_len != nullptr)
+        *match_len = 0;
+    if (k_max == 0 || k_max > 16) /* session.c:546-548 */
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "k_max outside 1..16");
+    if (history_n > INT32_MAX)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "history too long");
+    out_drafts[0] = seed;
+    *n_drafts     = 1;
+    if (history_n == 0 || k_max == 1) /* session.c:446-447 */
+        return GEIST_HIP_OK;
+    const int32_t in[2] = {seed, (int32_t) history_n};
+    int32_t       back[18];
+    if (geist_hip_upload(h->hs, h->d_ngram, in, sizeof in) != GEIST_HIP_OK ||
+        geist_hip_propose_drafts_ngram(h->hs, d_history, history_n, h->d_ngram + 1, h->d_ngram, 1,
+                                       k_max, /*max_suffix=*/4, h->d_ngram + 4, 16,
+                                       h->d_ngram + 2, h->d_ngram + 3) != GEIST_HIP_OK ||
+        geist_hip_download(h->hs, back, h->d_ngram + 2, (2 + k_max) * sizeof(int32_t)) !=
+                GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "n-gram drafts");
+    if (back[0] < 1 || (size_t) back[0] > k_max || back[1] < 0 || back[1] > 4)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "draft count out of range");
+    memcpy(out_drafts, back + 2, (size_t) back[0] * sizeof *out_drafts);
+    *n_drafts = (size_t) back[0];
+    if (match_len != nullptr)
+        *match_len = (size_t) back[1];
     return GEIST_HIP_OK;
 }
 

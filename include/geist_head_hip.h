@@ -10,6 +10,8 @@
  *   geist_hip_head_finalize_batch     sampler part of finalize_logits_batch (head.c:274-304)
  *   geist_hip_head_argmax_f32      the backend slot fused->argmax_f32
  *                                  (include/geist_backend.h:414-421)
+ *   geist_hip_head_propose_drafts  the n-gram drafter of geist_session_decode_speculative
+ *                                  (src/engine/session.c:437-513, 564-572)
  *   geist_hip_head_spec_accept     the accept loop of geist_session_decode_speculative
  *                                  (src/engine/session.c:599-625) over the rows verify_forward
  *                                  produced (src/archs/transformer/arch_ops.c:176-270)
@@ -62,6 +64,17 @@ int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logit
                                   int32_t *out_tokens);
 int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,
                               int32_t *out_index);
+
+/* The drafting step of one speculative round (session.c:564-572) for a token history kept in
+ * device memory: seed is the pending next token (what the finalize call of the step before
+ * returned; op_peek_next_token, src/archs/transformer/arch.c:156-161), the drafts come from the
+ * n-gram lookup with max_suffix = 4 (session.c:570-571). out_drafts holds k_max entries
+ * (1..16); out_drafts[0] = seed. *match_len is the matched suffix length: the reference goes
+ * on to verify_forward only when *n_drafts > 1 and *match_len >= 2 (session.c:572-592), and
+ * falls back to a single decode step otherwise. */
+int geist_hip_head_propose_drafts(struct geist_hip_head *h, const int32_t *d_history,
+                                  size_t history_n, int32_t seed, size_t k_max,
+                                  int32_t *out_drafts, size_t *n_drafts, size_t *match_len);
 
 /* The accept step of one speculative round. drafts[0..k) are the tokens fed to verify_forward
  * (drafts[0] is the already-sampled next token, session.c:563-568), d_logits the [k, vocab] rows

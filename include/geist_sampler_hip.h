@@ -144,6 +144,26 @@ int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t l
                            size_t n_vocab, float logit_softcap, const int32_t *d_tokens,
                            size_t tokens_ld, size_t k_per_row, double *d_out, size_t out_ld);
 
+/* The n-gram drafter of the reference's speculative loop (propose_drafts_ngram,
+ * src/engine/session.c:437-513; called with max_suffix = 4 at :570-571, capped at 8 at :455-456), for n_seq sequences
+ * whose token histories are on the device (the history layout of struct geist_hip_rows):
+ *   d_history [n_seq][history_ld], d_history_len [n_seq], d_seed [n_seq] (each sequence's
+ *   pending next token, op_peek_next_token, src/archs/transformer/arch.c:156-161: here the
+ *   output of the geist_hip_sample_rows call of the step before, still on the device)
+ * Finds the longest suffix of history + [seed], at most min(max_suffix, 8) tokens, that occurs
+ * earlier in the history; among the occurrences of that length the one with the most following
+ * tokens (counted up to k_max - 1), the most recent among equals.
+ *   d_out_drafts [n_seq][out_ld]: drafts[0] = seed, then the tokens that followed the match
+ *   d_out_count  [n_seq]: number of drafts written (>= 1; 1 = no usable match)
+ *   d_out_match_len [n_seq]: length of the matched suffix, 0 without a match (the reference
+ *                    skips verification below GEIST_SPEC_MIN_L = 2, session.c:575-592)
+ * 1 <= k_max <= 16 (GEIST_SPEC_KMAX_HARDCAP, session.c:515), out_ld >= k_max. */
+int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,
+                                   size_t history_ld, const int32_t *d_history_len,
+                                   const geist_hip_token_t *d_seed, size_t n_seq, size_t k_max,
+                                   size_t max_suffix, geist_hip_token_t *d_out_drafts,
+                                   size_t out_ld, int32_t *d_out_count, int32_t *d_out_match_len);
+
 /* Speculative-decode verification for n_seq sequences with draft length L (no reference
  * counterpart: include/geist_util.h:233-240 documents that the reference's speculative loop
  * omits rejection sampling; the batch shape is that of verify_forward,

@@ -13,6 +13,7 @@
 #include "sampler_oracle.h"
 
 #include <math.h>
+#include <stdbool.h>
 #include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
@@ -652,4 +653,49 @@ double oracle_logprob_at(size_t n, const float *logits, int32_t token) {
     for (size_t i = 0; i < n; i++)
         sum += exp((double) (logits[i] - maxv));
     return (double) (logits[token] - maxv) - log(sum);
+}
+
+/* src/engine/session.c:437-513. Lengths are tried longest first; for one length the history is
+ * walked from the most recent start position backwards, a later find only replaces an earlier
+ * one when more tokens follow it, and the walk stops once k_max - 1 follow. */
+size_t oracle_propose_drafts_ngram(const int32_t *history, size_t n, int32_t seed, size_t k_max,
+                                   size_t max_suffix, int32_t *out, size_t *match_len) {
+    out[0] = seed;
+    if (match_len)
+        *match_len = 0;
+    if (k_max <= 1 || n == 0)
+        return 1;
+    const size_t want = k_max - 1;
+    for (size_t len = max_suffix > 8 ? 8 : max_suffix; len >= 1; len--) {
+        const size_t ctx = len - 1; /* history tokens in the suffix; the seed is its last */
+        if (ctx > n)
+            continue;
+        const int32_t *tail  = history + (n - ctx);
+        bool           have  = false;
+        size_t         at    = 0, gain = 0;
+        for (size_t start = n - ctx; start-- > 0;) {
+            if (ctx && memcmp(history + start, tail, ctx * sizeof *history) != 0)
+                continue;
+            if (history[start + ctx] != seed)
+                continue;
+            const size_t next = start + len;
+            if (next >= n)
+                continue; /* nothing follows */
+            const size_t room = n - next < want ? n - next : want;
+            if (!have || room > gain) {
+                have = true;
+                at   = start;
+                gain = room;
+                if (gain >= want)
+                    break;
+            }
+        }
+        if (have) {
+            memcpy(out + 1, history + at + len, gain * sizeof *out);
+            if (match_len)
+                *match_len = len;
+            return 1 + gain;
+        }
+    }
+    return 1;
 }

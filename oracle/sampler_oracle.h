@@ -160,6 +160,16 @@ int  oracle_max_threads(void);
  * double sum, (double)(logits[token] - max) - log(sum). */
 double oracle_logprob_at(size_t n, const float *logits, int32_t token);
 
+/* The n-gram drafter of the speculative loop (propose_drafts_ngram,
+ * src/engine/session.c:437-513): out[0] = seed; then, for the longest suffix of history + [seed]
+ * (at most min(max_suffix, 8) tokens) found earlier in the history, the up to k_max - 1 tokens
+ * that followed its best occurrence (most following tokens, most recent among equals). Returns
+ * the number of drafts (>= 1); *match_len = length of the matched suffix or 0. `out` holds
+ * k_max entries. Pinned by a brute-force enumeration over (length, position) in the tests and
+ * by worked examples; the reference holds no test of this function. */
+size_t oracle_propose_drafts_ngram(const int32_t *history, size_t n, int32_t seed, size_t k_max,
+                                   size_t max_suffix, int32_t *out, size_t *match_len);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,9 @@ def load_oracle(fast=False):
     lib.oracle_softcap_inplace.argtypes = [C.c_size_t, c_float_p, C.c_float]
     lib.oracle_logprob_at.argtypes = [C.c_size_t, c_float_p, C.c_int32]
     lib.oracle_logprob_at.restype = C.c_double
+    lib.oracle_propose_drafts_ngram.restype = C.c_size_t
+    lib.oracle_propose_drafts_ngram.argtypes = [c_int32_p, C.c_size_t, C.c_int32, C.c_size_t,
+                                                C.c_size_t, c_int32_p, C.POINTER(C.c_size_t)]
     lib.oracle_finalize_row.restype = C.c_int32
     lib.oracle_finalize_row.argtypes = [C.POINTER(SessionSampler), C.c_size_t, c_float_p, C.c_float]
     lib.oracle_finalize_batch.argtypes = [C.POINTER(SessionSampler), C.c_size_t, C.c_size_t,
@@ -168,6 +171,15 @@ class Oracle:
     def logprob_at(self, row, token):
         row = np.ascontiguousarray(row, dtype=np.float32)
         return float(self.lib.oracle_logprob_at(row.size, _fp(row), int(token)))
+
+    def propose_drafts_ngram(self, history, seed, k_max, max_suffix):
+        """-> (drafts as a list, length of the matched suffix)"""
+        history = np.ascontiguousarray(history, dtype=np.int32)
+        out = np.full(max(int(k_max), 1), -1, dtype=np.int32)
+        match = C.c_size_t(99)
+        k = self.lib.oracle_propose_drafts_ngram(_ip(history), history.size, int(seed), int(k_max),
+                                                 int(max_suffix), _ip(out), C.byref(match))
+        return out[:k].tolist(), int(match.value)
 
     def softcap(self, row, cap):
         out = row.copy()

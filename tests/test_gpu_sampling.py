@@ -649,3 +649,58 @@ def test_argument_errors(hs):
     big.rows = 100000
     with pytest.raises(GeistHipError):     # beyond the workspace
         hs.sample(big, P(temperature=0.0), None, out)
+
+
+# ------------------------------------------------------------------------- n-gram drafter
+@pytest.mark.parametrize("seed", range(4))
+def test_ngram_drafter_matches_oracle(hs, oracle, seed):
+    """geist_hip_propose_drafts_ngram against the restated propose_drafts_ngram
+    (src/engine/session.c:437-513): drafts, their count and the matched length, exactly."""
+    g = np.random.default_rng(700 + seed)
+    for case in range(6):
+        n_seq = int(g.integers(1, 33))
+        H = int(g.choice([1, 2, 9, 300, 5000]))
+        alphabet = int(g.choice([2, 4, 30, 1000]))
+        k_max = int(g.integers(1, 17))
+        ms = int(g.choice([0, 1, 2, 4, 8, 11]))
+        pad = int(g.choice([0, 3]))
+        hist = g.integers(0, alphabet, (n_seq, H + pad)).astype(np.int32)
+        if alphabet == 1000 and H >= 300:          # text that repeats itself in long stretches
+            for s in range(n_seq):
+                period = int(g.integers(5, 60))
+                hist[s] = np.resize(hist[s, :period], H + pad)
+                hist[s, g.integers(0, H, 8)] = 7    # with a few edits
+        hl = g.integers(0, H + 1, n_seq).astype(np.int32)
+        hl[0] = H
+        seeds = np.array([hist[s, g.integers(0, max(int(hl[s]), 1))] for s in range(n_seq)],
+                         dtype=np.int32)
+        seeds[-1] = -1                              # a seed that occurs nowhere
+        print(f"drafter seed {seed} case {case}: n_seq={n_seq} H={H} alphabet={alphabet} "
+              f"k_max={k_max} max_suffix={ms}", flush=True)
+        out = torch.full((n_seq, k_max + 2), -9, dtype=torch.int32, device="cuda")
+        cnt = torch.full((n_seq,), -9, dtype=torch.int32, device="cuda")
+        mlen = torch.full((n_seq,), -9, dtype=torch.int32, device="cuda")
+        hs.propose_drafts_ngram(to_dev(hist, torch), to_dev(hl, torch), to_dev(seeds, torch), k_max,
+                                ms, out, cnt, mlen)
+        hs.sync()
+        out, cnt, mlen = out.cpu().numpy(), cnt.cpu().numpy(), mlen.cpu().numpy()
+        lengths = set()
+        for s in range(n_seq):
+            want, wl = oracle.propose_drafts_ngram(hist[s, :hl[s]], int(seeds[s]), k_max, ms)
+            assert cnt[s] == len(want) and mlen[s] == wl, (s, cnt[s], mlen[s], want, wl)
+            assert out[s, :cnt[s]].tolist() == want, (s, out[s], want)
+            assert np.all(out[s, cnt[s]:] == -9)    # nothing written beyond the drafts
+            lengths.add(wl)
+        print("  matched lengths seen:", sorted(lengths))
+
+
+def test_ngram_drafter_argument_errors(hs):
+    from geistlib_amd.binding import GeistHipError
+    h = torch.zeros((2, 8), dtype=torch.int32, device="cuda")
+    hl = torch.zeros(2, dtype=torch.int32, device="cuda")
+    sd = torch.zeros(2, dtype=torch.int32, device="cuda")
+    out = torch.zeros((2, 4), dtype=torch.int32, device="cuda")
+    c = torch.zeros(2, dtype=torch.int32, device="cuda")
+    for k_max in (0, 17, 5):                        # 5 > out_ld = 4
+        with pytest.raises(GeistHipError):
+            hs.propose_drafts_ngram(h, hl, sd, k_max, 4, out, c, c)
