@@ -22,7 +22,8 @@ class GeistHipError(RuntimeError):
 class Rows(C.Structure):
     _fields_ = [("d_logits", C.c_void_p), ("ld", C.c_size_t), ("rows", C.c_size_t),
                 ("n_vocab", C.c_size_t), ("d_history", C.c_void_p), ("history_ld", C.c_size_t),
-                ("d_history_len", C.c_void_p)]
+                ("d_history_len", C.c_void_p), ("d_allowed", C.c_void_p),
+                ("allowed_ld", C.c_size_t)]
 
 
 class SampleParams(C.Structure):
@@ -125,8 +126,9 @@ class HipSampler:
         self._check(self.lib.geist_hip_sampler_sync(self.h))
 
     @staticmethod
-    def rows(logits, history=None, history_len=None, n_vocab=None):
-        """logits: 2-D float32 device tensor (row stride = logits.stride(0))."""
+    def rows(logits, history=None, history_len=None, n_vocab=None, allowed=None):
+        """logits: 2-D float32 device tensor (row stride = logits.stride(0)). allowed: 2-D int32
+        device tensor of mask words, one row per logit row or a single row shared by all."""
         assert logits.dim() == 2 and logits.stride(1) == 1
         r = Rows()
         r.d_logits = logits.data_ptr()
@@ -138,6 +140,11 @@ class HipSampler:
             r.d_history = history.data_ptr()
             r.history_ld = history.stride(0) if history.shape[0] > 1 else history.shape[1]
             r.d_history_len = history_len.data_ptr()
+        if allowed is not None:
+            assert allowed.dim() == 2 and allowed.stride(1) == 1 and allowed.element_size() == 4
+            assert allowed.shape[0] in (1, r.rows) and allowed.shape[1] * 32 >= r.n_vocab
+            r.d_allowed = allowed.data_ptr()
+            r.allowed_ld = 0 if allowed.shape[0] == 1 else allowed.stride(0)
         return r
 
     def sample(self, rows, params, uniforms, out):

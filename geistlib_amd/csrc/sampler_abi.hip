@@ -112,6 +112,9 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
                     HISTORY_MAX);
     if (pen && !(p->repetition_penalty > 0.0f))
         return fail(s, GEIST_HIP_E_INVALID_ARG, "repetition_penalty must be > 0");
+    if (r->d_allowed && r->allowed_ld != 0 && r->allowed_ld < (r->n_vocab + 31) / 32)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "allowed_ld %zu < %zu mask words per row",
+                    r->allowed_ld, (r->n_vocab + 31) / 32);
     L.rv.logits    = r->d_logits;
     L.rv.ld        = (long) r->ld;
     L.rv.n_vocab   = (int) r->n_vocab;
@@ -127,6 +130,8 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
     L.rv.pres      = pen ? p->presence_penalty : 0.0f;
     /* the soft-cap is monotone, so greedy rows skip it (head.c:145-149) */
     L.rv.softcap   = (p && stochastic && p->logit_softcap > 0.0f) ? p->logit_softcap : 0.0f;
+    L.rv.allowed    = r->d_allowed;
+    L.rv.allowed_ld = (long) r->allowed_ld;
     L.rows         = (int) r->rows;
     L.nv           = nv;
     L.pen          = pen;

@@ -443,6 +443,17 @@ __device__ __forceinline__ void load_raw(const RowView &rv, const float *__restr
     }
 }
 
+/* Allowed-token mask: the four mask bits of elements e .. e + 3 of a row (e a multiple of 4,
+ * below n_vocab), bit c set = element e + c may be sampled. Only called with rv.allowed set. */
+__device__ __forceinline__ uint32_t allowed_nibble(const RowView &rv, long row, int e) {
+    const uint32_t *m = rv.allowed + row * rv.allowed_ld;
+    return (m[e >> 5] >> (e & 31)) & 0xfu;
+}
+__device__ __forceinline__ bool allowed_at(const RowView &rv, long row, int e) {
+    const uint32_t *m = rv.allowed + row * rv.allowed_ld;
+    return (m[e >> 5] >> (e & 31)) & 1u;
+}
+
 /* The logit soft-cap, tanhf(x / cap) * cap (head.c:148-159), kept out of line: few models have
  * one, and glibc's tanhf is some two hundred instructions per element -- inlined at every site
  * it would multiply the size of every kernel and evict the code that does run from the

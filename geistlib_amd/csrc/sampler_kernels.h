@@ -32,6 +32,8 @@ struct RowView {
     float          rep, freq, pres;
     double         inv_rep; /* 1.0 / (double) rep, see penalise() */
     float          softcap; /* 0 = off */
+    const uint32_t *allowed;   /* NULL = no mask; bit e of a row's mask set = token e allowed */
+    long            allowed_ld; /* words between rows, 0 = one mask for all rows */
 };
 
 struct Launch {

@@ -83,18 +83,25 @@ template <int NV>
 __device__ __forceinline__ void remask_padding(const RowView &rv, int base, int end,
                                                float4 (&v)[NV]) {
     if (rv.softcap > 0.0f && end - base < NV * TPB * 4) {
+        /* elements of this thread's first group that lie inside the row (<= 0: none). The empty
+         * asm makes the value opaque: callers fetch inside loops, and the 4 * NV comparisons
+         * would otherwise be hoisted out of them into as many scalar register pairs. */
+        int lim = end - base - 4 * (int) threadIdx.x;
+        asm volatile("" : "+v"(lim));
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            const int e = base + 4 * (j * TPB + (int) threadIdx.x);
-            if (e + 0 >= end) v[j].x = -INFINITY;
-            if (e + 1 >= end) v[j].y = -INFINITY;
-            if (e + 2 >= end) v[j].z = -INFINITY;
-            if (e + 3 >= end) v[j].w = -INFINITY;
+            const int l = lim - 4 * j * TPB;
+            v[j].x = l > 0 ? v[j].x : -INFINITY;
+            v[j].y = l > 1 ? v[j].y : -INFINITY;
+            v[j].z = l > 2 ? v[j].z : -INFINITY;
+            v[j].w = l > 3 ? v[j].w : -INFINITY;
         }
     }
 }
 
-template <int NV, bool PEN>
+/* MASK = false compiles the allowed-token mask out (for callers that know rv.allowed is NULL and
+ * are short of scalar registers). */
+template <int NV, bool PEN, bool MASK = true>
 __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_rows, int base,
                                             int end, uint32_t *cnt16, float4 (&v)[NV]) {
     const float *rowp = rv.logits + (long) row * rv.ld;
@@ -112,6 +119,19 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_ro
         apply_transform<NV>(rv, nullptr, v);
     }
     remask_padding<NV>(rv, base, end, v);
+    if (MASK && rv.allowed) { /* forbidden tokens weigh nothing, whatever the transforms made */
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + (int) threadIdx.x);
+            if (e < end) {
+                const uint32_t ok = allowed_nibble(rv, row, e);
+                v[j].x = (ok & 1u) ? v[j].x : -INFINITY;
+                v[j].y = (ok & 2u) ? v[j].y : -INFINITY;
+                v[j].z = (ok & 4u) ? v[j].z : -INFINITY;
+                v[j].w = (ok & 8u) ? v[j].w : -INFINITY;
+            }
+        }
+    }
 }
 
 /* Row maximum from the per-chunk results; every thread returns the same packed value. */
@@ -580,7 +600,7 @@ struct GeneralShared {
     int n;
 };
 
-template <int NV, bool PEN>
+template <int NV, bool PEN, bool MASK = true>
 __device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int k_want, uint64_t *spack,
                                 int spack_cap, uint32_t *cnt16, GeneralShared &gs_) {
     constexpr int TILE = NV * TPB * 4;
@@ -596,7 +616,7 @@ __device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int 
         __syncthreads();
         for (int base = 0; base < n; base += TILE) {
             const int end = base + TILE < n ? base + TILE : n;
-            fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, cnt16, v);
+            fetch_chunk<NV, PEN, MASK>(rv, row, (int) gridDim.x, base, end, cnt16, v);
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
                 const int e = base + 4 * (j * TPB + tid);
@@ -624,7 +644,7 @@ __device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int 
     int ties_before = 0;
     for (int base = 0; base < n; base += TILE) {
         const int end = base + TILE < n ? base + TILE : n;
-        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, cnt16, v);
+        fetch_chunk<NV, PEN, MASK>(rv, row, (int) gridDim.x, base, end, cnt16, v);
         int ties_here = 0;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
@@ -719,7 +739,7 @@ struct FinalArgs {
  * Returns true when the row has to take the general path instead (fewer than k real maxima,
  * long runs of equal values); otherwise k_out entries lie sorted in s_pack.
  * ========================================================================================== */
-template <int NV, bool PEN, int KPT>
+template <int NV, bool PEN, int KPT, bool MASK>
 __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArgs &a, int row,
                                                uint8_t *slot, uint32_t *s_mx, int *s_selid,
                                                uint32_t *s_pcnt, uint64_t *s_m, uint64_t *s_pack,
@@ -899,10 +919,12 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
             for (int c = 0; c < 4; ++c)
                 x4[c] = softcap1(x4[c], rv.softcap);
         }
-        const int nvalid = e1[q] - e0[q]; /* 4 but at the row's end */
+        const int      nvalid = e1[q] - e0[q]; /* 4 but at the row's end */
+        const uint32_t ok     = (MASK && rv.allowed) ? allowed_nibble(rv, row, e0[q]) : 0xfu;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            if (x4[c] >= bound && c < nvalid) { /* (a NaN fails the comparison: keys are > 0) */
+            /* (a NaN fails the comparison: keys are > 0) */
+            if (x4[c] >= bound && c < nvalid && ((ok >> c) & 1u)) {
                 ck[q][c] = f2key(x4[c]);
                 ++n_keep;
             }
@@ -973,8 +995,9 @@ __global__ __launch_bounds__(TPB) void k_final_argmax(RowView rv, FinalArgs a) {
     if (threadIdx.x == 0) {
         const float first = rv.logits[(long) row * rv.ld];
         /* a NaN at index 0 is never displaced by the strict '>' of the reference; after the
-         * transforms it stays NaN, so the raw value decides */
-        a.out[row] = (first != first) ? 0 : (int32_t) best_idx(b);
+         * transforms it stays NaN, so the raw value decides (unless token 0 is forbidden) */
+        const bool nan0 = first != first && (!rv.allowed || allowed_at(rv, row, 0));
+        a.out[row]      = nan0 ? 0 : (int32_t) best_idx(b);
     }
 }
 
@@ -1159,7 +1182,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
 /* top-k (sampler.c:178-228) and the chain behind it: select from the row's thread maxima, then
  * gather; rows the shortcut cannot serve (masked rows full of -inf, all-equal rows, tiny or huge
  * vocabularies) select over the whole row in place. */
-template <int NV, bool PEN>
+template <int NV, bool PEN, bool MASK>
 __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
     __shared__ uint64_t      s_tab[32];
     __shared__ GeneralShared s_gs;
@@ -1179,14 +1202,15 @@ __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
     int         k       = 0;
     bool        general = true;
     if (C <= 16)
-        general = topk_from_tmax<NV, PEN, 16>(rv, a, row, s_big, s_mx, s_selid, s_pcnt, s_m,
+        general = topk_from_tmax<NV, PEN, 16, MASK>(rv, a, row, s_big, s_mx, s_selid, s_pcnt, s_m,
                                               s_pack, &s_n, &s_n2, k);
     else if (C <= TMAX_LDS / TPB)
-        general = topk_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, s_big, s_mx, s_selid, s_pcnt,
+        general = topk_from_tmax<NV, PEN, TMAX_LDS / TPB, MASK>(rv, a, row, s_big, s_mx, s_selid,
+                                                                s_pcnt,
                                                           s_m, s_pack, &s_n, &s_n2, k);
     if (general) {
         __syncthreads();
-        k = topk_row_general<NV, PEN>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
+        k = topk_row_general<NV, PEN, MASK>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
     }
     GS_MARK(6);
     /* k <= TOPK_FAST_MAX = 128: the tail runs on one wavefront without barriers */
@@ -1539,8 +1563,10 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
             k_final_temperature<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
         else if (f.mode == FINAL_SORTED)
             k_final_sorted<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
+        else if (L.rv.allowed)
+            k_final_topk<GS_NV, GS_PEN, true><<<grid, block, 0, L.stream>>>(L.rv, a);
         else
-            k_final_topk<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(L.rv, a);
+            k_final_topk<GS_NV, GS_PEN, false><<<grid, block, 0, L.stream>>>(L.rv, a);
     });
 }
 

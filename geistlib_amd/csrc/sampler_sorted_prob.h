@@ -283,6 +283,8 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
                 }
                 if (rv.softcap > 0.0f)
                     x = softcap1(x, rv.softcap);
+                if (rv.allowed && !allowed_at(rv, row, e0[q] + c))
+                    continue;
                 if (x >= bound) { /* the logit for now; its probability below, one per thread */
                     const int at = atomicAdd(s_n2, 1);
                     if (at < TPB)

@@ -52,15 +52,25 @@ int geist_hip_sampler_set_stream(geist_hip_sampler *s, void *stream);
 
 /* A batch of logit rows in device memory. Row r starts at d_logits + r * ld.
  * The optional token history drives the penalties: row r owns d_history[r * history_ld ..
- * + d_history_len[r]) ; ids outside [0, n_vocab) are ignored. */
+ * + d_history_len[r]) ; ids outside [0, n_vocab) are ignored.
+ * The optional allowed-token mask is the device form of constrained decoding, which the
+ * reference leaves to a runtime that reads the logits back, masks what its grammar forbids and
+ * samples itself (docs/API_CONTRACT.md:35-44; geist_session_peek_logits,
+ * include/geist_util.h:195-211): bit (e % 32) of word d_allowed[r * allowed_ld + e / 32] set =
+ * token e may be sampled in row r; a forbidden token's logit is -inf, after the penalties and
+ * the soft-cap (peek_logits hands out capped values), in every mode, greedy included.
+ * allowed_ld = 0: one mask of (n_vocab + 31) / 32 words shared by all rows. Every row must
+ * allow at least one token with a logit above -inf. */
 struct geist_hip_rows {
-    const float   *d_logits;
-    size_t         ld;
-    size_t         rows;
-    size_t         n_vocab;
-    const int32_t *d_history;     /* NULL = no history */
-    size_t         history_ld;
-    const int32_t *d_history_len; /* rows entries */
+    const float    *d_logits;
+    size_t          ld;
+    size_t          rows;
+    size_t          n_vocab;
+    const int32_t  *d_history;     /* NULL = no history */
+    size_t          history_ld;
+    const int32_t  *d_history_len; /* rows entries */
+    const uint32_t *d_allowed;     /* NULL = every token allowed */
+    size_t          allowed_ld;    /* words between the masks of consecutive rows; 0 = shared */
 };
 
 /* Sampling configuration for one call. The first four fields are the sampler fields of

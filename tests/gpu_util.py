@@ -11,8 +11,18 @@ def to_dev(a, torch):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+def pack_allowed(allowed):
+    """bool [rows, n] -> int32 mask words [rows, ceil(n / 32)], bit e % 32 of word e / 32."""
+    rows, n = allowed.shape
+    words = (n + 31) // 32
+    bits = np.zeros((rows, words * 32), dtype=np.uint8)
+    bits[:, :n] = allowed
+    packed = np.packbits(bits.reshape(rows, words, 32), axis=-1, bitorder="little")
+    return np.ascontiguousarray(packed).view(np.uint32).reshape(rows, words).view(np.int32)
+
+
 def run_rows(sampler, torch, logits, uniforms, params, history=None, history_len=None,
-             pad=0, lead=0):
+             pad=0, lead=0, allowed=None):
     """pad: extra elements between rows; lead: elements before the first row (an unaligned base).
     Both gaps hold a huge logit, so a read outside a row changes the result."""
     from geistlib_amd import HipSampler
@@ -29,7 +39,8 @@ def run_rows(sampler, torch, logits, uniforms, params, history=None, history_len
     d_h = to_dev(history, torch) if history is not None else None
     d_hl = to_dev(history_len, torch) if history_len is not None else None
     out = torch.full((logits.shape[0],), -7, dtype=torch.int32, device="cuda")
-    rows = HipSampler.rows(d_logits, d_h, d_hl)
+    d_a = to_dev(pack_allowed(allowed), torch) if allowed is not None else None
+    rows = HipSampler.rows(d_logits, d_h, d_hl, allowed=d_a)
     sampler.sample(rows, params, d_u, out)
     sampler.sync()
     return out.cpu().numpy()

@@ -65,8 +65,18 @@ def _case(g):
     cap = float(g.choice([0.0, 0.0, 30.0, 5.0]))
     u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
     pad, lead = int(g.choice([0, 0, 1, 3, 4, 64])), int(g.choice([0, 0, 1, 2, 4]))
-    return x, u, prm, pen, cap, pad, lead, (f"{kind} rows={rows} n={n} {mode} {prm} "
-                                            f"pen={pen is not None} cap={cap} pad={pad} lead={lead}")
+    allowed = None
+    if g.random() < 0.35:                         # a grammar mask: from a handful to most tokens
+        density = float(g.choice([0.001, 0.05, 0.5, 0.97]))
+        shared = g.random() < 0.3
+        allowed = g.random((1 if shared else rows, n)) < density
+        allowed[:, int(g.integers(0, n))] = True
+        dens = density
+    else:
+        dens = None
+    return x, u, prm, pen, cap, pad, lead, allowed, (
+        f"{kind} rows={rows} n={n} {mode} {prm} pen={pen is not None} cap={cap} pad={pad} "
+        f"lead={lead} mask={dens}")
 
 
 @pytest.mark.parametrize("seed", range(16))
@@ -75,14 +85,14 @@ def test_random_configurations_match_oracle(hs, oracle, seed):
     g = np.random.default_rng(1000 + seed)
     near_total = 0
     for case in range(14):
-        x, u, prm, pen, cap, pad, lead, what = _case(g)
+        x, u, prm, pen, cap, pad, lead, allowed, what = _case(g)
         print(f"seed {seed} case {case}: {what}", flush=True)
         kw = dict(prm)
         if pen is not None:
             kw.update(rep=pen["rep"], freq=pen["freq"], pres=pen["pres"])
         p = SampleParams.make(softcap=cap, **kw)
         got = run_rows(hs, torch, x, u, p, None if pen is None else pen["hist"],
-                       None if pen is None else pen["hl"], pad=pad, lead=lead)
+                       None if pen is None else pen["hl"], pad=pad, lead=lead, allowed=allowed)
         res = []
         for r in range(x.shape[0]):
             row = x[r]
@@ -91,6 +101,9 @@ def test_random_configurations_match_oracle(hs, oracle, seed):
                                        pen["pres"])
             if cap > 0 and prm["temperature"] > 0:
                 row = oracle.softcap(row, cap)
+            if allowed is not None:               # after the penalties and the cap
+                row = np.where(allowed[r if allowed.shape[0] > 1 else 0], row, -np.inf)
+                row = row.astype(np.float32)
             if prm["temperature"] <= 0:
                 res.append((oracle.argmax(row), None))
             else:

@@ -704,3 +704,54 @@ def test_ngram_drafter_argument_errors(hs):
     for k_max in (0, 17, 5):                        # 5 > out_ld = 4
         with pytest.raises(GeistHipError):
             hs.propose_drafts_ngram(h, hl, sd, k_max, 4, out, c, c)
+
+
+# --------------------------------------------------------------------- allowed-token mask
+@pytest.mark.parametrize("mode", ["argmax", "temperature", "top_k", "top_p", "min_p", "chain"])
+def test_allowed_mask_equals_minus_inf_after_the_transforms(hs, oracle, mode):
+    """Constrained decoding on the device: a forbidden token weighs nothing. Equal to sampling
+    from the row with -inf written over the forbidden logits AFTER penalties and soft-cap (the
+    reference's runtime masks what geist_session_peek_logits hands out, which is capped)."""
+    from gpu_util import pack_allowed
+    rows, n, cap = 10, 50257, 8.0
+    g = np.random.default_rng(41)
+    x = (g.standard_normal((rows, n)) * 3).astype(np.float32)
+    u = (g.integers(0, 1 << 24, rows) / np.float32(1 << 24)).astype(np.float32)
+    hist = g.integers(0, n, (rows, 64)).astype(np.int32)
+    hl = np.full(rows, 64, dtype=np.int32)
+    allowed = g.random((rows, n)) < np.array([1e-4, 1e-3, 0.01, 0.1, 0.5, 0.9, 0.99, 1.0, 0.3,
+                                              0.3])[:, None]
+    allowed[np.arange(rows), g.integers(0, n, rows)] = True
+    allowed[8, np.argmax(x[8])] = False               # the favourite is forbidden
+    allowed[9, :] = False
+    allowed[9, 12345] = True                          # a single choice
+    x[7, 0] = np.nan
+    allowed[6, 0] = False
+    x[6, 0] = np.nan                                  # a forbidden NaN at index 0 does not win
+    kw = dict(temperature=0.0 if mode == "argmax" else 0.9,
+              top_k=40 if mode in ("top_k", "chain") else 0,
+              top_p=0.9 if mode in ("top_p", "chain") else 1.0,
+              min_p=0.02 if mode in ("min_p", "chain") else 0.0)
+    if mode != "argmax":
+        x[7, 0] = 0.5                                 # NaN rows are defined for argmax only
+    got = run_rows(hs, torch, x, u, P(softcap=cap, rep=1.2, freq=0.1, pres=0.1, **kw), hist, hl,
+                   allowed=allowed)
+    res = []
+    for r in range(rows):
+        row = oracle.penalties(x[r], hist[r], 1.2, 0.1, 0.1)
+        if mode != "argmax":
+            row = oracle.softcap(row, cap)
+        row = np.where(allowed[r], row, -np.inf).astype(np.float32)
+        res.append((oracle.argmax(row), None) if mode == "argmax"
+                   else oracle.chain_u(row, float(u[r]), **kw))
+    near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"mask {mode}")
+    assert near <= 1
+    assert all(allowed[r, got[r]] for r in range(rows))
+    assert got[9] == 12345
+    # one mask shared by every row (allowed_ld = 0)
+    shared = allowed[4:5]
+    got = run_rows(hs, torch, x[:6], u[:6], P(**kw), allowed=shared)
+    for r in range(6):
+        row = np.where(shared[0], x[r], -np.inf).astype(np.float32)
+        want = oracle.argmax(row) if mode == "argmax" else oracle.chain_u(row, float(u[r]), **kw)[0]
+        assert got[r] == want, (mode, r)
