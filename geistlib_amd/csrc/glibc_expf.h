@@ -96,15 +96,14 @@ GEIST_HD float geist_expf_glibc(float x, const uint64_t *tab) {
     return (float) y;
 }
 
-/* The same function for the sampler's arguments, (l - max) * inv_t <= 0, without branches or
- * selects: arguments below -104 are raised to -104, where the polynomial's result already rounds
- * to 0 as every smaller argument's does (the underflow edge -103.972 is where the rounding of
- * the same expression flips), and a NaN runs through the arithmetic and comes out a NaN. Positive
- * arguments take the general function. Equal to geist_expf_glibc() on every input (checked
- * exhaustively together with it). */
-GEIST_HD float geist_expf_glibc_nonpos(float x, const uint64_t *tab) {
-    if (__builtin_expect(x > 0.0f, 0))
-        return geist_expf_glibc(x, tab);
+/* The same function for arguments x <= 0 (and NaN), without branches or selects, so that the
+ * compiler can interleave the evaluations of many elements: arguments below -104 are raised to
+ * -104, where the polynomial's result already rounds to 0 as every smaller argument's does (the
+ * underflow edge -103.972 is where the rounding of the same expression flips), and a NaN runs
+ * through the arithmetic and comes out a NaN. Equal to geist_expf_glibc() on every such input
+ * (checked exhaustively). A positive argument is outside the contract: the sampler's arguments
+ * are (l - max) * inv_t with max taken over the same values. */
+GEIST_HD float geist_expf_glibc_le0(float x, const uint64_t *tab) {
     const double inv_ln2_n = 0x1.71547652b82fep+0 * 32.0;
     const double shift     = 0x1.8p+52;
     const double c0        = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
@@ -117,17 +116,26 @@ GEIST_HD float geist_expf_glibc_nonpos(float x, const uint64_t *tab) {
     const uint64_t ki = geist_double_as_u64(kd);
     kd -= shift;
     const double   r  = __builtin_fma(inv_ln2_n, xd, -kd);
-    /* ki << 47 only reaches the high word: add (low word of ki) << 15 there */
+    /* ki << 47 only reaches the high word: add (low word of ki) << 15 there, in 32-bit
+     * arithmetic (one shift-add on the device) */
+    typedef uint32_t geist_u32x2 __attribute__((vector_size(8)));
     const uint32_t kl = (uint32_t) ki;
-    const uint64_t t0 = tab[kl & 31];
-    const uint64_t t  = (t0 & 0xffffffffull) | ((uint64_t) ((uint32_t) (t0 >> 32) + (kl << 15)) << 32);
-    const double   s  = geist_u64_as_double(t);
+    geist_u32x2    w  = __builtin_bit_cast(geist_u32x2, tab[kl & 31]);
+    w[1] += kl << 15;
+    const double s = __builtin_bit_cast(double, w);
     const double   z  = __builtin_fma(c0, r, c1);
     const double   r2 = r * r;
     double         y  = __builtin_fma(c2, r, 1.0);
     y                 = __builtin_fma(z, r2, y);
     y                 = y * s;
     return (float) y;
+}
+
+/* Any argument: positive ones take the general function. */
+GEIST_HD float geist_expf_glibc_nonpos(float x, const uint64_t *tab) {
+    if (__builtin_expect(x > 0.0f, 0))
+        return geist_expf_glibc(x, tab);
+    return geist_expf_glibc_le0(x, tab);
 }
 
 #endif /* GEIST_GLIBC_EXPF_H */

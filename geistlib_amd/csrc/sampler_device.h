@@ -500,6 +500,45 @@ __device__ __forceinline__ void apply_transform(const RowView &rv, const uint32_
     }
 }
 
+/* The transforms of one float4 group of a chunk in registers -- elements base + off .. + 3,
+ * off = 4 * (j * TPB + tid) -- for kernels that work through a chunk group by group while the
+ * later groups' loads are still in flight: penalties from the count table, soft-cap, chunk
+ * padding back to -inf, allowed-token mask. The same values as fetch_chunk() produces. */
+template <bool PEN, bool EXTRAS = true>
+__device__ __forceinline__ void transform_group(const RowView &rv, long row, const uint32_t *cnt16,
+                                                int off, int base, int end, float4 &q) {
+    if (PEN) {
+        const uint2 w = *reinterpret_cast<const uint2 *>(cnt16 + (off >> 1));
+        if (w.x | w.y) {
+            if (w.x & 0xffffu)
+                q.x = penalise(q.x, w.x & 0xffffu, rv.rep, rv.inv_rep, rv.freq, rv.pres);
+            if (w.x >> 16)
+                q.y = penalise(q.y, w.x >> 16, rv.rep, rv.inv_rep, rv.freq, rv.pres);
+            if (w.y & 0xffffu)
+                q.z = penalise(q.z, w.y & 0xffffu, rv.rep, rv.inv_rep, rv.freq, rv.pres);
+            if (w.y >> 16)
+                q.w = penalise(q.w, w.y >> 16, rv.rep, rv.inv_rep, rv.freq, rv.pres);
+        }
+    }
+    if (!EXTRAS) /* the caller knows: no soft-cap, no padding, no mask */
+        return;
+    if (rv.softcap > 0.0f) {
+        q           = softcap4(q, rv.softcap);
+        const int l = end - base - off; /* elements of the group inside the row */
+        q.x         = l > 0 ? q.x : -__builtin_inff();
+        q.y         = l > 1 ? q.y : -__builtin_inff();
+        q.z         = l > 2 ? q.z : -__builtin_inff();
+        q.w         = l > 3 ? q.w : -__builtin_inff();
+    }
+    if (rv.allowed && base + off < end) {
+        const uint32_t ok = allowed_nibble(rv, row, base + off);
+        q.x               = (ok & 1u) ? q.x : -__builtin_inff();
+        q.y               = (ok & 2u) ? q.y : -__builtin_inff();
+        q.z               = (ok & 4u) ? q.z : -__builtin_inff();
+        q.w               = (ok & 8u) ? q.w : -__builtin_inff();
+    }
+}
+
 /* max of three floats in one instruction. Unlike fmaxf() no canonicalising self-max is emitted
  * per operand; a quiet NaN operand is ignored (a signalling NaN may come back quieted, which
  * only makes the caller keep more candidates). */

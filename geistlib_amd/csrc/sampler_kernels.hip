@@ -149,31 +149,32 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
  * Optionally records p at one token of the row (spec verification needs p(x_j)).
  * ========================================================================================== */
-template <int NV, bool PEN, bool LISTM, bool SLABS>
-__global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
-                                                      const uint64_t *__restrict__ chunk_best,
-                                                      double *__restrict__ chunk_sum,
-                                                      double *__restrict__ slab_sum,
-                                                      const int32_t *__restrict__ probe_token,
-                                                      int probe_L, float *__restrict__ probe_p,
-                                                      CandSpace list, int zb_list) {
-    static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
-    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ uint64_t s_red[NWAVES];
-    __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
-    __shared__ uint64_t s_tab[32];
-    __shared__ int      s_listed, s_base;
-    int                 row, chunk;
-    xcd_row_chunk(row, chunk);
+/* The work of one workgroup. PLAIN: a full, 16-byte aligned chunk without soft-cap or
+ * allowed-token mask -- the common case, kept free of everything that would make the compiler
+ * wait for all of the chunk's loads before the first group is summed (a merge with the
+ * element-wise loads of a ragged chunk, a branch around a mask load). */
+template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN>
+__device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chunk, int n_rows,
+                                             int base, int end, float inv_t,
+                                             const uint64_t *__restrict__ chunk_best,
+                                             double *__restrict__ chunk_sum,
+                                             double *__restrict__ slab_sum,
+                                             const int32_t *__restrict__ probe_token, int probe_L,
+                                             float *__restrict__ probe_p, const CandSpace &list,
+                                             int zb_list, uint32_t *s_cnt16, double *s_sum,
+                                             const uint64_t *s_tab, int *s_listed, int *s_base) {
     const int tid = threadIdx.x;
-    if (tid < 32)
-        s_tab[tid] = g_expf_tab[tid];
-    int base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
-    const float mx = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
-
+    /* Order of the loads: the chunk results of the row (each wavefront reduces them for itself,
+     * no barrier), the probed token, the history, then the chunk. The groups of the chunk are
+     * then transformed and summed one by one, each as soon as its own load has arrived: a
+     * barrier with a full fence, or a transform over the whole chunk first, would keep the
+     * arithmetic waiting for the last load, and the launch would alternate between a phase
+     * that only loads and one that only computes. */
+    uint64_t bb = 0;
+    for (int c = tid & (WAVE - 1); c < rv.n_chunks; c += WAVE) {
+        const uint64_t p = chunk_best[(long) row * rv.n_chunks + c];
+        bb               = p > bb ? p : bb;
+    }
     /* spec verification: target row s*(L+1)+j is probed at draft token j of sequence s */
     int tok = -1;
     if (probe_token) {
@@ -181,8 +182,29 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
         if (j < probe_L)
             tok = probe_token[(long) (row / (probe_L + 1)) * probe_L + j];
     }
+    HistPrefetch pf;
+    if (PEN)
+        pf = history_prefetch(rv, row, n_rows);
+    float4       v[NV];
+    const float *rowp = rv.logits + (long) row * rv.ld;
+    if (PLAIN) {
+        const float4 *p = reinterpret_cast<const float4 *>(rowp + base) + tid;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            v[j] = p[j * TPB];
+    } else {
+        load_raw<NV>(rv, rowp, base, end, v);
+    }
     if (LISTM && tid == 0)
-        s_listed = 0;
+        *s_listed = 0;
+    if (PEN) {
+        history_clear<NV * TPB * 4>(s_cnt16);
+        history_count(rv, row, pf, base, end, s_cnt16);
+    } else {
+        lds_barrier(); /* publishes s_tab (the history's barriers do when PEN) */
+    }
+    const float mx = key2f(best_key(wave_max_u64(bb)));
+
     double      acc  = 0.0;
     double      accs[SLABS ? NV : 1];
     uint32_t    mask = 0u;
@@ -191,11 +213,13 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
      * bin, so the loop carries no bound tests */
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        double a4 = 0.0;
+        transform_group<PEN, !PLAIN>(rv, row, s_cnt16, 4 * (j * TPB + tid), base, end, v[j]);
+        double a4;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
-            a4 += (double) geist_expf_glibc_nonpos(arg, s_tab);
+            const float  arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
+            const double p   = (double) geist_expf_glibc_le0(arg, s_tab);
+            a4               = c == 0 ? p : a4 + p;
             if (LISTM)
                 mask |= (uint32_t) (arg > list_thr) << (4 * j + c);
         }
@@ -203,6 +227,17 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             accs[j] = a4;
         else
             acc += a4;
+        /* four evaluations in flight are enough to cover the latencies; left alone, the
+         * compiler interleaves all 4 * NV of them and the registers that takes cost most of the
+         * occupancy. The empty asm ties the next group's inputs to this group's sum. */
+        if (j + 1 < NV) {
+            if (SLABS)
+                asm volatile("" : "+v"(accs[j]), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
+                                  "+v"(v[j + 1].z), "+v"(v[j + 1].w));
+            else
+                asm volatile("" : "+v"(acc), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
+                                  "+v"(v[j + 1].z), "+v"(v[j + 1].w));
+        }
     }
     if (tok >= base && tok < end) {
         /* the thread that holds the probed element evaluates it once more */
@@ -214,7 +249,7 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             for (int jj = 0; jj < NV; ++jj)
                 if (jj == j)
                     x = f4_get(v[jj], off & 3);
-            probe_p[row] = geist_expf_glibc_nonpos(softmax_arg(x, mx, inv_t), s_tab);
+            probe_p[row] = geist_expf_glibc_le0(softmax_arg(x, mx, inv_t), s_tab);
         }
     }
     if (SLABS) {
@@ -230,18 +265,18 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             chunk_sum[at] = acc;
         }
     } else {
-        acc = block_sum_f64(acc, s_sum); /* (its barriers publish s_listed = 0) */
+        acc = block_sum_f64(acc, s_sum);
         if (tid == 0)
             chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
     }
     if (LISTM) {
         /* places in the row's list: one LDS counter for the workgroup, one global add for all */
-        int pos = wave_reserve(__popc(mask), &s_listed);
+        int pos = wave_reserve(__popc(mask), s_listed);
         __syncthreads();
         if (tid == 0)
-            s_base = s_listed ? atomicAdd(&list.count[row], s_listed) : 0;
+            *s_base = *s_listed ? atomicAdd(&list.count[row], *s_listed) : 0;
         __syncthreads();
-        pos += s_base;
+        pos += *s_base;
         uint32_t *ck = list.key + (long) row * CAND_CAP;
         uint32_t *ci = list.idx + (long) row * CAND_CAP;
 #pragma unroll
@@ -251,8 +286,11 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             for (int c = 0; c < 4; ++c) {
                 if ((mask >> (4 * j + c)) & 1u) {
                     if (pos < CAND_CAP) {
-                        ck[pos] = __float_as_uint(
-                            geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab));
+                        float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
+                        /* (opaque, so that the evaluation stays under its condition: few
+                         * elements are listed) */
+                        asm volatile("" : "+v"(arg));
+                        ck[pos] = __float_as_uint(geist_expf_glibc_le0(arg, s_tab));
                         ci[pos] = (uint32_t) (e + c);
                     }
                     ++pos;
@@ -260,6 +298,39 @@ __global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
             }
         }
     }
+}
+
+template <int NV, bool PEN, bool LISTM, bool SLABS>
+__global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
+                                                      const uint64_t *__restrict__ chunk_best,
+                                                      double *__restrict__ chunk_sum,
+                                                      double *__restrict__ slab_sum,
+                                                      const int32_t *__restrict__ probe_token,
+                                                      int probe_L, float *__restrict__ probe_p,
+                                                      CandSpace list, int zb_list) {
+    static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
+    __shared__ uint64_t s_tab[32];
+    __shared__ int      s_listed, s_base;
+    int                 row, chunk;
+    xcd_row_chunk(row, chunk);
+    if (threadIdx.x < 32)
+        s_tab[threadIdx.x] = g_expf_tab[threadIdx.x];
+    int base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
+                       rv.allowed == nullptr;
+    if (plain)
+        expsum_chunk<NV, PEN, LISTM, SLABS, true>(rv, row, chunk, (int) gridDim.y, base, end, inv_t,
+                                                  chunk_best, chunk_sum, slab_sum, probe_token,
+                                                  probe_L, probe_p, list, zb_list, s_cnt16, s_sum,
+                                                  s_tab, &s_listed, &s_base);
+    else
+        expsum_chunk<NV, PEN, LISTM, SLABS, false>(rv, row, chunk, (int) gridDim.y, base, end,
+                                                   inv_t, chunk_best, chunk_sum, slab_sum,
+                                                   probe_token, probe_L, probe_p, list, zb_list,
+                                                   s_cnt16, s_sum, s_tab, &s_listed, &s_base);
 }
 
 /* ============================================================================================
@@ -362,7 +433,7 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
     }
     __syncthreads();
     const float l0 = key2f(best_key(spack[0]));
-#define GS_P(i) geist_expf_glibc_nonpos(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), fs.tab)
+#define GS_P(i) geist_expf_glibc_le0(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), fs.tab)
 
     double part = 0.0;
     for (int i = lo; i < hi; ++i)
@@ -451,7 +522,7 @@ __device__ int finish_sorted_wave(int n, const uint64_t *spack, float inv_t, flo
 #pragma unroll
     for (int t = 0; t < IPT; ++t) {
         const int i = IPT * lane + t;
-        w[t] = i < n ? geist_expf_glibc_nonpos(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), tab)
+        w[t] = i < n ? geist_expf_glibc_le0(softmax_arg(key2f(best_key(spack[i])), l0, inv_t), tab)
                      : 0.0f;
         part += (double) w[t];
     }
@@ -1064,7 +1135,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */
         if (tid == 0) {
             const int   B      = a.zb_min_p;
-            const float p_out  = geist_expf_glibc_nonpos(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float p_out  = geist_expf_glibc_le0(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
             const float pn_out = (float) ((double) p_out / sum);
             a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
             a.cand.row_bound[row] = B;
@@ -1167,7 +1238,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
             /* an element outside the list has z >= (B + 1) / ZBIN_PER_NAT (the product in zbin()
              * is exact), so its p is at most expf of minus that; one step up covers any
              * non-monotonic last bit of expf or of the division */
-            const float p_out  = geist_expf_glibc_nonpos(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
+            const float p_out  = geist_expf_glibc_le0(-(float) (B + 1) / (float) ZBIN_PER_NAT, s_tab);
             const float pn_out = (float) ((double) p_out / sum);
             a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
             a.cand.row_bound[row] = B;
@@ -1279,7 +1350,7 @@ __global__ __launch_bounds__(TPB) void k_write_probs(RowView rv, float inv_t,
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             if (e + c < end) {
-                const float p = geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
                 out[e + c]    = (float) ((double) p / tot);
             }
         }

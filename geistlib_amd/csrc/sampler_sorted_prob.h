@@ -157,7 +157,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     const uint32_t mkey = f2key(mxf);
     float          wt   = 0.0f;
     if (mkey)
-        wt = (float) ((double) geist_expf_glibc_nonpos(softmax_arg(mxf, mx, a.inv_t), tab) / sum);
+        wt = (float) ((double) geist_expf_glibc_le0(softmax_arg(mxf, mx, a.inv_t), tab) / sum);
     s_mx[tid] = mkey;
     s_wt[tid] = wt;
     __syncthreads();
@@ -302,7 +302,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
         const uint64_t ent = s_m[tid];
         const float    x   = __uint_as_float((uint32_t) (ent >> 32));
         const float    pn  =
-            (float) ((double) geist_expf_glibc_nonpos(softmax_arg(x, mx, a.inv_t), tab) / sum);
+            (float) ((double) geist_expf_glibc_le0(softmax_arg(x, mx, a.inv_t), tab) / sum);
         s_m[tid] = pack_best(__float_as_uint(pn), (uint32_t) ent);
     }
     __syncthreads();
@@ -745,7 +745,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(RowView rv, float inv_t,
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (e + c < end) {
-                    const float p = geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
                     pn[e + c]     = (float) ((double) p / tot);
                 }
             }
@@ -847,7 +847,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
         const int gbase = s_base;
         for (int i = tid; i < n_blk; i += TPB) {
             if (gbase + i < CAND_CAP) {
-                const float p   = geist_expf_glibc_nonpos(s_arg[i], s_tab);
+                const float p   = geist_expf_glibc_le0(s_arg[i], s_tab);
                 ck[gbase + i]   = __float_as_uint((float) ((double) p / tot));
                 ci[gbase + i]   = s_id[i];
             }
@@ -863,7 +863,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
                 if ((mask >> (4 * j + c)) & 1u) {
                     if (pos < CAND_CAP) {
                         const float p =
-                            geist_expf_glibc_nonpos(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                            geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
                         ck[pos] = __float_as_uint((float) ((double) p / tot));
                         ci[pos] = (uint32_t) (e + c);
                     }

@@ -26,7 +26,7 @@ __device__ __forceinline__ void slab_weights(const float4 &v, const float4 &qv, 
     for (int c = 0; c < 4; ++c) {
         float x = 0.0f;
         if (e + c < end) {
-            const float p = geist_expf_glibc_nonpos(softmax_arg(f4_get(v, c), mx, inv_t), tab);
+            const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v, c), mx, inv_t), tab);
             if (RESID) {
                 const float r = __fsub_rn((float) ((double) p / sum), f4_get(qv, c));
                 x             = r > 0.0f ? r : 0.0f;

@@ -20,15 +20,19 @@ int main(int argc, char **argv) {
         float          x;
         memcpy(&x, &u, 4);
         const float want = expf(x), got = geist_expf_glibc(x, TAB),
-                    got2 = geist_expf_glibc_nonpos(x, TAB); /* the branch-free variant */
-        uint32_t    uw, ug, ug2;
+                    got2 = geist_expf_glibc_nonpos(x, TAB),
+                    /* the branch-free variant, defined for x <= 0 and NaN */
+                    got3 = x > 0.0f ? want : geist_expf_glibc_le0(x, TAB);
+        uint32_t    uw, ug, ug2, ug3;
         memcpy(&uw, &want, 4);
         memcpy(&ug, &got, 4);
         memcpy(&ug2, &got2, 4);
+        memcpy(&ug3, &got3, 4);
         const bool both_nan  = want != want && got != got;
         const bool both_nan2 = want != want && got2 != got2;
+        const bool both_nan3 = want != want && got3 != got3;
         ++total;
-        if ((uw != ug && !both_nan) || (uw != ug2 && !both_nan2))
+        if ((uw != ug && !both_nan) || (uw != ug2 && !both_nan2) || (uw != ug3 && !both_nan3))
             ++bad;
     }
     printf("%ld %ld\n", bad, total);
