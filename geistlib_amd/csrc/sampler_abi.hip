@@ -392,6 +392,10 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     const int zb_m    = zbin_of_min_p(rs.min_p);
     f.cand            = s->cand;
     f.minp_listed     = rs.use_m && zb_m < ZBINS - 1;
+    /* A min-p of a few percent keeps the list short on any plausible row, and the walk can follow
+     * the exp-sum pass at once. Below that a flat row may overflow the list, and the row-final
+     * kernel should get the chance to bound it by top-p instead. */
+    f.minp_direct     = f.minp_listed && rs.min_p >= 0.02f;
     if (!stream_only(s))
         launch_tmax_scan(L, s->tmax, s->chunk_best, f.minp_listed ? s->cand.count : nullptr);
     launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
@@ -400,10 +404,13 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;
     f.row_flag = s->row_flag;
-    launch_row_final(L, f);
-    /* rows whose kept prefix is too wide for the shortcut flagged themselves 1: their candidates
-     * are listed and walked; what that cannot serve either is flagged 2 for the last two kernels.
-     * Each of these kernels returns at once for every row not flagged for it. */
+    /* rows whose kept prefix is too wide for the shortcut of the row-final kernel flag themselves
+     * 1: their candidates are listed and walked; what that cannot serve either is flagged 2 for
+     * the whole-row walk. Each of these kernels returns at once for every row not flagged for
+     * it. With the candidates already listed by the exp-sum pass the list walk comes first and
+     * alone. */
+    if (!f.minp_direct)
+        launch_row_final(L, f);
     launch_candidates(L, f);
     launch_sorted_general(L, f, s->probs, (long) s->max_vocab);
     return after_launch(s, "top-p / min-p");

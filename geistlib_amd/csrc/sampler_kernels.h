@@ -67,6 +67,9 @@ struct CandSpace {
 struct FinalLaunch {
     CandSpace       cand;
     bool            minp_listed; /* the exp-sum pass already listed the rows under the min-p bound */
+    bool            minp_direct; /* ... and the list walk runs straight after it: no row-final
+                                    kernel, no listing pass; a row whose list overflowed goes to
+                                    the whole-row walk */
     int             mode, k, k_sel;
     float           inv_t, top_p, min_p;
     const float    *uniforms;

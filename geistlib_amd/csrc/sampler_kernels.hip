@@ -357,11 +357,31 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
     chunk_bounds<NV>(rv, chunk, base, end);
     GS_MARK(0);
     float4 v[NV];
-    fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
-    float tm = -__builtin_inff();
+    float  tm = -__builtin_inff();
+    if (PEN && rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
+        rv.allowed == nullptr) {
+        /* the common case with penalties: each group is penalised as soon as its own load has
+         * arrived, while the later ones are still in flight (fetch_chunk() transforms the chunk
+         * as a whole, after its last load) */
+        const HistPrefetch pf = history_prefetch(rv, row, (int) gridDim.y);
+        const float4      *p =
+            reinterpret_cast<const float4 *>(rv.logits + (long) row * rv.ld + base) + tid;
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
-        tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
+        for (int j = 0; j < NV; ++j)
+            v[j] = p[j * TPB];
+        history_clear<NV * TPB * 4>(s_cnt16);
+        history_count(rv, row, pf, base, end, s_cnt16);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            transform_group<PEN, false>(rv, row, s_cnt16, 4 * (j * TPB + tid), base, end, v[j]);
+            tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
+        }
+    } else {
+        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
+    }
     if (base + 4 * tid >= end)
         tm = __builtin_nanf("");
     GS_MARK(1);
@@ -1689,13 +1709,24 @@ int configure_device_kernels() {
 
 void launch_candidates(const Launch &L, const FinalLaunch &f) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    const int  dyn = CAND_CAP * (int) sizeof(uint32_t); /* see configure_device_kernels() */
+    if (f.minp_direct) {
+        /* the exp-sum pass has listed every row: no row-final kernel, no listing pass. An
+         * unlisted element lies in z bin zb + 1 or beyond; the same expf as on the device. */
+        static const uint64_t tab[32] = GEIST_EXPF_TABLE_INIT;
+        const int             zb      = zbin_of_min_p(f.min_p);
+        const float p_out = geist_expf_glibc_le0(-(float) (zb + 1) / (float) ZBIN_PER_NAT, tab);
+        k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(
+            f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, f.chunk_sum, L.rv.n_chunks,
+            p_out);
+        return;
+    }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
             L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
     });
-    const int dyn = CAND_CAP * (int) sizeof(uint32_t); /* see configure_device_kernels() */
-    k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(f.cand, f.top_p, f.min_p, f.uniforms,
-                                                               f.row_flag, f.out);
+    k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(
+        f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f);
 }
 
 void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {

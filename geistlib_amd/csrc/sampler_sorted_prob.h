@@ -1107,13 +1107,20 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
     return (int) best_idx(sh.out_pack);
 }
 
-/* k_sorted_candidates: one workgroup per row flagged 1 or 4 walks the row's list (staged in LDS when
- * it fits). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
- * prefix that may reach past the list -- is flagged 2 for k_sorted_general. */
+/* k_sorted_candidates: one workgroup per row flagged 1 or 4 walks the row's list (staged in LDS
+ * when it fits; flag 4: listed by the exp-sum pass, holding p). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
+ * prefix that may reach past the list -- is flagged 2 for k_sorted_general.
+ * direct_sum != NULL: every row was listed by the exp-sum pass under the min-p bound (the list
+ * holds p, not pn) and no other kernel ran in between: the row's sum is taken from the chunk
+ * sums here (in chunk order, as everywhere), the bound on an unlisted element's pn from
+ * direct_p_out = expf of the first z bin outside the list, and the flag is written for every
+ * row. */
 __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float top_p, float min_p,
                                                            const float *__restrict__ uniforms,
                                                            int32_t *__restrict__ row_flag,
-                                                           int32_t *__restrict__ out) {
+                                                           int32_t *__restrict__ out,
+                                                           const double *__restrict__ direct_sum,
+                                                           int n_chunks, float direct_p_out) {
     extern __shared__ uint32_t s_key[]; /* CAND_CAP keys: every list is walked from LDS */
     __shared__ union {
         SortedGenShared gen;
@@ -1123,17 +1130,29 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
     __shared__ int      s_pick;
     __shared__ uint32_t s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
-    const int flag = row_flag[row];
-    if (flag != 1 && flag != 4)
+    const int flag = direct_sum ? 5 : row_flag[row];
+    if (flag != 1 && flag != 4 && flag != 5)
         return;
     const int n   = cand.count[row];
     int       tok = -1;
     GS_MARK(0);
+    double   sum  = 1.0;
+    uint32_t kout = 0u;
+    if (direct_sum) {
+        /* every thread adds the chunk sums in chunk order (the loads are broadcasts) */
+        sum = 0.0;
+        for (int c = 0; c < n_chunks; ++c)
+            sum += direct_sum[(long) row * n_chunks + c];
+        kout = __float_as_uint((float) ((double) direct_p_out / sum)) + 1u;
+    } else {
+        kout = cand.out_key[row];
+        if (flag == 4)
+            sum = cand.row_sum[row];
+    }
     if (n >= 1 && n <= CAND_CAP) {
         const uint32_t *gk = cand.key + (long) row * CAND_CAP;
         const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
         /* flag 4: the list holds p; pn = (float)((double)p / sum), sampler.c:251-253 */
-        const double sum = flag == 4 ? cand.row_sum[row] : 1.0;
         for (int i0 = 0; i0 < n; i0 += 8 * TPB) { /* eight independent loads in flight per thread */
             uint32_t k[8];
 #pragma unroll
@@ -1143,7 +1162,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
             for (int q = 0; q < 8; ++q) {
                 const int i = i0 + q * TPB + tid;
                 if (i < n)
-                    s_key[i] = flag == 4 ? __float_as_uint((float) ((double) __uint_as_float(k[q]) / sum))
+                    s_key[i] = flag >= 4 ? __float_as_uint((float) ((double) __uint_as_float(k[q]) / sum))
                                          : k[q];
             }
         }
@@ -1156,11 +1175,11 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
         gk = s_key;
         GS_MARK(1);
         const float *keys = reinterpret_cast<const float *>(gk);
-        tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], cand.out_key[row], sh.fast);
+        tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], kout, sh.fast);
         if (tok == -2) {
             __syncthreads();
-            tok = sorted_descend<true>(keys, gi, n, top_p, min_p, uniforms[row], cand.out_key[row],
-                                       sh.gen, s_scan, &s_pick);
+            tok = sorted_descend<true>(keys, gi, n, top_p, min_p, uniforms[row], kout, sh.gen,
+                                       s_scan, &s_pick);
         }
     }
     GS_MARK(7);

@@ -285,6 +285,25 @@ def test_sorted_paths_all_three_in_one_batch(hs, oracle):
     assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
 
 
+def test_min_p_listed_by_the_exp_sum_pass(hs, oracle):
+    """min_p of a few percent: the exp-sum pass lists the candidates and the list walk follows
+    it directly. Peaked rows (a handful of candidates), ordinary rows (hundreds), and flat rows
+    whose list overflows and is served by the whole-row walk; with and without top-p."""
+    n = 60000
+    g = np.random.default_rng(321)
+    scale = np.array([8.0, 8.0, 3.0, 3.0, 2.0, 0.3, 0.3, 0.05])[:, None]
+    x = (g.standard_normal((8, n)) * scale).astype(np.float32)
+    u = g.random(8).astype(np.float32)
+    for top_p in (1.0, 0.9):
+        kw = dict(temperature=1.0, top_p=top_p, min_p=0.03)
+        got = run_rows(hs, torch, x, u, P(**kw))
+        paths = hs.row_paths(8).tolist()
+        res = [oracle.chain_u(x[r], float(u[r]), **kw) for r in range(8)]
+        near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"min-p listed {top_p}")
+        assert near <= 1
+        assert paths[:5] == [2] * 5 and paths[5:] == [3] * 3, paths
+
+
 def test_sorted_modes_many_rows_and_one_row(hs, oracle):
     """More rows than compute units share the list walk (one workgroup per row, 100 KB of LDS
     each), and the single-row call of decode_step."""
