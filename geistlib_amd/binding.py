@@ -63,6 +63,7 @@ def load_library():
     lib.geist_hip_sampler_last_error.restype = C.c_char_p
     lib.geist_hip_sampler_sync.argtypes = [vp]
     lib.geist_hip_sampler_set_stream.argtypes = [vp, vp]
+    lib.geist_hip_sampler_set_logits_hint.argtypes = [vp, i32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -124,6 +125,11 @@ class HipSampler:
 
     def sync(self):
         self._check(self.lib.geist_hip_sampler_sync(self.h))
+
+    def set_logits_hint(self, streamed):
+        """streamed=True: the rows come from HBM and are read once (non-temporal loads in the
+        single-pass modes); False (default): they may still be cache-resident."""
+        self._check(self.lib.geist_hip_sampler_set_logits_hint(self.h, int(streamed)))
 
     @staticmethod
     def rows(logits, history=None, history_len=None, n_vocab=None, allowed=None):

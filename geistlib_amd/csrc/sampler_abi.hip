@@ -42,6 +42,7 @@ struct geist_hip_sampler {
     gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
+    bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
 
     char err[512] = {0};
 };
@@ -121,6 +122,7 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
     L.rv.per_chunk = per;
     L.rv.n_chunks  = nc;
     L.rv.vec_ok    = (((uintptr_t) r->d_logits) % 16 == 0) && (r->ld % 4 == 0);
+    L.rv.stream_loads = 0; /* set by the flows for their last pass over the rows */
     L.rv.hist      = pen ? r->d_history : nullptr;
     L.rv.hist_ld   = (long) r->history_ld;
     L.rv.hist_len  = pen ? r->d_history_len : nullptr;
@@ -231,6 +233,15 @@ int geist_hip_sampler_sync(geist_hip_sampler *s) {
     return GEIST_HIP_OK;
 }
 
+int geist_hip_sampler_set_logits_hint(geist_hip_sampler *s, int hint) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (hint != GEIST_HIP_LOGITS_CACHED && hint != GEIST_HIP_LOGITS_STREAMED)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown logits hint %d", hint);
+    s->logits_streamed = hint == GEIST_HIP_LOGITS_STREAMED;
+    return GEIST_HIP_OK;
+}
+
 int geist_hip_sampler_set_stream(geist_hip_sampler *s, void *stream) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
@@ -310,6 +321,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     f.out        = d_out;
 
     if (rs.greedy) {
+        L.rv.stream_loads = s->logits_streamed;
         launch_tmax_scan(L, s->tmax, s->chunk_best);
         if (stream_only(s))
             return after_launch(s, "argmax scan");
@@ -348,6 +360,7 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
             const int margin = rs.k / 2 > 8 ? rs.k / 2 : 8;
             f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
         }
+        scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
         launch_tmax_scan(scan, s->tmax, nullptr);
         if (stream_only(s))
             return after_launch(s, "top-k scan");
@@ -711,6 +724,7 @@ int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_h
         const int rc = make_launch(s, &rows[i], nullptr, false, L[i]);
         if (rc)
             return rc;
+        L[i].rv.stream_loads = s->logits_streamed;
         L[i].nv           = 8; /* the geometry of the top-k scan */
         L[i].rv.per_chunk = 8192;
         L[i].rv.n_chunks  = (int) ((rows[i].n_vocab + 8191) / 8192);

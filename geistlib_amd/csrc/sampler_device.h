@@ -415,6 +415,16 @@ __device__ __forceinline__ void history_count(const RowView &rv, int row, const 
     lds_barrier();
 }
 
+/* A 16-byte load marked non-temporal: the line is not kept in the caches on its way. For rows
+ * that come from HBM and are read once this is the faster read (a launch over 32.8 MB: 6.4 us
+ * against 7.0 us); for rows still in the Infinity Cache it is the slower one (5.5 us against
+ * 3.4 us), so it is used only where the caller has said the logits are not cache-resident. */
+__device__ __forceinline__ float4 load_streaming(const float4 *p) {
+    typedef float nt_f4 __attribute__((ext_vector_type(4)));
+    const nt_f4 t = __builtin_nontemporal_load(reinterpret_cast<const nt_f4 *>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+
 /* Issues the loads of the chunk [base, end) of a row into registers (layout in the file
  * header). Positions at or beyond `end` hold -inf. */
 template <int NV>
@@ -424,9 +434,15 @@ __device__ __forceinline__ void load_raw(const RowView &rv, const float *__restr
     const float ninf = -__builtin_inff();
     if (rv.vec_ok && end - base == NV * TPB * 4) { /* full chunk: no per-element tests */
         const float4 *p = reinterpret_cast<const float4 *>(row + base) + tid;
+        if (rv.stream_loads) {
 #pragma unroll
-        for (int j = 0; j < NV; ++j)
-            v[j] = p[j * TPB];
+            for (int j = 0; j < NV; ++j)
+                v[j] = load_streaming(p + j * TPB);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+                v[j] = p[j * TPB];
+        }
         return;
     }
 #pragma unroll

@@ -26,6 +26,8 @@ struct RowView {
     int            per_chunk;
     int            n_chunks;
     int            vec_ok; /* rows are 16-byte aligned: float4 loads allowed */
+    int            stream_loads; /* this pass is the last to read the rows and they come from HBM:
+                                    non-temporal loads */
     const int32_t *hist;   /* NULL = no penalties */
     long           hist_ld;
     const int32_t *hist_len;

@@ -189,9 +189,15 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     const float *rowp = rv.logits + (long) row * rv.ld;
     if (PLAIN) {
         const float4 *p = reinterpret_cast<const float4 *>(rowp + base) + tid;
+        if (rv.stream_loads) {
 #pragma unroll
-        for (int j = 0; j < NV; ++j)
-            v[j] = p[j * TPB];
+            for (int j = 0; j < NV; ++j)
+                v[j] = load_streaming(p + j * TPB);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+                v[j] = p[j * TPB];
+        }
     } else {
         load_raw<NV>(rv, rowp, base, end, v);
     }

@@ -91,6 +91,7 @@ def test_random_configurations_match_oracle(hs, oracle, seed):
         if pen is not None:
             kw.update(rep=pen["rep"], freq=pen["freq"], pres=pen["pres"])
         p = SampleParams.make(softcap=cap, **kw)
+        hs.set_logits_hint(bool(g.random() < 0.5))     # either way of loading, the same ids
         got = run_rows(hs, torch, x, u, p, None if pen is None else pen["hist"],
                        None if pen is None else pen["hl"], pad=pad, lead=lead, allowed=allowed)
         res = []

@@ -285,6 +285,22 @@ def test_sorted_paths_all_three_in_one_batch(hs, oracle):
     assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
 
 
+def test_logits_hint_changes_nothing_but_the_loads(hs, oracle):
+    """GEIST_HIP_LOGITS_STREAMED: non-temporal loads in the single-pass modes, identical ids."""
+    from geistlib_amd.binding import GeistHipError
+    x, u = rows_rng(91, 16, 128256, scale=2.0)
+    want = {}
+    for streamed in (False, True, False):
+        hs.set_logits_hint(streamed)
+        for name, prm in (("argmax", P(temperature=0.0)), ("top_k", P(temperature=0.7, top_k=40)),
+                          ("chain", P(temperature=0.7, top_k=40, top_p=0.9))):
+            got = run_rows(hs, torch, x, u, prm).tolist()
+            assert want.setdefault(name, got) == got, (name, streamed)
+    assert want["argmax"] == [oracle.argmax(x[r]) for r in range(16)]
+    with pytest.raises(GeistHipError):
+        hs.set_logits_hint(7)
+
+
 def test_min_p_listed_by_the_exp_sum_pass(hs, oracle):
     """min_p of a few percent: the exp-sum pass lists the candidates and the list walk follows
     it directly. Peaked rows (a handful of candidates), ordinary rows (hundreds), and flat rows
