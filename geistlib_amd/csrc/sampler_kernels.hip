@@ -24,9 +24,6 @@
  * logit exactly once per kernel; the logits are never written (k_penalties excepted).
  */
 #include "sampler_kernels.h"
-#ifndef GS_XCD_REMAP
-#define GS_XCD_REMAP 1
-#endif
 
 #include "sampler_device.h"
 
@@ -37,18 +34,6 @@ namespace gs {
 
 __device__ const uint64_t g_expf_tab[32] = GEIST_EXPF_TABLE_INIT;
 
-/* Phase timestamps for kernel tuning; compiled in only by the tuning probe. */
-#ifdef GS_PHASES
-__device__ long long g_phase[16384 * 16];
-#define GS_MARK(i)                                                                             \
-    do {                                                                                       \
-        if (threadIdx.x == 0)                                                                  \
-            g_phase[((long) blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();   \
-    } while (0)
-#else
-#define GS_MARK(i) ((void) 0)
-#endif
-
 /* Which (row, chunk) a workgroup of a (chunks, rows) grid works on. Workgroups go to the eight
  * XCDs round-robin by their linear id, and each XCD has its own L2. With the rows dealt out so
  * that every chunk of row r is handled on XCD r mod 8 -- in every pass, and the one-workgroup-
@@ -57,7 +42,7 @@ __device__ long long g_phase[16384 * 16];
 __device__ __forceinline__ void xcd_row_chunk(int &row, int &chunk) {
     row   = blockIdx.y;
     chunk = blockIdx.x;
-    if ((gridDim.y & 7) == 0 && GS_XCD_REMAP) {
+    if ((gridDim.y & 7) == 0) {
         const int lin = blockIdx.y * gridDim.x + blockIdx.x, slot = lin >> 3;
         row           = (lin & 7) + 8 * (slot / (int) gridDim.x);
         chunk         = slot % (int) gridDim.x;
@@ -109,11 +94,8 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_ro
         const HistPrefetch pf = history_prefetch(rv, row, n_rows);
         load_raw<NV>(rv, rowp, base, end, v);
         history_clear<NV * TPB * 4>(cnt16);
-        GS_MARK(3);
         history_count(rv, row, pf, base, end, cnt16);
-        GS_MARK(4);
         apply_transform<NV>(rv, cnt16, v);
-        GS_MARK(5);
     } else {
         load_raw<NV>(rv, rowp, base, end, v);
         apply_transform<NV>(rv, nullptr, v);
@@ -361,7 +343,6 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
         zero_per_row[row] = 0; /* a counter the following pass adds to */
     int       base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
-    GS_MARK(0);
     float4 v[NV];
     float  tm = -__builtin_inff();
     if (PEN && rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
@@ -390,9 +371,7 @@ __global__ __launch_bounds__(TPB) void k_tmax_scan(RowView rv, float *__restrict
     }
     if (base + 4 * tid >= end)
         tm = __builtin_nanf("");
-    GS_MARK(1);
     tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
-    GS_MARK(2);
     if (BEST) {
         /* the chunk's maximum and the first index holding it (sampler.c:52-62): only threads
          * whose own maximum equals the chunk's look for the index */
@@ -872,7 +851,6 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         mxf = max3f(mxf, raw[q], raw[q + 1]);
     s_mx[tid] = f2key(mxf); /* 0 when the thread saw no real maximum */
     __syncthreads();
-    GS_MARK(1);
     /* 2 */
     const uint32_t a0 = s_mx[lane], a1 = s_mx[lane + 64], a2 = s_mx[lane + 128],
                    a3 = s_mx[lane + 192];
@@ -902,7 +880,6 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
                 tau = t;
         }
     }
-    GS_MARK(2);
     /* keys at or below that of -inf: the bound says nothing (masked rows) */
     if (real < a.k_sel || tau < 0x00800000u)
         return true;
@@ -912,9 +889,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #pragma unroll
     for (int q = 0; q < KPT; ++q)
         selmask |= (uint32_t) (raw[q] >= bound) << q;
-    GS_MARK(8);
     int pos = wave_reserve(__popc(selmask), s_n);
-    GS_MARK(9);
     while (selmask) { /* a few rounds: the selected maxima are spread over the threads */
         const int q = __ffs(selmask) - 1;
         selmask &= selmask - 1u;
@@ -924,10 +899,8 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         }
         ++pos;
     }
-    GS_MARK(10);
     __syncthreads();
     const int n_sel = *s_n;
-    GS_MARK(11);
     if (n_sel > SEL_MAX)
         return true; /* long runs of equal maxima */
     /* 4 */
@@ -960,7 +933,6 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
             }
         }
     }
-    GS_MARK(3);
     if (PEN) {
         const int shift = 31 - __clz(rv.per_chunk); /* per_chunk = 1024 * NV */
         history_for_each_batched(
@@ -979,14 +951,9 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
             });
         __syncthreads();
     }
-    GS_MARK(4);
     /* survivors are appended in any order (the ranking below orders them): their keys wait in
      * registers until the lane has seen all its tasks, so that it asks for places once -- every
      * LDS atomic that returns a value costs the wavefront a round trip */
-#ifdef GS_PHASES
-    __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): when have the gathered values arrived? */
-    GS_MARK(14);
-#endif
     uint32_t ck[TASKS][4];
     int      n_keep = 0;
 #pragma unroll
@@ -998,11 +965,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
         if (e0[q] >= e1[q])
             continue; /* no task (whole wavefronts beyond the list skip the block) */
         float x4[4] = {r[q].x, r[q].y, r[q].z, r[q].w};
-#ifdef GS_EXP_NOPEN_TRANSFORM
-        if (false) {
-#else
         if (PEN) {
-#endif
             const uint4 hc = *reinterpret_cast<const uint4 *>(&s_pcnt[t * 4]);
             if (hc.x | hc.y | hc.z | hc.w) { /* few float4 groups hold a history token */
                 x4[0] = hc.x ? penalise(x4[0], hc.x, rv.rep, rv.inv_rep, rv.freq, rv.pres) : x4[0];
@@ -1041,10 +1004,8 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
             }
         }
     }
-    GS_MARK(12);
     __syncthreads();
     const int m = *s_n2;
-    GS_MARK(5);
     /* m > 256: long runs of equal values at the bound. m < k can only happen when the thread
      * maxima were taken before the penalties (see the launch code): then too many of the
      * leading logits were penalised below the bound and it certifies nothing. */
@@ -1139,7 +1100,6 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __shared__ int      s_n, s_n2;
     __shared__ double   s_sum;
     const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
-    GS_MARK(0);
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid < C)
@@ -1155,7 +1115,6 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __syncthreads();
     const double sum = s_sum;
     int          tok = -1;
-    GS_MARK(1);
     if (a.minp_listed && a.cand.count[row] <= CAND_CAP) {
         /* the exp-sum pass listed the row under the min-p bound (holding p, not pn): the list
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */
@@ -1178,7 +1137,6 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         tok = sorted_from_tmax<NV, PEN, TMAX_LDS / TPB>(rv, a, row, mx, sum, u_row, s_big, s_mx,
                                                         s_wt, s_selid, s_pcnt, s_m, s_srt, &s_n,
                                                         &s_n2, s_tab);
-    GS_MARK(6);
     if (tok >= 0) {
         if (tid == 0) {
             a.row_flag[row]  = 0;
@@ -1222,7 +1180,6 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         }
     }
     __syncthreads();
-    GS_MARK(7);
     if (tid < WAVE) {
         int B = ZBINS - 1;
         if (want_p) {
@@ -1273,7 +1230,6 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
             a.out[row]            = -1;
         }
     }
-    GS_MARK(8);
 }
 
 /* top-k (sampler.c:178-228) and the chain behind it: select from the row's thread maxima, then
@@ -1292,7 +1248,6 @@ __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ int           s_n, s_n2;
     const int row = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks;
-    GS_MARK(0);
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     const float u_row   = a.uniforms[row];
@@ -1309,7 +1264,6 @@ __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
         __syncthreads();
         k = topk_row_general<NV, PEN, MASK>(rv, row, a.k, s_pack, TOPK_FAST_MAX, s_cnt16, s_gs);
     }
-    GS_MARK(6);
     /* k <= TOPK_FAST_MAX = 128: the tail runs on one wavefront without barriers */
     if (tid < WAVE) {
         const int tok =
@@ -1318,7 +1272,6 @@ __global__ __launch_bounds__(TPB) void k_final_topk(RowView rv, FinalArgs a) {
         if (tid == 0)
             a.out[row] = tok;
     }
-    GS_MARK(7);
 }
 
 /* ============================================================================================

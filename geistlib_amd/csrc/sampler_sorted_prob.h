@@ -161,7 +161,6 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     s_mx[tid] = mkey;
     s_wt[tid] = wt;
     __syncthreads();
-    GS_MARK(2);
     /* 2 */
     uint32_t key_lo = 0u;
     if (use_p) {
@@ -195,7 +194,6 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     if (key_lo < 0x00800000u)
         return -1;
     const float bound = key2f(key_lo);
-    GS_MARK(3);
     /* 3 */
     uint32_t selmask = 0u;
 #pragma unroll
@@ -213,7 +211,6 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     }
     __syncthreads();
     const int n_sel = *s_n;
-    GS_MARK(4);
     if (n_sel > SEL_MAX)
         return -1;
     constexpr int TASKS = SEL_MAX * NV / TPB;
@@ -295,7 +292,6 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     }
     __syncthreads();
     const int m = *s_n2;
-    GS_MARK(5);
     if (m > TPB || m < 1)
         return -1;
     if (tid < m) {
@@ -588,7 +584,6 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
             mass_m = pn_fx(__uint_as_float(kmax));
         }
     }
-    GS_MARK(2);
     /* nucleus edge */
     bool     limited   = false;
     uint32_t edge_key  = 0u, edge_ties = 0u;
@@ -640,7 +635,6 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
         mass_keep = block_sum_u64(lm, sh.red64);
         limited   = false;
     }
-    GS_MARK(3);
     /* the draw: first entry of the kept prefix at which the running mass exceeds u * mass */
     /* running mass > u * mass  <=>  running mass >= floor(u * mass) + 1 in integers */
     const uint64_t target2 = (uint64_t) __double2ull_rd((double) u * (double) mass_keep) + 1ull;
@@ -655,7 +649,6 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
             j = 1;
         if (j > ties_d)
             j = ties_d;
-        GS_MARK(4);
         if (LIST) {
             tok = list_jth_id(pn, ids, n, kd, (int) j, sh, s_scan, s_pick);
         } else {
@@ -789,7 +782,6 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     const int tid = threadIdx.x;
     if (row_flag[row] != 1)
         return;
-    GS_MARK(0);
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid == 0) {
@@ -803,12 +795,10 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     chunk_bounds<NV>(rv, chunk, base, end);
     float4 v[NV];
     fetch_chunk<NV, PEN>(rv, row, (int) gridDim.y, base, end, s_cnt16, v);
-    GS_MARK(1);
     const float  mx  = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, s_red)));
     const double tot = s_total;
     const int    B   = cand.row_bound[row];
     const float  thr = zbin_threshold(B); /* zbin(arg) <= B */
-    GS_MARK(2);
     uint32_t     mask = 0u;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -819,14 +809,12 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
             mask |= (uint32_t) in << (4 * j + c);
         }
     }
-    GS_MARK(6);
     /* places: inside the workgroup through LDS, one global add for the workgroup */
     int pos = wave_reserve(__popc(mask), &s_count);
     __syncthreads();
     const int n_blk = s_count;
     if (tid == 0)
         s_base = n_blk ? atomicAdd(&cand.count[row], n_blk) : 0;
-    GS_MARK(7);
     uint32_t *ck = cand.key + (long) row * CAND_CAP;
     uint32_t *ci = cand.idx + (long) row * CAND_CAP;
     if (n_blk <= LIST_STAGE) {
@@ -872,7 +860,6 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
             }
         }
     }
-    GS_MARK(8);
 }
 
 /* ============================================================================================
@@ -1001,7 +988,6 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
             kmax = k[q] > kmax ? k[q] : kmax;
     }
     kmax = (uint32_t) block_max_u64((uint64_t) wave_max_u32(kmax), sh.red64);
-    GS_MARK(8);
     if (kmax <= kout)
         return -1;
     const int   bits    = 32 - __clz((int) (kmax - kout));
@@ -1030,7 +1016,6 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
         }
     }
     __syncthreads();
-    GS_MARK(9);
     const uint64_t mass_m = use_m ? block_sum_u64(lm, sh.red64) : 0ull;
     /* exclusive prefix of the bins: thread t owns bins 8t .. 8t+7 */
     constexpr int PER = SG_BINS / TPB;
@@ -1045,7 +1030,6 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
     for (int w = 0; w < tid / WAVE; ++w)
         excl += sh.scan64[w];
     excl -= own;
-    GS_MARK(10);
     /* the bin at which the running mass reaches `target`; optionally the mass before bin `be` */
     auto locate = [&](uint64_t target, int be) {
         if (tid == 0)
@@ -1081,7 +1065,6 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
             mass_keep = sh.out_mass;
         }
     }
-    GS_MARK(11);
     const uint32_t kf = __float_as_uint(floor_w);
     if (use_m && (!have_p || kf > best_key(edge_pack))) {
         if (kf <= kout)
@@ -1097,7 +1080,6 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
     locate(target2, be);
     int      bd     = sh.res_bin;
     uint64_t before = sh.res_before;
-    GS_MARK(12);
     if (bd < 0 || bd >= be) { /* inside the partly kept bin of the edge */
         bd     = be;
         before = sh.res_before_edge;
@@ -1135,7 +1117,6 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
         return;
     const int n   = cand.count[row];
     int       tok = -1;
-    GS_MARK(0);
     double   sum  = 1.0;
     uint32_t kout = 0u;
     if (direct_sum) {
@@ -1173,7 +1154,6 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
         }
         __syncthreads();
         gk = s_key;
-        GS_MARK(1);
         const float *keys = reinterpret_cast<const float *>(gk);
         tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], kout, sh.fast);
         if (tok == -2) {
@@ -1182,7 +1162,6 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
                                        s_scan, &s_pick);
         }
     }
-    GS_MARK(7);
     if (tid == 0) {
         row_flag[row] = tok < 0 ? 2 : 0;
         out[row]      = tok;

@@ -191,7 +191,6 @@ __global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a,
     const int seq = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks, L = a.L;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
-    GS_MARK(0);
     const SpecVerdict vd  = verdict[seq];
     const int         js  = vd.js;
     const long        row = (long) seq * (L + 1) + js;
@@ -203,7 +202,6 @@ __global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a,
         const float  mx    = vd.mx;
         const double sum   = vd.sum;
         bool         resid = js < L;
-        GS_MARK(1);
         if (resid) {
             if (tid < C)
                 s_w[tid] = a.resid_sum[(long) seq * C + tid];
