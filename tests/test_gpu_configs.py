@@ -127,3 +127,26 @@ def test_config5_speculative_verification(hs, oracle):
     print("config 5: accepted lengths", sorted(lens), flush=True)
     assert min(lens) < L            # the workload exercises rejections ...
     assert max(lens) > 0            # ... and acceptances
+
+
+@pytest.mark.parametrize("seed", range(100, 108))
+def test_config2_other_seeds_at_full_size(hs, oracle, seed):
+    """The headline shape (64 x 128256, top-k 40 -> top-p 0.9) on other draws of the workload,
+    with and without the penalty stage, under both load hints."""
+    from geistlib_amd import workloads as W
+    w = W.config2(seed=seed, with_penalties=bool(seed & 1))
+    hs.set_logits_hint(bool(seed & 2))
+    got = sample(hs, w)
+    hs.set_logits_hint(False)
+    kw = dict(temperature=w.temperature, top_k=w.top_k, top_p=w.top_p, min_p=w.min_p)
+    want = oracle.batch_chain_u(w.logits, w.uniforms, hist=w.history, hist_len=w.history_len,
+                                rep=w.rep, freq=w.freq, pres=w.pres, threads=8, **kw)
+    near = 0
+    for r in np.nonzero(got != want)[0]:
+        row = w.logits[r]
+        if w.history is not None:
+            row = oracle.penalties(row, w.history[r, :w.history_len[r]], w.rep, w.freq, w.pres)
+        _, info = oracle.chain_u(row, float(w.uniforms[r]), **kw)
+        assert info.boundary_dist < BOUNDARY_TOL, (seed, int(r), int(got[r]), int(want[r]))
+        near += 1
+    assert near <= 1
