@@ -87,6 +87,8 @@ def load_library():
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
+    lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
+    lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     _LIB = lib
     return lib
 
@@ -200,6 +202,23 @@ class HipSampler:
         self._check(self.lib.geist_hip_propose_drafts_ngram(
             self.h, _ptr(history), hld, _ptr(history_len), _ptr(seeds), n_seq, int(k_max),
             int(max_suffix), _ptr(out_drafts), old, _ptr(out_count), _ptr(out_match_len)))
+
+    def rmsnorm(self, x, weight, eps, y):
+        """x, y: [rows, n] float32 device tensors (y may be x); weight: [n]."""
+        rows, n = x.shape
+        self._check(self.lib.geist_hip_rmsnorm_rows(self.h, _ptr(x), x.stride(0) if rows > 1 else n,
+                                                    _ptr(weight), eps, rows, n, _ptr(y),
+                                                    y.stride(0) if rows > 1 else n))
+
+    def f16_gemv(self, w_f16, x, y):
+        """w_f16: [n_out, n_in] float16 (or int16 bit patterns), x: [m, n_in] float32,
+        y: [m, n_out] float32: y[m] = W x[m] in the reference's order of summation."""
+        n_out, n_in = w_f16.shape
+        m = x.shape[0]
+        assert w_f16.is_contiguous() and w_f16.element_size() == 2 and x.shape[1] == n_in
+        self._check(self.lib.geist_hip_f16_gemv_rows(
+            self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
 
     def time_stream_kernel(self, rows, params, uniforms, out, launches):
         """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around

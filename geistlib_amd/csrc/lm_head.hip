@@ -1,0 +1,240 @@
+/*
+ * lm_head.hip -- the two steps between the last transformer layer and the sampler
+ * (src/archs/transformer/forward/head.c:94-129 of the reference), for gfx950:
+ *
+ *   k_rmsnorm_rows   cpu_scalar_rmsnorm               src/backends/cpu_scalar/elementwise.c:241-280
+ *   k_f16_gemv       f16_gemv_m1 (tied F16 lm_head)   src/backends/cpu_x86/kernel_f16_gemv.c:34-64
+ *
+ * Both reproduce the reference's results bit for bit, which fixes the order of every sum.
+ *
+ * k_f16_gemv. The reference adds the products of a row in sixteen chains of fused multiply-adds
+ * (two 8-lane AVX accumulators: element k belongs to chain k % 16 and is added at step k / 16),
+ * then folds the chains in a fixed tree. A chain is sequential, so one lane owns eight chains of
+ * one weight row -- the 16 bytes it needs per step are exactly one accumulator's 8 weights --
+ * and two neighbouring lanes own a row. A wavefront therefore works on 32 rows at a time, and
+ * reading 16 bytes per lane straight from those rows would touch 32 different lines per load.
+ * Instead the wavefront streams the rows through a private LDS tile: it loads 128 bytes of each
+ * of its 32 rows with fully coalesced 16-byte loads (8 lanes per row), two stages ahead in
+ * registers, writes them to the tile (row pitch 144 bytes against bank conflicts), and each lane
+ * reads its own 16 bytes per step back. No workgroup barrier is involved: the tile belongs to
+ * one wavefront, whose LDS operations execute in order. The activations of the stage take the
+ * same way (they come from L2). The kernel is bound by the one pass over the weights: 2 bytes
+ * per multiply-add for one activation row, 2 / n_m bytes with n_m rows, whose accumulators
+ * (8 per row and lane) share each converted weight.
+ */
+#include "lm_head_kernels.h"
+
+#include <hip/hip_fp16.h>
+
+namespace gs {
+
+namespace {
+
+constexpr int LM_TPB       = 256;
+constexpr int LM_WAVE      = 64;
+constexpr int LM_WAVES     = LM_TPB / LM_WAVE;
+constexpr int ROWS_WAVE    = 32;                   /* two lanes per weight row */
+constexpr int ROWS_BLOCK   = ROWS_WAVE * LM_WAVES; /* 128 */
+constexpr int STAGE_COLS   = 64;                   /* 128 bytes of a row: four steps of 16 */
+constexpr int STAGE_LOADS  = 4;                    /* 32 rows x 8 segments / 64 lanes */
+constexpr int TILE_PITCH   = STAGE_COLS * 2 + 16;  /* bytes */
+constexpr int TILE_BYTES   = ROWS_WAVE * TILE_PITCH;
+
+__device__ __forceinline__ float dadd(float a, float b) { return __fadd_rn(a, b); }
+
+/* The weights of one stage for this lane: segment (lane & 7) of rows 8 i + (lane >> 3). */
+struct StageRegs {
+    uint4 w[STAGE_LOADS];
+};
+
+template <int MT>
+struct StageX {
+    float x[MT];
+};
+
+__device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long row0, long n_out,
+                                           int n_in, int stage, int lane, StageRegs &g) {
+    const int seg = lane & 7;
+    const int col = stage * STAGE_COLS + seg * 8;
+#pragma unroll
+    for (int i = 0; i < STAGE_LOADS; ++i) {
+        const long row = row0 + 8 * i + (lane >> 3);
+        g.w[i]         = make_uint4(0u, 0u, 0u, 0u);
+        if (row < n_out && col < n_in)
+            g.w[i] = *reinterpret_cast<const uint4 *>(w + row * n_in + col);
+    }
+}
+
+template <int MT>
+__device__ __forceinline__ void stage_load_x(const float *__restrict__ x, long ld_x, int n_m,
+                                             int n_in, int stage, int lane, StageX<MT> &gx) {
+    const int col = stage * STAGE_COLS + lane;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int mm = m < n_m ? m : n_m - 1; /* rows beyond n_m repeat the last one, unstored */
+        gx.x[m]      = col < n_in ? x[mm * ld_x + col] : 0.0f;
+    }
+}
+
+} // namespace
+
+template <int MT>
+__global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict__ w, long n_out,
+                                                     int n_in, const float *__restrict__ x,
+                                                     long ld_x, int n_m, float *__restrict__ y,
+                                                     long ld_y) {
+    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][TILE_BYTES];
+    __shared__ __align__(16) float   s_x[LM_WAVES][MT][STAGE_COLS];
+    const int  lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
+    const long row0 = (long) blockIdx.x * ROWS_BLOCK + wave * ROWS_WAVE;
+    if (row0 >= n_out)
+        return; /* (no workgroup barrier below) */
+    uint8_t *tile = s_tile[wave];
+    float(*xs)[STAGE_COLS] = s_x[wave];
+    const int my_row = lane >> 1, half = lane & 1;
+
+    float acc[MT][8];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc[m][i] = 0.0f;
+
+    const int n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    StageRegs  g0, g1;
+    StageX<MT> x0, x1;
+    stage_load(w, row0, n_out, n_in, 0, lane, g0);
+    stage_load_x<MT>(x, ld_x, n_m, n_in, 0, lane, x0);
+    if (n_stage > 1) {
+        stage_load(w, row0, n_out, n_in, 1, lane, g1);
+        stage_load_x<MT>(x, ld_x, n_m, n_in, 1, lane, x1);
+    }
+    for (int s = 0; s < n_stage; ++s) {
+        /* registers -> tile (this waits for the loads issued two stages ago) */
+#pragma unroll
+        for (int i = 0; i < STAGE_LOADS; ++i)
+            *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
+                g0.w[i];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            xs[m][lane] = x0.x[m];
+        g0 = g1;
+        x0 = x1;
+        if (s + 2 < n_stage) {
+            stage_load(w, row0, n_out, n_in, s + 2, lane, g1);
+            stage_load_x<MT>(x, ld_x, n_m, n_in, s + 2, lane, x1);
+        }
+        /* steps of this stage: whole blocks of 16 columns, and at the end of the row possibly
+         * a block of 8, which only extends chains 0..7 (the lanes with half == 0) */
+        const int left  = n_in - s * STAGE_COLS;
+        const int full  = left >= STAGE_COLS ? 4 : left / 16;
+        const bool tail8 = left < STAGE_COLS && (left & 15) == 8;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const bool whole = t < full;
+            const bool eight = tail8 && t == full && half == 0;
+            if (!whole && !(tail8 && t == full))
+                continue;
+            const uint4 q = *reinterpret_cast<const uint4 *>(tile + my_row * TILE_PITCH + t * 32 +
+                                                             half * 16);
+            const __half2 h01 = *reinterpret_cast<const __half2 *>(&q.x);
+            const __half2 h23 = *reinterpret_cast<const __half2 *>(&q.y);
+            const __half2 h45 = *reinterpret_cast<const __half2 *>(&q.z);
+            const __half2 h67 = *reinterpret_cast<const __half2 *>(&q.w);
+            const float2  f01 = __half22float2(h01), f23 = __half22float2(h23);
+            const float2  f45 = __half22float2(h45), f67 = __half22float2(h67);
+            const float   wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const float4 xa = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8]);
+                const float4 xb = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8 + 4]);
+                const float  xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float f = __builtin_fmaf(wf[i], xv[i], acc[m][i]);
+                    acc[m][i]     = (whole || eight) ? f : acc[m][i];
+                }
+            }
+        }
+    }
+    /* (chain j + chain j+8), (lane i + lane i+4), ((0+1) + (2+3)): kernel_f16_gemv.c:25-32, 59 */
+    const long row = row0 + my_row;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            v[i] = dadd(acc[m][i], __shfl_xor(acc[m][i], 1, LM_WAVE));
+        const float q0 = dadd(v[0], v[4]), q1 = dadd(v[1], v[5]);
+        const float q2 = dadd(v[2], v[6]), q3 = dadd(v[3], v[7]);
+        const float sum = dadd(dadd(q0, q1), dadd(q2, q3));
+        if (half == 0 && row < n_out && m < n_m)
+            y[m * ld_y + row] = sum;
+    }
+}
+
+/* One workgroup per row. The reference adds the squares in double in index order; the order of
+ * a double sum only shows in the binary32 result when 1 / sqrt(mean + eps) lies within the
+ * sum's error of the middle between two binary32 values. The workgroup adds in a fixed parallel
+ * order and, in that rare case, one thread repeats the sum in the reference's order. */
+__global__ __launch_bounds__(LM_TPB) void k_rmsnorm_rows(const float *__restrict__ x, long ld_x,
+                                                         const float *__restrict__ w, float eps,
+                                                         int n, float *__restrict__ y, long ld_y) {
+    __shared__ double s_part[LM_TPB];
+    __shared__ float  s_inv;
+    const int    tid = threadIdx.x;
+    const float *xr  = x + (long) blockIdx.x * ld_x;
+    float       *yr  = y + (long) blockIdx.x * ld_y;
+    double       a   = 0.0;
+    for (int i = tid; i < n; i += LM_TPB)
+        a += (double) xr[i] * (double) xr[i];
+    s_part[tid] = a;
+    __syncthreads();
+    for (int step = LM_TPB / 2; step > 0; step >>= 1) {
+        if (tid < step)
+            s_part[tid] += s_part[tid + step];
+        __syncthreads();
+    }
+    if (tid == 0) {
+        double      sumsq = s_part[0];
+        double      r     = 1.0 / sqrt(sumsq / (double) n + (double) eps);
+        float       f     = (float) r;
+        /* distance of r from the nearer rounding boundary of f, relative to r; the two sums
+         * differ by less than n * 2^-52 relative, and r by half of that */
+        const float  fn  = r > (double) f ? nextafterf(f, __builtin_inff()) : nextafterf(f, -__builtin_inff());
+        const double mid = 0.5 * ((double) f + (double) fn);
+        if (fabs(r - mid) <= fabs(r) * (double) n * 0x1p-50) {
+            sumsq = 0.0;
+            for (int i = 0; i < n; ++i)
+                sumsq += (double) xr[i] * (double) xr[i];
+            f = (float) (1.0 / sqrt(sumsq / (double) n + (double) eps));
+        }
+        s_inv = f;
+    }
+    __syncthreads();
+    const float inv = s_inv;
+    for (int i = tid; i < n; i += LM_TPB)
+        yr[i] = __fmul_rn(__fmul_rn(xr[i], inv), w[i]);
+}
+
+void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const float *w, float eps,
+                         int n_rows, int n, float *y, long ld_y) {
+    k_rmsnorm_rows<<<dim3(n_rows), dim3(LM_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y);
+}
+
+void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
+                     const float *x, long ld_x, int n_m, float *y, long ld_y) {
+    const dim3 grid((unsigned) ((n_out + ROWS_BLOCK - 1) / ROWS_BLOCK)), block(LM_TPB);
+    if (n_m <= 1)
+        k_f16_gemv<1><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+    else if (n_m <= 2)
+        k_f16_gemv<2><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+    else if (n_m <= 4)
+        k_f16_gemv<4><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+    else if (n_m <= 8)
+        k_f16_gemv<8><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+    else
+        k_f16_gemv<16><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+}
+
+} // namespace gs

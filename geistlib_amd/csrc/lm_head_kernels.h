@@ -1,0 +1,25 @@
+/* Launchers of the output-head kernels (lm_head.hip): the RMS norm in front of the lm_head and
+ * the F16 lm_head projection itself, so that logits are born in device memory and the sampler
+ * reads them there. */
+#ifndef GEIST_LM_HEAD_KERNELS_H
+#define GEIST_LM_HEAD_KERNELS_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace gs {
+
+constexpr int GEMV_M_MAX = 16; /* activation rows one pass over the weights serves */
+
+/* y = x * w * rsqrt(mean(x^2) + eps) per row; y may alias x. */
+void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const float *w, float eps,
+                         int n_rows, int n, float *y, long ld_y);
+
+/* y[m][r] = sum_i f16(W[r][i]) * x[m][i] for m < n_m <= GEMV_M_MAX; n_in a multiple of 8. */
+void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
+                     const float *x, long ld_x, int n_m, float *y, long ld_y);
+
+} // namespace gs
+#endif

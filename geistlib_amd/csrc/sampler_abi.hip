@@ -13,6 +13,8 @@
 #include <new>
 #include <vector>
 
+#include "../../include/geist_lm_head_hip.h"
+#include "lm_head_kernels.h"
 #include "sampler_kernels.h"
 
 using namespace gs;
@@ -557,6 +559,46 @@ int geist_hip_logprob_rows(geist_hip_sampler *s, const float *d_logits, size_t l
     launch_logprob(L, s->chunk_best, s->chunk_sum, d_tokens, (long) tokens_ld, (int) k_per_row,
                    d_out, (long) out_ld);
     return after_launch(s, "log-probabilities");
+}
+
+int geist_hip_rmsnorm_rows(geist_hip_sampler *s, const float *d_x, size_t ld_x,
+                           const float *d_weight, float eps, size_t n_rows, size_t n, float *d_y,
+                           size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_x || !d_weight || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || n == 0 || n > 0x7fffffffu || n_rows > 0x7fffffffu || ld_x < n || ld_y < n)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "rmsnorm: %zu rows of %zu, strides %zu / %zu",
+                    n_rows, n, ld_x, ld_y);
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_rmsnorm_rows(s->stream, d_x, (long) ld_x, d_weight, eps, (int) n_rows, (int) n, d_y,
+                        (long) ld_y);
+    return after_launch(s, "rmsnorm");
+}
+
+int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
+                            size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
+                            size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_f16 || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_out == 0 || n_in == 0 || n_rows == 0 || n_in > 0x7ffffff8u || ld_x < n_in ||
+        ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "gemv: %zu x %zu, %zu rows, strides %zu / %zu",
+                    n_out, n_in, n_rows, ld_x, ld_y);
+    if (n_in % 8 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "gemv: n_in %zu is not a multiple of 8", n_in);
+    if (((uintptr_t) d_w_f16) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "gemv: weights not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    for (size_t m0 = 0; m0 < n_rows; m0 += GEMV_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) GEMV_M_MAX ? n_rows - m0 : (size_t) GEMV_M_MAX;
+        launch_f16_gemv(s->stream, d_w_f16, (long) n_out, (int) n_in, d_x + m0 * ld_x, (long) ld_x,
+                        (int) m, d_y + m0 * ld_y, (long) ld_y);
+    }
+    return after_launch(s, "f16 gemv");
 }
 
 int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,

@@ -1,0 +1,42 @@
+/*
+ * geist_lm_head_hip.h -- the output head in front of the sampler, on the device: the RMS norm and
+ * the tied F16 lm_head projection of the reference's finalize step
+ * (src/archs/transformer/forward/head.c:94-129). With them the logits are written by the GPU
+ * into the buffer the sampler reads (include/geist_sampler_hip.h); nothing of vocabulary size
+ * crosses to the host. Both functions enqueue on the sampler's stream and reproduce the
+ * reference's CPU results bit for bit.
+ */
+#ifndef GEIST_LM_HEAD_HIP_H
+#define GEIST_LM_HEAD_HIP_H
+
+#include "geist_sampler_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Replaces prims->rmsnorm as head.c:99-101 calls it (cpu_scalar_rmsnorm,
+ * src/backends/cpu_scalar/elementwise.c:241-280): for each of n_rows rows of n floats,
+ *   inv = (float)(1.0 / sqrt(sum_i (double)x_i^2 / n + (double)eps)),  y_i = (x_i * inv) * w_i.
+ * Row r of x starts at d_x + r * ld_x, of y at d_y + r * ld_y; d_y may be d_x. */
+int geist_hip_rmsnorm_rows(geist_hip_sampler *s, const float *d_x, size_t ld_x,
+                           const float *d_weight, float eps, size_t n_rows, size_t n, float *d_y,
+                           size_t ld_y);
+
+/* Replaces f16_gemv_m1 (src/backends/cpu_x86/kernel_f16_gemv.h:22-25, kernel_f16_gemv.c:34-64;
+ * bound as linear_m1 of an F16 weight at src/backends/cpu_x86/backend.c:318-324, 406-411), the
+ * kernel behind the tied F16 lm_head at head.c:114-126:
+ *   d_y[m * ld_y + r] = sum_i f16_to_f32(d_w_f16[r * n_in + i]) * d_x[m * ld_x + i]
+ * for every activation row m < n_rows, with the reference's order of summation (sixteen chains
+ * of fused multiply-adds folded in a fixed tree), so each row equals what f16_gemv_m1 returns
+ * for it. The weights are read once for up to 16 activation rows. n_in must be a multiple of 8
+ * (GEIST_HIP_E_UNSUPPORTED otherwise: the reference adds a remainder element by element, with
+ * rounding that depends on how it was compiled); d_w_f16 must be 16-byte aligned. */
+int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
+                            size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
+                            size_t ld_y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

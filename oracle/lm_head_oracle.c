@@ -1,0 +1,104 @@
+/*
+ * lm_head_oracle.c -- see lm_head_oracle.h. Test infrastructure only.
+ */
+#include "lm_head_oracle.h"
+
+#include <math.h>
+#include <string.h>
+
+/* src/formats/gguf/common.c:29-62 */
+float oracle_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t) (h >> 15) << 31;
+    const uint32_t e    = (h >> 10) & 0x1fu;
+    uint32_t       m    = h & 0x3ffu;
+    uint32_t       bits;
+    if (e == 0x1fu) {
+        bits = sign | 0x7f800000u | (m << 13);
+    } else if (e != 0) {
+        bits = sign | ((e + 112u) << 23) | (m << 13);
+    } else if (m == 0) {
+        bits = sign;
+    } else { /* subnormal: value m * 2^-24, normalised */
+        uint32_t e32 = 113u;
+        while (!(m & 0x400u)) {
+            m <<= 1;
+            e32--;
+        }
+        bits = sign | (e32 << 23) | ((m & 0x3ffu) << 13);
+    }
+    float f;
+    memcpy(&f, &bits, sizeof f);
+    return f;
+}
+
+uint16_t oracle_f32_to_f16(float v) {
+    uint32_t b;
+    memcpy(&b, &v, sizeof b);
+    const uint16_t sign = (uint16_t) ((b >> 16) & 0x8000u);
+    const uint32_t a    = b & 0x7fffffffu;
+    if (a >= 0x7f800000u) /* inf, NaN (quiet) */
+        return (uint16_t) (sign | 0x7c00u | (a > 0x7f800000u ? 0x200u | ((a >> 13) & 0x3ffu) : 0u));
+    if (a >= 0x477ff000u) /* rounds to or beyond 65520 */
+        return (uint16_t) (sign | 0x7c00u);
+    if (a < 0x33000001u) /* at most half of the smallest subnormal */
+        return sign;
+    int      e = (int) (a >> 23) - 127;
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;
+    int      shift;
+    uint32_t base;
+    if (e < -14) { /* subnormal result: value = m * 2^(e-23), unit 2^-24 */
+        shift = -1 - e; /* 13 + (-14 - e) */
+        base  = 0;
+    } else {
+        shift = 13;
+        base  = (uint32_t) (e + 15) << 10;
+        m &= 0x7fffffu;
+    }
+    const uint32_t q    = m >> shift;
+    const uint32_t rem  = m & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    uint32_t       r    = base + q;
+    if (rem > half || (rem == half && (q & 1u)))
+        r++; /* carries into the exponent as it should */
+    return (uint16_t) (sign | r);
+}
+
+/* src/backends/cpu_x86/kernel_f16_gemv.c:34-64 */
+void oracle_f16_gemv_m1(size_t n_out, size_t n_in, const float *x, const uint16_t *w_f16, float *y) {
+    for (size_t r = 0; r < n_out; r++) {
+        const uint16_t *wr = w_f16 + r * n_in;
+        float           chain[16];
+        for (int j = 0; j < 16; j++)
+            chain[j] = 0.0f;
+        size_t k = 0;
+        for (; k + 16 <= n_in; k += 16)
+            for (int j = 0; j < 16; j++)
+                chain[j] = fmaf(oracle_f16_to_f32(wr[k + j]), x[k + j], chain[j]);
+        for (; k + 8 <= n_in; k += 8)
+            for (int j = 0; j < 8; j++)
+                chain[j] = fmaf(oracle_f16_to_f32(wr[k + j]), x[k + j], chain[j]);
+        float v[8], q[4];
+        for (int i = 0; i < 8; i++)
+            v[i] = chain[i] + chain[i + 8];
+        for (int i = 0; i < 4; i++)
+            q[i] = v[i] + v[i + 4];
+        float s = (q[0] + q[1]) + (q[2] + q[3]);
+        for (; k < n_in; k++)
+            s += oracle_f16_to_f32(wr[k]) * x[k];
+        y[r] = s;
+    }
+}
+
+/* src/backends/cpu_scalar/elementwise.c:266-278 */
+void oracle_rmsnorm_rows(size_t n_rows, size_t n, const float *x, const float *w, float eps,
+                         float *y) {
+    for (size_t r = 0; r < n_rows; r++) {
+        const float *xr    = x + r * n;
+        double       sumsq = 0.0;
+        for (size_t i = 0; i < n; i++)
+            sumsq += (double) xr[i] * (double) xr[i];
+        const float inv = (float) (1.0 / sqrt(sumsq / (double) n + (double) eps));
+        for (size_t i = 0; i < n; i++)
+            y[r * n + i] = xr[i] * inv * w[i];
+    }
+}

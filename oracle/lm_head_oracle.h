@@ -1,0 +1,46 @@
+/*
+ * lm_head_oracle.h -- TEST INFRASTRUCTURE, not part of the shipped library: a scalar CPU
+ * restatement of the two steps the reference runs between the last layer and the sampler
+ * (src/archs/transformer/forward/head.c:94-129): the output RMS norm and the tied lm_head
+ * projection for F16 weights. Only tests/, the smoke check and the cpu_baseline leg of bench.py
+ * may load it.
+ *
+ * Pinned by: the reference's own kernel compiled from its tree (oracle/_ref/libgeist_ref_f16gemv
+ * .so, src/backends/cpu_x86/kernel_f16_gemv.c) bit for bit on random and adversarial inputs
+ * (tests/test_lm_head_oracle.py); the exact-double reference of the reference's unit test
+ * (tests/test_q8w_gemv_unit.c:49-56) within the bound of fp32 accumulation; closed forms for the
+ * norm (constant rows, unit weights) and numpy in float64.
+ */
+#ifndef GEIST_LM_HEAD_ORACLE_H
+#define GEIST_LM_HEAD_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* IEEE binary16 -> binary32, exact (src/formats/gguf/common.c:29-62). */
+float oracle_f16_to_f32(uint16_t h);
+/* binary32 -> binary16, round to nearest even (what tests/test_q8w_gemv_unit.c:24-26 gets from
+ * F16C); used to build test weights. */
+uint16_t oracle_f32_to_f16(float v);
+
+/* y[r] = sum_i f16_to_f32(W[r,i]) * x[i] in the summation order of f16_gemv_m1
+ * (src/backends/cpu_x86/kernel_f16_gemv.c:34-64): sixteen chains of fused multiply-adds --
+ * chain j takes the elements 16 t + j in order of t; a trailing block of eight extends chains
+ * 0..7 --, then (chain j + chain j+8), then (lane i + lane i+4), then ((0+1) + (2+3)), then the
+ * elements of an n_in % 8 tail one by one. */
+void oracle_f16_gemv_m1(size_t n_out, size_t n_in, const float *x, const uint16_t *w_f16, float *y);
+
+/* y = x * weight * rsqrt(mean(x^2) + eps) per row (cpu_scalar_rmsnorm,
+ * src/backends/cpu_scalar/elementwise.c:241-280): sum of squares in double in index order,
+ * inv = (float)(1.0 / sqrt(sum / n + (double) eps)), y_i = (x_i * inv) * w_i in binary32. */
+void oracle_rmsnorm_rows(size_t n_rows, size_t n, const float *x, const float *w, float eps,
+                         float *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -106,6 +106,14 @@ def load_oracle(fast=False):
                                          C.c_float, C.c_float, C.c_float, c_float_p, c_int32_p,
                                          C.c_int]
     lib.oracle_max_threads.restype = C.c_int
+    c_u16_p = C.POINTER(C.c_uint16)
+    lib.oracle_f16_to_f32.restype = C.c_float
+    lib.oracle_f16_to_f32.argtypes = [C.c_uint16]
+    lib.oracle_f32_to_f16.restype = C.c_uint16
+    lib.oracle_f32_to_f16.argtypes = [C.c_float]
+    lib.oracle_f16_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, c_u16_p, c_float_p]
+    lib.oracle_rmsnorm_rows.argtypes = [C.c_size_t, C.c_size_t, c_float_p, c_float_p, C.c_float,
+                                        c_float_p]
     return lib
 
 
@@ -181,6 +189,25 @@ class Oracle:
                                                  int(max_suffix), _ip(out), C.byref(match))
         return out[:k].tolist(), int(match.value)
 
+    def f16_gemv(self, w_f16, x):
+        """w_f16: uint16 [n_out, n_in] (binary16 bit patterns), x: float32 [n_in] or [m, n_in]
+        -> float32 [n_out] or [m, n_out], each row of x through oracle_f16_gemv_m1."""
+        w = np.ascontiguousarray(w_f16, dtype=np.uint16)
+        xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+        n_out, n_in = w.shape
+        y = np.empty((xs.shape[0], n_out), dtype=np.float32)
+        for m in range(xs.shape[0]):
+            self.lib.oracle_f16_gemv_m1(n_out, n_in, _fp(xs[m]),
+                                        w.ctypes.data_as(C.POINTER(C.c_uint16)), _fp(y[m]))
+        return y[0] if np.ndim(x) == 1 else y
+
+    def rmsnorm(self, x, w, eps):
+        xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        y = np.empty_like(xs)
+        self.lib.oracle_rmsnorm_rows(xs.shape[0], xs.shape[1], _fp(xs), _fp(w), eps, _fp(y))
+        return y[0] if np.ndim(x) == 1 else y
+
     def softcap(self, row, cap):
         out = row.copy()
         self.lib.oracle_softcap_inplace(out.size, _fp(out), cap)
@@ -239,6 +266,22 @@ class RefWorkspace(C.Structure):
 def ref_path(fast=False):
     return os.path.join(ORACLE_DIR, "_ref",
                         "libgeist_ref_sampler_fast.so" if fast else "libgeist_ref_sampler.so")
+
+
+def load_ref_f16gemv(fast=False):
+    """The reference's f16_gemv_m1 compiled from its own sources, or None where not built. Loaded
+    with lazy binding: the unit that defines fp16_to_fp32 also holds GGUF functions whose
+    dependencies are not linked and are never called."""
+    path = os.path.join(ORACLE_DIR, "_ref",
+                        "libgeist_ref_f16gemv_fast.so" if fast else "libgeist_ref_f16gemv.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path, mode=os.RTLD_LAZY)
+    lib.f16_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.POINTER(C.c_uint16), c_float_p]
+    lib.f16_gemv_m1.restype = None
+    lib.fp16_to_fp32.restype = C.c_float
+    lib.fp16_to_fp32.argtypes = [C.c_uint16]
+    return lib
 
 
 def load_ref(fast=False):

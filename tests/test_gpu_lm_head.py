@@ -1,0 +1,128 @@
+"""The output head in front of the sampler on the device -- RMS norm and the tied F16 lm_head
+(src/archs/transformer/forward/head.c:94-129 of the reference) -- through the C ABI against the
+oracle, which is itself pinned bit for bit to the reference's compiled kernel
+(tests/test_lm_head_oracle.py). Every float must agree in every bit."""
+import numpy as np
+import pytest
+
+from gpu_util import to_dev
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hs():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=32, max_vocab=40000)
+    yield s
+    s.close()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def run_gemv(hs, w16, x):
+    d_w = to_dev(w16.view(np.int16), torch)
+    d_x = to_dev(x, torch)
+    y = torch.full((x.shape[0], w16.shape[0]), 7.0, dtype=torch.float32, device="cuda")
+    hs.f16_gemv(d_w, d_x, y)
+    hs.sync()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(1000, 2560, 1), (130, 64, 1), (129, 128, 3),
+                                          (4097, 1536, 2), (300, 8, 1), (300, 16, 5), (257, 24, 4),
+                                          (31, 2568, 8), (640, 4096, 16), (500, 2560, 17),
+                                          (50, 72, 16), (33, 40, 9), (1, 2560, 1)])
+def test_f16_gemv_rows_bit_exact(hs, oracle, n_out, n_in, m):
+    print(f"gemv n_out={n_out} n_in={n_in} m={m}", flush=True)
+    g = np.random.default_rng(n_out * 7 + n_in + m)
+    w16 = (g.standard_normal((n_out, n_in)) * g.choice([0.02, 1.0])).astype(np.float16).view(np.uint16)
+    x = (g.standard_normal((m, n_in)) * g.choice([0.1, 1.0, 30.0], (m, 1))).astype(np.float32)
+    got = run_gemv(hs, w16, x)
+    want = oracle.f16_gemv(w16, x)
+    assert (bits(got) == bits(want)).all(), np.argwhere(bits(got) != bits(want))[:5]
+
+
+def test_f16_gemv_special_values(hs, oracle):
+    """Subnormal and extreme binary16 weights, zeros of both signs, a row of zeros with negative
+    activations (the sign of a zero result is part of the result)."""
+    n_out, n_in = 64, 96
+    g = np.random.default_rng(3)
+    w = g.standard_normal((n_out, n_in)).astype(np.float16)
+    w[0, :] = 0.0
+    w[1, :] = -0.0
+    w[2, :] = np.float16(6e-8)                     # smallest subnormals
+    w[3, :] = np.float16(65504.0)
+    w[4, ::2] = np.float16(-65504.0)
+    w[5, :] = np.float16(2.0 ** -14)
+    w16 = w.view(np.uint16)
+    x = np.stack([g.standard_normal(n_in), -np.abs(g.standard_normal(n_in)),
+                  np.full(n_in, 1e-30), np.full(n_in, 3e30)]).astype(np.float32)
+    got = run_gemv(hs, w16, x)
+    want = oracle.f16_gemv(w16, x)
+    same = (bits(got) == bits(want)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), np.argwhere(~same)[:5]
+
+
+def test_f16_gemv_strides_and_errors(hs, oracle):
+    from geistlib_amd.binding import GeistHipError
+    g = np.random.default_rng(4)
+    n_out, n_in, m = 200, 256, 3
+    w16 = g.standard_normal((n_out, n_in)).astype(np.float16).view(np.uint16)
+    xbuf = np.full((m, n_in + 5), 1e30, dtype=np.float32)
+    xbuf[:, :n_in] = g.standard_normal((m, n_in))
+    d_x = to_dev(xbuf, torch)[:, :n_in]
+    ybuf = torch.full((m, n_out + 3), -1.0, dtype=torch.float32, device="cuda")
+    hs.f16_gemv(to_dev(w16.view(np.int16), torch), d_x, ybuf[:, :n_out])
+    hs.sync()
+    got = ybuf.cpu().numpy()
+    assert (bits(got[:, :n_out]) == bits(oracle.f16_gemv(w16, xbuf[:, :n_in]))).all()
+    assert (got[:, n_out:] == -1.0).all()
+    bad = torch.zeros((4, 20), dtype=torch.float16, device="cuda")        # n_in % 8 != 0
+    with pytest.raises(GeistHipError):
+        hs.f16_gemv(bad, torch.zeros((1, 20), device="cuda"), torch.zeros((1, 4), device="cuda"))
+
+
+@pytest.mark.parametrize("rows,n", [(1, 2560), (5, 1536), (17, 4096), (3, 7), (2, 300)])
+def test_rmsnorm_rows_bit_exact(hs, oracle, rows, n):
+    g = np.random.default_rng(rows * 100 + n)
+    x = (g.standard_normal((rows, n)) * g.choice([1e-3, 1.0, 50.0], (rows, 1))).astype(np.float32)
+    w = (1.0 + 0.2 * g.standard_normal(n)).astype(np.float32)
+    for eps in (1e-6, 1e-5):
+        d_x = to_dev(x, torch)
+        y = torch.empty_like(d_x)
+        hs.rmsnorm(d_x, to_dev(w, torch), eps, y)
+        hs.sync()
+        assert (bits(y.cpu().numpy()) == bits(oracle.rmsnorm(x, w, eps))).all()
+        hs.rmsnorm(d_x, to_dev(w, torch), eps, d_x)                        # in place
+        hs.sync()
+        assert (bits(d_x.cpu().numpy()) == bits(oracle.rmsnorm(x, w, eps))).all()
+
+
+def test_head_to_token_without_leaving_the_device(hs, oracle):
+    """head.c:94-188 end to end: norm -> lm_head -> sampler, logits never on the host. Equal to
+    the oracle's chain on the oracle's logits, token for token."""
+    from geistlib_amd import HipSampler, SampleParams
+    g = np.random.default_rng(12)
+    vocab, d_model, k = 32000, 2560, 6
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16).view(np.uint16)
+    hidden = (g.standard_normal((k, d_model)) * 3).astype(np.float32)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    u = g.random(k).astype(np.float32)
+    d_h = to_dev(hidden, torch)
+    hs.rmsnorm(d_h, to_dev(norm_w, torch), 1e-6, d_h)
+    logits = torch.empty((k, vocab), dtype=torch.float32, device="cuda")
+    hs.f16_gemv(to_dev(w16.view(np.int16), torch), d_h, logits)
+    out = torch.empty(k, dtype=torch.int32, device="cuda")
+    prm = dict(temperature=0.8, top_k=40, top_p=0.95)
+    hs.sample(HipSampler.rows(logits), SampleParams.make(**prm), to_dev(u, torch), out)
+    hs.sync()
+    want_logits = oracle.f16_gemv(w16, oracle.rmsnorm(hidden, norm_w, 1e-6))
+    assert (bits(logits.cpu().numpy()) == bits(want_logits)).all()
+    want = [oracle.chain_u(want_logits[r], float(u[r]), **prm)[0] for r in range(k)]
+    assert out.cpu().tolist() == want
