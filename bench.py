@@ -144,6 +144,105 @@ def bench_spec(w, args):
     print(json.dumps(result))
 
 
+def bench_lm_head(args, m_rows):
+    """Workload lm_head[_mN]: the tail of a decode step for BitNet-2B-4T's geometry, the case the
+    reference's F16 lm_head kernel was written for (cpu_x86/kernel_f16_gemv.h:7-12): RMS norm of
+    the hidden row(s), the tied F16 lm_head [128256 x 2560] (657 MB, read once per step), then the
+    headline sampler configuration on the logits, which never leave the device. A step is one
+    such tail for m_rows rows; the dominant kernel is the projection."""
+    import torch
+    from geistlib_amd import HipSampler, SampleParams
+    from geistlib_amd.workloads import xorshift_units
+    vocab, d_model = 128256, 2560
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    # three copies of the table (1.97 GB): every step's weights come from HBM
+    tables = [(torch.randn((vocab, d_model), device=dev, generator=g) * 0.05).to(torch.float16)
+              for _ in range(3)]
+    hidden = torch.randn((m_rows, d_model), device=dev, generator=g) * 3
+    norm_w = 1.0 + 0.1 * torch.randn((d_model,), device=dev, generator=g)
+    u, _ = xorshift_units(7, m_rows)
+    d_u = torch.from_numpy(u).to(dev)
+    normed = torch.empty_like(hidden)
+    logits = torch.empty((m_rows, vocab), dtype=torch.float32, device=dev)
+    out = torch.empty(m_rows, dtype=torch.int32, device=dev)
+    hs = HipSampler(max_rows=max(m_rows, 1), max_vocab=vocab)
+    prm = SampleParams.make(temperature=0.7, top_k=40, top_p=0.9)
+    rows = HipSampler.rows(logits)
+
+    def step(i=0):
+        hs.rmsnorm(hidden, norm_w, 1e-6, normed)
+        hs.f16_gemv(tables[i % len(tables)], normed, logits)
+        hs.sample(rows, prm, d_u, out)
+
+    for i in range(args.warmup):
+        step(i)
+    hs.sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    hs.sync()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed * 1e3 / args.steps
+    ids_gpu = out.cpu().numpy()
+    kernel_us = hs.time_f16_gemv(tables, normed, logits, args.steps)
+    w_bytes = vocab * d_model * 2
+    achieved = w_bytes / (kernel_us * 1e-6) / 1e9
+    result = {
+        "metric": "sampled rows/s", "value": round(m_rows * args.steps / elapsed, 1),
+        "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 weights x f32 activations, f32 accumulation",
+        "data": "synthetic",
+        "config": {"workload": f"lm_head_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
+                   "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
+                   "top_p": 0.9},
+        "us_per_step": round(ms * 1e3, 3),
+        "weight_copies_rotated": len(tables),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_f16_gemv", "kernel_us": round(kernel_us, 3),
+                     "kernel_algorithmic_bytes": w_bytes,
+                     "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
+    }
+    if not args.no_cpu:
+        # the reference's own kernel, compiled from its tree (oracle/_ref), on this host's cores;
+        # where it was not built, the oracle's scalar restatement on one core
+        from oracle_lib import Oracle, load_ref_f16gemv
+        wt = tables[(args.steps - 1) % len(tables)].cpu().numpy().view(np.uint16)
+        x_host = normed.cpu().numpy()
+        o = Oracle()
+        ref = load_ref_f16gemv(fast=True)
+        y = np.empty(vocab, dtype=np.float32)
+        reps, t_used = 0, 0.0
+        while reps < 10 and t_used < 10.0:
+            t1 = time.perf_counter()
+            if ref is not None:
+                ref.f16_gemv_m1(vocab, d_model, x_host[0].ctypes.data_as(C.POINTER(C.c_float)),
+                                wt.ctypes.data_as(C.POINTER(C.c_uint16)),
+                                y.ctypes.data_as(C.POINTER(C.c_float)))
+            else:
+                y = o.f16_gemv(wt, x_host[0])
+            t_used += time.perf_counter() - t1
+            reps += 1
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 10 ** 6)
+        result["cpu_baseline"] = {
+            "value": round(reps / t_used, 2), "unit": "rows/s",
+            "cores": cores if ref is not None else 1,
+            "kind": "reference" if ref is not None else "port",
+            "sample": f"{reps} calls of f16_gemv_m1 on one hidden row (the projection only, "
+                      "no norm, no sampling)"}
+        # parity of the whole tail on the last step's inputs
+        want_logits = o.f16_gemv(wt, o.rmsnorm(hidden.cpu().numpy(), norm_w.cpu().numpy(), 1e-6))
+        same_bits = bool((want_logits.view(np.uint32) == logits.cpu().numpy().view(np.uint32)).all())
+        want_ids = [o.chain_u(want_logits[r], float(u[r]), temperature=0.7, top_k=40, top_p=0.9)[0]
+                    for r in range(m_rows)]
+        result["parity"] = {"rows": m_rows, "logits_bit_identical": same_bits,
+                            "ids_differ": int((np.array(want_ids) != ids_gpu).sum())}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -168,6 +267,9 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: the sampling path has no CPU fallback")
 
+    if args.workload.startswith("lm_head"):
+        m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
+        return bench_lm_head(args, m)
     w = build_workload(args.workload)
     if args.workload == "cfg5":
         return bench_spec(w, args)

@@ -89,6 +89,8 @@ def load_library():
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
     lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_time_f16_gemv_rows.argtypes = [vp, C.POINTER(vp), sz, sz, sz, vp, sz, sz, vp, sz,
+                                                 i32, C.POINTER(C.c_double)]
     _LIB = lib
     return lib
 
@@ -219,6 +221,18 @@ class HipSampler:
         self._check(self.lib.geist_hip_f16_gemv_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
+
+    def time_f16_gemv(self, weight_copies, x, y, launches):
+        """Mean duration in microseconds of one f16_gemv call (HIP events on the sampler's stream
+        around `launches` back-to-back calls rotating over the weight copies)."""
+        n_out, n_in = weight_copies[0].shape
+        m = x.shape[0]
+        arr = (C.c_void_p * len(weight_copies))(*[w.data_ptr() for w in weight_copies])
+        ms = C.c_double()
+        self._check(self.lib.geist_hip_time_f16_gemv_rows(
+            self.h, arr, len(weight_copies), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in,
+            m, _ptr(y), y.stride(0) if m > 1 else n_out, int(launches), C.byref(ms)))
+        return ms.value * 1e3 / launches
 
     def time_stream_kernel(self, rows, params, uniforms, out, launches):
         """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around

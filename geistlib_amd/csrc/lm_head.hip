@@ -60,8 +60,13 @@ __device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long 
     for (int i = 0; i < STAGE_LOADS; ++i) {
         const long row = row0 + 8 * i + (lane >> 3);
         g.w[i]         = make_uint4(0u, 0u, 0u, 0u);
-        if (row < n_out && col < n_in)
-            g.w[i] = *reinterpret_cast<const uint4 *>(w + row * n_in + col);
+        if (row < n_out && col < n_in) {
+            /* read once, and far more than the caches hold: non-temporal */
+            typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+            const nt_u4 t =
+                __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(w + row * n_in + col));
+            g.w[i] = make_uint4(t.x, t.y, t.z, t.w);
+        }
     }
 }
 
@@ -73,6 +78,32 @@ __device__ __forceinline__ void stage_load_x(const float *__restrict__ x, long l
     for (int m = 0; m < MT; ++m) {
         const int mm = m < n_m ? m : n_m - 1; /* rows beyond n_m repeat the last one, unstored */
         gx.x[m]      = col < n_in ? x[mm * ld_x + col] : 0.0f;
+    }
+}
+
+/* One step of the chains: eight weights of this lane's row and half against the activations of
+ * the same columns. MASKED: lanes with keep == false leave their chains alone. */
+template <int MT, bool MASKED>
+__device__ __forceinline__ void gemv_step(const uint8_t *tile, const float (*xs)[STAGE_COLS],
+                                          int my_row, int half, int t, bool keep,
+                                          float (&acc)[MT][8]) {
+    const uint4 q =
+        *reinterpret_cast<const uint4 *>(tile + my_row * TILE_PITCH + t * 32 + half * 16);
+    const float2 f01 = __half22float2(*reinterpret_cast<const __half2 *>(&q.x));
+    const float2 f23 = __half22float2(*reinterpret_cast<const __half2 *>(&q.y));
+    const float2 f45 = __half22float2(*reinterpret_cast<const __half2 *>(&q.z));
+    const float2 f67 = __half22float2(*reinterpret_cast<const __half2 *>(&q.w));
+    const float  wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const float4 xa = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8]);
+        const float4 xb = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8 + 4]);
+        const float  xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float f = __builtin_fmaf(wf[i], xv[i], acc[m][i]);
+            acc[m][i]     = (!MASKED || keep) ? f : acc[m][i];
+        }
     }
 }
 
@@ -126,35 +157,18 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         }
         /* steps of this stage: whole blocks of 16 columns, and at the end of the row possibly
          * a block of 8, which only extends chains 0..7 (the lanes with half == 0) */
-        const int left  = n_in - s * STAGE_COLS;
-        const int full  = left >= STAGE_COLS ? 4 : left / 16;
-        const bool tail8 = left < STAGE_COLS && (left & 15) == 8;
+        const int left = n_in - s * STAGE_COLS;
+        if (left >= STAGE_COLS) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const bool whole = t < full;
-            const bool eight = tail8 && t == full && half == 0;
-            if (!whole && !(tail8 && t == full))
-                continue;
-            const uint4 q = *reinterpret_cast<const uint4 *>(tile + my_row * TILE_PITCH + t * 32 +
-                                                             half * 16);
-            const __half2 h01 = *reinterpret_cast<const __half2 *>(&q.x);
-            const __half2 h23 = *reinterpret_cast<const __half2 *>(&q.y);
-            const __half2 h45 = *reinterpret_cast<const __half2 *>(&q.z);
-            const __half2 h67 = *reinterpret_cast<const __half2 *>(&q.w);
-            const float2  f01 = __half22float2(h01), f23 = __half22float2(h23);
-            const float2  f45 = __half22float2(h45), f67 = __half22float2(h67);
-            const float   wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const float4 xa = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8]);
-                const float4 xb = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8 + 4]);
-                const float  xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float f = __builtin_fmaf(wf[i], xv[i], acc[m][i]);
-                    acc[m][i]     = (whole || eight) ? f : acc[m][i];
-                }
-            }
+            for (int t = 0; t < 4; ++t)
+                gemv_step<MT, false>(tile, xs, my_row, half, t, true, acc);
+        } else {
+            const int  full  = left / 16;
+            const bool tail8 = (left & 15) == 8;
+            for (int t = 0; t < full; ++t)
+                gemv_step<MT, false>(tile, xs, my_row, half, t, true, acc);
+            if (tail8)
+                gemv_step<MT, true>(tile, xs, my_row, half, full, half == 0, acc);
         }
     }
     /* (chain j + chain j+8), (lane i + lane i+4), ((0+1) + (2+3)): kernel_f16_gemv.c:25-32, 59 */

@@ -790,6 +790,36 @@ int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_h
     return rc ? rc : after_launch(s, "plain read");
 }
 
+int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_w_f16,
+                                 size_t n_weights, size_t n_out, size_t n_in, const float *d_x,
+                                 size_t ld_x, size_t n_rows, float *d_y, size_t ld_y, int launches,
+                                 double *ms_total) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (launches < 1 || !ms_total || !d_w_f16 || n_weights < 1)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no weights or null result");
+    for (size_t i = 0; i < n_weights; ++i) { /* argument checks and a warm-up of each copy */
+        const int rc = geist_hip_f16_gemv_rows(s, d_w_f16[i], n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+        if (rc)
+            return rc;
+    }
+    hipEvent_t a, b;
+    HIPCHK(s, hipEventCreate(&a));
+    HIPCHK(s, hipEventCreate(&b));
+    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
+    for (int i = 0; i < launches && !rc; ++i)
+        rc = geist_hip_f16_gemv_rows(s, d_w_f16[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
+                                     n_rows, d_y, ld_y);
+    float ms = 0.0f;
+    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
+                hipEventElapsedTime(&ms, a, b) != hipSuccess))
+        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
+    (void) hipEventDestroy(a);
+    (void) hipEventDestroy(b);
+    *ms_total = ms;
+    return rc;
+}
+
 int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,
                              float *d_out_units) {
     if (!s)

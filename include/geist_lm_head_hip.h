@@ -36,6 +36,14 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                             size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
                             size_t ld_y);
 
+/* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
+ * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
+ * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */
+int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_w_f16,
+                                 size_t n_weights, size_t n_out, size_t n_in, const float *d_x,
+                                 size_t ld_x, size_t n_rows, float *d_y, size_t ld_y, int launches,
+                                 double *ms_total);
+
 #ifdef __cplusplus
 }
 #endif
