@@ -5,6 +5,7 @@
  */
 #include "geist_head_hip.h"
 #include "geist_sampler_hip.h"
+#include "geist_lm_head_hip.h"
 
 #include <stdio.h>
 #include <stdlib.h>
@@ -25,6 +26,9 @@ struct geist_hip_head {
     int32_t  *d_drafts; /* m_max */
     int32_t  *d_nacc;
     int32_t  *d_ngram;  /* seed, history length, count, matched length, 16 drafts */
+    float    *d_normed; /* m_max x d_model_cap: the normed hidden rows */
+    size_t    d_model_cap;
+    float    *d_logits; /* m_max x vocab, written by the lm_head, read by the sampler */
     char      err[256];
 };
 
@@ -95,6 +99,8 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         geist_hip_free(h->hs, h->d_drafts);
         geist_hip_free(h->hs, h->d_nacc);
         geist_hip_free(h->hs, h->d_ngram);
+        geist_hip_free(h->hs, h->d_normed);
+        geist_hip_free(h->hs, h->d_logits);
         geist_hip_sampler_destroy(h->hs);
     }
     free(h);
@@ -151,6 +157,45 @@ int geist_hip_head_finalize_one_row(struct geist_hip_head *h, const float *d_log
 int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logits, size_t k,
                                   int32_t *out_tokens) {
     return finalize(h, d_logits, k, out_tokens);
+}
+
+int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
+                                    size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                    float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
+                                    int32_t *out_tokens) {
+    if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed_f16 == nullptr ||
+        out_tokens == nullptr || k == 0 || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (k > h->m_max)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
+    void *p = nullptr;
+    if (h->d_logits == nullptr) {
+        if (geist_hip_malloc(h->hs, h->m_max * h->vocab * sizeof(float), &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "logit buffer");
+        h->d_logits = p;
+    }
+    if (h->d_model_cap < d_model) {
+        geist_hip_free(h->hs, h->d_normed);
+        h->d_normed    = nullptr;
+        h->d_model_cap = 0;
+        if (geist_hip_malloc(h->hs, h->m_max * d_model * sizeof(float), &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
+        h->d_normed    = p;
+        h->d_model_cap = d_model;
+    }
+    /* head.c:99-101, then 114-126 */
+    int rc = geist_hip_rmsnorm_rows(h->hs, d_hidden, ld_hidden, d_norm_weight, rms_eps, k, d_model,
+                                    h->d_normed, d_model);
+    if (rc == GEIST_HIP_OK)
+        rc = geist_hip_f16_gemv_rows(h->hs, d_embed_f16, h->vocab, d_model, h->d_normed, d_model, k,
+                                     h->d_logits, h->vocab);
+    if (rc != GEIST_HIP_OK)
+        return head_fail(h, rc, "output head");
+    return finalize(h, h->d_logits, k, out_tokens);
+}
+
+const float *geist_hip_head_logits(const struct geist_hip_head *h) {
+    return h != nullptr ? h->d_logits : nullptr;
 }
 
 int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,

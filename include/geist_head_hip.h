@@ -10,6 +10,8 @@
  *   geist_hip_head_finalize_batch     sampler part of finalize_logits_batch (head.c:274-304)
  *   geist_hip_head_argmax_f32      the backend slot fused->argmax_f32
  *                                  (include/geist_backend.h:414-421)
+ *   geist_hip_head_project_finalize  output norm + tied F16 lm_head + the above, logits never
+ *                                  on the host (head.c:94-188, 224-304)
  *   geist_hip_head_propose_drafts  the n-gram drafter of geist_session_decode_speculative
  *                                  (src/engine/session.c:437-513, 564-572)
  *   geist_hip_head_spec_accept     the accept loop of geist_session_decode_speculative
@@ -64,6 +66,23 @@ int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logit
                                   int32_t *out_tokens);
 int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,
                               int32_t *out_index);
+
+/* The whole tail of a forward pass for k <= m_max rows of final hidden states, on the device
+ * (head.c:94-188 for one row, 224-304 for a batch): RMS norm with the output-norm weight
+ * (head.c:99-101), the tied F16 lm_head (head.c:114-126; [vocab, d_model] binary16, row-major,
+ * 16-byte aligned, d_model a multiple of 8), the soft-cap and the session's sampler. The logits
+ * live in a buffer of the head and are never copied out; they equal, bit for bit, what the
+ * reference's cpu_scalar_rmsnorm and f16_gemv_m1 produce, so the tokens are those of
+ * geist_hip_head_finalize_batch on the reference's logits. Row r of d_hidden starts at
+ * d_hidden + r * ld_hidden and is left untouched. */
+int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
+                                    size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                    float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
+                                    int32_t *out_tokens);
+/* The logits of the last geist_hip_head_project_finalize call ([k, vocab], row stride vocab,
+ * device memory; soft-cap not applied: the sampler applies it while reading), for scoring with
+ * geist_hip_logprob_rows in place of geist_session_peek_logits. NULL before the first call. */
+const float *geist_hip_head_logits(const struct geist_hip_head *h);
 
 /* The drafting step of one speculative round (session.c:564-572) for a token history kept in
  * device memory: seed is the pending next token (what the finalize call of the step before

@@ -58,6 +58,11 @@ def host():
     lib.geist_hip_head_propose_drafts.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int32,
                                                   C.c_size_t, C.POINTER(C.c_int32),
                                                   C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    lib.geist_hip_head_project_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                                    C.c_void_p, C.c_float, C.c_void_p, C.c_size_t,
+                                                    C.POINTER(C.c_int32)]
+    lib.geist_hip_head_logits.restype = C.c_void_p
+    lib.geist_hip_head_logits.argtypes = [C.c_void_p]
     lib.geist_hip_head_spec_accept.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
                                                C.POINTER(C.c_int32), C.c_int, C.c_size_t,
                                                C.POINTER(C.c_int32), C.POINTER(C.c_size_t)]
@@ -371,3 +376,35 @@ def test_head_propose_drafts_follows_the_reference_drafter(host, oracle):
     assert host.geist_hip_head_propose_drafts(h, None, 0, 3, 4, out, C.byref(n_out), None) == 0
     assert n_out.value == 1 and out[0] == 3
     host.geist_hip_head_destroy(h)
+
+
+def test_head_project_finalize_keeps_the_logits_on_the_device(host, oracle):
+    """head.c:94-188 / 224-304 in one call: output norm, tied F16 lm_head, soft-cap, sampler with
+    the session's RNG. The tokens are those of the oracle's session on the oracle's logits."""
+    g = np.random.default_rng(77)
+    vocab, d_model, k, cap = 20000, 1536, 5, 30.0
+    w16 = (g.standard_normal((vocab, d_model)) * 0.08).astype(np.float16)
+    hidden = (g.standard_normal((k, d_model + 4)) * 2).astype(np.float32)   # padded row stride
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    d_w = torch.from_numpy(w16.view(np.int16)).cuda()
+    d_hid = torch.from_numpy(hidden).cuda()
+    d_nw = torch.from_numpy(norm_w).cuda()
+    want_logits = oracle.f16_gemv(w16.view(np.uint16), oracle.rmsnorm(hidden[:, :d_model], norm_w, 1e-6))
+    for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.9, 0), (1.1, 1.0, 0)]:
+        h = make_head(host, vocab, 0, cap)
+        opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        out = (C.c_int32 * k)()
+        rc = host.geist_hip_head_project_finalize(h, C.c_void_p(d_hid.data_ptr()), d_model + 4, k,
+                                                  C.c_void_p(d_nw.data_ptr()), 1e-6,
+                                                  C.c_void_p(d_w.data_ptr()), d_model, out)
+        assert rc == 0, host.geist_hip_head_errmsg(h)
+        sess = oracle.session(T, p, top_k, seed=4242)
+        assert list(out) == oracle.finalize_batch(sess, want_logits, softcap=cap).tolist(), (T, p, top_k)
+        ptr = host.geist_hip_head_logits(h)
+        got = torch.empty((k, vocab), dtype=torch.float32, device="cuda")
+        C.cdll.LoadLibrary("libamdhip64.so").hipMemcpy(C.c_void_p(got.data_ptr()), C.c_void_p(ptr),
+                                                       C.c_size_t(k * vocab * 4), 3)
+        assert (got.cpu().numpy().view(np.uint32) == want_logits.view(np.uint32)).all()
+        host.geist_hip_head_destroy(h)
+    assert (d_hid.cpu().numpy() == hidden).all()                             # input untouched
