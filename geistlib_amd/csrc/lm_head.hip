@@ -187,6 +187,130 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
     }
 }
 
+/* The projection for several activation rows. Here a lane owns all sixteen chains of one weight
+ * row (a wavefront works on 64 rows), so the activations of a step are the same for every lane
+ * and come from scalar registers: each converted weight feeds n_m multiply-adds whose second
+ * operand costs neither LDS traffic nor vector registers. The weights take the same way through
+ * a private LDS tile as in k_f16_gemv. */
+constexpr int ROWS_WAVE_B  = 64;
+constexpr int ROWS_BLOCK_B = ROWS_WAVE_B * LM_WAVES;
+constexpr int STAGE_LOADS_B = 8; /* 64 rows x 8 segments / 64 lanes */
+
+struct StageRegsB {
+    uint4 w[STAGE_LOADS_B];
+};
+
+__device__ __forceinline__ void stage_load_b(const uint16_t *__restrict__ w, long row0, long n_out,
+                                             int n_in, int stage, int lane, StageRegsB &g) {
+    const int col = stage * STAGE_COLS + (lane & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < STAGE_LOADS_B; ++i) {
+        const long row = row0 + 8 * i + (lane >> 3);
+        g.w[i]         = make_uint4(0u, 0u, 0u, 0u);
+        if (row < n_out && col < n_in) {
+            typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+            const nt_u4 t =
+                __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(w + row * n_in + col));
+            g.w[i] = make_uint4(t.x, t.y, t.z, t.w);
+        }
+    }
+}
+
+/* Eight chains (one accumulator of the reference) of this lane's row against the activations
+ * x[m][col .. col + 8), which are uniform over the wavefront. */
+template <int MT>
+__device__ __forceinline__ void gemv_half_step(const uint8_t *row_tile, int byte_off,
+                                               const float *__restrict__ x, long ld_x, int n_m,
+                                               int col, float (&acc)[MT][16], int chain0) {
+    const uint4  q   = *reinterpret_cast<const uint4 *>(row_tile + byte_off);
+    const float2 f01 = __half22float2(*reinterpret_cast<const __half2 *>(&q.x));
+    const float2 f23 = __half22float2(*reinterpret_cast<const __half2 *>(&q.y));
+    const float2 f45 = __half22float2(*reinterpret_cast<const __half2 *>(&q.z));
+    const float2 f67 = __half22float2(*reinterpret_cast<const __half2 *>(&q.w));
+    float        wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
+    /* keep the conversion a separate instruction: folded into a mixed-precision multiply-add it
+     * is repeated per activation row, and that instruction takes no scalar operand, so every
+     * activation would be copied to a vector register first */
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        asm("" : "+v"(wf[i]));
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const float *xm = x + (long) (m < n_m ? m : n_m - 1) * ld_x + col; /* uniform address */
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc[m][chain0 + i] = __builtin_fmaf(wf[i], xm[i], acc[m][chain0 + i]);
+    }
+}
+
+template <int MT>
+__global__ __launch_bounds__(LM_TPB) void k_f16_gemv_batched(const uint16_t *__restrict__ w,
+                                                             long n_out, int n_in,
+                                                             const float *__restrict__ x, long ld_x,
+                                                             int n_m, float *__restrict__ y,
+                                                             long ld_y) {
+    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
+    const int  lane = threadIdx.x & (LM_WAVE - 1);
+    const int  wave = __builtin_amdgcn_readfirstlane(threadIdx.x / LM_WAVE);
+    const long row0 = (long) blockIdx.x * ROWS_BLOCK_B + wave * ROWS_WAVE_B;
+    if (row0 >= n_out)
+        return;
+    uint8_t       *tile     = s_tile[wave];
+    const uint8_t *row_tile = tile + lane * TILE_PITCH;
+
+    float acc[MT][16];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc[m][i] = 0.0f;
+
+    const int  n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    StageRegsB g0, g1;
+    stage_load_b(w, row0, n_out, n_in, 0, lane, g0);
+    if (n_stage > 1)
+        stage_load_b(w, row0, n_out, n_in, 1, lane, g1);
+    for (int s = 0; s < n_stage; ++s) {
+#pragma unroll
+        for (int i = 0; i < STAGE_LOADS_B; ++i)
+            *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
+                g0.w[i];
+        g0 = g1;
+        if (s + 2 < n_stage)
+            stage_load_b(w, row0, n_out, n_in, s + 2, lane, g1);
+        const int col0 = s * STAGE_COLS;
+        const int left = n_in - col0;
+        if (left >= STAGE_COLS) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                gemv_half_step<MT>(row_tile, t * 32, x, ld_x, n_m, col0 + t * 16, acc, 0);
+                gemv_half_step<MT>(row_tile, t * 32 + 16, x, ld_x, n_m, col0 + t * 16 + 8, acc, 8);
+            }
+        } else {
+            const int full = left / 16;
+            for (int t = 0; t < full; ++t) {
+                gemv_half_step<MT>(row_tile, t * 32, x, ld_x, n_m, col0 + t * 16, acc, 0);
+                gemv_half_step<MT>(row_tile, t * 32 + 16, x, ld_x, n_m, col0 + t * 16 + 8, acc, 8);
+            }
+            if ((left & 15) == 8) /* the block of eight extends chains 0..7 */
+                gemv_half_step<MT>(row_tile, full * 32, x, ld_x, n_m, col0 + full * 16, acc, 0);
+        }
+    }
+    const long row = row0 + lane;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            v[i] = dadd(acc[m][i], acc[m][i + 8]);
+        const float q0 = dadd(v[0], v[4]), q1 = dadd(v[1], v[5]);
+        const float q2 = dadd(v[2], v[6]), q3 = dadd(v[3], v[7]);
+        const float sum = dadd(dadd(q0, q1), dadd(q2, q3));
+        if (row < n_out && m < n_m)
+            y[m * ld_y + row] = sum;
+    }
+}
+
 /* One workgroup per row. The reference adds the squares in double in index order; the order of
  * a double sum only shows in the binary32 result when 1 / sqrt(mean + eps) lies within the
  * sum's error of the middle between two binary32 values. The workgroup adds in a fixed parallel
@@ -239,16 +363,15 @@ void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const fl
 void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
                      const float *x, long ld_x, int n_m, float *y, long ld_y) {
     const dim3 grid((unsigned) ((n_out + ROWS_BLOCK - 1) / ROWS_BLOCK)), block(LM_TPB);
+    const dim3 grid_b((unsigned) ((n_out + ROWS_BLOCK_B - 1) / ROWS_BLOCK_B));
     if (n_m <= 1)
         k_f16_gemv<1><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
     else if (n_m <= 2)
         k_f16_gemv<2><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
-    else if (n_m <= 4)
-        k_f16_gemv<4><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
-    else if (n_m <= 8)
-        k_f16_gemv<8><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+    else if (n_m <= 4) /* (with 8 rows the batched kernel's 128 accumulators leave no room) */
+        k_f16_gemv_batched<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
     else
-        k_f16_gemv<16><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+        k_f16_gemv<8><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
 }
 
 } // namespace gs

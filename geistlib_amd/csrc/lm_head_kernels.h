@@ -11,7 +11,7 @@
 
 namespace gs {
 
-constexpr int GEMV_M_MAX = 16; /* activation rows one pass over the weights serves */
+constexpr int GEMV_M_MAX = 8; /* activation rows one pass over the weights serves */
 
 /* y = x * w * rsqrt(mean(x^2) + eps) per row; y may alias x. */
 void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const float *w, float eps,

@@ -29,7 +29,7 @@ int geist_hip_rmsnorm_rows(geist_hip_sampler *s, const float *d_x, size_t ld_x,
  *   d_y[m * ld_y + r] = sum_i f16_to_f32(d_w_f16[r * n_in + i]) * d_x[m * ld_x + i]
  * for every activation row m < n_rows, with the reference's order of summation (sixteen chains
  * of fused multiply-adds folded in a fixed tree), so each row equals what f16_gemv_m1 returns
- * for it. The weights are read once for up to 16 activation rows. n_in must be a multiple of 8
+ * for it. The weights are read once for up to 8 activation rows. n_in must be a multiple of 8
  * (GEIST_HIP_E_UNSUPPORTED otherwise: the reference adds a remainder element by element, with
  * rounding that depends on how it was compiled); d_w_f16 must be 16-byte aligned. */
 int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
