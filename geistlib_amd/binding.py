@@ -89,6 +89,8 @@ def load_library():
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
     lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
+                                                  C.POINTER(SampleParams), vp, vp, i32, vp]
     lib.geist_hip_time_f16_gemv_rows.argtypes = [vp, C.POINTER(vp), sz, sz, sz, vp, sz, sz, vp, sz,
                                                  i32, C.POINTER(C.c_double)]
     _LIB = lib
@@ -221,6 +223,18 @@ class HipSampler:
         self._check(self.lib.geist_hip_f16_gemv_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
+
+    def project_sample(self, hidden, norm_w, eps, embed_f16, logits, params, uniforms, out,
+                       normed=None, rng_states=None, shared=True):
+        """Norm -> F16 lm_head -> sampler for hidden [rows, d_model]; logits [rows, vocab] is
+        written on the way."""
+        rows, d_model = hidden.shape
+        vocab = embed_f16.shape[0]
+        self._check(self.lib.geist_hip_project_sample_rows(
+            self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
+            _ptr(norm_w), eps, _ptr(embed_f16), vocab, _ptr(normed), _ptr(logits),
+            logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
+            _ptr(rng_states), int(shared), _ptr(out)))
 
     def time_f16_gemv(self, weight_copies, x, y, launches):
         """Mean duration in microseconds of one f16_gemv call (HIP events on the sampler's stream

@@ -52,13 +52,26 @@ struct StageX {
     float x[MT];
 };
 
-__device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long row0, long n_out,
+/* Which weight row a wavefront's virtual row r (0..31) is. Plain: 32 consecutive rows per
+ * wavefront task. Sampler layout: task (chunk, t) is thread t of chunk `chunk` of the sampler's
+ * top-k scan (chunks of 8192 logits, thread t owns the float4 groups 4 * (j * 256 + t), j < 8),
+ * so that the maximum over the task's 32 results is that thread's maximum. */
+template <bool SL>
+__device__ __forceinline__ long virtual_row(long task, int r) {
+    if (!SL)
+        return task * ROWS_WAVE + r;
+    const long chunk = task >> 8, t = task & 255;
+    return chunk * 8192 + 4 * ((long) (r >> 2) * 256 + t) + (r & 3);
+}
+
+template <bool SL>
+__device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long task, long n_out,
                                            int n_in, int stage, int lane, StageRegs &g) {
     const int seg = lane & 7;
     const int col = stage * STAGE_COLS + seg * 8;
 #pragma unroll
     for (int i = 0; i < STAGE_LOADS; ++i) {
-        const long row = row0 + 8 * i + (lane >> 3);
+        const long row = virtual_row<SL>(task, 8 * i + (lane >> 3));
         g.w[i]         = make_uint4(0u, 0u, 0u, 0u);
         if (row < n_out && col < n_in) {
             /* read once, and far more than the caches hold: non-temporal */
@@ -79,6 +92,24 @@ __device__ __forceinline__ void stage_load_x(const float *__restrict__ x, long l
         const int mm = m < n_m ? m : n_m - 1; /* rows beyond n_m repeat the last one, unstored */
         gx.x[m]      = col < n_in ? x[mm * ld_x + col] : 0.0f;
     }
+}
+
+/* 1 / sqrt(mean(x^2) + eps) as cpu_scalar_rmsnorm rounds it (elementwise.c:270-274). The
+ * reference adds the squares in double in index order; the order of a double sum only shows in
+ * the binary32 result when the value lies within the sums' error of the middle between two
+ * binary32 values, and then `sequential` repeats the sum in the reference's order. */
+__device__ __forceinline__ bool rms_inv_is_safe(double sumsq, int n, float eps, float &f) {
+    const double r  = 1.0 / sqrt(sumsq / (double) n + (double) eps);
+    f               = (float) r;
+    const float  fn = r > (double) f ? nextafterf(f, __builtin_inff()) : nextafterf(f, -__builtin_inff());
+    const double mid = 0.5 * ((double) f + (double) fn);
+    return !(fabs(r - mid) <= fabs(r) * (double) n * 0x1p-50);
+}
+__device__ __forceinline__ float rms_inv_sequential(const float *__restrict__ xr, int n, float eps) {
+    double sumsq = 0.0;
+    for (int i = 0; i < n; ++i)
+        sumsq += (double) xr[i] * (double) xr[i];
+    return (float) (1.0 / sqrt(sumsq / (double) n + (double) eps));
 }
 
 /* One step of the chains: eight weights of this lane's row and half against the activations of
@@ -109,17 +140,21 @@ __device__ __forceinline__ void gemv_step(const uint8_t *tile, const float (*xs)
 
 } // namespace
 
-template <int MT>
+template <int MT, bool SL>
 __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict__ w, long n_out,
                                                      int n_in, const float *__restrict__ x,
                                                      long ld_x, int n_m, float *__restrict__ y,
-                                                     long ld_y) {
+                                                     long ld_y, GemvFuse fuse) {
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][TILE_BYTES];
     __shared__ __align__(16) float   s_x[LM_WAVES][MT][STAGE_COLS];
     const int  lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
-    const long row0 = (long) blockIdx.x * ROWS_BLOCK + wave * ROWS_WAVE;
-    if (row0 >= n_out)
-        return; /* (no workgroup barrier below) */
+    const long task = (long) blockIdx.x * LM_WAVES + wave;
+    if (virtual_row<SL>(task, 0) >= n_out) { /* (no workgroup barrier below) */
+        if (SL && lane < n_m && task < (long) fuse.n_chunks * 256)
+            fuse.tmax[((long) lane * fuse.n_chunks + (task >> 8)) * 256 + (task & 255)] =
+                __builtin_nanf(""); /* a scanning thread without an element is never chosen */
+        return;
+    }
     uint8_t *tile = s_tile[wave];
     float(*xs)[STAGE_COLS] = s_x[wave];
     const int my_row = lane >> 1, half = lane & 1;
@@ -134,12 +169,12 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
     const int n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
     StageRegs  g0, g1;
     StageX<MT> x0, x1;
-    stage_load(w, row0, n_out, n_in, 0, lane, g0);
+    stage_load<SL>(w, task, n_out, n_in, 0, lane, g0);
+    if (n_stage > 1)
+        stage_load<SL>(w, task, n_out, n_in, 1, lane, g1);
     stage_load_x<MT>(x, ld_x, n_m, n_in, 0, lane, x0);
-    if (n_stage > 1) {
-        stage_load(w, row0, n_out, n_in, 1, lane, g1);
+    if (n_stage > 1)
         stage_load_x<MT>(x, ld_x, n_m, n_in, 1, lane, x1);
-    }
     for (int s = 0; s < n_stage; ++s) {
         /* registers -> tile (this waits for the loads issued two stages ago) */
 #pragma unroll
@@ -152,7 +187,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         g0 = g1;
         x0 = x1;
         if (s + 2 < n_stage) {
-            stage_load(w, row0, n_out, n_in, s + 2, lane, g1);
+            stage_load<SL>(w, task, n_out, n_in, s + 2, lane, g1);
             stage_load_x<MT>(x, ld_x, n_m, n_in, s + 2, lane, x1);
         }
         /* steps of this stage: whole blocks of 16 columns, and at the end of the row possibly
@@ -172,7 +207,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         }
     }
     /* (chain j + chain j+8), (lane i + lane i+4), ((0+1) + (2+3)): kernel_f16_gemv.c:25-32, 59 */
-    const long row = row0 + my_row;
+    const long row = virtual_row<SL>(task, my_row);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         float v[8];
@@ -184,6 +219,16 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         const float sum = dadd(dadd(q0, q1), dadd(q2, q3));
         if (half == 0 && row < n_out && m < n_m)
             y[m * ld_y + row] = sum;
+        if (SL) {
+            /* the scanning thread's maximum over its elements of the row (NaN ignored, as the
+             * scan's v_max3_f32 does) */
+            float mx = row < n_out ? sum : -__builtin_inff();
+#pragma unroll
+            for (int d = 1; d < LM_WAVE; d <<= 1)
+                mx = __builtin_fmaxf(mx, __shfl_xor(mx, d, LM_WAVE));
+            if (lane == 0 && m < n_m)
+                fuse.tmax[((long) m * fuse.n_chunks + (task >> 8)) * 256 + (task & 255)] = mx;
+        }
     }
 }
 
@@ -334,19 +379,9 @@ __global__ __launch_bounds__(LM_TPB) void k_rmsnorm_rows(const float *__restrict
         __syncthreads();
     }
     if (tid == 0) {
-        double      sumsq = s_part[0];
-        double      r     = 1.0 / sqrt(sumsq / (double) n + (double) eps);
-        float       f     = (float) r;
-        /* distance of r from the nearer rounding boundary of f, relative to r; the two sums
-         * differ by less than n * 2^-52 relative, and r by half of that */
-        const float  fn  = r > (double) f ? nextafterf(f, __builtin_inff()) : nextafterf(f, -__builtin_inff());
-        const double mid = 0.5 * ((double) f + (double) fn);
-        if (fabs(r - mid) <= fabs(r) * (double) n * 0x1p-50) {
-            sumsq = 0.0;
-            for (int i = 0; i < n; ++i)
-                sumsq += (double) xr[i] * (double) xr[i];
-            f = (float) (1.0 / sqrt(sumsq / (double) n + (double) eps));
-        }
+        float f;
+        if (!rms_inv_is_safe(s_part[0], n, eps, f))
+            f = rms_inv_sequential(xr, n, eps);
         s_inv = f;
     }
     __syncthreads();
@@ -360,18 +395,31 @@ void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const fl
     k_rmsnorm_rows<<<dim3(n_rows), dim3(LM_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y);
 }
 
+bool f16_gemv_can_fuse(int n_m) { return n_m >= 1 && n_m <= 2; }
+
 void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
-                     const float *x, long ld_x, int n_m, float *y, long ld_y) {
-    const dim3 grid((unsigned) ((n_out + ROWS_BLOCK - 1) / ROWS_BLOCK)), block(LM_TPB);
+                     const float *x, long ld_x, int n_m, float *y, long ld_y,
+                     const GemvFuse *fuse) {
+    const dim3 block(LM_TPB);
+    const dim3 grid((unsigned) ((n_out + ROWS_BLOCK - 1) / ROWS_BLOCK));
     const dim3 grid_b((unsigned) ((n_out + ROWS_BLOCK_B - 1) / ROWS_BLOCK_B));
+    GemvFuse   none{};
+    if (fuse && fuse->tmax) { /* (the caller has asked f16_gemv_can_fuse) */
+        const dim3 grid_s((unsigned) (fuse->n_chunks * 256 / LM_WAVES));
+        if (n_m <= 1)
+            k_f16_gemv<1, true><<<grid_s, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, *fuse);
+        else
+            k_f16_gemv<2, true><<<grid_s, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, *fuse);
+        return;
+    }
     if (n_m <= 1)
-        k_f16_gemv<1><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+        k_f16_gemv<1, false><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
     else if (n_m <= 2)
-        k_f16_gemv<2><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+        k_f16_gemv<2, false><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
     else if (n_m <= 4) /* (with 8 rows the batched kernel's 128 accumulators leave no room) */
         k_f16_gemv_batched<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
     else
-        k_f16_gemv<8><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
+        k_f16_gemv<8, false><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
 }
 
 } // namespace gs

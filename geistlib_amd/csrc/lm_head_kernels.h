@@ -17,9 +17,22 @@ constexpr int GEMV_M_MAX = 8; /* activation rows one pass over the weights serve
 void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const float *w, float eps,
                          int n_rows, int n, float *y, long ld_y);
 
+/* What the projection can do on its way, for n_m <= 2 activation rows (f16_gemv_can_fuse):
+ * with tmax != NULL the work is dealt out in the layout of the sampler's top-k scan (chunks of
+ * 8192 logits, 256 threads) and tmax[(m * n_chunks + chunk) * 256 + t] receives the maximum of
+ * scanning thread t's logits of row m, so that the sampler can skip its own pass over the
+ * logits. (Folding the RMS norm into the projection as well was tried: the registers it takes
+ * cost the projection more than the small kernel it saves.) */
+struct GemvFuse {
+    float *tmax;
+    int    n_chunks;
+};
+bool f16_gemv_can_fuse(int n_m);
+
 /* y[m][r] = sum_i f16(W[r][i]) * x[m][i] for m < n_m <= GEMV_M_MAX; n_in a multiple of 8. */
 void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
-                     const float *x, long ld_x, int n_m, float *y, long ld_y);
+                     const float *x, long ld_x, int n_m, float *y, long ld_y,
+                     const GemvFuse *fuse = nullptr);
 
 } // namespace gs
 #endif

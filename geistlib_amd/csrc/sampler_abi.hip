@@ -45,6 +45,8 @@ struct geist_hip_sampler {
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
+    bool tmax_ready         = false; /* the projection has written the top-k scan's thread maxima
+                                        for the rows about to be sampled */
 
     char err[512] = {0};
 };
@@ -363,7 +365,8 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
             f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
         }
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
-        launch_tmax_scan(scan, s->tmax, nullptr);
+        if (!s->tmax_ready)
+            launch_tmax_scan(scan, s->tmax, nullptr);
         if (stream_only(s))
             return after_launch(s, "top-k scan");
         f.mode = FINAL_TOPK;
@@ -599,6 +602,68 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                         (int) m, d_y + m0 * ld_y, (long) ld_y);
     }
     return after_launch(s, "f16 gemv");
+}
+
+int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
+                                  size_t rows, size_t d_model, const float *d_norm_weight,
+                                  float rms_eps, const uint16_t *d_embed_f16, size_t n_vocab,
+                                  float *d_normed, float *d_logits, size_t ld_logits,
+                                  const struct geist_hip_sample_params *params,
+                                  const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                  geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_hidden || !d_norm_weight || !d_embed_f16 || !d_logits || !params || !d_out_tokens)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (rows == 0 || rows > s->max_rows || d_model == 0 || d_model > 0x7ffffff8u ||
+        n_vocab == 0 || n_vocab > s->max_vocab || ld_hidden < d_model || ld_logits < n_vocab)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "projection: %zu rows, d_model %zu, vocab %zu",
+                    rows, d_model, n_vocab);
+    if (d_model % 8 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "projection: d_model %zu is not a multiple of 8",
+                    d_model);
+    if (((uintptr_t) d_embed_f16) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "projection: weights not 16-byte aligned");
+    Resolved rs;
+    int      rc = resolve(s, params, n_vocab, rs);
+    if (rc)
+        return rc;
+    if (!rs.greedy && !d_uniforms && !d_rng_states)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic configuration without draws");
+    HIPCHK(s, hipSetDevice(s->device));
+    const bool fuse_ok = f16_gemv_can_fuse((int) rows);
+    /* the top-k path's scan is the projection's epilogue when nothing changes the logits
+     * between the two (no soft-cap) */
+    const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX &&
+                           !(params->logit_softcap > 0.0f);
+    if (!d_normed)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "no buffer for the normed rows");
+    launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps, (int) rows,
+                        (int) d_model, d_normed, (long) d_model);
+    if (topk_scan) {
+        GemvFuse f{};
+        f.tmax     = s->tmax;
+        f.n_chunks = (int) ((n_vocab + 8191) / 8192);
+        launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
+                        (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+    } else {
+        for (size_t m0 = 0; m0 < rows; m0 += GEMV_M_MAX) {
+            const size_t m = rows - m0 < (size_t) GEMV_M_MAX ? rows - m0 : (size_t) GEMV_M_MAX;
+            launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model,
+                            d_normed + m0 * d_model, (long) d_model, (int) m,
+                            d_logits + m0 * ld_logits, (long) ld_logits);
+        }
+    }
+    if (!rs.greedy && d_rng_states) {
+        launch_rng_units(s->stream, d_rng_states, shared, (int) rows, s->uniforms);
+        d_uniforms = s->uniforms;
+    }
+    const struct geist_hip_rows r = {d_logits, ld_logits, rows, n_vocab, nullptr, 0, nullptr,
+                                     nullptr, 0};
+    s->tmax_ready = topk_scan;
+    rc            = sample_impl(s, &r, params, rs.greedy ? nullptr : d_uniforms, d_out_tokens);
+    s->tmax_ready = false;
+    return rc;
 }
 
 int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,

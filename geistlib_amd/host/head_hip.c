@@ -183,15 +183,24 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
         h->d_normed    = p;
         h->d_model_cap = d_model;
     }
-    /* head.c:99-101, then 114-126 */
-    int rc = geist_hip_rmsnorm_rows(h->hs, d_hidden, ld_hidden, d_norm_weight, rms_eps, k, d_model,
-                                    h->d_normed, d_model);
-    if (rc == GEIST_HIP_OK)
-        rc = geist_hip_f16_gemv_rows(h->hs, d_embed_f16, h->vocab, d_model, h->d_normed, d_model, k,
-                                     h->d_logits, h->vocab);
-    if (rc != GEIST_HIP_OK)
-        return head_fail(h, rc, "output head");
-    return finalize(h, h->d_logits, k, out_tokens);
+    /* head.c:99-101, 114-126, then the dispatch of 172-183 / 291-302 with the session's RNG */
+    const struct geist_hip_sample_params prm = {.temperature        = h->temperature,
+                                                .top_p              = h->top_p,
+                                                .top_k              = h->top_k,
+                                                .repetition_penalty = 1.0f,
+                                                .logit_softcap      = h->logit_softcap,
+                                                .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
+    if (geist_hip_project_sample_rows(h->hs, d_hidden, ld_hidden, k, d_model, d_norm_weight,
+                                      rms_eps, d_embed_f16, h->vocab, h->d_normed, h->d_logits,
+                                      h->vocab, &prm, nullptr, h->d_rng, /*shared=*/1,
+                                      h->d_tokens) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
+    if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
+    for (size_t r = 0; r < k; r++)
+        if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
+            return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
+    return GEIST_HIP_OK;
 }
 
 const float *geist_hip_head_logits(const struct geist_hip_head *h) {

@@ -36,6 +36,24 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                             size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
                             size_t ld_y);
 
+/* The tail of a forward pass in one call (head.c:94-188 / 224-304): norm, projection, sampling
+ * of `rows` hidden rows. Equal in results to geist_hip_rmsnorm_rows + geist_hip_f16_gemv_rows +
+ * geist_hip_sample_rows[_rng] on d_logits; for one or two rows whose configuration takes the
+ * top-k path without a soft-cap, the projection also leaves the per-thread maxima the sampler's
+ * first pass would compute, and that pass is skipped.
+ *   d_normed   [rows, d_model] receives the normed rows
+ *   d_logits   [rows, ld_logits] receives the logits (row stride ld_logits >= n_vocab)
+ *   d_uniforms one draw per row, or NULL with d_rng_states != NULL: xorshift64* states as in
+ *              geist_hip_sample_rows_rng (`shared` as there); both NULL only for greedy params
+ * rows <= max_rows and n_vocab <= max_vocab of the sampler. */
+int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
+                                  size_t rows, size_t d_model, const float *d_norm_weight,
+                                  float rms_eps, const uint16_t *d_embed_f16, size_t n_vocab,
+                                  float *d_normed, float *d_logits, size_t ld_logits,
+                                  const struct geist_hip_sample_params *params,
+                                  const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                  geist_hip_token_t *d_out_tokens);
+
 /* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
  * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
  * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */

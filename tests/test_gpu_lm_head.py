@@ -126,3 +126,64 @@ def test_head_to_token_without_leaving_the_device(hs, oracle):
     assert (bits(logits.cpu().numpy()) == bits(want_logits)).all()
     want = [oracle.chain_u(want_logits[r], float(u[r]), **prm)[0] for r in range(k)]
     assert out.cpu().tolist() == want
+
+
+@pytest.mark.parametrize("rows", [1, 2, 5])
+@pytest.mark.parametrize("vocab,d_model", [(32000, 2560), (20001, 136), (8192, 64), (8193, 1536)])
+def test_project_sample_rows_equals_the_separate_steps(hs, oracle, rows, vocab, d_model):
+    """geist_hip_project_sample_rows: for one or two rows the norm runs inside the projection and,
+    on the top-k path without soft-cap, the projection's epilogue replaces the sampler's scan.
+    Logits bit-identical to the oracle's, tokens those of the oracle's chain."""
+    from geistlib_amd import SampleParams
+    print(f"project rows={rows} vocab={vocab} d_model={d_model}", flush=True)
+    g = np.random.default_rng(rows * 1000 + vocab + d_model)
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16).view(np.uint16)
+    hidden = (g.standard_normal((rows, d_model)) * 3).astype(np.float32)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    u = g.random(rows).astype(np.float32)
+    want_logits = oracle.f16_gemv(w16, oracle.rmsnorm(hidden, norm_w, 1e-6))
+    d_w, d_h, d_nw, d_u = (to_dev(w16.view(np.int16), torch), to_dev(hidden, torch),
+                           to_dev(norm_w, torch), to_dev(u, torch))
+    normed = torch.empty((rows, d_model), dtype=torch.float32, device="cuda")
+    for prm in (dict(temperature=0.8, top_k=40, top_p=0.95), dict(temperature=0.7, top_k=5),
+                dict(temperature=0.0), dict(temperature=1.0), dict(temperature=0.9, top_p=0.9),
+                dict(temperature=0.8, top_k=40, softcap=20.0), dict(temperature=0.8, top_k=300)):
+        logits = torch.full((rows, vocab), 7.0, dtype=torch.float32, device="cuda")
+        out = torch.full((rows,), -3, dtype=torch.int32, device="cuda")
+        hs.project_sample(d_h, d_nw, 1e-6, d_w, logits, SampleParams.make(**prm), d_u, out,
+                          normed=normed)
+        hs.sync()
+        assert (bits(logits.cpu().numpy()) == bits(want_logits)).all(), prm
+        kw = {k: v for k, v in prm.items() if k != "softcap"}
+        want = []
+        for r in range(rows):
+            row = want_logits[r]
+            if prm.get("softcap") and prm["temperature"] > 0:
+                row = oracle.softcap(row, prm["softcap"])
+            want.append(oracle.argmax(row) if prm["temperature"] <= 0
+                        else oracle.chain_u(row, float(u[r]), **kw)[0])
+        assert out.cpu().tolist() == want, prm
+    assert (d_h.cpu().numpy() == hidden).all()
+
+
+def test_project_sample_rows_with_the_device_rng(hs, oracle):
+    from geistlib_amd import SampleParams
+    from geistlib_amd.workloads import xorshift_units
+    g = np.random.default_rng(2)
+    vocab, d_model, rows = 30000, 512, 2
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16).view(np.uint16)
+    hidden = (g.standard_normal((rows, d_model)) * 3).astype(np.float32)
+    norm_w = np.ones(d_model, dtype=np.float32)
+    st = torch.tensor([0xABCDEF], dtype=torch.int64, device="cuda")
+    logits = torch.empty((rows, vocab), dtype=torch.float32, device="cuda")
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    hs.project_sample(to_dev(hidden, torch), to_dev(norm_w, torch), 1e-5,
+                      to_dev(w16.view(np.int16), torch), logits,
+                      SampleParams.make(temperature=0.8, top_k=40), None, out, rng_states=st,
+                      normed=torch.empty((rows, d_model), dtype=torch.float32, device="cuda"))
+    hs.sync()
+    u, after = xorshift_units(0xABCDEF, rows)
+    want_logits = oracle.f16_gemv(w16, oracle.rmsnorm(hidden, norm_w, 1e-5))
+    want = [oracle.top_k_u(want_logits[r], 40, 0.8, float(u[r]))[0] for r in range(rows)]
+    assert out.cpu().tolist() == want
+    assert int(st.cpu().numpy().view(np.uint64)[0]) == after
