@@ -89,6 +89,8 @@ def load_library():
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
     lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_f16_to_q8w.argtypes = [vp, vp, sz, sz, vp, vp]
+    lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
                                                   C.POINTER(SampleParams), vp, vp, i32, vp]
     lib.geist_hip_time_f16_gemv_rows.argtypes = [vp, C.POINTER(vp), sz, sz, sz, vp, sz, sz, vp, sz,
@@ -223,6 +225,20 @@ class HipSampler:
         self._check(self.lib.geist_hip_f16_gemv_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
+
+    def f16_to_q8w(self, w_f16, wq, scales):
+        """w_f16 [n_out, n_in] float16 -> wq int8 [n_out, n_in], scales float32 [n_out]."""
+        n_out, n_in = w_f16.shape
+        self._check(self.lib.geist_hip_f16_to_q8w(self.h, _ptr(w_f16), n_out, n_in, _ptr(wq),
+                                                  _ptr(scales)))
+
+    def q8w_gemv(self, wq, scales, x, y):
+        n_out, n_in = wq.shape
+        m = x.shape[0]
+        assert wq.is_contiguous() and wq.element_size() == 1
+        self._check(self.lib.geist_hip_q8w_gemv_rows(
+            self.h, _ptr(wq), _ptr(scales), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in,
+            m, _ptr(y), y.stride(0) if m > 1 else n_out))
 
     def project_sample(self, hidden, norm_w, eps, embed_f16, logits, params, uniforms, out,
                        normed=None, rng_states=None, shared=True):

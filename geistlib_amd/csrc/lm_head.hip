@@ -35,10 +35,19 @@ constexpr int LM_WAVE      = 64;
 constexpr int LM_WAVES     = LM_TPB / LM_WAVE;
 constexpr int ROWS_WAVE    = 32;                   /* two lanes per weight row */
 constexpr int ROWS_BLOCK   = ROWS_WAVE * LM_WAVES; /* 128 */
-constexpr int STAGE_COLS   = 64;                   /* 128 bytes of a row: four steps of 16 */
+constexpr int STAGE_BYTES  = 128;                  /* of a row per stage */
+constexpr int STAGE_COLS   = 64;                   /* ... which is 64 binary16 weights */
 constexpr int STAGE_LOADS  = 4;                    /* 32 rows x 8 segments / 64 lanes */
-constexpr int TILE_PITCH   = STAGE_COLS * 2 + 16;  /* bytes */
+constexpr int TILE_PITCH   = STAGE_BYTES + 16;     /* bytes */
 constexpr int TILE_BYTES   = ROWS_WAVE * TILE_PITCH;
+/* EB = bytes per weight: 2 (binary16) or 1 (int8 with a scale per row). A stage then holds
+ * 128 / EB columns, 8 / EB steps of 16, and each lane stages 2 / EB activations per row. */
+template <int EB>
+struct Geom {
+    static constexpr int COLS  = STAGE_BYTES / EB;
+    static constexpr int STEPS = COLS / 16;
+    static constexpr int XL    = COLS / LM_WAVE;
+};
 
 __device__ __forceinline__ float dadd(float a, float b) { return __fadd_rn(a, b); }
 
@@ -47,9 +56,9 @@ struct StageRegs {
     uint4 w[STAGE_LOADS];
 };
 
-template <int MT>
+template <int MT, int XL>
 struct StageX {
-    float x[MT];
+    float x[MT][XL];
 };
 
 /* Which weight row a wavefront's virtual row r (0..31) is. Plain: 32 consecutive rows per
@@ -64,11 +73,11 @@ __device__ __forceinline__ long virtual_row(long task, int r) {
     return chunk * 8192 + 4 * ((long) (r >> 2) * 256 + t) + (r & 3);
 }
 
-template <bool SL>
-__device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long task, long n_out,
+template <int EB, bool SL>
+__device__ __forceinline__ void stage_load(const uint8_t *__restrict__ w, long task, long n_out,
                                            int n_in, int stage, int lane, StageRegs &g) {
     const int seg = lane & 7;
-    const int col = stage * STAGE_COLS + seg * 8;
+    const int col = stage * Geom<EB>::COLS + seg * (16 / EB);
 #pragma unroll
     for (int i = 0; i < STAGE_LOADS; ++i) {
         const long row = virtual_row<SL>(task, 8 * i + (lane >> 3));
@@ -76,21 +85,25 @@ __device__ __forceinline__ void stage_load(const uint16_t *__restrict__ w, long 
         if (row < n_out && col < n_in) {
             /* read once, and far more than the caches hold: non-temporal */
             typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
-            const nt_u4 t =
-                __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(w + row * n_in + col));
+            const nt_u4 t = __builtin_nontemporal_load(
+                reinterpret_cast<const nt_u4 *>(w + (row * n_in + col) * EB));
             g.w[i] = make_uint4(t.x, t.y, t.z, t.w);
         }
     }
 }
 
-template <int MT>
+template <int EB, int MT>
 __device__ __forceinline__ void stage_load_x(const float *__restrict__ x, long ld_x, int n_m,
-                                             int n_in, int stage, int lane, StageX<MT> &gx) {
-    const int col = stage * STAGE_COLS + lane;
+                                             int n_in, int stage, int lane,
+                                             StageX<MT, Geom<EB>::XL> &gx) {
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int mm = m < n_m ? m : n_m - 1; /* rows beyond n_m repeat the last one, unstored */
-        gx.x[m]      = col < n_in ? x[mm * ld_x + col] : 0.0f;
+    for (int q = 0; q < Geom<EB>::XL; ++q) {
+        const int col = stage * Geom<EB>::COLS + q * LM_WAVE + lane;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int mm = m < n_m ? m : n_m - 1; /* rows beyond n_m repeat the last, unstored */
+            gx.x[m][q]   = col < n_in ? x[mm * ld_x + col] : 0.0f;
+        }
     }
 }
 
@@ -114,17 +127,29 @@ __device__ __forceinline__ float rms_inv_sequential(const float *__restrict__ xr
 
 /* One step of the chains: eight weights of this lane's row and half against the activations of
  * the same columns. MASKED: lanes with keep == false leave their chains alone. */
-template <int MT, bool MASKED>
-__device__ __forceinline__ void gemv_step(const uint8_t *tile, const float (*xs)[STAGE_COLS],
+template <int EB, int MT, bool MASKED>
+__device__ __forceinline__ void gemv_step(const uint8_t *tile, const float (*xs)[Geom<EB>::COLS],
                                           int my_row, int half, int t, bool keep,
                                           float (&acc)[MT][8]) {
-    const uint4 q =
-        *reinterpret_cast<const uint4 *>(tile + my_row * TILE_PITCH + t * 32 + half * 16);
-    const float2 f01 = __half22float2(*reinterpret_cast<const __half2 *>(&q.x));
-    const float2 f23 = __half22float2(*reinterpret_cast<const __half2 *>(&q.y));
-    const float2 f45 = __half22float2(*reinterpret_cast<const __half2 *>(&q.z));
-    const float2 f67 = __half22float2(*reinterpret_cast<const __half2 *>(&q.w));
-    const float  wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
+    float wf[8];
+    if (EB == 2) {
+        const uint4 q =
+            *reinterpret_cast<const uint4 *>(tile + my_row * TILE_PITCH + t * 32 + half * 16);
+        const float2 f01 = __half22float2(*reinterpret_cast<const __half2 *>(&q.x));
+        const float2 f23 = __half22float2(*reinterpret_cast<const __half2 *>(&q.y));
+        const float2 f45 = __half22float2(*reinterpret_cast<const __half2 *>(&q.z));
+        const float2 f67 = __half22float2(*reinterpret_cast<const __half2 *>(&q.w));
+        wf[0] = f01.x, wf[1] = f01.y, wf[2] = f23.x, wf[3] = f23.y;
+        wf[4] = f45.x, wf[5] = f45.y, wf[6] = f67.x, wf[7] = f67.y;
+    } else {
+        const uint2 q =
+            *reinterpret_cast<const uint2 *>(tile + my_row * TILE_PITCH + t * 16 + half * 8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wf[i]     = (float) (int) (int8_t) (q.x >> (8 * i));
+            wf[4 + i] = (float) (int) (int8_t) (q.y >> (8 * i));
+        }
+    }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const float4 xa = *reinterpret_cast<const float4 *>(&xs[m][t * 16 + half * 8]);
@@ -138,15 +163,15 @@ __device__ __forceinline__ void gemv_step(const uint8_t *tile, const float (*xs)
     }
 }
 
-} // namespace
-
-template <int MT, bool SL>
-__global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict__ w, long n_out,
-                                                     int n_in, const float *__restrict__ x,
-                                                     long ld_x, int n_m, float *__restrict__ y,
-                                                     long ld_y, GemvFuse fuse) {
+/* The work of one workgroup; `scales` != NULL (int8 weights): y = sum * scales[row]. */
+template <int EB, int MT, bool SL>
+__device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w,
+                                          const float *__restrict__ scales, long n_out, int n_in,
+                                          const float *__restrict__ x, long ld_x, int n_m,
+                                          float *__restrict__ y, long ld_y, const GemvFuse &fuse) {
+    constexpr int COLS = Geom<EB>::COLS, STEPS = Geom<EB>::STEPS, XL = Geom<EB>::XL;
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][TILE_BYTES];
-    __shared__ __align__(16) float   s_x[LM_WAVES][MT][STAGE_COLS];
+    __shared__ __align__(16) float   s_x[LM_WAVES][MT][COLS];
     const int  lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
     const long task = (long) blockIdx.x * LM_WAVES + wave;
     if (virtual_row<SL>(task, 0) >= n_out) { /* (no workgroup barrier below) */
@@ -156,7 +181,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         return;
     }
     uint8_t *tile = s_tile[wave];
-    float(*xs)[STAGE_COLS] = s_x[wave];
+    float(*xs)[COLS] = s_x[wave];
     const int my_row = lane >> 1, half = lane & 1;
 
     float acc[MT][8];
@@ -166,15 +191,15 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
         for (int i = 0; i < 8; ++i)
             acc[m][i] = 0.0f;
 
-    const int n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
-    StageRegs  g0, g1;
-    StageX<MT> x0, x1;
-    stage_load<SL>(w, task, n_out, n_in, 0, lane, g0);
+    const int n_stage = (n_in + COLS - 1) / COLS;
+    StageRegs      g0, g1;
+    StageX<MT, XL> x0, x1;
+    stage_load<EB, SL>(w, task, n_out, n_in, 0, lane, g0);
     if (n_stage > 1)
-        stage_load<SL>(w, task, n_out, n_in, 1, lane, g1);
-    stage_load_x<MT>(x, ld_x, n_m, n_in, 0, lane, x0);
+        stage_load<EB, SL>(w, task, n_out, n_in, 1, lane, g1);
+    stage_load_x<EB, MT>(x, ld_x, n_m, n_in, 0, lane, x0);
     if (n_stage > 1)
-        stage_load_x<MT>(x, ld_x, n_m, n_in, 1, lane, x1);
+        stage_load_x<EB, MT>(x, ld_x, n_m, n_in, 1, lane, x1);
     for (int s = 0; s < n_stage; ++s) {
         /* registers -> tile (this waits for the loads issued two stages ago) */
 #pragma unroll
@@ -183,27 +208,29 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
                 g0.w[i];
 #pragma unroll
         for (int m = 0; m < MT; ++m)
-            xs[m][lane] = x0.x[m];
+#pragma unroll
+            for (int q = 0; q < XL; ++q)
+                xs[m][q * LM_WAVE + lane] = x0.x[m][q];
         g0 = g1;
         x0 = x1;
         if (s + 2 < n_stage) {
-            stage_load<SL>(w, task, n_out, n_in, s + 2, lane, g1);
-            stage_load_x<MT>(x, ld_x, n_m, n_in, s + 2, lane, x1);
+            stage_load<EB, SL>(w, task, n_out, n_in, s + 2, lane, g1);
+            stage_load_x<EB, MT>(x, ld_x, n_m, n_in, s + 2, lane, x1);
         }
         /* steps of this stage: whole blocks of 16 columns, and at the end of the row possibly
          * a block of 8, which only extends chains 0..7 (the lanes with half == 0) */
-        const int left = n_in - s * STAGE_COLS;
-        if (left >= STAGE_COLS) {
+        const int left = n_in - s * COLS;
+        if (left >= COLS) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                gemv_step<MT, false>(tile, xs, my_row, half, t, true, acc);
+            for (int t = 0; t < STEPS; ++t)
+                gemv_step<EB, MT, false>(tile, xs, my_row, half, t, true, acc);
         } else {
             const int  full  = left / 16;
             const bool tail8 = (left & 15) == 8;
             for (int t = 0; t < full; ++t)
-                gemv_step<MT, false>(tile, xs, my_row, half, t, true, acc);
+                gemv_step<EB, MT, false>(tile, xs, my_row, half, t, true, acc);
             if (tail8)
-                gemv_step<MT, true>(tile, xs, my_row, half, full, half == 0, acc);
+                gemv_step<EB, MT, true>(tile, xs, my_row, half, full, half == 0, acc);
         }
     }
     /* (chain j + chain j+8), (lane i + lane i+4), ((0+1) + (2+3)): kernel_f16_gemv.c:25-32, 59 */
@@ -216,7 +243,9 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
             v[i] = dadd(acc[m][i], __shfl_xor(acc[m][i], 1, LM_WAVE));
         const float q0 = dadd(v[0], v[4]), q1 = dadd(v[1], v[5]);
         const float q2 = dadd(v[2], v[6]), q3 = dadd(v[3], v[7]);
-        const float sum = dadd(dadd(q0, q1), dadd(q2, q3));
+        float sum = dadd(dadd(q0, q1), dadd(q2, q3));
+        if (EB == 1) /* q8w_gemv_m1: y[r] = s * scales[r], kernel_f16_gemv.c:125 */
+            sum = __fmul_rn(sum, row < n_out ? scales[row] : 0.0f);
         if (half == 0 && row < n_out && m < n_m)
             y[m * ld_y + row] = sum;
         if (SL) {
@@ -230,6 +259,29 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict_
                 fuse.tmax[((long) m * fuse.n_chunks + (task >> 8)) * 256 + (task & 255)] = mx;
         }
     }
+}
+
+} // namespace
+
+template <int MT, bool SL>
+__global__ __launch_bounds__(LM_TPB) void k_f16_gemv(const uint16_t *__restrict__ w, long n_out,
+                                                     int n_in, const float *__restrict__ x,
+                                                     long ld_x, int n_m, float *__restrict__ y,
+                                                     long ld_y, GemvFuse fuse) {
+    gemv_body<2, MT, SL>(reinterpret_cast<const uint8_t *>(w), nullptr, n_out, n_in, x, ld_x, n_m,
+                         y, ld_y, fuse);
+}
+
+/* q8w_gemv_m1 (kernel_f16_gemv.c:95-127): the same chains over int8 weights, times the row's
+ * scale. Half the bytes per weight, so twice the columns per stage. */
+template <int MT, bool SL>
+__global__ __launch_bounds__(LM_TPB) void k_q8w_gemv(const int8_t *__restrict__ wq,
+                                                     const float *__restrict__ scales, long n_out,
+                                                     int n_in, const float *__restrict__ x,
+                                                     long ld_x, int n_m, float *__restrict__ y,
+                                                     long ld_y, GemvFuse fuse) {
+    gemv_body<1, MT, SL>(reinterpret_cast<const uint8_t *>(wq), scales, n_out, n_in, x, ld_x, n_m,
+                         y, ld_y, fuse);
 }
 
 /* The projection for several activation rows. Here a lane owns all sixteen chains of one weight
@@ -420,6 +472,69 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
         k_f16_gemv_batched<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
     else
         k_f16_gemv<8, false><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+}
+
+/* f16_to_q8w (kernel_f16_gemv.c:66-93): per row scale = max|w| / 127, q = lrintf(w * (127 /
+ * max|w|)) clamped to +-127. One workgroup per row. */
+__global__ __launch_bounds__(LM_TPB) void k_f16_to_q8w(const uint16_t *__restrict__ w, int n_in,
+                                                       int8_t *__restrict__ wq,
+                                                       float *__restrict__ scales) {
+    __shared__ float s_max[LM_TPB];
+    const int        tid = threadIdx.x;
+    const uint16_t  *wr  = w + (long) blockIdx.x * n_in;
+    float            a   = 0.0f;
+    for (int k = tid; k < n_in; k += LM_TPB) {
+        const float v = fabsf(__half2float(*reinterpret_cast<const __half *>(wr + k)));
+        a             = v > a ? v : a; /* (a NaN never replaces the maximum, as in the reference) */
+    }
+    s_max[tid] = a;
+    __syncthreads();
+    for (int step = LM_TPB / 2; step > 0; step >>= 1) {
+        if (tid < step)
+            s_max[tid] = s_max[tid + step] > s_max[tid] ? s_max[tid + step] : s_max[tid];
+        __syncthreads();
+    }
+    const float amax = s_max[0];
+    const float id   = amax > 0.0f ? __fdiv_rn(127.0f, amax) : 0.0f;
+    if (tid == 0)
+        scales[blockIdx.x] = __fdiv_rn(amax, 127.0f);
+    int8_t *qr = wq + (long) blockIdx.x * n_in;
+    for (int k = tid; k < n_in; k += LM_TPB) {
+        const float v = __fmul_rn(__half2float(*reinterpret_cast<const __half *>(wr + k)), id);
+        int         q = __float2int_rn(v); /* lrintf: to nearest, ties to even */
+        q             = q > 127 ? 127 : q;
+        q             = q < -127 ? -127 : q;
+        qr[k]         = (int8_t) q;
+    }
+}
+
+void launch_f16_to_q8w(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in, int8_t *wq,
+                       float *scales) {
+    k_f16_to_q8w<<<dim3((unsigned) n_out), dim3(LM_TPB), 0, stream>>>(w_f16, n_in, wq, scales);
+}
+
+void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, long n_out,
+                     int n_in, const float *x, long ld_x, int n_m, float *y, long ld_y,
+                     const GemvFuse *fuse) {
+    const dim3 block(LM_TPB);
+    const dim3 grid((unsigned) ((n_out + ROWS_BLOCK - 1) / ROWS_BLOCK));
+    GemvFuse   none{};
+    if (fuse && fuse->tmax) {
+        const dim3 grid_s((unsigned) (fuse->n_chunks * 256 / LM_WAVES));
+        if (n_m <= 1)
+            k_q8w_gemv<1, true><<<grid_s, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, *fuse);
+        else
+            k_q8w_gemv<2, true><<<grid_s, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, *fuse);
+        return;
+    }
+    if (n_m <= 1)
+        k_q8w_gemv<1, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+    else if (n_m <= 2)
+        k_q8w_gemv<2, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+    else if (n_m <= 4)
+        k_q8w_gemv<4, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+    else
+        k_q8w_gemv<8, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
 }
 
 } // namespace gs

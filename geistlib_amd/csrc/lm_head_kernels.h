@@ -34,5 +34,14 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
                      const float *x, long ld_x, int n_m, float *y, long ld_y,
                      const GemvFuse *fuse = nullptr);
 
+/* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *
+ * scales[r]; n_in a multiple of 16. */
+void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, long n_out,
+                     int n_in, const float *x, long ld_x, int n_m, float *y, long ld_y,
+                     const GemvFuse *fuse = nullptr);
+/* f16_to_q8w: wq [n_out][n_in] and scales [n_out] from the binary16 table. */
+void launch_f16_to_q8w(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in, int8_t *wq,
+                       float *scales);
+
 } // namespace gs
 #endif

@@ -604,6 +604,42 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
     return after_launch(s, "f16 gemv");
 }
 
+int geist_hip_f16_to_q8w(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out, size_t n_in,
+                         int8_t *d_wq, float *d_scales) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_f16 || !d_wq || !d_scales || n_out == 0 || n_in == 0 || n_in > 0x7fffffffu ||
+        n_out > 0x7fffffffu)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "f16_to_q8w: null argument or bad shape");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_f16_to_q8w(s->stream, d_w_f16, (long) n_out, (int) n_in, d_wq, d_scales);
+    return after_launch(s, "f16_to_q8w");
+}
+
+int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const float *d_scales,
+                            size_t n_out, size_t n_in, const float *d_x, size_t ld_x,
+                            size_t n_rows, float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_wq || !d_scales || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_out == 0 || n_in == 0 || n_rows == 0 || n_in > 0x7ffffff0u || ld_x < n_in ||
+        ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "q8w gemv: %zu x %zu, %zu rows, strides %zu / %zu",
+                    n_out, n_in, n_rows, ld_x, ld_y);
+    if (n_in % 16 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "q8w gemv: n_in %zu is not a multiple of 16", n_in);
+    if (((uintptr_t) d_wq) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "q8w gemv: weights not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    for (size_t m0 = 0; m0 < n_rows; m0 += GEMV_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) GEMV_M_MAX ? n_rows - m0 : (size_t) GEMV_M_MAX;
+        launch_q8w_gemv(s->stream, d_wq, d_scales, (long) n_out, (int) n_in, d_x + m0 * ld_x,
+                        (long) ld_x, (int) m, d_y + m0 * ld_y, (long) ld_y);
+    }
+    return after_launch(s, "q8w gemv");
+}
+
 int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
                                   size_t rows, size_t d_model, const float *d_norm_weight,
                                   float rms_eps, const uint16_t *d_embed_f16, size_t n_vocab,

@@ -36,6 +36,23 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                             size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
                             size_t ld_y);
 
+/* The int8 form of the tied table, which the reference's x86 backend uses for the lm_head unless
+ * GEIST_Q8_LMHEAD=0 (src/backends/cpu_x86/backend.c:344-372): half the bytes per decode step.
+ *
+ * geist_hip_f16_to_q8w replaces f16_to_q8w (kernel_f16_gemv.c:66-93), run once at load:
+ *   scales[r] = max_k |w[r][k]| / 127,  wq[r][k] = clamp(lrintf(w[r][k] * (127 / max|w[r]|)), +-127)
+ * with IEEE divisions (the reference's release build compiles with -ffast-math, which may form
+ * the first quotient by a reciprocal; its strict build is matched bit for bit).
+ * geist_hip_q8w_gemv_rows replaces q8w_gemv_m1 (kernel_f16_gemv.c:95-127):
+ *   d_y[m * ld_y + r] = (sum_i (float)wq[r][i] * d_x[m * ld_x + i]) * scales[r]
+ * in the reference's order of summation (the chains and the tree of f16_gemv_m1), bit for bit.
+ * n_in must be a multiple of 16, d_wq 16-byte aligned. */
+int geist_hip_f16_to_q8w(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out, size_t n_in,
+                         int8_t *d_wq, float *d_scales);
+int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const float *d_scales,
+                            size_t n_out, size_t n_in, const float *d_x, size_t ld_x,
+                            size_t n_rows, float *d_y, size_t ld_y);
+
 /* The tail of a forward pass in one call (head.c:94-188 / 224-304): norm, projection, sampling
  * of `rows` hidden rows. Equal in results to geist_hip_rmsnorm_rows + geist_hip_f16_gemv_rows +
  * geist_hip_sample_rows[_rng] on d_logits; for one or two rows whose configuration takes the

@@ -89,6 +89,56 @@ void oracle_f16_gemv_m1(size_t n_out, size_t n_in, const float *x, const uint16_
     }
 }
 
+/* src/backends/cpu_x86/kernel_f16_gemv.c:66-93 */
+void oracle_f16_to_q8w(size_t n_out, size_t n_in, const uint16_t *w_f16, int8_t *wq, float *scales) {
+    for (size_t r = 0; r < n_out; r++) {
+        const uint16_t *wr   = w_f16 + r * n_in;
+        float           amax = 0.0f;
+        for (size_t k = 0; k < n_in; k++) {
+            const float a = fabsf(oracle_f16_to_f32(wr[k]));
+            if (a > amax)
+                amax = a;
+        }
+        scales[r]      = amax / 127.0f;
+        const float id = amax > 0.0f ? 127.0f / amax : 0.0f;
+        for (size_t k = 0; k < n_in; k++) {
+            long q = lrintf(oracle_f16_to_f32(wr[k]) * id);
+            if (q > 127)
+                q = 127;
+            if (q < -127)
+                q = -127;
+            wq[r * n_in + k] = (int8_t) q;
+        }
+    }
+}
+
+/* src/backends/cpu_x86/kernel_f16_gemv.c:95-127 */
+void oracle_q8w_gemv_m1(size_t n_out, size_t n_in, const float *x, const int8_t *wq,
+                        const float *scales, float *y) {
+    for (size_t r = 0; r < n_out; r++) {
+        const int8_t *qr = wq + r * n_in;
+        float         chain[16];
+        for (int j = 0; j < 16; j++)
+            chain[j] = 0.0f;
+        size_t k = 0;
+        for (; k + 16 <= n_in; k += 16)
+            for (int j = 0; j < 16; j++)
+                chain[j] = fmaf((float) qr[k + j], x[k + j], chain[j]);
+        for (; k + 8 <= n_in; k += 8)
+            for (int j = 0; j < 8; j++)
+                chain[j] = fmaf((float) qr[k + j], x[k + j], chain[j]);
+        float v[8], q[4];
+        for (int i = 0; i < 8; i++)
+            v[i] = chain[i] + chain[i + 8];
+        for (int i = 0; i < 4; i++)
+            q[i] = v[i] + v[i + 4];
+        float s = (q[0] + q[1]) + (q[2] + q[3]);
+        for (; k < n_in; k++)
+            s += (float) qr[k] * x[k];
+        y[r] = s * scales[r];
+    }
+}
+
 /* src/backends/cpu_scalar/elementwise.c:266-278 */
 void oracle_rmsnorm_rows(size_t n_rows, size_t n, const float *x, const float *w, float eps,
                          float *y) {

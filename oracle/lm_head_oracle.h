@@ -34,6 +34,14 @@ uint16_t oracle_f32_to_f16(float v);
  * elements of an n_in % 8 tail one by one. */
 void oracle_f16_gemv_m1(size_t n_out, size_t n_in, const float *x, const uint16_t *w_f16, float *y);
 
+/* The int8 form of the table. f16_to_q8w (kernel_f16_gemv.c:66-93): scales[r] = max|w| / 127,
+ * wq = clamp(lrintf(w * (127 / max|w|)), -127, 127), a row of zeros gets scale 0 and zeros.
+ * q8w_gemv_m1 (kernel_f16_gemv.c:95-127): the chains and tree of f16_gemv_m1 over (float) wq,
+ * then times scales[r]. */
+void oracle_f16_to_q8w(size_t n_out, size_t n_in, const uint16_t *w_f16, int8_t *wq, float *scales);
+void oracle_q8w_gemv_m1(size_t n_out, size_t n_in, const float *x, const int8_t *wq,
+                        const float *scales, float *y);
+
 /* y = x * weight * rsqrt(mean(x^2) + eps) per row (cpu_scalar_rmsnorm,
  * src/backends/cpu_scalar/elementwise.c:241-280): sum of squares in double in index order,
  * inv = (float)(1.0 / sqrt(sum / n + (double) eps)), y_i = (x_i * inv) * w_i in binary32. */

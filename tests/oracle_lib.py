@@ -112,6 +112,10 @@ def load_oracle(fast=False):
     lib.oracle_f32_to_f16.restype = C.c_uint16
     lib.oracle_f32_to_f16.argtypes = [C.c_float]
     lib.oracle_f16_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, c_u16_p, c_float_p]
+    c_i8_p = C.POINTER(C.c_int8)
+    lib.oracle_f16_to_q8w.argtypes = [C.c_size_t, C.c_size_t, c_u16_p, c_i8_p, c_float_p]
+    lib.oracle_q8w_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, c_i8_p, c_float_p,
+                                       c_float_p]
     lib.oracle_rmsnorm_rows.argtypes = [C.c_size_t, C.c_size_t, c_float_p, c_float_p, C.c_float,
                                         c_float_p]
     return lib
@@ -201,6 +205,26 @@ class Oracle:
                                         w.ctypes.data_as(C.POINTER(C.c_uint16)), _fp(y[m]))
         return y[0] if np.ndim(x) == 1 else y
 
+    def f16_to_q8w(self, w_f16):
+        w = np.ascontiguousarray(w_f16, dtype=np.uint16)
+        n_out, n_in = w.shape
+        wq = np.empty((n_out, n_in), dtype=np.int8)
+        scales = np.empty(n_out, dtype=np.float32)
+        self.lib.oracle_f16_to_q8w(n_out, n_in, w.ctypes.data_as(C.POINTER(C.c_uint16)),
+                                   wq.ctypes.data_as(C.POINTER(C.c_int8)), _fp(scales))
+        return wq, scales
+
+    def q8w_gemv(self, wq, scales, x):
+        wq = np.ascontiguousarray(wq, dtype=np.int8)
+        scales = np.ascontiguousarray(scales, dtype=np.float32)
+        xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+        n_out, n_in = wq.shape
+        y = np.empty((xs.shape[0], n_out), dtype=np.float32)
+        for m in range(xs.shape[0]):
+            self.lib.oracle_q8w_gemv_m1(n_out, n_in, _fp(xs[m]),
+                                        wq.ctypes.data_as(C.POINTER(C.c_int8)), _fp(scales), _fp(y[m]))
+        return y[0] if np.ndim(x) == 1 else y
+
     def rmsnorm(self, x, w, eps):
         xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
         w = np.ascontiguousarray(w, dtype=np.float32)
@@ -281,6 +305,12 @@ def load_ref_f16gemv(fast=False):
     lib.f16_gemv_m1.restype = None
     lib.fp16_to_fp32.restype = C.c_float
     lib.fp16_to_fp32.argtypes = [C.c_uint16]
+    lib.f16_to_q8w.argtypes = [C.c_size_t, C.c_size_t, C.POINTER(C.c_uint16), C.POINTER(C.c_int8),
+                               c_float_p]
+    lib.f16_to_q8w.restype = None
+    lib.q8w_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.POINTER(C.c_int8), c_float_p,
+                                c_float_p]
+    lib.q8w_gemv_m1.restype = None
     return lib
 
 

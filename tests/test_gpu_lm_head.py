@@ -187,3 +187,30 @@ def test_project_sample_rows_with_the_device_rng(hs, oracle):
     want = [oracle.top_k_u(want_logits[r], 40, 0.8, float(u[r]))[0] for r in range(rows)]
     assert out.cpu().tolist() == want
     assert int(st.cpu().numpy().view(np.uint64)[0]) == after
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(1000, 2560, 1), (130, 128, 1), (129, 256, 3),
+                                          (4097, 1536, 2), (300, 16, 1), (300, 32, 5), (257, 48, 4),
+                                          (640, 4096, 8), (500, 2560, 11), (33, 144, 2)])
+def test_q8w_quantise_and_gemv_bit_exact(hs, oracle, n_out, n_in, m):
+    """geist_hip_f16_to_q8w and geist_hip_q8w_gemv_rows against the oracle's restatement of
+    f16_to_q8w / q8w_gemv_m1 (kernel_f16_gemv.c:66-127): int8 values, scales and results equal in
+    every bit."""
+    print(f"q8w n_out={n_out} n_in={n_in} m={m}", flush=True)
+    g = np.random.default_rng(n_out + 3 * n_in + m)
+    w16 = (g.standard_normal((n_out, n_in)) * g.choice([0.02, 1.0])).astype(np.float16)
+    w16[0, :] = 0
+    x = (g.standard_normal((m, n_in)) * g.choice([0.1, 1.0, 30.0], (m, 1))).astype(np.float32)
+    d_w = to_dev(w16.view(np.int16), torch)
+    d_wq = torch.empty((n_out, n_in), dtype=torch.int8, device="cuda")
+    d_sc = torch.empty(n_out, dtype=torch.float32, device="cuda")
+    hs.f16_to_q8w(d_w, d_wq, d_sc)
+    y = torch.full((m, n_out), 7.0, dtype=torch.float32, device="cuda")
+    hs.q8w_gemv(d_wq, d_sc, to_dev(x, torch), y)
+    hs.sync()
+    wq, sc = oracle.f16_to_q8w(w16.view(np.uint16))
+    assert (d_wq.cpu().numpy() == wq).all()
+    assert (bits(d_sc.cpu().numpy()) == bits(sc)).all()
+    want = oracle.q8w_gemv(wq, sc, x)
+    got = y.cpu().numpy()
+    assert (bits(got) == bits(want)).all(), np.argwhere(bits(got) != bits(want))[:5]

@@ -122,3 +122,52 @@ def test_rmsnorm_closed_forms(oracle):
         want = (xs[r] * inv).astype(np.float32) * ws
         assert (got[r].view(np.uint32) == want.astype(np.float32).view(np.uint32)).all()
     assert oracle.rmsnorm(np.zeros(n, dtype=np.float32), w, eps).tolist() == [0.0] * n
+
+
+@pytest.mark.parametrize("fast", [False, True])
+def test_q8w_equals_the_compiled_reference_kernels(oracle, fast):
+    """f16_to_q8w and q8w_gemv_m1 of the reference (kernel_f16_gemv.c:66-127). The quantiser is
+    compared with the strict build in every bit; against the release build (-ffast-math, which
+    may form max|w| / 127 through a reciprocal) the scales may differ in the last bit, the int8
+    values not. The GEMV is identical under both builds."""
+    ref = load_ref_f16gemv(fast)
+    if ref is None:
+        pytest.skip("oracle/_ref not built (needs the reference tree: make -C oracle ref)")
+    g = np.random.default_rng(15)
+    for n_out, n_in, scale in [(64, 2560, 0.05), (33, 1536, 1.0), (9, 16, 3.0), (20, 48, 1e-3),
+                               (5, 4096, 100.0)]:
+        w = weights(g, n_out, n_in, scale)
+        w[0, :] = 0                                  # a row of zeros: scale 0, zeros
+        wq_ref = np.empty((n_out, n_in), dtype=np.int8)
+        sc_ref = np.empty(n_out, dtype=np.float32)
+        ref.f16_to_q8w(n_out, n_in, w.ctypes.data_as(C.POINTER(C.c_uint16)),
+                       wq_ref.ctypes.data_as(C.POINTER(C.c_int8)),
+                       sc_ref.ctypes.data_as(C.POINTER(C.c_float)))
+        wq, sc = oracle.f16_to_q8w(w)
+        assert (wq == wq_ref).all(), (n_out, n_in)
+        if fast:
+            assert (np.abs(sc.view(np.int32) - sc_ref.view(np.int32)) <= 1).all()
+        else:
+            assert (sc.view(np.uint32) == sc_ref.view(np.uint32)).all()
+        x = (g.standard_normal(n_in) * g.choice([0.01, 1.0, 50.0])).astype(np.float32)
+        y = np.zeros(n_out, dtype=np.float32)
+        ref.q8w_gemv_m1(n_out, n_in, x.ctypes.data_as(C.POINTER(C.c_float)),
+                        wq_ref.ctypes.data_as(C.POINTER(C.c_int8)),
+                        sc_ref.ctypes.data_as(C.POINTER(C.c_float)),
+                        y.ctypes.data_as(C.POINTER(C.c_float)))
+        mine = oracle.q8w_gemv(wq_ref, sc_ref, x)
+        assert (mine.view(np.uint32) == y.view(np.uint32)).all(), (n_out, n_in)
+
+
+def test_q8w_keeps_the_reference_tests_bar(oracle):
+    """tests/test_q8w_gemv_unit.c: cosine similarity with the exact product >= 0.999."""
+    g = np.random.default_rng(16)
+    n_out, n_in = 512, 2560
+    w = ((g.integers(0, 65536, (n_out, n_in)) / 65536.0 * 2 - 1)).astype(np.float16).view(np.uint16)
+    x = (g.integers(0, 65536, n_in) / 65536.0 * 2 - 1).astype(np.float32)
+    exact = w.view(np.float16).astype(np.float64) @ x.astype(np.float64)
+    wq, sc = oracle.f16_to_q8w(w)
+    y = oracle.q8w_gemv(wq, sc, x).astype(np.float64)
+    cos = (y @ exact) / np.sqrt((y @ y) * (exact @ exact))
+    assert cos >= 0.999
+    assert np.abs(wq).max() <= 127 and (np.abs(wq).max(axis=1) == 127).all()
