@@ -200,22 +200,22 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w,
     stage_load_x<EB, MT>(x, ld_x, n_m, n_in, 0, lane, x0);
     if (n_stage > 1)
         stage_load_x<EB, MT>(x, ld_x, n_m, n_in, 1, lane, x1);
-    for (int s = 0; s < n_stage; ++s) {
-        /* registers -> tile (this waits for the loads issued two stages ago) */
+    /* One stage: registers -> tile (this waits for the loads issued two stages ago), the same
+     * registers are reloaded with the stage after next, then the steps. Two register sets take
+     * turns, so nothing is copied. */
+    auto do_stage = [&](int s, StageRegs &g, StageX<MT, XL> &gx) {
 #pragma unroll
         for (int i = 0; i < STAGE_LOADS; ++i)
             *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
-                g0.w[i];
+                g.w[i];
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int q = 0; q < XL; ++q)
-                xs[m][q * LM_WAVE + lane] = x0.x[m][q];
-        g0 = g1;
-        x0 = x1;
+                xs[m][q * LM_WAVE + lane] = gx.x[m][q];
         if (s + 2 < n_stage) {
-            stage_load<EB, SL>(w, task, n_out, n_in, s + 2, lane, g1);
-            stage_load_x<EB, MT>(x, ld_x, n_m, n_in, s + 2, lane, x1);
+            stage_load<EB, SL>(w, task, n_out, n_in, s + 2, lane, g);
+            stage_load_x<EB, MT>(x, ld_x, n_m, n_in, s + 2, lane, gx);
         }
         /* steps of this stage: whole blocks of 16 columns, and at the end of the row possibly
          * a block of 8, which only extends chains 0..7 (the lanes with half == 0) */
@@ -232,6 +232,11 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w,
             if (tail8)
                 gemv_step<EB, MT, true>(tile, xs, my_row, half, full, half == 0, acc);
         }
+    };
+    for (int s = 0; s < n_stage; s += 2) {
+        do_stage(s, g0, x0);
+        if (s + 1 < n_stage)
+            do_stage(s + 1, g1, x1);
     }
     /* (chain j + chain j+8), (lane i + lane i+4), ((0+1) + (2+3)): kernel_f16_gemv.c:25-32, 59 */
     const long row = virtual_row<SL>(task, my_row);
