@@ -144,12 +144,14 @@ def bench_spec(w, args):
     print(json.dumps(result))
 
 
-def bench_lm_head(args, m_rows):
-    """Workload lm_head[_mN]: the tail of a decode step for BitNet-2B-4T's geometry, the case the
+def bench_lm_head(args, m_rows, q8=False):
+    """Workload lm_head[_q8][_mN]: the tail of a decode step for BitNet-2B-4T's geometry, the case the
     reference's F16 lm_head kernel was written for (cpu_x86/kernel_f16_gemv.h:7-12): RMS norm of
     the hidden row(s), the tied F16 lm_head [128256 x 2560] (657 MB, read once per step), then the
     headline sampler configuration on the logits, which never leave the device. A step is one
-    such tail for m_rows rows; the dominant kernel is the projection."""
+    such tail for m_rows rows; the dominant kernel is the projection. With q8 the table is the
+    int8 form the reference's x86 backend decodes with (cpu_x86/backend.c:332-372: 328 MB + one
+    scale per row), quantised on the device from the same F16 tables."""
     import torch
     from geistlib_amd import HipSampler, SampleParams
     from geistlib_amd.workloads import xorshift_units
@@ -169,11 +171,21 @@ def bench_lm_head(args, m_rows):
     out = torch.empty(m_rows, dtype=torch.int32, device=dev)
     hs = HipSampler(max_rows=max(m_rows, 1), max_vocab=vocab)
     prm = SampleParams.make(temperature=0.7, top_k=40, top_p=0.9)
-    rows = HipSampler.rows(logits)
+    if q8:
+        tables_q8 = [torch.empty((vocab, d_model), dtype=torch.int8, device=dev) for _ in tables]
+        scales = [torch.empty(vocab, dtype=torch.float32, device=dev) for _ in tables]
+        for t, tq, sc in zip(tables, tables_q8, scales):
+            hs.f16_to_q8w(t, tq, sc)
+        hs.sync()
 
     def step(i=0):
-        hs.project_sample(hidden, norm_w, 1e-6, tables[i % len(tables)], logits, prm, d_u, out,
-                          normed=normed)
+        j = i % len(tables)
+        if q8:
+            hs.project_sample_q8w(hidden, norm_w, 1e-6, tables_q8[j], scales[j], logits, prm, d_u,
+                                  out, normed=normed)
+        else:
+            hs.project_sample(hidden, norm_w, 1e-6, tables[j], logits, prm, d_u, out,
+                              normed=normed)
 
     for i in range(args.warmup):
         step(i)
@@ -186,23 +198,28 @@ def bench_lm_head(args, m_rows):
     ms = elapsed * 1e3 / args.steps
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-    kernel_us = hs.time_f16_gemv(tables, normed, logits, args.steps)  # the projection alone
-    w_bytes = vocab * d_model * 2
+    # the projection alone
+    kernel_us = (hs.time_q8w_gemv(tables_q8, scales, normed, logits, args.steps) if q8
+                 else hs.time_f16_gemv(tables, normed, logits, args.steps))
+    w_bytes = vocab * d_model + vocab * 4 if q8 else vocab * d_model * 2
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
         "metric": "sampled rows/s", "value": round(m_rows * args.steps / elapsed, 1),
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 weights x f32 activations, f32 accumulation",
+        "vs_baseline": None,
+        "dtype": ("int8" if q8 else "f16") + " weights x f32 activations, f32 accumulation",
         "data": "synthetic",
-        "config": {"workload": f"lm_head_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
+        "config": {"workload": f"lm_head{'_q8' if q8 else ''}_v{vocab}_d{d_model}_m{m_rows}",
+                   "rows": m_rows,
                    "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
                    "top_p": 0.9},
         "us_per_step": round(ms * 1e3, 3),
         "weight_copies_rotated": len(tables),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_f16_gemv", "kernel_us": round(kernel_us, 3),
+                     "kernel": "k_q8w_gemv" if q8 else "k_f16_gemv",
+                     "kernel_us": round(kernel_us, 3),
                      "kernel_algorithmic_bytes": w_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
@@ -215,13 +232,21 @@ def bench_lm_head(args, m_rows):
         o = Oracle()
         ref = load_ref_f16gemv(fast=True)
         y = np.empty(vocab, dtype=np.float32)
+        if q8:
+            wq, sc = o.f16_to_q8w(wt)
+        fp = C.POINTER(C.c_float)
         reps, t_used = 0, 0.0
         while reps < 10 and t_used < 10.0:
             t1 = time.perf_counter()
-            if ref is not None:
-                ref.f16_gemv_m1(vocab, d_model, x_host[0].ctypes.data_as(C.POINTER(C.c_float)),
-                                wt.ctypes.data_as(C.POINTER(C.c_uint16)),
-                                y.ctypes.data_as(C.POINTER(C.c_float)))
+            if ref is not None and q8:
+                ref.q8w_gemv_m1(vocab, d_model, x_host[0].ctypes.data_as(fp),
+                                wq.ctypes.data_as(C.POINTER(C.c_int8)), sc.ctypes.data_as(fp),
+                                y.ctypes.data_as(fp))
+            elif ref is not None:
+                ref.f16_gemv_m1(vocab, d_model, x_host[0].ctypes.data_as(fp),
+                                wt.ctypes.data_as(C.POINTER(C.c_uint16)), y.ctypes.data_as(fp))
+            elif q8:
+                y = o.q8w_gemv(wq, sc, x_host[0])
             else:
                 y = o.f16_gemv(wt, x_host[0])
             t_used += time.perf_counter() - t1
@@ -231,15 +256,21 @@ def bench_lm_head(args, m_rows):
             "value": round(reps / t_used, 2), "unit": "rows/s",
             "cores": cores if ref is not None else 1,
             "kind": "reference" if ref is not None else "port",
-            "sample": f"{reps} calls of f16_gemv_m1 on one hidden row (the projection only, "
-                      "no norm, no sampling)"}
+            "sample": f"{reps} calls of {'q8w' if q8 else 'f16'}_gemv_m1 on one hidden row (the "
+                      "projection only, no norm, no sampling)"}
         # parity of the whole tail on the last step's inputs
-        want_logits = o.f16_gemv(wt, o.rmsnorm(hidden.cpu().numpy(), norm_w.cpu().numpy(), 1e-6))
+        x_normed = o.rmsnorm(hidden.cpu().numpy(), norm_w.cpu().numpy(), 1e-6)
+        want_logits = o.q8w_gemv(wq, sc, x_normed) if q8 else o.f16_gemv(wt, x_normed)
         same_bits = bool((want_logits.view(np.uint32) == logits.cpu().numpy().view(np.uint32)).all())
         want_ids = [o.chain_u(want_logits[r], float(u[r]), temperature=0.7, top_k=40, top_p=0.9)[0]
                     for r in range(m_rows)]
         result["parity"] = {"rows": m_rows, "logits_bit_identical": same_bits,
                             "ids_differ": int((np.array(want_ids) != ids_gpu).sum())}
+        if q8:
+            j = (args.steps - 1) % len(tables)
+            result["parity"]["table_bit_identical"] = bool(
+                (tables_q8[j].cpu().numpy() == wq).all()
+                and (scales[j].cpu().numpy().view(np.uint32) == sc.view(np.uint32)).all())
     print(json.dumps(result))
 
 
@@ -269,7 +300,7 @@ def main():
 
     if args.workload.startswith("lm_head"):
         m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
-        return bench_lm_head(args, m)
+        return bench_lm_head(args, m, q8=args.workload.startswith("lm_head_q8"))
     w = build_workload(args.workload)
     if args.workload == "cfg5":
         return bench_spec(w, args)

@@ -95,6 +95,11 @@ def load_library():
                                                   C.POINTER(SampleParams), vp, vp, i32, vp]
     lib.geist_hip_time_f16_gemv_rows.argtypes = [vp, C.POINTER(vp), sz, sz, sz, vp, sz, sz, vp, sz,
                                                  i32, C.POINTER(C.c_double)]
+    lib.geist_hip_project_sample_rows_q8w.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, vp, sz, vp,
+                                                      vp, sz, C.POINTER(SampleParams), vp, vp,
+                                                      i32, vp]
+    lib.geist_hip_time_q8w_gemv_rows.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), sz, sz, sz, vp,
+                                                 sz, sz, vp, sz, i32, C.POINTER(C.c_double)]
     _LIB = lib
     return lib
 
@@ -251,6 +256,30 @@ class HipSampler:
             _ptr(norm_w), eps, _ptr(embed_f16), vocab, _ptr(normed), _ptr(logits),
             logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
             _ptr(rng_states), int(shared), _ptr(out)))
+
+    def project_sample_q8w(self, hidden, norm_w, eps, embed_q8, scales, logits, params, uniforms,
+                           out, normed=None, rng_states=None, shared=True):
+        """project_sample over the int8 table [vocab, d_model] and its per-row scales."""
+        rows, d_model = hidden.shape
+        vocab = embed_q8.shape[0]
+        self._check(self.lib.geist_hip_project_sample_rows_q8w(
+            self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
+            _ptr(norm_w), eps, _ptr(embed_q8), _ptr(scales), vocab, _ptr(normed), _ptr(logits),
+            logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
+            _ptr(rng_states), int(shared), _ptr(out)))
+
+    def time_q8w_gemv(self, weight_copies, scale_copies, x, y, launches):
+        """As time_f16_gemv for q8w_gemv."""
+        n_out, n_in = weight_copies[0].shape
+        m = x.shape[0]
+        wa = (C.c_void_p * len(weight_copies))(*[w.data_ptr() for w in weight_copies])
+        sa = (C.c_void_p * len(scale_copies))(*[w.data_ptr() for w in scale_copies])
+        ms = C.c_double()
+        self._check(self.lib.geist_hip_time_q8w_gemv_rows(
+            self.h, wa, sa, len(weight_copies), n_out, n_in, _ptr(x),
+            x.stride(0) if m > 1 else n_in, m, _ptr(y), y.stride(0) if m > 1 else n_out,
+            int(launches), C.byref(ms)))
+        return ms.value * 1e3 / launches
 
     def time_f16_gemv(self, weight_copies, x, y, launches):
         """Mean duration in microseconds of one f16_gemv call (HIP events on the sampler's stream

@@ -640,25 +640,29 @@ int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const floa
     return after_launch(s, "q8w gemv");
 }
 
-int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
-                                  size_t rows, size_t d_model, const float *d_norm_weight,
-                                  float rms_eps, const uint16_t *d_embed_f16, size_t n_vocab,
-                                  float *d_normed, float *d_logits, size_t ld_logits,
-                                  const struct geist_hip_sample_params *params,
-                                  const float *d_uniforms, uint64_t *d_rng_states, int shared,
-                                  geist_hip_token_t *d_out_tokens) {
-    if (!s)
-        return GEIST_HIP_E_INVALID_ARG;
-    if (!d_hidden || !d_norm_weight || !d_embed_f16 || !d_logits || !params || !d_out_tokens)
+/* Norm, projection and sampling; the table is binary16 (d_scales == NULL) or int8 with one
+ * scale per row. */
+static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
+                               size_t rows, size_t d_model, const float *d_norm_weight,
+                               float rms_eps, const void *d_embed, const float *d_scales,
+                               size_t n_vocab, float *d_normed, float *d_logits, size_t ld_logits,
+                               const struct geist_hip_sample_params *params,
+                               const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                               geist_hip_token_t *d_out_tokens) {
+    const bool      q8          = d_scales != nullptr;
+    const size_t    in_multiple = q8 ? 16 : 8;
+    const uint16_t *d_embed_f16 = (const uint16_t *) d_embed;
+    const int8_t   *d_embed_q8  = (const int8_t *) d_embed;
+    if (!d_hidden || !d_norm_weight || !d_embed || !d_logits || !params || !d_out_tokens)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
     if (rows == 0 || rows > s->max_rows || d_model == 0 || d_model > 0x7ffffff8u ||
         n_vocab == 0 || n_vocab > s->max_vocab || ld_hidden < d_model || ld_logits < n_vocab)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "projection: %zu rows, d_model %zu, vocab %zu",
                     rows, d_model, n_vocab);
-    if (d_model % 8 != 0)
-        return fail(s, GEIST_HIP_E_UNSUPPORTED, "projection: d_model %zu is not a multiple of 8",
-                    d_model);
-    if (((uintptr_t) d_embed_f16) % 16 != 0)
+    if (d_model % in_multiple != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "projection: d_model %zu is not a multiple of %zu",
+                    d_model, in_multiple);
+    if (((uintptr_t) d_embed) % 16 != 0)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "projection: weights not 16-byte aligned");
     Resolved rs;
     int      rc = resolve(s, params, n_vocab, rs);
@@ -680,14 +684,23 @@ int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, s
         GemvFuse f{};
         f.tmax     = s->tmax;
         f.n_chunks = (int) ((n_vocab + 8191) / 8192);
-        launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
-                        (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+        if (q8)
+            launch_q8w_gemv(s->stream, d_embed_q8, d_scales, (long) n_vocab, (int) d_model,
+                            d_normed, (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+        else
+            launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
+                            (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
     } else {
         for (size_t m0 = 0; m0 < rows; m0 += GEMV_M_MAX) {
             const size_t m = rows - m0 < (size_t) GEMV_M_MAX ? rows - m0 : (size_t) GEMV_M_MAX;
-            launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model,
-                            d_normed + m0 * d_model, (long) d_model, (int) m,
-                            d_logits + m0 * ld_logits, (long) ld_logits);
+            if (q8)
+                launch_q8w_gemv(s->stream, d_embed_q8, d_scales, (long) n_vocab, (int) d_model,
+                                d_normed + m0 * d_model, (long) d_model, (int) m,
+                                d_logits + m0 * ld_logits, (long) ld_logits);
+            else
+                launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model,
+                                d_normed + m0 * d_model, (long) d_model, (int) m,
+                                d_logits + m0 * ld_logits, (long) ld_logits);
         }
     }
     if (!rs.greedy && d_rng_states) {
@@ -700,6 +713,38 @@ int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, s
     rc            = sample_impl(s, &r, params, rs.greedy ? nullptr : d_uniforms, d_out_tokens);
     s->tmax_ready = false;
     return rc;
+}
+
+int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
+                                  size_t rows, size_t d_model, const float *d_norm_weight,
+                                  float rms_eps, const uint16_t *d_embed_f16, size_t n_vocab,
+                                  float *d_normed, float *d_logits, size_t ld_logits,
+                                  const struct geist_hip_sample_params *params,
+                                  const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                  geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
+                               d_embed_f16, nullptr, n_vocab, d_normed, d_logits, ld_logits,
+                               params, d_uniforms, d_rng_states, shared, d_out_tokens);
+}
+
+int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidden,
+                                      size_t ld_hidden, size_t rows, size_t d_model,
+                                      const float *d_norm_weight, float rms_eps,
+                                      const int8_t *d_embed_q8, const float *d_scales,
+                                      size_t n_vocab, float *d_normed, float *d_logits,
+                                      size_t ld_logits,
+                                      const struct geist_hip_sample_params *params,
+                                      const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                      geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_scales)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
+                               d_embed_q8, d_scales, n_vocab, d_normed, d_logits, ld_logits,
+                               params, d_uniforms, d_rng_states, shared, d_out_tokens);
 }
 
 int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,
@@ -910,6 +955,38 @@ int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_
     int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
     for (int i = 0; i < launches && !rc; ++i)
         rc = geist_hip_f16_gemv_rows(s, d_w_f16[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
+                                     n_rows, d_y, ld_y);
+    float ms = 0.0f;
+    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
+                hipEventElapsedTime(&ms, a, b) != hipSuccess))
+        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
+    (void) hipEventDestroy(a);
+    (void) hipEventDestroy(b);
+    *ms_total = ms;
+    return rc;
+}
+
+int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,
+                                 const float *const *d_scales, size_t n_weights, size_t n_out,
+                                 size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                 float *d_y, size_t ld_y, int launches, double *ms_total) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (launches < 1 || !ms_total || !d_wq || !d_scales || n_weights < 1)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no weights or null result");
+    for (size_t i = 0; i < n_weights; ++i) { /* argument checks and a warm-up of each copy */
+        const int rc = geist_hip_q8w_gemv_rows(s, d_wq[i], d_scales[i], n_out, n_in, d_x, ld_x,
+                                               n_rows, d_y, ld_y);
+        if (rc)
+            return rc;
+    }
+    hipEvent_t a, b;
+    HIPCHK(s, hipEventCreate(&a));
+    HIPCHK(s, hipEventCreate(&b));
+    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
+    for (int i = 0; i < launches && !rc; ++i)
+        rc = geist_hip_q8w_gemv_rows(s, d_wq[(size_t) i % n_weights],
+                                     d_scales[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
                                      n_rows, d_y, ld_y);
     float ms = 0.0f;
     if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||

@@ -159,11 +159,12 @@ int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logit
     return finalize(h, d_logits, k, out_tokens);
 }
 
-int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
-                                    size_t ld_hidden, size_t k, const float *d_norm_weight,
-                                    float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
-                                    int32_t *out_tokens) {
-    if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed_f16 == nullptr ||
+/* The table is binary16 (d_scales == nullptr) or int8 with one scale per row. */
+static int project_finalize(struct geist_hip_head *h, const float *d_hidden, size_t ld_hidden,
+                            size_t k, const float *d_norm_weight, float rms_eps,
+                            const void *d_embed, const float *d_scales, size_t d_model,
+                            int32_t *out_tokens) {
+    if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed == nullptr ||
         out_tokens == nullptr || k == 0 || d_model == 0)
         return GEIST_HIP_E_INVALID_ARG;
     if (k > h->m_max)
@@ -190,10 +191,18 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
                                                 .repetition_penalty = 1.0f,
                                                 .logit_softcap      = h->logit_softcap,
                                                 .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
-    if (geist_hip_project_sample_rows(h->hs, d_hidden, ld_hidden, k, d_model, d_norm_weight,
-                                      rms_eps, d_embed_f16, h->vocab, h->d_normed, h->d_logits,
-                                      h->vocab, &prm, nullptr, h->d_rng, /*shared=*/1,
-                                      h->d_tokens) != GEIST_HIP_OK)
+    const int rc =
+            d_scales != nullptr
+                    ? geist_hip_project_sample_rows_q8w(h->hs, d_hidden, ld_hidden, k, d_model,
+                                                        d_norm_weight, rms_eps, d_embed, d_scales,
+                                                        h->vocab, h->d_normed, h->d_logits,
+                                                        h->vocab, &prm, nullptr, h->d_rng,
+                                                        /*shared=*/1, h->d_tokens)
+                    : geist_hip_project_sample_rows(h->hs, d_hidden, ld_hidden, k, d_model,
+                                                    d_norm_weight, rms_eps, d_embed, h->vocab,
+                                                    h->d_normed, h->d_logits, h->vocab, &prm,
+                                                    nullptr, h->d_rng, /*shared=*/1, h->d_tokens);
+    if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
     if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
@@ -201,6 +210,25 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
             return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
     return GEIST_HIP_OK;
+}
+
+int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
+                                    size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                    float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
+                                    int32_t *out_tokens) {
+    return project_finalize(h, d_hidden, ld_hidden, k, d_norm_weight, rms_eps, d_embed_f16, nullptr,
+                            d_model, out_tokens);
+}
+
+int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const int8_t *d_embed_q8,
+                                        const float *d_scales, size_t d_model,
+                                        int32_t *out_tokens) {
+    if (d_scales == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    return project_finalize(h, d_hidden, ld_hidden, k, d_norm_weight, rms_eps, d_embed_q8, d_scales,
+                            d_model, out_tokens);
 }
 
 const float *geist_hip_head_logits(const struct geist_hip_head *h) {

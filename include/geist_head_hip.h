@@ -12,6 +12,8 @@
  *                                  (include/geist_backend.h:414-421)
  *   geist_hip_head_project_finalize  output norm + tied F16 lm_head + the above, logits never
  *                                  on the host (head.c:94-188, 224-304)
+ *   geist_hip_head_project_finalize_q8w  the same with the int8 table of the x86 backend
+ *                                  (src/backends/cpu_x86/backend.c:332-372)
  *   geist_hip_head_propose_drafts  the n-gram drafter of geist_session_decode_speculative
  *                                  (src/engine/session.c:437-513, 564-572)
  *   geist_hip_head_spec_accept     the accept loop of geist_session_decode_speculative
@@ -79,7 +81,16 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
                                     size_t ld_hidden, size_t k, const float *d_norm_weight,
                                     float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
                                     int32_t *out_tokens);
-/* The logits of the last geist_hip_head_project_finalize call ([k, vocab], row stride vocab,
+/* The same over the int8 form of the table, which the reference's x86 backend substitutes for
+ * the F16 table in a decode step (src/backends/cpu_x86/backend.c:332-372): d_embed_q8 [vocab,
+ * d_model] int8 and d_scales [vocab] as geist_hip_f16_to_q8w produces them, d_model a multiple
+ * of 16. The logits equal those of the reference's q8w_gemv_m1 bit for bit. */
+int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const int8_t *d_embed_q8,
+                                        const float *d_scales, size_t d_model,
+                                        int32_t *out_tokens);
+/* The logits of the last geist_hip_head_project_finalize[_q8w] call ([k, vocab], row stride vocab,
  * device memory; soft-cap not applied: the sampler applies it while reading), for scoring with
  * geist_hip_logprob_rows in place of geist_session_peek_logits. NULL before the first call. */
 const float *geist_hip_head_logits(const struct geist_hip_head *h);

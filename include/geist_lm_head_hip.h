@@ -71,6 +71,20 @@ int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, s
                                   const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                   geist_hip_token_t *d_out_tokens);
 
+/* The same tail over the int8 form of the table (the reference's default for a decode step on
+ * x86, src/backends/cpu_x86/backend.c:332-342 behind head.c:114-126): d_embed_q8 [n_vocab,
+ * d_model] and d_scales [n_vocab] as geist_hip_f16_to_q8w writes them; d_model a multiple of 16.
+ * Equal in results to geist_hip_rmsnorm_rows + geist_hip_q8w_gemv_rows + the sampler. */
+int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidden,
+                                      size_t ld_hidden, size_t rows, size_t d_model,
+                                      const float *d_norm_weight, float rms_eps,
+                                      const int8_t *d_embed_q8, const float *d_scales,
+                                      size_t n_vocab, float *d_normed, float *d_logits,
+                                      size_t ld_logits,
+                                      const struct geist_hip_sample_params *params,
+                                      const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                      geist_hip_token_t *d_out_tokens);
+
 /* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
  * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
  * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */
@@ -78,6 +92,12 @@ int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_
                                  size_t n_weights, size_t n_out, size_t n_in, const float *d_x,
                                  size_t ld_x, size_t n_rows, float *d_y, size_t ld_y, int launches,
                                  double *ms_total);
+/* The same for geist_hip_q8w_gemv_rows: call i reads d_wq[i % n_weights] and d_scales[i %
+ * n_weights]. */
+int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,
+                                 const float *const *d_scales, size_t n_weights, size_t n_out,
+                                 size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                 float *d_y, size_t ld_y, int launches, double *ms_total);
 
 #ifdef __cplusplus
 }

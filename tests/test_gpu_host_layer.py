@@ -61,6 +61,10 @@ def host():
     lib.geist_hip_head_project_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
                                                     C.c_void_p, C.c_float, C.c_void_p, C.c_size_t,
                                                     C.POINTER(C.c_int32)]
+    lib.geist_hip_head_project_finalize_q8w.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
+                                                        C.c_size_t, C.c_void_p, C.c_float,
+                                                        C.c_void_p, C.c_void_p, C.c_size_t,
+                                                        C.POINTER(C.c_int32)]
     lib.geist_hip_head_logits.restype = C.c_void_p
     lib.geist_hip_head_logits.argtypes = [C.c_void_p]
     lib.geist_hip_head_spec_accept.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
@@ -408,3 +412,33 @@ def test_head_project_finalize_keeps_the_logits_on_the_device(host, oracle):
         assert (got.cpu().numpy().view(np.uint32) == want_logits.view(np.uint32)).all()
         host.geist_hip_head_destroy(h)
     assert (d_hid.cpu().numpy() == hidden).all()                             # input untouched
+
+
+def test_head_project_finalize_q8w_is_the_decode_step_of_the_x86_backend(host, oracle):
+    """The int8 table behind the head (src/backends/cpu_x86/backend.c:332-372 under
+    head.c:114-126): tokens are those of the oracle's session on rmsnorm + q8w_gemv_m1 logits."""
+    g = np.random.default_rng(78)
+    vocab, d_model, cap = 20000, 1536, 30.0
+    w16 = (g.standard_normal((vocab, d_model)) * 0.08).astype(np.float16)
+    wq, sc = oracle.f16_to_q8w(w16.view(np.uint16))
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    d_wq, d_sc, d_nw = torch.from_numpy(wq).cuda(), torch.from_numpy(sc).cuda(), torch.from_numpy(norm_w).cuda()
+    for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.9, 0)]:
+        h = make_head(host, vocab, 0, cap)
+        opts = SessionOpts(0, T, p, top_k, 99, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        sess = oracle.session(T, p, top_k, seed=99)
+        for step in range(3):                                   # three decode steps, one row each
+            hidden = (g.standard_normal((1, d_model)) * 2).astype(np.float32)
+            d_hid = torch.from_numpy(hidden).cuda()
+            out = (C.c_int32 * 1)()
+            rc = host.geist_hip_head_project_finalize_q8w(
+                h, C.c_void_p(d_hid.data_ptr()), d_model, 1, C.c_void_p(d_nw.data_ptr()), 1e-6,
+                C.c_void_p(d_wq.data_ptr()), C.c_void_p(d_sc.data_ptr()), d_model, out)
+            assert rc == 0, host.geist_hip_head_errmsg(h)
+            want_logits = oracle.q8w_gemv(wq, sc, oracle.rmsnorm(hidden, norm_w, 1e-6))
+            assert list(out) == oracle.finalize_batch(sess, want_logits, softcap=cap).tolist(), (T, p, top_k, step)
+        assert host.geist_hip_head_project_finalize_q8w(
+            h, C.c_void_p(d_hid.data_ptr()), d_model, 1, C.c_void_p(d_nw.data_ptr()), 1e-6,
+            C.c_void_p(d_wq.data_ptr()), None, d_model, out) != 0
+        host.geist_hip_head_destroy(h)

@@ -214,3 +214,58 @@ def test_q8w_quantise_and_gemv_bit_exact(hs, oracle, n_out, n_in, m):
     want = oracle.q8w_gemv(wq, sc, x)
     got = y.cpu().numpy()
     assert (bits(got) == bits(want)).all(), np.argwhere(bits(got) != bits(want))[:5]
+
+
+@pytest.mark.parametrize("rows,vocab,d_model", [(1, 40000, 256), (1, 20000, 2560), (2, 9000, 512),
+                                                (3, 8200, 128), (9, 5000, 64)])
+def test_project_sample_rows_q8w_equals_the_separate_steps(hs, oracle, rows, vocab, d_model):
+    """geist_hip_project_sample_rows_q8w: the int8 table in the fused tail. Logits bit-identical
+    to the oracle's rmsnorm + q8w_gemv_m1, tokens those of the oracle's chain on them."""
+    from geistlib_amd import SampleParams
+    print(f"project q8w rows={rows} vocab={vocab} d_model={d_model}", flush=True)
+    g = np.random.default_rng(rows * 77 + vocab + d_model)
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16).view(np.uint16)
+    wq, sc = oracle.f16_to_q8w(w16)
+    hidden = (g.standard_normal((rows, d_model)) * 3).astype(np.float32)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    u = g.random(rows).astype(np.float32)
+    want_logits = oracle.q8w_gemv(wq, sc, oracle.rmsnorm(hidden, norm_w, 1e-6))
+    d_wq, d_sc, d_h, d_nw, d_u = (to_dev(wq, torch), to_dev(sc, torch), to_dev(hidden, torch),
+                                  to_dev(norm_w, torch), to_dev(u, torch))
+    normed = torch.empty((rows, d_model), dtype=torch.float32, device="cuda")
+    for prm in (dict(temperature=0.8, top_k=40, top_p=0.95), dict(temperature=0.0),
+                dict(temperature=0.9, top_p=0.9), dict(temperature=0.8, top_k=40, softcap=20.0),
+                dict(temperature=0.8, top_k=300)):
+        logits = torch.full((rows, vocab), 7.0, dtype=torch.float32, device="cuda")
+        out = torch.full((rows,), -3, dtype=torch.int32, device="cuda")
+        hs.project_sample_q8w(d_h, d_nw, 1e-6, d_wq, d_sc, logits, SampleParams.make(**prm), d_u,
+                              out, normed=normed)
+        hs.sync()
+        assert (bits(logits.cpu().numpy()) == bits(want_logits)).all(), prm
+        kw = {k: v for k, v in prm.items() if k != "softcap"}
+        want = []
+        for r in range(rows):
+            row = want_logits[r]
+            if prm.get("softcap") and prm["temperature"] > 0:
+                row = oracle.softcap(row, prm["softcap"])
+            want.append(oracle.argmax(row) if prm["temperature"] <= 0
+                        else oracle.chain_u(row, float(u[r]), **kw)[0])
+        assert out.cpu().tolist() == want, prm
+
+
+def test_project_sample_rows_q8w_rejects_what_it_cannot_take(hs):
+    from geistlib_amd import SampleParams
+    from geistlib_amd.binding import GeistHipError
+    vocab, d_model = 4096, 72                      # a multiple of 8, not of 16
+    wq = torch.zeros((vocab, d_model), dtype=torch.int8, device="cuda")
+    sc = torch.ones(vocab, dtype=torch.float32, device="cuda")
+    h = torch.ones((1, d_model), dtype=torch.float32, device="cuda")
+    nw = torch.ones(d_model, dtype=torch.float32, device="cuda")
+    logits = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
+    out = torch.empty(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(GeistHipError):
+        hs.project_sample_q8w(h, nw, 1e-6, wq, sc, logits, SampleParams.make(temperature=0.0),
+                              None, out, normed=torch.empty_like(h))
+    with pytest.raises(GeistHipError):
+        hs.project_sample_q8w(h, nw, 1e-6, wq, None, logits, SampleParams.make(temperature=0.0),
+                              None, out, normed=torch.empty_like(h))
