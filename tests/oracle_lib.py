@@ -232,6 +232,18 @@ class Oracle:
         self.lib.oracle_rmsnorm_rows(xs.shape[0], xs.shape[1], _fp(xs), _fp(w), eps, _fp(y))
         return y[0] if np.ndim(x) == 1 else y
 
+    def spec_head_geometry(self, vocab, d_model, stride=0, topk=0):
+        """(sketch_dim, topk) or None where the reference builds no sketch."""
+        sd, k = C.c_size_t(), C.c_size_t()
+        self.lib.oracle_spec_head_geometry.argtypes = [C.c_size_t] * 4 + [C.POINTER(C.c_size_t)] * 2
+        if self.lib.oracle_spec_head_geometry(vocab, d_model, stride, topk, C.byref(sd), C.byref(k)):
+            return None
+        return sd.value, k.value
+
+    def spec_head_build(self, w_f16, stride=0, topk=0):
+        """The reference's sketch of a [vocab, d_model] binary16 table, or None."""
+        return OracleSpecHead(self.lib, w_f16, stride, topk)._or_none()
+
     def softcap(self, row, cap):
         out = row.copy()
         self.lib.oracle_softcap_inplace(out.size, _fp(out), cap)
@@ -336,3 +348,56 @@ def load_ref(fast=False):
     lib.geist_sampler_top_p_ws.argtypes = [C.POINTER(RefWorkspace), c_float_p, C.c_float, C.c_float,
                                            C.POINTER(OracleRng)]
     return lib
+
+
+class _SpecHeadStruct(C.Structure):
+    _fields_ = [("vocab", C.c_size_t), ("d_model", C.c_size_t), ("sketch_dim", C.c_size_t),
+                ("topk", C.c_size_t), ("dims", C.POINTER(C.c_uint32)),
+                ("sketch", C.POINTER(C.c_int8)), ("row_scale", c_float_p),
+                ("w_drop", c_float_p), ("w_l1", c_float_p)]
+
+
+class OracleSpecHead:
+    """oracle_spec_head_build / _try (oracle/spec_head_oracle.h)."""
+
+    def __init__(self, lib, w_f16, stride=0, topk=0):
+        self.lib = lib
+        self.w = np.ascontiguousarray(w_f16, dtype=np.uint16)
+        V, H = self.w.shape
+        lib.oracle_spec_head_build.restype = C.POINTER(_SpecHeadStruct)
+        lib.oracle_spec_head_build.argtypes = [C.POINTER(C.c_uint16)] + [C.c_size_t] * 4
+        lib.oracle_spec_head_free.argtypes = [C.POINTER(_SpecHeadStruct)]
+        lib.oracle_spec_head_free.restype = None
+        lib.oracle_spec_head_try.argtypes = [C.POINTER(_SpecHeadStruct), C.POINTER(C.c_uint16),
+                                             c_float_p, C.c_int, C.POINTER(C.c_int32), c_float_p,
+                                             C.POINTER(C.c_size_t), c_float_p]
+        self.p = lib.oracle_spec_head_build(self.w.ctypes.data_as(C.POINTER(C.c_uint16)), V, H,
+                                            stride, topk)
+        if self.p:
+            st = self.p.contents
+            self.sketch_dim, self.topk = st.sketch_dim, st.topk
+            self.dims = np.ctypeslib.as_array(st.dims, (st.sketch_dim,)).copy()
+            self.sketch = np.ctypeslib.as_array(st.sketch, (V, st.sketch_dim)).copy()
+            self.row_scale = np.ctypeslib.as_array(st.row_scale, (V,)).copy()
+            self.w_drop = np.ctypeslib.as_array(st.w_drop, (V,)).copy()
+            self.w_l1 = np.ctypeslib.as_array(st.w_l1, (V,)).copy()
+
+    def _or_none(self):
+        return self if self.p else None
+
+    def try_row(self, h, verify=False):
+        """-> dict(token, certain, rough, n_finalists, cutoff)."""
+        h = np.ascontiguousarray(h, dtype=np.float32)
+        V = self.w.shape[0]
+        rough = np.empty(V, dtype=np.float32)
+        tok, nf, cut = C.c_int32(), C.c_size_t(), C.c_float()
+        certain = self.lib.oracle_spec_head_try(self.p, self.w.ctypes.data_as(C.POINTER(C.c_uint16)),
+                                                _fp(h), int(verify), C.byref(tok), _fp(rough),
+                                                C.byref(nf), C.byref(cut))
+        return dict(token=tok.value, certain=bool(certain), rough=rough, n_finalists=nf.value,
+                    cutoff=cut.value)
+
+    def __del__(self):
+        if getattr(self, "p", None):
+            self.lib.oracle_spec_head_free(self.p)
+            self.p = None
