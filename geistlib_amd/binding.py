@@ -38,6 +38,20 @@ class SampleParams(C.Structure):
         return cls(temperature, top_p, top_k, min_p, rep, freq, pres, softcap, precedence)
 
 
+class SpecResult(C.Structure):
+    """struct geist_hip_spec_result."""
+    _fields_ = [("token", C.c_int32), ("answered", C.c_int32), ("n_finalists", C.c_int32),
+                ("n_listed", C.c_int32), ("cutoff", C.c_float), ("best_exact", C.c_float)]
+
+
+class SpecHeadView(C.Structure):
+    """struct geist_hip_spec_head_view."""
+    _fields_ = [("n_vocab", C.c_size_t), ("d_model", C.c_size_t), ("sketch_dim", C.c_size_t),
+                ("topk", C.c_size_t), ("d_dims", C.c_void_p), ("d_sketch", C.c_void_p),
+                ("d_row_scale", C.c_void_p), ("d_w_drop", C.c_void_p), ("d_w_l1", C.c_void_p),
+                ("d_rough", C.c_void_p)]
+
+
 def library_path(name="libgeist_sampler_hip.so"):
     return os.path.join(HERE, "lib", name)
 
@@ -100,6 +114,12 @@ def load_library():
                                                       i32, vp]
     lib.geist_hip_time_q8w_gemv_rows.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), sz, sz, sz, vp,
                                                  sz, sz, vp, sz, i32, C.POINTER(C.c_double)]
+    lib.geist_hip_spec_head_geometry.argtypes = [sz, sz, sz, sz, C.POINTER(sz), C.POINTER(sz)]
+    lib.geist_hip_spec_head_build.argtypes = [vp, vp, sz, sz, sz, sz, C.POINTER(vp)]
+    lib.geist_hip_spec_head_destroy.argtypes = [vp, vp]
+    lib.geist_hip_spec_head_destroy.restype = None
+    lib.geist_hip_spec_head_view.argtypes = [vp, C.POINTER(SpecHeadView)]
+    lib.geist_hip_spec_head_try.argtypes = [vp, vp, vp, i32, vp]
     _LIB = lib
     return lib
 
@@ -267,6 +287,34 @@ class HipSampler:
             _ptr(norm_w), eps, _ptr(embed_q8), _ptr(scales), vocab, _ptr(normed), _ptr(logits),
             logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
             _ptr(rng_states), int(shared), _ptr(out)))
+
+    def spec_head_geometry(self, vocab, d_model, stride=0, topk=0):
+        """(sketch_dim, topk), or None where no sketch head is built."""
+        sd, k = C.c_size_t(), C.c_size_t()
+        rc = self.lib.geist_hip_spec_head_geometry(vocab, d_model, stride, topk, C.byref(sd),
+                                                   C.byref(k))
+        return None if rc else (sd.value, k.value)
+
+    def spec_head_build(self, embed_f16, stride=0, topk=0):
+        """Handle of the sketch head over the [vocab, d_model] binary16 table."""
+        vocab, d_model = embed_f16.shape
+        h = C.c_void_p()
+        self._check(self.lib.geist_hip_spec_head_build(self.h, _ptr(embed_f16), vocab, d_model,
+                                                       stride, topk, C.byref(h)))
+        return h
+
+    def spec_head_destroy(self, sh):
+        self.lib.geist_hip_spec_head_destroy(self.h, sh)
+
+    def spec_head_view(self, sh):
+        v = SpecHeadView()
+        self._check(self.lib.geist_hip_spec_head_view(sh, C.byref(v)))
+        return v
+
+    def spec_head_try(self, sh, hidden_normed, result, verify=False):
+        """result: a device buffer of 24 bytes that receives struct geist_hip_spec_result."""
+        self._check(self.lib.geist_hip_spec_head_try(self.h, sh, _ptr(hidden_normed), int(verify),
+                                                     _ptr(result)))
 
     def time_q8w_gemv(self, weight_copies, scale_copies, x, y, launches):
         """As time_f16_gemv for q8w_gemv."""

@@ -11,10 +11,12 @@
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <algorithm>
 #include <vector>
 
 #include "../../include/geist_lm_head_hip.h"
 #include "lm_head_kernels.h"
+#include "spec_head_kernels.h"
 #include "sampler_kernels.h"
 
 using namespace gs;
@@ -964,6 +966,161 @@ int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_
     (void) hipEventDestroy(b);
     *ms_total = ms;
     return rc;
+}
+
+/* ---- speculative output head -------------------------------------------------------------- */
+
+struct geist_hip_spec_head {
+    gs::SpecHeadDev d      = {};
+    int             device = 0;
+};
+
+int geist_hip_spec_head_geometry(size_t n_vocab, size_t d_model, size_t stride_override,
+                                 size_t topk_override, size_t *sketch_dim, size_t *topk) {
+    if (!sketch_dim || !topk || n_vocab == 0 || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    auto clamp = [](size_t v, size_t lo, size_t hi) { return v < lo ? lo : (v > hi ? hi : v); };
+    /* spec_head.c:431-452 */
+    const size_t stride_dflt = d_model > 640 ? d_model / 640 : 1;
+    size_t       sub         = stride_override ? clamp(stride_override, 1, d_model) : stride_dflt;
+    while (sub > 1 && d_model % sub != 0)
+        sub--;
+    const size_t k = topk_override ? clamp(topk_override, 16, n_vocab)
+                                   : (n_vocab >= 200000 ? (size_t) 4096 : (size_t) 1024);
+    if (n_vocab < 8192)
+        return GEIST_HIP_E_UNSUPPORTED;
+    const size_t sd = d_model / sub;
+    if ((double) (2 * d_model) / (double) sd < 3.0)
+        return GEIST_HIP_E_UNSUPPORTED;
+    /* what the kernels take */
+    if (sd % 16 != 0 || sd > (size_t) gs::SPEC_SKETCH_DIM_MAX || d_model % 8 != 0 ||
+        d_model > (size_t) gs::SPEC_D_MODEL_MAX || k > n_vocab / 64 || n_vocab > 0x7fffff00u)
+        return GEIST_HIP_E_UNSUPPORTED;
+    *sketch_dim = sd;
+    *topk       = k;
+    return GEIST_HIP_OK;
+}
+
+void geist_hip_spec_head_destroy(geist_hip_sampler *s, geist_hip_spec_head *sh) {
+    if (!sh)
+        return;
+    (void) s;
+    (void) hipSetDevice(sh->device);
+    gs::SpecHeadDev &d = sh->d;
+    void *ptrs[] = {d.sketch, d.row_scale, d.w_drop, d.w_l1, d.dims, d.kept, d.act, d.rough,
+                    d.tmax, d.sc, d.list_idx, d.list_rough, d.list_exact};
+    for (void *p : ptrs)
+        if (p)
+            (void) hipFree(p);
+    delete sh;
+}
+
+int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16, size_t n_vocab,
+                              size_t d_model, size_t stride_override, size_t topk_override,
+                              geist_hip_spec_head **out) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_embed_f16 || !out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (((uintptr_t) d_embed_f16) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sketch head: table not 16-byte aligned");
+    size_t sd = 0, topk = 0;
+    const int rc = geist_hip_spec_head_geometry(n_vocab, d_model, stride_override, topk_override,
+                                                &sd, &topk);
+    if (rc)
+        return fail(s, rc, "sketch head: no sketch for vocab %zu, d_model %zu", n_vocab, d_model);
+    HIPCHK(s, hipSetDevice(s->device));
+    geist_hip_spec_head *sh = new (std::nothrow) geist_hip_spec_head;
+    if (!sh)
+        return fail(s, GEIST_HIP_E_OOM, "sketch head");
+    sh->device         = s->device;
+    gs::SpecHeadDev &d = sh->d;
+    d.vocab = (long) n_vocab, d.d_model = (int) d_model, d.sketch_dim = (int) sd;
+    d.topk = (int) topk, d.n_chunks = (int) ((n_vocab + 8191) / 8192);
+    d.list_cap = (int) (4 * topk);
+    d.w        = d_embed_f16;
+    float *d_var = nullptr;
+    auto   alloc = [&](auto &p, size_t bytes) {
+        return hipMalloc(reinterpret_cast<void **>(&p), bytes) == hipSuccess;
+    };
+    bool ok = alloc(d.sketch, n_vocab * sd) && alloc(d.row_scale, n_vocab * 4) &&
+              alloc(d.w_drop, n_vocab * 4) && alloc(d.w_l1, n_vocab * 4) && alloc(d.dims, sd * 4) &&
+              alloc(d.kept, d_model) && alloc(d.act, sd * 4) && alloc(d.rough, n_vocab * 4) &&
+              alloc(d.tmax, (size_t) d.n_chunks * 256 * 4) && alloc(d.sc, sizeof(gs::SpecScalars)) &&
+              alloc(d.list_idx, (size_t) d.list_cap * 4) &&
+              alloc(d.list_rough, (size_t) d.list_cap * 4) &&
+              alloc(d.list_exact, (size_t) d.list_cap * 4) && alloc(d_var, d_model * 4);
+    int err = ok ? 0 : GEIST_HIP_E_OOM;
+    std::vector<float>    var(d_model);
+    std::vector<uint32_t> dims(sd);
+    std::vector<uint8_t>  kept(d_model, 0);
+    if (!err) {
+        /* spec_head.c:505-522 on the device, :526-548 here */
+        const long vstep = n_vocab > 512 ? (long) (n_vocab / 512) : 1;
+        gs::launch_spec_dim_stats(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, vstep, d_var);
+        if (hipMemcpyAsync(var.data(), d_var, d_model * 4, hipMemcpyDeviceToHost, s->stream) != hipSuccess ||
+            hipStreamSynchronize(s->stream) != hipSuccess)
+            err = GEIST_HIP_E_BACKEND;
+    }
+    if (!err) {
+        for (size_t k = 0; k < sd; ++k) { /* the first of equals, as the reference's scan */
+            size_t best = 0;
+            for (size_t i = 1; i < d_model; ++i)
+                if (var[i] > var[best])
+                    best = i;
+            dims[k]   = (uint32_t) best;
+            var[best] = -1.0f;
+        }
+        std::sort(dims.begin(), dims.end());
+        for (uint32_t i : dims)
+            kept[i] = 1;
+        if (hipMemcpyAsync(d.dims, dims.data(), sd * 4, hipMemcpyHostToDevice, s->stream) != hipSuccess ||
+            hipMemcpyAsync(d.kept, kept.data(), d_model, hipMemcpyHostToDevice, s->stream) != hipSuccess)
+            err = GEIST_HIP_E_BACKEND;
+    }
+    if (!err) {
+        gs::launch_spec_sketch_rows(s->stream, d);
+        if (hipGetLastError() != hipSuccess || hipStreamSynchronize(s->stream) != hipSuccess)
+            err = GEIST_HIP_E_BACKEND;
+    }
+    if (d_var)
+        (void) hipFree(d_var);
+    if (err) {
+        geist_hip_spec_head_destroy(s, sh);
+        return fail(s, err, err == GEIST_HIP_E_OOM ? "sketch head: out of device memory"
+                                                   : "sketch head: build failed");
+    }
+    *out = sh;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_spec_head_view(const geist_hip_spec_head *sh, struct geist_hip_spec_head_view *out) {
+    if (!sh || !out)
+        return GEIST_HIP_E_INVALID_ARG;
+    const gs::SpecHeadDev &d = sh->d;
+    out->n_vocab = (size_t) d.vocab, out->d_model = (size_t) d.d_model;
+    out->sketch_dim = (size_t) d.sketch_dim, out->topk = (size_t) d.topk;
+    out->d_dims = d.dims, out->d_sketch = d.sketch, out->d_row_scale = d.row_scale;
+    out->d_w_drop = d.w_drop, out->d_w_l1 = d.w_l1, out->d_rough = d.rough;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_spec_head_try(geist_hip_sampler *s, geist_hip_spec_head *sh,
+                            const float *d_hidden_normed, int verify,
+                            struct geist_hip_spec_result *d_result) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!sh || !d_hidden_normed || !d_result)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (sh->device != s->device)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sketch head built on another device");
+    if (((uintptr_t) d_hidden_normed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sketch head: hidden row not 16-byte aligned");
+    static_assert(sizeof(gs::SpecResult) == sizeof(struct geist_hip_spec_result), "result layout");
+    HIPCHK(s, hipSetDevice(s->device));
+    gs::launch_spec_try(s->stream, sh->d, d_hidden_normed, verify != 0,
+                        reinterpret_cast<gs::SpecResult *>(d_result));
+    return after_launch(s, "sketch head");
 }
 
 int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,

@@ -1,0 +1,71 @@
+/* Launchers of the speculative output head (spec_head.hip): the reference's greedy-only
+ * sketch head (src/archs/transformer/forward/spec_head.c) for a tied F16 table in device
+ * memory. */
+#ifndef GEIST_SPEC_HEAD_KERNELS_H
+#define GEIST_SPEC_HEAD_KERNELS_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace gs {
+
+/* Scalars of one call, in device memory. */
+struct SpecScalars {
+    float inv_xq;     /* max|h| / 127 */
+    float h_l1_kept;  /* L1 norm of h over the kept dimensions */
+    float h_l2_drop;  /* L2 norm of h over the dropped dimensions */
+    float threshold;  /* the topk-th largest thread maximum: every row of the topk best is >= it */
+    int   n_listed;   /* rows >= threshold found so far */
+};
+
+/* What a call answers (mirrors struct geist_hip_spec_result). */
+struct SpecResult {
+    int32_t token;
+    int32_t answered;
+    int32_t n_finalists;
+    int32_t n_listed;
+    float   cutoff;
+    float   best_exact;
+};
+
+struct SpecHeadDev {
+    long vocab;
+    int  d_model, sketch_dim, topk, n_chunks, list_cap;
+    const uint16_t *w; /* [vocab, d_model] binary16, not owned */
+    /* built once */
+    int8_t   *sketch;    /* [vocab, sketch_dim] */
+    float    *row_scale; /* [vocab] */
+    float    *w_drop;    /* [vocab] */
+    float    *w_l1;      /* [vocab] */
+    uint32_t *dims;      /* [sketch_dim] ascending */
+    uint8_t  *kept;      /* [d_model] 1 where the sketch keeps the dimension */
+    /* per call */
+    float       *act;   /* [sketch_dim] the kept dimensions of the int8 activation, as floats */
+    float       *rough; /* [vocab] */
+    float       *tmax;  /* [n_chunks * 256] thread maxima of the rough scores */
+    SpecScalars *sc;
+    int32_t     *list_idx;   /* [list_cap] rows >= threshold, any order */
+    float       *list_rough; /* [list_cap] */
+    float       *list_exact; /* [list_cap] their exact logits */
+};
+
+/* Largest d_model the finalist kernel stages in LDS. */
+constexpr int SPEC_D_MODEL_MAX = 5120;
+/* The rough scores are sums of products of two int8 values (|v| <= 127) formed in binary32:
+ * exact while sketch_dim * 127 * 127 < 2^24. */
+constexpr int SPEC_SKETCH_DIM_MAX = 1040;
+
+/* dvar[i] = variance of dimension i over the rows 0, vstep, 2 vstep, ... (spec_head.c:505-522,
+ * binary32, rows in order). */
+void launch_spec_dim_stats(hipStream_t stream, const uint16_t *w, long vocab, int d_model,
+                           long vstep, float *dvar);
+/* sketch, row_scale, w_drop, w_l1 from w, dims and kept (spec_head.c:563-603). */
+void launch_spec_sketch_rows(hipStream_t stream, const SpecHeadDev &d);
+/* transformer_spec_head_try for one normed hidden row h [d_model] (spec_head.c:624-889). */
+void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, bool verify,
+                     SpecResult *result);
+
+} // namespace gs
+#endif

@@ -85,6 +85,65 @@ int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidde
                                       const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                       geist_hip_token_t *d_out_tokens);
 
+/* The reference's speculative output head for greedy decoding
+ * (src/archs/transformer/forward/spec_head.c), over a tied F16 table in device memory: an int8
+ * sketch of the table ranks the vocabulary, only the best-ranked rows get their exact logit.
+ *
+ * geist_hip_spec_head_geometry: the sizes spec_head_build would choose (spec_head.c:431-452):
+ * sketch width d_model / stride, stride = d_model / 640 lowered until it divides d_model
+ * (stride_override > 0 as GEIST_SPEC_STRIDE), finalists 1024 or, from 200000 tokens on, 4096
+ * (topk_override > 0 as GEIST_SPEC_TOPK, clamped to 16..n_vocab). GEIST_HIP_E_UNSUPPORTED where
+ * the reference builds no sketch (n_vocab < 8192, or a sketch row not 3x smaller than a table
+ * row) and where this implementation does not: sketch width not a multiple of 16 or above 1040,
+ * d_model not a multiple of 8 or above 5120, more finalists than n_vocab / 64 (the finalists
+ * are found among the rows that reach the topk-th largest maximum of groups of 32 scores; with
+ * at most every second group involved that is about 1.4 x topk rows).
+ *
+ * geist_hip_spec_head_build replaces spec_head_build (spec_head.c:402-607), run once per model:
+ * the sketch_dim dimensions of largest variance over every (n_vocab / 512)-th row, each row's
+ * values there as int8 with one scale per row, and the two row norms of the certainty bound.
+ * Kept dimensions, int8 values and scales equal the reference's as written (strict IEEE
+ * evaluation); the norms agree to rounding. d_embed_f16 must stay valid while the head is used.
+ *
+ * geist_hip_spec_head_try replaces transformer_spec_head_try (spec_head.c:624-889) for one
+ * normed hidden row: rough scores over the sketch, the topk best of them, exact logits of those
+ * rows in the arithmetic of f16_gemv_m1, the best of them (lowest index first). *d_result
+ * (device memory) receives the token and answered = 1, or answered = 0 when the head declines
+ * and the caller has to run the dense head: with verify != 0 (GEIST_SPEC_VERIFY=1) whenever an
+ * excluded row's upper bound reaches the winner (spec_head.c:846-872); without it only if more
+ * rows tie around the cutoff than the candidate list holds (4 x topk), which the reference's
+ * heap would resolve by its insertion order. Greedy only, as in the reference (spec_head.c:645).
+ * Calls that overlap on one head race: it owns the buffers of a call. */
+typedef struct geist_hip_spec_head geist_hip_spec_head;
+struct geist_hip_spec_result {
+    int32_t token;       /* -1 when not answered without verification */
+    int32_t answered;
+    int32_t n_finalists; /* rows scored exactly that belong to the topk best rough scores */
+    int32_t n_listed;    /* rows scored exactly in all */
+    float   cutoff;      /* the smallest rough score among the finalists */
+    float   best_exact;  /* the winner's logit */
+};
+/* Device pointers into a built head, for inspection. */
+struct geist_hip_spec_head_view {
+    size_t          n_vocab, d_model, sketch_dim, topk;
+    const uint32_t *d_dims;      /* [sketch_dim] ascending */
+    const int8_t   *d_sketch;    /* [n_vocab, sketch_dim] */
+    const float    *d_row_scale; /* [n_vocab] */
+    const float    *d_w_drop;    /* [n_vocab] */
+    const float    *d_w_l1;      /* [n_vocab] */
+    const float    *d_rough;     /* [n_vocab] rough scores of the last try */
+};
+int geist_hip_spec_head_geometry(size_t n_vocab, size_t d_model, size_t stride_override,
+                                 size_t topk_override, size_t *sketch_dim, size_t *topk);
+int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16, size_t n_vocab,
+                              size_t d_model, size_t stride_override, size_t topk_override,
+                              geist_hip_spec_head **out);
+void geist_hip_spec_head_destroy(geist_hip_sampler *s, geist_hip_spec_head *sh);
+int  geist_hip_spec_head_view(const geist_hip_spec_head *sh, struct geist_hip_spec_head_view *out);
+int  geist_hip_spec_head_try(geist_hip_sampler *s, geist_hip_spec_head *sh,
+                             const float *d_hidden_normed, int verify,
+                             struct geist_hip_spec_result *d_result);
+
 /* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
  * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
  * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */

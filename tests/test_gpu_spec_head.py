@@ -1,0 +1,161 @@
+"""The speculative output head on the device (geist_hip_spec_head_*) against the oracle's
+restatement of src/archs/transformer/forward/spec_head.c, through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+from oracle_lib import Oracle  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hs():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=4, max_vocab=70000)
+    yield s
+    s.close()
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    return Oracle()
+
+
+def dev_array(ptr, shape, dtype):
+    """A device array behind a raw pointer, copied to the host."""
+    n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+    out = np.empty(shape, dtype=dtype)
+    rc = C.cdll.LoadLibrary("libamdhip64.so").hipMemcpy(out.ctypes.data_as(C.c_void_p),
+                                                        C.c_void_p(ptr), C.c_size_t(n), 2)
+    assert rc == 0
+    return out
+
+
+def result_of(buf):
+    from geistlib_amd import SpecResult
+    raw = buf.cpu().numpy().tobytes()
+    return SpecResult.from_buffer_copy(raw)
+
+
+def table(g, vocab, d_model, scale=0.05, hot=None):
+    w = (g.standard_normal((vocab, d_model)) * scale).astype(np.float32)
+    if hot is not None:
+        w[:, hot] *= 6.0
+    return w.astype(np.float16)
+
+
+def test_geometry_matches_the_oracle_where_the_device_builds(hs, oracle):
+    for vocab, d_model, stride, topk in [(128256, 2560, 0, 0), (262144, 1536, 0, 0),
+                                         (70000, 4096, 0, 0), (8191, 2560, 0, 0),
+                                         (50000, 512, 0, 0), (70000, 2560, 8, 0),
+                                         (50000, 2560, 0, 300)]:
+        assert hs.spec_head_geometry(vocab, d_model, stride, topk) == \
+            oracle.spec_head_geometry(vocab, d_model, stride, topk), (vocab, d_model, stride, topk)
+    # what the reference would build and the kernels do not take
+    assert hs.spec_head_geometry(40000, 2560) is None          # 1024 finalists > 40000 / 64
+    assert hs.spec_head_geometry(50000, 2560, stride=1) is None   # (and the reference: 2x < 3x)
+    assert hs.spec_head_geometry(50000, 6144) is None          # d_model above the LDS staging
+
+
+@pytest.mark.parametrize("vocab,d_model,topk", [(40000, 1280, 512), (66000, 2560, 0),
+                                                (16500, 1536, 256)])
+def test_build_equals_the_oracle(hs, oracle, vocab, d_model, topk):
+    print(f"spec build vocab={vocab} d_model={d_model} topk={topk}", flush=True)
+    g = np.random.default_rng(vocab + d_model)
+    hot = g.choice(d_model, d_model // 3, replace=False)
+    w16 = table(g, vocab, d_model, hot=hot)
+    w16[5, :] = 0                                             # a row of zeros: scale 1e-8 / 127
+    want = oracle.spec_head_build(w16.view(np.uint16), topk=topk)
+    d_w = torch.from_numpy(w16.view(np.int16)).cuda()
+    sh = hs.spec_head_build(d_w, topk=topk)
+    v = hs.spec_head_view(sh)
+    assert (v.sketch_dim, v.topk) == (want.sketch_dim, want.topk)
+    sd = want.sketch_dim
+    assert (dev_array(v.d_dims, (sd,), np.uint32) == want.dims).all()
+    assert (dev_array(v.d_sketch, (vocab, sd), np.int8) == want.sketch).all()
+    assert (dev_array(v.d_row_scale, (vocab,), np.uint32) == want.row_scale.view(np.uint32)).all()
+    assert np.allclose(dev_array(v.d_w_drop, (vocab,), np.float32), want.w_drop, rtol=2e-6)
+    assert np.allclose(dev_array(v.d_w_l1, (vocab,), np.float32), want.w_l1, rtol=2e-6)
+    hs.spec_head_destroy(sh)
+
+
+@pytest.mark.parametrize("vocab,d_model,topk", [(40000, 1280, 512), (66000, 2560, 0),
+                                                (16500, 1536, 256), (65536, 1280, 1024)])
+def test_try_equals_the_oracle(hs, oracle, vocab, d_model, topk):
+    """Rough scores bit for bit, the same cutoff, finalists and token; with the bound on, the same
+    verdict (and any answer is the dense head's argmax)."""
+    print(f"spec try vocab={vocab} d_model={d_model} topk={topk}", flush=True)
+    g = np.random.default_rng(7 * vocab + d_model)
+    hot = g.choice(d_model, d_model // 3, replace=False)
+    w16 = table(g, vocab, d_model, hot=hot)
+    want_sh = oracle.spec_head_build(w16.view(np.uint16), topk=topk)
+    d_w = torch.from_numpy(w16.view(np.int16)).cuda()
+    sh = hs.spec_head_build(d_w, topk=topk)
+    v = hs.spec_head_view(sh)
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    answered = 0
+    for trial in range(6):
+        h = (g.standard_normal(d_model) * g.choice([0.3, 1.0, 5.0])).astype(np.float32)
+        if trial == 4:
+            h[:] = 0                                        # every rough score equal
+        if trial == 5:                                      # one row far above the rest
+            h = np.zeros(d_model, dtype=np.float32)
+            h[want_sh.dims] = w16[777, want_sh.dims].astype(np.float32) * 100
+        d_h = torch.from_numpy(h).cuda()
+        for verify in (False, True):
+            want = want_sh.try_row(h, verify=verify)
+            hs.spec_head_try(sh, d_h, res, verify=verify)
+            hs.sync()
+            got = result_of(res)
+            rough = dev_array(v.d_rough, (vocab,), np.uint32)
+            assert (rough == want["rough"].view(np.uint32)).all(), (trial, verify)
+            if trial == 4:
+                # all scores tie: more rows around the cutoff than the list holds, no answer
+                assert got.answered == 0 and got.token == -1
+                continue
+            assert got.n_finalists == want["n_finalists"] == want_sh.topk
+            assert got.cutoff == want["cutoff"], (trial, verify)
+            assert got.n_listed >= got.n_finalists
+            assert got.token == want["token"], (trial, verify)
+            assert bool(got.answered) == want["certain"], (trial, verify)
+            if verify and got.answered:
+                answered += 1
+                dense = oracle.f16_gemv(w16.view(np.uint16), h)
+                assert got.token == int(np.flatnonzero(dense == dense.max())[0])
+                assert np.float32(got.best_exact) == dense.max()
+    assert answered >= 1                                    # trial 5 is certified
+    hs.spec_head_destroy(sh)
+
+
+def test_finalist_logits_are_the_dense_heads(hs, oracle):
+    """Without the bound the answer is the best exact logit among the finalists; its value must
+    be the dense kernel's in every bit."""
+    g = np.random.default_rng(99)
+    for vocab, d_model in [(66000, 1536), (70000, 2560)]:
+        w16 = table(g, vocab, d_model, scale=0.3)
+        d_w = torch.from_numpy(w16.view(np.int16)).cuda()
+        sh = hs.spec_head_build(d_w)
+        res = torch.zeros(6, dtype=torch.int32, device="cuda")
+        for _ in range(4):
+            h = (g.standard_normal(d_model) * 3).astype(np.float32)
+            hs.spec_head_try(sh, torch.from_numpy(h).cuda(), res)
+            hs.sync()
+            got = result_of(res)
+            assert got.answered == 1
+            y = oracle.f16_gemv(w16.view(np.uint16)[got.token:got.token + 1], h)
+            assert np.float32(got.best_exact).view(np.uint32) == y.view(np.uint32)[0]
+        hs.spec_head_destroy(sh)
+
+
+def test_rejects_what_it_cannot_take(hs):
+    from geistlib_amd.binding import GeistHipError
+    w = torch.zeros((9000, 2560), dtype=torch.float16, device="cuda")
+    with pytest.raises(GeistHipError):
+        hs.spec_head_build(w)                                # 1024 finalists > 9000 / 64
+    with pytest.raises(GeistHipError):
+        hs.spec_head_build(torch.zeros((40000, 512), dtype=torch.float16, device="cuda"))
