@@ -274,6 +274,112 @@ def bench_lm_head(args, m_rows, q8=False):
     print(json.dumps(result))
 
 
+class _DevPtr:
+    """A device array known by its address only, for the timing entry points."""
+
+    def __init__(self, ptr, shape):
+        self.ptr, self.shape = ptr, shape
+
+    def data_ptr(self):
+        return self.ptr
+
+
+def bench_lm_head_spec(args):
+    """Workload lm_head_spec: the tail of a greedy decode step for BitNet-2B-4T's geometry through
+    the reference's speculative output head (forward/spec_head.c): RMS norm of the hidden row,
+    rough scores of the 128256 rows over a 640-dimension int8 sketch (82 MB), the 1024 best-ranked
+    rows scored exactly against the F16 table, the best of them. A step is one such tail; the
+    dominant kernel is the int8 projection over the sketch."""
+    import torch
+    from geistlib_amd import HipSampler, SpecResult
+    vocab, d_model = 128256, 2560
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    hs = HipSampler(max_rows=1, max_vocab=vocab)
+    # three tables and their sketches (3 x 739 MB): every step's sketch and finalist rows come
+    # from HBM
+    tables = [(torch.randn((vocab, d_model), device=dev, generator=g) * 0.05).to(torch.float16)
+              for _ in range(3)]
+    heads = [hs.spec_head_build(t) for t in tables]
+    views = [hs.spec_head_view(sh) for sh in heads]
+    sd, topk = views[0].sketch_dim, views[0].topk
+    hidden = torch.randn((1, d_model), device=dev, generator=g) * 3
+    norm_w = 1.0 + 0.1 * torch.randn((d_model,), device=dev, generator=g)
+    normed = torch.empty_like(hidden)
+    res = torch.zeros(6, dtype=torch.int32, device=dev)
+
+    def step(i=0):
+        hs.rmsnorm(hidden, norm_w, 1e-6, normed)
+        hs.spec_head_try(heads[i % len(heads)], normed, res)
+
+    for i in range(args.warmup):
+        step(i)
+    hs.sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    hs.sync()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed * 1e3 / args.steps
+    got = SpecResult.from_buffer_copy(res.cpu().numpy().tobytes())
+    # the projection over the sketch alone
+    act = torch.randint(-127, 128, (1, sd), device=dev, generator=g).to(torch.float32)
+    rough = torch.empty((1, vocab), dtype=torch.float32, device=dev)
+    kernel_us = hs.time_q8w_gemv([_DevPtr(v.d_sketch, (vocab, sd)) for v in views],
+                                 [_DevPtr(v.d_row_scale, (vocab,)) for v in views], act, rough,
+                                 args.steps)
+    k_bytes = vocab * sd + vocab * 4
+    achieved = k_bytes / (kernel_us * 1e-6) / 1e9
+    result = {
+        "metric": "sampled rows/s", "value": round(args.steps / elapsed, 1), "unit": "rows/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 sketch x int8 activations (exact in f32), f16 x f32 finalists",
+        "data": "synthetic",
+        "config": {"workload": f"lm_head_spec_v{vocab}_d{d_model}", "rows": 1, "n_vocab": vocab,
+                   "d_model": d_model, "sketch_dim": sd, "finalists": topk, "temperature": 0.0},
+        "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": len(tables),
+        "finalists_scored": got.n_listed,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_q8w_gemv", "kernel_us": round(kernel_us, 3),
+                     "kernel_algorithmic_bytes": k_bytes,
+                     "step_algorithmic_bytes": k_bytes + vocab * 8 + got.n_listed * d_model * 2
+                     + d_model * 8},
+    }
+    if not args.no_cpu:
+        # the oracle's restatement of spec_head.c on this host's cores (its rough-score loop runs
+        # on OpenMP threads as the reference's does; heap and finalists are serial there too)
+        from oracle_lib import Oracle
+        o = Oracle()
+        j = (args.steps - 1) % len(tables)
+        wt = tables[j].cpu().numpy().view(np.uint16)
+        sh = o.spec_head_build(wt)
+        x_host = normed.cpu().numpy()[0]
+        reps, t_used = 0, 0.0
+        while reps < 20 and t_used < 10.0:
+            t1 = time.perf_counter()
+            want = sh.try_row(x_host)
+            t_used += time.perf_counter() - t1
+            reps += 1
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 10 ** 6)
+        result["cpu_baseline"] = {"value": round(reps / t_used, 2), "unit": "rows/s", "cores": cores,
+                                  "kind": "port",
+                                  "sample": f"{reps} calls of the sketch head on one normed row "
+                                            "(sketch built beforehand, no norm)"}
+        dense = o.f16_gemv(wt, x_host)
+        result["parity"] = {"rows": 1, "ids_differ": int(got.token != want["token"]),
+                            "cutoff_identical": bool(got.cutoff == want["cutoff"]),
+                            "token_is_dense_argmax": bool(got.token == int(np.argmax(dense))),
+                            "winner_logit_bit_identical": bool(
+                                np.float32(got.best_exact).view(np.uint32)
+                                == dense[got.token].view(np.uint32))}
+    for sh_ in heads:
+        hs.spec_head_destroy(sh_)
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -298,6 +404,8 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: the sampling path has no CPU fallback")
 
+    if args.workload == "lm_head_spec":
+        return bench_lm_head_spec(args)
     if args.workload.startswith("lm_head"):
         m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
         return bench_lm_head(args, m, q8=args.workload.startswith("lm_head_q8"))

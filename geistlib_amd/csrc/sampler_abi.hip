@@ -993,8 +993,9 @@ int geist_hip_spec_head_geometry(size_t n_vocab, size_t d_model, size_t stride_o
     if ((double) (2 * d_model) / (double) sd < 3.0)
         return GEIST_HIP_E_UNSUPPORTED;
     /* what the kernels take */
-    if (sd % 16 != 0 || sd > (size_t) gs::SPEC_SKETCH_DIM_MAX || d_model % 8 != 0 ||
-        d_model > (size_t) gs::SPEC_D_MODEL_MAX || k > n_vocab / 64 || n_vocab > 0x7fffff00u)
+    if (sd % 16 != 0 || sd > (size_t) gs::SPEC_SKETCH_DIM_MAX || d_model % 16 != 0 ||
+        d_model > (size_t) gs::SPEC_D_MODEL_MAX || k > n_vocab / 64 ||
+        k > (size_t) gs::SPEC_TOPK_MAX || n_vocab > (size_t) gs::SPEC_VOCAB_MAX)
         return GEIST_HIP_E_UNSUPPORTED;
     *sketch_dim = sd;
     *topk       = k;
@@ -1008,7 +1009,7 @@ void geist_hip_spec_head_destroy(geist_hip_sampler *s, geist_hip_spec_head *sh) 
     (void) hipSetDevice(sh->device);
     gs::SpecHeadDev &d = sh->d;
     void *ptrs[] = {d.sketch, d.row_scale, d.w_drop, d.w_l1, d.dims, d.kept, d.act, d.rough,
-                    d.tmax, d.sc, d.list_idx, d.list_rough, d.list_exact};
+                    d.tmax, d.sc, d.list_idx, d.list_rough, d.fin_idx, d.fin_exact};
     for (void *p : ptrs)
         if (p)
             (void) hipFree(p);
@@ -1037,7 +1038,7 @@ int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16,
     gs::SpecHeadDev &d = sh->d;
     d.vocab = (long) n_vocab, d.d_model = (int) d_model, d.sketch_dim = (int) sd;
     d.topk = (int) topk, d.n_chunks = (int) ((n_vocab + 8191) / 8192);
-    d.list_cap = (int) (4 * topk);
+    d.list_cap = (int) (2 * topk);
     d.w        = d_embed_f16;
     float *d_var = nullptr;
     auto   alloc = [&](auto &p, size_t bytes) {
@@ -1049,7 +1050,8 @@ int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16,
               alloc(d.tmax, (size_t) d.n_chunks * 256 * 4) && alloc(d.sc, sizeof(gs::SpecScalars)) &&
               alloc(d.list_idx, (size_t) d.list_cap * 4) &&
               alloc(d.list_rough, (size_t) d.list_cap * 4) &&
-              alloc(d.list_exact, (size_t) d.list_cap * 4) && alloc(d_var, d_model * 4);
+              alloc(d.fin_idx, topk * 4) && alloc(d.fin_exact, topk * 4) &&
+              alloc(d_var, d_model * 4);
     int err = ok ? 0 : GEIST_HIP_E_OOM;
     std::vector<float>    var(d_model);
     std::vector<uint32_t> dims(sd);

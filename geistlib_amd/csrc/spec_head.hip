@@ -13,13 +13,13 @@
  *                     sums below 2^24 (sketch_dim <= 1040), so the scores equal the reference's
  *                     integer dot bit for bit. Its epilogue leaves the maxima of groups of 32
  *                     scores (the sampler's thread maxima).
- *   k_spec_threshold  the topk-th largest of those maxima: at least topk scores reach it, so
- *                     the topk best rows are among the rows >= it (about 1.1 topk rows)
- *   k_spec_gather     finds those rows and computes their exact logits, one wavefront per row,
- *                     in the order of summation of f16_gemv_m1 (16 chains, fixed tree), so that
- *                     a finalist's logit is the dense head's in every bit
- *   k_spec_final      the topk best rough scores among the listed rows (the reference's heap),
- *                     the best exact logit among them, lowest index first
+ *   k_spec_select     the topk-th largest of those maxima: at least topk scores reach it, so
+ *                     the topk best rows are among the rows >= it (about 1.1 topk rows); it
+ *                     reads those groups again and keeps the topk best (the reference's heap)
+ *   k_spec_exact      their exact logits, one wavefront per row, in the order of summation of
+ *                     f16_gemv_m1 (16 chains, fixed tree), so that a finalist's logit is the
+ *                     dense head's in every bit
+ *   k_spec_final      the best exact logit among them, lowest index first
  *   k_spec_verify     (optional, GEIST_SPEC_VERIFY) the upper bound of every excluded row
  *                     against the winner; any row that could have won withdraws the answer
  *
@@ -71,54 +71,77 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-/* Inclusive scan over the 256 threads of a workgroup; s_w[4] is scratch. */
-__device__ __forceinline__ int block_incl_scan(int v, int *s_w) {
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    int       x    = v;
-#pragma unroll
-    for (int d = 1; d < SP_WAVE; d <<= 1) {
-        const int y = __shfl_up(x, d, SP_WAVE);
-        if (lane >= d)
-            x += y;
-    }
-    if (lane == 63)
-        s_w[wv] = x;
-    __syncthreads();
-    int add = 0;
-    for (int i = 0; i < wv; ++i)
-        add += s_w[i];
-    __syncthreads();
-    return x + add;
+/* One count for this lane's digit (if valid). Keys that order like floats share their leading
+ * digits, and atomics of one wavefront on one LDS word are serialised: the lanes that hold the
+ * digit of the first valid lane add their count in one operation, the others one by one. */
+__device__ __forceinline__ void hist_add(int *s_hist, uint32_t digit, bool valid) {
+    const unsigned long long todo = __ballot(valid);
+    if (todo == 0)
+        return;
+    const int                leader = __builtin_ctzll(todo);
+    const uint32_t           dl = (uint32_t) __builtin_amdgcn_readlane((int) digit, leader);
+    const unsigned long long m  = __ballot(valid && digit == dl);
+    if ((int) (threadIdx.x & 63) == leader)
+        atomicAdd(&s_hist[dl], __builtin_popcountll(m));
+    if (valid && digit != dl)
+        atomicAdd(&s_hist[digit], 1);
 }
 
-/* The k-th largest (1 <= k <= n) of the n keys key_at(i), by four 8-bit radix passes of the
- * whole workgroup; need_ties = how many of the keys equal to it belong to the k largest. */
-template <typename KeyAt>
-__device__ uint32_t block_kth_largest(KeyAt key_at, int n, int k, int *s_hist, int *s_w, int *s_sel,
-                                      int &need_ties) {
-    const int tid    = threadIdx.x;
-    uint32_t  prefix = 0, mask = 0;
-    int       remaining = k;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        s_hist[tid] = 0;
+/* The k-th largest (1 <= k <= n) of the keys the workgroup's threads hold in registers (thread t
+ * holds keys[e] for the elements e * blockDim.x + t < n), by four 8-bit radix passes;
+ * need_ties = how many of the keys equal to it belong to the k largest. s_hist is [4][256].
+ * With PASSES < 4 only the leading 8 * PASSES bits are resolved: the result is the k-th largest
+ * key with its other bits cleared (a lower bound of it that at least k keys reach).
+ * Each pass costs two workgroup barriers: all wavefronts count their digits, then the first
+ * wavefront alone finds the digit that holds the k-th key (lane l owns the digits 255 - 4 l ..
+ * 252 - 4 l, so that a scan over the lanes runs from the largest digit down). */
+template <int EPT, int PASSES = 4>
+__device__ uint32_t block_kth_largest(const uint32_t (&keys)[EPT], int n, int k, int (*s_hist)[256],
+                                      int *s_sel, int &need_ties) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < 4 * 256; i += (int) blockDim.x)
+        (&s_hist[0][0])[i] = 0;
+    __syncthreads();
+    uint32_t prefix = 0, mask = 0;
+    int      remaining = k;
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+        const int shift = 24 - 8 * pass;
+#pragma unroll
+        for (int e = 0; e < EPT; ++e)
+            hist_add(s_hist[pass], (keys[e] >> shift) & 255u,
+                     e * (int) blockDim.x + tid < n && (keys[e] & mask) == prefix);
         __syncthreads();
-        for (int i = tid; i < n; i += SP_TPB) {
-            const uint32_t key = key_at(i);
-            if ((key & mask) == prefix)
-                atomicAdd(&s_hist[(key >> shift) & 255u], 1);
-        }
-        __syncthreads();
-        const int mine = s_hist[255 - tid]; /* thread t owns digit 255 - t: descending order */
-        const int incl = block_incl_scan(mine, s_w);
-        if (incl >= remaining && incl - mine < remaining) {
-            s_sel[0] = 255 - tid;
-            s_sel[1] = remaining - (incl - mine);
+        if (tid < SP_WAVE) {
+            int c[4], local = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                c[j] = s_hist[pass][255 - 4 * lane - j];
+                local += c[j];
+            }
+            int incl = local;
+#pragma unroll
+            for (int d = 1; d < SP_WAVE; d <<= 1) {
+                const int y = __shfl_up(incl, d, SP_WAVE);
+                if (lane >= d)
+                    incl += y;
+            }
+            int r = remaining - (incl - local);
+            if (r >= 1 && r <= local) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (r >= 1 && r <= c[j]) {
+                        s_sel[0] = 255 - 4 * lane - j;
+                        s_sel[1] = r;
+                    }
+                    r -= c[j];
+                }
+            }
         }
         __syncthreads();
         prefix |= (uint32_t) s_sel[0] << shift;
         mask |= 255u << shift;
         remaining = s_sel[1];
-        __syncthreads();
     }
     need_ties = remaining;
     return prefix;
@@ -229,131 +252,279 @@ __global__ __launch_bounds__(SP_TPB) void k_spec_act(SpecHeadDev d, const float 
         d.sc->inv_xq      = __fdiv_rn(1.0f, x_q);
         d.sc->h_l1_kept   = (float) b;
         d.sc->h_l2_drop   = (float) sqrt(drop);
-        d.sc->n_listed    = 0;
     }
 }
 
-__global__ __launch_bounds__(SP_TPB) void k_spec_threshold(SpecHeadDev d) {
-    __shared__ int s_hist[256], s_w[4], s_sel[2];
-    const float   *tm = d.tmax;
+constexpr int SP_SEL_TPB = 1024; /* the two selection kernels: keys live in registers */
+
+/* Phase 2 of the head (spec_head.c:728-770), one workgroup of 1024 threads:
+ *   1. the topk-th largest thread maximum: at least topk rough scores reach it, so the topk best
+ *      rows are among the rows >= it. Thread maximum i (chunk i / 256, scanning thread t =
+ *      i % 256) covers the rows chunk * 8192 + 4 * (j * 256 + t) + c, j < 8, c < 4 (the
+ *      sampler's top-k scan layout, which the projection's epilogue writes);
+ *   2. only the groups whose maximum reaches that threshold are read again, their rows >= it
+ *      are the candidates (about 1.1 topk, at most 2 topk);
+ *   3. the topk-th largest candidate is the reference's cutoff (its heap's smallest entry); the
+ *      finalists are the candidates above it and, of those equal to it, as many as complete
+ *      topk rows -- the lowest indices first.
+ * Thread t holds the maxima e * 1024 + t and later the candidates e * 1024 + t. */
+template <int EPT, int EPT2>
+__global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    int *s_ent = reinterpret_cast<int *>(smem); /* [list_cap] groups to read again */
+    __shared__ int s_hist[4][256], s_w[16], s_sel[2], s_n[3];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int n   = d.n_chunks * 256;
+    uint32_t  keys[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int i = e * SP_SEL_TPB + tid;
+        keys[e]     = i < n ? ordered_key(d.tmax[i]) : 0u;
+    }
+    if (tid < 3)
+        s_n[tid] = 0;
+    /* (16 bits of the threshold are enough: it only has to be reached by at least topk maxima
+     * and by few more rows than topk; the exact cutoff comes from the candidates below) */
     int            ties;
-    const uint32_t key = block_kth_largest([tm](int i) { return ordered_key(tm[i]); },
-                                           d.n_chunks * 256, d.topk, s_hist, s_w, s_sel, ties);
-    if (threadIdx.x == 0)
-        d.sc->threshold = key_to_float(key);
+    const uint32_t tkey = block_kth_largest<EPT, 2>(keys, n, d.topk, s_hist, s_sel, ties);
+    const float    thr  = key_to_float(tkey);
+    /* 2a. the groups that reach the threshold */
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int  i   = e * SP_SEL_TPB + tid;
+        const bool hit = i < n && keys[e] >= tkey && keys[e] != 0u;
+        const unsigned long long m = __ballot(hit);
+        if (m == 0)
+            continue;
+        int base = 0;
+        if (lane == 0)
+            base = atomicAdd(&s_n[0], __builtin_popcountll(m));
+        base = __builtin_amdgcn_readfirstlane(base);
+        const int slot = base + __builtin_popcountll(m & ((1ull << lane) - 1ull));
+        if (hit && slot < d.list_cap)
+            s_ent[slot] = i;
+    }
+    __syncthreads();
+    const int n_ent = s_n[0] < d.list_cap ? s_n[0] : d.list_cap;
+    /* 2b. their rows that reach it */
+    for (int it = tid; it - lane < n_ent; it += SP_SEL_TPB) { /* (whole wavefronts) */
+        const bool live = it < n_ent;
+        const int  i    = live ? s_ent[it] : 0;
+        const long base = (long) (i >> 8) * 8192 + 4 * (i & 255);
+        float      v[32];
+        int        c = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const long r0 = base + (long) j * 1024;
+            if (live && r0 + 3 < d.vocab) { /* (rough is 16-byte aligned, r0 a multiple of 4) */
+                const float4 f = *reinterpret_cast<const float4 *>(d.rough + r0);
+                v[4 * j] = f.x, v[4 * j + 1] = f.y, v[4 * j + 2] = f.z, v[4 * j + 3] = f.w;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    v[4 * j + q] = (live && r0 + q < d.vocab) ? d.rough[r0 + q] : -__builtin_inff();
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 32; ++j)
+            c += v[j] >= thr ? 1 : 0;
+        int incl = c;
+#pragma unroll
+        for (int sft = 1; sft < SP_WAVE; sft <<= 1) {
+            const int y = __shfl_up(incl, sft, SP_WAVE);
+            if (lane >= sft)
+                incl += y;
+        }
+        int wbase = 0;
+        if (lane == 63)
+            wbase = atomicAdd(&s_n[1], incl);
+        wbase    = __shfl(wbase, 63, SP_WAVE);
+        int slot = wbase + incl - c;
+#pragma unroll
+        for (int j = 0; j < 32; ++j)
+            if (v[j] >= thr) {
+                if (slot < d.list_cap) {
+                    d.list_idx[slot]   = (int32_t) (base + (long) (j >> 2) * 1024 + (j & 3));
+                    d.list_rough[slot] = v[j];
+                }
+                ++slot;
+            }
+    }
+    __syncthreads(); /* (the candidates written above are visible to the whole workgroup) */
+    const int n_cand = s_n[1];
+    if (s_n[0] > d.list_cap || n_cand > d.list_cap || n_cand < d.topk) { /* (uniform) */
+        if (tid == 0) {
+            d.sc->threshold = thr, d.sc->cutoff = thr, d.sc->n_cand = n_cand, d.sc->n_final = 0;
+        }
+        return;
+    }
+    /* 3. the cutoff and the finalists */
+    uint32_t ck[EPT2];
+    int32_t  ci[EPT2];
+#pragma unroll
+    for (int e = 0; e < EPT2; ++e) {
+        const int i = e * SP_SEL_TPB + tid;
+        ck[e]       = i < n_cand ? ordered_key(d.list_rough[i]) : 0u;
+        ci[e]       = i < n_cand ? d.list_idx[i] : -1;
+    }
+    int            need_ties;
+    const uint32_t ckey = block_kth_largest<EPT2>(ck, n_cand, d.topk, s_hist, s_sel, need_ties);
+    int tie_cnt = 0;
+#pragma unroll
+    for (int e = 0; e < EPT2; ++e)
+        tie_cnt += (ci[e] >= 0 && ck[e] == ckey) ? 1 : 0;
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1)
+        tie_cnt += __shfl_xor(tie_cnt, sft, SP_WAVE);
+    if (lane == 0)
+        s_w[tid >> 6] = tie_cnt;
+    __syncthreads();
+    tie_cnt = 0;
+    for (int i = 0; i < SP_SEL_TPB / SP_WAVE; ++i)
+        tie_cnt += s_w[i];
+#pragma unroll
+    for (int e = 0; e < EPT2; ++e) {
+        bool in = ci[e] >= 0 && ck[e] > ckey;
+        if (ci[e] >= 0 && ck[e] == ckey) {
+            in = true;
+            if (tie_cnt > need_ties) { /* the lowest indices among the rows that tie */
+                int before = 0;
+                for (int j = 0; j < n_cand; ++j)
+                    before += (d.list_idx[j] < ci[e] && ordered_key(d.list_rough[j]) == ckey) ? 1 : 0;
+                in = before < need_ties;
+            }
+        }
+        const unsigned long long m = __ballot(in);
+        if (m == 0)
+            continue;
+        int base = 0;
+        if (lane == 0)
+            base = atomicAdd(&s_n[2], __builtin_popcountll(m));
+        base = __builtin_amdgcn_readfirstlane(base);
+        const int slot = base + __builtin_popcountll(m & ((1ull << lane) - 1ull));
+        if (in && slot < d.topk)
+            d.fin_idx[slot] = ci[e];
+    }
+    __syncthreads();
+    if (tid == 0) {
+        d.sc->threshold = thr;
+        d.sc->cutoff    = key_to_float(ckey);
+        d.sc->n_cand    = n_cand;
+        d.sc->n_final   = s_n[2]; /* == topk */
+    }
 }
 
-/* Rows whose rough score reaches the threshold, and their exact logits. Thread t of workgroup b
- * looks at row 256 b + t; every such row is then worked on by its whole wavefront: the row comes
- * into LDS with coalesced 16-byte loads, lanes 0..15 each run one of f16_gemv_m1's sixteen
- * chains over it (element k belongs to chain k % 16; a trailing block of eight extends chains
- * 0..7), and the chains are folded as there: (j + j+8), (i + i+4), ((0+1) + (2+3))
- * (src/backends/cpu_x86/kernel_f16_gemv.c:25-32, 40-59). */
-__global__ __launch_bounds__(SP_TPB) void k_spec_gather(SpecHeadDev d, const float *__restrict__ h) {
+/* Phase 3 (spec_head.c:802-826): the exact logit of every finalist, one wavefront per row, in
+ * f16_gemv_m1's order of summation (src/backends/cpu_x86/kernel_f16_gemv.c:25-32, 40-59):
+ * sixteen chains of fused multiply-adds, element k in chain k % 16, folded as (j + j+8),
+ * (i + i+4), ((0+1) + (2+3)). Lane c < 16 runs chain c. Row and activations are laid out in LDS
+ * by chain (element k at (k % 16) * pitch + k / 16), so that a lane reads its chain's next
+ * eight weights with one 16-byte load. d_model is a multiple of 16. */
+__global__ __launch_bounds__(SP_TPB) void k_spec_exact(SpecHeadDev d, const float *__restrict__ h) {
     extern __shared__ __align__(16) uint8_t smem[];
-    float    *s_x   = reinterpret_cast<float *>(smem);
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    uint16_t *s_row = reinterpret_cast<uint16_t *>(smem + (size_t) d.d_model * 4) +
-                      (size_t) wv * d.d_model;
-    const long  r   = (long) blockIdx.x * SP_TPB + tid;
-    const float thr = d.sc->threshold;
-    const float val = r < d.vocab ? d.rough[r] : -__builtin_inff();
-    const bool  hit = r < d.vocab && val >= thr;
-    if (__syncthreads_or(hit) == 0)
-        return;
-    for (int i = tid * 4; i < d.d_model; i += SP_TPB * 4)
-        *reinterpret_cast<float4 *>(s_x + i) = *reinterpret_cast<const float4 *>(h + i);
-    __syncthreads();
-    unsigned long long mask = __ballot(hit);
-    const int          n16  = d.d_model & ~15;
-    while (mask) {
-        const int  bit = __builtin_ctzll(mask);
-        mask &= mask - 1;
-        const long cr  = (long) blockIdx.x * SP_TPB + wv * SP_WAVE + bit;
-        const uint16_t *src = d.w + cr * d.d_model;
-        for (int o = lane * 8; o < d.d_model; o += SP_WAVE * 8)
-            *reinterpret_cast<nt_u4 *>(s_row + o) =
-                __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(src + o));
-        float acc = 0.0f;
-        if (lane < 16) {
-            for (int k = lane; k < n16; k += 16)
-                acc = __builtin_fmaf(h2f(s_row[k]), s_x[k], acc);
-            if ((d.d_model & 15) == 8 && lane < 8)
-                acc = __builtin_fmaf(h2f(s_row[n16 + lane]), s_x[n16 + lane], acc);
-        }
-        const float v   = __fadd_rn(acc, __shfl_down(acc, 8, SP_WAVE));
-        const float q   = __fadd_rn(v, __shfl_down(v, 4, SP_WAVE));
-        const float a   = __fadd_rn(q, __shfl_down(q, 1, SP_WAVE));
-        const float sum = __fadd_rn(a, __shfl_down(a, 2, SP_WAVE));
-        const float rv  = __shfl(val, bit, SP_WAVE);
-        if (lane == 0) {
-            const int slot = atomicAdd(&d.sc->n_listed, 1);
-            if (slot < d.list_cap) {
-                d.list_idx[slot]   = (int32_t) cr;
-                d.list_rough[slot] = rv;
-                d.list_exact[slot] = sum;
+    const int per   = d.d_model >> 4;     /* elements per chain */
+    const int pitch = (per + 7) & ~7;
+    float    *s_x   = reinterpret_cast<float *>(smem);                       /* [16][pitch] */
+    uint16_t *s_row = reinterpret_cast<uint16_t *>(smem + (size_t) 16 * pitch * 4) +
+                      (size_t) wv * 16 * pitch;                              /* [16][pitch] */
+    const int n_final = d.sc->n_final;
+    if ((int) blockIdx.x * (SP_TPB / SP_WAVE) >= n_final)
+        return; /* (uniform) */
+    /* the activations are requested first and stored last, so that their latency and the row's
+     * overlap */
+    constexpr int X_PER_THREAD = SPEC_D_MODEL_MAX / SP_TPB;
+    float         xv[X_PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; ++i)
+        xv[i] = i * SP_TPB + tid < d.d_model ? h[i * SP_TPB + tid] : 0.0f;
+    const int slot = (int) blockIdx.x * (SP_TPB / SP_WAVE) + wv;
+    if (slot < n_final) {
+        const uint16_t *src = d.w + (long) d.fin_idx[slot] * d.d_model;
+        for (int o = lane * 8; o < d.d_model; o += SP_WAVE * 8) {
+            const nt_u4 q = __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(src + o));
+            /* elements o .. o+7: chains (o & 15) .. (o & 15) + 7 at position o / 16 */
+            uint16_t *dst = s_row + (o & 15) * pitch + (o >> 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                dst[(2 * i) * pitch]     = (uint16_t) (q[i] & 0xffffu);
+                dst[(2 * i + 1) * pitch] = (uint16_t) (q[i] >> 16);
             }
         }
     }
+#pragma unroll
+    for (int i = 0; i < X_PER_THREAD; ++i) {
+        const int k = i * SP_TPB + tid;
+        if (k < d.d_model)
+            s_x[(k & 15) * pitch + (k >> 4)] = xv[i];
+    }
+    __syncthreads();
+    if (slot >= n_final)
+        return; /* (no workgroup barrier below) */
+    float acc = 0.0f;
+    if (lane < 16) {
+        const uint16_t *wr = s_row + lane * pitch;
+        const float    *xr = s_x + lane * pitch;
+        int             p  = 0;
+        for (; p + 8 <= per; p += 8) {
+            const uint4  q  = *reinterpret_cast<const uint4 *>(wr + p);
+            const float4 xa = *reinterpret_cast<const float4 *>(xr + p);
+            const float4 xb = *reinterpret_cast<const float4 *>(xr + p + 4);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.x & 0xffffu)), xa.x, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.x >> 16)), xa.y, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.y & 0xffffu)), xa.z, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.y >> 16)), xa.w, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.z & 0xffffu)), xb.x, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.z >> 16)), xb.y, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.w & 0xffffu)), xb.z, acc);
+            acc = __builtin_fmaf(h2f((uint16_t) (q.w >> 16)), xb.w, acc);
+        }
+        for (; p < per; ++p)
+            acc = __builtin_fmaf(h2f(wr[p]), xr[p], acc);
+    }
+    const float v   = __fadd_rn(acc, __shfl_down(acc, 8, SP_WAVE));
+    const float q   = __fadd_rn(v, __shfl_down(v, 4, SP_WAVE));
+    const float a   = __fadd_rn(q, __shfl_down(q, 1, SP_WAVE));
+    const float sum = __fadd_rn(a, __shfl_down(a, 2, SP_WAVE));
+    if (lane == 0)
+        d.fin_exact[slot] = sum;
 }
 
-/* The topk best rough scores among the listed rows and the best exact logit among those
- * (spec_head.c:728-770, 802-827), one workgroup. */
-__global__ __launch_bounds__(SP_TPB) void k_spec_final(SpecHeadDev d, SpecResult *__restrict__ res) {
-    __shared__ int      s_hist[256], s_w[4], s_sel[2];
-    __shared__ uint64_t s_best[SP_TPB / SP_WAVE];
-    __shared__ int      s_cnt[SP_TPB / SP_WAVE];
+/* The best exact logit among the finalists, the lowest index among equals (spec_head.c:827),
+ * one workgroup. */
+__global__ __launch_bounds__(SP_SEL_TPB) void k_spec_final(SpecHeadDev d, SpecResult *__restrict__ res) {
+    __shared__ uint64_t s_best[SP_SEL_TPB / SP_WAVE];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int listed = d.sc->n_listed;
-    if (listed > d.list_cap || listed < d.topk) { /* (uniform) more equal scores than the list holds */
+    const int n_final = d.sc->n_final;
+    if (n_final == 0) { /* (uniform) more candidates around the cutoff than the list holds */
         if (tid == 0) {
-            res->token = -1, res->answered = 0, res->n_finalists = 0, res->n_listed = listed;
-            res->cutoff = d.sc->threshold, res->best_exact = 0.0f;
+            res->token = -1, res->answered = 0, res->n_finalists = 0, res->n_listed = d.sc->n_cand;
+            res->cutoff = d.sc->cutoff, res->best_exact = 0.0f;
         }
         return;
     }
-    const float *lr = d.list_rough;
-    int          need_ties;
-    const uint32_t ckey = block_kth_largest([lr](int i) { return ordered_key(lr[i]); }, listed,
-                                            d.topk, s_hist, s_w, s_sel, need_ties);
     uint64_t best = 0;
-    int      cnt  = 0;
-    for (int i = tid; i < listed; i += SP_TPB) {
-        const uint32_t key = ordered_key(lr[i]);
-        bool           in  = key > ckey;
-        if (key == ckey) { /* the lowest indices among the rows that tie at the cutoff */
-            const int32_t me = d.list_idx[i];
-            int           before = 0;
-            for (int j = 0; j < listed; ++j)
-                before += (ordered_key(lr[j]) == ckey && d.list_idx[j] < me) ? 1 : 0;
-            in = before < need_ties;
-        }
-        if (in) {
-            ++cnt;
-            const uint64_t p = ((uint64_t) ordered_key(d.list_exact[i]) << 32) |
-                               (uint32_t) (0x7fffffff - d.list_idx[i]);
-            best = p > best ? p : best;
-        }
+    for (int i = tid; i < n_final; i += SP_SEL_TPB) {
+        const uint64_t p = ((uint64_t) ordered_key(d.fin_exact[i]) << 32) |
+                           (uint32_t) (0x7fffffff - d.fin_idx[i]);
+        best = p > best ? p : best;
     }
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) {
         const uint64_t o = __shfl_xor(best, s, SP_WAVE);
         best             = o > best ? o : best;
-        cnt += __shfl_xor(cnt, s, SP_WAVE);
     }
     if (lane == 0)
-        s_best[wv] = best, s_cnt[wv] = cnt;
+        s_best[wv] = best;
     __syncthreads();
     if (tid == 0) {
-        for (int i = 1; i < SP_TPB / SP_WAVE; ++i) {
+        for (int i = 1; i < SP_SEL_TPB / SP_WAVE; ++i)
             best = s_best[i] > best ? s_best[i] : best;
-            cnt += s_cnt[i];
-        }
         res->token       = 0x7fffffff - (int32_t) (uint32_t) (best & 0xffffffffu);
         res->answered    = 1;
-        res->n_finalists = cnt;
-        res->n_listed    = listed;
-        res->cutoff      = key_to_float(ckey);
+        res->n_finalists = n_final;
+        res->n_listed    = d.sc->n_cand;
+        res->cutoff      = d.sc->cutoff;
         res->best_exact  = key_to_float((uint32_t) (best >> 32));
     }
 }
@@ -393,17 +564,24 @@ void launch_spec_sketch_rows(hipStream_t stream, const SpecHeadDev &d) {
 
 void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, bool verify,
                      SpecResult *result) {
-    const dim3 one(1), block(SP_TPB), rows((unsigned) ((d.vocab + SP_TPB - 1) / SP_TPB));
+    const dim3 one(1), block(SP_TPB), sel(SP_SEL_TPB);
+    const dim3 rows((unsigned) ((d.vocab + SP_TPB - 1) / SP_TPB));
     k_spec_act<<<one, block, 0, stream>>>(d, h);
     GemvFuse f{};
     f.tmax     = d.tmax;
     f.n_chunks = d.n_chunks;
     launch_q8w_gemv(stream, d.sketch, d.row_scale, d.vocab, d.sketch_dim, d.act, d.sketch_dim, 1,
                     d.rough, d.vocab, &f);
-    k_spec_threshold<<<one, block, 0, stream>>>(d);
-    const size_t lds = (size_t) d.d_model * (sizeof(float) + (SP_TPB / SP_WAVE) * sizeof(uint16_t));
-    k_spec_gather<<<rows, block, lds, stream>>>(d, h);
-    k_spec_final<<<one, block, 0, stream>>>(d, result);
+    /* thread maxima: 256 per chunk of 8192 rows; candidates: at most 2 topk */
+    const size_t lds_sel = (size_t) d.list_cap * sizeof(int);
+    if (d.n_chunks * 256 <= 8 * SP_SEL_TPB && d.list_cap <= 2 * SP_SEL_TPB)
+        k_spec_select<8, 2><<<one, sel, lds_sel, stream>>>(d);
+    else
+        k_spec_select<SPEC_TMAX_EPT_MAX, SPEC_LIST_EPT_MAX><<<one, sel, lds_sel, stream>>>(d);
+    const int    pitch = ((d.d_model >> 4) + 7) & ~7;
+    const size_t lds   = (size_t) 16 * pitch * (sizeof(float) + (SP_TPB / SP_WAVE) * sizeof(uint16_t));
+    k_spec_exact<<<dim3((unsigned) ((d.topk + 3) / 4)), block, lds, stream>>>(d, h);
+    k_spec_final<<<one, sel, 0, stream>>>(d, result);
     if (verify)
         k_spec_verify<<<rows, block, 0, stream>>>(d, result);
 }

@@ -17,7 +17,9 @@ struct SpecScalars {
     float h_l1_kept;  /* L1 norm of h over the kept dimensions */
     float h_l2_drop;  /* L2 norm of h over the dropped dimensions */
     float threshold;  /* the topk-th largest thread maximum: every row of the topk best is >= it */
-    int   n_listed;   /* rows >= threshold found so far */
+    float cutoff;     /* the topk-th largest rough score */
+    int   n_cand;     /* rows >= threshold */
+    int   n_final;    /* topk, or 0 when the candidates did not fit the list */
 };
 
 /* What a call answers (mirrors struct geist_hip_spec_result). */
@@ -32,7 +34,8 @@ struct SpecResult {
 
 struct SpecHeadDev {
     long vocab;
-    int  d_model, sketch_dim, topk, n_chunks, list_cap;
+    int  d_model, sketch_dim, topk, n_chunks;
+    int  list_cap; /* 2 topk candidates */
     const uint16_t *w; /* [vocab, d_model] binary16, not owned */
     /* built once */
     int8_t   *sketch;    /* [vocab, sketch_dim] */
@@ -48,9 +51,16 @@ struct SpecHeadDev {
     SpecScalars *sc;
     int32_t     *list_idx;   /* [list_cap] rows >= threshold, any order */
     float       *list_rough; /* [list_cap] */
-    float       *list_exact; /* [list_cap] their exact logits */
+    int32_t     *fin_idx;    /* [topk] the finalists, any order */
+    float       *fin_exact;  /* [topk] their exact logits */
 };
 
+/* The selection kernels hold their keys in registers, 1024 threads: up to 32 thread maxima each
+ * (a vocabulary of 2^20 rows) and up to 8 candidates each (2 x 4096). */
+constexpr int SPEC_TMAX_EPT_MAX = 32;
+constexpr int SPEC_LIST_EPT_MAX = 8;
+constexpr int SPEC_VOCAB_MAX    = SPEC_TMAX_EPT_MAX * 1024 / 256 * 8192;
+constexpr int SPEC_TOPK_MAX     = 4096;
 /* Largest d_model the finalist kernel stages in LDS. */
 constexpr int SPEC_D_MODEL_MAX = 5120;
 /* The rough scores are sums of products of two int8 values (|v| <= 127) formed in binary32:

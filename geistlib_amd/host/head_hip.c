@@ -29,6 +29,10 @@ struct geist_hip_head {
     float    *d_normed; /* m_max x d_model_cap: the normed hidden rows */
     size_t    d_model_cap;
     float    *d_logits; /* m_max x vocab, written by the lm_head, read by the sampler */
+    bool      logits_sparse; /* the last token came from the sketch head: no dense logits */
+    geist_hip_spec_head          *spec;        /* sketch of the tied table, or nullptr */
+    struct geist_hip_spec_result *d_spec_result;
+    size_t                        spec_d_model;
     char      err[256];
 };
 
@@ -101,6 +105,8 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         geist_hip_free(h->hs, h->d_ngram);
         geist_hip_free(h->hs, h->d_normed);
         geist_hip_free(h->hs, h->d_logits);
+        geist_hip_free(h->hs, h->d_spec_result);
+        geist_hip_spec_head_destroy(h->hs, h->spec);
         geist_hip_sampler_destroy(h->hs);
     }
     free(h);
@@ -204,6 +210,7 @@ static int project_finalize(struct geist_hip_head *h, const float *d_hidden, siz
                                                     nullptr, h->d_rng, /*shared=*/1, h->d_tokens);
     if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
+    h->logits_sparse = false;
     if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++)
@@ -231,8 +238,73 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
                             d_model, out_tokens);
 }
 
+int geist_hip_head_spec_build(struct geist_hip_head *h, const uint16_t *d_embed_f16, size_t d_model,
+                              size_t stride_override, size_t topk_override) {
+    if (h == nullptr || d_embed_f16 == nullptr || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    geist_hip_spec_head_destroy(h->hs, h->spec);
+    h->spec = nullptr;
+    void *p = nullptr;
+    if (h->d_spec_result == nullptr) {
+        if (geist_hip_malloc(h->hs, sizeof *h->d_spec_result, &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "sketch head result");
+        h->d_spec_result = p;
+    }
+    /* transformer_spec_head_init, spec_head.c:616-622: a head that is not eligible simply has no
+     * sketch; the caller keeps the dense path */
+    const int rc = geist_hip_spec_head_build(h->hs, d_embed_f16, h->vocab, d_model, stride_override,
+                                             topk_override, &h->spec);
+    if (rc != GEIST_HIP_OK)
+        return head_fail(h, rc, "sketch head");
+    h->spec_d_model = d_model;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_project_finalize_spec(struct geist_hip_head *h, const float *d_hidden,
+                                         const float *d_norm_weight, float rms_eps,
+                                         const uint16_t *d_embed_f16, size_t d_model, int verify,
+                                         int32_t *out_token, int *used_sketch) {
+    if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed_f16 == nullptr ||
+        out_token == nullptr || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (used_sketch != nullptr)
+        *used_sketch = 0;
+    /* spec_head.c:645-647: greedy only; spec_state != 1: no sketch */
+    if (h->spec == nullptr || h->temperature != 0.0f || d_model != h->spec_d_model)
+        return project_finalize(h, d_hidden, d_model, 1, d_norm_weight, rms_eps, d_embed_f16,
+                                nullptr, d_model, out_token);
+    void *p = nullptr;
+    if (h->d_model_cap < d_model) {
+        geist_hip_free(h->hs, h->d_normed);
+        h->d_normed    = nullptr;
+        h->d_model_cap = 0;
+        if (geist_hip_malloc(h->hs, h->m_max * d_model * sizeof(float), &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
+        h->d_normed    = p;
+        h->d_model_cap = d_model;
+    }
+    /* head.c:99-101, then head.c:109 */
+    struct geist_hip_spec_result res;
+    if (geist_hip_rmsnorm_rows(h->hs, d_hidden, d_model, d_norm_weight, rms_eps, 1, d_model,
+                               h->d_normed, d_model) != GEIST_HIP_OK ||
+        geist_hip_spec_head_try(h->hs, h->spec, h->d_normed, verify, h->d_spec_result) !=
+                GEIST_HIP_OK ||
+        geist_hip_download(h->hs, &res, h->d_spec_result, sizeof res) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "sketch head");
+    if (res.answered == 0) /* head.c:114-188: the dense head */
+        return project_finalize(h, d_hidden, d_model, 1, d_norm_weight, rms_eps, d_embed_f16,
+                                nullptr, d_model, out_token);
+    if (res.token < 0 || (size_t) res.token >= h->vocab)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
+    *out_token       = res.token;
+    h->logits_sparse = true; /* spec_head.c:880 */
+    if (used_sketch != nullptr)
+        *used_sketch = 1;
+    return GEIST_HIP_OK;
+}
+
 const float *geist_hip_head_logits(const struct geist_hip_head *h) {
-    return h != nullptr ? h->d_logits : nullptr;
+    return h != nullptr && !h->logits_sparse ? h->d_logits : nullptr;
 }
 
 int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, size_t n,

@@ -14,6 +14,8 @@
  *                                  on the host (head.c:94-188, 224-304)
  *   geist_hip_head_project_finalize_q8w  the same with the int8 table of the x86 backend
  *                                  (src/backends/cpu_x86/backend.c:332-372)
+ *   geist_hip_head_spec_build, geist_hip_head_project_finalize_spec  the speculative int8
+ *                                  sketch head of greedy decoding (forward/spec_head.c)
  *   geist_hip_head_propose_drafts  the n-gram drafter of geist_session_decode_speculative
  *                                  (src/engine/session.c:437-513, 564-572)
  *   geist_hip_head_spec_accept     the accept loop of geist_session_decode_speculative
@@ -90,9 +92,27 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
                                         float rms_eps, const int8_t *d_embed_q8,
                                         const float *d_scales, size_t d_model,
                                         int32_t *out_tokens);
+/* The speculative output head of greedy decoding (src/archs/transformer/forward/spec_head.c;
+ * include/geist_lm_head_hip.h has the device entry points). geist_hip_head_spec_build is
+ * transformer_spec_head_init (spec_head.c:616-622) for a tied F16 table in device memory, which
+ * must stay valid: it returns GEIST_HIP_E_UNSUPPORTED, and the head keeps no sketch, where the
+ * reference or the device kernels build none. geist_hip_head_project_finalize_spec is
+ * finalize_logits_one_row with the sketch in front (head.c:99-112) for one hidden row: output
+ * norm, then the sketch head if the session is greedy and a sketch exists; when it declines
+ * (verify != 0, as GEIST_SPEC_VERIFY=1, and an excluded row could have won) or does not apply,
+ * the dense F16 head of geist_hip_head_project_finalize. *used_sketch (may be NULL) says which
+ * of the two produced the token. */
+int geist_hip_head_spec_build(struct geist_hip_head *h, const uint16_t *d_embed_f16, size_t d_model,
+                              size_t stride_override, size_t topk_override);
+int geist_hip_head_project_finalize_spec(struct geist_hip_head *h, const float *d_hidden,
+                                         const float *d_norm_weight, float rms_eps,
+                                         const uint16_t *d_embed_f16, size_t d_model, int verify,
+                                         int32_t *out_token, int *used_sketch);
 /* The logits of the last geist_hip_head_project_finalize[_q8w] call ([k, vocab], row stride vocab,
  * device memory; soft-cap not applied: the sampler applies it while reading), for scoring with
- * geist_hip_logprob_rows in place of geist_session_peek_logits. NULL before the first call. */
+ * geist_hip_logprob_rows in place of geist_session_peek_logits. NULL before the first call and
+ * after a token that the sketch head produced (there are no dense logits then: the reference
+ * recomputes them on demand, arch.c:179; here the caller runs geist_hip_head_project_finalize). */
 const float *geist_hip_head_logits(const struct geist_hip_head *h);
 
 /* The drafting step of one speculative round (session.c:564-572) for a token history kept in

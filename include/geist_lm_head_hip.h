@@ -111,15 +111,16 @@ int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidde
  * (device memory) receives the token and answered = 1, or answered = 0 when the head declines
  * and the caller has to run the dense head: with verify != 0 (GEIST_SPEC_VERIFY=1) whenever an
  * excluded row's upper bound reaches the winner (spec_head.c:846-872); without it only if more
- * rows tie around the cutoff than the candidate list holds (4 x topk), which the reference's
+ * than 2 x topk rows reach the topk-th largest maximum of groups of 32 scores (rough scores
+ * that tie in their thousands), which the reference's
  * heap would resolve by its insertion order. Greedy only, as in the reference (spec_head.c:645).
  * Calls that overlap on one head race: it owns the buffers of a call. */
 typedef struct geist_hip_spec_head geist_hip_spec_head;
 struct geist_hip_spec_result {
     int32_t token;       /* -1 when not answered without verification */
     int32_t answered;
-    int32_t n_finalists; /* rows scored exactly that belong to the topk best rough scores */
-    int32_t n_listed;    /* rows scored exactly in all */
+    int32_t n_finalists; /* rows scored exactly: the topk best rough scores */
+    int32_t n_listed;    /* candidate rows the finalists were chosen from */
     float   cutoff;      /* the smallest rough score among the finalists */
     float   best_exact;  /* the winner's logit */
 };

@@ -65,6 +65,11 @@ def host():
                                                         C.c_size_t, C.c_void_p, C.c_float,
                                                         C.c_void_p, C.c_void_p, C.c_size_t,
                                                         C.POINTER(C.c_int32)]
+    lib.geist_hip_head_spec_build.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                              C.c_size_t]
+    lib.geist_hip_head_project_finalize_spec.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p,
+                                                         C.c_float, C.c_void_p, C.c_size_t, C.c_int,
+                                                         C.POINTER(C.c_int32), C.POINTER(C.c_int)]
     lib.geist_hip_head_logits.restype = C.c_void_p
     lib.geist_hip_head_logits.argtypes = [C.c_void_p]
     lib.geist_hip_head_spec_accept.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
@@ -442,3 +447,52 @@ def test_head_project_finalize_q8w_is_the_decode_step_of_the_x86_backend(host, o
             h, C.c_void_p(d_hid.data_ptr()), d_model, 1, C.c_void_p(d_nw.data_ptr()), 1e-6,
             C.c_void_p(d_wq.data_ptr()), None, d_model, out) != 0
         host.geist_hip_head_destroy(h)
+
+
+def test_head_project_finalize_spec_follows_head_c(host, oracle):
+    """head.c:99-129 with the sketch head in front: greedy sessions take the sketch's answer
+    (the oracle's token), with the bound on a declined step falls back to the dense head, and a
+    session that samples never uses the sketch."""
+    g = np.random.default_rng(79)
+    vocab, d_model = 66000, 1280
+    w16 = (g.standard_normal((vocab, d_model)) * 0.08).astype(np.float16)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    d_w, d_nw = torch.from_numpy(w16.view(np.int16)).cuda(), torch.from_numpy(norm_w).cuda()
+    sh = oracle.spec_head_build(w16.view(np.uint16))
+    h = make_head(host, vocab, 0, 30.0)
+    assert host.geist_hip_head_spec_build(h, C.c_void_p(d_w.data_ptr()), d_model, 0, 0) == 0, \
+        host.geist_hip_head_errmsg(h)
+    out, used = C.c_int32(), C.c_int()
+    for step in range(4):
+        hidden = (g.standard_normal(d_model) * 2).astype(np.float32)
+        d_hid = torch.from_numpy(hidden).cuda()
+        normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
+        dense = oracle.f16_gemv(w16.view(np.uint16), normed)
+        for verify in (0, 1):
+            rc = host.geist_hip_head_project_finalize_spec(
+                h, C.c_void_p(d_hid.data_ptr()), C.c_void_p(d_nw.data_ptr()), 1e-6,
+                C.c_void_p(d_w.data_ptr()), d_model, verify, C.byref(out), C.byref(used))
+            assert rc == 0, host.geist_hip_head_errmsg(h)
+            want = sh.try_row(normed, verify=bool(verify))
+            assert bool(used.value) == want["certain"]
+            if used.value:
+                assert out.value == want["token"]
+                assert host.geist_hip_head_logits(h) is None
+            else:
+                assert out.value == int(np.flatnonzero(dense == dense.max())[0])
+                assert host.geist_hip_head_logits(h) is not None
+    # a sampling session: the sketch is not consulted (spec_head.c:645)
+    opts = SessionOpts(0, 0.8, 1.0, 40, 5, None, 0, 0)
+    assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+    rc = host.geist_hip_head_project_finalize_spec(
+        h, C.c_void_p(d_hid.data_ptr()), C.c_void_p(d_nw.data_ptr()), 1e-6,
+        C.c_void_p(d_w.data_ptr()), d_model, 0, C.byref(out), C.byref(used))
+    assert rc == 0 and used.value == 0
+    sess = oracle.session(0.8, 1.0, 40, seed=5)
+    assert out.value == oracle.finalize_batch(sess, dense[None, :], softcap=30.0).tolist()[0]
+    # no sketch where the reference builds none: the call reports it and the head stays dense
+    h2 = make_head(host, 9000, 0, 0.0)
+    d_small = torch.zeros((9000, d_model), dtype=torch.float16, device="cuda")
+    assert host.geist_hip_head_spec_build(h2, C.c_void_p(d_small.data_ptr()), d_model, 0, 0) != 0
+    host.geist_hip_head_destroy(h2)
+    host.geist_hip_head_destroy(h)
