@@ -262,6 +262,13 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w,
                 mx = __builtin_fmaxf(mx, __shfl_xor(mx, d, LM_WAVE));
             if (lane == 0 && m < n_m)
                 fuse.tmax[((long) m * fuse.n_chunks + (task >> 8)) * 256 + (task & 255)] = mx;
+        } else if (fuse.gmax != nullptr && m == 0) { /* (uniform) */
+            float mx = row < n_out ? sum : -__builtin_inff();
+#pragma unroll
+            for (int d = 1; d < LM_WAVE; d <<= 1)
+                mx = __builtin_fmaxf(mx, __shfl_xor(mx, d, LM_WAVE));
+            if (lane == 0)
+                fuse.gmax[task] = mx;
         }
     }
 }
@@ -533,7 +540,8 @@ void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, 
         return;
     }
     if (n_m <= 1)
-        k_q8w_gemv<1, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+        k_q8w_gemv<1, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y,
+                                                         fuse ? *fuse : none);
     else if (n_m <= 2)
         k_q8w_gemv<2, false><<<grid, block, 0, stream>>>(wq, scales, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
     else if (n_m <= 4)

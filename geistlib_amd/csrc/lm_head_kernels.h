@@ -26,6 +26,9 @@ void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const fl
 struct GemvFuse {
     float *tmax;
     int    n_chunks;
+    /* Independent of tmax, for one activation row in the plain layout: gmax[g] receives the
+     * maximum of the results of the rows 32 g .. 32 g + 31 (the rows one wavefront computes). */
+    float *gmax;
 };
 bool f16_gemv_can_fuse(int n_m);
 

@@ -11,8 +11,8 @@
  *   k_q8w_gemv        rough[r] = (float)(a . sketch[r]) * row_scale[r]: the int8 projection kernel
  *                     of the dense head. The dot is formed in binary32 there, which is exact for
  *                     sums below 2^24 (sketch_dim <= 1040), so the scores equal the reference's
- *                     integer dot bit for bit. Its epilogue leaves the maxima of groups of 32
- *                     scores (the sampler's thread maxima).
+ *                     integer dot bit for bit. Its epilogue leaves the maximum of every group
+ *                     of 32 consecutive scores (the rows one wavefront computes).
  *   k_spec_select     the topk-th largest of those maxima: at least topk scores reach it, so
  *                     the topk best rows are among the rows >= it (about 1.1 topk rows); it
  *                     reads those groups again and keeps the topk best (the reference's heap)
@@ -258,10 +258,9 @@ __global__ __launch_bounds__(SP_TPB) void k_spec_act(SpecHeadDev d, const float 
 constexpr int SP_SEL_TPB = 1024; /* the two selection kernels: keys live in registers */
 
 /* Phase 2 of the head (spec_head.c:728-770), one workgroup of 1024 threads:
- *   1. the topk-th largest thread maximum: at least topk rough scores reach it, so the topk best
- *      rows are among the rows >= it. Thread maximum i (chunk i / 256, scanning thread t =
- *      i % 256) covers the rows chunk * 8192 + 4 * (j * 256 + t) + c, j < 8, c < 4 (the
- *      sampler's top-k scan layout, which the projection's epilogue writes);
+ *   1. the topk-th largest group maximum (group g = rows 32 g .. 32 g + 31, written by the
+ *      projection's epilogue), to 16 bits: at least topk rough scores reach it, so the topk
+ *      best rows are among the rows >= it;
  *   2. only the groups whose maximum reaches that threshold are read again, their rows >= it
  *      are the candidates (about 1.1 topk, at most 2 topk);
  *   3. the topk-th largest candidate is the reference's cutoff (its heap's smallest entry); the
@@ -274,12 +273,12 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
     int *s_ent = reinterpret_cast<int *>(smem); /* [list_cap] groups to read again */
     __shared__ int s_hist[4][256], s_w[16], s_sel[2], s_n[3];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int n   = d.n_chunks * 256;
+    const int n   = d.n_groups;
     uint32_t  keys[EPT];
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
         const int i = e * SP_SEL_TPB + tid;
-        keys[e]     = i < n ? ordered_key(d.tmax[i]) : 0u;
+        keys[e]     = i < n ? ordered_key(d.gmax[i]) : 0u;
     }
     if (tid < 3)
         s_n[tid] = 0;
@@ -310,12 +309,12 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
     for (int it = tid; it - lane < n_ent; it += SP_SEL_TPB) { /* (whole wavefronts) */
         const bool live = it < n_ent;
         const int  i    = live ? s_ent[it] : 0;
-        const long base = (long) (i >> 8) * 8192 + 4 * (i & 255);
+        const long base = (long) i * 32;
         float      v[32];
         int        c = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const long r0 = base + (long) j * 1024;
+            const long r0 = base + 4 * j;
             if (live && r0 + 3 < d.vocab) { /* (rough is 16-byte aligned, r0 a multiple of 4) */
                 const float4 f = *reinterpret_cast<const float4 *>(d.rough + r0);
                 v[4 * j] = f.x, v[4 * j + 1] = f.y, v[4 * j + 2] = f.z, v[4 * j + 3] = f.w;
@@ -344,7 +343,7 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
         for (int j = 0; j < 32; ++j)
             if (v[j] >= thr) {
                 if (slot < d.list_cap) {
-                    d.list_idx[slot]   = (int32_t) (base + (long) (j >> 2) * 1024 + (j & 3));
+                    d.list_idx[slot]   = (int32_t) (base + j);
                     d.list_rough[slot] = v[j];
                 }
                 ++slot;
@@ -568,14 +567,15 @@ void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, b
     const dim3 rows((unsigned) ((d.vocab + SP_TPB - 1) / SP_TPB));
     k_spec_act<<<one, block, 0, stream>>>(d, h);
     GemvFuse f{};
-    f.tmax     = d.tmax;
-    f.n_chunks = d.n_chunks;
+    f.gmax = d.gmax;
     launch_q8w_gemv(stream, d.sketch, d.row_scale, d.vocab, d.sketch_dim, d.act, d.sketch_dim, 1,
                     d.rough, d.vocab, &f);
-    /* thread maxima: 256 per chunk of 8192 rows; candidates: at most 2 topk */
+    /* group maxima: one per 32 rows; candidates: at most 2 topk */
     const size_t lds_sel = (size_t) d.list_cap * sizeof(int);
-    if (d.n_chunks * 256 <= 8 * SP_SEL_TPB && d.list_cap <= 2 * SP_SEL_TPB)
-        k_spec_select<8, 2><<<one, sel, lds_sel, stream>>>(d);
+    if (d.n_groups <= 4 * SP_SEL_TPB && d.list_cap <= 2 * SP_SEL_TPB)
+        k_spec_select<4, 2><<<one, sel, lds_sel, stream>>>(d);
+    else if (d.n_groups <= 8 * SP_SEL_TPB)
+        k_spec_select<8, SPEC_LIST_EPT_MAX><<<one, sel, lds_sel, stream>>>(d);
     else
         k_spec_select<SPEC_TMAX_EPT_MAX, SPEC_LIST_EPT_MAX><<<one, sel, lds_sel, stream>>>(d);
     const int    pitch = ((d.d_model >> 4) + 7) & ~7;

@@ -16,7 +16,7 @@ struct SpecScalars {
     float inv_xq;     /* max|h| / 127 */
     float h_l1_kept;  /* L1 norm of h over the kept dimensions */
     float h_l2_drop;  /* L2 norm of h over the dropped dimensions */
-    float threshold;  /* the topk-th largest thread maximum: every row of the topk best is >= it */
+    float threshold;  /* a lower bound of the topk-th largest group maximum: the topk best rows are >= it */
     float cutoff;     /* the topk-th largest rough score */
     int   n_cand;     /* rows >= threshold */
     int   n_final;    /* topk, or 0 when the candidates did not fit the list */
@@ -34,7 +34,8 @@ struct SpecResult {
 
 struct SpecHeadDev {
     long vocab;
-    int  d_model, sketch_dim, topk, n_chunks;
+    int  d_model, sketch_dim, topk;
+    int  n_groups; /* ceil(vocab / 32): groups of consecutive rows whose maximum the projection leaves */
     int  list_cap; /* 2 topk candidates */
     const uint16_t *w; /* [vocab, d_model] binary16, not owned */
     /* built once */
@@ -47,7 +48,7 @@ struct SpecHeadDev {
     /* per call */
     float       *act;   /* [sketch_dim] the kept dimensions of the int8 activation, as floats */
     float       *rough; /* [vocab] */
-    float       *tmax;  /* [n_chunks * 256] thread maxima of the rough scores */
+    float       *gmax;  /* [n_groups] maxima of the rough scores of 32 consecutive rows */
     SpecScalars *sc;
     int32_t     *list_idx;   /* [list_cap] rows >= threshold, any order */
     float       *list_rough; /* [list_cap] */
@@ -55,11 +56,11 @@ struct SpecHeadDev {
     float       *fin_exact;  /* [topk] their exact logits */
 };
 
-/* The selection kernels hold their keys in registers, 1024 threads: up to 32 thread maxima each
+/* The selection kernels hold their keys in registers, 1024 threads: up to 32 group maxima each
  * (a vocabulary of 2^20 rows) and up to 8 candidates each (2 x 4096). */
 constexpr int SPEC_TMAX_EPT_MAX = 32;
 constexpr int SPEC_LIST_EPT_MAX = 8;
-constexpr int SPEC_VOCAB_MAX    = SPEC_TMAX_EPT_MAX * 1024 / 256 * 8192;
+constexpr int SPEC_VOCAB_MAX    = SPEC_TMAX_EPT_MAX * 1024 * 32;
 constexpr int SPEC_TOPK_MAX     = 4096;
 /* Largest d_model the finalist kernel stages in LDS. */
 constexpr int SPEC_D_MODEL_MAX = 5120;
