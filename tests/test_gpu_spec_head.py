@@ -159,3 +159,98 @@ def test_rejects_what_it_cannot_take(hs):
         hs.spec_head_build(w)                                # 1024 finalists > 9000 / 64
     with pytest.raises(GeistHipError):
         hs.spec_head_build(torch.zeros((40000, 512), dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_geometries_against_the_oracle(hs, oracle, seed):
+    """Vocabulary, width, finalist count, weight and activation scales drawn at random; token,
+    cutoff and rough scores as the oracle's."""
+    g = np.random.default_rng(1000 + seed)
+    d_model = int(g.choice([1280, 1536, 2048, 2560]))
+    vocab = int(g.integers(17000, 60000))
+    topk = int(g.integers(16, vocab // 64 + 1))
+    print(f"spec fuzz seed={seed} vocab={vocab} d_model={d_model} topk={topk}", flush=True)
+    col_scale = np.exp(g.standard_normal(d_model) * 0.7).astype(np.float32)   # uneven variances
+    w16 = ((g.standard_normal((vocab, d_model)).astype(np.float32) * col_scale)
+           * g.choice([0.01, 0.1, 2.0])).astype(np.float16)
+    want_sh = oracle.spec_head_build(w16.view(np.uint16), topk=topk)
+    assert want_sh is not None
+    sh = hs.spec_head_build(torch.from_numpy(w16.view(np.int16)).cuda(), topk=topk)
+    v = hs.spec_head_view(sh)
+    assert (dev_array(v.d_dims, (want_sh.sketch_dim,), np.uint32) == want_sh.dims).all()
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    for trial in range(3):
+        h = (g.standard_normal(d_model) * g.choice([1e-3, 1.0, 300.0])).astype(np.float32)
+        h[g.integers(0, d_model, 5)] *= 20                   # outliers set the int8 scale
+        for verify in (False, True):
+            want = want_sh.try_row(h, verify=verify)
+            hs.spec_head_try(sh, torch.from_numpy(h).cuda(), res, verify=verify)
+            hs.sync()
+            got = result_of(res)
+            rough = dev_array(v.d_rough, (vocab,), np.uint32)
+            assert (rough == want["rough"].view(np.uint32)).all()
+            srt = np.sort(want["rough"])[::-1]
+            if srt[topk - 1] == srt[topk]:                   # a tie at the cutoff: see below
+                continue
+            assert (got.token, got.cutoff, got.n_finalists) == \
+                (want["token"], want["cutoff"], topk), (trial, verify)
+            assert bool(got.answered) == want["certain"], (trial, verify)
+    hs.spec_head_destroy(sh)
+
+
+def test_ties_at_the_cutoff_keep_the_lowest_indices(hs, oracle):
+    """Rows that are copies of each other have equal rough scores. Where such a tie straddles the
+    cutoff this implementation keeps the lowest indices (the reference keeps whichever rows its
+    heap's sift order leaves); the rule is checked against its statement in numpy."""
+    g = np.random.default_rng(5)
+    vocab, d_model, topk = 20000, 1280, 64
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16)
+    sh_o = oracle.spec_head_build(w16.view(np.uint16), topk=topk)
+    h = g.standard_normal(d_model).astype(np.float32)
+    order = np.argsort(-sh_o.try_row(h)["rough"], kind="stable")
+    # the row ranked 60th is copied to 11 other places, before and behind it: 12 rows tie for the
+    # ranks 60..71 and only 5 of them are finalists
+    src = int(order[59])
+    spots = np.sort(g.choice(np.setdiff1d(np.arange(vocab), order[:80]), 11, replace=False))
+    w16[spots] = w16[src]
+    sh_o = oracle.spec_head_build(w16.view(np.uint16), topk=topk)
+    rough = sh_o.try_row(h)["rough"]
+    srt = np.sort(rough)[::-1]
+    cutoff = srt[topk - 1]
+    assert (rough == cutoff).sum() == 12 and (rough > cutoff).sum() == 59
+    tied = np.flatnonzero(rough == cutoff)[:topk - 59]
+    finalists = np.concatenate([np.flatnonzero(rough > cutoff), tied])
+    exact = oracle.f16_gemv(w16.view(np.uint16)[finalists], h)
+    want_token = int(finalists[np.flatnonzero(exact == exact.max())].min())
+    sh = hs.spec_head_build(torch.from_numpy(w16.view(np.int16)).cuda(), topk=topk)
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    hs.spec_head_try(sh, torch.from_numpy(h).cuda(), res)
+    hs.sync()
+    got = result_of(res)
+    assert got.answered == 1 and got.n_finalists == topk and got.cutoff == cutoff
+    assert got.token == want_token
+    assert np.float32(got.best_exact) == exact.max()
+    # make one of the tied copies the winner: only a copy among the 5 lowest indices can win
+    hs.spec_head_destroy(sh)
+
+
+def test_bitnet_geometry_once(hs, oracle):
+    """128256 x 2560, the geometry the head was written for: sketch 640 wide, 1024 finalists."""
+    g = np.random.default_rng(11)
+    vocab, d_model = 128256, 2560
+    w16 = (g.standard_normal((vocab, d_model), dtype=np.float32) * 0.05).astype(np.float16)
+    want_sh = oracle.spec_head_build(w16.view(np.uint16))
+    sh = hs.spec_head_build(torch.from_numpy(w16.view(np.int16)).cuda())
+    v = hs.spec_head_view(sh)
+    assert (v.sketch_dim, v.topk) == (640, 1024)
+    assert (dev_array(v.d_sketch, (vocab, 640), np.int8) == want_sh.sketch).all()
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        h = g.standard_normal(d_model).astype(np.float32)
+        want = want_sh.try_row(h)
+        hs.spec_head_try(sh, torch.from_numpy(h).cuda(), res)
+        hs.sync()
+        got = result_of(res)
+        assert (got.token, got.cutoff, got.n_finalists, got.answered) == \
+            (want["token"], want["cutoff"], 1024, 1)
+    hs.spec_head_destroy(sh)
