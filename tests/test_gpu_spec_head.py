@@ -254,3 +254,29 @@ def test_bitnet_geometry_once(hs, oracle):
         assert (got.token, got.cutoff, got.n_finalists, got.answered) == \
             (want["token"], want["cutoff"], 1024, 1)
     hs.spec_head_destroy(sh)
+
+
+@pytest.mark.parametrize("vocab,d_model", [(262144, 1536), (300000, 1280)])
+def test_large_vocabularies_take_the_wider_selection_kernels(hs, oracle, vocab, d_model):
+    """From 200000 tokens on the reference keeps 4096 finalists (Gemma's 262144 x 1536 head):
+    more group maxima and candidates per thread of the selection workgroup."""
+    print(f"spec large vocab={vocab} d_model={d_model}", flush=True)
+    g = np.random.default_rng(vocab)
+    w16 = (g.standard_normal((vocab, d_model), dtype=np.float32) * 0.05).astype(np.float16)
+    want_sh = oracle.spec_head_build(w16.view(np.uint16))
+    assert want_sh.topk == 4096
+    sh = hs.spec_head_build(torch.from_numpy(w16.view(np.int16)).cuda())
+    v = hs.spec_head_view(sh)
+    assert (v.sketch_dim, v.topk) == (want_sh.sketch_dim, 4096)
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    for verify in (False, True):
+        h = g.standard_normal(d_model).astype(np.float32)
+        want = want_sh.try_row(h, verify=verify)
+        hs.spec_head_try(sh, torch.from_numpy(h).cuda(), res, verify=verify)
+        hs.sync()
+        got = result_of(res)
+        rough = dev_array(v.d_rough, (vocab,), np.uint32)
+        assert (rough == want["rough"].view(np.uint32)).all()
+        assert (got.token, got.cutoff, got.n_finalists) == (want["token"], want["cutoff"], 4096)
+        assert bool(got.answered) == want["certain"]
+    hs.spec_head_destroy(sh)
