@@ -310,8 +310,7 @@ def bench_lm_head_spec(args):
     res = torch.zeros(6, dtype=torch.int32, device=dev)
 
     def step(i=0):
-        hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-        hs.spec_head_try(heads[i % len(heads)], normed, res)
+        hs.spec_head_try_hidden(heads[i % len(heads)], hidden, norm_w, 1e-6, normed, res)
 
     for i in range(args.warmup):
         step(i)

@@ -120,6 +120,7 @@ def load_library():
     lib.geist_hip_spec_head_destroy.restype = None
     lib.geist_hip_spec_head_view.argtypes = [vp, C.POINTER(SpecHeadView)]
     lib.geist_hip_spec_head_try.argtypes = [vp, vp, vp, i32, vp]
+    lib.geist_hip_spec_head_try_hidden.argtypes = [vp, vp, vp, vp, f32, vp, i32, vp]
     _LIB = lib
     return lib
 
@@ -315,6 +316,11 @@ class HipSampler:
         """result: a device buffer of 24 bytes that receives struct geist_hip_spec_result."""
         self._check(self.lib.geist_hip_spec_head_try(self.h, sh, _ptr(hidden_normed), int(verify),
                                                      _ptr(result)))
+
+    def spec_head_try_hidden(self, sh, hidden, norm_w, eps, normed, result, verify=False):
+        """spec_head_try with the output norm in front; normed receives the normed row."""
+        self._check(self.lib.geist_hip_spec_head_try_hidden(
+            self.h, sh, _ptr(hidden), _ptr(norm_w), eps, _ptr(normed), int(verify), _ptr(result)))
 
     def time_q8w_gemv(self, weight_copies, scale_copies, x, y, launches):
         """As time_f16_gemv for q8w_gemv."""

@@ -23,6 +23,7 @@
  * (8 per row and lane) share each converted weight.
  */
 #include "lm_head_kernels.h"
+#include "rmsnorm_device.h"
 
 #include <hip/hip_fp16.h>
 
@@ -105,24 +106,6 @@ __device__ __forceinline__ void stage_load_x(const float *__restrict__ x, long l
             gx.x[m][q]   = col < n_in ? x[mm * ld_x + col] : 0.0f;
         }
     }
-}
-
-/* 1 / sqrt(mean(x^2) + eps) as cpu_scalar_rmsnorm rounds it (elementwise.c:270-274). The
- * reference adds the squares in double in index order; the order of a double sum only shows in
- * the binary32 result when the value lies within the sums' error of the middle between two
- * binary32 values, and then `sequential` repeats the sum in the reference's order. */
-__device__ __forceinline__ bool rms_inv_is_safe(double sumsq, int n, float eps, float &f) {
-    const double r  = 1.0 / sqrt(sumsq / (double) n + (double) eps);
-    f               = (float) r;
-    const float  fn = r > (double) f ? nextafterf(f, __builtin_inff()) : nextafterf(f, -__builtin_inff());
-    const double mid = 0.5 * ((double) f + (double) fn);
-    return !(fabs(r - mid) <= fabs(r) * (double) n * 0x1p-50);
-}
-__device__ __forceinline__ float rms_inv_sequential(const float *__restrict__ xr, int n, float eps) {
-    double sumsq = 0.0;
-    for (int i = 0; i < n; ++i)
-        sumsq += (double) xr[i] * (double) xr[i];
-    return (float) (1.0 / sqrt(sumsq / (double) n + (double) eps));
 }
 
 /* One step of the chains: eight weights of this lane's row and half against the activations of
@@ -432,24 +415,7 @@ __global__ __launch_bounds__(LM_TPB) void k_rmsnorm_rows(const float *__restrict
     const int    tid = threadIdx.x;
     const float *xr  = x + (long) blockIdx.x * ld_x;
     float       *yr  = y + (long) blockIdx.x * ld_y;
-    double       a   = 0.0;
-    for (int i = tid; i < n; i += LM_TPB)
-        a += (double) xr[i] * (double) xr[i];
-    s_part[tid] = a;
-    __syncthreads();
-    for (int step = LM_TPB / 2; step > 0; step >>= 1) {
-        if (tid < step)
-            s_part[tid] += s_part[tid + step];
-        __syncthreads();
-    }
-    if (tid == 0) {
-        float f;
-        if (!rms_inv_is_safe(s_part[0], n, eps, f))
-            f = rms_inv_sequential(xr, n, eps);
-        s_inv = f;
-    }
-    __syncthreads();
-    const float inv = s_inv;
+    const float inv = block_rms_inv<LM_TPB>(xr, n, eps, s_part, &s_inv);
     for (int i = tid; i < n; i += LM_TPB)
         yr[i] = __fmul_rn(__fmul_rn(xr[i], inv), w[i]);
 }

@@ -1125,6 +1125,25 @@ int geist_hip_spec_head_try(geist_hip_sampler *s, geist_hip_spec_head *sh,
     return after_launch(s, "sketch head");
 }
 
+int geist_hip_spec_head_try_hidden(geist_hip_sampler *s, geist_hip_spec_head *sh,
+                                   const float *d_hidden, const float *d_norm_weight,
+                                   float rms_eps, float *d_normed, int verify,
+                                   struct geist_hip_spec_result *d_result) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!sh || !d_hidden || !d_norm_weight || !d_normed || !d_result)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (sh->device != s->device)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sketch head built on another device");
+    if (((uintptr_t) d_normed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sketch head: normed row not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    gs::launch_spec_try(s->stream, sh->d, d_hidden, verify != 0,
+                        reinterpret_cast<gs::SpecResult *>(d_result), d_norm_weight, rms_eps,
+                        d_normed);
+    return after_launch(s, "sketch head");
+}
+
 int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,
                                  const float *const *d_scales, size_t n_weights, size_t n_out,
                                  size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,

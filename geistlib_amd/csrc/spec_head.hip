@@ -31,6 +31,7 @@
 #include "spec_head_kernels.h"
 
 #include "lm_head_kernels.h"
+#include "rmsnorm_device.h"
 
 #include <hip/hip_fp16.h>
 
@@ -209,11 +210,30 @@ __global__ __launch_bounds__(SP_TPB) void k_spec_sketch_rows(SpecHeadDev d) {
 
 /* ---- per token --------------------------------------------------------------------------- */
 
-/* spec_head.c:672-694 and 712-724, one workgroup. */
-__global__ __launch_bounds__(SP_TPB) void k_spec_act(SpecHeadDev d, const float *__restrict__ h) {
+/* spec_head.c:672-694 and 712-724, one workgroup. With NORM the output norm of head.c:99-101
+ * runs in front: h = (x * inv_rms) * norm_w, written to h_out for the finalist kernel, in the
+ * arithmetic of the norm kernel of the dense head. */
+template <bool NORM>
+__global__ __launch_bounds__(SP_TPB) void k_spec_act(SpecHeadDev d, const float *__restrict__ h_in,
+                                                     const float *__restrict__ norm_w, float eps,
+                                                     float *__restrict__ h_out) {
     __shared__ float  s_max[SP_TPB / SP_WAVE];
     __shared__ double s_sum[3][SP_TPB / SP_WAVE];
+    __shared__ double s_part[NORM ? SP_TPB : 1];
+    __shared__ float  s_inv;
+    __shared__ float  s_h[NORM ? SPEC_D_MODEL_MAX : 1];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const float *h = h_in;
+    if (NORM) {
+        const float inv = block_rms_inv<SP_TPB>(h_in, d.d_model, eps, s_part, &s_inv);
+        for (int i = tid; i < d.d_model; i += SP_TPB) {
+            const float y = __fmul_rn(__fmul_rn(h_in[i], inv), norm_w[i]);
+            s_h[i]        = y;
+            h_out[i]      = y;
+        }
+        __syncthreads();
+        h = s_h;
+    }
     float     amax = 0.0f;
     double    all2 = 0.0;
     for (int i = tid; i < d.d_model; i += SP_TPB) {
@@ -562,10 +582,15 @@ void launch_spec_sketch_rows(hipStream_t stream, const SpecHeadDev &d) {
 }
 
 void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, bool verify,
-                     SpecResult *result) {
+                     SpecResult *result, const float *norm_w, float eps, float *h_normed) {
     const dim3 one(1), block(SP_TPB), sel(SP_SEL_TPB);
     const dim3 rows((unsigned) ((d.vocab + SP_TPB - 1) / SP_TPB));
-    k_spec_act<<<one, block, 0, stream>>>(d, h);
+    if (norm_w != nullptr) {
+        k_spec_act<true><<<one, block, 0, stream>>>(d, h, norm_w, eps, h_normed);
+        h = h_normed;
+    } else {
+        k_spec_act<false><<<one, block, 0, stream>>>(d, h, nullptr, 0.0f, nullptr);
+    }
     GemvFuse f{};
     f.gmax = d.gmax;
     launch_q8w_gemv(stream, d.sketch, d.row_scale, d.vocab, d.sketch_dim, d.act, d.sketch_dim, 1,

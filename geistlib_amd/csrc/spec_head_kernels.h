@@ -74,9 +74,12 @@ void launch_spec_dim_stats(hipStream_t stream, const uint16_t *w, long vocab, in
                            long vstep, float *dvar);
 /* sketch, row_scale, w_drop, w_l1 from w, dims and kept (spec_head.c:563-603). */
 void launch_spec_sketch_rows(hipStream_t stream, const SpecHeadDev &d);
-/* transformer_spec_head_try for one normed hidden row h [d_model] (spec_head.c:624-889). */
+/* transformer_spec_head_try for one normed hidden row h [d_model] (spec_head.c:624-889). With
+ * norm_w != NULL, h is the hidden row before the output norm: the norm (weights norm_w, eps) runs
+ * in the first kernel and h_normed [d_model] receives the normed row. */
 void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, bool verify,
-                     SpecResult *result);
+                     SpecResult *result, const float *norm_w = nullptr, float eps = 0.0f,
+                     float *h_normed = nullptr);
 
 } // namespace gs
 #endif

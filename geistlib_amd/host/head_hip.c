@@ -285,10 +285,8 @@ int geist_hip_head_project_finalize_spec(struct geist_hip_head *h, const float *
     }
     /* head.c:99-101, then head.c:109 */
     struct geist_hip_spec_result res;
-    if (geist_hip_rmsnorm_rows(h->hs, d_hidden, d_model, d_norm_weight, rms_eps, 1, d_model,
-                               h->d_normed, d_model) != GEIST_HIP_OK ||
-        geist_hip_spec_head_try(h->hs, h->spec, h->d_normed, verify, h->d_spec_result) !=
-                GEIST_HIP_OK ||
+    if (geist_hip_spec_head_try_hidden(h->hs, h->spec, d_hidden, d_norm_weight, rms_eps,
+                                       h->d_normed, verify, h->d_spec_result) != GEIST_HIP_OK ||
         geist_hip_download(h->hs, &res, h->d_spec_result, sizeof res) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "sketch head");
     if (res.answered == 0) /* head.c:114-188: the dense head */

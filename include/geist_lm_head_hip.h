@@ -145,6 +145,15 @@ int  geist_hip_spec_head_try(geist_hip_sampler *s, geist_hip_spec_head *sh,
                              const float *d_hidden_normed, int verify,
                              struct geist_hip_spec_result *d_result);
 
+/* geist_hip_spec_head_try with the output norm of head.c:99-101 in front, in the same launch as
+ * the activation's quantisation: d_hidden is the row before the norm, d_normed [d_model]
+ * receives geist_hip_rmsnorm_rows' result for it (bit for bit) and is what the finalists are
+ * scored against. */
+int geist_hip_spec_head_try_hidden(geist_hip_sampler *s, geist_hip_spec_head *sh,
+                                   const float *d_hidden, const float *d_norm_weight,
+                                   float rms_eps, float *d_normed, int verify,
+                                   struct geist_hip_spec_result *d_result);
+
 /* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
  * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
  * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */

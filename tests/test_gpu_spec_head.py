@@ -280,3 +280,27 @@ def test_large_vocabularies_take_the_wider_selection_kernels(hs, oracle, vocab, 
         assert (got.token, got.cutoff, got.n_finalists) == (want["token"], want["cutoff"], 4096)
         assert bool(got.answered) == want["certain"]
     hs.spec_head_destroy(sh)
+
+
+def test_try_hidden_norms_in_the_same_launch(hs, oracle):
+    """geist_hip_spec_head_try_hidden: the normed row equals geist_hip_rmsnorm_rows' bit for bit,
+    and the answer is that of geist_hip_spec_head_try on it."""
+    g = np.random.default_rng(21)
+    vocab, d_model = 40000, 2560
+    w16 = table(g, vocab, d_model)
+    sh = hs.spec_head_build(torch.from_numpy(w16.view(np.int16)).cuda(), topk=512)
+    want_sh = oracle.spec_head_build(w16.view(np.uint16), topk=512)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    d_nw = torch.from_numpy(norm_w).cuda()
+    res = torch.zeros(6, dtype=torch.int32, device="cuda")
+    for scale in (1e-3, 2.0, 1e4):
+        hidden = (g.standard_normal(d_model) * scale).astype(np.float32)
+        normed = torch.full((d_model,), 7.0, dtype=torch.float32, device="cuda")
+        hs.spec_head_try_hidden(sh, torch.from_numpy(hidden).cuda(), d_nw, 1e-6, normed, res)
+        hs.sync()
+        got = result_of(res)
+        want_normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
+        assert (normed.cpu().numpy().view(np.uint32) == want_normed.view(np.uint32)).all()
+        want = want_sh.try_row(want_normed)
+        assert (got.token, got.cutoff, got.answered) == (want["token"], want["cutoff"], 1)
+    hs.spec_head_destroy(sh)
