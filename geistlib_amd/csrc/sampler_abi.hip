@@ -1009,7 +1009,7 @@ void geist_hip_spec_head_destroy(geist_hip_sampler *s, geist_hip_spec_head *sh) 
     (void) hipSetDevice(sh->device);
     gs::SpecHeadDev &d = sh->d;
     void *ptrs[] = {d.sketch, d.row_scale, d.w_drop, d.w_l1, d.dims, d.kept, d.act, d.rough,
-                    d.gmax, d.sc, d.list_idx, d.list_rough, d.fin_idx, d.fin_exact};
+                    d.gmax, d.sc, d.fin_idx, d.fin_exact};
     for (void *p : ptrs)
         if (p)
             (void) hipFree(p);
@@ -1046,10 +1046,8 @@ int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16,
     };
     bool ok = alloc(d.sketch, n_vocab * sd) && alloc(d.row_scale, n_vocab * 4) &&
               alloc(d.w_drop, n_vocab * 4) && alloc(d.w_l1, n_vocab * 4) && alloc(d.dims, sd * 4) &&
-              alloc(d.kept, d_model) && alloc(d.act, sd * 4) && alloc(d.rough, n_vocab * 4) &&
+              alloc(d.kept, d_model) && alloc(d.act, sd * 4) && alloc(d.rough, (size_t) ((n_vocab + 31) / 32) * 32 * 4) &&
               alloc(d.gmax, (size_t) d.n_groups * 4) && alloc(d.sc, sizeof(gs::SpecScalars)) &&
-              alloc(d.list_idx, (size_t) d.list_cap * 4) &&
-              alloc(d.list_rough, (size_t) d.list_cap * 4) &&
               alloc(d.fin_idx, topk * 4) && alloc(d.fin_exact, topk * 4) &&
               alloc(d_var, d_model * 4);
     int err = ok ? 0 : GEIST_HIP_E_OOM;

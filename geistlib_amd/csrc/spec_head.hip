@@ -287,10 +287,12 @@ constexpr int SP_SEL_TPB = 1024; /* the two selection kernels: keys live in regi
  *      finalists are the candidates above it and, of those equal to it, as many as complete
  *      topk rows -- the lowest indices first.
  * Thread t holds the maxima e * 1024 + t and later the candidates e * 1024 + t. */
-template <int EPT, int EPT2>
+template <int EPT, int EPT2, int IT>
 __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
     extern __shared__ __align__(16) uint8_t smem[];
-    int *s_ent = reinterpret_cast<int *>(smem); /* [list_cap] groups to read again */
+    int      *s_ent = reinterpret_cast<int *>(smem); /* [list_cap] groups to read again */
+    int32_t  *s_ci  = s_ent + d.list_cap;             /* [list_cap] candidate rows */
+    uint32_t *s_ck  = reinterpret_cast<uint32_t *>(s_ci + d.list_cap); /* ... and their keys */
     __shared__ int s_hist[4][256], s_w[16], s_sel[2], s_n[3];
     const int tid = threadIdx.x, lane = tid & 63;
     const int n   = d.n_groups;
@@ -325,51 +327,57 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
     }
     __syncthreads();
     const int n_ent = s_n[0] < d.list_cap ? s_n[0] : d.list_cap;
-    /* 2b. their rows that reach it */
-    for (int it = tid; it - lane < n_ent; it += SP_SEL_TPB) { /* (whole wavefronts) */
-        const bool live = it < n_ent;
-        const int  i    = live ? s_ent[it] : 0;
-        const long base = (long) i * 32;
-        float      v[32];
-        int        c = 0;
+    /* 2b. their rows that reach it, into the candidate list in LDS: IT groups per thread and
+     * round with all their loads in flight together. A wavefront counts its hits with one ballot
+     * per row position, takes its slots with one atomic and hands them out by ballot again
+     * (candidates are stored in no particular order). */
+    for (int round = 0; round < n_ent; round += IT * SP_SEL_TPB) { /* (uniform) */
+        float v[IT][32];
+        long  base[IT];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const long r0 = base + 4 * j;
-            if (live && r0 + 3 < d.vocab) { /* (rough is 16-byte aligned, r0 a multiple of 4) */
-                const float4 f = *reinterpret_cast<const float4 *>(d.rough + r0);
-                v[4 * j] = f.x, v[4 * j + 1] = f.y, v[4 * j + 2] = f.z, v[4 * j + 3] = f.w;
-            } else {
+        for (int u = 0; u < IT; ++u) {
+            const int  it   = round + u * SP_SEL_TPB + tid;
+            const bool live = it < n_ent;
+            const int  i    = live ? s_ent[it] : 0;
+            base[u]         = (long) i * 32;
+            /* (no branch around a load, so that all of them are in flight together: rough is
+             * allocated in whole groups, rows beyond the vocabulary are masked afterwards) */
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    v[4 * j + q] = (live && r0 + q < d.vocab) ? d.rough[r0 + q] : -__builtin_inff();
+            for (int j = 0; j < 8; ++j) {
+                const long   r0 = base[u] + 4 * j;
+                const float4 f  = *reinterpret_cast<const float4 *>(d.rough + r0);
+                v[u][4 * j]     = live && r0 + 0 < d.vocab ? f.x : -__builtin_inff();
+                v[u][4 * j + 1] = live && r0 + 1 < d.vocab ? f.y : -__builtin_inff();
+                v[u][4 * j + 2] = live && r0 + 2 < d.vocab ? f.z : -__builtin_inff();
+                v[u][4 * j + 3] = live && r0 + 3 < d.vocab ? f.w : -__builtin_inff();
             }
         }
 #pragma unroll
-        for (int j = 0; j < 32; ++j)
-            c += v[j] >= thr ? 1 : 0;
-        int incl = c;
+        for (int u = 0; u < IT; ++u) {
+            if (round + u * SP_SEL_TPB + tid - lane >= n_ent)
+                continue; /* (whole wavefronts) */
+            int total = 0;
 #pragma unroll
-        for (int sft = 1; sft < SP_WAVE; sft <<= 1) {
-            const int y = __shfl_up(incl, sft, SP_WAVE);
-            if (lane >= sft)
-                incl += y;
-        }
-        int wbase = 0;
-        if (lane == 63)
-            wbase = atomicAdd(&s_n[1], incl);
-        wbase    = __shfl(wbase, 63, SP_WAVE);
-        int slot = wbase + incl - c;
+            for (int j = 0; j < 32; ++j)
+                total += __builtin_popcountll(__ballot(v[u][j] >= thr));
+            int wbase = 0;
+            if (lane == 0)
+                wbase = atomicAdd(&s_n[1], total);
+            wbase = __builtin_amdgcn_readfirstlane(wbase);
 #pragma unroll
-        for (int j = 0; j < 32; ++j)
-            if (v[j] >= thr) {
-                if (slot < d.list_cap) {
-                    d.list_idx[slot]   = (int32_t) (base + j);
-                    d.list_rough[slot] = v[j];
+            for (int j = 0; j < 32; ++j) {
+                const bool               hit = v[u][j] >= thr;
+                const unsigned long long m   = __ballot(hit);
+                const int slot = wbase + __builtin_popcountll(m & ((1ull << lane) - 1ull));
+                if (hit && slot < d.list_cap) {
+                    s_ci[slot] = (int32_t) (base[u] + j);
+                    s_ck[slot] = ordered_key(v[u][j]);
                 }
-                ++slot;
+                wbase += __builtin_popcountll(m);
             }
+        }
     }
-    __syncthreads(); /* (the candidates written above are visible to the whole workgroup) */
+    __syncthreads();
     const int n_cand = s_n[1];
     if (s_n[0] > d.list_cap || n_cand > d.list_cap || n_cand < d.topk) { /* (uniform) */
         if (tid == 0) {
@@ -383,8 +391,8 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
 #pragma unroll
     for (int e = 0; e < EPT2; ++e) {
         const int i = e * SP_SEL_TPB + tid;
-        ck[e]       = i < n_cand ? ordered_key(d.list_rough[i]) : 0u;
-        ci[e]       = i < n_cand ? d.list_idx[i] : -1;
+        ck[e]       = i < n_cand ? s_ck[i] : 0u;
+        ci[e]       = i < n_cand ? s_ci[i] : -1;
     }
     int            need_ties;
     const uint32_t ckey = block_kth_largest<EPT2>(ck, n_cand, d.topk, s_hist, s_sel, need_ties);
@@ -409,7 +417,7 @@ __global__ __launch_bounds__(SP_SEL_TPB) void k_spec_select(SpecHeadDev d) {
             if (tie_cnt > need_ties) { /* the lowest indices among the rows that tie */
                 int before = 0;
                 for (int j = 0; j < n_cand; ++j)
-                    before += (d.list_idx[j] < ci[e] && ordered_key(d.list_rough[j]) == ckey) ? 1 : 0;
+                    before += (s_ci[j] < ci[e] && s_ck[j] == ckey) ? 1 : 0;
                 in = before < need_ties;
             }
         }
@@ -596,13 +604,23 @@ void launch_spec_try(hipStream_t stream, const SpecHeadDev &d, const float *h, b
     launch_q8w_gemv(stream, d.sketch, d.row_scale, d.vocab, d.sketch_dim, d.act, d.sketch_dim, 1,
                     d.rough, d.vocab, &f);
     /* group maxima: one per 32 rows; candidates: at most 2 topk */
-    const size_t lds_sel = (size_t) d.list_cap * sizeof(int);
-    if (d.n_groups <= 4 * SP_SEL_TPB && d.list_cap <= 2 * SP_SEL_TPB)
-        k_spec_select<4, 2><<<one, sel, lds_sel, stream>>>(d);
-    else if (d.n_groups <= 8 * SP_SEL_TPB)
-        k_spec_select<8, SPEC_LIST_EPT_MAX><<<one, sel, lds_sel, stream>>>(d);
-    else
-        k_spec_select<SPEC_TMAX_EPT_MAX, SPEC_LIST_EPT_MAX><<<one, sel, lds_sel, stream>>>(d);
+    const size_t lds_sel = (size_t) d.list_cap * 3 * sizeof(int);
+    if (d.n_groups <= 4 * SP_SEL_TPB && d.list_cap <= 2 * SP_SEL_TPB) {
+        k_spec_select<4, 2, 2><<<one, sel, lds_sel, stream>>>(d);
+    } else { /* up to 96 KB of LDS, above what a launch may take by default */
+        if (d.n_groups <= 8 * SP_SEL_TPB) {
+            (void) hipFuncSetAttribute(
+                reinterpret_cast<const void *>(k_spec_select<8, SPEC_LIST_EPT_MAX, 1>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_sel);
+            k_spec_select<8, SPEC_LIST_EPT_MAX, 1><<<one, sel, lds_sel, stream>>>(d);
+        } else {
+            (void) hipFuncSetAttribute(
+                reinterpret_cast<const void *>(
+                    k_spec_select<SPEC_TMAX_EPT_MAX, SPEC_LIST_EPT_MAX, 1>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_sel);
+            k_spec_select<SPEC_TMAX_EPT_MAX, SPEC_LIST_EPT_MAX, 1><<<one, sel, lds_sel, stream>>>(d);
+        }
+    }
     const int    pitch = ((d.d_model >> 4) + 7) & ~7;
     const size_t lds   = (size_t) 16 * pitch * (sizeof(float) + (SP_TPB / SP_WAVE) * sizeof(uint16_t));
     k_spec_exact<<<dim3((unsigned) ((d.topk + 3) / 4)), block, lds, stream>>>(d, h);

@@ -47,11 +47,9 @@ struct SpecHeadDev {
     uint8_t  *kept;      /* [d_model] 1 where the sketch keeps the dimension */
     /* per call */
     float       *act;   /* [sketch_dim] the kept dimensions of the int8 activation, as floats */
-    float       *rough; /* [vocab] */
+    float       *rough; /* [vocab], allocated up to a multiple of 32 */
     float       *gmax;  /* [n_groups] maxima of the rough scores of 32 consecutive rows */
     SpecScalars *sc;
-    int32_t     *list_idx;   /* [list_cap] rows >= threshold, any order */
-    float       *list_rough; /* [list_cap] */
     int32_t     *fin_idx;    /* [topk] the finalists, any order */
     float       *fin_exact;  /* [topk] their exact logits */
 };
