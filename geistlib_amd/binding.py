@@ -103,6 +103,7 @@ def load_library():
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
     lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_f16_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_f16_to_q8w.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
@@ -249,6 +250,15 @@ class HipSampler:
         m = x.shape[0]
         assert w_f16.is_contiguous() and w_f16.element_size() == 2 and x.shape[1] == n_in
         self._check(self.lib.geist_hip_f16_gemv_rows(
+            self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def f16_linear(self, w_f16, x, y):
+        """As f16_gemv in the portable kernel's arithmetic: the sum in double, rounded once."""
+        n_out, n_in = w_f16.shape
+        m = x.shape[0]
+        assert w_f16.is_contiguous() and w_f16.element_size() == 2 and x.shape[1] == n_in
+        self._check(self.lib.geist_hip_f16_linear_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 

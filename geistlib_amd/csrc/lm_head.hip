@@ -403,6 +403,150 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv_batched(const uint16_t *__r
     }
 }
 
+/* ---- the portable kernel's arithmetic: double accumulation -------------------------------- *
+ * cpu_scalar_w_quant_m1 / _mN for F16 weights (src/backends/cpu_scalar/weight_resolve.c:186-241),
+ * which the x86 backend also runs whenever more than one activation row is projected:
+ *   y[i][j] = (float) sum_k (double) x[i][k] * (double) f16(W[j][k])   (double, index order).
+ * Every product is exact in double (24 + 11 significant bits), so only the order of the
+ * additions could differ from the reference, and that shows in the binary32 result only when
+ * the sum lies within the additions' error of a binary32 rounding boundary. A lane owns a
+ * weight row and adds in its own order (two partial sums per activation row); an output that
+ * close to a boundary -- about two in a thousand -- is added once more in index order by the
+ * same lane. The error bound uses |sum_k x_k w_k| terms <= ||x||_2 ||w||_2 (the row's norm is
+ * accumulated on the way in binary32, the activations' norm comes with their double copy). */
+
+/* xd[m][k] = (double) x[m][k], xn[m] = ||x[m]||_2 (rounded up a little). One workgroup per row. */
+__global__ __launch_bounds__(LM_TPB) void k_x_to_f64(const float *__restrict__ x, long ld_x,
+                                                     int n_in, double *__restrict__ xd,
+                                                     double *__restrict__ xn) {
+    __shared__ double s_part[LM_TPB];
+    const int    tid = threadIdx.x;
+    const float *xr  = x + (long) blockIdx.x * ld_x;
+    double       a   = 0.0;
+    for (int k = tid; k < n_in; k += LM_TPB) {
+        const double v = (double) xr[k];
+        xd[(long) blockIdx.x * n_in + k] = v;
+        a += v * v;
+    }
+    s_part[tid] = a;
+    __syncthreads();
+    for (int step = LM_TPB / 2; step > 0; step >>= 1) {
+        if (tid < step)
+            s_part[tid] += s_part[tid + step];
+        __syncthreads();
+    }
+    if (tid == 0)
+        xn[blockIdx.x] = sqrt(s_part[0]) * (1.0 + 0x1p-40);
+}
+
+/* (float) s, and whether every value within err of s rounds to the same binary32. */
+__device__ __forceinline__ bool f32_rounding_is_safe(double s, double err, float &f) {
+    f = (float) s;
+    if (!(__builtin_fabsf(f) < __builtin_inff()))
+        return true; /* overflow or NaN: the order of the sum does not decide it */
+    const double up = 0.5 * ((double) f + (double) nextafterf(f, __builtin_inff()));
+    const double dn = 0.5 * ((double) f + (double) nextafterf(f, -__builtin_inff()));
+    return up - s > err && s - dn > err;
+}
+
+/* The reference's own order, by one lane. */
+__device__ float f16_dot_f64_sequential(const uint16_t *__restrict__ wr,
+                                        const double *__restrict__ xr, int n_in) {
+    double acc = 0.0;
+    for (int k = 0; k < n_in; k += 8) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(wr + k);
+        const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
+            acc = __builtin_fma(xr[k + 2 * i], (double) f.x, acc);
+            acc = __builtin_fma(xr[k + 2 * i + 1], (double) f.y, acc);
+        }
+    }
+    return (float) acc;
+}
+
+template <int MT>
+__global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__restrict__ w,
+                                                           long n_out, int n_in,
+                                                           const double *__restrict__ xd,
+                                                           const double *__restrict__ xn, int n_m,
+                                                           float *__restrict__ y, long ld_y) {
+    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
+    const int  lane = threadIdx.x & (LM_WAVE - 1);
+    const int  wave = __builtin_amdgcn_readfirstlane(threadIdx.x / LM_WAVE);
+    const long row0 = (long) blockIdx.x * ROWS_BLOCK_B + wave * ROWS_WAVE_B;
+    if (row0 >= n_out)
+        return;
+    uint8_t       *tile     = s_tile[wave];
+    const uint8_t *row_tile = tile + lane * TILE_PITCH;
+
+    double acc[MT][2];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m][0] = acc[m][1] = 0.0;
+    float w2 = 0.0f;
+
+    const int  n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    StageRegsB g0, g1;
+    stage_load_b(w, row0, n_out, n_in, 0, lane, g0);
+    if (n_stage > 1)
+        stage_load_b(w, row0, n_out, n_in, 1, lane, g1);
+    auto do_stage = [&](int s, StageRegsB &g) {
+#pragma unroll
+        for (int i = 0; i < STAGE_LOADS_B; ++i)
+            *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
+                g.w[i];
+        if (s + 2 < n_stage)
+            stage_load_b(w, row0, n_out, n_in, s + 2, lane, g);
+        const int col0  = s * STAGE_COLS;
+        const int left  = n_in - col0;
+        const int steps = left >= STAGE_COLS ? STAGE_COLS / 8 : left / 8;
+        for (int t = 0; t < steps; ++t) {
+            const uint4    q    = *reinterpret_cast<const uint4 *>(row_tile + t * 16);
+            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+            double         wd[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
+                w2             = __builtin_fmaf(f.x, f.x, w2);
+                w2             = __builtin_fmaf(f.y, f.y, w2);
+                wd[2 * i]      = (double) f.x;
+                wd[2 * i + 1]  = (double) f.y;
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                /* (uniform address: the activations come as scalar operands) */
+                const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in + col0 + t * 8;
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    acc[m][i & 1] = __builtin_fma(wd[i], xm[i], acc[m][i & 1]);
+            }
+        }
+    };
+    for (int s = 0; s < n_stage; s += 2) {
+        do_stage(s, g0);
+        if (s + 1 < n_stage)
+            do_stage(s + 1, g1);
+    }
+    const long row = row0 + lane;
+    if (row >= n_out)
+        return;
+    /* ||w||_2 from the binary32 sum of squares: rounded up by more than its error */
+    const double wn = sqrt((double) w2) * (1.0 + 1e-3);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if (m >= n_m)
+            break;
+        const double sum = acc[m][0] + acc[m][1];
+        const double err = (double) n_in * 0x1p-52 * wn * xn[m];
+        float        f;
+        if (!f32_rounding_is_safe(sum, err, f))
+            f = f16_dot_f64_sequential(w + row * n_in, xd + (long) m * n_in, n_in);
+        y[m * ld_y + row] = f;
+    }
+}
+
 /* One workgroup per row. The reference adds the squares in double in index order; the order of
  * a double sum only shows in the binary32 result when 1 / sqrt(mean + eps) lies within the
  * sum's error of the middle between two binary32 values. The workgroup adds in a fixed parallel
@@ -450,6 +594,22 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
         k_f16_gemv_batched<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y);
     else
         k_f16_gemv<8, false><<<grid, block, 0, stream>>>(w_f16, n_out, n_in, x, ld_x, n_m, y, ld_y, none);
+}
+
+void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
+                           const float *x, long ld_x, int n_m, double *xd, double *xn, float *y,
+                           long ld_y) {
+    const dim3 block(LM_TPB);
+    const dim3 grid_b((unsigned) ((n_out + ROWS_BLOCK_B - 1) / ROWS_BLOCK_B));
+    k_x_to_f64<<<dim3(n_m), block, 0, stream>>>(x, ld_x, n_in, xd, xn);
+    if (n_m <= 1)
+        k_f16_linear_f64<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+    else if (n_m <= 2)
+        k_f16_linear_f64<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+    else if (n_m <= 4)
+        k_f16_linear_f64<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+    else
+        k_f16_linear_f64<8><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
 }
 
 /* f16_to_q8w (kernel_f16_gemv.c:66-93): per row scale = max|w| / 127, q = lrintf(w * (127 /

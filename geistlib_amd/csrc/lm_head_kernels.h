@@ -37,6 +37,13 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
                      const float *x, long ld_x, int n_m, float *y, long ld_y,
                      const GemvFuse *fuse = nullptr);
 
+/* The portable kernel (cpu_scalar_w_quant_mN for F16): y[m][r] = (float) sum_i (double) x[m][i] *
+ * (double) f16(W[r][i]), the sum as if in index order; n_m <= GEMV_M_MAX, n_in a multiple of 8.
+ * xd [n_m * n_in] and xn [n_m] are scratch (the activations in double, their norms). */
+void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
+                           const float *x, long ld_x, int n_m, double *xd, double *xn, float *y,
+                           long ld_y);
+
 /* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *
  * scales[r]; n_in a multiple of 16. */
 void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, long n_out,

@@ -44,6 +44,9 @@ struct geist_hip_sampler {
     float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
                                      * full-vocabulary top-p / min-p path */
     gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
+    double  *xd          = nullptr; /* [GEMV_M_MAX][xd_cap] + GEMV_M_MAX: activations in double and
+                                     * their norms, allocated on first use by the f64 projection */
+    size_t   xd_cap      = 0;
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
@@ -218,6 +221,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
+    (void) hipFree(s->xd);
     (void) hipFree(s->cand.row_bound);
     (void) hipFree(s->cand.out_key);
     (void) hipFree(s->cand.key);
@@ -604,6 +608,56 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                         (int) m, d_y + m0 * ld_y, (long) ld_y);
     }
     return after_launch(s, "f16 gemv");
+}
+
+/* The double copy of the activations of one pass and their norms. */
+static int ensure_xd(geist_hip_sampler *s, size_t n_in) {
+    if (s->xd_cap >= n_in)
+        return GEIST_HIP_OK;
+    if (s->xd) {
+        HIPCHK(s, hipStreamSynchronize(s->stream));
+        (void) hipFree(s->xd);
+        s->xd = nullptr, s->xd_cap = 0;
+    }
+    if (hipMalloc(reinterpret_cast<void **>(&s->xd), (size_t) GEMV_M_MAX * (n_in + 1) * sizeof(double)) !=
+        hipSuccess)
+        return fail(s, GEIST_HIP_E_OOM, "f64 projection: activations in double");
+    s->xd_cap = n_in;
+    return GEIST_HIP_OK;
+}
+
+static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out, size_t n_in,
+                           const float *d_x, size_t ld_x, size_t n_rows, float *d_y, size_t ld_y) {
+    const int rc = ensure_xd(s, n_in);
+    if (rc)
+        return rc;
+    double *xn = s->xd + (size_t) GEMV_M_MAX * s->xd_cap;
+    for (size_t m0 = 0; m0 < n_rows; m0 += GEMV_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) GEMV_M_MAX ? n_rows - m0 : (size_t) GEMV_M_MAX;
+        launch_f16_linear_f64(s->stream, d_w_f16, (long) n_out, (int) n_in, d_x + m0 * ld_x,
+                              (long) ld_x, (int) m, s->xd, xn, d_y + m0 * ld_y, (long) ld_y);
+    }
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
+                              size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                              float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_f16 || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_out == 0 || n_in == 0 || n_rows == 0 || n_in > 0x7ffffff8u || ld_x < n_in ||
+        ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "linear: %zu x %zu, %zu rows, strides %zu / %zu",
+                    n_out, n_in, n_rows, ld_x, ld_y);
+    if (n_in % 8 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "linear: n_in %zu is not a multiple of 8", n_in);
+    if (((uintptr_t) d_w_f16) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "linear: weights not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    const int rc = f16_linear_impl(s, d_w_f16, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "f16 linear");
 }
 
 int geist_hip_f16_to_q8w(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out, size_t n_in,

@@ -36,6 +36,18 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
                             size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
                             size_t ld_y);
 
+/* geist_hip_f16_linear_rows replaces the portable kernel cpu_scalar_w_quant_m1 / _mN for F16
+ * weights (src/backends/cpu_scalar/weight_resolve.c:186-241), which is also what the x86 backend
+ * runs for more than one activation row (its F16 and int8 kernels are decode-only, linear_m1):
+ *   d_y[m * ld_y + r] = (float) sum_i (double) d_x[m * ld_x + i] * (double) f16(W[r][i])
+ * with the sum in double in index order, bit for bit: the device adds in another order and
+ * repeats, in the reference's order, the few sums that lie close enough to a binary32 rounding
+ * boundary for the order to matter. Same argument rules as geist_hip_f16_gemv_rows. The first
+ * call allocates a small buffer in the sampler (the activations in double). */
+int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
+                              size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                              float *d_y, size_t ld_y);
+
 /* The int8 form of the tied table, which the reference's x86 backend uses for the lm_head unless
  * GEIST_Q8_LMHEAD=0 (src/backends/cpu_x86/backend.c:344-372): half the bytes per decode step.
  *

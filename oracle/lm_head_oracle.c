@@ -152,3 +152,19 @@ void oracle_rmsnorm_rows(size_t n_rows, size_t n, const float *x, const float *w
             y[r * n + i] = xr[i] * inv * w[i];
     }
 }
+
+
+void oracle_f16_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const uint16_t *w_f16, float *y) {
+    /* weight_resolve.c:221-238 with dequant_one_row_for's F16 case (:62-68) */
+#pragma omp parallel for schedule(static)
+    for (size_t j = 0; j < n_out; j++) {
+        const uint16_t *wr = w_f16 + j * n_in;
+        for (size_t i = 0; i < m; i++) {
+            double acc = 0.0;
+            for (size_t k = 0; k < n_in; k++)
+                acc += (double) x[i * n_in + k] * (double) oracle_f16_to_f32(wr[k]);
+            y[i * n_out + j] = (float) acc;
+        }
+    }
+}

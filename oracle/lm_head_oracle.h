@@ -42,6 +42,15 @@ void oracle_f16_to_q8w(size_t n_out, size_t n_in, const uint16_t *w_f16, int8_t 
 void oracle_q8w_gemv_m1(size_t n_out, size_t n_in, const float *x, const int8_t *wq,
                         const float *scales, float *y);
 
+/* The portable kernel, which the x86 backend also runs for more than one activation row
+ * (cpu_scalar_w_quant_m1 / _mN, src/backends/cpu_scalar/weight_resolve.c:186-241, for F16
+ * weights): y[i][j] = (float) sum_k (double) x[i][k] * (double) f16(W[j][k]), the sum in double in
+ * index order. (The products are exact in double, so a fused multiply-add gives the same bits.)
+ * Pinned by numpy's float64 dot wherever that is not within the sums' error of a binary32
+ * rounding boundary, and by exactly representable cases. */
+void oracle_f16_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const uint16_t *w_f16, float *y);
+
 /* y = x * weight * rsqrt(mean(x^2) + eps) per row (cpu_scalar_rmsnorm,
  * src/backends/cpu_scalar/elementwise.c:241-280): sum of squares in double in index order,
  * inv = (float)(1.0 / sqrt(sum / n + (double) eps)), y_i = (x_i * inv) * w_i in binary32. */

@@ -225,6 +225,18 @@ class Oracle:
                                         wq.ctypes.data_as(C.POINTER(C.c_int8)), _fp(scales), _fp(y[m]))
         return y[0] if np.ndim(x) == 1 else y
 
+    def f16_linear_f64(self, w_f16, x):
+        """cpu_scalar_w_quant_mN for F16 weights: [m, n_in] x [n_out, n_in] -> [m, n_out]."""
+        w = np.ascontiguousarray(w_f16, dtype=np.uint16)
+        xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+        n_out, n_in = w.shape
+        y = np.empty((xs.shape[0], n_out), dtype=np.float32)
+        self.lib.oracle_f16_linear_f64.argtypes = [C.c_size_t] * 3 + [c_float_p, C.POINTER(C.c_uint16),
+                                                                      c_float_p]
+        self.lib.oracle_f16_linear_f64(xs.shape[0], n_out, n_in, _fp(xs),
+                                       w.ctypes.data_as(C.POINTER(C.c_uint16)), _fp(y))
+        return y[0] if np.ndim(x) == 1 else y
+
     def rmsnorm(self, x, w, eps):
         xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
         w = np.ascontiguousarray(w, dtype=np.float32)

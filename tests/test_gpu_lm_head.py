@@ -269,3 +269,27 @@ def test_project_sample_rows_q8w_rejects_what_it_cannot_take(hs):
     with pytest.raises(GeistHipError):
         hs.project_sample_q8w(h, nw, 1e-6, wq, None, logits, SampleParams.make(temperature=0.0),
                               None, out, normed=torch.empty_like(h))
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(1000, 2560, 1), (130, 128, 1), (129, 256, 3),
+                                          (4097, 1536, 2), (300, 8, 1), (300, 40, 5), (257, 72, 4),
+                                          (640, 4096, 8), (500, 2560, 11), (20000, 2560, 8)])
+def test_f16_linear_in_double_bit_exact(hs, oracle, n_out, n_in, m):
+    """geist_hip_f16_linear_rows against cpu_scalar_w_quant_mN (weight_resolve.c:215-241): the
+    double sum in index order, rounded once -- equal in every bit, also where the sum lies at a
+    binary32 rounding boundary (integer inputs make many sums land exactly on one)."""
+    print(f"f16 linear f64 n_out={n_out} n_in={n_in} m={m}", flush=True)
+    g = np.random.default_rng(n_out + 5 * n_in + m)
+    w16 = (g.standard_normal((n_out, n_in)) * g.choice([0.02, 1.0])).astype(np.float16)
+    x = (g.standard_normal((m, n_in)) * g.choice([0.1, 1.0, 30.0], (m, 1))).astype(np.float32)
+    if n_out > 256:
+        # rows whose sums are exact halves of a binary32 step: every order must agree there too
+        w16[:128] = g.integers(-4, 5, (128, n_in)).astype(np.float16)
+        x[0] = g.integers(-3, 4, n_in).astype(np.float32)
+        x[0, 0] += np.float32(2.0 ** -20)
+    y = torch.full((m, n_out), 7.0, dtype=torch.float32, device="cuda")
+    hs.f16_linear(to_dev(w16.view(np.int16), torch), to_dev(x, torch), y)
+    hs.sync()
+    want = oracle.f16_linear_f64(w16.view(np.uint16), x)
+    got = y.cpu().numpy()
+    assert (bits(got) == bits(want)).all(), np.argwhere(bits(got) != bits(want))[:5]

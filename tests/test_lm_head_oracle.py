@@ -171,3 +171,27 @@ def test_q8w_keeps_the_reference_tests_bar(oracle):
     cos = (y @ exact) / np.sqrt((y @ y) * (exact @ exact))
     assert cos >= 0.999
     assert np.abs(wq).max() <= 127 and (np.abs(wq).max(axis=1) == 127).all()
+
+
+def test_f16_linear_f64_against_numpy(oracle):
+    """cpu_scalar_w_quant_mN for F16 weights (weight_resolve.c:215-241): the double sum in index
+    order, rounded once. numpy's float64 dot adds in another order; the two agree wherever the
+    value is not within the sums' error of a binary32 rounding boundary, which is checked, and on
+    integer-valued inputs (every partial sum exact) in every bit."""
+    g = np.random.default_rng(31)
+    n_out, n_in, m = 700, 2560, 3
+    w = (g.standard_normal((n_out, n_in)) * 0.05).astype(np.float16)
+    x = (g.standard_normal((m, n_in)) * 2).astype(np.float32)
+    y = oracle.f16_linear_f64(w.view(np.uint16), x)
+    exact = x.astype(np.float64) @ w.astype(np.float64).T
+    bound = n_in * 2.0 ** -52 * (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T)
+    lo, hi = (exact - bound).astype(np.float32), (exact + bound).astype(np.float32)
+    sure = lo == hi
+    assert sure.mean() > 0.99
+    assert (y[sure] == lo[sure]).all()
+    assert ((y >= lo) & (y <= hi)).all()
+    wi = g.integers(-8, 9, (50, 64)).astype(np.float16)
+    xi = g.integers(-100, 101, (2, 64)).astype(np.float32)
+    assert (oracle.f16_linear_f64(wi.view(np.uint16), xi) == (xi @ wi.astype(np.float32).T)).all()
+    # one row, one-dimensional in and out
+    assert (oracle.f16_linear_f64(w.view(np.uint16), x[1]) == y[1]).all()
