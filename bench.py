@@ -199,8 +199,20 @@ def bench_lm_head(args, m_rows, q8=False):
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
     # the projection alone
-    kernel_us = (hs.time_q8w_gemv(tables_q8, scales, normed, logits, args.steps) if q8
-                 else hs.time_f16_gemv(tables, normed, logits, args.steps))
+    f64_batch = (not q8) and m_rows > 1   # what project_sample runs for more than one F16 row
+    if q8:
+        kernel_us = hs.time_q8w_gemv(tables_q8, scales, normed, logits, args.steps)
+    elif not f64_batch:
+        kernel_us = hs.time_f16_gemv(tables, normed, logits, args.steps)
+    else:
+        for i in range(3):
+            hs.f16_linear(tables[i % len(tables)], normed, logits)
+        hs.sync()
+        t1 = time.perf_counter()
+        for i in range(args.steps):
+            hs.f16_linear(tables[i % len(tables)], normed, logits)
+        hs.sync()
+        kernel_us = (time.perf_counter() - t1) * 1e6 / args.steps
     w_bytes = vocab * d_model + vocab * 4 if q8 else vocab * d_model * 2
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -208,7 +220,8 @@ def bench_lm_head(args, m_rows, q8=False):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("int8" if q8 else "f16") + " weights x f32 activations, f32 accumulation",
+        "dtype": ("int8" if q8 else "f16") + " weights x f32 activations, "
+                 + ("f64" if (not q8 and m_rows > 1) else "f32") + " accumulation",
         "data": "synthetic",
         "config": {"workload": f"lm_head{'_q8' if q8 else ''}_v{vocab}_d{d_model}_m{m_rows}",
                    "rows": m_rows,
@@ -218,7 +231,9 @@ def bench_lm_head(args, m_rows, q8=False):
         "weight_copies_rotated": len(tables),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_q8w_gemv" if q8 else "k_f16_gemv",
+                     "kernel": ("k_q8w_gemv" if q8 else
+                                "k_f16_linear_f64 (+ activations to double, listed outputs)"
+                                if f64_batch else "k_f16_gemv"),
                      "kernel_us": round(kernel_us, 3),
                      "kernel_algorithmic_bytes": w_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
@@ -260,7 +275,8 @@ def bench_lm_head(args, m_rows, q8=False):
                       "projection only, no norm, no sampling)"}
         # parity of the whole tail on the last step's inputs
         x_normed = o.rmsnorm(hidden.cpu().numpy(), norm_w.cpu().numpy(), 1e-6)
-        want_logits = o.q8w_gemv(wq, sc, x_normed) if q8 else o.f16_gemv(wt, x_normed)
+        want_logits = (o.q8w_gemv(wq, sc, x_normed) if q8 else
+                       o.f16_linear_f64(wt, x_normed) if f64_batch else o.f16_gemv(wt, x_normed))
         same_bits = bool((want_logits.view(np.uint32) == logits.cpu().numpy().view(np.uint32)).all())
         want_ids = [o.chain_u(want_logits[r], float(u[r]), temperature=0.7, top_k=40, top_p=0.9)[0]
                     for r in range(m_rows)]

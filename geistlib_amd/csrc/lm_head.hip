@@ -411,32 +411,39 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_gemv_batched(const uint16_t *__r
  * additions could differ from the reference, and that shows in the binary32 result only when
  * the sum lies within the additions' error of a binary32 rounding boundary. A lane owns a
  * weight row and adds in its own order (two partial sums per activation row); an output that
- * close to a boundary -- about two in a thousand -- is added once more in index order by the
- * same lane. The error bound uses |sum_k x_k w_k| terms <= ||x||_2 ||w||_2 (the row's norm is
- * accumulated on the way in binary32, the activations' norm comes with their double copy). */
+ * close to a boundary -- a few in a hundred thousand -- goes on a list, and a second kernel adds
+ * those once more in index order, one lane per output. The error of either order is at most
+ * n * 2^-53 times the largest partial sum on its way; the lane's two partial sums cover the
+ * columns in ascending order, so after every stage of 64 columns |a0| + |a1| bounds both orders'
+ * partial sums there, and within a stage a partial sum moves by at most ||w_stage|| ||x_stage||
+ * (the weights' part is accumulated on the way in binary32, the activations' part comes with
+ * their double copy). */
 
-/* xd[m][k] = (double) x[m][k], xn[m] = ||x[m]||_2 (rounded up a little). One workgroup per row. */
+/* xd[m][k] = (double) x[m][k]; xs[m][s] = ||x[m][64 s .. 64 s + 63]||_2, rounded up; the count
+ * of outputs left to the second kernel starts at zero. One workgroup per row, a wavefront per
+ * stage of 64 columns. */
 __global__ __launch_bounds__(LM_TPB) void k_x_to_f64(const float *__restrict__ x, long ld_x,
                                                      int n_in, double *__restrict__ xd,
-                                                     double *__restrict__ xn) {
-    __shared__ double s_part[LM_TPB];
-    const int    tid = threadIdx.x;
-    const float *xr  = x + (long) blockIdx.x * ld_x;
-    double       a   = 0.0;
-    for (int k = tid; k < n_in; k += LM_TPB) {
-        const double v = (double) xr[k];
-        xd[(long) blockIdx.x * n_in + k] = v;
-        a += v * v;
+                                                     double *__restrict__ xs, int *amb_count) {
+    const int    lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
+    const float *xr   = x + (long) blockIdx.x * ld_x;
+    const int    n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        *amb_count = 0;
+    for (int st = wave; st < n_stage; st += LM_WAVES) {
+        const int k = st * STAGE_COLS + lane;
+        double    v = 0.0;
+        if (k < n_in) {
+            v = (double) xr[k];
+            xd[(long) blockIdx.x * n_in + k] = v;
+        }
+        double a = v * v;
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1)
+            a += __shfl_xor(a, d, LM_WAVE);
+        if (lane == 0)
+            xs[(long) blockIdx.x * n_stage + st] = sqrt(a) * (1.0 + 0x1p-40);
     }
-    s_part[tid] = a;
-    __syncthreads();
-    for (int step = LM_TPB / 2; step > 0; step >>= 1) {
-        if (tid < step)
-            s_part[tid] += s_part[tid + step];
-        __syncthreads();
-    }
-    if (tid == 0)
-        xn[blockIdx.x] = sqrt(s_part[0]) * (1.0 + 0x1p-40);
 }
 
 /* (float) s, and whether every value within err of s rounds to the same binary32. */
@@ -449,29 +456,41 @@ __device__ __forceinline__ bool f32_rounding_is_safe(double s, double err, float
     return up - s > err && s - dn > err;
 }
 
-/* The reference's own order, by one lane. */
-__device__ float f16_dot_f64_sequential(const uint16_t *__restrict__ wr,
-                                        const double *__restrict__ xr, int n_in) {
-    double acc = 0.0;
-    for (int k = 0; k < n_in; k += 8) {
-        const uint4 q = *reinterpret_cast<const uint4 *>(wr + k);
-        const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+/* One step of eight columns: this lane's weights against activations that are uniform over the
+ * wavefront (scalar operands). */
+template <int MT>
+__device__ __forceinline__ void linear_f64_step(const uint8_t *row_tile, int byte_off,
+                                                const double *__restrict__ xd, int n_in, int n_m,
+                                                int col, double (&acc)[MT][2], float &w2) {
+    const uint4  q   = *reinterpret_cast<const uint4 *>(row_tile + byte_off);
+    const float2 f01 = __half22float2(*reinterpret_cast<const __half2 *>(&q.x));
+    const float2 f23 = __half22float2(*reinterpret_cast<const __half2 *>(&q.y));
+    const float2 f45 = __half22float2(*reinterpret_cast<const __half2 *>(&q.z));
+    const float2 f67 = __half22float2(*reinterpret_cast<const __half2 *>(&q.w));
+    const float  wf[8] = {f01.x, f01.y, f23.x, f23.y, f45.x, f45.y, f67.x, f67.y};
+    double       wd[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
-            acc = __builtin_fma(xr[k + 2 * i], (double) f.x, acc);
-            acc = __builtin_fma(xr[k + 2 * i + 1], (double) f.y, acc);
-        }
+    for (int i = 0; i < 8; ++i) {
+        w2    = __builtin_fmaf(wf[i], wf[i], w2);
+        wd[i] = (double) wf[i];
     }
-    return (float) acc;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in + col; /* uniform address */
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc[m][i & 1] = __builtin_fma(wd[i], xm[i], acc[m][i & 1]);
+    }
 }
 
 template <int MT>
 __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__restrict__ w,
                                                            long n_out, int n_in,
                                                            const double *__restrict__ xd,
-                                                           const double *__restrict__ xn, int n_m,
-                                                           float *__restrict__ y, long ld_y) {
+                                                           const double *__restrict__ xs, int n_m,
+                                                           float *__restrict__ y, long ld_y,
+                                                           int *__restrict__ amb_count,
+                                                           int2 *__restrict__ amb_list) {
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
     const int  lane = threadIdx.x & (LM_WAVE - 1);
     const int  wave = __builtin_amdgcn_readfirstlane(threadIdx.x / LM_WAVE);
@@ -481,69 +500,142 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__res
     uint8_t       *tile     = s_tile[wave];
     const uint8_t *row_tile = tile + lane * TILE_PITCH;
 
-    double acc[MT][2];
+    double acc[MT][2], pmax[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
-        acc[m][0] = acc[m][1] = 0.0;
-    float w2 = 0.0f;
+        acc[m][0] = acc[m][1] = pmax[m] = 0.0;
 
     const int  n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
     StageRegsB g0, g1;
     stage_load_b(w, row0, n_out, n_in, 0, lane, g0);
     if (n_stage > 1)
         stage_load_b(w, row0, n_out, n_in, 1, lane, g1);
-    auto do_stage = [&](int s, StageRegsB &g) {
+    for (int s = 0; s < n_stage; ++s) {
 #pragma unroll
         for (int i = 0; i < STAGE_LOADS_B; ++i)
             *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
-                g.w[i];
+                g0.w[i];
+        g0 = g1;
         if (s + 2 < n_stage)
-            stage_load_b(w, row0, n_out, n_in, s + 2, lane, g);
-        const int col0  = s * STAGE_COLS;
-        const int left  = n_in - col0;
-        const int steps = left >= STAGE_COLS ? STAGE_COLS / 8 : left / 8;
-        for (int t = 0; t < steps; ++t) {
-            const uint4    q    = *reinterpret_cast<const uint4 *>(row_tile + t * 16);
-            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-            double         wd[8];
+            stage_load_b(w, row0, n_out, n_in, s + 2, lane, g1);
+        const int col0 = s * STAGE_COLS;
+        const int left = n_in - col0;
+        double    p0[MT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
-                w2             = __builtin_fmaf(f.x, f.x, w2);
-                w2             = __builtin_fmaf(f.y, f.y, w2);
-                wd[2 * i]      = (double) f.x;
-                wd[2 * i + 1]  = (double) f.y;
-            }
+        for (int m = 0; m < MT; ++m)
+            p0[m] = fabs(acc[m][0]) + fabs(acc[m][1]);
+        float w2 = 0.0f;
+        if (left >= STAGE_COLS) {
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                /* (uniform address: the activations come as scalar operands) */
-                const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in + col0 + t * 8;
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    acc[m][i & 1] = __builtin_fma(wd[i], xm[i], acc[m][i & 1]);
-            }
+            for (int t = 0; t < STAGE_COLS / 8; ++t)
+                linear_f64_step<MT>(row_tile, t * 16, xd, n_in, n_m, col0 + t * 8, acc, w2);
+        } else {
+            for (int t = 0; t < left / 8; ++t)
+                linear_f64_step<MT>(row_tile, t * 16, xd, n_in, n_m, col0 + t * 8, acc, w2);
         }
-    };
-    for (int s = 0; s < n_stage; s += 2) {
-        do_stage(s, g0);
-        if (s + 1 < n_stage)
-            do_stage(s + 1, g1);
+        /* ||w_stage||_2 from its binary32 sum of squares, rounded up by more than its error */
+        const double wn = (double) __builtin_sqrtf(w2) * (1.0 + 1e-4);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const double p = p0[m] + wn * xs[(long) (m < n_m ? m : n_m - 1) * n_stage + s];
+            pmax[m]        = p > pmax[m] ? p : pmax[m];
+        }
     }
     const long row = row0 + lane;
     if (row >= n_out)
         return;
-    /* ||w||_2 from the binary32 sum of squares: rounded up by more than its error */
-    const double wn = sqrt((double) w2) * (1.0 + 1e-3);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         if (m >= n_m)
             break;
         const double sum = acc[m][0] + acc[m][1];
-        const double err = (double) n_in * 0x1p-52 * wn * xn[m];
+        /* n 2^-53 (largest partial sum) for each of the two orders, and a little room for the
+         * rounding of the bound itself */
+        const double err = (double) n_in * 0x1p-52 * 1.01 * pmax[m];
         float        f;
         if (!f32_rounding_is_safe(sum, err, f))
-            f = f16_dot_f64_sequential(w + row * n_in, xd + (long) m * n_in, n_in);
+            amb_list[atomicAdd(amb_count, 1)] = make_int2((int) row, m);
         y[m * ld_y + row] = f;
+    }
+}
+
+/* The listed outputs once more, in the reference's order: a lane per output (weight row r,
+ * activation row m), a wavefront streams its 64 weight rows through its LDS tile as above and
+ * every lane adds its row's products one after the other. The activations of a stage lie in LDS
+ * for all activation rows; a lane reads those of its own. */
+__global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
+    const uint16_t *__restrict__ w, int n_in, const double *__restrict__ xd, int n_m,
+    float *__restrict__ y, long ld_y, const int *__restrict__ amb_count,
+    const int2 *__restrict__ amb_list) {
+    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
+    __shared__ double                s_x[LM_WAVES][GEMV_M_MAX][STAGE_COLS];
+    const int lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
+    const int count = *amb_count;
+    uint8_t  *tile  = s_tile[wave];
+    const int n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    for (int it0 = ((int) blockIdx.x * LM_WAVES + wave) * LM_WAVE; it0 < count;
+         it0 += (int) gridDim.x * LM_WAVES * LM_WAVE) { /* (uniform over the wavefront) */
+        const int2 mine = amb_list[it0 + lane < count ? it0 + lane : count - 1];
+        /* the rows whose segment (lane & 7) this lane fetches: items 8 i + (lane >> 3) */
+        long fetch_row[STAGE_LOADS_B];
+#pragma unroll
+        for (int i = 0; i < STAGE_LOADS_B; ++i) {
+            const int it  = it0 + 8 * i + (lane >> 3);
+            fetch_row[i] = (long) amb_list[it < count ? it : count - 1].x;
+        }
+        /* weights two stages ahead in registers, activations one stage ahead */
+        auto fetch_w = [&](int s, StageRegsB &g) {
+            const int col = s * STAGE_COLS + (lane & 7) * 8;
+#pragma unroll
+            for (int i = 0; i < STAGE_LOADS_B; ++i) {
+                g.w[i] = make_uint4(0u, 0u, 0u, 0u);
+                if (col < n_in)
+                    g.w[i] = *reinterpret_cast<const uint4 *>(w + fetch_row[i] * n_in + col);
+            }
+        };
+        auto fetch_x = [&](int s, double (&xr)[GEMV_M_MAX]) {
+            const int k = s * STAGE_COLS + lane;
+#pragma unroll
+            for (int m = 0; m < GEMV_M_MAX; ++m)
+                xr[m] = (m < n_m && k < n_in) ? xd[(long) m * n_in + k] : 0.0;
+        };
+        StageRegsB g0, g1;
+        double     x0[GEMV_M_MAX];
+        fetch_w(0, g0);
+        fetch_x(0, x0);
+        if (n_stage > 1)
+            fetch_w(1, g1);
+        double acc = 0.0;
+        for (int s = 0; s < n_stage; ++s) {
+            const int col0 = s * STAGE_COLS;
+#pragma unroll
+            for (int i = 0; i < STAGE_LOADS_B; ++i)
+                *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH +
+                                           (lane & 7) * 16) = g0.w[i];
+#pragma unroll
+            for (int m = 0; m < GEMV_M_MAX; ++m)
+                s_x[wave][m][lane] = x0[m];
+            g0 = g1;
+            if (s + 2 < n_stage)
+                fetch_w(s + 2, g1);
+            if (s + 1 < n_stage)
+                fetch_x(s + 1, x0);
+            const uint8_t *row_tile = tile + lane * TILE_PITCH;
+            const double  *xm       = s_x[wave][mine.y];
+            const int      steps    = (n_in - col0 >= STAGE_COLS ? STAGE_COLS : n_in - col0) / 8;
+            for (int t = 0; t < steps; ++t) {
+                const uint4    q    = *reinterpret_cast<const uint4 *>(row_tile + t * 16);
+                const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
+                    acc = __builtin_fma(xm[t * 8 + 2 * i], (double) f.x, acc);
+                    acc = __builtin_fma(xm[t * 8 + 2 * i + 1], (double) f.y, acc);
+                }
+            }
+        }
+        if (it0 + lane < count)
+            y[mine.y * ld_y + mine.x] = (float) acc;
     }
 }
 
@@ -597,19 +689,22 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
 }
 
 void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
-                           const float *x, long ld_x, int n_m, double *xd, double *xn, float *y,
+                           const float *x, long ld_x, int n_m, const F64Scratch &ws, float *y,
                            long ld_y) {
     const dim3 block(LM_TPB);
     const dim3 grid_b((unsigned) ((n_out + ROWS_BLOCK_B - 1) / ROWS_BLOCK_B));
-    k_x_to_f64<<<dim3(n_m), block, 0, stream>>>(x, ld_x, n_in, xd, xn);
+    k_x_to_f64<<<dim3(n_m), block, 0, stream>>>(x, ld_x, n_in, ws.xd, ws.xs, ws.amb_count);
     if (n_m <= 1)
-        k_f16_linear_f64<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+        k_f16_linear_f64<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else if (n_m <= 2)
-        k_f16_linear_f64<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+        k_f16_linear_f64<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else if (n_m <= 4)
-        k_f16_linear_f64<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+        k_f16_linear_f64<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else
-        k_f16_linear_f64<8><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, xd, xn, n_m, y, ld_y);
+        k_f16_linear_f64<8><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    /* normally a few dozen outputs: one wavefront's worth; the grid strides over longer lists */
+    k_f16_linear_f64_listed<<<dim3(64), block, 0, stream>>>(w_f16, n_in, ws.xd, n_m, y, ld_y,
+                                                           ws.amb_count, ws.amb_list);
 }
 
 /* f16_to_q8w (kernel_f16_gemv.c:66-93): per row scale = max|w| / 127, q = lrintf(w * (127 /

@@ -37,11 +37,17 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
                      const float *x, long ld_x, int n_m, float *y, long ld_y,
                      const GemvFuse *fuse = nullptr);
 
+/* Scratch of the double-accumulation projection, for one pass of up to GEMV_M_MAX rows. */
+struct F64Scratch {
+    double *xd;        /* [GEMV_M_MAX][n_in] the activations in double */
+    double *xs;        /* [GEMV_M_MAX][ceil(n_in / 64)] their norms per stage of 64 columns */
+    int    *amb_count; /* outputs whose rounding depends on the order of the sum ... */
+    int2   *amb_list;  /* ... [n_out * GEMV_M_MAX] (weight row, activation row) */
+};
 /* The portable kernel (cpu_scalar_w_quant_mN for F16): y[m][r] = (float) sum_i (double) x[m][i] *
- * (double) f16(W[r][i]), the sum as if in index order; n_m <= GEMV_M_MAX, n_in a multiple of 8.
- * xd [n_m * n_in] and xn [n_m] are scratch (the activations in double, their norms). */
+ * (double) f16(W[r][i]), the sum as if in index order; n_m <= GEMV_M_MAX, n_in a multiple of 8. */
 void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
-                           const float *x, long ld_x, int n_m, double *xd, double *xn, float *y,
+                           const float *x, long ld_x, int n_m, const F64Scratch &ws, float *y,
                            long ld_y);
 
 /* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *

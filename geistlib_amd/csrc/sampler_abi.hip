@@ -44,9 +44,9 @@ struct geist_hip_sampler {
     float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
                                      * full-vocabulary top-p / min-p path */
     gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
-    double  *xd          = nullptr; /* [GEMV_M_MAX][xd_cap] + GEMV_M_MAX: activations in double and
-                                     * their norms, allocated on first use by the f64 projection */
-    size_t   xd_cap      = 0;
+    void    *f64_ws      = nullptr; /* scratch of the f64 projection for n_in <= f64_in and
+                                     * n_out <= f64_out, allocated on first use */
+    size_t   f64_in = 0, f64_out = 0;
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
@@ -221,7 +221,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
-    (void) hipFree(s->xd);
+    (void) hipFree(s->f64_ws);
     (void) hipFree(s->cand.row_bound);
     (void) hipFree(s->cand.out_key);
     (void) hipFree(s->cand.key);
@@ -610,32 +610,41 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
     return after_launch(s, "f16 gemv");
 }
 
-/* The double copy of the activations of one pass and their norms. */
-static int ensure_xd(geist_hip_sampler *s, size_t n_in) {
-    if (s->xd_cap >= n_in)
-        return GEIST_HIP_OK;
-    if (s->xd) {
-        HIPCHK(s, hipStreamSynchronize(s->stream));
-        (void) hipFree(s->xd);
-        s->xd = nullptr, s->xd_cap = 0;
+/* Scratch of the f64 projection: activations in double, their stage norms, the list of outputs
+ * for the second kernel. */
+static int f64_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, F64Scratch &ws) {
+    if (s->f64_in < n_in || s->f64_out < n_out) {
+        if (s->f64_ws) {
+            HIPCHK(s, hipStreamSynchronize(s->stream));
+            (void) hipFree(s->f64_ws);
+            s->f64_ws = nullptr, s->f64_in = s->f64_out = 0;
+        }
+        const size_t in = n_in > s->f64_in ? n_in : s->f64_in;
+        const size_t out = n_out > s->f64_out ? n_out : s->f64_out;
+        const size_t bytes = (size_t) GEMV_M_MAX * (in + in / 64 + 2) * sizeof(double) + 16 +
+                             out * GEMV_M_MAX * sizeof(int2);
+        if (hipMalloc(&s->f64_ws, bytes) != hipSuccess)
+            return fail(s, GEIST_HIP_E_OOM, "f64 projection: scratch");
+        s->f64_in = in, s->f64_out = out;
     }
-    if (hipMalloc(reinterpret_cast<void **>(&s->xd), (size_t) GEMV_M_MAX * (n_in + 1) * sizeof(double)) !=
-        hipSuccess)
-        return fail(s, GEIST_HIP_E_OOM, "f64 projection: activations in double");
-    s->xd_cap = n_in;
+    char *p      = static_cast<char *>(s->f64_ws);
+    ws.xd        = reinterpret_cast<double *>(p);
+    ws.xs        = ws.xd + (size_t) GEMV_M_MAX * s->f64_in;
+    ws.amb_count = reinterpret_cast<int *>(ws.xs + (size_t) GEMV_M_MAX * (s->f64_in / 64 + 2));
+    ws.amb_list  = reinterpret_cast<int2 *>(reinterpret_cast<char *>(ws.amb_count) + 16);
     return GEIST_HIP_OK;
 }
 
 static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out, size_t n_in,
                            const float *d_x, size_t ld_x, size_t n_rows, float *d_y, size_t ld_y) {
-    const int rc = ensure_xd(s, n_in);
+    F64Scratch ws;
+    const int  rc = f64_scratch(s, n_out, n_in, ws);
     if (rc)
         return rc;
-    double *xn = s->xd + (size_t) GEMV_M_MAX * s->xd_cap;
     for (size_t m0 = 0; m0 < n_rows; m0 += GEMV_M_MAX) {
         const size_t m = n_rows - m0 < (size_t) GEMV_M_MAX ? n_rows - m0 : (size_t) GEMV_M_MAX;
         launch_f16_linear_f64(s->stream, d_w_f16, (long) n_out, (int) n_in, d_x + m0 * ld_x,
-                              (long) ld_x, (int) m, s->xd, xn, d_y + m0 * ld_y, (long) ld_y);
+                              (long) ld_x, (int) m, ws, d_y + m0 * ld_y, (long) ld_y);
     }
     return GEIST_HIP_OK;
 }
@@ -727,7 +736,7 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     if (!rs.greedy && !d_uniforms && !d_rng_states)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic configuration without draws");
     HIPCHK(s, hipSetDevice(s->device));
-    const bool fuse_ok = f16_gemv_can_fuse((int) rows);
+    const bool fuse_ok = f16_gemv_can_fuse((int) rows) && (q8 || rows == 1);
     /* the top-k path's scan is the projection's epilogue when nothing changes the logits
      * between the two (no soft-cap) */
     const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX &&
@@ -746,6 +755,13 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+    } else if (!q8 && rows > 1) {
+        /* more than one row: the reference's batch kernel (cpu_scalar_w_quant_mN), its x86
+         * kernels being decode-only */
+        rc = f16_linear_impl(s, d_embed_f16, n_vocab, d_model, d_normed, d_model, rows, d_logits,
+                             ld_logits);
+        if (rc)
+            return rc;
     } else {
         for (size_t m0 = 0; m0 < rows; m0 += GEMV_M_MAX) {
             const size_t m = rows - m0 < (size_t) GEMV_M_MAX ? rows - m0 : (size_t) GEMV_M_MAX;

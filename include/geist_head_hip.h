@@ -76,8 +76,10 @@ int geist_hip_head_argmax_f32(struct geist_hip_head *h, const float *d_logits, s
  * (head.c:99-101), the tied F16 lm_head (head.c:114-126; [vocab, d_model] binary16, row-major,
  * 16-byte aligned, d_model a multiple of 8), the soft-cap and the session's sampler. The logits
  * live in a buffer of the head and are never copied out; they equal, bit for bit, what the
- * reference's cpu_scalar_rmsnorm and f16_gemv_m1 produce, so the tokens are those of
- * geist_hip_head_finalize_batch on the reference's logits. Row r of d_hidden starts at
+ * reference's cpu_scalar_rmsnorm and its x86 backend's projection produce -- f16_gemv_m1 for
+ * k == 1, the portable cpu_scalar_w_quant_mN (double accumulation) for k > 1, which is what that
+ * backend runs for a batch -- so the tokens are those of geist_hip_head_finalize_batch on the
+ * reference's logits. Row r of d_hidden starts at
  * d_hidden + r * ld_hidden and is left untouched. */
 int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
                                     size_t ld_hidden, size_t k, const float *d_norm_weight,

@@ -66,8 +66,11 @@ int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const floa
                             size_t n_rows, float *d_y, size_t ld_y);
 
 /* The tail of a forward pass in one call (head.c:94-188 / 224-304): norm, projection, sampling
- * of `rows` hidden rows. Equal in results to geist_hip_rmsnorm_rows + geist_hip_f16_gemv_rows +
- * geist_hip_sample_rows[_rng] on d_logits; for one or two rows whose configuration takes the
+ * of `rows` hidden rows. Equal in results to geist_hip_rmsnorm_rows, the projection and
+ * geist_hip_sample_rows[_rng] on d_logits. The projection is the one the reference's x86 backend
+ * runs: for one row its decode kernel (geist_hip_f16_gemv_rows), for more rows the portable
+ * kernel (geist_hip_f16_linear_rows; the x86 kernels are linear_m1 only,
+ * src/archs/transformer/forward/linear.c:34-56). For one row whose configuration takes the
  * top-k path without a soft-cap, the projection also leaves the per-thread maxima the sampler's
  * first pass would compute, and that pass is skipped.
  *   d_normed   [rows, d_model] receives the normed rows
@@ -86,7 +89,8 @@ int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, s
 /* The same tail over the int8 form of the table (the reference's default for a decode step on
  * x86, src/backends/cpu_x86/backend.c:332-342 behind head.c:114-126): d_embed_q8 [n_vocab,
  * d_model] and d_scales [n_vocab] as geist_hip_f16_to_q8w writes them; d_model a multiple of 16.
- * Equal in results to geist_hip_rmsnorm_rows + geist_hip_q8w_gemv_rows + the sampler. */
+ * Equal in results to geist_hip_rmsnorm_rows + geist_hip_q8w_gemv_rows + the sampler, for any
+ * number of rows (the reference has the int8 table for one row at a time only). */
 int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidden,
                                       size_t ld_hidden, size_t rows, size_t d_model,
                                       const float *d_norm_weight, float rms_eps,

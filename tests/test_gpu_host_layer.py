@@ -398,7 +398,8 @@ def test_head_project_finalize_keeps_the_logits_on_the_device(host, oracle):
     d_w = torch.from_numpy(w16.view(np.int16)).cuda()
     d_hid = torch.from_numpy(hidden).cuda()
     d_nw = torch.from_numpy(norm_w).cuda()
-    want_logits = oracle.f16_gemv(w16.view(np.uint16), oracle.rmsnorm(hidden[:, :d_model], norm_w, 1e-6))
+    want_logits = oracle.f16_linear_f64(w16.view(np.uint16),
+                                        oracle.rmsnorm(hidden[:, :d_model], norm_w, 1e-6))
     for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.9, 0), (1.1, 1.0, 0)]:
         h = make_head(host, vocab, 0, cap)
         opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 0)
