@@ -559,6 +559,133 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__res
     }
 }
 
+/* The same projection for 5 to 16 activation rows on the double-precision matrix cores. A
+ * wavefront owns 64 weight rows (four tiles of 16) against up to 16 activation rows; one
+ * v_mfma_f64_16x16x4 adds four columns to a 16 x 16 tile: A = activations [m][k], B = weights
+ * [k][row], lane l holds A[l % 16][l / 16] and B[l / 16][l % 16], and of the result the rows
+ * l / 16, 4 + l / 16, 8 + l / 16, 12 + l / 16 of column l % 16. Within a stage of 64 columns instruction t takes
+ * the columns t, 16 + t, 32 + t, 48 + t, so that a lane converts 16 consecutive weights of its
+ * row and reads 16 consecutive activations. The order inside a stage is therefore not the
+ * reference's either; the bound and the list are those of the vector kernel (partial sums are
+ * sampled at the stage boundaries, where all earlier columns have been added; the room for the
+ * error is doubled for the matrix cores' internal additions). */
+typedef double mfma_d4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_mfma(
+    const uint16_t *__restrict__ w, long n_out, int n_in, const double *__restrict__ xd,
+    const double *__restrict__ xs, int n_m, float *__restrict__ y, long ld_y,
+    int *__restrict__ amb_count, int2 *__restrict__ amb_list) {
+    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
+    const int  lane = threadIdx.x & (LM_WAVE - 1);
+    const int  wave = __builtin_amdgcn_readfirstlane(threadIdx.x / LM_WAVE);
+    const long row0 = (long) blockIdx.x * ROWS_BLOCK_B + wave * ROWS_WAVE_B;
+    if (row0 >= n_out)
+        return;
+    uint8_t  *tile = s_tile[wave];
+    const int j = lane & 15, kq = lane >> 4;
+    /* this lane's activation row as the A operand; rows beyond n_m contribute zeros */
+    const double *xa_row = xd + (long) (j < n_m ? j : 0) * n_in;
+    const bool    xa_on  = j < n_m;
+
+    mfma_d4 acc[4];
+    double  pmax[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        acc[t] = mfma_d4{0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            pmax[t][r] = 0.0;
+    }
+    const int  n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
+    StageRegsB g0, g1;
+    stage_load_b(w, row0, n_out, n_in, 0, lane, g0);
+    if (n_stage > 1)
+        stage_load_b(w, row0, n_out, n_in, 1, lane, g1);
+    for (int s = 0; s < n_stage; ++s) {
+        const int col0 = s * STAGE_COLS;
+        /* activations of the stage: columns col0 + 16 kq .. + 15 of row j */
+        double xa[16];
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int c = col0 + 16 * kq + t;
+            xa[t]       = (xa_on && c < n_in) ? xa_row[c] : 0.0;
+        }
+        double xst[4]; /* ||x_stage|| of the four activation rows this lane holds results of */
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = 4 * r + kq;
+            xst[r]      = xs[(long) (m < n_m ? m : n_m - 1) * n_stage + s];
+        }
+#pragma unroll
+        for (int i = 0; i < STAGE_LOADS_B; ++i)
+            *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH + (lane & 7) * 16) =
+                g0.w[i];
+        g0 = g1;
+        if (s + 2 < n_stage)
+            stage_load_b(w, row0, n_out, n_in, s + 2, lane, g1);
+        /* the four tiles' instructions interleaved: consecutive ones do not wait for each other */
+        uint32_t u[4][8];
+        double   p0[4][4];
+        float    w2[4];
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            const uint8_t *src = tile + (16 * tl + j) * TILE_PITCH + kq * 32;
+            const uint4    qa  = *reinterpret_cast<const uint4 *>(src);
+            const uint4    qb  = *reinterpret_cast<const uint4 *>(src + 16);
+            u[tl][0] = qa.x, u[tl][1] = qa.y, u[tl][2] = qa.z, u[tl][3] = qa.w;
+            u[tl][4] = qb.x, u[tl][5] = qb.y, u[tl][6] = qb.z, u[tl][7] = qb.w;
+            w2[tl] = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                p0[tl][r] = fabs(acc[tl][r]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
+                w2[tl]         = __builtin_fmaf(f.x, f.x, w2[tl]);
+                w2[tl]         = __builtin_fmaf(f.y, f.y, w2[tl]);
+                acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i], (double) f.x, acc[tl], 0, 0, 0);
+            }
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
+                acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i + 1], (double) f.y, acc[tl], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            /* ||w_stage|| of row j: the four lanes j, j + 16, j + 32, j + 48 hold a quarter each */
+            float ws2 = w2[tl];
+            ws2 += __shfl_xor(ws2, 16, LM_WAVE);
+            ws2 += __shfl_xor(ws2, 32, LM_WAVE);
+            const double wn = (double) __builtin_sqrtf(ws2) * (1.0 + 1e-4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const double p = p0[tl][r] + wn * xst[r];
+                pmax[tl][r]    = p > pmax[tl][r] ? p : pmax[tl][r];
+            }
+        }
+    }
+#pragma unroll
+    for (int tl = 0; tl < 4; ++tl) {
+        const long row = row0 + 16 * tl + j;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = 4 * r + kq;
+            if (row >= n_out || m >= n_m)
+                continue;
+            const double sum = acc[tl][r];
+            const double err = (double) n_in * 0x1p-51 * 1.01 * pmax[tl][r];
+            float        f;
+            if (!f32_rounding_is_safe(sum, err, f))
+                amb_list[atomicAdd(amb_count, 1)] = make_int2((int) row, m);
+            y[m * ld_y + row] = f;
+        }
+    }
+}
+
 /* The listed outputs once more, in the reference's order: a lane per output (weight row r,
  * activation row m), a wavefront streams its 64 weight rows through its LDS tile as above and
  * every lane adds its row's products one after the other. The activations of a stage lie in LDS
@@ -568,7 +695,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
     float *__restrict__ y, long ld_y, const int *__restrict__ amb_count,
     const int2 *__restrict__ amb_list) {
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
-    __shared__ double                s_x[LM_WAVES][GEMV_M_MAX][STAGE_COLS];
+    __shared__ double                s_x[LM_WAVES][F64_M_MAX][STAGE_COLS];
     const int lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
     const int count = *amb_count;
     uint8_t  *tile  = s_tile[wave];
@@ -593,14 +720,14 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
                     g.w[i] = *reinterpret_cast<const uint4 *>(w + fetch_row[i] * n_in + col);
             }
         };
-        auto fetch_x = [&](int s, double (&xr)[GEMV_M_MAX]) {
+        auto fetch_x = [&](int s, double (&xr)[F64_M_MAX]) {
             const int k = s * STAGE_COLS + lane;
 #pragma unroll
-            for (int m = 0; m < GEMV_M_MAX; ++m)
+            for (int m = 0; m < F64_M_MAX; ++m)
                 xr[m] = (m < n_m && k < n_in) ? xd[(long) m * n_in + k] : 0.0;
         };
         StageRegsB g0, g1;
-        double     x0[GEMV_M_MAX];
+        double     x0[F64_M_MAX];
         fetch_w(0, g0);
         fetch_x(0, x0);
         if (n_stage > 1)
@@ -613,7 +740,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
                 *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH +
                                            (lane & 7) * 16) = g0.w[i];
 #pragma unroll
-            for (int m = 0; m < GEMV_M_MAX; ++m)
+            for (int m = 0; m < F64_M_MAX; ++m)
                 s_x[wave][m][lane] = x0[m];
             g0 = g1;
             if (s + 2 < n_stage)
@@ -700,8 +827,8 @@ void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out
         k_f16_linear_f64<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else if (n_m <= 4)
         k_f16_linear_f64<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    else
-        k_f16_linear_f64<8><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else /* 5 .. F64_M_MAX rows: one matrix-core tile of activation rows */
+        k_f16_linear_f64_mfma<<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     /* normally a few dozen outputs: one wavefront's worth; the grid strides over longer lists */
     k_f16_linear_f64_listed<<<dim3(64), block, 0, stream>>>(w_f16, n_in, ws.xd, n_m, y, ld_y,
                                                            ws.amb_count, ws.amb_list);

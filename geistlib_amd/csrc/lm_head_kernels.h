@@ -12,6 +12,7 @@
 namespace gs {
 
 constexpr int GEMV_M_MAX = 8; /* activation rows one pass over the weights serves */
+constexpr int F64_M_MAX  = 16; /* ... in the double-accumulation projection (a matrix-core tile) */
 
 /* y = x * w * rsqrt(mean(x^2) + eps) per row; y may alias x. */
 void launch_rmsnorm_rows(hipStream_t stream, const float *x, long ld_x, const float *w, float eps,
@@ -37,15 +38,15 @@ void launch_f16_gemv(hipStream_t stream, const uint16_t *w_f16, long n_out, int 
                      const float *x, long ld_x, int n_m, float *y, long ld_y,
                      const GemvFuse *fuse = nullptr);
 
-/* Scratch of the double-accumulation projection, for one pass of up to GEMV_M_MAX rows. */
+/* Scratch of the double-accumulation projection, for one pass of up to F64_M_MAX rows. */
 struct F64Scratch {
-    double *xd;        /* [GEMV_M_MAX][n_in] the activations in double */
-    double *xs;        /* [GEMV_M_MAX][ceil(n_in / 64)] their norms per stage of 64 columns */
+    double *xd;        /* [F64_M_MAX][n_in] the activations in double */
+    double *xs;        /* [F64_M_MAX][ceil(n_in / 64)] their norms per stage of 64 columns */
     int    *amb_count; /* outputs whose rounding depends on the order of the sum ... */
-    int2   *amb_list;  /* ... [n_out * GEMV_M_MAX] (weight row, activation row) */
+    int2   *amb_list;  /* ... [n_out * F64_M_MAX] (weight row, activation row) */
 };
 /* The portable kernel (cpu_scalar_w_quant_mN for F16): y[m][r] = (float) sum_i (double) x[m][i] *
- * (double) f16(W[r][i]), the sum as if in index order; n_m <= GEMV_M_MAX, n_in a multiple of 8. */
+ * (double) f16(W[r][i]), the sum as if in index order; n_m <= F64_M_MAX, n_in a multiple of 8. */
 void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out, int n_in,
                            const float *x, long ld_x, int n_m, const F64Scratch &ws, float *y,
                            long ld_y);

@@ -621,16 +621,16 @@ static int f64_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, F64Scrat
         }
         const size_t in = n_in > s->f64_in ? n_in : s->f64_in;
         const size_t out = n_out > s->f64_out ? n_out : s->f64_out;
-        const size_t bytes = (size_t) GEMV_M_MAX * (in + in / 64 + 2) * sizeof(double) + 16 +
-                             out * GEMV_M_MAX * sizeof(int2);
+        const size_t bytes = (size_t) F64_M_MAX * (in + in / 64 + 2) * sizeof(double) + 16 +
+                             out * F64_M_MAX * sizeof(int2);
         if (hipMalloc(&s->f64_ws, bytes) != hipSuccess)
             return fail(s, GEIST_HIP_E_OOM, "f64 projection: scratch");
         s->f64_in = in, s->f64_out = out;
     }
     char *p      = static_cast<char *>(s->f64_ws);
     ws.xd        = reinterpret_cast<double *>(p);
-    ws.xs        = ws.xd + (size_t) GEMV_M_MAX * s->f64_in;
-    ws.amb_count = reinterpret_cast<int *>(ws.xs + (size_t) GEMV_M_MAX * (s->f64_in / 64 + 2));
+    ws.xs        = ws.xd + (size_t) F64_M_MAX * s->f64_in;
+    ws.amb_count = reinterpret_cast<int *>(ws.xs + (size_t) F64_M_MAX * (s->f64_in / 64 + 2));
     ws.amb_list  = reinterpret_cast<int2 *>(reinterpret_cast<char *>(ws.amb_count) + 16);
     return GEIST_HIP_OK;
 }
@@ -641,8 +641,8 @@ static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t
     const int  rc = f64_scratch(s, n_out, n_in, ws);
     if (rc)
         return rc;
-    for (size_t m0 = 0; m0 < n_rows; m0 += GEMV_M_MAX) {
-        const size_t m = n_rows - m0 < (size_t) GEMV_M_MAX ? n_rows - m0 : (size_t) GEMV_M_MAX;
+    for (size_t m0 = 0; m0 < n_rows; m0 += F64_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) F64_M_MAX ? n_rows - m0 : (size_t) F64_M_MAX;
         launch_f16_linear_f64(s->stream, d_w_f16, (long) n_out, (int) n_in, d_x + m0 * ld_x,
                               (long) ld_x, (int) m, ws, d_y + m0 * ld_y, (long) ld_y);
     }
