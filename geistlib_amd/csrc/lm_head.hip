@@ -571,7 +571,7 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__res
  * error is doubled for the matrix cores' internal additions). */
 typedef double mfma_d4 __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_mfma(
+__global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     const uint16_t *__restrict__ w, long n_out, int n_in, const double *__restrict__ xd,
     const double *__restrict__ xs, int n_m, float *__restrict__ y, long ld_y,
     int *__restrict__ amb_count, int2 *__restrict__ amb_list) {
@@ -625,7 +625,6 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_mfma(
             stage_load_b(w, row0, n_out, n_in, s + 2, lane, g1);
         /* the four tiles' instructions interleaved: consecutive ones do not wait for each other */
         uint32_t u[4][8];
-        double   p0[4][4];
         float    w2[4];
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl) {
@@ -635,9 +634,6 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_mfma(
             u[tl][0] = qa.x, u[tl][1] = qa.y, u[tl][2] = qa.z, u[tl][3] = qa.w;
             u[tl][4] = qb.x, u[tl][5] = qb.y, u[tl][6] = qb.z, u[tl][7] = qb.w;
             w2[tl] = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                p0[tl][r] = fabs(acc[tl][r]);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -663,7 +659,9 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_mfma(
             const double wn = (double) __builtin_sqrtf(ws2) * (1.0 + 1e-4);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const double p = p0[tl][r] + wn * xst[r];
+                /* (a partial sum inside the stage differs from the one at its end by at most
+                 * the stage's ||w|| ||x||, as from the one at its start) */
+                const double p = fabs(acc[tl][r]) + wn * xst[r];
                 pmax[tl][r]    = p > pmax[tl][r] ? p : pmax[tl][r];
             }
         }
