@@ -693,7 +693,9 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
     float *__restrict__ y, long ld_y, const int *__restrict__ amb_count,
     const int2 *__restrict__ amb_list) {
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
-    __shared__ double                s_x[LM_WAVES][F64_M_MAX][STAGE_COLS];
+    /* (rows two doubles apart in the banks: lanes of different activation rows read the same
+     * column without conflict) */
+    __shared__ double                s_x[LM_WAVES][F64_M_MAX][STAGE_COLS + 2];
     const int lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
     const int count = *amb_count;
     uint8_t  *tile  = s_tile[wave];
