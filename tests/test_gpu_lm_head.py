@@ -296,3 +296,34 @@ def test_f16_linear_in_double_bit_exact(hs, oracle, n_out, n_in, m):
     want = oracle.f16_linear_f64(w16.view(np.uint16), x)
     got = y.cpu().numpy()
     assert (bits(got) == bits(want)).all(), np.argwhere(bits(got) != bits(want))[:5]
+
+
+@pytest.mark.parametrize("m", [1, 3, 7])
+def test_f16_linear_in_double_at_the_ends_of_the_range(hs, oracle, m):
+    """Sums that overflow binary32, sums in its subnormal range, zero rows, weights that are
+    binary16 subnormals and infinities: the vector kernels (m <= 4) and the matrix-core kernel
+    agree with the oracle in every bit (NaN where it has NaN)."""
+    g = np.random.default_rng(m)
+    n_out, n_in = 700, 512
+    w16 = (g.standard_normal((n_out, n_in)) * 0.05).astype(np.float16)
+    w16[0] = 0
+    w16[1] = np.float16(6.0e-8)                       # the smallest binary16 subnormals
+    w16[2] = np.float16(65504.0)                      # the largest binary16
+    w16[3, 5] = np.float16(np.inf)
+    w16[4, 7] = np.float16(-np.inf)
+    w16[4, 9] = np.float16(np.inf)                    # inf - inf
+    x = (g.standard_normal((m, n_in)) * 3).astype(np.float32)
+    x[0] = np.float32(1.0e-38)                        # subnormal results against rows of 0.05
+    if m > 1:
+        x[1] = np.float32(3.0e38)                     # overflows against every row of one sign
+        x[1, ::2] *= -1
+        x[1, :4] = np.float32(3.0e38)
+    y = torch.full((m, n_out), 7.0, dtype=torch.float32, device="cuda")
+    hs.f16_linear(to_dev(w16.view(np.int16), torch), to_dev(x, torch), y)
+    hs.sync()
+    want = oracle.f16_linear_f64(w16.view(np.uint16), x)
+    got = y.cpu().numpy()
+    nan = np.isnan(want)
+    assert (np.isnan(got) == nan).all()
+    assert (bits(got)[~nan] == bits(want)[~nan]).all(), np.argwhere(bits(got) != bits(want))[:5]
+    assert np.isinf(want).any() and nan.any() and (np.abs(want[0, 5:]) < 1.2e-38).any()
