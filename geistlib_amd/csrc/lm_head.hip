@@ -576,16 +576,30 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     const double *__restrict__ xs, int n_m, float *__restrict__ y, long ld_y,
     int *__restrict__ amb_count, int2 *__restrict__ amb_list) {
     __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
+    /* the activations of a stage, for the whole workgroup, two stages alternating (rows two
+     * doubles apart in the banks) */
+    __shared__ __align__(16) double s_xa[2][F64_M_MAX][STAGE_COLS + 2];
     const int  lane = threadIdx.x & (LM_WAVE - 1);
     const int  wave = __builtin_amdgcn_readfirstlane(threadIdx.x / LM_WAVE);
     const long row0 = (long) blockIdx.x * ROWS_BLOCK_B + wave * ROWS_WAVE_B;
-    if (row0 >= n_out)
-        return;
+    /* (a wavefront without rows stays for the workgroup's barriers; its loads are masked) */
     uint8_t  *tile = s_tile[wave];
     const int j = lane & 15, kq = lane >> 4;
-    /* this lane's activation row as the A operand; rows beyond n_m contribute zeros */
-    const double *xa_row = xd + (long) (j < n_m ? j : 0) * n_in;
-    const bool    xa_on  = j < n_m;
+    /* this thread's share of a stage's activations: four columns of row tid / 16 */
+    const int     xl_row = (int) threadIdx.x >> 4, xl_col = ((int) threadIdx.x & 15) * 4;
+    const double *xl_src = xd + (long) (xl_row < n_m ? xl_row : 0) * n_in + xl_col;
+    auto load_x = [&](int s, double (&xr)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = s * STAGE_COLS + xl_col + q;
+            xr[q]       = (xl_row < n_m && c < n_in) ? xl_src[s * STAGE_COLS + q] : 0.0;
+        }
+    };
+    auto store_x = [&](int buf, const double (&xr)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            s_xa[buf][xl_row][xl_col + q] = xr[q];
+    };
 
     mfma_d4 acc[4];
     double  pmax[4][4];
@@ -601,15 +615,22 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     stage_load_b(w, row0, n_out, n_in, 0, lane, g0);
     if (n_stage > 1)
         stage_load_b(w, row0, n_out, n_in, 1, lane, g1);
+    {
+        double xr[4];
+        load_x(0, xr);
+        store_x(0, xr);
+    }
+    __syncthreads();
     for (int s = 0; s < n_stage; ++s) {
-        const int col0 = s * STAGE_COLS;
-        /* activations of the stage: columns col0 + 16 kq .. + 15 of row j */
+        /* the next stage's activations are requested now and stored at the end of this stage */
+        double xnext[4];
+        if (s + 1 < n_stage)
+            load_x(s + 1, xnext);
+        /* activations of the stage: columns 16 kq .. 16 kq + 15 of row j */
         double xa[16];
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            const int c = col0 + 16 * kq + t;
-            xa[t]       = (xa_on && c < n_in) ? xa_row[c] : 0.0;
-        }
+        for (int t = 0; t < 16; ++t)
+            xa[t] = s_xa[s & 1][j][16 * kq + t];
         double xst[4]; /* ||x_stage|| of the four activation rows this lane holds results of */
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -665,6 +686,9 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
                 pmax[tl][r]    = p > pmax[tl][r] ? p : pmax[tl][r];
             }
         }
+        if (s + 1 < n_stage)
+            store_x((s + 1) & 1, xnext);
+        __syncthreads();
     }
 #pragma unroll
     for (int tl = 0; tl < 4; ++tl) {
