@@ -327,3 +327,21 @@ def test_f16_linear_in_double_at_the_ends_of_the_range(hs, oracle, m):
     assert (np.isnan(got) == nan).all()
     assert (bits(got)[~nan] == bits(want)[~nan]).all(), np.argwhere(bits(got) != bits(want))[:5]
     assert np.isinf(want).any() and nan.any() and (np.abs(want[0, 5:]) < 1.2e-38).any()
+
+
+@pytest.mark.parametrize("m", [2, 9, 19])
+def test_f16_linear_in_double_with_row_strides(hs, oracle, m):
+    """Padded rows on both sides (row strides above the row lengths), 19 rows in two passes of the
+    matrix-core kernel; the padding of the output is left alone."""
+    g = np.random.default_rng(40 + m)
+    n_out, n_in = 3000, 1536
+    w16 = (g.standard_normal((n_out, n_in)) * 0.05).astype(np.float16)
+    xbuf = (g.standard_normal((m, n_in + 24)) * 2).astype(np.float32)
+    d_x = to_dev(xbuf, torch)
+    y = torch.full((m, n_out + 8), 7.0, dtype=torch.float32, device="cuda")
+    hs.f16_linear(to_dev(w16.view(np.int16), torch), d_x[:, :n_in], y[:, :n_out])
+    hs.sync()
+    got = y.cpu().numpy()
+    want = oracle.f16_linear_f64(w16.view(np.uint16), xbuf[:, :n_in])
+    assert (bits(got[:, :n_out]) == bits(want)).all()
+    assert (got[:, n_out:] == 7.0).all()
