@@ -78,6 +78,7 @@ def load_library():
     lib.geist_hip_sampler_sync.argtypes = [vp]
     lib.geist_hip_sampler_set_stream.argtypes = [vp, vp]
     lib.geist_hip_sampler_set_logits_hint.argtypes = [vp, i32]
+    lib.geist_hip_sampler_set_projection.argtypes = [vp, i32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -252,6 +253,10 @@ class HipSampler:
         self._check(self.lib.geist_hip_f16_gemv_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
+
+    def set_projection(self, portable):
+        """Which reference backend project_sample's F16 projection stands for (False: x86)."""
+        self._check(self.lib.geist_hip_sampler_set_projection(self.h, 1 if portable else 0))
 
     def f16_linear(self, w_f16, x, y):
         """As f16_gemv in the portable kernel's arithmetic: the sum in double, rounded once."""

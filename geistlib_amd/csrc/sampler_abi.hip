@@ -50,6 +50,7 @@ struct geist_hip_sampler {
 
     bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
+    bool projection_portable = false; /* see geist_hip_sampler_set_projection */
     bool tmax_ready         = false; /* the projection has written the top-k scan's thread maxima
                                         for the rows about to be sampled */
 
@@ -249,6 +250,15 @@ int geist_hip_sampler_set_logits_hint(geist_hip_sampler *s, int hint) {
     if (hint != GEIST_HIP_LOGITS_CACHED && hint != GEIST_HIP_LOGITS_STREAMED)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown logits hint %d", hint);
     s->logits_streamed = hint == GEIST_HIP_LOGITS_STREAMED;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_set_projection(geist_hip_sampler *s, int mode) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (mode != GEIST_HIP_PROJECTION_X86 && mode != GEIST_HIP_PROJECTION_PORTABLE)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown projection mode %d", mode);
+    s->projection_portable = mode == GEIST_HIP_PROJECTION_PORTABLE;
     return GEIST_HIP_OK;
 }
 
@@ -736,7 +746,8 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     if (!rs.greedy && !d_uniforms && !d_rng_states)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic configuration without draws");
     HIPCHK(s, hipSetDevice(s->device));
-    const bool fuse_ok = f16_gemv_can_fuse((int) rows) && (q8 || rows == 1);
+    const bool f64     = !q8 && (rows > 1 || s->projection_portable);
+    const bool fuse_ok = f16_gemv_can_fuse((int) rows) && !f64;
     /* the top-k path's scan is the projection's epilogue when nothing changes the logits
      * between the two (no soft-cap) */
     const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX &&
@@ -755,9 +766,9 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
-    } else if (!q8 && rows > 1) {
+    } else if (f64) {
         /* more than one row: the reference's batch kernel (cpu_scalar_w_quant_mN), its x86
-         * kernels being decode-only */
+         * kernels being decode-only; or the portable backend asked for */
         rc = f16_linear_impl(s, d_embed_f16, n_vocab, d_model, d_normed, d_model, rows, d_logits,
                              ld_logits);
         if (rc)

@@ -219,6 +219,14 @@ static int project_finalize(struct geist_hip_head *h, const float *d_hidden, siz
     return GEIST_HIP_OK;
 }
 
+int geist_hip_head_set_projection(struct geist_hip_head *h, int mode) {
+    if (h == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (geist_hip_sampler_set_projection(h->hs, mode) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "projection mode");
+    return GEIST_HIP_OK;
+}
+
 int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hidden,
                                     size_t ld_hidden, size_t k, const float *d_norm_weight,
                                     float rms_eps, const uint16_t *d_embed_f16, size_t d_model,

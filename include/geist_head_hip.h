@@ -85,6 +85,9 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
                                     size_t ld_hidden, size_t k, const float *d_norm_weight,
                                     float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
                                     int32_t *out_tokens);
+/* GEIST_HIP_PROJECTION_X86 (default) or _PORTABLE (include/geist_lm_head_hip.h): which backend's
+ * arithmetic geist_hip_head_project_finalize uses for one row. */
+int geist_hip_head_set_projection(struct geist_hip_head *h, int mode);
 /* The same over the int8 form of the table, which the reference's x86 backend substitutes for
  * the F16 table in a decode step (src/backends/cpu_x86/backend.c:332-372): d_embed_q8 [vocab,
  * d_model] int8 and d_scales [vocab] as geist_hip_f16_to_q8w produces them, d_model a multiple

@@ -48,6 +48,16 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
                               size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                               float *d_y, size_t ld_y);
 
+/* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
+ * the head's project_finalize calls) stands for:
+ *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1; more rows: the portable kernel (default)
+ *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
+ *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
+ *                                  linear_m1 and linear_mN alike) */
+#define GEIST_HIP_PROJECTION_X86 0
+#define GEIST_HIP_PROJECTION_PORTABLE 1
+int geist_hip_sampler_set_projection(geist_hip_sampler *s, int mode);
+
 /* The int8 form of the tied table, which the reference's x86 backend uses for the lm_head unless
  * GEIST_Q8_LMHEAD=0 (src/backends/cpu_x86/backend.c:344-372): half the bytes per decode step.
  *

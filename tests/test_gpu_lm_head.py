@@ -345,3 +345,33 @@ def test_f16_linear_in_double_with_row_strides(hs, oracle, m):
     want = oracle.f16_linear_f64(w16.view(np.uint16), xbuf[:, :n_in])
     assert (bits(got[:, :n_out]) == bits(want)).all()
     assert (got[:, n_out:] == 7.0).all()
+
+
+def test_project_sample_rows_in_the_portable_backends_arithmetic(hs, oracle):
+    """geist_hip_sampler_set_projection(PORTABLE): one row goes through the double-accumulation
+    kernel too, as on the reference's cpu_scalar backend."""
+    from geistlib_amd import SampleParams
+    g = np.random.default_rng(61)
+    vocab, d_model = 30000, 1536
+    w16 = (g.standard_normal((vocab, d_model)) * 0.05).astype(np.float16).view(np.uint16)
+    hidden = (g.standard_normal((1, d_model)) * 3).astype(np.float32)
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    u = g.random(1).astype(np.float32)
+    normed_want = oracle.rmsnorm(hidden, norm_w, 1e-6)
+    logits = torch.empty((1, vocab), dtype=torch.float32, device="cuda")
+    out = torch.empty(1, dtype=torch.int32, device="cuda")
+    args = (to_dev(hidden, torch), to_dev(norm_w, torch), 1e-6, to_dev(w16.view(np.int16), torch),
+            logits, SampleParams.make(temperature=0.8, top_k=40), to_dev(u, torch), out)
+    normed = torch.empty((1, d_model), dtype=torch.float32, device="cuda")
+    try:
+        hs.set_projection(True)
+        hs.project_sample(*args, normed=normed)
+        hs.sync()
+        want = oracle.f16_linear_f64(w16, normed_want)
+        assert (bits(logits.cpu().numpy()) == bits(want)).all()
+        assert out.cpu().tolist() == [oracle.top_k_u(want[0], 40, 0.8, float(u[0]))[0]]
+    finally:
+        hs.set_projection(False)
+    hs.project_sample(*args, normed=normed)
+    hs.sync()
+    assert (bits(logits.cpu().numpy()) == bits(oracle.f16_gemv(w16, normed_want))).all()
