@@ -568,9 +568,15 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__res
  * row and reads 16 consecutive activations. The order inside a stage is therefore not the
  * reference's either; the bound and the list are those of the vector kernel (partial sums are
  * sampled at the stage boundaries, where all earlier columns have been added; the room for the
- * error is doubled for the matrix cores' internal additions). */
+ * error is doubled for the matrix cores' internal additions).
+ * SMALL (2 to 4 activation rows): v_mfma_f64_4x4x4 instead, four independent 4 x 4 x 4 blocks per
+ * instruction. Lane l holds A[l % 4][l / 16] of block (l / 4) % 4 -- the activations, the same
+ * in every block --, B[l / 16][l % 4] of that block -- weight row l % 16 of the tile, as above --
+ * and the result of activation row l / 16 and weight row l % 16. A quarter of the arithmetic
+ * for the same pass over the weights. */
 typedef double mfma_d4 __attribute__((ext_vector_type(4)));
 
+template <bool SMALL>
 __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     const uint16_t *__restrict__ w, long n_out, int n_in, const double *__restrict__ xd,
     const double *__restrict__ xs, int n_m, float *__restrict__ y, long ld_y,
@@ -601,13 +607,17 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
             s_xa[buf][xl_row][xl_col + q] = xr[q];
     };
 
+    /* results per lane and tile: rows 4 r + kq of the 16 x 16 tile, or row kq of the four
+     * 4 x 4 blocks */
+    constexpr int NR = SMALL ? 1 : 4;
+    const int     ja = SMALL ? (lane & 3) : j; /* the activation row this lane feeds as A */
     mfma_d4 acc[4];
-    double  pmax[4][4];
+    double  pmax[4][NR];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         acc[t] = mfma_d4{0.0, 0.0, 0.0, 0.0};
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < NR; ++r)
             pmax[t][r] = 0.0;
     }
     const int  n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
@@ -630,11 +640,11 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
         double xa[16];
 #pragma unroll
         for (int t = 0; t < 16; ++t)
-            xa[t] = s_xa[s & 1][j][16 * kq + t];
-        double xst[4]; /* ||x_stage|| of the four activation rows this lane holds results of */
+            xa[t] = s_xa[s & 1][ja][16 * kq + t];
+        double xst[NR]; /* ||x_stage|| of the activation rows this lane holds results of */
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = 4 * r + kq;
+        for (int r = 0; r < NR; ++r) {
+            const int m = SMALL ? kq : 4 * r + kq;
             xst[r]      = xs[(long) (m < n_m ? m : n_m - 1) * n_stage + s];
         }
 #pragma unroll
@@ -663,12 +673,18 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
                 const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
                 w2[tl]         = __builtin_fmaf(f.x, f.x, w2[tl]);
                 w2[tl]         = __builtin_fmaf(f.y, f.y, w2[tl]);
-                acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i], (double) f.x, acc[tl], 0, 0, 0);
+                if (SMALL)
+                    acc[tl][0] = __builtin_amdgcn_mfma_f64_4x4x4f64(xa[2 * i], (double) f.x, acc[tl][0], 0, 0, 0);
+                else
+                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i], (double) f.x, acc[tl], 0, 0, 0);
             }
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
                 const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
-                acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i + 1], (double) f.y, acc[tl], 0, 0, 0);
+                if (SMALL)
+                    acc[tl][0] = __builtin_amdgcn_mfma_f64_4x4x4f64(xa[2 * i + 1], (double) f.y, acc[tl][0], 0, 0, 0);
+                else
+                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i + 1], (double) f.y, acc[tl], 0, 0, 0);
             }
         }
 #pragma unroll
@@ -679,7 +695,7 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
             ws2 += __shfl_xor(ws2, 32, LM_WAVE);
             const double wn = (double) __builtin_sqrtf(ws2) * (1.0 + 1e-4);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int r = 0; r < NR; ++r) {
                 /* (a partial sum inside the stage differs from the one at its end by at most
                  * the stage's ||w|| ||x||, as from the one at its start) */
                 const double p = fabs(acc[tl][r]) + wn * xst[r];
@@ -694,8 +710,8 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     for (int tl = 0; tl < 4; ++tl) {
         const long row = row0 + 16 * tl + j;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = 4 * r + kq;
+        for (int r = 0; r < NR; ++r) {
+            const int m = SMALL ? kq : 4 * r + kq;
             if (row >= n_out || m >= n_m)
                 continue;
             const double sum = acc[tl][r];
@@ -847,12 +863,10 @@ void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out
     k_x_to_f64<<<dim3(n_m), block, 0, stream>>>(x, ld_x, n_in, ws.xd, ws.xs, ws.amb_count);
     if (n_m <= 1)
         k_f16_linear_f64<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    else if (n_m <= 2)
-        k_f16_linear_f64<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    else if (n_m <= 4)
-        k_f16_linear_f64<4><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    else /* 5 .. F64_M_MAX rows: one matrix-core tile of activation rows */
-        k_f16_linear_f64_mfma<<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else if (n_m <= 4) /* four 4 x 4 x 4 blocks per matrix-core instruction */
+        k_f16_linear_f64_mfma<true><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else /* 5 .. F64_M_MAX rows: one 16 x 16 tile of activation rows */
+        k_f16_linear_f64_mfma<false><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     /* normally a few dozen outputs: one wavefront's worth; the grid strides over longer lists */
     k_f16_linear_f64_listed<<<dim3(64), block, 0, stream>>>(w_f16, n_in, ws.xd, n_m, y, ld_y,
                                                            ws.amb_count, ws.amb_list);
