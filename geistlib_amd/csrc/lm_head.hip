@@ -569,14 +569,14 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64(const uint16_t *__res
  * reference's either; the bound and the list are those of the vector kernel (partial sums are
  * sampled at the stage boundaries, where all earlier columns have been added; the room for the
  * error is doubled for the matrix cores' internal additions).
- * SMALL (2 to 4 activation rows): v_mfma_f64_4x4x4 instead, four independent 4 x 4 x 4 blocks per
- * instruction. Lane l holds A[l % 4][l / 16] of block (l / 4) % 4 -- the activations, the same
+ * NS > 0 (2 to 12 activation rows): v_mfma_f64_4x4x4 instead, four independent 4 x 4 x 4 blocks
+ * per instruction, NS instructions for NS sets of four activation rows. Lane l holds A[l % 4][l / 16] of block (l / 4) % 4 -- the activations, the same
  * in every block --, B[l / 16][l % 4] of that block -- weight row l % 16 of the tile, as above --
- * and the result of activation row l / 16 and weight row l % 16. A quarter of the arithmetic
- * for the same pass over the weights. */
+ * and the result of activation row l / 16 (of its set) and weight row l % 16. A quarter of the
+ * arithmetic per set for the same pass over the weights. */
 typedef double mfma_d4 __attribute__((ext_vector_type(4)));
 
-template <bool SMALL>
+template <int NS>
 __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     const uint16_t *__restrict__ w, long n_out, int n_in, const double *__restrict__ xd,
     const double *__restrict__ xs, int n_m, float *__restrict__ y, long ld_y,
@@ -607,10 +607,12 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
             s_xa[buf][xl_row][xl_col + q] = xr[q];
     };
 
-    /* results per lane and tile: rows 4 r + kq of the 16 x 16 tile, or row kq of the four
-     * 4 x 4 blocks */
-    constexpr int NR = SMALL ? 1 : 4;
-    const int     ja = SMALL ? (lane & 3) : j; /* the activation row this lane feeds as A */
+    /* NS == 0: one 16 x 16 x 4 instruction per four columns; NS > 0: NS instructions of four
+     * 4 x 4 x 4 blocks, set q for the activation rows 4 q .. 4 q + 3. Either way a lane holds,
+     * per tile of 16 weight rows, the results of the activation rows 4 r + kq. */
+    constexpr bool SMALL = NS > 0;
+    constexpr int  NR = SMALL ? NS : 4, NA = SMALL ? NS : 1;
+    const int      ja = SMALL ? (lane & 3) : j; /* the activation row this lane feeds as A (+ 4 q) */
     mfma_d4 acc[4];
     double  pmax[4][NR];
 #pragma unroll
@@ -636,15 +638,11 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
         double xnext[4];
         if (s + 1 < n_stage)
             load_x(s + 1, xnext);
-        /* activations of the stage: columns 16 kq .. 16 kq + 15 of row j */
-        double xa[16];
-#pragma unroll
-        for (int t = 0; t < 16; ++t)
-            xa[t] = s_xa[s & 1][ja][16 * kq + t];
+        /* (activations of the stage: columns 16 kq .. 16 kq + 15 of row ja + 4 q, read below) */
         double xst[NR]; /* ||x_stage|| of the activation rows this lane holds results of */
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
-            const int m = SMALL ? kq : 4 * r + kq;
+            const int m = 4 * r + kq;
             xst[r]      = xs[(long) (m < n_m ? m : n_m - 1) * n_stage + s];
         }
 #pragma unroll
@@ -668,23 +666,35 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
+            double2 xv[NA];
+#pragma unroll
+            for (int q = 0; q < NA; ++q)
+                xv[q] = *reinterpret_cast<const double2 *>(&s_xa[s & 1][ja + 4 * q][16 * kq + 2 * i]);
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
                 const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
                 w2[tl]         = __builtin_fmaf(f.x, f.x, w2[tl]);
                 w2[tl]         = __builtin_fmaf(f.y, f.y, w2[tl]);
-                if (SMALL)
-                    acc[tl][0] = __builtin_amdgcn_mfma_f64_4x4x4f64(xa[2 * i], (double) f.x, acc[tl][0], 0, 0, 0);
-                else
-                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i], (double) f.x, acc[tl], 0, 0, 0);
+                const double wd = (double) f.x;
+                if (SMALL) {
+#pragma unroll
+                    for (int q = 0; q < NA; ++q)
+                        acc[tl][q] = __builtin_amdgcn_mfma_f64_4x4x4f64(xv[q].x, wd, acc[tl][q], 0, 0, 0);
+                } else {
+                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xv[0].x, wd, acc[tl], 0, 0, 0);
+                }
             }
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
                 const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[tl][i]));
-                if (SMALL)
-                    acc[tl][0] = __builtin_amdgcn_mfma_f64_4x4x4f64(xa[2 * i + 1], (double) f.y, acc[tl][0], 0, 0, 0);
-                else
-                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xa[2 * i + 1], (double) f.y, acc[tl], 0, 0, 0);
+                const double wd = (double) f.y;
+                if (SMALL) {
+#pragma unroll
+                    for (int q = 0; q < NA; ++q)
+                        acc[tl][q] = __builtin_amdgcn_mfma_f64_4x4x4f64(xv[q].y, wd, acc[tl][q], 0, 0, 0);
+                } else {
+                    acc[tl] = __builtin_amdgcn_mfma_f64_16x16x4f64(xv[0].y, wd, acc[tl], 0, 0, 0);
+                }
             }
         }
 #pragma unroll
@@ -711,7 +721,7 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
         const long row = row0 + 16 * tl + j;
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
-            const int m = SMALL ? kq : 4 * r + kq;
+            const int m = 4 * r + kq;
             if (row >= n_out || m >= n_m)
                 continue;
             const double sum = acc[tl][r];
@@ -864,9 +874,13 @@ void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out
     if (n_m <= 1)
         k_f16_linear_f64<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else if (n_m <= 4) /* four 4 x 4 x 4 blocks per matrix-core instruction */
-        k_f16_linear_f64_mfma<true><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    else /* 5 .. F64_M_MAX rows: one 16 x 16 tile of activation rows */
-        k_f16_linear_f64_mfma<false><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+        k_f16_linear_f64_mfma<1><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else if (n_m <= 8) /* ... two such instructions, for the rows 0..3 and 4..7 */
+        k_f16_linear_f64_mfma<2><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else if (n_m <= 12)
+        k_f16_linear_f64_mfma<3><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
+    else /* 13 .. F64_M_MAX rows: one 16 x 16 tile of activation rows */
+        k_f16_linear_f64_mfma<0><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     /* normally a few dozen outputs: one wavefront's worth; the grid strides over longer lists */
     k_f16_linear_f64_listed<<<dim3(64), block, 0, stream>>>(w_f16, n_in, ws.xd, n_m, y, ld_y,
                                                            ws.amb_count, ws.amb_list);
