@@ -1115,6 +1115,19 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __syncthreads();
     const double sum = s_sum;
     int          tok = -1;
+    if (sum != sum && !(a.min_p > 0.0f)) {
+        /* A NaN, a +inf or nothing finite in the row: the sum is NaN, the reference neither takes
+         * its argmax branch (sampler.c:243, `sum <= 0` is false) nor finds an end of the nucleus
+         * or a slot for the draw among normalised probabilities that are all NaN, and answers
+         * with the last entry of its sorted array (sampler.c:287-303) -- the last token, its
+         * comparator calling all entries equal and the sort keeping their order. */
+        if (tid == 0) {
+            a.row_flag[row]  = 0;
+            a.out[row]       = rv.n_vocab - 1;
+            a.cand.path[row] = 1;
+        }
+        return;
+    }
     if (a.minp_listed && a.cand.count[row] <= CAND_CAP) {
         /* the exp-sum pass listed the row under the min-p bound (holding p, not pn): the list
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */

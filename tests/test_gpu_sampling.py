@@ -790,3 +790,34 @@ def test_allowed_mask_equals_minus_inf_after_the_transforms(hs, oracle, mode):
         row = np.where(shared[0], x[r], -np.inf).astype(np.float32)
         want = oracle.argmax(row) if mode == "argmax" else oracle.chain_u(row, float(u[r]), **kw)[0]
         assert got[r] == want, (mode, r)
+
+
+@pytest.mark.parametrize("n", [300, 9000, 50257])
+def test_rows_that_are_not_finite_follow_the_reference(hs, oracle, n):
+    """Rows with a NaN, a +inf or nothing finite: the softmax sum is NaN. Temperature and top-p
+    then answer with the last token as the reference does (its loops find no slot; top-p:
+    sampler.c:243 is not taken, 287-303 fall through), the other modes as the oracle."""
+    from geistlib_amd import SampleParams
+    g = np.random.default_rng(n)
+    mods = [lambda x: x.__setitem__(150, np.nan), lambda x: x.__setitem__(0, np.nan),
+            lambda x: x.__setitem__(len(x) - 1, np.nan), lambda x: x.__setitem__(7, np.inf),
+            lambda x: (x.__setitem__(7, np.inf), x.__setitem__(9, np.inf)),
+            lambda x: x.fill(-np.inf), lambda x: x.fill(np.nan)]
+    rows = []
+    for mod in mods:
+        r = g.standard_normal(n).astype(np.float32)
+        mod(r)
+        rows.append(r)
+    x = np.stack(rows)
+    u = g.random(len(rows)).astype(np.float32)
+    for kw in (dict(temperature=1.3, top_k=0, top_p=0.3, min_p=0.0),
+               dict(temperature=1.0, top_k=0, top_p=0.9, min_p=0.05),
+               dict(temperature=1.0, top_k=0, top_p=1.0, min_p=0.05),
+               dict(temperature=1.0, top_k=0, top_p=1.0, min_p=0.0),
+               dict(temperature=1.0, top_k=40, top_p=1.0, min_p=0.0),
+               dict(temperature=0.7, top_k=40, top_p=0.9, min_p=0.0)):
+        want = [oracle.chain_u(x[r], float(u[r]), **kw)[0] for r in range(len(rows))]
+        got = [int(v) for v in run_rows(hs, torch, x, u, SampleParams.make(**kw), None, None)]
+        assert got == want, kw
+        if kw["top_k"] == 0 and kw["min_p"] == 0.0:
+            assert want == [n - 1] * len(rows)

@@ -69,3 +69,39 @@ def test_u_variants_equal_rng_variants(oracle):
         assert oracle.chain_u(row, u, temperature=0.7, top_p=0.9)[0] == oracle.top_p_u(row, 0.9, 0.7, u)[0]
         assert oracle.chain_u(row, u, temperature=0.7, top_k=40)[0] == oracle.top_k_u(row, 40, 0.7, u)[0]
         assert oracle.chain_u(row, u, temperature=0.7)[0] == oracle.temperature_u(row, 0.7, u)[0]
+
+
+NONFINITE_ROWS = [("nan mid", lambda x: x.__setitem__(len(x) // 2, np.nan)),
+                  ("nan first", lambda x: x.__setitem__(0, np.nan)),
+                  ("nan last", lambda x: x.__setitem__(len(x) - 1, np.nan)),
+                  ("+inf", lambda x: x.__setitem__(7 % len(x), np.inf)),
+                  ("all -inf", lambda x: x.fill(-np.inf)),
+                  ("all nan", lambda x: x.fill(np.nan))]
+
+
+@pytest.mark.parametrize("n", [64, 300, 9000])
+def test_rows_that_are_not_finite(oracle, ref, n):
+    """A NaN or +inf in the row, or nothing finite at all: the softmax sum is NaN and the
+    reference's functions fall through their loops (sampler.c:90-102, 243, 287-303). The oracle
+    follows the compiled reference in the temperature and top-p modes, and with top-k where the
+    row holds no NaN; with a NaN among finite values the reference's comparator is inconsistent
+    (sampler.c:166-176 returns 0 against a NaN) and the pick is whatever libc's qsort makes of
+    that: not pinned."""
+    g = np.random.default_rng(n)
+    for desc, mod in NONFINITE_ROWS:
+        row = g.standard_normal(n).astype(np.float32)
+        mod(row)
+        for mode, prm in [("temperature", (0.9,)), ("top_p", (0.3, 1.3)), ("top_p", (0.9, 1.0)),
+                          ("top_k", (40, 0.8))]:
+            if mode == "top_k" and np.isnan(row).any() and not np.isnan(row).all():
+                continue
+            ra, rb = OracleRng(), OracleRng()
+            ref.geist_rng_seed(C.byref(ra), C.c_uint64(5))
+            oracle.lib.oracle_rng_seed(C.byref(rb), C.c_uint64(5))
+            for _ in range(3):
+                want = _ref_call(ref, row, mode, prm, ra)
+                got = _oracle_call(oracle, row, mode, prm, rb)
+                assert got == want, (n, desc, mode, prm)
+            assert ra.state == rb.state
+            if mode != "top_k":
+                assert want == n - 1, (n, desc, mode)
