@@ -75,6 +75,17 @@ static int fail(geist_hip_sampler *s, int code, const char *fmt, ...) {
                         "%s: %s", #call, hipGetErrorString(e_));                               \
     } while (0)
 
+/* Two events for a timed region; neither is left behind when the second cannot be made. */
+static int event_pair(geist_hip_sampler *s, hipEvent_t *a, hipEvent_t *b) {
+    HIPCHK(s, hipEventCreate(a));
+    const hipError_t e = hipEventCreate(b);
+    if (e != hipSuccess) {
+        (void) hipEventDestroy(*a);
+        return fail(s, GEIST_HIP_E_BACKEND, "hipEventCreate: %s", hipGetErrorString(e));
+    }
+    return GEIST_HIP_OK;
+}
+
 static int after_launch(geist_hip_sampler *s, const char *what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess)
@@ -952,8 +963,8 @@ int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
         return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
     hipEvent_t a, b;
     HIPCHK(s, hipSetDevice(s->device));
-    HIPCHK(s, hipEventCreate(&a));
-    HIPCHK(s, hipEventCreate(&b));
+    if (const int ev = event_pair(s, &a, &b))
+        return ev;
     /* a complete call first, so that the kernel finds the inputs an earlier stage leaves it */
     int rc = 0;
     for (size_t i = 0; i < n_batches && !rc; ++i)
@@ -1002,8 +1013,8 @@ int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_h
     }
     hipEvent_t a, b;
     HIPCHK(s, hipSetDevice(s->device));
-    HIPCHK(s, hipEventCreate(&a));
-    HIPCHK(s, hipEventCreate(&b));
+    if (const int ev = event_pair(s, &a, &b))
+        return ev;
     for (size_t i = 0; i < n_batches; ++i)
         launch_plain_read(L[i], s->uniforms);
     int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
@@ -1033,8 +1044,8 @@ int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_
             return rc;
     }
     hipEvent_t a, b;
-    HIPCHK(s, hipEventCreate(&a));
-    HIPCHK(s, hipEventCreate(&b));
+    if (const int ev = event_pair(s, &a, &b))
+        return ev;
     int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
     for (int i = 0; i < launches && !rc; ++i)
         rc = geist_hip_f16_gemv_rows(s, d_w_f16[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
@@ -1238,8 +1249,8 @@ int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq
             return rc;
     }
     hipEvent_t a, b;
-    HIPCHK(s, hipEventCreate(&a));
-    HIPCHK(s, hipEventCreate(&b));
+    if (const int ev = event_pair(s, &a, &b))
+        return ev;
     int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
     for (int i = 0; i < launches && !rc; ++i)
         rc = geist_hip_q8w_gemv_rows(s, d_wq[(size_t) i % n_weights],
