@@ -1001,7 +1001,12 @@ int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_h
         return GEIST_HIP_E_INVALID_ARG;
     if (launches < 1 || !ms_total || !rows || n_batches < 1)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
-    std::vector<Launch> L(n_batches);
+    std::vector<Launch> L;
+    try { /* no exception leaves a C entry point */
+        L.resize(n_batches);
+    } catch (const std::bad_alloc &) {
+        return fail(s, GEIST_HIP_E_OOM, "plain read: %zu batches", n_batches);
+    }
     for (size_t i = 0; i < n_batches; ++i) {
         const int rc = make_launch(s, &rows[i], nullptr, false, L[i]);
         if (rc)
@@ -1143,9 +1148,14 @@ int geist_hip_spec_head_build(geist_hip_sampler *s, const uint16_t *d_embed_f16,
               alloc(d.fin_idx, topk * 4) && alloc(d.fin_exact, topk * 4) &&
               alloc(d_var, d_model * 4);
     int err = ok ? 0 : GEIST_HIP_E_OOM;
-    std::vector<float>    var(d_model);
-    std::vector<uint32_t> dims(sd);
-    std::vector<uint8_t>  kept(d_model, 0);
+    std::vector<float>    var;
+    std::vector<uint32_t> dims;
+    std::vector<uint8_t>  kept;
+    try { /* no exception leaves a C entry point */
+        var.resize(d_model), dims.resize(sd), kept.assign(d_model, 0);
+    } catch (const std::bad_alloc &) {
+        err = GEIST_HIP_E_OOM;
+    }
     if (!err) {
         /* spec_head.c:505-522 on the device, :526-548 here */
         const long vstep = n_vocab > 512 ? (long) (n_vocab / 512) : 1;
