@@ -1,6 +1,15 @@
 """Helpers of the GPU parity tests: move a workload to the device, run it through the C ABI and
 compare token ids with the oracle under the counted-exception rule."""
+import os
+
 import numpy as np
+
+
+def fuzz_seeds(n):
+    """The seeds of a randomised test: n by default, n * GEIST_TEST_FUZZ_SCALE for a long run
+    (GEIST_TEST_FUZZ_SCALE=60 python -m pytest tests -m gpu -k random)."""
+    return range(n * max(1, int(os.environ.get("GEIST_TEST_FUZZ_SCALE", "1"))))
+
 
 # A draw closer than this (relative to the mass of the walk) to an edge of its CDF slot may
 # legitimately land in the neighbouring slot on the device; such rows are counted, not failed.

@@ -5,7 +5,7 @@ the other parity tests."""
 import numpy as np
 import pytest
 
-from gpu_util import compare_ids, run_rows
+from gpu_util import compare_ids, fuzz_seeds, run_rows
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -79,7 +79,7 @@ def _case(g):
         f"lead={lead} mask={dens}")
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", fuzz_seeds(16))
 def test_random_configurations_match_oracle(hs, oracle, seed):
     from geistlib_amd import SampleParams
     g = np.random.default_rng(1000 + seed)
@@ -129,7 +129,7 @@ def _spec_matches(oracle, target, q, draft, u, T, nacc, out):
     return nacc == want_n and out[:want_n + 1].tolist() == want[:want_n + 1].tolist()
 
 
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", fuzz_seeds(8))
 def test_random_spec_verify_matches_oracle(hs_spec, oracle, seed):
     """Random draft length, batch, vocabulary, temperature, soft-cap and draft quality, dense and
     point-mass drafts. A sequence that differs must be explained by a uniform within 2e-6 of a
@@ -182,7 +182,7 @@ def test_random_spec_verify_matches_oracle(hs_spec, oracle, seed):
 
 
 # --------------------------------------------------------- probabilities and log-probabilities
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", fuzz_seeds(6))
 def test_random_softmax_and_logprob_rows(hs, oracle, seed):
     """geist_hip_softmax_rows and geist_hip_logprob_rows over random shapes, strides, penalties,
     temperatures and caps: probabilities within 2e-7 relative of the oracle's (the contract is

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
 
-from gpu_util import compare_ids, run_rows, to_dev  # noqa: E402
+from gpu_util import compare_ids, fuzz_seeds, run_rows, to_dev  # noqa: E402
 
 
 @pytest.fixture(scope="module")
@@ -687,7 +687,7 @@ def test_argument_errors(hs):
 
 
 # ------------------------------------------------------------------------- n-gram drafter
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", fuzz_seeds(4))
 def test_ngram_drafter_matches_oracle(hs, oracle, seed):
     """geist_hip_propose_drafts_ngram against the restated propose_drafts_ngram
     (src/engine/session.c:437-513): drafts, their count and the matched length, exactly."""

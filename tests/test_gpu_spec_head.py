@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 torch = pytest.importorskip("torch")
+from gpu_util import fuzz_seeds  # noqa: E402
 from oracle_lib import Oracle  # noqa: E402
 
 pytestmark = pytest.mark.gpu
@@ -161,7 +162,7 @@ def test_rejects_what_it_cannot_take(hs):
         hs.spec_head_build(torch.zeros((40000, 512), dtype=torch.float16, device="cuda"))
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", fuzz_seeds(6))
 def test_random_geometries_against_the_oracle(hs, oracle, seed):
     """Vocabulary, width, finalist count, weight and activation scales drawn at random; token,
     cutoff and rough scores as the oracle's."""
