@@ -644,8 +644,10 @@ static int f64_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, F64Scrat
         const size_t out = n_out > s->f64_out ? n_out : s->f64_out;
         const size_t bytes = (size_t) F64_M_MAX * (in + in / 64 + 2) * sizeof(double) + 16 +
                              out * F64_M_MAX * sizeof(int2);
-        if (hipMalloc(&s->f64_ws, bytes) != hipSuccess)
+        if (hipMalloc(&s->f64_ws, bytes) != hipSuccess) {
+            s->f64_ws = nullptr;
             return fail(s, GEIST_HIP_E_OOM, "f64 projection: scratch");
+        }
         s->f64_in = in, s->f64_out = out;
     }
     char *p      = static_cast<char *>(s->f64_ws);
