@@ -5,7 +5,7 @@ oracle, which is itself pinned bit for bit to the reference's compiled kernel
 import numpy as np
 import pytest
 
-from gpu_util import to_dev
+from gpu_util import fuzz_seeds, to_dev
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -375,3 +375,55 @@ def test_project_sample_rows_in_the_portable_backends_arithmetic(hs, oracle):
     hs.project_sample(*args, normed=normed)
     hs.sync()
     assert (bits(logits.cpu().numpy()) == bits(oracle.f16_gemv(w16, normed_want))).all()
+
+
+@pytest.mark.parametrize("seed", fuzz_seeds(4))
+def test_random_projection_shapes(hs, oracle, seed):
+    """Norm, F16 and int8 projections, the quantiser and the projection in double on random
+    shapes, scales and row counts, each against the oracle in every bit. Integer-valued and
+    cancelling data put the sums in double on rounding boundaries of binary32."""
+    g = np.random.default_rng(9000 + seed)
+    for case in range(5):
+        n_out = int(g.integers(1, 5000))
+        n_in = 16 * int(g.integers(1, 257)) + (8 if g.random() < 0.3 else 0)
+        m = int(g.integers(1, 21))
+        kind = int(g.integers(0, 3))
+        print(f"projection seed {seed} case {case}: n_out={n_out} n_in={n_in} m={m} kind={kind}",
+              flush=True)
+        w = (g.standard_normal((n_out, n_in)) * g.choice([1e-3, 0.05, 1.0, 30.0])).astype(np.float16)
+        x = (g.standard_normal((m, n_in)) * g.choice([1e-3, 1.0, 100.0], (m, 1))).astype(np.float32)
+        if kind == 1:
+            w = g.integers(-6, 7, (n_out, n_in)).astype(np.float16)
+            x = g.integers(-5, 6, (m, n_in)).astype(np.float32)
+            x[:, 0] += np.float32(2.0 ** -int(g.integers(10, 30)))
+        if kind == 2:
+            w[:, 1::2] = -w[:, ::2]
+            x[:, 1::2] = x[:, ::2] * np.float32(1 + 2.0 ** -12)
+        w16 = w.view(np.uint16)
+        d_w, d_x = to_dev(w.view(np.int16), torch), to_dev(x, torch)
+        y = torch.full((m, n_out), 7.0, dtype=torch.float32, device="cuda")
+        hs.f16_gemv(d_w, d_x, y)
+        hs.sync()
+        assert (bits(y.cpu().numpy()) == bits(oracle.f16_gemv(w16, x))).all()
+        y.fill_(7.0)
+        hs.f16_linear(d_w, d_x, y)
+        hs.sync()
+        assert (bits(y.cpu().numpy()) == bits(oracle.f16_linear_f64(w16, x))).all()
+        if n_in % 16 == 0:
+            wq = torch.empty((n_out, n_in), dtype=torch.int8, device="cuda")
+            sc = torch.empty(n_out, dtype=torch.float32, device="cuda")
+            hs.f16_to_q8w(d_w, wq, sc)
+            hs.sync()
+            wq_want, sc_want = oracle.f16_to_q8w(w16)
+            assert (wq.cpu().numpy() == wq_want).all()
+            assert (bits(sc.cpu().numpy()) == bits(sc_want)).all()
+            y.fill_(7.0)
+            hs.q8w_gemv(wq, sc, d_x, y)
+            hs.sync()
+            assert (bits(y.cpu().numpy()) == bits(oracle.q8w_gemv(wq_want, sc_want, x))).all()
+        norm_w = g.standard_normal(n_in).astype(np.float32)
+        eps = float(g.choice([1e-5, 1e-6, 0.0]))
+        normed = torch.empty((m, n_in), dtype=torch.float32, device="cuda")
+        hs.rmsnorm(d_x, to_dev(norm_w, torch), eps, normed)
+        hs.sync()
+        assert (bits(normed.cpu().numpy()) == bits(oracle.rmsnorm(x, norm_w, eps))).all()
