@@ -5,4 +5,4 @@ plus a C23 host layer with the reference's own sampler symbols). This Python pac
 them with ctypes for tests and benchmarks; it contains no sampling arithmetic and no fallback.
 """
 from .binding import (HipSampler, SampleParams, SpecResult, load_library,  # noqa: F401
-                      library_path)
+                      library_path, sample_rows_static)

@@ -82,6 +82,8 @@ def load_library():
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
+    lib.geist_hip_sample_rows_static.argtypes = [i32, vp, C.POINTER(Rows), C.POINTER(SampleParams),
+                                                 vp, vp, C.c_char_p, sz]
     lib.geist_hip_argmax_f32.argtypes = [vp, vp, sz, C.POINTER(C.c_int32)]
     lib.geist_hip_apply_penalties.argtypes = [vp, vp, sz, sz, sz, vp, sz, vp, f32, f32, f32]
     lib.geist_hip_softmax_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, sz]
@@ -129,6 +131,17 @@ def load_library():
 
 def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def sample_rows_static(rows, params, uniforms, out, device=0, stream=None):
+    """geist_hip_sample_rows_static: sampling without a sampler object and without any
+    allocation (the workspace is an array inside the library)."""
+    lib = load_library()
+    err = C.create_string_buffer(512)
+    rc = lib.geist_hip_sample_rows_static(device, stream, C.byref(rows), C.byref(params),
+                                          _ptr(uniforms), _ptr(out), err, len(err))
+    if rc != GEIST_HIP_OK:
+        raise GeistHipError(rc, err.value.decode())
 
 
 class HipSampler:

@@ -7,6 +7,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <pthread.h>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -166,7 +168,58 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
  * set, a sampling call enqueues that kernel and nothing after it. */
 static inline bool stream_only(const geist_hip_sampler *s) { return s->stream_kernel_only; }
 
+/* ---- sampling without any allocation --------------------------------------------------------
+ * The workspace of geist_hip_sample_rows_static: a device array that belongs to the code object,
+ * so neither a sampler object nor hipMalloc is needed. In host code `scratch` is only the
+ * symbol's host-side stand-in; the device address is looked up once per device with
+ * hipGetSymbolAddress and kept in g_static_ws[]. Every GPU holds its own copy of the array. */
+namespace {
+constexpr size_t STATIC_UNITS = GEIST_HIP_STATIC_MAX_UNITS; /* (row, chunk) pairs */
+constexpr size_t STATIC_TMAX  = 0;                                     /* float [units][256]  */
+constexpr size_t STATIC_BEST  = STATIC_TMAX + STATIC_UNITS * 256 * 4;  /* u64   [units]       */
+constexpr size_t STATIC_CSUM  = STATIC_BEST + STATIC_UNITS * 8;        /* double[units]       */
+constexpr size_t STATIC_SLAB  = STATIC_CSUM + STATIC_UNITS * 8;        /* double[units][8]    */
+constexpr size_t STATIC_BYTES = STATIC_SLAB + STATIC_UNITS * 8 * 8;
+constexpr int    STATIC_MAX_DEVICES = 64;
+} // namespace
+static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
+
+static unsigned char *g_static_ws[STATIC_MAX_DEVICES]; /* device address of `scratch`, per device */
+static bool           g_static_ws_tried[STATIC_MAX_DEVICES];
+static hipError_t     g_static_ws_err[STATIC_MAX_DEVICES];
+static pthread_mutex_t g_static_ws_lock = PTHREAD_MUTEX_INITIALIZER;
+
+/* The device address of `scratch` on `device` (which must be current). Looked up on the first
+ * call per device; later calls return the kept pointer without touching the runtime. */
+static hipError_t static_workspace(int device, unsigned char **out) {
+    if (device < 0 || device >= STATIC_MAX_DEVICES)
+        return hipErrorInvalidDevice;
+    pthread_mutex_lock(&g_static_ws_lock);
+    if (!g_static_ws_tried[device]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        g_static_ws_err[device]   = e;
+        g_static_ws[device]       = e == hipSuccess ? static_cast<unsigned char *>(p) : nullptr;
+        g_static_ws_tried[device] = e == hipSuccess; /* a failed lookup is tried again */
+    }
+    const hipError_t e = g_static_ws_err[device];
+    *out               = g_static_ws[device];
+    pthread_mutex_unlock(&g_static_ws_lock);
+    return e;
+}
+
 /* ============================================================================================ */
+/* failure text into a caller's buffer (an entry point without a sampler object has no error slot) */
+static int report(char *err, size_t err_len, int code, const char *fmt, ...) {
+    if (err && err_len) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(err, err_len, fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
 extern "C" {
 
 int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void *stream,
@@ -195,6 +248,11 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     const size_t rc = max_rows * mc;
     hipError_t   e  = hipSetDevice(device);
     if (e == hipSuccess) e = (hipError_t) configure_device_kernels();
+    if (e == hipSuccess) { /* the address of the static workspace, so that the allocation-free
+                            * entry point finds it ready (a failure is reported by that call) */
+        unsigned char *ws = nullptr;
+        (void) static_workspace(device, &ws);
+    }
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
@@ -465,6 +523,51 @@ int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *row
                           const struct geist_hip_sample_params *params, const float *d_uniforms,
                           geist_hip_token_t *d_out_tokens) {
     return sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+}
+
+int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hip_rows *rows,
+                                 const struct geist_hip_sample_params *params,
+                                 const float *d_uniforms, geist_hip_token_t *d_out_tokens,
+                                 char *err, size_t err_len) {
+    if (err && err_len)
+        err[0] = 0;
+    if (!rows || !params)
+        return report(err, err_len, GEIST_HIP_E_INVALID_ARG, "null rows or params");
+    /* a sampler object on the stack whose workspace is the device array: the flows below are
+     * those of geist_hip_sample_rows, with the modes that need more than this left out */
+    geist_hip_sampler tmp;
+    tmp.device = device;
+    tmp.stream = (hipStream_t) stream;
+    Resolved rs;
+    int      rc = resolve(&tmp, params, rows->n_vocab, rs);
+    if (rc)
+        return report(err, err_len, rc, "%s", tmp.err);
+    if (!rs.greedy && !rs.use_k && (rs.use_p || rs.use_m))
+        return report(err, err_len, GEIST_HIP_E_UNSUPPORTED,
+                      "top-p / min-p over the whole vocabulary needs a row of probabilities per "
+                      "logit row: use geist_hip_sample_rows");
+    const size_t units = rows->rows * ((rows->n_vocab + 2047) / 2048);
+    if (rows->rows == 0 || rows->n_vocab == 0 || units > STATIC_UNITS)
+        return report(err, err_len, GEIST_HIP_E_INVALID_ARG,
+                      "rows x ceil(n_vocab / 2048) = %zu x %zu exceeds the static workspace of %zu "
+                      "(or the batch is empty)",
+                      rows->rows, (rows->n_vocab + 2047) / 2048, (size_t) STATIC_UNITS);
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess)
+        return report(err, err_len, GEIST_HIP_E_BACKEND, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+    unsigned char *ws = nullptr;
+    e                 = static_workspace(device, &ws);
+    if (e != hipSuccess || !ws)
+        return report(err, err_len, GEIST_HIP_E_BACKEND, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    tmp.max_rows   = rows->rows;
+    tmp.max_vocab  = rows->n_vocab;
+    tmp.max_chunks = (int) std::min<size_t>((rows->n_vocab + 2047) / 2048, (size_t) MAX_CHUNKS);
+    tmp.tmax       = reinterpret_cast<float *>(ws + STATIC_TMAX);
+    tmp.chunk_best = reinterpret_cast<uint64_t *>(ws + STATIC_BEST);
+    tmp.chunk_sum  = reinterpret_cast<double *>(ws + STATIC_CSUM);
+    tmp.slab_sum   = reinterpret_cast<double *>(ws + STATIC_SLAB);
+    rc = sample_impl(&tmp, rows, params, d_uniforms, d_out_tokens);
+    return rc ? report(err, err_len, rc, "%s", tmp.err) : GEIST_HIP_OK;
 }
 
 int geist_hip_sample_rows_rng(geist_hip_sampler *s, const struct geist_hip_rows *rows,

@@ -122,6 +122,26 @@ int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *row
                           const struct geist_hip_sample_params *params, const float *d_uniforms,
                           geist_hip_token_t *d_out_tokens);
 
+/* geist_hip_sample_rows for callers that cannot allocate. It has no counterpart in the reference;
+ * it is for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc: no sampler object is needed and the call allocates nothing, on the host or on the
+ * device. Its workspace is an array of device memory inside the library's code object
+ * (GEIST_HIP_STATIC_MAX_UNITS x 1104 bytes = 4.3 MiB per GPU, held until the process ends).
+ *   device, stream   where the kernels are enqueued (stream NULL = the default stream)
+ *   err, err_len     optional buffer for the text of a failure
+ * Served: greedy, temperature, and every top-k configuration (with top-p / min-p behind it,
+ * penalties, soft-cap, allowed-token mask). Top-p / min-p WITHOUT top-k returns
+ * GEIST_HIP_E_UNSUPPORTED. rows x ceil(n_vocab / 2048) must not exceed
+ * GEIST_HIP_STATIC_MAX_UNITS (e.g. 64 rows of 128256 logits), else GEIST_HIP_E_INVALID_ARG.
+ * Same tokens as geist_hip_sample_rows. All calls on one GPU share the one array: calls that
+ * overlap on a GPU (two streams, two threads) race; calls on one stream are ordered. The first
+ * call on a device looks the array's address up (geist_hip_sampler_create does so too). */
+#define GEIST_HIP_STATIC_MAX_UNITS 4096
+int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hip_rows *rows,
+                                 const struct geist_hip_sample_params *params,
+                                 const float *d_uniforms, geist_hip_token_t *d_out_tokens,
+                                 char *err, size_t err_len);
+
 /* Same, drawing the uniforms on the device from xorshift64* states (struct geist_rng,
  * src/engine/sampler.h:28-32; sampler.c:35-48) held in device memory.
  *   shared != 0: one state for the whole batch, row r takes the (r+1)-th draw and the state
