@@ -38,6 +38,8 @@ struct geist_hip_sampler {
     double   *resid_slab = nullptr; /* [max_rows][max_chunks][8] spec verification */
     void     *verdict    = nullptr; /* [max_rows] acceptance results of spec verification */
     float    *tmax       = nullptr; /* [max_rows][max_chunks][256] per-thread maxima */
+    void     *wcands     = nullptr; /* what the top-k scan's wavefronts hand on (WaveCands) */
+    size_t    wcands_row_waves = 0; /* (row, wavefront) pairs it has room for */
     int32_t  *row_flag   = nullptr; /* [max_rows] */
     float    *uniforms   = nullptr; /* [max_rows] */
     float    *probe_p    = nullptr; /* [max_rows] */
@@ -179,7 +181,10 @@ constexpr size_t STATIC_TMAX  = 0;                                     /* float 
 constexpr size_t STATIC_BEST  = STATIC_TMAX + STATIC_UNITS * 256 * 4;  /* u64   [units]       */
 constexpr size_t STATIC_CSUM  = STATIC_BEST + STATIC_UNITS * 8;        /* double[units]       */
 constexpr size_t STATIC_SLAB  = STATIC_CSUM + STATIC_UNITS * 8;        /* double[units][8]    */
-constexpr size_t STATIC_BYTES = STATIC_SLAB + STATIC_UNITS * 8 * 8;
+constexpr size_t STATIC_ROW_WAVES = STATIC_UNITS + 512;            /* (row, wavefront) pairs */
+constexpr size_t STATIC_WCANDS = STATIC_SLAB + STATIC_UNITS * 8 * 8;   /* WaveCands           */
+constexpr size_t STATIC_BYTES  = STATIC_WCANDS + STATIC_ROW_WAVES * 648;
+static_assert(STATIC_WCANDS % 16 == 0, "float4 slots");
 constexpr int    STATIC_MAX_DEVICES = 64;
 } // namespace
 static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
@@ -259,6 +264,12 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     if (e == hipSuccess) e = hipMalloc((void **) &s->slab_sum, rc * 8 * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_slab, rc * 8 * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->tmax, rc * 256 * sizeof(float));
+    {
+        const size_t chunks8k = (max_vocab + 8191) / 8192;
+        s->wcands_row_waves   = max_rows * NWAVES_PER_CHUNK *
+                              (chunks8k < (size_t) CAND_CHUNKS_MAX ? chunks8k : (size_t) CAND_CHUNKS_MAX);
+        if (e == hipSuccess) e = hipMalloc(&s->wcands, wave_cands_bytes(s->wcands_row_waves));
+    }
     if (e == hipSuccess) e = hipMalloc(&s->verdict, max_rows * SPEC_VERDICT_BYTES);
     if (e == hipSuccess) e = hipMalloc((void **) &s->row_flag, max_rows * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->uniforms, max_rows * sizeof(float));
@@ -285,6 +296,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->slab_sum);
     (void) hipFree(s->resid_slab);
     (void) hipFree(s->tmax);
+    (void) hipFree(s->wcands);
     (void) hipFree(s->verdict);
     (void) hipFree(s->row_flag);
     (void) hipFree(s->uniforms);
@@ -450,12 +462,29 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
             f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
         }
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
+        f.mode = FINAL_TOPK;
+        f.k    = rs.k;
+        /* Plain rows (aligned, no soft-cap, no mask, penalties absent or left to the final kernel)
+         * take the candidate path: the scan's wavefronts hand their leading groups on and the
+         * row-final kernel gathers nothing. */
+        const size_t row_waves = rows->rows * (size_t) L.rv.n_chunks * NWAVES_PER_CHUNK;
+        const bool   plain = rs.k <= CAND_K_MAX && L.rv.vec_ok && !(L.rv.softcap > 0.0f) &&
+                           !L.rv.allowed &&
+                           L.rv.n_chunks <= CAND_CHUNKS_MAX && (!L.pen || !scan.pen) &&
+                           !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves;
+        const int m = plain ? cand_lanes_for(f.k_sel, rows->n_vocab) : 0;
+        if (m) {
+            const WaveCands wc = wave_cands_at(s->wcands, row_waves);
+            launch_cand_scan(scan, s->tmax, wc, m);
+            if (stream_only(s))
+                return after_launch(s, "top-k scan");
+            launch_final_cand(L, f, wc);
+            return after_launch(s, "top-k");
+        }
         if (!s->tmax_ready)
             launch_tmax_scan(scan, s->tmax, nullptr);
         if (stream_only(s))
             return after_launch(s, "top-k scan");
-        f.mode = FINAL_TOPK;
-        f.k    = rs.k;
         launch_row_final(L, f);
         return after_launch(s, "top-k");
     }
@@ -566,6 +595,8 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
     tmp.chunk_best = reinterpret_cast<uint64_t *>(ws + STATIC_BEST);
     tmp.chunk_sum  = reinterpret_cast<double *>(ws + STATIC_CSUM);
     tmp.slab_sum   = reinterpret_cast<double *>(ws + STATIC_SLAB);
+    tmp.wcands     = ws + STATIC_WCANDS;
+    tmp.wcands_row_waves = STATIC_ROW_WAVES;
     rc = sample_impl(&tmp, rows, params, d_uniforms, d_out_tokens);
     return rc ? report(err, err_len, rc, "%s", tmp.err) : GEIST_HIP_OK;
 }

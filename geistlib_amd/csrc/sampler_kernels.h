@@ -66,6 +66,38 @@ struct CandSpace {
                           * 3 whole row */
 };
 
+/* Workspace of the candidate path of the top-k modes: what each scanning wavefront hands on to
+ * the row-final kernel. A row is scanned by n_chunks * 4 wavefronts; wavefront w of row r owns
+ * CAND_GROUPS slots. */
+constexpr int NWAVES_PER_CHUNK = 4; /* a chunk is scanned by one workgroup of four wavefronts */
+constexpr int CAND_SLOTS     = 32;  /* float4 groups a wavefront has room for ... */
+constexpr int CAND_GROUPS    = 24;  /* ... and how many it may hand on (the rest is never read) */
+constexpr int CAND_CHUNKS_MAX = 32; /* rows of up to 32 chunks of 8192 logits take this path */
+constexpr int CAND_K_MAX     = 64;  /* largest k: the survivors are ordered one per lane */
+constexpr int CAND_LANES_MAX = 18;  /* largest `m` (see k_cand_scan) that leaves room in the slots */
+struct WaveCands {
+    float4   *val;   /* [rows][waves][CAND_SLOTS] the groups */
+    int32_t  *idx;   /* [rows][waves][CAND_SLOTS] index of each group's first element, -1 = unused */
+    uint32_t *bound; /* [rows][waves] key of the wavefront's bound T; 0xffffffff = it had too many
+                      * groups and handed none on */
+};
+/* bytes of the three arrays for `row_waves` = rows * waves per row */
+inline size_t wave_cands_bytes(size_t row_waves) {
+    return row_waves * (CAND_SLOTS * (sizeof(float4) + sizeof(int32_t)) + 8); /* 648 */
+}
+inline WaveCands wave_cands_at(void *base, size_t row_waves) {
+    WaveCands w;
+    w.val   = static_cast<float4 *>(base);
+    w.idx   = reinterpret_cast<int32_t *>(w.val + row_waves * CAND_SLOTS);
+    w.bound = reinterpret_cast<uint32_t *>(w.idx + row_waves * CAND_SLOTS);
+    return w;
+}
+/* `m` for a row of n_vocab logits of which about k_eff lead: the smallest number of lanes such
+ * that a wavefront (2048 logits) holding that many of the k_eff is a one-in-10^8 event when the
+ * logits' order is unrelated to the vocabulary's. 0 = the candidate path does not pay
+ * (m would exceed CAND_LANES_MAX). */
+int cand_lanes_for(int k_eff, size_t n_vocab);
+
 struct FinalLaunch {
     CandSpace       cand;
     bool            minp_listed; /* the exp-sum pass already listed the rows under the min-p bound */
@@ -125,6 +157,11 @@ void launch_spec(const Launch &L, const SpecLaunch &sp);
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best,
                       int32_t *zero_per_row = nullptr);
 void launch_row_final(const Launch &L, const FinalLaunch &f);
+/* the candidate path of top-k (sampler_cands.h): L.nv == 8, no soft-cap, no mask, 16-byte aligned
+ * rows of at most CAND_CHUNKS_MAX chunks; the scan reads the logits raw (penalties are the final
+ * kernel's) and also stores the thread maxima */
+void launch_cand_scan(const Launch &L, float *tmax, const WaveCands &wc, int m);
+void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &wc);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */

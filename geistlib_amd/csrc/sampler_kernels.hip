@@ -10,6 +10,9 @@
  *                    index-order CDF draw, top-k select + sorted softmax + top-p + min-p +
  *                    draw, top-p / min-p shortcut                             sampler.c:90-102, 209-222, 272-299
  *   k_topk_general   top-k for k above 128 and degenerate rows                 sampler.c:178-228
+ *   k_cand_scan, k_final_cand (sampler_cands.h)   the top-k path for plain rows: the scan hands
+ *                    each wavefront's leading groups on, the row-final kernel gathers nothing
+ *                                                                              sampler.c:178-228
  *   k_list_candidates, k_sorted_candidates, k_sorted_general (sampler_sorted_prob.h)
  *                    full-vocabulary top-p / min-p for kept prefixes the shortcut cannot
  *                    serve: candidate list, then the whole row                 sampler.c:246-304
@@ -1039,6 +1042,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #include "sampler_sorted_prob.h"
 #include "sampler_spec.h"
 #include "sampler_draft.h"
+#include "sampler_cands.h"
 namespace gs {
 
 /* ============================================================================================
@@ -1597,7 +1601,7 @@ void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best, int32_
     });
 }
 
-void launch_row_final(const Launch &L, const FinalLaunch &f) {
+static FinalArgs final_args(const FinalLaunch &f) {
     FinalArgs a;
     a.mode       = f.mode;
     a.k          = f.k;
@@ -1616,6 +1620,47 @@ void launch_row_final(const Launch &L, const FinalLaunch &f) {
     a.ln_min_p   = f.min_p > 0.0f ? std::log((double) f.min_p) : 0.0;
     a.zb_min_p    = zbin_of_min_p(f.min_p);
     a.minp_listed = f.minp_listed;
+    return a;
+}
+
+int cand_lanes_for(int k_eff, size_t n_vocab) {
+    const double lam = 2048.0 * (double) k_eff / (double) n_vocab;
+    double       p = std::exp(-lam), cdf = p; /* P(X <= m) for X ~ Poisson(lam) */
+    int          m = 0;
+    while (1.0 - cdf > 1e-8 && m < 64) {
+        ++m;
+        p *= lam / m;
+        cdf += p;
+    }
+    ++m; /* P(X >= m) <= 1e-8 */
+    if (m < 4)
+        m = 4;
+    return m <= CAND_LANES_MAX ? m : 0;
+}
+
+void launch_cand_scan(const Launch &L, float *tmax, const WaveCands &wc, int m) {
+    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    k_cand_scan<8><<<grid, block, 0, L.stream>>>(L.rv, tmax, wc, m);
+}
+
+void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &wc) {
+    const FinalArgs a = final_args(f);
+    const dim3      grid(L.rows), block(FC_THREADS);
+    if (L.rv.n_chunks <= 16) { /* up to 64 scanning wavefronts per row */
+        if (L.pen)
+            k_final_cand<8, true, false><<<grid, block, 0, L.stream>>>(L.rv, a, wc);
+        else
+            k_final_cand<8, false, false><<<grid, block, 0, L.stream>>>(L.rv, a, wc);
+    } else {
+        if (L.pen)
+            k_final_cand<8, true, true><<<grid, block, 0, L.stream>>>(L.rv, a, wc);
+        else
+            k_final_cand<8, false, true><<<grid, block, 0, L.stream>>>(L.rv, a, wc);
+    }
+}
+
+void launch_row_final(const Launch &L, const FinalLaunch &f) {
+    const FinalArgs a = final_args(f);
     const dim3 grid(L.rows), block(TPB);
     if (f.mode == FINAL_ARGMAX) {
         k_final_argmax<<<grid, block, 0, L.stream>>>(L.rv, a);
