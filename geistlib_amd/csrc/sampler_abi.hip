@@ -471,7 +471,8 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         const bool   plain = rs.k <= CAND_K_MAX && L.rv.vec_ok && !(L.rv.softcap > 0.0f) &&
                            !L.rv.allowed &&
                            L.rv.n_chunks <= CAND_CHUNKS_MAX && (!L.pen || !scan.pen) &&
-                           !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves;
+                           !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves &&
+                           (!L.pen || rows->history_ld <= (size_t) HT_HISTORY_MAX);
         const int m = plain ? cand_lanes_for(f.k_sel, rows->n_vocab) : 0;
         if (m) {
             const WaveCands wc = wave_cands_at(s->wcands, row_waves);

@@ -39,15 +39,19 @@ __device__ long long g_phase[4096 * 16];
         if (threadIdx.x == 0)                                                                  \
             g_phase[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (p)] = wall_clock64();        \
     } while (0)
+#define GS_JOB_PHASE(row, p)                                                                   \
+    do {                                                                                       \
+        if (threadIdx.x == 0)                                                                  \
+            g_phase[(2048 + (row)) * 16 + (p)] = wall_clock64();                               \
+    } while (0)
 #else
 #define GS_PHASE(p) do { } while (0)
+#define GS_JOB_PHASE(row, p) do { } while (0)
 #endif
 
 constexpr uint32_t KEY_LOWEST_FINITE = 0x00800000u; /* f2key(-FLT_MAX) */
 constexpr int      CAND_PER_WAVE     = 256;  /* groups / elements at or above B that one wavefront
                                               * of the final kernel holds */
-constexpr int      CAND_HASH         = 2048; /* slots of the candidates' id table */
-constexpr int      CAND_PROBES       = 64;   /* longest probe sequence in that table */
 constexpr int      CAND_CUT_MAX      = CAND_K_MAX; /* entries the last wavefront orders */
 static_assert(CAND_CUT_MAX == WAVE, "one entry per lane");
 
@@ -63,6 +67,10 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ __forceinline__ uint32_t hist_hash(int id) {
+    return ((uint32_t) id * 0x9E3779B1u) >> 20; /* 12 bits: HT_SLOTS slots */
 }
 
 template <int NV>
@@ -144,7 +152,6 @@ struct CandShared {
     int      n_real;    /* elements that still reach B after the penalties */
     int      n_cut;     /* entries listed for the final ordering */
     int      give_up;   /* the row cannot be served here */
-    int      n_el[16];  /* elements at or above B in each wavefront's share */
 };
 
 constexpr int FC_THREADS = 1024;             /* threads of the final kernel */
@@ -157,9 +164,9 @@ constexpr int FC_STRIDE  = 2 * FC_LIST;      /* its list in LDS: FC_LIST entries
  * path, when a row falls back to it, reuses the arena from its start. */
 constexpr int CA_EVAL = 0;                                   /* u32 [16][FC_STRIDE] bits, then keys */
 constexpr int CA_EIDX = CA_EVAL + FC_WAVES * FC_STRIDE * 4;  /* u32 [16][FC_STRIDE] vocabulary ids  */
-constexpr int CA_HKEY = CA_EIDX + FC_WAVES * FC_STRIDE * 4;  /* int [CAND_HASH] ids                 */
-constexpr int CA_HCNT = CA_HKEY + CAND_HASH * 4;             /* u32 [CAND_HASH] occurrences         */
-constexpr int CA_HIST = CA_HCNT + CAND_HASH * 4;             /* u32 [256] key bins                  */
+constexpr int CA_HKEY = CA_EIDX + FC_WAVES * FC_STRIDE * 4;  /* int [HT_SLOTS] the history table    */
+constexpr int CA_HCNT = CA_HKEY + HT_SLOTS * 4;              /* u32 [HT_SLOTS / 2] occurrences      */
+constexpr int CA_HIST = CA_HCNT + HT_SLOTS * 2;              /* u32 [256] key bins                  */
 constexpr int CA_CUT  = CA_HIST + 256 * 4;                   /* u64 [2 * CAND_CUT_MAX]              */
 constexpr int CA_END  = CA_CUT + 2 * CAND_CUT_MAX * 8;
 
@@ -210,9 +217,6 @@ __device__ __forceinline__ int cand_fallback(const RowView *rvp, const FinalArgs
     return k;
 }
 
-__device__ __forceinline__ uint32_t cand_hash(int id) {
-    return ((uint32_t) id * 0x9E3779B1u) >> 21; /* 11 bits: CAND_HASH slots */
-}
 __device__ __forceinline__ double readlane_f64(double v, int lane) {
     const uint64_t u = (uint64_t) __double_as_longlong(v);
     return __longlong_as_double((long long) (((uint64_t) readlane_u32((uint32_t) (u >> 32), lane) << 32) |
@@ -306,11 +310,12 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         }
     }
     uint32_t bk = tid < W ? wc.bound[row * W + tid] : 0u;
-    /* the row's history, two ids a thread (the rest, if any, is read when it is looked up) */
-    int hid0 = -1, hid1 = -1, hlen = 0;
+    /* the row's history, two ids a thread (at most HT_HISTORY_MAX = 2 * 1024: the launch code
+     * sends longer histories down another path) */
+    int hid0 = -1, hid1 = -1;
     if (PEN) {
-        hlen = rv.hist_len[row];
-        hlen = hlen > rv.hist_ld ? (int) rv.hist_ld : hlen;
+        int hlen = rv.hist_len[row];
+        hlen     = hlen > rv.hist_ld ? (int) rv.hist_ld : hlen;
         const int32_t *h = rv.hist + (long) row * rv.hist_ld;
         if (tid < hlen)
             hid0 = h[tid];
@@ -328,12 +333,11 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         s_c.n_cut   = 0;
         s_c.give_up = 0;
     }
-    if (PEN) {
-        uint4 *zk = reinterpret_cast<uint4 *>(hkey), *zc = reinterpret_cast<uint4 *>(hcnt);
-        if (tid < CAND_HASH / 4) {
-            zk[tid] = make_uint4(~0u, ~0u, ~0u, ~0u);
-            zc[tid] = make_uint4(0u, 0u, 0u, 0u);
-        }
+    if (PEN) { /* the history table starts empty */
+        static_assert(HT_SLOTS == 4 * FC_THREADS, "one 16-byte piece of each array per thread");
+        reinterpret_cast<uint4 *>(hkey)[tid] = make_uint4(~0u, ~0u, ~0u, ~0u);
+        if (tid < HT_SLOTS / 8)
+            reinterpret_cast<uint4 *>(hcnt)[tid] = make_uint4(0u, 0u, 0u, 0u);
     }
     /* B: the largest bound of the row's wavefronts (they sit in the first W <= 128 threads) */
     if (wv < 2) {
@@ -348,11 +352,21 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     bool           give_up = bk == 0xffffffffu;
     const uint32_t lo      = bk < KEY_LOWEST_FINITE ? KEY_LOWEST_FINITE : bk;
     const float    B       = key2f(lo);
+    /* With penalties: the row's history goes into an open-addressing table in LDS (ids and how
+     * often each occurs). The first attempt at each id's slot is issued here and settled after
+     * the candidates have been listed, so that the two round trips overlap. */
+    const bool     have0 = PEN && (unsigned) hid0 < (unsigned) rv.n_vocab;
+    const bool     have1 = PEN && (unsigned) hid1 < (unsigned) rv.n_vocab;
+    const uint32_t hs0 = hist_hash(hid0), hs1 = hist_hash(hid1);
+    int            old0 = 0, old1 = 0;
+    if (have0)
+        old0 = atomicCAS(&hkey[hs0], -1, hid0);
+    if (have1)
+        old1 = atomicCAS(&hkey[hs1], -1, hid1);
     /* this wavefront's elements at or above B, into its list in LDS. A lane's place is the
      * number of kept elements before it; what is not kept is written to the lane's spare slot,
      * so that no branch is needed. */
     unsigned n_e = 0;
-    uint32_t mxk = 0u; /* largest key among this lane's elements */
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
 #pragma unroll
@@ -363,93 +377,65 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
             const unsigned p    = n_e + lanes_before(mk);
             const bool     put  = keep && p < (unsigned) FC_LIST;
             const unsigned at   = put ? p : (unsigned) (FC_LIST + lane);
-            const uint32_t ky   = f2key(xc);
-            e_val[at]           = PEN ? __float_as_uint(xc) : ky;
+            e_val[at]           = PEN ? __float_as_uint(xc) : f2key(xc);
             e_idx[at]           = (uint32_t) (gi[r] + c);
-            mxk                 = put && ky > mxk ? ky : mxk;
             n_e += (unsigned) __popcll(mk);
         }
     }
     give_up = give_up || n_e > (unsigned) FC_LIST;
     GS_PHASE(2);
-    if (PEN && !give_up) {
-        /* the candidates' ids go into an open-addressing table in LDS ... */
-        wave_lds_sync();
-        if (lane < (int) n_e) {
-            const int id = (int) e_idx[lane];
-            uint32_t  h  = cand_hash(id);
-            bool      in = false;
-#pragma unroll 1
-            for (int pr = 0; pr < CAND_PROBES && !in; ++pr) {
-                in = atomicCAS(&hkey[h], -1, id) == -1;
-                h  = (h + 1u) & (CAND_HASH - 1);
-            }
-            give_up = !in;
-        }
-    }
-    if (give_up)
-        s_c.give_up = 1;
-    if (!PEN) { /* (with penalties the keys are not final yet) */
-        mxk = wave_max_u32(mxk);
-        if (lane == 0 && n_e) {
-            atomicMax(&s_c.mx, mxk);
-            atomicAdd(&s_c.n_real, (int) n_e);
-        }
-    }
-    if (lane == 0)
-        s_c.n_el[wv] = (int) n_e;
-    __syncthreads();
-    GS_PHASE(3);
-    give_up = s_c.give_up != 0;
     if (PEN) {
-        if (!give_up) {
-            /* ... every id of the row's history is looked up there and counted at its
-             * candidate's slot */
-            auto look = [&](int id) {
-                if ((unsigned) id >= (unsigned) rv.n_vocab)
-                    return;
-                uint32_t hq = cand_hash(id);
-                int      kq = hkey[hq];
+        /* claim the slot or find it taken by the same id, then count (16-bit counters, two a
+         * word: a history holds fewer than 65536 ids) */
+        auto settle = [&](int id, uint32_t h, int old) {
 #pragma unroll 1
-                for (int pr = 0; pr < CAND_PROBES && kq != id && kq != -1; ++pr) {
-                    hq = (hq + 1u) & (CAND_HASH - 1);
-                    kq = hkey[hq];
-                }
-                if (kq == id)
-                    atomicAdd(&hcnt[hq], 1u);
-            };
-            look(hid0);
-            look(hid1);
-            const int32_t *h = rv.hist + (long) row * rv.hist_ld;
-#pragma unroll 1
-            for (int i = 2 * FC_THREADS + tid; i < hlen; i += FC_THREADS)
-                look(h[i]);
-        }
+            for (int pr = 0; pr < HT_SLOTS && old != -1 && old != id; ++pr) {
+                h   = (h + 1u) & (HT_SLOTS - 1);
+                old = atomicCAS(&hkey[h], -1, id);
+            }
+            atomicAdd(&hcnt[h >> 1], 1u << (16 * (h & 1u)));
+        };
+        if (have0)
+            settle(hid0, hs0, old0);
+        if (have1)
+            settle(hid1, hs1, old1);
         __syncthreads();
-        GS_PHASE(4);
-        /* each wavefront penalises its own elements; one that no longer reaches B gets key 0 */
-        uint32_t ky = 0u;
-        if (!give_up && lane < (int) n_e) {
+    }
+    /* one element per lane from here on. With penalties: how often the row's history names it
+     * is read from the table; an element that no longer reaches B gets key 0. */
+    wave_lds_sync();
+    uint32_t my_key = 0u;
+    if (!give_up && lane < (int) n_e) {
+        my_key = e_val[lane];
+        if (PEN) {
             const int id = (int) e_idx[lane];
-            float     x  = __uint_as_float(e_val[lane]);
-            uint32_t  hq = cand_hash(id);
+            float     x  = __uint_as_float(my_key);
+            uint32_t  hq = hist_hash(id);
+            int       kq = hkey[hq];
 #pragma unroll 1
-            for (int pr = 0; pr < CAND_PROBES && hkey[hq] != id; ++pr)
-                hq = (hq + 1u) & (CAND_HASH - 1);
-            const uint32_t hc = hcnt[hq];
-            if (hc)
-                x = penalise(x, hc, rv.rep, rv.inv_rep, rv.freq, rv.pres);
-            ky          = x >= B ? f2key(x) : 0u;
-            e_val[lane] = ky;
+            for (int pr = 0; pr < HT_SLOTS && kq != id && kq != -1; ++pr) {
+                hq = (hq + 1u) & (HT_SLOTS - 1);
+                kq = hkey[hq];
+            }
+            if (kq == id)
+                x = penalise(x, (hcnt[hq >> 1] >> (16 * (hq & 1u))) & 0xffffu, rv.rep, rv.inv_rep,
+                             rv.freq, rv.pres);
+            my_key = x >= B ? f2key(x) : 0u;
         }
-        const int real = __popcll(ballot64(ky != 0u));
-        mxk            = wave_max_u32(ky);
+    }
+    {
+        const int      real = __popcll(ballot64(my_key != 0u));
+        const uint32_t mxk  = wave_max_u32(my_key);
         if (lane == 0 && real) {
             atomicMax(&s_c.mx, mxk);
             atomicAdd(&s_c.n_real, real);
         }
-        __syncthreads();
     }
+    if (give_up)
+        s_c.give_up = 1;
+    __syncthreads();
+    GS_PHASE(3);
+    give_up = s_c.give_up != 0;
     GS_PHASE(5);
     /* The k largest. The keys lie in [lo, mx]; 256 bins over that range, counted by all
      * wavefronts, then every wavefront finds the bin in which the count from above reaches k.
@@ -457,8 +443,7 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
      * bin is split again. */
     const int n_real = s_c.n_real;
     give_up = give_up || n_real < a.k; /* fewer than k at or above B: B certifies nothing */
-    const uint32_t my_key = lane < (int) n_e ? e_val[lane] : 0u;
-    uint32_t       cut    = lo;        /* entries with key >= cut are listed */
+    uint32_t cut = lo; /* entries with key >= cut are listed */
     if (!give_up && n_real > CAND_CUT_MAX) {
         uint32_t base_k = lo, top_k = s_c.mx; /* the range being split, inclusive */
         int      need        = a.k;       /* entries wanted from this range: its `need` largest */
@@ -553,10 +538,7 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     GS_PHASE(8);
 #ifdef GS_PHASES
     if (tid == 0) {
-        int t = 0;
-        for (int w = 0; w < FC_WAVES; ++w)
-            t += s_c.n_el[w];
-        g_phase[blockIdx.x * 16 + 12] = t;
+        g_phase[blockIdx.x * 16 + 12] = 0;
         g_phase[blockIdx.x * 16 + 13] = s_c.n_real;
         g_phase[blockIdx.x * 16 + 14] = s_c.n_cut;
         g_phase[blockIdx.x * 16 + 15] = give_up;
