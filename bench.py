@@ -35,12 +35,11 @@ HBM_PEAK_GBS = 8000.0
 COLD_WORKING_SET = 640 * 1024 * 1024   # bytes of logits the timed loops cycle through
 
 # HBM bytes moved by one launch of the streaming kernel, from rocprofv3's FETCH_SIZE and
-# WRITE_SIZE scaled by what the same counters read for a plain copy of the logit buffer
-# (fetch x 1.9985, write x 1.0000); the summaries are profiles/k_tmax_scan_k_final_topk__*.md.
-# A counter run cannot happen inside a timed benchmark, so the figure is carried here.
+# WRITE_SIZE scaled by what the same counters read for a plain copy of the logit buffer. A
+# counter run cannot happen inside a timed benchmark, so the figure is carried here together
+# with the summary it was taken from (`roofline.traffic_source`); workloads without a counter
+# run report null.
 PROFILED_TRAFFIC = {
-    "cfg2_b64_v128256_pen2048": 33950691,
-    "cfg2_b64_v128256": 33950691,
 }
 
 
@@ -200,19 +199,23 @@ def bench_lm_head(args, m_rows, q8=False):
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
     # the projection alone
     f64_batch = (not q8) and m_rows > 1   # what project_sample runs for more than one F16 row
-    if q8:
-        kernel_us = hs.time_q8w_gemv(tables_q8, scales, normed, logits, args.steps)
-    elif not f64_batch:
-        kernel_us = hs.time_f16_gemv(tables, normed, logits, args.steps)
-    else:
-        for i in range(3):
-            hs.f16_linear(tables[i % len(tables)], normed, logits)
-        hs.sync()
-        t1 = time.perf_counter()
+    from geistlib_amd.bench_hooks import Timer
+
+    def projection(i):
+        j = i % len(tables)
+        if q8:
+            hs.q8w_gemv(tables_q8[j], scales[j], normed, logits)
+        elif not f64_batch:
+            hs.f16_gemv(tables[j], normed, logits)
+        else:
+            hs.f16_linear(tables[j], normed, logits)
+
+    for i in range(len(tables)):
+        projection(i)
+    with Timer() as tm:       # HIP events on the sampler's stream around the launches
         for i in range(args.steps):
-            hs.f16_linear(tables[i % len(tables)], normed, logits)
-        hs.sync()
-        kernel_us = (time.perf_counter() - t1) * 1e6 / args.steps
+            projection(i)
+    kernel_us = tm.ms * 1e3 / args.steps
     w_bytes = vocab * d_model + vocab * 4 if q8 else vocab * d_model * 2
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -320,6 +323,12 @@ class _DevPtr:
     def data_ptr(self):
         return self.ptr
 
+    def is_contiguous(self):
+        return True
+
+    def element_size(self):
+        return 1
+
 
 def bench_lm_head_spec(args):
     """Workload lm_head_spec: the tail of a greedy decode step for BitNet-2B-4T's geometry through
@@ -362,9 +371,15 @@ def bench_lm_head_spec(args):
     # the projection over the sketch alone
     act = torch.randint(-127, 128, (1, sd), device=dev, generator=g).to(torch.float32)
     rough = torch.empty((1, vocab), dtype=torch.float32, device=dev)
-    kernel_us = hs.time_q8w_gemv([_DevPtr(v.d_sketch, (vocab, sd)) for v in views],
-                                 [_DevPtr(v.d_row_scale, (vocab,)) for v in views], act, rough,
-                                 args.steps)
+    from geistlib_amd.bench_hooks import Timer
+    sketches = [_DevPtr(v.d_sketch, (vocab, sd)) for v in views]
+    row_scales = [_DevPtr(v.d_row_scale, (vocab,)) for v in views]
+    for i in range(len(views)):
+        hs.q8w_gemv(sketches[i], row_scales[i], act, rough)
+    with Timer() as tm:
+        for i in range(args.steps):
+            hs.q8w_gemv(sketches[i % len(views)], row_scales[i % len(views)], act, rough)
+    kernel_us = tm.ms * 1e3 / args.steps
     k_bytes = vocab * sd + vocab * 4
     achieved = k_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -480,9 +495,17 @@ def main():
     def step(i=0):
         hs.sample(rows_cold[i % n_copies], prm, d_u, d_out)
 
+    from geistlib_amd import bench_hooks as bh
+
     # The cold legs tell the sampler what they are: logits that come from HBM and are read once
     # (GEIST_HIP_LOGITS_STREAMED). The cache-resident legs run with the default hint.
     hs.set_logits_hint(True)
+    # Untimed and reported: one pass over every copy before the counted warm-up, so that a short
+    # run (the driver's 20 steps) does not time first touches of 690 MB and idle clocks.
+    prewarm = 3 * n_copies
+    for i in range(prewarm):
+        step(i)
+    hs.sync()
     for i in range(args.warmup):
         step(i)
     hs.sync()
@@ -513,13 +536,14 @@ def main():
     # the logit-streaming kernel on its own: HIP events on the sampler's stream around K
     # back-to-back launches of that kernel (same configuration), again over the rotating copies
     hs.set_logits_hint(True)
-    kernel_us = hs.time_stream_kernel_multi(rows_cold, prm, d_u, d_out, args.steps)
+    kernel_us, kernel_name = bh.time_stream_kernel(hs, rows_cold, prm, d_u, d_out, args.steps)
     # calibration: a kernel that only reads the same rows with the same geometry
-    plain_us = hs.time_plain_read(rows_cold, args.steps)
+    plain_us = bh.time_plain_read(rows_cold, args.steps, streamed=True)
     hs.set_logits_hint(False)
-    plain_us_resident = None if args.cold_only else hs.time_plain_read([rows], args.steps)
+    plain_us_resident = None if args.cold_only else bh.time_plain_read([rows], args.steps,
+                                                                       streamed=False)
     kernel_us_resident = (None if args.cold_only
-                          else hs.time_stream_kernel(rows, prm, d_u, d_out, args.steps))
+                          else bh.time_stream_kernel(hs, [rows], prm, d_u, d_out, args.steps)[0])
     hs.set_logits_hint(True)
 
     # one-step latency: enqueue + wait, median
@@ -557,11 +581,13 @@ def main():
         "rows_per_s_cache_resident": None if ms_resident is None else round(
             w.rows / (ms_resident * 1e-3), 1),
         "input_copies_rotated": n_copies,
+        "prewarm_steps": prewarm,
         "step_latency_us_median": round(lat[len(lat) // 2], 2) if lat else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": PROFILED_TRAFFIC.get(w.name),
-                     "kernel": "k_tmax_scan" if (w.top_k > 1 or w.temperature <= 0) else "k_chunk_expsum",
+                     "traffic": PROFILED_TRAFFIC.get(w.name, (None, None))[0],
+                     "traffic_source": PROFILED_TRAFFIC.get(w.name, (None, None))[1],
+                     "kernel": kernel_name,
                      "kernel_us": round(kernel_us, 3),
                      "kernel_us_cache_resident": None if kernel_us_resident is None else round(
                          kernel_us_resident, 3),

@@ -79,6 +79,7 @@ def load_library():
     lib.geist_hip_sampler_set_stream.argtypes = [vp, vp]
     lib.geist_hip_sampler_set_logits_hint.argtypes = [vp, i32]
     lib.geist_hip_sampler_set_projection.argtypes = [vp, i32]
+    lib.geist_hip_sampler_prepare.argtypes = [vp, C.POINTER(SampleParams), sz]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -93,15 +94,8 @@ def load_library():
     lib.geist_hip_free.argtypes = [vp, vp]
     lib.geist_hip_upload.argtypes = [vp, vp, vp, sz]
     lib.geist_hip_download.argtypes = [vp, vp, vp, sz]
-    lib.geist_hip_sampler_time_stream_kernel.argtypes = [vp, C.POINTER(Rows),
-                                                         C.POINTER(SampleParams), vp, vp, i32,
-                                                         C.POINTER(C.c_double)]
-    lib.geist_hip_sampler_time_stream_kernel_multi.argtypes = [vp, C.POINTER(Rows), sz,
-                                                               C.POINTER(SampleParams), vp, vp, i32,
-                                                               C.POINTER(C.c_double)]
-    lib.geist_hip_sampler_time_plain_read.argtypes = [vp, C.POINTER(Rows), sz, i32,
-                                                      C.POINTER(C.c_double)]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
+    lib.geist_hip_sampler_topk_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
     lib.geist_hip_propose_drafts_ngram.argtypes = [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, vp, vp]
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
@@ -111,13 +105,9 @@ def load_library():
     lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
                                                   C.POINTER(SampleParams), vp, vp, i32, vp]
-    lib.geist_hip_time_f16_gemv_rows.argtypes = [vp, C.POINTER(vp), sz, sz, sz, vp, sz, sz, vp, sz,
-                                                 i32, C.POINTER(C.c_double)]
     lib.geist_hip_project_sample_rows_q8w.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, vp, sz, vp,
                                                       vp, sz, C.POINTER(SampleParams), vp, vp,
                                                       i32, vp]
-    lib.geist_hip_time_q8w_gemv_rows.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), sz, sz, sz, vp,
-                                                 sz, sz, vp, sz, i32, C.POINTER(C.c_double)]
     lib.geist_hip_spec_head_geometry.argtypes = [sz, sz, sz, sz, C.POINTER(sz), C.POINTER(sz)]
     lib.geist_hip_spec_head_build.argtypes = [vp, vp, sz, sz, sz, sz, C.POINTER(vp)]
     lib.geist_hip_spec_head_destroy.argtypes = [vp, vp]
@@ -168,6 +158,11 @@ class HipSampler:
     def _check(self, rc):
         if rc != GEIST_HIP_OK:
             raise GeistHipError(rc, self.lib.geist_hip_sampler_last_error(self.h).decode())
+
+    def prepare(self, params, n_vocab=0):
+        """Sizes whatever workspace `params` needs beyond the sampler's own, ahead of the first
+        sampling call (the reference does so when a session's options are applied)."""
+        self._check(self.lib.geist_hip_sampler_prepare(self.h, C.byref(params), int(n_vocab)))
 
     def set_stream(self, stream_ptr):
         self._check(self.lib.geist_hip_sampler_set_stream(self.h, stream_ptr))
@@ -350,57 +345,6 @@ class HipSampler:
         self._check(self.lib.geist_hip_spec_head_try_hidden(
             self.h, sh, _ptr(hidden), _ptr(norm_w), eps, _ptr(normed), int(verify), _ptr(result)))
 
-    def time_q8w_gemv(self, weight_copies, scale_copies, x, y, launches):
-        """As time_f16_gemv for q8w_gemv."""
-        n_out, n_in = weight_copies[0].shape
-        m = x.shape[0]
-        wa = (C.c_void_p * len(weight_copies))(*[w.data_ptr() for w in weight_copies])
-        sa = (C.c_void_p * len(scale_copies))(*[w.data_ptr() for w in scale_copies])
-        ms = C.c_double()
-        self._check(self.lib.geist_hip_time_q8w_gemv_rows(
-            self.h, wa, sa, len(weight_copies), n_out, n_in, _ptr(x),
-            x.stride(0) if m > 1 else n_in, m, _ptr(y), y.stride(0) if m > 1 else n_out,
-            int(launches), C.byref(ms)))
-        return ms.value * 1e3 / launches
-
-    def time_f16_gemv(self, weight_copies, x, y, launches):
-        """Mean duration in microseconds of one f16_gemv call (HIP events on the sampler's stream
-        around `launches` back-to-back calls rotating over the weight copies)."""
-        n_out, n_in = weight_copies[0].shape
-        m = x.shape[0]
-        arr = (C.c_void_p * len(weight_copies))(*[w.data_ptr() for w in weight_copies])
-        ms = C.c_double()
-        self._check(self.lib.geist_hip_time_f16_gemv_rows(
-            self.h, arr, len(weight_copies), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in,
-            m, _ptr(y), y.stride(0) if m > 1 else n_out, int(launches), C.byref(ms)))
-        return ms.value * 1e3 / launches
-
-    def time_stream_kernel(self, rows, params, uniforms, out, launches):
-        """Mean duration in microseconds of the logit-streaming kernel alone (HIP events around
-        `launches` back-to-back launches on the sampler's stream)."""
-        ms = C.c_double()
-        self._check(self.lib.geist_hip_sampler_time_stream_kernel(
-            self.h, C.byref(rows), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
-            C.byref(ms)))
-        return ms.value * 1e3 / launches
-
-    def time_stream_kernel_multi(self, rows_list, params, uniforms, out, launches):
-        """As time_stream_kernel, launch i reading rows_list[i % len(rows_list)]."""
-        arr = (Rows * len(rows_list))(*rows_list)
-        ms = C.c_double()
-        self._check(self.lib.geist_hip_sampler_time_stream_kernel_multi(
-            self.h, arr, len(rows_list), C.byref(params), _ptr(uniforms), _ptr(out), int(launches),
-            C.byref(ms)))
-        return ms.value * 1e3 / launches
-
-    def time_plain_read(self, rows_list, launches):
-        """Mean duration in microseconds of a kernel that only reads the rows (calibration)."""
-        arr = (Rows * len(rows_list))(*rows_list)
-        ms = C.c_double()
-        self._check(self.lib.geist_hip_sampler_time_plain_read(self.h, arr, len(rows_list),
-                                                               int(launches), C.byref(ms)))
-        return ms.value * 1e3 / launches
-
     def logprob(self, logits, tokens, out, softcap=0.0):
         """out[r, j] = log_softmax(logits[r])[tokens[r, j]] (float64), logits soft-capped first
         when softcap > 0."""
@@ -409,6 +353,15 @@ class HipSampler:
         self._check(self.lib.geist_hip_logprob_rows(
             self.h, _ptr(logits), logits.stride(0), rows, n, softcap, _ptr(tokens),
             tokens.stride(0), tokens.shape[1], _ptr(out), out.stride(0)))
+
+    def topk_paths(self, rows):
+        """Which path served each row of the last top-k call (0 candidates handed on by the scan,
+        1 per-thread maxima, 2 whole row; -1: the call did not take the candidate path)."""
+        import numpy as np
+        out = np.zeros(int(rows), dtype=np.int32)
+        self._check(self.lib.geist_hip_sampler_topk_paths(self.h, out.ctypes.data_as(C.c_void_p),
+                                                          int(rows)))
+        return out
 
     def row_paths(self, rows):
         """Which walk served each row of the last full-vocabulary top-p / min-p call

@@ -20,6 +20,7 @@
 #include "lm_head_kernels.h"
 #include "spec_head_kernels.h"
 #include "sampler_kernels.h"
+#include "sampler_host.h"
 
 using namespace gs;
 
@@ -52,7 +53,7 @@ struct geist_hip_sampler {
                                      * n_out <= f64_out, allocated on first use */
     size_t   f64_in = 0, f64_out = 0;
 
-    bool stream_kernel_only = false; /* see geist_hip_sampler_time_stream_kernel */
+    size_t topk_paths_rows  = 0;     /* rows of the last top-k call that took the candidate path */ /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
     bool projection_portable = false; /* see geist_hip_sampler_set_projection */
     bool tmax_ready         = false; /* the projection has written the top-k scan's thread maxima
@@ -78,17 +79,6 @@ static int fail(geist_hip_sampler *s, int code, const char *fmt, ...) {
             return fail((s), e_ == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND, \
                         "%s: %s", #call, hipGetErrorString(e_));                               \
     } while (0)
-
-/* Two events for a timed region; neither is left behind when the second cannot be made. */
-static int event_pair(geist_hip_sampler *s, hipEvent_t *a, hipEvent_t *b) {
-    HIPCHK(s, hipEventCreate(a));
-    const hipError_t e = hipEventCreate(b);
-    if (e != hipSuccess) {
-        (void) hipEventDestroy(*a);
-        return fail(s, GEIST_HIP_E_BACKEND, "hipEventCreate: %s", hipGetErrorString(e));
-    }
-    return GEIST_HIP_OK;
-}
 
 static int after_launch(geist_hip_sampler *s, const char *what) {
     hipError_t e = hipGetLastError();
@@ -166,9 +156,6 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
     return GEIST_HIP_OK;
 }
 
-/* Benchmarks time the logit-streaming kernel of a configuration on its own: while this flag is
- * set, a sampling call enqueues that kernel and nothing after it. */
-static inline bool stream_only(const geist_hip_sampler *s) { return s->stream_kernel_only; }
 
 /* ---- sampling without any allocation --------------------------------------------------------
  * The workspace of geist_hip_sample_rows_static: a device array that belongs to the code object,
@@ -395,6 +382,52 @@ static int resolve(geist_hip_sampler *s, const struct geist_hip_sample_params *p
 static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                        const struct geist_hip_sample_params *params, const float *d_uniforms,
                        geist_hip_token_t *d_out) {
+    return gs_host::sample_stages(s, rows, params, d_uniforms, d_out, gs_host::STAGE_ALL, nullptr);
+}
+
+/* The buffers of the full-vocabulary top-p / min-p path (a row of probabilities per logit row
+ * among them: hence not part of every sampler). All or nothing: a failure leaves no pointer set. */
+static int reserve_sorted_workspace(geist_hip_sampler *s) {
+    if (s->probs)
+        return GEIST_HIP_OK;
+    const size_t  R = s->max_rows;
+    gs::CandSpace c = {};
+    float        *probs = nullptr;
+    hipError_t    e = hipSetDevice(s->device);
+    if (e == hipSuccess) e = hipMalloc((void **) &c.row_bound, R * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.out_key, R * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.key, R * CAND_CAP * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.idx, R * CAND_CAP * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.count, R * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.row_sum, R * sizeof(double));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.path, R * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &probs, R * s->max_vocab * sizeof(float));
+    if (e != hipSuccess) {
+        void *ptrs[] = {c.row_bound, c.out_key, c.key, c.idx, c.count, c.row_sum, c.path, probs};
+        for (void *q : ptrs)
+            if (q)
+                (void) hipFree(q);
+        return fail(s, e == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND,
+                    "workspace of the top-p / min-p path: %s", hipGetErrorString(e));
+    }
+    s->cand  = c;
+    s->probs = probs;
+    return GEIST_HIP_OK;
+}
+
+} /* extern "C" */
+
+/* One sampling call is enqueued in up to three stages: a first pass over the rows where the mode
+ * needs two (the row maxima before the exp-sum), the pass that streams the logits, and what
+ * follows it per row. geist_hip_sample_rows runs all three. */
+int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                           const struct geist_hip_sample_params *params, const float *d_uniforms,
+                           geist_hip_token_t *d_out, unsigned stages, const char **stream_kernel) {
+    const bool do_pre = stages & gs_host::STAGE_PRE, do_stream = stages & gs_host::STAGE_STREAM,
+               do_tail = stages & gs_host::STAGE_TAIL;
+    const char *unused_name;
+    if (!stream_kernel)
+        stream_kernel = &unused_name;
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     if (!d_out)
@@ -423,19 +456,21 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
 
     if (rs.greedy) {
         L.rv.stream_loads = s->logits_streamed;
-        launch_tmax_scan(L, s->tmax, s->chunk_best);
-        if (stream_only(s))
-            return after_launch(s, "argmax scan");
+        *stream_kernel    = "k_tmax_scan";
+        if (do_stream)
+            launch_tmax_scan(L, s->tmax, s->chunk_best);
         f.mode = FINAL_ARGMAX;
-        launch_row_final(L, f);
+        if (do_tail)
+            launch_row_final(L, f);
         return after_launch(s, "argmax");
     }
     if (rs.use_k) {
         if (rs.k > TOPK_FAST_MAX) {
-            f.mode = FINAL_TOPK;
-            f.k    = rs.k;
-                const int e = launch_topk_general(L, f);
-                if (e != 0)
+            f.mode         = FINAL_TOPK;
+            f.k            = rs.k;
+            *stream_kernel = "k_topk_general";
+            const int e    = do_stream ? launch_topk_general(L, f) : 0;
+            if (e != 0)
                 return fail(s, GEIST_HIP_E_BACKEND, "top-k (general) launch: %s",
                             hipGetErrorString((hipError_t) e));
             return after_launch(s, "top-k (general)");
@@ -476,43 +511,40 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
         const int m = plain ? cand_lanes_for(f.k_sel, rows->n_vocab) : 0;
         if (m) {
             const WaveCands wc = wave_cands_at(s->wcands, row_waves);
-            launch_cand_scan(scan, s->tmax, wc, m);
-            if (stream_only(s))
-                return after_launch(s, "top-k scan");
-            launch_final_cand(L, f, wc);
+            f.row_flag         = s->row_flag; /* which path served each row, for diagnostics */
+            s->topk_paths_rows = rows->rows;
+            *stream_kernel     = "k_cand_scan";
+            if (do_stream)
+                launch_cand_scan(scan, s->tmax, wc, m);
+            if (do_tail)
+                launch_final_cand(L, f, wc);
             return after_launch(s, "top-k");
         }
-        if (!s->tmax_ready)
+        s->topk_paths_rows = 0;
+        *stream_kernel     = "k_tmax_scan";
+        if (!s->tmax_ready && do_stream)
             launch_tmax_scan(scan, s->tmax, nullptr);
-        if (stream_only(s))
-            return after_launch(s, "top-k scan");
-        launch_row_final(L, f);
+        if (do_tail)
+            launch_row_final(L, f);
         return after_launch(s, "top-k");
     }
     if (!rs.use_p && !rs.use_m) {
-        if (!stream_only(s))
+        *stream_kernel = "k_chunk_expsum";
+        if (do_pre)
             launch_tmax_scan(L, s->tmax, s->chunk_best);
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr, 0,
-                            s->slab_sum);
-        if (stream_only(s))
-            return after_launch(s, "exp-sum scan");
+        if (do_stream)
+            launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr,
+                                0, s->slab_sum);
         f.mode     = FINAL_TEMPERATURE;
         f.slab_sum = s->slab_sum;
-        launch_row_final(L, f);
+        if (do_tail)
+            launch_row_final(L, f);
         return after_launch(s, "temperature");
     }
     /* top-p and/or min-p over the whole vocabulary */
-    if (!s->probs) {
-        const size_t R = s->max_rows;
-        HIPCHK(s, hipMalloc((void **) &s->cand.row_bound, R * sizeof(int32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.out_key, R * sizeof(uint32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.key, R * CAND_CAP * sizeof(uint32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.idx, R * CAND_CAP * sizeof(uint32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.count, R * sizeof(int32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.row_sum, R * sizeof(double)));
-        HIPCHK(s, hipMalloc((void **) &s->cand.path, R * sizeof(int32_t)));
-        HIPCHK(s, hipMalloc((void **) &s->probs, R * s->max_vocab * sizeof(float)));
-    }
+    rc = reserve_sorted_workspace(s); /* a no-op after geist_hip_sampler_prepare() or a first call */
+    if (rc)
+        return rc;
     L.nv           = 8;
     L.rv.per_chunk = 8192;
     L.rv.n_chunks  = (int) ((rows->n_vocab + 8191) / 8192);
@@ -529,11 +561,14 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
      * the exp-sum pass at once. Below that a flat row may overflow the list, and the row-final
      * kernel should get the chance to bound it by top-p instead. */
     f.minp_direct     = f.minp_listed && rs.min_p >= 0.02f;
-    if (!stream_only(s))
+    *stream_kernel = "k_chunk_expsum";
+    if (do_pre)
         launch_tmax_scan(L, s->tmax, s->chunk_best, f.minp_listed ? s->cand.count : nullptr);
-    launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
-                        f.minp_listed && !stream_only(s) ? &f.cand : nullptr, zb_m);
-    if (stream_only(s))
+    /* (the pass lists candidates only when the pass before it has cleared the lists' counters) */
+    if (do_stream)
+        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
+                            f.minp_listed && do_pre ? &f.cand : nullptr, zb_m);
+    if (!do_tail)
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;
     f.row_flag = s->row_flag;
@@ -549,10 +584,25 @@ static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     return after_launch(s, "top-p / min-p");
 }
 
+extern "C" {
+
 int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                           const struct geist_hip_sample_params *params, const float *d_uniforms,
                           geist_hip_token_t *d_out_tokens) {
     return sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+}
+
+int geist_hip_sampler_prepare(geist_hip_sampler *s, const struct geist_hip_sample_params *params,
+                              size_t n_vocab) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    Resolved rs;
+    int      rc = resolve(s, params, n_vocab ? n_vocab : s->max_vocab, rs);
+    if (rc)
+        return rc;
+    if (!rs.greedy && !rs.use_k && (rs.use_p || rs.use_m))
+        rc = reserve_sorted_workspace(s);
+    return rc;
 }
 
 int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hip_rows *rows,
@@ -1088,120 +1138,6 @@ int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, siz
     return GEIST_HIP_OK;
 }
 
-int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
-                                               const struct geist_hip_rows *rows, size_t n_batches,
-                                               const struct geist_hip_sample_params *params,
-                                               const float *d_uniforms,
-                                               geist_hip_token_t *d_out_tokens, int launches,
-                                               double *ms_total) {
-    if (!s)
-        return GEIST_HIP_E_INVALID_ARG;
-    if (launches < 1 || !ms_total || !rows || n_batches < 1)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
-    hipEvent_t a, b;
-    HIPCHK(s, hipSetDevice(s->device));
-    if (const int ev = event_pair(s, &a, &b))
-        return ev;
-    /* a complete call first, so that the kernel finds the inputs an earlier stage leaves it */
-    int rc = 0;
-    for (size_t i = 0; i < n_batches && !rc; ++i)
-        rc = sample_impl(s, &rows[i], params, d_uniforms, d_out_tokens);
-    s->stream_kernel_only = true;
-    for (size_t i = 0; i < n_batches && !rc; ++i) /* warm the code object, cycle the caches */
-        rc = sample_impl(s, &rows[i], params, d_uniforms, d_out_tokens);
-    if (!rc)
-        rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
-    for (int i = 0; i < launches && !rc; ++i)
-        rc = sample_impl(s, &rows[(size_t) i % n_batches], params, d_uniforms, d_out_tokens);
-    s->stream_kernel_only = false;
-    float ms = 0.0f;
-    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
-                hipEventElapsedTime(&ms, a, b) != hipSuccess))
-        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
-    (void) hipEventDestroy(a);
-    (void) hipEventDestroy(b);
-    *ms_total = ms;
-    return rc;
-}
-
-int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geist_hip_rows *rows,
-                                         const struct geist_hip_sample_params *params,
-                                         const float *d_uniforms, geist_hip_token_t *d_out_tokens,
-                                         int launches, double *ms_total) {
-    return geist_hip_sampler_time_stream_kernel_multi(s, rows, 1, params, d_uniforms, d_out_tokens,
-                                                      launches, ms_total);
-}
-
-int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_hip_rows *rows,
-                                      size_t n_batches, int launches, double *ms_total) {
-    if (!s)
-        return GEIST_HIP_E_INVALID_ARG;
-    if (launches < 1 || !ms_total || !rows || n_batches < 1)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no batch or null result");
-    std::vector<Launch> L;
-    try { /* no exception leaves a C entry point */
-        L.resize(n_batches);
-    } catch (const std::bad_alloc &) {
-        return fail(s, GEIST_HIP_E_OOM, "plain read: %zu batches", n_batches);
-    }
-    for (size_t i = 0; i < n_batches; ++i) {
-        const int rc = make_launch(s, &rows[i], nullptr, false, L[i]);
-        if (rc)
-            return rc;
-        L[i].rv.stream_loads = s->logits_streamed;
-        L[i].nv           = 8; /* the geometry of the top-k scan */
-        L[i].rv.per_chunk = 8192;
-        L[i].rv.n_chunks  = (int) ((rows[i].n_vocab + 8191) / 8192);
-    }
-    hipEvent_t a, b;
-    HIPCHK(s, hipSetDevice(s->device));
-    if (const int ev = event_pair(s, &a, &b))
-        return ev;
-    for (size_t i = 0; i < n_batches; ++i)
-        launch_plain_read(L[i], s->uniforms);
-    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
-    for (int i = 0; i < launches && !rc; ++i)
-        launch_plain_read(L[(size_t) i % n_batches], s->uniforms);
-    float ms = 0.0f;
-    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
-                hipEventElapsedTime(&ms, a, b) != hipSuccess))
-        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
-    (void) hipEventDestroy(a);
-    (void) hipEventDestroy(b);
-    *ms_total = ms;
-    return rc ? rc : after_launch(s, "plain read");
-}
-
-int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_w_f16,
-                                 size_t n_weights, size_t n_out, size_t n_in, const float *d_x,
-                                 size_t ld_x, size_t n_rows, float *d_y, size_t ld_y, int launches,
-                                 double *ms_total) {
-    if (!s)
-        return GEIST_HIP_E_INVALID_ARG;
-    if (launches < 1 || !ms_total || !d_w_f16 || n_weights < 1)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no weights or null result");
-    for (size_t i = 0; i < n_weights; ++i) { /* argument checks and a warm-up of each copy */
-        const int rc = geist_hip_f16_gemv_rows(s, d_w_f16[i], n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
-        if (rc)
-            return rc;
-    }
-    hipEvent_t a, b;
-    if (const int ev = event_pair(s, &a, &b))
-        return ev;
-    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
-    for (int i = 0; i < launches && !rc; ++i)
-        rc = geist_hip_f16_gemv_rows(s, d_w_f16[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
-                                     n_rows, d_y, ld_y);
-    float ms = 0.0f;
-    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
-                hipEventElapsedTime(&ms, a, b) != hipSuccess))
-        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
-    (void) hipEventDestroy(a);
-    (void) hipEventDestroy(b);
-    *ms_total = ms;
-    return rc;
-}
-
 /* ---- speculative output head -------------------------------------------------------------- */
 
 struct geist_hip_spec_head {
@@ -1381,38 +1317,6 @@ int geist_hip_spec_head_try_hidden(geist_hip_sampler *s, geist_hip_spec_head *sh
     return after_launch(s, "sketch head");
 }
 
-int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,
-                                 const float *const *d_scales, size_t n_weights, size_t n_out,
-                                 size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
-                                 float *d_y, size_t ld_y, int launches, double *ms_total) {
-    if (!s)
-        return GEIST_HIP_E_INVALID_ARG;
-    if (launches < 1 || !ms_total || !d_wq || !d_scales || n_weights < 1)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "launches < 1, no weights or null result");
-    for (size_t i = 0; i < n_weights; ++i) { /* argument checks and a warm-up of each copy */
-        const int rc = geist_hip_q8w_gemv_rows(s, d_wq[i], d_scales[i], n_out, n_in, d_x, ld_x,
-                                               n_rows, d_y, ld_y);
-        if (rc)
-            return rc;
-    }
-    hipEvent_t a, b;
-    if (const int ev = event_pair(s, &a, &b))
-        return ev;
-    int rc = hipEventRecord(a, s->stream) == hipSuccess ? 0 : GEIST_HIP_E_BACKEND;
-    for (int i = 0; i < launches && !rc; ++i)
-        rc = geist_hip_q8w_gemv_rows(s, d_wq[(size_t) i % n_weights],
-                                     d_scales[(size_t) i % n_weights], n_out, n_in, d_x, ld_x,
-                                     n_rows, d_y, ld_y);
-    float ms = 0.0f;
-    if (!rc && (hipEventRecord(b, s->stream) != hipSuccess || hipEventSynchronize(b) != hipSuccess ||
-                hipEventElapsedTime(&ms, a, b) != hipSuccess))
-        rc = fail(s, GEIST_HIP_E_BACKEND, "event timing failed");
-    (void) hipEventDestroy(a);
-    (void) hipEventDestroy(b);
-    *ms_total = ms;
-    return rc;
-}
-
 int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t n,
                              float *d_out_units) {
     if (!s)
@@ -1422,6 +1326,21 @@ int geist_hip_rng_draw_units(geist_hip_sampler *s, uint64_t *d_rng_state, size_t
     HIPCHK(s, hipSetDevice(s->device));
     launch_rng_units(s->stream, d_rng_state, /*shared=*/1, (int) n, d_out_units);
     return after_launch(s, "rng draws");
+}
+
+int geist_hip_sampler_topk_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows) {
+    if (!s || !h_paths)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (rows > s->max_rows)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "rows %zu > max_rows %zu", rows, s->max_rows);
+    if (s->topk_paths_rows == 0 || rows > s->topk_paths_rows) {
+        /* the last top-k call ran the thread-maxima path for every row (or there was none) */
+        HIPCHK(s, hipStreamSynchronize(s->stream));
+        for (size_t r = 0; r < rows; ++r)
+            h_paths[r] = -1;
+        return GEIST_HIP_OK;
+    }
+    return geist_hip_download(s, h_paths, s->row_flag, rows * sizeof(int32_t));
 }
 
 int geist_hip_sampler_row_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows) {

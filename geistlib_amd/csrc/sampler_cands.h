@@ -264,15 +264,15 @@ __device__ __forceinline__ int finish_sorted_lanes(int n, const uint64_t *spack,
     return (int) (0xffffffffu - readlane_u32((uint32_t) mine, at));
 }
 
-static_assert(CAND_GROUPS == 24 && CAND_SLOTS == 32, "the slot-to-thread maps below");
+static_assert(CAND_GROUPS == 32 && CAND_SLOTS == 32, "the slot-to-thread maps below");
 
 /* One workgroup of 1024 threads per row, so that every wavefront has little to do and a SIMD's
  * four wavefronts cover each other's waits. WIDE = false: up to 64 scanning wavefronts per row;
- * thread t reads slots (t & 15) and 16 + (t & 15) (the latter if below CAND_GROUPS) of scanning
- * wavefront t >> 4. WIDE = true: up to 128; slots (t & 7) + 8 r, r < 3, of wavefront t >> 3. */
+ * thread t reads slots (t & 15) and 16 + (t & 15) of scanning wavefront t >> 4. WIDE = true: up
+ * to 128; slots (t & 7) + 8 r, r < 4, of wavefront t >> 3. */
 template <int NV, bool PEN, bool WIDE>
 __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs a, WaveCands wc) {
-    constexpr int ROUNDS = WIDE ? 3 : 2;
+    constexpr int ROUNDS = WIDE ? 4 : 2;
     constexpr int ARENA = CA_END > FallbackArena<NV, PEN>::END ? CA_END : FallbackArena<NV, PEN>::END;
     __shared__ __align__(16) uint8_t s_arena[ARENA];
     __shared__ uint64_t      s_tab[32];

@@ -71,10 +71,10 @@ struct CandSpace {
  * CAND_GROUPS slots. */
 constexpr int NWAVES_PER_CHUNK = 4; /* a chunk is scanned by one workgroup of four wavefronts */
 constexpr int CAND_SLOTS     = 32;  /* float4 groups a wavefront has room for ... */
-constexpr int CAND_GROUPS    = 24;  /* ... and how many it may hand on (the rest is never read) */
+constexpr int CAND_GROUPS    = 32;  /* ... and how many it may hand on */
 constexpr int CAND_CHUNKS_MAX = 32; /* rows of up to 32 chunks of 8192 logits take this path */
 constexpr int CAND_K_MAX     = 64;  /* largest k: the survivors are ordered one per lane */
-constexpr int CAND_LANES_MAX = 18;  /* largest `m` (see k_cand_scan) that leaves room in the slots */
+constexpr int CAND_LANES_MAX = 16;  /* largest `m` (see k_cand_scan) that leaves room in the slots */
 struct WaveCands {
     float4   *val;   /* [rows][waves][CAND_SLOTS] the groups */
     int32_t  *idx;   /* [rows][waves][CAND_SLOTS] index of each group's first element, -1 = unused */
@@ -184,8 +184,6 @@ void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, 
 /* after launch_tmax_scan(L, tmax, chunk_best): out[row][j] = log_softmax(row)[tokens[row][j]] */
 void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,
                     const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld);
-/* calibration: reads the rows as the streaming kernels do and stores nothing */
-void launch_plain_read(const Launch &L, float *sink);
 void launch_ngram_draft(hipStream_t stream, const int32_t *history, long history_ld,
                         const int32_t *history_len, const int32_t *seeds, int n_seq, int k_max,
                         int max_suffix, int32_t *out, long out_ld, int32_t *out_count,

@@ -1421,27 +1421,6 @@ __global__ __launch_bounds__(TPB) void k_final_logprob(RowView rv,
 }
 
 /* ============================================================================================
- * k_plain_read: calibration. Reads the rows with the geometry of the streaming kernels and does
- * nothing else (a maximum nobody stores keeps the loads alive). Its duration is the floor of
- * any one-pass kernel over the same bytes on this device and launch size.
- * ========================================================================================== */
-template <int NV>
-__global__ __launch_bounds__(TPB) void k_plain_read(RowView rv, float *__restrict__ sink) {
-    int row, chunk;
-    xcd_row_chunk(row, chunk);
-    int base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    float4 v[NV];
-    load_raw<NV>(rv, rv.logits + (long) row * rv.ld, base, end, v);
-    float m = -__builtin_inff();
-#pragma unroll
-    for (int j = 0; j < NV; ++j)
-        m = max3f(m, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
-    if (m == 0x1.234568p+100f) /* never among the inputs: nothing is written */
-        sink[0] = m;
-}
-
-/* ============================================================================================
  * k_penalties: in-place penalties; only the penalised positions are written back.
  * ========================================================================================== */
 template <int NV>
@@ -1772,14 +1751,6 @@ void launch_ngram_draft(hipStream_t stream, const int32_t *history, long history
     k_ngram_draft<<<dim3(n_seq), dim3(TPB), 0, stream>>>(history, history_ld, history_len, seeds,
                                                          k_max, max_suffix, out, out_ld, out_count,
                                                          out_match);
-}
-
-void launch_plain_read(const Launch &L, float *sink) {
-    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
-    if (L.nv == 8)
-        k_plain_read<8><<<grid, block, 0, L.stream>>>(L.rv, sink);
-    else
-        k_plain_read<2><<<grid, block, 0, L.stream>>>(L.rv, sink);
 }
 
 void launch_penalties(const Launch &L, float *logits_rw) {

@@ -180,20 +180,6 @@ int geist_hip_spec_head_try_hidden(geist_hip_sampler *s, geist_hip_spec_head *sh
                                    float rms_eps, float *d_normed, int verify,
                                    struct geist_hip_spec_result *d_result);
 
-/* For benchmarks: total duration in milliseconds, from HIP events on the sampler's stream, of
- * `launches` back-to-back geist_hip_f16_gemv_rows calls, call i reading the weight copy
- * d_w_f16[i % n_weights] (several copies keep every call's weights out of the caches). */
-int geist_hip_time_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *const *d_w_f16,
-                                 size_t n_weights, size_t n_out, size_t n_in, const float *d_x,
-                                 size_t ld_x, size_t n_rows, float *d_y, size_t ld_y, int launches,
-                                 double *ms_total);
-/* The same for geist_hip_q8w_gemv_rows: call i reads d_wq[i % n_weights] and d_scales[i %
- * n_weights]. */
-int geist_hip_time_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *const *d_wq,
-                                 const float *const *d_scales, size_t n_weights, size_t n_out,
-                                 size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
-                                 float *d_y, size_t ld_y, int launches, double *ms_total);
-
 #ifdef __cplusplus
 }
 #endif

@@ -126,7 +126,7 @@ int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *row
  * it is for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc: no sampler object is needed and the call allocates nothing, on the host or on the
  * device. Its workspace is an array of device memory inside the library's code object
- * (GEIST_HIP_STATIC_MAX_UNITS x 1104 bytes = 4.3 MiB per GPU, held until the process ends).
+ * (7.2 MiB per GPU, held until the process ends).
  *   device, stream   where the kernels are enqueued (stream NULL = the default stream)
  *   err, err_len     optional buffer for the text of a failure
  * Served: greedy, temperature, and every top-k configuration (with top-p / min-p behind it,
@@ -141,6 +141,15 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
                                  const struct geist_hip_sample_params *params,
                                  const float *d_uniforms, geist_hip_token_t *d_out_tokens,
                                  char *err, size_t err_len);
+
+/* Sizes, ahead of the first sampling call, whatever workspace the configuration needs beyond
+ * what geist_hip_sampler_create made -- the reference sizes its workspace when the options are
+ * applied (transformer_session_apply_opts, src/archs/transformer/forward/step.c:398-409), so that
+ * the per-token call allocates nothing. Today that is the full-vocabulary top-p / min-p path (a
+ * row of probabilities per logit row). n_vocab = 0: the sampler's max_vocab. A sampling call
+ * made without it sizes the same workspace on first use. */
+int geist_hip_sampler_prepare(geist_hip_sampler *s, const struct geist_hip_sample_params *params,
+                              size_t n_vocab);
 
 /* Same, drawing the uniforms on the device from xorshift64* states (struct geist_rng,
  * src/engine/sampler.h:28-32; sampler.c:35-48) held in device memory.
@@ -241,36 +250,17 @@ int geist_hip_free(geist_hip_sampler *s, void *d_ptr);
 int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes);   /* sync */
 int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, size_t bytes); /* sync */
 
-/* For benchmarks (no reference counterpart): enqueues ONLY the logit-streaming kernel of the given
- * configuration `launches` times back to back on the sampler's stream, between two HIP events
- * recorded on that stream, waits, and returns the elapsed milliseconds. Dividing by `launches`
- * gives the mean duration of that kernel (thread-maxima scan for top-k and argmax, exp-sum scan
- * for temperature / top-p / min-p). One complete sampling call is made first. */
-int geist_hip_sampler_time_stream_kernel(geist_hip_sampler *s, const struct geist_hip_rows *rows,
-                                         const struct geist_hip_sample_params *params,
-                                         const float *d_uniforms, geist_hip_token_t *d_out_tokens,
-                                         int launches, double *ms_total);
-
-/* The same over n_batches batches of equal shape, launch i reading rows[i % n_batches]: with
- * enough batches to exceed the caches (256 MB of Infinity Cache on an MI355X) every launch streams
- * its logits from HBM, which is what a roofline against the HBM rate has to time. */
-int geist_hip_sampler_time_stream_kernel_multi(geist_hip_sampler *s,
-                                               const struct geist_hip_rows *rows, size_t n_batches,
-                                               const struct geist_hip_sample_params *params,
-                                               const float *d_uniforms,
-                                               geist_hip_token_t *d_out_tokens, int launches,
-                                               double *ms_total);
-
-/* Calibration for benchmarks (no reference counterpart): the same timing loop around a kernel
- * that only reads the rows, with the launch geometry of the top-k scan, and stores nothing. Its
- * mean duration is the floor of any one-pass kernel over these bytes on this device. */
-int geist_hip_sampler_time_plain_read(geist_hip_sampler *s, const struct geist_hip_rows *rows,
-                                      size_t n_batches, int launches, double *ms_total);
-
 /* Diagnostics (no reference counterpart): after a full-vocabulary top-p / min-p call, which walk
  * served each row: 1 = shortcut over the per-thread maxima, 2 = candidate list, 3 = the whole
  * row. Synchronous; h_paths receives `rows` entries. */
 int geist_hip_sampler_row_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows);
+
+/* Diagnostics (no reference counterpart): after a top-k call, which path served each row:
+ * 0 = the candidates handed on by the scan, 1 = the per-thread maxima (rows whose leading logits
+ * crowd into few wavefronts' elements, runs of equal values), 2 = the selection over the whole
+ * row; -1 for every row when the call did not take the candidate path at all (soft-cap, mask,
+ * unaligned rows, k above 64, penalties that can raise a logit). Synchronous. */
+int geist_hip_sampler_topk_paths(geist_hip_sampler *s, int32_t *h_paths, size_t rows);
 
 #ifdef __cplusplus
 }

@@ -11,6 +11,7 @@ LIBDIR = os.path.join(ROOT, "geistlib_amd", "lib")
 
 HEADERS = {
     "geist_sampler_hip.h": "libgeist_sampler_hip.so",
+    "geist_lm_head_hip.h": "libgeist_sampler_hip.so",
     "geist_sampler_dropin.h": "libgeist_sampler_host.so",
     "geist_head_hip.h": "libgeist_sampler_host.so",
 }
@@ -33,6 +34,19 @@ def test_library_exports_every_declared_symbol(header, lib):
     assert len(names) >= 8
     missing = [n for n in names if not hasattr(handle, n)]
     assert not missing, f"{lib} lacks {missing}"
+
+
+def test_no_measurement_code_in_the_product_abi():
+    """Timing helpers live in libgeist_bench_hip.so (geistlib_amd/bench/), outside include/."""
+    import subprocess
+    for header in os.listdir(os.path.join(ROOT, "include")):
+        assert not [n for n in declared_functions(header) if "_time_" in n or "bench" in n], header
+    for lib in ("libgeist_sampler_hip.so", "libgeist_sampler_host.so"):
+        out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(LIBDIR, lib)],
+                             capture_output=True, text=True, check=True).stdout
+        bad = [l for l in out.splitlines() if "_time_" in l or "plain_read" in l]
+        assert not bad, (lib, bad)
+    assert os.path.exists(os.path.join(LIBDIR, "libgeist_bench_hip.so"))
 
 
 def test_reference_symbol_set_is_complete():

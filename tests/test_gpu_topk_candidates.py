@@ -1,0 +1,149 @@
+"""The candidate path of top-k (the scan's wavefronts hand their leading groups on, the row-final
+kernel gathers nothing) against the oracle, on the rows it was built for and on the rows it has to
+pass on to the thread-maxima path and the whole-row selection. Token ids bit for bit; which path
+served each row is read back and asserted, so that every branch is known to have run."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from gpu_util import compare_ids, run_rows  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def hs():
+    from geistlib_amd import HipSampler
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a device; the sampling path has no CPU fallback")
+    s = HipSampler(max_rows=256, max_vocab=262144)
+    yield s
+    s.close()
+
+
+def P(**kw):
+    from geistlib_amd import SampleParams
+    return SampleParams.make(**kw)
+
+
+def units(g, rows):
+    return (g.integers(0, 1 << 24, rows).astype(np.float32) / np.float32(1 << 24)).astype(np.float32)
+
+
+def want_rows(oracle, x, u, hist=None, pen=None, **kw):
+    res = []
+    for r in range(x.shape[0]):
+        row = x[r] if hist is None else oracle.penalties(x[r], hist[r], *pen)
+        res.append(oracle.chain_u(row, float(u[r]), **kw))
+    return [t for t, _ in res], [i for _, i in res]
+
+
+@pytest.mark.parametrize("n,k", [(128256, 40), (151936, 40), (262144, 64), (32000, 2), (70000, 64),
+                                 (8192 * 3, 17)])
+def test_plain_rows_take_the_candidate_path(hs, oracle, n, k):
+    print(f"candidates n={n} k={k}", flush=True)
+    g = np.random.default_rng(n + k)
+    rows = 24
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    x[1, g.integers(0, n, 5)] += 10        # a few leaders far above the rest
+    x[2] = (g.standard_t(3, n) * 2.5).astype(np.float32)
+    u = units(g, rows)
+    got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9))
+    paths = hs.topk_paths(rows).tolist()
+    want, infos = want_rows(oracle, x, u, temperature=0.7, top_k=k, top_p=0.9)
+    compare_ids(got, want, infos, f"candidates n={n} k={k}")
+    assert paths == [0] * rows, paths
+
+
+def test_rows_the_candidates_cannot_certify(hs, oracle):
+    """Leading logits crowded into one wavefront's elements (a sorted row, a cluster of
+    consecutive ids), runs of equal values across the cut, rows with fewer than k finite logits:
+    each falls back inside the same launch and still gives the oracle's token."""
+    g = np.random.default_rng(5)
+    n, k, rows = 128256, 40, 16
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    x[0] = -np.sort(-x[0])                          # sorted: the top 40 sit in 10 threads
+    x[1, 70000:70040] = x[1].max() + 1 + g.random(40).astype(np.float32)   # a cluster
+    x[2, :] = np.round(x[2])                        # long runs of equal values
+    x[3, :] = 1.5                                   # all equal
+    x[4, :] = -np.inf
+    x[4, g.integers(0, n, 25)] = g.standard_normal(25).astype(np.float32)  # < k finite
+    x[5, ::2] = -np.inf                             # half the row forbidden by value
+    x[6, :1000] = 9.0                               # 1000 equal leaders in the first chunk
+    x[7, n - 3:] = 50.0                             # leaders in the ragged last chunk
+    u = units(g, rows)
+    got = run_rows(hs, torch, x, u, P(temperature=0.8, top_k=k, top_p=0.95))
+    paths = hs.topk_paths(rows).tolist()
+    want, infos = want_rows(oracle, x, u, temperature=0.8, top_k=k, top_p=0.95)
+    compare_ids(got, want, infos, "rows passed on")
+    print("paths:", paths)
+    assert paths[0] != 0 and paths[1] != 0 and paths[2] != 0 and paths[3] != 0 and paths[4] != 0
+    assert paths[5] == 0 and paths[7] == 0 and all(p == 0 for p in paths[8:])
+
+
+@pytest.mark.parametrize("H,dup", [(2048, True), (2048, False), (300, True), (1, False), (0, False)])
+def test_penalties_from_the_history_table(hs, oracle, H, dup):
+    """Penalties on the candidate path: the history goes into a table in LDS. Heavily repeated
+    ids, ids outside the vocabulary, rows with shorter histories, leaders penalised away."""
+    g = np.random.default_rng(100 + H + dup)
+    n, k, rows = 128256, 40, 32
+    Hl = max(H, 4)
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    hist = (g.zipf(1.1, (rows, Hl)) % n if dup else g.integers(0, n, (rows, Hl))).astype(np.int32)
+    lead = np.argsort(-x, axis=1)[:, :60]
+    m = min(Hl, 30)
+    hist[::2, :m] = lead[::2, :m]                   # every other row: its leaders are in the history
+    hist[3, : min(Hl, 3)] = [-1, n, n + 5][: min(Hl, 3)]   # ids outside the vocabulary: ignored
+    hl = np.full(rows, H, dtype=np.int32)
+    hl[5] = H // 2
+    hl[6] = 0
+    u = units(g, rows)
+    for pen in [(1.1, 0.5, 0.3), (1.0, 0.0, 4.0), (3.0, 0.0, 0.0)]:
+        got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9, rep=pen[0],
+                                          freq=pen[1], pres=pen[2]), hist, hl)
+        paths = hs.topk_paths(rows).tolist()
+        hh = [hist[r, :hl[r]] for r in range(rows)]
+        want, infos = want_rows(oracle, x, u, hist=hh, pen=pen, temperature=0.7, top_k=k, top_p=0.9)
+        compare_ids(got, want, infos, f"history table H={H} dup={dup} pen={pen}")
+        assert set(paths) <= {0, 1, 2} and paths.count(0) >= rows // 2, paths
+
+
+def test_penalties_that_empty_the_candidates(hs, oracle):
+    """The 500 leading logits of a row are all penalised far down: fewer than k of the candidates
+    still reach the bound, which then certifies nothing, and the row is passed on."""
+    g = np.random.default_rng(77)
+    n, k, rows, H = 128256, 40, 8, 512
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    hist = g.integers(0, n, (rows, H)).astype(np.int32)
+    hist[:4, :500] = np.argsort(-x[:4], axis=1)[:, :500]
+    hl = np.full(rows, H, dtype=np.int32)
+    u = units(g, rows)
+    got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9, rep=1.0, freq=0.0, pres=8.0),
+                   hist, hl)
+    paths = hs.topk_paths(rows).tolist()
+    want, infos = want_rows(oracle, x, u, hist=hist, pen=(1.0, 0.0, 8.0), temperature=0.7, top_k=k,
+                            top_p=0.9)
+    compare_ids(got, want, infos, "emptied candidates")
+    assert all(p != 0 for p in paths[:4]) and paths[4:] == [0] * 4, paths
+
+
+def test_calls_that_stay_off_the_candidate_path(hs, oracle):
+    """Soft-cap, k above 64, a history longer than the table takes, penalties that can raise a
+    logit: the thread-maxima path serves the whole call, and says so."""
+    g = np.random.default_rng(9)
+    n, rows = 60000, 8
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    u = units(g, rows)
+    hist = g.integers(0, n, (rows, 2500)).astype(np.int32)
+    hl = np.full(rows, 2500, dtype=np.int32)
+    cases = [(dict(temperature=0.7, top_k=100), None, None),
+             (dict(temperature=0.7, top_k=40, rep=1.2), hist, (1.2, 0.0, 0.0)),
+             (dict(temperature=0.7, top_k=40, rep=0.8), hist[:, :100].copy(), (0.8, 0.0, 0.0))]
+    for kw, h, pen in cases:
+        hlen = None if h is None else np.full(rows, h.shape[1], dtype=np.int32)
+        got = run_rows(hs, torch, x, u, P(**kw), h, hlen)
+        assert hs.topk_paths(rows).tolist() == [-1] * rows
+        okw = {k_: v for k_, v in kw.items() if k_ in ("temperature", "top_k", "top_p", "min_p")}
+        want, infos = want_rows(oracle, x, u, hist=h, pen=pen, **okw)
+        compare_ids(got, want, infos, f"off the candidate path {kw}")
