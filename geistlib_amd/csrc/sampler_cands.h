@@ -32,26 +32,7 @@
 
 namespace gs {
 
-#ifdef GS_PHASES
-__device__ long long g_phase[4096 * 16];
-#define GS_PHASE(p)                                                                            \
-    do {                                                                                       \
-        if (threadIdx.x == 0)                                                                  \
-            g_phase[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (p)] = wall_clock64();        \
-    } while (0)
-#define GS_JOB_PHASE(row, p)                                                                   \
-    do {                                                                                       \
-        if (threadIdx.x == 0)                                                                  \
-            g_phase[(2048 + (row)) * 16 + (p)] = wall_clock64();                               \
-    } while (0)
-#else
-#define GS_PHASE(p) do { } while (0)
-#define GS_JOB_PHASE(row, p) do { } while (0)
-#endif
-
 constexpr uint32_t KEY_LOWEST_FINITE = 0x00800000u; /* f2key(-FLT_MAX) */
-constexpr int      CAND_PER_WAVE     = 256;  /* groups / elements at or above B that one wavefront
-                                              * of the final kernel holds */
 constexpr int      CAND_CUT_MAX      = CAND_K_MAX; /* entries the last wavefront orders */
 static_assert(CAND_CUT_MAX == WAVE, "one entry per lane");
 
@@ -289,8 +270,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     uint32_t *hcnt  = reinterpret_cast<uint32_t *>(s_arena + CA_HCNT);
     uint32_t *hist  = reinterpret_cast<uint32_t *>(s_arena + CA_HIST);
     uint64_t *s_cut = reinterpret_cast<uint64_t *>(s_arena + CA_CUT);
-
-    GS_PHASE(0);
     /* every load this kernel needs from memory is issued here, before anything is waited for */
     float4 gv[ROUNDS];
     int    gi[ROUNDS];
@@ -347,7 +326,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     }
     __syncthreads();
     bk = s_c.red_b[0] > s_c.red_b[1] ? s_c.red_b[0] : s_c.red_b[1];
-    GS_PHASE(1);
     /* 0xffffffff: a wavefront of the scan had more groups than slots */
     bool           give_up = bk == 0xffffffffu;
     const uint32_t lo      = bk < KEY_LOWEST_FINITE ? KEY_LOWEST_FINITE : bk;
@@ -383,7 +361,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         }
     }
     give_up = give_up || n_e > (unsigned) FC_LIST;
-    GS_PHASE(2);
     if (PEN) {
         /* claim the slot or find it taken by the same id, then count (16-bit counters, two a
          * word: a history holds fewer than 65536 ids) */
@@ -434,9 +411,7 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     if (give_up)
         s_c.give_up = 1;
     __syncthreads();
-    GS_PHASE(3);
     give_up = s_c.give_up != 0;
-    GS_PHASE(5);
     /* The k largest. The keys lie in [lo, mx]; 256 bins over that range, counted by all
      * wavefronts, then every wavefront finds the bin in which the count from above reaches k.
      * The entries from that bin upwards are listed; should they be more than CAND_CUT_MAX the
@@ -497,7 +472,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         }
         give_up = give_up || listed > CAND_CUT_MAX; /* runs of equal values */
     }
-    GS_PHASE(6);
     if (!give_up) {
         /* the entries that reach the cut: each wavefront lists its own, after asking for places
          * (cut > 0: a dropped entry's key 0 never passes) */
@@ -513,7 +487,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         s_c.give_up = 1;
     }
     __syncthreads();
-    GS_PHASE(7);
     give_up = s_c.give_up != 0 || s_c.n_cut > CAND_CUT_MAX;
     if (!give_up) {
         /* order by counting (logit descending, index ascending): entry i is compared with the
@@ -535,31 +508,14 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
             s_pack[rank] = me;
     }
     __syncthreads();
-    GS_PHASE(8);
-#ifdef GS_PHASES
-    if (tid == 0) {
-        g_phase[blockIdx.x * 16 + 12] = 0;
-        g_phase[blockIdx.x * 16 + 13] = s_c.n_real;
-        g_phase[blockIdx.x * 16 + 14] = s_c.n_cut;
-        g_phase[blockIdx.x * 16 + 15] = give_up;
-    }
-#endif
     /* all but the first wavefront are done, or all but the first four when the row falls back
      * (the slower paths are written for 256 threads) */
     if (tid >= (give_up ? TPB : WAVE))
         return;
     int k = a.k;
-#ifdef GS_NO_FALLBACK
-    if (give_up) {
-        a.out[row] = -1;
-        return;
-    }
-#else
     if (give_up)
         k = cand_fallback<NV, PEN>(&rv, &a, row, s_arena, s_pack, &s_gs, &s_n, &s_n2);
-    else
-#endif
-    if (a.row_flag && tid == 0)
+    else if (a.row_flag && tid == 0)
         a.row_flag[row] = 0;
     if (tid < WAVE) {
         /* (k <= CAND_K_MAX = 64 on this path) */
@@ -567,7 +523,6 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         if (tid == 0)
             a.out[row] = tok;
     }
-    GS_PHASE(9);
 }
 
 } // namespace gs
