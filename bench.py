@@ -90,9 +90,65 @@ def cpu_baseline(w, budget_s=20.0):
     v_1, reps_1, _ = out["1"]
     return {"value": round(v_all, 2), "unit": "rows/s", "cores": cores, "kind": "port",
             "single_core_rows_per_s": round(v_1, 2),
+            **reference_top_k_baseline(w, cores, budget_s / 2),
             "sample": f"whole batch of {w.rows} rows x {reps_all} repeats on {cores} threads "
                       f"(one row per thread) and x {reps_1} repeats on 1 thread; oracle built with "
                       "-O3 -ffast-math -march=x86-64-v3 -fopenmp"}, ids
+
+
+def reference_top_k_baseline(w, cores, budget_s):
+    """Times the reference's own geist_sampler_top_k_ws (src/engine/sampler.c:178-228, compiled
+    from its sources with its release flags) on the same rows: k and temperature of the workload,
+    reference precedence (top-k alone, no top-p, no penalties). One workspace and one generator
+    per thread, as the reference's sessions hold them. Empty where that library was not built."""
+    import ctypes as C
+    import threading
+    from oracle_lib import load_ref, RefWorkspace, OracleRng
+    lib = load_ref(fast=True)
+    if lib is None or w.top_k <= 0 or w.temperature <= 0:
+        return {}
+    fp = C.POINTER(C.c_float)
+    rows = [np.ascontiguousarray(r, dtype=np.float32) for r in w.logits]
+
+    def work(mine, reps, counter):
+        ws, rng = RefWorkspace(), OracleRng()
+        if lib.geist_sampler_workspace_init(C.byref(ws), w.n_vocab) != 0:
+            return
+        lib.geist_rng_seed(C.byref(rng), 1234)
+        for _ in range(reps):
+            for i in mine:
+                lib.geist_sampler_top_k_ws(C.byref(ws), rows[i].ctypes.data_as(fp), w.top_k,
+                                           w.temperature, C.byref(rng))
+                counter[0] += 1
+        lib.geist_sampler_workspace_destroy(C.byref(ws))
+
+    res = {}
+    for label, threads in (("1", 1), ("all", cores)):
+        # size the sample from one timed row so that each leg takes a few seconds
+        c = [0]
+        t0 = time.perf_counter()
+        work([0], 1, c)
+        per_row = max(time.perf_counter() - t0, 1e-6)
+        want = budget_s / 2 / per_row * threads
+        reps = max(1, min(10, int(want / w.rows)))
+        n_rows = w.rows if want >= w.rows else max(threads, int(want))
+        shares = [list(range(t, n_rows, threads)) for t in range(threads)]
+        counters = [[0] for _ in range(threads)]
+        th = [threading.Thread(target=work, args=(shares[t], reps, counters[t]))
+              for t in range(threads)]
+        t0 = time.perf_counter()
+        for t in th:
+            t.start()
+        for t in th:
+            t.join()
+        dt = time.perf_counter() - t0
+        res[label] = (sum(c[0] for c in counters) / dt, n_rows, reps)
+    return {"reference_top_k_rows_per_s": round(res["all"][0], 2),
+            "reference_top_k_single_core_rows_per_s": round(res["1"][0], 2),
+            "reference_top_k_sample": f"geist_sampler_top_k_ws(k={w.top_k}, T={w.temperature}) from "
+                                      f"oracle/_ref (release flags): {res['all'][1]} rows x "
+                                      f"{res['all'][2]} on {cores} threads, {res['1'][1]} rows x "
+                                      f"{res['1'][2]} on 1 thread"}
 
 
 def bench_spec(w, args):
