@@ -379,6 +379,23 @@ static int resolve(geist_hip_sampler *s, const struct geist_hip_sample_params *p
     return GEIST_HIP_OK;
 }
 
+/* Everything that can make a sampling call fail on its arguments, without side effects: the
+ * entry points that draw from a generator check first, so that a rejected call consumes no
+ * draw. */
+static int check_call(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                      const struct geist_hip_sample_params *params, const void *d_out) {
+    if (!rows || !params)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null rows or params");
+    if (!d_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null output");
+    Resolved rs;
+    const int rc = resolve(s, params, rows->n_vocab, rs);
+    if (rc)
+        return rc;
+    Launch L{};
+    return make_launch(s, rows, params, !rs.greedy, L);
+}
+
 static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                        const struct geist_hip_sample_params *params, const float *d_uniforms,
                        geist_hip_token_t *d_out) {
@@ -660,8 +677,9 @@ int geist_hip_sample_rows_rng(geist_hip_sampler *s, const struct geist_hip_rows 
         return GEIST_HIP_E_INVALID_ARG;
     if (!rows || !params)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "null rows or params");
-    if (rows->rows > s->max_rows)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "too many rows");
+    const int rc = check_call(s, rows, params, d_out_tokens);
+    if (rc)
+        return rc;
     const bool greedy = !(params->temperature > 0.0f);
     if (!greedy) {
         if (!d_rng_states)
@@ -857,6 +875,16 @@ static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t
     return GEIST_HIP_OK;
 }
 
+int geist_hip_f16_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (n_out == 0 || n_in == 0 || n_in > 0x7ffffff8u)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "linear: %zu x %zu", n_out, n_in);
+    HIPCHK(s, hipSetDevice(s->device));
+    F64Scratch ws;
+    return f64_scratch(s, n_out, n_in, ws);
+}
+
 int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
                               size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                               float *d_y, size_t ld_y) {
@@ -943,6 +971,10 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         return rc;
     if (!rs.greedy && !d_uniforms && !d_rng_states)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "stochastic configuration without draws");
+    const struct geist_hip_rows r = {d_logits, ld_logits, rows, n_vocab, nullptr, 0, nullptr,
+                                     nullptr, 0};
+    if ((rc = check_call(s, &r, params, d_out_tokens)) != GEIST_HIP_OK)
+        return rc; /* before any draw */
     HIPCHK(s, hipSetDevice(s->device));
     const bool f64     = !q8 && (rows > 1 || s->projection_portable);
     const bool fuse_ok = f16_gemv_can_fuse((int) rows) && !f64;
@@ -988,8 +1020,6 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         launch_rng_units(s->stream, d_rng_states, shared, (int) rows, s->uniforms);
         d_uniforms = s->uniforms;
     }
-    const struct geist_hip_rows r = {d_logits, ld_logits, rows, n_vocab, nullptr, 0, nullptr,
-                                     nullptr, 0};
     s->tmax_ready = topk_scan;
     rc            = sample_impl(s, &r, params, rs.greedy ? nullptr : d_uniforms, d_out_tokens);
     s->tmax_ready = false;

@@ -73,10 +73,10 @@ struct WalkShared {
  * u * (sum of chunk_w). chunk_w: C per-chunk weights in LDS; slab_w: the row's C * SLABS_MAX slab
  * weights in global memory; NV: slabs per chunk of the pass that wrote them; qrow / qx: the
  * draft probabilities of the residual walk (see load_q_chunk). Returns the id to
- * every thread. Should rounding leave the target beyond the located slab, the following slabs of
- * the chunk are walked too; beyond those the chunk's last index (the reference returns the last
- * index of the row, sampler.c:100-101; the located chunk is then the last one), for the residual
- * walk the last element seen with a positive weight. */
+ * every thread. Should rounding leave the target beyond the located slab, the walk goes on through
+ * the following slabs and chunks, as the reference's single loop does (sampler.c:93-99); past the
+ * end of the row it returns the row's last index (sampler.c:100-101), for the residual walk the
+ * last element seen with a positive weight. */
 template <int NV, bool PEN, bool RESID>
 __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const double *chunk_w,
                                 const double *__restrict__ slab_w, int C, float u, float mx,
@@ -123,46 +123,52 @@ __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const do
         }
     }
     __syncthreads();
-    const int    chunk  = sh.chunk;
+    const int    chunk0 = sh.chunk, slab0 = sh.slab;
     double       carry  = sh.before;
     const double target = sh.target;
-    int          base, end;
-    chunk_bounds<NV>(rv, chunk, base, end);
-    for (int j = sh.slab; j < NV; ++j) {
-        const int sbase = base + j * 4 * TPB;
-        if (sbase >= end)
-            break;
-        const int send = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
-        float4    v[1], qv[1];
-        fetch_chunk<1, PEN>(rv, row, n_rows, sbase, send, s_cnt16, v); /* a slab is a chunk of 1024 */
-        qv[0] = v[0];
-        if (RESID)
-            load_q_chunk<1>(qrow, qvec, qx, sbase, send, qv);
-        const int e = sbase + 4 * tid;
-        float     w[4];
-        slab_weights<RESID>(v[0], qv[0], e, send, mx, inv_t, sum, tab, w);
-        const double part = (double) w[0] + (double) w[1] + (double) w[2] + (double) w[3];
-        double       slab;
-        const double incl = block_scan_f64(part, sh.scan, &slab);
-        double       run  = carry + (incl - part);
-        int          lastpos = -1;
+    int          base, end = 0;
+    bool         found = false;
+    for (int chunk = chunk0; chunk < C && !found; ++chunk) {
+        chunk_bounds<NV>(rv, chunk, base, end);
+        for (int j = chunk == chunk0 ? slab0 : 0; j < NV; ++j) {
+            const int sbase = base + j * 4 * TPB;
+            if (sbase >= end)
+                break;
+            const int send = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
+            float4    v[1], qv[1];
+            /* a slab is a chunk of 1024 */
+            fetch_chunk<1, PEN>(rv, row, n_rows, sbase, send, s_cnt16, v);
+            qv[0] = v[0];
+            if (RESID)
+                load_q_chunk<1>(qrow, qvec, qx, sbase, send, qv);
+            const int e = sbase + 4 * tid;
+            float     w[4];
+            slab_weights<RESID>(v[0], qv[0], e, send, mx, inv_t, sum, tab, w);
+            const double part = (double) w[0] + (double) w[1] + (double) w[2] + (double) w[3];
+            double       slab;
+            const double incl = block_scan_f64(part, sh.scan, &slab);
+            double       run  = carry + (incl - part);
+            int          lastpos = -1;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            run += (double) w[c];
-            if (w[c] > 0.0f)
-                lastpos = e + c;
-            if (e + c < send && w[c] > 0.0f && target < run) {
-                atomicMin(&sh.pick, e + c);
+            for (int c = 0; c < 4; ++c) {
+                run += (double) w[c];
+                if (w[c] > 0.0f)
+                    lastpos = e + c;
+                if (e + c < send && w[c] > 0.0f && target < run) {
+                    atomicMin(&sh.pick, e + c);
+                    break;
+                }
+            }
+            if (RESID && lastpos >= 0)
+                atomicMax(&sh.last_pos, lastpos);
+            __syncthreads();
+            if (sh.pick != 0x7fffffff) {
+                found = true;
                 break;
             }
+            carry += slab;
+            __syncthreads();
         }
-        if (RESID && lastpos >= 0)
-            atomicMax(&sh.last_pos, lastpos);
-        __syncthreads();
-        if (sh.pick != 0x7fffffff)
-            break;
-        carry += slab;
-        __syncthreads();
     }
     __syncthreads();
     int tok = sh.pick;

@@ -114,6 +114,17 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
 
 const char *geist_hip_head_errmsg(const struct geist_hip_head *h) { return h ? h->err : ""; }
 
+/* The session's sampling options as the device layer takes them: the reference's precedence,
+ * no penalties, the model's soft-cap. */
+static struct geist_hip_sample_params head_params(const struct geist_hip_head *h) {
+    return (struct geist_hip_sample_params) {.temperature        = h->temperature,
+                                             .top_p              = h->top_p,
+                                             .top_k              = h->top_k,
+                                             .repetition_penalty = 1.0f,
+                                             .logit_softcap      = h->logit_softcap,
+                                             .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
+}
+
 int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_session_opts *opts) {
     if (h == nullptr)
         return GEIST_HIP_E_INVALID_ARG;
@@ -125,7 +136,36 @@ int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_sessi
     h->top_k       = opts->top_k;
     if (opts->random_seed != 0 && seed_rng(h, opts->random_seed) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "seeding the device RNG");
-    /* step.c:398-409 sizes the host workspace here; the device workspace was sized at create */
+    /* step.c:398-409 sizes the sampler workspace here, once top_p is known, so that no decode
+     * step allocates; so does this */
+    const struct geist_hip_sample_params prm = head_params(h);
+    if (geist_hip_sampler_prepare(h->hs, &prm, h->vocab) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_OOM, "sampler workspace");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_reserve_projection(struct geist_hip_head *h, size_t d_model) {
+    if (h == nullptr || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    void *p = nullptr;
+    if (h->d_logits == nullptr) {
+        if (geist_hip_malloc(h->hs, h->m_max * h->vocab * sizeof(float), &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "logit buffer");
+        h->d_logits = p;
+    }
+    if (h->d_model_cap < d_model) {
+        geist_hip_free(h->hs, h->d_normed);
+        h->d_normed    = nullptr;
+        h->d_model_cap = 0;
+        if (geist_hip_malloc(h->hs, h->m_max * d_model * sizeof(float), &p) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
+        h->d_normed    = p;
+        h->d_model_cap = d_model;
+        /* a batch of rows goes through the double-precision projection, which has scratch */
+        if (h->m_max > 1 && d_model % 8 == 0 &&
+            geist_hip_f16_linear_reserve(h->hs, h->vocab, d_model) != GEIST_HIP_OK)
+            return head_fail(h, GEIST_HIP_E_OOM, "scratch of the batch projection");
+    }
     return GEIST_HIP_OK;
 }
 
@@ -138,12 +178,7 @@ static int finalize(struct geist_hip_head *h, const float *d_logits, size_t k, i
         .d_logits = d_logits, .ld = h->vocab, .rows = k, .n_vocab = h->vocab};
     /* head.c:172-183 / 291-302: T == 0 -> argmax; top_k > 1 -> top-k; 0 < top_p < 1 -> top-p;
      * else temperature. Rows in order, one shared RNG (head.c:274-304). */
-    const struct geist_hip_sample_params prm = {.temperature        = h->temperature,
-                                                .top_p              = h->top_p,
-                                                .top_k              = h->top_k,
-                                                .repetition_penalty = 1.0f,
-                                                .logit_softcap      = h->logit_softcap,
-                                                .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
+    const struct geist_hip_sample_params prm = head_params(h);
     if (geist_hip_sample_rows_rng(h->hs, &rows, &prm, h->d_rng, /*shared=*/1, h->d_tokens) !=
         GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "sampling");
@@ -175,28 +210,12 @@ static int project_finalize(struct geist_hip_head *h, const float *d_hidden, siz
         return GEIST_HIP_E_INVALID_ARG;
     if (k > h->m_max)
         return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
-    void *p = nullptr;
-    if (h->d_logits == nullptr) {
-        if (geist_hip_malloc(h->hs, h->m_max * h->vocab * sizeof(float), &p) != GEIST_HIP_OK)
-            return head_fail(h, GEIST_HIP_E_OOM, "logit buffer");
-        h->d_logits = p;
-    }
-    if (h->d_model_cap < d_model) {
-        geist_hip_free(h->hs, h->d_normed);
-        h->d_normed    = nullptr;
-        h->d_model_cap = 0;
-        if (geist_hip_malloc(h->hs, h->m_max * d_model * sizeof(float), &p) != GEIST_HIP_OK)
-            return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
-        h->d_normed    = p;
-        h->d_model_cap = d_model;
-    }
+    /* a no-op after geist_hip_head_reserve_projection with this d_model */
+    const int rrc = geist_hip_head_reserve_projection(h, d_model);
+    if (rrc != GEIST_HIP_OK)
+        return rrc;
     /* head.c:99-101, 114-126, then the dispatch of 172-183 / 291-302 with the session's RNG */
-    const struct geist_hip_sample_params prm = {.temperature        = h->temperature,
-                                                .top_p              = h->top_p,
-                                                .top_k              = h->top_k,
-                                                .repetition_penalty = 1.0f,
-                                                .logit_softcap      = h->logit_softcap,
-                                                .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
+    const struct geist_hip_sample_params prm = head_params(h);
     const int rc =
             d_scales != nullptr
                     ? geist_hip_project_sample_rows_q8w(h->hs, d_hidden, ld_hidden, k, d_model,
@@ -281,15 +300,10 @@ int geist_hip_head_project_finalize_spec(struct geist_hip_head *h, const float *
     if (h->spec == nullptr || h->temperature != 0.0f || d_model != h->spec_d_model)
         return project_finalize(h, d_hidden, d_model, 1, d_norm_weight, rms_eps, d_embed_f16,
                                 nullptr, d_model, out_token);
-    void *p = nullptr;
     if (h->d_model_cap < d_model) {
-        geist_hip_free(h->hs, h->d_normed);
-        h->d_normed    = nullptr;
-        h->d_model_cap = 0;
-        if (geist_hip_malloc(h->hs, h->m_max * d_model * sizeof(float), &p) != GEIST_HIP_OK)
-            return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
-        h->d_normed    = p;
-        h->d_model_cap = d_model;
+        const int rrc = geist_hip_head_reserve_projection(h, d_model);
+        if (rrc != GEIST_HIP_OK)
+            return rrc;
     }
     /* head.c:99-101, then head.c:109 */
     struct geist_hip_spec_result res;

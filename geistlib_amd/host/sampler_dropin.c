@@ -8,6 +8,8 @@
 #include "geist_sampler_dropin.h"
 #include "geist_sampler_hip.h"
 
+#include <pthread.h>
+#include <stdatomic.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -31,9 +33,27 @@ struct ws_header {
     uint64_t          pad; /* keeps probs 16-byte aligned */
 };
 
-[[noreturn]] static void die(const char *what, geist_hip_sampler *hs) {
-    fprintf(stderr, "geist sampler (HIP): %s: %s\n", what,
-            hs ? geist_hip_sampler_last_error(hs) : "no device context");
+/* A device failure (no device, out of device memory, a failed copy or launch) goes to the failure
+ * handler. The reference's samplers cannot fail (on a failed allocation they degrade to the
+ * arg-max on the host, sampler.c:125-127); there is no host path here, so the default handler
+ * ends the process with a message. A handler installed by the application may return instead:
+ * the sampling call then returns GEIST_SAMPLER_DROPIN_FAILED_TOKEN. */
+static _Atomic(geist_sampler_dropin_failure_fn) g_on_failure;
+static _Atomic(void *)                          g_on_failure_user;
+
+void geist_sampler_dropin_on_failure(geist_sampler_dropin_failure_fn fn, void *user) {
+    atomic_store(&g_on_failure_user, user);
+    atomic_store(&g_on_failure, fn);
+}
+
+static geist_token_t fail(const char *what, geist_hip_sampler *hs) {
+    const char *detail = hs ? geist_hip_sampler_last_error(hs) : "no device context";
+    const geist_sampler_dropin_failure_fn fn = atomic_load(&g_on_failure);
+    if (fn != nullptr) {
+        fn(what, detail, atomic_load(&g_on_failure_user));
+        return GEIST_SAMPLER_DROPIN_FAILED_TOKEN;
+    }
+    fprintf(stderr, "geist sampler (HIP): %s: %s\n", what, detail);
     abort();
 }
 
@@ -67,24 +87,61 @@ static int ctx_setup(struct dropin_ctx *c, size_t n_vocab) {
     return GEIST_HIP_OK;
 }
 
-static thread_local struct dropin_ctx tl_ctx;
+/* The context of geist_sampler_argmax / _temperature lives under a thread-specific key whose
+ * destructor gives the device memory back when the thread ends: a server that runs each
+ * session on a short-lived thread (tests/test_multi_session_parallel_int.c:1-24) leaks
+ * nothing. The main thread's context lives until the process ends. */
+static pthread_key_t  g_ctx_key;
+static pthread_once_t g_ctx_once = PTHREAD_ONCE_INIT;
+static int            g_ctx_key_ok;
 
-static struct dropin_ctx *thread_ctx(size_t n_vocab) {
-    if (tl_ctx.hs == nullptr || tl_ctx.n_vocab < n_vocab) {
-        ctx_release(&tl_ctx);
-        if (ctx_setup(&tl_ctx, n_vocab) != GEIST_HIP_OK)
-            die("no device workspace for this thread", nullptr);
+static void thread_ctx_destroy(void *p) {
+    struct dropin_ctx *c = p;
+    if (c != nullptr) {
+        ctx_release(c);
+        free(c);
     }
-    return &tl_ctx;
+}
+
+static void thread_ctx_key_make(void) {
+    g_ctx_key_ok = pthread_key_create(&g_ctx_key, thread_ctx_destroy) == 0;
+}
+
+/* The calling thread's context for rows of n_vocab logits, or null after a reported failure. */
+static struct dropin_ctx *thread_ctx(size_t n_vocab) {
+    pthread_once(&g_ctx_once, thread_ctx_key_make);
+    if (!g_ctx_key_ok) {
+        fail("no thread-specific key for the device workspace", nullptr);
+        return nullptr;
+    }
+    struct dropin_ctx *c = pthread_getspecific(g_ctx_key);
+    if (c == nullptr) {
+        c = calloc(1, sizeof *c);
+        if (c == nullptr || pthread_setspecific(g_ctx_key, c) != 0) {
+            free(c);
+            fail("no memory for this thread's device workspace", nullptr);
+            return nullptr;
+        }
+    }
+    if (c->hs == nullptr || c->n_vocab < n_vocab) {
+        ctx_release(c);
+        if (ctx_setup(c, n_vocab) != GEIST_HIP_OK) {
+            fail("no device workspace for this thread", nullptr);
+            return nullptr;
+        }
+    }
+    return c;
 }
 
 /* One row through the device path with the reference's precedence. */
 static geist_token_t sample_one(struct dropin_ctx *c, size_t n, const float *logits,
                                 float temperature, int top_k, float top_p, const float *u) {
+    if (c == nullptr) /* the failure has been reported */
+        return GEIST_SAMPLER_DROPIN_FAILED_TOKEN;
     if (geist_hip_upload(c->hs, c->d_row, logits, n * sizeof(float)) != GEIST_HIP_OK)
-        die("upload of the logit row", c->hs);
+        return fail("upload of the logit row", c->hs);
     if (u != nullptr && geist_hip_upload(c->hs, c->d_u, u, sizeof(float)) != GEIST_HIP_OK)
-        die("upload of the draw", c->hs);
+        return fail("upload of the draw", c->hs);
     const struct geist_hip_rows rows = {
         .d_logits = c->d_row, .ld = n, .rows = 1, .n_vocab = n};
     const struct geist_hip_sample_params prm = {.temperature        = temperature,
@@ -94,10 +151,10 @@ static geist_token_t sample_one(struct dropin_ctx *c, size_t n, const float *log
                                                 .precedence = GEIST_HIP_PRECEDENCE_REFERENCE};
     if (geist_hip_sample_rows(c->hs, &rows, &prm, u != nullptr ? c->d_u : nullptr, c->d_out) !=
         GEIST_HIP_OK)
-        die("sampling", c->hs);
+        return fail("sampling", c->hs);
     int32_t tok = -1;
     if (geist_hip_download(c->hs, &tok, c->d_out, sizeof tok) != GEIST_HIP_OK)
-        die("download of the token id", c->hs);
+        return fail("download of the token id", c->hs);
     return tok;
 }
 
@@ -174,8 +231,10 @@ void geist_sampler_workspace_destroy(struct geist_sampler_workspace *ws) {
 
 static struct dropin_ctx *ws_ctx(struct geist_sampler_workspace *ws) {
     struct ws_header *h = ws->probs != nullptr ? (struct ws_header *) ws->probs - 1 : nullptr;
-    if (h == nullptr || h->magic != DROPIN_MAGIC)
-        die("workspace was not made by geist_sampler_workspace_init", nullptr);
+    if (h == nullptr || h->magic != DROPIN_MAGIC) {
+        fail("workspace was not made by geist_sampler_workspace_init", nullptr);
+        return nullptr;
+    }
     return &h->ctx;
 }
 

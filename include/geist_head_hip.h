@@ -59,8 +59,15 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
 void geist_hip_head_destroy(struct geist_hip_head *h);
 const char *geist_hip_head_errmsg(const struct geist_hip_head *h);
 
-/* opts == NULL keeps the greedy defaults (geist_session_create's NULL opts). */
+/* opts == NULL keeps the greedy defaults (geist_session_create's NULL opts). Sizes the sampler's
+ * workspace for the options it sets, as step.c:398-409 does, so that no later call allocates. */
 int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_session_opts *opts);
+/* Sizes what geist_hip_head_project_finalize[_q8w|_spec] need for hidden rows of d_model floats:
+ * the [m_max, vocab] logit buffer, the normed rows and the scratch of the batch projection
+ * (where the reference's session allocator sizes scratch_logits and scratch_normed,
+ * src/archs/transformer/arch_state.c). Call it at set-up; a projection call for which nothing
+ * was reserved reserves on its first use. */
+int geist_hip_head_reserve_projection(struct geist_hip_head *h, size_t d_model);
 
 /* d_logits: [1, vocab] / [k, vocab] fp32 in device memory, row stride vocab. Synchronous: the
  * token ids are in host memory on return, as in the reference. */

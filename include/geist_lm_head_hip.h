@@ -42,8 +42,12 @@ int geist_hip_f16_gemv_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_
  *   d_y[m * ld_y + r] = (float) sum_i (double) d_x[m * ld_x + i] * (double) f16(W[r][i])
  * with the sum in double in index order, bit for bit: the device adds in another order and
  * repeats, in the reference's order, the few sums that lie close enough to a binary32 rounding
- * boundary for the order to matter. Same argument rules as geist_hip_f16_gemv_rows. The first
- * call allocates a small buffer in the sampler (the activations in double). */
+ * boundary for the order to matter. Same argument rules as geist_hip_f16_gemv_rows. The kernels
+ * use a buffer in the sampler (the activations in double, the list of outputs to repeat):
+ * geist_hip_f16_linear_reserve sizes it for weights of up to n_out x n_in at set-up, where the
+ * reference sizes its scratch (forward/step.c:398-409); a call for a larger shape than was
+ * reserved sizes it again, with a device synchronisation. */
+int geist_hip_f16_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in);
 int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t n_out,
                               size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                               float *d_y, size_t ld_y);

@@ -6,7 +6,13 @@
  * sampler.o leaves head.c, step.c, arch_state.c, spec_head.c and tests/test_sampler_unit.c
  * unchanged. The logit row a caller passes lives in host memory, as in the reference; it is
  * uploaded, sampled by the HIP kernels and only the 4-byte token id returns. There is no CPU
- * path behind these symbols: a missing or failing device aborts with a message.
+ * path behind these symbols: a missing or failing device goes to the failure handler below,
+ * which by default ends the process with a message.
+ *
+ * Threads: every entry point may be called from any number of threads at once
+ * (src/engine/sampler.h:8). A workspace belongs to one thread at a time, as in the reference;
+ * geist_sampler_argmax / _temperature keep a device context per calling thread, made on the
+ * thread's first call and given back when the thread ends.
  *
  * A translation unit that already includes the reference's <geist.h> / sampler.h must not
  * include this file (the declarations would repeat); it is for callers built without the
@@ -68,6 +74,17 @@ geist_token_t geist_sampler_top_k_ws(struct geist_sampler_workspace *ws, const f
 geist_token_t geist_sampler_top_p_ws(struct geist_sampler_workspace *ws, const float *logits,
                                      float top_p, float temperature, struct geist_rng *rng);
 #endif
+
+/* No counterpart in the reference, whose samplers cannot fail. What a sampling call returns
+ * after a device failure when the installed handler returns. */
+#define GEIST_SAMPLER_DROPIN_FAILED_TOKEN ((geist_token_t) -1)
+/* `what` names the step that failed, `detail` is the device layer's message. */
+typedef void (*geist_sampler_dropin_failure_fn)(const char *what, const char *detail, void *user);
+/* Installs the process-wide handler of device failures inside the sampling calls; null restores
+ * the default, which prints the message to stderr and calls abort(). A handler may log and
+ * return (the call then returns GEIST_SAMPLER_DROPIN_FAILED_TOKEN and consumes the draw it had
+ * taken), or not return (longjmp, exit). It is called on the thread whose call failed. */
+void geist_sampler_dropin_on_failure(geist_sampler_dropin_failure_fn fn, void *user);
 
 #ifdef __cplusplus
 }
