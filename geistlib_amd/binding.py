@@ -80,6 +80,7 @@ def load_library():
     lib.geist_hip_sampler_set_logits_hint.argtypes = [vp, i32]
     lib.geist_hip_sampler_set_projection.argtypes = [vp, i32]
     lib.geist_hip_sampler_prepare.argtypes = [vp, C.POINTER(SampleParams), sz]
+    lib.geist_hip_sampler_set_wait_limit.argtypes = [vp, C.c_uint32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -158,6 +159,9 @@ class HipSampler:
     def _check(self, rc):
         if rc != GEIST_HIP_OK:
             raise GeistHipError(rc, self.lib.geist_hip_sampler_last_error(self.h).decode())
+
+    def set_wait_limit(self, polls):
+        self._check(self.lib.geist_hip_sampler_set_wait_limit(self.h, C.c_uint32(polls)))
 
     def prepare(self, params, n_vocab=0):
         """Sizes whatever workspace `params` needs beyond the sampler's own, ahead of the first

@@ -24,6 +24,16 @@
 
 using namespace gs;
 
+/* Host side of gs::MeetSpace: the two slot arrays ([max_rows * max_chunks] each, zeroed when
+ * made), how many slots the last launch on each array used, and whose turn it is. */
+struct MeetState {
+    uint64_t *slots[2] = {nullptr, nullptr};
+    uint32_t  used[2]  = {0, 0};
+    int       turn     = 0;
+    uint32_t  capacity = 0;     /* slots per array */
+    bool      suspect  = false; /* a launch failed after the bookkeeping: zero both arrays */
+};
+
 struct geist_hip_sampler {
     int         device     = 0;
     hipStream_t stream     = nullptr;
@@ -33,6 +43,9 @@ struct geist_hip_sampler {
 
     /* device workspace */
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
+    MeetState  meet_own;             /* where the workgroups of the one-pass exp-sum kernel meet */
+    MeetState *meet      = &meet_own; /* (the allocation-free entry point shares one per device) */
+    uint32_t  wait_limit = 1u << 16; /* polls a workgroup of that kernel waits for its row */
     double   *chunk_sum  = nullptr; /* [max_rows][max_chunks] */
     double   *resid_sum  = nullptr; /* [max_rows][max_chunks] spec verification */
     double   *slab_sum   = nullptr; /* [max_rows][max_chunks][8] slab sums of the exp-sum pass */
@@ -82,8 +95,11 @@ static int fail(geist_hip_sampler *s, int code, const char *fmt, ...) {
 
 static int after_launch(geist_hip_sampler *s, const char *what) {
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess)
+    if (e != hipSuccess) {
+        if (s->meet)
+            s->meet->suspect = true; /* the slots may not be what the bookkeeping says */
         return fail(s, GEIST_HIP_E_BACKEND, "launch of %s failed: %s", what, hipGetErrorString(e));
+    }
     return GEIST_HIP_OK;
 }
 
@@ -170,12 +186,17 @@ constexpr size_t STATIC_CSUM  = STATIC_BEST + STATIC_UNITS * 8;        /* double
 constexpr size_t STATIC_SLAB  = STATIC_CSUM + STATIC_UNITS * 8;        /* double[units][8]    */
 constexpr size_t STATIC_ROW_WAVES = STATIC_UNITS + 512;            /* (row, wavefront) pairs */
 constexpr size_t STATIC_WCANDS = STATIC_SLAB + STATIC_UNITS * 8 * 8;   /* WaveCands           */
-constexpr size_t STATIC_BYTES  = STATIC_WCANDS + STATIC_ROW_WAVES * 648;
+constexpr size_t STATIC_MEET   = STATIC_WCANDS + STATIC_ROW_WAVES * 648; /* u64 [2][units]: the
+                                                                            meeting slots, zero
+                                                                            when loaded */
+constexpr size_t STATIC_BYTES  = STATIC_MEET + 2 * STATIC_UNITS * 8;
+static_assert(STATIC_MEET % 16 == 0, "64-bit atomics");
 static_assert(STATIC_WCANDS % 16 == 0, "float4 slots");
 constexpr int    STATIC_MAX_DEVICES = 64;
 } // namespace
 static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
 
+static MeetState      g_static_meet[STATIC_MAX_DEVICES]; /* turn and use of its meeting slots */
 static unsigned char *g_static_ws[STATIC_MAX_DEVICES]; /* device address of `scratch`, per device */
 static bool           g_static_ws_tried[STATIC_MAX_DEVICES];
 static hipError_t     g_static_ws_err[STATIC_MAX_DEVICES];
@@ -247,6 +268,12 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     }
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
+    for (int t = 0; t < 2; ++t) {
+        if (e == hipSuccess) e = hipMalloc((void **) &s->meet_own.slots[t], rc * sizeof(uint64_t));
+        if (e == hipSuccess) e = hipMemsetAsync(s->meet_own.slots[t], 0, rc * sizeof(uint64_t), s->stream);
+    }
+    s->meet_own.capacity = (uint32_t) rc;
+    if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->slab_sum, rc * 8 * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_slab, rc * 8 * sizeof(double));
@@ -279,6 +306,8 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipStreamSynchronize(s->stream);
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
+    (void) hipFree(s->meet_own.slots[0]);
+    (void) hipFree(s->meet_own.slots[1]);
     (void) hipFree(s->resid_sum);
     (void) hipFree(s->slab_sum);
     (void) hipFree(s->resid_slab);
@@ -396,6 +425,28 @@ static int check_call(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     return make_launch(s, rows, params, !rs.greedy, L);
 }
 
+/* The meeting slots for a launch of rows * n_chunks workgroups: this launch takes the array
+ * whose turn it is, which the launch before left zero, and zeroes what that launch used in the
+ * other. */
+static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L) {
+    MeetState &st = *s->meet;
+    if (st.suspect) { /* only after a failed launch: start again from two zeroed arrays */
+        for (int t = 0; t < 2; ++t)
+            (void) hipMemsetAsync(st.slots[t], 0, st.capacity * sizeof(uint64_t), s->stream);
+        st.used[0] = st.used[1] = 0;
+        st.suspect              = false;
+    }
+    MeetSpace  m;
+    m.slots       = st.slots[st.turn];
+    m.stale       = st.slots[st.turn ^ 1];
+    m.stale_count = st.used[st.turn ^ 1];
+    m.wait_limit  = s->wait_limit;
+    st.used[st.turn]     = (uint32_t) L.rows * (uint32_t) L.rv.n_chunks;
+    st.used[st.turn ^ 1] = 0;
+    st.turn ^= 1;
+    return m;
+}
+
 static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                        const struct geist_hip_sample_params *params, const float *d_uniforms,
                        geist_hip_token_t *d_out) {
@@ -436,11 +487,11 @@ static int reserve_sorted_workspace(geist_hip_sampler *s) {
 
 /* One sampling call is enqueued in up to three stages: a first pass over the rows where the mode
  * needs two (the row maxima before the exp-sum), the pass that streams the logits, and what
- * follows it per row. geist_hip_sample_rows runs all three. */
+ * follows it per row. geist_hip_sample_rows runs both. */
 int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                            const struct geist_hip_sample_params *params, const float *d_uniforms,
                            geist_hip_token_t *d_out, unsigned stages, const char **stream_kernel) {
-    const bool do_pre = stages & gs_host::STAGE_PRE, do_stream = stages & gs_host::STAGE_STREAM,
+    const bool do_stream = stages & gs_host::STAGE_STREAM,
                do_tail = stages & gs_host::STAGE_TAIL;
     const char *unused_name;
     if (!stream_kernel)
@@ -471,6 +522,8 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
     f.tmax       = s->tmax;
     f.out        = d_out;
 
+    if (!rs.greedy && !rs.use_k && !(s->meet && s->meet->slots[0] && s->meet->slots[1]))
+        return fail(s, GEIST_HIP_E_INTERNAL, "no meeting slots for the one-pass kernel");
     if (rs.greedy) {
         L.rv.stream_loads = s->logits_streamed;
         *stream_kernel    = "k_tmax_scan";
@@ -546,12 +599,13 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         return after_launch(s, "top-k");
     }
     if (!rs.use_p && !rs.use_m) {
-        *stream_kernel = "k_chunk_expsum";
-        if (do_pre)
-            launch_tmax_scan(L, s->tmax, s->chunk_best);
-        if (do_stream)
-            launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr, nullptr,
-                                0, s->slab_sum);
+        *stream_kernel = "k_scan_expsum";
+        Launch scan          = L;
+        scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
+        if (do_stream &&
+            launch_scan_expsum(scan, rs.inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0,
+                               nullptr, nullptr, 0, s->slab_sum, meet_space(s, scan)))
+            return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
         f.mode     = FINAL_TEMPERATURE;
         f.slab_sum = s->slab_sum;
         if (do_tail)
@@ -578,13 +632,14 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
      * the exp-sum pass at once. Below that a flat row may overflow the list, and the row-final
      * kernel should get the chance to bound it by top-p instead. */
     f.minp_direct     = f.minp_listed && rs.min_p >= 0.02f;
-    *stream_kernel = "k_chunk_expsum";
-    if (do_pre)
-        launch_tmax_scan(L, s->tmax, s->chunk_best, f.minp_listed ? s->cand.count : nullptr);
-    /* (the pass lists candidates only when the pass before it has cleared the lists' counters) */
-    if (do_stream)
-        launch_chunk_expsum(L, rs.inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
-                            f.minp_listed && do_pre ? &f.cand : nullptr, zb_m);
+    *stream_kernel = "k_scan_expsum";
+    Launch scan          = L;
+    scan.rv.stream_loads = s->logits_streamed; /* the one pass over whole rows */
+    if (do_stream &&
+        launch_scan_expsum(scan, rs.inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0,
+                           nullptr, f.minp_listed ? &f.cand : nullptr, zb_m, nullptr,
+                           meet_space(s, scan)))
+        return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     if (!do_tail)
         return after_launch(s, "exp-sum scan");
     f.mode     = FINAL_SORTED;
@@ -607,6 +662,13 @@ int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *row
                           const struct geist_hip_sample_params *params, const float *d_uniforms,
                           geist_hip_token_t *d_out_tokens) {
     return sample_impl(s, rows, params, d_uniforms, d_out_tokens);
+}
+
+int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->wait_limit = polls;
+    return GEIST_HIP_OK;
 }
 
 int geist_hip_sampler_prepare(geist_hip_sampler *s, const struct geist_hip_sample_params *params,
@@ -665,6 +727,11 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
     tmp.slab_sum   = reinterpret_cast<double *>(ws + STATIC_SLAB);
     tmp.wcands     = ws + STATIC_WCANDS;
     tmp.wcands_row_waves = STATIC_ROW_WAVES;
+    MeetState &ms = g_static_meet[device];
+    ms.slots[0]   = reinterpret_cast<uint64_t *>(ws + STATIC_MEET);
+    ms.slots[1]   = ms.slots[0] + STATIC_UNITS;
+    ms.capacity   = (uint32_t) STATIC_UNITS;
+    tmp.meet      = &ms;
     rc = sample_impl(&tmp, rows, params, d_uniforms, d_out_tokens);
     return rc ? report(err, err_len, rc, "%s", tmp.err) : GEIST_HIP_OK;
 }
@@ -760,8 +827,9 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
         return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_probs < n_vocab");
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
-    launch_tmax_scan(L, s->tmax, s->chunk_best);
-    launch_chunk_expsum(L, inv_t, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr);
+    if (launch_scan_expsum(L, inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
+                           nullptr, 0, nullptr, meet_space(s, L)))
+        return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
 }
@@ -1113,10 +1181,11 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
         return rc;
     HIPCHK(s, hipSetDevice(s->device));
     const float inv_t = greedy ? 1.0f : 1.0f / temperature;
-    launch_tmax_scan(La, s->tmax, s->chunk_best);
-    if (!greedy)
-        launch_chunk_expsum(La, inv_t, s->chunk_best, s->chunk_sum, d_draft, (int) L, s->probe_p,
-                            nullptr, 0, s->slab_sum);
+    if (greedy)
+        launch_tmax_scan(La, s->tmax, s->chunk_best);
+    else if (launch_scan_expsum(La, inv_t, s->tmax, s->chunk_best, s->chunk_sum, d_draft, (int) L,
+                                s->probe_p, nullptr, 0, s->slab_sum, meet_space(s, La)))
+        return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     SpecLaunch sp{};
     sp.n_seq      = (int) n_seq;
     sp.L          = (int) L;

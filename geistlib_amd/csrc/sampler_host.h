@@ -10,10 +10,9 @@
 namespace gs_host {
 
 enum : unsigned {
-    STAGE_PRE    = 1u, /* a first pass over the rows, in the modes that read them twice */
     STAGE_STREAM = 2u, /* the pass that streams the logits */
     STAGE_TAIL   = 4u, /* what follows per row */
-    STAGE_ALL    = 7u,
+    STAGE_ALL    = 6u,
 };
 
 /* geist_hip_sample_rows restricted to the stages in `stages` (same checks, same geometry, same

@@ -38,6 +38,17 @@ struct RowView {
     long            allowed_ld; /* words between rows, 0 = one mask for all rows */
 };
 
+/* Where the workgroups of a row meet in the one-pass exp-sum kernel (k_scan_expsum): one 64-bit
+ * slot per (row, chunk), zero until the chunk's workgroup stores its packed maximum there (never
+ * zero). Two such arrays take turns from launch to launch: a launch finds its own array all
+ * zero and zeroes the slots that the launch before it used in the other. */
+struct MeetSpace {
+    uint64_t *slots;       /* [rows * n_chunks] of this launch, zero on entry */
+    uint64_t *stale;       /* the slots of the launch before, zeroed by this one */
+    uint32_t  stale_count;
+    uint32_t  wait_limit;  /* polls before a workgroup reads the row for itself; 0 = do not wait */
+};
+
 struct Launch {
     RowView     rv;
     int         rows;
@@ -121,17 +132,20 @@ struct FinalLaunch {
     int32_t        *row_flag;
 };
 
-/* probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
- * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id */
-/* list != NULL (min-p set): the pass also lists, per row, every element up to z bin zb_list with
- * its unnormalised p -- the min-p bound needs nothing but the row maximum. list->count must be
- * zero on entry (launch_tmax_scan can clear it).
+/* The one pass over the rows of the modes that weigh every element (k_scan_expsum): tmax and
+ * chunk_best as launch_tmax_scan writes them, and chunk_sum[row][chunk], the sum of
+ * expf((l - max) * inv_t) over the chunk in double.
+ * probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
+ * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id.
+ * list != NULL (min-p set): the pass also lists, per row, every element up to z bin zb_list with
+ * its unnormalised p -- the min-p bound needs nothing but the row maximum (the pass clears
+ * list->count itself).
  * slab_sum != NULL (and no list): also the sums of the chunk's slabs of 1024 elements,
- * [rows][chunks][8], which the index-order walks locate their starting point with. */
-void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                         double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, const CandSpace *list = nullptr, int zb_list = 0,
-                         double *slab_sum = nullptr);
+ * [rows][chunks][8], which the index-order walks locate their starting point with.
+ * Returns 0 or a hipError_t value (the launch itself is checked by the caller as usual). */
+int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
+                       double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
+                       const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet);
 /* last z bin that can hold an entry passing min_p (with slack); ZBINS - 1 when min_p is off or
  * that deep */
 int zbin_of_min_p(float min_p);

@@ -4,8 +4,10 @@
  * Kernel map (reference lines the arithmetic follows are cited at each kernel):
  *   k_tmax_scan      per-thread maxima (the single pass of the top-k path) and,
  *                    on request, the per-chunk maximum with its first index       sampler.c:52-62, 202-207
- *   k_chunk_expsum   per-(row, chunk) sum of expf((l - max) * inv_t); on request the sums of
- *                    the chunk's slabs, or the min-p candidates of the row        sampler.c:77-83
+ *   k_scan_expsum    the one pass of the modes that weigh every element: per (row, chunk) the
+ *                    maxima as above and the sum of expf((l - max) * inv_t); on request the
+ *                    sums of the chunk's slabs, or the min-p candidates of the row
+ *                                                                              sampler.c:52-62, 77-83
  *   k_final_argmax / _temperature / _topk / _sorted   per-row combine of each mode: argmax,
  *                    index-order CDF draw, top-k select + sorted softmax + top-p + min-p +
  *                    draw, top-p / min-p shortcut                             sampler.c:90-102, 209-222, 272-299
@@ -131,35 +133,125 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
 }
 
 /* ============================================================================================
- * k_chunk_expsum: sum over the chunk of p_i = expf((l_i - max) * inv_t), in double.
- * Optionally records p at one token of the row (spec verification needs p(x_j)).
+ * k_scan_expsum: the one pass over the logits of the modes that weigh every element --
+ * temperature, top-p / min-p, softmax, speculative verification. Per (row, chunk): the thread
+ * maxima and the chunk's maximum with its first index (what k_tmax_scan writes;
+ * sampler.c:52-62), then, once the row's maximum is known, the chunk's sum of
+ * p_i = expf((l_i - max) * inv_t) in double (sampler.c:77-83); on request the sums of the
+ * chunk's slabs, p at one token of the row (speculative verification needs p(x_j)), or the
+ * row's min-p candidates.
+ *
+ * The row's maximum needs every chunk of the row, so the workgroups of a row meet half way
+ * (row_best_meet): each keeps its chunk in registers, reports the chunk's maximum, waits for the
+ * others' and sums the exponentials from the registers. The rows are read once.
  * ========================================================================================== */
+/* Where the thread maxima and the chunk results go, and the slots through which the workgroups
+ * of a row meet. */
+struct FusedScan {
+    float    *tmax;
+    uint64_t *chunk_best;
+    uint64_t *slots;
+    uint32_t  wait_limit;
+    uint64_t *s_red; /* LDS, NWAVES words */
+    uint64_t *s_bb;  /* LDS, one word */
+};
+
+/* The row's maximum (packed with its first index) once every chunk of the row has reported its
+ * own, for the workgroup that has just found `mine`. Every thread returns the same value.
+ *
+ * The workgroup stores `mine` (never zero) into its slot and its first wavefront polls the row's
+ * n_chunks <= 2 * WAVE slots, a lane per slot, until none reads zero; the maximum of what it then
+ * holds is the row's. Stores and polls are device-scope atomics (plain stores and loads, no
+ * read-modify-write: the slots of a row share a few cache lines, and contended atomic updates of
+ * one line are what would make this wait slow), so no fence is needed; `prior` (thread 0's) is a
+ * value returned by an earlier atomic of the caller's, made an operand of the store so that the
+ * row's other workgroups find that atomic performed when they leave the wait.
+ *
+ * A workgroup waits only for workgroups of its own row. The grid is dealt out so that a row's
+ * workgroups have neighbouring ids and are started together; the wait is bounded all the same:
+ * past `wait_limit` polls (0: at once) the workgroup stops waiting and finds the row's maximum
+ * itself by reading the whole row, so every workgroup ends whatever the others do. */
+template <int NV, bool PEN>
+__device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, int chunk,
+                                                  int n_rows, uint64_t mine, uint32_t prior,
+                                                  const FusedScan &fs, uint32_t *s_cnt16) {
+    static_assert(MAX_CHUNKS <= 2 * WAVE, "two slots per polling lane");
+    const int tid = threadIdx.x;
+    const int C   = rv.n_chunks;
+    uint64_t *row_slots = fs.slots + (long) row * C;
+    if (tid < WAVE) {
+        if (tid == 0) {
+            uint64_t v = mine;
+            asm volatile("" : "+v"(v) : "v"(prior));
+            __hip_atomic_store(row_slots + chunk, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        uint64_t a = 0, b = 0;
+        uint32_t polls = 0;
+        bool     met   = fs.wait_limit != 0;
+        while (met) {
+            a = tid < C ? __hip_atomic_load(row_slots + tid, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT)
+                        : 0;
+            b = tid + WAVE < C ? __hip_atomic_load(row_slots + tid + WAVE, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT)
+                               : 0;
+            const bool missing = (tid < C && a == 0) || (tid + WAVE < C && b == 0);
+            if (__builtin_amdgcn_ballot_w64(missing) == 0)
+                break;
+            if (++polls > fs.wait_limit)
+                met = false;
+            else
+                __builtin_amdgcn_s_sleep(8);
+        }
+        /* 1 is never a packed value: a row's first index is below 2^32 - 2 */
+        const uint64_t got = met ? wave_max_u64(a > b ? a : b) : 1;
+        if (tid == 0)
+            *fs.s_bb = got;
+    }
+    __syncthreads();
+    uint64_t bb = *fs.s_bb;
+    __syncthreads();
+    if (bb != 1)
+        return bb;
+    /* not met: the row's maximum from the row itself, 1024 elements at a time */
+    bb = 0;
+    for (int b0 = 0; b0 < rv.n_vocab; b0 += 4 * TPB) {
+        const int e0 = b0 + 4 * TPB < rv.n_vocab ? b0 + 4 * TPB : rv.n_vocab;
+        float4    w[1];
+        fetch_chunk<1, PEN>(rv, row, n_rows, b0, e0, s_cnt16, w);
+#pragma unroll
+        for (int c = 3; c >= 0; --c) {
+            const int e = b0 + 4 * tid + c;
+            if (e < e0) {
+                const uint64_t p = pack_best(f2key(f4_get(w[0], c)), (uint32_t) e);
+                bb               = p > bb ? p : bb;
+            }
+        }
+        __syncthreads(); /* the count table is rebuilt by the next round */
+    }
+    bb = block_max_u64(bb, fs.s_red);
+    return bb ? bb : pack_best(0u, 0u);
+}
+
 /* The work of one workgroup. PLAIN: a full, 16-byte aligned chunk without soft-cap or
  * allowed-token mask -- the common case, kept free of everything that would make the compiler
- * wait for all of the chunk's loads before the first group is summed (a merge with the
+ * wait for all of the chunk's loads before the first group is looked at (a merge with the
  * element-wise loads of a ragged chunk, a branch around a mask load). */
 template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN>
 __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chunk, int n_rows,
                                              int base, int end, float inv_t,
-                                             const uint64_t *__restrict__ chunk_best,
                                              double *__restrict__ chunk_sum,
                                              double *__restrict__ slab_sum,
                                              const int32_t *__restrict__ probe_token, int probe_L,
                                              float *__restrict__ probe_p, const CandSpace &list,
                                              int zb_list, uint32_t *s_cnt16, double *s_sum,
-                                             const uint64_t *s_tab, int *s_listed, int *s_base) {
+                                             const uint64_t *s_tab, int *s_listed, int *s_base,
+                                             const FusedScan &fs) {
     const int tid = threadIdx.x;
-    /* Order of the loads: the chunk results of the row (each wavefront reduces them for itself,
-     * no barrier), the probed token, the history, then the chunk. The groups of the chunk are
-     * then transformed and summed one by one, each as soon as its own load has arrived: a
-     * barrier with a full fence, or a transform over the whole chunk first, would keep the
-     * arithmetic waiting for the last load, and the launch would alternate between a phase
-     * that only loads and one that only computes. */
-    uint64_t bb = 0;
-    for (int c = tid & (WAVE - 1); c < rv.n_chunks; c += WAVE) {
-        const uint64_t p = chunk_best[(long) row * rv.n_chunks + c];
-        bb               = p > bb ? p : bb;
-    }
+    /* Order of the loads: the probed token, the history, then the chunk. The groups of the
+     * chunk are transformed one by one, each as soon as its own load has arrived: a barrier
+     * with a full fence, or a transform over the whole chunk first, would keep the arithmetic
+     * waiting for the last load. */
     /* spec verification: target row s*(L+1)+j is probed at draft token j of sequence s */
     int tok = -1;
     if (probe_token) {
@@ -194,7 +286,49 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     } else {
         lds_barrier(); /* publishes s_tab (the history's barriers do when PEN) */
     }
-    const float mx = key2f(best_key(wave_max_u64(bb)));
+    uint64_t bb;
+    {
+        /* first half of the one pass: transform each group as its load arrives, keep the
+         * thread's maximum (k_tmax_scan's output) and the chunk's (sampler.c:52-62), then meet
+         * the row's other chunks */
+        float tm = -__builtin_inff();
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            transform_group<PEN, !PLAIN>(rv, row, s_cnt16, 4 * (j * TPB + tid), base, end, v[j]);
+            tm = max3f(tm, max3f(v[j].x, v[j].y, v[j].z), v[j].w);
+        }
+        if (base + 4 * tid >= end)
+            tm = __builtin_nanf("");
+        fs.tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
+        const uint32_t mykey = f2key(tm);
+        uint32_t       bk    = wave_max_u32(mykey);
+        bk = (uint32_t) (block_max_u64((uint64_t) bk, fs.s_red));
+        uint64_t best = 0;
+        if (mykey == bk) {
+            int first = 0x7fffffff;
+#pragma unroll
+            for (int j = NV - 1; j >= 0; --j) {
+                const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+                for (int c = 3; c >= 0; --c)
+                    if (e + c < end && f2key(f4_get(v[j], c)) == bk)
+                        first = e + c;
+            }
+            if (first != 0x7fffffff)
+                best = pack_best(bk, (uint32_t) first);
+        }
+        best = block_max_u64(best, fs.s_red);
+        if (!best) /* an all-NaN chunk reports key 0 at its first index */
+            best = pack_best(0u, (uint32_t) base);
+        uint32_t prior = 0;
+        if (tid == 0) {
+            fs.chunk_best[(long) row * rv.n_chunks + chunk] = best;
+            if (LISTM && chunk == 0) /* the list the second half appends to starts empty */
+                prior = (uint32_t) atomicExch(&list.count[row], 0);
+        }
+        bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, prior, fs, s_cnt16);
+    }
+    const float mx = key2f(best_key(bb));
 
     double      acc  = 0.0;
     double      accs[SLABS ? NV : 1];
@@ -204,7 +338,6 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
      * bin, so the loop carries no bound tests */
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        transform_group<PEN, !PLAIN>(rv, row, s_cnt16, 4 * (j * TPB + tid), base, end, v[j]);
         double a4;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -292,36 +425,52 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
 }
 
 template <int NV, bool PEN, bool LISTM, bool SLABS>
-__global__ __launch_bounds__(TPB) void k_chunk_expsum(RowView rv, float inv_t,
-                                                      const uint64_t *__restrict__ chunk_best,
-                                                      double *__restrict__ chunk_sum,
-                                                      double *__restrict__ slab_sum,
-                                                      const int32_t *__restrict__ probe_token,
-                                                      int probe_L, float *__restrict__ probe_p,
-                                                      CandSpace list, int zb_list) {
+__global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
+                                                     float *__restrict__ tmax,
+                                                     uint64_t *__restrict__ chunk_best,
+                                                     double *__restrict__ chunk_sum,
+                                                     double *__restrict__ slab_sum,
+                                                     const int32_t *__restrict__ probe_token,
+                                                     int probe_L, float *__restrict__ probe_p,
+                                                     CandSpace list, int zb_list, MeetSpace meet) {
     static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
     __shared__ uint64_t s_tab[32];
+    __shared__ uint64_t s_red[NWAVES], s_bb;
     __shared__ int      s_listed, s_base;
-    int                 row, chunk;
+    const int tid = threadIdx.x;
+    int       row, chunk;
     xcd_row_chunk(row, chunk);
-    if (threadIdx.x < 32)
-        s_tab[threadIdx.x] = g_expf_tab[threadIdx.x];
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    /* the slots that the launch before this one used, back to zero for the launch after */
+    {
+        const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, n_wg = gridDim.x * gridDim.y;
+        for (uint32_t i = wg * TPB + tid; i < meet.stale_count; i += n_wg * TPB)
+            meet.stale[i] = 0;
+    }
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
+    FusedScan fs;
+    fs.tmax       = tmax;
+    fs.chunk_best = chunk_best;
+    fs.slots      = meet.slots;
+    fs.wait_limit = meet.wait_limit;
+    fs.s_red      = s_red;
+    fs.s_bb       = &s_bb;
     const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
                        rv.allowed == nullptr;
     if (plain)
-        expsum_chunk<NV, PEN, LISTM, SLABS, true>(rv, row, chunk, (int) gridDim.y, base, end, inv_t,
-                                                  chunk_best, chunk_sum, slab_sum, probe_token,
-                                                  probe_L, probe_p, list, zb_list, s_cnt16, s_sum,
-                                                  s_tab, &s_listed, &s_base);
+        expsum_chunk<NV, PEN, LISTM, SLABS, true>(
+            rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, &s_listed, &s_base,
+            fs);
     else
-        expsum_chunk<NV, PEN, LISTM, SLABS, false>(rv, row, chunk, (int) gridDim.y, base, end,
-                                                   inv_t, chunk_best, chunk_sum, slab_sum,
-                                                   probe_token, probe_L, probe_p, list, zb_list,
-                                                   s_cnt16, s_sum, s_tab, &s_listed, &s_base);
+        expsum_chunk<NV, PEN, LISTM, SLABS, false>(
+            rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, &s_listed, &s_base,
+            fs);
 }
 
 /* ============================================================================================
@@ -1500,31 +1649,32 @@ static void dispatch(int nv, bool pen, F &&f) {
 #define GS_NV decltype(nv)::value
 #define GS_PEN decltype(pen)::value
 
-void launch_chunk_expsum(const Launch &L, float inv_t, const uint64_t *chunk_best,
-                         double *chunk_sum, const int32_t *probe_token, int probe_L,
-                         float *probe_p, const CandSpace *list, int zb_list, double *slab_sum) {
+int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
+                        double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
+                        const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     if (list && L.nv == 8) {
         if (L.pen)
-            k_chunk_expsum<8, true, true, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p, *list,
-                zb_list);
+            k_scan_expsum<8, true, true, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
+                *list, zb_list, meet);
         else
-            k_chunk_expsum<8, false, true, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p, *list,
-                zb_list);
-        return;
+            k_scan_expsum<8, false, true, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
+                *list, zb_list, meet);
+        return 0;
     }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         if (slab_sum)
-            k_chunk_expsum<GS_NV, GS_PEN, false, true><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, slab_sum, probe_token, probe_L, probe_p,
-                CandSpace{}, 0);
+            k_scan_expsum<GS_NV, GS_PEN, false, true><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, tmax, chunk_best, chunk_sum, slab_sum, probe_token, probe_L, probe_p,
+                CandSpace{}, 0, meet);
         else
-            k_chunk_expsum<GS_NV, GS_PEN, false, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
-                CandSpace{}, 0);
+            k_scan_expsum<GS_NV, GS_PEN, false, false><<<grid, block, 0, L.stream>>>(
+                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
+                CandSpace{}, 0, meet);
     });
+    return 0;
 }
 
 int zbin_of_min_p(float min_p) {

@@ -11,7 +11,7 @@
  *   j* < L : token ~ max(0, p_j* - q_j*) / R, walked in index order with u_L;
  *   j* = L : token ~ p_L, the temperature sampler's walk (sampler.c:90-102) with u_L.
  *
- * Kernels (after k_tmax_scan + k_chunk_expsum over all n_seq * (L+1) target rows):
+ * Kernels (after k_scan_expsum over all n_seq * (L+1) target rows):
  *   k_spec_accept  grid (n_seq): row sums and maxima, j*, the accepted ids and their count
  *   k_spec_resid   grid (chunks, n_seq): sums max(0, p - q) over its chunk of row j*
  *   k_spec_final   grid (n_seq): draws the last token

@@ -142,6 +142,14 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
                                  const float *d_uniforms, geist_hip_token_t *d_out_tokens,
                                  char *err, size_t err_len);
 
+/* No counterpart in the reference. The modes that need a row's maximum before they can sum its
+ * exponentials (temperature, top-p, min-p, softmax, speculative verification) read the rows
+ * once: the workgroups that share a row wait for one another inside the kernel. `polls` bounds
+ * that wait (default 65536 polls, tens of milliseconds); a workgroup that reaches the bound
+ * finds the row's maximum by reading the row itself, so the results never depend on it. 0 makes
+ * every workgroup do that at once, which is slow and meant for tests of that path. */
+int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
+
 /* Sizes, ahead of the first sampling call, whatever workspace the configuration needs beyond
  * what geist_hip_sampler_create made -- the reference sizes its workspace when the options are
  * applied (transformer_session_apply_opts, src/archs/transformer/forward/step.c:398-409), so that

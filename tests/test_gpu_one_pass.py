@@ -1,0 +1,103 @@
+"""The one-pass form of the modes that need a row's maximum before its exponentials (temperature,
+top-p / min-p, softmax, speculative verification): the workgroups of a row wait for one another
+inside the kernel, and one that stops waiting reads the row for itself. Both ways must give the
+oracle's ids; the second is forced from the host with a wait limit of 0 polls, so every workgroup
+still ends normally."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+from gpu_util import compare_ids, run_rows, to_dev  # noqa: E402
+
+
+@pytest.fixture()
+def hs():
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=256, max_vocab=160000)
+    yield s
+    s.close()
+
+
+def P(**kw):
+    from geistlib_amd import SampleParams
+    return SampleParams.make(**kw)
+
+
+def history_for(g, rows, n, length=300):
+    hist = g.integers(0, n, (rows, length)).astype(np.int32)
+    hist[:, :40] = hist[:, 40:80]          # repeated ids: counts above 1
+    hl = np.full(rows, length, dtype=np.int32)
+    hl[1] = 0
+    return hist, hl
+
+
+CASES = [
+    # (rows, n, sampling parameters, penalties)
+    (3, 5000, dict(temperature=0.8), False),
+    (8, 50000, dict(temperature=1.0), True),
+    (16, 128256, dict(temperature=0.7), False),
+    (8, 60000, dict(temperature=1.0, top_p=0.9), False),
+    (8, 60000, dict(temperature=1.0, top_p=0.95, min_p=0.05), True),
+    (5, 151936, dict(temperature=1.0, top_p=0.95, min_p=0.05), True),
+    (1, 128256, dict(temperature=0.8), False),
+]
+
+
+@pytest.mark.parametrize("wait_limit", [None, 0, 3])
+@pytest.mark.parametrize("rows,n,kw,pen", CASES)
+def test_waiting_and_not_waiting_give_the_oracles_ids(hs, oracle, rows, n, kw, pen, wait_limit):
+    print(f"one pass rows={rows} n={n} {kw} pen={pen} wait_limit={wait_limit}", flush=True)
+    g = np.random.default_rng(rows * 7 + n)
+    x = (g.standard_normal((rows, n)) * 2.5).astype(np.float32)
+    x[0, n // 3] = x[0].max()              # the maximum twice: the first index counts
+    u = g.random(rows).astype(np.float32)
+    hist = hl = None
+    pk = {}
+    if pen:
+        hist, hl = history_for(g, rows, n)
+        pk = dict(rep=1.2, freq=0.4, pres=0.2)
+    if wait_limit is not None:
+        hs.set_wait_limit(wait_limit)
+    for call in range(2):                  # the second call finds the meeting words as the first left them
+        got = run_rows(hs, torch, x, u, P(**kw, **pk), history=hist, history_len=hl)
+        res = []
+        for r in range(rows):
+            row = oracle.penalties(x[r], hist[r, :hl[r]], 1.2, 0.4, 0.2) if pen else x[r]
+            res.append(oracle.chain_u(row, float(u[r]), **kw))
+        near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"call {call}")
+        assert near <= 1
+
+
+@pytest.mark.parametrize("wait_limit", [None, 0])
+def test_normalised_probabilities_one_pass(hs, oracle, wait_limit):
+    rows, n, T = 4, 70001, 0.9
+    g = np.random.default_rng(9)
+    x = (g.standard_normal((rows, n)) * 3).astype(np.float32)
+    if wait_limit is not None:
+        hs.set_wait_limit(wait_limit)
+    d = to_dev(x, torch)
+    probs = torch.empty((rows, n), dtype=torch.float32, device="cuda")
+    from geistlib_amd import HipSampler
+    hs.softmax(HipSampler.rows(d), P(temperature=T), probs)
+    hs.sync()
+    got = probs.cpu().numpy()
+    for r in range(rows):
+        want, _ = oracle.softmax_normalised(x[r], T)
+        assert np.array_equal(got[r], want), r
+
+
+@pytest.mark.parametrize("wait_limit", [None, 0])
+def test_spec_verify_one_pass(hs, oracle, wait_limit):
+    from test_gpu_sampling import _run_spec, _spec_case
+    n_seq, L, n, T = 5, 6, 40000, 0.9
+    if wait_limit is not None:
+        hs.set_wait_limit(wait_limit)
+    target, q, draft, u = _spec_case(77, n_seq, L, n)
+    for call in range(2):
+        nacc, out = _run_spec(hs, target, q, draft, u, T)
+        for s in range(n_seq):
+            want_n, want = oracle.spec_verify(target[s], q[s], draft[s], u[s], T)
+            assert nacc[s] == want_n, (call, s)
+            assert out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), (call, s)
