@@ -4,6 +4,7 @@
 #include "lm_head_oracle.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* src/formats/gguf/common.c:29-62 */
@@ -166,5 +167,47 @@ void oracle_f16_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
                 acc += (double) x[i * n_in + k] * (double) oracle_f16_to_f32(wr[k]);
             y[i * n_out + j] = (float) acc;
         }
+    }
+}
+
+void oracle_dequant_q6_K_row(const void *blocks, float *out, size_t n_elems) {
+    /* q6_K.c:13-45; the block layout of src/quant/quant_blocks.h:67-73 by offsets */
+    const uint8_t *p = (const uint8_t *) blocks;
+    for (size_t b = 0; b < n_elems / 256; b++, p += 210) {
+        const uint8_t *ql = p, *qh = p + 128;
+        const int8_t  *sc = (const int8_t *) (p + 192);
+        const float    d  = oracle_f16_to_f32((uint16_t) (p[208] | (p[209] << 8)));
+        float         *y  = out + b * 256;
+        for (int h = 0; h < 2; h++)
+            for (int j = 0; j < 4; j++)
+                for (int l = 0; l < 32; l++) {
+                    const uint8_t lo = ql[64 * h + 32 * (j & 1) + l];
+                    const int     q  = (int) (((j >> 1) ? lo >> 4 : lo & 0xF) |
+                                             (((qh[32 * h + l] >> (2 * j)) & 3) << 4)) - 32;
+                    y[128 * h + 32 * j + l] = d * (float) sc[8 * h + 2 * j + l / 16] * (float) (int8_t) q;
+                }
+    }
+}
+
+void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const void *w_q6k, float *y) {
+    /* weight_resolve.c:186-241 */
+    const size_t row_bytes = n_in / 256 * 210;
+#pragma omp parallel
+    {
+        float *row = (float *) malloc(n_in * sizeof(float));
+#pragma omp for schedule(static)
+        for (size_t j = 0; j < n_out; j++) {
+            if (!row)
+                continue;
+            oracle_dequant_q6_K_row((const uint8_t *) w_q6k + j * row_bytes, row, n_in);
+            for (size_t i = 0; i < m; i++) {
+                double acc = 0.0;
+                for (size_t k = 0; k < n_in; k++)
+                    acc += (double) x[i * n_in + k] * (double) row[k];
+                y[i * n_out + j] = (float) acc;
+            }
+        }
+        free(row);
     }
 }

@@ -51,6 +51,23 @@ void oracle_q8w_gemv_m1(size_t n_out, size_t n_in, const float *x, const int8_t 
 void oracle_f16_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
                            const uint16_t *w_f16, float *y);
 
+/* Q6_K weights: super-blocks of 256 elements in 210 bytes -- ql[128] (low 4 bits), qh[64] (high
+ * 2 bits), scales[16] (int8, one per 16 elements), d (binary16) -- src/quant/quant_blocks.h:67-73.
+ * dequant_q6_K_row (src/formats/gguf/q6_K.c:13-45): element 128 h + 32 j + l of a block
+ * (h < 2, j < 4, l < 32) is d * scales[8 h + 2 j + l / 16] * (q - 32) with
+ * q = nibble (j >> 1) of ql[64 h + 32 (j & 1) + l] | ((qh[32 h + l] >> 2 j) & 3) << 4,
+ * multiplied left to right in binary32. (Both products are exact: 11 + 8 + 6 significant bits.)
+ * n_elems a multiple of 256. */
+void oracle_dequant_q6_K_row(const void *blocks, float *out, size_t n_elems);
+/* cpu_scalar_w_quant_m1 / _mN over a Q6_K table (src/backends/cpu_scalar/weight_resolve.c:
+ * 186-241 with the Q6_K case of dequant_one_row_for, :86-88): row j of the table is
+ * n_in / 256 blocks; y[i][j] = (float) sum_k (double) x[i][k] * (double) w[j][k], the sum in
+ * double in index order. Pinned by the reference's own weight_resolve.c and q6_K.c compiled from
+ * its tree (oracle/_ref/libgeist_ref_wquant.so, tests/test_q6k_oracle.py) bit for bit, and by
+ * golden vectors written from that build. */
+void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const void *w_q6k, float *y);
+
 /* y = x * weight * rsqrt(mean(x^2) + eps) per row (cpu_scalar_rmsnorm,
  * src/backends/cpu_scalar/elementwise.c:241-280): sum of squares in double in index order,
  * inv = (float)(1.0 / sqrt(sum / n + (double) eps)), y_i = (x_i * inv) * w_i in binary32. */

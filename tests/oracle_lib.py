@@ -413,3 +413,77 @@ class OracleSpecHead:
         if getattr(self, "p", None):
             self.lib.oracle_spec_head_free(self.p)
             self.p = None
+
+
+# ---- Q6_K tables ---------------------------------------------------------------------------
+Q6K_BLOCK_BYTES, Q6K_BLOCK_ELEMS = 210, 256
+
+
+def random_q6k_table(g, n_out, n_in, scale_mode="mixed"):
+    """A [n_out, n_in] table of Q6_K super-blocks as uint8 [n_out, n_in / 256 * 210]: every bit
+    pattern of ql / qh, int8 scales over their whole range (with 0, 127 and -128 forced in),
+    binary16 super-block scales that are normal, subnormal, zero or negative (never inf / NaN)."""
+    assert n_in % Q6K_BLOCK_ELEMS == 0
+    nb = n_in // Q6K_BLOCK_ELEMS
+    t = g.integers(0, 256, (n_out, nb, Q6K_BLOCK_BYTES), dtype=np.uint8)
+    sc = g.integers(-128, 128, (n_out, nb, 16)).astype(np.int8)
+    if scale_mode == "mixed":
+        sc[g.random((n_out, nb, 16)) < 0.05] = 0
+        sc[g.random((n_out, nb, 16)) < 0.02] = 127
+        sc[g.random((n_out, nb, 16)) < 0.02] = -128
+    t[:, :, 192:208] = sc.view(np.uint8)
+    d = (g.standard_normal((n_out, nb)) * 0.01).astype(np.float16)
+    kind = g.random((n_out, nb))
+    d[kind < 0.03] = np.float16(0.0)
+    d = d.view(np.uint16).copy()
+    sub = (kind >= 0.03) & (kind < 0.08)           # subnormal: exponent bits 0, mantissa random
+    d[sub] = (g.integers(1, 1024, int(sub.sum())) | (g.integers(0, 2, int(sub.sum())) << 15)).astype(np.uint16)
+    t[:, :, 208] = (d & 0xFF).astype(np.uint8)
+    t[:, :, 209] = (d >> 8).astype(np.uint8)
+    return np.ascontiguousarray(t.reshape(n_out, nb * Q6K_BLOCK_BYTES))
+
+
+def oracle_q6k_linear(lib, w_q6k, x, n_in):
+    """(float) sum_k (double) x[i][k] * (double) dequant(w[j][k]) for every activation row."""
+    xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    n_out = w_q6k.shape[0]
+    y = np.empty((xs.shape[0], n_out), dtype=np.float32)
+    lib.oracle_q6k_linear_f64.argtypes = [C.c_size_t] * 3 + [c_float_p, C.c_void_p, c_float_p]
+    lib.oracle_q6k_linear_f64.restype = None
+    lib.oracle_q6k_linear_f64(xs.shape[0], n_out, n_in, _fp(xs), w_q6k.ctypes.data_as(C.c_void_p),
+                              _fp(y))
+    return y
+
+
+def oracle_dequant_q6k(lib, w_q6k, n_in):
+    out = np.empty((w_q6k.shape[0], n_in), dtype=np.float32)
+    lib.oracle_dequant_q6_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
+    lib.oracle_dequant_q6_K_row.restype = None
+    for j in range(w_q6k.shape[0]):
+        lib.oracle_dequant_q6_K_row(w_q6k[j].ctypes.data_as(C.c_void_p), _fp(out[j]), n_in)
+    return out
+
+
+def load_ref_wquant(fast=False):
+    """The reference's portable linear kernels compiled from its tree, or None where not built
+    (lazy binding, as for load_ref_f16gemv)."""
+    path = os.path.join(ORACLE_DIR, "_ref",
+                        "libgeist_ref_wquant_fast.so" if fast else "libgeist_ref_wquant.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path, mode=os.RTLD_LAZY)
+    lib.ref_wquant_linear.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, c_float_p, C.c_size_t,
+                                      c_float_p]
+    lib.dequant_q6_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
+    lib.dequant_q6_K_row.restype = None
+    return lib
+
+
+def ref_q6k_linear(ref, w_q6k, x, n_in):
+    xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    n_out = w_q6k.shape[0]
+    y = np.full((xs.shape[0], n_out), np.nan, dtype=np.float32)
+    rc = ref.ref_wquant_linear(ref.ref_dtype_q6_K(), w_q6k.ctypes.data_as(C.c_void_p), n_out, n_in,
+                               _fp(xs), xs.shape[0], _fp(y))
+    assert rc == 0
+    return y
