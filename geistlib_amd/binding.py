@@ -102,6 +102,8 @@ def load_library():
     lib.geist_hip_rmsnorm_rows.argtypes = [vp, vp, sz, vp, f32, sz, sz, vp, sz]
     lib.geist_hip_f16_gemv_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_f16_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q6k_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q6k_linear_reserve.argtypes = [vp, sz, sz]
     lib.geist_hip_f16_to_q8w.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
@@ -277,6 +279,17 @@ class HipSampler:
         assert w_f16.is_contiguous() and w_f16.element_size() == 2 and x.shape[1] == n_in
         self._check(self.lib.geist_hip_f16_linear_rows(
             self.h, _ptr(w_f16), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def q6k_linear(self, w_q6k, n_in, x, y):
+        """w_q6k: uint8 [n_out, n_in / 256 * 210], the Q6_K super-blocks of each table row; the
+        portable kernel's arithmetic (sum in double in index order, rounded once)."""
+        n_out = w_q6k.shape[0]
+        m = x.shape[0]
+        assert w_q6k.is_contiguous() and w_q6k.element_size() == 1 and x.shape[1] == n_in
+        assert w_q6k.shape[1] == n_in // 256 * 210
+        self._check(self.lib.geist_hip_q6k_linear_rows(
+            self.h, _ptr(w_q6k), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 
     def f16_to_q8w(self, w_f16, wq, scales):

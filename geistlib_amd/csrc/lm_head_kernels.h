@@ -51,6 +51,22 @@ void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out
                            const float *x, long ld_x, int n_m, const F64Scratch &ws, float *y,
                            long ld_y);
 
+/* Scratch of the Q6_K projection, for one pass of up to Q6K_M_MAX rows. */
+constexpr int Q6K_M_MAX = 4;
+struct Q6KScratch {
+    double *xd;        /* [Q6K_M_MAX][n_in] the activations in double */
+    double *xsum;      /* [Q6K_M_MAX][n_in / 16] their sums per group of 16 */
+    double *xabs;      /* [Q6K_M_MAX][n_in / 16] the sums of their magnitudes */
+    int    *amb_count; /* outputs whose rounding depends on the order of the sum ... */
+    int2   *amb_list;  /* ... [n_out * Q6K_M_MAX] (table row, activation row) */
+};
+/* The portable kernel over a Q6_K table (cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row):
+ * y[m][r] = (float) sum_k (double) x[m][k] * (double) w[r][k], the sum as if in index order;
+ * n_m <= Q6K_M_MAX, n_in a multiple of 256, the table 4-byte aligned. */
+void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
+                       const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                       long ld_y);
+
 /* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *
  * scales[r]; n_in a multiple of 16. */
 void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, long n_out,

@@ -1,0 +1,263 @@
+/*
+ * lm_head_q6k.hip -- the lm_head projection over a Q6_K table (gfx950), with the results of the
+ * reference's portable kernels cpu_scalar_w_quant_m1 / _mN
+ * (src/backends/cpu_scalar/weight_resolve.c:186-241) after dequant_q6_K_row
+ * (src/formats/gguf/q6_K.c:13-45):
+ *   y[m][r] = (float) sum_k (double) x[m][k] * (double) w[r][k]        (double, index order)
+ *   w[r][k] = d * scale * (q - 32)                                     (binary32, left to right)
+ * A Q6_K super-block is 256 elements in 210 bytes (src/quant/quant_blocks.h:67-73): ql[128],
+ * qh[64], sixteen int8 scales, one binary16 d. Element 128 h + 32 j + l of a block has
+ * q = nibble (j >> 1) of ql[64 h + 32 (j & 1) + l] | ((qh[32 h + l] >> 2 j) & 3) << 4 and the
+ * scale 8 h + 2 j + l / 16.
+ *
+ * Arithmetic. d * scale has at most 11 + 8 significant bits and (q - 32) at most 6, so both
+ * binary32 products of the dequantisation are exact, and so is every product x * w in double
+ * (24 + 24 bits): the reference's result is the exact sum of the products but for the rounding
+ * of its 1 + n_in additions. Here a lane owns a table row. It adds, per group of 16 elements
+ * that share a scale, t = sum x * q_unsigned in double (exact products again), and then
+ * ds * (t - 32 * sum x) to the row's sum, ds = d * scale; the sums of x and |x| per group come
+ * with the double copy of the activations. The result differs from the reference's by at most
+ *   err = 2^-53 * (32 * sum_g (n_in - 16 g) |ds_g| X_g  +  (1700 + 96 n_g) * sum_g |ds_g| X_g),
+ * X_g = sum |x| over group g: the first term bounds the rounding of the reference's sequential
+ * additions (the k-th addition's error is at most 2^-53 times the sum of the |products| so
+ * far, and |w| <= 32 |ds|), the second everything this kernel rounds (16 additions per group on
+ * values below 63 X_g, the subtraction, the product with ds, one addition per group of the row's
+ * sum, n_g = n_in / 16 of them). When every value within err of the sum rounds to the same
+ * binary32 the reference's result is that binary32; otherwise -- a few outputs in ten thousand -- the output goes on a
+ * list and a second kernel adds its products once more one after the other in index order.
+ *
+ * Memory. A lane reads its row's blocks with aligned 16-byte loads straight from the table:
+ * consecutive loads of a lane use up the cache lines that its first load fetched, and all bytes
+ * of the table are read once. Blocks start on 2-byte boundaries; a block is fetched as the 53
+ * aligned dwords that hold it and shifted into place. The activations are uniform over the
+ * wavefront and come as scalar operands.
+ */
+#include "lm_head_kernels.h"
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gs {
+
+constexpr int Q6K_BLOCK_BYTES = 210;
+constexpr int Q6K_BLOCK_ELEMS = 256;
+constexpr int Q6K_TPB         = 256;
+
+/* (float) s, and whether every value within err of s rounds to the same binary32. */
+__device__ __forceinline__ bool q6k_rounding_is_safe(double s, double err, float &f) {
+    f = (float) s;
+    if (!(__builtin_fabsf(f) < __builtin_inff()))
+        return true; /* overflow or NaN: the order of the sum does not decide it */
+    const double up = 0.5 * ((double) f + (double) nextafterf(f, __builtin_inff()));
+    const double dn = 0.5 * ((double) f + (double) nextafterf(f, -__builtin_inff()));
+    return up - s > err && s - dn > err;
+}
+
+/* xd[m][k] = (double) x[m][k]; per group of 16 elements xsum = sum x and xabs = sum |x| (rounded
+ * up); the count of listed outputs starts at zero. One workgroup per activation row. */
+__global__ __launch_bounds__(Q6K_TPB) void k_q6k_x_prep(const float *__restrict__ x, long ld_x,
+                                                        int n_in, double *__restrict__ xd,
+                                                        double *__restrict__ xsum,
+                                                        double *__restrict__ xabs,
+                                                        int *amb_count) {
+    const int    m  = blockIdx.x;
+    const float *xr = x + (long) m * ld_x;
+    if (m == 0 && threadIdx.x == 0)
+        *amb_count = 0;
+    for (int k = threadIdx.x; k < n_in; k += Q6K_TPB)
+        xd[(long) m * n_in + k] = (double) xr[k];
+    const int n_g = n_in / 16;
+    for (int g = threadIdx.x; g < n_g; g += Q6K_TPB) {
+        double s = 0.0, a = 0.0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const double v = (double) xr[16 * g + i];
+            s += v;
+            a += __builtin_fabs(v);
+        }
+        xsum[(long) m * n_g + g] = s;
+        xabs[(long) m * n_g + g] = a * (1.0 + 0x1p-40);
+    }
+}
+
+typedef uint32_t q6k_u32x4 __attribute__((ext_vector_type(4), aligned(4)));
+
+/* The 53 dwords of the block at `bp` (2-byte aligned), shifted into place: d[0..31] ql,
+ * d[32..47] qh, d[48..51] the scales, the low half of d[52] the binary16 d. The aligned dwords
+ * that hold the block are read whole; what they hold beyond the block lies in the same aligned
+ * dword as a byte of the block, so no load leaves the table's pages. */
+__device__ __forceinline__ void q6k_load_block(const uint8_t *bp, uint32_t (&d)[53]) {
+    const uintptr_t a     = reinterpret_cast<uintptr_t>(bp);
+    const uint32_t  shift = (uint32_t) (a & 2) * 8; /* 0 or 16 */
+    const uint32_t *p     = reinterpret_cast<const uint32_t *>(a & ~(uintptr_t) 3);
+    uint32_t        raw[54];
+#pragma unroll
+    for (int i = 0; i < 52; i += 4) {
+        const q6k_u32x4 q = *reinterpret_cast<const q6k_u32x4 *>(p + i);
+        raw[i] = q.x, raw[i + 1] = q.y, raw[i + 2] = q.z, raw[i + 3] = q.w;
+    }
+    raw[52] = p[52];
+    raw[53] = 0u; /* (only the low half of d[52] is used, and raw[52] holds it either way) */
+#pragma unroll
+    for (int i = 0; i < 53; ++i)
+        d[i] = __builtin_amdgcn_alignbit(raw[i + 1], raw[i], shift);
+}
+
+/* byte i of v as a float (one conversion instruction per byte) */
+__device__ __forceinline__ float q6k_ubyte(uint32_t v, int i) {
+    return (float) ((v >> (8 * i)) & 0xffu);
+}
+
+template <int MT>
+__global__ __launch_bounds__(Q6K_TPB) void k_q6k_linear(const uint8_t *__restrict__ w, long n_out,
+                                                        int n_in, const double *__restrict__ xd,
+                                                        const double *__restrict__ xsum,
+                                                        const double *__restrict__ xabs, int n_m,
+                                                        float *__restrict__ y, long ld_y,
+                                                        int *__restrict__ amb_count,
+                                                        int2 *__restrict__ amb_list) {
+    const long row = (long) blockIdx.x * Q6K_TPB + threadIdx.x;
+    if (row >= n_out)
+        return;
+    const int      nb  = n_in / Q6K_BLOCK_ELEMS, n_g = n_in / 16;
+    const uint8_t *rp  = w + row * (long) nb * Q6K_BLOCK_BYTES;
+    double         S[MT], B[MT], Bw[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        S[m] = B[m] = Bw[m] = 0.0;
+    for (int b = 0; b < nb; ++b) {
+        uint32_t d[53];
+        q6k_load_block(rp + (long) b * Q6K_BLOCK_BYTES, d);
+        const float dd = __half2float(__ushort_as_half((unsigned short) (d[52] & 0xffffu)));
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int is = 0; is < 2; ++is) {
+                double t[4][MT];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m)
+                        t[j][m] = 0.0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint32_t ql_a = d[16 * h + 4 * is + s];
+                    const uint32_t ql_b = d[16 * h + 8 + 4 * is + s];
+                    const uint32_t qh4  = d[32 + 8 * h + 4 * is + s];
+                    uint32_t       qu[4]; /* the unsigned 6-bit values of four elements, a byte each */
+                    qu[0] = (ql_a & 0x0F0F0F0Fu) | ((qh4 << 4) & 0x30303030u);
+                    qu[1] = (ql_b & 0x0F0F0F0Fu) | ((qh4 << 2) & 0x30303030u);
+                    qu[2] = ((ql_a >> 4) & 0x0F0F0F0Fu) | (qh4 & 0x30303030u);
+                    qu[3] = ((ql_b >> 4) & 0x0F0F0F0Fu) | ((qh4 >> 2) & 0x30303030u);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        /* elements 256 b + 128 h + 32 j + 16 is + 4 s + i */
+                        const int k0 = Q6K_BLOCK_ELEMS * b + 128 * h + 32 * j + 16 * is + 4 * s;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const double q = (double) q6k_ubyte(qu[j], i);
+#pragma unroll
+                            for (int m = 0; m < MT; ++m) {
+                                const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in;
+                                t[j][m] = __builtin_fma(xm[k0 + i], q, t[j][m]); /* uniform address */
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int    si = 8 * h + 2 * j + is; /* scale of the group within the block */
+                    const int    sc = (int) (int8_t) (d[48 + si / 4] >> (8 * (si % 4)));
+                    const double ds = (double) (dd * (float) sc);
+                    const int    g  = 16 * b + si;        /* the group's place in the row */
+                    const double pos = (double) (n_in - 16 * g);
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) {
+                        const long   at = (long) (m < n_m ? m : n_m - 1) * n_g + g;
+                        const double v  = __builtin_fma(-32.0, xsum[at], t[j][m]);
+                        S[m]            = __builtin_fma(ds, v, S[m]);
+                        const double bx = __builtin_fabs(ds) * xabs[at];
+                        B[m] += bx;
+                        Bw[m] = __builtin_fma(pos, bx, Bw[m]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if (m < n_m) {
+            const double err =
+                0x1p-53 * (32.0 * Bw[m] + (1700.0 + 96.0 * n_g) * B[m]) * (1.0 + 0x1p-30);
+            float        f;
+            if (!q6k_rounding_is_safe(S[m], err, f))
+                amb_list[atomicAdd(amb_count, 1)] = make_int2((int) row, m);
+            y[m * ld_y + row] = f;
+        }
+    }
+}
+
+/* The listed outputs once more: a lane per output (table row r, activation row m) adds its
+ * row's products one after the other in index order, as the reference does. */
+__global__ __launch_bounds__(64) void k_q6k_linear_listed(const uint8_t *__restrict__ w, int n_in,
+                                                          const double *__restrict__ xd,
+                                                          float *__restrict__ y, long ld_y,
+                                                          const int *__restrict__ amb_count,
+                                                          const int2 *__restrict__ amb_list) {
+    const int count = *amb_count;
+    const int nb    = n_in / Q6K_BLOCK_ELEMS;
+    for (int it = blockIdx.x * 64 + threadIdx.x; it < count; it += gridDim.x * 64) {
+        const int2     mine = amb_list[it];
+        const uint8_t *rp   = w + (long) mine.x * nb * Q6K_BLOCK_BYTES;
+        const double  *xm   = xd + (long) mine.y * n_in;
+        double         acc  = 0.0;
+        for (int b = 0; b < nb; ++b) {
+            const uint8_t *p  = rp + (long) b * Q6K_BLOCK_BYTES;
+            const float    dd = __half2float(
+                __ushort_as_half((unsigned short) (p[208] | ((unsigned) p[209] << 8))));
+            for (int h = 0; h < 2; ++h)
+                for (int j = 0; j < 4; ++j) {
+                    const uint8_t *ql = p + 64 * h + 32 * (j & 1);
+                    const uint8_t *qh = p + 128 + 32 * h;
+                    for (int l = 0; l < 32; ++l) {
+                        const uint32_t lo = ql[l];
+                        const int      q  = (int) (((j >> 1) ? lo >> 4 : lo & 0xFu) |
+                                                  (((qh[l] >> (2 * j)) & 3u) << 4)) - 32;
+                        const int   sc = (int) (int8_t) p[192 + 8 * h + 2 * j + l / 16];
+                        const float wv = dd * (float) sc * (float) q; /* q6_K.c:37-40 */
+                        acc = __builtin_fma(xm[Q6K_BLOCK_ELEMS * b + 128 * h + 32 * j + l],
+                                            (double) wv, acc);
+                    }
+                }
+        }
+        y[mine.y * ld_y + mine.x] = (float) acc;
+    }
+}
+
+void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
+                       const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                       long ld_y) {
+    k_q6k_x_prep<<<dim3(n_m), dim3(Q6K_TPB), 0, stream>>>(x, ld_x, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                         ws.amb_count);
+    const dim3 grid((unsigned) ((n_out + Q6K_TPB - 1) / Q6K_TPB)), block(Q6K_TPB);
+    switch (n_m) {
+    case 1:
+        k_q6k_linear<1><<<grid, block, 0, stream>>>(w_q6k, n_out, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                    n_m, y, ld_y, ws.amb_count, ws.amb_list);
+        break;
+    case 2:
+        k_q6k_linear<2><<<grid, block, 0, stream>>>(w_q6k, n_out, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                    n_m, y, ld_y, ws.amb_count, ws.amb_list);
+        break;
+    default:
+        k_q6k_linear<4><<<grid, block, 0, stream>>>(w_q6k, n_out, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                    n_m, y, ld_y, ws.amb_count, ws.amb_list);
+        break;
+    }
+    /* the list is short (a few outputs in ten thousand): a handful of wavefronts */
+    k_q6k_linear_listed<<<dim3(64), dim3(64), 0, stream>>>(w_q6k, n_in, ws.xd, y, ld_y,
+                                                           ws.amb_count, ws.amb_list);
+}
+
+} // namespace gs

@@ -62,6 +62,8 @@ struct geist_hip_sampler {
     float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
                                      * full-vocabulary top-p / min-p path */
     gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
+    void    *q6k_ws      = nullptr; /* scratch of the Q6_K projection, sized like f64_ws */
+    size_t   q6k_in = 0, q6k_out = 0;
     void    *f64_ws      = nullptr; /* scratch of the f64 projection for n_in <= f64_in and
                                      * n_out <= f64_out, allocated on first use */
     size_t   f64_in = 0, f64_out = 0;
@@ -320,6 +322,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
     (void) hipFree(s->f64_ws);
+    (void) hipFree(s->q6k_ws);
     (void) hipFree(s->cand.row_bound);
     (void) hipFree(s->cand.out_key);
     (void) hipFree(s->cand.key);
@@ -943,6 +946,89 @@ static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t
     return GEIST_HIP_OK;
 }
 
+/* Scratch of the Q6_K projection: the activations in double, their sums and magnitudes per
+ * group of 16, the list of outputs for the second kernel. */
+static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScratch &ws) {
+    if (s->q6k_in < n_in || s->q6k_out < n_out) {
+        if (s->q6k_ws) {
+            HIPCHK(s, hipStreamSynchronize(s->stream));
+            (void) hipFree(s->q6k_ws);
+            s->q6k_ws = nullptr, s->q6k_in = s->q6k_out = 0;
+        }
+        const size_t in = n_in > s->q6k_in ? n_in : s->q6k_in;
+        const size_t out = n_out > s->q6k_out ? n_out : s->q6k_out;
+        const size_t bytes = (size_t) Q6K_M_MAX * (in + in / 8) * sizeof(double) + 16 +
+                             out * Q6K_M_MAX * sizeof(int2);
+        if (hipMalloc(&s->q6k_ws, bytes) != hipSuccess) {
+            s->q6k_ws = nullptr;
+            return fail(s, GEIST_HIP_E_OOM, "Q6_K projection: scratch");
+        }
+        s->q6k_in = in, s->q6k_out = out;
+    }
+    char *p      = static_cast<char *>(s->q6k_ws);
+    ws.xd        = reinterpret_cast<double *>(p);
+    ws.xsum      = ws.xd + (size_t) Q6K_M_MAX * s->q6k_in;
+    ws.xabs      = ws.xsum + (size_t) Q6K_M_MAX * (s->q6k_in / 16);
+    ws.amb_count = reinterpret_cast<int *>(ws.xabs + (size_t) Q6K_M_MAX * (s->q6k_in / 16));
+    ws.amb_list  = reinterpret_cast<int2 *>(reinterpret_cast<char *>(ws.amb_count) + 16);
+    return GEIST_HIP_OK;
+}
+
+static int q6k_linear_impl(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
+                           const float *d_x, size_t ld_x, size_t n_rows, float *d_y, size_t ld_y) {
+    Q6KScratch ws;
+    const int  rc = q6k_scratch(s, n_out, n_in, ws);
+    if (rc)
+        return rc;
+    for (size_t m0 = 0; m0 < n_rows; m0 += Q6K_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) Q6K_M_MAX ? n_rows - m0 : (size_t) Q6K_M_MAX;
+        launch_q6k_linear(s->stream, static_cast<const uint8_t *>(d_w_q6k), (long) n_out,
+                          (int) n_in, d_x + m0 * ld_x, (long) ld_x, (int) m, ws, d_y + m0 * ld_y,
+                          (long) ld_y);
+    }
+    return GEIST_HIP_OK;
+}
+
+static int q6k_check(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in) {
+    if (n_out == 0 || n_in == 0 || n_in > 0x7fffff00u || n_out > 0x7fffffffu)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K table: %zu x %zu", n_out, n_in);
+    if (n_in % 256 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED,
+                    "Q6_K table: n_in %zu is not a multiple of the 256-element block", n_in);
+    if (((uintptr_t) d_w_q6k) % 4 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K table not 4-byte aligned");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_q6k_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    const int rc = q6k_check(s, nullptr, n_out, n_in);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    Q6KScratch ws;
+    return q6k_scratch(s, n_out, n_in, ws);
+}
+
+int geist_hip_q6k_linear_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
+                              const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
+                              size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_q6k || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K linear: %zu rows, strides %zu / %zu", n_rows,
+                    ld_x, ld_y);
+    int rc = q6k_check(s, d_w_q6k, n_out, n_in);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q6k_linear_impl(s, d_w_q6k, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q6_K linear");
+}
+
 int geist_hip_f16_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
@@ -1009,17 +1095,20 @@ int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const floa
     return after_launch(s, "q8w gemv");
 }
 
-/* Norm, projection and sampling; the table is binary16 (d_scales == NULL) or int8 with one
- * scale per row. */
+/* Norm, projection and sampling; the table is binary16, int8 with one scale per row (d_scales),
+ * or Q6_K super-blocks. */
+enum { TABLE_F16 = 0, TABLE_Q8W = 1, TABLE_Q6K = 2 };
 static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
                                size_t rows, size_t d_model, const float *d_norm_weight,
-                               float rms_eps, const void *d_embed, const float *d_scales,
-                               size_t n_vocab, float *d_normed, float *d_logits, size_t ld_logits,
+                               float rms_eps, int table, const void *d_embed,
+                               const float *d_scales, size_t n_vocab, float *d_normed,
+                               float *d_logits, size_t ld_logits,
                                const struct geist_hip_sample_params *params,
                                const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                geist_hip_token_t *d_out_tokens) {
-    const bool      q8          = d_scales != nullptr;
-    const size_t    in_multiple = q8 ? 16 : 8;
+    const bool      q8          = table == TABLE_Q8W;
+    const bool      q6k         = table == TABLE_Q6K;
+    const size_t    in_multiple = q6k ? 256 : q8 ? 16 : 8;
     const uint16_t *d_embed_f16 = (const uint16_t *) d_embed;
     const int8_t   *d_embed_q8  = (const int8_t *) d_embed;
     if (!d_hidden || !d_norm_weight || !d_embed || !d_logits || !params || !d_out_tokens)
@@ -1044,8 +1133,8 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     if ((rc = check_call(s, &r, params, d_out_tokens)) != GEIST_HIP_OK)
         return rc; /* before any draw */
     HIPCHK(s, hipSetDevice(s->device));
-    const bool f64     = !q8 && (rows > 1 || s->projection_portable);
-    const bool fuse_ok = f16_gemv_can_fuse((int) rows) && !f64;
+    const bool f64     = table == TABLE_F16 && (rows > 1 || s->projection_portable);
+    const bool fuse_ok = f16_gemv_can_fuse((int) rows) && !f64 && !q6k;
     /* the top-k path's scan is the projection's epilogue when nothing changes the logits
      * between the two (no soft-cap) */
     const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX &&
@@ -1064,6 +1153,12 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+    } else if (q6k) {
+        /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
+        rc = q6k_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows, d_logits,
+                             ld_logits);
+        if (rc)
+            return rc;
     } else if (f64) {
         /* more than one row: the reference's batch kernel (cpu_scalar_w_quant_mN), its x86
          * kernels being decode-only; or the portable backend asked for */
@@ -1104,7 +1199,7 @@ int geist_hip_project_sample_rows(geist_hip_sampler *s, const float *d_hidden, s
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
-                               d_embed_f16, nullptr, n_vocab, d_normed, d_logits, ld_logits,
+                               TABLE_F16, d_embed_f16, nullptr, n_vocab, d_normed, d_logits, ld_logits,
                                params, d_uniforms, d_rng_states, shared, d_out_tokens);
 }
 
@@ -1122,8 +1217,23 @@ int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidde
     if (!d_scales)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
     return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
-                               d_embed_q8, d_scales, n_vocab, d_normed, d_logits, ld_logits,
+                               TABLE_Q8W, d_embed_q8, d_scales, n_vocab, d_normed, d_logits, ld_logits,
                                params, d_uniforms, d_rng_states, shared, d_out_tokens);
+}
+
+int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
+                                      size_t ld_hidden, size_t rows, size_t d_model,
+                                      const float *d_norm_weight, float rms_eps,
+                                      const void *d_embed_q6k, size_t n_vocab, float *d_normed,
+                                      float *d_logits, size_t ld_logits,
+                                      const struct geist_hip_sample_params *params,
+                                      const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                      geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
+                               TABLE_Q6K, d_embed_q6k, nullptr, n_vocab, d_normed, d_logits,
+                               ld_logits, params, d_uniforms, d_rng_states, shared, d_out_tokens);
 }
 
 int geist_hip_propose_drafts_ngram(geist_hip_sampler *s, const int32_t *d_history,

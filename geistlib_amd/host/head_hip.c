@@ -144,7 +144,10 @@ int geist_hip_head_apply_opts(struct geist_hip_head *h, const struct geist_sessi
     return GEIST_HIP_OK;
 }
 
-int geist_hip_head_reserve_projection(struct geist_hip_head *h, size_t d_model) {
+/* The [m_max, vocab] logit buffer and the normed rows; *grown says whether d_model outgrew what
+ * was there. */
+static int reserve_head_buffers(struct geist_hip_head *h, size_t d_model, bool *grown) {
+    *grown = false;
     if (h == nullptr || d_model == 0)
         return GEIST_HIP_E_INVALID_ARG;
     void *p = nullptr;
@@ -161,11 +164,20 @@ int geist_hip_head_reserve_projection(struct geist_hip_head *h, size_t d_model) 
             return head_fail(h, GEIST_HIP_E_OOM, "buffer of normed rows");
         h->d_normed    = p;
         h->d_model_cap = d_model;
-        /* a batch of rows goes through the double-precision projection, which has scratch */
-        if (h->m_max > 1 && d_model % 8 == 0 &&
-            geist_hip_f16_linear_reserve(h->hs, h->vocab, d_model) != GEIST_HIP_OK)
-            return head_fail(h, GEIST_HIP_E_OOM, "scratch of the batch projection");
+        *grown         = true;
     }
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_reserve_projection(struct geist_hip_head *h, size_t d_model) {
+    bool      grown;
+    const int rc = reserve_head_buffers(h, d_model, &grown);
+    if (rc != GEIST_HIP_OK)
+        return rc;
+    /* a batch of rows goes through the double-precision projection, which has scratch */
+    if (grown && h->m_max > 1 && d_model % 8 == 0 &&
+        geist_hip_f16_linear_reserve(h->hs, h->vocab, d_model) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_OOM, "scratch of the batch projection");
     return GEIST_HIP_OK;
 }
 
@@ -200,24 +212,42 @@ int geist_hip_head_finalize_batch(struct geist_hip_head *h, const float *d_logit
     return finalize(h, d_logits, k, out_tokens);
 }
 
-/* The table is binary16 (d_scales == nullptr) or int8 with one scale per row. */
+static int project_finalize_table(struct geist_hip_head *h, const float *d_hidden,
+                                  size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                  float rms_eps, const void *d_embed, const float *d_scales,
+                                  bool q6k, size_t d_model, int32_t *out_tokens);
+
+/* The table is binary16 (d_scales == nullptr), int8 with one scale per row, or Q6_K blocks. */
 static int project_finalize(struct geist_hip_head *h, const float *d_hidden, size_t ld_hidden,
                             size_t k, const float *d_norm_weight, float rms_eps,
                             const void *d_embed, const float *d_scales, size_t d_model,
                             int32_t *out_tokens) {
+    return project_finalize_table(h, d_hidden, ld_hidden, k, d_norm_weight, rms_eps, d_embed,
+                                  d_scales, false, d_model, out_tokens);
+}
+
+static int project_finalize_table(struct geist_hip_head *h, const float *d_hidden,
+                                  size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                  float rms_eps, const void *d_embed, const float *d_scales,
+                                  bool q6k, size_t d_model, int32_t *out_tokens) {
     if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed == nullptr ||
         out_tokens == nullptr || k == 0 || d_model == 0)
         return GEIST_HIP_E_INVALID_ARG;
     if (k > h->m_max)
         return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
-    /* a no-op after geist_hip_head_reserve_projection with this d_model */
-    const int rrc = geist_hip_head_reserve_projection(h, d_model);
+    /* a no-op after geist_hip_head_reserve_projection[_q6k] with this d_model */
+    const int rrc = q6k ? geist_hip_head_reserve_projection_q6k(h, d_model)
+                        : geist_hip_head_reserve_projection(h, d_model);
     if (rrc != GEIST_HIP_OK)
         return rrc;
     /* head.c:99-101, 114-126, then the dispatch of 172-183 / 291-302 with the session's RNG */
     const struct geist_hip_sample_params prm = head_params(h);
     const int rc =
-            d_scales != nullptr
+            q6k ? geist_hip_project_sample_rows_q6k(h->hs, d_hidden, ld_hidden, k, d_model,
+                                                    d_norm_weight, rms_eps, d_embed, h->vocab,
+                                                    h->d_normed, h->d_logits, h->vocab, &prm,
+                                                    nullptr, h->d_rng, /*shared=*/1, h->d_tokens)
+            : d_scales != nullptr
                     ? geist_hip_project_sample_rows_q8w(h->hs, d_hidden, ld_hidden, k, d_model,
                                                         d_norm_weight, rms_eps, d_embed, d_scales,
                                                         h->vocab, h->d_normed, h->d_logits,
@@ -235,6 +265,24 @@ static int project_finalize(struct geist_hip_head *h, const float *d_hidden, siz
     for (size_t r = 0; r < k; r++)
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
             return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const void *d_embed_q6k, size_t d_model,
+                                        int32_t *out_tokens) {
+    return project_finalize_table(h, d_hidden, ld_hidden, k, d_norm_weight, rms_eps, d_embed_q6k,
+                                  nullptr, true, d_model, out_tokens);
+}
+
+int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model) {
+    bool      grown;
+    const int rc = reserve_head_buffers(h, d_model, &grown);
+    if (rc != GEIST_HIP_OK)
+        return rc;
+    if (geist_hip_q6k_linear_reserve(h->hs, h->vocab, d_model) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_OOM, "scratch of the Q6_K projection");
     return GEIST_HIP_OK;
 }
 

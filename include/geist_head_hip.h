@@ -104,6 +104,23 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
                                         float rms_eps, const int8_t *d_embed_q8,
                                         const float *d_scales, size_t d_model,
                                         int32_t *out_tokens);
+/* The same over a Q6_K table as it lies in a GGUF file (the tied embedding of the Gemma models,
+ * whose logit soft-cap the head was created with): d_embed_q6k holds vocab rows of d_model / 256
+ * super-blocks of 210 bytes, d_model a multiple of 256. The logits equal, bit for bit, those of
+ * the reference's portable kernel cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row
+ * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch; the
+ * x86 backend's one-row path through cblas_sgemv (src/backends/cpu_x86/backend.c:395-397) sums
+ * in the order of the BLAS library it is linked with and is not reproduced. The other GGUF
+ * block formats the reference resolves for an embedding table (Q4_K, I2_S) and an F32 table have
+ * no device kernel here: their callers project on the host or with their own kernel and pass
+ * the logits to geist_hip_head_finalize_one_row / _batch.
+ * geist_hip_head_reserve_projection_q6k is geist_hip_head_reserve_projection plus the scratch of
+ * this kernel. */
+int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const void *d_embed_q6k, size_t d_model,
+                                        int32_t *out_tokens);
+int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model);
 /* The speculative output head of greedy decoding (src/archs/transformer/forward/spec_head.c;
  * include/geist_lm_head_hip.h has the device entry points). geist_hip_head_spec_build is
  * transformer_spec_head_init (spec_head.c:616-622) for a tied F16 table in device memory, which

@@ -115,6 +115,36 @@ int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidde
                                       const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                       geist_hip_token_t *d_out_tokens);
 
+/* The lm_head over a Q6_K table, the tied embedding of the Gemma models (which also carry the
+ * soft-cap that the sampler applies): d_w_q6k holds n_out rows of n_in / 256 super-blocks of 210
+ * bytes (src/quant/quant_blocks.h:67-73), as they lie in a GGUF file, 4-byte aligned, n_in a
+ * multiple of 256 (GEIST_HIP_E_UNSUPPORTED otherwise: the format has no partial blocks).
+ * geist_hip_q6k_linear_rows replaces cpu_scalar_w_quant_m1 / _mN for that dtype
+ * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241; decoder: src/formats/gguf/q6_K.c):
+ *   d_y[m * ld_y + r] = (float) sum_k (double) d_x[m * ld_x + k] * (double) w[r][k],
+ * w = d * scale * (q - 32) in binary32, the sum in double in index order, bit for bit (the device
+ * adds in another order and repeats, in the reference's order, the few sums that lie close enough
+ * to a binary32 rounding boundary for the order to matter). This is the arithmetic of the
+ * reference's portable backend for any number of rows and of its x86 backend for more than one
+ * row; for one row the x86 backend decodes the table to binary32 once and calls cblas_sgemv
+ * (src/backends/cpu_x86/backend.c:395-397), whose order of summation belongs to the BLAS library
+ * and is not reproduced. geist_hip_q6k_linear_reserve sizes the scratch ahead of the first call,
+ * as geist_hip_f16_linear_reserve does. */
+int geist_hip_q6k_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in);
+int geist_hip_q6k_linear_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
+                              const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
+                              size_t ld_y);
+/* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, geist_hip_q6k_linear_rows
+ * and the sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. */
+int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
+                                      size_t ld_hidden, size_t rows, size_t d_model,
+                                      const float *d_norm_weight, float rms_eps,
+                                      const void *d_embed_q6k, size_t n_vocab, float *d_normed,
+                                      float *d_logits, size_t ld_logits,
+                                      const struct geist_hip_sample_params *params,
+                                      const float *d_uniforms, uint64_t *d_rng_states, int shared,
+                                      geist_hip_token_t *d_out_tokens);
+
 /* The reference's speculative output head for greedy decoding
  * (src/archs/transformer/forward/spec_head.c), over a tied F16 table in device memory: an int8
  * sketch of the table ranks the vocabulary, only the best-ranked rows get their exact logit.
