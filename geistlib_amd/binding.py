@@ -111,6 +111,8 @@ def load_library():
     lib.geist_hip_project_sample_rows_q8w.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, vp, sz, vp,
                                                       vp, sz, C.POINTER(SampleParams), vp, vp,
                                                       i32, vp]
+    lib.geist_hip_project_sample_rows_q6k.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp,
+                                                      sz, C.POINTER(SampleParams), vp, vp, i32, vp]
     lib.geist_hip_spec_head_geometry.argtypes = [sz, sz, sz, sz, C.POINTER(sz), C.POINTER(sz)]
     lib.geist_hip_spec_head_build.argtypes = [vp, vp, sz, sz, sz, sz, C.POINTER(vp)]
     lib.geist_hip_spec_head_destroy.argtypes = [vp, vp]
@@ -326,6 +328,18 @@ class HipSampler:
         self._check(self.lib.geist_hip_project_sample_rows_q8w(
             self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
             _ptr(norm_w), eps, _ptr(embed_q8), _ptr(scales), vocab, _ptr(normed), _ptr(logits),
+            logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
+            _ptr(rng_states), int(shared), _ptr(out)))
+
+    def project_sample_q6k(self, hidden, norm_w, eps, embed_q6k, logits, params, uniforms, out,
+                           normed=None, rng_states=None, shared=True):
+        """project_sample over a Q6_K table: uint8 [vocab, d_model / 256 * 210]."""
+        rows, d_model = hidden.shape
+        vocab = embed_q6k.shape[0]
+        assert embed_q6k.is_contiguous() and embed_q6k.shape[1] == d_model // 256 * 210
+        self._check(self.lib.geist_hip_project_sample_rows_q6k(
+            self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
+            _ptr(norm_w), eps, _ptr(embed_q6k), vocab, _ptr(normed), _ptr(logits),
             logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
             _ptr(rng_states), int(shared), _ptr(out)))
 

@@ -198,40 +198,58 @@ __global__ __launch_bounds__(Q6K_TPB) void k_q6k_linear(const uint8_t *__restric
     }
 }
 
-/* The listed outputs once more: a lane per output (table row r, activation row m) adds its
- * row's products one after the other in index order, as the reference does. */
-__global__ __launch_bounds__(64) void k_q6k_linear_listed(const uint8_t *__restrict__ w, int n_in,
-                                                          const double *__restrict__ xd,
-                                                          float *__restrict__ y, long ld_y,
-                                                          const int *__restrict__ amb_count,
-                                                          const int2 *__restrict__ amb_list) {
+/* The listed outputs once more, the products added one after the other in index order as the
+ * reference adds them. A wavefront per output (table row r, activation row m): its lanes form 64
+ * products at a time -- each exact in double, whichever way it is computed -- and the sum takes
+ * them in order, lane by lane, as scalar operands. The chain of n_in dependent additions
+ * is what this kernel takes; there are few listed outputs and each has a wavefront to itself. */
+constexpr int Q6K_LISTED_WAVES = 4;
+__global__ __launch_bounds__(64 * Q6K_LISTED_WAVES) void k_q6k_linear_listed(
+    const uint8_t *__restrict__ w, int n_in, const double *__restrict__ xd, float *__restrict__ y,
+    long ld_y, const int *__restrict__ amb_count, const int2 *__restrict__ amb_list) {
     const int count = *amb_count;
     const int nb    = n_in / Q6K_BLOCK_ELEMS;
-    for (int it = blockIdx.x * 64 + threadIdx.x; it < count; it += gridDim.x * 64) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int it0 = blockIdx.x * Q6K_LISTED_WAVES; it0 < count;
+         it0 += gridDim.x * Q6K_LISTED_WAVES) {
+        const int      it   = it0 + wave < count ? it0 + wave : count - 1;
         const int2     mine = amb_list[it];
         const uint8_t *rp   = w + (long) mine.x * nb * Q6K_BLOCK_BYTES;
         const double  *xm   = xd + (long) mine.y * n_in;
         double         acc  = 0.0;
         for (int b = 0; b < nb; ++b) {
-            const uint8_t *p  = rp + (long) b * Q6K_BLOCK_BYTES;
+            /* the four 64-element rounds of a block: their loads first, all in flight together */
+            const uint8_t *p = rp + (long) b * Q6K_BLOCK_BYTES;
+            const int      l = lane & 31;
             const float    dd = __half2float(
                 __ushort_as_half((unsigned short) (p[208] | ((unsigned) p[209] << 8))));
-            for (int h = 0; h < 2; ++h)
-                for (int j = 0; j < 4; ++j) {
-                    const uint8_t *ql = p + 64 * h + 32 * (j & 1);
-                    const uint8_t *qh = p + 128 + 32 * h;
-                    for (int l = 0; l < 32; ++l) {
-                        const uint32_t lo = ql[l];
-                        const int      q  = (int) (((j >> 1) ? lo >> 4 : lo & 0xFu) |
-                                                  (((qh[l] >> (2 * j)) & 3u) << 4)) - 32;
-                        const int   sc = (int) (int8_t) p[192 + 8 * h + 2 * j + l / 16];
-                        const float wv = dd * (float) sc * (float) q; /* q6_K.c:37-40 */
-                        acc = __builtin_fma(xm[Q6K_BLOCK_ELEMS * b + 128 * h + 32 * j + l],
-                                            (double) wv, acc);
-                    }
+            double prod[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { /* element 64 r + lane: h = r / 2, j = 2 (r & 1) + lane / 32 */
+                const int      h = r >> 1, j = 2 * (r & 1) + (lane >> 5);
+                const uint32_t lo = p[64 * h + 32 * (j & 1) + l];
+                const int      q  = (int) (((j >> 1) ? lo >> 4 : lo & 0xFu) |
+                                          (((p[128 + 32 * h + l] >> (2 * j)) & 3u) << 4)) - 32;
+                const int   sc = (int) (int8_t) p[192 + 8 * h + 2 * j + l / 16];
+                const float wv = dd * (float) sc * (float) q; /* q6_K.c:37-40 */
+                prod[r]        = xm[Q6K_BLOCK_ELEMS * b + 64 * r + lane] * (double) wv;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                /* lane i's product as a scalar operand, i = 0 .. 63 in order: the additions are
+                 * the only dependent chain (every lane runs it; the first lane's copy is used) */
+                const uint2 pw = __builtin_bit_cast(uint2, prod[r]);
+#pragma unroll
+                for (int i = 0; i < 64; ++i) {
+                    uint2 t;
+                    t.x = (uint32_t) __builtin_amdgcn_readlane((int) pw.x, i);
+                    t.y = (uint32_t) __builtin_amdgcn_readlane((int) pw.y, i);
+                    acc += __builtin_bit_cast(double, t);
                 }
+            }
         }
-        y[mine.y * ld_y + mine.x] = (float) acc;
+        if (lane == 0 && it0 + wave < count)
+            y[mine.y * ld_y + mine.x] = (float) acc;
     }
 }
 
@@ -255,9 +273,13 @@ void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int
                                                     n_m, y, ld_y, ws.amb_count, ws.amb_list);
         break;
     }
-    /* the list is short (a few outputs in ten thousand): a handful of wavefronts */
-    k_q6k_linear_listed<<<dim3(64), dim3(64), 0, stream>>>(w_q6k, n_in, ws.xd, y, ld_y,
-                                                           ws.amb_count, ws.amb_list);
+    /* the list is short (a few outputs in ten thousand) but its length is only known on the
+     * device: a workgroup per four listed outputs for up to one output in 256, most of which
+     * return at once; longer lists (rows that cancel) go round the loop */
+    const long     want_wgs   = ((long) n_out * n_m / 256 + Q6K_LISTED_WAVES - 1) / Q6K_LISTED_WAVES + 1;
+    const unsigned listed_wgs = (unsigned) (want_wgs < 2048 ? want_wgs : 2048);
+    k_q6k_linear_listed<<<dim3(listed_wgs), dim3(64 * Q6K_LISTED_WAVES), 0, stream>>>(
+        w_q6k, n_in, ws.xd, y, ld_y, ws.amb_count, ws.amb_list);
 }
 
 } // namespace gs
