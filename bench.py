@@ -159,23 +159,27 @@ def bench_spec(w, args):
     x = w.extra
     n_seq, L = x["n_seq"], x["draft_len"]
     dev = torch.device("cuda:0")
-    t = torch.from_numpy(x["target"]).to(dev)
-    q = torch.from_numpy(x["q"]).to(dev)
+    # three copies of the inputs (840 MB against the 256 MB Infinity Cache): every step reads its
+    # target rows and draft probabilities from HBM
+    n_copies = 3
+    ts = [torch.from_numpy(x["target"]).to(dev) for _ in range(n_copies)]
+    qs = [torch.from_numpy(x["q"]).to(dev) for _ in range(n_copies)]
     d = torch.from_numpy(x["draft"]).to(dev)
     u = torch.from_numpy(x["uniforms"]).to(dev)
     out = torch.full((n_seq, L + 1), -1, dtype=torch.int32, device=dev)
     nacc = torch.full((n_seq,), -1, dtype=torch.int32, device=dev)
     hs = HipSampler(max_rows=n_seq * (L + 1), max_vocab=w.n_vocab)
+    hs.set_logits_hint(1)   # the rows come from HBM and are read once
 
-    def step():
-        hs.spec_verify(t, q, d, u, w.temperature, out, nacc)
+    def step(i):
+        hs.spec_verify(ts[i % n_copies], qs[i % n_copies], d, u, w.temperature, out, nacc)
 
-    for _ in range(args.warmup):
-        step()
+    for i in range(max(args.warmup, n_copies)):
+        step(i)
     hs.sync()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        step(i)
     hs.sync()
     elapsed = time.perf_counter() - t0
     ms = elapsed * 1e3 / args.steps
@@ -195,10 +199,47 @@ def bench_spec(w, args):
         "sequences_per_s": round(n_seq * args.steps / elapsed, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "whole step (five kernels)", "step_algorithmic_bytes": alg},
+                     "kernel": "whole step (four kernels)", "step_algorithmic_bytes": alg},
+        "input_copies_rotated": n_copies,
         "accepted_lengths": sorted(nacc.cpu().numpy().tolist()),
     }
+    if not args.no_cpu:
+        result["cpu_baseline"], want = spec_cpu_baseline(w)
+        got_n, got_out = nacc.cpu().numpy(), out.cpu().numpy()
+        differ = sum(int(got_n[s_] != n_) or got_out[s_, :n_ + 1].tolist() != o_[:n_ + 1].tolist()
+                     for s_, (n_, o_) in enumerate(want))
+        result["parity"] = {"sequences": n_seq, "verdicts_differ": int(differ)}
     print(json.dumps(result))
+
+
+def spec_cpu_baseline(w, budget_s=15.0):
+    """The oracle's speculative verification (built with the reference's release flags) on this
+    host: every sequence of the batch, one sequence per thread; repeated to fill the budget."""
+    from concurrent.futures import ThreadPoolExecutor
+    from oracle_lib import Oracle
+    x = w.extra
+    n_seq = x["n_seq"]
+    o = Oracle(fast=True)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 10 ** 6)
+
+    def one(s):
+        return o.spec_verify(x["target"][s], x["q"][s], x["draft"][s], x["uniforms"][s],
+                             w.temperature)
+
+    with ThreadPoolExecutor(cores) as pool:
+        list(pool.map(one, range(min(cores, n_seq))))        # warm-up
+        reps, t_used, res = 0, 0.0, None
+        while reps < 10 and t_used < budget_s:
+            t0 = time.perf_counter()
+            res = list(pool.map(one, range(n_seq)))
+            t_used += time.perf_counter() - t0
+            reps += 1
+    rows = n_seq * (x["draft_len"] + 1)
+    return {"value": round(rows * reps / t_used, 2), "unit": "rows/s", "cores": cores,
+            "kind": "port",
+            "sample": f"the whole batch of {n_seq} sequences x {reps} repeats on {cores} threads "
+                      "(one sequence per thread); oracle built with -O3 -ffast-math "
+                      "-march=x86-64-v3"}, res
 
 
 def bench_lm_head(args, m_rows, q8=False):
@@ -424,9 +465,17 @@ def bench_lm_head_q6k(args, m_rows):
     hs = HipSampler(max_rows=max(m_rows, 1), max_vocab=vocab)
     prm = SampleParams.make(temperature=0.7, top_k=40, top_p=0.9, softcap=30.0)
 
+    # the copies of the tables in the order the device reads them (geist_hip_q6k_pack, once per
+    # model at load); the tables themselves are not read again
+    packed = [torch.empty((hs.q6k_packed_bytes(vocab, d_model),), dtype=torch.uint8, device=dev)
+              for _ in tables]
+    for t, pk in zip(tables, packed):
+        hs.q6k_pack(t, d_model, pk)
+    hs.sync()
+
     def step(i=0):
-        hs.project_sample_q6k(hidden, norm_w, 1e-6, tables[i % 3], logits, prm, d_u, out,
-                              normed=normed)
+        hs.project_sample_q6k_packed(hidden, norm_w, 1e-6, packed[i % 3], vocab, logits, prm, d_u,
+                                     out, normed=normed)
 
     for i in range(args.warmup):
         step(i)
@@ -440,11 +489,15 @@ def bench_lm_head_q6k(args, m_rows):
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
     for i in range(3):
-        hs.q6k_linear(tables[i], d_model, normed, logits)
+        hs.q6k_packed_linear(packed[i], vocab, d_model, normed, logits)
     with Timer() as tm:       # HIP events on the sampler's stream around the launches
         for i in range(args.steps):
-            hs.q6k_linear(tables[i % 3], d_model, normed, logits)
+            hs.q6k_packed_linear(packed[i % 3], vocab, d_model, normed, logits)
     kernel_us = tm.ms * 1e3 / args.steps
+    with Timer() as tm:       # the table as it lies in the file, for comparison
+        for i in range(args.steps):
+            hs.q6k_linear(tables[i % 3], d_model, normed, logits)
+    unpacked_us = tm.ms * 1e3 / args.steps
     w_bytes = vocab * nb * 210
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -459,8 +512,10 @@ def bench_lm_head_q6k(args, m_rows):
         "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_q6k_linear (+ activations to double, listed outputs)",
-                     "kernel_us": round(kernel_us, 3), "kernel_algorithmic_bytes": w_bytes,
+                     "kernel": "k_q6k_packed_linear (+ activations to double)",
+                     "kernel_us": round(kernel_us, 3),
+                     "kernel_us_table_as_in_file": round(unpacked_us, 3),
+                     "kernel_algorithmic_bytes": w_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
     if not args.no_cpu:
@@ -473,7 +528,7 @@ def bench_lm_head_q6k(args, m_rows):
         t0 = time.perf_counter()
         want = oracle_q6k_linear(lib, w_s, x_s, d_model)
         dt = time.perf_counter() - t0
-        hs.q6k_linear(tables[0], d_model, normed, logits)
+        hs.q6k_packed_linear(packed[0], vocab, d_model, normed, logits)
         hs.sync()
         got = logits[:, :n_s].cpu().numpy()
         result["cpu_baseline"] = {

@@ -104,6 +104,13 @@ def load_library():
     lib.geist_hip_f16_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q6k_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q6k_linear_reserve.argtypes = [vp, sz, sz]
+    lib.geist_hip_q6k_packed_bytes.argtypes = [sz, sz]
+    lib.geist_hip_q6k_packed_bytes.restype = sz
+    lib.geist_hip_q6k_pack.argtypes = [vp, vp, sz, sz, vp]
+    lib.geist_hip_q6k_packed_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_project_sample_rows_q6k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
+                                                             vp, vp, sz, C.POINTER(SampleParams),
+                                                             vp, vp, i32, vp]
     lib.geist_hip_f16_to_q8w.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
@@ -294,6 +301,21 @@ class HipSampler:
             self.h, _ptr(w_q6k), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 
+    def q6k_packed_bytes(self, n_out, n_in):
+        return int(self.lib.geist_hip_q6k_packed_bytes(n_out, n_in))
+
+    def q6k_pack(self, w_q6k, n_in, packed):
+        """packed: uint8 tensor of q6k_packed_bytes(n_out, n_in) bytes, 16-byte aligned."""
+        n_out = w_q6k.shape[0]
+        assert packed.numel() * packed.element_size() >= self.q6k_packed_bytes(n_out, n_in)
+        self._check(self.lib.geist_hip_q6k_pack(self.h, _ptr(w_q6k), n_out, n_in, _ptr(packed)))
+
+    def q6k_packed_linear(self, packed, n_out, n_in, x, y):
+        m = x.shape[0]
+        self._check(self.lib.geist_hip_q6k_packed_linear_rows(
+            self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
     def f16_to_q8w(self, w_f16, wq, scales):
         """w_f16 [n_out, n_in] float16 -> wq int8 [n_out, n_in], scales float32 [n_out]."""
         n_out, n_in = w_f16.shape
@@ -340,6 +362,16 @@ class HipSampler:
         self._check(self.lib.geist_hip_project_sample_rows_q6k(
             self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
             _ptr(norm_w), eps, _ptr(embed_q6k), vocab, _ptr(normed), _ptr(logits),
+            logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
+            _ptr(rng_states), int(shared), _ptr(out)))
+
+    def project_sample_q6k_packed(self, hidden, norm_w, eps, packed, vocab, logits, params,
+                                  uniforms, out, normed=None, rng_states=None, shared=True):
+        """project_sample over the packed copy of a Q6_K table (q6k_pack)."""
+        rows, d_model = hidden.shape
+        self._check(self.lib.geist_hip_project_sample_rows_q6k_packed(
+            self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
+            _ptr(norm_w), eps, _ptr(packed), vocab, _ptr(normed), _ptr(logits),
             logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
             _ptr(rng_states), int(shared), _ptr(out)))
 

@@ -734,84 +734,46 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
     }
 }
 
-/* The listed outputs once more, in the reference's order: a lane per output (weight row r,
- * activation row m), a wavefront streams its 64 weight rows through its LDS tile as above and
- * every lane adds its row's products one after the other. The activations of a stage lie in LDS
- * for all activation rows; a lane reads those of its own. */
+/* The listed outputs once more, the products added one after the other in index order as the
+ * reference adds them. A wavefront per output (weight row r, activation row m): its lanes form
+ * 64 products at a time -- each exact in double -- and the sum takes them in order, lane by
+ * lane, as scalar operands. The chain of n_in dependent additions is what this kernel takes;
+ * there are few listed outputs and each has a wavefront to itself. */
 __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
-    const uint16_t *__restrict__ w, int n_in, const double *__restrict__ xd, int n_m,
-    float *__restrict__ y, long ld_y, const int *__restrict__ amb_count,
-    const int2 *__restrict__ amb_list) {
-    __shared__ __align__(16) uint8_t s_tile[LM_WAVES][ROWS_WAVE_B * TILE_PITCH];
-    /* (rows two doubles apart in the banks: lanes of different activation rows read the same
-     * column without conflict) */
-    __shared__ double                s_x[LM_WAVES][F64_M_MAX][STAGE_COLS + 2];
+    const uint16_t *__restrict__ w, int n_in, const double *__restrict__ xd, float *__restrict__ y,
+    long ld_y, const int *__restrict__ amb_count, const int2 *__restrict__ amb_list) {
     const int lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
     const int count = *amb_count;
-    uint8_t  *tile  = s_tile[wave];
-    const int n_stage = (n_in + STAGE_COLS - 1) / STAGE_COLS;
-    for (int it0 = ((int) blockIdx.x * LM_WAVES + wave) * LM_WAVE; it0 < count;
-         it0 += (int) gridDim.x * LM_WAVES * LM_WAVE) { /* (uniform over the wavefront) */
-        const int2 mine = amb_list[it0 + lane < count ? it0 + lane : count - 1];
-        /* the rows whose segment (lane & 7) this lane fetches: items 8 i + (lane >> 3) */
-        long fetch_row[STAGE_LOADS_B];
+    for (int it = (int) blockIdx.x * LM_WAVES + wave; it < count;
+         it += (int) gridDim.x * LM_WAVES) { /* (uniform over the wavefront) */
+        const int2      mine = amb_list[it];
+        const uint16_t *wr   = w + (long) mine.x * n_in;
+        const double   *xm   = xd + (long) mine.y * n_in;
+        double          acc  = 0.0;
+        for (int k0 = 0; k0 < n_in; k0 += 4 * LM_WAVE) {
+            /* four rounds of 64 products, their loads in flight together; a short last round
+             * adds zeros, which change nothing (the sum never is -0 after a +0 start) */
+            double prod[4];
 #pragma unroll
-        for (int i = 0; i < STAGE_LOADS_B; ++i) {
-            const int it  = it0 + 8 * i + (lane >> 3);
-            fetch_row[i] = (long) amb_list[it < count ? it : count - 1].x;
-        }
-        /* weights two stages ahead in registers, activations one stage ahead */
-        auto fetch_w = [&](int s, StageRegsB &g) {
-            const int col = s * STAGE_COLS + (lane & 7) * 8;
-#pragma unroll
-            for (int i = 0; i < STAGE_LOADS_B; ++i) {
-                g.w[i] = make_uint4(0u, 0u, 0u, 0u);
-                if (col < n_in)
-                    g.w[i] = *reinterpret_cast<const uint4 *>(w + fetch_row[i] * n_in + col);
+            for (int r = 0; r < 4; ++r) {
+                const int k = k0 + r * LM_WAVE + lane;
+                prod[r]     = k < n_in ? xm[k] * (double) __half2float(__ushort_as_half(wr[k])) : 0.0;
             }
-        };
-        auto fetch_x = [&](int s, double (&xr)[F64_M_MAX]) {
-            const int k = s * STAGE_COLS + lane;
 #pragma unroll
-            for (int m = 0; m < F64_M_MAX; ++m)
-                xr[m] = (m < n_m && k < n_in) ? xd[(long) m * n_in + k] : 0.0;
-        };
-        StageRegsB g0, g1;
-        double     x0[F64_M_MAX];
-        fetch_w(0, g0);
-        fetch_x(0, x0);
-        if (n_stage > 1)
-            fetch_w(1, g1);
-        double acc = 0.0;
-        for (int s = 0; s < n_stage; ++s) {
-            const int col0 = s * STAGE_COLS;
+            for (int r = 0; r < 4; ++r) {
+                if (k0 + r * LM_WAVE >= n_in)
+                    break;
+                const uint2 pw = __builtin_bit_cast(uint2, prod[r]);
 #pragma unroll
-            for (int i = 0; i < STAGE_LOADS_B; ++i)
-                *reinterpret_cast<uint4 *>(tile + (8 * i + (lane >> 3)) * TILE_PITCH +
-                                           (lane & 7) * 16) = g0.w[i];
-#pragma unroll
-            for (int m = 0; m < F64_M_MAX; ++m)
-                s_x[wave][m][lane] = x0[m];
-            g0 = g1;
-            if (s + 2 < n_stage)
-                fetch_w(s + 2, g1);
-            if (s + 1 < n_stage)
-                fetch_x(s + 1, x0);
-            const uint8_t *row_tile = tile + lane * TILE_PITCH;
-            const double  *xm       = s_x[wave][mine.y];
-            const int      steps    = (n_in - col0 >= STAGE_COLS ? STAGE_COLS : n_in - col0) / 8;
-            for (int t = 0; t < steps; ++t) {
-                const uint4    q    = *reinterpret_cast<const uint4 *>(row_tile + t * 16);
-                const uint32_t u[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&u[i]));
-                    acc = __builtin_fma(xm[t * 8 + 2 * i], (double) f.x, acc);
-                    acc = __builtin_fma(xm[t * 8 + 2 * i + 1], (double) f.y, acc);
+                for (int i = 0; i < LM_WAVE; ++i) {
+                    uint2 t;
+                    t.x = (uint32_t) __builtin_amdgcn_readlane((int) pw.x, i);
+                    t.y = (uint32_t) __builtin_amdgcn_readlane((int) pw.y, i);
+                    acc += __builtin_bit_cast(double, t);
                 }
             }
         }
-        if (it0 + lane < count)
+        if (lane == 0)
             y[mine.y * ld_y + mine.x] = (float) acc;
     }
 }
@@ -881,9 +843,12 @@ void launch_f16_linear_f64(hipStream_t stream, const uint16_t *w_f16, long n_out
         k_f16_linear_f64_mfma<3><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
     else /* 13 .. F64_M_MAX rows: one 16 x 16 tile of activation rows */
         k_f16_linear_f64_mfma<0><<<grid_b, block, 0, stream>>>(w_f16, n_out, n_in, ws.xd, ws.xs, n_m, y, ld_y, ws.amb_count, ws.amb_list);
-    /* normally a few dozen outputs: one wavefront's worth; the grid strides over longer lists */
-    k_f16_linear_f64_listed<<<dim3(64), block, 0, stream>>>(w_f16, n_in, ws.xd, n_m, y, ld_y,
-                                                           ws.amb_count, ws.amb_list);
+    /* normally a few dozen outputs, whose number is only known on the device: a wavefront for
+     * up to one output in 256, most of which return at once; longer lists go round the loop */
+    const long     want_wgs   = (n_out * n_m / 256 + LM_WAVES - 1) / LM_WAVES + 1;
+    const unsigned listed_wgs = (unsigned) (want_wgs < 2048 ? want_wgs : 2048);
+    k_f16_linear_f64_listed<<<dim3(listed_wgs), block, 0, stream>>>(w_f16, n_in, ws.xd, y, ld_y,
+                                                                   ws.amb_count, ws.amb_list);
 }
 
 /* f16_to_q8w (kernel_f16_gemv.c:66-93): per row scale = max|w| / 127, q = lrintf(w * (127 /

@@ -67,6 +67,15 @@ void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int
                        const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
                        long ld_y);
 
+/* The Q6_K table in the order the device reads it (lm_head_q6k.hip): bytes of the packed copy,
+ * the packing kernel (once per model), and the projection over the packed copy, which adds in
+ * the reference's order and needs no second kernel. */
+size_t q6k_packed_bytes(long n_out, int n_in);
+void launch_q6k_pack(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in, void *packed);
+void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
+                              const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                              long ld_y);
+
 /* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *
  * scales[r]; n_in a multiple of 16. */
 void launch_q8w_gemv(hipStream_t stream, const int8_t *wq, const float *scales, long n_out,

@@ -253,6 +253,146 @@ __global__ __launch_bounds__(64 * Q6K_LISTED_WAVES) void k_q6k_linear_listed(
     }
 }
 
+/* ---- the table repacked for the device --------------------------------------------------------
+ * The GGUF layout puts a row's blocks one after the other, 210 bytes each: lanes that own
+ * neighbouring rows read addresses a row apart, and a block shares its first and last cache line
+ * with its neighbours. geist_hip_q6k_pack (once per model, at load) writes the same bytes in the
+ * order the kernel reads them: the table rows in groups of 64 (a wavefront), per group the blocks
+ * in order, per block the 53 dwords of each of the 64 rows with the rows innermost --
+ *   dwords 4 p .. 4 p + 3 of row r (p < 13) at  base + p * 256 + 4 r,   dword 52 at base + 3328 + r
+ * (in dwords; base = (group * blocks + b) * 3392) -- so that a wavefront's 16-byte loads read one
+ * kilobyte of consecutive addresses and every byte of the table is read once. Rows beyond n_out
+ * in the last group are zero blocks.
+ *
+ * With the loads out of the way the kernel can afford the reference's own order of additions:
+ * a lane owns a table row and adds its products one after the other in index order,
+ *   acc = fma(x[k], w[k], acc),  w = fma(ds, q_unsigned, -32 ds)   (both exact, see the header)
+ * which is cpu_scalar_w_quant_m1's sum bit for bit, with nothing to bound and nothing to repeat.
+ * The chain of dependent additions is hidden by the conversions of the following elements and
+ * by the other wavefronts of the SIMD. */
+constexpr int Q6K_PACK_DWORDS = 53 * 64; /* per (group of 64 rows, block) */
+
+__global__ __launch_bounds__(Q6K_TPB) void k_q6k_pack(const uint8_t *__restrict__ w, long n_out,
+                                                      int nb, uint32_t *__restrict__ packed) {
+    const long item = (long) blockIdx.x * (Q6K_TPB / 64) + threadIdx.x / 64; /* (group, block) */
+    const int  r    = threadIdx.x & 63;
+    const long n_groups = (n_out + 63) / 64;
+    if (item >= n_groups * nb)
+        return;
+    const long g = item / nb, row = g * 64 + r;
+    const int  b = (int) (item - g * nb);
+    uint32_t   d[53];
+    if (row < n_out) {
+        q6k_load_block(w + (row * nb + b) * (long) Q6K_BLOCK_BYTES, d);
+        d[52] &= 0xffffu;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 53; ++i)
+            d[i] = 0u;
+    }
+    uint32_t *base = packed + item * Q6K_PACK_DWORDS;
+#pragma unroll
+    for (int p = 0; p < 13; ++p)
+        *reinterpret_cast<uint4 *>(base + p * 256 + 4 * r) =
+            make_uint4(d[4 * p], d[4 * p + 1], d[4 * p + 2], d[4 * p + 3]);
+    base[3328 + r] = d[52];
+}
+
+template <int MT>
+__global__ __launch_bounds__(Q6K_TPB) void k_q6k_packed_linear(const uint32_t *__restrict__ packed,
+                                                               long n_out, int n_in,
+                                                               const double *__restrict__ xd,
+                                                               int n_m, float *__restrict__ y,
+                                                               long ld_y) {
+    const int  r = threadIdx.x & 63;
+    const long g = (long) blockIdx.x * (Q6K_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long row = g * 64 + r;
+    const int  nb  = n_in / Q6K_BLOCK_ELEMS;
+    double     acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m] = 0.0;
+    for (int b = 0; b < nb; ++b) {
+        const uint32_t *base = packed + (g * nb + b) * Q6K_PACK_DWORDS;
+        uint32_t        d[53];
+#pragma unroll
+        for (int p = 0; p < 13; ++p) {
+            typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+            const nt_u4 q = __builtin_nontemporal_load(
+                reinterpret_cast<const nt_u4 *>(base + p * 256 + 4 * r));
+            d[4 * p] = q.x, d[4 * p + 1] = q.y, d[4 * p + 2] = q.z, d[4 * p + 3] = q.w;
+        }
+        d[52] = __builtin_nontemporal_load(base + 3328 + r);
+        const float dd = __half2float(__ushort_as_half((unsigned short) (d[52] & 0xffffu)));
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int l4 = 0; l4 < 8; ++l4) {
+                    const int      si  = 8 * h + 2 * j + l4 / 4;
+                    const int      sc  = (int) (int8_t) (d[48 + si / 4] >> (8 * (si % 4)));
+                    const double   ds  = (double) (dd * (float) sc), m32ds = -32.0 * ds;
+                    const uint32_t qlw = d[16 * h + 8 * (j & 1) + l4];
+                    const uint32_t qhw = d[32 + 8 * h + l4];
+                    const uint32_t lo4 = ((j >> 1) ? qlw >> 4 : qlw) & 0x0F0F0F0Fu;
+                    const uint32_t hi4 = (j == 0   ? qhw << 4
+                                          : j == 1 ? qhw << 2
+                                          : j == 2 ? qhw
+                                                   : qhw >> 2) &
+                                         0x30303030u;
+                    const uint32_t qu = lo4 | hi4; /* four unsigned 6-bit values, a byte each */
+                    const int      k0 = Q6K_BLOCK_ELEMS * b + 128 * h + 32 * j + 4 * l4;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const double wv = __builtin_fma(ds, (double) q6k_ubyte(qu, i), m32ds);
+#pragma unroll
+                        for (int m = 0; m < MT; ++m) {
+                            const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in;
+                            acc[m] = __builtin_fma(xm[k0 + i], wv, acc[m]); /* uniform address */
+                        }
+                    }
+                }
+            }
+        }
+    }
+    if (row < n_out) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m < n_m)
+                y[m * ld_y + row] = (float) acc[m];
+    }
+}
+
+size_t q6k_packed_bytes(long n_out, int n_in) {
+    return (size_t) ((n_out + 63) / 64) * (size_t) (n_in / Q6K_BLOCK_ELEMS) * Q6K_PACK_DWORDS * 4;
+}
+
+void launch_q6k_pack(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
+                     void *packed) {
+    const int  nb    = n_in / Q6K_BLOCK_ELEMS;
+    const long items = (n_out + 63) / 64 * nb;
+    k_q6k_pack<<<dim3((unsigned) ((items + 3) / 4)), dim3(Q6K_TPB), 0, stream>>>(
+        w_q6k, n_out, nb, static_cast<uint32_t *>(packed));
+}
+
+void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
+                              const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                              long ld_y) {
+    k_q6k_x_prep<<<dim3(n_m), dim3(Q6K_TPB), 0, stream>>>(x, ld_x, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                         ws.amb_count);
+    const long     groups = (n_out + 63) / 64;
+    const dim3     grid((unsigned) ((groups + 3) / 4)), block(Q6K_TPB);
+    const uint32_t *p = static_cast<const uint32_t *>(packed);
+    switch (n_m) {
+    case 1: k_q6k_packed_linear<1><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    case 2: k_q6k_packed_linear<2><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    default: k_q6k_packed_linear<4><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    }
+}
+
 void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
                        const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
                        long ld_y) {

@@ -26,6 +26,9 @@ struct geist_hip_head {
     int32_t  *d_drafts; /* m_max */
     int32_t  *d_nacc;
     int32_t  *d_ngram;  /* seed, history length, count, matched length, 16 drafts */
+    void       *d_q6k_packed; /* the Q6_K table of geist_hip_head_q6k_load, repacked */
+    const void *q6k_source;   /* ... the table it was packed from, and its row length */
+    size_t      q6k_d_model;
     float    *d_normed; /* m_max x d_model_cap: the normed hidden rows */
     size_t    d_model_cap;
     float    *d_logits; /* m_max x vocab, written by the lm_head, read by the sampler */
@@ -104,6 +107,7 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         geist_hip_free(h->hs, h->d_nacc);
         geist_hip_free(h->hs, h->d_ngram);
         geist_hip_free(h->hs, h->d_normed);
+        geist_hip_free(h->hs, h->d_q6k_packed);
         geist_hip_free(h->hs, h->d_logits);
         geist_hip_free(h->hs, h->d_spec_result);
         geist_hip_spec_head_destroy(h->hs, h->spec);
@@ -242,11 +246,18 @@ static int project_finalize_table(struct geist_hip_head *h, const float *d_hidde
         return rrc;
     /* head.c:99-101, 114-126, then the dispatch of 172-183 / 291-302 with the session's RNG */
     const struct geist_hip_sample_params prm = head_params(h);
+    /* the table that geist_hip_head_q6k_load repacked is read from its packed copy */
+    const bool packed = q6k && h->d_q6k_packed != nullptr && d_embed == h->q6k_source &&
+                        d_model == h->q6k_d_model;
     const int rc =
-            q6k ? geist_hip_project_sample_rows_q6k(h->hs, d_hidden, ld_hidden, k, d_model,
-                                                    d_norm_weight, rms_eps, d_embed, h->vocab,
-                                                    h->d_normed, h->d_logits, h->vocab, &prm,
-                                                    nullptr, h->d_rng, /*shared=*/1, h->d_tokens)
+            packed ? geist_hip_project_sample_rows_q6k_packed(
+                             h->hs, d_hidden, ld_hidden, k, d_model, d_norm_weight, rms_eps,
+                             h->d_q6k_packed, h->vocab, h->d_normed, h->d_logits, h->vocab, &prm,
+                             nullptr, h->d_rng, /*shared=*/1, h->d_tokens)
+            : q6k ? geist_hip_project_sample_rows_q6k(h->hs, d_hidden, ld_hidden, k, d_model,
+                                                      d_norm_weight, rms_eps, d_embed, h->vocab,
+                                                      h->d_normed, h->d_logits, h->vocab, &prm,
+                                                      nullptr, h->d_rng, /*shared=*/1, h->d_tokens)
             : d_scales != nullptr
                     ? geist_hip_project_sample_rows_q8w(h->hs, d_hidden, ld_hidden, k, d_model,
                                                         d_norm_weight, rms_eps, d_embed, d_scales,
@@ -274,6 +285,29 @@ int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d
                                         int32_t *out_tokens) {
     return project_finalize_table(h, d_hidden, ld_hidden, k, d_norm_weight, rms_eps, d_embed_q6k,
                                   nullptr, true, d_model, out_tokens);
+}
+
+int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, size_t d_model) {
+    if (h == nullptr || d_embed_q6k == nullptr || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    const size_t bytes = geist_hip_q6k_packed_bytes(h->vocab, d_model);
+    if (bytes == 0)
+        return head_fail(h, GEIST_HIP_E_UNSUPPORTED, "Q6_K table: d_model not a multiple of 256");
+    geist_hip_free(h->hs, h->d_q6k_packed);
+    h->d_q6k_packed = nullptr;
+    h->q6k_source   = nullptr;
+    void *p         = nullptr;
+    if (geist_hip_malloc(h->hs, bytes, &p) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_OOM, "packed Q6_K table");
+    if (geist_hip_q6k_pack(h->hs, d_embed_q6k, h->vocab, d_model, p) != GEIST_HIP_OK ||
+        geist_hip_sampler_sync(h->hs) != GEIST_HIP_OK) {
+        geist_hip_free(h->hs, p);
+        return head_fail(h, GEIST_HIP_E_BACKEND, "packing the Q6_K table");
+    }
+    h->d_q6k_packed = p;
+    h->q6k_source   = d_embed_q6k;
+    h->q6k_d_model  = d_model;
+    return geist_hip_head_reserve_projection_q6k(h, d_model);
 }
 
 int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model) {

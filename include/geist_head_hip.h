@@ -115,12 +115,18 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
  * no device kernel here: their callers project on the host or with their own kernel and pass
  * the logits to geist_hip_head_finalize_one_row / _batch.
  * geist_hip_head_reserve_projection_q6k is geist_hip_head_reserve_projection plus the scratch of
- * this kernel. */
+ * this kernel. geist_hip_head_q6k_load, once per model: keeps a copy of the table in the order
+ * the device reads it (geist_hip_q6k_pack; 1 % more device memory than the table itself, the
+ * x86 backend's counterpart being its binary32 predecode at load) and reserves the buffers;
+ * geist_hip_head_project_finalize_q6k with that same table pointer and d_model then streams the
+ * copy, 1.5 times as fast, with the same logits bit for bit. The table itself is not kept
+ * alive by the head and may be changed or freed only together with a new load. */
 int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d_hidden,
                                         size_t ld_hidden, size_t k, const float *d_norm_weight,
                                         float rms_eps, const void *d_embed_q6k, size_t d_model,
                                         int32_t *out_tokens);
 int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model);
+int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, size_t d_model);
 /* The speculative output head of greedy decoding (src/archs/transformer/forward/spec_head.c;
  * include/geist_lm_head_hip.h has the device entry points). geist_hip_head_spec_build is
  * transformer_spec_head_init (spec_head.c:616-622) for a tied F16 table in device memory, which

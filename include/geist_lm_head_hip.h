@@ -134,6 +134,21 @@ int geist_hip_q6k_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in
 int geist_hip_q6k_linear_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
                               const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
                               size_t ld_y);
+/* No counterpart in the reference (its x86 backend likewise re-lays the table at load, into
+ * binary32: cpu_x86_linear_q6k_resolve). The same bytes in the order the device reads them, so
+ * that the projection streams the table at the rate of the memory: the rows in groups of 64, per
+ * group the blocks in order, per block the 53 dwords of the 64 rows with the rows innermost
+ * (geistlib_amd/csrc/lm_head_q6k.hip has the exact layout). geist_hip_q6k_packed_bytes: size of
+ * the packed copy (1 % above the table's; 0 for a shape the format does not allow).
+ * geist_hip_q6k_pack: once per model, d_packed 16-byte aligned. geist_hip_q6k_packed_linear_rows:
+ * geist_hip_q6k_linear_rows over the packed copy, same results bit for bit; it adds every row's
+ * products in index order itself, so nothing is repeated. */
+size_t geist_hip_q6k_packed_bytes(size_t n_out, size_t n_in);
+int geist_hip_q6k_pack(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
+                       void *d_packed);
+int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                     size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                     float *d_y, size_t ld_y);
 /* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, geist_hip_q6k_linear_rows
  * and the sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. */
 int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
@@ -144,6 +159,15 @@ int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidde
                                       const struct geist_hip_sample_params *params,
                                       const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                       geist_hip_token_t *d_out_tokens);
+
+int geist_hip_project_sample_rows_q6k_packed(geist_hip_sampler *s, const float *d_hidden,
+                                             size_t ld_hidden, size_t rows, size_t d_model,
+                                             const float *d_norm_weight, float rms_eps,
+                                             const void *d_embed_packed, size_t n_vocab,
+                                             float *d_normed, float *d_logits, size_t ld_logits,
+                                             const struct geist_hip_sample_params *params,
+                                             const float *d_uniforms, uint64_t *d_rng_states,
+                                             int shared, geist_hip_token_t *d_out_tokens);
 
 /* The reference's speculative output head for greedy decoding
  * (src/archs/transformer/forward/spec_head.c), over a tied F16 table in device memory: an int8

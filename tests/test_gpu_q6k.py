@@ -40,6 +40,16 @@ def test_q6k_linear_equals_the_portable_kernel(hs, oracle, n_out, n_in, m):
         got = y.cpu().numpy()
         bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, (scale, bad[:5], got[tuple(bad[0])], want[tuple(bad[0])])
+        # the same over the table repacked for the device
+        packed = torch.full((hs.q6k_packed_bytes(n_out, n_in),), 0xA5, dtype=torch.uint8,
+                            device="cuda")
+        hs.q6k_pack(d_w, n_in, packed)
+        y2 = torch.full((m, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q6k_packed_linear(packed, n_out, n_in, d_x, y2)
+        hs.sync()
+        got = y2.cpu().numpy()
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, ("packed", scale, bad[:5], got[tuple(bad[0])], want[tuple(bad[0])])
 
 
 def test_q6k_linear_rows_whose_sums_cancel(hs, oracle):
@@ -54,7 +64,14 @@ def test_q6k_linear_rows_whose_sums_cancel(hs, oracle):
         x[:, 1::2] = -x[:, 0::2] * np.float32(1 + 2.0 ** -(8 + 4 * trial))
         want = oracle_q6k_linear(oracle.lib, w, x, n_in)
         y = torch.empty((2, n_out), dtype=torch.float32, device="cuda")
-        hs.q6k_linear(torch.from_numpy(w).cuda(), n_in, torch.from_numpy(x).cuda(), y)
+        d_w, d_x = torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda()
+        hs.q6k_linear(d_w, n_in, d_x, y)
+        hs.sync()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32)), trial
+        packed = torch.empty((hs.q6k_packed_bytes(n_out, n_in),), dtype=torch.uint8, device="cuda")
+        hs.q6k_pack(d_w, n_in, packed)
+        y.fill_(0)
+        hs.q6k_packed_linear(packed, n_out, n_in, d_x, y)
         hs.sync()
         assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32)), trial
 
@@ -84,6 +101,7 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
                                                          C.c_void_p, C.c_size_t,
                                                          C.POINTER(C.c_int32)]
     host.geist_hip_head_reserve_projection_q6k.argtypes = [C.c_void_p, C.c_size_t]
+    host.geist_hip_head_q6k_load.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
     g = np.random.default_rng(2026)
     vocab, d_model, cap = 262144, 1536, 30.0
     w = random_q6k_table(g, vocab, d_model, scale_mode="plain")
@@ -94,7 +112,11 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
         h = make_head(host, vocab, 4, cap)
         opts = SessionOpts(0, T, p, top_k, 31337, None, 0, 4)
         assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
-        assert host.geist_hip_head_reserve_projection_q6k(h, d_model) == 0
+        if top_k == 0:      # one configuration reads the table as it lies, the others packed
+            assert host.geist_hip_head_reserve_projection_q6k(h, d_model) == 0
+        else:
+            assert host.geist_hip_head_q6k_load(h, C.c_void_p(d_w.data_ptr()), d_model) == 0, \
+                host.geist_hip_head_errmsg(h)
         sess = oracle.session(T, p, top_k, seed=31337)
         for k in (1, 1, 3):
             hidden = (g.standard_normal((k, d_model)) * 4).astype(np.float32)
