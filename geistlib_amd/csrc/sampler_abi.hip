@@ -570,14 +570,19 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
             f.k_sel          = rs.k + margin < TOPK_FAST_MAX ? rs.k + margin : TOPK_FAST_MAX;
         }
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
+        /* The soft-cap keeps the order of the logits, so the scan runs on the logits as they are
+         * and the row-final kernel caps what it keeps (with the thread maxima already there from
+         * a projection's epilogue they are uncapped as well). */
+        f.cap_after = L.rv.softcap > 0.0f;
+        if (f.cap_after)
+            scan.rv.softcap = 0.0f;
         f.mode = FINAL_TOPK;
         f.k    = rs.k;
-        /* Plain rows (aligned, no soft-cap, no mask, penalties absent or left to the final kernel)
+        /* Plain rows (aligned, no mask, penalties absent or left to the final kernel)
          * take the candidate path: the scan's wavefronts hand their leading groups on and the
          * row-final kernel gathers nothing. */
         const size_t row_waves = rows->rows * (size_t) L.rv.n_chunks * NWAVES_PER_CHUNK;
-        const bool   plain = rs.k <= CAND_K_MAX && L.rv.vec_ok && !(L.rv.softcap > 0.0f) &&
-                           !L.rv.allowed &&
+        const bool   plain = rs.k <= CAND_K_MAX && L.rv.vec_ok && !L.rv.allowed &&
                            L.rv.n_chunks <= CAND_CHUNKS_MAX && (!L.pen || !scan.pen) &&
                            !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves &&
                            (!L.pen || rows->history_ld <= (size_t) HT_HISTORY_MAX);
@@ -1193,10 +1198,9 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     HIPCHK(s, hipSetDevice(s->device));
     const bool f64     = table == TABLE_F16 && (rows > 1 || s->projection_portable);
     const bool fuse_ok = f16_gemv_can_fuse((int) rows) && !f64 && !q6k;
-    /* the top-k path's scan is the projection's epilogue when nothing changes the logits
-     * between the two (no soft-cap) */
-    const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX &&
-                           !(params->logit_softcap > 0.0f);
+    /* the top-k path's scan is the projection's epilogue (its thread maxima are those of the
+     * logits before the soft-cap, which the row-final kernel applies to what it keeps) */
+    const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX;
     if (!d_normed)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "no buffer for the normed rows");
     launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps, (int) rows,

@@ -355,7 +355,7 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
             const unsigned p    = n_e + lanes_before(mk);
             const bool     put  = keep && p < (unsigned) FC_LIST;
             const unsigned at   = put ? p : (unsigned) (FC_LIST + lane);
-            e_val[at]           = PEN ? __float_as_uint(xc) : f2key(xc);
+            e_val[at]           = (PEN || a.cap_after) ? __float_as_uint(xc) : f2key(xc);
             e_idx[at]           = (uint32_t) (gi[r] + c);
             n_e += (unsigned) __popcll(mk);
         }
@@ -382,22 +382,35 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
      * is read from the table; an element that no longer reaches B gets key 0. */
     wave_lds_sync();
     uint32_t my_key = 0u;
+    /* With the soft-cap left to this kernel (FinalArgs::cap_after) an entry counts when its
+     * capped value lies strictly above the capped bound: those are certain to be all there are. */
+    const float Bc = a.cap_after ? softcap1(B, rv.softcap) : B;
     if (!give_up && lane < (int) n_e) {
         my_key = e_val[lane];
-        if (PEN) {
-            const int id = (int) e_idx[lane];
-            float     x  = __uint_as_float(my_key);
-            uint32_t  hq = hist_hash(id);
-            int       kq = hkey[hq];
+        if (PEN || a.cap_after) {
+            float x = __uint_as_float(my_key);
+            if (PEN) {
+                const int id = (int) e_idx[lane];
+                uint32_t  hq = hist_hash(id);
+                int       kq = hkey[hq];
 #pragma unroll 1
-            for (int pr = 0; pr < HT_SLOTS && kq != id && kq != -1; ++pr) {
-                hq = (hq + 1u) & (HT_SLOTS - 1);
-                kq = hkey[hq];
+                for (int pr = 0; pr < HT_SLOTS && kq != id && kq != -1; ++pr) {
+                    hq = (hq + 1u) & (HT_SLOTS - 1);
+                    kq = hkey[hq];
+                }
+                if (kq == id)
+                    x = penalise(x, (hcnt[hq >> 1] >> (16 * (hq & 1u))) & 0xffffu, rv.rep,
+                                 rv.inv_rep, rv.freq, rv.pres);
             }
-            if (kq == id)
-                x = penalise(x, (hcnt[hq >> 1] >> (16 * (hq & 1u))) & 0xffffu, rv.rep, rv.inv_rep,
-                             rv.freq, rv.pres);
-            my_key = x >= B ? f2key(x) : 0u;
+            if (a.cap_after) {
+                my_key = 0u;
+                if (x >= B) {
+                    const float xc = softcap1(x, rv.softcap);
+                    my_key         = xc > Bc ? f2key(xc) : 0u;
+                }
+            } else {
+                my_key = x >= B ? f2key(x) : 0u;
+            }
         }
     }
     {
@@ -412,15 +425,17 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
         s_c.give_up = 1;
     __syncthreads();
     give_up = s_c.give_up != 0;
-    /* The k largest. The keys lie in [lo, mx]; 256 bins over that range, counted by all
+    /* The k largest. The keys lie in [lo_k, mx]; 256 bins over that range, counted by all
      * wavefronts, then every wavefront finds the bin in which the count from above reaches k.
      * The entries from that bin upwards are listed; should they be more than CAND_CUT_MAX the
      * bin is split again. */
     const int n_real = s_c.n_real;
     give_up = give_up || n_real < a.k; /* fewer than k at or above B: B certifies nothing */
-    uint32_t cut = lo; /* entries with key >= cut are listed */
+    /* (keys of capped values lie above the capped bound's, which is below the raw bound's) */
+    const uint32_t lo_k = a.cap_after ? f2key(Bc) : lo;
+    uint32_t cut = lo_k; /* entries with key >= cut are listed */
     if (!give_up && n_real > CAND_CUT_MAX) {
-        uint32_t base_k = lo, top_k = s_c.mx; /* the range being split, inclusive */
+        uint32_t base_k = lo_k, top_k = s_c.mx; /* the range being split, inclusive */
         int      need        = a.k;       /* entries wanted from this range: its `need` largest */
         int      above_total = 0;         /* entries above the range: all of them are wanted */
         int      listed      = n_real;    /* entries at or above the cut */

@@ -122,6 +122,8 @@ struct FinalLaunch {
                                     kernel, no listing pass; a row whose list overflowed goes to
                                     the whole-row walk */
     int             mode, k, k_sel;
+    bool            cap_after; /* top-k: the scan ran before the soft-cap, the row-final kernel
+                                  applies it to what it keeps */
     float           inv_t, top_p, min_p;
     const float    *uniforms;
     const uint64_t *chunk_best;

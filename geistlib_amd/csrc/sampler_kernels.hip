@@ -950,6 +950,14 @@ struct FinalArgs {
     int             zb_min_p; /* last z bin that can hold an entry passing min_p (with slack);
                                * ZBINS - 1 when min_p is off or that deep */
     bool            minp_listed; /* the exp-sum pass listed every row up to that bin */
+    bool            cap_after;   /* top-k: the scan ran on the logits before the soft-cap (the
+                                  * thread maxima, the candidates); the row-final kernel applies
+                                  * it to what it keeps. The cap tanhf(x / c) * c never turns the
+                                  * order of two logits round (tanhf is monotone over every
+                                  * binary32, tests/test_tanhf_exact.py), but it maps neighbouring
+                                  * logits to the same value: only entries whose capped value lies
+                                  * strictly above the capped bound are certain to be all there
+                                  * is, and k of those are needed. */
 };
 
 /* ============================================================================================
@@ -1036,6 +1044,9 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
     if (real < a.k_sel || tau < 0x00800000u)
         return true;
     const float bound = key2f(tau);
+    /* what a kept element has to reach: the bound itself, or -- when the maxima were taken
+     * before the soft-cap -- more than the capped bound (see FinalArgs::cap_after) */
+    const float bound_kept = a.cap_after ? softcap1(bound, rv.softcap) : bound;
     /* 3 */
     uint32_t selmask = 0u;
 #pragma unroll
@@ -1136,7 +1147,8 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             /* (a NaN fails the comparison: keys are > 0) */
-            if (x4[c] >= bound && c < nvalid && ((ok >> c) & 1u)) {
+            if ((a.cap_after ? x4[c] > bound_kept : x4[c] >= bound_kept) && c < nvalid &&
+                ((ok >> c) & 1u)) {
                 ck[q][c] = f2key(x4[c]);
                 ++n_keep;
             }
@@ -1749,6 +1761,7 @@ static FinalArgs final_args(const FinalLaunch &f) {
     a.ln_min_p   = f.min_p > 0.0f ? std::log((double) f.min_p) : 0.0;
     a.zb_min_p    = zbin_of_min_p(f.min_p);
     a.minp_listed = f.minp_listed;
+    a.cap_after   = f.cap_after;
     return a;
 }
 

@@ -9,9 +9,34 @@
 
 #include "../../geistlib_amd/csrc/glibc_tanhf.h"
 
+// "mono" as third argument: counts instead the floats x in the range whose successor has a
+// smaller tanhf (the function would then not be monotone); same three numbers.
+static int monotone(uint32_t lo, uint32_t hi) {
+    long    bad = 0, total = 0;
+    int64_t first = -1;
+#pragma omp parallel for reduction(+ : bad, total) schedule(static)
+    for (int64_t b = lo; b < (int64_t) hi; ++b) {
+        const uint32_t u0 = (uint32_t) b, u1 = u0 + 1u;
+        float          x0, x1;
+        memcpy(&x0, &u0, 4);
+        memcpy(&x1, &u1, 4);
+        ++total;
+        if (geist_tanhf_glibc(x1) < geist_tanhf_glibc(x0)) {
+            ++bad;
+#pragma omp critical
+            if (first < 0 || b < first)
+                first = b;
+        }
+    }
+    printf("%ld %ld %lld\n", bad, total, (long long) first);
+    return 0;
+}
+
 int main(int argc, char **argv) {
     const uint32_t lo = argc > 1 ? (uint32_t) strtoul(argv[1], nullptr, 0) : 0u;
     const uint32_t hi = argc > 2 ? (uint32_t) strtoul(argv[2], nullptr, 0) : 0x7f800000u;
+    if (argc > 3 && strcmp(argv[3], "mono") == 0)
+        return monotone(lo, hi);
     long           bad = 0, total = 0;
     int64_t        first = -1;
 #pragma omp parallel for reduction(+ : bad, total) schedule(static)

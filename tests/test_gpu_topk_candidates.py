@@ -147,3 +147,59 @@ def test_calls_that_stay_off_the_candidate_path(hs, oracle):
         okw = {k_: v for k_, v in kw.items() if k_ in ("temperature", "top_k", "top_p", "min_p")}
         want, infos = want_rows(oracle, x, u, hist=h, pen=pen, **okw)
         compare_ids(got, want, infos, f"off the candidate path {kw}")
+
+
+def test_soft_capped_rows_select_on_raw_logits_and_cap_what_they_keep(hs, oracle):
+    """The soft-cap (head.c:148-159) keeps the order of the logits, so the scan hands on raw
+    values and the row-final kernel caps its candidates. Ordinary rows stay on the candidate
+    path; rows whose leaders the cap presses into one value (logits far beyond the cap) cannot
+    be certified from candidates -- ties are broken by index over the whole row -- and are passed
+    on. Penalties come before the cap, as in the exact scan."""
+    g = np.random.default_rng(314)
+    n, k, rows, cap = 128256, 40, 12, 30.0
+    x = (g.standard_normal((rows, n)) * 4).astype(np.float32)
+    x[1] *= 2                                        # bent by the cap, still distinct
+    x[2] = (g.standard_normal(n) * 400).astype(np.float32)     # thousands saturate at +-cap
+    x[3, g.integers(0, n, 60)] = 1e4                 # 60 equal leaders: all of them candidates
+    x[4, :7] = [np.inf, 500.0, 499.0, 200.0, 30.0, 29.999, -np.inf]
+    u = units(g, rows)
+    kw = dict(temperature=0.8, top_k=k, top_p=0.95)
+    got = run_rows(hs, torch, x, u, P(softcap=cap, **kw))
+    paths = hs.topk_paths(rows).tolist()
+    res = [oracle.chain_u(oracle.softcap(x[r], cap), float(u[r]), **kw) for r in range(rows)]
+    compare_ids(got, [t for t, _ in res], [i for _, i in res], "soft-capped candidates")
+    print("paths:", paths)
+    assert paths[0] == 0 and paths[1] == 0 and all(p == 0 for p in paths[5:]), paths
+    assert paths[2] != 0, paths
+    # with penalties in front of the cap
+    H = 300
+    hist = g.integers(0, n, (rows, H)).astype(np.int32)
+    top = np.argsort(-x, axis=1)[:, :10].astype(np.int32)
+    hist[:, :10] = top
+    hl = np.full(rows, H, dtype=np.int32)
+    pen = (1.2, 0.3, 0.1)
+    got = run_rows(hs, torch, x, u, P(softcap=cap, rep=pen[0], freq=pen[1], pres=pen[2], **kw),
+                   hist, hl)
+    res = [oracle.chain_u(oracle.softcap(oracle.penalties(x[r], hist[r], *pen), cap), float(u[r]),
+                          **kw) for r in range(rows)]
+    compare_ids(got, [t for t, _ in res], [i for _, i in res], "soft-capped, penalised")
+
+
+def test_soft_capped_rows_on_the_thread_maxima_path(oracle):
+    """The same split of work where the candidate path does not apply (k above its limit, a mask,
+    an unaligned row): thread maxima of the raw logits, the cap on what the row-final kernel
+    gathers, strict comparison with the capped bound."""
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=16, max_vocab=70000)
+    g = np.random.default_rng(99)
+    n, rows, cap = 65537, 8, 20.0
+    x = (g.standard_normal((rows, n)) * 6).astype(np.float32)
+    x[1] = (g.standard_normal(n) * 300).astype(np.float32)     # saturated leaders: passed on
+    x[2, g.integers(0, n, 200)] = 77.0
+    u = units(g, rows)
+    for k in (100, 40):
+        kw = dict(temperature=0.9, top_k=k, top_p=0.9)
+        got = run_rows(s, torch, x, u, P(softcap=cap, **kw))
+        res = [oracle.chain_u(oracle.softcap(x[r], cap), float(u[r]), **kw) for r in range(rows)]
+        compare_ids(got, [t for t, _ in res], [i for _, i in res], f"soft-capped maxima k={k}")
+    s.close()

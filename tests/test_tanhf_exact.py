@@ -39,3 +39,13 @@ def test_nans_stay_nans(checker):
     assert bad == 0
     bad, _, _ = run(checker, 0xFF800001, 0xFF800100)
     assert bad == 0
+
+
+def test_monotone_over_every_float(checker):
+    """tanhf(next float) >= tanhf(float) for every non-negative float (the function is odd by
+    construction): the soft-cap tanhf(x / cap) * cap then keeps the order of the logits, which is
+    what lets the top-k path select on raw logits and cap only the candidates."""
+    out = subprocess.run([checker, hex(0), hex(0x7F800000), "mono"], capture_output=True,
+                         text=True, check=True)
+    bad, total, first = map(int, out.stdout.split())
+    assert total == 0x7F800000 and bad == 0, hex(first)
