@@ -653,14 +653,13 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
     f.mode     = FINAL_SORTED;
     f.row_flag = s->row_flag;
     /* rows whose kept prefix is too wide for the shortcut of the row-final kernel flag themselves
-     * 1: their candidates are listed and walked; what that cannot serve either is flagged 2 for
-     * the whole-row walk. Each of these kernels returns at once for every row not flagged for
-     * it. With the candidates already listed by the exp-sum pass the list walk comes first and
-     * alone. */
+     * 1: their candidates are listed and walked; what that cannot serve either takes the
+     * whole-row walk inside the list-walk kernel. Each of these kernels returns at once for every
+     * row not flagged for it. With the candidates already listed by the exp-sum pass the list
+     * walk comes first and alone. */
     if (!f.minp_direct)
         launch_row_final(L, f);
-    launch_candidates(L, f);
-    launch_sorted_general(L, f, s->probs, (long) s->max_vocab);
+    launch_candidates(L, f, s->probs, (long) s->max_vocab);
     return after_launch(s, "top-p / min-p");
 }
 

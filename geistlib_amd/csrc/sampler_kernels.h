@@ -189,14 +189,13 @@ int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */
 int configure_device_kernels();
 /* rows flagged 1 by the sorted row-final kernel: list their candidates, then draw from the
- * list; rows the list cannot serve are flagged 2 for the two kernels below */
-void launch_candidates(const Launch &L, const FinalLaunch &f);
+ * list; rows the list cannot serve (and rows the row-final kernel flagged 2) take the whole-row
+ * walk in the same launch: probabilities of the whole row into `probs`, then the walk over them */
+void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs);
 /* row_flag != NULL: only rows flagged 2 are written */
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
                         const double *chunk_sum, float *probs, long ld_probs,
                         const int32_t *row_flag);
-/* rows flagged 2: probabilities of the whole row into `probs`, then the walk over them */
-void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs);
 /* after launch_tmax_scan(L, tmax, chunk_best): out[row][j] = log_softmax(row)[tokens[row][j]] */
 void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,
                     const int32_t *tokens, long tokens_ld, int k_per_row, double *out, long out_ld);

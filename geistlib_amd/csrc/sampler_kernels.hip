@@ -15,7 +15,7 @@
  *   k_cand_scan, k_final_cand (sampler_cands.h)   the top-k path for plain rows: the scan hands
  *                    each wavefront's leading groups on, the row-final kernel gathers nothing
  *                                                                              sampler.c:178-228
- *   k_list_candidates, k_sorted_candidates, k_sorted_general (sampler_sorted_prob.h)
+ *   k_list_candidates, k_sorted_candidates (sampler_sorted_prob.h)
  *                    full-vocabulary top-p / min-p for kept prefixes the shortcut cannot
  *                    serve: candidate list, then the whole row                 sampler.c:246-304
  *   k_write_probs    normalised probabilities of a row                        sampler.c:246-253
@@ -944,7 +944,7 @@ struct FinalArgs {
     const float    *tmax;
     int32_t        *out;
     int32_t        *row_flag; /* FINAL_SORTED: 1 = the row goes on to the candidate list,
-                               * 2 = to k_sorted_general */
+                               * 2 = to the whole-row walk */
     CandSpace       cand;
     double          ln_min_p; /* log(min_p), taken on the host */
     int             zb_min_p; /* last z bin that can hold an entry passing min_p (with slack);
@@ -1249,7 +1249,7 @@ __global__ __launch_bounds__(TPB) void k_final_temperature(RowView rv, FinalArgs
 }
 
 /* top-p / min-p over the whole vocabulary (sampler.c:232-305): the thread-maxima shortcut; a
- * row it cannot serve raises its flag for k_sorted_general. */
+ * row it cannot serve raises its flag for the whole-row walk. */
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
     __shared__ uint64_t s_red[NWAVES];
@@ -1861,38 +1861,47 @@ void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best
 
 int configure_device_kernels() {
     /* k_sorted_candidates keeps a whole candidate list in LDS: more than the static limit */
-    return (int) hipFuncSetAttribute((const void *) k_sorted_candidates,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     CAND_CAP * (int) sizeof(uint32_t));
+    const int   dyn = CAND_CAP * (int) sizeof(uint32_t);
+    const void *kernels[] = {(const void *) k_sorted_candidates<2, false>,
+                             (const void *) k_sorted_candidates<2, true>,
+                             (const void *) k_sorted_candidates<8, false>,
+                             (const void *) k_sorted_candidates<8, true>};
+    for (const void *k : kernels) {
+        const hipError_t e =
+            hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
+        if (e != hipSuccess)
+            return (int) e;
+    }
+    return 0;
 }
 
-void launch_candidates(const Launch &L, const FinalLaunch &f) {
+void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     const int  dyn = CAND_CAP * (int) sizeof(uint32_t); /* see configure_device_kernels() */
+    SortedRowArgs g;
+    g.inv_t      = f.inv_t;
+    g.chunk_best = f.chunk_best;
+    g.chunk_sum  = f.chunk_sum;
+    g.probs      = probs;
+    g.ld_probs   = ld_probs;
     if (f.minp_direct) {
         /* the exp-sum pass has listed every row: no row-final kernel, no listing pass. An
          * unlisted element lies in z bin zb + 1 or beyond; the same expf as on the device. */
         static const uint64_t tab[32] = GEIST_EXPF_TABLE_INIT;
         const int             zb      = zbin_of_min_p(f.min_p);
         const float p_out = geist_expf_glibc_le0(-(float) (zb + 1) / (float) ZBIN_PER_NAT, tab);
-        k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(
-            f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, f.chunk_sum, L.rv.n_chunks,
-            p_out);
+        dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
+            k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
+                L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, f.chunk_sum,
+                L.rv.n_chunks, p_out);
+        });
         return;
     }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
             L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
-    });
-    k_sorted_candidates<<<dim3(L.rows), block, dyn, L.stream>>>(
-        f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f);
-}
-
-void launch_sorted_general(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {
-    dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_sorted_general<GS_NV, GS_PEN><<<dim3(L.rows), dim3(TPB), 0, L.stream>>>(
-            L.rv, f.inv_t, f.chunk_best, f.chunk_sum, probs, ld_probs, f.top_p, f.min_p, f.uniforms,
-            f.row_flag, f.out, f.cand.path);
+        k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
+            L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f);
     });
 }
 

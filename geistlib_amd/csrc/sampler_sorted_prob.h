@@ -13,7 +13,7 @@
  *                                every element up to a z bin is listed with its normalised
  *                                probability; one mass histogram over the list locates the
  *                                nucleus edge and the draw. Kept prefixes of thousands.
- *   whole row (flag 2: k_sorted_general)   the row's probabilities are written once, then a
+ *   whole row (flag 2: sorted_general_row)  the row's probabilities are written once, then a
  *                                mass-weighted radix descent over their bit patterns finds the
  *                                edge and the drawn entry. Anything else.
  */
@@ -338,7 +338,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
 }
 
 /* ============================================================================================
- * k_sorted_general: rows the fast path handed on (row_flag != 0). One workgroup per row works
+ * The whole-row walk: rows the fast path handed on (row_flag != 0). One workgroup per row works
  * on the row's normalised probabilities pn (written by k_write_probs).
  *
  * The sorted order of the reference (pn descending, equal pn by ascending index) is never
@@ -693,52 +693,49 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
     return tok;
 }
 
-/* k_sorted_general: rows flagged 2. One workgroup per row first writes the row's normalised
- * probabilities pn_i = (float)((double)p_i / sum) (sampler.c:246-253) into the probs workspace,
- * chunk by chunk, then walks them. The rows that get here are rare (kept prefixes of tens of
- * thousands of entries, rows of equal values), so the row is not spread over more workgroups. */
+/* The whole-row walk, for rows that neither the shortcut nor the list can serve (kept prefixes
+ * of tens of thousands of entries, rows of equal values): the workgroup first writes the row's
+ * normalised probabilities pn_i = (float)((double)p_i / sum) (sampler.c:246-253) into the probs
+ * workspace, chunk by chunk, then walks them. Such rows are rare, so the row is not spread over
+ * more workgroups. Called by every thread of a 256-thread workgroup. */
+struct SortedRowArgs {
+    float           inv_t;
+    const uint64_t *chunk_best;
+    const double   *chunk_sum;
+    float          *probs;
+    long            ld_probs;
+};
 template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_sorted_general(RowView rv, float inv_t,
-                                                        const uint64_t *__restrict__ chunk_best,
-                                                        const double *__restrict__ chunk_sum,
-                                                        float *__restrict__ probs, long ld_probs,
-                                                        float top_p, float min_p,
-                                                        const float *__restrict__ uniforms,
-                                                        const int32_t *__restrict__ row_flag,
-                                                        int32_t *__restrict__ out,
-                                                        int32_t *__restrict__ path) {
-    __shared__ SortedGenShared sh;
-    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
-    __shared__ uint64_t s_tab[32];
-    __shared__ int      s_scan[NWAVES];
-    __shared__ int      s_pick;
-    __shared__ double   s_total;
-    const int row = blockIdx.x, tid = threadIdx.x;
-    if (row_flag[row] != 2)
-        return;
+__device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, int n_rows,
+                                                  const SortedRowArgs &g, float top_p, float min_p,
+                                                  float u, SortedGenShared &sh, uint32_t *s_cnt16,
+                                                  uint64_t *s_tab, int *s_scan, int *s_pick,
+                                                  double *s_total) {
+    const int tid = threadIdx.x;
+    __syncthreads(); /* the caller's use of the shared words is over */
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
     if (tid == 0) {
         double t = 0.0;
         for (int c = 0; c < rv.n_chunks; ++c)
-            t += chunk_sum[(long) row * rv.n_chunks + c];
-        s_total = t;
+            t += g.chunk_sum[(long) row * rv.n_chunks + c];
+        *s_total = t;
     }
-    const float  mx = key2f(best_key(row_best_from_chunks(chunk_best, row, rv.n_chunks, sh.red64)));
-    const double tot = s_total;
-    float       *pn  = probs + (long) row * ld_probs;
+    const float  mx = key2f(best_key(row_best_from_chunks(g.chunk_best, row, rv.n_chunks, sh.red64)));
+    const double tot = *s_total;
+    float       *pn  = g.probs + (long) row * g.ld_probs;
     for (int chunk = 0; chunk < rv.n_chunks; ++chunk) {
         int base, end;
         chunk_bounds<NV>(rv, chunk, base, end);
         float4 v[NV];
-        fetch_chunk<NV, PEN>(rv, row, (int) gridDim.x, base, end, s_cnt16, v);
+        fetch_chunk<NV, PEN>(rv, row, n_rows, base, end, s_cnt16, v);
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int e = base + 4 * (j * TPB + tid);
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 if (e + c < end) {
-                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, g.inv_t), s_tab);
                     pn[e + c]     = (float) ((double) p / tot);
                 }
             }
@@ -747,12 +744,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_general(RowView rv, float inv_t,
     }
     __threadfence_block();
     __syncthreads();
-    const int tok = sorted_descend<false>(pn, nullptr, rv.n_vocab, top_p, min_p, uniforms[row], 0u,
-                                          sh, s_scan, &s_pick);
-    if (tid == 0) {
-        out[row]  = tok;
-        path[row] = 3;
-    }
+    return sorted_descend<false>(pn, nullptr, rv.n_vocab, top_p, min_p, u, 0u, sh, s_scan, s_pick);
 }
 
 /* ============================================================================================
@@ -1091,13 +1083,15 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
 
 /* k_sorted_candidates: one workgroup per row flagged 1 or 4 walks the row's list (staged in LDS
  * when it fits; flag 4: listed by the exp-sum pass, holding p). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
- * prefix that may reach past the list -- is flagged 2 for k_sorted_general.
+ * prefix that may reach past the list -- takes the whole-row walk (flag 2).
  * direct_sum != NULL: every row was listed by the exp-sum pass under the min-p bound (the list
  * holds p, not pn) and no other kernel ran in between: the row's sum is taken from the chunk
  * sums here (in chunk order, as everywhere), the bound on an unlisted element's pn from
  * direct_p_out = expf of the first z bin outside the list, and the flag is written for every
  * row. */
-__global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float top_p, float min_p,
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRowArgs g,
+                                                           CandSpace cand, float top_p, float min_p,
                                                            const float *__restrict__ uniforms,
                                                            int32_t *__restrict__ row_flag,
                                                            int32_t *__restrict__ out,
@@ -1108,11 +1102,24 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
         SortedGenShared gen;
         ListWalkShared  fast;
     } sh;
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ uint64_t s_tab[32];
+    __shared__ double   s_total;
     __shared__ int      s_scan[NWAVES];
     __shared__ int      s_pick;
     __shared__ uint32_t s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int flag = direct_sum ? 5 : row_flag[row];
+    if (flag == 2) { /* sent past the list by the row-final kernel */
+        const int t = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p,
+                                                  uniforms[row], sh.gen, s_cnt16, s_tab, s_scan,
+                                                  &s_pick, &s_total);
+        if (tid == 0) {
+            out[row]       = t;
+            cand.path[row] = 3;
+        }
+        return;
+    }
     if (flag != 1 && flag != 4 && flag != 5)
         return;
     const int n   = cand.count[row];
@@ -1162,11 +1169,18 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(CandSpace cand, float
                                        s_scan, &s_pick);
         }
     }
+    /* what the list cannot certify takes the whole-row walk here and now (tok is the same in
+     * every thread) */
+    int path = 2;
+    if (tok < 0) {
+        tok  = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p, uniforms[row],
+                                           sh.gen, s_cnt16, s_tab, s_scan, &s_pick, &s_total);
+        path = 3;
+    }
     if (tid == 0) {
-        row_flag[row] = tok < 0 ? 2 : 0;
-        out[row]      = tok;
-        if (tok >= 0)
-            cand.path[row] = 2;
+        row_flag[row]  = path == 3 ? 2 : 0;
+        out[row]       = tok;
+        cand.path[row] = path;
     }
 }
 
