@@ -140,7 +140,7 @@ struct FinalLaunch {
  * probe_token != NULL: the rows are n_seq * (probe_L + 1) target rows of a speculative batch and
  * probe_token holds the n_seq * probe_L draft ids; probe_p[row] receives p at the row's draft id.
  * list != NULL (min-p set): the pass also lists, per row, every element up to z bin zb_list with
- * its unnormalised p -- the min-p bound needs nothing but the row maximum (the pass clears
+ * its softmax argument -- the min-p bound needs nothing but the row maximum (the pass clears
  * list->count itself).
  * slab_sum != NULL (and no list): also the sums of the chunk's slabs of 1024 elements,
  * [rows][chunks][8], which the index-order walks locate their starting point with.

@@ -410,11 +410,10 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
             for (int c = 0; c < 4; ++c) {
                 if ((mask >> (4 * j + c)) & 1u) {
                     if (pos < CAND_CAP) {
-                        float arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
-                        /* (opaque, so that the evaluation stays under its condition: few
-                         * elements are listed) */
-                        asm volatile("" : "+v"(arg));
-                        ck[pos] = __float_as_uint(geist_expf_glibc_le0(arg, s_tab));
+                        /* the softmax argument; the list walk takes the exponential of the few
+                         * hundred entries it reads (here it would run under divergence, once
+                         * per listed element for the whole wavefront) */
+                        ck[pos] = __float_as_uint(softmax_arg(f4_get(v[j], c), mx, inv_t));
                         ci[pos] = (uint32_t) (e + c);
                     }
                     ++pos;
@@ -1294,7 +1293,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         return;
     }
     if (a.minp_listed && a.cand.count[row] <= CAND_CAP) {
-        /* the exp-sum pass listed the row under the min-p bound (holding p, not pn): the list
+        /* the exp-sum pass listed the row under the min-p bound (holding softmax arguments, not pn): the list
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */
         if (tid == 0) {
             const int   B      = a.zb_min_p;

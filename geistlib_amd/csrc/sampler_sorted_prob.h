@@ -1085,7 +1085,7 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
  * when it fits; flag 4: listed by the exp-sum pass, holding p). On success the flag is cleared; a row the list cannot serve -- too long, or a kept
  * prefix that may reach past the list -- takes the whole-row walk (flag 2).
  * direct_sum != NULL: every row was listed by the exp-sum pass under the min-p bound (the list
- * holds p, not pn) and no other kernel ran in between: the row's sum is taken from the chunk
+ * holds softmax arguments, not pn) and no other kernel ran in between: the row's sum is taken from the chunk
  * sums here (in chunk order, as everywhere), the bound on an unlisted element's pn from
  * direct_p_out = expf of the first z bin outside the list, and the flag is written for every
  * row. */
@@ -1110,6 +1110,9 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
     __shared__ uint32_t s_idx[CAND_LDS];
     const int row = blockIdx.x, tid = threadIdx.x;
     const int flag = direct_sum ? 5 : row_flag[row];
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    __syncthreads();
     if (flag == 2) { /* sent past the list by the row-final kernel */
         const int t = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p,
                                                   uniforms[row], sh.gen, s_cnt16, s_tab, s_scan,
@@ -1140,7 +1143,8 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
     if (n >= 1 && n <= CAND_CAP) {
         const uint32_t *gk = cand.key + (long) row * CAND_CAP;
         const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
-        /* flag 4: the list holds p; pn = (float)((double)p / sum), sampler.c:251-253 */
+        /* flags 4, 5: the list holds the softmax arguments; p = expf(argument),
+         * pn = (float)((double)p / sum), sampler.c:80, 251-253 */
         for (int i0 = 0; i0 < n; i0 += 8 * TPB) { /* eight independent loads in flight per thread */
             uint32_t k[8];
 #pragma unroll
@@ -1150,7 +1154,9 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
             for (int q = 0; q < 8; ++q) {
                 const int i = i0 + q * TPB + tid;
                 if (i < n)
-                    s_key[i] = flag >= 4 ? __float_as_uint((float) ((double) __uint_as_float(k[q]) / sum))
+                    s_key[i] = flag >= 4 ? __float_as_uint((float) ((double) geist_expf_glibc_le0(
+                                                                        __uint_as_float(k[q]), s_tab) /
+                                                                    sum))
                                          : k[q];
             }
         }
