@@ -255,17 +255,22 @@ __global__ __launch_bounds__(64 * Q6K_LISTED_WAVES) void k_q6k_linear_listed(
 
 /* ---- the table repacked for the device --------------------------------------------------------
  * The GGUF layout puts a row's blocks one after the other, 210 bytes each: lanes that own
- * neighbouring rows read addresses a row apart, and a block shares its first and last cache line
- * with its neighbours. geist_hip_q6k_pack (once per model, at load) writes the same bytes in the
- * order the kernel reads them: the table rows in groups of 64 (a wavefront), per group the blocks
- * in order, per block the 53 dwords of each of the 64 rows with the rows innermost --
+ * neighbouring rows read addresses a row apart, a block shares its first and last cache line
+ * with its neighbours, and an element's six bits lie in two places. geist_hip_q6k_pack (once per
+ * model, at load) writes the same information in the order and form the kernel wants: the table
+ * rows in groups of 64 (a wavefront), per group the blocks in order, per block 53 dwords for
+ * each of the 64 rows with the rows innermost --
  *   dwords 4 p .. 4 p + 3 of row r (p < 13) at  base + p * 256 + 4 r,   dword 52 at base + 3328 + r
  * (in dwords; base = (group * blocks + b) * 3392) -- so that a wavefront's 16-byte loads read one
- * kilobyte of consecutive addresses and every byte of the table is read once. Rows beyond n_out
- * in the last group are zero blocks.
+ * kilobyte of consecutive addresses and every byte is read once. A row's 53 dwords hold the
+ * block's 256 six-bit values in the order of the elements, element e in bits 6 e .. 6 e + 5 of
+ * dwords 0..47 (one extraction per element; two of every sixteen straddle a dword), the sixteen
+ * scales in dwords 48..51 and d in the low half of dword 52. Rows beyond n_out in the last group
+ * are zero blocks.
  *
- * With the loads out of the way the kernel can afford the reference's own order of additions:
- * a lane owns a table row and adds its products one after the other in index order,
+ * With the loads and the bit assembly out of the way the kernel can afford the reference's own
+ * order of additions: a lane owns a table row and adds its products one after the other in index
+ * order,
  *   acc = fma(x[k], w[k], acc),  w = fma(ds, q_unsigned, -32 ds)   (both exact, see the header)
  * which is cpu_scalar_w_quant_m1's sum bit for bit, with nothing to bound and nothing to repeat.
  * The chain of dependent additions is hidden by the conversions of the following elements and
@@ -290,12 +295,33 @@ __global__ __launch_bounds__(Q6K_TPB) void k_q6k_pack(const uint8_t *__restrict_
         for (int i = 0; i < 53; ++i)
             d[i] = 0u;
     }
+    /* the six-bit values in element order: element 128 h + 32 j + l takes nibble (j >> 1) of
+     * ql[64 h + 32 (j & 1) + l] and bits 2 j, 2 j + 1 of qh[32 h + l] (q6_K.c:30-36) */
+    uint32_t o[53];
+#pragma unroll
+    for (int i = 0; i < 48; ++i)
+        o[i] = 0u;
+#pragma unroll
+    for (int e = 0; e < 256; ++e) {
+        const int      h = e >> 7, j = (e >> 5) & 3, l = e & 31;
+        const int      qlb = 64 * h + 32 * (j & 1) + l, qhb = 32 * h + l;
+        const uint32_t lo = (d[qlb / 4] >> (8 * (qlb % 4) + 4 * (j >> 1))) & 0xFu;
+        const uint32_t hi = (d[32 + qhb / 4] >> (8 * (qhb % 4) + 2 * j)) & 3u;
+        const uint32_t q  = lo | (hi << 4);
+        const int      bit = 6 * e, w0 = bit >> 5, off = bit & 31;
+        o[w0] |= q << off;
+        if (off > 26)
+            o[w0 + 1] |= q >> (32 - off);
+    }
+#pragma unroll
+    for (int i = 48; i < 53; ++i)
+        o[i] = d[i];
     uint32_t *base = packed + item * Q6K_PACK_DWORDS;
 #pragma unroll
     for (int p = 0; p < 13; ++p)
         *reinterpret_cast<uint4 *>(base + p * 256 + 4 * r) =
-            make_uint4(d[4 * p], d[4 * p + 1], d[4 * p + 2], d[4 * p + 3]);
-    base[3328 + r] = d[52];
+            make_uint4(o[4 * p], o[4 * p + 1], o[4 * p + 2], o[4 * p + 3]);
+    base[3328 + r] = o[52];
 }
 
 template <int MT>
@@ -327,33 +353,22 @@ __global__ __launch_bounds__(Q6K_TPB) void k_q6k_packed_linear(const uint32_t *_
         d[52] = __builtin_nontemporal_load(base + 3328 + r);
         const float dd = __half2float(__ushort_as_half((unsigned short) (d[52] & 0xffffu)));
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int g16 = 0; g16 < 16; ++g16) { /* the sixteen scale groups, in element order */
+            const int    sc = (int) (int8_t) (d[48 + g16 / 4] >> (8 * (g16 % 4)));
+            const double ds = (double) (dd * (float) sc), m32ds = -32.0 * ds;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int i = 0; i < 16; ++i) {
+                const int bit = 6 * (16 * g16 + i), w0 = bit >> 5, off = bit & 31;
+                /* (straddling values: the funnel shift's low six bits) */
+                const uint32_t q  = off <= 26
+                                        ? (d[w0] >> off) & 63u
+                                        : __builtin_amdgcn_alignbit(d[w0 + 1], d[w0], off) & 63u;
+                const double   wv = __builtin_fma(ds, (double) q, m32ds);
+                const int      k  = Q6K_BLOCK_ELEMS * b + 16 * g16 + i;
 #pragma unroll
-                for (int l4 = 0; l4 < 8; ++l4) {
-                    const int      si  = 8 * h + 2 * j + l4 / 4;
-                    const int      sc  = (int) (int8_t) (d[48 + si / 4] >> (8 * (si % 4)));
-                    const double   ds  = (double) (dd * (float) sc), m32ds = -32.0 * ds;
-                    const uint32_t qlw = d[16 * h + 8 * (j & 1) + l4];
-                    const uint32_t qhw = d[32 + 8 * h + l4];
-                    const uint32_t lo4 = ((j >> 1) ? qlw >> 4 : qlw) & 0x0F0F0F0Fu;
-                    const uint32_t hi4 = (j == 0   ? qhw << 4
-                                          : j == 1 ? qhw << 2
-                                          : j == 2 ? qhw
-                                                   : qhw >> 2) &
-                                         0x30303030u;
-                    const uint32_t qu = lo4 | hi4; /* four unsigned 6-bit values, a byte each */
-                    const int      k0 = Q6K_BLOCK_ELEMS * b + 128 * h + 32 * j + 4 * l4;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const double wv = __builtin_fma(ds, (double) q6k_ubyte(qu, i), m32ds);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m) {
-                            const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in;
-                            acc[m] = __builtin_fma(xm[k0 + i], wv, acc[m]); /* uniform address */
-                        }
-                    }
+                for (int m = 0; m < MT; ++m) {
+                    const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in;
+                    acc[m] = __builtin_fma(xm[k], wv, acc[m]); /* uniform address */
                 }
             }
         }
