@@ -469,7 +469,7 @@ static int reserve_sorted_workspace(geist_hip_sampler *s) {
     if (e == hipSuccess) e = hipMalloc((void **) &c.out_key, R * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &c.key, R * CAND_CAP * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &c.idx, R * CAND_CAP * sizeof(uint32_t));
-    if (e == hipSuccess) e = hipMalloc((void **) &c.count, R * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void **) &c.count, R * gs::CAND_COUNT_STRIDE * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &c.row_sum, R * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &c.path, R * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &probs, R * s->max_vocab * sizeof(float));

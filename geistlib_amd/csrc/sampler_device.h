@@ -171,6 +171,21 @@ __device__ __forceinline__ int wave_reserve(int cnt, int *counter) {
 }
 
 /* ---- workgroup combines through LDS -------------------------------------------------------- */
+/* Combining without a barrier: every wavefront of the workgroup deposits its part in LDS and
+ * then calls this; the call returns true (in all lanes) in the wavefront that arrives last,
+ * which finds every part deposited -- the LDS operations of a workgroup are performed in the
+ * order they were issued. The others go on without waiting. `counter` (LDS) must hold zero, and
+ * a barrier must have published that, before the first arrival. */
+__device__ __forceinline__ bool wave_arrives_last(uint32_t *counter) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    uint32_t ticket = 0;
+    if ((threadIdx.x & (WAVE - 1)) == 0)
+        ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_WORKGROUP);
+    ticket = readlane_u32(ticket, 0);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return ticket == NWAVES - 1;
+}
 /* All 256 threads call; every thread receives the maximum. `scratch` holds NWAVES entries. */
 __device__ __forceinline__ uint64_t block_max_u64(uint64_t v, uint64_t *scratch) {
     v = wave_max_u64(v);

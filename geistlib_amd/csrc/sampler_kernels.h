@@ -66,12 +66,14 @@ constexpr int ZBINS        = 128;
 constexpr int ZBIN_PER_NAT = 4;
 constexpr int CAND_CAP     = 16384; /* list entries per row */
 constexpr int CAND_LDS     = 4096;  /* lists up to this length are staged in LDS */
+constexpr int CAND_COUNT_STRIDE = 32;
 struct CandSpace {
     int32_t  *row_bound; /* [rows] last z bin listed */
     uint32_t *out_key;   /* [rows] bits of a pn no element past that bin can exceed */
     uint32_t *key;       /* [rows][CAND_CAP] bits of pn */
     uint32_t *idx;       /* [rows][CAND_CAP] vocabulary ids */
-    int32_t  *count;     /* [rows] */
+    int32_t  *count;     /* [rows * CAND_COUNT_STRIDE]: a row's counter has a cache line to itself
+                          * (the appending wavefronts' atomic adds to one line serialise) */
     double   *row_sum;   /* [rows] the row's exp-sum, for lists that hold p instead of pn */
     int32_t  *path;      /* [rows] which walk served the row: 1 thread-maxima shortcut, 2 list,
                           * 3 whole row */

@@ -145,6 +145,39 @@ __device__ __forceinline__ uint64_t row_best_from_chunks(const uint64_t *__restr
  * (row_best_meet): each keeps its chunk in registers, reports the chunk's maximum, waits for the
  * others' and sums the exponentials from the registers. The rows are read once.
  * ========================================================================================== */
+/* The first index among a wavefront's elements whose key is `bk`, the wavefront's greatest,
+ * packed with it; 0 when no element has that key (bk == 0: nothing but NaN). Every lane receives
+ * it. Element c of group j of lane l sits at base + 4 (j TPB + tid) + c, so the first index is in
+ * the first group that holds the value, there in the first lane, there in the first component:
+ * a ballot per group instead of a search through each lane's elements and a reduction. Equal
+ * keys are equal floats (f2key merges the zeros and gives every NaN key 0, which no float's
+ * comparison matches). `bounded`: positions at or beyond `end` may hold anything. */
+template <int NV, bool PLAIN>
+__device__ __forceinline__ uint64_t wave_first_of(const float4 (&v)[NV], uint32_t bk, int base,
+                                                  int end) {
+    const float m   = key2f(bk);
+    const int   tid = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int e = base + 4 * (j * TPB + tid);
+        bool h0 = v[j].x == m, h1 = v[j].y == m, h2 = v[j].z == m, h3 = v[j].w == m;
+        if (!PLAIN) {
+            h0 = h0 && e < end;
+            h1 = h1 && e + 1 < end;
+            h2 = h2 && e + 2 < end;
+            h3 = h3 && e + 3 < end;
+        }
+        const uint64_t hit = __builtin_amdgcn_ballot_w64(h0 || h1 || h2 || h3);
+        if (hit) {
+            const int lane = __builtin_ctzll(hit);
+            const int c    = h0 ? 0 : h1 ? 1 : h2 ? 2 : 3;
+            const int idx  = __builtin_amdgcn_readlane(e + c, lane);
+            return pack_best(bk, (uint32_t) idx);
+        }
+    }
+    return 0;
+}
+
 /* Where the thread maxima and the chunk results go, and the slots through which the workgroups
  * of a row meet. */
 struct FusedScan {
@@ -152,20 +185,22 @@ struct FusedScan {
     uint64_t *chunk_best;
     uint64_t *slots;
     uint32_t  wait_limit;
-    uint64_t *s_red; /* LDS, NWAVES words */
-    uint64_t *s_bb;  /* LDS, one word */
+    uint64_t *s_red;    /* LDS, NWAVES words */
+    uint64_t *s_bb;     /* LDS, one word */
+    uint32_t *s_arrive; /* LDS, two arrival counters, zero and published before use */
 };
 
 /* The row's maximum (packed with its first index) once every chunk of the row has reported its
  * own, for the workgroup that has just found `mine`. Every thread returns the same value.
  *
- * The workgroup stores `mine` (never zero) into its slot and its first wavefront polls the row's
- * n_chunks <= 2 * WAVE slots, a lane per slot, until none reads zero; the maximum of what it then
- * holds is the row's. Stores and polls are device-scope atomics (plain stores and loads, no
- * read-modify-write: the slots of a row share a few cache lines, and contended atomic updates of
- * one line are what would make this wait slow), so no fence is needed; `prior` (thread 0's) is a
- * value returned by an earlier atomic of the caller's, made an operand of the store so that the
- * row's other workgroups find that atomic performed when they leave the wait.
+ * One wavefront of the workgroup (`reporter`: the one that combined the chunk's maximum) stores
+ * `mine` (never zero) into the chunk's slot and polls the row's n_chunks <= 2 * WAVE slots, a
+ * lane per slot, until none reads zero; the maximum of what it then holds is the row's, which
+ * the other wavefronts receive through LDS behind a barrier. Stores and polls are device-scope
+ * atomics (plain stores and loads, no read-modify-write: the slots of a row share a few cache
+ * lines, and contended atomic updates of one line are what would make this wait slow), so no
+ * fence is needed. An atomic of the caller's that the row's other workgroups must find
+ * performed when they leave the wait has to have returned before the reporter gets here.
  *
  * A workgroup waits only for workgroups of its own row. The grid is dealt out so that a row's
  * workgroups have neighbouring ids and are started together; the wait is bounded all the same:
@@ -173,29 +208,27 @@ struct FusedScan {
  * itself by reading the whole row, so every workgroup ends whatever the others do. */
 template <int NV, bool PEN>
 __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, int chunk,
-                                                  int n_rows, uint64_t mine, uint32_t prior,
+                                                  int n_rows, uint64_t mine, bool reporter,
                                                   const FusedScan &fs, uint32_t *s_cnt16) {
     static_assert(MAX_CHUNKS <= 2 * WAVE, "two slots per polling lane");
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
     const int C   = rv.n_chunks;
     uint64_t *row_slots = fs.slots + (long) row * C;
-    if (tid < WAVE) {
-        if (tid == 0) {
-            uint64_t v = mine;
-            asm volatile("" : "+v"(v) : "v"(prior));
-            __hip_atomic_store(row_slots + chunk, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    if (reporter) { /* one wavefront, all its lanes */
+        if (lane == 0)
+            __hip_atomic_store(row_slots + chunk, mine, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
         uint64_t a = 0, b = 0;
         uint32_t polls = 0;
         bool     met   = fs.wait_limit != 0;
         while (met) {
-            a = tid < C ? __hip_atomic_load(row_slots + tid, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT)
-                        : 0;
-            b = tid + WAVE < C ? __hip_atomic_load(row_slots + tid + WAVE, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT)
-                               : 0;
-            const bool missing = (tid < C && a == 0) || (tid + WAVE < C && b == 0);
+            a = lane < C ? __hip_atomic_load(row_slots + lane, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT)
+                         : 0;
+            b = lane + WAVE < C ? __hip_atomic_load(row_slots + lane + WAVE, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT)
+                                : 0;
+            const bool missing = (lane < C && a == 0) || (lane + WAVE < C && b == 0);
             if (__builtin_amdgcn_ballot_w64(missing) == 0)
                 break;
             if (++polls > fs.wait_limit)
@@ -205,12 +238,11 @@ __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, in
         }
         /* 1 is never a packed value: a row's first index is below 2^32 - 2 */
         const uint64_t got = met ? wave_max_u64(a > b ? a : b) : 1;
-        if (tid == 0)
+        if (lane == 0)
             *fs.s_bb = got;
     }
     __syncthreads();
     uint64_t bb = *fs.s_bb;
-    __syncthreads();
     if (bb != 1)
         return bb;
     /* not met: the row's maximum from the row itself, 1024 elements at a time */
@@ -245,7 +277,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
                                              const int32_t *__restrict__ probe_token, int probe_L,
                                              float *__restrict__ probe_p, const CandSpace &list,
                                              int zb_list, uint32_t *s_cnt16, double *s_sum,
-                                             const uint64_t *s_tab, int *s_listed, int *s_base,
+                                             uint64_t *s_tab, uint64_t tabv, double *s_tr,
                                              const FusedScan &fs) {
     const int tid = threadIdx.x;
     /* Order of the loads: the probed token, the history, then the chunk. The groups of the
@@ -278,8 +310,10 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     } else {
         load_raw<NV>(rv, rowp, base, end, v);
     }
-    if (LISTM && tid == 0)
-        *s_listed = 0;
+    if (tid < 32)
+        s_tab[tid] = tabv;
+    if (tid < 2)
+        fs.s_arrive[tid] = 0;
     if (PEN) {
         history_clear<NV * TPB * 4>(s_cnt16);
         history_count(rv, row, pf, base, end, s_cnt16);
@@ -300,33 +334,32 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
         if (base + 4 * tid >= end)
             tm = __builtin_nanf("");
         fs.tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
-        const uint32_t mykey = f2key(tm);
-        uint32_t       bk    = wave_max_u32(mykey);
-        bk = (uint32_t) (block_max_u64((uint64_t) bk, fs.s_red));
-        uint64_t best = 0;
-        if (mykey == bk) {
-            int first = 0x7fffffff;
-#pragma unroll
-            for (int j = NV - 1; j >= 0; --j) {
-                const int e = base + 4 * (j * TPB + tid);
-#pragma unroll
-                for (int c = 3; c >= 0; --c)
-                    if (e + c < end && f2key(f4_get(v[j], c)) == bk)
-                        first = e + c;
-            }
-            if (first != 0x7fffffff)
-                best = pack_best(bk, (uint32_t) first);
-        }
-        best = block_max_u64(best, fs.s_red);
-        if (!best) /* an all-NaN chunk reports key 0 at its first index */
-            best = pack_best(0u, (uint32_t) base);
+        /* the wavefront's best, then the chunk's: each wavefront deposits its own in LDS and
+         * the one that arrives last (no barrier: the others need not wait for it) combines
+         * them, reports the chunk's and waits for the row's */
+        const uint32_t bk   = wave_max_u32(f2key(tm));
+        uint64_t       best = wave_first_of<NV, PLAIN>(v, bk, base, end);
         uint32_t prior = 0;
-        if (tid == 0) {
-            fs.chunk_best[(long) row * rv.n_chunks + chunk] = best;
-            if (LISTM && chunk == 0) /* the list the second half appends to starts empty */
-                prior = (uint32_t) atomicExch(&list.count[row], 0);
+        if (LISTM && chunk == 0 && tid == 0) /* the list the second half appends to starts empty */
+            prior = (uint32_t) atomicExch(&list.count[(long) row * CAND_COUNT_STRIDE], 0);
+        if ((tid & (WAVE - 1)) == 0) {
+            /* `prior` an operand of the deposit: the exchange above has returned before this
+             * wavefront arrives, so before the chunk's slot is stored */
+            asm volatile("" : "+v"(best) : "v"(prior));
+            fs.s_red[tid / WAVE] = best;
         }
-        bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, prior, fs, s_cnt16);
+        const bool last = wave_arrives_last(fs.s_arrive);
+        if (last) {
+            best = fs.s_red[0];
+#pragma unroll
+            for (int w = 1; w < NWAVES; ++w)
+                best = fs.s_red[w] > best ? fs.s_red[w] : best;
+            if (!best) /* an all-NaN chunk reports key 0 at its first index */
+                best = pack_best(0u, (uint32_t) base);
+            if ((tid & (WAVE - 1)) == 0)
+                fs.chunk_best[(long) row * rv.n_chunks + chunk] = best;
+        }
+        bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, last, fs, s_cnt16);
     }
     const float mx = key2f(best_key(bb));
 
@@ -376,31 +409,65 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
             probe_p[row] = geist_expf_glibc_le0(softmax_arg(x, mx, inv_t), s_tab);
         }
     }
-    if (SLABS) {
-        /* the chunk's sum is the sum of its slab sums, in slab order */
-        block_sum_f64_multi<SLABS ? NV : 1>(accs, s_sum);
-        if (tid == 0) {
-            const long at = (long) row * rv.n_chunks + chunk;
+    /* The chunk's sums: wavefront totals (lane 63 of the DPP scan) deposited in LDS, combined by
+     * the wavefront that arrives last, in the order wavefront 0..3 (and slab 0..NV-1 for the
+     * chunk's sum, which is the sum of its slab sums). No barrier: a wavefront that is done
+     * leaves. */
+    {
+        const int  lane = tid & (WAVE - 1), w = tid / WAVE;
+        const long at   = (long) row * rv.n_chunks + chunk;
+        if (SLABS && NV == 8) {
+            /* eight sums over the wavefront at once, through LDS: sum j of lane l goes to place
+             * [j][l] of the wavefront's 8 x 64 table, then lane l adds the eight entries
+             * [l / 8][8 (l % 8) ..] in order and three DPP steps add up the eight lanes of a
+             * group: lane 8 j + 7 ends with sum j. (Eight DPP reductions one after the other
+             * took as long as a third of the exponentials.) Places are swizzled by the row
+             * number, so that the lanes of a read hit different banks. */
+            volatile double *tr = s_tr + w * (8 * WAVE);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                tr[j * WAVE + (lane ^ j)] = accs[j < NV ? j : 0];
+            const int g = lane >> 3, first = 8 * (lane & 7);
+            double    r = tr[g * WAVE + (first ^ g)];
+#pragma unroll
+            for (int i = 1; i < 8; ++i)
+                r += tr[g * WAVE + ((first + i) ^ g)];
+            r += dpp_fetch_f64<0x111, 0xf>(r); /* row_shr:1, 2, 4: the lane and the seven */
+            r += dpp_fetch_f64<0x112, 0xf>(r); /* before it                               */
+            r += dpp_fetch_f64<0x114, 0xf>(r);
+            if ((lane & 7) == 7)
+                s_sum[w * NV + g] = r;
+        } else if (SLABS) {
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
-                slab_sum[at * SLABS_MAX + j] = accs[j];
-                acc += accs[j];
+                const double t = wave_scan_f64_dpp(accs[j]);
+                if (lane == WAVE - 1)
+                    s_sum[w * NV + j] = t;
             }
-            chunk_sum[at] = acc;
+        } else {
+            const double t = wave_scan_f64_dpp(acc);
+            if (lane == WAVE - 1)
+                s_sum[w] = t;
         }
-    } else {
-        acc = block_sum_f64(acc, s_sum);
-        if (tid == 0)
-            chunk_sum[(long) row * rv.n_chunks + chunk] = acc;
+        if (wave_arrives_last(fs.s_arrive + 1) && lane == 0) {
+            constexpr int NS = SLABS ? NV : 1;
+            double        total = 0.0;
+#pragma unroll
+            for (int j = 0; j < NS; ++j) {
+                double r = s_sum[j];
+#pragma unroll
+                for (int x = 1; x < NWAVES; ++x)
+                    r += s_sum[x * NS + j];
+                if (SLABS)
+                    slab_sum[at * SLABS_MAX + j] = r;
+                total += r;
+            }
+            chunk_sum[at] = total;
+        }
     }
     if (LISTM) {
-        /* places in the row's list: one LDS counter for the workgroup, one global add for all */
-        int pos = wave_reserve(__popc(mask), s_listed);
-        __syncthreads();
-        if (tid == 0)
-            *s_base = *s_listed ? atomicAdd(&list.count[row], *s_listed) : 0;
-        __syncthreads();
-        pos += *s_base;
+        /* places in the row's list: one add to the row's counter per wavefront */
+        int pos = wave_reserve(__popc(mask), &list.count[(long) row * CAND_COUNT_STRIDE]);
         uint32_t *ck = list.key + (long) row * CAND_CAP;
         uint32_t *ci = list.idx + (long) row * CAND_CAP;
 #pragma unroll
@@ -437,12 +504,19 @@ __global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
     __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ uint64_t s_red[NWAVES], s_bb;
-    __shared__ int      s_listed, s_base;
+    __shared__ uint32_t s_arrive[2];
+    /* the table the slab sums are transposed through: the history's count table has the size
+     * and is free once the row's workgroups have met */
+    __shared__ __align__(16) double s_tr_own[(SLABS && NV == 8 && !PEN) ? NWAVES * 8 * WAVE : 1];
+    static_assert(!(SLABS && NV == 8 && PEN) || sizeof(s_cnt16) >= NWAVES * 8 * WAVE * sizeof(double),
+                  "the count table holds the transposed sums");
+    double *s_tr = PEN ? reinterpret_cast<double *>(s_cnt16) : s_tr_own;
     const int tid = threadIdx.x;
     int       row, chunk;
     xcd_row_chunk(row, chunk);
-    if (tid < 32)
-        s_tab[tid] = g_expf_tab[tid];
+    /* the table's words are asked for here and put into LDS after the chunk's loads have been
+     * issued: written at once, the wait for them would stand before those loads */
+    const uint64_t tabv = g_expf_tab[tid & 31];
     /* the slots that the launch before this one used, back to zero for the launch after */
     {
         const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, n_wg = gridDim.x * gridDim.y;
@@ -458,18 +532,17 @@ __global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
     fs.wait_limit = meet.wait_limit;
     fs.s_red      = s_red;
     fs.s_bb       = &s_bb;
+    fs.s_arrive   = s_arrive;
     const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
                        rv.allowed == nullptr;
     if (plain)
         expsum_chunk<NV, PEN, LISTM, SLABS, true>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
-            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, &s_listed, &s_base,
-            fs);
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, fs);
     else
         expsum_chunk<NV, PEN, LISTM, SLABS, false>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
-            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, &s_listed, &s_base,
-            fs);
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, fs);
 }
 
 /* ============================================================================================
@@ -1292,7 +1365,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
         }
         return;
     }
-    if (a.minp_listed && a.cand.count[row] <= CAND_CAP) {
+    if (a.minp_listed && a.cand.count[(long) row * CAND_COUNT_STRIDE] <= CAND_CAP) {
         /* the exp-sum pass listed the row under the min-p bound (holding softmax arguments, not pn): the list
          * walk serves it, top-p included -- the kept prefix is the shorter of the two */
         if (tid == 0) {
@@ -1402,7 +1475,7 @@ __global__ __launch_bounds__(TPB) void k_final_sorted(RowView rv, FinalArgs a) {
             const float pn_out = (float) ((double) p_out / sum);
             a.cand.out_key[row]   = __float_as_uint(pn_out) + 1u;
             a.cand.row_bound[row] = B;
-            a.cand.count[row]     = 0;
+            a.cand.count[(long) row * CAND_COUNT_STRIDE]     = 0;
             a.row_flag[row]       = B < ZBINS - 1 ? 1 : 2;
             a.out[row]            = -1;
         }

@@ -806,7 +806,7 @@ __global__ __launch_bounds__(TPB) void k_list_candidates(RowView rv, float inv_t
     __syncthreads();
     const int n_blk = s_count;
     if (tid == 0)
-        s_base = n_blk ? atomicAdd(&cand.count[row], n_blk) : 0;
+        s_base = n_blk ? atomicAdd(&cand.count[(long) row * CAND_COUNT_STRIDE], n_blk) : 0;
     uint32_t *ck = cand.key + (long) row * CAND_CAP;
     uint32_t *ci = cand.idx + (long) row * CAND_CAP;
     if (n_blk <= LIST_STAGE) {
@@ -1125,7 +1125,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
     }
     if (flag != 1 && flag != 4 && flag != 5)
         return;
-    const int n   = cand.count[row];
+    const int n   = cand.count[(long) row * CAND_COUNT_STRIDE];
     int       tok = -1;
     double   sum  = 1.0;
     uint32_t kout = 0u;
