@@ -363,8 +363,26 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     }
     const float mx = key2f(best_key(bb));
 
+    if (tok >= base && tok < end) {
+        /* the thread that holds the probed element evaluates it by itself (before the sums, so
+         * that each group's registers are free once it has been added up) */
+        const int off = tok - base, f = off >> 2;
+        if ((f & (TPB - 1)) == tid) {
+            const int j = f / TPB;
+            float     x = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < NV; ++jj)
+                if (jj == j)
+                    x = f4_get(v[jj], off & 3);
+            probe_p[row] = geist_expf_glibc_le0(softmax_arg(x, mx, inv_t), s_tab);
+        }
+    }
+    /* SLABS with eight groups: a group's sum goes straight into the table through which the
+     * wavefront's eight sums are transposed (below), so no sum stays in a register */
+    constexpr bool TRANSPOSED = SLABS && NV == 8;
+    volatile double *tr = s_tr + (tid / WAVE) * (8 * WAVE);
     double      acc  = 0.0;
-    double      accs[SLABS ? NV : 1];
+    double      accs[SLABS && !TRANSPOSED ? NV : 1];
     uint32_t    mask = 0u;
     const float list_thr = zbin_threshold(zb_list); /* zbin(arg) <= zb_list */
     /* positions at or beyond `end` hold -inf (load_raw): they weigh exactly 0 and land in no
@@ -380,7 +398,9 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
             if (LISTM)
                 mask |= (uint32_t) (arg > list_thr) << (4 * j + c);
         }
-        if (SLABS)
+        if (TRANSPOSED)
+            tr[j * WAVE + ((tid & (WAVE - 1)) ^ j)] = a4;
+        else if (SLABS)
             accs[j] = a4;
         else
             acc += a4;
@@ -388,25 +408,15 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
          * compiler interleaves all 4 * NV of them and the registers that takes cost most of the
          * occupancy. The empty asm ties the next group's inputs to this group's sum. */
         if (j + 1 < NV) {
-            if (SLABS)
+            if (TRANSPOSED)
+                asm volatile("" : "+v"(a4), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
+                                  "+v"(v[j + 1].z), "+v"(v[j + 1].w));
+            else if (SLABS)
                 asm volatile("" : "+v"(accs[j]), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
                                   "+v"(v[j + 1].z), "+v"(v[j + 1].w));
             else
                 asm volatile("" : "+v"(acc), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
                                   "+v"(v[j + 1].z), "+v"(v[j + 1].w));
-        }
-    }
-    if (tok >= base && tok < end) {
-        /* the thread that holds the probed element evaluates it once more */
-        const int off = tok - base, f = off >> 2;
-        if ((f & (TPB - 1)) == tid) {
-            const int j = f / TPB;
-            float     x = 0.0f;
-#pragma unroll
-            for (int jj = 0; jj < NV; ++jj)
-                if (jj == j)
-                    x = f4_get(v[jj], off & 3);
-            probe_p[row] = geist_expf_glibc_le0(softmax_arg(x, mx, inv_t), s_tab);
         }
     }
     /* The chunk's sums: wavefront totals (lane 63 of the DPP scan) deposited in LDS, combined by
@@ -416,17 +426,13 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     {
         const int  lane = tid & (WAVE - 1), w = tid / WAVE;
         const long at   = (long) row * rv.n_chunks + chunk;
-        if (SLABS && NV == 8) {
-            /* eight sums over the wavefront at once, through LDS: sum j of lane l goes to place
-             * [j][l] of the wavefront's 8 x 64 table, then lane l adds the eight entries
+        if (TRANSPOSED) {
+            /* eight sums over the wavefront at once, through LDS: sum j of lane l went to place
+             * [j][l] of the wavefront's 8 x 64 table, now lane l adds the eight entries
              * [l / 8][8 (l % 8) ..] in order and three DPP steps add up the eight lanes of a
              * group: lane 8 j + 7 ends with sum j. (Eight DPP reductions one after the other
              * took as long as a third of the exponentials.) Places are swizzled by the row
              * number, so that the lanes of a read hit different banks. */
-            volatile double *tr = s_tr + w * (8 * WAVE);
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                tr[j * WAVE + (lane ^ j)] = accs[j < NV ? j : 0];
             const int g = lane >> 3, first = 8 * (lane & 7);
             double    r = tr[g * WAVE + (first ^ g)];
 #pragma unroll
@@ -440,7 +446,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
         } else if (SLABS) {
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
-                const double t = wave_scan_f64_dpp(accs[j]);
+                const double t = wave_scan_f64_dpp(accs[TRANSPOSED ? 0 : j]);
                 if (lane == WAVE - 1)
                     s_sum[w * NV + j] = t;
             }
@@ -1788,8 +1794,9 @@ void launch_spec(const Launch &L, const SpecLaunch &sp) {
     a.n_accepted = sp.n_accepted;
     const dim3   block(TPB);
     SpecVerdict *vd = static_cast<SpecVerdict *>(sp.verdict);
-    k_spec_accept<<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
-    if (!sp.greedy) {
+    if (sp.greedy) {
+        k_spec_accept<<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
+    } else {
         const dim3 grid(L.rv.n_chunks, sp.n_seq);
         if (L.nv == 8)
             k_spec_resid<8><<<grid, block, 0, L.stream>>>(L.rv, a, vd);

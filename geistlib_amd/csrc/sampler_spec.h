@@ -12,9 +12,10 @@
  *   j* = L : token ~ p_L, the temperature sampler's walk (sampler.c:90-102) with u_L.
  *
  * Kernels (after k_scan_expsum over all n_seq * (L+1) target rows):
- *   k_spec_accept  grid (n_seq): row sums and maxima, j*, the accepted ids and their count
- *   k_spec_resid   grid (chunks, n_seq): sums max(0, p - q) over its chunk of row j*
+ *   k_spec_resid   grid (chunks, n_seq): row sums and maxima, j*, the accepted ids and their
+ *                  count (spec_accept_seq), then the sum of max(0, p - q) over its chunk of row j*
  *   k_spec_final   grid (n_seq): draws the last token
+ *   k_spec_accept  grid (n_seq): the verdicts alone, for the greedy mode (no residual)
  */
 #ifndef GEIST_SAMPLER_SPEC_H
 #define GEIST_SAMPLER_SPEC_H
@@ -41,7 +42,7 @@ struct SpecArgs {
 
 constexpr int SPEC_L_MAX = 63;
 
-/* What k_spec_accept leaves per sequence for the two kernels behind it. */
+/* The outcome of the acceptance test of one sequence (spec_accept_seq). */
 struct SpecVerdict {
     double sum;   /* exp-sum of target row j* */
     float  mx;    /* its maximum */
@@ -51,14 +52,23 @@ struct SpecVerdict {
 };
 static_assert(sizeof(SpecVerdict) == SPEC_VERDICT_BYTES, "workspace is sized by the constant");
 
-/* ---- k_spec_accept --------------------------------------------------------------------------- */
-/* One workgroup per sequence. Groups of 16 lanes each take one target row: the lanes share the
+/* ---- the acceptance test --------------------------------------------------------------------- */
+/* By one workgroup, for one sequence. Groups of 16 lanes each take one target row: the lanes share the
  * row's chunks, partial maxima / sums are combined inside the group in a fixed order (DPP row
  * steps). Then lane j of the first wavefront tests position j and a ballot gives j*. */
-__global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, SpecVerdict *verdict) {
-    __shared__ double   s_sum[SPEC_L_MAX + 1];
-    __shared__ uint64_t s_best[SPEC_L_MAX + 1];
-    const int seq = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks, L = a.L;
+struct SpecAcceptShared {
+    double      sum[SPEC_L_MAX + 1];
+    uint64_t    best[SPEC_L_MAX + 1];
+    SpecVerdict vd;
+};
+/* The verdict of sequence `seq`, to every thread of the workgroup. `publish`: this workgroup is
+ * the one that writes the accepted ids, their count and the verdict for the kernels behind. */
+__device__ __forceinline__ SpecVerdict spec_accept_seq(const RowView &rv, const SpecArgs &a, int seq,
+                                                       SpecAcceptShared &sh, bool publish,
+                                                       SpecVerdict *verdict) {
+    double   *s_sum  = sh.sum;
+    uint64_t *s_best = sh.best;
+    const int tid = threadIdx.x, C = rv.n_chunks, L = a.L;
     const int part = tid & 15;
     for (int j = tid >> 4; j <= L; j += TPB / 16) {
         const long row = (long) seq * (L + 1) + j;
@@ -95,8 +105,7 @@ __global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, Spe
         }
     }
     __syncthreads();
-    if (tid >= WAVE)
-        return;
+    if (tid < WAVE) {
     bool ok = true; /* lanes at or beyond L never reject */
     if (tid < L) {
         const long row = (long) seq * (L + 1) + tid;
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, Spe
     }
     const uint64_t rej = __ballot(!ok);
     const int      js  = rej ? __ffsll((long long) rej) - 1 : L;
-    if (tid < js)
+    if (publish && tid < js)
         a.out_tokens[(long) seq * (L + 1) + tid] = a.draft[(long) seq * L + tid];
     if (tid == 0) {
         const long  row   = (long) seq * (L + 1) + js;
@@ -127,28 +136,42 @@ __global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, Spe
         v.js   = js;
         v.amax = (first != first) ? 0 : (int) best_idx(s_best[js]);
         v.pad  = 0;
-        verdict[seq]      = v;
-        a.n_accepted[seq] = js;
+        sh.vd  = v;
+        if (publish) {
+            verdict[seq]      = v;
+            a.n_accepted[seq] = js;
+        }
     }
+    }
+    __syncthreads();
+    return sh.vd;
+}
+
+/* the verdicts alone: the greedy mode, which has no residual pass */
+__global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, SpecVerdict *verdict) {
+    __shared__ SpecAcceptShared sh;
+    (void) spec_accept_seq(rv, a, (int) blockIdx.x, sh, true, verdict);
 }
 
 /* ---- k_spec_resid ---------------------------------------------------------------------------- */
 template <int NV>
-__global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a,
-                                                    const SpecVerdict *__restrict__ verdict) {
+__global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a, SpecVerdict *verdict) {
     __shared__ double   s_sum[NWAVES * NV];
     __shared__ uint64_t s_tab[32];
     const int seq = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 32)
         s_tab[tid] = g_expf_tab[tid];
-    const SpecVerdict vd = verdict[seq];
+    /* every workgroup of the sequence works out the verdict for itself (a few hundred chunk
+     * results from L2: cheaper than a kernel of its own in front of this one); the first one
+     * leaves it for k_spec_final */
+    __shared__ SpecAcceptShared s_acc;
+    const SpecVerdict vd = spec_accept_seq(rv, a, seq, s_acc, chunk == 0, verdict);
     const int         js = vd.js;
     if (a.greedy || js >= a.L)
         return; /* nothing to resample from */
     const long   row = (long) seq * (a.L + 1) + js;
     const float  mx  = vd.mx;
     const double sum = vd.sum;
-    __syncthreads();
     int          base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4       v[NV], qv[NV];
