@@ -324,8 +324,115 @@ __global__ __launch_bounds__(Q6K_TPB) void k_q6k_pack(const uint8_t *__restrict_
     base[3328 + r] = o[52];
 }
 
+/* six of a lane's 16-byte pieces of a packed block, from piece p0 on: 24 dwords, the six-bit
+ * values of half a block */
+__device__ __forceinline__ void q6k_packed_load6(const uint32_t *__restrict__ base, int r, int p0,
+                                                 uint32_t (&q)[24]) {
+#pragma unroll
+    for (int p = 0; p < 6; ++p) {
+        typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+        const nt_u4 t = __builtin_nontemporal_load(
+            reinterpret_cast<const nt_u4 *>(base + (p0 + p) * 256 + 4 * r));
+        q[4 * p] = t.x, q[4 * p + 1] = t.y, q[4 * p + 2] = t.z, q[4 * p + 3] = t.w;
+    }
+}
+/* the sixteen scales (four dwords) and d of a lane's block */
+__device__ __forceinline__ void q6k_packed_load_scales(const uint32_t *__restrict__ base, int r,
+                                                       uint32_t (&sc)[4], uint32_t &d52) {
+    typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+    const nt_u4 t =
+        __builtin_nontemporal_load(reinterpret_cast<const nt_u4 *>(base + 12 * 256 + 4 * r));
+    sc[0] = t.x, sc[1] = t.y, sc[2] = t.z, sc[3] = t.w;
+    d52   = __builtin_nontemporal_load(base + 3328 + r);
+}
+/* acc[m] += the 128 products of half a block with activation row m, one after the other in
+ * index order; `q` the half's six-bit values, `sc_lo`, `sc_hi` its eight scales, `x0` the
+ * half's first activation of row 0 */
 template <int MT>
-__global__ __launch_bounds__(Q6K_TPB) void k_q6k_packed_linear(const uint32_t *__restrict__ packed,
+__device__ __forceinline__ void q6k_packed_half(uint32_t (&q)[24], uint32_t sc_lo,
+                                                uint32_t sc_hi, float dd,
+                                                const double *__restrict__ x0, int n_m, int n_in,
+                                                double (&acc)[MT]) {
+#pragma unroll
+    for (int g16 = 0; g16 < 8; ++g16) { /* eight scale groups, in element order */
+        const int    sc = (int) (int8_t) ((g16 < 4 ? sc_lo : sc_hi) >> (8 * (g16 % 4)));
+        const double ds = (double) (dd * (float) sc), m32ds = -32.0 * ds;
+        const double *xg = x0 + 16 * g16;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int bit = 6 * (16 * g16 + i), w0 = bit >> 5, off = bit & 31;
+            /* (straddling values: the funnel shift's low six bits) */
+            const uint32_t v  = off <= 26
+                                    ? (q[w0] >> off) & 63u
+                                    : __builtin_amdgcn_alignbit(q[w0 + 1 < 24 ? w0 + 1 : 23], q[w0],
+                                                                off) & 63u;
+            const double   wv = __builtin_fma(ds, (double) v, m32ds);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const double *xm = xg + (long) (m < n_m ? m : n_m - 1) * n_in;
+                acc[m] = __builtin_fma(xm[i], wv, acc[m]); /* uniform address */
+            }
+        }
+        /* one scale group at a time: left alone the scheduler converts far ahead and runs out of
+         * registers. The empty asm makes the next group's three dwords wait for this group's
+         * sum. */
+        if (g16 + 1 < 8) {
+            asm volatile("" : "+v"(acc[0]), "+v"(q[3 * g16 + 3]), "+v"(q[3 * g16 + 4]),
+                              "+v"(q[3 * g16 + 5]));
+        }
+    }
+}
+
+template <int MT>
+__global__ __launch_bounds__(Q6K_TPB, 4) void k_q6k_packed_linear(const uint32_t *__restrict__ packed,
+                                                               long n_out, int n_in,
+                                                               const double *__restrict__ xd,
+                                                               int n_m, float *__restrict__ y,
+                                                               long ld_y) {
+    const int  r = threadIdx.x & 63;
+    const long g = (long) blockIdx.x * (Q6K_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long row = g * 64 + r;
+    const int  nb  = n_in / Q6K_BLOCK_ELEMS;
+    double     acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m] = 0.0;
+    /* Loads run half a block ahead of the arithmetic (a wavefront has few neighbours on its SIMD
+     * to cover a wait: the whole table is 4 wavefronts per SIMD): a block's second half is asked
+     * for when its first half is about to be added up, the next block's first half and scales
+     * when this block's second half is. */
+    const uint32_t *base = packed + g * nb * Q6K_PACK_DWORDS;
+    uint32_t        qa[24], qb[24], sc[4], d52;
+    q6k_packed_load_scales(base, r, sc, d52);
+    q6k_packed_load6(base, r, 0, qa);
+    for (int b = 0; b < nb; ++b) {
+        const uint32_t *blk = base + (long) b * Q6K_PACK_DWORDS;
+        const double   *x0  = xd + (long) b * Q6K_BLOCK_ELEMS;
+        q6k_packed_load6(blk, r, 6, qb);
+        const float    dd  = __half2float(__ushort_as_half((unsigned short) (d52 & 0xffffu)));
+        const uint32_t sc2 = sc[2], sc3 = sc[3];
+        q6k_packed_half<MT>(qa, sc[0], sc[1], dd, x0, n_m, n_in, acc);
+        if (b + 1 < nb) {
+            q6k_packed_load_scales(blk + Q6K_PACK_DWORDS, r, sc, d52);
+            q6k_packed_load6(blk + Q6K_PACK_DWORDS, r, 0, qa);
+        }
+        q6k_packed_half<MT>(qb, sc2, sc3, dd, x0 + 128, n_m, n_in, acc);
+    }
+    if (row < n_out) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m < n_m)
+                y[m * ld_y + row] = (float) acc[m];
+    }
+}
+
+/* Several activation rows at once: a block at a time, every weight converted once and used for
+ * each row (the scalar registers that hold the rows' activations leave no room for running the
+ * loads ahead). */
+template <int MT>
+__global__ __launch_bounds__(Q6K_TPB) void k_q6k_packed_linear_rows(const uint32_t *__restrict__ packed,
                                                                long n_out, int n_in,
                                                                const double *__restrict__ xd,
                                                                int n_m, float *__restrict__ y,
@@ -403,8 +510,8 @@ void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out
     const uint32_t *p = static_cast<const uint32_t *>(packed);
     switch (n_m) {
     case 1: k_q6k_packed_linear<1><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
-    case 2: k_q6k_packed_linear<2><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
-    default: k_q6k_packed_linear<4><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    case 2: k_q6k_packed_linear_rows<2><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    default: k_q6k_packed_linear_rows<4><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
     }
 }
 
