@@ -180,6 +180,7 @@ __device__ __forceinline__ uint64_t wave_first_of(const float4 (&v)[NV], uint32_
 
 /* Where the thread maxima and the chunk results go, and the slots through which the workgroups
  * of a row meet. */
+constexpr uint32_t SCAN_STAGE = 2048; /* candidates a workgroup stages in LDS */
 struct FusedScan {
     float    *tmax;
     uint64_t *chunk_best;
@@ -187,7 +188,8 @@ struct FusedScan {
     uint32_t  wait_limit;
     uint64_t *s_red;    /* LDS, NWAVES words */
     uint64_t *s_bb;     /* LDS, one word */
-    uint32_t *s_arrive; /* LDS, two arrival counters, zero and published before use */
+    uint32_t *s_arrive; /* LDS, three arrival counters (and a fourth word), zero and published
+                         * before use */
 };
 
 /* The row's maximum (packed with its first index) once every chunk of the row has reported its
@@ -278,6 +280,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
                                              float *__restrict__ probe_p, const CandSpace &list,
                                              int zb_list, uint32_t *s_cnt16, double *s_sum,
                                              uint64_t *s_tab, uint64_t tabv, double *s_tr,
+                                             uint2 *s_stage, uint32_t *s_nstage,
                                              const FusedScan &fs) {
     const int tid = threadIdx.x;
     /* Order of the loads: the probed token, the history, then the chunk. The groups of the
@@ -312,7 +315,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     }
     if (tid < 32)
         s_tab[tid] = tabv;
-    if (tid < 2)
+    if (tid < 4) /* three arrival counters and the staging list's length */
         fs.s_arrive[tid] = 0;
     if (PEN) {
         history_clear<NV * TPB * 4>(s_cnt16);
@@ -383,20 +386,37 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     volatile double *tr = s_tr + (tid / WAVE) * (8 * WAVE);
     double      acc  = 0.0;
     double      accs[SLABS && !TRANSPOSED ? NV : 1];
-    uint32_t    mask = 0u;
     const float list_thr = zbin_threshold(zb_list); /* zbin(arg) <= zb_list */
     /* positions at or beyond `end` hold -inf (load_raw): they weigh exactly 0 and land in no
      * bin, so the loop carries no bound tests */
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         double a4;
+        float  args[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const float  arg = softmax_arg(f4_get(v[j], c), mx, inv_t);
-            const double p   = (double) geist_expf_glibc_le0(arg, s_tab);
-            a4               = c == 0 ? p : a4 + p;
-            if (LISTM)
-                mask |= (uint32_t) (arg > list_thr) << (4 * j + c);
+            args[c]        = softmax_arg(f4_get(v[j], c), mx, inv_t);
+            const double p = (double) geist_expf_glibc_le0(args[c], s_tab);
+            a4             = c == 0 ? p : a4 + p;
+        }
+        if (LISTM) {
+            /* the group's candidates go to the workgroup's staging list in LDS right away (the
+             * softmax argument and the id; the list walk takes the exponential of the few
+             * hundred entries it reads), so that the group's registers are free afterwards */
+            const bool c0 = args[0] > list_thr, c1 = args[1] > list_thr, c2 = args[2] > list_thr,
+                       c3 = args[3] > list_thr;
+            if (__builtin_amdgcn_ballot_w64(c0 || c1 || c2 || c3)) {
+                const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (c == 0 ? c0 : c == 1 ? c1 : c == 2 ? c2 : c3) {
+                        const uint32_t at = __hip_atomic_fetch_add(
+                            s_nstage, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        if (at < SCAN_STAGE)
+                            s_stage[at] = make_uint2(__float_as_uint(args[c]), (uint32_t) (e + c));
+                    }
+                }
+            }
         }
         if (TRANSPOSED)
             tr[j * WAVE + ((tid & (WAVE - 1)) ^ j)] = a4;
@@ -472,24 +492,25 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
         }
     }
     if (LISTM) {
-        /* places in the row's list: one add to the row's counter per wavefront */
-        int pos = wave_reserve(__popc(mask), &list.count[(long) row * CAND_COUNT_STRIDE]);
-        uint32_t *ck = list.key + (long) row * CAND_CAP;
-        uint32_t *ci = list.idx + (long) row * CAND_CAP;
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int e = base + 4 * (j * TPB + tid);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if ((mask >> (4 * j + c)) & 1u) {
-                    if (pos < CAND_CAP) {
-                        /* the softmax argument; the list walk takes the exponential of the few
-                         * hundred entries it reads (here it would run under divergence, once
-                         * per listed element for the whole wavefront) */
-                        ck[pos] = __float_as_uint(softmax_arg(f4_get(v[j], c), mx, inv_t));
-                        ci[pos] = (uint32_t) (e + c);
-                    }
-                    ++pos;
+        /* the wavefront that arrives last moves the staged entries to the row's list: one add to
+         * the row's counter per workgroup. A workgroup with more candidates than the staging
+         * list holds reports more than the row's list can hold, which sends the row to the
+         * whole-row walk. */
+        if (wave_arrives_last(fs.s_arrive + 2)) {
+            const int      lane  = tid & (WAVE - 1);
+            const uint32_t n     = *s_nstage;
+            const uint32_t total = n > SCAN_STAGE ? (uint32_t) CAND_CAP + 1u : n;
+            int            at    = 0;
+            if (lane == 0 && total)
+                at = atomicAdd(&list.count[(long) row * CAND_COUNT_STRIDE], (int) total);
+            at = __builtin_amdgcn_readfirstlane(at);
+            uint32_t *ck = list.key + (long) row * CAND_CAP;
+            uint32_t *ci = list.idx + (long) row * CAND_CAP;
+            for (uint32_t i = lane; i < n && i < SCAN_STAGE; i += WAVE) {
+                const uint2 t = s_stage[i];
+                if (at + (int) i < CAND_CAP) {
+                    ck[at + i] = t.x;
+                    ci[at + i] = t.y;
                 }
             }
         }
@@ -505,12 +526,17 @@ __global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
                                                      const int32_t *__restrict__ probe_token,
                                                      int probe_L, float *__restrict__ probe_p,
                                                      CandSpace list, int zb_list, MeetSpace meet) {
-    static_assert(!LISTM || 4 * NV <= 32, "one mask bit per element of a thread");
+    
     __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
     __shared__ double   s_sum[SLABS ? NWAVES * NV : NWAVES];
     __shared__ uint64_t s_tab[32];
     __shared__ uint64_t s_red[NWAVES], s_bb;
-    __shared__ uint32_t s_arrive[2];
+    __shared__ uint32_t s_arrive[4];
+    /* the staging list of the candidates: in the history's count table when there is one */
+    __shared__ uint2 s_stage_own[(LISTM && !PEN) ? SCAN_STAGE : 1];
+    static_assert(!(LISTM && PEN) || sizeof(s_cnt16) >= SCAN_STAGE * sizeof(uint2),
+                  "the count table holds the staging list");
+    uint2 *s_stage = PEN ? reinterpret_cast<uint2 *>(s_cnt16) : s_stage_own;
     /* the table the slab sums are transposed through: the history's count table has the size
      * and is free once the row's workgroups have met */
     __shared__ __align__(16) double s_tr_own[(SLABS && NV == 8 && !PEN) ? NWAVES * 8 * WAVE : 1];
@@ -544,11 +570,13 @@ __global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
     if (plain)
         expsum_chunk<NV, PEN, LISTM, SLABS, true>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
-            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, fs);
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
+            s_arrive + 3, fs);
     else
         expsum_chunk<NV, PEN, LISTM, SLABS, false>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
-            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, fs);
+            probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
+            s_arrive + 3, fs);
 }
 
 /* ============================================================================================
