@@ -283,6 +283,10 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
                                              uint2 *s_stage, uint32_t *s_nstage,
                                              const FusedScan &fs) {
     const int tid = threadIdx.x;
+    /* with penalties the work before the meet is long, and the row's other workgroups wait for
+     * it: it is issued ahead of the exponentials of workgroups that have met */
+    if (PEN)
+        __builtin_amdgcn_s_setprio(3);
     /* Order of the loads: the probed token, the history, then the chunk. The groups of the
      * chunk are transformed one by one, each as soon as its own load has arrived: a barrier
      * with a full fence, or a transform over the whole chunk first, would keep the arithmetic
@@ -364,6 +368,8 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
         }
         bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, last, fs, s_cnt16);
     }
+    if (PEN)
+        __builtin_amdgcn_s_setprio(0);
     const float mx = key2f(best_key(bb));
 
     if (tok >= base && tok < end) {
