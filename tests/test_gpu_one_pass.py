@@ -101,3 +101,36 @@ def test_spec_verify_one_pass(hs, oracle, wait_limit):
             want_n, want = oracle.spec_verify(target[s], q[s], draft[s], u[s], T)
             assert nacc[s] == want_n, (call, s)
             assert out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), (call, s)
+
+
+@pytest.mark.parametrize("pen", [False, True])
+def test_min_p_lists_of_every_size(hs, oracle, pen):
+    """The exp-sum pass stages a chunk's min-p candidates in LDS (2048 places per chunk): rows whose
+    candidates are a handful per chunk, rows with about a thousand in one chunk, and rows with more
+    than a chunk can stage (which the pass must report as not listed, so that the whole row is
+    walked) all give the oracle's ids."""
+    rows, n = 6, 40000
+    g = np.random.default_rng(31 + pen)
+    x = (g.standard_normal((rows, n)) * 2.0).astype(np.float32)
+    x[1, 9000:10000] = x[1].max() - 0.01 * g.random(1000).astype(np.float32)   # ~1000 in one chunk
+    x[2, 17000:20000] = x[2].max() + 0.5                                       # 3000 equal leaders
+    x[3, :] = np.float32(0.25)                                                 # every element
+    x[4, 8190:8194] = x[4].max() + 1.0                                         # across a chunk edge
+    u = g.random(rows).astype(np.float32)
+    kw = dict(temperature=1.0, top_p=0.95, min_p=0.05)
+    hist = hl = None
+    pk = {}
+    if pen:
+        hist, hl = history_for(g, rows, n)
+        pk = dict(rep=1.2, freq=0.4, pres=0.2)
+    for call in range(2):
+        got = run_rows(hs, torch, x, u, P(**kw, **pk), history=hist, history_len=hl)
+        res = []
+        for r in range(rows):
+            row = oracle.penalties(x[r], hist[r, :hl[r]], 1.2, 0.4, 0.2) if pen else x[r]
+            res.append(oracle.chain_u(row, float(u[r]), **kw))
+        near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"call {call}")
+        assert near <= 1
+        paths = hs.row_paths(rows)
+        assert paths[0] == 2 and paths[1] == 2, paths     # listed
+        assert paths[2] == 3 and paths[3] == 3, paths     # more than a chunk stages: whole row
