@@ -188,10 +188,10 @@ constexpr size_t STATIC_CSUM  = STATIC_BEST + STATIC_UNITS * 8;        /* double
 constexpr size_t STATIC_SLAB  = STATIC_CSUM + STATIC_UNITS * 8;        /* double[units][8]    */
 constexpr size_t STATIC_ROW_WAVES = STATIC_UNITS + 512;            /* (row, wavefront) pairs */
 constexpr size_t STATIC_WCANDS = STATIC_SLAB + STATIC_UNITS * 8 * 8;   /* WaveCands           */
-constexpr size_t STATIC_MEET   = STATIC_WCANDS + STATIC_ROW_WAVES * 648; /* u64 [2][units]: the
-                                                                            meeting slots, zero
-                                                                            when loaded */
-constexpr size_t STATIC_BYTES  = STATIC_MEET + 2 * STATIC_UNITS * 8;
+constexpr size_t STATIC_MEET   = STATIC_WCANDS + STATIC_ROW_WAVES * 648; /* u64 [2][2 units]:
+                                                                            the meeting slots,
+                                                                            zero when loaded */
+constexpr size_t STATIC_BYTES  = STATIC_MEET + 2 * 2 * STATIC_UNITS * 8;
 static_assert(STATIC_MEET % 16 == 0, "64-bit atomics");
 static_assert(STATIC_WCANDS % 16 == 0, "float4 slots");
 constexpr int    STATIC_MAX_DEVICES = 64;
@@ -271,10 +271,11 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_best, rc * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **) &s->chunk_sum, rc * sizeof(double));
     for (int t = 0; t < 2; ++t) {
-        if (e == hipSuccess) e = hipMalloc((void **) &s->meet_own.slots[t], rc * sizeof(uint64_t));
-        if (e == hipSuccess) e = hipMemsetAsync(s->meet_own.slots[t], 0, rc * sizeof(uint64_t), s->stream);
+        /* two words per (row, chunk): the one-kernel temperature draw meets twice */
+        if (e == hipSuccess) e = hipMalloc((void **) &s->meet_own.slots[t], 2 * rc * sizeof(uint64_t));
+        if (e == hipSuccess) e = hipMemsetAsync(s->meet_own.slots[t], 0, 2 * rc * sizeof(uint64_t), s->stream);
     }
-    s->meet_own.capacity = (uint32_t) rc;
+    s->meet_own.capacity = (uint32_t) (2 * rc);
     if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->slab_sum, rc * 8 * sizeof(double));
@@ -428,10 +429,10 @@ static int check_call(geist_hip_sampler *s, const struct geist_hip_rows *rows,
     return make_launch(s, rows, params, !rs.greedy, L);
 }
 
-/* The meeting slots for a launch of rows * n_chunks workgroups: this launch takes the array
- * whose turn it is, which the launch before left zero, and zeroes what that launch used in the
- * other. */
-static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L) {
+/* The meeting slots for a launch of rows * n_chunks workgroups (`words` per workgroup): this
+ * launch takes the array whose turn it is, which the launch before left zero, and zeroes what
+ * that launch used in the other. */
+static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t words = 1) {
     MeetState &st = *s->meet;
     if (st.suspect) { /* only after a failed launch: start again from two zeroed arrays */
         for (int t = 0; t < 2; ++t)
@@ -444,7 +445,7 @@ static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L) {
     m.stale       = st.slots[st.turn ^ 1];
     m.stale_count = st.used[st.turn ^ 1];
     m.wait_limit  = s->wait_limit;
-    st.used[st.turn]     = (uint32_t) L.rows * (uint32_t) L.rv.n_chunks;
+    st.used[st.turn]     = words * (uint32_t) L.rows * (uint32_t) L.rv.n_chunks;
     st.used[st.turn ^ 1] = 0;
     st.turn ^= 1;
     return m;
@@ -607,9 +608,20 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         return after_launch(s, "top-k");
     }
     if (!rs.use_p && !rs.use_m) {
-        *stream_kernel = "k_scan_expsum";
         Launch scan          = L;
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over the rows */
+        if (scan.nv == 2 && (size_t) scan.rows * (size_t) scan.rv.n_chunks <= 256) {
+            /* A few rows: the step is a chain of waits, not of bytes, and a second launch is a
+             * tenth of it. Scan, sums and the draw in one kernel (10.9 against 11.8 us for one
+             * row of 128256, 12.0 against 12.7 for four; from 16 rows on the two kernels are the
+             * faster form, their workgroups being smaller and gone sooner). The measuring
+             * stages cannot split it: the streaming stage is the whole step. */
+            *stream_kernel = "k_temperature_draw";
+            if (do_stream)
+                launch_temperature_draw(scan, rs.inv_t, d_uniforms, d_out, meet_space(s, scan, 2));
+            return after_launch(s, "temperature");
+        }
+        *stream_kernel = "k_scan_expsum";
         if (do_stream &&
             launch_scan_expsum(scan, rs.inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0,
                                nullptr, nullptr, 0, s->slab_sum, meet_space(s, scan)))
@@ -736,8 +748,8 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
     tmp.wcands_row_waves = STATIC_ROW_WAVES;
     MeetState &ms = g_static_meet[device];
     ms.slots[0]   = reinterpret_cast<uint64_t *>(ws + STATIC_MEET);
-    ms.slots[1]   = ms.slots[0] + STATIC_UNITS;
-    ms.capacity   = (uint32_t) STATIC_UNITS;
+    ms.slots[1]   = ms.slots[0] + 2 * STATIC_UNITS;
+    ms.capacity   = (uint32_t) (2 * STATIC_UNITS);
     tmp.meet      = &ms;
     rc = sample_impl(&tmp, rows, params, d_uniforms, d_out_tokens);
     return rc ? report(err, err_len, rc, "%s", tmp.err) : GEIST_HIP_OK;

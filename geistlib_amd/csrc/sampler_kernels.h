@@ -150,6 +150,11 @@ struct FinalLaunch {
 int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
                        double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
                        const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet);
+/* The temperature draw in one kernel (sampler_draw.h): out[row] = the id drawn with
+ * uniforms[row]. For L.nv == 2. `meet.slots` holds 2 * rows * n_chunks zeroed words: the
+ * workgroups of a row meet twice. */
+void launch_temperature_draw(const Launch &L, float inv_t, const float *uniforms, int32_t *out,
+                             const MeetSpace &meet);
 /* last z bin that can hold an entry passing min_p (with slack); ZBINS - 1 when min_p is off or
  * that deep */
 int zbin_of_min_p(float min_p);

@@ -211,7 +211,8 @@ struct FusedScan {
 template <int NV, bool PEN>
 __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, int chunk,
                                                   int n_rows, uint64_t mine, bool reporter,
-                                                  const FusedScan &fs, uint32_t *s_cnt16) {
+                                                  const FusedScan &fs, uint32_t *s_cnt16,
+                                                  bool *met_out = nullptr) {
     static_assert(MAX_CHUNKS <= 2 * WAVE, "two slots per polling lane");
     const int tid = threadIdx.x, lane = tid & (WAVE - 1);
     const int C   = rv.n_chunks;
@@ -245,6 +246,8 @@ __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, in
     }
     __syncthreads();
     uint64_t bb = *fs.s_bb;
+    if (met_out)
+        *met_out = bb != 1;
     if (bb != 1)
         return bb;
     /* not met: the row's maximum from the row itself, 1024 elements at a time */
@@ -1312,6 +1315,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 
 } // namespace gs
 #include "sampler_walk.h"
+#include "sampler_draw.h"
 #include "sampler_sorted_prob.h"
 #include "sampler_spec.h"
 #include "sampler_draft.h"
@@ -1807,6 +1811,16 @@ int zbin_of_min_p(float min_p) {
     /* pn_i >= min_p * pn_0 needs z_i <= -ln(min_p); slack for the fp32 steps in between */
     const double z_m = -std::log((double) min_p) + 2e-3;
     return z_m * ZBIN_PER_NAT < (double) (ZBINS - 1) ? (int) (z_m * ZBIN_PER_NAT) : ZBINS - 1;
+}
+
+void launch_temperature_draw(const Launch &L, float inv_t, const float *uniforms, int32_t *out,
+                             const MeetSpace &meet) {
+    /* for launches of a few rows: the geometry of 2048 elements per workgroup only */
+    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    if (L.pen)
+        k_temperature_draw<2, true><<<grid, block, 0, L.stream>>>(L.rv, inv_t, uniforms, out, meet);
+    else
+        k_temperature_draw<2, false><<<grid, block, 0, L.stream>>>(L.rv, inv_t, uniforms, out, meet);
 }
 
 void launch_spec(const Launch &L, const SpecLaunch &sp) {

@@ -134,3 +134,57 @@ def test_min_p_lists_of_every_size(hs, oracle, pen):
         paths = hs.row_paths(rows)
         assert paths[0] == 2 and paths[1] == 2, paths     # listed
         assert paths[2] == 3 and paths[3] == 3, paths     # more than a chunk stages: whole row
+
+
+@pytest.mark.parametrize("wait_limit", [None, 0, 3])
+@pytest.mark.parametrize("rows,n,pen,extra", [
+    (1, 128256, False, ""),
+    (1, 2049, False, ""),            # two chunks, the second with one element
+    (2, 50001, True, ""),            # ragged rows (not a multiple of four), penalties
+    (4, 32000, False, "softcap"),
+    (3, 32003, True, "mask"),
+    (2, 10000, False, "nan"),
+    (1, 7, False, ""),               # one workgroup: nobody to meet
+])
+def test_temperature_draw_in_one_kernel(hs, oracle, rows, n, pen, extra, wait_limit):
+    """A few rows draw by temperature in a single kernel whose workgroups meet twice (for the
+    row's maximum, then for the chunks' sums) and whose draw is walked from the registers of
+    the workgroup it falls to. Ids equal the oracle's, also when every wait is given up at once
+    (wait limit 0: every workgroup forms maximum and sums from the row itself) or early (3)."""
+    from gpu_util import pack_allowed  # noqa: F401  (run_rows packs the mask)
+    print(f"one kernel rows={rows} n={n} pen={pen} {extra} wait_limit={wait_limit}", flush=True)
+    g = np.random.default_rng(rows * 131 + n)
+    x = (g.standard_normal((rows, n)) * 2.5).astype(np.float32)
+    x[0, n // 2] = x[0].max()
+    if extra == "nan":
+        x[1, 17] = np.nan
+        x[0, 5] = -np.inf
+    cap = 5.0 if extra == "softcap" else 0.0
+    allowed = (g.random((rows, n)) < 0.3) if extra == "mask" else None
+    if allowed is not None:
+        allowed[:, 0] = True
+    hist = hl = None
+    pk = {}
+    if pen:
+        hist, hl = history_for(g, max(rows, 2), n)
+        hist, hl = hist[:rows], hl[:rows]
+        pk = dict(rep=1.2, freq=0.4, pres=0.2)
+    if wait_limit is not None:
+        hs.set_wait_limit(wait_limit)
+    T = 0.8
+    for call in range(3):                  # meeting words alternate between two arrays
+        u = g.random(rows).astype(np.float32)
+        if call == 1:
+            u[0] = np.float32(0.99999994)  # the last float below one: the end of the row
+        got = run_rows(hs, torch, x, u, P(temperature=T, softcap=cap, **pk), history=hist,
+                       history_len=hl, allowed=allowed)
+        res = []
+        for r in range(rows):
+            row = oracle.penalties(x[r], hist[r, :hl[r]], 1.2, 0.4, 0.2) if pen else x[r]
+            if cap:
+                row = oracle.softcap(row, cap)
+            if allowed is not None:
+                row = np.where(allowed[r], row, -np.inf).astype(np.float32)
+            res.append(oracle.chain_u(row, float(u[r]), temperature=T))
+        near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"call {call}")
+        assert near <= 1
