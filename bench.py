@@ -755,6 +755,14 @@ def main():
     # back-to-back launches of that kernel (same configuration), again over the rotating copies
     hs.set_logits_hint(True)
     kernel_us, kernel_name = bh.time_stream_kernel(hs, rows_cold, prm, d_u, d_out, args.steps)
+    # where the step is one launch (scan and row-final together), the scan kernel of the
+    # two-launch form on its own as well: the rate at which the logits are streamed
+    scan_alone_us = scan_alone_name = None
+    if kernel_name == "k_cand_scan_final":
+        hs.one_launch_topk(False)
+        scan_alone_us, scan_alone_name = bh.time_stream_kernel(hs, rows_cold, prm, d_u, d_out,
+                                                               args.steps)
+        hs.one_launch_topk(True)
     # calibration: a kernel that only reads the same rows with the same geometry
     plain_us = bh.time_plain_read(rows_cold, args.steps, streamed=True)
     hs.set_logits_hint(False)
@@ -776,6 +784,9 @@ def main():
     alg_bytes = w.algorithmic_bytes()
     # the streaming kernel's own share of those bytes: every logit once
     kernel_bytes = w.rows * w.n_vocab * 4
+    scan_bytes = kernel_bytes
+    if kernel_name in ("k_cand_scan_final", "k_temperature_draw"):
+        kernel_bytes = alg_bytes  # the kernel is the whole step
     achieved = kernel_bytes / (kernel_us * 1e-6) / 1e9
     result = {
         "metric": "sampled rows/s",
@@ -816,6 +827,10 @@ def main():
                      "step_algorithmic_bytes": alg_bytes,
                      "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }
+    if scan_alone_us is not None:
+        result["roofline"]["scan_kernel_of_two_launch_form"] = {
+            "kernel": scan_alone_name, "kernel_us": round(scan_alone_us, 3),
+            "frac": round(scan_bytes / (scan_alone_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
     if not args.no_cpu:
         base, ids_cpu = cpu_baseline(w)
         result["cpu_baseline"] = base

@@ -81,6 +81,7 @@ def load_library():
     lib.geist_hip_sampler_set_projection.argtypes = [vp, i32]
     lib.geist_hip_sampler_prepare.argtypes = [vp, C.POINTER(SampleParams), sz]
     lib.geist_hip_sampler_set_wait_limit.argtypes = [vp, C.c_uint32]
+    lib.geist_hip_sampler_one_launch_topk.argtypes = [vp, i32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -173,6 +174,13 @@ class HipSampler:
 
     def set_wait_limit(self, polls):
         self._check(self.lib.geist_hip_sampler_set_wait_limit(self.h, C.c_uint32(polls)))
+
+    def one_launch_topk(self, enable=True):
+        """Whether the top-k candidate path runs as one launch for batches that qualify."""
+        rc = self.lib.geist_hip_sampler_one_launch_topk(self.h, 1 if enable else 0)
+        if rc < 0:
+            self._check(rc)
+        return bool(rc)
 
     def prepare(self, params, n_vocab=0):
         """Sizes whatever workspace `params` needs beyond the sampler's own, ahead of the first

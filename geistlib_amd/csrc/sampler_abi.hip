@@ -43,6 +43,9 @@ struct geist_hip_sampler {
 
     /* device workspace */
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
+    int32_t   *row_arrive = nullptr; /* per row: how many of its workgroups have scanned (k_cand_scan_final) */
+    int        fused_wg_limit = 0;   /* largest grid that kernel is used for */
+    int        fused_wg_default = 0; /* ... as the device allows */
     MeetState  meet_own;             /* where the workgroups of the one-pass exp-sum kernel meet */
     MeetState *meet      = &meet_own; /* (the allocation-free entry point shares one per device) */
     uint32_t  wait_limit = 1u << 16; /* polls a workgroup of that kernel waits for its row */
@@ -223,6 +226,28 @@ static hipError_t static_workspace(int device, unsigned char **out) {
     return e;
 }
 
+/* Whether the device (current) places workgroups as k_cand_scan_final needs; probed on the first
+ * call per device. */
+static bool g_placement_known[STATIC_MAX_DEVICES], g_placement_same[STATIC_MAX_DEVICES];
+static hipError_t placement_of(int device, hipStream_t stream, bool *same) {
+    *same = false;
+    if (device < 0 || device >= STATIC_MAX_DEVICES)
+        return hipSuccess;
+    pthread_mutex_lock(&g_static_ws_lock);
+    hipError_t e = hipSuccess;
+    if (!g_placement_known[device]) {
+        bool ok = false;
+        e       = (hipError_t) gs::probe_workgroup_placement(stream, &ok);
+        if (e == hipSuccess) {
+            g_placement_known[device] = true;
+            g_placement_same[device]  = ok;
+        }
+    }
+    *same = g_placement_known[device] && g_placement_same[device];
+    pthread_mutex_unlock(&g_static_ws_lock);
+    return e;
+}
+
 /* ============================================================================================ */
 /* failure text into a caller's buffer (an entry point without a sampler object has no error slot) */
 static int report(char *err, size_t err_len, int code, const char *fmt, ...) {
@@ -276,6 +301,23 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
         if (e == hipSuccess) e = hipMemsetAsync(s->meet_own.slots[t], 0, 2 * rc * sizeof(uint64_t), s->stream);
     }
     s->meet_own.capacity = (uint32_t) (2 * rc);
+    if (e == hipSuccess)
+        e = hipMalloc((void **) &s->row_arrive, max_rows * ARRIVE_STRIDE_INTS * sizeof(int32_t));
+    if (e == hipSuccess)
+        e = hipMemsetAsync(s->row_arrive, 0, max_rows * ARRIVE_STRIDE_INTS * sizeof(int32_t), s->stream);
+    {
+        /* the one-launch form of the top-k candidate path hands a row over through the L2 its
+         * workgroups share: used only where the device places them as that needs (looked at
+         * once per device) */
+        int cus = 0;
+        if (e == hipSuccess)
+            e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+        bool same = false;
+        if (e == hipSuccess)
+            e = placement_of(device, s->stream, &same);
+        s->fused_wg_default = same ? cus : 0; /* one workgroup of 1024 threads per compute unit */
+        s->fused_wg_limit   = s->fused_wg_default;
+    }
     if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
     if (e == hipSuccess) e = hipMalloc((void **) &s->resid_sum, rc * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &s->slab_sum, rc * 8 * sizeof(double));
@@ -309,6 +351,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipStreamSynchronize(s->stream);
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
+    (void) hipFree(s->row_arrive);
     (void) hipFree(s->meet_own.slots[0]);
     (void) hipFree(s->meet_own.slots[1]);
     (void) hipFree(s->resid_sum);
@@ -593,6 +636,16 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
             f.row_flag         = s->row_flag; /* which path served each row, for diagnostics */
             s->topk_paths_rows = rows->rows;
             *stream_kernel     = "k_cand_scan";
+            /* a batch that fits the device in one round of 1024-thread workgroups takes both
+             * kernels in one launch (the measuring stages cannot split it: the streaming stage
+             * is the whole step) */
+            const size_t wgs = rows->rows * (size_t) ((L.rv.n_chunks + 3) / 4);
+            if (s->row_arrive && rows->rows % 8 == 0 && wgs <= (size_t) s->fused_wg_limit) {
+                *stream_kernel = "k_cand_scan_final";
+                if (do_stream)
+                    launch_cand_scan_final(scan, L, f, s->tmax, wc, m, s->row_arrive);
+                return after_launch(s, "top-k");
+            }
             if (do_stream)
                 launch_cand_scan(scan, s->tmax, wc, m);
             if (do_tail)
@@ -688,6 +741,13 @@ int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls) {
         return GEIST_HIP_E_INVALID_ARG;
     s->wait_limit = polls;
     return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->fused_wg_limit = enable ? s->fused_wg_default : 0;
+    return s->fused_wg_limit > 0 ? 1 : 0;
 }
 
 int geist_hip_sampler_prepare(geist_hip_sampler *s, const struct geist_hip_sample_params *params,

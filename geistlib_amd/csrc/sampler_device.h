@@ -444,8 +444,8 @@ __device__ __forceinline__ float4 load_streaming(const float4 *p) {
  * header). Positions at or beyond `end` hold -inf. */
 template <int NV>
 __device__ __forceinline__ void load_raw(const RowView &rv, const float *__restrict__ row,
-                                         int base, int end, float4 (&v)[NV]) {
-    const int   tid  = threadIdx.x;
+                                         int base, int end, float4 (&v)[NV],
+                                         int tid = (int) threadIdx.x) {
     const float ninf = -__builtin_inff();
     if (rv.vec_ok && end - base == NV * TPB * 4) { /* full chunk: no per-element tests */
         const float4 *p = reinterpret_cast<const float4 *>(row + base) + tid;

@@ -191,6 +191,15 @@ void launch_row_final(const Launch &L, const FinalLaunch &f);
  * kernel's) and also stores the thread maxima */
 void launch_cand_scan(const Launch &L, float *tmax, const WaveCands &wc, int m);
 void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &wc);
+/* both in one launch (k_cand_scan_final): L.rows a multiple of 8; `arrive` holds one zeroed
+ * counter per row, ARRIVE_STRIDE_INTS apart, and is left zeroed */
+constexpr int ARRIVE_STRIDE_INTS = 32;
+/* *same_xcd: workgroups of a grid whose linear ids are equal modulo 8 run on one XCD (and so
+ * share an L2), which launch_cand_scan_final relies on. Runs a small kernel and waits for it.
+ * Returns a hipError_t value. */
+int probe_workgroup_placement(hipStream_t stream, bool *same_xcd);
+void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
+                            const WaveCands &wc, int m, int32_t *arrive);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */

@@ -1928,6 +1928,52 @@ void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &w
     }
 }
 
+void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
+                            const WaveCands &wc, int m, int32_t *arrive) {
+    const FinalArgs a = final_args(f);
+    const int       per_wg = FC_THREADS / TPB; /* chunks a workgroup scans */
+    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, L.rows), block(FC_THREADS);
+    if (L.rv.n_chunks <= 16) { /* up to 64 scanning wavefronts per row */
+        if (L.pen)
+            k_cand_scan_final<8, true, false><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
+                                                                          m, a, arrive);
+        else
+            k_cand_scan_final<8, false, false><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax,
+                                                                           wc, m, a, arrive);
+    } else {
+        if (L.pen)
+            k_cand_scan_final<8, true, true><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
+                                                                         m, a, arrive);
+        else
+            k_cand_scan_final<8, false, true><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
+                                                                          m, a, arrive);
+    }
+}
+
+int probe_workgroup_placement(hipStream_t stream, bool *same_xcd) {
+    /* a grid shaped like the fused kernel's: do workgroups whose linear ids are equal modulo 8
+     * run on one XCD? */
+    const int gx = 4, gy = 64, n = gx * gy;
+    int32_t  *d  = nullptr;
+    int32_t   h[gx * gy];
+    *same_xcd    = false;
+    hipError_t e = hipMalloc((void **) &d, n * sizeof(int32_t));
+    if (e != hipSuccess)
+        return (int) e;
+    k_xcd_of_workgroups<<<dim3(gx, gy), dim3(FC_THREADS), 0, stream>>>(d);
+    e = hipMemcpyAsync(h, d, n * sizeof(int32_t), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(stream);
+    (void) hipFree(d);
+    if (e != hipSuccess)
+        return (int) e;
+    bool ok = true;
+    for (int i = 8; i < n; ++i)
+        ok = ok && h[i] == h[i & 7];
+    *same_xcd = ok;
+    return 0;
+}
+
 void launch_row_final(const Launch &L, const FinalLaunch &f) {
     const FinalArgs a = final_args(f);
     const dim3 grid(L.rows), block(TPB);

@@ -150,6 +150,15 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
  * every workgroup do that at once, which is slow and meant for tests of that path. */
 int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
 
+/* No counterpart in the reference. The top-k candidate path runs as one launch (the workgroup of
+ * a row that finishes scanning last goes on as the row's final stage) when the batch is a
+ * multiple of 8 rows, fits the device in one round of workgroups and the device places the
+ * workgroups of a row where they share a second-level cache (looked at once per device);
+ * otherwise as two launches. Results are the same either way. enable = 0 keeps to two launches,
+ * 1 returns to the default. Returns 1 when the one-launch form is in use for batches that
+ * qualify, 0 when not, negative on error. */
+int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable);
+
 /* Sizes, ahead of the first sampling call, whatever workspace the configuration needs beyond
  * what geist_hip_sampler_create made -- the reference sizes its workspace when the options are
  * applied (transformer_session_apply_opts, src/archs/transformer/forward/step.c:398-409), so that

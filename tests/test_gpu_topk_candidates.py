@@ -203,3 +203,41 @@ def test_soft_capped_rows_on_the_thread_maxima_path(oracle):
         res = [oracle.chain_u(oracle.softcap(x[r], cap), float(u[r]), **kw) for r in range(rows)]
         compare_ids(got, [t for t, _ in res], [i for _, i in res], f"soft-capped maxima k={k}")
     s.close()
+
+
+@pytest.mark.parametrize("pen", [False, True])
+def test_one_launch_and_two_launches_agree(hs, oracle, pen):
+    """The candidate path as one launch (the last workgroup of a row to finish scanning goes on
+    as the row's final stage) and as two give the oracle's ids, call after call on changing
+    rows -- what one workgroup wrote must be what another reads -- including rows that fall back
+    to the thread maxima and to the whole-row selection."""
+    n, k, rows = 128256, 40, 64
+    g = np.random.default_rng(77 + pen)
+    used = hs.one_launch_topk(True)
+    print("one launch available on this device:", used, flush=True)
+    hist = None
+    pk = {}
+    pen_t = None
+    if pen:
+        hist = g.integers(0, n, (rows, 1024)).astype(np.int32)
+        pk = dict(rep=1.1, freq=0.5, pres=0.2)
+        pen_t = (1.1, 0.5, 0.2)
+    try:
+        for call in range(4):
+            x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+            x[call] = -np.sort(-x[call])                # thread-maxima path
+            x[8 + call, :] = np.round(x[8 + call])      # runs of equal values
+            x[16 + call, :] = 0.5                       # all equal: whole-row selection
+            u = units(g, rows)
+            hl = None if hist is None else np.full(rows, hist.shape[1], dtype=np.int32)
+            want, infos = want_rows(oracle, x, u, hist=hist, pen=pen_t, temperature=0.7, top_k=k,
+                                    top_p=0.9)
+            for one in (True, False):
+                hs.one_launch_topk(one)
+                got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9, **pk),
+                               history=hist, history_len=hl)
+                compare_ids(got, want, infos, f"call {call} one launch {one}")
+                paths = hs.topk_paths(rows).tolist()
+                assert paths[call] != 0 and paths[16 + call] != 0, paths
+    finally:
+        hs.one_launch_topk(True)
