@@ -34,14 +34,14 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 COLD_WORKING_SET = 640 * 1024 * 1024   # bytes of logits the timed loops cycle through
 
-# HBM bytes moved by one launch of the streaming kernel, from rocprofv3's FETCH_SIZE and
+# HBM bytes moved by one launch of the step's kernel, from rocprofv3's FETCH_SIZE and
 # WRITE_SIZE scaled by what the same counters read for a plain copy of the logit buffer. A
 # counter run cannot happen inside a timed benchmark, so the figure is carried here together
 # with the summary it was taken from (`roofline.traffic_source`); workloads without a counter
 # run report null.
 PROFILED_TRAFFIC = {
-    "cfg2_b64_v128256_pen2048": (35322830, "profiles/k_cand_scan_k_final_cand__cfg2_pen.md"),
-    "cfg2_b64_v128256": (35234705, "profiles/k_cand_scan_k_final_cand__cfg2.md"),
+    "cfg2_b64_v128256_pen2048": (38628690, "profiles/k_cand_scan_final__cfg2_pen.md"),
+    "cfg2_b64_v128256": (38007434, "profiles/k_cand_scan_final__cfg2.md"),
 }
 
 
@@ -199,7 +199,7 @@ def bench_spec(w, args):
         "sequences_per_s": round(n_seq * args.steps / elapsed, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "whole step (four kernels)", "step_algorithmic_bytes": alg},
+                     "kernel": "whole step (three kernels)", "step_algorithmic_bytes": alg},
         "input_copies_rotated": n_copies,
         "accepted_lengths": sorted(nacc.cpu().numpy().tolist()),
     }
@@ -788,6 +788,9 @@ def main():
     if kernel_name in ("k_cand_scan_final", "k_temperature_draw"):
         kernel_bytes = alg_bytes  # the kernel is the whole step
     achieved = kernel_bytes / (kernel_us * 1e-6) / 1e9
+    # (the counter runs were taken with the one-launch kernel)
+    traffic = (PROFILED_TRAFFIC.get(w.name, (None, None)) if kernel_name == "k_cand_scan_final"
+               else (None, None))
     result = {
         "metric": "sampled rows/s",
         "value": round(w.rows * args.steps / elapsed, 1),
@@ -814,8 +817,7 @@ def main():
         "step_latency_us_median": round(lat[len(lat) // 2], 2) if lat else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": PROFILED_TRAFFIC.get(w.name, (None, None))[0],
-                     "traffic_source": PROFILED_TRAFFIC.get(w.name, (None, None))[1],
+                     "traffic": traffic[0], "traffic_source": traffic[1],
                      "kernel": kernel_name,
                      "kernel_us": round(kernel_us, 3),
                      "kernel_us_cache_resident": None if kernel_us_resident is None else round(
