@@ -126,7 +126,7 @@ int geist_hip_sample_rows(geist_hip_sampler *s, const struct geist_hip_rows *row
  * it is for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc: no sampler object is needed and the call allocates nothing, on the host or on the
  * device. Its workspace is an array of device memory inside the library's code object
- * (7.2 MiB per GPU, held until the process ends).
+ * (7.3 MiB per GPU, held until the process ends).
  *   device, stream   where the kernels are enqueued (stream NULL = the default stream)
  *   err, err_len     optional buffer for the text of a failure
  * Served: greedy, temperature, and every top-k configuration (with top-p / min-p behind it,
