@@ -211,3 +211,57 @@ void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
         free(row);
     }
 }
+
+void oracle_dequant_q4_K_row(const void *blocks, float *out, size_t n_elems) {
+    /* q4_K.c:18-49; the block layout of src/quant/quant_blocks.h:50-56 by offsets */
+    const uint8_t *p = (const uint8_t *) blocks;
+    for (size_t b = 0; b < n_elems / 256; b++, p += 144) {
+        const float    d    = oracle_f16_to_f32((uint16_t) (p[0] | (p[1] << 8)));
+        const float    dmin = oracle_f16_to_f32((uint16_t) (p[2] | (p[3] << 8)));
+        const uint8_t *sc = p + 4, *q = p + 16;
+        float         *y  = out + b * 256;
+        for (int s = 0; s < 4; s++, q += 32) {
+            uint8_t scale[2], min[2];
+            for (int t = 0; t < 2; t++) { /* get_scale_min_k4(2 s + t) */
+                const int j = 2 * s + t;
+                if (j < 4) {
+                    scale[t] = sc[j] & 63;
+                    min[t]   = sc[j + 4] & 63;
+                } else {
+                    scale[t] = (uint8_t) ((sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4));
+                    min[t]   = (uint8_t) ((sc[j + 4] >> 4) | ((sc[j] >> 6) << 4));
+                }
+            }
+            const float d1 = d * (float) scale[0], m1 = dmin * (float) min[0];
+            const float d2 = d * (float) scale[1], m2 = dmin * (float) min[1];
+            for (int l = 0; l < 32; l++) {
+                const float a = d1 * (float) (q[l] & 0xF);
+                y[64 * s + l] = a - m1;
+            }
+            for (int l = 0; l < 32; l++) {
+                const float a      = d2 * (float) (q[l] >> 4);
+                y[64 * s + 32 + l] = a - m2;
+            }
+        }
+    }
+}
+
+void oracle_q4k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const void *w_q4k, float *y) {
+    const size_t row_bytes = n_in / 256 * 144;
+#pragma omp parallel
+    {
+        float *row = (float *) malloc(n_in * sizeof(float));
+#pragma omp for schedule(static)
+        for (size_t j = 0; j < n_out; j++) {
+            oracle_dequant_q4_K_row((const uint8_t *) w_q4k + j * row_bytes, row, n_in);
+            for (size_t i = 0; i < m; i++) {
+                double acc = 0.0;
+                for (size_t k = 0; k < n_in; k++)
+                    acc += (double) x[i * n_in + k] * (double) row[k];
+                y[i * n_out + j] = (float) acc;
+            }
+        }
+        free(row);
+    }
+}

@@ -68,6 +68,19 @@ void oracle_dequant_q6_K_row(const void *blocks, float *out, size_t n_elems);
 void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
                            const void *w_q6k, float *y);
 
+/* The same pair for a Q4_K table (super-blocks of 144 bytes: d, dmin in binary16, eight 6-bit
+ * scales and eight 6-bit minima packed into 12 bytes, 128 bytes of 4-bit values;
+ * src/quant/quant_blocks.h:50-56). dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, scales by
+ * get_scale_min_k4, quant_blocks.h:103-111): element 64 s + l of a block is
+ * (d * sc[2s]) * (qs[32 s + l] & 15) - dmin * m[2s], element 64 s + 32 + l the same with the
+ * high nibble and sc / m[2s + 1], each step rounded to binary32 (the product with the 4-bit value
+ * is exact, so a fused multiply-subtract gives the same bits). The projection is
+ * cpu_scalar_w_quant_m1 / _mN as above. Pinned bit for bit by the reference's files compiled from
+ * its tree (tests/test_q4k_oracle.py) and by hand-built blocks. */
+void oracle_dequant_q4_K_row(const void *blocks, float *out, size_t n_elems);
+void oracle_q4k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
+                           const void *w_q4k, float *y);
+
 /* y = x * weight * rsqrt(mean(x^2) + eps) per row (cpu_scalar_rmsnorm,
  * src/backends/cpu_scalar/elementwise.c:241-280): sum of squares in double in index order,
  * inv = (float)(1.0 / sqrt(sum / n + (double) eps)), y_i = (x_i * inv) * w_i in binary32. */

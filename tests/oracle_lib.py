@@ -476,6 +476,8 @@ def load_ref_wquant(fast=False):
                                       c_float_p]
     lib.dequant_q6_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
     lib.dequant_q6_K_row.restype = None
+    lib.dequant_q4_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
+    lib.dequant_q4_K_row.restype = None
     return lib
 
 
@@ -484,6 +486,69 @@ def ref_q6k_linear(ref, w_q6k, x, n_in):
     n_out = w_q6k.shape[0]
     y = np.full((xs.shape[0], n_out), np.nan, dtype=np.float32)
     rc = ref.ref_wquant_linear(ref.ref_dtype_q6_K(), w_q6k.ctypes.data_as(C.c_void_p), n_out, n_in,
+                               _fp(xs), xs.shape[0], _fp(y))
+    assert rc == 0
+    return y
+
+
+# ---- Q4_K tables ---------------------------------------------------------------------------
+Q4K_BLOCK_BYTES, Q4K_BLOCK_ELEMS = 144, 256
+
+
+def _random_f16_scales(g, shape, sigma):
+    """binary16 values that are normal, subnormal, zero or negative, never inf / NaN, as uint16."""
+    d = (g.standard_normal(shape) * sigma).astype(np.float16)
+    kind = g.random(shape)
+    d[kind < 0.03] = np.float16(0.0)
+    d = d.view(np.uint16).copy()
+    sub = (kind >= 0.03) & (kind < 0.08)
+    d[sub] = (g.integers(1, 1024, int(sub.sum())) | (g.integers(0, 2, int(sub.sum())) << 15)).astype(np.uint16)
+    return d
+
+
+def random_q4k_table(g, n_out, n_in):
+    """A [n_out, n_in] table of Q4_K super-blocks as uint8 [n_out, n_in / 256 * 144]: every bit
+    pattern of the packed scales / minima and of the 4-bit values, binary16 d and dmin of either
+    sign and of very different magnitudes (so that d * sc * q - dmin * m does round)."""
+    assert n_in % Q4K_BLOCK_ELEMS == 0
+    nb = n_in // Q4K_BLOCK_ELEMS
+    t = g.integers(0, 256, (n_out, nb, Q4K_BLOCK_BYTES), dtype=np.uint8)
+    d = _random_f16_scales(g, (n_out, nb), 0.01)
+    dmin = _random_f16_scales(g, (n_out, nb), 0.01)
+    big = g.random((n_out, nb)) < 0.3      # dmin a few thousand times d: the subtraction rounds
+    dmin[big] = (g.standard_normal(int(big.sum())) * 8.0).astype(np.float16).view(np.uint16)
+    t[:, :, 0] = (d & 0xFF).astype(np.uint8)
+    t[:, :, 1] = (d >> 8).astype(np.uint8)
+    t[:, :, 2] = (dmin & 0xFF).astype(np.uint8)
+    t[:, :, 3] = (dmin >> 8).astype(np.uint8)
+    return np.ascontiguousarray(t.reshape(n_out, nb * Q4K_BLOCK_BYTES))
+
+
+def oracle_q4k_linear(lib, w_q4k, x, n_in):
+    xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    n_out = w_q4k.shape[0]
+    y = np.empty((xs.shape[0], n_out), dtype=np.float32)
+    lib.oracle_q4k_linear_f64.argtypes = [C.c_size_t] * 3 + [c_float_p, C.c_void_p, c_float_p]
+    lib.oracle_q4k_linear_f64.restype = None
+    lib.oracle_q4k_linear_f64(xs.shape[0], n_out, n_in, _fp(xs), w_q4k.ctypes.data_as(C.c_void_p),
+                              _fp(y))
+    return y
+
+
+def oracle_dequant_q4k(lib, w_q4k, n_in):
+    out = np.empty((w_q4k.shape[0], n_in), dtype=np.float32)
+    lib.oracle_dequant_q4_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
+    lib.oracle_dequant_q4_K_row.restype = None
+    for j in range(w_q4k.shape[0]):
+        lib.oracle_dequant_q4_K_row(w_q4k[j].ctypes.data_as(C.c_void_p), _fp(out[j]), n_in)
+    return out
+
+
+def ref_q4k_linear(ref, w_q4k, x, n_in):
+    xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    n_out = w_q4k.shape[0]
+    y = np.full((xs.shape[0], n_out), np.nan, dtype=np.float32)
+    rc = ref.ref_wquant_linear(ref.ref_dtype_q4_K(), w_q4k.ctypes.data_as(C.c_void_p), n_out, n_in,
                                _fp(xs), xs.shape[0], _fp(y))
     assert rc == 0
     return y
