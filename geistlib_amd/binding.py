@@ -112,6 +112,13 @@ def load_library():
     lib.geist_hip_project_sample_rows_q6k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
                                                              vp, vp, sz, C.POINTER(SampleParams),
                                                              vp, vp, i32, vp]
+    lib.geist_hip_q4k_packed_bytes.argtypes = [sz, sz]
+    lib.geist_hip_q4k_packed_bytes.restype = sz
+    lib.geist_hip_q4k_pack.argtypes = [vp, vp, sz, sz, vp]
+    lib.geist_hip_q4k_packed_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_project_sample_rows_q4k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
+                                                             vp, vp, sz, C.POINTER(SampleParams),
+                                                             vp, vp, i32, vp]
     lib.geist_hip_f16_to_q8w.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_q8w_gemv_rows.argtypes = [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz, vp, vp, sz,
@@ -378,6 +385,32 @@ class HipSampler:
         """project_sample over the packed copy of a Q6_K table (q6k_pack)."""
         rows, d_model = hidden.shape
         self._check(self.lib.geist_hip_project_sample_rows_q6k_packed(
+            self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
+            _ptr(norm_w), eps, _ptr(packed), vocab, _ptr(normed), _ptr(logits),
+            logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),
+            _ptr(rng_states), int(shared), _ptr(out)))
+
+    def q4k_packed_bytes(self, n_out, n_in):
+        return int(self.lib.geist_hip_q4k_packed_bytes(n_out, n_in))
+
+    def q4k_pack(self, w_q4k, n_in, packed):
+        """w_q4k: uint8 [n_out, n_in / 256 * 144]; packed: uint8 tensor of q4k_packed_bytes(n_out,
+        n_in) bytes, 16-byte aligned."""
+        n_out = w_q4k.shape[0]
+        assert packed.numel() * packed.element_size() >= self.q4k_packed_bytes(n_out, n_in)
+        self._check(self.lib.geist_hip_q4k_pack(self.h, _ptr(w_q4k), n_out, n_in, _ptr(packed)))
+
+    def q4k_packed_linear(self, packed, n_out, n_in, x, y):
+        m = x.shape[0]
+        self._check(self.lib.geist_hip_q4k_packed_linear_rows(
+            self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def project_sample_q4k_packed(self, hidden, norm_w, eps, packed, vocab, logits, params,
+                                  uniforms, out, normed=None, rng_states=None, shared=True):
+        """project_sample over the packed copy of a Q4_K table (q4k_pack)."""
+        rows, d_model = hidden.shape
+        self._check(self.lib.geist_hip_project_sample_rows_q4k_packed(
             self.h, _ptr(hidden), hidden.stride(0) if rows > 1 else d_model, rows, d_model,
             _ptr(norm_w), eps, _ptr(packed), vocab, _ptr(normed), _ptr(logits),
             logits.stride(0) if rows > 1 else vocab, C.byref(params), _ptr(uniforms),

@@ -75,6 +75,13 @@ void launch_q6k_pack(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n
 void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
                               const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
                               long ld_y);
+/* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
+ * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
+size_t q4k_packed_bytes(long n_out, int n_in);
+void launch_q4k_pack(hipStream_t stream, const uint8_t *w_q4k, long n_out, int n_in, void *packed);
+void launch_q4k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
+                              const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                              long ld_y);
 
 /* The same for the int8 form of the table (q8w_gemv_m1): y[m][r] = (sum_i wq[r][i] * x[m][i]) *
  * scales[r]; n_in a multiple of 16. */

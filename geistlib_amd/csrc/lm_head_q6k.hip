@@ -544,4 +544,189 @@ void launch_q6k_linear(hipStream_t stream, const uint8_t *w_q6k, long n_out, int
         w_q6k, n_in, ws.xd, y, ld_y, ws.amb_count, ws.amb_list);
 }
 
+
+/* ==== Q4_K ==================================================================================
+ * Super-blocks of 144 bytes: d and dmin (binary16), eight 6-bit scales and eight 6-bit minima
+ * in 12 bytes, 128 bytes of 4-bit values (src/quant/quant_blocks.h:50-56). dequant_q4_K_row
+ * (src/formats/gguf/q4_K.c:18-49): element 64 s + l of a block is
+ *   (d * sc[2 s]) * (qs[32 s + l] & 15) - dmin * m[2 s],
+ * element 64 s + 32 + l the same with the high nibble and sc / m[2 s + 1]. d * sc (11 + 6 bits)
+ * and its product with the 4-bit value are exact in binary32, so the element is one rounding
+ * of an exact difference: a fused multiply-add gives the reference's bits whether or not its
+ * compiler contracted the expression. The projection adds (double) x * (double) w in index
+ * order (cpu_scalar_w_quant_m1 / _mN), as for Q6_K.
+ *
+ * Only the packed form has a kernel. geist_hip_q4k_pack writes, per group of 64 table rows and
+ * block, 37 dwords for each row with the rows innermost (dwords 4 p .. 4 p + 3 of row r, p < 9,
+ * at base + p * 256 + 4 r, dword 36 at base + 2304 + r; base = (group * blocks + b) * 2368):
+ * dwords 0..31 the 4-bit values in element order (element e in bits 4 (e % 8) .. of dword e / 8),
+ * 32..33 the eight scales and 34..35 the eight minima as bytes, 36 d (low half) and dmin. 148
+ * bytes for a block's 144: the 6-bit fields are spread to bytes once, at load.
+ * ========================================================================================== */
+constexpr int Q4K_BLOCK_BYTES = 144;
+constexpr int Q4K_ROW_DWORDS  = 37;
+constexpr int Q4K_PACK_DWORDS = Q4K_ROW_DWORDS * 64;
+
+__global__ __launch_bounds__(Q6K_TPB) void k_q4k_pack(const uint8_t *__restrict__ w, long n_out,
+                                                      int nb, uint32_t *__restrict__ packed) {
+    const int  r    = threadIdx.x & 63;
+    const long item = (long) blockIdx.x * (Q6K_TPB / 64) + threadIdx.x / 64; /* (group, block) */
+    const long g    = item / nb;
+    const int  b    = (int) (item % nb);
+    if (g * 64 >= n_out)
+        return;
+    const long row = g * 64 + r;
+    uint32_t   d[36]; /* the block's 144 bytes; a row beyond the table is a block of zeros */
+#pragma unroll
+    for (int i = 0; i < 36; ++i)
+        d[i] = 0u;
+    if (row < n_out) {
+        const uint8_t *src = w + ((size_t) row * nb + b) * Q4K_BLOCK_BYTES; /* 4-byte aligned: 144 = 36 * 4 */
+        const uint32_t *s4 = reinterpret_cast<const uint32_t *>(src);
+#pragma unroll
+        for (int i = 0; i < 36; ++i)
+            d[i] = s4[i];
+    }
+    uint32_t o[Q4K_ROW_DWORDS];
+    /* bytes 16 + 32 s + l hold elements 64 s + l (low nibble) and 64 s + 32 + l (high) */
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+        o[i] = 0u;
+#pragma unroll
+    for (int e = 0; e < 256; ++e) {
+        const int      s = e >> 6, hi = (e >> 5) & 1, l = e & 31;
+        const int      byte = 16 + 32 * s + l;
+        const uint32_t q = (d[byte / 4] >> (8 * (byte % 4) + 4 * hi)) & 0xFu;
+        o[e >> 3] |= q << (4 * (e & 7));
+    }
+    /* get_scale_min_k4 (quant_blocks.h:103-111) over the 12 bytes at offset 4 */
+    auto sbyte = [&](int i) { return (d[1 + i / 4] >> (8 * (i % 4))) & 0xFFu; };
+    o[32] = o[33] = o[34] = o[35] = 0u;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t sc, mn;
+        if (j < 4) {
+            sc = sbyte(j) & 63u;
+            mn = sbyte(j + 4) & 63u;
+        } else {
+            sc = (sbyte(j + 4) & 0xFu) | ((sbyte(j - 4) >> 6) << 4);
+            mn = (sbyte(j + 4) >> 4) | ((sbyte(j) >> 6) << 4);
+        }
+        o[32 + j / 4] |= sc << (8 * (j % 4));
+        o[34 + j / 4] |= mn << (8 * (j % 4));
+    }
+    o[36] = d[0]; /* d, dmin */
+    uint32_t *base = packed + item * Q4K_PACK_DWORDS;
+#pragma unroll
+    for (int p = 0; p < 9; ++p)
+        *reinterpret_cast<uint4 *>(base + p * 256 + 4 * r) =
+            make_uint4(o[4 * p], o[4 * p + 1], o[4 * p + 2], o[4 * p + 3]);
+    base[2304 + r] = o[36];
+}
+
+/* A lane owns a table row and adds its products one after the other in index order. Per weight:
+ * its byte (the nibbles of a dword are spread to bytes by two masks for eight weights), the
+ * conversion, one fused multiply-add in binary32 (the element), its conversion to double, one
+ * in double (the sum). */
+template <int MT>
+__global__ __launch_bounds__(Q6K_TPB) void k_q4k_packed_linear(const uint32_t *__restrict__ packed,
+                                                               long n_out, int n_in,
+                                                               const double *__restrict__ xd,
+                                                               int n_m, float *__restrict__ y,
+                                                               long ld_y) {
+    const int  r = threadIdx.x & 63;
+    const long g = (long) blockIdx.x * (Q6K_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long row = g * 64 + r;
+    const int  nb  = n_in / Q6K_BLOCK_ELEMS;
+    double     acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m] = 0.0;
+    for (int b = 0; b < nb; ++b) {
+        const uint32_t *base = packed + (g * nb + b) * Q4K_PACK_DWORDS;
+        uint32_t        d[Q4K_ROW_DWORDS];
+        /* scales, minima and d first: the arithmetic can start when they and the first values
+         * have arrived */
+        {
+            typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+            const nt_u4 q = __builtin_nontemporal_load(
+                reinterpret_cast<const nt_u4 *>(base + 8 * 256 + 4 * r));
+            d[32] = q.x, d[33] = q.y, d[34] = q.z, d[35] = q.w;
+            d[36] = __builtin_nontemporal_load(base + 2304 + r);
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+            const nt_u4 q = __builtin_nontemporal_load(
+                reinterpret_cast<const nt_u4 *>(base + p * 256 + 4 * r));
+            d[4 * p] = q.x, d[4 * p + 1] = q.y, d[4 * p + 2] = q.z, d[4 * p + 3] = q.w;
+        }
+        const float dd   = __half2float(__ushort_as_half((unsigned short) (d[36] & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short) (d[36] >> 16)));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { /* the eight sub-blocks of 32 elements */
+            const float d1  = dd * (float) ((d[32 + j / 4] >> (8 * (j % 4))) & 0xFFu);
+            const float nm1 = -(dmin * (float) ((d[34 + j / 4] >> (8 * (j % 4))) & 0xFFu));
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t v  = d[4 * j + t];
+                uint32_t lo = v & 0x0F0F0F0Fu, hi = (v >> 4) & 0x0F0F0F0Fu;
+                /* (opaque, so that each byte is converted by one v_cvt_f32_ubyteN instead of
+                 * being extracted from `v` again) */
+                asm volatile("" : "+v"(lo), "+v"(hi));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t src = (i & 1) ? hi : lo;
+                    const float    qf  = (float) ((src >> (8 * (i >> 1))) & 0xFFu);
+                    const double   wv  = (double) __builtin_fmaf(d1, qf, nm1);
+                    const int      k   = Q6K_BLOCK_ELEMS * b + 32 * j + 8 * t + i;
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) {
+                        const double *xm = xd + (long) (m < n_m ? m : n_m - 1) * n_in;
+                        acc[m] = __builtin_fma(xm[k], wv, acc[m]); /* uniform address */
+                    }
+                }
+            }
+            if (j + 1 < 8) /* one sub-block at a time (see q6k_packed_half) */
+                asm volatile("" : "+v"(acc[0]), "+v"(d[4 * j + 4]), "+v"(d[4 * j + 5]),
+                                  "+v"(d[4 * j + 6]), "+v"(d[4 * j + 7]));
+        }
+    }
+    if (row < n_out) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m < n_m)
+                y[m * ld_y + row] = (float) acc[m];
+    }
+}
+
+size_t q4k_packed_bytes(long n_out, int n_in) {
+    return (size_t) ((n_out + 63) / 64) * (size_t) (n_in / Q6K_BLOCK_ELEMS) * Q4K_PACK_DWORDS * 4;
+}
+
+void launch_q4k_pack(hipStream_t stream, const uint8_t *w_q4k, long n_out, int n_in,
+                     void *packed) {
+    const int  nb    = n_in / Q6K_BLOCK_ELEMS;
+    const long items = (n_out + 63) / 64 * nb;
+    k_q4k_pack<<<dim3((unsigned) ((items + 3) / 4)), dim3(Q6K_TPB), 0, stream>>>(
+        w_q4k, n_out, nb, static_cast<uint32_t *>(packed));
+}
+
+void launch_q4k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
+                              const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
+                              long ld_y) {
+    k_q6k_x_prep<<<dim3(n_m), dim3(Q6K_TPB), 0, stream>>>(x, ld_x, n_in, ws.xd, ws.xsum, ws.xabs,
+                                                         ws.amb_count);
+    const long     groups = (n_out + 63) / 64;
+    const dim3     grid((unsigned) ((groups + 3) / 4)), block(Q6K_TPB);
+    const uint32_t *p = static_cast<const uint32_t *>(packed);
+    switch (n_m) {
+    case 1: k_q4k_packed_linear<1><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    case 2: k_q4k_packed_linear<2><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    default: k_q4k_packed_linear<4><<<grid, block, 0, stream>>>(p, n_out, n_in, ws.xd, n_m, y, ld_y); break;
+    }
+}
+
 } // namespace gs

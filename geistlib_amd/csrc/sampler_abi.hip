@@ -1163,6 +1163,64 @@ int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
     return rc ? rc : after_launch(s, "Q6_K linear (packed)");
 }
 
+static int q4k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                  size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                  float *d_y, size_t ld_y) {
+    Q6KScratch ws; /* the activations in double: the Q6_K projection's scratch */
+    const int  rc = q6k_scratch(s, n_out, n_in, ws);
+    if (rc)
+        return rc;
+    for (size_t m0 = 0; m0 < n_rows; m0 += Q6K_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) Q6K_M_MAX ? n_rows - m0 : (size_t) Q6K_M_MAX;
+        launch_q4k_packed_linear(s->stream, d_packed, (long) n_out, (int) n_in, d_x + m0 * ld_x,
+                                 (long) ld_x, (int) m, ws, d_y + m0 * ld_y, (long) ld_y);
+    }
+    return GEIST_HIP_OK;
+}
+
+size_t geist_hip_q4k_packed_bytes(size_t n_out, size_t n_in) {
+    if (n_out == 0 || n_in == 0 || n_in % 256 != 0 || n_in > 0x7fffff00u)
+        return 0;
+    return q4k_packed_bytes((long) n_out, (int) n_in);
+}
+
+int geist_hip_q4k_pack(geist_hip_sampler *s, const void *d_w_q4k, size_t n_out, size_t n_in,
+                       void *d_packed) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_q4k || !d_packed)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    const int rc = q6k_check(s, d_w_q4k, n_out, n_in); /* the same shape rules */
+    if (rc)
+        return rc;
+    if (((uintptr_t) d_packed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q4_K table not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_q4k_pack(s->stream, static_cast<const uint8_t *>(d_w_q4k), (long) n_out, (int) n_in,
+                    d_packed);
+    return after_launch(s, "Q4_K pack");
+}
+
+int geist_hip_q4k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                     size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                     float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K linear: %zu rows, strides %zu / %zu", n_rows,
+                    ld_x, ld_y);
+    int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (((uintptr_t) d_packed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q4_K table not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q4k_packed_linear_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q4_K linear (packed)");
+}
+
 int geist_hip_f16_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
@@ -1231,7 +1289,7 @@ int geist_hip_q8w_gemv_rows(geist_hip_sampler *s, const int8_t *d_wq, const floa
 
 /* Norm, projection and sampling; the table is binary16, int8 with one scale per row (d_scales),
  * or Q6_K super-blocks. */
-enum { TABLE_F16 = 0, TABLE_Q8W = 1, TABLE_Q6K = 2, TABLE_Q6K_PACKED = 3 };
+enum { TABLE_F16 = 0, TABLE_Q8W = 1, TABLE_Q6K = 2, TABLE_Q6K_PACKED = 3, TABLE_Q4K_PACKED = 4 };
 static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size_t ld_hidden,
                                size_t rows, size_t d_model, const float *d_norm_weight,
                                float rms_eps, int table, const void *d_embed,
@@ -1241,7 +1299,8 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
                                const float *d_uniforms, uint64_t *d_rng_states, int shared,
                                geist_hip_token_t *d_out_tokens) {
     const bool      q8          = table == TABLE_Q8W;
-    const bool      q6k         = table == TABLE_Q6K || table == TABLE_Q6K_PACKED;
+    const bool      q6k         = table == TABLE_Q6K || table == TABLE_Q6K_PACKED ||
+                                  table == TABLE_Q4K_PACKED; /* the block formats */
     const size_t    in_multiple = q6k ? 256 : q8 ? 16 : 8;
     const uint16_t *d_embed_f16 = (const uint16_t *) d_embed;
     const int8_t   *d_embed_q8  = (const int8_t *) d_embed;
@@ -1288,7 +1347,10 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
-        rc = table == TABLE_Q6K_PACKED
+        rc = table == TABLE_Q4K_PACKED
+                 ? q4k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
+                                          d_logits, ld_logits)
+             : table == TABLE_Q6K_PACKED
                  ? q6k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)
                  : q6k_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows, d_logits,
@@ -1384,6 +1446,22 @@ int geist_hip_project_sample_rows_q6k_packed(geist_hip_sampler *s, const float *
         return GEIST_HIP_E_INVALID_ARG;
     return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
                                TABLE_Q6K_PACKED, d_embed_packed, nullptr, n_vocab, d_normed,
+                               d_logits, ld_logits, params, d_uniforms, d_rng_states, shared,
+                               d_out_tokens);
+}
+
+int geist_hip_project_sample_rows_q4k_packed(geist_hip_sampler *s, const float *d_hidden,
+                                             size_t ld_hidden, size_t rows, size_t d_model,
+                                             const float *d_norm_weight, float rms_eps,
+                                             const void *d_embed_packed, size_t n_vocab,
+                                             float *d_normed, float *d_logits, size_t ld_logits,
+                                             const struct geist_hip_sample_params *params,
+                                             const float *d_uniforms, uint64_t *d_rng_states,
+                                             int shared, geist_hip_token_t *d_out_tokens) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    return project_sample_impl(s, d_hidden, ld_hidden, rows, d_model, d_norm_weight, rms_eps,
+                               TABLE_Q4K_PACKED, d_embed_packed, nullptr, n_vocab, d_normed,
                                d_logits, ld_logits, params, d_uniforms, d_rng_states, shared,
                                d_out_tokens);
 }

@@ -29,6 +29,9 @@ struct geist_hip_head {
     void       *d_q6k_packed; /* the Q6_K table of geist_hip_head_q6k_load, repacked */
     const void *q6k_source;   /* ... the table it was packed from, and its row length */
     size_t      q6k_d_model;
+    void       *d_q4k_packed; /* the same for a Q4_K table (geist_hip_head_q4k_load) */
+    const void *q4k_source;
+    size_t      q4k_d_model;
     float    *d_normed; /* m_max x d_model_cap: the normed hidden rows */
     size_t    d_model_cap;
     float    *d_logits; /* m_max x vocab, written by the lm_head, read by the sampler */
@@ -108,6 +111,7 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         geist_hip_free(h->hs, h->d_ngram);
         geist_hip_free(h->hs, h->d_normed);
         geist_hip_free(h->hs, h->d_q6k_packed);
+        geist_hip_free(h->hs, h->d_q4k_packed);
         geist_hip_free(h->hs, h->d_logits);
         geist_hip_free(h->hs, h->d_spec_result);
         geist_hip_spec_head_destroy(h->hs, h->spec);
@@ -308,6 +312,61 @@ int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, s
     h->q6k_source   = d_embed_q6k;
     h->q6k_d_model  = d_model;
     return geist_hip_head_reserve_projection_q6k(h, d_model);
+}
+
+/* Q4_K: only the packed copy has a kernel, so the table has to have been loaded. */
+int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const void *d_embed_q4k, size_t d_model,
+                                        int32_t *out_tokens) {
+    if (h == nullptr || d_hidden == nullptr || d_norm_weight == nullptr || d_embed_q4k == nullptr ||
+        out_tokens == nullptr || k == 0 || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (k > h->m_max)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "more rows than m_max");
+    if (h->d_q4k_packed == nullptr || d_embed_q4k != h->q4k_source || d_model != h->q4k_d_model)
+        return head_fail(h, GEIST_HIP_E_UNSUPPORTED,
+                         "Q4_K table not loaded (geist_hip_head_q4k_load)");
+    const int rrc = geist_hip_head_reserve_projection_q6k(h, d_model); /* a no-op after the load */
+    if (rrc != GEIST_HIP_OK)
+        return rrc;
+    const struct geist_hip_sample_params prm = head_params(h);
+    const int rc = geist_hip_project_sample_rows_q4k_packed(
+            h->hs, d_hidden, ld_hidden, k, d_model, d_norm_weight, rms_eps, h->d_q4k_packed,
+            h->vocab, h->d_normed, h->d_logits, h->vocab, &prm, nullptr, h->d_rng, /*shared=*/1,
+            h->d_tokens);
+    if (rc != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
+    h->logits_sparse = false;
+    if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
+    for (size_t r = 0; r < k; r++)
+        if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
+            return head_fail(h, GEIST_HIP_E_BACKEND, "token id out of range");
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_head_q4k_load(struct geist_hip_head *h, const void *d_embed_q4k, size_t d_model) {
+    if (h == nullptr || d_embed_q4k == nullptr || d_model == 0)
+        return GEIST_HIP_E_INVALID_ARG;
+    const size_t bytes = geist_hip_q4k_packed_bytes(h->vocab, d_model);
+    if (bytes == 0)
+        return head_fail(h, GEIST_HIP_E_UNSUPPORTED, "Q4_K table: d_model not a multiple of 256");
+    geist_hip_free(h->hs, h->d_q4k_packed);
+    h->d_q4k_packed = nullptr;
+    h->q4k_source   = nullptr;
+    void *p         = nullptr;
+    if (geist_hip_malloc(h->hs, bytes, &p) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_OOM, "packed Q4_K table");
+    if (geist_hip_q4k_pack(h->hs, d_embed_q4k, h->vocab, d_model, p) != GEIST_HIP_OK ||
+        geist_hip_sampler_sync(h->hs) != GEIST_HIP_OK) {
+        geist_hip_free(h->hs, p);
+        return head_fail(h, GEIST_HIP_E_BACKEND, "packing the Q4_K table");
+    }
+    h->d_q4k_packed = p;
+    h->q4k_source   = d_embed_q4k;
+    h->q4k_d_model  = d_model;
+    return geist_hip_head_reserve_projection_q6k(h, d_model); /* the same buffers and scratch */
 }
 
 int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model) {

@@ -110,8 +110,8 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
  * the reference's portable kernel cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row
  * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch; the
  * x86 backend's one-row path through cblas_sgemv (src/backends/cpu_x86/backend.c:395-397) sums
- * in the order of the BLAS library it is linked with and is not reproduced. The other GGUF
- * block formats the reference resolves for an embedding table (Q4_K, I2_S) and an F32 table have
+ * in the order of the BLAS library it is linked with and is not reproduced. Q4_K: below. The
+ * other formats the reference resolves for an embedding table (I2_S, an F32 table) have
  * no device kernel here: their callers project on the host or with their own kernel and pass
  * the logits to geist_hip_head_finalize_one_row / _batch.
  * geist_hip_head_reserve_projection_q6k is geist_hip_head_reserve_projection plus the scratch of
@@ -127,6 +127,21 @@ int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d
                                         int32_t *out_tokens);
 int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_model);
 int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, size_t d_model);
+/* A Q4_K table (super-blocks of 144 bytes): geist_hip_head_q4k_load, once per model, keeps a
+ * copy in the order the device reads it (geist_hip_q4k_pack, 3 % more device memory than the
+ * table) and reserves the buffers; geist_hip_head_project_finalize_q4k with that same table
+ * pointer and d_model then runs norm -> projection -> soft-cap -> sampler on the device.
+ * Without the load the call is refused (GEIST_HIP_E_UNSUPPORTED): only the packed copy has a
+ * kernel. The logits equal, bit for bit, those of the portable kernel cpu_scalar_w_quant_m1 /
+ * _mN after dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, weight_resolve.c:82-83, 186-241),
+ * for one row and for a batch. The x86 and NEON backends decode this dtype with int8
+ * activations (W4A8: src/backends/cpu_x86/linear_q4k.c), a different arithmetic with different
+ * logits, which is not reproduced. */
+int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d_hidden,
+                                        size_t ld_hidden, size_t k, const float *d_norm_weight,
+                                        float rms_eps, const void *d_embed_q4k, size_t d_model,
+                                        int32_t *out_tokens);
+int geist_hip_head_q4k_load(struct geist_hip_head *h, const void *d_embed_q4k, size_t d_model);
 /* The speculative output head of greedy decoding (src/archs/transformer/forward/spec_head.c;
  * include/geist_lm_head_hip.h has the device entry points). geist_hip_head_spec_build is
  * transformer_spec_head_init (spec_head.c:616-622) for a tied F16 table in device memory, which

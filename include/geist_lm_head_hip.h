@@ -169,6 +169,30 @@ int geist_hip_project_sample_rows_q6k_packed(geist_hip_sampler *s, const float *
                                              const float *d_uniforms, uint64_t *d_rng_states,
                                              int shared, geist_hip_token_t *d_out_tokens);
 
+/* A Q4_K table (n_out rows of n_in / 256 super-blocks of 144 bytes: d and dmin in binary16, eight
+ * 6-bit scales and minima, 256 four-bit values; src/quant/quant_blocks.h:50-56), packed form
+ * only. geist_hip_q4k_packed_bytes: size of the packed copy (148 bytes per block; 0 for a shape
+ * that is not supported); geist_hip_q4k_pack: once per model, table 4-byte and d_packed 16-byte
+ * aligned; geist_hip_q4k_packed_linear_rows: d_y[i][j] = (float) sum_k (double) d_x[i][k] *
+ * (double) w[j][k] in index order, w as dequant_q4_K_row forms it (src/formats/gguf/q4_K.c:18-49)
+ * -- cpu_scalar_w_quant_m1 / _mN for that dtype (weight_resolve.c:82-83, 186-241), bit for bit.
+ * geist_hip_q6k_linear_reserve sizes the scratch. geist_hip_project_sample_rows_q4k_packed: the
+ * tail of a forward pass over the packed table, as geist_hip_project_sample_rows_q6k_packed. */
+size_t geist_hip_q4k_packed_bytes(size_t n_out, size_t n_in);
+int geist_hip_q4k_pack(geist_hip_sampler *s, const void *d_w_q4k, size_t n_out, size_t n_in,
+                       void *d_packed);
+int geist_hip_q4k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                     size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                     float *d_y, size_t ld_y);
+int geist_hip_project_sample_rows_q4k_packed(geist_hip_sampler *s, const float *d_hidden,
+                                             size_t ld_hidden, size_t rows, size_t d_model,
+                                             const float *d_norm_weight, float rms_eps,
+                                             const void *d_embed_packed, size_t n_vocab,
+                                             float *d_normed, float *d_logits, size_t ld_logits,
+                                             const struct geist_hip_sample_params *params,
+                                             const float *d_uniforms, uint64_t *d_rng_states,
+                                             int shared, geist_hip_token_t *d_out_tokens);
+
 /* The reference's speculative output head for greedy decoding
  * (src/archs/transformer/forward/spec_head.c), over a tied F16 table in device memory: an int8
  * sketch of the table ranks the vocabulary, only the best-ranked rows get their exact logit.

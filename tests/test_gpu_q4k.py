@@ -1,0 +1,131 @@
+"""The lm_head over a Q4_K table on the GPU against the oracle, which is pinned to the reference's
+own q4_K.c and weight_resolve.c (tests/test_q4k_oracle.py): logits bit for bit, for one activation
+row and for batches, and token ids through the head with a soft-cap."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle_lib import oracle_q4k_linear, random_q4k_table
+from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def hs():
+    from geistlib_amd import HipSampler
+    s = HipSampler(max_rows=16, max_vocab=262144)
+    yield s
+    s.close()
+
+
+def packed_copy(hs, w, n_in):
+    d_w = torch.from_numpy(w).cuda()
+    packed = torch.full((hs.q4k_packed_bytes(w.shape[0], n_in),), 0xA5, dtype=torch.uint8,
+                        device="cuda")
+    hs.q4k_pack(d_w, n_in, packed)
+    return packed
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(1, 256, 1), (64, 256, 1), (300, 512, 1), (1000, 768, 3),
+                                          (5000, 1536, 1), (4097, 1536, 5), (2000, 2560, 9),
+                                          (70000, 1024, 2)])
+def test_q4k_linear_equals_the_portable_kernel(hs, oracle, n_out, n_in, m):
+    print(f"q4k linear {n_out} x {n_in}, {m} rows", flush=True)
+    g = np.random.default_rng(n_out + n_in + m)
+    w = random_q4k_table(g, n_out, n_in)
+    packed = packed_copy(hs, w, n_in)
+    for scale in (1.0, 1e-4, 300.0):
+        x = (g.standard_normal((m, n_in)) * scale).astype(np.float32)
+        x[0, ::5] = 0.0
+        want = oracle_q4k_linear(oracle.lib, w, x, n_in)
+        d_x = torch.from_numpy(x).cuda()
+        y = torch.full((m, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q4k_packed_linear(packed, n_out, n_in, d_x, y)
+        hs.sync()
+        got = y.cpu().numpy()
+        bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+        assert bad.size == 0, (scale, bad[:5], got[tuple(bad[0])], want[tuple(bad[0])])
+
+
+def test_q4k_linear_rows_whose_sums_cancel(hs, oracle):
+    """Activations that repeat with alternating sign make pairs of products cancel: sums close to
+    rounding boundaries, which only the reference's order of additions gets right."""
+    g = np.random.default_rng(6)
+    n_out, n_in = 3000, 1536
+    w = random_q4k_table(g, n_out, n_in)
+    packed = packed_copy(hs, w, n_in)
+    for trial in range(3):
+        x = (g.standard_normal((2, n_in)) * 3).astype(np.float32)
+        x[:, 1::2] = -x[:, 0::2] * np.float32(1 + 2.0 ** -(8 + 4 * trial))
+        want = oracle_q4k_linear(oracle.lib, w, x, n_in)
+        y = torch.empty((2, n_out), dtype=torch.float32, device="cuda")
+        hs.q4k_packed_linear(packed, n_out, n_in, torch.from_numpy(x).cuda(), y)
+        hs.sync()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32)), trial
+
+
+def test_q4k_argument_errors(hs):
+    from geistlib_amd.binding import GeistHipError
+    assert hs.q4k_packed_bytes(4, 200) == 0                   # not a whole number of blocks
+    assert hs.q4k_packed_bytes(4, 256) == 64 * 37 * 4         # one group of 64 rows, one block
+    w = torch.zeros((4, 144), dtype=torch.uint8, device="cuda")
+    packed = torch.zeros((hs.q4k_packed_bytes(4, 256) + 16,), dtype=torch.uint8, device="cuda")
+    x = torch.ones((1, 256), dtype=torch.float32, device="cuda")
+    y = torch.full((1, 4), 7.0, dtype=torch.float32, device="cuda")
+    hs.q4k_pack(w, 256, packed)
+    hs.q4k_packed_linear(packed, 4, 256, x, y)
+    hs.sync()
+    assert not y.cpu().numpy().any()                          # a table of zeros
+    with pytest.raises(GeistHipError):                        # packed copy not 16-byte aligned
+        hs._check(hs.lib.geist_hip_q4k_packed_linear_rows(hs.h, packed.data_ptr() + 4, 4, 256,
+                                                          x.data_ptr(), 256, 1, y.data_ptr(), 4))
+    with pytest.raises(GeistHipError):                        # table not 4-byte aligned
+        hs._check(hs.lib.geist_hip_q4k_pack(hs.h, w.data_ptr() + 2, 3, 256, packed.data_ptr()))
+
+
+def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
+    """262144 x 1536 Q4_K behind the head with soft-cap 30 (head.c:94-188): norm, projection,
+    soft-cap, dispatch, one shared generator. Tokens equal the oracle's session on the oracle's
+    logits, for decode steps and for a batch; without geist_hip_head_q4k_load the call is
+    refused."""
+    host.geist_hip_head_project_finalize_q4k.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
+                                                         C.c_size_t, C.c_void_p, C.c_float,
+                                                         C.c_void_p, C.c_size_t,
+                                                         C.POINTER(C.c_int32)]
+    host.geist_hip_head_q4k_load.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    g = np.random.default_rng(2027)
+    vocab, d_model, cap = 262144, 1536, 30.0
+    w = random_q4k_table(g, vocab, d_model)
+    w[:, 2::144] = 0                      # dmin = 0.0 or tiny: logits stay within the cap's range
+    w[:, 3::144] &= 0x03
+    norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
+    d_w, d_nw = torch.from_numpy(w).cuda(), torch.from_numpy(norm_w).cuda()
+    for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.95, 0)]:
+        print(f"q4k table T={T} p={p} k={top_k}", flush=True)
+        h = make_head(host, vocab, 4, cap)
+        opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 4)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        hidden = (g.standard_normal((1, d_model)) * 4).astype(np.float32)
+        d_hid = torch.from_numpy(hidden).cuda()
+        out1 = (C.c_int32 * 1)()
+        assert host.geist_hip_head_project_finalize_q4k(
+            h, C.c_void_p(d_hid.data_ptr()), d_model, 1, C.c_void_p(d_nw.data_ptr()), 1e-6,
+            C.c_void_p(d_w.data_ptr()), d_model, out1) != 0     # not loaded yet
+        assert host.geist_hip_head_q4k_load(h, C.c_void_p(d_w.data_ptr()), d_model) == 0, \
+            host.geist_hip_head_errmsg(h)
+        sess = oracle.session(T, p, top_k, seed=4242)
+        for k in (1, 1, 3):
+            hidden = (g.standard_normal((k, d_model)) * 4).astype(np.float32)
+            d_hid = torch.from_numpy(hidden).cuda()
+            out = (C.c_int32 * k)()
+            rc = host.geist_hip_head_project_finalize_q4k(
+                h, C.c_void_p(d_hid.data_ptr()), d_model, k, C.c_void_p(d_nw.data_ptr()), 1e-6,
+                C.c_void_p(d_w.data_ptr()), d_model, out)
+            assert rc == 0, host.geist_hip_head_errmsg(h)
+            logits = oracle_q4k_linear(oracle.lib, w, oracle.rmsnorm(hidden, norm_w, 1e-6), d_model)
+            want = oracle.finalize_batch(sess, logits, softcap=cap).tolist()
+            assert list(out) == want, (T, p, top_k, k)
+        host.geist_hip_head_destroy(h)
