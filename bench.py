@@ -545,6 +545,110 @@ def bench_lm_head_q6k(args, m_rows):
     return 0
 
 
+def bench_lm_head_q4k(args, m_rows):
+    """Workload lm_head_q4k[_mN]: as lm_head_q6k over a Q4_K table of the same geometry
+    ([262144 x 1536], super-blocks of 144 bytes: 226 MB, read once per step; the portable kernel
+    of src/backends/cpu_scalar/weight_resolve.c:82-83, 186-241 after src/formats/gguf/q4_K.c),
+    from the packed copy the head keeps (148 bytes per block)."""
+    import torch
+    from geistlib_amd import HipSampler, SampleParams
+    from geistlib_amd.bench_hooks import Timer
+    from geistlib_amd.workloads import xorshift_units
+    vocab, d_model = 262144, 1536
+    nb = d_model // 256
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(13)
+    hs = HipSampler(max_rows=max(m_rows, 1), max_vocab=vocab)
+    tables, packed = [], []
+    for _ in range(3):          # three copies (0.7 GB packed): every step's table comes from HBM
+        t = torch.randint(0, 256, (vocab, nb, 144), dtype=torch.uint8, device=dev, generator=g)
+        # d = binary16 0x0C6D = 2.7e-4 and dmin = 8 d in every block: logits of a few units
+        t[:, :, 0], t[:, :, 1] = 0x6D, 0x0C
+        t[:, :, 2], t[:, :, 3] = 0x6D, 0x18
+        t = t.reshape(vocab, nb * 144).contiguous()
+        pk = torch.empty((hs.q4k_packed_bytes(vocab, d_model),), dtype=torch.uint8, device=dev)
+        hs.q4k_pack(t, d_model, pk)
+        tables.append(t)
+        packed.append(pk)
+    hs.sync()
+    hidden = torch.randn((m_rows, d_model), device=dev, generator=g) * 3
+    norm_w = 1.0 + 0.1 * torch.randn((d_model,), device=dev, generator=g)
+    u, _ = xorshift_units(7, m_rows)
+    d_u = torch.from_numpy(u).to(dev)
+    normed = torch.empty_like(hidden)
+    logits = torch.empty((m_rows, vocab), dtype=torch.float32, device=dev)
+    out = torch.empty(m_rows, dtype=torch.int32, device=dev)
+    prm = SampleParams.make(temperature=0.7, top_k=40, top_p=0.9, softcap=30.0)
+
+    def step(i=0):
+        hs.project_sample_q4k_packed(hidden, norm_w, 1e-6, packed[i % 3], vocab, logits, prm, d_u,
+                                     out, normed=normed)
+
+    for i in range(args.warmup):
+        step(i)
+    hs.sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    hs.sync()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed * 1e3 / args.steps
+    ids_gpu = out.cpu().numpy()
+    hs.rmsnorm(hidden, norm_w, 1e-6, normed)
+    for i in range(3):
+        hs.q4k_packed_linear(packed[i], vocab, d_model, normed, logits)
+    with Timer() as tm:       # HIP events on the sampler's stream around the launches
+        for i in range(args.steps):
+            hs.q4k_packed_linear(packed[i % 3], vocab, d_model, normed, logits)
+    kernel_us = tm.ms * 1e3 / args.steps
+    w_bytes = vocab * nb * 144
+    read_bytes = vocab * nb * 148
+    achieved = w_bytes / (kernel_us * 1e-6) / 1e9
+    result = {
+        "metric": "sampled rows/s", "value": round(m_rows * args.steps / elapsed, 1),
+        "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "Q4_K weights x f32 activations, f64 accumulation", "data": "synthetic",
+        "config": {"workload": f"lm_head_q4k_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
+                   "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
+                   "top_p": 0.9, "logit_softcap": 30.0},
+        "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "k_q4k_packed_linear (+ activations to double)",
+                     "kernel_us": round(kernel_us, 3),
+                     "kernel_algorithmic_bytes": w_bytes,
+                     "packed_bytes_read": read_bytes,
+                     "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
+    }
+    if not args.no_cpu:
+        from oracle_lib import load_oracle, oracle_q4k_linear
+        lib = load_oracle(fast=True)
+        n_s = 16384
+        w_s = tables[0][:n_s].cpu().numpy()
+        x_s = normed.cpu().numpy()
+        t0 = time.perf_counter()
+        want = oracle_q4k_linear(lib, w_s, x_s, d_model)
+        dt = time.perf_counter() - t0
+        hs.q4k_packed_linear(packed[0], vocab, d_model, normed, logits)
+        hs.sync()
+        got = logits[:, :n_s].cpu().numpy()
+        result["cpu_baseline"] = {
+            "value": round(m_rows / (dt * vocab / n_s), 2), "unit": "rows/s",
+            "cores": int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1),
+            "kind": "port",
+            "sample": f"the projection of {m_rows} row(s) over the first {n_s} of {vocab} table rows "
+                      "(dequantise a row, accumulate in double), scaled to the whole table; the "
+                      "sampler's share of the step is not included"}
+        result["parity"] = {"logits_compared": int(want.size),
+                            "logits_differ": int((got.view(np.uint32) != want.view(np.uint32)).sum())}
+    result["token_ids"] = [int(t) for t in ids_gpu[:8]]
+    print(json.dumps(result))
+    return 0
+
+
 def bench_lm_head_spec(args):
     """Workload lm_head_spec: the tail of a greedy decode step for BitNet-2B-4T's geometry through
     the reference's speculative output head (forward/spec_head.c): RMS norm of the hidden row,
@@ -675,6 +779,9 @@ def main():
     if args.workload.startswith("lm_head_q6k"):
         m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
         return bench_lm_head_q6k(args, m)
+    if args.workload.startswith("lm_head_q4k"):
+        m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
+        return bench_lm_head_q4k(args, m)
     if args.workload.startswith("lm_head"):
         m = int(args.workload.split("_m")[1]) if "_m" in args.workload else 1
         return bench_lm_head(args, m, q8=args.workload.startswith("lm_head_q8"))
