@@ -339,17 +339,13 @@ __device__ __forceinline__ void final_cand_row(const RowView &rv, const FinalArg
     bool           give_up = bk == 0xffffffffu;
     const uint32_t lo      = bk < KEY_LOWEST_FINITE ? KEY_LOWEST_FINITE : bk;
     const float    B       = key2f(lo);
-    /* With penalties: the row's history goes into an open-addressing table in LDS (ids and how
-     * often each occurs). The first attempt at each id's slot is issued here and settled after
-     * the candidates have been listed, so that the two round trips overlap. */
-    const bool     have0 = PEN && (unsigned) hid0 < (unsigned) rv.n_vocab;
-    const bool     have1 = PEN && (unsigned) hid1 < (unsigned) rv.n_vocab;
-    const uint32_t hs0 = hist_hash(hid0), hs1 = hist_hash(hid1);
-    int            old0 = 0, old1 = 0;
-    if (have0)
-        old0 = atomicCAS(&hkey[hs0], -1, hid0);
-    if (have1)
-        old1 = atomicCAS(&hkey[hs1], -1, hid1);
+    /* With penalties the table in LDS is of the CANDIDATES (a few hundred ids, each once), and
+     * the row's history is looked up in it: an id of the history that is no candidate -- nearly
+     * all of them -- costs one LDS read, and only hits count, with an atomic add. (A table of
+     * the history's 2048 ids took two to three returning atomics per id, and the most frequent
+     * ids' additions queued behind one another.) */
+    const bool have0 = PEN && (unsigned) hid0 < (unsigned) rv.n_vocab;
+    const bool have1 = PEN && (unsigned) hid1 < (unsigned) rv.n_vocab;
     /* this wavefront's elements at or above B, into its list in LDS. A lane's place is the
      * number of kept elements before it; what is not kept is written to the lane's spare slot,
      * so that no branch is needed. */
@@ -370,26 +366,41 @@ __device__ __forceinline__ void final_cand_row(const RowView &rv, const FinalArg
         }
     }
     give_up = give_up || n_e > (unsigned) FC_LIST;
+    /* one element per lane from here on */
+    wave_lds_sync();
+    uint32_t my_slot = 0u;
     if (PEN) {
-        /* claim the slot or find it taken by the same id, then count (16-bit counters, two a
-         * word: a history holds fewer than 65536 ids) */
-        auto settle = [&](int id, uint32_t h, int old) {
+        /* every listed element claims a slot (ids of a row are distinct: a claim never meets
+         * its own id; at most 16 x 64 elements for 4096 slots) */
+        if (lane < (int) (n_e < (unsigned) FC_LIST ? n_e : (unsigned) FC_LIST)) {
+            const int id = (int) e_idx[lane];
+            my_slot      = hist_hash(id);
 #pragma unroll 1
-            for (int pr = 0; pr < HT_SLOTS && old != -1 && old != id; ++pr) {
-                h   = (h + 1u) & (HT_SLOTS - 1);
-                old = atomicCAS(&hkey[h], -1, id);
+            for (int pr = 0; pr < HT_SLOTS && atomicCAS(&hkey[my_slot], -1, id) != -1; ++pr)
+                my_slot = (my_slot + 1u) & (HT_SLOTS - 1);
+        }
+        __syncthreads();
+        /* the history: a hit adds one to the element's counter (16-bit counters, two a word: a
+         * history holds fewer than 65536 ids) */
+        auto look_up = [&](int id) {
+            uint32_t h = hist_hash(id);
+            int      k = hkey[h];
+#pragma unroll 1
+            for (int pr = 0; pr < HT_SLOTS && k != id && k != -1; ++pr) {
+                h = (h + 1u) & (HT_SLOTS - 1);
+                k = hkey[h];
             }
-            atomicAdd(&hcnt[h >> 1], 1u << (16 * (h & 1u)));
+            if (k == id)
+                atomicAdd(&hcnt[h >> 1], 1u << (16 * (h & 1u)));
         };
         if (have0)
-            settle(hid0, hs0, old0);
+            look_up(hid0);
         if (have1)
-            settle(hid1, hs1, old1);
+            look_up(hid1);
         __syncthreads();
     }
-    /* one element per lane from here on. With penalties: how often the row's history names it
-     * is read from the table; an element that no longer reaches B gets key 0. */
-    wave_lds_sync();
+    /* With penalties: how often the row's history names the element is read from its slot; an
+     * element that no longer reaches B gets key 0. */
     uint32_t my_key = 0u;
     /* With the soft-cap left to this kernel (FinalArgs::cap_after) an entry counts when its
      * capped value lies strictly above the capped bound: those are certain to be all there are. */
@@ -399,17 +410,9 @@ __device__ __forceinline__ void final_cand_row(const RowView &rv, const FinalArg
         if (PEN || a.cap_after) {
             float x = __uint_as_float(my_key);
             if (PEN) {
-                const int id = (int) e_idx[lane];
-                uint32_t  hq = hist_hash(id);
-                int       kq = hkey[hq];
-#pragma unroll 1
-                for (int pr = 0; pr < HT_SLOTS && kq != id && kq != -1; ++pr) {
-                    hq = (hq + 1u) & (HT_SLOTS - 1);
-                    kq = hkey[hq];
-                }
-                if (kq == id)
-                    x = penalise(x, (hcnt[hq >> 1] >> (16 * (hq & 1u))) & 0xffffu, rv.rep,
-                                 rv.inv_rep, rv.freq, rv.pres);
+                const uint32_t times = (hcnt[my_slot >> 1] >> (16 * (my_slot & 1u))) & 0xffffu;
+                if (times)
+                    x = penalise(x, times, rv.rep, rv.inv_rep, rv.freq, rv.pres);
             }
             if (a.cap_after) {
                 my_key = 0u;
