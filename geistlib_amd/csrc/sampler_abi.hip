@@ -628,8 +628,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         const size_t row_waves = rows->rows * (size_t) L.rv.n_chunks * NWAVES_PER_CHUNK;
         const bool   plain = rs.k <= CAND_K_MAX && L.rv.vec_ok && !L.rv.allowed &&
                            L.rv.n_chunks <= CAND_CHUNKS_MAX && (!L.pen || !scan.pen) &&
-                           !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves &&
-                           (!L.pen || rows->history_ld <= (size_t) HT_HISTORY_MAX);
+                           !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves;
         const int m = plain ? cand_lanes_for(f.k_sel, rows->n_vocab) : 0;
         if (m) {
             const WaveCands wc = wave_cands_at(s->wcands, row_waves);

@@ -298,17 +298,18 @@ __device__ __forceinline__ void final_cand_row(const RowView &rv, const FinalArg
         }
     }
     uint32_t bk = tid < W ? wc.bound[row * W + tid] : 0u;
-    /* the row's history, two ids a thread (at most HT_HISTORY_MAX = 2 * 1024: the launch code
-     * sends longer histories down another path) */
-    int hid0 = -1, hid1 = -1;
+    /* the row's history: the first two ids of each thread are asked for here (2048 ids: all of
+     * most histories), the rest when the history is looked up */
+    int            hid0 = -1, hid1 = -1, hlen = 0;
+    const int32_t *hrow = nullptr;
     if (PEN) {
-        int hlen = rv.hist_len[row];
-        hlen     = hlen > rv.hist_ld ? (int) rv.hist_ld : hlen;
-        const int32_t *h = rv.hist + (long) row * rv.hist_ld;
+        hlen = rv.hist_len[row];
+        hlen = hlen > rv.hist_ld ? (int) rv.hist_ld : hlen;
+        hrow = rv.hist + (long) row * rv.hist_ld;
         if (tid < hlen)
-            hid0 = h[tid];
+            hid0 = hrow[tid];
         if (tid + FC_THREADS < hlen)
-            hid1 = h[tid + FC_THREADS];
+            hid1 = hrow[tid + FC_THREADS];
     }
     const float u_row = a.uniforms[row];
     if (tid < 32)
@@ -397,6 +398,12 @@ __device__ __forceinline__ void final_cand_row(const RowView &rv, const FinalArg
             look_up(hid0);
         if (have1)
             look_up(hid1);
+#pragma unroll 1
+        for (int i = tid + 2 * FC_THREADS; i < hlen; i += FC_THREADS) {
+            const int id = hrow[i];
+            if ((unsigned) id < (unsigned) rv.n_vocab)
+                look_up(id);
+        }
         __syncthreads();
     }
     /* With penalties: how often the row's history names the element is read from its slot; an

@@ -105,11 +105,9 @@ inline WaveCands wave_cands_at(void *base, size_t row_waves) {
     w.bound = reinterpret_cast<uint32_t *>(w.idx + row_waves * CAND_SLOTS);
     return w;
 }
-/* The final kernel of that path keeps the row's token history as an open-addressing table in LDS
- * (HT_SLOTS slots: a row's distinct ids and how often each occurs), for histories of up to
- * HT_HISTORY_MAX ids, so that the table stays at most half full. */
+/* The final stage of that path keeps its candidates (at most 16 x 64 ids) in an open-addressing
+ * table of HT_SLOTS slots in LDS and looks the row's token history up in it. */
 constexpr int HT_SLOTS       = 4096;
-constexpr int HT_HISTORY_MAX = 2048;
 
 /* `m` for a row of n_vocab logits of which about k_eff lead: the smallest number of lanes such
  * that a wavefront (2048 logits) holding that many of the k_eff is a one-in-10^8 event when the

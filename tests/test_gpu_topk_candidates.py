@@ -129,8 +129,8 @@ def test_penalties_that_empty_the_candidates(hs, oracle):
 
 
 def test_calls_that_stay_off_the_candidate_path(hs, oracle):
-    """Soft-cap, k above 64, a history longer than the table takes, penalties that can raise a
-    logit: the thread-maxima path serves the whole call, and says so."""
+    """k above 64 and penalties that can raise a logit: the thread-maxima path serves the whole
+    call, and says so."""
     g = np.random.default_rng(9)
     n, rows = 60000, 8
     x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
@@ -138,7 +138,6 @@ def test_calls_that_stay_off_the_candidate_path(hs, oracle):
     hist = g.integers(0, n, (rows, 2500)).astype(np.int32)
     hl = np.full(rows, 2500, dtype=np.int32)
     cases = [(dict(temperature=0.7, top_k=100), None, None),
-             (dict(temperature=0.7, top_k=40, rep=1.2), hist, (1.2, 0.0, 0.0)),
              (dict(temperature=0.7, top_k=40, rep=0.8), hist[:, :100].copy(), (0.8, 0.0, 0.0))]
     for kw, h, pen in cases:
         hlen = None if h is None else np.full(rows, h.shape[1], dtype=np.int32)
@@ -147,6 +146,32 @@ def test_calls_that_stay_off_the_candidate_path(hs, oracle):
         okw = {k_: v for k_, v in kw.items() if k_ in ("temperature", "top_k", "top_p", "min_p")}
         want, infos = want_rows(oracle, x, u, hist=h, pen=pen, **okw)
         compare_ids(got, want, infos, f"off the candidate path {kw}")
+
+
+@pytest.mark.parametrize("H", [2500, 9000, 40000])
+def test_histories_of_any_length_on_the_candidate_path(hs, oracle, H):
+    """The final stage keeps its candidates in a table and looks the history up in it, so the
+    history's length does not matter: thousands of ids, many of them repeated and many of them
+    among the leading logits, still on the candidate path."""
+    g = np.random.default_rng(H)
+    n, rows, k = 128256, 16, 40
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    hist = g.integers(0, n, (rows, H)).astype(np.int32)
+    for r in range(rows):                       # the row's leaders, over and over
+        top = np.argsort(-x[r])[:60]
+        hist[r, : H // 2] = g.choice(top, H // 2)
+    hist[0, :] = int(np.argmax(x[0]))           # one id H times
+    hl = np.full(rows, H, dtype=np.int32)
+    hl[1] = H - 777
+    u = units(g, rows)
+    pen = (1.3, 0.02, 0.1)
+    got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9, rep=pen[0], freq=pen[1],
+                                      pres=pen[2]), hist, hl)
+    paths = hs.topk_paths(rows).tolist()
+    want, infos = want_rows(oracle, x, u, hist=[hist[r, :hl[r]] for r in range(rows)], pen=pen,
+                            temperature=0.7, top_k=k, top_p=0.9)
+    compare_ids(got, want, infos, f"history of {H}")
+    assert all(p_ >= 0 for p_ in paths), paths   # the candidate path served the call
 
 
 def test_soft_capped_rows_select_on_raw_logits_and_cap_what_they_keep(hs, oracle):
