@@ -526,8 +526,11 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
     }
 }
 
+/* The penalised list-making form needs 82 registers when left alone, two more than let a sixth
+ * workgroup share a compute unit; held to 80 it spills nothing and a launch of 128 x 151936 is
+ * about a microsecond shorter. (Held to 72 or 64 it spills and is slower.) */
 template <int NV, bool PEN, bool LISTM, bool SLABS>
-__global__ __launch_bounds__(TPB) void k_scan_expsum(RowView rv, float inv_t,
+__global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan_expsum(RowView rv, float inv_t,
                                                      float *__restrict__ tmax,
                                                      uint64_t *__restrict__ chunk_best,
                                                      double *__restrict__ chunk_sum,
