@@ -1565,6 +1565,24 @@ int geist_hip_free(geist_hip_sampler *s, void *d_ptr) {
     HIPCHK(s, hipFree(d_ptr));
     return GEIST_HIP_OK;
 }
+/* Page-locked host memory that the device addresses in place (hipHostMalloc: the pointer is valid
+ * on both sides). What a kernel stores there is in host memory once its stream has been waited
+ * for, and what the host stores there is what a kernel launched afterwards reads: a few words of
+ * results or arguments cross without a copy command. */
+int geist_hip_host_malloc(geist_hip_sampler *s, size_t bytes, void **h_ptr) {
+    if (!s || !h_ptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    HIPCHK(s, hipSetDevice(s->device));
+    HIPCHK(s, hipHostMalloc(h_ptr, bytes ? bytes : 1, hipHostMallocDefault));
+    return GEIST_HIP_OK;
+}
+int geist_hip_host_free(geist_hip_sampler *s, void *h_ptr) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (h_ptr)
+        HIPCHK(s, hipHostFree(h_ptr));
+    return GEIST_HIP_OK;
+}
 int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;

@@ -21,6 +21,9 @@ struct geist_hip_head {
     size_t   m_max;
     geist_hip_sampler *hs;
     uint64_t *d_rng;   /* the session's struct geist_rng, in device memory */
+    /* d_tokens, d_nacc, d_ngram and d_spec_result are page-locked host memory that the device
+     * writes in place (geist_hip_host_malloc): reading them takes a wait for the stream and no
+     * copy command (read_back) */
     int32_t  *d_tokens; /* m_max */
     float    *d_units;  /* m_max uniforms of one speculative round */
     int32_t  *d_drafts; /* m_max */
@@ -49,6 +52,14 @@ static int head_fail(struct geist_hip_head *h, int code, const char *what) {
     return code;
 }
 
+/* What the kernels queued so far have left in one of the page-locked result buffers. */
+static int read_back(struct geist_hip_head *h, void *dst, const void *pinned, size_t bytes) {
+    if (geist_hip_sampler_sync(h->hs) != GEIST_HIP_OK)
+        return GEIST_HIP_E_BACKEND;
+    memcpy(dst, pinned, bytes);
+    return GEIST_HIP_OK;
+}
+
 static int seed_rng(struct geist_hip_head *h, uint64_t seed) {
     /* geist_rng_seed, src/engine/sampler.c:27-33 */
     const uint64_t state = seed != 0 ? seed : UINT64_C(0x9E3779B97F4A7C15);
@@ -75,7 +86,7 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
     if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(h->hs, sizeof(uint64_t), &p)) == GEIST_HIP_OK)
         h->d_rng = p;
     if (rc == GEIST_HIP_OK &&
-        (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        (rc = geist_hip_host_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_tokens = p;
     if (rc == GEIST_HIP_OK &&
         (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(float), &p)) == GEIST_HIP_OK)
@@ -83,10 +94,11 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
     if (rc == GEIST_HIP_OK &&
         (rc = geist_hip_malloc(h->hs, h->m_max * sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_drafts = p;
-    if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(h->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_host_malloc(h->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_nacc = p;
     if (rc == GEIST_HIP_OK &&
-        (rc = geist_hip_malloc(h->hs, 20 * sizeof(int32_t), &p)) == GEIST_HIP_OK)
+        (rc = geist_hip_host_malloc(h->hs, 20 * sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_ngram = p;
     /* arch_state.c:1173: the default seed */
     if (rc == GEIST_HIP_OK)
@@ -104,16 +116,16 @@ void geist_hip_head_destroy(struct geist_hip_head *h) {
         return;
     if (h->hs != nullptr) {
         geist_hip_free(h->hs, h->d_rng);
-        geist_hip_free(h->hs, h->d_tokens);
+        geist_hip_host_free(h->hs, h->d_tokens);
         geist_hip_free(h->hs, h->d_units);
         geist_hip_free(h->hs, h->d_drafts);
-        geist_hip_free(h->hs, h->d_nacc);
-        geist_hip_free(h->hs, h->d_ngram);
+        geist_hip_host_free(h->hs, h->d_nacc);
+        geist_hip_host_free(h->hs, h->d_ngram);
         geist_hip_free(h->hs, h->d_normed);
         geist_hip_free(h->hs, h->d_q6k_packed);
         geist_hip_free(h->hs, h->d_q4k_packed);
         geist_hip_free(h->hs, h->d_logits);
-        geist_hip_free(h->hs, h->d_spec_result);
+        geist_hip_host_free(h->hs, h->d_spec_result);
         geist_hip_spec_head_destroy(h->hs, h->spec);
         geist_hip_sampler_destroy(h->hs);
     }
@@ -202,7 +214,7 @@ static int finalize(struct geist_hip_head *h, const float *d_logits, size_t k, i
     if (geist_hip_sample_rows_rng(h->hs, &rows, &prm, h->d_rng, /*shared=*/1, h->d_tokens) !=
         GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "sampling");
-    if (geist_hip_download(h->hs, out, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_back(h, out, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++) /* head.c:137-139: an id outside the vocabulary is an error */
         if (out[r] < 0 || (size_t) out[r] >= h->vocab)
@@ -275,7 +287,7 @@ static int project_finalize_table(struct geist_hip_head *h, const float *d_hidde
     if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
     h->logits_sparse = false;
-    if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_back(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++)
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
@@ -338,7 +350,7 @@ int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d
     if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
     h->logits_sparse = false;
-    if (geist_hip_download(h->hs, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_back(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++)
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
@@ -414,7 +426,7 @@ int geist_hip_head_spec_build(struct geist_hip_head *h, const uint16_t *d_embed_
     h->spec = nullptr;
     void *p = nullptr;
     if (h->d_spec_result == nullptr) {
-        if (geist_hip_malloc(h->hs, sizeof *h->d_spec_result, &p) != GEIST_HIP_OK)
+        if (geist_hip_host_malloc(h->hs, sizeof *h->d_spec_result, &p) != GEIST_HIP_OK)
             return head_fail(h, GEIST_HIP_E_OOM, "sketch head result");
         h->d_spec_result = p;
     }
@@ -450,7 +462,7 @@ int geist_hip_head_project_finalize_spec(struct geist_hip_head *h, const float *
     struct geist_hip_spec_result res;
     if (geist_hip_spec_head_try_hidden(h->hs, h->spec, d_hidden, d_norm_weight, rms_eps,
                                        h->d_normed, verify, h->d_spec_result) != GEIST_HIP_OK ||
-        geist_hip_download(h->hs, &res, h->d_spec_result, sizeof res) != GEIST_HIP_OK)
+        read_back(h, &res, h->d_spec_result, sizeof res) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "sketch head");
     if (res.answered == 0) /* head.c:114-188: the dense head */
         return project_finalize(h, d_hidden, d_model, 1, d_norm_weight, rms_eps, d_embed_f16,
@@ -496,14 +508,13 @@ int geist_hip_head_propose_drafts(struct geist_hip_head *h, const int32_t *d_his
     *n_drafts     = 1;
     if (history_n == 0 || k_max == 1) /* session.c:446-447 */
         return GEIST_HIP_OK;
-    const int32_t in[2] = {seed, (int32_t) history_n};
-    int32_t       back[18];
-    if (geist_hip_upload(h->hs, h->d_ngram, in, sizeof in) != GEIST_HIP_OK ||
-        geist_hip_propose_drafts_ngram(h->hs, d_history, history_n, h->d_ngram + 1, h->d_ngram, 1,
+    int32_t back[18];
+    h->d_ngram[0] = seed; /* the kernel reads both in place */
+    h->d_ngram[1] = (int32_t) history_n;
+    if (geist_hip_propose_drafts_ngram(h->hs, d_history, history_n, h->d_ngram + 1, h->d_ngram, 1,
                                        k_max, /*max_suffix=*/4, h->d_ngram + 4, 16,
                                        h->d_ngram + 2, h->d_ngram + 3) != GEIST_HIP_OK ||
-        geist_hip_download(h->hs, back, h->d_ngram + 2, (2 + k_max) * sizeof(int32_t)) !=
-                GEIST_HIP_OK)
+        read_back(h, back, h->d_ngram + 2, (2 + k_max) * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "n-gram drafts");
     if (back[0] < 1 || (size_t) back[0] > k_max || back[1] < 0 || back[1] > 4)
         return head_fail(h, GEIST_HIP_E_BACKEND, "draft count out of range");
@@ -562,11 +573,10 @@ int geist_hip_head_spec_accept(struct geist_hip_head *h, const float *d_logits, 
                               h->d_nacc) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "verification");
     int32_t n_acc = 0;
-    if (geist_hip_download(h->hs, &n_acc, h->d_nacc, sizeof n_acc) != GEIST_HIP_OK ||
-        n_acc < 0 || (size_t) n_acc > L ||
-        geist_hip_download(h->hs, out_tokens + 1, h->d_tokens,
-                           ((size_t) n_acc + 1) * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_back(h, &n_acc, h->d_nacc, sizeof n_acc) != GEIST_HIP_OK || n_acc < 0 ||
+        (size_t) n_acc > L)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the verdict");
+    memcpy(out_tokens + 1, h->d_tokens, ((size_t) n_acc + 1) * sizeof(int32_t));
     out_tokens[0] = drafts[0];
     *n_out        = (size_t) n_acc + 2;
     for (size_t i = 0; i < *n_out; i++)

@@ -60,8 +60,8 @@ static geist_token_t fail(const char *what, geist_hip_sampler *hs) {
 static void ctx_release(struct dropin_ctx *c) {
     if (c->hs != nullptr) {
         geist_hip_free(c->hs, c->d_row);
-        geist_hip_free(c->hs, c->d_u);
-        geist_hip_free(c->hs, c->d_out);
+        geist_hip_host_free(c->hs, c->d_u);
+        geist_hip_host_free(c->hs, c->d_out);
         geist_hip_sampler_destroy(c->hs);
     }
     *c = (struct dropin_ctx) {0};
@@ -75,9 +75,13 @@ static int ctx_setup(struct dropin_ctx *c, size_t n_vocab) {
     void *p = nullptr;
     if ((rc = geist_hip_malloc(c->hs, n_vocab * sizeof(float), &p)) == GEIST_HIP_OK)
         c->d_row = p;
-    if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(c->hs, sizeof(float), &p)) == GEIST_HIP_OK)
+    /* the draw and the token id: page-locked host memory that the kernels read and write in
+     * place, so neither is copied */
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_host_malloc(c->hs, sizeof(float), &p)) == GEIST_HIP_OK)
         c->d_u = p;
-    if (rc == GEIST_HIP_OK && (rc = geist_hip_malloc(c->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
+    if (rc == GEIST_HIP_OK &&
+        (rc = geist_hip_host_malloc(c->hs, sizeof(int32_t), &p)) == GEIST_HIP_OK)
         c->d_out = p;
     if (rc != GEIST_HIP_OK) {
         ctx_release(c);
@@ -140,8 +144,8 @@ static geist_token_t sample_one(struct dropin_ctx *c, size_t n, const float *log
         return GEIST_SAMPLER_DROPIN_FAILED_TOKEN;
     if (geist_hip_upload(c->hs, c->d_row, logits, n * sizeof(float)) != GEIST_HIP_OK)
         return fail("upload of the logit row", c->hs);
-    if (u != nullptr && geist_hip_upload(c->hs, c->d_u, u, sizeof(float)) != GEIST_HIP_OK)
-        return fail("upload of the draw", c->hs);
+    if (u != nullptr)
+        *c->d_u = *u;
     const struct geist_hip_rows rows = {
         .d_logits = c->d_row, .ld = n, .rows = 1, .n_vocab = n};
     const struct geist_hip_sample_params prm = {.temperature        = temperature,
@@ -152,10 +156,9 @@ static geist_token_t sample_one(struct dropin_ctx *c, size_t n, const float *log
     if (geist_hip_sample_rows(c->hs, &rows, &prm, u != nullptr ? c->d_u : nullptr, c->d_out) !=
         GEIST_HIP_OK)
         return fail("sampling", c->hs);
-    int32_t tok = -1;
-    if (geist_hip_download(c->hs, &tok, c->d_out, sizeof tok) != GEIST_HIP_OK)
-        return fail("download of the token id", c->hs);
-    return tok;
+    if (geist_hip_sampler_sync(c->hs) != GEIST_HIP_OK)
+        return fail("waiting for the token id", c->hs);
+    return *c->d_out;
 }
 
 /* ---- RNG: sampler.c:27-48, exact integer arithmetic, stays on the host -------------------- */

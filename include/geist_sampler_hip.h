@@ -266,6 +266,12 @@ int geist_hip_malloc(geist_hip_sampler *s, size_t bytes, void **d_ptr);
 int geist_hip_free(geist_hip_sampler *s, void *d_ptr);
 int geist_hip_upload(geist_hip_sampler *s, void *d_dst, const void *h_src, size_t bytes);   /* sync */
 int geist_hip_download(geist_hip_sampler *s, void *h_dst, const void *d_src, size_t bytes); /* sync */
+/* Page-locked host memory that the device reads and writes in place (the same pointer on both
+ * sides): a kernel's stores are in host memory once the stream has been waited for
+ * (geist_hip_sampler_sync), the host's stores are read by kernels launched afterwards. For the
+ * few words of results and arguments of a decode step, which then need no copy command. */
+int geist_hip_host_malloc(geist_hip_sampler *s, size_t bytes, void **h_ptr);
+int geist_hip_host_free(geist_hip_sampler *s, void *h_ptr);
 
 /* Diagnostics (no reference counterpart): after a full-vocabulary top-p / min-p call, which walk
  * served each row: 1 = shortcut over the per-thread maxima, 2 = candidate list, 3 = the whole
