@@ -91,6 +91,23 @@ __device__ __forceinline__ void remask_padding(const RowView &rv, int base, int 
 
 /* MASK = false compiles the allowed-token mask out (for callers that know rv.allowed is NULL and
  * are short of scalar registers). */
+template <int NV, bool MASK = true>
+__device__ __forceinline__ void mask_forbidden(const RowView &rv, int row, int base, int end,
+                                               float4 (&v)[NV]) {
+    if (MASK && rv.allowed) { /* forbidden tokens weigh nothing, whatever the transforms made */
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + (int) threadIdx.x);
+            if (e < end) {
+                const uint32_t ok = allowed_nibble(rv, row, e);
+                v[j].x = (ok & 1u) ? v[j].x : -INFINITY;
+                v[j].y = (ok & 2u) ? v[j].y : -INFINITY;
+                v[j].z = (ok & 4u) ? v[j].z : -INFINITY;
+                v[j].w = (ok & 8u) ? v[j].w : -INFINITY;
+            }
+        }
+    }
+}
 template <int NV, bool PEN, bool MASK = true>
 __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_rows, int base,
                                             int end, uint32_t *cnt16, float4 (&v)[NV]) {
@@ -106,19 +123,24 @@ __device__ __forceinline__ void fetch_chunk(const RowView &rv, int row, int n_ro
         apply_transform<NV>(rv, nullptr, v);
     }
     remask_padding<NV>(rv, base, end, v);
-    if (MASK && rv.allowed) { /* forbidden tokens weigh nothing, whatever the transforms made */
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int e = base + 4 * (j * TPB + (int) threadIdx.x);
-            if (e < end) {
-                const uint32_t ok = allowed_nibble(rv, row, e);
-                v[j].x = (ok & 1u) ? v[j].x : -INFINITY;
-                v[j].y = (ok & 2u) ? v[j].y : -INFINITY;
-                v[j].z = (ok & 4u) ? v[j].z : -INFINITY;
-                v[j].w = (ok & 8u) ? v[j].w : -INFINITY;
-            }
-        }
+    mask_forbidden<NV, MASK>(rv, row, base, end, v);
+}
+/* fetch_chunk() without its loads: `v` holds what load_raw() brought for the chunk. For a
+ * caller that asks for the next chunk before it works on this one. */
+template <int NV, bool PEN>
+__device__ __forceinline__ void transform_loaded_chunk(const RowView &rv, int row, int n_rows,
+                                                       int base, int end, uint32_t *cnt16,
+                                                       float4 (&v)[NV]) {
+    if (PEN) {
+        const HistPrefetch pf = history_prefetch(rv, row, n_rows);
+        history_clear<NV * TPB * 4>(cnt16);
+        history_count(rv, row, pf, base, end, cnt16);
+        apply_transform<NV>(rv, cnt16, v);
+    } else {
+        apply_transform<NV>(rv, nullptr, v);
     }
+    remask_padding<NV>(rv, base, end, v);
+    mask_forbidden<NV, true>(rv, row, base, end, v);
 }
 
 /* Row maximum from the per-chunk results; every thread returns the same packed value. */

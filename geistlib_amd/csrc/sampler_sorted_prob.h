@@ -382,6 +382,57 @@ __device__ __forceinline__ uint64_t block_sum_u64(uint64_t v, uint64_t *scratch)
     return r;
 }
 
+/* f(i, pn[i]) for every i < n, the workgroup's threads sharing the entries. Many loads of a
+ * thread are in flight together (eight of 16 bytes where pn is aligned, eight words otherwise):
+ * with one load and its use per turn a pass over a row of 128 k probabilities is 500 round
+ * trips to L2 one after the other, and the whole-row walk makes seven such passes; this way a
+ * pass that adds nothing to a histogram takes 16 us, about what one compute unit reads from L2.
+ * (The order in which entries are visited does not matter to the callers: integer sums and
+ * maxima.) */
+template <typename F>
+__device__ __forceinline__ void for_each_entry(const float *pn, int n, F &&f) {
+    int i = 0;
+    if ((((uintptr_t) pn) & 15) == 0) {
+        const float4 *p4 = reinterpret_cast<const float4 *>(pn);
+        const int     n4 = n >> 2;
+        int           g  = threadIdx.x;
+        for (; g + 7 * TPB < n4; g += 8 * TPB) {
+            float4 p[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                p[k] = p4[g + k * TPB];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int e = 4 * (g + k * TPB);
+                f(e, p[k].x);
+                f(e + 1, p[k].y);
+                f(e + 2, p[k].z);
+                f(e + 3, p[k].w);
+            }
+        }
+        for (; g < n4; g += TPB) {
+            const float4 q = p4[g];
+            f(4 * g, q.x);
+            f(4 * g + 1, q.y);
+            f(4 * g + 2, q.z);
+            f(4 * g + 3, q.w);
+        }
+        i = n4 << 2;
+    }
+    i += threadIdx.x;
+    for (; i + 7 * TPB < n; i += 8 * TPB) {
+        float p[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            p[k] = pn[i + k * TPB];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            f(i + k * TPB, p[k]);
+    }
+    for (; i < n; i += TPB)
+        f(i, pn[i]);
+}
+
 /* One descent. `limit_key`/`limit_ties`: only entries that precede the (limit_key, limit_ties)
  * edge of a previous descent take part -- entries with key > limit_key, plus the first
  * limit_ties (by index) of those equal to it, whose mass is limit_ties * fx(limit_key); pass
@@ -407,17 +458,16 @@ __device__ bool sg_descent(const float *pn, int n, uint64_t target, bool limited
             sh.mass[i] = 0ull;
         }
         __syncthreads();
-        for (int i = tid; i < n; i += TPB) {
-            const float    p   = pn[i];
+        for_each_entry(pn, n, [&](int, float p) {
             const uint32_t key = __float_as_uint(p);
             if ((key & mask) != prefix)
-                continue;
+                return;
             if (limited && key <= limit_key)
-                continue; /* entries equal to the limit are added below, as a block */
+                return; /* entries equal to the limit are added below, as a block */
             const uint32_t d = (key >> shf) & dm;
             atomicAdd(&sh.cnt[d], 1u);
             atomicAdd((unsigned long long *) &sh.mass[d], (unsigned long long) pn_fx(p));
-        }
+        });
         if (limited && tid == 0 && limit_ties && (limit_key & mask) == prefix) {
             const uint32_t d = (limit_key >> shf) & dm;
             atomicAdd(&sh.cnt[d], limit_ties);
@@ -549,20 +599,24 @@ __device__ int list_jth_id(const float *pn, const uint32_t *ids, int n, uint32_t
  * order, every entry of the row up to some z bin; no entry outside the list has a pn whose bits
  * exceed `kout`, so the walk is exact as long as the kept prefix ends strictly above kout --
  * otherwise -1 is returned and the row is walked in full. */
+/* `seen_max`: the largest key among the entries this thread has itself written to pn[] (the
+ * threads together having written all of them), or SEEN_NONE to have the maximum looked for. */
+constexpr uint32_t SEEN_NONE = 0xffffffffu;
 template <bool LIST>
 __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float top_p, float min_p,
                               float u, uint32_t kout, SortedGenShared &sh, int *s_scan,
-                              int *s_pick) {
+                              int *s_pick, uint32_t seen_max = SEEN_NONE) {
     const int  tid   = threadIdx.x;
     const bool use_p = top_p > 0.0f && top_p < 1.0f;
     const bool use_m = min_p > 0.0f;
 
     /* largest probability, then the min-p prefix: count and mass of pn >= min_p * pn_0 */
-    uint32_t kmax = 0u;
-    for (int i = tid; i < n; i += TPB) {
-        const uint32_t key = __float_as_uint(pn[i]);
-        kmax               = key > kmax ? key : kmax;
-    }
+    uint32_t kmax = seen_max != SEEN_NONE ? seen_max : 0u;
+    if (seen_max == SEEN_NONE)
+        for_each_entry(pn, n, [&](int, float p) {
+            const uint32_t key = __float_as_uint(p);
+            kmax               = key > kmax ? key : kmax;
+        });
     kmax = (uint32_t) block_max_u64((uint64_t) wave_max_u32(kmax), sh.red64);
     uint32_t n_m    = (uint32_t) n;
     uint64_t mass_m = 0;
@@ -570,13 +624,12 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
         const float floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
         uint64_t    lm      = 0;
         uint64_t    lc      = 0;
-        for (int i = tid; i < n; i += TPB) {
-            const float p = pn[i];
+        for_each_entry(pn, n, [&](int, float p) {
             if (p >= floor_w) {
                 lm += pn_fx(p);
                 ++lc;
             }
-        }
+        });
         mass_m = block_sum_u64(lm, sh.red64);
         n_m    = (uint32_t) block_sum_u64(lc, sh.red64);
         if (n_m < 1u) { /* cannot happen (pn_0 >= min_p * pn_0 for min_p <= 1); keep the max */
@@ -630,8 +683,7 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
         if (LIST)
             return -1;
         uint64_t lm = 0;
-        for (int i = tid; i < n; i += TPB)
-            lm += pn_fx(pn[i]);
+        for_each_entry(pn, n, [&](int, float p) { lm += pn_fx(p); });
         mass_keep = block_sum_u64(lm, sh.red64);
         limited   = false;
     }
@@ -651,14 +703,38 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
             j = ties_d;
         if (LIST) {
             tok = list_jth_id(pn, ids, n, kd, (int) j, sh, s_scan, s_pick);
+        } else if (j == 1) {
+            /* the first entry (index order) with pn == kd */
+            if (tid == 0)
+                *s_pick = 0x7fffffff;
+            __syncthreads();
+            for_each_entry(pn, n, [&](int i, float p) {
+                if (__float_as_uint(p) == kd)
+                    atomicMin(s_pick, i);
+            });
+            __syncthreads();
+            tok = *s_pick == 0x7fffffff ? -1 : *s_pick;
+            __syncthreads();
         } else {
             /* the j-th entry (index order) with pn == kd: each thread takes a contiguous range */
             const int span = (n + TPB - 1) / TPB;
             const int lo   = tid * span < n ? tid * span : n;
             const int hi   = lo + span < n ? lo + span : n;
             int       mine = 0;
-            for (int i = lo; i < hi; ++i)
-                mine += __float_as_uint(pn[i]) == kd;
+            {
+                int i = lo; /* (eight loads in flight, as in for_each_entry) */
+                for (; i + 8 <= hi; i += 8) {
+                    float p[8];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        p[k] = pn[i + k];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        mine += __float_as_uint(p[k]) == kd;
+                }
+                for (; i < hi; ++i)
+                    mine += __float_as_uint(pn[i]) == kd;
+            }
             const int incl = block_scan_i32(mine, s_scan, nullptr);
             if (tid == 0)
                 *s_pick = -1;
@@ -683,9 +759,10 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
         if (tid == 0)
             *s_pick = 0x7fffffff;
         __syncthreads();
-        for (int i = tid; i < n; i += TPB)
-            if (__float_as_uint(pn[i]) == kmax)
+        for_each_entry(pn, n, [&](int i, float p) {
+            if (__float_as_uint(p) == kmax)
                 atomicMin(s_pick, i);
+        });
         __syncthreads();
         tok = *s_pick == 0x7fffffff ? 0 : *s_pick;
     }
@@ -698,6 +775,24 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
  * normalised probabilities pn_i = (float)((double)p_i / sum) (sampler.c:246-253) into the probs
  * workspace, chunk by chunk, then walks them. Such rows are rare, so the row is not spread over
  * more workgroups. Called by every thread of a 256-thread workgroup. */
+/* (float) ((double) p / tot) without the division, rtot = 1 / tot: the quotient from the
+ * reciprocal and one correction step (the remainder is exact in the fused multiply-add) is the
+ * correctly rounded one or its neighbour, and both round to the same binary32 unless they lie
+ * within a few units of the middle between two of them, or the result is tiny, infinite or not
+ * a number: there the division itself decides. */
+__device__ __forceinline__ float quotient_f32(float p, double tot, double rtot) {
+    const double pd = (double) p;
+    double       q  = pd * rtot;
+    const double r  = __builtin_fma(-q, tot, pd);
+    q               = __builtin_fma(r, rtot, q);
+    const uint64_t b   = (uint64_t) __double_as_longlong(q);
+    const uint32_t low = (uint32_t) b & 0x1fffffffu; /* the 29 bits that a binary32 drops */
+    const int      ex  = (int) ((b >> 52) & 0x7ff);
+    if ((low - 0x0ffffffeu) <= 4u || ex < 1023 - 120 || ex == 0x7ff)
+        return (float) (pd / tot);
+    return (float) q;
+}
+
 struct SortedRowArgs {
     float           inv_t;
     const uint64_t *chunk_best;
@@ -722,13 +817,26 @@ __device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, in
         *s_total = t;
     }
     const float  mx = key2f(best_key(row_best_from_chunks(g.chunk_best, row, rv.n_chunks, sh.red64)));
-    const double tot = *s_total;
+    const double tot = *s_total, rtot = 1.0 / tot;
     float       *pn  = g.probs + (long) row * g.ld_probs;
+    const float *rowp = rv.logits + (long) row * rv.ld;
+    /* the next chunk's logits are asked for before this chunk is worked on */
+    float4   v[NV], vnext[NV];
+    uint32_t seen = 0u;
+    {
+        int base, end;
+        chunk_bounds<NV>(rv, 0, base, end);
+        load_raw<NV>(rv, rowp, base, end, v);
+    }
     for (int chunk = 0; chunk < rv.n_chunks; ++chunk) {
         int base, end;
         chunk_bounds<NV>(rv, chunk, base, end);
-        float4 v[NV];
-        fetch_chunk<NV, PEN>(rv, row, n_rows, base, end, s_cnt16, v);
+        if (chunk + 1 < rv.n_chunks) {
+            int nb, ne;
+            chunk_bounds<NV>(rv, chunk + 1, nb, ne);
+            load_raw<NV>(rv, rowp, nb, ne, vnext);
+        }
+        transform_loaded_chunk<NV, PEN>(rv, row, n_rows, base, end, s_cnt16, v);
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int e = base + 4 * (j * TPB + tid);
@@ -736,15 +844,21 @@ __device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, in
             for (int c = 0; c < 4; ++c) {
                 if (e + c < end) {
                     const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, g.inv_t), s_tab);
-                    pn[e + c]     = (float) ((double) p / tot);
+                    const float q = quotient_f32(p, tot, rtot);
+                    pn[e + c]     = q;
+                    seen          = __float_as_uint(q) > seen ? __float_as_uint(q) : seen;
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            v[j] = vnext[j];
         __syncthreads(); /* the history table is rebuilt for the next chunk */
     }
     __threadfence_block();
     __syncthreads();
-    return sorted_descend<false>(pn, nullptr, rv.n_vocab, top_p, min_p, u, 0u, sh, s_scan, s_pick);
+    return sorted_descend<false>(pn, nullptr, rv.n_vocab, top_p, min_p, u, 0u, sh, s_scan, s_pick,
+                                 seen);
 }
 
 /* ============================================================================================

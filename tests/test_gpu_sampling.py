@@ -285,6 +285,43 @@ def test_sorted_paths_all_three_in_one_batch(hs, oracle):
     assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
 
 
+@pytest.mark.parametrize("n,lead,pad", [(128256, 0, 0), (50001, 0, 0), (33333, 3, 5),
+                                        (70001, 1, 2)])
+def test_whole_row_walk_with_penalties_cap_and_mask(hs, oracle, n, lead, pad):
+    """Rows close to uniform, so that every one of them is walked in full, with everything the
+    walk's own pass over the logits has to apply: penalties from a history, the soft-cap, the
+    allowed-token mask; vocabularies that are no multiple of four and rows that start off a
+    16-byte boundary; nucleus and min-p. Row 1 is quantised (index order among equal
+    probabilities), row 2 has a few values far below the rest (tiny probabilities)."""
+    print(f"whole-row walk n={n} lead={lead} pad={pad}", flush=True)
+    g = np.random.default_rng(n + lead)
+    rows = 5
+    x = (g.standard_normal((rows, n)) * 0.4).astype(np.float32)
+    x[1] = np.round(x[1] * 4) / 4
+    x[2, g.integers(0, n, 50)] = -90.0
+    u = g.random(rows).astype(np.float32)
+    hist = g.integers(0, n, (rows, 300)).astype(np.int32)
+    hlen = np.array([300, 0, 17, 300, 128], dtype=np.int32)
+    allowed = g.random((rows, n)) < 0.8
+    allowed[3] = True
+    rep, freq, pres, cap = 1.3, 0.05, 0.1, 4.0
+    for kw in (dict(temperature=1.0, top_p=0.9), dict(temperature=0.8, top_p=0.95, min_p=1e-4)):
+        got = run_rows(hs, torch, x, u, P(rep=rep, freq=freq, pres=pres, softcap=cap, **kw),
+                       history=hist, history_len=hlen, lead=lead, pad=pad, allowed=allowed)
+        paths = hs.row_paths(rows).tolist()
+        want, infos = [], []
+        for r in range(rows):
+            row = oracle.penalties(x[r], hist[r, :hlen[r]], rep, freq, pres)
+            row = oracle.softcap(row, cap)
+            row[~allowed[r]] = -np.inf
+            t, i = oracle.chain_u(row, float(u[r]), **kw)
+            want.append(t)
+            infos.append(i)
+        near = compare_ids(got, want, infos, f"whole-row walk n={n} {kw}")
+        assert near <= 1
+        assert paths == [3] * rows, paths
+
+
 def test_logits_hint_changes_nothing_but_the_loads(hs, oracle):
     """GEIST_HIP_LOGITS_STREAMED: non-temporal loads in the single-pass modes, identical ids."""
     from geistlib_amd.binding import GeistHipError
