@@ -887,6 +887,20 @@ def main():
         hs.sync()
         lat.append((time.perf_counter() - t1) * 1e6)
     lat.sort()
+    # the same with the ids landing in page-locked host memory (the kernels write them there in
+    # place): from the call to token ids the host can read, no copy in between
+    lat_host = []
+    if not args.cold_only:
+        out_host = hs.host_buffer(w.rows * 4)
+        ids_host = out_host.view(np.int32)
+        for i in range(200):
+            t1 = time.perf_counter()
+            hs.sample(rows_cold[i % n_copies], prm, d_u, out_host)
+            hs.sync()
+            lat_host.append((time.perf_counter() - t1) * 1e6)
+        lat_host.sort()
+        assert ids_host.tolist() == d_out.cpu().numpy().tolist()
+        out_host.close()
 
     alg_bytes = w.algorithmic_bytes()
     # the streaming kernel's own share of those bytes: every logit once
@@ -922,6 +936,8 @@ def main():
         "input_copies_rotated": n_copies,
         "prewarm_steps": prewarm,
         "step_latency_us_median": round(lat[len(lat) // 2], 2) if lat else None,
+        "step_latency_ids_on_host_us_median": (round(lat_host[len(lat_host) // 2], 2)
+                                               if lat_host else None),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic[0], "traffic_source": traffic[1],

@@ -96,6 +96,8 @@ def load_library():
     lib.geist_hip_free.argtypes = [vp, vp]
     lib.geist_hip_upload.argtypes = [vp, vp, vp, sz]
     lib.geist_hip_download.argtypes = [vp, vp, vp, sz]
+    lib.geist_hip_host_malloc.argtypes = [vp, sz, C.POINTER(vp)]
+    lib.geist_hip_host_free.argtypes = [vp, vp]
     lib.geist_hip_sampler_row_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_sampler_topk_paths.argtypes = [vp, vp, sz]
     lib.geist_hip_logprob_rows.argtypes = [vp, vp, sz, sz, sz, f32, vp, sz, sz, vp, sz]
@@ -141,6 +143,31 @@ def load_library():
 
 def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+class HostBuffer:
+    """Page-locked host memory that the device addresses in place (geist_hip_host_malloc): pass it
+    where a device tensor is expected (it has data_ptr()), read or write it through view()."""
+
+    def __init__(self, sampler, nbytes):
+        self.sampler, self.nbytes = sampler, int(nbytes)
+        p = C.c_void_p()
+        sampler._check(sampler.lib.geist_hip_host_malloc(sampler.h, self.nbytes, C.byref(p)))
+        self.p = p
+
+    def data_ptr(self):
+        return self.p.value
+
+    def view(self, dtype):
+        import numpy as np
+        dtype = np.dtype(dtype)
+        buf = (C.c_char * self.nbytes).from_address(self.p.value)
+        return np.frombuffer(buf, dtype=dtype, count=self.nbytes // dtype.itemsize)
+
+    def close(self):
+        if self.p and self.sampler.h:
+            self.sampler.lib.geist_hip_host_free(self.sampler.h, self.p)
+        self.p = C.c_void_p()
 
 
 def sample_rows_static(rows, params, uniforms, out, device=0, stream=None):
@@ -199,6 +226,9 @@ class HipSampler:
 
     def sync(self):
         self._check(self.lib.geist_hip_sampler_sync(self.h))
+
+    def host_buffer(self, nbytes):
+        return HostBuffer(self, nbytes)
 
     def set_logits_hint(self, streamed):
         """streamed=True: the rows come from HBM and are read once (non-temporal loads in the

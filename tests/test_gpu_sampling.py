@@ -322,6 +322,30 @@ def test_whole_row_walk_with_penalties_cap_and_mask(hs, oracle, n, lead, pad):
         assert paths == [3] * rows, paths
 
 
+def test_ids_and_draws_in_page_locked_host_memory(hs):
+    """geist_hip_host_malloc: the kernels write the ids into host memory and read the draws from
+    it, in place; the ids equal those of the same call with device buffers, for every mode that
+    has a kernel of its own to finish a row."""
+    from geistlib_amd import HipSampler
+    x, u = rows_rng(77, 24, 50000, scale=3.0)
+    out_h, u_h = hs.host_buffer(24 * 4), hs.host_buffer(24 * 4)
+    try:
+        u_h.view(np.float32)[:] = u
+        d = to_dev(x, torch)
+        for prm in (P(temperature=0.0), P(temperature=0.9), P(temperature=0.7, top_k=40),
+                    P(temperature=0.7, top_k=40, top_p=0.9), P(temperature=1.0, top_p=0.9),
+                    P(temperature=1.0, min_p=0.05), P(temperature=1.0, top_p=0.9, precedence=0)):
+            want = run_rows(hs, torch, x, u, prm)
+            ids = out_h.view(np.int32)
+            ids[:] = -7
+            hs.sample(HipSampler.rows(d), prm, u_h, out_h)
+            hs.sync()
+            assert ids.tolist() == want.tolist(), prm
+    finally:
+        out_h.close()
+        u_h.close()
+
+
 def test_logits_hint_changes_nothing_but_the_loads(hs, oracle):
     """GEIST_HIP_LOGITS_STREAMED: non-temporal loads in the single-pass modes, identical ids."""
     from geistlib_amd.binding import GeistHipError
