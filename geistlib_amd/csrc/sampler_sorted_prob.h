@@ -775,24 +775,6 @@ __device__ int sorted_descend(const float *pn, const uint32_t *ids, int n, float
  * normalised probabilities pn_i = (float)((double)p_i / sum) (sampler.c:246-253) into the probs
  * workspace, chunk by chunk, then walks them. Such rows are rare, so the row is not spread over
  * more workgroups. Called by every thread of a 256-thread workgroup. */
-/* (float) ((double) p / tot) without the division, rtot = 1 / tot: the quotient from the
- * reciprocal and one correction step (the remainder is exact in the fused multiply-add) is the
- * correctly rounded one or its neighbour, and both round to the same binary32 unless they lie
- * within a few units of the middle between two of them, or the result is tiny, infinite or not
- * a number: there the division itself decides. */
-__device__ __forceinline__ float quotient_f32(float p, double tot, double rtot) {
-    const double pd = (double) p;
-    double       q  = pd * rtot;
-    const double r  = __builtin_fma(-q, tot, pd);
-    q               = __builtin_fma(r, rtot, q);
-    const uint64_t b   = (uint64_t) __double_as_longlong(q);
-    const uint32_t low = (uint32_t) b & 0x1fffffffu; /* the 29 bits that a binary32 drops */
-    const int      ex  = (int) ((b >> 52) & 0x7ff);
-    if ((low - 0x0ffffffeu) <= 4u || ex < 1023 - 120 || ex == 0x7ff)
-        return (float) (pd / tot);
-    return (float) q;
-}
-
 struct SortedRowArgs {
     float           inv_t;
     const uint64_t *chunk_best;
@@ -844,7 +826,7 @@ __device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, in
             for (int c = 0; c < 4; ++c) {
                 if (e + c < end) {
                     const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, g.inv_t), s_tab);
-                    const float q = quotient_f32(p, tot, rtot);
+                    const float q = geist_quotient_f32(p, tot, rtot);
                     pn[e + c]     = q;
                     seen          = __float_as_uint(q) > seen ? __float_as_uint(q) : seen;
                 }
