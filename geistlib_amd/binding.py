@@ -82,6 +82,7 @@ def load_library():
     lib.geist_hip_sampler_prepare.argtypes = [vp, C.POINTER(SampleParams), sz]
     lib.geist_hip_sampler_set_wait_limit.argtypes = [vp, C.c_uint32]
     lib.geist_hip_sampler_one_launch_topk.argtypes = [vp, i32]
+    lib.geist_hip_sampler_one_launch_spec.argtypes = [vp, i32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -212,6 +213,14 @@ class HipSampler:
     def one_launch_topk(self, enable=True):
         """Whether the top-k candidate path runs as one launch for batches that qualify."""
         rc = self.lib.geist_hip_sampler_one_launch_topk(self.h, 1 if enable else 0)
+        if rc < 0:
+            self._check(rc)
+        return bool(rc)
+
+    def one_launch_spec(self, enable=True):
+        """Whether stochastic verification sums the residual and draws in one launch for
+        batches that qualify."""
+        rc = self.lib.geist_hip_sampler_one_launch_spec(self.h, 1 if enable else 0)
         if rc < 0:
             self._check(rc)
         return bool(rc)

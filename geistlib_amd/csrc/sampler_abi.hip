@@ -45,6 +45,8 @@ struct geist_hip_sampler {
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     int32_t   *row_arrive = nullptr; /* per row: how many of its workgroups have scanned (k_cand_scan_final) */
     int        fused_wg_limit = 0;   /* largest grid that kernel is used for */
+    bool       spec_one_launch = true; /* residual sums and draw of spec verification in one launch */
+    int        cu_count = 0;
     int        fused_wg_default = 0; /* ... as the device allows */
     MeetState  meet_own;             /* where the workgroups of the one-pass exp-sum kernel meet */
     MeetState *meet      = &meet_own; /* (the allocation-free entry point shares one per device) */
@@ -315,6 +317,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
         bool same = false;
         if (e == hipSuccess)
             e = placement_of(device, s->stream, &same);
+        s->cu_count         = cus;
         s->fused_wg_default = same ? cus : 0; /* one workgroup of 1024 threads per compute unit */
         s->fused_wg_limit   = s->fused_wg_default;
     }
@@ -747,6 +750,13 @@ int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable) {
         return GEIST_HIP_E_INVALID_ARG;
     s->fused_wg_limit = enable ? s->fused_wg_default : 0;
     return s->fused_wg_limit > 0 ? 1 : 0;
+}
+
+int geist_hip_sampler_one_launch_spec(geist_hip_sampler *s, int enable) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->spec_one_launch = enable != 0;
+    return s->spec_one_launch ? 1 : 0;
 }
 
 int geist_hip_sampler_prepare(geist_hip_sampler *s, const struct geist_hip_sample_params *params,
@@ -1547,7 +1557,17 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     sp.verdict    = s->verdict;
     sp.out_tokens = d_out_tokens;
     sp.n_accepted = d_n_accepted;
-    launch_spec(La, sp);
+    /* the residual pass and the draw in one launch while its workgroups, at the two per compute
+     * unit their registers allow, run in one round; past that the two kernels are the lighter */
+    if (!greedy && s->spec_one_launch &&
+        n_seq * (size_t) La.rv.n_chunks <= (size_t) gs::SPEC_ONE_LAUNCH_WGS_PER_CU * (size_t) s->cu_count) {
+        Launch per_seq = La;
+        per_seq.rows   = (int) n_seq;
+        const MeetSpace m = meet_space(s, per_seq);
+        launch_spec(La, sp, &m);
+    } else {
+        launch_spec(La, sp);
+    }
     return after_launch(s, "spec verification");
 }
 

@@ -25,7 +25,8 @@ namespace gs {
 /* A wavefront's share of a chunk's slab sums: sum j over the lanes of Σ_c expf(arg) of group j,
  * into s_sum[w * NV + j]. NV == 8 goes through the wavefront's 8 x 64 table `tr` in LDS (see
  * expsum_chunk), NV == 2 through two DPP scans: the same operations in the same order as the
- * SLABS form of expsum_chunk. */
+ * SLABS form of expsum_chunk. On return v[] holds the weights themselves (expf of each element's
+ * argument; 0 at positions beyond the row, which were -inf) in place of the logits. */
 template <int NV>
 __device__ __forceinline__ void chunk_slab_totals(float4 (&v)[NV], float mx, float inv_t,
                                                   const uint64_t *s_tab, double *s_tr,
@@ -37,12 +38,14 @@ __device__ __forceinline__ void chunk_slab_totals(float4 (&v)[NV], float mx, flo
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
         double a4;
+        float  pw[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const double p =
-                (double) geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+            pw[c]          = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, inv_t), s_tab);
+            const double p = (double) pw[c];
             a4 = c == 0 ? p : a4 + p;
         }
+        v[j] = make_float4(pw[0], pw[1], pw[2], pw[3]); /* kept for the walk */
         if (TRANSPOSED)
             tr[j * WAVE + (lane ^ j)] = a4;
         else
@@ -264,24 +267,27 @@ __device__ __forceinline__ void draw_chunk(const RowView &rv, int row, int chunk
         return; /* another workgroup's */
     const double target = sh.walk.target;
     double       carry  = sh.walk.before;
-    const int    js     = sh.walk.slab;
+    const int    js     = __builtin_amdgcn_readfirstlane(sh.walk.slab);
     int          end_w  = end;
     bool         found  = false;
     if (from_registers) {
-        /* this chunk's slabs from the registers, from slab js on */
+        /* the located slab's weights, which the summation left in the registers (one workgroup
+         * of the row comes here and fetches this code from memory, at tens of nanoseconds per
+         * cache line: the exponentials taken again here took longer to fetch than to run).
+         * Should rounding have left the target beyond the slab, the walk goes on through the
+         * row from memory. */
+        float4 vs = v[0];
 #pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int sbase = base + j * 4 * TPB;
-            if (j < js || found || sbase >= end)
-                continue; /* (the same for every thread) */
-            const int send = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
-            const int e    = sbase + 4 * tid;
-            float     w[4];
-            slab_weights<false>(v[j], v[j], e, send, mx, inv_t, 0.0, s_tab, w);
-            found = walk_slab_step<false>(w, e, send, target, carry, sh.walk);
-        }
-        if (!found) /* rounding left the target beyond this chunk: on through the row */
-            walk_from<NV, PEN, false>(rv, row, n_rows, C, chunk + 1, 0, carry, target, mx, inv_t,
+        for (int j = 1; j < NV; ++j)
+            if (j == js)
+                vs = v[j];
+        const int   sbase = base + js * 4 * TPB;
+        const int   send  = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
+        const int   e     = sbase + 4 * tid;
+        const float w[4]  = {vs.x, vs.y, vs.z, vs.w};
+        found = walk_slab_step<false>(w, e, send, target, carry, sh.walk);
+        if (!found)
+            walk_from<NV, PEN, false>(rv, row, n_rows, C, chunk, js + 1, carry, target, mx, inv_t,
                                       0.0, nullptr, false, -1, s_tab, s_cnt16, sh.walk, end_w);
     } else {
         walk_from<NV, PEN, false>(rv, row, n_rows, C, chunk, js, carry, target, mx, inv_t, 0.0,

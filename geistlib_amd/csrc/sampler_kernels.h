@@ -179,7 +179,10 @@ constexpr int SPEC_DRAFT_MAX      = 63;
 constexpr int NGRAM_SUFFIX_MAX    = 8;  /* session.c:455-456 */
 constexpr int NGRAM_DRAFT_MAX     = 16; /* GEIST_SPEC_KMAX_HARDCAP, session.c:515 */
 constexpr int SPEC_VERDICT_BYTES = 24;
-void launch_spec(const Launch &L, const SpecLaunch &sp);
+/* meet != NULL (stochastic verification only): the residual sums and the draw in one launch (the
+ * workgroups of a sequence wait for one another); NULL: two launches */
+void launch_spec(const Launch &L, const SpecLaunch &sp, const MeetSpace *meet = nullptr);
+constexpr int SPEC_ONE_LAUNCH_WGS_PER_CU = 2; /* what the one-launch kernel's 171 registers allow */
 /* chunk_best may be NULL when only the thread maxima are wanted */
 void launch_tmax_scan(const Launch &L, float *tmax, uint64_t *chunk_best,
                       int32_t *zero_per_row = nullptr);

@@ -1848,7 +1848,7 @@ void launch_temperature_draw(const Launch &L, float inv_t, const float *uniforms
         k_temperature_draw<2, false><<<grid, block, 0, L.stream>>>(L.rv, inv_t, uniforms, out, meet);
 }
 
-void launch_spec(const Launch &L, const SpecLaunch &sp) {
+void launch_spec(const Launch &L, const SpecLaunch &sp, const MeetSpace *meet) {
     SpecArgs a;
     a.L          = sp.L;
     a.greedy     = sp.greedy;
@@ -1869,6 +1869,13 @@ void launch_spec(const Launch &L, const SpecLaunch &sp) {
     SpecVerdict *vd = static_cast<SpecVerdict *>(sp.verdict);
     if (sp.greedy) {
         k_spec_accept<<<dim3(sp.n_seq), block, 0, L.stream>>>(L.rv, a, vd);
+    } else if (meet) { /* the residual and the draw in one launch */
+        const dim3 grid(L.rv.n_chunks, sp.n_seq);
+        if (L.nv == 8)
+            k_spec_resid_draw<8><<<grid, block, 0, L.stream>>>(L.rv, a, vd, *meet);
+        else
+            k_spec_resid_draw<2><<<grid, block, 0, L.stream>>>(L.rv, a, vd, *meet);
+        return;
     } else {
         const dim3 grid(L.rv.n_chunks, sp.n_seq);
         if (L.nv == 8)

@@ -15,6 +15,9 @@
  *   k_spec_resid   grid (chunks, n_seq): row sums and maxima, j*, the accepted ids and their
  *                  count (spec_accept_seq), then the sum of max(0, p - q) over its chunk of row j*
  *   k_spec_final   grid (n_seq): draws the last token
+ *   k_spec_resid_draw  grid (chunks, n_seq): the two above in one launch, for batches whose
+ *                  workgroups are all resident at once; the chunks of a sequence meet for their
+ *                  residual sums and the one in whose chunk the draw falls walks it from registers
  *   k_spec_accept  grid (n_seq): the verdicts alone, for the greedy mode (no residual)
  */
 #ifndef GEIST_SAMPLER_SPEC_H
@@ -69,6 +72,20 @@ __device__ __forceinline__ SpecVerdict spec_accept_seq(const RowView &rv, const 
     double   *s_sum  = sh.sum;
     uint64_t *s_best = sh.best;
     const int tid = threadIdx.x, C = rv.n_chunks, L = a.L;
+    /* what the test of position `tid` needs, asked for before the chunk results: the draft's
+     * probability is a read that depends on the draft id, and is under way while those results
+     * are fetched and combined */
+    int   x  = -1;
+    float uu = 0.0f, pp = 0.0f, qt = 0.0f;
+    if (tid < L) {
+        x = a.draft[(long) seq * L + tid];
+        if (!a.greedy) {
+            uu = a.uniforms[(long) seq * (L + 1) + tid];
+            pp = a.probe_p[(long) seq * (L + 1) + tid];
+            if (x >= 0 && x < rv.n_vocab)
+                qt = a.q ? a.q[((long) seq * L + tid) * a.ld_q + x] : 1.0f; /* NULL: point mass */
+        }
+    }
     const int part = tid & 15;
     for (int j = tid >> 4; j <= L; j += TPB / 16) {
         const long row = (long) seq * (L + 1) + j;
@@ -108,28 +125,24 @@ __device__ __forceinline__ SpecVerdict spec_accept_seq(const RowView &rv, const 
     if (tid < WAVE) {
     bool ok = true; /* lanes at or beyond L never reject */
     if (tid < L) {
-        const long row = (long) seq * (L + 1) + tid;
-        const int  x   = a.draft[(long) seq * L + tid];
         if (a.greedy) {
             /* a NaN at index 0 keeps the argmax at 0 (sampler.c:52-62) */
-            const float first = rv.logits[row * rv.ld];
+            const float first = rv.logits[((long) seq * (L + 1) + tid) * rv.ld];
             ok                = x == ((first != first) ? 0 : (int) best_idx(s_best[tid]));
         } else {
-            float pn = 0.0f, qt = 0.0f;
-            if (x >= 0 && x < rv.n_vocab) {
-                pn = (float) ((double) a.probe_p[row] / s_sum[tid]);
-                qt = a.q ? a.q[((long) seq * L + tid) * a.ld_q + x] : 1.0f; /* NULL: point mass */
-            }
-            ok = (double) a.uniforms[(long) seq * (L + 1) + tid] * (double) qt < (double) pn;
+            /* (a draft id outside the vocabulary has q = 0 and p = 0: rejected) */
+            const float pn =
+                x >= 0 && x < rv.n_vocab ? (float) ((double) pp / s_sum[tid]) : 0.0f;
+            ok = (double) uu * (double) qt < (double) pn;
         }
     }
     const uint64_t rej = __ballot(!ok);
     const int      js  = rej ? __ffsll((long long) rej) - 1 : L;
     if (publish && tid < js)
-        a.out_tokens[(long) seq * (L + 1) + tid] = a.draft[(long) seq * L + tid];
+        a.out_tokens[(long) seq * (L + 1) + tid] = x;
     if (tid == 0) {
-        const long  row   = (long) seq * (L + 1) + js;
-        const float first = rv.logits[row * rv.ld];
+        /* (the argmax is the greedy mode's answer; only there is the row's first logit read) */
+        const float first = a.greedy ? rv.logits[((long) seq * (L + 1) + js) * rv.ld] : 0.0f;
         SpecVerdict v;
         v.sum  = a.greedy ? 0.0 : s_sum[js];
         v.mx   = key2f(best_key(s_best[js]));
@@ -153,6 +166,32 @@ __global__ __launch_bounds__(TPB) void k_spec_accept(RowView rv, SpecArgs a, Spe
     (void) spec_accept_seq(rv, a, (int) blockIdx.x, sh, true, verdict);
 }
 
+/* The residual weights max(0, p - q) of chunk [base, end) of target row `row`, summed per slab
+ * over the workgroup: every thread receives the NV slab sums in acc[]; v[] returns the thread's
+ * weights themselves (group j: the four elements it owns in slab j), qv[] is scratch. */
+template <int NV>
+__device__ __forceinline__ void resid_chunk_sums(const RowView &rv, long row, int base, int end,
+                                                 const float *qrow, bool qvec, int qx, float mx,
+                                                 float inv_t, double sum, const uint64_t *s_tab,
+                                                 double *s_sum, float4 (&v)[NV], float4 (&qv)[NV],
+                                                 double (&acc)[NV]) {
+    const int tid = threadIdx.x;
+    load_raw<NV>(rv, rv.logits + row * rv.ld, base, end, v);
+    load_q_chunk<NV>(qrow, qvec, qx, base, end, qv);
+    apply_transform<NV>(rv, nullptr, v); /* the soft-cap, as in the passes before */
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        float w[4];
+        slab_weights<true>(v[j], qv[j], base + 4 * (j * TPB + tid), end, mx, inv_t, sum, s_tab, w);
+        acc[j] = (double) w[0];
+        acc[j] += (double) w[1];
+        acc[j] += (double) w[2];
+        acc[j] += (double) w[3];
+        v[j] = make_float4(w[0], w[1], w[2], w[3]);
+    }
+    block_sum_f64_multi<NV>(acc, s_sum);
+}
+
 /* ---- k_spec_resid ---------------------------------------------------------------------------- */
 template <int NV>
 __global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a, SpecVerdict *verdict) {
@@ -172,26 +211,15 @@ __global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a, Spec
     const long   row = (long) seq * (a.L + 1) + js;
     const float  mx  = vd.mx;
     const double sum = vd.sum;
-    int          base, end;
+    int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     float4       v[NV], qv[NV];
     const float *qrow = a.q ? a.q + ((long) seq * a.L + js) * a.ld_q : nullptr;
     const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
     const int    qx   = a.draft[(long) seq * a.L + js];
-    load_raw<NV>(rv, rv.logits + row * rv.ld, base, end, v);
-    load_q_chunk<NV>(qrow, qvec, qx, base, end, qv);
-    apply_transform<NV>(rv, nullptr, v); /* the soft-cap, as in the passes before */
-    double acc[NV];
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-        float w[4];
-        slab_weights<true>(v[j], qv[j], base + 4 * (j * TPB + tid), end, mx, a.inv_t, sum, s_tab, w);
-        acc[j] = (double) w[0];
-        acc[j] += (double) w[1];
-        acc[j] += (double) w[2];
-        acc[j] += (double) w[3];
-    }
-    block_sum_f64_multi<NV>(acc, s_sum);
+    double       acc[NV];
+    resid_chunk_sums<NV>(rv, row, base, end, qrow, qvec, qx, mx, a.inv_t, sum, s_tab, s_sum, v, qv,
+                         acc);
     if (tid == 0) {
         const long at  = (long) seq * rv.n_chunks + chunk;
         double     tot = 0.0;
@@ -202,6 +230,21 @@ __global__ __launch_bounds__(TPB) void k_spec_resid(RowView rv, SpecArgs a, Spec
         }
         a.resid_sum[at] = tot;
     }
+}
+
+/* A draw from p of target row `row` (the bonus token, or the fallback when the residual is
+ * empty): the temperature walk over the sums the exp-sum pass left. `s_w`: MAX_CHUNKS doubles. */
+template <int NV>
+__device__ __forceinline__ int spec_draw_from_p(const RowView &rv, const SpecArgs &a, long row,
+                                                float u, float mx, double sum, double *s_w,
+                                                const uint64_t *s_tab, WalkShared &s_walk) {
+    const int tid = threadIdx.x, C = rv.n_chunks;
+    if (tid < C)
+        s_w[tid] = a.chunk_sum[row * C + tid];
+    __syncthreads();
+    return index_order_walk<NV, false, false>(rv, (int) row, 0, s_w,
+                                              a.slab_sum + row * C * SLABS_MAX, C, u, mx, a.inv_t,
+                                              sum, nullptr, false, -1, s_tab, nullptr, s_walk);
 }
 
 /* ---- k_spec_final ---------------------------------------------------------------------------- */
@@ -244,17 +287,164 @@ __global__ __launch_bounds__(TPB) void k_spec_final(RowView rv, SpecArgs a,
                                                     mx, a.inv_t, sum, qrow, qvec, qx, s_tab,
                                                     nullptr, s_walk);
         } else {
-            if (tid < C)
-                s_w[tid] = a.chunk_sum[row * C + tid];
-            __syncthreads();
-            tok = index_order_walk<NV, false, false>(rv, (int) row, 0, s_w,
-                                                     a.slab_sum + row * C * SLABS_MAX, C, u, mx,
-                                                     a.inv_t, sum, nullptr, false, -1, s_tab,
-                                                     nullptr, s_walk);
+            tok = spec_draw_from_p<NV>(rv, a, row, u, mx, sum, s_w, s_tab, s_walk);
         }
     }
     if (tid == 0)
         a.out_tokens[(long) seq * (L + 1) + js] = tok;
+}
+
+/* ---- k_spec_resid_draw ----------------------------------------------------------------------- */
+/* k_spec_resid and k_spec_final in one launch (stochastic verification only). The workgroups of
+ * a sequence work out the verdict, sum the residual of their chunks, and meet for those sums
+ * (row_sums_meet, as the temperature draw's workgroups do); each then adds them up in chunk
+ * order and locates the draw with the same arithmetic on the same numbers, so exactly one finds
+ * it in its own chunk and walks that chunk from the registers it still holds. The sums, the
+ * location and the walk are those of the two kernels (resid_chunk_sums, walk_locate_chunk,
+ * walk_slab_step), so the token is the same bit for bit. A sequence whose drafts are all accepted,
+ * or whose residual is empty, has its token drawn from p by its first workgroup, from the sums of
+ * the exp-sum pass. A workgroup that gives up the wait forms the other chunks' sums itself (the
+ * same summation, so it still agrees with the others on the chunk) and walks from memory. */
+template <int NV>
+__global__ __launch_bounds__(TPB) void k_spec_resid_draw(RowView rv, SpecArgs a,
+                                                         SpecVerdict *verdict, MeetSpace meet) {
+    __shared__ double           s_sum[NWAVES * NV];
+    __shared__ uint64_t         s_tab[32];
+    __shared__ SpecAcceptShared s_acc;
+    __shared__ DrawShared       s_draw;
+    const int seq = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x, C = rv.n_chunks, L = a.L;
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    {
+        const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, n_wg = gridDim.x * gridDim.y;
+        for (uint32_t i = wg * TPB + tid; i < meet.stale_count; i += n_wg * TPB)
+            meet.stale[i] = 0;
+    }
+    const SpecVerdict vd  = spec_accept_seq(rv, a, seq, s_acc, chunk == 0, verdict);
+    const int         js  = vd.js;
+    const long        row = (long) seq * (L + 1) + js;
+    const float       u   = a.uniforms[(long) seq * (L + 1) + L];
+    const float       mx  = vd.mx;
+    const double      sum = vd.sum;
+    if (js >= L) { /* every draft accepted: the bonus token, a draw from p_L */
+        if (chunk != 0)
+            return;
+        const int tok = spec_draw_from_p<NV>(rv, a, row, u, mx, sum, s_draw.csum, s_tab, s_draw.walk);
+        if (tid == 0)
+            a.out_tokens[row] = tok;
+        return;
+    }
+    int base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    float4       v[NV], qv[NV];
+    const float *qrow = a.q ? a.q + ((long) seq * L + js) * a.ld_q : nullptr;
+    const bool   qvec = ((((uintptr_t) a.q) & 15) == 0) && (a.ld_q % 4 == 0);
+    const int    qx   = a.draft[(long) seq * L + js];
+    double       acc[NV];
+    resid_chunk_sums<NV>(rv, row, base, end, qrow, qvec, qx, mx, a.inv_t, sum, s_tab, s_sum, v, qv,
+                         acc);
+    if (tid == 0) {
+        double tot = 0.0;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            s_draw.slab[j] = acc[j];
+            tot += acc[j];
+        }
+        s_draw.total = tot;
+    }
+    __syncthreads();
+    row_sums_meet(meet.slots + (long) seq * C, chunk, C, s_draw.total, tid < WAVE, true,
+                  meet.wait_limit, s_draw);
+    const bool from_registers = s_draw.have_sums != 0;
+    if (!from_registers) {
+        /* not met: every other chunk's sum by this workgroup, with the same summation */
+        if (tid == 0)
+            s_draw.csum[chunk] = s_draw.total;
+        for (int c2 = 0; c2 < C; ++c2) {
+            if (c2 == chunk)
+                continue;
+            int b2, e2;
+            chunk_bounds<NV>(rv, c2, b2, e2);
+            double acc2[NV];
+            resid_chunk_sums<NV>(rv, row, b2, e2, qrow, qvec, qx, mx, a.inv_t, sum, s_tab, s_sum, v,
+                                 qv, acc2);
+            if (tid == 0) {
+                double tot = 0.0;
+#pragma unroll
+                for (int j = 0; j < NV; ++j)
+                    tot += acc2[j];
+                s_draw.csum[c2] = tot;
+            }
+        }
+        __syncthreads();
+    }
+    /* the residual's mass, added up as k_spec_final adds it */
+    double R = 0.0;
+    for (int c = 0; c < C; ++c)
+        R += s_draw.csum[c];
+    if (!(R > 0.0)) { /* p == q everywhere it matters: a draw from p */
+        if (chunk != 0)
+            return;
+        __syncthreads(); /* csum is about to hold the sums of p */
+        const int tok = spec_draw_from_p<NV>(rv, a, row, u, mx, sum, s_draw.csum, s_tab, s_draw.walk);
+        if (tid == 0)
+            a.out_tokens[row] = tok;
+        return;
+    }
+    /* where the draw falls: the same arithmetic in every workgroup of the sequence */
+    if (tid < WAVE) {
+        double    run, target;
+        const int at = walk_locate_chunk(s_draw.csum, C, u, &run, &target);
+        int       sl = 0;
+        if (at == chunk)
+            sl = walk_locate_slab<NV>(s_draw.slab, target, &run);
+        if (tid == 0) {
+            s_draw.walk.chunk    = at;
+            s_draw.walk.slab     = sl;
+            s_draw.walk.before   = run;
+            s_draw.walk.target   = target;
+            s_draw.walk.pick     = 0x7fffffff;
+            s_draw.walk.last_pos = -1;
+        }
+    }
+    __syncthreads();
+    if (s_draw.walk.chunk != chunk)
+        return; /* another workgroup's */
+    const double target = s_draw.walk.target;
+    double       carry  = s_draw.walk.before;
+    const int    sl     = __builtin_amdgcn_readfirstlane(s_draw.walk.slab);
+    int          end_w  = end;
+    bool         found  = false;
+    if (from_registers) {
+        /* the located slab's weights, which the summation left in the registers (few workgroups
+         * come here and each fetches this code from memory, at tens of nanoseconds per cache
+         * line: the exponentials and quotients taken again here took longer to fetch than to
+         * run). Should rounding have left the target beyond the slab, the walk goes on through
+         * the row from memory. */
+        float4 vs = v[0];
+#pragma unroll
+        for (int j = 1; j < NV; ++j)
+            if (j == sl)
+                vs = v[j];
+        const int   sbase = base + sl * 4 * TPB;
+        const int   send  = sbase + 4 * TPB < end ? sbase + 4 * TPB : end;
+        const int   e     = sbase + 4 * tid;
+        const float w[4]  = {vs.x, vs.y, vs.z, vs.w};
+        found = walk_slab_step<true>(w, e, send, target, carry, s_draw.walk);
+        if (!found)
+            walk_from<NV, false, true>(rv, (int) row, 0, C, chunk, sl + 1, carry, target, mx,
+                                       a.inv_t, sum, qrow, qvec, qx, s_tab, nullptr, s_draw.walk,
+                                       end_w);
+    } else {
+        walk_from<NV, false, true>(rv, (int) row, 0, C, chunk, sl, carry, target, mx, a.inv_t, sum,
+                                   qrow, qvec, qx, s_tab, nullptr, s_draw.walk, end_w);
+    }
+    __syncthreads();
+    int tok = s_draw.walk.pick;
+    if (tok == 0x7fffffff)
+        tok = s_draw.walk.last_pos >= 0 ? s_draw.walk.last_pos : end_w - 1;
+    if (tid == 0)
+        a.out_tokens[row] = tok;
 }
 
 } // namespace gs

@@ -125,18 +125,26 @@ __device__ __forceinline__ bool walk_slab_step(const float (&w)[4], int e, int s
     const double incl = block_scan_f64(part, sh.scan, &slab);
     double       run  = carry + (incl - part);
     int          lastpos = -1;
+    uint32_t     pick    = 0x7fffffffu;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         run += (double) w[c];
         if (w[c] > 0.0f)
             lastpos = e + c;
-        if (e + c < send && w[c] > 0.0f && target < run) {
-            atomicMin(&sh.pick, e + c);
-            break;
-        }
+        if (pick == 0x7fffffffu && e + c < send && w[c] > 0.0f && target < run)
+            pick = (uint32_t) (e + c); /* the thread's first: the running sum only grows */
     }
-    if (RESID && lastpos >= 0)
-        atomicMax(&sh.last_pos, lastpos);
+    /* one atomic per wavefront: nearly every thread has a last position to report, and 256
+     * atomics on one word of LDS took 4 us */
+    pick = ~wave_max_u32(~pick);
+    if (RESID)
+        lastpos = (int) wave_max_u32((uint32_t) (lastpos + 1)) - 1;
+    if ((threadIdx.x & (WAVE - 1)) == 0) {
+        if (pick != 0x7fffffffu)
+            atomicMin(&sh.pick, (int) pick);
+        if (RESID && lastpos >= 0)
+            atomicMax(&sh.last_pos, lastpos);
+    }
     __syncthreads();
     if (sh.pick != 0x7fffffff)
         return true;

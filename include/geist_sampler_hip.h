@@ -159,6 +159,14 @@ int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
  * qualify, 0 when not, negative on error. */
 int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable);
 
+/* No counterpart in the reference. Stochastic speculative verification sums the residual
+ * max(0, p - q) and draws from it in one launch (the workgroups of a sequence wait for one
+ * another's sums, the wait bounded by geist_hip_sampler_set_wait_limit) when sequences x chunks
+ * of 8192 logits is at most two per compute unit (512 on an MI355X), one round of that kernel's
+ * workgroups; otherwise, and with enable = 0, in two launches. Results are the same either way. Returns 1 when the one-launch
+ * form is in use for batches that qualify, 0 when not, negative on error. */
+int geist_hip_sampler_one_launch_spec(geist_hip_sampler *s, int enable);
+
 /* Sizes, ahead of the first sampling call, whatever workspace the configuration needs beyond
  * what geist_hip_sampler_create made -- the reference sizes its workspace when the options are
  * applied (transformer_session_apply_opts, src/archs/transformer/forward/step.c:398-409), so that

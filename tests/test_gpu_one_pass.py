@@ -103,6 +103,48 @@ def test_spec_verify_one_pass(hs, oracle, wait_limit):
             assert out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), (call, s)
 
 
+@pytest.mark.parametrize("n_seq,L,n,T", [(28, 8, 128256, 1.0), (7, 5, 50001, 0.8), (3, 63, 9000, 1.2),
+                                         (1, 4, 128256, 1.0), (40, 2, 20000, 1.0)])
+def test_spec_verify_one_launch_and_two_launches_agree(hs, oracle, n_seq, L, n, T):
+    """The residual sums and the draw in one launch (the workgroups of a sequence meet for their
+    sums and one of them walks its chunk from registers), in two launches, and in one launch
+    with every wait given up at once (each workgroup then forms the other chunks' sums itself):
+    the same accepted counts and tokens, equal to the oracle's. One sequence accepts every draft
+    (the bonus token), one is rejected where the residual is empty (the token is drawn from p)."""
+    from test_gpu_sampling import _run_spec, _spec_case
+    print(f"spec one launch n_seq={n_seq} L={L} n={n}", flush=True)
+    target, q, draft, u = _spec_case(n_seq * 31 + L, n_seq, L, n)
+    if n_seq >= 3:
+        # sequence 1: q == p on every row, so every draft is accepted whatever the draws
+        q[1] = np.stack([oracle.softmax_normalised(target[1, j], T)[0] for j in range(L)])
+        # sequence 2: at row 0 every q is one step above p and the draw is the largest there
+        # is, so the draft is rejected there and the residual max(0, p - q) is empty
+        q[2, 0] = np.nextafter(oracle.softmax_normalised(target[2, 0], T)[0], np.float32(2.0))
+        u[2, 0] = np.float32(1 - 2.0 ** -24)
+    results = []
+    try:
+        for one_launch, wait_limit in ((True, None), (False, None), (True, 0)):
+            hs.one_launch_spec(one_launch)
+            if wait_limit is not None:
+                hs.set_wait_limit(wait_limit)
+            results.append(_run_spec(hs, target, q, draft, u, T))
+    finally:
+        hs.one_launch_spec(True)
+        hs.set_wait_limit(65536)
+    for nacc, out in results[1:]:
+        assert np.array_equal(nacc, results[0][0]) and np.array_equal(out, results[0][1])
+    nacc, out = results[0]
+    seen = set()
+    for s in range(n_seq):
+        want_n, want = oracle.spec_verify(target[s], q[s], draft[s], u[s], T)
+        assert nacc[s] == want_n, (s, nacc[s], want_n)
+        assert out[s, :want_n + 1].tolist() == want[:want_n + 1].tolist(), (s, out[s], want)
+        seen.add(int(want_n))
+    print("  accepted lengths seen:", sorted(seen))
+    if n_seq >= 3:
+        assert nacc[1] == L and nacc[2] == 0
+
+
 @pytest.mark.parametrize("pen", [False, True])
 def test_min_p_lists_of_every_size(hs, oracle, pen):
     """The exp-sum pass stages a chunk's min-p candidates in LDS (2048 places per chunk): rows whose
