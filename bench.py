@@ -199,7 +199,7 @@ def bench_spec(w, args):
         "sequences_per_s": round(n_seq * args.steps / elapsed, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "whole step (three kernels)", "step_algorithmic_bytes": alg},
+                     "kernel": "whole step (two kernels)", "step_algorithmic_bytes": alg},
         "input_copies_rotated": n_copies,
         "accepted_lengths": sorted(nacc.cpu().numpy().tolist()),
     }

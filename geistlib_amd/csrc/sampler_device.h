@@ -14,7 +14,6 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "exact_quotient.h"
 #include "glibc_expf.h"
 #include "glibc_tanhf.h"
 #include "sampler_kernels.h"

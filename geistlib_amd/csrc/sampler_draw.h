@@ -271,11 +271,9 @@ __device__ __forceinline__ void draw_chunk(const RowView &rv, int row, int chunk
     int          end_w  = end;
     bool         found  = false;
     if (from_registers) {
-        /* the located slab's weights, which the summation left in the registers (one workgroup
-         * of the row comes here and fetches this code from memory, at tens of nanoseconds per
-         * cache line: the exponentials taken again here took longer to fetch than to run).
-         * Should rounding have left the target beyond the slab, the walk goes on through the
-         * row from memory. */
+        /* the located slab's weights, which the summation left in the registers: nothing is
+         * computed again. Should rounding have left the target beyond the slab, the walk goes
+         * on through the row from memory. */
         float4 vs = v[0];
 #pragma unroll
         for (int j = 1; j < NV; ++j)

@@ -799,7 +799,7 @@ __device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, in
         *s_total = t;
     }
     const float  mx = key2f(best_key(row_best_from_chunks(g.chunk_best, row, rv.n_chunks, sh.red64)));
-    const double tot = *s_total, rtot = 1.0 / tot;
+    const double tot = *s_total;
     float       *pn  = g.probs + (long) row * g.ld_probs;
     const float *rowp = rv.logits + (long) row * rv.ld;
     /* the next chunk's logits are asked for before this chunk is worked on */
@@ -826,7 +826,7 @@ __device__ __forceinline__ int sorted_general_row(const RowView &rv, int row, in
             for (int c = 0; c < 4; ++c) {
                 if (e + c < end) {
                     const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, g.inv_t), s_tab);
-                    const float q = geist_quotient_f32(p, tot, rtot);
+                    const float q = (float) ((double) p / tot);
                     pn[e + c]     = q;
                     seen          = __float_as_uint(q) > seen ? __float_as_uint(q) : seen;
                 }

@@ -416,11 +416,9 @@ __global__ __launch_bounds__(TPB) void k_spec_resid_draw(RowView rv, SpecArgs a,
     int          end_w  = end;
     bool         found  = false;
     if (from_registers) {
-        /* the located slab's weights, which the summation left in the registers (few workgroups
-         * come here and each fetches this code from memory, at tens of nanoseconds per cache
-         * line: the exponentials and quotients taken again here took longer to fetch than to
-         * run). Should rounding have left the target beyond the slab, the walk goes on through
-         * the row from memory. */
+        /* the located slab's weights, which the summation left in the registers: nothing is
+         * computed again. Should rounding have left the target beyond the slab, the walk goes
+         * on through the row from memory. */
         float4 vs = v[0];
 #pragma unroll
         for (int j = 1; j < NV; ++j)
