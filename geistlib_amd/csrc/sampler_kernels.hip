@@ -763,10 +763,19 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
             if (use_m && w >= floor_w)
                 ++cnt_m;
         }
-        if (use_p && first_p != 0x7fffffff)
-            atomicMin(&fs.n_p, first_p);
-        if (use_m && cnt_m)
-            atomicAdd(&fs.n_m, cnt_m);
+        /* one atomic per wavefront: every thread past the nucleus' end has a position to
+         * report, and that many atomics on one word of LDS take microseconds */
+        {
+            const uint32_t fp = ~wave_max_u32(~(uint32_t) first_p);
+            const int      wave_m =
+                __builtin_amdgcn_readlane(wave_scan_i32_dpp(cnt_m), WAVE - 1);
+            if ((tid & (WAVE - 1)) == 0) {
+                if (use_p && fp != 0x7fffffffu)
+                    atomicMin(&fs.n_p, (int) fp);
+                if (use_m && wave_m)
+                    atomicAdd(&fs.n_m, wave_m);
+            }
+        }
         __syncthreads();
         keep = fs.n_p;
         if (use_m) {
@@ -787,14 +796,18 @@ __device__ int finish_sorted(int n, const uint64_t *spack, float inv_t, float to
     __syncthreads();
     const double target = (double) u * fs.mass;
     {
-        double run = off;
+        double   run  = off;
+        uint32_t mine = 0x7fffffffu;
         for (int i = lo; i < hi && i < keep; ++i) {
             run += (double) GS_W(i);
             if (target < run) {
-                atomicMin(&fs.pick, i);
+                mine = (uint32_t) i;
                 break;
             }
         }
+        mine = ~wave_max_u32(~mine); /* (as above: one atomic per wavefront) */
+        if ((tid & (WAVE - 1)) == 0 && mine != 0x7fffffffu)
+            atomicMin(&fs.pick, (int) mine);
     }
     __syncthreads();
 #undef GS_P
