@@ -15,8 +15,8 @@
  *   k_spec_resid   grid (chunks, n_seq): row sums and maxima, j*, the accepted ids and their
  *                  count (spec_accept_seq), then the sum of max(0, p - q) over its chunk of row j*
  *   k_spec_final   grid (n_seq): draws the last token
- *   k_spec_resid_draw  grid (chunks, n_seq): the two above in one launch, for batches whose
- *                  workgroups are all resident at once; the chunks of a sequence meet for their
+ *   k_spec_resid_draw  grid (chunks, n_seq): the two above in one launch, for batches of up to
+ *                  two workgroups per compute unit; the chunks of a sequence meet for their
  *                  residual sums and the one in whose chunk the draw falls walks it from registers
  *   k_spec_accept  grid (n_seq): the verdicts alone, for the greedy mode (no residual)
  */
