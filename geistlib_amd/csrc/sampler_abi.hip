@@ -1535,8 +1535,10 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     else {
         Launch scan          = La;
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over whole rows */
+        /* no slab sums: of the n_seq * (L + 1) rows at most n_seq are drawn from, each by a
+         * workgroup that walks the located chunk from its start */
         if (launch_scan_expsum(scan, inv_t, s->tmax, s->chunk_best, s->chunk_sum, d_draft, (int) L,
-                               s->probe_p, nullptr, 0, s->slab_sum, meet_space(s, scan)))
+                               s->probe_p, nullptr, 0, nullptr, meet_space(s, scan)))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     }
     SpecLaunch sp{};
@@ -1553,7 +1555,7 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
     sp.probe_p    = s->probe_p;
     sp.resid_sum  = s->resid_sum;
     sp.resid_slab = s->resid_slab;
-    sp.slab_sum   = s->slab_sum;
+    sp.slab_sum   = nullptr;
     sp.verdict    = s->verdict;
     sp.out_tokens = d_out_tokens;
     sp.n_accepted = d_n_accepted;

@@ -38,7 +38,7 @@ struct SpecArgs {
     const float    *probe_p; /* unnormalised p_j(x_j) per target row */
     double         *resid_sum; /* [n_seq][chunks] */
     double         *resid_slab; /* [n_seq][chunks][SLABS_MAX] */
-    const double   *slab_sum;  /* [rows][chunks][SLABS_MAX] of the exp-sum pass */
+    const double   *slab_sum;  /* [rows][chunks][SLABS_MAX] of the exp-sum pass, or NULL */
     int32_t        *out_tokens; /* [n_seq][L+1] */
     int32_t        *n_accepted; /* [n_seq] */
 };
@@ -242,9 +242,11 @@ __device__ __forceinline__ int spec_draw_from_p(const RowView &rv, const SpecArg
     if (tid < C)
         s_w[tid] = a.chunk_sum[row * C + tid];
     __syncthreads();
-    return index_order_walk<NV, false, false>(rv, (int) row, 0, s_w,
-                                              a.slab_sum + row * C * SLABS_MAX, C, u, mx, a.inv_t,
-                                              sum, nullptr, false, -1, s_tab, nullptr, s_walk);
+    /* (the exp-sum pass of the verification keeps no slab sums: few rows are drawn from, and
+     * those by a workgroup that has nothing else to do) */
+    return index_order_walk<NV, false, false>(
+        rv, (int) row, 0, s_w, a.slab_sum ? a.slab_sum + row * C * SLABS_MAX : nullptr, C, u, mx,
+        a.inv_t, sum, nullptr, false, -1, s_tab, nullptr, s_walk);
 }
 
 /* ---- k_spec_final ---------------------------------------------------------------------------- */

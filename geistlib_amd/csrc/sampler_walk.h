@@ -192,7 +192,8 @@ __device__ __forceinline__ void walk_from(const RowView &rv, int row, int n_rows
 
 /* Walks row `row` in index order for the first element at which the running weight exceeds
  * u * (sum of chunk_w). chunk_w: C per-chunk weights in LDS; slab_w: the row's C * SLABS_MAX slab
- * weights in global memory; NV: slabs per chunk of the pass that wrote them; qrow / qx: the
+ * weights in global memory, or NULL where the pass did not keep them (the located chunk is then
+ * walked from its first slab); NV: slabs per chunk of the pass that wrote them; qrow / qx: the
  * draft probabilities of the residual walk (see load_q_chunk). Returns the id to
  * every thread. Should rounding leave the target beyond the located slab, the walk goes on through
  * the following slabs and chunks, as the reference's single loop does (sampler.c:93-99); past the
@@ -207,7 +208,8 @@ __device__ int index_order_walk(const RowView &rv, int row, int n_rows, const do
     if (tid < WAVE) {
         double    run, target;
         const int at = walk_locate_chunk(chunk_w, C, u, &run, &target);
-        const int js = walk_locate_slab<NV>(slab_w + at * SLABS_MAX, target, &run);
+        /* without slab weights the located chunk is walked from its first slab */
+        const int js = slab_w ? walk_locate_slab<NV>(slab_w + at * SLABS_MAX, target, &run) : 0;
         if (tid == 0) {
             sh.chunk    = at;
             sh.slab     = js;
