@@ -678,7 +678,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         }
         *stream_kernel = "k_scan_expsum";
         if (do_stream &&
-            launch_scan_expsum(scan, rs.inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0,
+            launch_scan_expsum(scan, rs.inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0,
                                nullptr, nullptr, 0, s->slab_sum, meet_space(s, scan)))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
         f.mode     = FINAL_TEMPERATURE;
@@ -711,9 +711,11 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
     Launch scan          = L;
     scan.rv.stream_loads = s->logits_streamed; /* the one pass over whole rows */
     if (do_stream &&
-        launch_scan_expsum(scan, rs.inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0,
-                           nullptr, f.minp_listed ? &f.cand : nullptr, zb_m, nullptr,
-                           meet_space(s, scan)))
+        /* (the thread maxima are the row-final kernel's; with the list walk coming first and
+         * alone nobody reads them) */
+        launch_scan_expsum(scan, rs.inv_t, f.minp_direct ? nullptr : s->tmax, s->chunk_best,
+                           s->chunk_sum, nullptr, 0, nullptr, f.minp_listed ? &f.cand : nullptr,
+                           zb_m, nullptr, meet_space(s, scan)))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     if (!do_tail)
         return after_launch(s, "exp-sum scan");
@@ -915,7 +917,7 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
         return fail(s, GEIST_HIP_E_INVALID_ARG, "ld_probs < n_vocab");
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
-    if (launch_scan_expsum(L, inv_t, s->tmax, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
+    if (launch_scan_expsum(L, inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
                            nullptr, 0, nullptr, meet_space(s, L)))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
@@ -1537,7 +1539,7 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
         scan.rv.stream_loads = s->logits_streamed; /* the one pass over whole rows */
         /* no slab sums: of the n_seq * (L + 1) rows at most n_seq are drawn from, each by a
          * workgroup that walks the located chunk from its start */
-        if (launch_scan_expsum(scan, inv_t, s->tmax, s->chunk_best, s->chunk_sum, d_draft, (int) L,
+        if (launch_scan_expsum(scan, inv_t, nullptr, s->chunk_best, s->chunk_sum, d_draft, (int) L,
                                s->probe_p, nullptr, 0, nullptr, meet_space(s, scan)))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     }

@@ -365,7 +365,8 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
         }
         if (base + 4 * tid >= end)
             tm = __builtin_nanf("");
-        fs.tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
+        if (fs.tmax) /* (wanted by the row-final kernel of the top-p path only) */
+            fs.tmax[((long) row * rv.n_chunks + chunk) * TPB + tid] = tm;
         /* the wavefront's best, then the chunk's: each wavefront deposits its own in LDS and
          * the one that arrives last (no barrier: the others need not wait for it) combines
          * them, reports the chunk's and waits for the row's */
