@@ -1204,14 +1204,31 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
     __shared__ int      s_scan[NWAVES];
     __shared__ int      s_pick;
     __shared__ uint32_t s_idx[CAND_LDS];
+    __shared__ double   s_csum[MAX_CHUNKS];
     const int row = blockIdx.x, tid = threadIdx.x;
-    const int flag = direct_sum ? 5 : row_flag[row];
+    /* what the first steps need from memory is asked for at once, not one wait after the other:
+     * the row's flag, the length of its list, the table of expf, the chunk sums (a thread each)
+     * and the first two list entries of every thread (within the row's CAND_CAP places whatever
+     * the length turns out to be) */
+    const int       flag = direct_sum ? 5 : row_flag[row];
+    const uint64_t  tabv = g_expf_tab[tid & 31];
+    const int       n    = cand.count[(long) row * CAND_COUNT_STRIDE];
+    const uint32_t *gk   = cand.key + (long) row * CAND_CAP;
+    const uint32_t *gi   = cand.idx + (long) row * CAND_CAP;
+    const double    csum = direct_sum && tid < n_chunks ? direct_sum[(long) row * n_chunks + tid] : 0.0;
+    const float     u_row = uniforms[row];
+    uint32_t        kpre[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+        kpre[q] = gk[q * TPB + tid];
     if (tid < 32)
-        s_tab[tid] = g_expf_tab[tid];
+        s_tab[tid] = tabv;
+    if (tid < MAX_CHUNKS)
+        s_csum[tid] = csum;
     __syncthreads();
     if (flag == 2) { /* sent past the list by the row-final kernel */
         const int t = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p,
-                                                  uniforms[row], sh.gen, s_cnt16, s_tab, s_scan,
+                                                  u_row, sh.gen, s_cnt16, s_tab, s_scan,
                                                   &s_pick, &s_total);
         if (tid == 0) {
             out[row]       = t;
@@ -1221,15 +1238,14 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
     }
     if (flag != 1 && flag != 4 && flag != 5)
         return;
-    const int n   = cand.count[(long) row * CAND_COUNT_STRIDE];
     int       tok = -1;
     double   sum  = 1.0;
     uint32_t kout = 0u;
     if (direct_sum) {
-        /* every thread adds the chunk sums in chunk order (the loads are broadcasts) */
+        /* every thread adds the chunk sums in chunk order */
         sum = 0.0;
         for (int c = 0; c < n_chunks; ++c)
-            sum += direct_sum[(long) row * n_chunks + c];
+            sum += s_csum[c];
         kout = __float_as_uint((float) ((double) direct_p_out / sum)) + 1u;
     } else {
         kout = cand.out_key[row];
@@ -1237,11 +1253,18 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
             sum = cand.row_sum[row];
     }
     if (n >= 1 && n <= CAND_CAP) {
-        const uint32_t *gk = cand.key + (long) row * CAND_CAP;
-        const uint32_t *gi = cand.idx + (long) row * CAND_CAP;
         /* flags 4, 5: the list holds the softmax arguments; p = expf(argument),
          * pn = (float)((double)p / sum), sampler.c:80, 251-253 */
-        for (int i0 = 0; i0 < n; i0 += 8 * TPB) { /* eight independent loads in flight per thread */
+#pragma unroll
+        for (int q = 0; q < 2; ++q) { /* the entries asked for at the start */
+            const int i = q * TPB + tid;
+            if (i < n)
+                s_key[i] = flag >= 4 ? __float_as_uint((float) ((double) geist_expf_glibc_le0(
+                                                                    __uint_as_float(kpre[q]), s_tab) /
+                                                                sum))
+                                     : kpre[q];
+        }
+        for (int i0 = 2 * TPB; i0 < n; i0 += 8 * TPB) { /* eight independent loads in flight per thread */
             uint32_t k[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q)
@@ -1264,10 +1287,10 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
         __syncthreads();
         gk = s_key;
         const float *keys = reinterpret_cast<const float *>(gk);
-        tok = list_walk_fast(keys, gi, n, top_p, min_p, uniforms[row], kout, sh.fast);
+        tok = list_walk_fast(keys, gi, n, top_p, min_p, u_row, kout, sh.fast);
         if (tok == -2) {
             __syncthreads();
-            tok = sorted_descend<true>(keys, gi, n, top_p, min_p, uniforms[row], kout, sh.gen,
+            tok = sorted_descend<true>(keys, gi, n, top_p, min_p, u_row, kout, sh.gen,
                                        s_scan, &s_pick);
         }
     }
@@ -1275,7 +1298,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
      * every thread) */
     int path = 2;
     if (tok < 0) {
-        tok  = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p, uniforms[row],
+        tok  = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p, u_row,
                                            sh.gen, s_cnt16, s_tab, s_scan, &s_pick, &s_total);
         path = 3;
     }
