@@ -83,6 +83,7 @@ def load_library():
     lib.geist_hip_sampler_set_wait_limit.argtypes = [vp, C.c_uint32]
     lib.geist_hip_sampler_one_launch_topk.argtypes = [vp, i32]
     lib.geist_hip_sampler_one_launch_spec.argtypes = [vp, i32]
+    lib.geist_hip_sampler_handoff_scope.argtypes = [vp, i32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -216,6 +217,11 @@ class HipSampler:
         if rc < 0:
             self._check(rc)
         return bool(rc)
+
+    def handoff_scope(self, always_agent=False):
+        """always_agent=True: the one-launch top-k kernel reads every row's hand-over with
+        agent-scope loads, as it does for a row whose workgroups ran on different XCDs."""
+        self._check(self.lib.geist_hip_sampler_handoff_scope(self.h, 1 if always_agent else 0))
 
     def one_launch_spec(self, enable=True):
         """Whether stochastic verification sums the residual and draws in one launch for

@@ -45,6 +45,8 @@ struct geist_hip_sampler {
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     int32_t   *row_arrive = nullptr; /* per row: how many of its workgroups have scanned (k_cand_scan_final) */
     int        fused_wg_limit = 0;   /* largest grid that kernel is used for */
+    bool       handoff_far = false;  /* that kernel reads the hand-over with agent-scope loads
+                                      * whatever the placement (geist_hip_sampler_handoff_scope) */
     bool       spec_one_launch = true; /* residual sums and draw of spec verification in one launch */
     int        cu_count = 0;
     int        fused_wg_default = 0; /* ... as the device allows */
@@ -170,6 +172,7 @@ static int make_launch(geist_hip_sampler *s, const struct geist_hip_rows *r,
     L.rv.pres      = pen ? p->presence_penalty : 0.0f;
     /* the soft-cap is monotone, so greedy rows skip it (head.c:145-149) */
     L.rv.softcap   = (p && stochastic && p->logit_softcap > 0.0f) ? p->logit_softcap : 0.0f;
+    L.rv.n_rows     = (int) r->rows;
     L.rv.allowed    = r->d_allowed;
     L.rv.allowed_ld = (long) r->allowed_ld;
     L.rows         = (int) r->rows;
@@ -633,21 +636,35 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
                            L.rv.n_chunks <= CAND_CHUNKS_MAX && (!L.pen || !scan.pen) &&
                            !s->tmax_ready && s->wcands && row_waves <= s->wcands_row_waves;
         const int m = plain ? cand_lanes_for(f.k_sel, rows->n_vocab) : 0;
-        if (m) {
-            const WaveCands wc = wave_cands_at(s->wcands, row_waves);
+        /* a batch that fits the device in one round of 1024-thread workgroups takes scan and
+         * row-final stage in one launch (the measuring stages cannot split it: the streaming
+         * stage is the whole step) */
+        const size_t wgs_row = (size_t) ((L.rv.n_chunks + 3) / 4);
+        const size_t wgs     = rows->rows * wgs_row;
+        const bool   one     = plain && s->row_arrive && rows->rows % 8 == 0 &&
+                             wgs <= (size_t) s->fused_wg_limit && rows->n_vocab % 4 == 0 &&
+                             wg_cands_bytes(rows->rows, wgs_row) <= wave_cands_bytes(s->wcands_row_waves);
+        const size_t per_wg  = 32768;
+        const size_t e_full  = rows->n_vocab < per_wg ? rows->n_vocab : per_wg;
+        const int    r_full  = one ? cand_rank_for(f.k_sel, rows->n_vocab, e_full) : 0;
+        const int    r_last  = one ? cand_rank_for(f.k_sel, rows->n_vocab,
+                                                   rows->n_vocab - (wgs_row - 1) * per_wg) : 0;
+        const int    r_w     = r_full && r_last ? r_full : 0;
+        if (r_w) {
             f.row_flag         = s->row_flag; /* which path served each row, for diagnostics */
             s->topk_paths_rows = rows->rows;
+            *stream_kernel     = "k_cand_scan_final";
+            if (do_stream)
+                launch_cand_scan_final(scan, L, f, s->tmax, wg_cands_at(s->wcands, rows->rows, wgs_row),
+                                       r_w, r_last, reinterpret_cast<uint32_t *>(s->row_arrive),
+                                       s->handoff_far);
+            return after_launch(s, "top-k");
+        }
+        if (m) {
+            const WaveCands wc = wave_cands_at(s->wcands, row_waves);
+            f.row_flag         = s->row_flag;
+            s->topk_paths_rows = rows->rows;
             *stream_kernel     = "k_cand_scan";
-            /* a batch that fits the device in one round of 1024-thread workgroups takes both
-             * kernels in one launch (the measuring stages cannot split it: the streaming stage
-             * is the whole step) */
-            const size_t wgs = rows->rows * (size_t) ((L.rv.n_chunks + 3) / 4);
-            if (s->row_arrive && rows->rows % 8 == 0 && wgs <= (size_t) s->fused_wg_limit) {
-                *stream_kernel = "k_cand_scan_final";
-                if (do_stream)
-                    launch_cand_scan_final(scan, L, f, s->tmax, wc, m, s->row_arrive);
-                return after_launch(s, "top-k");
-            }
             if (do_stream)
                 launch_cand_scan(scan, s->tmax, wc, m);
             if (do_tail)
@@ -752,6 +769,13 @@ int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable) {
         return GEIST_HIP_E_INVALID_ARG;
     s->fused_wg_limit = enable ? s->fused_wg_default : 0;
     return s->fused_wg_limit > 0 ? 1 : 0;
+}
+
+int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->handoff_far = always_agent != 0;
+    return GEIST_HIP_OK;
 }
 
 int geist_hip_sampler_one_launch_spec(geist_hip_sampler *s, int enable) {

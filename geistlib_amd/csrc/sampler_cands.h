@@ -564,53 +564,5 @@ __global__ __launch_bounds__(FC_THREADS) void k_final_cand(RowView rv, FinalArgs
     final_cand_row<NV, PEN, WIDE>(rv, a, wc, (int) blockIdx.x);
 }
 
-/* Scan and row-final in one launch, for batches that fit the device at one workgroup of 1024
- * threads per compute unit: a workgroup scans four chunks of its row (a wavefront does what it
- * does in k_cand_scan), and the workgroup of a row that finishes last goes on as the row's
- * k_final_cand. What that saves is the boundary between two kernels (about 1.2 us) and the wait
- * of the early rows for the late ones: a row's final starts when the row has been scanned.
- *
- * The handover goes through the L2 the row's workgroups share (the grid is dealt out so that
- * a row's workgroups run on one XCD; the host launches this kernel only with a multiple of 8
- * rows): every wavefront waits for its stores to be acknowledged, the workgroup adds one to the
- * row's counter (a device-scope atomic, its line the row's own), and the one that finds the
- * others' arrivals there invalidates its first-level cache and reads what they wrote. It also
- * puts the counter back to zero for the next launch. */
-template <int NV, bool PEN, bool WIDE>
-__global__ __launch_bounds__(FC_THREADS) void k_cand_scan_final(RowView rv_scan, RowView rv,
-                                                                float *__restrict__ tmax,
-                                                                WaveCands wc, int m, FinalArgs a,
-                                                                int32_t *__restrict__ arrive) {
-    __shared__ int s_last;
-    const int G   = (int) gridDim.x; /* workgroups per row */
-    const int lin = (int) (blockIdx.y * gridDim.x + blockIdx.x), slot = lin >> 3;
-    const int row = (lin & 7) + 8 * (slot / G), grp = slot % G;
-    const int chunk = (FC_THREADS / TPB) * grp + (int) (threadIdx.x / TPB);
-    if (chunk < rv_scan.n_chunks)
-        cand_scan_chunk<NV>(rv_scan, tmax, wc, m, row, chunk, (int) (threadIdx.x % TPB));
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int32_t  *ctr = arrive + (long) row * ARRIVE_STRIDE;
-        const int t   = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last        = t == G - 1;
-        if (t == G - 1)
-            __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last)
-        return;
-    asm volatile("buffer_inv sc0" ::: "memory"); /* the first-level cache only */
-    final_cand_row<NV, PEN, WIDE>(rv, a, wc, row);
-}
-
-/* Writes, per workgroup of a (gx, gy) grid of 1024 threads, the number of the XCD it runs on:
- * what the host checks before it trusts k_cand_scan_final's placement of a row's workgroups. */
-__global__ __launch_bounds__(FC_THREADS) void k_xcd_of_workgroups(int32_t *__restrict__ out) {
-    if (threadIdx.x == 0) /* hwreg 20 (XCC_ID), bits 3:0 */
-        out[blockIdx.y * gridDim.x + blockIdx.x] =
-            (int32_t) __builtin_amdgcn_s_getreg(((4 - 1) << 11) | (0 << 6) | 20);
-}
-
 } // namespace gs
 #endif

@@ -34,6 +34,7 @@ struct RowView {
     float          rep, freq, pres;
     double         inv_rep; /* 1.0 / (double) rep, see penalise() */
     float          softcap; /* 0 = off */
+    int            n_rows; /* rows of the batch (hist_len has that many entries) */
     const uint32_t *allowed;   /* NULL = no mask; bit e of a row's mask set = token e allowed */
     long            allowed_ld; /* words between rows, 0 = one mask for all rows */
 };
@@ -105,6 +106,38 @@ inline WaveCands wave_cands_at(void *base, size_t row_waves) {
     w.bound = reinterpret_cast<uint32_t *>(w.idx + row_waves * CAND_SLOTS);
     return w;
 }
+/* What the wavefronts of the one-launch form of that path (k_cand_scan_final) hand on to the
+ * workgroup that finishes the row: per scanning wavefront (16 per workgroup, G workgroups per row)
+ * OL_SLOTS float4 groups -- those that hold an element at or above the workgroup's bound T_w --
+ * with the index of each group's first element, and their number (more than OL_SLOTS: it had too
+ * many and the row cannot be certified); per workgroup the key of T_w. */
+constexpr int OL_TOP      = 8;   /* maxima a wavefront enters for its workgroup's bound */
+constexpr int OL_SLOTS    = 16;  /* groups a scanning wavefront may hand on */
+constexpr int OL_WG_MAX   = 8;   /* workgroups per row (CAND_CHUNKS_MAX chunks, four each) */
+constexpr int OL_RANK_MAX = 64;  /* largest rank `r` of the workgroup's bound the path is used for */
+struct WgCands {
+    float4   *val;   /* [rows][G][16][OL_SLOTS] the float4 groups */
+    uint32_t *idx;   /* [rows][G][16][OL_SLOTS] index of each group's first element */
+    uint32_t *count; /* [rows][G][16] */
+    uint32_t *bound; /* [rows][G] */
+};
+inline size_t wg_cands_bytes(size_t rows, size_t wgs_per_row) {
+    return rows * wgs_per_row * (16 * OL_SLOTS * 20 + 16 * sizeof(uint32_t) + sizeof(uint32_t));
+}
+inline WgCands wg_cands_at(void *base, size_t rows, size_t wgs_per_row) {
+    WgCands w;
+    w.val   = static_cast<float4 *>(base);
+    w.idx   = reinterpret_cast<uint32_t *>(w.val + rows * wgs_per_row * 16 * OL_SLOTS);
+    w.count = w.idx + rows * wgs_per_row * 16 * OL_SLOTS;
+    w.bound = w.count + rows * wgs_per_row * 16;
+    return w;
+}
+/* `r` for a workgroup that holds `elems` of a row's n_vocab logits, of which about k_eff lead:
+ * the smallest rank such that the workgroup holding that many of the k_eff is a one-in-10^8 event
+ * when the logits' order is unrelated to the vocabulary's (all of them when it holds the whole
+ * row). 0 = the one-launch form does not pay (r would exceed OL_RANK_MAX). */
+int cand_rank_for(int k_eff, size_t n_vocab, size_t elems);
+
 /* The final stage of that path keeps its candidates (at most 16 x 64 ids) in an open-addressing
  * table of HT_SLOTS slots in LDS and looks the row's token history up in it. */
 constexpr int HT_SLOTS       = 4096;
@@ -192,15 +225,19 @@ void launch_row_final(const Launch &L, const FinalLaunch &f);
  * kernel's) and also stores the thread maxima */
 void launch_cand_scan(const Launch &L, float *tmax, const WaveCands &wc, int m);
 void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &wc);
-/* both in one launch (k_cand_scan_final): L.rows a multiple of 8; `arrive` holds one zeroed
- * counter per row, ARRIVE_STRIDE_INTS apart, and is left zeroed */
+/* both in one launch (k_cand_scan_final): `arrive` holds one zeroed counter per row,
+ * ARRIVE_STRIDE_INTS apart, and is left zeroed; `tmax` receives the thread maxima of the rows that
+ * fall back to the slower paths. r_w / r_last: the rank of the bound of a full workgroup and of
+ * the row's last one (cand_rank_for). far_always: read the hand-over with agent-scope loads whatever
+ * the placement of the row's workgroups (for tests of that branch). */
 constexpr int ARRIVE_STRIDE_INTS = 32;
 /* *same_xcd: workgroups of a grid whose linear ids are equal modulo 8 run on one XCD (and so
- * share an L2), which launch_cand_scan_final relies on. Runs a small kernel and waits for it.
- * Returns a hipError_t value. */
+ * share an L2): then launch_cand_scan_final hands a row over through that L2. Runs a small
+ * kernel and waits for it. Returns a hipError_t value. */
 int probe_workgroup_placement(hipStream_t stream, bool *same_xcd);
 void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
-                            const WaveCands &wc, int m, int32_t *arrive);
+                            const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
+                            bool far_always);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */

@@ -998,7 +998,7 @@ __device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int 
         __syncthreads();
         for (int base = 0; base < n; base += TILE) {
             const int end = base + TILE < n ? base + TILE : n;
-            fetch_chunk<NV, PEN, MASK>(rv, row, (int) gridDim.x, base, end, cnt16, v);
+            fetch_chunk<NV, PEN, MASK>(rv, row, rv.n_rows, base, end, cnt16, v);
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
                 const int e = base + 4 * (j * TPB + tid);
@@ -1026,7 +1026,7 @@ __device__ __forceinline__ int topk_row_general(const RowView &rv, int row, int 
     int ties_before = 0;
     for (int base = 0; base < n; base += TILE) {
         const int end = base + TILE < n ? base + TILE : n;
-        fetch_chunk<NV, PEN, MASK>(rv, row, (int) gridDim.x, base, end, cnt16, v);
+        fetch_chunk<NV, PEN, MASK>(rv, row, rv.n_rows, base, end, cnt16, v);
         int ties_here = 0;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
@@ -1138,7 +1138,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
     const int C   = rv.n_chunks;
     HistPrefetch pf;
     if (PEN)
-        pf = history_prefetch(rv, row, (int) gridDim.x);
+        pf = history_prefetch(rv, row, rv.n_rows);
     /* 1 */
     const float *tm = a.tmax + (long) row * C * TPB + tid;
     float        raw[KPT];
@@ -1359,6 +1359,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #include "sampler_spec.h"
 #include "sampler_draft.h"
 #include "sampler_cands.h"
+#include "sampler_cands_one_launch.h"
 namespace gs {
 
 /* ============================================================================================
@@ -1974,26 +1975,39 @@ void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &w
     }
 }
 
-void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
-                            const WaveCands &wc, int m, int32_t *arrive) {
-    const FinalArgs a = final_args(f);
-    const int       per_wg = FC_THREADS / TPB; /* chunks a workgroup scans */
-    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, L.rows), block(FC_THREADS);
-    if (L.rv.n_chunks <= 16) { /* up to 64 scanning wavefronts per row */
-        if (L.pen)
-            k_cand_scan_final<8, true, false><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
-                                                                          m, a, arrive);
-        else
-            k_cand_scan_final<8, false, false><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax,
-                                                                           wc, m, a, arrive);
-    } else {
-        if (L.pen)
-            k_cand_scan_final<8, true, true><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
-                                                                         m, a, arrive);
-        else
-            k_cand_scan_final<8, false, true><<<grid, block, 0, L.stream>>>(scan.rv, L.rv, tmax, wc,
-                                                                          m, a, arrive);
+int cand_rank_for(int k_eff, size_t n_vocab, size_t elems) {
+    if (k_eff < 1 || elems == 0 || elems > n_vocab)
+        return 0;
+    int r = k_eff; /* the workgroup holds the whole row */
+    if (elems < n_vocab) {
+        /* P(X >= r) <= 1e-8 for X ~ Binomial(k_eff, share) */
+        const double share = (double) elems / (double) n_vocab;
+        double       p = std::pow(1.0 - share, k_eff), cdf = p;
+        int          x = 0;
+        while (1.0 - cdf > 1e-8 && x < k_eff) {
+            p *= (double) (k_eff - x) / (double) (x + 1) * share / (1.0 - share);
+            ++x;
+            cdf += p;
+        }
+        r = x + 1 < k_eff ? x + 1 : k_eff;
     }
+    return r <= OL_RANK_MAX ? r : 0;
+}
+
+void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
+                            const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
+                            bool far_always) {
+    const FinalArgs a = final_args(f);
+    const int       per_wg = OL_THREADS / TPB; /* chunks a workgroup scans */
+    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, L.rows), block(OL_THREADS);
+    auto go = [&](auto kernel) {
+        kernel<<<grid, block, 0, L.stream>>>(scan.rv, L.rv, wc, r_w, r_last, a, tmax, arrive,
+                                             far_always ? 1 : 0);
+    };
+    if (L.pen)
+        scan.rv.stream_loads ? go(k_cand_scan_final<true, true>) : go(k_cand_scan_final<true, false>);
+    else
+        scan.rv.stream_loads ? go(k_cand_scan_final<false, true>) : go(k_cand_scan_final<false, false>);
 }
 
 int probe_workgroup_placement(hipStream_t stream, bool *same_xcd) {
@@ -2006,7 +2020,7 @@ int probe_workgroup_placement(hipStream_t stream, bool *same_xcd) {
     hipError_t e = hipMalloc((void **) &d, n * sizeof(int32_t));
     if (e != hipSuccess)
         return (int) e;
-    k_xcd_of_workgroups<<<dim3(gx, gy), dim3(FC_THREADS), 0, stream>>>(d);
+    k_xcd_of_workgroups<<<dim3(gx, gy), dim3(OL_THREADS), 0, stream>>>(d);
     e = hipMemcpyAsync(h, d, n * sizeof(int32_t), hipMemcpyDeviceToHost, stream);
     if (e == hipSuccess)
         e = hipStreamSynchronize(stream);

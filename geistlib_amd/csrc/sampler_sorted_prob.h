@@ -129,7 +129,7 @@ __device__ __forceinline__ int sorted_from_tmax(const RowView &rv, const FinalAr
     const bool use_m = a.min_p > 0.0f;
     HistPrefetch pf;
     if (PEN)
-        pf = history_prefetch(rv, row, (int) gridDim.x);
+        pf = history_prefetch(rv, row, rv.n_rows);
     /* 1 */
     const float *tm = a.tmax + (long) row * C * TPB + tid;
     float        raw[KPT];
@@ -1227,7 +1227,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
         s_csum[tid] = csum;
     __syncthreads();
     if (flag == 2) { /* sent past the list by the row-final kernel */
-        const int t = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p,
+        const int t = sorted_general_row<NV, PEN>(rv, row, rv.n_rows, g, top_p, min_p,
                                                   u_row, sh.gen, s_cnt16, s_tab, s_scan,
                                                   &s_pick, &s_total);
         if (tid == 0) {
@@ -1298,7 +1298,7 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
      * every thread) */
     int path = 2;
     if (tok < 0) {
-        tok  = sorted_general_row<NV, PEN>(rv, row, (int) gridDim.x, g, top_p, min_p, u_row,
+        tok  = sorted_general_row<NV, PEN>(rv, row, rv.n_rows, g, top_p, min_p, u_row,
                                            sh.gen, s_cnt16, s_tab, s_scan, &s_pick, &s_total);
         path = 3;
     }

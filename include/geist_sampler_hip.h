@@ -153,11 +153,21 @@ int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
 /* No counterpart in the reference. The top-k candidate path runs as one launch (the workgroup of
  * a row that finishes scanning last goes on as the row's final stage) when the batch is a
  * multiple of 8 rows, fits the device in one round of workgroups and the device places the
- * workgroups of a row where they share a second-level cache (looked at once per device);
- * otherwise as two launches. Results are the same either way. enable = 0 keeps to two launches,
- * 1 returns to the default. Returns 1 when the one-launch form is in use for batches that
- * qualify, 0 when not, negative on error. */
+ * workgroups of a row where they share a second-level cache (looked at once per device: it
+ * decides which form is faster, not whether the one launch is correct -- every launch checks the
+ * placement of each row for itself, see geist_hip_sampler_handoff_scope); otherwise as two
+ * launches. Results are the same either way. enable = 0 keeps to two launches, 1 returns to the
+ * default. Returns 1 when the one-launch form is in use for batches that qualify, 0 when not,
+ * negative on error. */
 int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable);
+
+/* No counterpart in the reference. In the one-launch form the workgroups of a row hand their
+ * candidates to the one that finishes the row. Each arrival reports the XCD it ran on; when all
+ * of a row ran on one XCD the finishing workgroup reads the hand-over from the second-level cache
+ * they share, otherwise with agent-scope loads (the hand-over is always written with agent-scope
+ * stores). always_agent = 1 makes every row take the second branch whatever its placement -- for
+ * tests of that branch; 0 returns to the default. Results are the same either way. */
+int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent);
 
 /* No counterpart in the reference. Stochastic speculative verification sums the residual
  * max(0, p - q) and draws from it in one launch (the workgroups of a sequence wait for one

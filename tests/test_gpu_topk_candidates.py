@@ -31,10 +31,11 @@ def units(g, rows):
     return (g.integers(0, 1 << 24, rows).astype(np.float32) / np.float32(1 << 24)).astype(np.float32)
 
 
-def want_rows(oracle, x, u, hist=None, pen=None, **kw):
+def want_rows(oracle, x, u, hist=None, pen=None, hist_len=None, **kw):
     res = []
     for r in range(x.shape[0]):
-        row = x[r] if hist is None else oracle.penalties(x[r], hist[r], *pen)
+        h = None if hist is None else (hist[r] if hist_len is None else hist[r][:hist_len[r]])
+        row = x[r] if hist is None else oracle.penalties(x[r], h, *pen)
         res.append(oracle.chain_u(row, float(u[r]), **kw))
     return [t for t, _ in res], [i for _, i in res]
 
@@ -78,7 +79,9 @@ def test_rows_the_candidates_cannot_certify(hs, oracle):
     want, infos = want_rows(oracle, x, u, temperature=0.8, top_k=k, top_p=0.95)
     compare_ids(got, want, infos, "rows passed on")
     print("paths:", paths)
-    assert paths[0] != 0 and paths[1] != 0 and paths[2] != 0 and paths[3] != 0 and paths[4] != 0
+    # (the cluster of row 1 and the short runs of equal values of row 2 are within what some forms
+    # of the path hand on and beyond others)
+    assert paths[0] != 0 and paths[3] != 0 and paths[4] != 0
     assert paths[5] == 0 and paths[7] == 0 and all(p == 0 for p in paths[8:])
 
 
@@ -254,15 +257,24 @@ def test_one_launch_and_two_launches_agree(hs, oracle, pen):
             x[8 + call, :] = np.round(x[8 + call])      # runs of equal values
             x[16 + call, :] = 0.5                       # all equal: whole-row selection
             u = units(g, rows)
-            hl = None if hist is None else np.full(rows, hist.shape[1], dtype=np.int32)
+            # every row its own history length: the slower paths read the length of THEIR row
+            hl = None if hist is None else g.integers(0, hist.shape[1] + 1, rows).astype(np.int32)
             want, infos = want_rows(oracle, x, u, hist=hist, pen=pen_t, temperature=0.7, top_k=k,
-                                    top_p=0.9)
-            for one in (True, False):
+                                    top_p=0.9, hist_len=hl)
+            # one launch with the hand-over read from the shared second-level cache (where the
+            # placement allows), one launch with every row treated as spread over XCDs, two launches
+            for one, far in ((True, False), (True, True), (False, False)):
                 hs.one_launch_topk(one)
+                hs.handoff_scope(far)
                 got = run_rows(hs, torch, x, u, P(temperature=0.7, top_k=k, top_p=0.9, **pk),
                                history=hist, history_len=hl)
-                compare_ids(got, want, infos, f"call {call} one launch {one}")
+                compare_ids(got, want, infos, f"call {call} one launch {one} far {far}")
                 paths = hs.topk_paths(rows).tolist()
                 assert paths[call] != 0 and paths[16 + call] != 0, paths
+                if far:   # no row trusts what the others handed on: all served from the logits
+                    assert all(p != 0 for p in paths), paths
+                else:
+                    assert sum(p == 0 for p in paths) >= rows - 8, paths
     finally:
         hs.one_launch_topk(True)
+        hs.handoff_scope(False)
