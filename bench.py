@@ -900,6 +900,16 @@ def main():
             lat_host.append((time.perf_counter() - t1) * 1e6)
         lat_host.sort()
         assert ids_host.tolist() == d_out.cpu().numpy().tolist()
+        # the same measured from C, call to ids readable on the host (clock_gettime around
+        # geist_hip_sample_rows + the wait), first with the wait for the stream, then with the
+        # sampler telling the host when the ids are written (geist_hip_sampler_notify_ids /
+        # _wait_ids): the figure a caller of the synchronous entry points sees
+        lat_c_sync = sorted(bh.step_latency(hs, rows_cold, prm, d_u, out_host, 200, wait_ids=False))
+        hs.notify_ids(True)
+        bh.step_latency(hs, rows_cold, prm, d_u, out_host, 20, wait_ids=True)
+        lat_c_wait = sorted(bh.step_latency(hs, rows_cold, prm, d_u, out_host, 200, wait_ids=True))
+        hs.notify_ids(False)
+        assert ids_host.tolist() == d_out.cpu().numpy().tolist()
         out_host.close()
 
     alg_bytes = w.algorithmic_bytes()
@@ -936,6 +946,12 @@ def main():
         "input_copies_rotated": n_copies,
         "prewarm_steps": prewarm,
         "step_latency_us_median": round(lat[len(lat) // 2], 2) if lat else None,
+        "step_latency_from_c_stream_wait_us_median": (round(lat_c_sync[len(lat_c_sync) // 2], 2)
+                                                      if lat_host else None),
+        "step_latency_from_c_ids_on_host_us_median": (round(lat_c_wait[len(lat_c_wait) // 2], 2)
+                                                      if lat_host else None),
+        "step_latency_from_c_ids_on_host_us_p90": (round(lat_c_wait[len(lat_c_wait) * 9 // 10], 2)
+                                                   if lat_host else None),
         "step_latency_ids_on_host_us_median": (round(lat_host[len(lat_host) // 2], 2)
                                                if lat_host else None),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,

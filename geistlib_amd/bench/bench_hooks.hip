@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <time.h>
 #include <cstring>
 #include <new>
 
@@ -119,6 +120,27 @@ int geist_bench_time_stream_kernel(geist_hip_sampler *s, void *stream,
     if (kernel_name && kernel_name_len)
         snprintf(kernel_name, kernel_name_len, "%s", name);
     return rc;
+}
+
+int geist_bench_step_latency(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                             size_t n_batches, const struct geist_hip_sample_params *params,
+                             const float *d_uniforms, geist_hip_token_t *out_tokens, int wait_ids,
+                             int samples, double *us_each) {
+    if (!s || !rows || n_batches < 1 || samples < 1 || !us_each)
+        return GEIST_HIP_E_INVALID_ARG;
+    for (int i = 0; i < samples; ++i) {
+        struct timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        int rc = geist_hip_sample_rows(s, &rows[(size_t) i % n_batches], params, d_uniforms,
+                                       out_tokens);
+        if (rc == GEIST_HIP_OK)
+            rc = wait_ids ? geist_hip_sampler_wait_ids(s) : geist_hip_sampler_sync(s);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        if (rc != GEIST_HIP_OK)
+            return rc;
+        us_each[i] = (double) (t1.tv_sec - t0.tv_sec) * 1e6 + (double) (t1.tv_nsec - t0.tv_nsec) * 1e-3;
+    }
+    return GEIST_HIP_OK;
 }
 
 int geist_bench_time_plain_read(void *stream, const struct geist_hip_rows *rows, size_t n_batches,

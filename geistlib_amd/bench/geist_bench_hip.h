@@ -30,6 +30,15 @@ int geist_bench_time_stream_kernel(geist_hip_sampler *s, void *stream,
                                    int launches, double *ms_total, char *kernel_name,
                                    size_t kernel_name_len);
 
+/* One-step latency measured from C: `samples` times geist_hip_sample_rows on rows[i % n_batches]
+ * followed by geist_hip_sampler_wait_ids (wait_ids != 0) or geist_hip_sampler_sync, each timed
+ * with clock_gettime(CLOCK_MONOTONIC) from before the call to after the wait; us_each receives
+ * the microseconds of every sample. */
+int geist_bench_step_latency(geist_hip_sampler *s, const struct geist_hip_rows *rows,
+                             size_t n_batches, const struct geist_hip_sample_params *params,
+                             const float *d_uniforms, geist_hip_token_t *out_tokens, int wait_ids,
+                             int samples, double *us_each);
+
 /* Calibration: the same loop around a kernel that only reads the rows (8192 logits per workgroup
  * of 256 threads, 16-byte loads, non-temporal when `streamed`) and stores nothing: the floor of
  * any one-pass kernel over these bytes on this device. */

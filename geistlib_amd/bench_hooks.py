@@ -20,6 +20,8 @@ def _lib():
                                                        C.POINTER(C.c_double), C.c_char_p, sz]
         lib.geist_bench_time_plain_read.argtypes = [vp, C.POINTER(Rows), sz, i32, i32,
                                                     C.POINTER(C.c_double)]
+        lib.geist_bench_step_latency.argtypes = [vp, C.POINTER(Rows), sz, C.POINTER(SampleParams),
+                                                 vp, vp, i32, i32, C.POINTER(C.c_double)]
         _LIB = lib
     return _LIB
 
@@ -58,6 +60,19 @@ def time_stream_kernel(sampler, rows_list, params, uniforms, out, launches, stre
     if rc:
         raise GeistHipError(rc, sampler.lib.geist_hip_sampler_last_error(sampler.h).decode())
     return ms.value * 1e3 / launches, name.value.decode()
+
+
+def step_latency(sampler, rows_list, params, uniforms, out, samples, wait_ids):
+    """Microseconds of `samples` single steps, each from before geist_hip_sample_rows to after
+    geist_hip_sampler_wait_ids (wait_ids=True) or geist_hip_sampler_sync, timed in C."""
+    arr = (Rows * len(rows_list))(*rows_list)
+    us = (C.c_double * samples)()
+    rc = _lib().geist_bench_step_latency(sampler.h, arr, len(rows_list), C.byref(params),
+                                         _ptr(uniforms), _ptr(out), int(bool(wait_ids)),
+                                         int(samples), us)
+    if rc:
+        raise GeistHipError(rc, sampler.lib.geist_hip_sampler_last_error(sampler.h).decode())
+    return list(us)
 
 
 def time_plain_read(rows_list, launches, streamed, stream=None):

@@ -84,6 +84,9 @@ def load_library():
     lib.geist_hip_sampler_one_launch_topk.argtypes = [vp, i32]
     lib.geist_hip_sampler_one_launch_spec.argtypes = [vp, i32]
     lib.geist_hip_sampler_handoff_scope.argtypes = [vp, i32]
+    lib.geist_hip_sampler_notify_ids.argtypes = [vp, i32]
+    lib.geist_hip_sampler_wait_ids.argtypes = [vp]
+    lib.geist_hip_sampler_set_wait_spin.argtypes = [vp, C.c_uint32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
                                               vp]
@@ -222,6 +225,17 @@ class HipSampler:
         """always_agent=True: the one-launch top-k kernel reads every row's hand-over with
         agent-scope loads, as it does for a row whose workgroups ran on different XCDs."""
         self._check(self.lib.geist_hip_sampler_handoff_scope(self.h, 1 if always_agent else 0))
+
+    def notify_ids(self, enable=True):
+        """Every sampling call reports into page-locked memory when its ids are written."""
+        self._check(self.lib.geist_hip_sampler_notify_ids(self.h, 1 if enable else 0))
+
+    def wait_ids(self):
+        """Returns when the ids of the last sampling call are written (see notify_ids)."""
+        self._check(self.lib.geist_hip_sampler_wait_ids(self.h))
+
+    def set_wait_spin(self, microseconds):
+        self._check(self.lib.geist_hip_sampler_set_wait_spin(self.h, microseconds))
 
     def one_launch_spec(self, enable=True):
         """Whether stochastic verification sums the residual and draws in one launch for

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <pthread.h>
+#include <time.h>
 
 #include <cstdarg>
 #include <cstdio>
@@ -45,6 +46,13 @@ struct geist_hip_sampler {
     uint64_t *chunk_best = nullptr; /* [max_rows][max_chunks] */
     int32_t   *row_arrive = nullptr; /* per row: how many of its workgroups have scanned (k_cand_scan_final) */
     int        fused_wg_limit = 0;   /* largest grid that kernel is used for */
+    /* geist_hip_sampler_notify_ids: every sampling call reports when its ids are written */
+    bool       notify = false;
+    uint64_t  *h_done = nullptr;     /* page-locked: the epoch of the last call whose ids are written */
+    uint64_t   epoch = 0;            /* of the last call enqueued */
+    uint32_t  *rows_done = nullptr;  /* device counter of the one-launch top-k kernel */
+    bool       epoch_by_kernel = false; /* the call being enqueued reports from its own kernel */
+    uint32_t   wait_spin_us = 2000;  /* geist_hip_sampler_wait_ids: how long it watches the word */
     bool       handoff_far = false;  /* that kernel reads the hand-over with agent-scope loads
                                       * whatever the placement (geist_hip_sampler_handoff_scope) */
     bool       spec_one_launch = true; /* residual sums and draw of spec verification in one launch */
@@ -358,6 +366,9 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->chunk_best);
     (void) hipFree(s->chunk_sum);
     (void) hipFree(s->row_arrive);
+    (void) hipFree(s->rows_done);
+    if (s->h_done)
+        (void) hipHostFree(s->h_done);
     (void) hipFree(s->meet_own.slots[0]);
     (void) hipFree(s->meet_own.slots[1]);
     (void) hipFree(s->resid_sum);
@@ -503,7 +514,17 @@ static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t word
 static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                        const struct geist_hip_sample_params *params, const float *d_uniforms,
                        geist_hip_token_t *d_out) {
-    return gs_host::sample_stages(s, rows, params, d_uniforms, d_out, gs_host::STAGE_ALL, nullptr);
+    if (s)
+        s->epoch_by_kernel = false;
+    const int rc = gs_host::sample_stages(s, rows, params, d_uniforms, d_out, gs_host::STAGE_ALL, nullptr);
+    if (rc == GEIST_HIP_OK && s->notify && s->h_done) {
+        /* the ids of this call are written when the word holds this epoch */
+        const Notify nt = {s->h_done, s->epoch + 1, s->rows_done};
+        if (!s->epoch_by_kernel)
+            launch_publish_epoch(s->stream, nt);
+        s->epoch += 1;
+    }
+    return rc;
 }
 
 /* The buffers of the full-vocabulary top-p / min-p path (a row of probabilities per logit row
@@ -654,10 +675,16 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
             f.row_flag         = s->row_flag; /* which path served each row, for diagnostics */
             s->topk_paths_rows = rows->rows;
             *stream_kernel     = "k_cand_scan_final";
+            /* with both stages in this call, the kernel itself reports the ids written */
+            Notify nt = {nullptr, 0, nullptr};
+            if (s->notify && s->h_done && s->rows_done && do_stream && do_tail) {
+                nt                 = Notify{s->h_done, s->epoch + 1, s->rows_done};
+                s->epoch_by_kernel = true;
+            }
             if (do_stream)
                 launch_cand_scan_final(scan, L, f, s->tmax, wg_cands_at(s->wcands, rows->rows, wgs_row),
                                        r_w, r_last, reinterpret_cast<uint32_t *>(s->row_arrive),
-                                       s->handoff_far);
+                                       s->handoff_far, nt);
             return after_launch(s, "top-k");
         }
         if (m) {
@@ -775,6 +802,64 @@ int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     s->handoff_far = always_agent != 0;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_notify_ids(geist_hip_sampler *s, int enable) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (enable && !s->h_done) {
+        HIPCHK(s, hipSetDevice(s->device));
+        uint64_t *h = nullptr;
+        uint32_t *d = nullptr;
+        hipError_t e = hipHostMalloc((void **) &h, 64, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipMalloc((void **) &d, 64);
+        if (e == hipSuccess) e = hipMemsetAsync(d, 0, 64, s->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
+        if (e != hipSuccess) {
+            if (h) (void) hipHostFree(h);
+            if (d) (void) hipFree(d);
+            return fail(s, e == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND,
+                        "the word that reports written ids: %s", hipGetErrorString(e));
+        }
+        *h           = 0;
+        s->h_done    = h;
+        s->rows_done = d;
+    }
+    s->notify = enable != 0;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_wait_ids(geist_hip_sampler *s) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (s->notify && s->h_done && s->epoch != 0) {
+        const volatile uint64_t *w = s->h_done;
+        struct timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        for (;;) {
+            for (int i = 0; i < 256; ++i) {
+                if (*w >= s->epoch) {
+                    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+                    return GEIST_HIP_OK;
+                }
+                __builtin_ia32_pause();
+            }
+            clock_gettime(CLOCK_MONOTONIC, &t1);
+            const double us = (double) (t1.tv_sec - t0.tv_sec) * 1e6 + (double) (t1.tv_nsec - t0.tv_nsec) * 1e-3;
+            if (us > (double) s->wait_spin_us)
+                break;
+        }
+    }
+    /* not told within the time (or telling is off): wait for the stream, which also reports a
+     * failed launch or kernel */
+    return geist_hip_sampler_sync(s);
+}
+
+int geist_hip_sampler_set_wait_spin(geist_hip_sampler *s, uint32_t microseconds) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    s->wait_spin_us = microseconds;
     return GEIST_HIP_OK;
 }
 

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
                                                                 FinalArgs a,
                                                                 float *__restrict__ tmax_rw,
                                                                 uint32_t *__restrict__ arrive,
-                                                                int far_always) {
+                                                                int far_always, Notify nt) {
     /* the table of the row's history (PEN): OL_HT_SLOTS ids and as many 16-bit counters */
     constexpr int ARENA_HT = PEN ? OL_HT_SLOTS * 6 : 16;
     constexpr int ARENA = ARENA_HT > FallbackArena<8, PEN>::END ? ARENA_HT
@@ -273,23 +273,23 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
     }
     lds_barrier();
     /* T_w: sixteen leading key bits of the r-th largest of the 128 entered maxima (at least r lane
-     * maxima reach it). Every entry is ranked by counting, eight lanes to an entry, sixteen
-     * comparisons a lane; the one of rank r - 1 is it. A workgroup with fewer than r maxima -- a
-     * few elements at the row's end -- finds an empty entry there and hands on all it has. */
+     * maxima reach it). Every wavefront ranks the eight it entered itself: a lane holds two of the
+     * 128, an entry travels as a scalar, and two ballots count the entries above it; the entry of
+     * rank r - 1 is it. A workgroup with fewer than r maxima -- a few elements at the row's end --
+     * finds an empty entry there and hands on all it has. */
     {
-        const uint32_t mine = s_top[tid >> 3];
-        const uint4   *q    = reinterpret_cast<const uint4 *>(s_top) + 4 * (tid & 7);
-        const uint4    q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
-        int c = (int) (q0.x > mine) + (int) (q0.y > mine) + (int) (q0.z > mine) + (int) (q0.w > mine) +
-                (int) (q1.x > mine) + (int) (q1.y > mine) + (int) (q1.z > mine) + (int) (q1.w > mine) +
-                (int) (q2.x > mine) + (int) (q2.y > mine) + (int) (q2.z > mine) + (int) (q2.w > mine) +
-                (int) (q3.x > mine) + (int) (q3.y > mine) + (int) (q3.z > mine) + (int) (q3.w > mine);
-        c += __builtin_amdgcn_update_dpp(0, c, 0x111, 0xf, 0xf, false); /* row_shr:1 */
-        c += __builtin_amdgcn_update_dpp(0, c, 0x112, 0xf, 0xf, false); /* row_shr:2 */
-        c += __builtin_amdgcn_update_dpp(0, c, 0x114, 0xf, 0xf, false); /* row_shr:4 */
-        const int r = grp == G - 1 ? r_last : r_w; /* the row's last workgroup holds less */
-        if ((tid & 7) == 7 && c == r - 1) {
-            const uint32_t q16 = mine & 0xffff0000u;
+        const uint32_t sa = s_top[lane], sb = s_top[lane + WAVE];
+        const uint32_t own = wv < OL_WAVES / 2 ? sa : sb;
+        const int      r = grp == G - 1 ? r_last : r_w; /* the row's last workgroup holds less */
+        uint32_t       found = 0u;
+#pragma unroll
+        for (int e = 0; e < OL_TOP; ++e) {
+            const uint32_t x = readlane_u32(own, (wv & (OL_WAVES / 2 - 1)) * OL_TOP + e);
+            const int      c = __popcll(ballot64(sa > x)) + __popcll(ballot64(sb > x));
+            found            = c == r - 1 ? (x | 1u) : found; /* (never 0 when found) */
+        }
+        if (found != 0u && lane == 0) {
+            const uint32_t q16 = found & 0xffff0000u;
             /* never below the lowest finite value: -inf (padding, forbidden tokens) is not
              * handed on */
             s_o.tw = q16 < KEY_LOWEST_FINITE ? KEY_LOWEST_FINITE : q16;
@@ -305,8 +305,11 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
      * be certified. The first wavefront adds T_w. */
     {
         const long sw  = ((long) row * G + grp) * OL_WAVES + wv; /* this scanning wavefront */
-        float4    *dv  = wc.val + sw * OL_SLOTS;
-        uint32_t  *di  = wc.idx + sw * OL_SLOTS;
+        /* slot p of this wavefront lies at [row][p][wavefront of the row]: the final stage reads
+         * one slot of all the row's wavefronts at a time */
+        const int  Wr  = G * OL_WAVES;
+        float4    *dv  = wc.val + (long) row * OL_SLOTS * Wr + grp * OL_WAVES + wv;
+        uint32_t  *di  = wc.idx + (long) row * OL_SLOTS * Wr + grp * OL_WAVES + wv;
         const int  e0  = base + 4 * t;
         unsigned   cnt = 0;
 #pragma unroll
@@ -317,16 +320,15 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
                 continue;
             const unsigned p = cnt + lanes_before(mj);
             if (in_j && p < (unsigned) OL_SLOTS) {
-                dv[p] = v[j];
-                di[p] = (uint32_t) (e0 + 4 * j * TPB);
+                dv[p * Wr] = v[j];
+                di[p * Wr] = (uint32_t) (e0 + 4 * j * TPB);
             }
             cnt += (unsigned) __popcll(mj);
         }
-        if (lane == 0) {
-            wc.count[sw] = cnt;
-            if (wv == 0)
-                wc.bound[(long) row * G + grp] = tw;
-        }
+        /* the number of groups (more than OL_SLOTS: too many) beside the sixteen leading bits of
+         * T_w, which are all it has */
+        if (lane == 0)
+            wc.count[sw] = tw | (cnt < 0xffffu ? cnt : 0xffffu);
     }
     if (PEN && table_ok && hlen > 2 * OL_THREADS) { /* a long history: the rest of it */
         for (int i = tid + 2 * OL_THREADS; i < hlen; i += OL_THREADS) {
@@ -386,20 +388,17 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
         gi[h] = 0u;
         cw[h] = 0u;
         if (on) {
-            gv[h] = wc.val[(sw0 + w) * OL_SLOTS + wv];
-            gi[h] = wc.idx[(sw0 + w) * OL_SLOTS + wv];
+            gv[h] = wc.val[((long) row * OL_SLOTS + wv) * W + w];
+            gi[h] = wc.idx[((long) row * OL_SLOTS + wv) * W + w];
             cw[h] = wc.count[sw0 + w]; /* how many groups that scanning wavefront handed on */
         }
         cw[h] = lane + 64 * h < W ? cw[h] : 0u;
     }
-    uint32_t tb[OL_WG_MAX];
-#pragma unroll
-    for (int g = 0; g < OL_WG_MAX; ++g)
-        tb[g] = wc.bound[(long) row * G + (g < G ? g : 0)];
-    uint32_t bk = 0u;
-#pragma unroll
-    for (int g = 0; g < OL_WG_MAX; ++g)
-        bk = (g < G && tb[g] > bk) ? tb[g] : bk;
+    /* B: the largest T_w of the row (each scanning wavefront wrote its workgroup's beside its
+     * count) */
+    const uint32_t bk = wave_max_u32((cw[0] > cw[1] ? cw[0] : cw[1]) & 0xffff0000u);
+    cw[0] &= 0xffffu;
+    cw[1] &= 0xffffu;
     const uint32_t lo = bk < KEY_LOWEST_FINITE ? KEY_LOWEST_FINITE : bk;
     GS_STAMP(8);
     const float    B  = key2f(lo);
@@ -569,8 +568,20 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
     if (tid < WAVE) {
         /* (k <= CAND_K_MAX = 64 on this path) */
         const int tok = finish_sorted_lanes(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_tab);
-        if (tid == 0)
+        if (tid == 0) {
             a.out[row] = tok;
+            if (nt.h_done) {
+                /* the id has left for where `out` lies before the row counts as done; the row
+                 * that completes the batch tells the host */
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                const uint32_t done = __hip_atomic_fetch_add(nt.rows_done, 1u, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT) + 1u;
+                if (done == gridDim.y) {
+                    __hip_atomic_store(nt.rows_done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(nt.h_done, nt.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+            }
+        }
     }
     GS_STAMP(11);
 }

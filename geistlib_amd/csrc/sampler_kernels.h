@@ -50,6 +50,18 @@ struct MeetSpace {
     uint32_t  wait_limit;  /* polls before a workgroup reads the row for itself; 0 = do not wait */
 };
 
+/* Where a sampling step reports that the ids of all its rows are written: `epoch` goes into
+ * *h_done (page-locked host memory) after them. h_done == NULL: nobody is told. `rows_done` is a
+ * zeroed device counter that the one-launch top-k kernel leaves zeroed (its rows finish in any
+ * order; the last one reports). */
+struct Notify {
+    uint64_t *h_done;
+    uint64_t  epoch;
+    uint32_t *rows_done;
+};
+/* the same report from a launch of its own, for the steps whose last kernel does not make it */
+void launch_publish_epoch(hipStream_t stream, const Notify &nt);
+
 struct Launch {
     RowView     rv;
     int         rows;
@@ -110,26 +122,24 @@ inline WaveCands wave_cands_at(void *base, size_t row_waves) {
  * workgroup that finishes the row: per scanning wavefront (16 per workgroup, G workgroups per row)
  * OL_SLOTS float4 groups -- those that hold an element at or above the workgroup's bound T_w --
  * with the index of each group's first element, and their number (more than OL_SLOTS: it had too
- * many and the row cannot be certified); per workgroup the key of T_w. */
+ * many and the row cannot be certified) beside the key of T_w. */
 constexpr int OL_TOP      = 8;   /* maxima a wavefront enters for its workgroup's bound */
 constexpr int OL_SLOTS    = 16;  /* groups a scanning wavefront may hand on */
 constexpr int OL_WG_MAX   = 8;   /* workgroups per row (CAND_CHUNKS_MAX chunks, four each) */
 constexpr int OL_RANK_MAX = 64;  /* largest rank `r` of the workgroup's bound the path is used for */
 struct WgCands {
-    float4   *val;   /* [rows][G][16][OL_SLOTS] the float4 groups */
-    uint32_t *idx;   /* [rows][G][16][OL_SLOTS] index of each group's first element */
-    uint32_t *count; /* [rows][G][16] */
-    uint32_t *bound; /* [rows][G] */
+    float4   *val;   /* [rows][OL_SLOTS][G * 16] the float4 groups */
+    uint32_t *idx;   /* [rows][OL_SLOTS][G * 16] index of each group's first element */
+    uint32_t *count; /* [rows][G][16] key of T_w (its sixteen leading bits) | number of groups */
 };
 inline size_t wg_cands_bytes(size_t rows, size_t wgs_per_row) {
-    return rows * wgs_per_row * (16 * OL_SLOTS * 20 + 16 * sizeof(uint32_t) + sizeof(uint32_t));
+    return rows * wgs_per_row * (16 * OL_SLOTS * 20 + 16 * sizeof(uint32_t));
 }
 inline WgCands wg_cands_at(void *base, size_t rows, size_t wgs_per_row) {
     WgCands w;
     w.val   = static_cast<float4 *>(base);
     w.idx   = reinterpret_cast<uint32_t *>(w.val + rows * wgs_per_row * 16 * OL_SLOTS);
     w.count = w.idx + rows * wgs_per_row * 16 * OL_SLOTS;
-    w.bound = w.count + rows * wgs_per_row * 16;
     return w;
 }
 /* `r` for a workgroup that holds `elems` of a row's n_vocab logits, of which about k_eff lead:
@@ -237,7 +247,7 @@ constexpr int ARRIVE_STRIDE_INTS = 32;
 int probe_workgroup_placement(hipStream_t stream, bool *same_xcd);
 void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
                             const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
-                            bool far_always);
+                            bool far_always, const Notify &nt);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */

@@ -1975,6 +1975,9 @@ void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &w
     }
 }
 
+#ifndef GS_RANK_TAIL
+#define GS_RANK_TAIL 1e-8
+#endif
 int cand_rank_for(int k_eff, size_t n_vocab, size_t elems) {
     if (k_eff < 1 || elems == 0 || elems > n_vocab)
         return 0;
@@ -1984,7 +1987,7 @@ int cand_rank_for(int k_eff, size_t n_vocab, size_t elems) {
         const double share = (double) elems / (double) n_vocab;
         double       p = std::pow(1.0 - share, k_eff), cdf = p;
         int          x = 0;
-        while (1.0 - cdf > 1e-8 && x < k_eff) {
+        while (1.0 - cdf > GS_RANK_TAIL && x < k_eff) {
             p *= (double) (k_eff - x) / (double) (x + 1) * share / (1.0 - share);
             ++x;
             cdf += p;
@@ -1996,18 +1999,29 @@ int cand_rank_for(int k_eff, size_t n_vocab, size_t elems) {
 
 void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
                             const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
-                            bool far_always) {
+                            bool far_always, const Notify &nt) {
     const FinalArgs a = final_args(f);
     const int       per_wg = OL_THREADS / TPB; /* chunks a workgroup scans */
     const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, L.rows), block(OL_THREADS);
     auto go = [&](auto kernel) {
         kernel<<<grid, block, 0, L.stream>>>(scan.rv, L.rv, wc, r_w, r_last, a, tmax, arrive,
-                                             far_always ? 1 : 0);
+                                             far_always ? 1 : 0, nt);
     };
     if (L.pen)
         scan.rv.stream_loads ? go(k_cand_scan_final<true, true>) : go(k_cand_scan_final<true, false>);
     else
         scan.rv.stream_loads ? go(k_cand_scan_final<false, true>) : go(k_cand_scan_final<false, false>);
+}
+
+__global__ void k_publish_epoch(Notify nt) {
+    /* (the kernels before this one on the stream have ended: their stores are where the host
+     * reads them) */
+    __hip_atomic_store(nt.h_done, nt.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+void launch_publish_epoch(hipStream_t stream, const Notify &nt) {
+    if (nt.h_done)
+        k_publish_epoch<<<dim3(1), dim3(1), 0, stream>>>(nt);
 }
 
 int probe_workgroup_placement(hipStream_t stream, bool *same_xcd) {

@@ -60,6 +60,17 @@ static int read_back(struct geist_hip_head *h, void *dst, const void *pinned, si
     return GEIST_HIP_OK;
 }
 
+/* The token ids of the sampling call enqueued last: the call returns with the tokens, as the
+ * reference's does (forward/head.c:165-186), as soon as the kernels have written them -- the
+ * sampler reports that into page-locked memory (geist_hip_sampler_notify_ids), and only a call
+ * that is not reported in time waits for the stream. */
+static int read_ids(struct geist_hip_head *h, void *dst, const void *pinned, size_t bytes) {
+    if (geist_hip_sampler_wait_ids(h->hs) != GEIST_HIP_OK)
+        return GEIST_HIP_E_BACKEND;
+    memcpy(dst, pinned, bytes);
+    return GEIST_HIP_OK;
+}
+
 static int seed_rng(struct geist_hip_head *h, uint64_t seed) {
     /* geist_rng_seed, src/engine/sampler.c:27-33 */
     const uint64_t state = seed != 0 ? seed : UINT64_C(0x9E3779B97F4A7C15);
@@ -100,6 +111,8 @@ int geist_hip_head_create(int device, size_t vocab, size_t m_max, float logit_so
     if (rc == GEIST_HIP_OK &&
         (rc = geist_hip_host_malloc(h->hs, 20 * sizeof(int32_t), &p)) == GEIST_HIP_OK)
         h->d_ngram = p;
+    if (rc == GEIST_HIP_OK)
+        rc = geist_hip_sampler_notify_ids(h->hs, 1); /* see read_ids() */
     /* arch_state.c:1173: the default seed */
     if (rc == GEIST_HIP_OK)
         rc = seed_rng(h, UINT64_C(0xCAFEBABE1234));
@@ -214,7 +227,7 @@ static int finalize(struct geist_hip_head *h, const float *d_logits, size_t k, i
     if (geist_hip_sample_rows_rng(h->hs, &rows, &prm, h->d_rng, /*shared=*/1, h->d_tokens) !=
         GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "sampling");
-    if (read_back(h, out, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_ids(h, out, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++) /* head.c:137-139: an id outside the vocabulary is an error */
         if (out[r] < 0 || (size_t) out[r] >= h->vocab)
@@ -287,7 +300,7 @@ static int project_finalize_table(struct geist_hip_head *h, const float *d_hidde
     if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
     h->logits_sparse = false;
-    if (read_back(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_ids(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++)
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)
@@ -350,7 +363,7 @@ int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d
     if (rc != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "output head");
     h->logits_sparse = false;
-    if (read_back(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
+    if (read_ids(h, out_tokens, h->d_tokens, k * sizeof(int32_t)) != GEIST_HIP_OK)
         return head_fail(h, GEIST_HIP_E_BACKEND, "reading back the token ids");
     for (size_t r = 0; r < k; r++)
         if (out_tokens[r] < 0 || (size_t) out_tokens[r] >= h->vocab)

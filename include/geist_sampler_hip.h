@@ -47,6 +47,22 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s);
 const char *geist_hip_sampler_last_error(const geist_hip_sampler *s);
 /* Blocks until everything enqueued on the sampler's stream has finished. */
 int geist_hip_sampler_sync(geist_hip_sampler *s);
+
+/* The reference's sample call returns with the token (forward/head.c:165-186). Here the ids of a
+ * sampling call are written by kernels, and a caller that waits for the stream pays the runtime's
+ * completion path on top of them. With enable = 1 every sampling call of `s` also stores, after
+ * the ids of all its rows, the call's number into a word of page-locked host memory -- the kernel
+ * that writes the last id does it where the step is one launch, a launch of its own otherwise.
+ * geist_hip_sampler_wait_ids() then watches that word: it returns as soon as the ids of the last
+ * call enqueued are written (meant for ids that go to page-locked memory, geist_hip_host_malloc,
+ * which the host can then read at once) and falls back to waiting for the stream -- which also
+ * reports a failed launch -- when the word has not changed within a bounded time
+ * (geist_hip_sampler_set_wait_spin, default 2000 us; 0 = do not watch at all). With enable = 0
+ * (the default) wait_ids is geist_hip_sampler_sync. Other work enqueued on the stream after the
+ * sampling call is not waited for. */
+int geist_hip_sampler_notify_ids(geist_hip_sampler *s, int enable);
+int geist_hip_sampler_wait_ids(geist_hip_sampler *s);
+int geist_hip_sampler_set_wait_spin(geist_hip_sampler *s, uint32_t microseconds);
 /* Rebinds the stream later calls are enqueued on (NULL = default stream). */
 int geist_hip_sampler_set_stream(geist_hip_sampler *s, void *stream);
 
