@@ -29,6 +29,9 @@ using namespace gs;
  * made), how many slots the last launch on each array used, and whose turn it is. */
 struct MeetState {
     uint64_t *slots[2] = {nullptr, nullptr};
+    uint64_t *recorded = nullptr; /* a third array, for launches recorded into a HIP graph: a graph
+                                   * is replayed with the arguments it was recorded with, so the
+                                   * turns of the two arrays above mean nothing to it */
     uint32_t  used[2]  = {0, 0};
     int       turn     = 0;
     uint32_t  capacity = 0;     /* slots per array */
@@ -52,6 +55,7 @@ struct geist_hip_sampler {
     uint64_t   epoch = 0;            /* of the last call enqueued */
     uint32_t  *rows_done = nullptr;  /* device counter of the one-launch top-k kernel */
     bool       epoch_by_kernel = false; /* the call being enqueued reports from its own kernel */
+    bool       tell = false;            /* the call being enqueued reports at all */
     uint32_t   wait_spin_us = 2000;  /* geist_hip_sampler_wait_ids: how long it watches the word */
     bool       handoff_far = false;  /* that kernel reads the hand-over with agent-scope loads
                                       * whatever the placement (geist_hip_sampler_handoff_scope) */
@@ -207,7 +211,9 @@ constexpr size_t STATIC_WCANDS = STATIC_SLAB + STATIC_UNITS * 8 * 8;   /* WaveCa
 constexpr size_t STATIC_MEET   = STATIC_WCANDS + STATIC_ROW_WAVES * 648; /* u64 [2][2 units]:
                                                                             the meeting slots,
                                                                             zero when loaded */
-constexpr size_t STATIC_BYTES  = STATIC_MEET + 2 * 2 * STATIC_UNITS * 8;
+constexpr size_t STATIC_BYTES  = STATIC_MEET + 3 * 2 * STATIC_UNITS * 8; /* (the third array: for
+                                                                           launches recorded into a
+                                                                           HIP graph) */
 static_assert(STATIC_MEET % 16 == 0, "64-bit atomics");
 static_assert(STATIC_WCANDS % 16 == 0, "float4 slots");
 constexpr int    STATIC_MAX_DEVICES = 64;
@@ -313,6 +319,7 @@ int geist_hip_sampler_create(int device, size_t max_rows, size_t max_vocab, void
         if (e == hipSuccess) e = hipMalloc((void **) &s->meet_own.slots[t], 2 * rc * sizeof(uint64_t));
         if (e == hipSuccess) e = hipMemsetAsync(s->meet_own.slots[t], 0, 2 * rc * sizeof(uint64_t), s->stream);
     }
+    if (e == hipSuccess) e = hipMalloc((void **) &s->meet_own.recorded, 2 * rc * sizeof(uint64_t));
     s->meet_own.capacity = (uint32_t) (2 * rc);
     if (e == hipSuccess)
         e = hipMalloc((void **) &s->row_arrive, max_rows * ARRIVE_STRIDE_INTS * sizeof(int32_t));
@@ -371,6 +378,7 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
         (void) hipHostFree(s->h_done);
     (void) hipFree(s->meet_own.slots[0]);
     (void) hipFree(s->meet_own.slots[1]);
+    (void) hipFree(s->meet_own.recorded);
     (void) hipFree(s->resid_sum);
     (void) hipFree(s->slab_sum);
     (void) hipFree(s->resid_slab);
@@ -496,11 +504,24 @@ static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t word
     MeetState &st = *s->meet;
     if (st.suspect) { /* only after a failed launch: start again from two zeroed arrays */
         for (int t = 0; t < 2; ++t)
-            (void) hipMemsetAsync(st.slots[t], 0, st.capacity * sizeof(uint64_t), s->stream);
+            launch_zero_words(s->stream, st.slots[t], st.capacity);
         st.used[0] = st.used[1] = 0;
         st.suspect              = false;
     }
     MeetSpace  m;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (st.recorded && hipStreamIsCapturing(s->stream, &capture) == hipSuccess &&
+        capture == hipStreamCaptureStatusActive) {
+        /* being recorded: the launch meets in the array kept for graphs, and a fill kernel
+         * recorded in front of it clears what it uses on every replay */
+        const uint32_t n = words * (uint32_t) L.rows * (uint32_t) L.rv.n_chunks;
+        launch_zero_words(s->stream, st.recorded, n);
+        m.slots       = st.recorded;
+        m.stale       = st.recorded;
+        m.stale_count = 0;
+        m.wait_limit  = s->wait_limit;
+        return m;
+    }
     m.slots       = st.slots[st.turn];
     m.stale       = st.slots[st.turn ^ 1];
     m.stale_count = st.used[st.turn ^ 1];
@@ -514,10 +535,19 @@ static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t word
 static int sample_impl(geist_hip_sampler *s, const struct geist_hip_rows *rows,
                        const struct geist_hip_sample_params *params, const float *d_uniforms,
                        geist_hip_token_t *d_out) {
-    if (s)
+    if (s) {
         s->epoch_by_kernel = false;
+        s->tell = false;
+        if (s->notify && s->h_done) {
+            /* (a launch recorded into a graph would report the same number at every replay:
+             * recorded calls report nothing) */
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            s->tell = hipStreamIsCapturing(s->stream, &capture) != hipSuccess ||
+                      capture != hipStreamCaptureStatusActive;
+        }
+    }
     const int rc = gs_host::sample_stages(s, rows, params, d_uniforms, d_out, gs_host::STAGE_ALL, nullptr);
-    if (rc == GEIST_HIP_OK && s->notify && s->h_done) {
+    if (rc == GEIST_HIP_OK && s->tell) {
         /* the ids of this call are written when the word holds this epoch */
         const Notify nt = {s->h_done, s->epoch + 1, s->rows_done};
         if (!s->epoch_by_kernel)
@@ -677,7 +707,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
             *stream_kernel     = "k_cand_scan_final";
             /* with both stages in this call, the kernel itself reports the ids written */
             Notify nt = {nullptr, 0, nullptr};
-            if (s->notify && s->h_done && s->rows_done && do_stream && do_tail) {
+            if (s->tell && s->rows_done && do_stream && do_tail) {
                 nt                 = Notify{s->h_done, s->epoch + 1, s->rows_done};
                 s->epoch_by_kernel = true;
             }
@@ -929,6 +959,7 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
     MeetState &ms = g_static_meet[device];
     ms.slots[0]   = reinterpret_cast<uint64_t *>(ws + STATIC_MEET);
     ms.slots[1]   = ms.slots[0] + 2 * STATIC_UNITS;
+    ms.recorded   = ms.slots[1] + 2 * STATIC_UNITS;
     ms.capacity   = (uint32_t) (2 * STATIC_UNITS);
     tmp.meet      = &ms;
     rc = sample_impl(&tmp, rows, params, d_uniforms, d_out_tokens);

@@ -59,6 +59,9 @@ struct Notify {
     uint64_t  epoch;
     uint32_t *rows_done;
 };
+/* a small fill kernel: n 64-bit words at p become zero (recorded into HIP graphs in place of a
+ * memset node) */
+void launch_zero_words(hipStream_t stream, uint64_t *p, uint32_t n);
 /* the same report from a launch of its own, for the steps whose last kernel does not make it */
 void launch_publish_epoch(hipStream_t stream, const Notify &nt);
 

@@ -2013,6 +2013,18 @@ void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaun
         scan.rv.stream_loads ? go(k_cand_scan_final<false, true>) : go(k_cand_scan_final<false, false>);
 }
 
+__global__ __launch_bounds__(TPB) void k_zero_words(uint64_t *__restrict__ p, uint32_t n) {
+    for (uint32_t i = blockIdx.x * TPB + threadIdx.x; i < n; i += gridDim.x * TPB)
+        p[i] = 0ull;
+}
+
+void launch_zero_words(hipStream_t stream, uint64_t *p, uint32_t n) {
+    if (n == 0)
+        return;
+    const uint32_t blocks = (n + TPB - 1) / TPB;
+    k_zero_words<<<dim3(blocks < 64u ? blocks : 64u), dim3(TPB), 0, stream>>>(p, n);
+}
+
 __global__ void k_publish_epoch(Notify nt) {
     /* (the kernels before this one on the stream have ended: their stores are where the host
      * reads them) */
