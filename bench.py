@@ -151,6 +151,105 @@ def reference_top_k_baseline(w, cores, budget_s):
                                       f"{res['1'][2]} on 1 thread"}
 
 
+def time_other_configs(steps=50, warmup=10):
+    """The other four benchmark configurations under the same clock as the headline workload:
+    `steps` HBM-cold steps each (the inputs rotate over copies that together exceed the Infinity
+    Cache), wall-clock per step, and -- for the configurations that are one sampling call -- the
+    logit-streaming kernel on its own by HIP events. Inputs are drawn on the device with the
+    configurations' distributions (parity of these configurations at full size is the business of
+    tests/test_gpu_configs.py, not of this leg); no CPU leg."""
+    import torch
+    from geistlib_amd import HipSampler, SampleParams
+    from geistlib_amd import bench_hooks as bh
+    from geistlib_amd.workloads import zipf_history
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    out = {}
+
+    def normal(shape, scale):
+        return torch.randn(shape, device=dev, generator=g) * scale
+
+    def run(name, make_copy, n_copies, rows, n_vocab, prm_kw, hist_len=0, extra_bytes=0):
+        copies = [make_copy() for _ in range(n_copies)]
+        d_u = torch.rand(rows, device=dev, generator=g)
+        d_out = torch.empty(rows, dtype=torch.int32, device=dev)
+        d_h = d_hl = None
+        if hist_len:
+            hg = np.random.default_rng(3)
+            d_h = torch.from_numpy(zipf_history(hg, rows, hist_len, n_vocab)).to(dev)
+            d_hl = torch.full((rows,), hist_len, dtype=torch.int32, device=dev)
+        hs = HipSampler(max_rows=rows, max_vocab=n_vocab)
+        hs.set_logits_hint(True)
+        prm = SampleParams.make(**prm_kw)
+        hs.prepare(prm, n_vocab)
+        rl = [HipSampler.rows(c, d_h, d_hl) for c in copies]
+        for i in range(max(warmup, n_copies)):
+            hs.sample(rl[i % n_copies], prm, d_u, d_out)
+        hs.sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            hs.sample(rl[i % n_copies], prm, d_u, d_out)
+        hs.sync()
+        us = (time.perf_counter() - t0) * 1e6 / steps
+        k_us, k_name = bh.time_stream_kernel(hs, rl, prm, d_u, d_out, steps)
+        alg = rows * (4 * n_vocab + 8) + extra_bytes
+        out[name] = {"us_per_step": round(us, 2), "rows_per_s": round(rows / (us * 1e-6), 1),
+                     "step_frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     "step_algorithmic_bytes": int(alg), "kernel": k_name,
+                     "kernel_us": round(k_us, 2), "steps": steps, "input_copies_rotated": n_copies}
+        hs.close()
+
+    # cfg1: one row of 128256, N(0, 3^2), T = 0.8 (the rows of a [1400 x V] buffer take turns)
+    big = normal((1400, 128256), 3.0)
+    run("cfg1", iter([big[i:i + 1] for i in range(1400)]).__next__, 1400, 1, 128256,
+        dict(temperature=0.8))
+    del big
+    # cfg3: 128 x 151936, N(0, 2^2), Zipf history of 2048, penalties, T = 1, top-p 0.95, min-p 0.05
+    hist_bytes = 128 * (4 * 2048 + 8 * 1000)   # ids read + about 1000 distinct per row gathered
+    run("cfg3", lambda: normal((128, 151936), 2.0), 9, 128, 151936,
+        dict(temperature=1.0, top_p=0.95, min_p=0.05, rep=1.1, freq=0.5, pres=0.3), hist_len=2048,
+        extra_bytes=hist_bytes)
+    # cfg4: 256 x 262144, Student-t(3) x 2.5, top-k 64 -> top-p 0.9, T = 0.6
+    def student_t():
+        z = torch.randn((256, 262144), device=dev, generator=g)
+        chi = (torch.randn((3, 256, 262144), device=dev, generator=g) ** 2).sum(0)
+        return (z / torch.sqrt(chi / 3.0) * 2.5).contiguous()
+    run("cfg4", student_t, 3, 256, 262144, dict(temperature=0.6, top_k=64, top_p=0.9))
+    # cfg5: 32 sequences x 9 target rows of 128256, q = softmax(target + N(0, 0.5^2))
+    n_seq, L, V = 32, 8, 128256
+    ts, qs = [], []
+    for _ in range(3):
+        t = normal((n_seq, L + 1, V), 2.0)
+        q = torch.softmax((t[:, :L, :] + normal((n_seq, L, V), 0.5)).double(), dim=-1).float()
+        ts.append(t)
+        qs.append(q.contiguous())
+    draft = torch.multinomial(qs[0].reshape(-1, V), 1, generator=g).reshape(n_seq, L).to(torch.int32)
+    u = torch.rand((n_seq, L + 1), device=dev, generator=g)
+    o_tok = torch.full((n_seq, L + 1), -1, dtype=torch.int32, device=dev)
+    nacc = torch.full((n_seq,), -1, dtype=torch.int32, device=dev)
+    hs = HipSampler(max_rows=n_seq * (L + 1), max_vocab=V)
+    hs.set_logits_hint(1)
+    for i in range(max(warmup, 3)):
+        hs.spec_verify(ts[i % 3], qs[i % 3], draft, u, 1.0, o_tok, nacc)
+    hs.sync()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        hs.spec_verify(ts[i % 3], qs[i % 3], draft, u, 1.0, o_tok, nacc)
+    hs.sync()
+    us = (time.perf_counter() - t0) * 1e6 / steps
+    rows = n_seq * (L + 1)
+    alg = rows * V * 4 + n_seq * V * 4 + rows * 8 + n_seq * 4
+    out["cfg5"] = {"us_per_step": round(us, 2), "rows_per_s": round(rows / (us * 1e-6), 1),
+                   "sequences_per_s": round(n_seq / (us * 1e-6), 1),
+                   "step_frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                   "step_algorithmic_bytes": int(alg),
+                   "kernel": "k_scan_expsum + k_spec_resid_draw (whole step)", "kernel_us": None,
+                   "steps": steps, "input_copies_rotated": 3}
+    hs.close()
+    return out
+
+
 def bench_spec(w, args):
     """Configuration 5: speculative verification of n_seq sequences x (L + 1) target rows. A step
     is one geist_hip_spec_verify call; rows/s counts target rows."""
@@ -761,6 +860,9 @@ def main():
                     help="skip the cache-resident legs and the latency probe, so that every launch "
                          "of the run streams its logits from HBM (for rocprofv3 runs whose "
                          "per-kernel averages are to be compared with roofline.kernel_us)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the legs that time configurations 1, 3, 4 and 5 beside the headline "
+                         "workload")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="instead of sampling, run a plain device copy of the logit buffer "
                          "(a kernel of known traffic, for scaling rocprof's FETCH_SIZE/WRITE_SIZE)")
@@ -978,6 +1080,12 @@ def main():
         if ids_cpu is not None:
             result["parity"] = {"rows": int(w.rows),
                                 "ids_differ": int(np.sum(ids_cpu != ids_gpu))}
+    if args.workload == "cfg2_pen" and not args.cold_only and not args.no_configs:
+        # the headline run also carries the other four configurations' figures
+        hs.close()
+        del copies, rows_cold
+        torch.cuda.empty_cache()
+        result["configs"] = time_other_configs()
     print(json.dumps(result))
 
 
