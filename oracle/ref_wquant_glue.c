@@ -33,5 +33,6 @@ int ref_wquant_linear(int dtype, const void *raw, int n_out, int n_in, const flo
     return 0;
 }
 
+int ref_dtype_f16(void) { return (int) GEIST_DTYPE_F16; }
 int ref_dtype_q6_K(void) { return (int) GEIST_DTYPE_Q6_K; }
 int ref_dtype_q4_K(void) { return (int) GEIST_DTYPE_Q4_K; }

@@ -481,6 +481,19 @@ def load_ref_wquant(fast=False):
     return lib
 
 
+def ref_f16_linear(ref, w_f16_bits, x):
+    """cpu_scalar_w_quant_m1 / _mN over an F16 table (uint16 bit patterns [n_out, n_in]), compiled
+    from the reference's tree."""
+    xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
+    w = np.ascontiguousarray(w_f16_bits, dtype=np.uint16)
+    n_out, n_in = w.shape
+    y = np.full((xs.shape[0], n_out), np.nan, dtype=np.float32)
+    rc = ref.ref_wquant_linear(ref.ref_dtype_f16(), w.ctypes.data_as(C.c_void_p), n_out, n_in,
+                               _fp(xs), xs.shape[0], _fp(y))
+    assert rc == 0
+    return y
+
+
 def ref_q6k_linear(ref, w_q6k, x, n_in):
     xs = np.ascontiguousarray(np.atleast_2d(x), dtype=np.float32)
     n_out = w_q6k.shape[0]

@@ -427,3 +427,29 @@ def test_random_projection_shapes(hs, oracle, seed):
         hs.rmsnorm(d_x, to_dev(norm_w, torch), eps, normed)
         hs.sync()
         assert (bits(normed.cpu().numpy()) == bits(oracle.rmsnorm(x, norm_w, eps))).all()
+
+
+@pytest.mark.parametrize("m", [1, 2, 5, 9, 14])
+def test_f16_linear_in_double_on_order_sensitive_rows(hs, oracle, m):
+    """Rows whose last quarter cancels a huge first quarter: the small terms in between are added
+    to a sum 2^24 times their size, so the binary32 result depends on the ORDER of the additions in
+    double (numpy's own float64 product rounds some of these outputs to another value). The
+    device kernels add in another order and re-add, in index order, what their bound cannot
+    decide: every bit equals the oracle, which equals the reference's cpu_scalar_w_quant_mN
+    compiled from its tree (tests/test_lm_head_oracle.py)."""
+    g = np.random.default_rng(900 + m)
+    n_out, n_in = 3000, 1024
+    q = n_in // 4
+    w = (g.standard_normal((n_out, n_in)) * 4).astype(np.float16)
+    x = (g.standard_normal((m, n_in)) * 100).astype(np.float32)
+    x[:, :q] *= np.float32(2.0 ** 24)
+    w[:, 3 * q: 4 * q] = -w[:, :q]
+    x[:, 3 * q: 4 * q] = x[:, :q]
+    y = torch.full((m, n_out), float("nan"), dtype=torch.float32, device="cuda")
+    hs.f16_linear(to_dev(w.view(np.int16), torch), to_dev(x, torch), y)
+    hs.sync()
+    want = np.atleast_2d(oracle.f16_linear_f64(w.view(np.uint16), x if m > 1 else x[0]))
+    got = y.cpu().numpy()
+    other = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32)
+    assert (other != want).any()          # the case does hang on the order
+    assert (got.view(np.uint32) == want.view(np.uint32)).all(), int((got != want).sum())

@@ -195,3 +195,69 @@ def test_f16_linear_f64_against_numpy(oracle):
     assert (oracle.f16_linear_f64(wi.view(np.uint16), xi) == (xi @ wi.astype(np.float32).T)).all()
     # one row, one-dimensional in and out
     assert (oracle.f16_linear_f64(w.view(np.uint16), x[1]) == y[1]).all()
+
+
+def _cancelling(g, n_out, n_in, m):
+    q = n_in // 4
+    w = (g.standard_normal((n_out, n_in)) * 4).astype(np.float16)
+    x = (g.standard_normal((m, n_in)) * 100).astype(np.float32)
+    x[:, :q] *= np.float32(2.0 ** 24)       # a huge first quarter ...
+    w[:, 3 * q: 4 * q] = -w[:, :q]          # ... that the last quarter takes away again:
+    x[:, 3 * q: 4 * q] = x[:, :q]           # the small terms in between are added to a huge sum
+    return w, x
+
+
+@pytest.mark.parametrize("fast", [False, True])
+def test_f16_linear_f64_equals_the_compiled_reference(oracle, fast):
+    """oracle_f16_linear_f64 against the reference's own cpu_scalar_w_quant_m1 / _mN over an F16
+    table (weight_resolve.c:186-241), compiled from its tree with strict and with release flags:
+    every bit, for one row and for batches, on random data and on rows whose last quarter cancels a huge first quarter -- there the binary32 result depends on the ORDER of the double-precision additions,
+    which is what the device kernel claims to reproduce."""
+    from oracle_lib import load_ref_wquant, ref_f16_linear
+    ref = load_ref_wquant(fast=fast)
+    if ref is None:
+        pytest.skip("oracle/_ref/libgeist_ref_wquant*.so not built (needs the reference tree)")
+    g = np.random.default_rng(77 + fast)
+    for n_out, n_in, m in [(40, 64, 1), (33, 2560, 1), (21, 1536, 5), (17, 320, 9)]:
+        for kind in ("random", "cancelling", "integers"):
+            if kind == "random":
+                w = (g.standard_normal((n_out, n_in)) * 0.05).astype(np.float16)
+                x = (g.standard_normal((m, n_in)) * g.choice([1e-3, 1.0, 300.0])).astype(np.float32)
+            elif kind == "cancelling":
+                w, x = _cancelling(g, n_out, n_in, m)
+            else:
+                w = g.integers(-8, 9, (n_out, n_in)).astype(np.float16)
+                x = g.integers(-100, 101, (m, n_in)).astype(np.float32)
+            want = ref_f16_linear(ref, w.view(np.uint16), x)
+            got = np.atleast_2d(oracle.f16_linear_f64(w.view(np.uint16), x if m > 1 else x[0]))
+            if fast and kind == "cancelling":
+                # -ffast-math lets the compiler add in another order, and on these rows it shows:
+                # the release build is pinned to a few units in the last place only. It is the
+                # strict build -- the order the source states -- that oracle and device reproduce.
+                assert np.allclose(got, want, rtol=1e-5, atol=1e-3)
+                continue
+            assert (got.view(np.uint32) == want.view(np.uint32)).all(), (n_out, n_in, m, kind, fast)
+    # the cancelling rows do hang on the order: numpy's pairwise float64 dot rounds some of them
+    # to another binary32 value (if it never did, the case would pin nothing)
+    if not fast:
+        w, x = _cancelling(np.random.default_rng(5), 400, 1024, 2)
+        other = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32)
+        assert (other != ref_f16_linear(ref, w.view(np.uint16), x)).any()
+
+
+def test_f16_linear_f64_golden_vectors(oracle):
+    """The same against vectors written from the compiled reference
+    (tests/golden/make_f16_linear_golden.py): these travel to where the reference does not."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                        "f16_linear_ref_vectors.json")
+    with open(path) as f:
+        cases = json.load(f)["cases"]
+    assert len(cases) >= 5
+    for c in cases:
+        w = np.frombuffer(bytes.fromhex(c["w_hex"]), dtype=np.uint16).reshape(c["n_out"], c["n_in"])
+        x = np.frombuffer(bytes.fromhex(c["x_hex"]), dtype=np.float32).reshape(c["m"], c["n_in"])
+        want = np.frombuffer(bytes.fromhex(c["y_hex"]), dtype=np.float32).reshape(c["m"], c["n_out"])
+        got = np.atleast_2d(oracle.f16_linear_f64(w, x if c["m"] > 1 else x[0]))
+        assert (got.view(np.uint32) == want.view(np.uint32)).all(), c["kind"]
