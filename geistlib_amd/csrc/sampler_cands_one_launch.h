@@ -47,10 +47,15 @@ namespace gs {
  * looking at where the time goes; the library as shipped has none of it). */
 #ifdef GS_PHASE_STAMPS
 __device__ unsigned long long g_phase_stamps[4096 * 16];
+#ifndef GS_PHASE_STAMP_MASK
+#define GS_PHASE_STAMP_MASK 0xffff /* which of the stamps are taken (each costs its wavefront time) */
+#endif
 #define GS_STAMP(i)                                                                            \
     do {                                                                                       \
-        if (threadIdx.x == 0)                                                                  \
-            g_phase_stamps[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();  \
+        if (((GS_PHASE_STAMP_MASK) >> (i)) & 1)                                                \
+            if (threadIdx.x == 0)                                                              \
+                g_phase_stamps[(blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] =             \
+                    wall_clock64();                                                            \
     } while (0)
 #else
 #define GS_STAMP(i) do { } while (0)

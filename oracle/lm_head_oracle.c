@@ -212,6 +212,86 @@ void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
     }
 }
 
+/* ---- the x86 backend's decode kernel over a Q6_K table ---------------------------------------
+ * src/backends/cpu_x86/kernel_q6k_gemv.c (q6k_gemv_m1, reached from cpu_x86_linear_q6k_m1,
+ * linear_q6k.c:187-208, whenever the raw table is at hand): the activation row is quantised to
+ * int8 per super-block of 256, the products are integers, and each super-block contributes one
+ * binary32 multiply-add per lane of an eight-lane accumulator. Restated in scalar C: the AVX2
+ * lanes become loops, every rounding stays where the vector code has it. */
+void oracle_q8k_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                         int16_t *bsums_out) {
+    /* kernel_q6k_gemv.c:43-67: d = amax / 127, qs = lrintf(x * (127 / amax)), sums per 16 */
+    for (size_t s = 0; s < n_super; s++) {
+        const float *xs   = x + s * 256;
+        float        amax = 0.0f;
+        for (int k = 0; k < 256; k++) {
+            const float ax = fabsf(xs[k]);
+            if (ax > amax)
+                amax = ax;
+        }
+        const float id = amax > 0.0f ? 127.0f / amax : 0.0f;
+        d_out[s]       = amax / 127.0f;
+        for (int g = 0; g < 16; g++) {
+            int sum = 0;
+            for (int i = 0; i < 16; i++) {
+                const int v = (int) lrintf(xs[g * 16 + i] * id);
+                qs_out[s * 256 + g * 16 + i] = (int8_t) v;
+                sum += v;
+            }
+            bsums_out[s * 16 + g] = (int16_t) sum;
+        }
+    }
+}
+
+/* One row's dot product, kernel_q6k_gemv.c:90-157. Lane u of the eight-lane integer sum takes,
+ * from each of the super-block's eight runs of 32 elements, the four elements 4u .. 4u + 3 of
+ * the run times the scale of their group of sixteen (run v, elements below 16: scale 2v, else
+ * 2v + 1); the uniform offset of 32 leaves through the activations' sums per sixteen, which the
+ * vector code pairs by SCALE index: lane u loses 32 (bsums[2u] scale[2u] + bsums[2u+1]
+ * scale[2u+1]). Each lane's integer is converted to binary32 and joins the lane's accumulator by
+ * one fused multiply-add with d = d_act * d_weight; the lanes are added as hsum_ps_avx adds them:
+ * ((a0 + a4) + (a1 + a5)) + ((a2 + a6) + (a3 + a7)). */
+static float oracle_dot_q6k_q8k(size_t n_super, const uint8_t *row, const float *d_act,
+                                const int8_t *qs, const int16_t *bsums) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t i = 0; i < n_super; i++, row += 210) {
+        const uint8_t *ql = row, *qh = row + 128;
+        const int8_t  *sc = (const int8_t *) (row + 192);
+        const float    d  = d_act[i] * oracle_f16_to_f32((uint16_t) (row[208] | (row[209] << 8)));
+        const int8_t  *q8 = qs + i * 256;
+        int32_t        lane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int v = 0; v < 8; v++) { /* run v: elements 32 v .. 32 v + 31 */
+            const int h = v >> 2, j = v & 3;
+            for (int b = 0; b < 32; b++) {
+                const uint8_t lo = ql[64 * h + 32 * (j & 1) + b];
+                const int     q  = ((j >> 1) ? lo >> 4 : lo & 0xF) | (((qh[32 * h + b] >> (2 * j)) & 3) << 4);
+                lane[b >> 2] += (int32_t) sc[2 * v + (b >> 4)] * (q * (int32_t) q8[32 * v + b]);
+            }
+        }
+        for (int u = 0; u < 8; u++) {
+            lane[u] -= ((int32_t) bsums[i * 16 + 2 * u] * sc[2 * u] +
+                        (int32_t) bsums[i * 16 + 2 * u + 1] * sc[2 * u + 1]) * 32;
+            acc[u] = fmaf(d, (float) lane[u], acc[u]);
+        }
+    }
+    return ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
+}
+
+int oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q6k, float *y) {
+    /* kernel_q6k_gemv.c:159-179 */
+    const size_t n_super = n_in / 256;
+    if (n_super == 0 || n_super > 64 || n_in % 256 != 0)
+        return 1; /* the reference's caller falls back */
+    float   d_act[64];
+    int8_t  qs[64 * 256];
+    int16_t bsums[64 * 16];
+    oracle_q8k_quantize(n_super, x, d_act, qs, bsums);
+#pragma omp parallel for schedule(static)
+    for (size_t r = 0; r < n_out; r++)
+        y[r] = oracle_dot_q6k_q8k(n_super, (const uint8_t *) w_q6k + r * n_super * 210, d_act, qs, bsums);
+    return 0;
+}
+
 void oracle_dequant_q4_K_row(const void *blocks, float *out, size_t n_elems) {
     /* q4_K.c:18-49; the block layout of src/quant/quant_blocks.h:50-56 by offsets */
     const uint8_t *p = (const uint8_t *) blocks;

@@ -68,6 +68,19 @@ void oracle_dequant_q6_K_row(const void *blocks, float *out, size_t n_elems);
 void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
                            const void *w_q6k, float *y);
 
+/* What the reference's x86 backend decodes a Q6_K table with when it has the raw table (one
+ * row: cpu_x86_linear_q6k_m1, src/backends/cpu_x86/linear_q6k.c:187-208 -> q6k_gemv_m1,
+ * kernel_q6k_gemv.c:159-179): the activation row quantised per super-block of 256 to int8
+ * (d = amax / 127, q = lrintf(x * (127 / amax)), sums per sixteen; kernel_q6k_gemv.c:43-67),
+ * integer dot products, and per super-block one fused multiply-add per lane of an eight-lane
+ * binary32 accumulator (kernel_q6k_gemv.c:90-157), the lanes added as hsum_ps_avx adds them.
+ * Returns 1 where the reference's kernel returns without a result (n_in / 256 outside 1 .. 64).
+ * Pinned bit for bit by that translation unit compiled from the reference's tree
+ * (tests/test_q6k_x86_oracle.py) and by golden vectors written from it. */
+void oracle_q8k_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                         int16_t *bsums_out);
+int  oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q6k, float *y);
+
 /* The same pair for a Q4_K table (super-blocks of 144 bytes: d, dmin in binary16, eight 6-bit
  * scales and eight 6-bit minima packed into 12 bytes, 128 bytes of 4-bit values;
  * src/quant/quant_blocks.h:50-56). dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, scales by

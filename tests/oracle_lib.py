@@ -455,6 +455,52 @@ def oracle_q6k_linear(lib, w_q6k, x, n_in):
     return y
 
 
+def oracle_q6k_gemv_x86(lib, w_q6k, x, n_in):
+    """oracle_q6k_gemv_x86: the x86 backend's one-row decode kernel over a Q6_K table."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    n_out = w_q6k.shape[0]
+    y = np.full(n_out, np.nan, dtype=np.float32)
+    lib.oracle_q6k_gemv_x86.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_void_p, c_float_p]
+    lib.oracle_q6k_gemv_x86.restype = C.c_int
+    rc = lib.oracle_q6k_gemv_x86(n_out, n_in, _fp(x), w_q6k.ctypes.data_as(C.c_void_p), _fp(y))
+    assert rc == 0
+    return y
+
+
+def oracle_q8k_quantize(lib, x):
+    """(d [n_super], qs int8 [n_in], bsums int16 [n_in / 16]) of one activation row."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    ns = x.size // 256
+    d = np.empty(ns, dtype=np.float32)
+    qs = np.empty(ns * 256, dtype=np.int8)
+    bs = np.empty(ns * 16, dtype=np.int16)
+    lib.oracle_q8k_quantize.argtypes = [C.c_size_t, c_float_p, c_float_p, C.c_void_p, C.c_void_p]
+    lib.oracle_q8k_quantize.restype = None
+    lib.oracle_q8k_quantize(ns, _fp(x), _fp(d), qs.ctypes.data_as(C.c_void_p),
+                            bs.ctypes.data_as(C.c_void_p))
+    return d, qs, bs
+
+
+def load_ref_q6kgemv(fast=False):
+    """The reference's q6k_gemv_m1 compiled from its tree, or None where not built."""
+    path = os.path.join(ORACLE_DIR, "_ref",
+                        "libgeist_ref_q6kgemv_fast.so" if fast else "libgeist_ref_q6kgemv.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path, mode=os.RTLD_LAZY)
+    lib.q6k_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_void_p, c_float_p]
+    lib.q6k_gemv_m1.restype = None
+    return lib
+
+
+def ref_q6k_gemv_m1(ref, w_q6k, x, n_in):
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    n_out = w_q6k.shape[0]
+    y = np.full(n_out, np.nan, dtype=np.float32)
+    ref.q6k_gemv_m1(n_out, n_in, _fp(x), w_q6k.ctypes.data_as(C.c_void_p), _fp(y))
+    return y
+
+
 def oracle_dequant_q6k(lib, w_q6k, n_in):
     out = np.empty((w_q6k.shape[0], n_in), dtype=np.float32)
     lib.oracle_dequant_q6_K_row.argtypes = [C.c_void_p, c_float_p, C.c_size_t]
