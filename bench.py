@@ -587,16 +587,23 @@ def bench_lm_head_q6k(args, m_rows):
     ms = elapsed * 1e3 / args.steps
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-    for i in range(3):
-        hs.q6k_packed_linear(packed[i], vocab, d_model, normed, logits)
-    with Timer() as tm:       # HIP events on the sampler's stream around the launches
-        for i in range(args.steps):
-            hs.q6k_packed_linear(packed[i % 3], vocab, d_model, normed, logits)
-    kernel_us = tm.ms * 1e3 / args.steps
-    with Timer() as tm:       # the table as it lies in the file, for comparison
-        for i in range(args.steps):
-            hs.q6k_linear(tables[i % 3], d_model, normed, logits)
-    unpacked_us = tm.ms * 1e3 / args.steps
+    # One row is a decode step of the reference's x86 backend: its integer kernel q6k_gemv_m1
+    # (src/backends/cpu_x86/kernel_q6k_gemv.c), which the step above ran. A batch runs the
+    # portable arithmetic (double accumulation); for one row that kernel is timed beside.
+    x86 = m_rows == 1
+
+    def timed(fn, tabs):
+        for i in range(3):
+            fn(tabs[i], i)
+        with Timer() as tm:   # HIP events on the sampler's stream around the launches
+            for i in range(args.steps):
+                fn(tabs[i % 3], i)
+        return tm.ms * 1e3 / args.steps
+
+    portable_us = timed(lambda t, i: hs.q6k_packed_linear(t, vocab, d_model, normed, logits), packed)
+    unpacked_us = timed(lambda t, i: hs.q6k_linear(t, d_model, normed, logits), tables)
+    kernel_us = (timed(lambda t, i: hs.q6k_packed_gemv_x86(t, vocab, d_model, normed, logits),
+                       packed) if x86 else portable_us)
     w_bytes = vocab * nb * 210
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -604,39 +611,72 @@ def bench_lm_head_q6k(args, m_rows):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "Q6_K weights x f32 activations, f64 accumulation", "data": "synthetic",
+        "dtype": ("Q6_K weights x int8 activations, int32 dot products, f32 accumulation" if x86
+                  else "Q6_K weights x f32 activations, f64 accumulation"),
+        "data": "synthetic",
         "config": {"workload": f"lm_head_q6k_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
                    "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
-                   "top_p": 0.9, "logit_softcap": 30.0},
+                   "top_p": 0.9, "logit_softcap": 30.0,
+                   "projection": "x86 decode kernel (q6k_gemv_m1)" if x86
+                                 else "portable kernel (cpu_scalar_w_quant_mN)"},
         "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_q6k_packed_linear (+ activations to double)",
+                     "kernel": ("k_q6k_packed_gemv_x86 (+ k_q8k_quantize)" if x86 else
+                                "k_q6k_packed_linear (+ activations to double)"),
                      "kernel_us": round(kernel_us, 3),
-                     "kernel_us_table_as_in_file": round(unpacked_us, 3),
+                     "kernel_us_portable_arithmetic": round(portable_us, 3),
+                     "kernel_us_portable_table_as_in_file": round(unpacked_us, 3),
                      "kernel_algorithmic_bytes": w_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
     if not args.no_cpu:
-        # the oracle's restatement of the portable kernel on a bounded sample of the table rows
-        from oracle_lib import load_oracle, oracle_q6k_linear
-        lib = load_oracle(fast=True)
-        n_s = 16384
+        # CPU side on a bounded sample of the table rows. One row: the reference's own AVX2
+        # kernel (release flags, OpenMP over the table rows) where it was compiled from the
+        # reference's tree, else the oracle's scalar restatement; parity against the strict
+        # oracle, which is the one pinned to the reference bit for bit. A batch: the oracle's
+        # restatement of the portable kernel.
+        from oracle_lib import (load_oracle, load_ref_q6kgemv, oracle_q6k_gemv_x86,
+                                oracle_q6k_linear, ref_q6k_gemv_m1)
+        n_s = 65536 if x86 else 16384
         w_s = tables[0][:n_s].cpu().numpy()
         x_s = normed.cpu().numpy()
-        t0 = time.perf_counter()
-        want = oracle_q6k_linear(lib, w_s, x_s, d_model)
-        dt = time.perf_counter() - t0
-        hs.q6k_packed_linear(packed[0], vocab, d_model, normed, logits)
+        kind = "port"
+        if x86:
+            want = oracle_q6k_gemv_x86(load_oracle(fast=False), w_s, x_s[0], d_model)[None, :]
+            ref = load_ref_q6kgemv(fast=True)
+            if ref is not None:
+                kind = "reference"
+                ref_q6k_gemv_m1(ref, w_s[:1024], x_s[0], d_model)       # threads started
+                reps = 20
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    ref_q6k_gemv_m1(ref, w_s, x_s[0], d_model)
+                dt = (time.perf_counter() - t0) / reps
+            else:
+                lib = load_oracle(fast=True)
+                t0 = time.perf_counter()
+                oracle_q6k_gemv_x86(lib, w_s, x_s[0], d_model)
+                dt = time.perf_counter() - t0
+            hs.q6k_packed_gemv_x86(packed[0], vocab, d_model, normed, logits)
+        else:
+            lib = load_oracle(fast=True)
+            t0 = time.perf_counter()
+            want = oracle_q6k_linear(lib, w_s, x_s, d_model)
+            dt = time.perf_counter() - t0
+            hs.q6k_packed_linear(packed[0], vocab, d_model, normed, logits)
         hs.sync()
         got = logits[:, :n_s].cpu().numpy()
         result["cpu_baseline"] = {
             "value": round(m_rows / (dt * vocab / n_s), 2), "unit": "rows/s",
             "cores": int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1),
-            "kind": "port",
+            "kind": kind,
             "sample": f"the projection of {m_rows} row(s) over the first {n_s} of {vocab} table rows "
-                      "(dequantise a row, accumulate in double), scaled to the whole table; the "
-                      "sampler's share of the step is not included"}
+                      + (("(q6k_gemv_m1: int8 activations, integer dot products"
+                          + (", AVX2, mean of 20 passes)" if kind == "reference" else ", scalar C)"))
+                         if x86 else "(dequantise a row, accumulate in double)")
+                      + ", scaled to the whole table; the sampler's share of the step is not "
+                        "included"}
         result["parity"] = {"logits_compared": int(want.size),
                             "logits_differ": int((got.view(np.uint32) != want.view(np.uint32)).sum())}
     result["token_ids"] = [int(t) for t in ids_gpu[:8]]

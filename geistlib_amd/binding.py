@@ -116,6 +116,7 @@ def load_library():
     lib.geist_hip_q6k_packed_bytes.restype = sz
     lib.geist_hip_q6k_pack.argtypes = [vp, vp, sz, sz, vp]
     lib.geist_hip_q6k_packed_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q6k_packed_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_project_sample_rows_q6k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
                                                              vp, vp, sz, C.POINTER(SampleParams),
                                                              vp, vp, i32, vp]
@@ -387,6 +388,13 @@ class HipSampler:
     def q6k_packed_linear(self, packed, n_out, n_in, x, y):
         m = x.shape[0]
         self._check(self.lib.geist_hip_q6k_packed_linear_rows(
+            self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def q6k_packed_gemv_x86(self, packed, n_out, n_in, x, y):
+        """The x86 backend's integer decode kernel over the packed copy, row by row."""
+        m = x.shape[0]
+        self._check(self.lib.geist_hip_q6k_packed_gemv_x86_rows(
             self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 

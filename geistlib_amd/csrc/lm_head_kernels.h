@@ -59,7 +59,11 @@ struct Q6KScratch {
     double *xabs;      /* [Q6K_M_MAX][n_in / 16] the sums of their magnitudes */
     int    *amb_count; /* outputs whose rounding depends on the order of the sum ... */
     int2   *amb_list;  /* ... [n_out * Q6K_M_MAX] (table row, activation row) */
+    uint32_t *act8;    /* [n_in / 256][Q8K_ACT_DWORDS] one row's activations as int8 (x86 decode) */
 };
+/* One super-block of int8 activations: 64 dwords of four int8 each in element order, sixteen
+ * int32 sums per group of sixteen, the scale d_a (binary32 bits), padding. */
+constexpr int Q8K_ACT_DWORDS = 96;
 /* The portable kernel over a Q6_K table (cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row):
  * y[m][r] = (float) sum_k (double) x[m][k] * (double) w[r][k], the sum as if in index order;
  * n_m <= Q6K_M_MAX, n_in a multiple of 256, the table 4-byte aligned. */
@@ -75,6 +79,12 @@ void launch_q6k_pack(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n
 void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out, int n_in,
                               const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
                               long ld_y);
+/* The x86 backend's decode kernel (q6k_gemv_m1, src/backends/cpu_x86/kernel_q6k_gemv.c) over the
+ * packed copy: int8 activations per super-block, integer dot products, binary32 accumulation in
+ * the reference's order; one pass over the table per activation row (lm_head_q6k_x86.hip). */
+void launch_q6k_packed_gemv_x86(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const float *x, long ld_x, int n_m, uint32_t *act, float *y,
+                                long ld_y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
  * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
 size_t q4k_packed_bytes(long n_out, int n_in);

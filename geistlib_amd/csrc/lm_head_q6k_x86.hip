@@ -1,0 +1,199 @@
+/*
+ * lm_head_q6k_x86.hip -- the lm_head projection of one activation row over a Q6_K table with the
+ * results of the reference's x86 decode kernel q6k_gemv_m1
+ * (src/backends/cpu_x86/kernel_q6k_gemv.c:43-67 the activation quantiser, :90-157 the dot
+ * product, called from cpu_x86_linear_q6k_m1, src/backends/cpu_x86/linear_q6k.c:205-207).
+ *
+ * Arithmetic of the reference, per super-block of 256 elements:
+ *   activations  amax = max |x|, d_a = amax / 127, a = lrintf(x * (127 / amax)) as int8 (all zero
+ *                when amax is zero), s[g] = sum of a over group g of sixteen;
+ *   weights      q in 0..63 (six bits), a scale per sixteen elements (int8), d_w (binary16);
+ *   integers     eight lanes: lane u adds, over the eight runs v of 32 elements, scale[2 v +
+ *                (u >> 2)] * (the four products q * a of elements 32 v + 4 u .. + 3), and loses
+ *                32 * (s[2 u] scale[2 u] + s[2 u + 1] scale[2 u + 1]);
+ *   binary32     acc[u] = fmaf(d_a * d_w, (float) lane[u], acc[u]); after the last block
+ *                y = ((acc0 + acc4) + (acc1 + acc5)) + ((acc2 + acc6) + (acc3 + acc7)).
+ * The integer part cannot overflow (|lane| < 2^26), so its order is free; the binary32 part is
+ * done here in the reference's order, which makes the result the reference's bit for bit.
+ * Activations are taken to be finite (a NaN or an infinity sends lrintf out of int8's range,
+ * where the reference's own result is whatever the conversion leaves).
+ *
+ * The table is read from the packed copy of geist_hip_q6k_pack (lm_head_q6k.hip): a lane owns a
+ * table row and gets a block as thirteen 16-byte pieces and one dword, the six-bit values in
+ * element order. The four values of one integer dot product are 24 consecutive bits; five
+ * bit-field instructions spread them over the four bytes of a dword, v_dot4_i32_i8 multiplies
+ * them with four int8 activations (a scalar operand: the activations are uniform over the
+ * wavefront), and v_mad_i32_i24 applies the scale.
+ */
+#include "lm_head_kernels.h"
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gs {
+
+constexpr int Q6X_TPB         = 256;
+constexpr int Q6X_PACK_DWORDS = 53 * 64; /* the packed copy's dwords per (64 rows, block) */
+
+/* One workgroup per (super-block, activation row): the 256 activations as int8 (64 dwords, four
+ * to a dword in element order), the sixteen sums per group of sixteen as int32, and d_a. */
+__global__ __launch_bounds__(Q6X_TPB) void k_q8k_quantize(const float *__restrict__ x, long ld_x,
+                                                         int nb, uint32_t *__restrict__ act) {
+    __shared__ float s_max[Q6X_TPB / 64];
+    const int        b = blockIdx.x, m = blockIdx.y, t = threadIdx.x;
+    const float      xv = x[(long) m * ld_x + (long) b * 256 + t];
+    float            ax = __builtin_fabsf(xv);
+    /* the reference keeps the running maximum when a comparison with a NaN fails; fmaxf drops
+     * the NaN in the same way */
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1)
+        ax = __builtin_fmaxf(ax, __shfl_xor(ax, o));
+    if ((t & 63) == 0)
+        s_max[t >> 6] = ax;
+    __syncthreads();
+    const float amax = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]),
+                                       __builtin_fmaxf(s_max[2], s_max[3]));
+    const float id   = amax > 0.0f ? __fdiv_rn(127.0f, amax) : 0.0f;
+    const int   q    = __float2int_rn(__fmul_rn(xv, id)); /* lrintf: to nearest, ties to even */
+    int         sum  = q;
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1)
+        sum += __shfl_xor(sum, o);
+    const uint32_t b0 = (uint32_t) q & 0xffu;
+    const uint32_t b1 = (uint32_t) __shfl_down(q, 1) & 0xffu;
+    const uint32_t b2 = (uint32_t) __shfl_down(q, 2) & 0xffu;
+    const uint32_t b3 = (uint32_t) __shfl_down(q, 3) & 0xffu;
+    uint32_t      *o  = act + ((long) m * nb + b) * Q8K_ACT_DWORDS;
+    if ((t & 3) == 0)
+        o[t >> 2] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    if ((t & 15) == 0)
+        o[64 + (t >> 4)] = (uint32_t) sum;
+    if (t == 0)
+        o[80] = __float_as_uint(__fdiv_rn(amax, 127.0f));
+}
+
+typedef uint32_t q6x_u4 __attribute__((ext_vector_type(4)));
+
+/* six of a lane's 16-byte pieces of a packed block, from piece p0 on: half a block's values */
+__device__ __forceinline__ void q6x_load6(const uint32_t *__restrict__ base, int r, int p0,
+                                          uint32_t (&q)[24]) {
+#pragma unroll
+    for (int p = 0; p < 6; ++p) {
+        const q6x_u4 t = __builtin_nontemporal_load(
+            reinterpret_cast<const q6x_u4 *>(base + (p0 + p) * 256 + 4 * r));
+        q[4 * p] = t.x, q[4 * p + 1] = t.y, q[4 * p + 2] = t.z, q[4 * p + 3] = t.w;
+    }
+}
+__device__ __forceinline__ void q6x_load_scales(const uint32_t *__restrict__ base, int r,
+                                                uint32_t (&sc)[4], uint32_t &d52) {
+    const q6x_u4 t =
+        __builtin_nontemporal_load(reinterpret_cast<const q6x_u4 *>(base + 12 * 256 + 4 * r));
+    sc[0] = t.x, sc[1] = t.y, sc[2] = t.z, sc[3] = t.w;
+    d52   = __builtin_nontemporal_load(base + 3328 + r);
+}
+/* scale k of a block (k = 0..15), sign extended */
+__device__ __forceinline__ int q6x_scale(const uint32_t (&sc)[4], int k) {
+    return __builtin_amdgcn_sbfe((int) sc[k >> 2], 8 * (k & 3), 8);
+}
+/* The four six-bit values in bits 8 sh .. 8 sh + 23 of the 64 bits hi:lo, one to a byte: twelve
+ * bits to each half first (bits 12..15 and 28..31 of y hold strays), then six to each byte. The
+ * empty asm keeps the two steps apart: merged, they cost the compiler three instructions more. */
+template <int SH>
+__device__ __forceinline__ uint32_t q6x_spread(uint32_t lo, uint32_t hi) {
+    uint32_t x, t; /* the field from bit 0 on, and the same shifted left by four */
+    if (SH == 0)
+        x = lo, t = lo << 4;
+    else if (SH == 1)
+        x = lo >> 8, t = lo >> 4;
+    else
+        x = __builtin_amdgcn_alignbit(hi, lo, 8 * SH), t = __builtin_amdgcn_alignbit(hi, lo, 8 * SH - 4);
+    uint32_t y = (x & 0xfffu) | (t & ~0xfffu);
+    asm("" : "+v"(y));
+    return ((y << 2) & 0x3f003f00u) | (y & 0x003f003fu);
+}
+/* The 128 elements of half a block (runs 4 half .. 4 half + 3): lane[u] += scale * (q . a). */
+__device__ __forceinline__ void q6x_half(const uint32_t (&q)[24], const uint32_t (&sc)[4],
+                                         int half, const uint32_t *__restrict__ a,
+                                         int (&lane)[8]) {
+#pragma unroll
+    for (int vl = 0; vl < 4; ++vl) {
+        const int v   = 4 * half + vl;
+        const int s_a = q6x_scale(sc, 2 * v), s_b = q6x_scale(sc, 2 * v + 1);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            /* field f of the half: bits 24 f .. 24 f + 23 of its 24 dwords */
+            const int      f = 8 * vl + u, w0 = (3 * f) >> 2, sh = (3 * f) & 3;
+            const uint32_t lo = q[w0], hi = q[w0 + 1 < 24 ? w0 + 1 : 23];
+            const uint32_t z  = sh == 0   ? q6x_spread<0>(lo, hi)
+                                : sh == 1 ? q6x_spread<1>(lo, hi)
+                                : sh == 2 ? q6x_spread<2>(lo, hi)
+                                          : q6x_spread<3>(lo, hi);
+            const int dot = __builtin_amdgcn_sdot4((int) z, (int) a[8 * v + u], 0, false);
+            lane[u] += __mul24(u < 4 ? s_a : s_b, dot);
+        }
+    }
+}
+
+__global__ __launch_bounds__(Q6X_TPB, 4) void k_q6k_packed_gemv_x86(
+    const uint32_t *__restrict__ packed, long n_out, int nb, const uint32_t *__restrict__ act,
+    float *__restrict__ y) {
+    const int  r = threadIdx.x & 63;
+    const long g = (long) blockIdx.x * (Q6X_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long row = g * 64 + r;
+    float      acc[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        acc[u] = 0.0f;
+    /* loads run half a block ahead of the arithmetic, as in k_q6k_packed_linear */
+    const uint32_t *base = packed + g * nb * Q6X_PACK_DWORDS;
+    uint32_t        qa[24], qb[24], sc[4], d52;
+    q6x_load_scales(base, r, sc, d52);
+    q6x_load6(base, r, 0, qa);
+    for (int b = 0; b < nb; ++b) {
+        const uint32_t *blk = base + (long) b * Q6X_PACK_DWORDS;
+        const uint32_t *a   = act + (long) b * Q8K_ACT_DWORDS; /* uniform: scalar loads */
+        q6x_load6(blk, r, 6, qb);
+        const float d = __uint_as_float(a[80]) *
+                        __half2float(__ushort_as_half((unsigned short) (d52 & 0xffffu)));
+        /* the offset of 32 leaves through the activations' sums, paired by scale index */
+        int lane[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            lane[u] = -32 * (__mul24((int) a[64 + 2 * u], q6x_scale(sc, 2 * u)) +
+                             __mul24((int) a[64 + 2 * u + 1], q6x_scale(sc, 2 * u + 1)));
+        uint32_t sc_now[4] = {sc[0], sc[1], sc[2], sc[3]};
+        q6x_half(qa, sc_now, 0, a, lane);
+        if (b + 1 < nb) {
+            q6x_load_scales(blk + Q6X_PACK_DWORDS, r, sc, d52);
+            q6x_load6(blk + Q6X_PACK_DWORDS, r, 0, qa);
+        }
+        q6x_half(qb, sc_now, 1, a, lane);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            acc[u] = __builtin_fmaf(d, (float) lane[u], acc[u]);
+    }
+    if (row < n_out)
+        y[row] = ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
+}
+
+size_t q8k_act_bytes(int n_in, int n_m) {
+    return (size_t) n_m * (size_t) (n_in / 256) * Q8K_ACT_DWORDS * 4;
+}
+
+void launch_q6k_packed_gemv_x86(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const float *x, long ld_x, int n_m, uint32_t *act, float *y,
+                                long ld_y) {
+    const int nb = n_in / 256;
+    k_q8k_quantize<<<dim3(nb, n_m), dim3(Q6X_TPB), 0, stream>>>(x, ld_x, nb, act);
+    const long groups = (n_out + 63) / 64;
+    const dim3 grid((unsigned) ((groups + 3) / 4)), block(Q6X_TPB);
+    for (int m = 0; m < n_m; ++m) /* a decode kernel: one pass over the table per row */
+        k_q6k_packed_gemv_x86<<<grid, block, 0, stream>>>(
+            static_cast<const uint32_t *>(packed), n_out, nb,
+            act + (size_t) m * nb * Q8K_ACT_DWORDS, y + (long) m * ld_y);
+}
+
+} // namespace gs

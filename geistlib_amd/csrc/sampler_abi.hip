@@ -1185,7 +1185,8 @@ static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScrat
         const size_t in = n_in > s->q6k_in ? n_in : s->q6k_in;
         const size_t out = n_out > s->q6k_out ? n_out : s->q6k_out;
         const size_t bytes = (size_t) Q6K_M_MAX * (in + in / 8) * sizeof(double) + 16 +
-                             out * Q6K_M_MAX * sizeof(int2);
+                             out * Q6K_M_MAX * sizeof(int2) +
+                             (in / 256) * Q8K_ACT_DWORDS * sizeof(uint32_t);
         if (hipMalloc(&s->q6k_ws, bytes) != hipSuccess) {
             s->q6k_ws = nullptr;
             return fail(s, GEIST_HIP_E_OOM, "Q6_K projection: scratch");
@@ -1198,6 +1199,7 @@ static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScrat
     ws.xabs      = ws.xsum + (size_t) Q6K_M_MAX * (s->q6k_in / 16);
     ws.amb_count = reinterpret_cast<int *>(ws.xabs + (size_t) Q6K_M_MAX * (s->q6k_in / 16));
     ws.amb_list  = reinterpret_cast<int2 *>(reinterpret_cast<char *>(ws.amb_count) + 16);
+    ws.act8      = reinterpret_cast<uint32_t *>(ws.amb_list + s->q6k_out * Q6K_M_MAX);
     return GEIST_HIP_OK;
 }
 
@@ -1228,6 +1230,21 @@ static int q6k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, si
         launch_q6k_packed_linear(s->stream, d_packed, (long) n_out, (int) n_in, d_x + m0 * ld_x,
                                  (long) ld_x, (int) m, ws, d_y + m0 * ld_y, (long) ld_y);
     }
+    return GEIST_HIP_OK;
+}
+
+/* The x86 backend's decode kernel, row by row (each row is a pass over the table, as each call
+ * of q6k_gemv_m1 is). */
+static int q6k_packed_gemv_x86_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                    size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                    float *d_y, size_t ld_y) {
+    Q6KScratch ws;
+    const int  rc = q6k_scratch(s, n_out, n_in, ws);
+    if (rc)
+        return rc;
+    for (size_t m = 0; m < n_rows; ++m)
+        launch_q6k_packed_gemv_x86(s->stream, d_packed, (long) n_out, (int) n_in, d_x + m * ld_x,
+                                   (long) ld_x, 1, ws.act8, d_y + m * ld_y, (long) ld_y);
     return GEIST_HIP_OK;
 }
 
@@ -1312,6 +1329,26 @@ int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
     HIPCHK(s, hipSetDevice(s->device));
     rc = q6k_packed_linear_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
     return rc ? rc : after_launch(s, "Q6_K linear (packed)");
+}
+
+int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                       float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K decode: %zu rows, strides %zu / %zu", n_rows,
+                    ld_x, ld_y);
+    int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (((uintptr_t) d_packed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q6_K table not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q6k_packed_gemv_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q6_K decode (packed)");
 }
 
 static int q4k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
@@ -1501,6 +1538,10 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         rc = table == TABLE_Q4K_PACKED
                  ? q4k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)
+             : table == TABLE_Q6K_PACKED && rows == 1 && !s->projection_portable
+                 /* one row on the x86 backend: its integer decode kernel (q6k_gemv_m1) */
+                 ? q6k_packed_gemv_x86_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
+                                            d_logits, ld_logits)
              : table == TABLE_Q6K_PACKED
                  ? q6k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)

@@ -108,19 +108,25 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
  * whose logit soft-cap the head was created with): d_embed_q6k holds vocab rows of d_model / 256
  * super-blocks of 210 bytes, d_model a multiple of 256. The logits equal, bit for bit, those of
  * the reference's portable kernel cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row
- * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch; the
- * x86 backend's one-row path through cblas_sgemv (src/backends/cpu_x86/backend.c:395-397) sums
- * in the order of the BLAS library it is linked with and is not reproduced. Q4_K: below. The
+ * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch. After
+ * geist_hip_head_q6k_load, and unless geist_hip_head_set_projection chose the portable backend,
+ * one row gets the logits of the x86 backend's decode kernel q6k_gemv_m1 instead
+ * (src/backends/cpu_x86/kernel_q6k_gemv.c, resolved at src/backends/cpu_x86/backend.c:395-397),
+ * again bit for bit; that backend's batch kernel, a GEMM over an int8 copy of the table
+ * (src/backends/cpu_x86/linear_q6k.c:234-300), is not reproduced. Q4_K: below. The
  * other formats the reference resolves for an embedding table (I2_S, an F32 table) have
  * no device kernel here: their callers project on the host or with their own kernel and pass
  * the logits to geist_hip_head_finalize_one_row / _batch.
  * geist_hip_head_reserve_projection_q6k is geist_hip_head_reserve_projection plus the scratch of
  * this kernel. geist_hip_head_q6k_load, once per model: keeps a copy of the table in the order
  * the device reads it (geist_hip_q6k_pack; 1 % more device memory than the table itself, the
- * x86 backend's counterpart being its binary32 predecode at load) and reserves the buffers;
+ * x86 backend's counterpart being the int8 copy it builds at load) and reserves the buffers;
  * geist_hip_head_project_finalize_q6k with that same table pointer and d_model then streams the
- * copy, 1.5 times as fast, with the same logits bit for bit. The table itself is not kept
- * alive by the head and may be changed or freed only together with a new load. */
+ * copy (in the portable arithmetic 1.5 times as fast as the table, with the same logits bit for
+ * bit). The packed copy is recognised by the table's address and d_model alone: the table is not
+ * kept alive by the head, and after any change to its bytes -- a reload, merged adapter weights,
+ * another table at the same address -- geist_hip_head_q6k_load must be called again, or the old
+ * weights keep being used. */
 int geist_hip_head_project_finalize_q6k(struct geist_hip_head *h, const float *d_hidden,
                                         size_t ld_hidden, size_t k, const float *d_norm_weight,
                                         float rms_eps, const void *d_embed_q6k, size_t d_model,

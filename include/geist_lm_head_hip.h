@@ -54,7 +54,8 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
 
 /* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
  * the head's project_finalize calls) stands for:
- *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1; more rows: the portable kernel (default)
+ *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a packed Q6_K table q6k_gemv_m1;
+ *                                  more rows: the portable kernel (default)
  *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
  *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
  *                                  linear_m1 and linear_mN alike) */
@@ -125,11 +126,13 @@ int geist_hip_project_sample_rows_q8w(geist_hip_sampler *s, const float *d_hidde
  * w = d * scale * (q - 32) in binary32, the sum in double in index order, bit for bit (the device
  * adds in another order and repeats, in the reference's order, the few sums that lie close enough
  * to a binary32 rounding boundary for the order to matter). This is the arithmetic of the
- * reference's portable backend for any number of rows and of its x86 backend for more than one
- * row; for one row the x86 backend decodes the table to binary32 once and calls cblas_sgemv
- * (src/backends/cpu_x86/backend.c:395-397), whose order of summation belongs to the BLAS library
- * and is not reproduced. geist_hip_q6k_linear_reserve sizes the scratch ahead of the first call,
- * as geist_hip_f16_linear_reserve does. */
+ * reference's portable backend for any number of rows. Its x86 backend runs other kernels over
+ * such a table (cpu_x86_linear_q6k_resolve, src/backends/cpu_x86/backend.c:395-397): for one row
+ * the integer decode kernel q6k_gemv_m1, which geist_hip_q6k_packed_gemv_x86_rows below
+ * reproduces; for more rows a GEMM over an int8 copy of the table and int8 activations
+ * (cpu_x86_linear_q6k_mN, src/backends/cpu_x86/linear_q6k.c:234-300), which is not reproduced:
+ * batches get the portable arithmetic. geist_hip_q6k_linear_reserve sizes the scratch ahead of
+ * the first call, as geist_hip_f16_linear_reserve does. */
 int geist_hip_q6k_linear_reserve(geist_hip_sampler *s, size_t n_out, size_t n_in);
 int geist_hip_q6k_linear_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, size_t n_in,
                               const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
@@ -149,8 +152,24 @@ int geist_hip_q6k_pack(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out, 
 int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                      size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                      float *d_y, size_t ld_y);
-/* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, geist_hip_q6k_linear_rows
- * and the sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. */
+/* The x86 backend's decode kernel over the packed copy: replaces q6k_gemv_m1
+ * (src/backends/cpu_x86/kernel_q6k_gemv.c:43-157, called from cpu_x86_linear_q6k_m1,
+ * src/backends/cpu_x86/linear_q6k.c:205-207), bit for bit. Per super-block of 256 elements the
+ * activations become int8 with one scale (amax / 127, round to nearest even), the products with
+ * the six-bit weights are summed as integers in eight lanes, each lane's sum joins a binary32
+ * accumulator by one fused multiply-add, and the eight accumulators are added as the AVX2
+ * horizontal sum adds them. Each activation row is a pass of its own over the table, as each
+ * call of the reference's kernel is. Activations must be finite. */
+int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                       float *d_y, size_t ld_y);
+/* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, the projection and the
+ * sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. The
+ * projection is geist_hip_q6k_linear_rows (the portable arithmetic) over the table as it lies in
+ * the file. Over the packed copy it follows geist_hip_sampler_set_projection: in the default
+ * mode GEIST_HIP_PROJECTION_X86 one row gets geist_hip_q6k_packed_gemv_x86_rows, as on the
+ * reference's x86 backend; a batch, and any call in mode _PORTABLE, gets
+ * geist_hip_q6k_packed_linear_rows. */
 int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
                                       size_t ld_hidden, size_t rows, size_t d_model,
                                       const float *d_norm_weight, float rms_eps,

@@ -7,7 +7,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import oracle_q6k_linear, random_q6k_table
+from oracle_lib import oracle_q6k_gemv_x86, oracle_q6k_linear, random_q6k_table
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -76,6 +76,33 @@ def test_q6k_linear_rows_whose_sums_cancel(hs, oracle):
         assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32)), trial
 
 
+@pytest.mark.parametrize("n_out,n_in", [(1, 256), (64, 256), (300, 512), (5000, 1536),
+                                        (4097, 2560), (70000, 1024)])
+def test_q6k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
+    """The x86 backend's integer decode kernel (kernel_q6k_gemv.c), to which the oracle is pinned
+    by the compiled reference (tests/test_q6k_x86_oracle.py): logits bit for bit, row by row."""
+    print(f"q6k x86 decode {n_out} x {n_in}", flush=True)
+    g = np.random.default_rng(n_out + n_in)
+    w = random_q6k_table(g, n_out, n_in)
+    d_w = torch.from_numpy(w).cuda()
+    packed = torch.full((hs.q6k_packed_bytes(n_out, n_in),), 0xA5, dtype=torch.uint8, device="cuda")
+    hs.q6k_pack(d_w, n_in, packed)
+    for scale in (1.0, 1e-4, 300.0, 0.0):
+        x = (g.standard_normal((3, n_in)) * scale).astype(np.float32)
+        x[0, ::5] = 0.0
+        x[1, :256] = 0.0                      # a super-block of zeros: its scale is zero
+        x[2, 7] = np.float32(1e30)            # one huge activation: the others round to zero
+        d_x = torch.from_numpy(x).cuda()
+        y = torch.full((3, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q6k_packed_gemv_x86(packed, n_out, n_in, d_x, y)
+        hs.sync()
+        got = y.cpu().numpy()
+        for m in range(3):
+            want = oracle_q6k_gemv_x86(oracle.lib, w, x[m], n_in)
+            bad = np.flatnonzero(got[m].view(np.uint32) != want.view(np.uint32))
+            assert bad.size == 0, (scale, m, bad[:5], got[m][bad[:3]], want[bad[:3]])
+
+
 def test_q6k_argument_errors(hs):
     from geistlib_amd.binding import GeistHipError
     w = torch.zeros((4, 210), dtype=torch.uint8, device="cuda")
@@ -107,12 +134,17 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
     w = random_q6k_table(g, vocab, d_model, scale_mode="plain")
     norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
     d_w, d_nw = torch.from_numpy(w).cuda(), torch.from_numpy(norm_w).cuda()
-    for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.95, 0)]:
-        print(f"gemma table T={T} p={p} k={top_k}", flush=True)
+    host.geist_hip_head_set_projection.argtypes = [C.c_void_p, C.c_int]
+    for T, p, top_k, portable in [(0.0, 1.0, 0, False), (0.8, 1.0, 40, False),
+                                  (0.9, 0.95, 0, False), (0.8, 1.0, 40, True)]:
+        print(f"gemma table T={T} p={p} k={top_k} portable={portable}", flush=True)
         h = make_head(host, vocab, 4, cap)
+        if portable:
+            assert host.geist_hip_head_set_projection(h, 1) == 0
         opts = SessionOpts(0, T, p, top_k, 31337, None, 0, 4)
         assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
-        if top_k == 0:      # one configuration reads the table as it lies, the others packed
+        packed = not (top_k == 0 and T == 0.0)
+        if not packed:      # one configuration reads the table as it lies, the others packed
             assert host.geist_hip_head_reserve_projection_q6k(h, d_model) == 0
         else:
             assert host.geist_hip_head_q6k_load(h, C.c_void_p(d_w.data_ptr()), d_model) == 0, \
@@ -126,7 +158,11 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
                 h, C.c_void_p(d_hid.data_ptr()), d_model, k, C.c_void_p(d_nw.data_ptr()), 1e-6,
                 C.c_void_p(d_w.data_ptr()), d_model, out)
             assert rc == 0, host.geist_hip_head_errmsg(h)
-            logits = oracle_q6k_linear(oracle.lib, w, oracle.rmsnorm(hidden, norm_w, 1e-6), d_model)
+            normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
+            if k == 1 and packed and not portable:     # the x86 backend's decode kernel
+                logits = oracle_q6k_gemv_x86(oracle.lib, w, normed[0], d_model)[None, :]
+            else:
+                logits = oracle_q6k_linear(oracle.lib, w, normed, d_model)
             want = oracle.finalize_batch(sess, logits, softcap=cap).tolist()
             assert list(out) == want, (T, p, top_k, k)
         host.geist_hip_head_destroy(h)
