@@ -117,6 +117,10 @@ def load_library():
     lib.geist_hip_q6k_pack.argtypes = [vp, vp, sz, sz, vp]
     lib.geist_hip_q6k_packed_linear_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q6k_packed_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q8k_act_bytes.argtypes = [sz, sz]
+    lib.geist_hip_q8k_act_bytes.restype = sz
+    lib.geist_hip_q8k_quantize_rows.argtypes = [vp, vp, sz, sz, sz, vp]
+    lib.geist_hip_q6k_packed_gemv_q8k.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_project_sample_rows_q6k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
                                                              vp, vp, sz, C.POINTER(SampleParams),
                                                              vp, vp, i32, vp]
@@ -397,6 +401,21 @@ class HipSampler:
         self._check(self.lib.geist_hip_q6k_packed_gemv_x86_rows(
             self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
+
+    def q8k_act_bytes(self, n_in, n_rows=1):
+        return int(self.lib.geist_hip_q8k_act_bytes(n_in, n_rows))
+
+    def q8k_quantize(self, x, act):
+        """x [m, n_in] float32 -> act: the rows as int8 super-blocks (q8k_act_bytes bytes)."""
+        m, n_in = x.shape
+        assert act.numel() * act.element_size() >= self.q8k_act_bytes(n_in, m)
+        self._check(self.lib.geist_hip_q8k_quantize_rows(
+            self.h, _ptr(x), x.stride(0) if m > 1 else n_in, m, n_in, _ptr(act)))
+
+    def q6k_packed_gemv_q8k(self, packed, n_out, n_in, act, y):
+        """One row of int8 activations (q8k_quantize) times the packed table: y [n_out]."""
+        self._check(self.lib.geist_hip_q6k_packed_gemv_q8k(self.h, _ptr(packed), n_out, n_in,
+                                                           _ptr(act), _ptr(y)))
 
     def f16_to_q8w(self, w_f16, wq, scales):
         """w_f16 [n_out, n_in] float16 -> wq int8 [n_out, n_in], scales float32 [n_out]."""

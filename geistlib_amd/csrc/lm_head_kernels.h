@@ -80,11 +80,16 @@ void launch_q6k_packed_linear(hipStream_t stream, const void *packed, long n_out
                               const float *x, long ld_x, int n_m, const Q6KScratch &ws, float *y,
                               long ld_y);
 /* The x86 backend's decode kernel (q6k_gemv_m1, src/backends/cpu_x86/kernel_q6k_gemv.c) over the
- * packed copy: int8 activations per super-block, integer dot products, binary32 accumulation in
- * the reference's order; one pass over the table per activation row (lm_head_q6k_x86.hip). */
-void launch_q6k_packed_gemv_x86(hipStream_t stream, const void *packed, long n_out, int n_in,
-                                const float *x, long ld_x, int n_m, uint32_t *act, float *y,
-                                long ld_y);
+ * packed copy (lm_head_q6k_x86.hip), in its two parts: the activations of n_m rows as int8 per
+ * super-block (act: [n_m][n_in / 256][Q8K_ACT_DWORDS]), and one row's integer dot products with
+ * binary32 accumulation in the reference's order. launch_rmsnorm_q8k_rows is launch_rmsnorm_rows
+ * and the quantiser in one launch (n a multiple of 256). */
+void launch_q8k_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                         uint32_t *act);
+void launch_rmsnorm_q8k_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                             float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act);
+void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const uint32_t *act, float *y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
  * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
 size_t q4k_packed_bytes(long n_out, int n_in);

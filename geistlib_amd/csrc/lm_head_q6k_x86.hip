@@ -26,6 +26,7 @@
  * wavefront), and v_mad_i32_i24 applies the scale.
  */
 #include "lm_head_kernels.h"
+#include "rmsnorm_device.h"
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -36,19 +37,19 @@ namespace gs {
 constexpr int Q6X_TPB         = 256;
 constexpr int Q6X_PACK_DWORDS = 53 * 64; /* the packed copy's dwords per (64 rows, block) */
 
-/* One workgroup per (super-block, activation row): the 256 activations as int8 (64 dwords, four
- * to a dword in element order), the sixteen sums per group of sixteen as int32, and d_a. */
-__global__ __launch_bounds__(Q6X_TPB) void k_q8k_quantize(const float *__restrict__ x, long ld_x,
-                                                         int nb, uint32_t *__restrict__ act) {
-    __shared__ float s_max[Q6X_TPB / 64];
-    const int        b = blockIdx.x, m = blockIdx.y, t = threadIdx.x;
-    const float      xv = x[(long) m * ld_x + (long) b * 256 + t];
-    float            ax = __builtin_fabsf(xv);
+/* One super-block's 256 activations, one to a thread of the workgroup, as int8 (64 dwords, four
+ * to a dword in element order), their sixteen sums per group of sixteen as int32, and d_a, written
+ * to o[0 .. Q8K_ACT_DWORDS). s_max: four floats that no thread still reads from an earlier call
+ * (the callers alternate between two). */
+__device__ __forceinline__ void q8k_quantize_block(float xv, uint32_t *__restrict__ o,
+                                                   float *s_max) {
+    const int t  = threadIdx.x;
+    float     ax = __builtin_fabsf(xv);
     /* the reference keeps the running maximum when a comparison with a NaN fails; fmaxf drops
      * the NaN in the same way */
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1)
-        ax = __builtin_fmaxf(ax, __shfl_xor(ax, o));
+    for (int s = 32; s >= 1; s >>= 1)
+        ax = __builtin_fmaxf(ax, __shfl_xor(ax, s));
     if ((t & 63) == 0)
         s_max[t >> 6] = ax;
     __syncthreads();
@@ -58,19 +59,50 @@ __global__ __launch_bounds__(Q6X_TPB) void k_q8k_quantize(const float *__restric
     const int   q    = __float2int_rn(__fmul_rn(xv, id)); /* lrintf: to nearest, ties to even */
     int         sum  = q;
 #pragma unroll
-    for (int o = 8; o >= 1; o >>= 1)
-        sum += __shfl_xor(sum, o);
+    for (int s = 8; s >= 1; s >>= 1)
+        sum += __shfl_xor(sum, s);
     const uint32_t b0 = (uint32_t) q & 0xffu;
     const uint32_t b1 = (uint32_t) __shfl_down(q, 1) & 0xffu;
     const uint32_t b2 = (uint32_t) __shfl_down(q, 2) & 0xffu;
     const uint32_t b3 = (uint32_t) __shfl_down(q, 3) & 0xffu;
-    uint32_t      *o  = act + ((long) m * nb + b) * Q8K_ACT_DWORDS;
     if ((t & 3) == 0)
         o[t >> 2] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
     if ((t & 15) == 0)
         o[64 + (t >> 4)] = (uint32_t) sum;
     if (t == 0)
         o[80] = __float_as_uint(__fdiv_rn(amax, 127.0f));
+}
+
+/* One workgroup per (super-block, activation row). */
+__global__ __launch_bounds__(Q6X_TPB) void k_q8k_quantize(const float *__restrict__ x, long ld_x,
+                                                         int nb, uint32_t *__restrict__ act) {
+    __shared__ float s_max[Q6X_TPB / 64];
+    const int        b = blockIdx.x, m = blockIdx.y;
+    q8k_quantize_block(x[(long) m * ld_x + (long) b * 256 + threadIdx.x],
+                       act + ((long) m * nb + b) * Q8K_ACT_DWORDS, s_max);
+}
+
+/* The output norm (cpu_scalar_rmsnorm, src/backends/cpu_scalar/elementwise.c:241-280, as
+ * k_rmsnorm_rows computes it) and the quantiser in one launch, one workgroup per row: the normed
+ * row goes to y and, as int8 super-blocks, to act. n a multiple of 256. */
+__global__ __launch_bounds__(Q6X_TPB) void k_rmsnorm_q8k_rows(const float *__restrict__ x,
+                                                             long ld_x,
+                                                             const float *__restrict__ w,
+                                                             float eps, int n,
+                                                             float *__restrict__ y, long ld_y,
+                                                             uint32_t *__restrict__ act) {
+    __shared__ double s_part[Q6X_TPB];
+    __shared__ float  s_inv;
+    __shared__ float  s_max[2][Q6X_TPB / 64];
+    const int    nb = n / 256, m = blockIdx.x, t = threadIdx.x;
+    const float *xr = x + (long) m * ld_x;
+    const float  inv = block_rms_inv<Q6X_TPB>(xr, n, eps, s_part, &s_inv);
+    for (int b = 0; b < nb; ++b) {
+        const int   i = 256 * b + t;
+        const float v = __fmul_rn(__fmul_rn(xr[i], inv), w[i]);
+        y[(long) m * ld_y + i] = v;
+        q8k_quantize_block(v, act + ((long) m * nb + b) * Q8K_ACT_DWORDS, s_max[b & 1]);
+    }
 }
 
 typedef uint32_t q6x_u4 __attribute__((ext_vector_type(4)));
@@ -112,7 +144,9 @@ __device__ __forceinline__ uint32_t q6x_spread(uint32_t lo, uint32_t hi) {
     asm("" : "+v"(y));
     return ((y << 2) & 0x3f003f00u) | (y & 0x003f003fu);
 }
-/* The 128 elements of half a block (runs 4 half .. 4 half + 3): lane[u] += scale * (q . a). */
+/* The 128 elements of half a block (runs 4 half .. 4 half + 3): lane[u] += scale * (q . a). A
+ * run's eight dot products are formed before any of them is used: a dependent instruction right
+ * behind a dot product waits. */
 __device__ __forceinline__ void q6x_half(const uint32_t (&q)[24], const uint32_t (&sc)[4],
                                          int half, const uint32_t *__restrict__ a,
                                          int (&lane)[8]) {
@@ -120,6 +154,10 @@ __device__ __forceinline__ void q6x_half(const uint32_t (&q)[24], const uint32_t
     for (int vl = 0; vl < 4; ++vl) {
         const int v   = 4 * half + vl;
         const int s_a = q6x_scale(sc, 2 * v), s_b = q6x_scale(sc, 2 * v + 1);
+        int       dot[8];
+        /* the run's 32 activations: one scalar load of eight dwords */
+        typedef uint32_t u8v __attribute__((ext_vector_type(8)));
+        const u8v av = *reinterpret_cast<const u8v *>(a + 8 * v);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             /* field f of the half: bits 24 f .. 24 f + 23 of its 24 dwords */
@@ -129,9 +167,11 @@ __device__ __forceinline__ void q6x_half(const uint32_t (&q)[24], const uint32_t
                                 : sh == 1 ? q6x_spread<1>(lo, hi)
                                 : sh == 2 ? q6x_spread<2>(lo, hi)
                                           : q6x_spread<3>(lo, hi);
-            const int dot = __builtin_amdgcn_sdot4((int) z, (int) a[8 * v + u], 0, false);
-            lane[u] += __mul24(u < 4 ? s_a : s_b, dot);
+            dot[u] = __builtin_amdgcn_sdot4((int) z, (int) av[u], 0, false);
         }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            lane[u] += __mul24(u < 4 ? s_a : s_b, dot[u]);
     }
 }
 
@@ -159,11 +199,13 @@ __global__ __launch_bounds__(Q6X_TPB, 4) void k_q6k_packed_gemv_x86(
         const float d = __uint_as_float(a[80]) *
                         __half2float(__ushort_as_half((unsigned short) (d52 & 0xffffu)));
         /* the offset of 32 leaves through the activations' sums, paired by scale index */
-        int lane[8];
+        typedef uint32_t u16v __attribute__((ext_vector_type(16)));
+        const u16v bs = *reinterpret_cast<const u16v *>(a + 64);
+        int        lane[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-            lane[u] = -32 * (__mul24((int) a[64 + 2 * u], q6x_scale(sc, 2 * u)) +
-                             __mul24((int) a[64 + 2 * u + 1], q6x_scale(sc, 2 * u + 1)));
+            lane[u] = -32 * (__mul24((int) bs[2 * u], q6x_scale(sc, 2 * u)) +
+                             __mul24((int) bs[2 * u + 1], q6x_scale(sc, 2 * u + 1)));
         uint32_t sc_now[4] = {sc[0], sc[1], sc[2], sc[3]};
         q6x_half(qa, sc_now, 0, a, lane);
         if (b + 1 < nb) {
@@ -179,21 +221,23 @@ __global__ __launch_bounds__(Q6X_TPB, 4) void k_q6k_packed_gemv_x86(
         y[row] = ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
 }
 
-size_t q8k_act_bytes(int n_in, int n_m) {
-    return (size_t) n_m * (size_t) (n_in / 256) * Q8K_ACT_DWORDS * 4;
-}
-
-void launch_q6k_packed_gemv_x86(hipStream_t stream, const void *packed, long n_out, int n_in,
-                                const float *x, long ld_x, int n_m, uint32_t *act, float *y,
-                                long ld_y) {
+void launch_q8k_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                         uint32_t *act) {
     const int nb = n_in / 256;
     k_q8k_quantize<<<dim3(nb, n_m), dim3(Q6X_TPB), 0, stream>>>(x, ld_x, nb, act);
+}
+
+void launch_rmsnorm_q8k_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                             float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act) {
+    k_rmsnorm_q8k_rows<<<dim3(n_rows), dim3(Q6X_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y,
+                                                                  act);
+}
+
+void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const uint32_t *act, float *y) {
     const long groups = (n_out + 63) / 64;
-    const dim3 grid((unsigned) ((groups + 3) / 4)), block(Q6X_TPB);
-    for (int m = 0; m < n_m; ++m) /* a decode kernel: one pass over the table per row */
-        k_q6k_packed_gemv_x86<<<grid, block, 0, stream>>>(
-            static_cast<const uint32_t *>(packed), n_out, nb,
-            act + (size_t) m * nb * Q8K_ACT_DWORDS, y + (long) m * ld_y);
+    k_q6k_packed_gemv_x86<<<dim3((unsigned) ((groups + 3) / 4)), dim3(Q6X_TPB), 0, stream>>>(
+        static_cast<const uint32_t *>(packed), n_out, n_in / 256, act, y);
 }
 
 } // namespace gs

@@ -1242,9 +1242,11 @@ static int q6k_packed_gemv_x86_impl(geist_hip_sampler *s, const void *d_packed, 
     const int  rc = q6k_scratch(s, n_out, n_in, ws);
     if (rc)
         return rc;
-    for (size_t m = 0; m < n_rows; ++m)
-        launch_q6k_packed_gemv_x86(s->stream, d_packed, (long) n_out, (int) n_in, d_x + m * ld_x,
-                                   (long) ld_x, 1, ws.act8, d_y + m * ld_y, (long) ld_y);
+    for (size_t m = 0; m < n_rows; ++m) {
+        launch_q8k_quantize(s->stream, d_x + m * ld_x, (long) ld_x, 1, (int) n_in, ws.act8);
+        launch_q6k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in, ws.act8,
+                                   d_y + m * ld_y);
+    }
     return GEIST_HIP_OK;
 }
 
@@ -1349,6 +1351,49 @@ int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packe
     HIPCHK(s, hipSetDevice(s->device));
     rc = q6k_packed_gemv_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
     return rc ? rc : after_launch(s, "Q6_K decode (packed)");
+}
+
+size_t geist_hip_q8k_act_bytes(size_t n_in, size_t n_rows) {
+    if (n_in == 0 || n_in % 256 != 0 || n_in > 0x7fffff00u)
+        return 0;
+    return n_rows * (n_in / 256) * Q8K_ACT_DWORDS * sizeof(uint32_t);
+}
+
+int geist_hip_q8k_quantize_rows(geist_hip_sampler *s, const float *d_x, size_t ld_x, size_t n_rows,
+                                size_t n_in, void *d_act) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_x || !d_act)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || n_rows > 65535 || n_in == 0 || n_in > 0x7fffff00u || ld_x < n_in)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "int8 activations: %zu rows of %zu, stride %zu",
+                    n_rows, n_in, ld_x);
+    if (n_in % 256 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "int8 activations: %zu is not a multiple of 256",
+                    n_in);
+    if (((uintptr_t) d_act) % 64 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "int8 activations: buffer not 64-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_q8k_quantize(s->stream, d_x, (long) ld_x, (int) n_rows, (int) n_in,
+                        static_cast<uint32_t *>(d_act));
+    return after_launch(s, "int8 activations");
+}
+
+int geist_hip_q6k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                  size_t n_in, const void *d_act, float *d_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_act || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    const int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (((uintptr_t) d_packed) % 16 != 0 || ((uintptr_t) d_act) % 64 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K decode: table or activations misaligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_q6k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in,
+                               static_cast<const uint32_t *>(d_act), d_y);
+    return after_launch(s, "Q6_K decode (packed)");
 }
 
 static int q4k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
@@ -1521,8 +1566,19 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX;
     if (!d_normed)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "no buffer for the normed rows");
-    launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps, (int) rows,
-                        (int) d_model, d_normed, (long) d_model);
+    /* one row over a packed Q6_K table on the x86 backend: its integer decode kernel
+     * (q6k_gemv_m1), whose activation quantiser rides on the norm's launch */
+    const bool q6k_x86 = table == TABLE_Q6K_PACKED && rows == 1 && !s->projection_portable;
+    Q6KScratch q6ws{};
+    if (q6k_x86) {
+        if ((rc = q6k_scratch(s, n_vocab, d_model, q6ws)) != GEIST_HIP_OK)
+            return rc;
+        launch_rmsnorm_q8k_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps, 1,
+                                (int) d_model, d_normed, (long) d_model, q6ws.act8);
+    } else {
+        launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
+                            (int) rows, (int) d_model, d_normed, (long) d_model);
+    }
     if (topk_scan) {
         GemvFuse f{};
         f.tmax     = s->tmax;
@@ -1533,15 +1589,14 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
+    } else if (q6k_x86) {
+        launch_q6k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,
+                                   d_logits);
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
         rc = table == TABLE_Q4K_PACKED
                  ? q4k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)
-             : table == TABLE_Q6K_PACKED && rows == 1 && !s->projection_portable
-                 /* one row on the x86 backend: its integer decode kernel (q6k_gemv_m1) */
-                 ? q6k_packed_gemv_x86_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
-                                            d_logits, ld_logits)
              : table == TABLE_Q6K_PACKED
                  ? q6k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)

@@ -163,6 +163,18 @@ int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
 int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                        size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                        float *d_y, size_t ld_y);
+/* The two halves of that kernel for callers that keep the int8 activations (several tables
+ * projected from one activation row, or the quantiser placed in an earlier launch):
+ * geist_hip_q8k_quantize_rows replaces the activation quantiser of kernel_q6k_gemv.c:43-67 --
+ * d_act, 64-byte aligned, geist_hip_q8k_act_bytes(n_in, n_rows) bytes, gets per row and
+ * super-block 96 dwords: the 256 activations as int8 in element order, their sixteen sums per
+ * group of sixteen as int32, the scale as binary32, padding. geist_hip_q6k_packed_gemv_q8k
+ * replaces the dot products of kernel_q6k_gemv.c:90-157 for one row of d_act. */
+size_t geist_hip_q8k_act_bytes(size_t n_in, size_t n_rows);
+int geist_hip_q8k_quantize_rows(geist_hip_sampler *s, const float *d_x, size_t ld_x, size_t n_rows,
+                                size_t n_in, void *d_act);
+int geist_hip_q6k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                  size_t n_in, const void *d_act, float *d_y);
 /* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, the projection and the
  * sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. The
  * projection is geist_hip_q6k_linear_rows (the portable arithmetic) over the table as it lies in

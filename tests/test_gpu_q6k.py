@@ -7,7 +7,8 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import oracle_q6k_gemv_x86, oracle_q6k_linear, random_q6k_table
+from oracle_lib import (oracle_q6k_gemv_x86, oracle_q6k_linear, oracle_q8k_quantize,
+                        random_q6k_table)
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -101,6 +102,21 @@ def test_q6k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
             want = oracle_q6k_gemv_x86(oracle.lib, w, x[m], n_in)
             bad = np.flatnonzero(got[m].view(np.uint32) != want.view(np.uint32))
             assert bad.size == 0, (scale, m, bad[:5], got[m][bad[:3]], want[bad[:3]])
+        # the kernel's two halves: the int8 activations as the reference's quantiser leaves
+        # them, and the dot products over them
+        nb = n_in // 256
+        act = torch.full((hs.q8k_act_bytes(n_in, 3) // 4,), -1, dtype=torch.int32, device="cuda")
+        hs.q8k_quantize(d_x, act)
+        y1 = torch.full((n_out,), np.nan, dtype=torch.float32, device="cuda")
+        hs.q6k_packed_gemv_q8k(packed, n_out, n_in, act[2 * nb * 96:], y1)
+        hs.sync()
+        a = act.cpu().numpy().reshape(3, nb, 96)
+        for m in range(3):
+            d, qs, bs = oracle_q8k_quantize(oracle.lib, x[m])
+            assert (a[m, :, :64].copy().view(np.int8).reshape(-1) == qs).all(), (scale, m)
+            assert (a[m, :, 64:80].reshape(-1) == bs.astype(np.int32)).all(), (scale, m)
+            assert (a[m, :, 80].copy().view(np.uint32) == d.view(np.uint32)).all(), (scale, m)
+        assert (y1.cpu().numpy().view(np.uint32) == got[2].view(np.uint32)).all(), scale
 
 
 def test_q6k_argument_errors(hs):
