@@ -692,7 +692,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
          * stage is the whole step) */
         const size_t wgs_row = (size_t) ((L.rv.n_chunks + 3) / 4);
         const size_t wgs     = rows->rows * wgs_row;
-        const bool   one     = plain && s->row_arrive && rows->rows % 8 == 0 &&
+        const bool   one     = plain && s->row_arrive &&
                              wgs <= (size_t) s->fused_wg_limit && rows->n_vocab % 4 == 0 &&
                              wg_cands_bytes(rows->rows, wgs_row) <= wave_cands_bytes(s->wcands_row_waves);
         const size_t per_wg  = 32768;

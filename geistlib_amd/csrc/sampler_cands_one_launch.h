@@ -140,12 +140,11 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
     const int tid = threadIdx.x, lane = tid & (WAVE - 1);
     const int wv  = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int G   = (int) gridDim.x; /* workgroups per row */
-    int       row = (int) blockIdx.y, grp = (int) blockIdx.x;
-    if ((gridDim.y & 7) == 0) { /* the workgroups of a row have linear ids equal modulo 8 */
-        const int lin = (int) (blockIdx.y * gridDim.x + blockIdx.x), slot = lin >> 3;
-        row           = (lin & 7) + 8 * (slot / G);
-        grp           = slot % G;
-    }
+    /* the grid holds the rows in eights: the workgroups of a row have linear ids equal modulo 8 */
+    const int lin = (int) (blockIdx.y * gridDim.x + blockIdx.x), slot = lin >> 3;
+    const int row = (lin & 7) + 8 * (slot / G), grp = slot % G;
+    if (row >= rv.n_rows)
+        return; /* the grid's padding */
     int      *hkey = reinterpret_cast<int *>(s_arena);                    /* -1 = empty */
     uint32_t *hcnt = reinterpret_cast<uint32_t *>(s_arena + OL_HT_SLOTS * 4); /* two a word */
     GS_STAMP(0);
@@ -574,14 +573,18 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
         /* (k <= CAND_K_MAX = 64 on this path) */
         const int tok = finish_sorted_lanes(k, s_pack, a.inv_t, a.top_p, a.min_p, u_row, s_tab);
         if (tid == 0) {
-            a.out[row] = tok;
-            if (nt.h_done) {
-                /* the id has left for where `out` lies before the row counts as done; the row
-                 * that completes the batch tells the host */
+            if (!nt.h_done) {
+                a.out[row] = tok;
+            } else {
+                /* The id is written through to where `out` lies (a plain store may stay in the
+                 * second-level cache until the kernel ends, and the host, told by the word below,
+                 * would read the id of the call before) and has arrived before the row counts as
+                 * done; the row that completes the batch tells the host. */
+                __hip_atomic_store(a.out + row, tok, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 const uint32_t done = __hip_atomic_fetch_add(nt.rows_done, 1u, __ATOMIC_RELAXED,
                                                              __HIP_MEMORY_SCOPE_AGENT) + 1u;
-                if (done == gridDim.y) {
+                if (done == (uint32_t) rv.n_rows) {
                     __hip_atomic_store(nt.rows_done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(nt.h_done, nt.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 }

@@ -2002,7 +2002,9 @@ void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaun
                             bool far_always, const Notify &nt) {
     const FinalArgs a = final_args(f);
     const int       per_wg = OL_THREADS / TPB; /* chunks a workgroup scans */
-    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, L.rows), block(OL_THREADS);
+    /* rows in eights: the workgroups of a row then have linear ids equal modulo 8 and share an
+     * XCD; the workgroups of the rows that are not there leave at once */
+    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, (L.rows + 7) & ~7), block(OL_THREADS);
     auto go = [&](auto kernel) {
         kernel<<<grid, block, 0, L.stream>>>(scan.rv, L.rv, wc, r_w, r_last, a, tmax, arrive,
                                              far_always ? 1 : 0, nt);

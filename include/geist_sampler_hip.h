@@ -167,8 +167,8 @@ int geist_hip_sample_rows_static(int device, void *stream, const struct geist_hi
 int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
 
 /* No counterpart in the reference. The top-k candidate path runs as one launch (the workgroup of
- * a row that finishes scanning last goes on as the row's final stage) when the batch is a
- * multiple of 8 rows, fits the device in one round of workgroups and the device places the
+ * a row that finishes scanning last goes on as the row's final stage) when the batch
+ * fits the device in one round of workgroups and the device places the
  * workgroups of a row where they share a second-level cache (looked at once per device: it
  * decides which form is faster, not whether the one launch is correct -- every launch checks the
  * placement of each row for itself, see geist_hip_sampler_handoff_scope); otherwise as two
@@ -178,11 +178,13 @@ int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
 int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable);
 
 /* No counterpart in the reference. In the one-launch form the workgroups of a row hand their
- * candidates to the one that finishes the row. Each arrival reports the XCD it ran on; when all
- * of a row ran on one XCD the finishing workgroup reads the hand-over from the second-level cache
- * they share, otherwise with agent-scope loads (the hand-over is always written with agent-scope
- * stores). always_agent = 1 makes every row take the second branch whatever its placement -- for
- * tests of that branch; 0 returns to the default. Results are the same either way. */
+ * candidates to the one that finishes the row, through plain stores that are only sure to be
+ * seen inside the second-level cache of the XCD that wrote them. Each arrival reports the XCD it
+ * ran on; when all of a row ran on one XCD the finishing workgroup reads the hand-over from the
+ * cache they share, otherwise it leaves the hand-over unread and finds the row's candidates from
+ * the logits themselves. always_agent = 1 makes every row take the second branch whatever its
+ * placement -- for tests of that branch; 0 returns to the default. Results are the same either
+ * way. */
 int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent);
 
 /* No counterpart in the reference. Stochastic speculative verification sums the residual

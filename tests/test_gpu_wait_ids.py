@@ -72,3 +72,35 @@ def test_ids_reported_into_host_memory(oracle, P, spin_us):
         out_host.close()
     finally:
         hs.close()
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+def test_short_rows_report_after_their_ids_have_arrived(oracle, P, rows):
+    """One workgroup per row and a few rows: the kernel that writes the ids tells the host within
+    a microsecond of writing them, so an id that lingered in a cache on its way would be read one
+    call late. Many calls in a row, every one checked right after the wait."""
+    from geistlib_amd import HipSampler
+    n = 32000
+    g = np.random.default_rng(rows)
+    hs = HipSampler(8, n)
+    try:
+        hs.notify_ids(True)
+        out_host = hs.host_buffer(rows * 4)
+        ids = out_host.view(np.int32)
+        kw = dict(temperature=0.8, top_k=40, top_p=0.95)
+        xs = (g.standard_normal((12, rows, n)) * 2).astype(np.float32)
+        d_xs = [to_dev(x, torch) for x in xs]
+        torch.cuda.synchronize()
+        for call in range(48):
+            x = xs[call % 12]
+            u = units(g, rows)
+            d_u = to_dev(u, torch)
+            hs.sample(HipSampler.rows(d_xs[call % 12]), P(**kw), d_u, out_host)
+            hs.wait_ids()
+            got = ids.copy()
+            want, infos = want_rows(oracle, x, u, **kw)
+            compare_ids(got, want, infos, f"call {call}, {rows} rows")
+        hs.sync()
+        out_host.close()
+    finally:
+        hs.close()
