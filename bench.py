@@ -40,8 +40,8 @@ COLD_WORKING_SET = 640 * 1024 * 1024   # bytes of logits the timed loops cycle t
 # with the summary it was taken from (`roofline.traffic_source`); workloads without a counter
 # run report null.
 PROFILED_TRAFFIC = {
-    "cfg2_b64_v128256_pen2048": (38628690, "profiles/k_cand_scan_final__cfg2_pen.md"),
-    "cfg2_b64_v128256": (38007434, "profiles/k_cand_scan_final__cfg2.md"),
+    "cfg2_b64_v128256_pen2048": (35264326, "profiles/k_cand_scan_final__cfg2_pen.md"),
+    "cfg2_b64_v128256": (34624496, "profiles/k_cand_scan_final__cfg2.md"),
 }
 
 

@@ -3,40 +3,51 @@
  * top-p and min-p of the chain) as ONE launch, for batches that fit the device at one workgroup of
  * 1024 threads per compute unit.
  *
- *   k_cand_scan_final   grid (G, rows), G = ceil(chunks / 4) workgroups per row. A workgroup
- *                       holds 32768 logits of its row in registers (a wavefront 2048, a lane 32).
- *                       It finds a bound T_w that about r of its lane maxima reach, hands on the
- *                       elements at or above T_w -- a few dozen (value, id) pairs -- and adds
- *                       itself to the row's arrival counter. The workgroup that arrives last
- *                       goes on as the row's final stage: B = the largest T_w of the row; every
- *                       element of the row at or above B was handed on by its workgroup (each
- *                       handed on everything >= its own T_w <= B). If k of them still reach B
- *                       after the penalties, the row's k largest are among them (sampler.c:202-215
+ *   k_cand_scan_final   G = ceil(chunks / 4) workgroups per row; the grid holds the rows in
+ *                       eights so that the workgroups of a row have linear ids equal modulo 8,
+ *                       which this device places on one XCD (workgroups of rows that are not
+ *                       there leave at once). A workgroup holds 32768 logits of its row in
+ *                       registers (a wavefront 2048, a lane 32 in eight groups of four). It
+ *                       finds a bound T_w that about r of its group maxima reach, hands on the
+ *                       groups whose maximum reaches T_w -- a few dozen (float4, index) pairs,
+ *                       in slots of their own per wavefront -- and adds itself to the row's
+ *                       arrival counter. The workgroup that arrives last goes on as the row's
+ *                       final stage: B = the largest T_w of the row; every element of the row at
+ *                       or above B was handed on by its workgroup (each handed on every group
+ *                       with an element >= its own T_w <= B). If k of them still reach B after
+ *                       the penalties, the row's k largest are among them (sampler.c:202-215
  *                       keeps the k largest of the sorted row): they are ordered by counting
  *                       (logit descending, index ascending: sampler.c:207 with a stable sort) and
  *                       the first wavefront finishes (softmax over the k, top-p, min-p, draw).
  *                       A row that cannot be certified this way -- leading logits crowded into
  *                       one workgroup, runs of equal values, rows of -inf, many penalised
- *                       leaders -- forms its thread maxima and takes the slower exact paths
- *                       inside the same launch.
+ *                       leaders, more groups than slots -- forms its thread maxima and takes the
+ *                       slower exact paths inside the same launch.
  *
  * `r` is chosen on the host so that a workgroup holding r of the row's k leading logits is a
- * one-in-10^8 event for logits whose order is unrelated to the vocabulary order; it only decides
- * how often the slower paths run, never the token.
+ * one-in-10^8 event for logits whose order is unrelated to the vocabulary order (r_last for the
+ * row's last workgroup, which may hold fewer elements); it only decides how often the slower
+ * paths run, never the token.
  *
  * What does not depend on the logits is done while their loads are in flight: the row's history
- * is read and entered into a bit set of the vocabulary in LDS (one bit per token id: which
- * tokens are penalised at all), the uniform and the expf table are fetched, the lists cleared.
- * The final stage then tests a candidate with one LDS read; the rare candidates that are in the
- * history are counted by comparing them with the history ids every thread still holds.
+ * is entered into an open-addressing table in LDS (16384 slots: token id and a 16-bit count),
+ * the uniform and the expf table are fetched, the lists cleared. The final stage then penalises a
+ * candidate after one probe of the table; only candidates are ever penalised (penalties that can
+ * only lower a logit leave the bound B valid: the check that k entries still reach B proves that
+ * nothing outside the hand-over belongs to the k largest).
  *
- * The hand-over between the workgroups of a row: a workgroup's list is written with agent-scope
- * stores (they are performed where every XCD sees them), the wavefront that wrote them waits for
- * their acknowledgement and adds the workgroup to the row's counter. The sum carries the XCD
- * number of every arrival (count, sum and sum of squares), so the last arrival knows whether all
- * of the row ran on its own XCD: then the lists are in the L2 it shares with them and it reads
- * them with ordinary loads after invalidating its first-level cache; otherwise it reads them
- * with agent-scope loads. Where a row's workgroups are placed can cost time, never a token.
+ * The hand-over between the workgroups of a row goes through plain stores: the wavefront that
+ * wrote its slots waits for their acknowledgement (they are then in the XCD's second-level
+ * cache), and the workgroup's last wavefront adds the workgroup to the row's counter with one
+ * agent-scope atomic. The sum carries the XCD number of every arrival (count, sum and sum of
+ * squares), so the last arrival knows whether all of the row ran on its own XCD: then the slots
+ * are in the L2 it shares with them and it reads them with ordinary loads after invalidating its
+ * first-level cache. Otherwise (or when the host asks for it, for tests) the hand-over is not
+ * read at all: the row takes the slower paths, which read the logits only. Where a row's
+ * workgroups are placed can cost time, never a token.
+ *
+ * With a word in page-locked memory to report to (Notify), the row that completes the batch
+ * publishes the call's number there, after every row's id has been written through to `out`.
  */
 #ifndef GEIST_SAMPLER_CANDS_ONE_LAUNCH_H
 #define GEIST_SAMPLER_CANDS_ONE_LAUNCH_H
