@@ -53,7 +53,9 @@ class SpecHeadView(C.Structure):
 
 
 def library_path(name="libgeist_sampler_hip.so"):
-    return os.path.join(HERE, "lib", name)
+    """Where the built library lies; GEIST_HIP_LIB_DIR names another directory (an instrumented
+    build, `make -C geistlib_amd phase-stamps`)."""
+    return os.path.join(os.environ.get("GEIST_HIP_LIB_DIR") or os.path.join(HERE, "lib"), name)
 
 
 _LIB = None

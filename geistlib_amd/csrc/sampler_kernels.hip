@@ -2202,3 +2202,13 @@ void launch_rng_units(hipStream_t stream, uint64_t *states, int shared, int rows
 }
 
 } // namespace gs
+
+#ifdef GS_PHASE_STAMPS
+/* Instrumented builds only (`make -C geistlib_amd phase-stamps`): the device timestamps that
+ * k_cand_scan_final's workgroups took at their phases during the launches so far, 16 per
+ * workgroup (sampler_cands_one_launch.h). */
+extern "C" int geist_hip_phase_stamps_read(unsigned long long *host, size_t n) {
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(gs::g_phase_stamps),
+                                     n * sizeof(unsigned long long));
+}
+#endif
