@@ -47,8 +47,11 @@ constexpr int Q6K_TPB         = 256;
 /* (float) s, and whether every value within err of s rounds to the same binary32. */
 __device__ __forceinline__ bool q6k_rounding_is_safe(double s, double err, float &f) {
     f = (float) s;
+    /* Not finite: with an infinite or NaN activation the sum's terms are infinities and NaNs,
+     * and this kernel's split into t - 32 * sum x can meet inf - inf where the reference's sum in
+     * index order does not. The kernel that adds in the reference's order decides. */
     if (!(__builtin_fabsf(f) < __builtin_inff()))
-        return true; /* overflow or NaN: the order of the sum does not decide it */
+        return false;
     const double up = 0.5 * ((double) f + (double) nextafterf(f, __builtin_inff()));
     const double dn = 0.5 * ((double) f + (double) nextafterf(f, -__builtin_inff()));
     return up - s > err && s - dn > err;

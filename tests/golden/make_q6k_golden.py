@@ -38,6 +38,20 @@ def main():
         cases.append({"n_out": n_out, "n_in": n_in, "m": m, "w_hex": w.tobytes().hex(),
                       "x_hex": x.tobytes().hex(), "y_hex": y.tobytes().hex(),
                       "dequant_row0_hex": row0.tobytes().hex()})
+    # activations that are not finite: an infinity, two of opposite sign in one row (their
+    # products meet as inf - inf wherever the weights' signs agree), a NaN
+    n_out, n_in, m = 12, 512, 3
+    w = random_q6k_table(g, n_out, n_in, scale_mode="plain")
+    x = g.standard_normal((m, n_in)).astype(np.float32)
+    x[0, 5] = np.inf
+    x[1, 9], x[1, 300] = -np.inf, np.inf
+    x[2, 17] = np.nan
+    y = ref_q6k_linear(ref, w, x, n_in)
+    row0 = np.empty(n_in, dtype=np.float32)
+    ref.dequant_q6_K_row(w[0].ctypes.data_as(C.c_void_p), _fp(row0), n_in)
+    cases.append({"n_out": n_out, "n_in": n_in, "m": m, "w_hex": w.tobytes().hex(),
+                  "x_hex": x.tobytes().hex(), "y_hex": y.tobytes().hex(),
+                  "dequant_row0_hex": row0.tobytes().hex(), "not_finite": True})
     out = os.path.join(HERE, "q6k_ref_vectors.json")
     with open(out, "w") as f:
         json.dump({"source": "oracle/_ref/libgeist_ref_wquant.so (reference weight_resolve.c + q6_K.c)",

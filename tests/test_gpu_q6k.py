@@ -119,6 +119,36 @@ def test_q6k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
         assert (y1.cpu().numpy().view(np.uint32) == got[2].view(np.uint32)).all(), scale
 
 
+def test_q6k_linear_with_activations_that_are_not_finite(hs, oracle):
+    """An infinity, two of opposite sign, a NaN among the activations: the reference's sum in
+    index order gives +-inf or NaN per output (golden case of tests/golden/q6k_ref_vectors.json,
+    written from the compiled reference), and both device kernels give the same -- the kernel
+    over the table as it lies sends every such output to its second, index-order kernel."""
+    g = np.random.default_rng(404)
+    n_out, n_in, m = 700, 768, 4
+    w = random_q6k_table(g, n_out, n_in, scale_mode="plain")
+    x = g.standard_normal((m, n_in)).astype(np.float32)
+    x[0, 5] = np.inf
+    x[1, 9], x[1, 300] = -np.inf, np.inf
+    x[2, 17] = np.nan
+    want = oracle_q6k_linear(oracle.lib, w, x, n_in)     # row 3 is finite
+    assert np.isinf(want[0]).any() and np.isnan(want[1]).any() and np.isinf(want[1]).any()
+    d_w, d_x = torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda()
+    packed = torch.zeros((hs.q6k_packed_bytes(n_out, n_in),), dtype=torch.uint8, device="cuda")
+    hs.q6k_pack(d_w, n_in, packed)
+    for name in ("as in the file", "packed"):
+        y = torch.full((m, n_out), 7.0, dtype=torch.float32, device="cuda")
+        if name == "packed":
+            hs.q6k_packed_linear(packed, n_out, n_in, d_x, y)
+        else:
+            hs.q6k_linear(d_w, n_in, d_x, y)
+        hs.sync()
+        got = y.cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want)), name
+        ok = ~np.isnan(want)
+        assert np.array_equal(got.view(np.uint32)[ok], want.view(np.uint32)[ok]), name
+
+
 def test_q6k_argument_errors(hs):
     from geistlib_amd.binding import GeistHipError
     w = torch.zeros((4, 210), dtype=torch.uint8, device="cuda")
