@@ -86,6 +86,7 @@ def load_library():
     lib.geist_hip_sampler_one_launch_topk.argtypes = [vp, i32]
     lib.geist_hip_sampler_one_launch_spec.argtypes = [vp, i32]
     lib.geist_hip_sampler_handoff_scope.argtypes = [vp, i32]
+    lib.geist_hip_sampler_set_whole_row_walk.argtypes = [vp, i32]
     lib.geist_hip_sampler_notify_ids.argtypes = [vp, i32]
     lib.geist_hip_sampler_wait_ids.argtypes = [vp]
     lib.geist_hip_sampler_set_wait_spin.argtypes = [vp, C.c_uint32]
@@ -220,6 +221,10 @@ class HipSampler:
 
     def set_wait_limit(self, polls):
         self._check(self.lib.geist_hip_sampler_set_wait_limit(self.h, C.c_uint32(polls)))
+
+    def set_whole_row_walk(self, mode):
+        """0 adaptive (default), 1 always spread over the row's chunks, 2 one workgroup."""
+        self._check(self.lib.geist_hip_sampler_set_whole_row_walk(self.h, int(mode)))
 
     def one_launch_topk(self, enable=True):
         """Whether the top-k candidate path runs as one launch for batches that qualify."""

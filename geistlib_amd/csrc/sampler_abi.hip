@@ -81,6 +81,15 @@ struct geist_hip_sampler {
     float    *probs      = nullptr; /* [max_rows][max_vocab], allocated on first use by the
                                      * full-vocabulary top-p / min-p path */
     gs::CandSpace cand   = {};      /* candidate lists of that path, allocated with probs */
+    void     *walk_rows  = nullptr; /* workspace of the whole-row walk spread over the row's
+                                     * chunks (sampler_walk_coop.h), allocated with probs */
+    uint32_t *walk_hint  = nullptr; /* pinned, two words: the number of the last call in which
+                                     * a row was walked in full / in which a wait ran out */
+    uint32_t  walk_steps = 0;       /* step numbers handed out so far */
+    uint32_t  walk_calls = 0;       /* calls of the top-p / min-p path so far */
+    uint32_t  walk_cleared = 0;     /* ... the one before which the workspace was last cleared */
+    int       walk_mode  = 0;       /* geist_hip_sampler_set_whole_row_walk */
+    bool      walk_clear = false;   /* clear the workspace before its next use */
     void    *q6k_ws      = nullptr; /* scratch of the Q6_K projection, sized like f64_ws */
     size_t   q6k_in = 0, q6k_out = 0;
     void    *f64_ws      = nullptr; /* scratch of the f64 projection for n_in <= f64_in and
@@ -390,6 +399,9 @@ void geist_hip_sampler_destroy(geist_hip_sampler *s) {
     (void) hipFree(s->probe_p);
     (void) hipFree(s->scalar_out);
     (void) hipFree(s->probs);
+    (void) hipFree(s->walk_rows);
+    if (s->walk_hint)
+        (void) hipHostFree(s->walk_hint);
     (void) hipFree(s->f64_ws);
     (void) hipFree(s->q6k_ws);
     (void) hipFree(s->cand.row_bound);
@@ -574,16 +586,28 @@ static int reserve_sorted_workspace(geist_hip_sampler *s) {
     if (e == hipSuccess) e = hipMalloc((void **) &c.row_sum, R * sizeof(double));
     if (e == hipSuccess) e = hipMalloc((void **) &c.path, R * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void **) &probs, R * s->max_vocab * sizeof(float));
+    void     *walk_rows = nullptr;
+    uint32_t *walk_hint = nullptr;
+    if (e == hipSuccess) e = hipMalloc(&walk_rows, gs::walk_coop_bytes(R));
+    if (e == hipSuccess) e = hipMemsetAsync(walk_rows, 0, gs::walk_coop_bytes(R), s->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
+    if (e == hipSuccess) e = hipHostMalloc((void **) &walk_hint, 64, hipHostMallocDefault);
     if (e != hipSuccess) {
-        void *ptrs[] = {c.row_bound, c.out_key, c.key, c.idx, c.count, c.row_sum, c.path, probs};
+        void *ptrs[] = {c.row_bound, c.out_key, c.key, c.idx, c.count, c.row_sum, c.path, probs,
+                        walk_rows};
         for (void *q : ptrs)
             if (q)
                 (void) hipFree(q);
+        if (walk_hint)
+            (void) hipHostFree(walk_hint);
         return fail(s, e == hipErrorOutOfMemory ? GEIST_HIP_E_OOM : GEIST_HIP_E_BACKEND,
                     "workspace of the top-p / min-p path: %s", hipGetErrorString(e));
     }
     s->cand  = c;
     s->probs = probs;
+    walk_hint[0] = walk_hint[1] = 0u;
+    s->walk_rows = walk_rows;
+    s->walk_hint = walk_hint;
     return GEIST_HIP_OK;
 }
 
@@ -802,7 +826,39 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
      * walk comes first and alone. */
     if (!f.minp_direct)
         launch_row_final(L, f);
-    launch_candidates(L, f, s->probs, (long) s->max_vocab);
+    /* Rows that neither shortcut nor list can serve are walked in full: by their one workgroup
+     * inside the list-walk kernel, or spread over the workgroups of their chunks by a kernel
+     * behind it. That kernel is a launch more for every call, so it is sent only while such rows
+     * keep turning up: the kernels say so in a page-locked word, which is looked at here without
+     * waiting for anything (a stale value costs time, never a token). */
+    WalkCoop wc = {};
+    wc.rows       = s->walk_rows;
+    wc.hint       = s->walk_hint;
+    wc.wait_limit = s->wait_limit;
+    if (s->walk_rows && s->walk_hint) {
+        /* (calls are numbered from 1; a hint from one of the last 64 calls counts: with
+         * several calls in flight the kernels' word lags behind) */
+        const uint32_t call   = ++s->walk_calls;
+        const uint32_t walked = __atomic_load_n(&s->walk_hint[0], __ATOMIC_RELAXED);
+        const uint32_t ranout = __atomic_load_n(&s->walk_hint[1], __ATOMIC_RELAXED);
+        wc.call   = call;
+        /* the spread form holds two workgroups per compute unit: beyond a few rounds of them the
+         * rows' own workgroups, all at once, are the faster way */
+        const bool fits = rows->rows * (size_t) L.rv.n_chunks <= 1280;
+        wc.spread = s->walk_mode == GEIST_HIP_WHOLE_ROW_WALK_SPREAD ||
+                    (s->walk_mode == GEIST_HIP_WHOLE_ROW_WALK_ADAPTIVE && fits && walked != 0u &&
+                     call - walked <= 64u);
+        if (wc.spread) {
+            wc.clear = (ranout != 0u && (int32_t) (ranout - s->walk_cleared) >= 0) ||
+                       s->walk_clear;
+            if (wc.clear)
+                s->walk_cleared = call;
+            s->walk_clear = s->wait_limit < 1024u; /* (a bound set for tests: clear behind it) */
+            wc.step_base  = s->walk_steps;
+            s->walk_steps += 16u;
+        }
+    }
+    launch_candidates(L, f, s->probs, (long) s->max_vocab, wc);
     return after_launch(s, "top-p / min-p");
 }
 
@@ -826,6 +882,16 @@ int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable) {
         return GEIST_HIP_E_INVALID_ARG;
     s->fused_wg_limit = enable ? s->fused_wg_default : 0;
     return s->fused_wg_limit > 0 ? 1 : 0;
+}
+
+int geist_hip_sampler_set_whole_row_walk(geist_hip_sampler *s, int mode) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (mode != GEIST_HIP_WHOLE_ROW_WALK_ADAPTIVE && mode != GEIST_HIP_WHOLE_ROW_WALK_SPREAD &&
+        mode != GEIST_HIP_WHOLE_ROW_WALK_ONE_WORKGROUP)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown whole-row walk mode %d", mode);
+    s->walk_mode = mode;
+    return GEIST_HIP_OK;
 }
 
 int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent) {

@@ -258,7 +258,25 @@ int configure_device_kernels();
 /* rows flagged 1 by the sorted row-final kernel: list their candidates, then draw from the
  * list; rows the list cannot serve (and rows the row-final kernel flagged 2) take the whole-row
  * walk in the same launch: probabilities of the whole row into `probs`, then the walk over them */
-void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs);
+/* The whole-row walk spread over the workgroups of the row's chunks (sampler_walk_coop.h), for
+ * the rows the list walk flags 2 when `spread` is set: `rows` is the workspace of
+ * walk_coop_bytes(max rows) bytes, zero before its first use and cleared again by this call when
+ * `clear` is set; the steps of this launch are numbered from step_base + 1 on (at most 16); `hint`
+ * (two words of page-locked host memory, or null): a launch in which a row was walked in full
+ * writes the call's number `call` to word 0, one in which a wait ran out (the workspace then has
+ * to be cleared) to word 1. */
+struct WalkCoop {
+    void     *rows;
+    bool      spread;
+    bool      clear;
+    uint32_t  step_base;
+    uint32_t  wait_limit;
+    uint32_t *hint;
+    uint32_t  call;
+};
+size_t walk_coop_bytes(size_t rows);
+void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs,
+                       const WalkCoop &wc);
 /* row_flag != NULL: only rows flagged 2 are written */
 void launch_write_probs(const Launch &L, float inv_t, const uint64_t *chunk_best,
                         const double *chunk_sum, float *probs, long ld_probs,

@@ -1356,6 +1356,7 @@ __device__ __forceinline__ bool topk_from_tmax(const RowView &rv, const FinalArg
 #include "sampler_walk.h"
 #include "sampler_draw.h"
 #include "sampler_sorted_prob.h"
+#include "sampler_walk_coop.h"
 #include "sampler_spec.h"
 #include "sampler_draft.h"
 #include "sampler_cands.h"
@@ -2136,7 +2137,10 @@ int configure_device_kernels() {
     return 0;
 }
 
-void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs) {
+size_t walk_coop_bytes(size_t rows) { return rows * sizeof(CoopRow); }
+
+void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long ld_probs,
+                       const WalkCoop &wc) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
     const int  dyn = CAND_CAP * (int) sizeof(uint32_t); /* see configure_device_kernels() */
     SortedRowArgs g;
@@ -2145,6 +2149,8 @@ void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long
     g.chunk_sum  = f.chunk_sum;
     g.probs      = probs;
     g.ld_probs   = ld_probs;
+    /* the cooperative whole-row walk holds a chunk of 8192 in registers */
+    const int defer = wc.rows != nullptr && wc.spread && L.nv == 8 ? 1 : 0;
     if (f.minp_direct) {
         /* the exp-sum pass has listed every row: no row-final kernel, no listing pass. An
          * unlisted element lies in z bin zb + 1 or beyond; the same expf as on the device. */
@@ -2154,16 +2160,39 @@ void launch_candidates(const Launch &L, const FinalLaunch &f, float *probs, long
         dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
             k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
                 L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, f.chunk_sum,
-                L.rv.n_chunks, p_out);
+                L.rv.n_chunks, p_out, defer, wc.hint, wc.call);
         });
-        return;
+    } else {
+        dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
+            k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
+                L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
+            k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
+                L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f,
+                defer, wc.hint, wc.call);
+        });
     }
-    dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
-        k_list_candidates<GS_NV, GS_PEN><<<grid, block, 0, L.stream>>>(
-            L.rv, f.inv_t, f.chunk_best, f.chunk_sum, f.row_flag, f.cand);
-        k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
-            L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f);
-    });
+    if (defer) {
+        /* the rows flagged 2, a workgroup per chunk */
+        if (wc.clear)
+            launch_zero_words(L.stream, static_cast<uint64_t *>(wc.rows),
+                              (uint32_t) (walk_coop_bytes((size_t) L.rows) / sizeof(uint64_t)));
+        CoopRow *cr = static_cast<CoopRow *>(wc.rows);
+        if (L.pen)
+            k_whole_row_coop<8, true><<<grid, block, 0, L.stream>>>(
+                L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, cr, wc.step_base,
+                wc.wait_limit, wc.hint, wc.call);
+        else
+            k_whole_row_coop<8, false><<<grid, block, 0, L.stream>>>(
+                L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, cr, wc.step_base,
+                wc.wait_limit, wc.hint, wc.call);
+        /* rows that are still flagged 2 (a wait ran out, sums that are not finite): one workgroup
+         * each, as without the spread walk */
+        dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
+            k_sorted_candidates<GS_NV, GS_PEN><<<dim3(L.rows), block, dyn, L.stream>>>(
+                L.rv, g, f.cand, f.top_p, f.min_p, f.uniforms, f.row_flag, f.out, nullptr, 0, 0.0f,
+                0, nullptr, 0u);
+        });
+    }
 }
 
 void launch_logprob(const Launch &L, const uint64_t *chunk_best, double *chunk_sum,

@@ -433,6 +433,67 @@ __device__ __forceinline__ void for_each_entry(const float *pn, int n, F &&f) {
         f(i, pn[i]);
 }
 
+/* The digit of a level's histogram (sh.cnt / sh.mass, complete and published by a barrier) at
+ * which the running mass, counted from the largest digit down and starting from mass_above,
+ * first reaches `target`: sh.res_digit (-1: not reached), sh.res_mass_above and
+ * sh.res_cnt_above (strictly greater digits, on top of mass_above / cnt_above). Called by every
+ * thread of the workgroup; ends with a barrier. */
+__device__ __forceinline__ void sg_select_digit(SortedGenShared &sh, uint64_t target,
+                                                uint64_t mass_above, uint32_t cnt_above) {
+    const int tid = threadIdx.x;
+    /* thread t owns the 8 digits SG_BINS-1-8t .. SG_BINS-8-8t, i.e. descending order */
+    uint64_t lm = 0;
+    uint32_t lc = 0;
+#pragma unroll
+    for (int q = 0; q < SG_BINS / TPB; ++q) {
+        const int d = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
+        lm += sh.mass[d];
+        lc += sh.cnt[d];
+    }
+    /* exclusive prefix over threads (descending digits) */
+    uint64_t im = lm;
+    uint32_t ic = lc;
+    {
+        const int lane = tid & (WAVE - 1), w = tid / WAVE;
+#pragma unroll
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const uint64_t om = ((uint64_t) (uint32_t) __shfl_up((int) (im >> 32), d, WAVE) << 32) |
+                                (uint32_t) __shfl_up((int) (uint32_t) im, d, WAVE);
+            const uint32_t oc = (uint32_t) __shfl_up((int) ic, d, WAVE);
+            if (lane >= d) {
+                im += om;
+                ic += oc;
+            }
+        }
+        if (lane == WAVE - 1) {
+            sh.scan64[w] = im;
+            sh.scan32[w] = ic;
+        }
+        if (tid == 0)
+            sh.res_digit = -1;
+        __syncthreads();
+        for (int x = 0; x < w; ++x) {
+            im += sh.scan64[x];
+            ic += sh.scan32[x];
+        }
+    }
+    uint64_t run_m = mass_above + (im - lm);
+    uint32_t run_c = cnt_above + (ic - lc);
+#pragma unroll
+    for (int q = 0; q < SG_BINS / TPB; ++q) {
+        const int      d  = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
+        const uint64_t bm = sh.mass[d];
+        if (sh.cnt[d] && run_m < target && run_m + bm >= target) {
+            sh.res_digit      = d;
+            sh.res_mass_above = run_m;
+            sh.res_cnt_above  = run_c;
+        }
+        run_m += bm;
+        run_c += sh.cnt[d];
+    }
+    __syncthreads();
+}
+
 /* One descent. `limit_key`/`limit_ties`: only entries that precede the (limit_key, limit_ties)
  * edge of a previous descent take part -- entries with key > limit_key, plus the first
  * limit_ties (by index) of those equal to it, whose mass is limit_ties * fx(limit_key); pass
@@ -475,57 +536,7 @@ __device__ bool sg_descent(const float *pn, int n, uint64_t target, bool limited
                       (unsigned long long) (pn_fx(__uint_as_float(limit_key)) * limit_ties));
         }
         __syncthreads();
-        /* thread t owns the 8 digits SG_BINS-1-8t .. SG_BINS-8-8t, i.e. descending order */
-        uint64_t lm = 0;
-        uint32_t lc = 0;
-#pragma unroll
-        for (int q = 0; q < SG_BINS / TPB; ++q) {
-            const int d = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
-            lm += sh.mass[d];
-            lc += sh.cnt[d];
-        }
-        /* exclusive prefix over threads (descending digits) */
-        uint64_t im = lm;
-        uint32_t ic = lc;
-        {
-            const int lane = tid & (WAVE - 1), w = tid / WAVE;
-#pragma unroll
-            for (int d = 1; d < WAVE; d <<= 1) {
-                const uint64_t om = ((uint64_t) (uint32_t) __shfl_up((int) (im >> 32), d, WAVE) << 32) |
-                                    (uint32_t) __shfl_up((int) (uint32_t) im, d, WAVE);
-                const uint32_t oc = (uint32_t) __shfl_up((int) ic, d, WAVE);
-                if (lane >= d) {
-                    im += om;
-                    ic += oc;
-                }
-            }
-            if (lane == WAVE - 1) {
-                sh.scan64[w] = im;
-                sh.scan32[w] = ic;
-            }
-            if (tid == 0)
-                sh.res_digit = -1;
-            __syncthreads();
-            for (int x = 0; x < w; ++x) {
-                im += sh.scan64[x];
-                ic += sh.scan32[x];
-            }
-        }
-        uint64_t run_m = mass_above + (im - lm);
-        uint32_t run_c = cnt_above + (ic - lc);
-#pragma unroll
-        for (int q = 0; q < SG_BINS / TPB; ++q) {
-            const int      d  = SG_BINS - 1 - (tid * (SG_BINS / TPB) + q);
-            const uint64_t bm = sh.mass[d];
-            if (sh.cnt[d] && run_m < target && run_m + bm >= target) {
-                sh.res_digit      = d;
-                sh.res_mass_above = run_m;
-                sh.res_cnt_above  = run_c;
-            }
-            run_m += bm;
-            run_c += sh.cnt[d];
-        }
-        __syncthreads();
+        sg_select_digit(sh, target, mass_above, cnt_above);
         const int d = sh.res_digit;
         if (d < 0)
             return false;
@@ -1184,7 +1195,11 @@ __device__ __forceinline__ int list_walk_fast(const float *pn, const uint32_t *i
  * holds softmax arguments, not pn) and no other kernel ran in between: the row's sum is taken from the chunk
  * sums here (in chunk order, as everywhere), the bound on an unlisted element's pn from
  * direct_p_out = expf of the first z bin outside the list, and the flag is written for every
- * row. */
+ * row.
+ * walk_hint (page-locked host memory, or null): set to walk_call, the call's number, when a row
+ * of the launch needs the whole-row walk -- the host then sends the next calls' such rows to
+ * k_whole_row_coop, which spreads the walk over the row's chunks: this launch is told so by
+ * defer_walk and only flags them 2. */
 template <int NV, bool PEN>
 __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRowArgs g,
                                                            CandSpace cand, float top_p, float min_p,
@@ -1192,7 +1207,10 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
                                                            int32_t *__restrict__ row_flag,
                                                            int32_t *__restrict__ out,
                                                            const double *__restrict__ direct_sum,
-                                                           int n_chunks, float direct_p_out) {
+                                                           int n_chunks, float direct_p_out,
+                                                           int defer_walk,
+                                                           uint32_t *__restrict__ walk_hint,
+                                                           uint32_t walk_call) {
     extern __shared__ uint32_t s_key[]; /* CAND_CAP keys: every list is walked from LDS */
     __shared__ union {
         SortedGenShared gen;
@@ -1227,6 +1245,10 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
         s_csum[tid] = csum;
     __syncthreads();
     if (flag == 2) { /* sent past the list by the row-final kernel */
+        if (tid == 0 && walk_hint)
+            *walk_hint = walk_call;
+        if (defer_walk)
+            return; /* k_whole_row_coop follows and serves the rows flagged 2 */
         const int t = sorted_general_row<NV, PEN>(rv, row, rv.n_rows, g, top_p, min_p,
                                                   u_row, sh.gen, s_cnt16, s_tab, s_scan,
                                                   &s_pick, &s_total);
@@ -1298,6 +1320,13 @@ __global__ __launch_bounds__(TPB) void k_sorted_candidates(RowView rv, SortedRow
      * every thread) */
     int path = 2;
     if (tok < 0) {
+        if (tid == 0 && walk_hint)
+            *walk_hint = walk_call;
+        if (defer_walk) {
+            if (tid == 0)
+                row_flag[row] = 2;
+            return;
+        }
         tok  = sorted_general_row<NV, PEN>(rv, row, rv.n_rows, g, top_p, min_p, u_row,
                                            sh.gen, s_cnt16, s_tab, s_scan, &s_pick, &s_total);
         path = 3;

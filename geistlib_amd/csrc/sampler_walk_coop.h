@@ -1,0 +1,509 @@
+/*
+ * sampler_walk_coop.h -- the whole-row walk of the top-p / min-p modes (sampler.c:246-304: sort
+ * by probability, keep the nucleus, draw) spread over the workgroups of the row's chunks.
+ *
+ * One workgroup walking a row of 128 k probabilities makes some nine passes over them, 275 to
+ * 300 us in all. Here the workgroup of each chunk keeps its 8192 probabilities in registers, and
+ * a pass is: every workgroup adds its share to a histogram of the row in global memory
+ * (agent-scope atomics; sums of integers, so their order does not matter), the workgroups meet at
+ * the row's arrival counter, the one that arrives last reads the histogram, selects the digit as
+ * the one-workgroup walk does (sg_select_digit), clears the histogram and publishes the result
+ * with the step's number; the others wait for that number. The steps: the first level of the
+ * nucleus descent together with the min-p sums, its two further levels, the three levels of the
+ * draw's descent, and the index-order count that finds the j-th entry equal to the drawn value.
+ * The arithmetic is that of sorted_descend<false> (sampler_sorted_prob.h) step for step: masses
+ * in 2^-62 fixed point, the same targets, the same edge rules.
+ *
+ * No fences: a workgroup's atomics are acknowledged (s_waitcnt vmcnt(0)) before it arrives, and
+ * what the last arrival publishes is written and read with agent-scope accesses. Every wait is
+ * bounded (`wait_limit` polls); a workgroup whose wait runs out leaves -- it is then missed at the
+ * next meeting, where the others' waits run out in turn --, the row keeps its flag, and the
+ * one-workgroup walk that the host launches behind this kernel serves it: a row is always served,
+ * whatever the others do. The last step has no wait: the workgroup that arrives last finds the chunk
+ * that holds the drawn entry and, if it is not its own, forms that chunk's probabilities once
+ * more. The row's workspace is zero before the first launch and left zero by every launch that
+ * ends without a wait running out (steps are numbered on from `step_base`, so the published
+ * number needs no clearing); a launch in which one did says so in the host's hint words (the
+ * call's number: in word 0 when a row was walked in full, in word 1 when a wait ran out), and the
+ * host clears the workspace before the next.
+ */
+#ifndef GEIST_SAMPLER_WALK_COOP_H
+#define GEIST_SAMPLER_WALK_COOP_H
+
+namespace gs {
+
+struct CoopRow {
+    uint32_t cnt[SG_BINS];
+    uint64_t mass[SG_BINS];
+    uint64_t aux[4];                /* sums of the first step, added by every workgroup */
+    uint32_t chunk_cnt[MAX_CHUNKS]; /* entries equal to the drawn value, per chunk */
+    uint32_t arrive;
+    uint32_t epoch; /* number of the last step whose result is published */
+    int32_t  res_digit;
+    uint32_t res_cnt_above;
+    uint32_t res_ties;
+    uint32_t pad;
+    uint64_t res_mass_above;
+};
+static_assert(sizeof(CoopRow) % 8 == 0, "rows of the workspace stay 8-byte aligned");
+
+__device__ __forceinline__ uint32_t coop_ld32(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t coop_ld64(const uint64_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coop_st32(uint32_t *p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coop_st64(uint64_t *p, uint64_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coop_add32(uint32_t *p, uint32_t v) {
+    (void) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coop_add64(uint64_t *p, uint64_t v) {
+    (void) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct CoopShared {
+    int last; /* this workgroup arrived last at the step's meeting */
+    int ok;   /* the step's result has been published */
+};
+
+/* What the workgroup has added to the row's workspace is performed; true in the workgroup that
+ * arrives last of the row's W. */
+__device__ __forceinline__ bool coop_arrive(CoopRow *cr, int W, CoopShared &cs) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t before =
+            __hip_atomic_fetch_add(&cr->arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        cs.last = before == (uint32_t) W - 1u;
+        if (cs.last)
+            coop_st32(&cr->arrive, 0u); /* (nobody arrives again before the step is published) */
+    }
+    __syncthreads();
+    return cs.last != 0;
+}
+/* The last arrival's results are written: publish the step. */
+__device__ __forceinline__ void coop_publish(CoopRow *cr, uint32_t step) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+        coop_st32(&cr->epoch, step);
+}
+/* Waits until the step is published; false when the wait ran out. */
+__device__ __forceinline__ bool coop_wait(const CoopRow *cr, uint32_t step, uint32_t limit,
+                                          CoopShared &cs) {
+    if (threadIdx.x == 0) {
+        int      ok = 0;
+        uint32_t polls = 0;
+        for (;;) {
+            if ((int32_t) (coop_ld32(&cr->epoch) - step) >= 0) {
+                ok = 1;
+                break;
+            }
+            if (polls++ >= limit)
+                break;
+            __builtin_amdgcn_s_sleep(8);
+        }
+        cs.ok = ok;
+    }
+    __syncthreads();
+    const bool ok = cs.ok != 0;
+    __syncthreads();
+    return ok;
+}
+
+/* One level of a descent over the row: `add(key)` says whether an entry of this workgroup takes
+ * part; its digit is (key >> shf) & dm. With `select` the last arrival picks the digit at which
+ * the running mass reaches `target` and publishes it; mass_above / cnt_above / ties are updated
+ * in every workgroup. Returns 1 (digit in `digit`), 0 (the target is not reached, or nothing
+ * was to be selected), -1 (the wait ran out). */
+template <int NK, typename Take>
+__device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, uint32_t limit,
+                                          SortedGenShared &sh, CoopShared &cs,
+                                          const uint32_t (&key)[NK], Take take, int shf,
+                                          uint32_t dm, bool select, bool clear_aux,
+                                          uint64_t target, uint64_t &mass_above,
+                                          uint32_t &cnt_above, uint32_t &ties, int &digit) {
+    const int tid = threadIdx.x;
+    for (int i = tid; i < SG_BINS; i += TPB) {
+        sh.cnt[i]  = 0u;
+        sh.mass[i] = 0ull;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        if (take(key[i])) {
+            const uint32_t d = (key[i] >> shf) & dm;
+            atomicAdd(&sh.cnt[d], 1u);
+            atomicAdd((unsigned long long *) &sh.mass[d],
+                      (unsigned long long) pn_fx(__uint_as_float(key[i])));
+        }
+        /* (four entries at a time: interleaving all of them costs registers, not time) */
+        if ((i & 3) == 3)
+            __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+    for (int i = tid; i < SG_BINS; i += TPB) {
+        const uint32_t c = sh.cnt[i];
+        if (c) {
+            coop_add32(&cr->cnt[i], c);
+            coop_add64(&cr->mass[i], sh.mass[i]);
+        }
+    }
+    ++step;
+    if (coop_arrive(cr, W, cs)) {
+        {
+            /* all of a thread's loads in flight together: one round trip, not sixteen */
+            constexpr int PER = SG_BINS / TPB;
+            uint32_t      c[PER];
+            uint64_t      m[PER];
+#pragma unroll
+            for (int q = 0; q < PER; ++q)
+                c[q] = coop_ld32(&cr->cnt[q * TPB + tid]);
+#pragma unroll
+            for (int q = 0; q < PER; ++q)
+                m[q] = coop_ld64(&cr->mass[q * TPB + tid]);
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                sh.cnt[q * TPB + tid]  = c[q];
+                sh.mass[q * TPB + tid] = m[q];
+            }
+        }
+        __syncthreads();
+        for (int i = tid; i < SG_BINS; i += TPB) { /* for the next level */
+            coop_st32(&cr->cnt[i], 0u);
+            coop_st64(&cr->mass[i], 0ull);
+        }
+        if (clear_aux && tid < 4) /* (every workgroup has read them before it arrived here) */
+            coop_st64(&cr->aux[tid], 0ull);
+        if (select)
+            sg_select_digit(sh, target, mass_above, cnt_above);
+        if (tid == 0) {
+            const int d = select ? sh.res_digit : -1;
+            coop_st32(reinterpret_cast<uint32_t *>(&cr->res_digit), (uint32_t) d);
+            if (d >= 0) {
+                coop_st32(&cr->res_cnt_above, sh.res_cnt_above);
+                coop_st64(&cr->res_mass_above, sh.res_mass_above);
+                coop_st32(&cr->res_ties, sh.cnt[d]);
+            }
+        }
+        coop_publish(cr, step);
+    } else if (!coop_wait(cr, step, limit, cs)) {
+        return -1;
+    }
+    /* (the last arrival reads its own stores back: program order, same addresses; the four
+     * loads go out together) */
+    digit                = (int) coop_ld32(reinterpret_cast<const uint32_t *>(&cr->res_digit));
+    const uint32_t r_cnt = coop_ld32(&cr->res_cnt_above);
+    const uint64_t r_mas = coop_ld64(&cr->res_mass_above);
+    const uint32_t r_tie = coop_ld32(&cr->res_ties);
+    if (digit < 0)
+        return 0;
+    cnt_above  = r_cnt;
+    mass_above = r_mas;
+    ties       = r_tie;
+    return 1;
+}
+
+/* Three levels (11, 11, 10 bits of the key): sg_descent over the row's workgroups. `lead` is
+ * the row's first workgroup, which adds the block of limit_ties entries equal to limit_key.
+ * Returns 1 / 0 / -1 as coop_level. */
+template <int NK>
+__device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, uint32_t limit,
+                                            SortedGenShared &sh, CoopShared &cs,
+                                            const uint32_t (&key)[NK], bool lead, bool clear_aux,
+                                            uint64_t target, bool limited, uint32_t limit_key,
+                                            uint32_t limit_ties,
+                                            uint32_t &kappa, uint32_t &cnt_above,
+                                            uint64_t &mass_above, uint32_t &ties_total) {
+    uint32_t prefix = 0u, mask = 0u;
+    cnt_above  = 0u;
+    mass_above = 0ull;
+    ties_total = 0u;
+#pragma unroll 1
+    for (int lv = 0; lv < 3; ++lv) {
+        const int      shf = lv == 0 ? 21 : lv == 1 ? 10 : 0;
+        const uint32_t dm  = lv == 2 ? 1023u : 2047u;
+        /* the block of entries equal to the limit, as one more key of the first workgroup's
+         * first thread: handled apart, its mass is limit_ties times the entry's */
+        const bool block_here = limited && lead && threadIdx.x == 0 && limit_ties &&
+                                (limit_key & mask) == prefix;
+        auto take = [&](uint32_t k) {
+            return k != 0xffffffffu && (k & mask) == prefix && !(limited && k <= limit_key);
+        };
+        /* the block is added after the level's own zeroing: through a key list of one more
+         * entry would cost every level a register; it goes straight to the global histogram */
+        if (block_here) {
+            const uint32_t d = (limit_key >> shf) & dm;
+            coop_add32(&cr->cnt[d], limit_ties);
+            coop_add64(&cr->mass[d], pn_fx(__uint_as_float(limit_key)) * (uint64_t) limit_ties);
+        }
+        int       digit = -1;
+        const int r = coop_level<NK>(cr, W, step, limit, sh, cs, key, take, shf, dm, true,
+                                     clear_aux && lv == 0, target, mass_above, cnt_above,
+                                     ties_total, digit);
+        if (r <= 0)
+            return r;
+        prefix |= (uint32_t) digit << shf;
+        mask |= dm << shf;
+    }
+    kappa = prefix;
+    return 1;
+}
+
+template <int NV, bool PEN>
+__global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRowArgs g, CandSpace cand,
+                                                        float top_p, float min_p,
+                                                        const float *__restrict__ uniforms,
+                                                        int32_t *__restrict__ row_flag,
+                                                        int32_t *__restrict__ out,
+                                                        CoopRow *__restrict__ coop,
+                                                        uint32_t step_base, uint32_t wait_limit,
+                                                        uint32_t *__restrict__ hint,
+                                                        uint32_t call) {
+    __shared__ SortedGenShared sh;
+    __shared__ CoopShared      cs;
+    __shared__ __align__(16) uint32_t s_cnt16[PEN ? NV * TPB * 2 : 1];
+    __shared__ uint64_t s_tab[32];
+    __shared__ double   s_total;
+    __shared__ int      s_scan[NWAVES];
+    int row, chunk;
+    xcd_row_chunk(row, chunk);
+    if (row_flag[row] != 2)
+        return;
+    const int   tid = threadIdx.x, W = rv.n_chunks;
+    const bool  lead = chunk == 0;
+    const float u    = uniforms[row];
+    CoopRow    *cr   = coop + row;
+    if (lead && tid == 0 && hint)
+        hint[0] = call; /* rows are being walked in full: the host keeps sending them here */
+    /* A row that is not served here keeps its flag, and the one-workgroup walk of the launch
+     * behind this one serves it: rows whose sums are not finite (the reference's own answer for
+     * those comes out of that walk), and rows of a launch in which a wait ran out -- then the
+     * row's workspace may hold a step's remains, and the host is told to clear it. */
+    auto alone = [&](bool dirty) {
+        if (dirty && lead && tid == 0 && hint)
+            hint[1] = call;
+    };
+    if (tid < 32)
+        s_tab[tid] = g_expf_tab[tid];
+    if (tid == 0) {
+        double t = 0.0;
+        for (int c = 0; c < rv.n_chunks; ++c)
+            t += g.chunk_sum[(long) row * rv.n_chunks + c];
+        s_total = t;
+    }
+    const float mx = key2f(best_key(row_best_from_chunks(g.chunk_best, row, rv.n_chunks, sh.red64)));
+    __syncthreads();
+    const double tot = s_total;
+    if (!(tot > 0.0 && tot < __builtin_inf() && mx > -__builtin_inff() && mx < __builtin_inff())) {
+        alone(false);
+        return;
+    }
+    /* this chunk's normalised probabilities pn = (float)((double)p / sum) (sampler.c:246-253),
+     * kept in registers as their bit patterns; 0xffffffff marks places beyond the row */
+    int base, end;
+    chunk_bounds<NV>(rv, chunk, base, end);
+    uint32_t key[4 * NV];
+    {
+        float4 v[NV];
+        fetch_chunk<NV, PEN>(rv, row, rv.n_rows, base, end, s_cnt16, v);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int e = base + 4 * (j * TPB + tid);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                uint32_t k = 0xffffffffu;
+                if (e + c < end) {
+                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[j], c), mx, g.inv_t), s_tab);
+                    k             = __float_as_uint((float) ((double) p / tot));
+                }
+                key[4 * j + c] = k;
+            }
+            /* one group of four at a time: left alone the compiler interleaves all 32
+             * evaluations, and the registers that takes cost the kernel its occupancy */
+            if (j + 1 < NV)
+                asm volatile("" : "+v"(key[4 * j + 3]), "+v"(v[j + 1].x), "+v"(v[j + 1].y),
+                                  "+v"(v[j + 1].z), "+v"(v[j + 1].w));
+        }
+    }
+    const bool use_p = top_p > 0.0f && top_p < 1.0f;
+    const bool use_m = min_p > 0.0f;
+    /* the largest probability is that of the row's maximum: expf(0) = 1 over the sum */
+    const uint32_t kmax    = __float_as_uint((float) (1.0 / tot));
+    const float    floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
+    uint32_t       step    = step_base;
+    /* ---- step 1: the first level of the nucleus descent, the min-p prefix, the row's mass ---- */
+    {
+        uint64_t a[4] = {0ull, 0ull, 0ull, 0ull};
+#pragma unroll
+        for (int i = 0; i < 4 * NV; ++i) {
+            if (key[i] == 0xffffffffu)
+                continue;
+            const float    p  = __uint_as_float(key[i]);
+            const uint64_t fx = pn_fx(p);
+            if (use_m && p >= floor_w) {
+                a[0] += fx;
+                a[1] += 1ull;
+            }
+            a[2] += fx;
+            a[3] += key[i] > kmax; /* (never: checked below) */
+            if ((i & 3) == 3)
+                __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint64_t t = block_sum_u64(a[q], sh.red64);
+            if (tid == 0 && t)
+                coop_add64(&cr->aux[q], t);
+        }
+    }
+    uint32_t kappa = 0u, cnt_above = 0u, ties = 0u;
+    uint64_t mass_above = 0ull;
+    const uint64_t target = (uint64_t) __double2ull_ru((double) top_p * 0x1p62);
+    int      r;
+    {
+        /* (the three levels of coop_descent, the first of them also carrying the sums above) */
+        r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, false,
+                                 use_p ? target : ~0ull, false, 0u, 0u, kappa, cnt_above,
+                                 mass_above, ties);
+        if (r < 0) {
+            alone(true);
+            return;
+        }
+    }
+    const uint64_t mass_m = coop_ld64(&cr->aux[0]);
+    uint32_t       n_m    = (uint32_t) coop_ld64(&cr->aux[1]);
+    const uint64_t mass_all = coop_ld64(&cr->aux[2]);
+    if (coop_ld64(&cr->aux[3]) != 0ull) { /* a probability above the maximum's: not this walk's case */
+        alone(true);
+        return;
+    }
+    uint64_t mass_m_use = mass_m;
+    if (use_m && n_m < 1u) {
+        n_m        = 1u;
+        mass_m_use = pn_fx(__uint_as_float(kmax));
+    }
+    /* ---- the kept prefix, as sorted_descend<false> decides it ---- */
+    bool     limited   = false;
+    uint32_t edge_key  = 0u, edge_ties = 0u;
+    uint64_t mass_keep = 0ull;
+    uint32_t n_keep    = (uint32_t) rv.n_vocab;
+    bool     have_p    = false;
+    if (use_p && r == 1) {
+        const uint64_t each = pn_fx(__uint_as_float(kappa));
+        uint64_t       j    = each ? (target - mass_above + each - 1) / each : 1;
+        if (j < 1)
+            j = 1;
+        if (j > ties)
+            j = ties;
+        have_p    = true;
+        limited   = true;
+        edge_key  = kappa;
+        edge_ties = (uint32_t) j;
+        n_keep    = cnt_above + (uint32_t) j;
+        mass_keep = mass_above + each * j;
+    }
+    if (use_m && (!have_p || n_m < n_keep)) {
+        limited   = true;
+        mass_keep = mass_m_use;
+        edge_key  = __float_as_uint(floor_w) ? __float_as_uint(floor_w) - 1u : 0u;
+        edge_ties = 0u;
+        if (__float_as_uint(floor_w) == 0u)
+            limited = false;
+    } else if (!have_p) {
+        mass_keep = mass_all;
+        limited   = false;
+    }
+    /* ---- the draw ---- */
+    const uint64_t target2 = (uint64_t) __double2ull_rd((double) u * (double) mass_keep) + 1ull;
+    uint32_t       kd = 0u, cnt_above_d = 0u, ties_d = 0u;
+    uint64_t       mass_above_d = 0ull;
+    r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, true, target2, limited,
+                             edge_key, edge_ties, kd, cnt_above_d, mass_above_d, ties_d);
+    if (r <= 0) { /* 0: not reachable with exact integer masses; the one-workgroup walk decides */
+        alone(true);
+        return;
+    }
+    const uint64_t each = pn_fx(__uint_as_float(kd));
+    uint64_t       j    = each ? (target2 - mass_above_d + each - 1) / each : 1;
+    if (j < 1)
+        j = 1;
+    if (j > ties_d)
+        j = ties_d;
+    /* ---- the j-th entry, in index order, equal to the drawn value: every workgroup reports how
+     * many its chunk holds and leaves; the one that arrives last finds the chunk and the entry ---- */
+    {
+        int mine = 0;
+#pragma unroll
+        for (int i = 0; i < 4 * NV; ++i)
+            mine += (int) (key[i] == kd);
+        const uint32_t here = (uint32_t) block_sum_u64((uint64_t) mine, sh.red64);
+        if (tid == 0)
+            coop_st32(&cr->chunk_cnt[chunk], here);
+    }
+    if (!coop_arrive(cr, W, cs))
+        return;
+    int      c_at = -1;
+    uint64_t before = 0;
+    for (int c = 0; c < W; ++c) { /* (uniform: every thread adds the same counts) */
+        const uint32_t n_c = coop_ld32(&cr->chunk_cnt[c]);
+        if (c_at < 0 && before < j && j <= before + n_c)
+            c_at = c;
+        if (c_at < 0)
+            before += n_c;
+    }
+    if (c_at < 0) { /* (the counts add up to ties_d >= j: not reachable) */
+        alone(true);
+        return;
+    }
+    if (c_at != chunk) { /* that chunk's probabilities once more */
+        chunk_bounds<NV>(rv, c_at, base, end);
+        float4 v[NV];
+        __syncthreads();
+        fetch_chunk<NV, PEN>(rv, row, rv.n_rows, base, end, s_cnt16, v);
+#pragma unroll
+        for (int q = 0; q < NV; ++q) {
+            const int e = base + 4 * (q * TPB + tid);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                uint32_t k = 0xffffffffu;
+                if (e + c < end) {
+                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[q], c), mx, g.inv_t), s_tab);
+                    k             = __float_as_uint((float) ((double) p / tot));
+                }
+                key[4 * q + c] = k;
+            }
+            if (q + 1 < NV)
+                asm volatile("" : "+v"(key[4 * q + 3]), "+v"(v[q + 1].x), "+v"(v[q + 1].y),
+                                  "+v"(v[q + 1].z), "+v"(v[q + 1].w));
+        }
+    }
+    int want = (int) (j - before); /* 1-based, among the chunk's entries in index order */
+#pragma unroll
+    for (int q = 0; q < NV; ++q) { /* a chunk's index order: group q, then thread, then element */
+        const int m_q = (int) (key[4 * q] == kd) + (int) (key[4 * q + 1] == kd) +
+                        (int) (key[4 * q + 2] == kd) + (int) (key[4 * q + 3] == kd);
+        int       total;
+        const int incl = block_scan_i32(m_q, s_scan, &total);
+        if (want >= 1 && want <= total && incl >= want && incl - m_q < want) {
+            int seen = incl - m_q;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (key[4 * q + c] == kd && ++seen == want) {
+                    out[row]       = base + 4 * (q * TPB + tid) + c;
+                    cand.path[row] = 4;
+                    row_flag[row]  = 0; /* served */
+                }
+            }
+        }
+        want -= total; /* (at or below zero once found: no later group matches) */
+    }
+}
+
+} // namespace gs
+#endif

@@ -177,6 +177,26 @@ int geist_hip_sampler_set_wait_limit(geist_hip_sampler *s, uint32_t polls);
  * negative on error. */
 int geist_hip_sampler_one_launch_topk(geist_hip_sampler *s, int enable);
 
+/* No counterpart in the reference. A top-p / min-p row whose kept prefix is too long for the
+ * candidate list (tens of thousands of entries: a flat row at a high temperature) is walked in
+ * full, as sampler.c:246-304 sorts and walks it. One workgroup takes 275 to 300 us for a row of
+ * 128 k logits; spread over the workgroups of the row's chunks, which keep their part of the row
+ * in registers and meet after every pass, the walk takes a fifth of that -- at the price of one
+ * more launch per call.
+ *   GEIST_HIP_WHOLE_ROW_WALK_ADAPTIVE       (default) the extra launch is sent while such rows
+ *                                           keep turning up: the kernels report them in a
+ *                                           page-locked word that the next call looks at
+ *   GEIST_HIP_WHOLE_ROW_WALK_SPREAD         always send it
+ *   GEIST_HIP_WHOLE_ROW_WALK_ONE_WORKGROUP  never
+ * Tokens are the same in every mode. geist_hip_sampler_row_paths reports 3 for a row walked by
+ * one workgroup, 4 for a row walked by its chunks' workgroups. The waits of the spread form are
+ * bounded by geist_hip_sampler_set_wait_limit like those of the one-pass kernels: a row whose
+ * workgroups do not all turn up in time is walked by its first workgroup alone. */
+#define GEIST_HIP_WHOLE_ROW_WALK_ADAPTIVE 0
+#define GEIST_HIP_WHOLE_ROW_WALK_SPREAD 1
+#define GEIST_HIP_WHOLE_ROW_WALK_ONE_WORKGROUP 2
+int geist_hip_sampler_set_whole_row_walk(geist_hip_sampler *s, int mode);
+
 /* No counterpart in the reference. In the one-launch form the workgroups of a row hand their
  * candidates to the one that finishes the row, through plain stores that are only sure to be
  * seen inside the second-level cache of the XCD that wrote them. Each arrival reports the XCD it

@@ -175,7 +175,7 @@ def test_min_p_lists_of_every_size(hs, oracle, pen):
         assert near <= 1
         paths = hs.row_paths(rows)
         assert paths[0] == 2 and paths[1] == 2, paths     # listed
-        assert paths[2] == 3 and paths[3] == 3, paths     # more than a chunk stages: whole row
+        assert paths[2] in (3, 4) and paths[3] in (3, 4), paths   # more than a chunk stages: whole row
 
 
 @pytest.mark.parametrize("wait_limit", [None, 0, 3])

@@ -243,7 +243,7 @@ def test_top_p_candidate_list_path(hs, oracle, n, scale, T, p, m):
            for r in range(x.shape[0])]
     near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"top-p list n={n}")
     assert near <= 1
-    assert set(paths.tolist()) <= {1, 2, 3}
+    assert set(paths.tolist()) <= {1, 2, 3, 4}     # (3 / 4: the whole row, by one workgroup / by its chunks')
     assert (paths == 2).sum() >= 6, f"paths {paths.tolist()}, kept {[i.n_keep for _, i in res]}"
 
 
@@ -262,7 +262,7 @@ def test_top_p_vocabulary_beyond_the_shortcut(oracle):
     res = [oracle.top_p_u(x[r], 0.9, 1.0, float(u[r])) for r in range(4)]
     near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "top-p n=300000")
     assert near <= 1
-    assert paths == [2, 2, 2, 3], paths
+    assert paths[:3] == [2, 2, 2] and paths[3] in (3, 4), paths
 
 
 def test_sorted_paths_all_three_in_one_batch(hs, oracle):
@@ -282,7 +282,7 @@ def test_sorted_paths_all_three_in_one_batch(hs, oracle):
     res = [oracle.top_p_u(x[r], 0.9, 1.0, float(u[r])) for r in range(6)]
     near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "three paths")
     assert near <= 1
-    assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and paths[4:] == [3, 3], paths
+    assert paths[:2] == [1, 1] and paths[2:4] == [2, 2] and set(paths[4:]) <= {3, 4}, paths
 
 
 @pytest.mark.parametrize("n,lead,pad", [(128256, 0, 0), (50001, 0, 0), (33333, 3, 5),
@@ -319,7 +319,7 @@ def test_whole_row_walk_with_penalties_cap_and_mask(hs, oracle, n, lead, pad):
             infos.append(i)
         near = compare_ids(got, want, infos, f"whole-row walk n={n} {kw}")
         assert near <= 1
-        assert paths == [3] * rows, paths
+        assert set(paths) <= {3, 4}, paths
 
 
 def test_ids_and_draws_in_page_locked_host_memory(hs):
@@ -378,7 +378,7 @@ def test_min_p_listed_by_the_exp_sum_pass(hs, oracle):
         res = [oracle.chain_u(x[r], float(u[r]), **kw) for r in range(8)]
         near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"min-p listed {top_p}")
         assert near <= 1
-        assert paths[:5] == [2] * 5 and paths[5:] == [3] * 3, paths
+        assert paths[:5] == [2] * 5 and set(paths[5:]) <= {3, 4}, paths
 
 
 def test_sorted_modes_many_rows_and_one_row(hs, oracle):
@@ -393,7 +393,7 @@ def test_sorted_modes_many_rows_and_one_row(hs, oracle):
     res = [oracle.chain_u(x[r], float(u[r]), temperature=1.0, top_p=0.9, min_p=0.001)
            for r in range(400)]
     near = compare_ids(got, [t for t, _ in res], [i for _, i in res], "400 rows")
-    assert near <= 2 and 2 in paths and set(paths.tolist()) <= {1, 2, 3}
+    assert near <= 2 and 2 in paths and set(paths.tolist()) <= {1, 2, 3, 4}
     for r in (0, 1, 2):
         one = run_rows(hs, torch, x[r:r + 1], u[r:r + 1], P(temperature=1.0, top_p=0.9, min_p=0.001))
         assert one[0] == got[r]
