@@ -2241,3 +2241,10 @@ extern "C" int geist_hip_phase_stamps_read(unsigned long long *host, size_t n) {
                                      n * sizeof(unsigned long long));
 }
 #endif
+
+#ifdef GS_WALK_STAMPS
+extern "C" int geist_hip_walk_stamps_read(unsigned long long *host, size_t n) {
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(gs::g_walk_stamps),
+                                     n * sizeof(unsigned long long));
+}
+#endif

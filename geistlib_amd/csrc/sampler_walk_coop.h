@@ -35,7 +35,7 @@ namespace gs {
 struct CoopRow {
     uint32_t cnt[SG_BINS];
     uint64_t mass[SG_BINS];
-    uint64_t aux[4];                /* sums of the first step, added by every workgroup */
+    uint64_t aux[4];                /* sums of the first step, added by every workgroup (three used) */
     uint32_t chunk_cnt[MAX_CHUNKS]; /* entries equal to the drawn value, per chunk */
     uint32_t arrive;
     uint32_t epoch; /* number of the last step whose result is published */
@@ -64,6 +64,29 @@ __device__ __forceinline__ void coop_add32(uint32_t *p, uint32_t v) {
 }
 __device__ __forceinline__ void coop_add64(uint64_t *p, uint64_t v) {
     (void) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* Device timestamps of the first row's workgroups, compiled in only with -DGS_WALK_STAMPS. */
+#ifdef GS_WALK_STAMPS
+__device__ unsigned long long g_walk_stamps[64 * 32];
+__device__ __forceinline__ void walk_stamp(int row, int chunk, int i) {
+    if (row == 0 && threadIdx.x == 0 && chunk < 64 && i < 32)
+        g_walk_stamps[chunk * 32 + i] = wall_clock64();
+}
+#define GS_WSTAMP(i) walk_stamp(row, chunk, (i))
+#else
+#define GS_WSTAMP(i) do { } while (0)
+#endif
+
+/* pn_fx() for the bits of a probability 0 <= p <= 1 without the trip through double: p * 2^62 is
+ * the 24-bit significand shifted by the exponent, truncated as __double2ull_rz truncates (the
+ * product is exact in double, so the two agree bit for bit: compared on the host for every
+ * binary32 in [0, 1]). */
+__device__ __forceinline__ uint64_t pn_fx_bits(uint32_t key) {
+    const uint32_t e  = key >> 23; /* (the sign is 0) */
+    const uint32_t m  = e ? (key & 0x7fffffu) | 0x800000u : key & 0x7fffffu;
+    const int      sh = (int) (e ? e : 1u) - 88; /* value = m * 2^sh, -87 <= sh <= 39 */
+    return sh >= 0 ? (uint64_t) m << sh : sh > -24 ? (uint64_t) (m >> -sh) : 0ull;
 }
 
 struct CoopShared {
@@ -106,7 +129,7 @@ __device__ __forceinline__ bool coop_wait(const CoopRow *cr, uint32_t step, uint
             }
             if (polls++ >= limit)
                 break;
-            __builtin_amdgcn_s_sleep(8);
+            __builtin_amdgcn_s_sleep(2);
         }
         cs.ok = ok;
     }
@@ -127,8 +150,10 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
                                           const uint32_t (&key)[NK], Take take, int shf,
                                           uint32_t dm, bool select, bool clear_aux,
                                           uint64_t target, uint64_t &mass_above,
-                                          uint32_t &cnt_above, uint32_t &ties, int &digit) {
+                                          uint32_t &cnt_above, uint32_t &ties, int &digit,
+                                          int row, int chunk, int sbase) {
     const int tid = threadIdx.x;
+    (void) row, (void) chunk, (void) sbase;
     for (int i = tid; i < SG_BINS; i += TPB) {
         sh.cnt[i]  = 0u;
         sh.mass[i] = 0ull;
@@ -139,8 +164,7 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
         if (take(key[i])) {
             const uint32_t d = (key[i] >> shf) & dm;
             atomicAdd(&sh.cnt[d], 1u);
-            atomicAdd((unsigned long long *) &sh.mass[d],
-                      (unsigned long long) pn_fx(__uint_as_float(key[i])));
+            atomicAdd((unsigned long long *) &sh.mass[d], (unsigned long long) pn_fx_bits(key[i]));
         }
         /* (four entries at a time: interleaving all of them costs registers, not time) */
         if ((i & 3) == 3)
@@ -155,7 +179,9 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
         }
     }
     ++step;
+    GS_WSTAMP(sbase);
     if (coop_arrive(cr, W, cs)) {
+        GS_WSTAMP(sbase + 1);
         {
             /* all of a thread's loads in flight together: one round trip, not sixteen */
             constexpr int PER = SG_BINS / TPB;
@@ -175,8 +201,10 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
         }
         __syncthreads();
         for (int i = tid; i < SG_BINS; i += TPB) { /* for the next level */
-            coop_st32(&cr->cnt[i], 0u);
-            coop_st64(&cr->mass[i], 0ull);
+            if (sh.cnt[i]) {
+                coop_st32(&cr->cnt[i], 0u);
+                coop_st64(&cr->mass[i], 0ull);
+            }
         }
         if (clear_aux && tid < 4) /* (every workgroup has read them before it arrived here) */
             coop_st64(&cr->aux[tid], 0ull);
@@ -195,6 +223,7 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
     } else if (!coop_wait(cr, step, limit, cs)) {
         return -1;
     }
+    GS_WSTAMP(sbase + 2);
     /* (the last arrival reads its own stores back: program order, same addresses; the four
      * loads go out together) */
     digit                = (int) coop_ld32(reinterpret_cast<const uint32_t *>(&cr->res_digit));
@@ -219,7 +248,8 @@ __device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, 
                                             uint64_t target, bool limited, uint32_t limit_key,
                                             uint32_t limit_ties,
                                             uint32_t &kappa, uint32_t &cnt_above,
-                                            uint64_t &mass_above, uint32_t &ties_total) {
+                                            uint64_t &mass_above, uint32_t &ties_total,
+                                            int row, int chunk, int sbase) {
     uint32_t prefix = 0u, mask = 0u;
     cnt_above  = 0u;
     mass_above = 0ull;
@@ -245,7 +275,7 @@ __device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, 
         int       digit = -1;
         const int r = coop_level<NK>(cr, W, step, limit, sh, cs, key, take, shf, dm, true,
                                      clear_aux && lv == 0, target, mass_above, cnt_above,
-                                     ties_total, digit);
+                                     ties_total, digit, row, chunk, sbase + 3 * lv);
         if (r <= 0)
             return r;
         prefix |= (uint32_t) digit << shf;
@@ -275,6 +305,7 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     xcd_row_chunk(row, chunk);
     if (row_flag[row] != 2)
         return;
+    GS_WSTAMP(0);
     const int   tid = threadIdx.x, W = rv.n_chunks;
     const bool  lead = chunk == 0;
     const float u    = uniforms[row];
@@ -331,37 +362,55 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
                                   "+v"(v[j + 1].z), "+v"(v[j + 1].w));
         }
     }
+    GS_WSTAMP(1);
     const bool use_p = top_p > 0.0f && top_p < 1.0f;
     const bool use_m = min_p > 0.0f;
     /* the largest probability is that of the row's maximum: expf(0) = 1 over the sum */
     const uint32_t kmax    = __float_as_uint((float) (1.0 / tot));
     const float    floor_w = __fmul_rn(min_p, __uint_as_float(kmax));
     uint32_t       step    = step_base;
-    /* ---- step 1: the first level of the nucleus descent, the min-p prefix, the row's mass ---- */
-    {
+    /* ---- step 1: the first level of the nucleus descent; with it the sums that the kept prefix
+     * may need: mass and count of the min-p prefix, or the row's mass where no nucleus is asked
+     * for ---- */
+    if (use_m || !use_p) {
         uint64_t a[4] = {0ull, 0ull, 0ull, 0ull};
 #pragma unroll
         for (int i = 0; i < 4 * NV; ++i) {
             if (key[i] == 0xffffffffu)
                 continue;
-            const float    p  = __uint_as_float(key[i]);
-            const uint64_t fx = pn_fx(p);
-            if (use_m && p >= floor_w) {
+            const uint64_t fx = pn_fx_bits(key[i]);
+            if (use_m && __uint_as_float(key[i]) >= floor_w) {
                 a[0] += fx;
                 a[1] += 1ull;
             }
             a[2] += fx;
-            a[3] += key[i] > kmax; /* (never: checked below) */
             if ((i & 3) == 3)
                 __builtin_amdgcn_sched_barrier(0);
         }
+        /* the sums over the workgroup with one barrier between them (the histogram's words are
+         * free until the first level clears them) */
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint64_t t = block_sum_u64(a[q], sh.red64);
-            if (tid == 0 && t)
-                coop_add64(&cr->aux[q], t);
+        for (int q = 0; q < 3; ++q)
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1)
+                a[q] += shfl_xor_u64(a[q], m);
+        if ((tid & (WAVE - 1)) == 0) {
+#pragma unroll
+            for (int q = 0; q < 3; ++q)
+                sh.mass[(tid / WAVE) * 4 + q] = a[q];
         }
+        __syncthreads();
+        if (tid < 3) {
+            uint64_t t = 0;
+#pragma unroll
+            for (int w = 0; w < NWAVES; ++w)
+                t += sh.mass[w * 4 + tid];
+            if (t)
+                coop_add64(&cr->aux[tid], t);
+        }
+        __syncthreads();
     }
+    GS_WSTAMP(2);
     uint32_t kappa = 0u, cnt_above = 0u, ties = 0u;
     uint64_t mass_above = 0ull;
     const uint64_t target = (uint64_t) __double2ull_ru((double) top_p * 0x1p62);
@@ -370,19 +419,16 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
         /* (the three levels of coop_descent, the first of them also carrying the sums above) */
         r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, false,
                                  use_p ? target : ~0ull, false, 0u, 0u, kappa, cnt_above,
-                                 mass_above, ties);
+                                 mass_above, ties, row, chunk, 8);
         if (r < 0) {
             alone(true);
             return;
         }
     }
+    GS_WSTAMP(3);
     const uint64_t mass_m = coop_ld64(&cr->aux[0]);
     uint32_t       n_m    = (uint32_t) coop_ld64(&cr->aux[1]);
     const uint64_t mass_all = coop_ld64(&cr->aux[2]);
-    if (coop_ld64(&cr->aux[3]) != 0ull) { /* a probability above the maximum's: not this walk's case */
-        alone(true);
-        return;
-    }
     uint64_t mass_m_use = mass_m;
     if (use_m && n_m < 1u) {
         n_m        = 1u;
@@ -424,11 +470,13 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     uint32_t       kd = 0u, cnt_above_d = 0u, ties_d = 0u;
     uint64_t       mass_above_d = 0ull;
     r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, true, target2, limited,
-                             edge_key, edge_ties, kd, cnt_above_d, mass_above_d, ties_d);
+                             edge_key, edge_ties, kd, cnt_above_d, mass_above_d, ties_d, row, chunk,
+                             17);
     if (r <= 0) { /* 0: not reachable with exact integer masses; the one-workgroup walk decides */
         alone(true);
         return;
     }
+    GS_WSTAMP(4);
     const uint64_t each = pn_fx(__uint_as_float(kd));
     uint64_t       j    = each ? (target2 - mass_above_d + each - 1) / each : 1;
     if (j < 1)
@@ -436,53 +484,30 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     if (j > ties_d)
         j = ties_d;
     /* ---- the j-th entry, in index order, equal to the drawn value: every workgroup reports how
-     * many its chunk holds and leaves; the one that arrives last finds the chunk and the entry ---- */
+     * many its chunk holds; once all have, the one whose chunk holds the entry finds it ---- */
+    uint32_t here;
     {
         int mine = 0;
 #pragma unroll
         for (int i = 0; i < 4 * NV; ++i)
             mine += (int) (key[i] == kd);
-        const uint32_t here = (uint32_t) block_sum_u64((uint64_t) mine, sh.red64);
+        here = (uint32_t) block_sum_u64((uint64_t) mine, sh.red64);
         if (tid == 0)
             coop_st32(&cr->chunk_cnt[chunk], here);
     }
-    if (!coop_arrive(cr, W, cs))
-        return;
-    int      c_at = -1;
-    uint64_t before = 0;
-    for (int c = 0; c < W; ++c) { /* (uniform: every thread adds the same counts) */
-        const uint32_t n_c = coop_ld32(&cr->chunk_cnt[c]);
-        if (c_at < 0 && before < j && j <= before + n_c)
-            c_at = c;
-        if (c_at < 0)
-            before += n_c;
-    }
-    if (c_at < 0) { /* (the counts add up to ties_d >= j: not reachable) */
+    ++step;
+    if (coop_arrive(cr, W, cs)) {
+        GS_WSTAMP(5);
+        coop_publish(cr, step);
+    } else if (!coop_wait(cr, step, wait_limit, cs)) {
         alone(true);
         return;
     }
-    if (c_at != chunk) { /* that chunk's probabilities once more */
-        chunk_bounds<NV>(rv, c_at, base, end);
-        float4 v[NV];
-        __syncthreads();
-        fetch_chunk<NV, PEN>(rv, row, rv.n_rows, base, end, s_cnt16, v);
-#pragma unroll
-        for (int q = 0; q < NV; ++q) {
-            const int e = base + 4 * (q * TPB + tid);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                uint32_t k = 0xffffffffu;
-                if (e + c < end) {
-                    const float p = geist_expf_glibc_le0(softmax_arg(f4_get(v[q], c), mx, g.inv_t), s_tab);
-                    k             = __float_as_uint((float) ((double) p / tot));
-                }
-                key[4 * q + c] = k;
-            }
-            if (q + 1 < NV)
-                asm volatile("" : "+v"(key[4 * q + 3]), "+v"(v[q + 1].x), "+v"(v[q + 1].y),
-                                  "+v"(v[q + 1].z), "+v"(v[q + 1].w));
-        }
-    }
+    /* the entries in the chunks before this one (a thread per chunk, then their sum) */
+    const uint64_t before =
+        block_sum_u64(tid < chunk ? (uint64_t) coop_ld32(&cr->chunk_cnt[tid]) : 0ull, sh.red64);
+    if (!(before < j && j <= before + here))
+        return; /* the entry lies in another chunk */
     int want = (int) (j - before); /* 1-based, among the chunk's entries in index order */
 #pragma unroll
     for (int q = 0; q < NV; ++q) { /* a chunk's index order: group q, then thread, then element */
@@ -503,6 +528,7 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
         }
         want -= total; /* (at or below zero once found: no later group matches) */
     }
+    GS_WSTAMP(6);
 }
 
 } // namespace gs
