@@ -902,6 +902,67 @@ def bench_lm_head_spec(args):
     print(json.dumps(result))
 
 
+def bench_whole_row_walk(args):
+    """Workload whole_row_walk: top-p rows whose kept prefix is tens of thousands of entries (flat
+    rows at temperature 1: logits N(0, 0.5^2), top-p 0.9), which neither the thread-maxima
+    shortcut nor the candidate list can serve: every row is walked in full
+    (src/engine/sampler.c:246-304 sorts and walks it). Timed per step for 1, 16 and 64 rows of
+    128256 with the walk by one workgroup per row and spread over the workgroups of the row's
+    chunks (geist_hip_sampler_set_whole_row_walk), the steps reading four copies of the batch in
+    turn; the ids of the two forms are compared with each other and, without --no-cpu, the
+    16-row batch with the oracle."""
+    import torch
+    from geistlib_amd import HipSampler, SampleParams
+    from geistlib_amd.bench_hooks import Timer
+    dev = torch.device("cuda:0")
+    n = 128256
+    prm = SampleParams.make(temperature=1.0, top_p=0.9)
+    legs, ids16, x16, u16 = {}, None, None, None
+    for rows in (1, 16, 64):
+        hs = HipSampler(max_rows=rows, max_vocab=n)
+        g = torch.Generator(device=dev)
+        g.manual_seed(100 + rows)
+        xs = [torch.randn((rows, n), device=dev, generator=g) * 0.5 for _ in range(4)]
+        u = torch.rand(rows, device=dev, generator=g)
+        out = torch.empty(rows, dtype=torch.int32, device=dev)
+        got = {}
+        for name, mode in (("one_workgroup", 2), ("spread", 1)):
+            hs.set_whole_row_walk(mode)
+            for i in range(8):
+                hs.sample(HipSampler.rows(xs[i % 4]), prm, u, out)
+            hs.sync()
+            steps = max(8, min(args.steps, 100))
+            with Timer() as tm:
+                for i in range(steps):
+                    hs.sample(HipSampler.rows(xs[i % 4]), prm, u, out)
+            hs.sample(HipSampler.rows(xs[0]), prm, u, out)
+            hs.sync()
+            got[name] = out.cpu().numpy().tolist()
+            legs[f"rows{rows}_{name}_us_per_step"] = round(tm.ms * 1e3 / steps, 2)
+            legs[f"rows{rows}_{name}_paths"] = sorted(set(hs.row_paths(rows).tolist()))
+        legs[f"rows{rows}_ids_equal"] = got["one_workgroup"] == got["spread"]
+        if rows == 16:
+            ids16, x16, u16 = got["spread"], xs[0].cpu().numpy(), u.cpu().numpy()
+        hs.close()
+    result = {
+        "metric": "sampled rows/s", "value": round(16 / (legs["rows16_spread_us_per_step"] * 1e-6), 1),
+        "unit": "rows/s", "n_gpus": 1, "steps": max(8, min(args.steps, 100)), "warmup": 8,
+        "ms_per_step": round(legs["rows16_spread_us_per_step"] * 1e-3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "whole_row_walk_b16_v128256", "rows": 16, "n_vocab": n,
+                   "temperature": 1.0, "top_p": 0.9, "logits": "N(0, 0.5^2)"},
+        "legs": legs,
+    }
+    if not args.no_cpu:
+        from oracle_lib import Oracle
+        o = Oracle(fast=True)
+        want = [int(o.top_p_u(x16[r], 0.9, 1.0, float(u16[r]))[0]) for r in range(16)]
+        result["parity"] = {"rows": 16, "ids_differ": int(sum(a != b for a, b in zip(ids16, want)))}
+    print(json.dumps(result))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -929,6 +990,8 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("no GPU visible: the sampling path has no CPU fallback")
 
+    if args.workload == "whole_row_walk":
+        return bench_whole_row_walk(args)
     if args.workload == "lm_head_spec":
         return bench_lm_head_spec(args)
     if args.workload.startswith("lm_head_q6k"):
