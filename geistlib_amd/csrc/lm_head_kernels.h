@@ -90,6 +90,9 @@ void launch_rmsnorm_q8k_rows(hipStream_t stream, const float *x, long ld_x, cons
                              float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act);
 void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
                                 const uint32_t *act, float *y);
+/* ... and over the table as it lies in the file (4-byte aligned). */
+void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
+                         const uint32_t *act, float *y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
  * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
 size_t q4k_packed_bytes(long n_out, int n_in);

@@ -26,6 +26,7 @@
  * wavefront), and v_mad_i32_i24 applies the scale.
  */
 #include "lm_head_kernels.h"
+#include "lm_head_q6k_block.h"
 #include "rmsnorm_device.h"
 
 #include <hip/hip_fp16.h>
@@ -219,6 +220,71 @@ __global__ __launch_bounds__(Q6X_TPB, 4) void k_q6k_packed_gemv_x86(
     }
     if (row < n_out)
         y[row] = ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
+}
+
+/* The same over the table as it lies in the file, for callers that keep no packed copy: a lane
+ * owns a table row and reads its 210-byte blocks whole. There the four low bits and the two high
+ * bits of an element lie apart, but in the order the dot product wants them: a dword of ql holds
+ * the low nibbles of elements 4u .. 4u + 3 of two runs, a dword of qh the high bits of the same
+ * elements of four runs, so a mask and a shift per run put four six-bit values into the bytes of
+ * a dword. */
+__global__ __launch_bounds__(Q6X_TPB) void k_q6k_gemv_x86(const uint8_t *__restrict__ w,
+                                                          long n_out, int nb,
+                                                          const uint32_t *__restrict__ act,
+                                                          float *__restrict__ y) {
+    const long row = (long) blockIdx.x * Q6X_TPB + threadIdx.x;
+    if (row >= n_out)
+        return;
+    const uint8_t *rp = w + row * (long) nb * 210;
+    float          acc[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        acc[u] = 0.0f;
+    for (int b = 0; b < nb; ++b) {
+        uint32_t d[53];
+        q6k_load_block(rp + (long) b * 210, d);
+        const uint32_t *a  = act + (long) b * Q8K_ACT_DWORDS; /* uniform: scalar loads */
+        const uint32_t  sc[4] = {d[48], d[49], d[50], d[51]};
+        const float     dd = __uint_as_float(a[80]) *
+                         __half2float(__ushort_as_half((unsigned short) (d[52] & 0xffffu)));
+        typedef uint32_t u16v __attribute__((ext_vector_type(16)));
+        const u16v bs = *reinterpret_cast<const u16v *>(a + 64);
+        int        lane[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            lane[u] = -32 * (__mul24((int) bs[2 * u], q6x_scale(sc, 2 * u)) +
+                             __mul24((int) bs[2 * u + 1], q6x_scale(sc, 2 * u + 1)));
+#pragma unroll
+        for (int v = 0; v < 8; ++v) { /* run v = 4 h + j: elements 128 h + 32 j .. + 31 */
+            const int h = v >> 2, j = v & 3;
+            typedef uint32_t u8v __attribute__((ext_vector_type(8)));
+            const u8v av  = *reinterpret_cast<const u8v *>(a + 8 * v);
+            const int s_a = q6x_scale(sc, 2 * v), s_b = q6x_scale(sc, 2 * v + 1);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                /* q = nibble (j >> 1) of ql[64 h + 32 (j & 1) + l] | ((qh[32 h + l] >> 2 j) & 3) << 4
+                 * for l = 4 u .. 4 u + 3 (src/formats/gguf/q6_K.c:30-36) */
+                const uint32_t ql = d[16 * h + 8 * (j & 1) + u], qh = d[32 + 8 * h + u];
+                const uint32_t lo = (j >> 1) ? (ql >> 4) & 0x0f0f0f0fu : ql & 0x0f0f0f0fu;
+                const uint32_t hi = j == 0   ? (qh << 4) & 0x30303030u
+                                    : j == 1 ? (qh << 2) & 0x30303030u
+                                    : j == 2 ? qh & 0x30303030u
+                                             : (qh >> 2) & 0x30303030u;
+                const int dot = __builtin_amdgcn_sdot4((int) (lo | hi), (int) av[u], 0, false);
+                lane[u] += __mul24(u < 4 ? s_a : s_b, dot);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            acc[u] = __builtin_fmaf(dd, (float) lane[u], acc[u]);
+    }
+    y[row] = ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
+}
+
+void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
+                         const uint32_t *act, float *y) {
+    k_q6k_gemv_x86<<<dim3((unsigned) ((n_out + Q6X_TPB - 1) / Q6X_TPB)), dim3(Q6X_TPB), 0, stream>>>(
+        w_q6k, n_out, n_in / 256, act, y);
 }
 
 void launch_q8k_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,

@@ -1301,17 +1301,21 @@ static int q6k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, si
 
 /* The x86 backend's decode kernel, row by row (each row is a pass over the table, as each call
  * of q6k_gemv_m1 is). */
-static int q6k_packed_gemv_x86_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
-                                    size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
-                                    float *d_y, size_t ld_y) {
+static int q6k_gemv_x86_impl(geist_hip_sampler *s, const void *d_table, bool packed, size_t n_out,
+                            size_t n_in, const float *d_x, size_t ld_x, size_t n_rows, float *d_y,
+                            size_t ld_y) {
     Q6KScratch ws;
     const int  rc = q6k_scratch(s, n_out, n_in, ws);
     if (rc)
         return rc;
     for (size_t m = 0; m < n_rows; ++m) {
         launch_q8k_quantize(s->stream, d_x + m * ld_x, (long) ld_x, 1, (int) n_in, ws.act8);
-        launch_q6k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in, ws.act8,
-                                   d_y + m * ld_y);
+        if (packed)
+            launch_q6k_packed_gemv_q8k(s->stream, d_table, (long) n_out, (int) n_in, ws.act8,
+                                       d_y + m * ld_y);
+        else
+            launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_table), (long) n_out,
+                                (int) n_in, ws.act8, d_y + m * ld_y);
     }
     return GEIST_HIP_OK;
 }
@@ -1415,8 +1419,26 @@ int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packe
     if (((uintptr_t) d_packed) % 16 != 0)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q6_K table not 16-byte aligned");
     HIPCHK(s, hipSetDevice(s->device));
-    rc = q6k_packed_gemv_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    rc = q6k_gemv_x86_impl(s, d_packed, true, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
     return rc ? rc : after_launch(s, "Q6_K decode (packed)");
+}
+
+int geist_hip_q6k_gemv_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out,
+                                size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_q6k || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K decode: %zu rows, strides %zu / %zu", n_rows,
+                    ld_x, ld_y);
+    int rc = q6k_check(s, d_w_q6k, n_out, n_in);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q6k_gemv_x86_impl(s, d_w_q6k, false, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q6_K decode");
 }
 
 size_t geist_hip_q8k_act_bytes(size_t n_in, size_t n_rows) {
@@ -1632,9 +1654,10 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     const bool topk_scan = fuse_ok && !rs.greedy && rs.use_k && rs.k <= TOPK_FAST_MAX;
     if (!d_normed)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "no buffer for the normed rows");
-    /* one row over a packed Q6_K table on the x86 backend: its integer decode kernel
+    /* one row over a Q6_K table on the x86 backend: its integer decode kernel
      * (q6k_gemv_m1), whose activation quantiser rides on the norm's launch */
-    const bool q6k_x86 = table == TABLE_Q6K_PACKED && rows == 1 && !s->projection_portable;
+    const bool q6k_x86 = (table == TABLE_Q6K_PACKED || table == TABLE_Q6K) && rows == 1 &&
+                         !s->projection_portable;
     Q6KScratch q6ws{};
     if (q6k_x86) {
         if ((rc = q6k_scratch(s, n_vocab, d_model, q6ws)) != GEIST_HIP_OK)
@@ -1656,8 +1679,12 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
             launch_f16_gemv(s->stream, d_embed_f16, (long) n_vocab, (int) d_model, d_normed,
                             (long) d_model, (int) rows, d_logits, (long) ld_logits, &f);
     } else if (q6k_x86) {
-        launch_q6k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,
-                                   d_logits);
+        if (table == TABLE_Q6K_PACKED)
+            launch_q6k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,
+                                       d_logits);
+        else
+            launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_embed), (long) n_vocab,
+                                (int) d_model, q6ws.act8, d_logits);
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
         rc = table == TABLE_Q4K_PACKED

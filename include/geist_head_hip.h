@@ -108,8 +108,8 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
  * whose logit soft-cap the head was created with): d_embed_q6k holds vocab rows of d_model / 256
  * super-blocks of 210 bytes, d_model a multiple of 256. The logits equal, bit for bit, those of
  * the reference's portable kernel cpu_scalar_w_quant_m1 / _mN after dequant_q6_K_row
- * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch. After
- * geist_hip_head_q6k_load, and unless geist_hip_head_set_projection chose the portable backend,
+ * (src/backends/cpu_scalar/weight_resolve.c:86-88, 186-241), for one row and for a batch. Unless
+ * geist_hip_head_set_projection chose the portable backend,
  * one row gets the logits of the x86 backend's decode kernel q6k_gemv_m1 instead
  * (src/backends/cpu_x86/kernel_q6k_gemv.c, resolved at src/backends/cpu_x86/backend.c:395-397),
  * again bit for bit; that backend's batch kernel, a GEMM over an int8 copy of the table

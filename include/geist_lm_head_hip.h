@@ -54,7 +54,7 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
 
 /* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
  * the head's project_finalize calls) stands for:
- *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a packed Q6_K table q6k_gemv_m1;
+ *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a Q6_K table q6k_gemv_m1;
  *                                  more rows: the portable kernel (default)
  *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
  *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
@@ -163,6 +163,11 @@ int geist_hip_q6k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
 int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                        size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                        float *d_y, size_t ld_y);
+/* The same over the table as it lies in the file (4-byte aligned), for callers that keep no
+ * packed copy: the same results bit for bit, at the price of the table's scattered reads. */
+int geist_hip_q6k_gemv_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out,
+                                size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                float *d_y, size_t ld_y);
 /* The two halves of that kernel for callers that keep the int8 activations (several tables
  * projected from one activation row, or the quantiser placed in an earlier launch):
  * geist_hip_q8k_quantize_rows replaces the activation quantiser of kernel_q6k_gemv.c:43-67 --
@@ -177,11 +182,12 @@ int geist_hip_q6k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, si
                                   size_t n_in, const void *d_act, float *d_y);
 /* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, the projection and the
  * sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. The
- * projection is geist_hip_q6k_linear_rows (the portable arithmetic) over the table as it lies in
- * the file. Over the packed copy it follows geist_hip_sampler_set_projection: in the default
- * mode GEIST_HIP_PROJECTION_X86 one row gets geist_hip_q6k_packed_gemv_x86_rows, as on the
- * reference's x86 backend; a batch, and any call in mode _PORTABLE, gets
- * geist_hip_q6k_packed_linear_rows. */
+ * projection follows geist_hip_sampler_set_projection: in the default mode
+ * GEIST_HIP_PROJECTION_X86 one row gets the x86 backend's decode kernel
+ * (geist_hip_q6k_gemv_x86_rows / geist_hip_q6k_packed_gemv_x86_rows); a batch, and any call in
+ * mode _PORTABLE, gets the portable arithmetic (geist_hip_q6k_linear_rows /
+ * geist_hip_q6k_packed_linear_rows). Over the packed copy and over the table as it lies in the
+ * file the logits are the same bit for bit. */
 int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
                                       size_t ld_hidden, size_t rows, size_t d_model,
                                       const float *d_norm_weight, float rms_eps,

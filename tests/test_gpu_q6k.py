@@ -102,6 +102,11 @@ def test_q6k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
             want = oracle_q6k_gemv_x86(oracle.lib, w, x[m], n_in)
             bad = np.flatnonzero(got[m].view(np.uint32) != want.view(np.uint32))
             assert bad.size == 0, (scale, m, bad[:5], got[m][bad[:3]], want[bad[:3]])
+        # the same over the table as it lies in the file
+        y0 = torch.full((3, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q6k_gemv_x86(d_w, n_in, d_x, y0)
+        hs.sync()
+        assert np.array_equal(y0.cpu().numpy().view(np.uint32), got.view(np.uint32)), scale
         # the kernel's two halves: the int8 activations as the reference's quantiser leaves
         # them, and the dot products over them
         nb = n_in // 256
@@ -205,7 +210,7 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
                 C.c_void_p(d_w.data_ptr()), d_model, out)
             assert rc == 0, host.geist_hip_head_errmsg(h)
             normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
-            if k == 1 and packed and not portable:     # the x86 backend's decode kernel
+            if k == 1 and not portable:     # the x86 backend's decode kernel, packed copy or not
                 logits = oracle_q6k_gemv_x86(oracle.lib, w, normed[0], d_model)[None, :]
             else:
                 logits = oracle_q6k_linear(oracle.lib, w, normed, d_model)
