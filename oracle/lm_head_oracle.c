@@ -292,6 +292,98 @@ int oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w
     return 0;
 }
 
+/* ---- the x86 backend's decode kernel over a Q4_K table ------------------------------------
+ * q4kx8_gemv_m1 (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:380-399) over the table that
+ * q4k_to_q4kx8_matrix (q4k_to_q4kx8.c:24-115) interleaves eight rows at a time. The interleaving
+ * only places the rows' bytes where the eight lanes of the vector kernel find them: each output
+ * row's arithmetic involves that row's blocks alone, and it is restated here row by row. */
+
+void oracle_q8k_row_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                             int16_t *bsums_out) {
+    /* quantize_q8k_row, kernel_q4kx8_gemm_avx512.c:47-77: ONE scale for the whole row,
+     * round half away from zero by truncation, clamp, sums per sixteen */
+    float amax = 0.0f;
+    for (size_t k = 0; k < n_super * 256; k++) {
+        const float a  = x[k];
+        const float ax = a < 0.0f ? -a : a;
+        if (ax > amax)
+            amax = ax;
+    }
+    const float scale = amax == 0.0f ? 1.0f : amax / 127.0f;
+    const float inv   = 1.0f / scale;
+    *d_out            = scale;
+    for (size_t k = 0; k < n_super * 256; k++) {
+        const float v = x[k] * inv;
+        const int   q = (int) (v < 0.0f ? v - 0.5f : v + 0.5f);
+        qs_out[k]     = (int8_t) (q < -128 ? -128 : q > 127 ? 127 : q);
+    }
+    for (size_t g = 0; g < n_super * 16; g++) {
+        int s = 0;
+        for (int i = 0; i < 16; i++)
+            s += qs_out[g * 16 + i];
+        bsums_out[g] = (int16_t) s;
+    }
+}
+
+/* One row: q4kx8_gemv_one_row_tile (kernel_q4kx8_gemm_avx512.c:81-304) for one of its eight
+ * lanes. Per super-block the products of the 4-bit values with the int8 activations are summed
+ * as integers per sub-block of 32 and weighted with the sub-block's 6-bit scale; the minima are
+ * weighted with the activations' sums per sub-block; each of the two integers joins a binary32
+ * accumulator by one fused multiply-add with (d * d_act) and (dmin * d_act) -- both products
+ * rounded to binary32 first --, and the result is the difference of the two accumulators. */
+static float oracle_dot_q4k_q8k(size_t n_super, const uint8_t *row, float d_act, const int8_t *qs,
+                                const int16_t *bsums) {
+    float acc = 0.0f, acc_min = 0.0f;
+    for (size_t b = 0; b < n_super; b++, row += 144) {
+        const float    d    = oracle_f16_to_f32((uint16_t) (row[0] | (row[1] << 8)));
+        const float    dmin = oracle_f16_to_f32((uint16_t) (row[2] | (row[3] << 8)));
+        const uint8_t *sc = row + 4, *q = row + 16;
+        const int8_t  *a  = qs + b * 256;
+        int32_t        iacc = 0, iacc_min = 0;
+        for (int j = 0; j < 8; j++) { /* sub-block j: elements 32 j .. 32 j + 31 */
+            int scale, min;          /* get_scale_min_k4(j), src/formats/gguf/q4_K.c */
+            if (j < 4) {
+                scale = sc[j] & 63;
+                min   = sc[j + 4] & 63;
+            } else {
+                scale = (sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4);
+                min   = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
+            }
+            int32_t dot = 0;
+            for (int l = 0; l < 32; l++) {
+                const int v = (j & 1) ? q[32 * (j >> 1) + l] >> 4 : q[32 * (j >> 1) + l] & 0xF;
+                dot += v * a[32 * j + l];
+            }
+            iacc += scale * dot;
+            iacc_min += min * (bsums[b * 16 + 2 * j] + bsums[b * 16 + 2 * j + 1]);
+        }
+        acc     = fmaf((float) iacc, d * d_act, acc);
+        acc_min = fmaf((float) iacc_min, dmin * d_act, acc_min);
+    }
+    return acc - acc_min;
+}
+
+int oracle_q4k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q4k, float *y) {
+    const size_t n_super = n_in / 256;
+    if (n_in % 256 != 0 || n_super == 0 || n_super > 64 || n_out % 8 != 0)
+        return -1; /* shapes the reference's kernel does not take */
+    float    d_act;
+    int8_t  *qs    = malloc(n_in);
+    int16_t *bsums = malloc(n_super * 16 * sizeof(int16_t));
+    if (!qs || !bsums) {
+        free(qs);
+        free(bsums);
+        return -2;
+    }
+    oracle_q8k_row_quantize(n_super, x, &d_act, qs, bsums);
+#pragma omp parallel for schedule(static)
+    for (size_t r = 0; r < n_out; r++)
+        y[r] = oracle_dot_q4k_q8k(n_super, (const uint8_t *) w_q4k + r * n_super * 144, d_act, qs, bsums);
+    free(qs);
+    free(bsums);
+    return 0;
+}
+
 void oracle_dequant_q4_K_row(const void *blocks, float *out, size_t n_elems) {
     /* q4_K.c:18-49; the block layout of src/quant/quant_blocks.h:50-56 by offsets */
     const uint8_t *p = (const uint8_t *) blocks;

@@ -81,6 +81,15 @@ void oracle_q8k_quantize(size_t n_super, const float *x, float *d_out, int8_t *q
                          int16_t *bsums_out);
 int  oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q6k, float *y);
 
+/* The x86 backend's decode kernel over a Q4_K table (q4kx8_gemv_m1,
+ * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:47-77 the activation quantiser -- one scale for
+ * the whole row, round half away from zero --, :81-304 the dot products), restated row by row.
+ * n_out a multiple of 8 and n_in / 256 <= 64, as the reference's kernel requires (-1 otherwise).
+ * oracle_q8k_row_quantize: d_out one float, qs_out n_super * 256 int8, bsums_out n_super * 16. */
+void oracle_q8k_row_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                             int16_t *bsums_out);
+int oracle_q4k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q4k, float *y);
+
 /* The same pair for a Q4_K table (super-blocks of 144 bytes: d, dmin in binary16, eight 6-bit
  * scales and eight 6-bit minima packed into 12 bytes, 128 bytes of 4-bit values;
  * src/quant/quant_blocks.h:50-56). dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, scales by

@@ -611,3 +611,60 @@ def ref_q4k_linear(ref, w_q4k, x, n_in):
                                _fp(xs), xs.shape[0], _fp(y))
     assert rc == 0
     return y
+
+
+def oracle_q4k_gemv_x86(lib, w_q4k, x, n_in):
+    """oracle_q4k_gemv_x86: the x86 backend's one-row decode kernel over a Q4_K table."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    n_out = w_q4k.shape[0]
+    y = np.full(n_out, np.nan, dtype=np.float32)
+    lib.oracle_q4k_gemv_x86.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_void_p, c_float_p]
+    lib.oracle_q4k_gemv_x86.restype = C.c_int
+    rc = lib.oracle_q4k_gemv_x86(n_out, n_in, _fp(x), w_q4k.ctypes.data_as(C.c_void_p), _fp(y))
+    assert rc == 0, rc
+    return y
+
+
+def oracle_q8k_row_quantize(lib, x):
+    """(d, qs int8 [n_in], bsums int16 [n_in / 16]) of one activation row, one scale per row."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    ns = x.size // 256
+    d = np.empty(1, dtype=np.float32)
+    qs = np.empty(ns * 256, dtype=np.int8)
+    bs = np.empty(ns * 16, dtype=np.int16)
+    lib.oracle_q8k_row_quantize.argtypes = [C.c_size_t, c_float_p, c_float_p, C.c_void_p, C.c_void_p]
+    lib.oracle_q8k_row_quantize.restype = None
+    lib.oracle_q8k_row_quantize(ns, _fp(x), _fp(d), qs.ctypes.data_as(C.c_void_p),
+                                bs.ctypes.data_as(C.c_void_p))
+    return float(d[0]), qs, bs
+
+
+Q4KX8_BLOCK_BYTES = 1152
+
+
+def load_ref_q4kgemv(fast=False):
+    """The reference's q4k_to_q4kx8_matrix and q4kx8_gemv_m1 compiled from its tree, or None where
+    not built."""
+    path = os.path.join(ORACLE_DIR, "_ref",
+                        "libgeist_ref_q4kgemv_fast.so" if fast else "libgeist_ref_q4kgemv.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path, mode=os.RTLD_LAZY)
+    lib.q4k_to_q4kx8_matrix.argtypes = [C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
+    lib.q4k_to_q4kx8_matrix.restype = None
+    lib.q4kx8_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_void_p, c_float_p]
+    lib.q4kx8_gemv_m1.restype = None
+    return lib
+
+
+def ref_q4k_gemv_m1(ref, w_q4k, x, n_in):
+    """The table interleaved by the reference's repacker, then its decode kernel."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    n_out = w_q4k.shape[0]
+    assert n_out % 8 == 0 and n_in % 256 == 0
+    blob = np.zeros(n_out // 8 * (n_in // 256) * Q4KX8_BLOCK_BYTES + 64, dtype=np.uint8)
+    w = np.ascontiguousarray(w_q4k)
+    ref.q4k_to_q4kx8_matrix(n_in, n_out, w.ctypes.data_as(C.c_void_p), blob.ctypes.data_as(C.c_void_p))
+    y = np.full(n_out, np.nan, dtype=np.float32)
+    ref.q4kx8_gemv_m1(n_out, n_in, _fp(x), blob.ctypes.data_as(C.c_void_p), _fp(y))
+    return y
