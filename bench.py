@@ -748,12 +748,22 @@ def bench_lm_head_q4k(args, m_rows):
     ms = elapsed * 1e3 / args.steps
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-    for i in range(3):
-        hs.q4k_packed_linear(packed[i], vocab, d_model, normed, logits)
-    with Timer() as tm:       # HIP events on the sampler's stream around the launches
-        for i in range(args.steps):
-            hs.q4k_packed_linear(packed[i % 3], vocab, d_model, normed, logits)
-    kernel_us = tm.ms * 1e3 / args.steps
+    # One row is a decode step of the reference's x86 backend: its integer kernel q4kx8_gemv_m1
+    # (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c), which the step above ran. A batch runs
+    # the portable arithmetic (double accumulation); for one row that kernel is timed beside.
+    x86 = m_rows == 1
+
+    def timed(fn):
+        for i in range(3):
+            fn(packed[i])
+        with Timer() as tm:   # HIP events on the sampler's stream around the launches
+            for i in range(args.steps):
+                fn(packed[i % 3])
+        return tm.ms * 1e3 / args.steps
+
+    portable_us = timed(lambda t: hs.q4k_packed_linear(t, vocab, d_model, normed, logits))
+    kernel_us = (timed(lambda t: hs.q4k_packed_gemv_x86(t, vocab, d_model, normed, logits))
+                 if x86 else portable_us)
     w_bytes = vocab * nb * 144
     read_bytes = vocab * nb * 148
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
@@ -762,38 +772,81 @@ def bench_lm_head_q4k(args, m_rows):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "Q4_K weights x f32 activations, f64 accumulation", "data": "synthetic",
+        "dtype": ("Q4_K weights x int8 activations, int32 dot products, f32 accumulation" if x86
+                  else "Q4_K weights x f32 activations, f64 accumulation"),
+        "data": "synthetic",
         "config": {"workload": f"lm_head_q4k_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
                    "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
-                   "top_p": 0.9, "logit_softcap": 30.0},
+                   "top_p": 0.9, "logit_softcap": 30.0,
+                   "projection": "x86 decode kernel (q4kx8_gemv_m1)" if x86
+                                 else "portable kernel (cpu_scalar_w_quant_mN)"},
         "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_q4k_packed_linear (+ activations to double)",
+                     "kernel": ("k_q4k_packed_gemv_x86 (+ k_q8k_row_quantize)" if x86 else
+                                "k_q4k_packed_linear (+ activations to double)"),
                      "kernel_us": round(kernel_us, 3),
+                     "kernel_us_portable_arithmetic": round(portable_us, 3),
                      "kernel_algorithmic_bytes": w_bytes,
                      "packed_bytes_read": read_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
     if not args.no_cpu:
-        from oracle_lib import load_oracle, oracle_q4k_linear
-        lib = load_oracle(fast=True)
-        n_s = 16384
+        # CPU side on a bounded sample of the table rows. One row: the reference's own AVX2
+        # kernel over the table its own repacker interleaves (release flags, OpenMP over the
+        # row tiles) where it was compiled from the reference's tree, else the oracle's scalar
+        # restatement; parity against the strict oracle, which is the one pinned to the reference
+        # bit for bit. A batch: the oracle's restatement of the portable kernel.
+        from oracle_lib import (load_oracle, load_ref_q4kgemv, oracle_q4k_gemv_x86,
+                                oracle_q4k_linear, ref_q4k_gemv_m1, Q4KX8_BLOCK_BYTES)
+        import ctypes as C
+        n_s = 65536 if x86 else 16384
         w_s = tables[0][:n_s].cpu().numpy()
         x_s = normed.cpu().numpy()
-        t0 = time.perf_counter()
-        want = oracle_q4k_linear(lib, w_s, x_s, d_model)
-        dt = time.perf_counter() - t0
-        hs.q4k_packed_linear(packed[0], vocab, d_model, normed, logits)
+        kind = "port"
+        if x86:
+            want = oracle_q4k_gemv_x86(load_oracle(fast=False), w_s, x_s[0], d_model)[None, :]
+            ref = load_ref_q4kgemv(fast=True)
+            if ref is not None:
+                kind = "reference"
+                blob = np.zeros(n_s // 8 * nb * Q4KX8_BLOCK_BYTES + 64, dtype=np.uint8)
+                ref.q4k_to_q4kx8_matrix(d_model, n_s, w_s.ctypes.data_as(C.c_void_p),
+                                        blob.ctypes.data_as(C.c_void_p))      # once, as at load
+                xr = np.ascontiguousarray(x_s[0])
+                yr = np.empty(n_s, dtype=np.float32)
+                fp = C.POINTER(C.c_float)
+                args_r = (n_s, d_model, xr.ctypes.data_as(fp), blob.ctypes.data_as(C.c_void_p),
+                          yr.ctypes.data_as(fp))
+                ref.q4kx8_gemv_m1(*args_r)                                   # threads started
+                reps = 20
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    ref.q4kx8_gemv_m1(*args_r)
+                dt = (time.perf_counter() - t0) / reps
+            else:
+                lib = load_oracle(fast=True)
+                t0 = time.perf_counter()
+                oracle_q4k_gemv_x86(lib, w_s, x_s[0], d_model)
+                dt = time.perf_counter() - t0
+            hs.q4k_packed_gemv_x86(packed[0], vocab, d_model, normed, logits)
+        else:
+            lib = load_oracle(fast=True)
+            t0 = time.perf_counter()
+            want = oracle_q4k_linear(lib, w_s, x_s, d_model)
+            dt = time.perf_counter() - t0
+            hs.q4k_packed_linear(packed[0], vocab, d_model, normed, logits)
         hs.sync()
         got = logits[:, :n_s].cpu().numpy()
         result["cpu_baseline"] = {
             "value": round(m_rows / (dt * vocab / n_s), 2), "unit": "rows/s",
             "cores": int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1),
-            "kind": "port",
+            "kind": kind,
             "sample": f"the projection of {m_rows} row(s) over the first {n_s} of {vocab} table rows "
-                      "(dequantise a row, accumulate in double), scaled to the whole table; the "
-                      "sampler's share of the step is not included"}
+                      + (("(q4kx8_gemv_m1: int8 activations, integer dot products"
+                          + (", AVX2, mean of 20 passes)" if kind == "reference" else ", scalar C)"))
+                         if x86 else "(dequantise a row, accumulate in double)")
+                      + ", scaled to the whole table; the sampler's share of the step is not "
+                        "included"}
         result["parity"] = {"logits_compared": int(want.size),
                             "logits_differ": int((got.view(np.uint32) != want.view(np.uint32)).sum())}
     result["token_ids"] = [int(t) for t in ids_gpu[:8]]

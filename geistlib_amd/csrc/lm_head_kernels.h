@@ -93,6 +93,17 @@ void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_o
 /* ... and over the table as it lies in the file (4-byte aligned). */
 void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
                          const uint32_t *act, float *y);
+/* The x86 backend's decode kernel over a Q4_K table (q4kx8_gemv_m1,
+ * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c) over the packed copy (lm_head_q4k_x86.hip):
+ * the activations of n_m rows as int8 with one scale per row (act: per row n_in / 256 *
+ * Q4X_ACT_DWORDS + 1 dwords), and one row's integer dot products with binary32 accumulation in
+ * the reference's order. */
+constexpr int Q4X_ACT_DWORDS = 72; /* 64 of int8 (even / odd elements of every eight), 8 sums */
+size_t q4k_x86_act_dwords(int n_in);
+void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                             uint32_t *act);
+void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const uint32_t *act, float *y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
  * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
 size_t q4k_packed_bytes(long n_out, int n_in);

@@ -1,0 +1,164 @@
+/*
+ * lm_head_q4k_x86.hip -- the lm_head projection of one activation row over a Q4_K table with the
+ * results of the reference's x86 decode kernel q4kx8_gemv_m1
+ * (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:47-77 the activation quantiser, :81-304 the dot
+ * products of one row against eight interleaved table rows, :380-399 the sweep; reached from
+ * cpu_x86_linear_q4k_m1, src/backends/cpu_x86/linear_q4k.c:163-166, for tables of a multiple of
+ * 8 rows). The reference interleaves eight table rows so that eight outputs fill the lanes of a
+ * vector; each output's arithmetic involves its own row alone:
+ *   activations  ONE scale for the row: amax = max |x|, d_a = amax / 127 (1 when amax is 0),
+ *                a = (int) (x / d_a +- 0.5) (round half away from zero), clamped to int8;
+ *   per block    integers: I = sum over the eight sub-blocks j of 32 of scale_j * (sum q * a),
+ *                M = sum_j min_j * (sum of a over sub-block j); binary32:
+ *                acc = fmaf((float) I, d * d_a, acc), acc_min = fmaf((float) M, dmin * d_a,
+ *                acc_min), the two products rounded to binary32 first;
+ *   result       y = acc - acc_min.
+ * The integers cannot overflow (|I| < 2^26), so their order is free; the binary32 steps are the
+ * reference's, which makes the result the reference's bit for bit. Finite activations only.
+ *
+ * The table is read from the packed copy of geist_hip_q4k_pack (lm_head_q6k.hip): a lane owns a
+ * table row; a dword holds the 4-bit values of eight consecutive elements, one mask gives the
+ * even ones as bytes and a shift and a mask the odd ones, and two v_dot4_i32_i8 multiply them
+ * with the activations, which the quantiser lays out to match (per eight elements a dword of the
+ * even ones and a dword of the odd ones) and which are scalar operands.
+ */
+#include "lm_head_kernels.h"
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gs {
+
+constexpr int Q4X_TPB         = 256;
+constexpr int Q4X_ROW_DWORDS  = 37;
+constexpr int Q4X_PACK_DWORDS = Q4X_ROW_DWORDS * 64; /* the packed copy's dwords per (64 rows, block) */
+
+/* One workgroup per activation row. act: per super-block Q4X_ACT_DWORDS dwords -- 64 of int8 (per
+ * eight elements the even ones, then the odd ones), eight int32 sums per sub-block of 32 --, and
+ * behind the row's last block the scale d_a as binary32. */
+__global__ __launch_bounds__(Q4X_TPB) void k_q8k_row_quantize(const float *__restrict__ x, long ld_x,
+                                                             int nb, uint32_t *__restrict__ act) {
+    __shared__ float s_max[Q4X_TPB / 64];
+    const int        m = blockIdx.x, t = threadIdx.x;
+    const float     *xr = x + (long) m * ld_x;
+    uint32_t        *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + 1);
+    float            ax = 0.0f;
+    for (int b = 0; b < nb; ++b)
+        ax = __builtin_fmaxf(ax, __builtin_fabsf(xr[256 * b + t])); /* (a NaN is passed over) */
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1)
+        ax = __builtin_fmaxf(ax, __shfl_xor(ax, s));
+    if ((t & 63) == 0)
+        s_max[t >> 6] = ax;
+    __syncthreads();
+    const float amax  = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]),
+                                        __builtin_fmaxf(s_max[2], s_max[3]));
+    const float scale = amax == 0.0f ? 1.0f : __fdiv_rn(amax, 127.0f);
+    const float inv   = __fdiv_rn(1.0f, scale);
+    if (t == 0)
+        o[(long) nb * Q4X_ACT_DWORDS] = __float_as_uint(scale);
+    for (int b = 0; b < nb; ++b) {
+        const float v = __fmul_rn(xr[256 * b + t], inv);
+        int         q = __float2int_rz(v < 0.0f ? __fsub_rn(v, 0.5f) : __fadd_rn(v, 0.5f));
+        q             = q < -128 ? -128 : q > 127 ? 127 : q;
+        int sum       = q;
+#pragma unroll
+        for (int s = 16; s >= 1; s >>= 1)
+            sum += __shfl_xor(sum, s);
+        const uint32_t b0 = (uint32_t) q & 0xffu;
+        const uint32_t b1 = (uint32_t) __shfl_down(q, 2) & 0xffu;
+        const uint32_t b2 = (uint32_t) __shfl_down(q, 4) & 0xffu;
+        const uint32_t b3 = (uint32_t) __shfl_down(q, 6) & 0xffu;
+        uint32_t      *ob = o + (long) b * Q4X_ACT_DWORDS;
+        if ((t & 7) < 2) /* elements 8 k + {0, 2, 4, 6} to dword 2 k, 8 k + {1, 3, 5, 7} to 2 k + 1 */
+            ob[2 * (t >> 3) + (t & 7)] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+        if ((t & 31) == 0)
+            ob[64 + (t >> 5)] = (uint32_t) sum;
+    }
+}
+
+typedef uint32_t q4x_u4 __attribute__((ext_vector_type(4)));
+
+struct Q4xBlock {
+    uint32_t q[32]; /* the 4-bit values, eight consecutive elements to a dword */
+    uint32_t sc[2]; /* the eight scales as bytes */
+    uint32_t mn[2]; /* the eight minima as bytes */
+    uint32_t dd;    /* d (low half) and dmin, binary16 */
+};
+__device__ __forceinline__ void q4x_load(const uint32_t *__restrict__ base, int r, Q4xBlock &k) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const q4x_u4 t =
+            __builtin_nontemporal_load(reinterpret_cast<const q4x_u4 *>(base + p * 256 + 4 * r));
+        k.q[4 * p] = t.x, k.q[4 * p + 1] = t.y, k.q[4 * p + 2] = t.z, k.q[4 * p + 3] = t.w;
+    }
+    const q4x_u4 t =
+        __builtin_nontemporal_load(reinterpret_cast<const q4x_u4 *>(base + 8 * 256 + 4 * r));
+    k.sc[0] = t.x, k.sc[1] = t.y, k.mn[0] = t.z, k.mn[1] = t.w;
+    k.dd    = __builtin_nontemporal_load(base + 2304 + r);
+}
+
+__global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
+    const uint32_t *__restrict__ packed, long n_out, int nb, const uint32_t *__restrict__ act,
+    float *__restrict__ y) {
+    const int  r = threadIdx.x & 63;
+    const long g = (long) blockIdx.x * (Q4X_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long      row  = g * 64 + r;
+    const uint32_t *base = packed + g * nb * Q4X_PACK_DWORDS;
+    const float     d_a  = __uint_as_float(act[(long) nb * Q4X_ACT_DWORDS]);
+    float           acc = 0.0f, acc_min = 0.0f;
+    /* a block ahead: the next block's loads are in flight while this one is worked on */
+    Q4xBlock cur, nxt;
+    q4x_load(base, r, cur);
+    for (int b = 0; b < nb; ++b) {
+        if (b + 1 < nb)
+            q4x_load(base + (long) (b + 1) * Q4X_PACK_DWORDS, r, nxt);
+        const uint32_t *a = act + (long) b * Q4X_ACT_DWORDS; /* uniform: scalar loads */
+        typedef uint32_t u8v __attribute__((ext_vector_type(8)));
+        const u8v bs = *reinterpret_cast<const u8v *>(a + 64);
+        int       iacc = 0, iacc_min = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { /* sub-block j: elements 32 j .. 32 j + 31, dwords 4 j .. */
+            const u8v av  = *reinterpret_cast<const u8v *>(a + 8 * j);
+            int       dot = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = cur.q[4 * j + k];
+                dot = __builtin_amdgcn_sdot4((int) (w & 0x0f0f0f0fu), (int) av[2 * k], dot, false);
+                dot = __builtin_amdgcn_sdot4((int) ((w >> 4) & 0x0f0f0f0fu), (int) av[2 * k + 1],
+                                             dot, false);
+            }
+            const int sc = (int) ((cur.sc[j >> 2] >> (8 * (j & 3))) & 0xffu);
+            const int mn = (int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu);
+            iacc += __mul24(sc, dot);
+            iacc_min += __mul24(mn, (int) bs[j]);
+        }
+        const float d    = __half2float(__ushort_as_half((unsigned short) (cur.dd & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short) (cur.dd >> 16)));
+        acc     = __builtin_fmaf((float) iacc, __fmul_rn(d, d_a), acc);
+        acc_min = __builtin_fmaf((float) iacc_min, __fmul_rn(dmin, d_a), acc_min);
+        if (b + 1 < nb)
+            cur = nxt;
+    }
+    if (row < n_out)
+        y[row] = __fsub_rn(acc, acc_min);
+}
+
+size_t q4k_x86_act_dwords(int n_in) { return (size_t) (n_in / 256) * Q4X_ACT_DWORDS + 1; }
+
+void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                             uint32_t *act) {
+    k_q8k_row_quantize<<<dim3(n_m), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, n_in / 256, act);
+}
+
+void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
+                                const uint32_t *act, float *y) {
+    const long groups = (n_out + 63) / 64;
+    k_q4k_packed_gemv_x86<<<dim3((unsigned) ((groups + 3) / 4)), dim3(Q4X_TPB), 0, stream>>>(
+        static_cast<const uint32_t *>(packed), n_out, n_in / 256, act, y);
+}
+
+} // namespace gs

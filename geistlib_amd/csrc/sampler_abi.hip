@@ -1499,6 +1499,51 @@ static int q4k_packed_linear_impl(geist_hip_sampler *s, const void *d_packed, si
     return GEIST_HIP_OK;
 }
 
+/* Shapes the reference's x86 decode kernel takes (q4kx8_gemv_m1: rows in eights, at most 64
+ * super-blocks per row); others go through other kernels of that backend, not reproduced. */
+static bool q4k_x86_shape(size_t n_out, size_t n_in) {
+    return n_out % 8 == 0 && n_in % 256 == 0 && n_in / 256 >= 1 && n_in / 256 <= 64;
+}
+
+static int q4k_packed_gemv_x86_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                    size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                    float *d_y, size_t ld_y) {
+    Q6KScratch ws; /* (its int8 activation area: 96 dwords per super-block, 73 needed) */
+    const int  rc = q6k_scratch(s, n_out, n_in, ws);
+    if (rc)
+        return rc;
+    for (size_t m = 0; m < n_rows; ++m) {
+        launch_q8k_row_quantize(s->stream, d_x + m * ld_x, (long) ld_x, 1, (int) n_in, ws.act8);
+        launch_q4k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in, ws.act8,
+                                   d_y + m * ld_y);
+    }
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                       float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K decode: %zu rows, strides %zu / %zu", n_rows,
+                    ld_x, ld_y);
+    int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (!q4k_x86_shape(n_out, n_in))
+        return fail(s, GEIST_HIP_E_UNSUPPORTED,
+                    "Q4_K decode: %zu x %zu is not a shape of the x86 kernel (rows in eights, at "
+                    "most 64 super-blocks per row)", n_out, n_in);
+    if (((uintptr_t) d_packed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q4_K table not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q4k_packed_gemv_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q4_K decode (packed)");
+}
+
 size_t geist_hip_q4k_packed_bytes(size_t n_out, size_t n_in) {
     if (n_out == 0 || n_in == 0 || n_in % 256 != 0 || n_in > 0x7fffff00u)
         return 0;
@@ -1687,7 +1732,12 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
                                 (int) d_model, q6ws.act8, d_logits);
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
-        rc = table == TABLE_Q4K_PACKED
+        rc = table == TABLE_Q4K_PACKED && rows == 1 && !s->projection_portable &&
+                     q4k_x86_shape(n_vocab, d_model)
+                 /* one row on the x86 backend: its integer decode kernel (q4kx8_gemv_m1) */
+                 ? q4k_packed_gemv_x86_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
+                                            d_logits, ld_logits)
+             : table == TABLE_Q4K_PACKED
                  ? q4k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)
              : table == TABLE_Q6K_PACKED

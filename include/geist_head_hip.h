@@ -140,9 +140,12 @@ int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, s
  * Without the load the call is refused (GEIST_HIP_E_UNSUPPORTED): only the packed copy has a
  * kernel. The logits equal, bit for bit, those of the portable kernel cpu_scalar_w_quant_m1 /
  * _mN after dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, weight_resolve.c:82-83, 186-241),
- * for one row and for a batch. The x86 and NEON backends decode this dtype with int8
- * activations (W4A8: src/backends/cpu_x86/linear_q4k.c), a different arithmetic with different
- * logits, which is not reproduced. */
+ * for one row and for a batch. Unless geist_hip_head_set_projection chose the portable backend,
+ * one row over a vocabulary of a multiple of 8 tokens (d_model <= 16384) gets the logits of the
+ * x86 backend's decode kernel q4kx8_gemv_m1 instead (int8 activations, integer dot products:
+ * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c, from src/backends/cpu_x86/linear_q4k.c:163-166),
+ * again bit for bit. That backend's batch kernels and its W4A8 kernels for other shapes, and
+ * the NEON backend's kernels, are not reproduced. */
 int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d_hidden,
                                         size_t ld_hidden, size_t k, const float *d_norm_weight,
                                         float rms_eps, const void *d_embed_q4k, size_t d_model,

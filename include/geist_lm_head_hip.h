@@ -54,7 +54,8 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
 
 /* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
  * the head's project_finalize calls) stands for:
- *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a Q6_K table q6k_gemv_m1;
+ *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a Q6_K table q6k_gemv_m1, over a
+ *                                  packed Q4_K table q4kx8_gemv_m1;
  *                                  more rows: the portable kernel (default)
  *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
  *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
@@ -221,6 +222,23 @@ int geist_hip_q4k_pack(geist_hip_sampler *s, const void *d_w_q4k, size_t n_out, 
 int geist_hip_q4k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                      size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                      float *d_y, size_t ld_y);
+/* The x86 backend's decode kernel over the packed copy: replaces q4kx8_gemv_m1
+ * (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:47-77, 81-304, 380-399; reached from
+ * cpu_x86_linear_q4k_m1, src/backends/cpu_x86/linear_q4k.c:163-166, over the table that
+ * q4k_to_q4kx8_matrix interleaves), bit for bit: the activation row becomes int8 with ONE scale
+ * (amax / 127, round half away from zero), the products with the 4-bit values are summed as
+ * integers per sub-block of 32 and weighted with the sub-block's scale, the minima with the
+ * activations' sums; per super-block each of the two integers joins a binary32 accumulator by a
+ * fused multiply-add, and the result is the difference of the accumulators. For the shapes that
+ * kernel takes -- n_out a multiple of 8, n_in / 256 <= 64 -- and GEIST_HIP_E_UNSUPPORTED for
+ * others (the reference sends those through its W4A8 kernels, which are not reproduced). Each
+ * activation row is a pass of its own over the table. Activations must be finite.
+ * geist_hip_project_sample_rows_q4k_packed follows geist_hip_sampler_set_projection: in the
+ * default mode GEIST_HIP_PROJECTION_X86 one row over a table of such a shape gets this kernel;
+ * a batch, other shapes and any call in mode _PORTABLE get geist_hip_q4k_packed_linear_rows. */
+int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                       float *d_y, size_t ld_y);
 int geist_hip_project_sample_rows_q4k_packed(geist_hip_sampler *s, const float *d_hidden,
                                              size_t ld_hidden, size_t rows, size_t d_model,
                                              const float *d_norm_weight, float rms_eps,

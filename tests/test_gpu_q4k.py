@@ -6,7 +6,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import oracle_q4k_linear, random_q4k_table
+from oracle_lib import oracle_q4k_gemv_x86, oracle_q4k_linear, random_q4k_table
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -48,6 +48,40 @@ def test_q4k_linear_equals_the_portable_kernel(hs, oracle, n_out, n_in, m):
         got = y.cpu().numpy()
         bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
         assert bad.size == 0, (scale, bad[:5], got[tuple(bad[0])], want[tuple(bad[0])])
+
+
+@pytest.mark.parametrize("n_out,n_in", [(8, 256), (64, 256), (304, 512), (5000, 1536),
+                                        (4104, 2560), (70000, 1024), (72, 16384)])
+def test_q4k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
+    """The x86 backend's integer decode kernel (q4kx8_gemv_m1 over the table its repacker
+    interleaves), to which the oracle is pinned by the compiled reference
+    (tests/test_q4k_x86_oracle.py): logits bit for bit, row by row."""
+    print(f"q4k x86 decode {n_out} x {n_in}", flush=True)
+    g = np.random.default_rng(n_out + n_in)
+    w = random_q4k_table(g, n_out, n_in)
+    packed = packed_copy(hs, w, n_in)
+    for scale in (1.0, 1e-4, 300.0, 0.0):
+        x = (g.standard_normal((3, n_in)) * scale).astype(np.float32)
+        x[0, ::5] = 0.0
+        x[2, 7] = np.float32(1e30)            # one huge activation: the others round to zero
+        d_x = torch.from_numpy(x).cuda()
+        y = torch.full((3, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q4k_packed_gemv_x86(packed, n_out, n_in, d_x, y)
+        hs.sync()
+        got = y.cpu().numpy()
+        for m in range(3):
+            want = oracle_q4k_gemv_x86(oracle.lib, w, x[m], n_in)
+            bad = np.flatnonzero(got[m].view(np.uint32) != want.view(np.uint32))
+            assert bad.size == 0, (scale, m, bad[:5], got[m][bad[:3]], want[bad[:3]])
+
+
+def test_q4k_decode_refuses_shapes_the_x86_kernel_does_not_take(hs):
+    from geistlib_amd.binding import GeistHipError
+    packed = torch.zeros((hs.q4k_packed_bytes(12, 256),), dtype=torch.uint8, device="cuda")
+    x = torch.zeros((1, 256), dtype=torch.float32, device="cuda")
+    y = torch.zeros((1, 12), dtype=torch.float32, device="cuda")
+    with pytest.raises(GeistHipError):                        # 12 rows: not a multiple of 8
+        hs.q4k_packed_gemv_x86(packed, 12, 256, x, y)
 
 
 def test_q4k_linear_rows_whose_sums_cancel(hs, oracle):
@@ -103,9 +137,13 @@ def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
     w[:, 3::144] &= 0x03
     norm_w = (1.0 + 0.1 * g.standard_normal(d_model)).astype(np.float32)
     d_w, d_nw = torch.from_numpy(w).cuda(), torch.from_numpy(norm_w).cuda()
-    for T, p, top_k in [(0.0, 1.0, 0), (0.8, 1.0, 40), (0.9, 0.95, 0)]:
-        print(f"q4k table T={T} p={p} k={top_k}", flush=True)
+    host.geist_hip_head_set_projection.argtypes = [C.c_void_p, C.c_int]
+    for T, p, top_k, portable in [(0.0, 1.0, 0, False), (0.8, 1.0, 40, False),
+                                  (0.9, 0.95, 0, False), (0.8, 1.0, 40, True)]:
+        print(f"q4k table T={T} p={p} k={top_k} portable={portable}", flush=True)
         h = make_head(host, vocab, 4, cap)
+        if portable:
+            assert host.geist_hip_head_set_projection(h, 1) == 0
         opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 4)
         assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
         hidden = (g.standard_normal((1, d_model)) * 4).astype(np.float32)
@@ -125,7 +163,11 @@ def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
                 h, C.c_void_p(d_hid.data_ptr()), d_model, k, C.c_void_p(d_nw.data_ptr()), 1e-6,
                 C.c_void_p(d_w.data_ptr()), d_model, out)
             assert rc == 0, host.geist_hip_head_errmsg(h)
-            logits = oracle_q4k_linear(oracle.lib, w, oracle.rmsnorm(hidden, norm_w, 1e-6), d_model)
+            normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
+            if k == 1 and not portable:      # the x86 backend's decode kernel
+                logits = oracle_q4k_gemv_x86(oracle.lib, w, normed[0], d_model)[None, :]
+            else:
+                logits = oracle_q4k_linear(oracle.lib, w, normed, d_model)
             want = oracle.finalize_batch(sess, logits, softcap=cap).tolist()
-            assert list(out) == want, (T, p, top_k, k)
+            assert list(out) == want, (T, p, top_k, k, portable)
         host.geist_hip_head_destroy(h)
