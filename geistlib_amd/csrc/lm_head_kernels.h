@@ -102,6 +102,9 @@ constexpr int Q4X_ACT_DWORDS = 72; /* 64 of int8 (even / odd elements of every e
 size_t q4k_x86_act_dwords(int n_in);
 void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
                              uint32_t *act);
+/* launch_rmsnorm_rows and that quantiser in one launch (n a multiple of 256) */
+void launch_rmsnorm_q8k_row_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                                 float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act);
 void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
                                 const uint32_t *act, float *y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of

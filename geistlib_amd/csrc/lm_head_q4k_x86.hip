@@ -23,6 +23,7 @@
  * even ones and a dword of the odd ones) and which are scalar operands.
  */
 #include "lm_head_kernels.h"
+#include "rmsnorm_device.h"
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -33,6 +34,27 @@ namespace gs {
 constexpr int Q4X_TPB         = 256;
 constexpr int Q4X_ROW_DWORDS  = 37;
 constexpr int Q4X_PACK_DWORDS = Q4X_ROW_DWORDS * 64; /* the packed copy's dwords per (64 rows, block) */
+
+/* Thread t's element of a super-block, given the reciprocal of the row's scale: its int8 value
+ * into the block's dwords (ob), the sums per sub-block of 32 behind them. */
+__device__ __forceinline__ void q4x_quantize_block(float xv, float inv, uint32_t *__restrict__ ob) {
+    const int   t = threadIdx.x;
+    const float v = __fmul_rn(xv, inv);
+    int         q = __float2int_rz(v < 0.0f ? __fsub_rn(v, 0.5f) : __fadd_rn(v, 0.5f));
+    q             = q < -128 ? -128 : q > 127 ? 127 : q;
+    int sum       = q;
+#pragma unroll
+    for (int s = 16; s >= 1; s >>= 1)
+        sum += __shfl_xor(sum, s);
+    const uint32_t b0 = (uint32_t) q & 0xffu;
+    const uint32_t b1 = (uint32_t) __shfl_down(q, 2) & 0xffu;
+    const uint32_t b2 = (uint32_t) __shfl_down(q, 4) & 0xffu;
+    const uint32_t b3 = (uint32_t) __shfl_down(q, 6) & 0xffu;
+    if ((t & 7) < 2) /* elements 8 k + {0, 2, 4, 6} to dword 2 k, 8 k + {1, 3, 5, 7} to 2 k + 1 */
+        ob[2 * (t >> 3) + (t & 7)] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    if ((t & 31) == 0)
+        ob[64 + (t >> 5)] = (uint32_t) sum;
+}
 
 /* One workgroup per activation row. act: per super-block Q4X_ACT_DWORDS dwords -- 64 of int8 (per
  * eight elements the even ones, then the odd ones), eight int32 sums per sub-block of 32 --, and
@@ -58,24 +80,48 @@ __global__ __launch_bounds__(Q4X_TPB) void k_q8k_row_quantize(const float *__res
     const float inv   = __fdiv_rn(1.0f, scale);
     if (t == 0)
         o[(long) nb * Q4X_ACT_DWORDS] = __float_as_uint(scale);
+    for (int b = 0; b < nb; ++b)
+        q4x_quantize_block(xr[256 * b + t], inv, o + (long) b * Q4X_ACT_DWORDS);
+}
+
+/* The output norm (cpu_scalar_rmsnorm, as k_rmsnorm_rows computes it) and that quantiser in one
+ * launch, one workgroup per row: the normed row goes to y and, as int8, to act. A thread reads
+ * back what it wrote itself. n a multiple of 256. */
+__global__ __launch_bounds__(Q4X_TPB) void k_rmsnorm_q8k_row_rows(const float *__restrict__ x,
+                                                                 long ld_x,
+                                                                 const float *__restrict__ w,
+                                                                 float eps, int n,
+                                                                 float *__restrict__ y, long ld_y,
+                                                                 uint32_t *__restrict__ act) {
+    __shared__ double s_part[Q4X_TPB];
+    __shared__ float  s_inv;
+    __shared__ float  s_max[Q4X_TPB / 64];
+    const int    nb = n / 256, m = blockIdx.x, t = threadIdx.x;
+    const float *xr = x + (long) m * ld_x;
+    float       *yr = y + (long) m * ld_y;
+    uint32_t    *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + 1);
+    const float  rinv = block_rms_inv<Q4X_TPB>(xr, n, eps, s_part, &s_inv);
+    float        ax = 0.0f;
     for (int b = 0; b < nb; ++b) {
-        const float v = __fmul_rn(xr[256 * b + t], inv);
-        int         q = __float2int_rz(v < 0.0f ? __fsub_rn(v, 0.5f) : __fadd_rn(v, 0.5f));
-        q             = q < -128 ? -128 : q > 127 ? 127 : q;
-        int sum       = q;
-#pragma unroll
-        for (int s = 16; s >= 1; s >>= 1)
-            sum += __shfl_xor(sum, s);
-        const uint32_t b0 = (uint32_t) q & 0xffu;
-        const uint32_t b1 = (uint32_t) __shfl_down(q, 2) & 0xffu;
-        const uint32_t b2 = (uint32_t) __shfl_down(q, 4) & 0xffu;
-        const uint32_t b3 = (uint32_t) __shfl_down(q, 6) & 0xffu;
-        uint32_t      *ob = o + (long) b * Q4X_ACT_DWORDS;
-        if ((t & 7) < 2) /* elements 8 k + {0, 2, 4, 6} to dword 2 k, 8 k + {1, 3, 5, 7} to 2 k + 1 */
-            ob[2 * (t >> 3) + (t & 7)] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-        if ((t & 31) == 0)
-            ob[64 + (t >> 5)] = (uint32_t) sum;
+        const int   i = 256 * b + t;
+        const float v = __fmul_rn(__fmul_rn(xr[i], rinv), w[i]);
+        yr[i]         = v;
+        ax            = __builtin_fmaxf(ax, __builtin_fabsf(v));
     }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1)
+        ax = __builtin_fmaxf(ax, __shfl_xor(ax, s));
+    if ((t & 63) == 0)
+        s_max[t >> 6] = ax;
+    __syncthreads();
+    const float amax  = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]),
+                                        __builtin_fmaxf(s_max[2], s_max[3]));
+    const float scale = amax == 0.0f ? 1.0f : __fdiv_rn(amax, 127.0f);
+    const float inv   = __fdiv_rn(1.0f, scale);
+    if (t == 0)
+        o[(long) nb * Q4X_ACT_DWORDS] = __float_as_uint(scale);
+    for (int b = 0; b < nb; ++b)
+        q4x_quantize_block(yr[256 * b + t], inv, o + (long) b * Q4X_ACT_DWORDS);
 }
 
 typedef uint32_t q4x_u4 __attribute__((ext_vector_type(4)));
@@ -152,6 +198,12 @@ size_t q4k_x86_act_dwords(int n_in) { return (size_t) (n_in / 256) * Q4X_ACT_DWO
 void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
                              uint32_t *act) {
     k_q8k_row_quantize<<<dim3(n_m), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, n_in / 256, act);
+}
+
+void launch_rmsnorm_q8k_row_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                                 float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act) {
+    k_rmsnorm_q8k_row_rows<<<dim3(n_rows), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y,
+                                                                      act);
 }
 
 void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,

@@ -1703,12 +1703,21 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
      * (q6k_gemv_m1), whose activation quantiser rides on the norm's launch */
     const bool q6k_x86 = (table == TABLE_Q6K_PACKED || table == TABLE_Q6K) && rows == 1 &&
                          !s->projection_portable;
+    /* ... and over a packed Q4_K table of a shape that backend's decode kernel takes
+     * (q4kx8_gemv_m1), likewise */
+    const bool q4k_x86 = table == TABLE_Q4K_PACKED && rows == 1 && !s->projection_portable &&
+                         q4k_x86_shape(n_vocab, d_model);
     Q6KScratch q6ws{};
-    if (q6k_x86) {
+    if (q6k_x86 || q4k_x86) {
         if ((rc = q6k_scratch(s, n_vocab, d_model, q6ws)) != GEIST_HIP_OK)
             return rc;
-        launch_rmsnorm_q8k_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps, 1,
-                                (int) d_model, d_normed, (long) d_model, q6ws.act8);
+        if (q6k_x86)
+            launch_rmsnorm_q8k_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
+                                    1, (int) d_model, d_normed, (long) d_model, q6ws.act8);
+        else
+            launch_rmsnorm_q8k_row_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight,
+                                        rms_eps, 1, (int) d_model, d_normed, (long) d_model,
+                                        q6ws.act8);
     } else {
         launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
                             (int) rows, (int) d_model, d_normed, (long) d_model);
@@ -1730,14 +1739,12 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_embed), (long) n_vocab,
                                 (int) d_model, q6ws.act8, d_logits);
+    } else if (q4k_x86) {
+        launch_q4k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,
+                                   d_logits);
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
-        rc = table == TABLE_Q4K_PACKED && rows == 1 && !s->projection_portable &&
-                     q4k_x86_shape(n_vocab, d_model)
-                 /* one row on the x86 backend: its integer decode kernel (q4kx8_gemv_m1) */
-                 ? q4k_packed_gemv_x86_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
-                                            d_logits, ld_logits)
-             : table == TABLE_Q4K_PACKED
+        rc = table == TABLE_Q4K_PACKED
                  ? q4k_packed_linear_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
                                           d_logits, ld_logits)
              : table == TABLE_Q6K_PACKED
