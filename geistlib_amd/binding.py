@@ -126,6 +126,10 @@ def load_library():
     lib.geist_hip_q8k_act_bytes.restype = sz
     lib.geist_hip_q8k_quantize_rows.argtypes = [vp, vp, sz, sz, sz, vp]
     lib.geist_hip_q6k_packed_gemv_q8k.argtypes = [vp, vp, sz, sz, vp, vp]
+    lib.geist_hip_q8k_row_act_bytes.argtypes = [sz]
+    lib.geist_hip_q8k_row_act_bytes.restype = sz
+    lib.geist_hip_q8k_row_quantize.argtypes = [vp, vp, sz, vp]
+    lib.geist_hip_q4k_packed_gemv_q8k.argtypes = [vp, vp, sz, sz, vp, vp]
     lib.geist_hip_project_sample_rows_q6k_packed.argtypes = [vp, vp, sz, sz, sz, vp, f32, vp, sz,
                                                              vp, vp, sz, C.POINTER(SampleParams),
                                                              vp, vp, i32, vp]
@@ -439,6 +443,20 @@ class HipSampler:
     def q6k_packed_gemv_q8k(self, packed, n_out, n_in, act, y):
         """One row of int8 activations (q8k_quantize) times the packed table: y [n_out]."""
         self._check(self.lib.geist_hip_q6k_packed_gemv_q8k(self.h, _ptr(packed), n_out, n_in,
+                                                           _ptr(act), _ptr(y)))
+
+    def q8k_row_act_bytes(self, n_in):
+        return int(self.lib.geist_hip_q8k_row_act_bytes(n_in))
+
+    def q8k_row_quantize(self, x, act):
+        """x [n_in] float32 -> act: the row as int8 with one scale (q8k_row_act_bytes bytes)."""
+        n_in = x.numel()
+        assert x.is_contiguous() and act.numel() * act.element_size() >= self.q8k_row_act_bytes(n_in)
+        self._check(self.lib.geist_hip_q8k_row_quantize(self.h, _ptr(x), n_in, _ptr(act)))
+
+    def q4k_packed_gemv_q8k(self, packed, n_out, n_in, act, y):
+        """One row of int8 activations (q8k_row_quantize) times the packed Q4_K table: y [n_out]."""
+        self._check(self.lib.geist_hip_q4k_packed_gemv_q8k(self.h, _ptr(packed), n_out, n_in,
                                                            _ptr(act), _ptr(y)))
 
     def f16_to_q8w(self, w_f16, wq, scales):

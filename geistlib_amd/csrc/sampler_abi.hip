@@ -1544,6 +1544,51 @@ int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packe
     return rc ? rc : after_launch(s, "Q4_K decode (packed)");
 }
 
+size_t geist_hip_q8k_row_act_bytes(size_t n_in) {
+    if (n_in == 0 || n_in % 256 != 0 || n_in > 0x7fffff00u)
+        return 0;
+    return q4k_x86_act_dwords((int) n_in) * sizeof(uint32_t);
+}
+
+int geist_hip_q8k_row_quantize(geist_hip_sampler *s, const float *d_x, size_t n_in, void *d_act) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_x || !d_act)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_in == 0 || n_in > 0x7fffff00u)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "int8 activation row of %zu", n_in);
+    if (n_in % 256 != 0)
+        return fail(s, GEIST_HIP_E_UNSUPPORTED, "int8 activation row: %zu is not a multiple of 256",
+                    n_in);
+    if (((uintptr_t) d_act) % 64 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "int8 activation row: buffer not 64-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_q8k_row_quantize(s->stream, d_x, (long) n_in, 1, (int) n_in,
+                            static_cast<uint32_t *>(d_act));
+    return after_launch(s, "int8 activation row");
+}
+
+int geist_hip_q4k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                  size_t n_in, const void *d_act, float *d_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_act || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    const int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (!q4k_x86_shape(n_out, n_in))
+        return fail(s, GEIST_HIP_E_UNSUPPORTED,
+                    "Q4_K decode: %zu x %zu is not a shape of the x86 kernel (rows in eights, at "
+                    "most 64 super-blocks per row)", n_out, n_in);
+    if (((uintptr_t) d_packed) % 16 != 0 || ((uintptr_t) d_act) % 64 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K decode: table or activations misaligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    launch_q4k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in,
+                               static_cast<const uint32_t *>(d_act), d_y);
+    return after_launch(s, "Q4_K decode (packed)");
+}
+
 size_t geist_hip_q4k_packed_bytes(size_t n_out, size_t n_in) {
     if (n_out == 0 || n_in == 0 || n_in % 256 != 0 || n_in > 0x7fffff00u)
         return 0;

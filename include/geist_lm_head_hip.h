@@ -239,6 +239,16 @@ int geist_hip_q4k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
 int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                        size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                        float *d_y, size_t ld_y);
+/* The two halves of that kernel, as for Q6_K: geist_hip_q8k_row_quantize replaces the activation
+ * quantiser of kernel_q4kx8_gemm_avx512.c:47-77 for one row -- d_act, 64-byte aligned,
+ * geist_hip_q8k_row_act_bytes(n_in) bytes, gets per super-block 72 dwords (the 256 activations as
+ * int8, per eight elements the even ones and then the odd ones; their eight sums per sub-block
+ * of 32 as int32) and behind the last block the row's scale as binary32 --, and
+ * geist_hip_q4k_packed_gemv_q8k replaces the dot products of :81-304 over it. */
+size_t geist_hip_q8k_row_act_bytes(size_t n_in);
+int geist_hip_q8k_row_quantize(geist_hip_sampler *s, const float *d_x, size_t n_in, void *d_act);
+int geist_hip_q4k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                  size_t n_in, const void *d_act, float *d_y);
 int geist_hip_project_sample_rows_q4k_packed(geist_hip_sampler *s, const float *d_hidden,
                                              size_t ld_hidden, size_t rows, size_t d_model,
                                              const float *d_norm_weight, float rms_eps,

@@ -6,7 +6,8 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import oracle_q4k_gemv_x86, oracle_q4k_linear, random_q4k_table
+from oracle_lib import (oracle_q4k_gemv_x86, oracle_q4k_linear, oracle_q8k_row_quantize,
+                        random_q4k_table)
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -73,6 +74,23 @@ def test_q4k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
             want = oracle_q4k_gemv_x86(oracle.lib, w, x[m], n_in)
             bad = np.flatnonzero(got[m].view(np.uint32) != want.view(np.uint32))
             assert bad.size == 0, (scale, m, bad[:5], got[m][bad[:3]], want[bad[:3]])
+        # the kernel's two halves: the int8 activations as the reference's quantiser leaves them
+        # (per eight elements the even ones, then the odd ones), and the dot products over them
+        nb = n_in // 256
+        act = torch.full((hs.q8k_row_act_bytes(n_in) // 4,), -1, dtype=torch.int32, device="cuda")
+        hs.q8k_row_quantize(d_x[1], act)
+        y1 = torch.full((n_out,), np.nan, dtype=torch.float32, device="cuda")
+        hs.q4k_packed_gemv_q8k(packed, n_out, n_in, act, y1)
+        hs.sync()
+        a = act.cpu().numpy()
+        d, qs, bs = oracle_q8k_row_quantize(oracle.lib, x[1])
+        blocks = a[:nb * 72].reshape(nb, 72)
+        q = blocks[:, :64].copy().view(np.int8).reshape(nb, 32, 2, 4)    # [block, eight, parity, i]
+        assert (q.transpose(0, 1, 3, 2).reshape(-1) == qs).all(), scale
+        assert (blocks[:, 64:].reshape(-1) ==
+                bs.astype(np.int32).reshape(-1, 2).sum(axis=1)).all(), scale
+        assert a[nb * 72:].view(np.float32)[0] == np.float32(d), scale
+        assert (y1.cpu().numpy().view(np.uint32) == got[1].view(np.uint32)).all(), scale
 
 
 def test_q4k_decode_refuses_shapes_the_x86_kernel_does_not_take(hs):
