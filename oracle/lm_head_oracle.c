@@ -332,7 +332,7 @@ void oracle_q8k_row_quantize(size_t n_super, const float *x, float *d_out, int8_
  * accumulator by one fused multiply-add with (d * d_act) and (dmin * d_act) -- both products
  * rounded to binary32 first --, and the result is the difference of the two accumulators. */
 static float oracle_dot_q4k_q8k(size_t n_super, const uint8_t *row, float d_act, const int8_t *qs,
-                                const int16_t *bsums) {
+                                const int16_t *bsums, int per_pair) {
     float acc = 0.0f, acc_min = 0.0f;
     for (size_t b = 0; b < n_super; b++, row += 144) {
         const float    d    = oracle_f16_to_f32((uint16_t) (row[0] | (row[1] << 8)));
@@ -356,7 +356,17 @@ static float oracle_dot_q4k_q8k(size_t n_super, const uint8_t *row, float d_act,
             }
             iacc += scale * dot;
             iacc_min += min * (bsums[b * 16 + 2 * j] + bsums[b * 16 + 2 * j + 1]);
+            if (per_pair && (j & 1)) {
+                /* the 16 x 16 tiles of kernel_q4kx8_gemm_avx512_full.c:94-779 join the
+                 * accumulators once per pair of sub-blocks, not once per super-block */
+                acc      = fmaf((float) iacc, d * d_act, acc);
+                acc_min  = fmaf((float) iacc_min, dmin * d_act, acc_min);
+                iacc     = 0;
+                iacc_min = 0;
+            }
         }
+        if (per_pair)
+            continue;
         acc     = fmaf((float) iacc, d * d_act, acc);
         acc_min = fmaf((float) iacc_min, dmin * d_act, acc_min);
     }
@@ -378,7 +388,73 @@ int oracle_q4k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w
     oracle_q8k_row_quantize(n_super, x, &d_act, qs, bsums);
 #pragma omp parallel for schedule(static)
     for (size_t r = 0; r < n_out; r++)
-        y[r] = oracle_dot_q4k_q8k(n_super, (const uint8_t *) w_q4k + r * n_super * 144, d_act, qs, bsums);
+        y[r] = oracle_dot_q4k_q8k(n_super, (const uint8_t *) w_q4k + r * n_super * 144, d_act, qs, bsums, 0);
+    free(qs);
+    free(bsums);
+    return 0;
+}
+
+/* ---- the x86 backend's batch kernel over a Q4_K table ----------------------------------------
+ * cpu_x86_linear_q4k_mN (src/backends/cpu_x86/linear_q4k.c:198-250). A batch whose row count is
+ * not a multiple of 4 is the decode kernel row by row (:222-229). Otherwise the rows are quantised
+ * four at a time by quantize_q8_Kx4 (q8_kx4.c:21-105) and go through q4kx8_gemm_avx512
+ * (kernel_q4kx8_gemm_avx512_full.c:800-860): the 16 x 16 tiles of an AVX-512 host for row counts
+ * that are multiples of 16, q4kx8_gemv_avx2_fallback (kernel_q4kx8_gemm_avx512.c:317-371) for the
+ * others and on hosts without AVX-512. The fallback is the decode kernel's arithmetic per output
+ * (it calls the same q4kx8_gemv_one_row_tile), so its rows differ from the decode kernel's only
+ * through the quantiser: still ONE scale per row, but lrintf (ties to even) and no clamp. The
+ * tiles form the same integers but join them to the binary32 accumulators once per pair of
+ * sub-blocks (full.c:94, 729-778), four times per super-block. */
+
+void oracle_q8kx4_row_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                               int16_t *bsums_out) {
+    /* quantize_q8_Kx4 for one of its four rows, the int8 values back in element order (the
+     * interleaving in stripes of eight only places them for the vector kernel) */
+    float amax = 0.0f;
+    for (size_t k = 0; k < n_super * 256; k++) {
+        const float a = fabsf(x[k]);
+        if (a > amax)
+            amax = a;
+    }
+    const float scale = amax == 0.0f ? 1.0f : amax / 127.0f;
+    const float inv   = 1.0f / scale;
+    *d_out            = scale;
+    for (size_t k = 0; k < n_super * 256; k++)
+        qs_out[k] = (int8_t) lrintf(x[k] * inv);
+    for (size_t g = 0; g < n_super * 16; g++) {
+        int s = 0;
+        for (int i = 0; i < 16; i++)
+            s += qs_out[g * 16 + i];
+        bsums_out[g] = (int16_t) s;
+    }
+}
+
+int oracle_q4k_linear_x86(size_t m, size_t n_out, size_t n_in, const float *x, const void *w_q4k,
+                          float *y, int avx512) {
+    const size_t n_super = n_in / 256;
+    if (n_in % 256 != 0 || n_super == 0 || n_super > 64 || n_out % 8 != 0 || m == 0)
+        return -1; /* shapes these kernels do not take */
+    const int kx4   = m > 1 && m % 4 == 0;
+    /* full.c:831-835: the tiles need both counts to be multiples of 16, and an AVX-512 host */
+    const int tiles = avx512 && kx4 && m % 16 == 0 && n_out % 16 == 0;
+    int8_t   *qs    = malloc(n_in);
+    int16_t  *bsums = malloc(n_super * 16 * sizeof(int16_t));
+    if (!qs || !bsums) {
+        free(qs);
+        free(bsums);
+        return -2;
+    }
+    for (size_t i = 0; i < m; i++) {
+        float d_act;
+        if (kx4)
+            oracle_q8kx4_row_quantize(n_super, x + i * n_in, &d_act, qs, bsums);
+        else
+            oracle_q8k_row_quantize(n_super, x + i * n_in, &d_act, qs, bsums);
+#pragma omp parallel for schedule(static)
+        for (size_t r = 0; r < n_out; r++)
+            y[i * n_out + r] = oracle_dot_q4k_q8k(
+                n_super, (const uint8_t *) w_q4k + r * n_super * 144, d_act, qs, bsums, tiles);
+    }
     free(qs);
     free(bsums);
     return 0;

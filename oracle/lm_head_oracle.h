@@ -89,6 +89,18 @@ int  oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *
 void oracle_q8k_row_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
                              int16_t *bsums_out);
 int oracle_q4k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q4k, float *y);
+/* The x86 backend's batch kernel over a Q4_K table (cpu_x86_linear_q4k_mN,
+ * src/backends/cpu_x86/linear_q4k.c:198-250): row counts that are no multiple of 4 are the decode
+ * kernel row by row; the others are quantised by quantize_q8_Kx4 (q8_kx4.c:21-105: one scale per
+ * row, lrintf) and multiplied by q4kx8_gemm_avx512: per output the decode kernel's arithmetic,
+ * except that with avx512 != 0 (a host with AVX-512) row counts that are multiples of 16 over a
+ * table of a multiple of 16 rows go through 16 x 16 tiles, which join the binary32 accumulators
+ * once per pair of sub-blocks. x [m, n_in], y [m, n_out]. Pinned to those translation units compiled from the
+ * reference's tree (tests/test_q4k_x86_oracle.py), the 16 x 16 AVX-512 tiles included. */
+void oracle_q8kx4_row_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
+                               int16_t *bsums_out);
+int oracle_q4k_linear_x86(size_t m, size_t n_out, size_t n_in, const float *x, const void *w_q4k,
+                          float *y, int avx512);
 
 /* The same pair for a Q4_K table (super-blocks of 144 bytes: d, dmin in binary16, eight 6-bit
  * scales and eight 6-bit minima packed into 12 bytes, 128 bytes of 4-bit values;

@@ -639,7 +639,37 @@ def oracle_q8k_row_quantize(lib, x):
     return float(d[0]), qs, bs
 
 
+def oracle_q8kx4_row_quantize(lib, x):
+    """(d, qs int8 [n_in], bsums int16 [n_in / 16]) of one row as quantize_q8_Kx4 leaves it."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    ns = x.size // 256
+    d = np.empty(1, dtype=np.float32)
+    qs = np.empty(ns * 256, dtype=np.int8)
+    bs = np.empty(ns * 16, dtype=np.int16)
+    lib.oracle_q8kx4_row_quantize.argtypes = [C.c_size_t, c_float_p, c_float_p, C.c_void_p,
+                                              C.c_void_p]
+    lib.oracle_q8kx4_row_quantize.restype = None
+    lib.oracle_q8kx4_row_quantize(ns, _fp(x), _fp(d), qs.ctypes.data_as(C.c_void_p),
+                                  bs.ctypes.data_as(C.c_void_p))
+    return float(d[0]), qs, bs
+
+
+def oracle_q4k_linear_x86(lib, w_q4k, x, n_in, avx512=True):
+    """oracle_q4k_linear_x86: the x86 backend's projection of a batch over a Q4_K table."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
+    m, n_out = x.shape[0], w_q4k.shape[0]
+    y = np.full((m, n_out), np.nan, dtype=np.float32)
+    lib.oracle_q4k_linear_x86.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t, c_float_p,
+                                          C.c_void_p, c_float_p, C.c_int]
+    lib.oracle_q4k_linear_x86.restype = C.c_int
+    rc = lib.oracle_q4k_linear_x86(m, n_out, n_in, _fp(x), w_q4k.ctypes.data_as(C.c_void_p), _fp(y),
+                                   1 if avx512 else 0)
+    assert rc == 0, rc
+    return y
+
+
 Q4KX8_BLOCK_BYTES = 1152
+Q8KX4_BLOCK_BYTES = 1168     # struct block_q8_Kx4: d[4] float, qs[1024] int8, bsums[64] int16
 
 
 def load_ref_q4kgemv(fast=False):
@@ -654,6 +684,11 @@ def load_ref_q4kgemv(fast=False):
     lib.q4k_to_q4kx8_matrix.restype = None
     lib.q4kx8_gemv_m1.argtypes = [C.c_size_t, C.c_size_t, c_float_p, C.c_void_p, c_float_p]
     lib.q4kx8_gemv_m1.restype = None
+    lib.quantize_q8_Kx4.argtypes = [C.c_size_t, c_float_p, C.c_void_p]
+    lib.quantize_q8_Kx4.restype = None
+    lib.q4kx8_gemm_avx512.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
+                                      c_float_p]
+    lib.q4kx8_gemm_avx512.restype = None
     return lib
 
 
@@ -667,4 +702,26 @@ def ref_q4k_gemv_m1(ref, w_q4k, x, n_in):
     ref.q4k_to_q4kx8_matrix(n_in, n_out, w.ctypes.data_as(C.c_void_p), blob.ctypes.data_as(C.c_void_p))
     y = np.full(n_out, np.nan, dtype=np.float32)
     ref.q4kx8_gemv_m1(n_out, n_in, _fp(x), blob.ctypes.data_as(C.c_void_p), _fp(y))
+    return y
+
+
+def ref_q4k_linear_mN(ref, w_q4k, x, n_in):
+    """The reference's calls in the order of cpu_x86_linear_q4k_mN (linear_q4k.c:198-250): a row
+    count that is no multiple of 4 runs the decode kernel row by row; otherwise quantize_q8_Kx4 per
+    four rows, then q4kx8_gemm_avx512 over the interleaved table."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
+    m, n_out, ns = x.shape[0], w_q4k.shape[0], n_in // 256
+    assert n_out % 8 == 0 and n_in % 256 == 0
+    if m % 4 != 0:
+        return np.stack([ref_q4k_gemv_m1(ref, w_q4k, x[i], n_in) for i in range(m)])
+    blob = np.zeros(n_out // 8 * ns * Q4KX8_BLOCK_BYTES + 64, dtype=np.uint8)
+    w = np.ascontiguousarray(w_q4k)
+    ref.q4k_to_q4kx8_matrix(n_in, n_out, w.ctypes.data_as(C.c_void_p), blob.ctypes.data_as(C.c_void_p))
+    acts = np.zeros(m // 4 * ns * Q8KX4_BLOCK_BYTES + 64, dtype=np.uint8)
+    for mt in range(m // 4):
+        ref.quantize_q8_Kx4(n_in, _fp(x[4 * mt:4 * mt + 4]),
+                            C.c_void_p(acts.ctypes.data + mt * ns * Q8KX4_BLOCK_BYTES))
+    y = np.full((m, n_out), np.nan, dtype=np.float32)
+    ref.q4kx8_gemm_avx512(m, n_out, n_in, acts.ctypes.data_as(C.c_void_p),
+                          blob.ctypes.data_as(C.c_void_p), _fp(y))
     return y

@@ -1,8 +1,9 @@
 """The oracle's restatement of the x86 backend's Q4_K decode kernel (oracle_q4k_gemv_x86) against
 the reference's own q4k_to_q4kx8_matrix + q4kx8_gemv_m1, compiled from its tree
 (oracle/_ref/libgeist_ref_q4kgemv.so: kernel_q4kx8_gemm_avx512.c, kernel_q4kx8_gemm_scalar.c,
-q4k_to_q4kx8.c), bit for bit with strict flags; against golden vectors written from that build;
-and against what the definition fixes."""
+q4k_to_q4kx8.c), bit for bit with strict flags; the batch path (oracle_q4k_linear_x86) against
+quantize_q8_Kx4 + q4kx8_gemm_avx512 of the same build; against golden vectors written from that
+build; and against what the definition fixes."""
 import json
 import os
 
@@ -10,7 +11,8 @@ import numpy as np
 import pytest
 
 from oracle_lib import (load_oracle, load_ref_q4kgemv, oracle_dequant_q4k, oracle_q4k_gemv_x86,
-                        oracle_q8k_row_quantize, random_q4k_table, ref_q4k_gemv_m1)
+                        oracle_q4k_linear_x86, oracle_q8k_row_quantize, oracle_q8kx4_row_quantize,
+                        random_q4k_table, ref_q4k_gemv_m1, ref_q4k_linear_mN)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -96,6 +98,80 @@ def test_golden_vectors_of_the_reference(lib):
         x = np.frombuffer(bytes.fromhex(c["x_hex"]), dtype=np.float32).copy()
         y = np.frombuffer(bytes.fromhex(c["y_hex"]), dtype=np.float32)
         assert np.array_equal(oracle_q4k_gemv_x86(lib, w, x, n_in).view(np.uint32), y.view(np.uint32))
+
+
+def host_has_avx512():
+    try:
+        flags = open("/proc/cpuinfo").read()
+    except OSError:
+        return False
+    return all(f in flags for f in ("avx512f", "avx512bw", "avx512dq", "avx512vl"))
+
+
+def tie_rows(g, m, n_in, scale):
+    """Rows with activations exactly between two int8 values, where the decode kernel's quantiser
+    (half away from zero) and the batch quantiser (lrintf) part ways."""
+    x = (g.standard_normal((m, n_in)) * scale).astype(np.float32)
+    x[:, ::7] = 0.0
+    d = np.float32(2.0) ** np.ceil(np.log2(scale) - 3)   # the row's scale: a power of two,
+    x[:, 0] = np.float32(127.0) * d                      # so that the ties are exact
+    for k, h in enumerate((0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -126.5)):
+        x[:, 1 + k] = np.float32(h) * d
+    return x
+
+
+def test_batch_kernel_equals_the_compiled_reference(lib):
+    """cpu_x86_linear_q4k_mN's calls (quantize_q8_Kx4, q4kx8_gemm_avx512; the decode kernel row by
+    row for row counts that are no multiple of 4) against oracle_q4k_linear_x86, bit for bit. On
+    a host with AVX-512 the reference takes its 16 x 16 tiles where both counts are multiples of
+    16; elsewhere, and on other hosts, the AVX2 kernel."""
+    ref = load_ref_q4kgemv(False)
+    if ref is None:
+        pytest.skip("built only where the reference tree is mounted (make -C oracle ref)")
+    if os.environ.get("GEIST_FORCE_ISA"):
+        pytest.skip("GEIST_FORCE_ISA changes which of the reference's kernels runs")
+    avx512 = host_has_avx512()
+    g = np.random.default_rng(77)
+    for n_out, n_in, m in [(64, 512, 2), (64, 512, 3), (64, 512, 4), (48, 768, 8), (64, 256, 12),
+                           (64, 1024, 16), (72, 512, 16), (128, 512, 32), (64, 256, 20),
+                           (32, 16384, 4)]:
+        w = random_q4k_table(g, n_out, n_in)
+        for scale in (1e-3, 1.0, 100.0):
+            x = tie_rows(g, m, n_in, scale)
+            a = oracle_q4k_linear_x86(lib, w, x, n_in, avx512=avx512)
+            b = ref_q4k_linear_mN(ref, w, x, n_in)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (n_out, n_in, m, scale)
+            if m % 16 == 0 and n_out % 16 == 0:          # the two hosts give different bits
+                c = oracle_q4k_linear_x86(lib, w, x, n_in, avx512=not avx512)
+                assert not np.array_equal(a.view(np.uint32), c.view(np.uint32))
+
+
+def test_batch_quantiser_against_the_definition(lib):
+    g = np.random.default_rng(8)
+    x = tie_rows(g, 1, 768, 2.5)[0]
+    d, qs, bs = oracle_q8kx4_row_quantize(lib, x)
+    d1, qs1, _ = oracle_q8k_row_quantize(lib, x)
+    assert np.float32(d) == np.float32(np.abs(x).max()) / np.float32(127.0) == np.float32(d1)
+    assert np.float32(d) == np.float32(0.5)
+    v = (x * (np.float32(1.0) / np.float32(d))).astype(np.float32)
+    assert np.array_equal(qs, np.rint(v).astype(np.int8))           # ties to even
+    assert np.array_equal(bs, qs.reshape(-1, 16).astype(np.int32).sum(1).astype(np.int16))
+    # the ties: 0.5 -> 0 here and 1 in the decode kernel, 2.5 -> 2 and 3, 1.5 -> 2 in both
+    assert list(qs[1:9]) == [0, 2, 2, 0, -2, -2, 64, -126]
+    assert list(qs1[1:9]) == [1, 2, 3, -1, -2, -3, 64, -127]
+
+
+def test_golden_batches_of_the_reference(lib):
+    with open(os.path.join(HERE, "golden", "q4k_x86_ref_vectors.json")) as f:
+        cases = json.load(f)["batch_cases"]
+    assert len(cases) >= 6 and any(c["tiles"] for c in cases)
+    for c in cases:
+        n_out, n_in, m = c["n_out"], c["n_in"], c["m"]
+        w = np.frombuffer(bytes.fromhex(c["w_hex"]), dtype=np.uint8).reshape(n_out, -1).copy()
+        x = np.frombuffer(bytes.fromhex(c["x_hex"]), dtype=np.float32).reshape(m, n_in).copy()
+        y = np.frombuffer(bytes.fromhex(c["y_hex"]), dtype=np.float32).reshape(m, n_out)
+        got = oracle_q4k_linear_x86(lib, w, x, n_in, avx512=True)   # written on an AVX-512 host
+        assert np.array_equal(got.view(np.uint32), y.view(np.uint32)), (n_out, n_in, m)
 
 
 def test_shapes_the_kernel_does_not_take(lib):
