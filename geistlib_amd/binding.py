@@ -122,6 +122,7 @@ def load_library():
     lib.geist_hip_q6k_packed_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q6k_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q4k_packed_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q4k_packed_linear_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q8k_act_bytes.argtypes = [sz, sz]
     lib.geist_hip_q8k_act_bytes.restype = sz
     lib.geist_hip_q8k_quantize_rows.argtypes = [vp, vp, sz, sz, sz, vp]
@@ -370,8 +371,9 @@ class HipSampler:
             y.stride(0) if m > 1 else n_out))
 
     def set_projection(self, portable):
-        """Which reference backend project_sample's F16 projection stands for (False: x86)."""
-        self._check(self.lib.geist_hip_sampler_set_projection(self.h, 1 if portable else 0))
+        """Which reference backend project_sample's projection stands for: False / 0 the x86
+        backend (on a host with AVX-512), True / 1 the portable one, 2 x86 without AVX-512."""
+        self._check(self.lib.geist_hip_sampler_set_projection(self.h, int(portable)))
 
     def f16_linear(self, w_f16, x, y):
         """As f16_gemv in the portable kernel's arithmetic: the sum in double, rounded once."""
@@ -427,6 +429,14 @@ class HipSampler:
         """The x86 backend's integer decode kernel over the packed Q4_K copy, row by row."""
         m = x.shape[0]
         self._check(self.lib.geist_hip_q4k_packed_gemv_x86_rows(
+            self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def q4k_packed_linear_x86(self, packed, n_out, n_in, x, y):
+        """The x86 backend's projection of a batch over the packed Q4_K copy
+        (cpu_x86_linear_q4k_mN; one row: the decode kernel)."""
+        m = x.shape[0]
+        self._check(self.lib.geist_hip_q4k_packed_linear_x86_rows(
             self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 

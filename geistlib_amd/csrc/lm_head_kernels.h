@@ -59,7 +59,8 @@ struct Q6KScratch {
     double *xabs;      /* [Q6K_M_MAX][n_in / 16] the sums of their magnitudes */
     int    *amb_count; /* outputs whose rounding depends on the order of the sum ... */
     int2   *amb_list;  /* ... [n_out * Q6K_M_MAX] (table row, activation row) */
-    uint32_t *act8;    /* [n_in / 256][Q8K_ACT_DWORDS] one row's activations as int8 (x86 decode) */
+    uint32_t *act8;    /* activations as int8 for the x86 kernels: one row of [n_in / 256][Q8K_ACT_DWORDS]
+                        * (Q6_K) or Q4X_M_MAX rows of q4k_x86_act_dwords (Q4_K) */
 };
 /* One super-block of int8 activations: 64 dwords of four int8 each in element order, sixteen
  * int32 sums per group of sixteen, the scale d_a (binary32 bits), padding. */
@@ -93,20 +94,27 @@ void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_o
 /* ... and over the table as it lies in the file (4-byte aligned). */
 void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
                          const uint32_t *act, float *y);
-/* The x86 backend's decode kernel over a Q4_K table (q4kx8_gemv_m1,
- * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c) over the packed copy (lm_head_q4k_x86.hip):
- * the activations of n_m rows as int8 with one scale per row (act: per row n_in / 256 *
- * Q4X_ACT_DWORDS + 1 dwords), and one row's integer dot products with binary32 accumulation in
- * the reference's order. */
+/* The x86 backend's kernels over a Q4_K table -- the decode kernel q4kx8_gemv_m1
+ * (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c) and the batch path of
+ * cpu_x86_linear_q4k_mN (linear_q4k.c:198-250) -- over the packed copy (lm_head_q4k_x86.hip):
+ * the activations of n_m rows as int8 with one scale per row (act: per row
+ * q4k_x86_act_dwords(n_in) dwords; ties_even: the batch quantiser quantize_q8_Kx4 instead of the
+ * decode kernel's), and the integer dot products of n_m <= Q4X_M_MAX rows in one pass over the
+ * table, with binary32 accumulation in the reference's order (pairs: that of its 16 x 16
+ * AVX-512 tiles, once per pair of sub-blocks). */
 constexpr int Q4X_ACT_DWORDS = 72; /* 64 of int8 (even / odd elements of every eight), 8 sums */
+constexpr int Q4X_ACT_TAIL   = 8;  /* the row's scale, and padding to 32 bytes */
+constexpr int Q4X_M_MAX      = 8;
+constexpr int Q4X_M_MAX_PAIRS = 4; /* with pairs: fewer rows per pass (registers) */
 size_t q4k_x86_act_dwords(int n_in);
 void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
-                             uint32_t *act);
+                             bool ties_even, uint32_t *act);
 /* launch_rmsnorm_rows and that quantiser in one launch (n a multiple of 256) */
 void launch_rmsnorm_q8k_row_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
-                                 float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act);
+                                 float eps, int n_rows, int n, float *y, long ld_y, bool ties_even,
+                                 uint32_t *act);
 void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
-                                const uint32_t *act, float *y);
+                                const uint32_t *act, int n_m, bool pairs, float *y, long ld_y);
 /* The same for a Q4_K table (packed form only; 148 bytes per block of 144): n_in a multiple of
  * 256, the table 4-byte aligned. The scratch is the Q6_K projection's. */
 size_t q4k_packed_bytes(long n_out, int n_in);

@@ -37,11 +37,15 @@ constexpr int Q4X_PACK_DWORDS = Q4X_ROW_DWORDS * 64; /* the packed copy's dwords
 
 /* Thread t's element of a super-block, given the reciprocal of the row's scale: its int8 value
  * into the block's dwords (ob), the sums per sub-block of 32 behind them. */
-__device__ __forceinline__ void q4x_quantize_block(float xv, float inv, uint32_t *__restrict__ ob) {
+__device__ __forceinline__ void q4x_quantize_block(float xv, float inv, bool ties_even,
+                                                   uint32_t *__restrict__ ob) {
     const int   t = threadIdx.x;
     const float v = __fmul_rn(xv, inv);
-    int         q = __float2int_rz(v < 0.0f ? __fsub_rn(v, 0.5f) : __fadd_rn(v, 0.5f));
-    q             = q < -128 ? -128 : q > 127 ? 127 : q;
+    /* the decode kernel's quantiser rounds half away from zero by truncation and clamps; the
+     * batch quantiser is lrintf (|v| <= 127 up to rounding: nothing to clamp) */
+    int q = ties_even ? __float2int_rn(v)
+                      : __float2int_rz(v < 0.0f ? __fsub_rn(v, 0.5f) : __fadd_rn(v, 0.5f));
+    q     = q < -128 ? -128 : q > 127 ? 127 : q;
     int sum       = q;
 #pragma unroll
     for (int s = 16; s >= 1; s >>= 1)
@@ -56,15 +60,18 @@ __device__ __forceinline__ void q4x_quantize_block(float xv, float inv, uint32_t
         ob[64 + (t >> 5)] = (uint32_t) sum;
 }
 
-/* One workgroup per activation row. act: per super-block Q4X_ACT_DWORDS dwords -- 64 of int8 (per
- * eight elements the even ones, then the odd ones), eight int32 sums per sub-block of 32 --, and
- * behind the row's last block the scale d_a as binary32. */
+/* One workgroup per activation row. act: per row q4k_x86_act_dwords dwords: per super-block
+ * Q4X_ACT_DWORDS -- 64 of int8 (per eight elements the even ones, then the odd ones), eight
+ * int32 sums per sub-block of 32 --, and behind the row's last block the scale d_a as binary32
+ * (and padding that keeps the next row 32-byte aligned). ties_even: the batch quantiser
+ * (quantize_q8_Kx4, q8_kx4.c:21-105) instead of the decode kernel's. */
 __global__ __launch_bounds__(Q4X_TPB) void k_q8k_row_quantize(const float *__restrict__ x, long ld_x,
-                                                             int nb, uint32_t *__restrict__ act) {
+                                                             int nb, bool ties_even,
+                                                             uint32_t *__restrict__ act) {
     __shared__ float s_max[Q4X_TPB / 64];
     const int        m = blockIdx.x, t = threadIdx.x;
     const float     *xr = x + (long) m * ld_x;
-    uint32_t        *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + 1);
+    uint32_t        *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + Q4X_ACT_TAIL);
     float            ax = 0.0f;
     for (int b = 0; b < nb; ++b)
         ax = __builtin_fmaxf(ax, __builtin_fabsf(xr[256 * b + t])); /* (a NaN is passed over) */
@@ -81,7 +88,7 @@ __global__ __launch_bounds__(Q4X_TPB) void k_q8k_row_quantize(const float *__res
     if (t == 0)
         o[(long) nb * Q4X_ACT_DWORDS] = __float_as_uint(scale);
     for (int b = 0; b < nb; ++b)
-        q4x_quantize_block(xr[256 * b + t], inv, o + (long) b * Q4X_ACT_DWORDS);
+        q4x_quantize_block(xr[256 * b + t], inv, ties_even, o + (long) b * Q4X_ACT_DWORDS);
 }
 
 /* The output norm (cpu_scalar_rmsnorm, as k_rmsnorm_rows computes it) and that quantiser in one
@@ -92,6 +99,7 @@ __global__ __launch_bounds__(Q4X_TPB) void k_rmsnorm_q8k_row_rows(const float *_
                                                                  const float *__restrict__ w,
                                                                  float eps, int n,
                                                                  float *__restrict__ y, long ld_y,
+                                                                 bool ties_even,
                                                                  uint32_t *__restrict__ act) {
     __shared__ double s_part[Q4X_TPB];
     __shared__ float  s_inv;
@@ -99,7 +107,7 @@ __global__ __launch_bounds__(Q4X_TPB) void k_rmsnorm_q8k_row_rows(const float *_
     const int    nb = n / 256, m = blockIdx.x, t = threadIdx.x;
     const float *xr = x + (long) m * ld_x;
     float       *yr = y + (long) m * ld_y;
-    uint32_t    *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + 1);
+    uint32_t    *o  = act + (long) m * ((long) nb * Q4X_ACT_DWORDS + Q4X_ACT_TAIL);
     const float  rinv = block_rms_inv<Q4X_TPB>(xr, n, eps, s_part, &s_inv);
     float        ax = 0.0f;
     for (int b = 0; b < nb; ++b) {
@@ -121,7 +129,7 @@ __global__ __launch_bounds__(Q4X_TPB) void k_rmsnorm_q8k_row_rows(const float *_
     if (t == 0)
         o[(long) nb * Q4X_ACT_DWORDS] = __float_as_uint(scale);
     for (int b = 0; b < nb; ++b)
-        q4x_quantize_block(yr[256 * b + t], inv, o + (long) b * Q4X_ACT_DWORDS);
+        q4x_quantize_block(yr[256 * b + t], inv, ties_even, o + (long) b * Q4X_ACT_DWORDS);
 }
 
 typedef uint32_t q4x_u4 __attribute__((ext_vector_type(4)));
@@ -145,17 +153,26 @@ __device__ __forceinline__ void q4x_load(const uint32_t *__restrict__ base, int 
     k.dd    = __builtin_nontemporal_load(base + 2304 + r);
 }
 
+/* M activation rows share a pass over the table. PAIRS: the binary32 accumulators are joined once
+ * per pair of sub-blocks (the reference's 16 x 16 AVX-512 tiles,
+ * kernel_q4kx8_gemm_avx512_full.c:94, 729-778) instead of once per super-block. */
+template <int M, bool PAIRS>
 __global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
     const uint32_t *__restrict__ packed, long n_out, int nb, const uint32_t *__restrict__ act,
-    float *__restrict__ y) {
+    float *__restrict__ y, long ld_y) {
     const int  r = threadIdx.x & 63;
     const long g = (long) blockIdx.x * (Q4X_TPB / 64) + threadIdx.x / 64;
     if (g * 64 >= n_out)
         return;
-    const long      row  = g * 64 + r;
-    const uint32_t *base = packed + g * nb * Q4X_PACK_DWORDS;
-    const float     d_a  = __uint_as_float(act[(long) nb * Q4X_ACT_DWORDS]);
-    float           acc = 0.0f, acc_min = 0.0f;
+    const long      row    = g * 64 + r;
+    const uint32_t *base   = packed + g * nb * Q4X_PACK_DWORDS;
+    const long      act_ld = (long) nb * Q4X_ACT_DWORDS + Q4X_ACT_TAIL;
+    float           d_a[M], acc[M], acc_min[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        d_a[m] = __uint_as_float(act[m * act_ld + (long) nb * Q4X_ACT_DWORDS]);
+        acc[m] = 0.0f, acc_min[m] = 0.0f;
+    }
     /* a block ahead: the next block's loads are in flight while this one is worked on */
     Q4xBlock cur, nxt;
     q4x_load(base, r, cur);
@@ -164,53 +181,129 @@ __global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
             q4x_load(base + (long) (b + 1) * Q4X_PACK_DWORDS, r, nxt);
         const uint32_t *a = act + (long) b * Q4X_ACT_DWORDS; /* uniform: scalar loads */
         typedef uint32_t u8v __attribute__((ext_vector_type(8)));
-        const u8v bs = *reinterpret_cast<const u8v *>(a + 64);
-        int       iacc = 0, iacc_min = 0;
+        const float d    = __half2float(__ushort_as_half((unsigned short) (cur.dd & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short) (cur.dd >> 16)));
+        int         iacc[M], iacc_min[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            iacc[m] = 0, iacc_min[m] = 0;
+        /* With several rows the scalar loads of a sub-block stay next to its arithmetic, four
+         * rows at a time: a fence that the loads may not pass and that needs the sums so far.
+         * Hoisted to the top of the block they would not fit the scalar registers. */
+        if (!PAIRS) { /* the minima against the activations' sums per sub-block */
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                if (M > 4 && m % 4 == 0)
+                    asm volatile("" : "+v"(acc_min[m > 0 ? m - 1 : 0])::"memory");
+                const u8v bs = *reinterpret_cast<const u8v *>(a + m * act_ld + 64);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    iacc_min[m] += __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu), (int) bs[j]);
+                acc_min[m] = __builtin_fmaf((float) iacc_min[m], __fmul_rn(dmin, d_a[m]), acc_min[m]);
+            }
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) { /* sub-block j: elements 32 j .. 32 j + 31, dwords 4 j .. */
-            const u8v av  = *reinterpret_cast<const u8v *>(a + 8 * j);
-            int       dot = 0;
+            uint32_t even[4], odd[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const uint32_t w = cur.q[4 * j + k];
-                dot = __builtin_amdgcn_sdot4((int) (w & 0x0f0f0f0fu), (int) av[2 * k], dot, false);
-                dot = __builtin_amdgcn_sdot4((int) ((w >> 4) & 0x0f0f0f0fu), (int) av[2 * k + 1],
-                                             dot, false);
+                even[k] = w & 0x0f0f0f0fu, odd[k] = (w >> 4) & 0x0f0f0f0fu;
             }
             const int sc = (int) ((cur.sc[j >> 2] >> (8 * (j & 3))) & 0xffu);
-            const int mn = (int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu);
-            iacc += __mul24(sc, dot);
-            iacc_min += __mul24(mn, (int) bs[j]);
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                if (M > 1 && m % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < M; ++i)
+                        asm volatile("" : "+v"(iacc[i])::"memory");
+                }
+                const u8v av  = *reinterpret_cast<const u8v *>(a + m * act_ld + 8 * j);
+                int       dot = 0;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    dot = __builtin_amdgcn_sdot4((int) even[k], (int) av[2 * k], dot, false);
+                    dot = __builtin_amdgcn_sdot4((int) odd[k], (int) av[2 * k + 1], dot, false);
+                }
+                iacc[m] += __mul24(sc, dot);
+                if (PAIRS && !(j & 1)) { /* the pair's minima */
+                    typedef uint32_t u2v __attribute__((ext_vector_type(2)));
+                    const u2v bs = *reinterpret_cast<const u2v *>(a + m * act_ld + 64 + j);
+                    iacc_min[m] =
+                        __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu), (int) bs[0]) +
+                        __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3) + 8)) & 0xffu), (int) bs[1]);
+                }
+            }
+            if (PAIRS && (j & 1)) {
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    acc[m]     = __builtin_fmaf((float) iacc[m], __fmul_rn(d, d_a[m]), acc[m]);
+                    acc_min[m] = __builtin_fmaf((float) iacc_min[m], __fmul_rn(dmin, d_a[m]),
+                                                acc_min[m]);
+                    iacc[m] = 0;
+                }
+            }
         }
-        const float d    = __half2float(__ushort_as_half((unsigned short) (cur.dd & 0xffffu)));
-        const float dmin = __half2float(__ushort_as_half((unsigned short) (cur.dd >> 16)));
-        acc     = __builtin_fmaf((float) iacc, __fmul_rn(d, d_a), acc);
-        acc_min = __builtin_fmaf((float) iacc_min, __fmul_rn(dmin, d_a), acc_min);
+        if (!PAIRS) {
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+                acc[m] = __builtin_fmaf((float) iacc[m], __fmul_rn(d, d_a[m]), acc[m]);
+        }
         if (b + 1 < nb)
             cur = nxt;
     }
-    if (row < n_out)
-        y[row] = __fsub_rn(acc, acc_min);
+    if (row < n_out) {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            y[m * ld_y + row] = __fsub_rn(acc[m], acc_min[m]);
+    }
 }
 
-size_t q4k_x86_act_dwords(int n_in) { return (size_t) (n_in / 256) * Q4X_ACT_DWORDS + 1; }
+size_t q4k_x86_act_dwords(int n_in) {
+    return (size_t) (n_in / 256) * Q4X_ACT_DWORDS + Q4X_ACT_TAIL;
+}
 
 void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
-                             uint32_t *act) {
-    k_q8k_row_quantize<<<dim3(n_m), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, n_in / 256, act);
+                             bool ties_even, uint32_t *act) {
+    k_q8k_row_quantize<<<dim3(n_m), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, n_in / 256, ties_even, act);
 }
 
 void launch_rmsnorm_q8k_row_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
-                                 float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act) {
+                                 float eps, int n_rows, int n, float *y, long ld_y, bool ties_even,
+                                 uint32_t *act) {
     k_rmsnorm_q8k_row_rows<<<dim3(n_rows), dim3(Q4X_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y,
-                                                                      act);
+                                                                      ties_even, act);
+}
+
+template <int M>
+static void q4x_launch(hipStream_t stream, const uint32_t *packed, long n_out, int nb,
+                       const uint32_t *act, bool pairs, float *y, long ld_y) {
+    const long groups = (n_out + 63) / 64;
+    const dim3 grid((unsigned) ((groups + 3) / 4)), block(Q4X_TPB);
+    if constexpr (M <= Q4X_M_MAX_PAIRS) {
+        if (pairs) {
+            k_q4k_packed_gemv_x86<M, true><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y,
+                                                                      ld_y);
+            return;
+        }
+    }
+    k_q4k_packed_gemv_x86<M, false><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y, ld_y);
 }
 
 void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,
-                                const uint32_t *act, float *y) {
-    const long groups = (n_out + 63) / 64;
-    k_q4k_packed_gemv_x86<<<dim3((unsigned) ((groups + 3) / 4)), dim3(Q4X_TPB), 0, stream>>>(
-        static_cast<const uint32_t *>(packed), n_out, n_in / 256, act, y);
+                                const uint32_t *act, int n_m, bool pairs, float *y, long ld_y) {
+    const uint32_t *p  = static_cast<const uint32_t *>(packed);
+    const int       nb = n_in / 256;
+    switch (n_m) {
+    case 1: q4x_launch<1>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 2: q4x_launch<2>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 3: q4x_launch<3>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 4: q4x_launch<4>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 5: q4x_launch<5>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 6: q4x_launch<6>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    case 7: q4x_launch<7>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    default: q4x_launch<8>(stream, p, n_out, nb, act, pairs, y, ld_y); break;
+    }
 }
 
 } // namespace gs

@@ -99,6 +99,7 @@ struct geist_hip_sampler {
     size_t topk_paths_rows  = 0;     /* rows of the last top-k call that took the candidate path */ /* see geist_hip_sampler_time_stream_kernel */
     bool logits_streamed    = false; /* see geist_hip_sampler_set_logits_hint */
     bool projection_portable = false; /* see geist_hip_sampler_set_projection */
+    bool projection_avx2     = false; /* the x86 backend on a host without AVX-512 */
     bool tmax_ready         = false; /* the projection has written the top-k scan's thread maxima
                                         for the rows about to be sampled */
 
@@ -437,9 +438,11 @@ int geist_hip_sampler_set_logits_hint(geist_hip_sampler *s, int hint) {
 int geist_hip_sampler_set_projection(geist_hip_sampler *s, int mode) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
-    if (mode != GEIST_HIP_PROJECTION_X86 && mode != GEIST_HIP_PROJECTION_PORTABLE)
+    if (mode != GEIST_HIP_PROJECTION_X86 && mode != GEIST_HIP_PROJECTION_PORTABLE &&
+        mode != GEIST_HIP_PROJECTION_X86_AVX2)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "unknown projection mode %d", mode);
     s->projection_portable = mode == GEIST_HIP_PROJECTION_PORTABLE;
+    s->projection_avx2     = mode == GEIST_HIP_PROJECTION_X86_AVX2;
     return GEIST_HIP_OK;
 }
 
@@ -1241,6 +1244,13 @@ static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t
 
 /* Scratch of the Q6_K projection: the activations in double, their sums and magnitudes per
  * group of 16, the list of outputs for the second kernel. */
+/* the int8 activations of the x86 kernels: one row for Q6_K, Q4X_M_MAX rows for Q4_K */
+static size_t q8_act_bytes(size_t n_in) {
+    const size_t q6 = (n_in / 256) * Q8K_ACT_DWORDS;
+    const size_t q4 = (size_t) Q4X_M_MAX * ((n_in / 256) * Q4X_ACT_DWORDS + Q4X_ACT_TAIL);
+    return (q6 > q4 ? q6 : q4) * sizeof(uint32_t);
+}
+
 static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScratch &ws) {
     if (s->q6k_in < n_in || s->q6k_out < n_out) {
         if (s->q6k_ws) {
@@ -1252,7 +1262,7 @@ static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScrat
         const size_t out = n_out > s->q6k_out ? n_out : s->q6k_out;
         const size_t bytes = (size_t) Q6K_M_MAX * (in + in / 8) * sizeof(double) + 16 +
                              out * Q6K_M_MAX * sizeof(int2) +
-                             (in / 256) * Q8K_ACT_DWORDS * sizeof(uint32_t);
+                             q8_act_bytes(in);
         if (hipMalloc(&s->q6k_ws, bytes) != hipSuccess) {
             s->q6k_ws = nullptr;
             return fail(s, GEIST_HIP_E_OOM, "Q6_K projection: scratch");
@@ -1505,43 +1515,64 @@ static bool q4k_x86_shape(size_t n_out, size_t n_in) {
     return n_out % 8 == 0 && n_in % 256 == 0 && n_in / 256 >= 1 && n_in / 256 <= 64;
 }
 
-static int q4k_packed_gemv_x86_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
-                                    size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
-                                    float *d_y, size_t ld_y) {
-    Q6KScratch ws; /* (its int8 activation area: 96 dwords per super-block, 73 needed) */
+/* batch: the rows are one call of cpu_x86_linear_q4k_mN (linear_q4k.c:198-250) -- a row count
+ * that is a multiple of 4 takes the batch quantiser, a multiple of 16 over 16 n table rows the
+ * arithmetic of the AVX-512 tiles unless the host reproduced has none; otherwise every row is a
+ * call of the decode kernel. Q4X_M_MAX rows share a pass over the table. */
+static int q4k_packed_x86_impl(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                               size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                               float *d_y, size_t ld_y, bool batch) {
+    Q6KScratch ws;
     const int  rc = q6k_scratch(s, n_out, n_in, ws);
     if (rc)
         return rc;
-    for (size_t m = 0; m < n_rows; ++m) {
-        launch_q8k_row_quantize(s->stream, d_x + m * ld_x, (long) ld_x, 1, (int) n_in, ws.act8);
-        launch_q4k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in, ws.act8,
-                                   d_y + m * ld_y);
+    const bool kx4   = batch && n_rows > 1 && n_rows % 4 == 0;
+    const bool pairs = kx4 && !s->projection_avx2 && n_rows % 16 == 0 && n_out % 16 == 0;
+    const size_t tile = pairs ? Q4X_M_MAX_PAIRS : Q4X_M_MAX;
+    for (size_t m0 = 0; m0 < n_rows; m0 += tile) {
+        const size_t m = n_rows - m0 < tile ? n_rows - m0 : tile;
+        launch_q8k_row_quantize(s->stream, d_x + m0 * ld_x, (long) ld_x, (int) m, (int) n_in, kx4,
+                                ws.act8);
+        launch_q4k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in, ws.act8, (int) m,
+                                   pairs, d_y + m0 * ld_y, (long) ld_y);
     }
     return GEIST_HIP_OK;
 }
 
-int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
-                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
-                                       float *d_y, size_t ld_y) {
+static int q4k_packed_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                               size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                               float *d_y, size_t ld_y, bool batch) {
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     if (!d_packed || !d_x || !d_y)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
     if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
-        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K decode: %zu rows, strides %zu / %zu", n_rows,
-                    ld_x, ld_y);
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K x86 kernels: %zu rows, strides %zu / %zu",
+                    n_rows, ld_x, ld_y);
     int rc = q6k_check(s, d_packed, n_out, n_in);
     if (rc)
         return rc;
     if (!q4k_x86_shape(n_out, n_in))
         return fail(s, GEIST_HIP_E_UNSUPPORTED,
-                    "Q4_K decode: %zu x %zu is not a shape of the x86 kernel (rows in eights, at "
+                    "Q4_K x86 kernels: %zu x %zu is not a shape they take (rows in eights, at "
                     "most 64 super-blocks per row)", n_out, n_in);
     if (((uintptr_t) d_packed) % 16 != 0)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q4_K table not 16-byte aligned");
     HIPCHK(s, hipSetDevice(s->device));
-    rc = q4k_packed_gemv_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
-    return rc ? rc : after_launch(s, "Q4_K decode (packed)");
+    rc = q4k_packed_x86_impl(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y, batch);
+    return rc ? rc : after_launch(s, "Q4_K x86 kernels (packed)");
+}
+
+int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                       size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                       float *d_y, size_t ld_y) {
+    return q4k_packed_x86_rows(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y, false);
+}
+
+int geist_hip_q4k_packed_linear_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                         size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                         float *d_y, size_t ld_y) {
+    return q4k_packed_x86_rows(s, d_packed, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y, true);
 }
 
 size_t geist_hip_q8k_row_act_bytes(size_t n_in) {
@@ -1563,7 +1594,7 @@ int geist_hip_q8k_row_quantize(geist_hip_sampler *s, const float *d_x, size_t n_
     if (((uintptr_t) d_act) % 64 != 0)
         return fail(s, GEIST_HIP_E_INVALID_ARG, "int8 activation row: buffer not 64-byte aligned");
     HIPCHK(s, hipSetDevice(s->device));
-    launch_q8k_row_quantize(s->stream, d_x, (long) n_in, 1, (int) n_in,
+    launch_q8k_row_quantize(s->stream, d_x, (long) n_in, 1, (int) n_in, false,
                             static_cast<uint32_t *>(d_act));
     return after_launch(s, "int8 activation row");
 }
@@ -1585,7 +1616,7 @@ int geist_hip_q4k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, si
         return fail(s, GEIST_HIP_E_INVALID_ARG, "Q4_K decode: table or activations misaligned");
     HIPCHK(s, hipSetDevice(s->device));
     launch_q4k_packed_gemv_q8k(s->stream, d_packed, (long) n_out, (int) n_in,
-                               static_cast<const uint32_t *>(d_act), d_y);
+                               static_cast<const uint32_t *>(d_act), 1, false, d_y, (long) n_out);
     return after_launch(s, "Q4_K decode (packed)");
 }
 
@@ -1748,12 +1779,14 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
      * (q6k_gemv_m1), whose activation quantiser rides on the norm's launch */
     const bool q6k_x86 = (table == TABLE_Q6K_PACKED || table == TABLE_Q6K) && rows == 1 &&
                          !s->projection_portable;
-    /* ... and over a packed Q4_K table of a shape that backend's decode kernel takes
-     * (q4kx8_gemv_m1), likewise */
-    const bool q4k_x86 = table == TABLE_Q4K_PACKED && rows == 1 && !s->projection_portable &&
-                         q4k_x86_shape(n_vocab, d_model);
+    /* ... and over a packed Q4_K table of a shape that backend's kernels take: one row likewise
+     * (q4kx8_gemv_m1), a batch as cpu_x86_linear_q4k_mN projects it */
+    const bool q4k_x86  = table == TABLE_Q4K_PACKED && !s->projection_portable &&
+                          q4k_x86_shape(n_vocab, d_model);
+    const bool q4k_kx4   = q4k_x86 && rows > 1 && rows % 4 == 0;
+    const bool q4k_fused = q4k_x86 && rows <= (size_t) Q4X_M_MAX;
     Q6KScratch q6ws{};
-    if (q6k_x86 || q4k_x86) {
+    if (q6k_x86 || q4k_fused) {
         if ((rc = q6k_scratch(s, n_vocab, d_model, q6ws)) != GEIST_HIP_OK)
             return rc;
         if (q6k_x86)
@@ -1761,8 +1794,8 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
                                     1, (int) d_model, d_normed, (long) d_model, q6ws.act8);
         else
             launch_rmsnorm_q8k_row_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight,
-                                        rms_eps, 1, (int) d_model, d_normed, (long) d_model,
-                                        q6ws.act8);
+                                        rms_eps, (int) rows, (int) d_model, d_normed,
+                                        (long) d_model, q4k_kx4, q6ws.act8);
     } else {
         launch_rmsnorm_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
                             (int) rows, (int) d_model, d_normed, (long) d_model);
@@ -1784,9 +1817,14 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_embed), (long) n_vocab,
                                 (int) d_model, q6ws.act8, d_logits);
-    } else if (q4k_x86) {
+    } else if (q4k_fused) {
+        /* (at most 8 rows: never the AVX-512 tiles' arithmetic) */
         launch_q4k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,
-                                   d_logits);
+                                   (int) rows, false, d_logits, (long) ld_logits);
+    } else if (q4k_x86) {
+        if ((rc = q4k_packed_x86_impl(s, d_embed, n_vocab, d_model, d_normed, d_model, rows,
+                                      d_logits, ld_logits, true)) != GEIST_HIP_OK)
+            return rc;
     } else if (q6k) {
         /* the portable kernel after dequant_q6_K_row, for one row and for a batch */
         rc = table == TABLE_Q4K_PACKED

@@ -92,8 +92,8 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
                                     size_t ld_hidden, size_t k, const float *d_norm_weight,
                                     float rms_eps, const uint16_t *d_embed_f16, size_t d_model,
                                     int32_t *out_tokens);
-/* GEIST_HIP_PROJECTION_X86 (default) or _PORTABLE (include/geist_lm_head_hip.h): which backend's
- * arithmetic geist_hip_head_project_finalize uses for one row. */
+/* GEIST_HIP_PROJECTION_X86 (default), _PORTABLE or _X86_AVX2 (include/geist_lm_head_hip.h): which
+ * backend's arithmetic the project_finalize calls use. */
 int geist_hip_head_set_projection(struct geist_hip_head *h, int mode);
 /* The same over the int8 form of the table, which the reference's x86 backend substitutes for
  * the F16 table in a decode step (src/backends/cpu_x86/backend.c:332-372): d_embed_q8 [vocab,
@@ -141,11 +141,12 @@ int geist_hip_head_q6k_load(struct geist_hip_head *h, const void *d_embed_q6k, s
  * kernel. The logits equal, bit for bit, those of the portable kernel cpu_scalar_w_quant_m1 /
  * _mN after dequant_q4_K_row (src/formats/gguf/q4_K.c:18-49, weight_resolve.c:82-83, 186-241),
  * for one row and for a batch. Unless geist_hip_head_set_projection chose the portable backend,
- * one row over a vocabulary of a multiple of 8 tokens (d_model <= 16384) gets the logits of the
- * x86 backend's decode kernel q4kx8_gemv_m1 instead (int8 activations, integer dot products:
- * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c, from src/backends/cpu_x86/linear_q4k.c:163-166),
- * again bit for bit. That backend's batch kernels and its W4A8 kernels for other shapes, and
- * the NEON backend's kernels, are not reproduced. */
+ * a vocabulary of a multiple of 8 tokens (d_model <= 16384) gets the logits of the x86 backend
+ * instead (int8 activations, integer dot products): one row those of its decode kernel
+ * q4kx8_gemv_m1 (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c, from
+ * src/backends/cpu_x86/linear_q4k.c:163-166), a batch those of cpu_x86_linear_q4k_mN
+ * (linear_q4k.c:198-250; see geist_hip_q4k_packed_linear_x86_rows), again bit for bit. That
+ * backend's W4A8 kernels for other shapes, and the NEON backend's kernels, are not reproduced. */
 int geist_hip_head_project_finalize_q4k(struct geist_hip_head *h, const float *d_hidden,
                                         size_t ld_hidden, size_t k, const float *d_norm_weight,
                                         float rms_eps, const void *d_embed_q4k, size_t d_model,

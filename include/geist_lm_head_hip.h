@@ -55,13 +55,20 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
 /* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
  * the head's project_finalize calls) stands for:
  *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a Q6_K table q6k_gemv_m1, over a
- *                                  packed Q4_K table q4kx8_gemv_m1;
- *                                  more rows: the portable kernel (default)
+ *                                  packed Q4_K table q4kx8_gemv_m1; more rows: over a packed
+ *                                  Q4_K table cpu_x86_linear_q4k_mN as a host with AVX-512 runs
+ *                                  it, over the other tables the portable kernel (default)
  *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
  *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
- *                                  linear_m1 and linear_mN alike) */
+ *                                  linear_m1 and linear_mN alike)
+ *   GEIST_HIP_PROJECTION_X86_AVX2  as _X86, for a host without AVX-512 (or one run with
+ *                                  GEIST_FORCE_ISA=avx2): the only difference is a Q4_K batch of
+ *                                  a multiple of 16 rows, which such a host sends through its AVX2
+ *                                  kernel instead of the 16 x 16 tiles
+ *                                  (kernel_q4kx8_gemm_avx512_full.c:816-835) */
 #define GEIST_HIP_PROJECTION_X86 0
 #define GEIST_HIP_PROJECTION_PORTABLE 1
+#define GEIST_HIP_PROJECTION_X86_AVX2 2
 int geist_hip_sampler_set_projection(geist_hip_sampler *s, int mode);
 
 /* The int8 form of the tied table, which the reference's x86 backend uses for the lm_head unless
@@ -231,19 +238,35 @@ int geist_hip_q4k_packed_linear_rows(geist_hip_sampler *s, const void *d_packed,
  * activations' sums; per super-block each of the two integers joins a binary32 accumulator by a
  * fused multiply-add, and the result is the difference of the accumulators. For the shapes that
  * kernel takes -- n_out a multiple of 8, n_in / 256 <= 64 -- and GEIST_HIP_E_UNSUPPORTED for
- * others (the reference sends those through its W4A8 kernels, which are not reproduced). Each
- * activation row is a pass of its own over the table. Activations must be finite.
+ * others (the reference sends those through its W4A8 kernels, which are not reproduced). Every
+ * row gets the decode kernel's result; up to four rows share a pass over the table. Activations
+ * must be finite.
+ *
+ * geist_hip_q4k_packed_linear_x86_rows replaces cpu_x86_linear_q4k_mN
+ * (src/backends/cpu_x86/linear_q4k.c:198-250) for n_rows > 1, and the decode kernel for one row:
+ * a row count that is no multiple of 4 is the decode kernel row by row (:222-229); a multiple of
+ * 4 is quantised by quantize_q8_Kx4 (q8_kx4.c:21-105: one scale per row, lrintf) and goes
+ * through q4kx8_gemm_avx512 (kernel_q4kx8_gemm_avx512_full.c:800-860), whose AVX2 kernel is the
+ * decode kernel's arithmetic per output and whose 16 x 16 tiles -- row counts that are
+ * multiples of 16 over a table of a multiple of 16 rows, on a host with AVX-512 -- join the
+ * binary32 accumulators once per pair of sub-blocks instead of once per super-block. Which host
+ * follows geist_hip_sampler_set_projection (_X86: with AVX-512; _X86_AVX2: without). Bit for bit
+ * in all three cases.
+ *
  * geist_hip_project_sample_rows_q4k_packed follows geist_hip_sampler_set_projection: in the
- * default mode GEIST_HIP_PROJECTION_X86 one row over a table of such a shape gets this kernel;
- * a batch, other shapes and any call in mode _PORTABLE get geist_hip_q4k_packed_linear_rows. */
+ * modes _X86 / _X86_AVX2 a table of such a shape gets geist_hip_q4k_packed_linear_x86_rows;
+ * other shapes and any call in mode _PORTABLE get geist_hip_q4k_packed_linear_rows. */
 int geist_hip_q4k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                        size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
                                        float *d_y, size_t ld_y);
+int geist_hip_q4k_packed_linear_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                         size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                         float *d_y, size_t ld_y);
 /* The two halves of that kernel, as for Q6_K: geist_hip_q8k_row_quantize replaces the activation
  * quantiser of kernel_q4kx8_gemm_avx512.c:47-77 for one row -- d_act, 64-byte aligned,
  * geist_hip_q8k_row_act_bytes(n_in) bytes, gets per super-block 72 dwords (the 256 activations as
  * int8, per eight elements the even ones and then the odd ones; their eight sums per sub-block
- * of 32 as int32) and behind the last block the row's scale as binary32 --, and
+ * of 32 as int32) and behind the last block the row's scale as binary32 and padding --, and
  * geist_hip_q4k_packed_gemv_q8k replaces the dot products of :81-304 over it. */
 size_t geist_hip_q8k_row_act_bytes(size_t n_in);
 int geist_hip_q8k_row_quantize(geist_hip_sampler *s, const float *d_x, size_t n_in, void *d_act);

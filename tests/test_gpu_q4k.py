@@ -6,8 +6,8 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import (oracle_q4k_gemv_x86, oracle_q4k_linear, oracle_q8k_row_quantize,
-                        random_q4k_table)
+from oracle_lib import (oracle_q4k_gemv_x86, oracle_q4k_linear, oracle_q4k_linear_x86,
+                        oracle_q8k_row_quantize, random_q4k_table)
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -93,6 +93,57 @@ def test_q4k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
         assert (y1.cpu().numpy().view(np.uint32) == got[1].view(np.uint32)).all(), scale
 
 
+def tie_rows(g, m, n_in, scale):
+    """Rows whose scale is a power of two, with activations exactly between two int8 values: there
+    the decode kernel's quantiser (half away from zero) and the batch quantiser (lrintf) differ."""
+    x = (g.standard_normal((m, n_in)) * scale).astype(np.float32)
+    x[:, ::7] = 0.0
+    d = np.float32(2.0) ** np.ceil(np.log2(scale) - 3)
+    x[:, 0] = np.float32(127.0) * d
+    for k, h in enumerate((0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -126.5)):
+        x[:, 1 + k] = np.float32(h) * d
+    return x
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(64, 512, 2), (64, 512, 3), (5000, 1536, 4), (304, 512, 5),
+                                          (4104, 2560, 8), (64, 256, 12), (4112, 1024, 16),
+                                          (4104, 1024, 16), (128, 512, 32), (72, 16384, 4),
+                                          (70000, 1024, 7)])
+def test_q4k_batch_equals_the_x86_backend(hs, oracle, n_out, n_in, m):
+    """cpu_x86_linear_q4k_mN over the packed copy, to which the oracle is pinned by the compiled
+    reference (tests/test_q4k_x86_oracle.py): row counts that are no multiple of 4 (the decode
+    kernel row by row), multiples of 4 (the batch quantiser), multiples of 16 over 16 n table rows
+    (the AVX-512 tiles' order of accumulation, and the AVX2 kernel's in projection mode
+    X86_AVX2), with activations on the quantisers' ties. Logits bit for bit."""
+    print(f"q4k x86 batch {n_out} x {n_in}, {m} rows", flush=True)
+    g = np.random.default_rng(n_out + n_in + m)
+    w = random_q4k_table(g, n_out, n_in)
+    packed = packed_copy(hs, w, n_in)
+    try:
+        for scale in (1.0, 1e-3, 100.0):
+            x = tie_rows(g, m, n_in, scale)
+            d_x = torch.from_numpy(x).cuda()
+            for mode, avx512 in ((0, True), (2, False)):
+                hs.set_projection(mode)
+                y = torch.full((m, n_out), np.nan, dtype=torch.float32, device="cuda")
+                hs.q4k_packed_linear_x86(packed, n_out, n_in, d_x, y)
+                hs.sync()
+                got = y.cpu().numpy()
+                want = oracle_q4k_linear_x86(oracle.lib, w, x, n_in, avx512=avx512)
+                bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+                assert bad.size == 0, (scale, mode, bad[:5])
+            # every row as a decode call of its own, whatever the batch
+            y = torch.full((m, n_out), np.nan, dtype=torch.float32, device="cuda")
+            hs.q4k_packed_gemv_x86(packed, n_out, n_in, d_x, y)
+            hs.sync()
+            got = y.cpu().numpy()
+            for i in range(m):
+                want = oracle_q4k_gemv_x86(oracle.lib, w, x[i], n_in)
+                assert np.array_equal(got[i].view(np.uint32), want.view(np.uint32)), (scale, i)
+    finally:
+        hs.set_projection(0)
+
+
 def test_q4k_decode_refuses_shapes_the_x86_kernel_does_not_take(hs):
     from geistlib_amd.binding import GeistHipError
     packed = torch.zeros((hs.q4k_packed_bytes(12, 256),), dtype=torch.uint8, device="cuda")
@@ -141,8 +192,9 @@ def test_q4k_argument_errors(hs):
 def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
     """262144 x 1536 Q4_K behind the head with soft-cap 30 (head.c:94-188): norm, projection,
     soft-cap, dispatch, one shared generator. Tokens equal the oracle's session on the oracle's
-    logits, for decode steps and for a batch; without geist_hip_head_q4k_load the call is
-    refused."""
+    logits, for decode steps and for batches (3 rows: the decode kernel row by row; 4 and 8: the
+    batch quantiser), in the x86 backend's arithmetic and in the portable one; without
+    geist_hip_head_q4k_load the call is refused."""
     host.geist_hip_head_project_finalize_q4k.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
                                                          C.c_size_t, C.c_void_p, C.c_float,
                                                          C.c_void_p, C.c_size_t,
@@ -159,10 +211,10 @@ def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
     for T, p, top_k, portable in [(0.0, 1.0, 0, False), (0.8, 1.0, 40, False),
                                   (0.9, 0.95, 0, False), (0.8, 1.0, 40, True)]:
         print(f"q4k table T={T} p={p} k={top_k} portable={portable}", flush=True)
-        h = make_head(host, vocab, 4, cap)
+        h = make_head(host, vocab, 8, cap)
         if portable:
             assert host.geist_hip_head_set_projection(h, 1) == 0
-        opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 4)
+        opts = SessionOpts(0, T, p, top_k, 4242, None, 0, 8)
         assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
         hidden = (g.standard_normal((1, d_model)) * 4).astype(np.float32)
         d_hid = torch.from_numpy(hidden).cuda()
@@ -173,7 +225,7 @@ def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
         assert host.geist_hip_head_q4k_load(h, C.c_void_p(d_w.data_ptr()), d_model) == 0, \
             host.geist_hip_head_errmsg(h)
         sess = oracle.session(T, p, top_k, seed=4242)
-        for k in (1, 1, 3):
+        for k in (1, 1, 3, 4, 8):
             hidden = (g.standard_normal((k, d_model)) * 4).astype(np.float32)
             d_hid = torch.from_numpy(hidden).cuda()
             out = (C.c_int32 * k)()
@@ -182,8 +234,8 @@ def test_head_over_a_q4k_table_with_a_soft_cap(host, oracle):
                 C.c_void_p(d_w.data_ptr()), d_model, out)
             assert rc == 0, host.geist_hip_head_errmsg(h)
             normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
-            if k == 1 and not portable:      # the x86 backend's decode kernel
-                logits = oracle_q4k_gemv_x86(oracle.lib, w, normed[0], d_model)[None, :]
+            if not portable:    # the x86 backend: its decode kernel, cpu_x86_linear_q4k_mN
+                logits = oracle_q4k_linear_x86(oracle.lib, w, normed, d_model)
             else:
                 logits = oracle_q4k_linear(oracle.lib, w, normed, d_model)
             want = oracle.finalize_batch(sess, logits, softcap=cap).tolist()
