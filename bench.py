@@ -699,9 +699,11 @@ def bench_lm_head_q6k(args, m_rows):
 
 def bench_lm_head_q4k(args, m_rows):
     """Workload lm_head_q4k[_mN]: as lm_head_q6k over a Q4_K table of the same geometry
-    ([262144 x 1536], super-blocks of 144 bytes: 226 MB, read once per step; the portable kernel
-    of src/backends/cpu_scalar/weight_resolve.c:82-83, 186-241 after src/formats/gguf/q4_K.c),
-    from the packed copy the head keeps (148 bytes per block)."""
+    ([262144 x 1536], super-blocks of 144 bytes: 226 MB, read once per step and eight rows) in
+    the arithmetic of the reference's x86 backend (src/backends/cpu_x86/linear_q4k.c:142-250),
+    from the packed copy the head keeps (148 bytes per block); the portable kernel
+    (src/backends/cpu_scalar/weight_resolve.c:82-83, 186-241 after src/formats/gguf/q4_K.c) is
+    timed beside it."""
     import torch
     from geistlib_amd import HipSampler, SampleParams
     from geistlib_amd.bench_hooks import Timer
@@ -748,10 +750,11 @@ def bench_lm_head_q4k(args, m_rows):
     ms = elapsed * 1e3 / args.steps
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-    # One row is a decode step of the reference's x86 backend: its integer kernel q4kx8_gemv_m1
-    # (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c), which the step above ran. A batch runs
-    # the portable arithmetic (double accumulation); for one row that kernel is timed beside.
-    x86 = m_rows == 1
+    # The step above ran the arithmetic of the reference's x86 backend: for one row its integer
+    # decode kernel q4kx8_gemv_m1 (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c), for a batch
+    # cpu_x86_linear_q4k_mN (linear_q4k.c:198-250: the same dot products after the batch
+    # quantiser). The portable arithmetic (double accumulation) is timed beside.
+    x86 = True
 
     def timed(fn):
         for i in range(3):
@@ -762,9 +765,8 @@ def bench_lm_head_q4k(args, m_rows):
         return tm.ms * 1e3 / args.steps
 
     portable_us = timed(lambda t: hs.q4k_packed_linear(t, vocab, d_model, normed, logits))
-    kernel_us = (timed(lambda t: hs.q4k_packed_gemv_x86(t, vocab, d_model, normed, logits))
-                 if x86 else portable_us)
-    if x86:
+    kernel_us = timed(lambda t: hs.q4k_packed_linear_x86(t, vocab, d_model, normed, logits))
+    if m_rows == 1:
         # geist_hip_q4k_packed_gemv_x86_rows is two launches, the activation quantiser and the
         # pass over the table; in the step the quantiser rides on the norm's launch
         act = torch.empty((hs.q8k_row_act_bytes(d_model),), dtype=torch.uint8, device=dev)
@@ -778,73 +780,78 @@ def bench_lm_head_q4k(args, m_rows):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("Q4_K weights x int8 activations, int32 dot products, f32 accumulation" if x86
-                  else "Q4_K weights x f32 activations, f64 accumulation"),
+        "dtype": "Q4_K weights x int8 activations, int32 dot products, f32 accumulation",
         "data": "synthetic",
         "config": {"workload": f"lm_head_q4k_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
                    "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
                    "top_p": 0.9, "logit_softcap": 30.0,
-                   "projection": "x86 decode kernel (q4kx8_gemv_m1)" if x86
-                                 else "portable kernel (cpu_scalar_w_quant_mN)"},
+                   "projection": "x86 decode kernel (q4kx8_gemv_m1)" if m_rows == 1
+                                 else "x86 batch path (cpu_x86_linear_q4k_mN)"},
         "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": ("k_q4k_packed_gemv_x86 (+ k_q8k_row_quantize)" if x86 else
-                                "k_q4k_packed_linear (+ activations to double)"),
+                     "kernel": f"k_q4k_packed_gemv_x86<{min(m_rows, 8)}> (+ k_q8k_row_quantize)",
                      "kernel_us": round(kernel_us, 3),
+                     "table_passes": (m_rows + 7) // 8,
                      **({"kernel_us_table_pass_alone": round(table_pass_us, 3),
                          "frac_table_pass_alone":
                              round(w_bytes / (table_pass_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
-                        if x86 else {}),
+                        if m_rows == 1 else {}),
                      "kernel_us_portable_arithmetic": round(portable_us, 3),
                      "kernel_algorithmic_bytes": w_bytes,
                      "packed_bytes_read": read_bytes,
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
     if not args.no_cpu:
-        # CPU side on a bounded sample of the table rows. One row: the reference's own AVX2
-        # kernel over the table its own repacker interleaves (release flags, OpenMP over the
-        # row tiles) where it was compiled from the reference's tree, else the oracle's scalar
-        # restatement; parity against the strict oracle, which is the one pinned to the reference
-        # bit for bit. A batch: the oracle's restatement of the portable kernel.
-        from oracle_lib import (load_oracle, load_ref_q4kgemv, oracle_q4k_gemv_x86,
-                                oracle_q4k_linear, ref_q4k_gemv_m1, Q4KX8_BLOCK_BYTES)
+        # CPU side on a bounded sample of the table rows: the reference's own kernels over the
+        # table its own repacker interleaves (release flags, OpenMP over the row tiles) where
+        # they were compiled from the reference's tree -- q4kx8_gemv_m1 for one row,
+        # quantize_q8_Kx4 + q4kx8_gemm_avx512 for a batch of a multiple of 4 rows, the decode
+        # kernel row by row for the others, as cpu_x86_linear_q4k_mN calls them --, else the
+        # oracle's scalar restatement; parity against the strict oracle, which is the one pinned
+        # to the reference bit for bit.
+        from oracle_lib import (load_oracle, load_ref_q4kgemv, oracle_q4k_linear_x86,
+                                Q4KX8_BLOCK_BYTES, Q8KX4_BLOCK_BYTES)
         import ctypes as C
-        n_s = 65536 if x86 else 16384
+        n_s = 65536
         w_s = tables[0][:n_s].cpu().numpy()
-        x_s = normed.cpu().numpy()
+        x_s = np.ascontiguousarray(normed.cpu().numpy())
         kind = "port"
-        if x86:
-            want = oracle_q4k_gemv_x86(load_oracle(fast=False), w_s, x_s[0], d_model)[None, :]
-            ref = load_ref_q4kgemv(fast=True)
-            if ref is not None:
-                kind = "reference"
-                blob = np.zeros(n_s // 8 * nb * Q4KX8_BLOCK_BYTES + 64, dtype=np.uint8)
-                ref.q4k_to_q4kx8_matrix(d_model, n_s, w_s.ctypes.data_as(C.c_void_p),
-                                        blob.ctypes.data_as(C.c_void_p))      # once, as at load
-                xr = np.ascontiguousarray(x_s[0])
-                yr = np.empty(n_s, dtype=np.float32)
-                fp = C.POINTER(C.c_float)
-                args_r = (n_s, d_model, xr.ctypes.data_as(fp), blob.ctypes.data_as(C.c_void_p),
-                          yr.ctypes.data_as(fp))
-                ref.q4kx8_gemv_m1(*args_r)                                   # threads started
-                reps = 20
-                t0 = time.perf_counter()
-                for _ in range(reps):
-                    ref.q4kx8_gemv_m1(*args_r)
-                dt = (time.perf_counter() - t0) / reps
-            else:
-                lib = load_oracle(fast=True)
-                t0 = time.perf_counter()
-                oracle_q4k_gemv_x86(lib, w_s, x_s[0], d_model)
-                dt = time.perf_counter() - t0
-            hs.q4k_packed_gemv_x86(packed[0], vocab, d_model, normed, logits)
+        want = oracle_q4k_linear_x86(load_oracle(fast=False), w_s, x_s, d_model)
+        ref = load_ref_q4kgemv(fast=True)
+        if ref is not None:
+            kind = "reference"
+            blob = np.zeros(n_s // 8 * nb * Q4KX8_BLOCK_BYTES + 64, dtype=np.uint8)
+            ref.q4k_to_q4kx8_matrix(d_model, n_s, w_s.ctypes.data_as(C.c_void_p),
+                                    blob.ctypes.data_as(C.c_void_p))      # once, as at load
+            yr = np.empty((m_rows, n_s), dtype=np.float32)
+            fp = C.POINTER(C.c_float)
+            acts = np.zeros(max(m_rows // 4, 1) * nb * Q8KX4_BLOCK_BYTES + 64, dtype=np.uint8)
+
+            def cpu_call():
+                if m_rows % 4 != 0:
+                    for i in range(m_rows):
+                        ref.q4kx8_gemv_m1(n_s, d_model, x_s[i].ctypes.data_as(fp),
+                                          blob.ctypes.data_as(C.c_void_p), yr[i].ctypes.data_as(fp))
+                    return
+                for mt in range(m_rows // 4):
+                    ref.quantize_q8_Kx4(d_model, x_s[4 * mt:4 * mt + 4].ctypes.data_as(fp),
+                                        C.c_void_p(acts.ctypes.data + mt * nb * Q8KX4_BLOCK_BYTES))
+                ref.q4kx8_gemm_avx512(m_rows, n_s, d_model, acts.ctypes.data_as(C.c_void_p),
+                                      blob.ctypes.data_as(C.c_void_p), yr.ctypes.data_as(fp))
+
+            cpu_call()                                                      # threads started
+            reps = 20
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                cpu_call()
+            dt = (time.perf_counter() - t0) / reps
         else:
             lib = load_oracle(fast=True)
             t0 = time.perf_counter()
-            want = oracle_q4k_linear(lib, w_s, x_s, d_model)
+            oracle_q4k_linear_x86(lib, w_s, x_s, d_model)
             dt = time.perf_counter() - t0
-            hs.q4k_packed_linear(packed[0], vocab, d_model, normed, logits)
+        hs.q4k_packed_linear_x86(packed[0], vocab, d_model, normed, logits)
         hs.sync()
         got = logits[:, :n_s].cpu().numpy()
         result["cpu_baseline"] = {
@@ -852,9 +859,10 @@ def bench_lm_head_q4k(args, m_rows):
             "cores": int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1),
             "kind": kind,
             "sample": f"the projection of {m_rows} row(s) over the first {n_s} of {vocab} table rows "
-                      + (("(q4kx8_gemv_m1: int8 activations, integer dot products"
-                          + (", AVX2, mean of 20 passes)" if kind == "reference" else ", scalar C)"))
-                         if x86 else "(dequantise a row, accumulate in double)")
+                      + ("(" + ("q4kx8_gemv_m1" if m_rows % 4 else "quantize_q8_Kx4 + q4kx8_gemm_avx512")
+                         + ": int8 activations, integer dot products"
+                         + (", the reference's vector kernels, mean of 20 passes)"
+                            if kind == "reference" else ", scalar C)"))
                       + ", scaled to the whole table; the sampler's share of the step is not "
                         "included"}
         result["parity"] = {"logits_compared": int(want.size),
