@@ -105,7 +105,6 @@ void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, i
 constexpr int Q4X_ACT_DWORDS = 72; /* 64 of int8 (even / odd elements of every eight), 8 sums */
 constexpr int Q4X_ACT_TAIL   = 8;  /* the row's scale, and padding to 32 bytes */
 constexpr int Q4X_M_MAX      = 8;
-constexpr int Q4X_M_MAX_PAIRS = 4; /* with pairs: fewer rows per pass (registers) */
 size_t q4k_x86_act_dwords(int n_in);
 void launch_q8k_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
                              bool ties_even, uint32_t *act);

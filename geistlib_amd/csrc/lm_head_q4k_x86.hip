@@ -157,7 +157,7 @@ __device__ __forceinline__ void q4x_load(const uint32_t *__restrict__ base, int 
  * per pair of sub-blocks (the reference's 16 x 16 AVX-512 tiles,
  * kernel_q4kx8_gemm_avx512_full.c:94, 729-778) instead of once per super-block. */
 template <int M, bool PAIRS>
-__global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
+__global__ __launch_bounds__(Q4X_TPB, PAIRS && M > 2 ? 3 : 4) void k_q4k_packed_gemv_x86(
     const uint32_t *__restrict__ packed, long n_out, int nb, const uint32_t *__restrict__ act,
     float *__restrict__ y, long ld_y) {
     const int  r = threadIdx.x & 63;
@@ -183,42 +183,71 @@ __global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
         typedef uint32_t u8v __attribute__((ext_vector_type(8)));
         const float d    = __half2float(__ushort_as_half((unsigned short) (cur.dd & 0xffffu)));
         const float dmin = __half2float(__ushort_as_half((unsigned short) (cur.dd >> 16)));
-        int         iacc[M], iacc_min[M];
+        int         iacc[M];
 #pragma unroll
         for (int m = 0; m < M; ++m)
-            iacc[m] = 0, iacc_min[m] = 0;
-        /* With several rows the scalar loads of a sub-block stay next to its arithmetic, four
-         * rows at a time: a fence that the loads may not pass and that needs the sums so far.
-         * Hoisted to the top of the block they would not fit the scalar registers. */
-        if (!PAIRS) { /* the minima against the activations' sums per sub-block */
+            iacc[m] = 0;
+        /* With several rows the scalar loads stay near their arithmetic, four rows at a time:
+         * a fence that loads may not pass and that needs the sums so far. Hoisted to the top of
+         * the block they would not fit the scalar registers. */
+        /* the minima against the activations' sums per sub-block: a chain of its own */
 #pragma unroll
-            for (int m = 0; m < M; ++m) {
-                if (M > 4 && m % 4 == 0)
-                    asm volatile("" : "+v"(acc_min[m > 0 ? m - 1 : 0])::"memory");
-                const u8v bs = *reinterpret_cast<const u8v *>(a + m * act_ld + 64);
+        for (int m = 0; m < M; ++m) {
+            if (M > 4 && m % 4 == 0)
+                asm volatile("" : "+v"(acc_min[m > 0 ? m - 1 : 0])::"memory");
+            const u8v   bs = *reinterpret_cast<const u8v *>(a + m * act_ld + 64);
+            const float dm = __fmul_rn(dmin, d_a[m]);
+            int         im = 0;
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    iacc_min[m] += __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu), (int) bs[j]);
-                acc_min[m] = __builtin_fmaf((float) iacc_min[m], __fmul_rn(dmin, d_a[m]), acc_min[m]);
+            for (int j = 0; j < 8; ++j) {
+                im += __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu), (int) bs[j]);
+                if (PAIRS ? (j & 1) : j == 7) {
+                    acc_min[m] = __builtin_fmaf((float) im, dm, acc_min[m]);
+                    im         = 0;
+                }
             }
         }
+        /* Steps of (sub-block j, group of up to four rows). The activations of a step are
+         * scalar loads issued one step ahead, before the fence that opens the step. */
+        constexpr int G  = M < 4 ? M : 4;
+        constexpr int NG = (M + G - 1) / G;
+        u8v           avc[G], avn[G];
+        uint32_t      even[4], odd[4];
+        int           sc = 0;
+        if (M > 1) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { /* sub-block j: elements 32 j .. 32 j + 31, dwords 4 j .. */
-            uint32_t even[4], odd[4];
+            for (int i = 0; i < G; ++i)
+                avc[i] = *reinterpret_cast<const u8v *>(a + i * act_ld);
+        }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t w = cur.q[4 * j + k];
-                even[k] = w & 0x0f0f0f0fu, odd[k] = (w >> 4) & 0x0f0f0f0fu;
-            }
-            const int sc = (int) ((cur.sc[j >> 2] >> (8 * (j & 3))) & 0xffu);
+        for (int st = 0; st < 8 * NG; ++st) {
+            const int j = st / NG, grp = st % NG; /* sub-block j: elements 32 j .. 32 j + 31 */
+            if (M > 1) {
+                if (st + 1 < 8 * NG) {
+                    const int jn = (st + 1) / NG, gn = (st + 1) % NG;
 #pragma unroll
-            for (int m = 0; m < M; ++m) {
-                if (M > 1 && m % 4 == 0) {
-#pragma unroll
-                    for (int i = 0; i < M; ++i)
-                        asm volatile("" : "+v"(iacc[i])::"memory");
+                    for (int i = 0; i < G; ++i)
+                        if (gn * G + i < M)
+                            avn[i] = *reinterpret_cast<const u8v *>(a + (gn * G + i) * act_ld + 8 * jn);
                 }
-                const u8v av  = *reinterpret_cast<const u8v *>(a + m * act_ld + 8 * j);
+#pragma unroll
+                for (int i = 0; i < M; ++i)
+                    asm volatile("" : "+v"(iacc[i])::"memory");
+            }
+            if (grp == 0) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t w = cur.q[4 * j + k];
+                    even[k] = w & 0x0f0f0f0fu, odd[k] = (w >> 4) & 0x0f0f0f0fu;
+                }
+                sc = (int) ((cur.sc[j >> 2] >> (8 * (j & 3))) & 0xffu);
+            }
+#pragma unroll
+            for (int i = 0; i < G; ++i) {
+                const int m = grp * G + i;
+                if (m >= M)
+                    continue;
+                const u8v av  = M > 1 ? avc[i] : *reinterpret_cast<const u8v *>(a + 8 * j);
                 int       dot = 0;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -226,22 +255,15 @@ __global__ __launch_bounds__(Q4X_TPB, 4) void k_q4k_packed_gemv_x86(
                     dot = __builtin_amdgcn_sdot4((int) odd[k], (int) av[2 * k + 1], dot, false);
                 }
                 iacc[m] += __mul24(sc, dot);
-                if (PAIRS && !(j & 1)) { /* the pair's minima */
-                    typedef uint32_t u2v __attribute__((ext_vector_type(2)));
-                    const u2v bs = *reinterpret_cast<const u2v *>(a + m * act_ld + 64 + j);
-                    iacc_min[m] =
-                        __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3))) & 0xffu), (int) bs[0]) +
-                        __mul24((int) ((cur.mn[j >> 2] >> (8 * (j & 3) + 8)) & 0xffu), (int) bs[1]);
-                }
-            }
-            if (PAIRS && (j & 1)) {
-#pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    acc[m]     = __builtin_fmaf((float) iacc[m], __fmul_rn(d, d_a[m]), acc[m]);
-                    acc_min[m] = __builtin_fmaf((float) iacc_min[m], __fmul_rn(dmin, d_a[m]),
-                                                acc_min[m]);
+                if (PAIRS && (j & 1)) {
+                    acc[m]  = __builtin_fmaf((float) iacc[m], __fmul_rn(d, d_a[m]), acc[m]);
                     iacc[m] = 0;
                 }
+            }
+            if (M > 1) {
+#pragma unroll
+                for (int i = 0; i < G; ++i)
+                    avc[i] = avn[i];
             }
         }
         if (!PAIRS) {
@@ -280,14 +302,10 @@ static void q4x_launch(hipStream_t stream, const uint32_t *packed, long n_out, i
                        const uint32_t *act, bool pairs, float *y, long ld_y) {
     const long groups = (n_out + 63) / 64;
     const dim3 grid((unsigned) ((groups + 3) / 4)), block(Q4X_TPB);
-    if constexpr (M <= Q4X_M_MAX_PAIRS) {
-        if (pairs) {
-            k_q4k_packed_gemv_x86<M, true><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y,
-                                                                      ld_y);
-            return;
-        }
-    }
-    k_q4k_packed_gemv_x86<M, false><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y, ld_y);
+    if (pairs)
+        k_q4k_packed_gemv_x86<M, true><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y, ld_y);
+    else
+        k_q4k_packed_gemv_x86<M, false><<<grid, block, 0, stream>>>(packed, n_out, nb, act, y, ld_y);
 }
 
 void launch_q4k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_out, int n_in,

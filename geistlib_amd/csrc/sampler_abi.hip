@@ -1528,7 +1528,7 @@ static int q4k_packed_x86_impl(geist_hip_sampler *s, const void *d_packed, size_
         return rc;
     const bool kx4   = batch && n_rows > 1 && n_rows % 4 == 0;
     const bool pairs = kx4 && !s->projection_avx2 && n_rows % 16 == 0 && n_out % 16 == 0;
-    const size_t tile = pairs ? Q4X_M_MAX_PAIRS : Q4X_M_MAX;
+    const size_t tile = Q4X_M_MAX;
     for (size_t m0 = 0; m0 < n_rows; m0 += tile) {
         const size_t m = n_rows - m0 < tile ? n_rows - m0 : tile;
         launch_q8k_row_quantize(s->stream, d_x + m0 * ld_x, (long) ld_x, (int) m, (int) n_in, kx4,
