@@ -292,6 +292,108 @@ int oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w
     return 0;
 }
 
+/* ---- the x86 backend's batch kernel over a Q6_K table ------------------------------------------
+ * cpu_x86_linear_q6k_mN (src/backends/cpu_x86/linear_q6k.c:234-300) over the copy that
+ * cpu_x86_linear_q6k_resolve (:84-156) makes at load: q6k_to_w8a8_row (q6k_to_w8a8.c:26-68) keeps
+ * the six-bit values q = 0..63 as bytes in element order and, per group of sixteen, the scale
+ * ws = d * (float) scale (binary32) and the offset wo = ws * 32. Every activation row is quantised
+ * by quantize_x_int8_sym (src/formats/gguf/common.c:204-250: ONE scale per row, amax / 127, 1 when
+ * that is zero; lrintf) and summed per sixteen (linear_q6k.c:271-279). Per output and group the
+ * integer d = sum of q * a; then
+ *   lanes != 0  w8x8_gemm / w8x16_gemm (kernel_w8a8_avx512_vnni.c:176-297), which a host with
+ *               AVX-512 VNNI takes for tables of a multiple of 8 rows: acc = fmaf(ws, (float) d,
+ *               acc); acc = fmaf(-wo, (float) sum_a, acc), group after group;
+ *   lanes == 0  w8a8_dot_scalar (kernel_w8a8_scalar.c:14-34) and the VNNI kernel for other tables
+ *               (kernel_w8a8_avx512_vnni.c:90-160), which write acc += ws * (float) d - wo * (float)
+ *               sum_a: restated without contraction, every operation rounded, as the reference's
+ *               strict build compiles it;
+ * and y = scale_x * acc. The interleaving of w8x8_repack / w8x16_repack only places eight or
+ * sixteen rows in the lanes of a vector. */
+
+void oracle_q8_sym_row_quantize(size_t n, const float *x, float *scale_out, int8_t *q_out,
+                                int32_t *sum16_out) {
+    float amax = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        const float a = fabsf(x[i]);
+        if (a > amax)
+            amax = a;
+    }
+    float scale = amax / 127.0f;
+    if (scale == 0.0f)
+        scale = 1.0f;
+    const float inv = 1.0f / scale;
+    for (size_t i = 0; i < n; i++)
+        q_out[i] = (int8_t) lrintf(x[i] * inv);
+    for (size_t g = 0; g < n / 16; g++) {
+        int32_t t = 0;
+        for (int i = 0; i < 16; i++)
+            t += q_out[16 * g + i];
+        sum16_out[g] = t;
+    }
+    *scale_out = scale;
+}
+
+static float oracle_dot_q6k_w8a8(size_t n_super, const uint8_t *row, float scale_x, const int8_t *a,
+                                 const int32_t *sum16, int lanes) {
+    float acc = 0.0f;
+    for (size_t b = 0; b < n_super; b++, row += 210, a += 256, sum16 += 16) {
+        const uint8_t *ql = row, *qh = row + 128;
+        const int8_t  *sc = (const int8_t *) (row + 192);
+        const float    d  = oracle_f16_to_f32((uint16_t) (row[208] | (row[209] << 8)));
+        int32_t        dot[16] = {0};
+        for (int h = 0; h < 2; h++)
+            for (int j = 0; j < 4; j++)
+                for (int l = 0; l < 32; l++) {
+                    const uint8_t lo = ql[64 * h + 32 * (j & 1) + l];
+                    const int     q  = ((j >> 1) ? lo >> 4 : lo & 0xF) |
+                                  (((qh[32 * h + l] >> (2 * j)) & 3) << 4);
+                    const int e = 128 * h + 32 * j + l;
+                    dot[e / 16] += q * a[e];
+                }
+        for (int k = 0; k < 16; k++) {
+            const float ws = d * (float) sc[k];
+            const float wo = ws * 32.0f;
+            if (lanes) {
+                acc = fmaf(ws, (float) dot[k], acc);
+                acc = fmaf(-wo, (float) sum16[k], acc);
+            } else {
+                const float t1 = ws * (float) dot[k];
+                const float t2 = wo * (float) sum16[k];
+                const float t  = t1 - t2;
+                acc            = acc + t;
+            }
+        }
+    }
+    return scale_x * acc;
+}
+
+int oracle_q6k_linear_x86(size_t m, size_t n_out, size_t n_in, const float *x, const void *w_q6k,
+                          float *y, int vnni) {
+    if (n_in % 256 != 0 || n_in == 0 || m == 0)
+        return -1;
+    if (m == 1) /* cpu_x86_linear_q6k_m1: the decode kernel over the table as it lies */
+        return oracle_q6k_gemv_x86(n_out, n_in, x, w_q6k, y);
+    const int lanes = vnni && n_out % 8 == 0; /* q6k_use_w8x8, linear_q6k.c:61-63 */
+    int8_t   *q     = malloc(n_in);
+    int32_t  *sum16 = malloc(n_in / 16 * sizeof(int32_t));
+    if (!q || !sum16) {
+        free(q);
+        free(sum16);
+        return -2;
+    }
+    for (size_t i = 0; i < m; i++) {
+        float scale_x;
+        oracle_q8_sym_row_quantize(n_in, x + i * n_in, &scale_x, q, sum16);
+#pragma omp parallel for schedule(static)
+        for (size_t r = 0; r < n_out; r++)
+            y[i * n_out + r] = oracle_dot_q6k_w8a8(
+                n_in / 256, (const uint8_t *) w_q6k + r * (n_in / 256) * 210, scale_x, q, sum16, lanes);
+    }
+    free(q);
+    free(sum16);
+    return 0;
+}
+
 /* ---- the x86 backend's decode kernel over a Q4_K table ------------------------------------
  * q4kx8_gemv_m1 (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:380-399) over the table that
  * q4k_to_q4kx8_matrix (q4k_to_q4kx8.c:24-115) interleaves eight rows at a time. The interleaving

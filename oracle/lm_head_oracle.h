@@ -80,6 +80,18 @@ void oracle_q6k_linear_f64(size_t m, size_t n_out, size_t n_in, const float *x,
 void oracle_q8k_quantize(size_t n_super, const float *x, float *d_out, int8_t *qs_out,
                          int16_t *bsums_out);
 int  oracle_q6k_gemv_x86(size_t n_out, size_t n_in, const float *x, const void *w_q6k, float *y);
+/* The x86 backend's projection of a batch over a Q6_K table (cpu_x86_linear_q6k_mN,
+ * src/backends/cpu_x86/linear_q6k.c:234-300, over the int8 copy of cpu_x86_linear_q6k_resolve):
+ * the rows quantised with one scale each (quantize_x_int8_sym), integer dot products per group
+ * of sixteen, binary32 accumulation group after group -- with vnni != 0 and a table of a multiple
+ * of 8 rows by two fused multiply-adds per group (w8x8_gemm / w8x16_gemm), otherwise by the
+ * rounded expression of w8a8_dot_scalar. One row is the decode kernel. x [m, n_in], y [m, n_out].
+ * Pinned to those translation units compiled from the reference's tree
+ * (tests/test_q6k_x86_oracle.py). */
+void oracle_q8_sym_row_quantize(size_t n, const float *x, float *scale_out, int8_t *q_out,
+                                int32_t *sum16_out);
+int  oracle_q6k_linear_x86(size_t m, size_t n_out, size_t n_in, const float *x, const void *w_q6k,
+                           float *y, int vnni);
 
 /* The x86 backend's decode kernel over a Q4_K table (q4kx8_gemv_m1,
  * src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c:47-77 the activation quantiser -- one scale for

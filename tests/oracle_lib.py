@@ -639,6 +639,95 @@ def oracle_q8k_row_quantize(lib, x):
     return float(d[0]), qs, bs
 
 
+def load_ref_q6kmn():
+    """The reference's int8 copy of a Q6_K table (q6k_to_w8a8_row, w8x8 / w8x16_repack), its
+    activation quantiser and its W8A8 kernels compiled from its tree (strict flags), or None where
+    not built."""
+    path = os.path.join(ORACLE_DIR, "_ref", "libgeist_ref_q6kmn.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path, mode=os.RTLD_LAZY)
+    vp, sz = C.c_void_p, C.c_size_t
+    lib.q6k_to_w8a8_row.argtypes = [sz, vp, vp, vp, vp]
+    lib.q6k_to_w8a8_row.restype = None
+    lib.w4a8_quantize_acts_row.argtypes = [sz, c_float_p, vp, vp]
+    lib.w4a8_quantize_acts_row.restype = C.c_float
+    lib.w8a8_isa_is_vnni.restype = C.c_int
+    for name in ("w8x8_repack", "w8x16_repack"):
+        getattr(lib, name).argtypes = [sz, sz, vp, vp, vp, vp, vp, vp]
+        getattr(lib, name).restype = None
+    for name in ("w8a8_gemm", "w8x8_gemm", "w8x16_gemm"):
+        getattr(lib, name).argtypes = [sz, sz, sz, vp, vp, vp, vp, vp, vp, c_float_p]
+        getattr(lib, name).restype = None
+    return lib
+
+
+def ref_q6k_linear_mN(ref, w_q6k, x, n_in):
+    """The reference's calls in the order of cpu_x86_linear_q6k_resolve (linear_q6k.c:84-156: the
+    int8 copy row by row, interleaved in eights or sixteens on a VNNI host) and
+    cpu_x86_linear_q6k_mN (:234-300: w4a8_quantize_acts_row per row, the sums again per sixteen,
+    then the kernel the host and the table's row count select). Returns (y, lanes)."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
+    m, n_out, nblk = x.shape[0], w_q6k.shape[0], n_in // 16
+    w = np.ascontiguousarray(w_q6k)
+    row_bytes = n_in // 256 * 210
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
+    wq = np.zeros((n_out, n_in), dtype=np.uint8)
+    ws = np.zeros((n_out, nblk), dtype=np.float32)
+    wo = np.zeros((n_out, nblk), dtype=np.float32)
+    for r in range(n_out):
+        ref.q6k_to_w8a8_row(n_in, C.c_void_p(w.ctypes.data + r * row_bytes),
+                            C.c_void_p(wq.ctypes.data + r * n_in),
+                            C.c_void_p(ws.ctypes.data + r * nblk * 4),
+                            C.c_void_p(wo.ctypes.data + r * nblk * 4))
+    acts = np.zeros((m, n_in), dtype=np.int8)
+    sum_a = np.zeros((m, nblk), dtype=np.int32)
+    scale_x = np.zeros(m, dtype=np.float32)
+    for j in range(m):
+        scale_x[j] = ref.w4a8_quantize_acts_row(n_in, _fp(x[j]), C.c_void_p(acts.ctypes.data + j * n_in),
+                                                C.c_void_p(sum_a.ctypes.data + j * nblk * 4))
+        # linear_q6k.c:271-279: the sums again at the W8A8 granularity of sixteen
+        sum_a[j] = acts[j].reshape(nblk, 16).astype(np.int32).sum(axis=1)
+    y = np.full((m, n_out), np.nan, dtype=np.float32)
+    lanes = bool(ref.w8a8_isa_is_vnni()) and n_out % 8 == 0
+    if lanes:
+        il_q, il_s, il_o = np.zeros_like(wq), np.zeros_like(ws), np.zeros_like(wo)
+        which = "w8x16" if n_out % 16 == 0 else "w8x8"
+        getattr(ref, which + "_repack")(n_out, n_in, vp(wq), vp(ws), vp(wo), vp(il_q), vp(il_s), vp(il_o))
+        getattr(ref, which + "_gemm")(m, n_out, nblk, vp(il_q), vp(il_s), vp(il_o), vp(acts),
+                                      vp(sum_a), vp(scale_x), _fp(y))
+    else:
+        ref.w8a8_gemm(m, n_out, nblk, vp(wq), vp(ws), vp(wo), vp(acts), vp(sum_a), vp(scale_x), _fp(y))
+    return y, lanes
+
+
+def oracle_q8_sym_row_quantize(lib, x):
+    """(scale, q int8 [n], sums int32 [n / 16]) of one row as quantize_x_int8_sym leaves it."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    d = np.empty(1, dtype=np.float32)
+    q = np.empty(x.size, dtype=np.int8)
+    sm = np.empty(x.size // 16, dtype=np.int32)
+    lib.oracle_q8_sym_row_quantize.argtypes = [C.c_size_t, c_float_p, c_float_p, C.c_void_p, C.c_void_p]
+    lib.oracle_q8_sym_row_quantize.restype = None
+    lib.oracle_q8_sym_row_quantize(x.size, _fp(x), _fp(d), q.ctypes.data_as(C.c_void_p),
+                                   sm.ctypes.data_as(C.c_void_p))
+    return float(d[0]), q, sm
+
+
+def oracle_q6k_linear_x86(lib, w_q6k, x, n_in, vnni=True):
+    """oracle_q6k_linear_x86: the x86 backend's projection of a batch over a Q6_K table."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
+    m, n_out = x.shape[0], w_q6k.shape[0]
+    y = np.full((m, n_out), np.nan, dtype=np.float32)
+    lib.oracle_q6k_linear_x86.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t, c_float_p,
+                                          C.c_void_p, c_float_p, C.c_int]
+    lib.oracle_q6k_linear_x86.restype = C.c_int
+    rc = lib.oracle_q6k_linear_x86(m, n_out, n_in, _fp(x), w_q6k.ctypes.data_as(C.c_void_p), _fp(y),
+                                   1 if vnni else 0)
+    assert rc == 0, rc
+    return y
+
+
 def oracle_q8kx4_row_quantize(lib, x):
     """(d, qs int8 [n_in], bsums int16 [n_in / 16]) of one row as quantize_q8_Kx4 leaves it."""
     x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
