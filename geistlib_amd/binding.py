@@ -123,6 +123,8 @@ def load_library():
     lib.geist_hip_q6k_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q4k_packed_gemv_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q4k_packed_linear_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q6k_packed_linear_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
+    lib.geist_hip_q6k_linear_x86_rows.argtypes = [vp, vp, sz, sz, vp, sz, sz, vp, sz]
     lib.geist_hip_q8k_act_bytes.argtypes = [sz, sz]
     lib.geist_hip_q8k_act_bytes.restype = sz
     lib.geist_hip_q8k_quantize_rows.argtypes = [vp, vp, sz, sz, sz, vp]
@@ -430,6 +432,22 @@ class HipSampler:
         m = x.shape[0]
         self._check(self.lib.geist_hip_q4k_packed_gemv_x86_rows(
             self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def q6k_packed_linear_x86(self, packed, n_out, n_in, x, y):
+        """The x86 backend's projection of a batch over the packed Q6_K copy
+        (cpu_x86_linear_q6k_mN; one row: the decode kernel)."""
+        m = x.shape[0]
+        self._check(self.lib.geist_hip_q6k_packed_linear_x86_rows(
+            self.h, _ptr(packed), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
+            y.stride(0) if m > 1 else n_out))
+
+    def q6k_linear_x86(self, w_q6k, n_in, x, y):
+        """The same over the table as it lies in the file."""
+        n_out, m = w_q6k.shape[0], x.shape[0]
+        assert w_q6k.is_contiguous() and w_q6k.shape[1] == n_in // 256 * 210
+        self._check(self.lib.geist_hip_q6k_linear_x86_rows(
+            self.h, _ptr(w_q6k), n_out, n_in, _ptr(x), x.stride(0) if m > 1 else n_in, m, _ptr(y),
             y.stride(0) if m > 1 else n_out))
 
     def q4k_packed_linear_x86(self, packed, n_out, n_in, x, y):

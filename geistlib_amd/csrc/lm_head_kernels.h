@@ -94,6 +94,21 @@ void launch_q6k_packed_gemv_q8k(hipStream_t stream, const void *packed, long n_o
 /* ... and over the table as it lies in the file (4-byte aligned). */
 void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
                          const uint32_t *act, float *y);
+/* The x86 backend's batch path over a Q6_K table (cpu_x86_linear_q6k_mN,
+ * src/backends/cpu_x86/linear_q6k.c:234-300) over the packed copy or the table as it lies: the rows as int8 with one scale
+ * each (quantize_x_int8_sym; act: per row q6k_x86_batch_act_dwords(n_in) dwords), and the integer
+ * dot products per group of sixteen of n_m <= Q6X_M_MAX rows in one pass over the table, joined
+ * in binary32 as the W8A8 lane kernels of a VNNI host join them (lanes) or as the scalar kernel
+ * does. */
+constexpr int Q6X_M_MAX = 8;
+size_t q6k_x86_batch_act_dwords(int n_in);
+void launch_q8s_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                             uint32_t *act);
+void launch_rmsnorm_q8s_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                             float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act);
+/* table: the packed copy (packed) or the table as it lies in the file (4-byte aligned) */
+void launch_q6k_gemm_q8s(hipStream_t stream, const void *table, bool packed, long n_out, int n_in,
+                         const uint32_t *act, int n_m, bool lanes, float *y, long ld_y);
 /* The x86 backend's kernels over a Q4_K table -- the decode kernel q4kx8_gemv_m1
  * (src/backends/cpu_x86/kernel_q4kx8_gemm_avx512.c) and the batch path of
  * cpu_x86_linear_q4k_mN (linear_q4k.c:198-250) -- over the packed copy (lm_head_q4k_x86.hip):

@@ -281,6 +281,350 @@ __global__ __launch_bounds__(Q6X_TPB) void k_q6k_gemv_x86(const uint8_t *__restr
     y[row] = ((acc[0] + acc[4]) + (acc[1] + acc[5])) + ((acc[2] + acc[6]) + (acc[3] + acc[7]));
 }
 
+/* ---- batches: cpu_x86_linear_q6k_mN (src/backends/cpu_x86/linear_q6k.c:234-300) ---------------
+ * The reference multiplies an int8 copy of the table (q6k_to_w8a8_row, q6k_to_w8a8.c:26-68: the
+ * six-bit values as bytes, per group of sixteen ws = d * (float) scale and wo = ws * 32) with the
+ * rows quantised by quantize_x_int8_sym (src/formats/gguf/common.c:204-250: ONE scale per row,
+ * amax / 127, 1 when that is zero; lrintf). Per output and group of sixteen the integer
+ * dot = sum of q * a, then in binary32, group after group,
+ *   LANES   acc = fmaf(ws, (float) dot, acc); acc = fmaf(-wo, (float) sum_a, acc)   (w8x8_gemm /
+ *           w8x16_gemm, kernel_w8a8_avx512_vnni.c:176-297: a host with AVX-512 VNNI, tables of a
+ *           multiple of 8 rows)
+ *   else    acc = acc + (ws * (float) dot - wo * (float) sum_a), every operation rounded
+ *           (w8a8_dot_scalar, kernel_w8a8_scalar.c:14-34, and the VNNI kernel for other tables)
+ * and y = scale_x * acc. The device reads the same packed copy as the decode kernel: the values
+ * and scales of the int8 copy are in it, and ws is formed as the reference forms it.
+ *
+ * act, per row (Q8S_ACT_TAIL dwords behind nb blocks of Q8K_ACT_DWORDS): per run of 32 elements
+ * twelve dwords -- eight of four int8 each in element order, (float) sum_a of its two groups,
+ * -32 * (float) sum_a of the two (exact; fmaf(-wo, s, acc) == fmaf(ws, -32 s, acc) as wo = 32 ws
+ * is exact) --, and behind the last block the row's scale. */
+constexpr int Q8S_ACT_TAIL = 8;
+
+__device__ __forceinline__ void q8s_quantize_block(float xv, float inv, uint32_t *__restrict__ ob) {
+    const int t = threadIdx.x;
+    const int q = __float2int_rn(__fmul_rn(xv, inv)); /* lrintf; |x * inv| <= 127 up to rounding */
+    int       sum = q;
+#pragma unroll
+    for (int s = 8; s >= 1; s >>= 1)
+        sum += __shfl_xor(sum, s);
+    const uint32_t b0 = (uint32_t) q & 0xffu;
+    const uint32_t b1 = (uint32_t) __shfl_down(q, 1) & 0xffu;
+    const uint32_t b2 = (uint32_t) __shfl_down(q, 2) & 0xffu;
+    const uint32_t b3 = (uint32_t) __shfl_down(q, 3) & 0xffu;
+    uint32_t      *run = ob + 12 * (t >> 5);
+    if ((t & 3) == 0)
+        run[(t & 31) >> 2] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    if ((t & 15) == 0) {
+        run[8 + ((t >> 4) & 1)]  = __float_as_uint((float) sum);
+        run[10 + ((t >> 4) & 1)] = __float_as_uint((float) (-32 * sum));
+    }
+}
+
+/* the reciprocal of the row's scale from the row's largest magnitude, the scale to *o_scale */
+__device__ __forceinline__ float q8s_row_inv(float ax, float *s_max, uint32_t *o_scale) {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1)
+        ax = __builtin_fmaxf(ax, __shfl_xor(ax, s));
+    if ((t & 63) == 0)
+        s_max[t >> 6] = ax;
+    __syncthreads();
+    const float amax = __builtin_fmaxf(__builtin_fmaxf(s_max[0], s_max[1]),
+                                       __builtin_fmaxf(s_max[2], s_max[3]));
+    float scale = __fdiv_rn(amax, 127.0f);
+    if (scale == 0.0f)
+        scale = 1.0f;
+    if (t == 0)
+        *o_scale = __float_as_uint(scale);
+    return __fdiv_rn(1.0f, scale);
+}
+
+/* One workgroup per activation row. */
+__global__ __launch_bounds__(Q6X_TPB) void k_q8s_row_quantize(const float *__restrict__ x, long ld_x,
+                                                             int nb, uint32_t *__restrict__ act) {
+    __shared__ float s_max[Q6X_TPB / 64];
+    const int        m = blockIdx.x, t = threadIdx.x;
+    const float     *xr = x + (long) m * ld_x;
+    uint32_t        *o  = act + (long) m * ((long) nb * Q8K_ACT_DWORDS + Q8S_ACT_TAIL);
+    float            ax = 0.0f;
+    for (int b = 0; b < nb; ++b)
+        ax = __builtin_fmaxf(ax, __builtin_fabsf(xr[256 * b + t])); /* (a NaN is passed over) */
+    const float inv = q8s_row_inv(ax, s_max, o + (long) nb * Q8K_ACT_DWORDS);
+    for (int b = 0; b < nb; ++b)
+        q8s_quantize_block(xr[256 * b + t], inv, o + (long) b * Q8K_ACT_DWORDS);
+}
+
+/* The output norm (as k_rmsnorm_rows computes it) and that quantiser in one launch, one workgroup
+ * per row; a thread reads back what it wrote itself. n a multiple of 256. */
+__global__ __launch_bounds__(Q6X_TPB) void k_rmsnorm_q8s_rows(const float *__restrict__ x, long ld_x,
+                                                             const float *__restrict__ w, float eps,
+                                                             int n, float *__restrict__ y, long ld_y,
+                                                             uint32_t *__restrict__ act) {
+    __shared__ double s_part[Q6X_TPB];
+    __shared__ float  s_inv;
+    __shared__ float  s_max[Q6X_TPB / 64];
+    const int    nb = n / 256, m = blockIdx.x, t = threadIdx.x;
+    const float *xr = x + (long) m * ld_x;
+    float       *yr = y + (long) m * ld_y;
+    uint32_t    *o  = act + (long) m * ((long) nb * Q8K_ACT_DWORDS + Q8S_ACT_TAIL);
+    const float  rinv = block_rms_inv<Q6X_TPB>(xr, n, eps, s_part, &s_inv);
+    float        ax = 0.0f;
+    for (int b = 0; b < nb; ++b) {
+        const int   i = 256 * b + t;
+        const float v = __fmul_rn(__fmul_rn(xr[i], rinv), w[i]);
+        yr[i]         = v;
+        ax            = __builtin_fmaxf(ax, __builtin_fabsf(v));
+    }
+    const float inv = q8s_row_inv(ax, s_max, o + (long) nb * Q8K_ACT_DWORDS);
+    for (int b = 0; b < nb; ++b)
+        q8s_quantize_block(yr[256 * b + t], inv, o + (long) b * Q8K_ACT_DWORDS);
+}
+
+typedef uint32_t q8s_u8v __attribute__((ext_vector_type(8), aligned(16)));
+
+/* The rows grp * G .. of a step: each adds the run's two groups of sixteen to its accumulator.
+ * z: the run's 32 values as bytes, four to a dword; ws0 / ws1: the groups' scales; av: the rows'
+ * activations of the run; a_run: the run's twelve dwords of row 0. */
+template <int M, int G, bool LANES>
+__device__ __forceinline__ void q6x_group_rows(const uint32_t (&z)[8], float ws0, float ws1,
+                                               const q8s_u8v (&av)[G],
+                                               const uint32_t *__restrict__ a_run, long act_ld,
+                                               int grp, float (&acc)[M]) {
+    typedef float f2v __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+        const int m = grp * G + i;
+        if (m >= M)
+            continue;
+        const f2v sa = *reinterpret_cast<const f2v *>(a_run + m * act_ld + (LANES ? 10 : 8));
+        int       d0 = 0, d1 = 0;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            d0 = __builtin_amdgcn_sdot4((int) z[u], (int) av[i][u], d0, false);
+            d1 = __builtin_amdgcn_sdot4((int) z[4 + u], (int) av[i][4 + u], d1, false);
+        }
+        if (LANES) {
+            acc[m] = __builtin_fmaf(ws0, (float) d0, acc[m]);
+            acc[m] = __builtin_fmaf(ws0, sa[0], acc[m]);
+            acc[m] = __builtin_fmaf(ws1, (float) d1, acc[m]);
+            acc[m] = __builtin_fmaf(ws1, sa[1], acc[m]);
+        } else {
+            const float wo0 = __fmul_rn(ws0, 32.0f), wo1 = __fmul_rn(ws1, 32.0f);
+            acc[m] = __fadd_rn(acc[m], __fsub_rn(__fmul_rn(ws0, (float) d0), __fmul_rn(wo0, sa[0])));
+            acc[m] = __fadd_rn(acc[m], __fsub_rn(__fmul_rn(ws1, (float) d1), __fmul_rn(wo1, sa[1])));
+        }
+    }
+}
+
+/* M activation rows share a pass over the packed table. Steps of (run of 32 elements, group of up
+ * to four rows): a run's eight fields are spread to bytes once; every row adds its own dot
+ * products, with its activations as scalar operands that were loaded one step ahead, before the
+ * fence that opens the step (an empty asm that loads may not pass and that needs the sums so
+ * far: hoisted to the top of the block the rows' activations would not fit the scalar
+ * registers). */
+template <int M, bool LANES>
+__global__ __launch_bounds__(Q6X_TPB, 4) void k_q6k_packed_gemm_x86(
+    const uint32_t *__restrict__ packed, long n_out, int nb, const uint32_t *__restrict__ act,
+    float *__restrict__ y, long ld_y) {
+    typedef q8s_u8v u8v;
+    constexpr int   G  = M < 4 ? M : 4;
+    constexpr int NG = (M + G - 1) / G;
+    const int     r  = threadIdx.x & 63;
+    const long    g  = (long) blockIdx.x * (Q6X_TPB / 64) + threadIdx.x / 64;
+    if (g * 64 >= n_out)
+        return;
+    const long row    = g * 64 + r;
+    const long act_ld = (long) nb * Q8K_ACT_DWORDS + Q8S_ACT_TAIL;
+    float      acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+        acc[m] = 0.0f;
+    /* loads run half a block ahead of the arithmetic, as in the decode kernel */
+    const uint32_t *base = packed + g * nb * Q6X_PACK_DWORDS;
+    uint32_t        qa[24], qb[24], sc[4], d52;
+    q6x_load_scales(base, r, sc, d52);
+    q6x_load6(base, r, 0, qa);
+    for (int b = 0; b < nb; ++b) {
+        const uint32_t *blk = base + (long) b * Q6X_PACK_DWORDS;
+        const uint32_t *a   = act + (long) b * Q8K_ACT_DWORDS; /* uniform: scalar loads */
+        q6x_load6(blk, r, 6, qb);
+        const float    d         = __half2float(__ushort_as_half((unsigned short) (d52 & 0xffffu)));
+        const uint32_t sc_now[4] = {sc[0], sc[1], sc[2], sc[3]};
+        u8v            avc[G], avn[G];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+            avc[i] = *reinterpret_cast<const u8v *>(a + i * act_ld);
+        uint32_t z[8];
+        float    ws0 = 0.0f, ws1 = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 8 * NG; ++st) {
+            const int v = st / NG, grp = st % NG; /* run v: elements 32 v .. 32 v + 31 */
+            if (st + 1 < 8 * NG) {
+                const int vn = (st + 1) / NG, gn = (st + 1) % NG;
+#pragma unroll
+                for (int i = 0; i < G; ++i)
+                    if (gn * G + i < M)
+                        avn[i] = *reinterpret_cast<const u8v *>(a + (gn * G + i) * act_ld + 12 * vn);
+            }
+#pragma unroll
+            for (int i = 0; i < M; ++i)
+                asm volatile("" : "+v"(acc[i])::"memory");
+            if (st == 4 * NG && b + 1 < nb) { /* the first half's values are used up */
+                q6x_load_scales(blk + Q6X_PACK_DWORDS, r, sc, d52);
+                q6x_load6(blk + Q6X_PACK_DWORDS, r, 0, qa);
+            }
+            if (grp == 0) {
+                const int vl = v & 3;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    /* field f of the half: bits 24 f .. 24 f + 23 of its 24 dwords */
+                    const int      f = 8 * vl + u, w0 = (3 * f) >> 2, sh = (3 * f) & 3;
+                    const int      w1 = w0 + 1 < 24 ? w0 + 1 : 23;
+                    const uint32_t lo = v < 4 ? qa[w0] : qb[w0], hi = v < 4 ? qa[w1] : qb[w1];
+                    z[u] = sh == 0   ? q6x_spread<0>(lo, hi)
+                           : sh == 1 ? q6x_spread<1>(lo, hi)
+                           : sh == 2 ? q6x_spread<2>(lo, hi)
+                                     : q6x_spread<3>(lo, hi);
+                }
+                ws0 = __fmul_rn(d, (float) q6x_scale(sc_now, 2 * v));
+                ws1 = __fmul_rn(d, (float) q6x_scale(sc_now, 2 * v + 1));
+            }
+            q6x_group_rows<M, G, LANES>(z, ws0, ws1, avc, a + 12 * v, act_ld, grp, acc);
+#pragma unroll
+            for (int i = 0; i < G; ++i)
+                avc[i] = avn[i];
+        }
+    }
+    if (row < n_out) {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            y[m * ld_y + row] =
+                __fmul_rn(__uint_as_float(act[m * act_ld + (long) nb * Q8K_ACT_DWORDS]), acc[m]);
+    }
+}
+
+/* The same over the table as it lies in the file: a lane owns a table row and reads its 210-byte
+ * blocks whole; a run's values come from ql and qh as in k_q6k_gemv_x86. */
+template <int M, bool LANES>
+__global__ __launch_bounds__(Q6X_TPB) void k_q6k_gemm_x86(const uint8_t *__restrict__ w, long n_out,
+                                                          int nb, const uint32_t *__restrict__ act,
+                                                          float *__restrict__ y, long ld_y) {
+    typedef q8s_u8v u8v;
+    constexpr int   G  = M < 4 ? M : 4;
+    constexpr int   NG = (M + G - 1) / G;
+    const long      row = (long) blockIdx.x * Q6X_TPB + threadIdx.x;
+    if (row >= n_out)
+        return;
+    const uint8_t *rp     = w + row * (long) nb * 210;
+    const long     act_ld = (long) nb * Q8K_ACT_DWORDS + Q8S_ACT_TAIL;
+    float          acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+        acc[m] = 0.0f;
+    for (int b = 0; b < nb; ++b) {
+        uint32_t dw[53];
+        q6k_load_block(rp + (long) b * 210, dw);
+        const uint32_t *a     = act + (long) b * Q8K_ACT_DWORDS; /* uniform: scalar loads */
+        const uint32_t  sc[4] = {dw[48], dw[49], dw[50], dw[51]};
+        const float     d = __half2float(__ushort_as_half((unsigned short) (dw[52] & 0xffffu)));
+        u8v             avc[G], avn[G];
+#pragma unroll
+        for (int i = 0; i < G; ++i)
+            avc[i] = *reinterpret_cast<const u8v *>(a + i * act_ld);
+        uint32_t z[8];
+        float    ws0 = 0.0f, ws1 = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 8 * NG; ++st) {
+            const int v = st / NG, grp = st % NG; /* run v = 4 h + j: elements 128 h + 32 j .. */
+            if (st + 1 < 8 * NG) {
+                const int vn = (st + 1) / NG, gn = (st + 1) % NG;
+#pragma unroll
+                for (int i = 0; i < G; ++i)
+                    if (gn * G + i < M)
+                        avn[i] = *reinterpret_cast<const u8v *>(a + (gn * G + i) * act_ld + 12 * vn);
+            }
+#pragma unroll
+            for (int i = 0; i < M; ++i)
+                asm volatile("" : "+v"(acc[i])::"memory");
+            if (grp == 0) {
+                const int h = v >> 2, j = v & 3;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const uint32_t ql = dw[16 * h + 8 * (j & 1) + u], qh = dw[32 + 8 * h + u];
+                    const uint32_t lo = (j >> 1) ? (ql >> 4) & 0x0f0f0f0fu : ql & 0x0f0f0f0fu;
+                    const uint32_t hi = j == 0   ? (qh << 4) & 0x30303030u
+                                        : j == 1 ? (qh << 2) & 0x30303030u
+                                        : j == 2 ? qh & 0x30303030u
+                                                 : (qh >> 2) & 0x30303030u;
+                    z[u] = lo | hi;
+                }
+                ws0 = __fmul_rn(d, (float) q6x_scale(sc, 2 * v));
+                ws1 = __fmul_rn(d, (float) q6x_scale(sc, 2 * v + 1));
+            }
+            q6x_group_rows<M, G, LANES>(z, ws0, ws1, avc, a + 12 * v, act_ld, grp, acc);
+#pragma unroll
+            for (int i = 0; i < G; ++i)
+                avc[i] = avn[i];
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+        y[m * ld_y + row] =
+            __fmul_rn(__uint_as_float(act[m * act_ld + (long) nb * Q8K_ACT_DWORDS]), acc[m]);
+}
+
+size_t q6k_x86_batch_act_dwords(int n_in) {
+    return (size_t) (n_in / 256) * Q8K_ACT_DWORDS + Q8S_ACT_TAIL;
+}
+
+void launch_q8s_row_quantize(hipStream_t stream, const float *x, long ld_x, int n_m, int n_in,
+                             uint32_t *act) {
+    k_q8s_row_quantize<<<dim3(n_m), dim3(Q6X_TPB), 0, stream>>>(x, ld_x, n_in / 256, act);
+}
+
+void launch_rmsnorm_q8s_rows(hipStream_t stream, const float *x, long ld_x, const float *w,
+                             float eps, int n_rows, int n, float *y, long ld_y, uint32_t *act) {
+    k_rmsnorm_q8s_rows<<<dim3(n_rows), dim3(Q6X_TPB), 0, stream>>>(x, ld_x, w, eps, n, y, ld_y,
+                                                                  act);
+}
+
+template <int M>
+static void q6x_gemm_launch(hipStream_t stream, const void *table, bool packed, long n_out, int nb,
+                            const uint32_t *act, bool lanes, float *y, long ld_y) {
+    if (packed) {
+        const uint32_t *p      = static_cast<const uint32_t *>(table);
+        const long      groups = (n_out + 63) / 64;
+        const dim3      grid((unsigned) ((groups + 3) / 4)), block(Q6X_TPB);
+        if (lanes)
+            k_q6k_packed_gemm_x86<M, true><<<grid, block, 0, stream>>>(p, n_out, nb, act, y, ld_y);
+        else
+            k_q6k_packed_gemm_x86<M, false><<<grid, block, 0, stream>>>(p, n_out, nb, act, y, ld_y);
+    } else {
+        const uint8_t *p = static_cast<const uint8_t *>(table);
+        const dim3     grid((unsigned) ((n_out + Q6X_TPB - 1) / Q6X_TPB)), block(Q6X_TPB);
+        if (lanes)
+            k_q6k_gemm_x86<M, true><<<grid, block, 0, stream>>>(p, n_out, nb, act, y, ld_y);
+        else
+            k_q6k_gemm_x86<M, false><<<grid, block, 0, stream>>>(p, n_out, nb, act, y, ld_y);
+    }
+}
+
+void launch_q6k_gemm_q8s(hipStream_t stream, const void *table, bool packed, long n_out, int n_in,
+                         const uint32_t *act, int n_m, bool lanes, float *y, long ld_y) {
+    const int nb = n_in / 256;
+    switch (n_m) {
+    case 1: q6x_gemm_launch<1>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 2: q6x_gemm_launch<2>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 3: q6x_gemm_launch<3>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 4: q6x_gemm_launch<4>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 5: q6x_gemm_launch<5>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 6: q6x_gemm_launch<6>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    case 7: q6x_gemm_launch<7>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    default: q6x_gemm_launch<8>(stream, table, packed, n_out, nb, act, lanes, y, ld_y); break;
+    }
+}
+
 void launch_q6k_gemv_q8k(hipStream_t stream, const uint8_t *w_q6k, long n_out, int n_in,
                          const uint32_t *act, float *y) {
     k_q6k_gemv_x86<<<dim3((unsigned) ((n_out + Q6X_TPB - 1) / Q6X_TPB)), dim3(Q6X_TPB), 0, stream>>>(

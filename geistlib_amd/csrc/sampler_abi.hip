@@ -1244,11 +1244,13 @@ static int f16_linear_impl(geist_hip_sampler *s, const uint16_t *d_w_f16, size_t
 
 /* Scratch of the Q6_K projection: the activations in double, their sums and magnitudes per
  * group of 16, the list of outputs for the second kernel. */
-/* the int8 activations of the x86 kernels: one row for Q6_K, Q4X_M_MAX rows for Q4_K */
+/* the int8 activations of the x86 kernels: one row for the Q6_K decode kernel, Q6X_M_MAX rows
+ * for its batch path, Q4X_M_MAX rows for Q4_K */
 static size_t q8_act_bytes(size_t n_in) {
     const size_t q6 = (n_in / 256) * Q8K_ACT_DWORDS;
     const size_t q4 = (size_t) Q4X_M_MAX * ((n_in / 256) * Q4X_ACT_DWORDS + Q4X_ACT_TAIL);
-    return (q6 > q4 ? q6 : q4) * sizeof(uint32_t);
+    const size_t qb = (size_t) Q6X_M_MAX * q6k_x86_batch_act_dwords((int) n_in);
+    return (q6 > q4 ? (q6 > qb ? q6 : qb) : (q4 > qb ? q4 : qb)) * sizeof(uint32_t);
 }
 
 static int q6k_scratch(geist_hip_sampler *s, size_t n_out, size_t n_in, Q6KScratch &ws) {
@@ -1326,6 +1328,29 @@ static int q6k_gemv_x86_impl(geist_hip_sampler *s, const void *d_table, bool pac
         else
             launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_table), (long) n_out,
                                 (int) n_in, ws.act8, d_y + m * ld_y);
+    }
+    return GEIST_HIP_OK;
+}
+
+/* cpu_x86_linear_q6k_mN (linear_q6k.c:234-300) over the packed copy or the table as it lies,
+ * Q6X_M_MAX rows per pass over the table; one row is cpu_x86_linear_q6k_m1's decode kernel. The lane kernels' arithmetic for
+ * tables of a multiple of 8 rows unless the host reproduced has no AVX-512 VNNI. */
+static int q6k_x86_batch_impl(geist_hip_sampler *s, const void *d_table, bool packed, size_t n_out,
+                              size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                              float *d_y, size_t ld_y) {
+    if (n_rows == 1)
+        return q6k_gemv_x86_impl(s, d_table, packed, n_out, n_in, d_x, ld_x, 1, d_y, ld_y);
+    Q6KScratch ws;
+    const int  rc = q6k_scratch(s, n_out, n_in, ws);
+    if (rc)
+        return rc;
+    const bool lanes = !s->projection_avx2 && n_out % 8 == 0;
+    for (size_t m0 = 0; m0 < n_rows; m0 += Q6X_M_MAX) {
+        const size_t m = n_rows - m0 < (size_t) Q6X_M_MAX ? n_rows - m0 : (size_t) Q6X_M_MAX;
+        launch_q8s_row_quantize(s->stream, d_x + m0 * ld_x, (long) ld_x, (int) m, (int) n_in,
+                                ws.act8);
+        launch_q6k_gemm_q8s(s->stream, d_table, packed, (long) n_out, (int) n_in, ws.act8, (int) m,
+                            lanes, d_y + m0 * ld_y, (long) ld_y);
     }
     return GEIST_HIP_OK;
 }
@@ -1431,6 +1456,44 @@ int geist_hip_q6k_packed_gemv_x86_rows(geist_hip_sampler *s, const void *d_packe
     HIPCHK(s, hipSetDevice(s->device));
     rc = q6k_gemv_x86_impl(s, d_packed, true, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
     return rc ? rc : after_launch(s, "Q6_K decode (packed)");
+}
+
+int geist_hip_q6k_packed_linear_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                         size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                         float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_packed || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K x86 batch: %zu rows, strides %zu / %zu",
+                    n_rows, ld_x, ld_y);
+    int rc = q6k_check(s, d_packed, n_out, n_in);
+    if (rc)
+        return rc;
+    if (((uintptr_t) d_packed) % 16 != 0)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "packed Q6_K table not 16-byte aligned");
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q6k_x86_batch_impl(s, d_packed, true, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q6_K x86 batch (packed)");
+}
+
+int geist_hip_q6k_linear_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out,
+                                  size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                  float *d_y, size_t ld_y) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (!d_w_q6k || !d_x || !d_y)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "null argument");
+    if (n_rows == 0 || ld_x < n_in || ld_y < n_out)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "Q6_K x86 batch: %zu rows, strides %zu / %zu",
+                    n_rows, ld_x, ld_y);
+    int rc = q6k_check(s, d_w_q6k, n_out, n_in);
+    if (rc)
+        return rc;
+    HIPCHK(s, hipSetDevice(s->device));
+    rc = q6k_x86_batch_impl(s, d_w_q6k, false, n_out, n_in, d_x, ld_x, n_rows, d_y, ld_y);
+    return rc ? rc : after_launch(s, "Q6_K x86 batch");
 }
 
 int geist_hip_q6k_gemv_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out,
@@ -1784,14 +1847,21 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
     const bool q4k_x86  = table == TABLE_Q4K_PACKED && !s->projection_portable &&
                           q4k_x86_shape(n_vocab, d_model);
     const bool q4k_kx4   = q4k_x86 && rows > 1 && rows % 4 == 0;
+    /* a batch over a Q6_K table as cpu_x86_linear_q6k_mN projects it */
+    const bool q6k_x86_mn    = (table == TABLE_Q6K_PACKED || table == TABLE_Q6K) && rows > 1 &&
+                               !s->projection_portable;
+    const bool q6k_mn_fused  = q6k_x86_mn && rows <= (size_t) Q6X_M_MAX;
     const bool q4k_fused = q4k_x86 && rows <= (size_t) Q4X_M_MAX;
     Q6KScratch q6ws{};
-    if (q6k_x86 || q4k_fused) {
+    if (q6k_x86 || q4k_fused || q6k_mn_fused) {
         if ((rc = q6k_scratch(s, n_vocab, d_model, q6ws)) != GEIST_HIP_OK)
             return rc;
         if (q6k_x86)
             launch_rmsnorm_q8k_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
                                     1, (int) d_model, d_normed, (long) d_model, q6ws.act8);
+        else if (q6k_mn_fused)
+            launch_rmsnorm_q8s_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight, rms_eps,
+                                    (int) rows, (int) d_model, d_normed, (long) d_model, q6ws.act8);
         else
             launch_rmsnorm_q8k_row_rows(s->stream, d_hidden, (long) ld_hidden, d_norm_weight,
                                         rms_eps, (int) rows, (int) d_model, d_normed,
@@ -1817,6 +1887,14 @@ static int project_sample_impl(geist_hip_sampler *s, const float *d_hidden, size
         else
             launch_q6k_gemv_q8k(s->stream, static_cast<const uint8_t *>(d_embed), (long) n_vocab,
                                 (int) d_model, q6ws.act8, d_logits);
+    } else if (q6k_mn_fused) {
+        launch_q6k_gemm_q8s(s->stream, d_embed, table == TABLE_Q6K_PACKED, (long) n_vocab,
+                            (int) d_model, q6ws.act8, (int) rows,
+                            !s->projection_avx2 && n_vocab % 8 == 0, d_logits, (long) ld_logits);
+    } else if (q6k_x86_mn) {
+        if ((rc = q6k_x86_batch_impl(s, d_embed, table == TABLE_Q6K_PACKED, n_vocab, d_model,
+                                     d_normed, d_model, rows, d_logits, ld_logits)) != GEIST_HIP_OK)
+            return rc;
     } else if (q4k_fused) {
         /* (at most 8 rows: never the AVX-512 tiles' arithmetic) */
         launch_q4k_packed_gemv_q8k(s->stream, d_embed, (long) n_vocab, (int) d_model, q6ws.act8,

@@ -188,6 +188,28 @@ int geist_hip_q8k_quantize_rows(geist_hip_sampler *s, const float *d_x, size_t l
                                 size_t n_in, void *d_act);
 int geist_hip_q6k_packed_gemv_q8k(geist_hip_sampler *s, const void *d_packed, size_t n_out,
                                   size_t n_in, const void *d_act, float *d_y);
+/* geist_hip_q6k_packed_linear_x86_rows replaces cpu_x86_linear_q6k_mN
+ * (src/backends/cpu_x86/linear_q6k.c:234-300) for n_rows > 1, and the decode kernel for one row,
+ * bit for bit. The reference multiplies an int8 copy of the table that it makes at load
+ * (cpu_x86_linear_q6k_resolve, :84-156; q6k_to_w8a8_row, q6k_to_w8a8.c:26-68: the six-bit values
+ * as bytes, a binary32 scale and offset per group of sixteen) with the rows quantised by
+ * quantize_x_int8_sym (src/formats/gguf/common.c:204-250: one scale per row, lrintf): integer dot
+ * products per group of sixteen, joined in binary32 group after group. The device needs no such
+ * copy: the packed copy holds the same values and scales. How the groups are joined depends on
+ * the host, and follows geist_hip_sampler_set_projection: _X86 stands for a host with AVX-512
+ * VNNI, whose lane kernels (w8x8_gemm / w8x16_gemm, kernel_w8a8_avx512_vnni.c:176-297: two fused
+ * multiply-adds per group) take tables of a multiple of 8 rows; other tables there, and every
+ * table in mode _X86_AVX2 (a host without VNNI, or GEIST_FORCE_ISA=avx2), get the expression of
+ * w8a8_dot_scalar (kernel_w8a8_scalar.c:14-34) with every operation rounded, as the reference's
+ * strict build compiles it. Up to eight rows share a pass over the table. Activations must be
+ * finite. */
+int geist_hip_q6k_packed_linear_x86_rows(geist_hip_sampler *s, const void *d_packed, size_t n_out,
+                                         size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                         float *d_y, size_t ld_y);
+/* The same over the table as it lies in the file (4-byte aligned): the same results bit for bit. */
+int geist_hip_q6k_linear_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, size_t n_out,
+                                  size_t n_in, const float *d_x, size_t ld_x, size_t n_rows,
+                                  float *d_y, size_t ld_y);
 /* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, the projection and the
  * sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. The
  * projection follows geist_hip_sampler_set_projection: in the default mode

@@ -7,8 +7,8 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from oracle_lib import (oracle_q6k_gemv_x86, oracle_q6k_linear, oracle_q8k_quantize,
-                        random_q6k_table)
+from oracle_lib import (oracle_q6k_gemv_x86, oracle_q6k_linear, oracle_q6k_linear_x86,
+                        oracle_q8k_quantize, random_q6k_table)
 from test_gpu_host_layer import SessionOpts, host, make_head  # noqa: F401 (fixture)
 
 pytestmark = pytest.mark.gpu
@@ -124,6 +124,59 @@ def test_q6k_decode_equals_the_x86_kernel(hs, oracle, n_out, n_in):
         assert (y1.cpu().numpy().view(np.uint32) == got[2].view(np.uint32)).all(), scale
 
 
+def tie_rows(g, m, n_in, scale):
+    """Rows whose scale is a power of two, with activations exactly between two int8 values."""
+    x = (g.standard_normal((m, n_in)) * scale).astype(np.float32)
+    x[:, ::7] = 0.0
+    d = np.float32(2.0) ** np.ceil(np.log2(scale) - 3)
+    x[:, 0] = np.float32(127.0) * d
+    for k, h in enumerate((0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -126.5)):
+        x[:, 1 + k] = np.float32(h) * d
+    return x
+
+
+@pytest.mark.parametrize("n_out,n_in,m", [(64, 512, 2), (300, 512, 3), (5000, 1536, 4), (304, 512, 5),
+                                          (4100, 2560, 8), (64, 256, 12), (4112, 1024, 16),
+                                          (72, 16384, 2), (70000, 1024, 7), (1, 256, 2)])
+def test_q6k_batch_equals_the_x86_backend(hs, oracle, n_out, n_in, m):
+    """cpu_x86_linear_q6k_mN, to which the oracle is pinned by the compiled reference
+    (tests/test_q6k_x86_oracle.py), over the packed copy and over the table as it lies: in
+    projection mode X86 the lane kernels' arithmetic for tables of a multiple of 8 rows and the
+    scalar kernel's for the others, in mode X86_AVX2 the scalar kernel's for all. Logits bit for
+    bit, one row included (the decode kernel)."""
+    print(f"q6k x86 batch {n_out} x {n_in}, {m} rows", flush=True)
+    g = np.random.default_rng(n_out + n_in + m)
+    w = random_q6k_table(g, n_out, n_in)
+    d_w = torch.from_numpy(w).cuda()
+    packed = torch.full((hs.q6k_packed_bytes(n_out, n_in),), 0xA5, dtype=torch.uint8, device="cuda")
+    hs.q6k_pack(d_w, n_in, packed)
+    try:
+        for scale in (1.0, 1e-3, 100.0):
+            x = tie_rows(g, m, n_in, scale)
+            d_x = torch.from_numpy(x).cuda()
+            for mode, vnni in ((0, True), (2, False)):
+                hs.set_projection(mode)
+                want = oracle_q6k_linear_x86(oracle.lib, w, x, n_in, vnni=vnni)
+                for over_packed in (True, False):
+                    y = torch.full((m, n_out), np.nan, dtype=torch.float32, device="cuda")
+                    if over_packed:
+                        hs.q6k_packed_linear_x86(packed, n_out, n_in, d_x, y)
+                    else:
+                        hs.q6k_linear_x86(d_w, n_in, d_x, y)
+                    hs.sync()
+                    got = y.cpu().numpy()
+                    bad = np.argwhere(got.view(np.uint32) != want.view(np.uint32))
+                    assert bad.size == 0, (scale, mode, over_packed, bad[:5])
+        x1 = tie_rows(g, 1, n_in, 1.0)
+        y = torch.full((1, n_out), np.nan, dtype=torch.float32, device="cuda")
+        hs.q6k_packed_linear_x86(packed, n_out, n_in, torch.from_numpy(x1).cuda(), y)
+        hs.sync()
+        want = oracle_q6k_gemv_x86(oracle.lib, w, x1[0], n_in)
+        assert np.array_equal(y.cpu().numpy()[0].view(np.uint32), want.view(np.uint32))
+    finally:
+        hs.set_projection(0)
+
+
 def test_q6k_linear_with_activations_that_are_not_finite(hs, oracle):
     """An infinity, two of opposite sign, a NaN among the activations: the reference's sum in
     index order gives +-inf or NaN per output (golden case of tests/golden/q6k_ref_vectors.json,
@@ -173,7 +226,9 @@ def test_q6k_argument_errors(hs):
 def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
     """262144 x 1536 Q6_K (the tied table of the Gemma models) behind the head with soft-cap 30
     (head.c:94-188): norm, projection, soft-cap, dispatch, one shared generator. Tokens equal the
-    oracle's session on the oracle's logits, for decode steps and for a batch."""
+    oracle's session on the oracle's logits, for decode steps and for batches of 3 and 8 rows, in
+    the x86 backend's arithmetic (over the packed copy and over the table as it lies) and in the
+    portable one."""
     host.geist_hip_head_project_finalize_q6k.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t,
                                                          C.c_size_t, C.c_void_p, C.c_float,
                                                          C.c_void_p, C.c_size_t,
@@ -189,10 +244,10 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
     for T, p, top_k, portable in [(0.0, 1.0, 0, False), (0.8, 1.0, 40, False),
                                   (0.9, 0.95, 0, False), (0.8, 1.0, 40, True)]:
         print(f"gemma table T={T} p={p} k={top_k} portable={portable}", flush=True)
-        h = make_head(host, vocab, 4, cap)
+        h = make_head(host, vocab, 8, cap)
         if portable:
             assert host.geist_hip_head_set_projection(h, 1) == 0
-        opts = SessionOpts(0, T, p, top_k, 31337, None, 0, 4)
+        opts = SessionOpts(0, T, p, top_k, 31337, None, 0, 8)
         assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
         packed = not (top_k == 0 and T == 0.0)
         if not packed:      # one configuration reads the table as it lies, the others packed
@@ -201,7 +256,7 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
             assert host.geist_hip_head_q6k_load(h, C.c_void_p(d_w.data_ptr()), d_model) == 0, \
                 host.geist_hip_head_errmsg(h)
         sess = oracle.session(T, p, top_k, seed=31337)
-        for k in (1, 1, 3):
+        for k in (1, 1, 3, 8):
             hidden = (g.standard_normal((k, d_model)) * 4).astype(np.float32)
             d_hid = torch.from_numpy(hidden).cuda()
             out = (C.c_int32 * k)()
@@ -210,8 +265,8 @@ def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
                 C.c_void_p(d_w.data_ptr()), d_model, out)
             assert rc == 0, host.geist_hip_head_errmsg(h)
             normed = oracle.rmsnorm(hidden, norm_w, 1e-6)
-            if k == 1 and not portable:     # the x86 backend's decode kernel, packed copy or not
-                logits = oracle_q6k_gemv_x86(oracle.lib, w, normed[0], d_model)[None, :]
+            if not portable:    # the x86 backend (decode kernel, batch path), packed copy or not
+                logits = oracle_q6k_linear_x86(oracle.lib, w, normed, d_model)
             else:
                 logits = oracle_q6k_linear(oracle.lib, w, normed, d_model)
             want = oracle.finalize_batch(sess, logits, softcap=cap).tolist()
