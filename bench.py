@@ -587,9 +587,11 @@ def bench_lm_head_q6k(args, m_rows):
     ms = elapsed * 1e3 / args.steps
     ids_gpu = out.cpu().numpy()
     hs.rmsnorm(hidden, norm_w, 1e-6, normed)
-    # One row is a decode step of the reference's x86 backend: its integer kernel q6k_gemv_m1
-    # (src/backends/cpu_x86/kernel_q6k_gemv.c), which the step above ran. A batch runs the
-    # portable arithmetic (double accumulation); for one row that kernel is timed beside.
+    # The step above ran the arithmetic of the reference's x86 backend: for one row its integer
+    # decode kernel q6k_gemv_m1 (src/backends/cpu_x86/kernel_q6k_gemv.c), for a batch
+    # cpu_x86_linear_q6k_mN (linear_q6k.c:234-300: one int8 scale per row, integer dot products
+    # per group of sixteen, joined as the W8A8 lane kernels of a VNNI host join them). The
+    # portable arithmetic (double accumulation) is timed beside.
     x86 = m_rows == 1
 
     def timed(fn, tabs):
@@ -612,7 +614,8 @@ def bench_lm_head_q6k(args, m_rows):
         table_pass_us = timed(lambda t, i: hs.q6k_packed_gemv_q8k(t, vocab, d_model, act,
                                                                   logits[0]), packed)
     else:
-        kernel_us = portable_us
+        kernel_us = timed(lambda t, i: hs.q6k_packed_linear_x86(t, vocab, d_model, normed, logits),
+                          packed)
     w_bytes = vocab * nb * 210
     achieved = w_bytes / (kernel_us * 1e-6) / 1e9
     result = {
@@ -620,20 +623,20 @@ def bench_lm_head_q6k(args, m_rows):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("Q6_K weights x int8 activations, int32 dot products, f32 accumulation" if x86
-                  else "Q6_K weights x f32 activations, f64 accumulation"),
+        "dtype": "Q6_K weights x int8 activations, int32 dot products, f32 accumulation",
         "data": "synthetic",
         "config": {"workload": f"lm_head_q6k_v{vocab}_d{d_model}_m{m_rows}", "rows": m_rows,
                    "n_vocab": vocab, "d_model": d_model, "temperature": 0.7, "top_k": 40,
                    "top_p": 0.9, "logit_softcap": 30.0,
                    "projection": "x86 decode kernel (q6k_gemv_m1)" if x86
-                                 else "portable kernel (cpu_scalar_w_quant_mN)"},
+                                 else "x86 batch path (cpu_x86_linear_q6k_mN)"},
         "us_per_step": round(ms * 1e3, 3), "weight_copies_rotated": 3,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": ("k_q6k_packed_gemv_x86 (+ k_q8k_quantize)" if x86 else
-                                "k_q6k_packed_linear (+ activations to double)"),
+                                f"k_q6k_packed_gemm_x86<{min(m_rows, 8)}> (+ k_q8s_row_quantize)"),
                      "kernel_us": round(kernel_us, 3),
+                     "table_passes": (m_rows + 7) // 8,
                      **({"kernel_us_table_pass_alone": round(table_pass_us, 3),
                          "frac_table_pass_alone":
                              round(w_bytes / (table_pass_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -644,13 +647,14 @@ def bench_lm_head_q6k(args, m_rows):
                      "step_algorithmic_bytes": w_bytes + m_rows * (d_model * 8 + vocab * 8 + 8)},
     }
     if not args.no_cpu:
-        # CPU side on a bounded sample of the table rows. One row: the reference's own AVX2
-        # kernel (release flags, OpenMP over the table rows) where it was compiled from the
-        # reference's tree, else the oracle's scalar restatement; parity against the strict
-        # oracle, which is the one pinned to the reference bit for bit. A batch: the oracle's
-        # restatement of the portable kernel.
-        from oracle_lib import (load_oracle, load_ref_q6kgemv, oracle_q6k_gemv_x86,
-                                oracle_q6k_linear, ref_q6k_gemv_m1)
+        # CPU side on a bounded sample of the table rows, by the reference's own kernels where
+        # they were compiled from its tree, else the oracle's scalar restatement; parity against
+        # the strict oracle, which is the one pinned to the reference bit for bit. One row:
+        # q6k_gemv_m1 (AVX2, release flags, OpenMP over the table rows). A batch:
+        # w4a8_quantize_acts_row + the W8A8 kernel this host selects, over the int8 copy the
+        # reference makes at load (strict flags; made before the clock starts).
+        from oracle_lib import (load_oracle, load_ref_q6kgemv, load_ref_q6kmn, oracle_q6k_gemv_x86,
+                                oracle_q6k_linear_x86, ref_q6k_gemv_m1, ref_q6k_mN_prepare)
         n_s = 65536 if x86 else 16384
         w_s = tables[0][:n_s].cpu().numpy()
         x_s = normed.cpu().numpy()
@@ -673,11 +677,23 @@ def bench_lm_head_q6k(args, m_rows):
                 dt = time.perf_counter() - t0
             hs.q6k_packed_gemv_x86(packed[0], vocab, d_model, normed, logits)
         else:
-            lib = load_oracle(fast=True)
-            t0 = time.perf_counter()
-            want = oracle_q6k_linear(lib, w_s, x_s, d_model)
-            dt = time.perf_counter() - t0
-            hs.q6k_packed_linear(packed[0], vocab, d_model, normed, logits)
+            want = oracle_q6k_linear_x86(load_oracle(fast=False), w_s, x_s, d_model)
+            ref = load_ref_q6kmn()
+            if ref is not None and ref.w8a8_isa_is_vnni():
+                kind = "reference"
+                run = ref_q6k_mN_prepare(ref, w_s, d_model)
+                run(x_s)                                                # threads started
+                reps = 10
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    run(x_s)
+                dt = (time.perf_counter() - t0) / reps
+            else:
+                lib = load_oracle(fast=True)
+                t0 = time.perf_counter()
+                oracle_q6k_linear_x86(lib, w_s, x_s, d_model)
+                dt = time.perf_counter() - t0
+            hs.q6k_packed_linear_x86(packed[0], vocab, d_model, normed, logits)
         hs.sync()
         got = logits[:, :n_s].cpu().numpy()
         result["cpu_baseline"] = {
@@ -687,7 +703,10 @@ def bench_lm_head_q6k(args, m_rows):
             "sample": f"the projection of {m_rows} row(s) over the first {n_s} of {vocab} table rows "
                       + (("(q6k_gemv_m1: int8 activations, integer dot products"
                           + (", AVX2, mean of 20 passes)" if kind == "reference" else ", scalar C)"))
-                         if x86 else "(dequantise a row, accumulate in double)")
+                         if x86 else
+                         ("(cpu_x86_linear_q6k_mN: int8 activations, integer dot products"
+                          + (", the reference's W8A8 lane kernel, mean of 10 passes)"
+                             if kind == "reference" else ", scalar C)")))
                       + ", scaled to the whole table; the sampler's share of the step is not "
                         "included"}
         result["parity"] = {"logits_compared": int(want.size),

@@ -662,13 +662,12 @@ def load_ref_q6kmn():
     return lib
 
 
-def ref_q6k_linear_mN(ref, w_q6k, x, n_in):
-    """The reference's calls in the order of cpu_x86_linear_q6k_resolve (linear_q6k.c:84-156: the
-    int8 copy row by row, interleaved in eights or sixteens on a VNNI host) and
-    cpu_x86_linear_q6k_mN (:234-300: w4a8_quantize_acts_row per row, the sums again per sixteen,
-    then the kernel the host and the table's row count select). Returns (y, lanes)."""
-    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
-    m, n_out, nblk = x.shape[0], w_q6k.shape[0], n_in // 16
+def ref_q6k_mN_prepare(ref, w_q6k, n_in):
+    """cpu_x86_linear_q6k_resolve (linear_q6k.c:84-156) by the reference's own calls: the int8 copy
+    row by row, interleaved in eights or sixteens on a VNNI host. Returns run(x) -> (y, lanes),
+    which is cpu_x86_linear_q6k_mN (:234-300): w4a8_quantize_acts_row per row, the sums again per
+    sixteen, then the kernel the host and the table's row count select."""
+    n_out, nblk = w_q6k.shape[0], n_in // 16
     w = np.ascontiguousarray(w_q6k)
     row_bytes = n_in // 256 * 210
     vp = lambda a: a.ctypes.data_as(C.c_void_p)  # noqa: E731
@@ -680,25 +679,39 @@ def ref_q6k_linear_mN(ref, w_q6k, x, n_in):
                             C.c_void_p(wq.ctypes.data + r * n_in),
                             C.c_void_p(ws.ctypes.data + r * nblk * 4),
                             C.c_void_p(wo.ctypes.data + r * nblk * 4))
-    acts = np.zeros((m, n_in), dtype=np.int8)
-    sum_a = np.zeros((m, nblk), dtype=np.int32)
-    scale_x = np.zeros(m, dtype=np.float32)
-    for j in range(m):
-        scale_x[j] = ref.w4a8_quantize_acts_row(n_in, _fp(x[j]), C.c_void_p(acts.ctypes.data + j * n_in),
-                                                C.c_void_p(sum_a.ctypes.data + j * nblk * 4))
-        # linear_q6k.c:271-279: the sums again at the W8A8 granularity of sixteen
-        sum_a[j] = acts[j].reshape(nblk, 16).astype(np.int32).sum(axis=1)
-    y = np.full((m, n_out), np.nan, dtype=np.float32)
     lanes = bool(ref.w8a8_isa_is_vnni()) and n_out % 8 == 0
+    which = "w8x16" if n_out % 16 == 0 else "w8x8"
     if lanes:
         il_q, il_s, il_o = np.zeros_like(wq), np.zeros_like(ws), np.zeros_like(wo)
-        which = "w8x16" if n_out % 16 == 0 else "w8x8"
         getattr(ref, which + "_repack")(n_out, n_in, vp(wq), vp(ws), vp(wo), vp(il_q), vp(il_s), vp(il_o))
-        getattr(ref, which + "_gemm")(m, n_out, nblk, vp(il_q), vp(il_s), vp(il_o), vp(acts),
-                                      vp(sum_a), vp(scale_x), _fp(y))
-    else:
-        ref.w8a8_gemm(m, n_out, nblk, vp(wq), vp(ws), vp(wo), vp(acts), vp(sum_a), vp(scale_x), _fp(y))
-    return y, lanes
+
+    def run(x):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, n_in)
+        m = x.shape[0]
+        acts = np.zeros((m, n_in), dtype=np.int8)
+        sum_a = np.zeros((m, nblk), dtype=np.int32)
+        scale_x = np.zeros(m, dtype=np.float32)
+        for j in range(m):
+            scale_x[j] = ref.w4a8_quantize_acts_row(n_in, _fp(x[j]),
+                                                    C.c_void_p(acts.ctypes.data + j * n_in),
+                                                    C.c_void_p(sum_a.ctypes.data + j * nblk * 4))
+            # linear_q6k.c:271-279: the sums again at the W8A8 granularity of sixteen
+            sum_a[j] = acts[j].reshape(nblk, 16).astype(np.int32).sum(axis=1)
+        y = np.full((m, n_out), np.nan, dtype=np.float32)
+        if lanes:
+            getattr(ref, which + "_gemm")(m, n_out, nblk, vp(il_q), vp(il_s), vp(il_o), vp(acts),
+                                          vp(sum_a), vp(scale_x), _fp(y))
+        else:
+            ref.w8a8_gemm(m, n_out, nblk, vp(wq), vp(ws), vp(wo), vp(acts), vp(sum_a), vp(scale_x),
+                          _fp(y))
+        return y, lanes
+
+    return run
+
+
+def ref_q6k_linear_mN(ref, w_q6k, x, n_in):
+    """(y, lanes) of the reference's load-time copy and batch projection, see ref_q6k_mN_prepare."""
+    return ref_q6k_mN_prepare(ref, w_q6k, n_in)(x)
 
 
 def oracle_q8_sym_row_quantize(lib, x):
