@@ -112,8 +112,10 @@ int geist_hip_head_project_finalize_q8w(struct geist_hip_head *h, const float *d
  * geist_hip_head_set_projection chose the portable backend,
  * one row gets the logits of the x86 backend's decode kernel q6k_gemv_m1 instead
  * (src/backends/cpu_x86/kernel_q6k_gemv.c, resolved at src/backends/cpu_x86/backend.c:395-397),
- * again bit for bit; that backend's batch kernel, a GEMM over an int8 copy of the table
- * (src/backends/cpu_x86/linear_q6k.c:234-300), is not reproduced. Q4_K: below. The
+ * again bit for bit, and a batch those of its batch path cpu_x86_linear_q6k_mN
+ * (src/backends/cpu_x86/linear_q6k.c:234-300; see geist_hip_q6k_packed_linear_x86_rows: as a host
+ * with AVX-512 VNNI computes them, or in mode GEIST_HIP_PROJECTION_X86_AVX2 one without).
+ * Q4_K: below. The
  * other formats the reference resolves for an embedding table (I2_S, an F32 table) have
  * no device kernel here: their callers project on the host or with their own kernel and pass
  * the logits to geist_hip_head_finalize_one_row / _batch.

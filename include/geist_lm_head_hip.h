@@ -55,17 +55,20 @@ int geist_hip_f16_linear_rows(geist_hip_sampler *s, const uint16_t *d_w_f16, siz
 /* Which of the reference's backends the projection inside geist_hip_project_sample_rows (and
  * the head's project_finalize calls) stands for:
  *   GEIST_HIP_PROJECTION_X86       one row: f16_gemv_m1, over a Q6_K table q6k_gemv_m1, over a
- *                                  packed Q4_K table q4kx8_gemv_m1; more rows: over a packed
- *                                  Q4_K table cpu_x86_linear_q4k_mN as a host with AVX-512 runs
- *                                  it, over the other tables the portable kernel (default)
+ *                                  packed Q4_K table q4kx8_gemv_m1; more rows: over a Q6_K table
+ *                                  cpu_x86_linear_q6k_mN and over a packed Q4_K table
+ *                                  cpu_x86_linear_q4k_mN, as a host with AVX-512 (VNNI) runs
+ *                                  them, over the F16 table and its int8 form the portable
+ *                                  kernel (default)
  *   GEIST_HIP_PROJECTION_PORTABLE  the portable kernel for any number of rows, as on the
  *                                  reference's cpu_scalar backend (weight_resolve.c:247-252 sets
  *                                  linear_m1 and linear_mN alike)
  *   GEIST_HIP_PROJECTION_X86_AVX2  as _X86, for a host without AVX-512 (or one run with
- *                                  GEIST_FORCE_ISA=avx2): the only difference is a Q4_K batch of
- *                                  a multiple of 16 rows, which such a host sends through its AVX2
- *                                  kernel instead of the 16 x 16 tiles
- *                                  (kernel_q4kx8_gemm_avx512_full.c:816-835) */
+ *                                  GEIST_FORCE_ISA=avx2). Two differences: a Q4_K batch of a
+ *                                  multiple of 16 rows goes through the AVX2 kernel instead of
+ *                                  the 16 x 16 tiles (kernel_q4kx8_gemm_avx512_full.c:816-835),
+ *                                  and a Q6_K batch through the scalar W8A8 kernel instead of
+ *                                  the lane kernels (linear_q6k.c:61-63, 281-295) */
 #define GEIST_HIP_PROJECTION_X86 0
 #define GEIST_HIP_PROJECTION_PORTABLE 1
 #define GEIST_HIP_PROJECTION_X86_AVX2 2
@@ -212,10 +215,11 @@ int geist_hip_q6k_linear_x86_rows(geist_hip_sampler *s, const void *d_w_q6k, siz
                                   float *d_y, size_t ld_y);
 /* The tail of a forward pass over that table: geist_hip_rmsnorm_rows, the projection and the
  * sampler (soft-cap included) in one call, arguments as geist_hip_project_sample_rows. The
- * projection follows geist_hip_sampler_set_projection: in the default mode
- * GEIST_HIP_PROJECTION_X86 one row gets the x86 backend's decode kernel
- * (geist_hip_q6k_gemv_x86_rows / geist_hip_q6k_packed_gemv_x86_rows); a batch, and any call in
- * mode _PORTABLE, gets the portable arithmetic (geist_hip_q6k_linear_rows /
+ * projection follows geist_hip_sampler_set_projection: in the modes GEIST_HIP_PROJECTION_X86
+ * (default) and _X86_AVX2 one row gets the x86 backend's decode kernel
+ * (geist_hip_q6k_gemv_x86_rows / geist_hip_q6k_packed_gemv_x86_rows) and a batch its batch path
+ * (geist_hip_q6k_linear_x86_rows / geist_hip_q6k_packed_linear_x86_rows); any call in mode
+ * _PORTABLE gets the portable arithmetic (geist_hip_q6k_linear_rows /
  * geist_hip_q6k_packed_linear_rows). Over the packed copy and over the table as it lies in the
  * file the logits are the same bit for bit. */
 int geist_hip_project_sample_rows_q6k(geist_hip_sampler *s, const float *d_hidden,
