@@ -151,6 +151,22 @@ def reference_top_k_baseline(w, cores, budget_s):
                                       f"{res['1'][2]} on 1 thread"}
 
 
+def topk_path_counts(hs, row_sets, prm, d_u, d_out, n_rows):
+    """Which path served the rows of a top-k configuration, over every input copy once
+    (geist_hip_sampler_topk_paths after each call): the candidates handed on by the scan, the
+    per-thread maxima, the selection over the whole row; fallback_rate = the share of rows that
+    did not take the first."""
+    counts = {"scan_candidates": 0, "thread_maxima": 0, "whole_row": 0, "other": 0}
+    for rs in row_sets:
+        hs.sample(rs, prm, d_u, d_out)
+        for p in hs.topk_paths(n_rows).tolist():
+            counts[{0: "scan_candidates", 1: "thread_maxima", 2: "whole_row"}.get(p, "other")] += 1
+    total = max(1, sum(counts.values()))
+    counts["rows"] = total
+    counts["fallback_rate"] = round(1.0 - counts["scan_candidates"] / total, 6)
+    return counts
+
+
 def time_other_configs(steps=50, warmup=10):
     """The other four benchmark configurations under the same clock as the headline workload:
     `steps` HBM-cold steps each (the inputs rotate over copies that together exceed the Infinity
@@ -198,6 +214,8 @@ def time_other_configs(steps=50, warmup=10):
                      "step_frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      "step_algorithmic_bytes": int(alg), "kernel": k_name,
                      "kernel_us": round(k_us, 2), "steps": steps, "input_copies_rotated": n_copies}
+        if prm_kw.get("top_k"):
+            out[name]["topk_paths"] = topk_path_counts(hs, rl, prm, d_u, d_out, rows)
         hs.close()
 
     # cfg1: one row of 128256, N(0, 3^2), T = 0.8 (the rows of a [1400 x V] buffer take turns)
@@ -1276,6 +1294,8 @@ def main():
                      "step_algorithmic_bytes": alg_bytes,
                      "step_frac": round(alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }
+    if w.top_k:
+        result["topk_paths"] = topk_path_counts(hs, rows_cold, prm, d_u, d_out, w.rows)
     if scan_alone_us is not None:
         result["roofline"]["scan_kernel_of_two_launch_form"] = {
             "kernel": scan_alone_name, "kernel_us": round(scan_alone_us, 3),
