@@ -32,20 +32,21 @@
 
 namespace gs {
 
+constexpr int COOP_HISTS = 4; /* 0: the first step's, kept for the draw; 1..3 take turns */
 struct CoopRow {
-    uint32_t cnt[SG_BINS];
-    uint64_t mass[SG_BINS];
+    uint32_t cnt[COOP_HISTS][SG_BINS];
+    uint64_t mass[COOP_HISTS][SG_BINS];
     uint64_t aux[4];                /* sums of the first step, added by every workgroup (three used) */
     uint32_t chunk_cnt[MAX_CHUNKS]; /* entries equal to the drawn value, per chunk */
-    uint32_t arrive;
-    uint32_t epoch; /* number of the last step whose result is published */
-    int32_t  res_digit;
-    uint32_t res_cnt_above;
-    uint32_t res_ties;
-    uint32_t pad;
+    /* what a waiting workgroup reads with one 16-byte load: the number of the last step whose
+     * result is published, and that result's digit, count above and ties */
+    __attribute__((aligned(16))) uint32_t pub[4];
     uint64_t res_mass_above;
+    uint32_t arrive;
+    uint32_t pad;
 };
-static_assert(sizeof(CoopRow) % 8 == 0, "rows of the workspace stay 8-byte aligned");
+static_assert(sizeof(CoopRow) % 16 == 0, "rows of the workspace stay 16-byte aligned");
+static_assert(offsetof(CoopRow, pub) % 16 == 0, "the published record is one aligned 16-byte load");
 
 __device__ __forceinline__ uint32_t coop_ld32(const uint32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -58,6 +59,16 @@ __device__ __forceinline__ void coop_st32(uint32_t *p, uint32_t v) {
 }
 __device__ __forceinline__ void coop_st64(uint64_t *p, uint64_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+/* four dwords with one agent-scope load (16-byte aligned: one request, one moment) */
+typedef uint32_t coop_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ coop_u32x4 coop_ld128(const uint32_t *p) {
+    coop_u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=v"(v)
+                 : "v"(p)
+                 : "memory");
+    return v;
 }
 __device__ __forceinline__ void coop_add32(uint32_t *p, uint32_t v) {
     (void) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -90,8 +101,9 @@ __device__ __forceinline__ uint64_t pn_fx_bits(uint32_t key) {
 }
 
 struct CoopShared {
-    int last; /* this workgroup arrived last at the step's meeting */
-    int ok;   /* the step's result has been published */
+    int      last;   /* this workgroup arrived last at the step's meeting */
+    int      ok;     /* the step's result has been published */
+    uint32_t pub[4]; /* ... and what was published with it */
 };
 
 /* What the workgroup has added to the row's workspace is performed; true in the workgroup that
@@ -114,7 +126,7 @@ __device__ __forceinline__ void coop_publish(CoopRow *cr, uint32_t step) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0)
-        coop_st32(&cr->epoch, step);
+        coop_st32(&cr->pub[0], step);
 }
 /* Waits until the step is published; false when the wait ran out. */
 __device__ __forceinline__ bool coop_wait(const CoopRow *cr, uint32_t step, uint32_t limit,
@@ -123,7 +135,10 @@ __device__ __forceinline__ bool coop_wait(const CoopRow *cr, uint32_t step, uint
         int      ok = 0;
         uint32_t polls = 0;
         for (;;) {
-            if ((int32_t) (coop_ld32(&cr->epoch) - step) >= 0) {
+            const coop_u32x4 v = coop_ld128(cr->pub);
+            if ((int32_t) (v.x - step) >= 0) {
+                /* (the result was written and acknowledged before the number was) */
+                cs.pub[1] = v.y, cs.pub[2] = v.z, cs.pub[3] = v.w;
                 ok = 1;
                 break;
             }
@@ -139,6 +154,30 @@ __device__ __forceinline__ bool coop_wait(const CoopRow *cr, uint32_t step, uint
     return ok;
 }
 
+/* This workgroup's share of clearing histogram hb (a W-th of its bins). The stores are
+ * acknowledged before the workgroup arrives at its next meeting. */
+__device__ __forceinline__ void coop_clear_slice(CoopRow *cr, int hb, int chunk, int W) {
+    if (hb < 0)
+        return;
+    const int per = (SG_BINS + W - 1) / W;
+    const int end = (chunk + 1) * per < SG_BINS ? (chunk + 1) * per : SG_BINS;
+    for (int i = chunk * per + (int) threadIdx.x; i < end; i += TPB) {
+        coop_st32(&cr->cnt[hb][i], 0u);
+        coop_st64(&cr->mass[hb][i], 0ull);
+    }
+}
+
+/* The histograms of the steps that meet. The first step's goes to histogram 0, which stays until
+ * the draw's first level has been read from it; the others take turns through 1..3. A
+ * histogram is cleared by all workgroups, a slice each, while they wait at the NEXT meeting
+ * (everyone has read it by then: only the last arrival reads it, before it publishes), and is
+ * used again no sooner than three meetings later -- with a meeting in between at which every
+ * workgroup's clearing stores are acknowledged. */
+struct CoopTurn {
+    int hb;     /* this step's histogram */
+    int clr[2]; /* histograms to clear while waiting at this step's meeting, or -1 */
+};
+
 /* One level of a descent over the row: `add(key)` says whether an entry of this workgroup takes
  * part; its digit is (key >> shf) & dm. With `select` the last arrival picks the digit at which
  * the running mass reaches `target` and publishes it; mass_above / cnt_above / ties are updated
@@ -148,12 +187,12 @@ template <int NK, typename Take>
 __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, uint32_t limit,
                                           SortedGenShared &sh, CoopShared &cs,
                                           const uint32_t (&key)[NK], Take take, int shf,
-                                          uint32_t dm, bool select, bool clear_aux,
+                                          uint32_t dm, CoopTurn turn, bool select, bool clear_aux,
                                           uint64_t target, uint64_t &mass_above,
                                           uint32_t &cnt_above, uint32_t &ties, int &digit,
                                           int row, int chunk, int sbase) {
     const int tid = threadIdx.x;
-    (void) row, (void) chunk, (void) sbase;
+    (void) row, (void) sbase;
     for (int i = tid; i < SG_BINS; i += TPB) {
         sh.cnt[i]  = 0u;
         sh.mass[i] = 0ull;
@@ -174,8 +213,8 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
     for (int i = tid; i < SG_BINS; i += TPB) {
         const uint32_t c = sh.cnt[i];
         if (c) {
-            coop_add32(&cr->cnt[i], c);
-            coop_add64(&cr->mass[i], sh.mass[i]);
+            coop_add32(&cr->cnt[turn.hb][i], c);
+            coop_add64(&cr->mass[turn.hb][i], sh.mass[i]);
         }
     }
     ++step;
@@ -189,10 +228,10 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
             uint64_t      m[PER];
 #pragma unroll
             for (int q = 0; q < PER; ++q)
-                c[q] = coop_ld32(&cr->cnt[q * TPB + tid]);
+                c[q] = coop_ld32(&cr->cnt[turn.hb][q * TPB + tid]);
 #pragma unroll
             for (int q = 0; q < PER; ++q)
-                m[q] = coop_ld64(&cr->mass[q * TPB + tid]);
+                m[q] = coop_ld64(&cr->mass[turn.hb][q * TPB + tid]);
 #pragma unroll
             for (int q = 0; q < PER; ++q) {
                 sh.cnt[q * TPB + tid]  = c[q];
@@ -200,53 +239,114 @@ __device__ __forceinline__ int coop_level(CoopRow *cr, int W, uint32_t &step, ui
             }
         }
         __syncthreads();
-        for (int i = tid; i < SG_BINS; i += TPB) { /* for the next level */
-            if (sh.cnt[i]) {
-                coop_st32(&cr->cnt[i], 0u);
-                coop_st64(&cr->mass[i], 0ull);
-            }
-        }
-        if (clear_aux && tid < 4) /* (every workgroup has read them before it arrived here) */
-            coop_st64(&cr->aux[tid], 0ull);
         if (select)
             sg_select_digit(sh, target, mass_above, cnt_above);
         if (tid == 0) {
             const int d = select ? sh.res_digit : -1;
-            coop_st32(reinterpret_cast<uint32_t *>(&cr->res_digit), (uint32_t) d);
+            cs.pub[1] = (uint32_t) d;
+            coop_st32(&cr->pub[1], (uint32_t) d);
             if (d >= 0) {
-                coop_st32(&cr->res_cnt_above, sh.res_cnt_above);
+                cs.pub[2] = sh.res_cnt_above, cs.pub[3] = sh.cnt[d];
+                coop_st32(&cr->pub[2], sh.res_cnt_above);
+                coop_st32(&cr->pub[3], sh.cnt[d]);
                 coop_st64(&cr->res_mass_above, sh.res_mass_above);
-                coop_st32(&cr->res_ties, sh.cnt[d]);
             }
         }
         coop_publish(cr, step);
-    } else if (!coop_wait(cr, step, limit, cs)) {
-        return -1;
+        /* (behind the publication: the others are on their way already) */
+        if (clear_aux && tid < 4) /* (every workgroup has read them before it arrived here) */
+            coop_st64(&cr->aux[tid], 0ull);
+        coop_clear_slice(cr, turn.clr[0], chunk, W);
+        coop_clear_slice(cr, turn.clr[1], chunk, W);
+    } else {
+        coop_clear_slice(cr, turn.clr[0], chunk, W);
+        coop_clear_slice(cr, turn.clr[1], chunk, W);
+        if (!coop_wait(cr, step, limit, cs))
+            return -1;
     }
     GS_WSTAMP(sbase + 2);
-    /* (the last arrival reads its own stores back: program order, same addresses; the four
-     * loads go out together) */
-    digit                = (int) coop_ld32(reinterpret_cast<const uint32_t *>(&cr->res_digit));
-    const uint32_t r_cnt = coop_ld32(&cr->res_cnt_above);
-    const uint64_t r_mas = coop_ld64(&cr->res_mass_above);
-    const uint32_t r_tie = coop_ld32(&cr->res_ties);
+    /* the digit, the count above and the ties came with the step's number (cs.pub: written by
+     * thread 0 before a barrier in either branch); the mass above is loaded now and not needed
+     * before the next meeting's selection or the descent's end */
+    digit = (int) cs.pub[1];
     if (digit < 0)
         return 0;
-    cnt_above  = r_cnt;
-    mass_above = r_mas;
-    ties       = r_tie;
+    cnt_above  = cs.pub[2];
+    ties       = cs.pub[3];
+    mass_above = cs.last ? sh.res_mass_above : coop_ld64(&cr->res_mass_above);
     return 1;
+}
+
+/* The first level of the draw's descent without a meeting. The first step's histogram (every
+ * entry of the row by the leading 11 bits of its key, histogram 0) holds what that level would
+ * collect again: the digits above the edge's are the same, those below it are empty, and the
+ * edge's own digit holds the entries greater than the edge -- their count and mass, gt_cnt and
+ * gt_mass, less those of the digits above -- and the block of limit_ties entries equal to it.
+ * Every workgroup reads the histogram and selects for itself (integers: the same result in
+ * all). Returns 1 with the digit, or 0 (the target is not reached). */
+__device__ __forceinline__ int coop_first_level_local(const CoopRow *cr, SortedGenShared &sh,
+                                                      uint64_t target, bool limited,
+                                                      uint32_t limit_key, uint32_t limit_ties,
+                                                      uint32_t gt_cnt, uint64_t gt_mass,
+                                                      uint64_t &mass_above, uint32_t &cnt_above,
+                                                      uint32_t &ties, int &digit) {
+    const int     tid = threadIdx.x;
+    constexpr int PER = SG_BINS / TPB;
+    const int     de  = limited ? (int) (limit_key >> 21) : -1;
+    uint32_t      c[PER];
+    uint64_t      m[PER];
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+        c[q] = coop_ld32(&cr->cnt[0][q * TPB + tid]);
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+        m[q] = coop_ld64(&cr->mass[0][q * TPB + tid]);
+    uint64_t above_c = 0ull, above_m = 0ull;
+#pragma unroll
+    for (int q = 0; q < PER; ++q) {
+        const int i = q * TPB + tid;
+        if (i > de) {
+            above_c += c[q];
+            above_m += m[q];
+        } else {
+            c[q] = 0u, m[q] = 0ull;
+        }
+        sh.cnt[i]  = c[q];
+        sh.mass[i] = m[q];
+    }
+    if (limited) {
+        above_c = block_sum_u64(above_c, sh.red64);
+        above_m = block_sum_u64(above_m, sh.red64);
+        if (tid == 0) {
+            sh.cnt[de]  = gt_cnt - (uint32_t) above_c + limit_ties;
+            sh.mass[de] = gt_mass - above_m + pn_fx(__uint_as_float(limit_key)) * (uint64_t) limit_ties;
+        }
+    }
+    __syncthreads();
+    sg_select_digit(sh, target, 0ull, 0u);
+    const int d = sh.res_digit;
+    if (d >= 0) {
+        mass_above = sh.res_mass_above;
+        cnt_above  = sh.res_cnt_above;
+        ties       = sh.cnt[d];
+    }
+    digit = d;
+    __syncthreads();
+    return d >= 0 ? 1 : 0;
 }
 
 /* Three levels (11, 11, 10 bits of the key): sg_descent over the row's workgroups. `lead` is
  * the row's first workgroup, which adds the block of limit_ties entries equal to limit_key.
- * Returns 1 / 0 / -1 as coop_level. */
+ * `meet` counts the row's meetings so far (it picks the histograms, see CoopTurn). With
+ * `local_first` the first level is coop_first_level_local. `last` is the row's last descent: its
+ * last level also clears histogram 0. Returns 1 / 0 / -1 as coop_level. */
 template <int NK>
 __device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, uint32_t limit,
                                             SortedGenShared &sh, CoopShared &cs,
                                             const uint32_t (&key)[NK], bool lead, bool clear_aux,
                                             uint64_t target, bool limited, uint32_t limit_key,
-                                            uint32_t limit_ties,
+                                            uint32_t limit_ties, int &meet, bool local_first,
+                                            uint32_t gt_cnt, uint64_t gt_mass, bool last,
                                             uint32_t &kappa, uint32_t &cnt_above,
                                             uint64_t &mass_above, uint32_t &ties_total,
                                             int row, int chunk, int sbase) {
@@ -258,6 +358,23 @@ __device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, 
     for (int lv = 0; lv < 3; ++lv) {
         const int      shf = lv == 0 ? 21 : lv == 1 ? 10 : 0;
         const uint32_t dm  = lv == 2 ? 1023u : 2047u;
+        if (lv == 0 && local_first) {
+            int       digit = -1;
+            const int r = coop_first_level_local(cr, sh, target, limited, limit_key, limit_ties,
+                                                 gt_cnt, gt_mass, mass_above, cnt_above,
+                                                 ties_total, digit);
+            if (r <= 0)
+                return r;
+            prefix |= (uint32_t) digit << shf;
+            mask |= dm << shf;
+            continue;
+        }
+        /* meeting number `meet` (0 = the row's first): its histogram, and what it clears */
+        CoopTurn turn;
+        turn.hb     = meet == 0 ? 0 : 1 + (meet - 1) % 3;
+        turn.clr[0] = meet >= 2 ? 1 + (meet - 2) % 3 : -1; /* the meeting before, unless the first */
+        turn.clr[1] = last && lv == 2 ? 0 : -1;
+        ++meet;
         /* the block of entries equal to the limit, as one more key of the first workgroup's
          * first thread: handled apart, its mass is limit_ties times the entry's */
         const bool block_here = limited && lead && threadIdx.x == 0 && limit_ties &&
@@ -269,13 +386,13 @@ __device__ __forceinline__ int coop_descent(CoopRow *cr, int W, uint32_t &step, 
          * entry would cost every level a register; it goes straight to the global histogram */
         if (block_here) {
             const uint32_t d = (limit_key >> shf) & dm;
-            coop_add32(&cr->cnt[d], limit_ties);
-            coop_add64(&cr->mass[d], pn_fx(__uint_as_float(limit_key)) * (uint64_t) limit_ties);
+            coop_add32(&cr->cnt[turn.hb][d], limit_ties);
+            coop_add64(&cr->mass[turn.hb][d], pn_fx(__uint_as_float(limit_key)) * (uint64_t) limit_ties);
         }
         int       digit = -1;
-        const int r = coop_level<NK>(cr, W, step, limit, sh, cs, key, take, shf, dm, true,
-                                     clear_aux && lv == 0, target, mass_above, cnt_above,
-                                     ties_total, digit, row, chunk, sbase + 3 * lv);
+        const int r = coop_level<NK>(cr, W, step, limit, sh, cs, key, take, shf, dm, turn, true,
+                                     clear_aux && lv == (local_first ? 1 : 0), target, mass_above,
+                                     cnt_above, ties_total, digit, row, chunk, sbase + 3 * lv);
         if (r <= 0)
             return r;
         prefix |= (uint32_t) digit << shf;
@@ -414,12 +531,12 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     uint32_t kappa = 0u, cnt_above = 0u, ties = 0u;
     uint64_t mass_above = 0ull;
     const uint64_t target = (uint64_t) __double2ull_ru((double) top_p * 0x1p62);
-    int      r;
+    int      r, meet = 0;
     {
         /* (the three levels of coop_descent, the first of them also carrying the sums above) */
         r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, false,
-                                 use_p ? target : ~0ull, false, 0u, 0u, kappa, cnt_above,
-                                 mass_above, ties, row, chunk, 8);
+                                 use_p ? target : ~0ull, false, 0u, 0u, meet, false, 0u, 0ull,
+                                 false, kappa, cnt_above, mass_above, ties, row, chunk, 8);
         if (r < 0) {
             alone(true);
             return;
@@ -430,9 +547,15 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     uint32_t       n_m    = (uint32_t) coop_ld64(&cr->aux[1]);
     const uint64_t mass_all = coop_ld64(&cr->aux[2]);
     uint64_t mass_m_use = mass_m;
+    /* the draw's first level can be read off the first step's histogram when the count and mass
+     * of the entries above the edge are at hand */
+    bool     local_first = true;
+    uint32_t gt_cnt = 0u;
+    uint64_t gt_mass = 0ull;
     if (use_m && n_m < 1u) {
-        n_m        = 1u;
-        mass_m_use = pn_fx(__uint_as_float(kmax));
+        n_m         = 1u;
+        mass_m_use  = pn_fx(__uint_as_float(kmax));
+        local_first = false;
     }
     /* ---- the kept prefix, as sorted_descend<false> decides it ---- */
     bool     limited   = false;
@@ -453,12 +576,16 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
         edge_ties = (uint32_t) j;
         n_keep    = cnt_above + (uint32_t) j;
         mass_keep = mass_above + each * j;
+        gt_cnt    = cnt_above;
+        gt_mass   = mass_above;
     }
     if (use_m && (!have_p || n_m < n_keep)) {
         limited   = true;
         mass_keep = mass_m_use;
         edge_key  = __float_as_uint(floor_w) ? __float_as_uint(floor_w) - 1u : 0u;
         edge_ties = 0u;
+        gt_cnt    = n_m;
+        gt_mass   = mass_m_use;
         if (__float_as_uint(floor_w) == 0u)
             limited = false;
     } else if (!have_p) {
@@ -470,8 +597,8 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
     uint32_t       kd = 0u, cnt_above_d = 0u, ties_d = 0u;
     uint64_t       mass_above_d = 0ull;
     r = coop_descent<4 * NV>(cr, W, step, wait_limit, sh, cs, key, lead, true, target2, limited,
-                             edge_key, edge_ties, kd, cnt_above_d, mass_above_d, ties_d, row, chunk,
-                             17);
+                             edge_key, edge_ties, meet, local_first, gt_cnt, gt_mass, true, kd,
+                             cnt_above_d, mass_above_d, ties_d, row, chunk, 17);
     if (r <= 0) { /* 0: not reachable with exact integer masses; the one-workgroup walk decides */
         alone(true);
         return;
@@ -496,12 +623,17 @@ __global__ __launch_bounds__(TPB, 2) void k_whole_row_coop(RowView rv, SortedRow
             coop_st32(&cr->chunk_cnt[chunk], here);
     }
     ++step;
+    const int last_hb = 1 + (meet - 2) % 3; /* (the draw's last level met: meet >= 3) */
     if (coop_arrive(cr, W, cs)) {
         GS_WSTAMP(5);
         coop_publish(cr, step);
-    } else if (!coop_wait(cr, step, wait_limit, cs)) {
-        alone(true);
-        return;
+        coop_clear_slice(cr, last_hb, chunk, W);
+    } else {
+        coop_clear_slice(cr, last_hb, chunk, W);
+        if (!coop_wait(cr, step, wait_limit, cs)) {
+            alone(true);
+            return;
+        }
     }
     /* the entries in the chunks before this one (a thread per chunk, then their sum) */
     const uint64_t before =
