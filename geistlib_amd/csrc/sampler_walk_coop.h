@@ -7,21 +7,24 @@
  * a pass is: every workgroup adds its share to a histogram of the row in global memory
  * (agent-scope atomics; sums of integers, so their order does not matter), the workgroups meet at
  * the row's arrival counter, the one that arrives last reads the histogram, selects the digit as
- * the one-workgroup walk does (sg_select_digit), clears the histogram and publishes the result
- * with the step's number; the others wait for that number. The steps: the first level of the
- * nucleus descent together with the min-p sums, its two further levels, the three levels of the
- * draw's descent, and the index-order count that finds the j-th entry equal to the drawn value.
- * The arithmetic is that of sorted_descend<false> (sampler_sorted_prob.h) step for step: masses
- * in 2^-62 fixed point, the same targets, the same edge rules.
+ * the one-workgroup walk does (sg_select_digit) and publishes the result with the step's number
+ * in one 16-byte record; the others wait for that number. The steps: the first level of the
+ * nucleus descent together with the min-p sums, its two further levels, the draw's descent --
+ * whose first level is read off the first step's histogram without a meeting
+ * (coop_first_level_local), two levels meet --, and the index-order count that finds the j-th
+ * entry equal to the drawn value. The histograms take turns, and each is cleared by the waiting
+ * workgroups of the meeting after its own (CoopTurn). The arithmetic is that of
+ * sorted_descend<false> (sampler_sorted_prob.h) step for step: masses in 2^-62 fixed point, the
+ * same targets, the same edge rules.
  *
  * No fences: a workgroup's atomics are acknowledged (s_waitcnt vmcnt(0)) before it arrives, and
  * what the last arrival publishes is written and read with agent-scope accesses. Every wait is
  * bounded (`wait_limit` polls); a workgroup whose wait runs out leaves -- it is then missed at the
  * next meeting, where the others' waits run out in turn --, the row keeps its flag, and the
  * one-workgroup walk that the host launches behind this kernel serves it: a row is always served,
- * whatever the others do. The last step has no wait: the workgroup that arrives last finds the chunk
- * that holds the drawn entry and, if it is not its own, forms that chunk's probabilities once
- * more. The row's workspace is zero before the first launch and left zero by every launch that
+ * whatever the others do. At the last step every workgroup reports how many entries equal to the
+ * drawn value its chunk holds, and once all have, the one whose chunk holds the j-th of them in
+ * index order writes the token. The row's workspace is zero before the first launch and left zero by every launch that
  * ends without a wait running out (steps are numbered on from `step_base`, so the published
  * number needs no clearing); a launch in which one did says so in the host's hint words (the
  * call's number: in word 0 when a row was walked in full, in word 1 when a wait ran out), and the
