@@ -153,6 +153,31 @@ def test_q4k_decode_refuses_shapes_the_x86_kernel_does_not_take(hs):
         hs.q4k_packed_gemv_x86(packed, 12, 256, x, y)
 
 
+def test_q4k_x86_argument_errors(hs):
+    from geistlib_amd.binding import GeistHipError
+    packed = torch.zeros((hs.q4k_packed_bytes(8, 256) + 16,), dtype=torch.uint8, device="cuda")
+    x = torch.zeros((4, 256), dtype=torch.float32, device="cuda")
+    y = torch.full((4, 8), 7.0, dtype=torch.float32, device="cuda")
+    hs.q4k_packed_linear_x86(packed, 8, 256, x, y)
+    hs.sync()
+    assert not y.cpu().numpy().any()                          # zeros: scale 1, every product 0
+    f = hs.lib.geist_hip_q4k_packed_linear_x86_rows
+    with pytest.raises(GeistHipError):                        # 12 rows: not a multiple of 8
+        hs._check(f(hs.h, packed.data_ptr(), 12, 256, x.data_ptr(), 256, 4, y.data_ptr(), 12))
+    with pytest.raises(GeistHipError):                        # packed copy not 16-byte aligned
+        hs._check(f(hs.h, packed.data_ptr() + 4, 8, 256, x.data_ptr(), 256, 4, y.data_ptr(), 8))
+    with pytest.raises(GeistHipError):                        # rows closer than their length
+        hs._check(f(hs.h, packed.data_ptr(), 8, 256, x.data_ptr(), 128, 4, y.data_ptr(), 8))
+    with pytest.raises(GeistHipError):                        # no rows
+        hs._check(f(hs.h, packed.data_ptr(), 8, 256, x.data_ptr(), 256, 0, y.data_ptr(), 8))
+    act = torch.zeros((hs.q8k_row_act_bytes(256) + 64,), dtype=torch.uint8, device="cuda")
+    with pytest.raises(GeistHipError):                        # activations not 64-byte aligned
+        hs._check(hs.lib.geist_hip_q8k_row_quantize(hs.h, x.data_ptr(), 256, act.data_ptr() + 4))
+    with pytest.raises(GeistHipError):                        # not a whole number of blocks
+        hs._check(hs.lib.geist_hip_q8k_row_quantize(hs.h, x.data_ptr(), 200, act.data_ptr()))
+    assert hs.q8k_row_act_bytes(200) == 0 and hs.q8k_row_act_bytes(256) == (72 + 8) * 4
+
+
 def test_q4k_linear_rows_whose_sums_cancel(hs, oracle):
     """Activations that repeat with alternating sign make pairs of products cancel: sums close to
     rounding boundaries, which only the reference's order of additions gets right."""

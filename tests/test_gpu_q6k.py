@@ -221,6 +221,25 @@ def test_q6k_argument_errors(hs):
     with pytest.raises(GeistHipError):                       # table not 4-byte aligned
         hs._check(hs.lib.geist_hip_q6k_linear_rows(hs.h, w.data_ptr() + 2, 3, 256, x.data_ptr(),
                                                    256, 1, y.data_ptr(), 4))
+    # the x86 backend's batch path: the same rules
+    x2 = torch.zeros((2, 256), dtype=torch.float32, device="cuda")
+    y2 = torch.full((2, 4), 7.0, dtype=torch.float32, device="cuda")
+    hs.q6k_linear_x86(w, 256, x2, y2)
+    hs.sync()
+    assert not y2.cpu().numpy().any()                        # zeros: scale 1, every product 0
+    packed = torch.zeros((hs.q6k_packed_bytes(4, 256) + 16,), dtype=torch.uint8, device="cuda")
+    for fn, table in ((hs.lib.geist_hip_q6k_linear_x86_rows, w.data_ptr() + 2),         # alignment
+                      (hs.lib.geist_hip_q6k_packed_linear_x86_rows, packed.data_ptr() + 4)):
+        with pytest.raises(GeistHipError):
+            hs._check(fn(hs.h, table, 4, 256, x2.data_ptr(), 256, 2, y2.data_ptr(), 4))
+    with pytest.raises(GeistHipError):                       # rows closer than their length
+        hs._check(hs.lib.geist_hip_q6k_packed_linear_x86_rows(hs.h, packed.data_ptr(), 4, 256,
+                                                              x2.data_ptr(), 128, 2, y2.data_ptr(), 4))
+    with pytest.raises(GeistHipError):                       # no rows
+        hs._check(hs.lib.geist_hip_q6k_packed_linear_x86_rows(hs.h, packed.data_ptr(), 4, 256,
+                                                              x2.data_ptr(), 256, 0, y2.data_ptr(), 4))
+    with pytest.raises(GeistHipError):                       # an unknown projection mode
+        hs.set_projection(3)
 
 
 def test_head_over_the_gemma_table_with_the_soft_cap(host, oracle):
