@@ -515,7 +515,11 @@ static int check_call(geist_hip_sampler *s, const struct geist_hip_rows *rows,
 /* The meeting slots for a launch of rows * n_chunks workgroups (`words` per workgroup): this
  * launch takes the array whose turn it is, which the launch before left zero, and zeroes what
  * that launch used in the other. */
-static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t words = 1) {
+/* `one_xcd`: the launch deals the workgroups that meet to one XCD (rows in eights,
+ * xcd_row_chunk); where the device was seen to place them so they meet through that XCD's L2
+ * (MeetSpace::local). geist_hip_sampler_handoff_scope(s, 1) switches that off as well. */
+static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t words = 1,
+                            bool one_xcd = false) {
     MeetState &st = *s->meet;
     if (st.suspect) { /* only after a failed launch: start again from two zeroed arrays */
         for (int t = 0; t < 2; ++t)
@@ -535,12 +539,14 @@ static MeetSpace meet_space(geist_hip_sampler *s, const Launch &L, uint32_t word
         m.stale       = st.recorded;
         m.stale_count = 0;
         m.wait_limit  = s->wait_limit;
+        m.local       = one_xcd && s->fused_wg_default != 0 && !s->handoff_far;
         return m;
     }
     m.slots       = st.slots[st.turn];
     m.stale       = st.slots[st.turn ^ 1];
     m.stale_count = st.used[st.turn ^ 1];
     m.wait_limit  = s->wait_limit;
+    m.local       = one_xcd && s->fused_wg_default != 0 && !s->handoff_far;
     st.used[st.turn]     = words * (uint32_t) L.rows * (uint32_t) L.rv.n_chunks;
     st.used[st.turn ^ 1] = 0;
     st.turn ^= 1;
@@ -774,13 +780,15 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
              * stages cannot split it: the streaming stage is the whole step. */
             *stream_kernel = "k_temperature_draw";
             if (do_stream)
-                launch_temperature_draw(scan, rs.inv_t, d_uniforms, d_out, meet_space(s, scan, 2));
+                launch_temperature_draw(scan, rs.inv_t, d_uniforms, d_out,
+                                        meet_space(s, scan, 2, true));
             return after_launch(s, "temperature");
         }
         *stream_kernel = "k_scan_expsum";
         if (do_stream &&
             launch_scan_expsum(scan, rs.inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0,
-                               nullptr, nullptr, 0, s->slab_sum, meet_space(s, scan)))
+                               nullptr, nullptr, 0, s->slab_sum,
+                               meet_space(s, scan, 1, (scan.rows & 7) == 0)))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
         f.mode     = FINAL_TEMPERATURE;
         f.slab_sum = s->slab_sum;
@@ -816,7 +824,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
          * alone nobody reads them) */
         launch_scan_expsum(scan, rs.inv_t, f.minp_direct ? nullptr : s->tmax, s->chunk_best,
                            s->chunk_sum, nullptr, 0, nullptr, f.minp_listed ? &f.cand : nullptr,
-                           zb_m, nullptr, meet_space(s, scan)))
+                           zb_m, nullptr, meet_space(s, scan, 1, (scan.rows & 7) == 0)))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     if (!do_tail)
         return after_launch(s, "exp-sum scan");
@@ -1127,7 +1135,7 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
     if (launch_scan_expsum(L, inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
-                           nullptr, 0, nullptr, meet_space(s, L)))
+                           nullptr, 0, nullptr, meet_space(s, L, 1, (L.rows & 7) == 0)))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
@@ -2087,7 +2095,8 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
         /* no slab sums: of the n_seq * (L + 1) rows at most n_seq are drawn from, each by a
          * workgroup that walks the located chunk from its start */
         if (launch_scan_expsum(scan, inv_t, nullptr, s->chunk_best, s->chunk_sum, d_draft, (int) L,
-                               s->probe_p, nullptr, 0, nullptr, meet_space(s, scan)))
+                               s->probe_p, nullptr, 0, nullptr,
+                               meet_space(s, scan, 1, (scan.rows & 7) == 0)))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     }
     SpecLaunch sp{};

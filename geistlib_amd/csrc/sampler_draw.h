@@ -111,12 +111,11 @@ struct DrawShared {
  * not even have started): sh.have_sums = 0. Ends with a barrier. */
 __device__ __forceinline__ void row_sums_meet(uint64_t *row_slots, int chunk, int C, double total,
                                               bool reporter, bool wait, uint32_t wait_limit,
-                                              DrawShared &sh) {
+                                              DrawShared &sh, uint32_t local = 0) {
     const int lane = threadIdx.x & (WAVE - 1);
     if (reporter) {
         if (lane == 0)
-            __hip_atomic_store(row_slots + chunk, (uint64_t) __double_as_longlong(total) + 1u,
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            meet_store(row_slots + chunk, (uint64_t) __double_as_longlong(total) + 1u, local);
         uint64_t a = 0, b = 0;
         uint32_t polls = 0;
         bool     met   = wait;
@@ -224,7 +223,7 @@ __device__ __forceinline__ void draw_chunk(const RowView &rv, int row, int chunk
         sh.total = combine_slab_totals<NV>(s_sum, sh.slab);
     /* (the reporter's lane 0 wrote sh.total: its own LDS write, read back in order) */
     row_sums_meet(sum_slots + (long) row * C, chunk, C, last2 ? sh.total : 0.0, last2, met_max,
-                  fs.wait_limit, sh);
+                  fs.wait_limit, sh, fs.local);
     const bool from_registers = sh.have_sums != 0;
     if (!from_registers) {
         /* not met: every other chunk's sum by this workgroup, with the same summation */
@@ -300,7 +299,7 @@ __device__ __forceinline__ void draw_chunk(const RowView &rv, int row, int chunk
 }
 
 template <int NV, bool PEN>
-__global__ __launch_bounds__(TPB) void k_temperature_draw(RowView rv, float inv_t,
+__global__ __launch_bounds__(TPB) void k_temperature_draw(RowView rv, int n_rows, float inv_t,
                                                           const float *__restrict__ uniforms,
                                                           int32_t *__restrict__ out,
                                                           MeetSpace meet) {
@@ -323,6 +322,8 @@ __global__ __launch_bounds__(TPB) void k_temperature_draw(RowView rv, float inv_
         for (uint32_t i = wg * TPB + tid; i < meet.stale_count; i += n_wg * TPB)
             meet.stale[i] = 0;
     }
+    if (row >= n_rows) /* the grid holds the rows in eights */
+        return;
     int base, end;
     chunk_bounds<NV>(rv, chunk, base, end);
     FusedScan fs;
@@ -330,17 +331,18 @@ __global__ __launch_bounds__(TPB) void k_temperature_draw(RowView rv, float inv_
     fs.chunk_best = nullptr;
     fs.slots      = meet.slots;
     fs.wait_limit = meet.wait_limit;
+    fs.local      = meet.local;
     fs.s_red      = s_red;
     fs.s_bb       = &s_bb;
     fs.s_arrive   = s_arrive;
-    uint64_t  *sum_slots = meet.slots + (long) gridDim.y * rv.n_chunks;
+    uint64_t  *sum_slots = meet.slots + (long) n_rows * rv.n_chunks;
     const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
                        rv.allowed == nullptr;
     if (plain)
-        draw_chunk<NV, PEN, true>(rv, row, chunk, (int) gridDim.y, base, end, inv_t, uniforms, out,
+        draw_chunk<NV, PEN, true>(rv, row, chunk, n_rows, base, end, inv_t, uniforms, out,
                                   sum_slots, s_cnt16, s_sum, s_tab, tabv, s_tr, s_draw, fs);
     else
-        draw_chunk<NV, PEN, false>(rv, row, chunk, (int) gridDim.y, base, end, inv_t, uniforms, out,
+        draw_chunk<NV, PEN, false>(rv, row, chunk, n_rows, base, end, inv_t, uniforms, out,
                                    sum_slots, s_cnt16, s_sum, s_tab, tabv, s_tr, s_draw, fs);
 }
 

@@ -48,6 +48,13 @@ struct MeetSpace {
     uint64_t *stale;       /* the slots of the launch before, zeroed by this one */
     uint32_t  stale_count;
     uint32_t  wait_limit;  /* polls before a workgroup reads the row for itself; 0 = do not wait */
+    uint32_t  local;       /* the workgroups that meet run on one XCD (the grid deals a row's
+                            * workgroups to one, and the device was seen to place them so): a slot
+                            * is written with a plain store, which that XCD's L2 holds and serves
+                            * to the polls -- a device-scope store is written through to memory
+                            * first (a meeting of 63 workgroups: 0.6 against 2.5 us). Should the
+                            * workgroups not share an XCD after all, the polls never see the slot,
+                            * the bounded wait runs out and each workgroup reads the row itself. */
 };
 
 /* Where a sampling step reports that the ids of all its rows are written: `epoch` goes into

@@ -208,6 +208,7 @@ struct FusedScan {
     uint64_t *chunk_best;
     uint64_t *slots;
     uint32_t  wait_limit;
+    uint32_t  local;    /* MeetSpace::local */
     uint64_t *s_red;    /* LDS, NWAVES words */
     uint64_t *s_bb;     /* LDS, one word */
     uint32_t *s_arrive; /* LDS, three arrival counters (and a fourth word), zero and published
@@ -230,6 +231,13 @@ struct FusedScan {
  * workgroups have neighbouring ids and are started together; the wait is bounded all the same:
  * past `wait_limit` polls (0: at once) the workgroup stops waiting and finds the row's maximum
  * itself by reading the whole row, so every workgroup ends whatever the others do. */
+/* A workgroup's word into its meeting slot: see MeetSpace::local. */
+__device__ __forceinline__ void meet_store(uint64_t *slot, uint64_t v, uint32_t local) {
+    if (local)
+        *reinterpret_cast<volatile uint64_t *>(slot) = v;
+    else
+        __hip_atomic_store(slot, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 template <int NV, bool PEN>
 __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, int chunk,
                                                   int n_rows, uint64_t mine, bool reporter,
@@ -241,8 +249,7 @@ __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, in
     uint64_t *row_slots = fs.slots + (long) row * C;
     if (reporter) { /* one wavefront, all its lanes */
         if (lane == 0)
-            __hip_atomic_store(row_slots + chunk, mine, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+            meet_store(row_slots + chunk, mine, fs.local);
         uint64_t a = 0, b = 0;
         uint32_t polls = 0;
         bool     met   = fs.wait_limit != 0;
@@ -597,6 +604,7 @@ __global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan
     fs.chunk_best = chunk_best;
     fs.slots      = meet.slots;
     fs.wait_limit = meet.wait_limit;
+    fs.local      = meet.local;
     fs.s_red      = s_red;
     fs.s_bb       = &s_bb;
     fs.s_arrive   = s_arrive;
@@ -1856,12 +1864,14 @@ int zbin_of_min_p(float min_p) {
 
 void launch_temperature_draw(const Launch &L, float inv_t, const float *uniforms, int32_t *out,
                              const MeetSpace &meet) {
-    /* for launches of a few rows: the geometry of 2048 elements per workgroup only */
-    const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    /* for launches of a few rows: the geometry of 2048 elements per workgroup only. Rows in
+     * eights, so that the workgroups of a row have linear ids equal modulo 8 and share an XCD
+     * (xcd_row_chunk); the workgroups of the rows that are not there leave at once. */
+    const dim3 grid(L.rv.n_chunks, (L.rows + 7) & ~7), block(TPB);
     if (L.pen)
-        k_temperature_draw<2, true><<<grid, block, 0, L.stream>>>(L.rv, inv_t, uniforms, out, meet);
+        k_temperature_draw<2, true><<<grid, block, 0, L.stream>>>(L.rv, L.rows, inv_t, uniforms, out, meet);
     else
-        k_temperature_draw<2, false><<<grid, block, 0, L.stream>>>(L.rv, inv_t, uniforms, out, meet);
+        k_temperature_draw<2, false><<<grid, block, 0, L.stream>>>(L.rv, L.rows, inv_t, uniforms, out, meet);
 }
 
 void launch_spec(const Launch &L, const SpecLaunch &sp, const MeetSpace *meet) {

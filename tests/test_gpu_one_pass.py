@@ -70,6 +70,37 @@ def test_waiting_and_not_waiting_give_the_oracles_ids(hs, oracle, rows, n, kw, p
         assert near <= 1
 
 
+@pytest.mark.parametrize("far", [False, True])
+@pytest.mark.parametrize("rows,n,kw,pen", [CASES[1], CASES[2], CASES[4], CASES[6], (4, 128256, dict(temperature=0.9), True)])
+def test_meeting_in_the_shared_l2_or_through_memory(hs, oracle, rows, n, kw, pen, far):
+    """Where a launch deals the workgroups of a row to one XCD they write their meeting slots
+    with plain stores, which that XCD's L2 serves to the polls; geist_hip_sampler_handoff_scope
+    (1) makes them store through to memory as launches of other shapes do. The ids are the
+    oracle's both ways, on two calls in a row (the slot arrays take turns)."""
+    print(f"meeting rows={rows} n={n} {kw} pen={pen} far={far}", flush=True)
+    g = np.random.default_rng(rows * 11 + n)
+    x = (g.standard_normal((rows, n)) * 2.5).astype(np.float32)
+    hist = hl = None
+    pk = {}
+    if pen:
+        hist, hl = history_for(g, max(rows, 2), n)
+        hist, hl = hist[:rows], hl[:rows]
+        pk = dict(rep=1.2, freq=0.4, pres=0.2)
+    hs.handoff_scope(far)
+    try:
+        for call in range(2):
+            u = g.random(rows).astype(np.float32)
+            got = run_rows(hs, torch, x, u, P(**kw, **pk), history=hist, history_len=hl)
+            res = []
+            for r in range(rows):
+                row = oracle.penalties(x[r], hist[r, :hl[r]], 1.2, 0.4, 0.2) if pen else x[r]
+                res.append(oracle.chain_u(row, float(u[r]), **kw))
+            near = compare_ids(got, [t for t, _ in res], [i for _, i in res], f"call {call}")
+            assert near <= 1
+    finally:
+        hs.handoff_scope(False)
+
+
 @pytest.mark.parametrize("wait_limit", [None, 0])
 def test_normalised_probabilities_one_pass(hs, oracle, wait_limit):
     rows, n, T = 4, 70001, 0.9
