@@ -51,6 +51,10 @@ def build_workload(name):
         return W.config2(with_penalties=True)
     if name == "cfg2":
         return W.config2(with_penalties=False)
+    if name.startswith("cfg2_pen_b") or name.startswith("cfg2_b"):
+        # the headline's parameters on another number of rows (cfg2_pen_b1: one decode step of
+        # one session, which is what the reference's geist_session_decode_step samples)
+        return W.config2(rows=int(name.split("_b")[1]), with_penalties=name.startswith("cfg2_pen"))
     if name == "cfg3":
         return W.config3()
     if name == "cfg4":
@@ -222,6 +226,11 @@ def time_other_configs(steps=50, warmup=10):
     big = normal((1400, 128256), 3.0)
     run("cfg1", iter([big[i:i + 1] for i in range(1400)]).__next__, 1400, 1, 128256,
         dict(temperature=0.8))
+    # one decode step of one session, which is what the reference's sample call serves
+    # (geist_session_decode_step): one row with the headline's parameters and penalties
+    run("decode_one_row", iter([big[i:i + 1] for i in range(1400)]).__next__, 1400, 1, 128256,
+        dict(temperature=0.7, top_k=40, top_p=0.9, rep=1.1, freq=0.5, pres=0.3), hist_len=2048,
+        extra_bytes=4 * 2048 + 8 * 1000)
     del big
     # cfg3: 128 x 151936, N(0, 2^2), Zipf history of 2048, penalties, T = 1, top-p 0.95, min-p 0.05
     hist_bytes = 128 * (4 * 2048 + 8 * 1000)   # ids read + about 1000 distinct per row gathered

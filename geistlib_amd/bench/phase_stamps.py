@@ -1,14 +1,14 @@
 """Where the time goes inside k_cand_scan_final: device timestamps of an instrumented build.
 
     make -C geistlib_amd phase-stamps [STAMP_MASK=0x...]
-    GEIST_HIP_LIB_DIR=geistlib_amd/lib/stamps python3 geistlib_amd/bench/phase_stamps.py [--no-pen]
+    GEIST_HIP_LIB_DIR=geistlib_amd/lib/stamps python3 geistlib_amd/bench/phase_stamps.py [--no-pen] [--rows N]
     GEIST_HIP_LIB_DIR=geistlib_amd/lib/stamps python3 geistlib_amd/bench/phase_stamps.py --walk [ROWS]
 
 Workload: 64 x 128256 fp32, T = 0.7, top-k 40 -> top-p 0.9, penalties over 2048 history ids per
 row (the default benchmark workload), 21 copies of the batch rotated so that every launch reads
 its logits from HBM. Prints, per stamp taken, minimum / median / maximum over the launch's
 workgroups in microseconds from the first workgroup's start, for the last of 40 launches, three
-times. Every stamp costs the wavefront that takes it time: the figures of a sparse mask are
+times (--rows N: the same on N rows, e.g. 1 for the decode step of one session). Every stamp costs the wavefront that takes it time: the figures of a sparse mask are
 closer to the uninstrumented kernel's than those of a dense one.
 
 --walk: the same for k_whole_row_coop (the whole-row top-p walk spread over the row's chunks) on
@@ -87,6 +87,8 @@ def main():
                  "GEIST_HIP_LIB_DIR=geistlib_amd/lib/stamps")
     lib.geist_hip_phase_stamps_read.argtypes = [C.c_void_p, C.c_size_t]
     rows, vocab, hist_n = 64, 128256, 2048
+    if "--rows" in sys.argv:
+        rows = int(sys.argv[sys.argv.index("--rows") + 1])
     pen = "--no-pen" not in sys.argv
     hs = HipSampler(rows, vocab)
     g = torch.Generator(device="cuda")
@@ -102,7 +104,7 @@ def main():
     hs.set_logits_hint(True)
     n = 4096 * 16
     buf = (C.c_ulonglong * n)()
-    wgs = rows * ((vocab + 32767) // 32768)
+    wgs = ((rows + 7) & ~7) * ((vocab + 32767) // 32768)   # the grid holds the rows in eights
     for rep in range(3):
         for i in range(40):
             hs.sample(hs.rows(copies[i % 21], hist if pen else None, hlen if pen else None), prm,
@@ -111,8 +113,10 @@ def main():
         if lib.geist_hip_phase_stamps_read(buf, n) != 0:
             sys.exit("reading the stamps failed")
         a = np.frombuffer(buf, dtype=np.uint64).reshape(-1, 16).astype(np.int64)[:wgs]
+        a = a[a[:, 0] != 0]                      # (the workgroups of the grid's padding take none)
+        wgs_run = a.shape[0]
         d = (a - a[:, 0].min()) / 100.0          # the device's clock ticks at 100 MHz
-        print(f"run {rep}: {wgs} workgroups; microseconds from the first workgroup's start")
+        print(f"run {rep}: {wgs_run} workgroups; microseconds from the first workgroup's start")
         for k in ORDER:
             col = d[:, k]
             col = col[col > 0] if k else col
