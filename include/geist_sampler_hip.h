@@ -204,7 +204,13 @@ int geist_hip_sampler_set_whole_row_walk(geist_hip_sampler *s, int mode);
  * cache they share, otherwise it leaves the hand-over unread and finds the row's candidates from
  * the logits themselves. always_agent = 1 makes every row take the second branch whatever its
  * placement -- for tests of that branch; 0 returns to the default. Results are the same either
- * way. */
+ * way.
+ * The one-pass kernels (temperature, top-p / min-p, verification) use the same cache for the
+ * slots through which the workgroups of a row meet, where the launch deals a row to one XCD
+ * (a row count that is a multiple of 8, and the one-kernel temperature draw): plain stores, which
+ * that XCD's cache serves to the polling workgroups. Workgroups that did not share an XCD would
+ * not see one another, their bounded waits would run out and each would read the row itself:
+ * slower, the same ids. always_agent = 1 makes these stores device-scope as well. */
 int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent);
 
 /* No counterpart in the reference. Stochastic speculative verification sums the residual
