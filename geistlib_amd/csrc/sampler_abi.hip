@@ -12,6 +12,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <algorithm>
@@ -723,12 +724,19 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         /* a batch that fits the device in one round of 1024-thread workgroups takes scan and
          * row-final stage in one launch (the measuring stages cannot split it: the streaming
          * stage is the whole step) */
-        const size_t wgs_row = (size_t) ((L.rv.n_chunks + 3) / 4);
+        /* a workgroup scans 32768 logits; launches of up to 128 workgroups halve that, so
+         * that twice the compute units fetch a row (64 x 128256: 13.1 us with whole, 14.9 with
+         * half workgroups; 32 rows 11.4 and 12.0; 16 rows 11.1 and 11.0; 4 rows 10.6 and 10.3;
+         * one row 10.2 and 9.9, without penalties 9.0 and 8.6) */
+        const size_t wgs_row8 = (size_t) ((L.rv.n_chunks + 3) / 4);
+        const size_t wgs_row4 = (rows->n_vocab + 16383) / 16384;
+        const bool   halves   = wgs_row4 <= (size_t) OL_WG_MAX && rows->rows * wgs_row4 <= 128;
+        const size_t wgs_row = halves ? wgs_row4 : wgs_row8;
         const size_t wgs     = rows->rows * wgs_row;
         const bool   one     = plain && s->row_arrive &&
                              wgs <= (size_t) s->fused_wg_limit && rows->n_vocab % 4 == 0 &&
                              wg_cands_bytes(rows->rows, wgs_row) <= wave_cands_bytes(s->wcands_row_waves);
-        const size_t per_wg  = 32768;
+        const size_t per_wg  = halves ? 16384 : 32768;
         const size_t e_full  = rows->n_vocab < per_wg ? rows->n_vocab : per_wg;
         const int    r_full  = one ? cand_rank_for(f.k_sel, rows->n_vocab, e_full) : 0;
         const int    r_last  = one ? cand_rank_for(f.k_sel, rows->n_vocab,
@@ -747,7 +755,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
             if (do_stream)
                 launch_cand_scan_final(scan, L, f, s->tmax, wg_cands_at(s->wcands, rows->rows, wgs_row),
                                        r_w, r_last, reinterpret_cast<uint32_t *>(s->row_arrive),
-                                       s->handoff_far, nt);
+                                       s->handoff_far, nt, (int) wgs_row, halves ? 4 : 8);
             return after_launch(s, "top-k");
         }
         if (m) {

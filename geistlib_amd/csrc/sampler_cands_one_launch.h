@@ -7,7 +7,9 @@
  *                       eights so that the workgroups of a row have linear ids equal modulo 8,
  *                       which this device places on one XCD (workgroups of rows that are not
  *                       there leave at once). A workgroup holds 32768 logits of its row in
- *                       registers (a wavefront 2048, a lane 32 in eight groups of four). It
+ *                       registers (a wavefront 2048, a lane 32 in eight groups of four; in
+ *                       launches of few rows half of that, NG = 4, so that twice the compute
+ *                       units fetch a row). It
  *                       finds a bound T_w that about r of its group maxima reach, hands on the
  *                       groups whose maximum reaches T_w -- a few dozen (float4, index) pairs,
  *                       in slots of their own per wavefront -- and adds itself to the row's
@@ -113,21 +115,29 @@ static_assert(OL_HT_SLOTS == 1 << 14, "ol_hash");
 /* The maxima of a thread's eight float4 groups of chunk `chunk` (loaded into v) and their
  * maximum, NaN for a thread whose first element lies beyond the row: what k_cand_scan stores as
  * the thread maximum. */
-__device__ __forceinline__ float group_maxima(const float4 (&v)[8], float (&gm)[8], int base,
+template <int NG>
+__device__ __forceinline__ float group_maxima(const float4 (&v)[NG], float (&gm)[NG], int base,
                                               int end, int t) {
+    static_assert(NG == 8 || NG == 4, "eight or four groups a lane");
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < NG; ++j)
         gm[j] = max3f(max3f(v[j].x, v[j].y, v[j].z), v[j].w, v[j].w);
     float tm = max3f(gm[0], gm[1], gm[2]);
-    tm       = max3f(tm, gm[3], gm[4]);
-    tm       = max3f(tm, gm[5], gm[6]);
-    tm       = max3f(tm, gm[7], gm[7]);
+    if (NG == 8) {
+        tm = max3f(tm, gm[3], gm[4]);
+        tm = max3f(tm, gm[5], gm[6]);
+        tm = max3f(tm, gm[NG - 1], gm[NG - 1]);
+    } else {
+        tm = max3f(tm, gm[3], gm[3]);
+    }
     if (base + 4 * t >= end)
         tm = __builtin_nanf("");
     return tm;
 }
 
-template <bool PEN, bool STREAM>
+/* NG: float4 groups a lane holds, 8 (a workgroup scans 32768 logits) or, for launches of few
+ * rows, 4 (16384: twice the workgroups to a row, so that twice the compute units fetch it). */
+template <bool PEN, bool STREAM, int NG>
 __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, RowView rv,
                                                                 WgCands wc, int r_w, int r_last,
                                                                 FinalArgs a,
@@ -186,16 +196,19 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
      * to -inf afterwards. (A second code path for partial chunks would make the loads of both
      * wait for everything asked for before.) Rows are 16-byte aligned and n_vocab a multiple of
      * four on this path. */
-    const int chunk = 4 * grp + (tid >> 8), t = tid & (TPB - 1);
-    int       base = rvs.n_vocab, end = rvs.n_vocab; /* a chunk beyond the row: nothing but -inf */
-    if (chunk < rvs.n_chunks)
-        chunk_bounds<8>(rvs, chunk, base, end);
+    constexpr int PIECE = NG * TPB * 4; /* what 256 threads hold: a chunk of the scan, or half */
+    const int piece = 4 * grp + (tid >> 8), t = tid & (TPB - 1);
+    int       base = rvs.n_vocab, end = rvs.n_vocab; /* a piece beyond the row: nothing but -inf */
+    if ((long) piece * PIECE < (long) rvs.n_vocab) {
+        base = piece * PIECE;
+        end  = base + PIECE < rvs.n_vocab ? base + PIECE : rvs.n_vocab;
+    }
     const int g0 = (base >> 2) + t, g_last = (rvs.n_vocab >> 2) - 1;
-    float4    v[8];
+    float4    v[NG];
     {
         const float4 *row4 = reinterpret_cast<const float4 *>(rvs.logits + (long) row * rvs.ld);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NG; ++j) {
             const int g = g0 + j * TPB;
             v[j] = STREAM ? load_streaming(row4 + (g < g_last ? g : g_last))
                           : row4[g < g_last ? g : g_last];
@@ -257,9 +270,9 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
 
     /* ---- the lane maxima; the largest of every eight neighbouring lanes is entered for the
      * workgroup's bound (three row shifts: lane 8 i + 7 ends with the maximum of its eight) */
-    if (ballot64(g0 + 7 * TPB > g_last) != 0ull) { /* a wavefront at the row's end */
+    if (ballot64(g0 + (NG - 1) * TPB > g_last) != 0ull) { /* a wavefront at the row's end */
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NG; ++j) {
             const bool out = g0 + j * TPB > g_last;
             v[j].x         = out ? -INFINITY : v[j].x;
             v[j].y         = out ? -INFINITY : v[j].y;
@@ -267,8 +280,8 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
             v[j].w         = out ? -INFINITY : v[j].w;
         }
     }
-    float gm[8];
-    const float tm = group_maxima(v, gm, base, end, t);
+    float gm[NG];
+    const float tm = group_maxima<NG>(v, gm, base, end, t);
     {
         uint32_t m8 = f2key(tm);
         GS_STAMP(2);
@@ -328,7 +341,7 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
         const int  e0  = base + 4 * t;
         unsigned   cnt = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NG; ++j) {
             const bool     in_j = gm[j] >= Tf;
             const uint64_t mj   = ballot64(in_j);
             if (mj == 0ull)
@@ -568,7 +581,7 @@ __global__ __launch_bounds__(OL_THREADS) void k_cand_scan_final(RowView rvs, Row
             float4 v2[8];
             float  gm2[8];
             load_raw<8>(rvs, rvs.logits + (long) row * rvs.ld, b2, e2, v2, t);
-            tmax_rw[((long) row * rvs.n_chunks + c) * TPB + t] = group_maxima(v2, gm2, b2, e2, t);
+            tmax_rw[((long) row * rvs.n_chunks + c) * TPB + t] = group_maxima<8>(v2, gm2, b2, e2, t);
         }
         __syncthreads();
         if (tid >= TPB)

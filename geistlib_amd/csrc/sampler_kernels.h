@@ -257,7 +257,7 @@ constexpr int ARRIVE_STRIDE_INTS = 32;
 int probe_workgroup_placement(hipStream_t stream, bool *same_xcd);
 void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
                             const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
-                            bool far_always, const Notify &nt);
+                            bool far_always, const Notify &nt, int wgs_per_row, int groups);
 /* returns a hipError_t value */
 int  launch_topk_general(const Launch &L, const FinalLaunch &f);
 /* Per-device kernel attributes; call once with the device current. Returns a hipError_t value. */

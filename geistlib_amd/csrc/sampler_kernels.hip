@@ -2010,20 +2010,26 @@ int cand_rank_for(int k_eff, size_t n_vocab, size_t elems) {
 
 void launch_cand_scan_final(const Launch &scan, const Launch &L, const FinalLaunch &f, float *tmax,
                             const WgCands &wc, int r_w, int r_last, uint32_t *arrive,
-                            bool far_always, const Notify &nt) {
+                            bool far_always, const Notify &nt, int wgs_per_row, int groups) {
     const FinalArgs a = final_args(f);
-    const int       per_wg = OL_THREADS / TPB; /* chunks a workgroup scans */
     /* rows in eights: the workgroups of a row then have linear ids equal modulo 8 and share an
      * XCD; the workgroups of the rows that are not there leave at once */
-    const dim3      grid((L.rv.n_chunks + per_wg - 1) / per_wg, (L.rows + 7) & ~7), block(OL_THREADS);
+    const dim3      grid(wgs_per_row, (L.rows + 7) & ~7), block(OL_THREADS);
     auto go = [&](auto kernel) {
         kernel<<<grid, block, 0, L.stream>>>(scan.rv, L.rv, wc, r_w, r_last, a, tmax, arrive,
                                              far_always ? 1 : 0, nt);
     };
+    if (groups == 4) { /* launches of few rows: half the logits to a workgroup */
+        if (L.pen)
+            scan.rv.stream_loads ? go(k_cand_scan_final<true, true, 4>) : go(k_cand_scan_final<true, false, 4>);
+        else
+            scan.rv.stream_loads ? go(k_cand_scan_final<false, true, 4>) : go(k_cand_scan_final<false, false, 4>);
+        return;
+    }
     if (L.pen)
-        scan.rv.stream_loads ? go(k_cand_scan_final<true, true>) : go(k_cand_scan_final<true, false>);
+        scan.rv.stream_loads ? go(k_cand_scan_final<true, true, 8>) : go(k_cand_scan_final<true, false, 8>);
     else
-        scan.rv.stream_loads ? go(k_cand_scan_final<false, true>) : go(k_cand_scan_final<false, false>);
+        scan.rv.stream_loads ? go(k_cand_scan_final<false, true, 8>) : go(k_cand_scan_final<false, false, 8>);
 }
 
 __global__ __launch_bounds__(TPB) void k_zero_words(uint64_t *__restrict__ p, uint32_t n) {
