@@ -736,13 +736,18 @@ __global__ __launch_bounds__(LM_TPB, 2) void k_f16_linear_f64_mfma(
 
 /* The listed outputs once more, the products added one after the other in index order as the
  * reference adds them. A wavefront per output (weight row r, activation row m): its lanes form
- * 64 products at a time -- each exact in double -- and the sum takes them in order, lane by
- * lane, as scalar operands. The chain of n_in dependent additions is what this kernel takes;
- * there are few listed outputs and each has a wavefront to itself. */
+ * 256 products at a time -- each exact in double -- and put them into the wavefront's part of
+ * LDS; the sum then takes them in order, two per 16-byte read that every lane makes of the same
+ * address. The chain of n_in dependent additions is what this kernel takes (a wavefront issues
+ * an instruction every few cycles whatever it is: 1.5 instructions per product here, where
+ * fetching each product from its lane as a scalar operand took three); there are few listed
+ * outputs and each has a wavefront to itself. */
 __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
     const uint16_t *__restrict__ w, int n_in, const double *__restrict__ xd, float *__restrict__ y,
     long ld_y, const int *__restrict__ amb_count, const int2 *__restrict__ amb_list) {
+    __shared__ __align__(16) double s_prod[LM_WAVES][4 * LM_WAVE];
     const int lane = threadIdx.x & (LM_WAVE - 1), wave = threadIdx.x / LM_WAVE;
+    double   *mine_p = s_prod[wave];
     const int count = *amb_count;
     for (int it = (int) blockIdx.x * LM_WAVES + wave; it < count;
          it += (int) gridDim.x * LM_WAVES) { /* (uniform over the wavefront) */
@@ -759,19 +764,25 @@ __global__ __launch_bounds__(LM_TPB) void k_f16_linear_f64_listed(
                 const int k = k0 + r * LM_WAVE + lane;
                 prod[r]     = k < n_in ? xm[k] * (double) __half2float(__ushort_as_half(wr[k])) : 0.0;
             }
+            /* (the wavefront's own reads of the block before are done: its LDS operations are
+             * performed in the order they were issued) */
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (k0 + r * LM_WAVE >= n_in)
-                    break;
-                const uint2 pw = __builtin_bit_cast(uint2, prod[r]);
-#pragma unroll
-                for (int i = 0; i < LM_WAVE; ++i) {
-                    uint2 t;
-                    t.x = (uint32_t) __builtin_amdgcn_readlane((int) pw.x, i);
-                    t.y = (uint32_t) __builtin_amdgcn_readlane((int) pw.y, i);
-                    acc += __builtin_bit_cast(double, t);
-                }
+            for (int r = 0; r < 4; ++r)
+                mine_p[r * LM_WAVE + lane] = prod[r];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int n_here = n_in - k0 < 4 * LM_WAVE ? n_in - k0 : 4 * LM_WAVE;
+            const int pairs  = (n_here + 1) >> 1; /* (an odd count ends with a zero) */
+            const double2 *pp = reinterpret_cast<const double2 *>(mine_p);
+#pragma unroll 16
+            for (int i = 0; i < pairs; ++i) {
+                const double2 t = pp[i];
+                acc += t.x;
+                acc += t.y;
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
         if (lane == 0)
             y[mine.y * ld_y + mine.x] = (float) acc;
