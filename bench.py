@@ -1243,6 +1243,12 @@ def main():
         hs.notify_ids(True)
         bh.step_latency(hs, rows_cold, prm, d_u, out_host, 20, wait_ids=True)
         lat_c_wait = sorted(bh.step_latency(hs, rows_cold, prm, d_u, out_host, 200, wait_ids=True))
+        # ... and on one buffer over and over, which stays cache-resident as logits are right
+        # after the projection that wrote them (with the default kind of load)
+        hs.set_logits_hint(False)
+        bh.step_latency(hs, [rows], prm, d_u, out_host, 20, wait_ids=True)
+        lat_c_wait_res = sorted(bh.step_latency(hs, [rows], prm, d_u, out_host, 200, wait_ids=True))
+        hs.set_logits_hint(True)
         hs.notify_ids(False)
         assert ids_host.tolist() == d_out.cpu().numpy().tolist()
         out_host.close()
@@ -1287,6 +1293,8 @@ def main():
                                                       if lat_host else None),
         "step_latency_from_c_ids_on_host_us_p90": (round(lat_c_wait[len(lat_c_wait) * 9 // 10], 2)
                                                    if lat_host else None),
+        "step_latency_from_c_ids_on_host_cache_resident_us_median": (
+            round(lat_c_wait_res[len(lat_c_wait_res) // 2], 2) if lat_host else None),
         "step_latency_ids_on_host_us_median": (round(lat_host[len(lat_host) // 2], 2)
                                                if lat_host else None),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
