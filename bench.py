@@ -190,7 +190,8 @@ def time_other_configs(steps=50, warmup=10):
     def normal(shape, scale):
         return torch.randn(shape, device=dev, generator=g) * scale
 
-    def run(name, make_copy, n_copies, rows, n_vocab, prm_kw, hist_len=0, extra_bytes=0):
+    def run(name, make_copy, n_copies, rows, n_vocab, prm_kw, hist_len=0, extra_bytes=0,
+            fast_sums_twin=False):
         copies = [make_copy() for _ in range(n_copies)]
         d_u = torch.rand(rows, device=dev, generator=g)
         d_out = torch.empty(rows, dtype=torch.int32, device=dev)
@@ -220,6 +221,20 @@ def time_other_configs(steps=50, warmup=10):
                      "kernel_us": round(k_us, 2), "steps": steps, "input_copies_rotated": n_copies}
         if prm_kw.get("top_k"):
             out[name]["topk_paths"] = topk_path_counts(hs, rl, prm, d_u, d_out, rows)
+        if fast_sums_twin:
+            # the same with the sums of exponentials from the hardware's 2^z (the contract's
+            # tolerance used, geist_hip_sampler_set_sums; off by default)
+            hs.set_sums(fast=True)
+            for i in range(max(warmup, n_copies)):
+                hs.sample(rl[i % n_copies], prm, d_u, d_out)
+            hs.sync()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                hs.sample(rl[i % n_copies], prm, d_u, d_out)
+            hs.sync()
+            out[name]["us_per_step_fast_sums"] = round((time.perf_counter() - t0) * 1e6 / steps, 2)
+            out[name]["kernel_us_fast_sums"] = round(
+                bh.time_stream_kernel(hs, rl, prm, d_u, d_out, steps)[0], 2)
         hs.close()
 
     # cfg1: one row of 128256, N(0, 3^2), T = 0.8 (the rows of a [1400 x V] buffer take turns)
@@ -236,7 +251,7 @@ def time_other_configs(steps=50, warmup=10):
     hist_bytes = 128 * (4 * 2048 + 8 * 1000)   # ids read + about 1000 distinct per row gathered
     run("cfg3", lambda: normal((128, 151936), 2.0), 9, 128, 151936,
         dict(temperature=1.0, top_p=0.95, min_p=0.05, rep=1.1, freq=0.5, pres=0.3), hist_len=2048,
-        extra_bytes=hist_bytes)
+        extra_bytes=hist_bytes, fast_sums_twin=True)
     # cfg4: 256 x 262144, Student-t(3) x 2.5, top-k 64 -> top-p 0.9, T = 0.6
     def student_t():
         z = torch.randn((256, 262144), device=dev, generator=g)
@@ -273,6 +288,15 @@ def time_other_configs(steps=50, warmup=10):
                    "step_algorithmic_bytes": int(alg),
                    "kernel": "k_scan_expsum + k_spec_resid_draw (whole step)", "kernel_us": None,
                    "steps": steps, "input_copies_rotated": 3}
+    hs.set_sums(fast=True)
+    for i in range(max(warmup, 3)):
+        hs.spec_verify(ts[i % 3], qs[i % 3], draft, u, 1.0, o_tok, nacc)
+    hs.sync()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        hs.spec_verify(ts[i % 3], qs[i % 3], draft, u, 1.0, o_tok, nacc)
+    hs.sync()
+    out["cfg5"]["us_per_step_fast_sums"] = round((time.perf_counter() - t0) * 1e6 / steps, 2)
     hs.close()
     return out
 
@@ -296,6 +320,8 @@ def bench_spec(w, args):
     nacc = torch.full((n_seq,), -1, dtype=torch.int32, device=dev)
     hs = HipSampler(max_rows=n_seq * (L + 1), max_vocab=w.n_vocab)
     hs.set_logits_hint(1)   # the rows come from HBM and are read once
+    if args.fast_sums:
+        hs.set_sums(fast=True)
 
     def step(i):
         hs.spec_verify(ts[i % n_copies], qs[i % n_copies], d, u, w.temperature, out, nacc)
@@ -319,7 +345,8 @@ def bench_spec(w, args):
         "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": w.name, "sequences": n_seq, "draft_len": L, "n_vocab": w.n_vocab,
+        "config": {"workload": w.name, "sums": "fast" if args.fast_sums else "exact",
+                   "sequences": n_seq, "draft_len": L, "n_vocab": w.n_vocab,
                    "temperature": w.temperature},
         "us_per_step": round(ms * 1e3, 3),
         "sequences_per_s": round(n_seq * args.steps / elapsed, 1),
@@ -1091,6 +1118,10 @@ def main():
                     help="skip the cache-resident legs and the latency probe, so that every launch "
                          "of the run streams its logits from HBM (for rocprofv3 runs whose "
                          "per-kernel averages are to be compared with roofline.kernel_us)")
+    ap.add_argument("--fast-sums", action="store_true",
+                    help="geist_hip_sampler_set_sums(GEIST_HIP_SUMS_FAST): the sums of exponentials "
+                         "from the hardware's 2^z (the tolerance of the sampling contract used; "
+                         "off by default, and never the headline figure)")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the legs that time configurations 1, 3, 4 and 5 beside the headline "
                          "workload")
@@ -1130,6 +1161,8 @@ def main():
     d_hl = torch.from_numpy(w.history_len).to(dev) if w.history is not None else None
     d_out = torch.empty(w.rows, dtype=torch.int32, device=dev)
     hs = HipSampler(max_rows=w.rows, max_vocab=w.n_vocab)
+    if args.fast_sums:
+        hs.set_sums(fast=True)
     rows = HipSampler.rows(d_logits, d_h, d_hl)
     prm = SampleParams.make(temperature=w.temperature, top_k=w.top_k, top_p=w.top_p,
                             min_p=w.min_p, rep=w.rep, freq=w.freq, pres=w.pres)
@@ -1276,7 +1309,8 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": w.name, "rows": w.rows, "n_vocab": w.n_vocab,
+        "config": {"workload": w.name, "sums": "fast" if args.fast_sums else "exact",
+                   "rows": w.rows, "n_vocab": w.n_vocab,
                    "temperature": w.temperature, "top_k": w.top_k, "top_p": w.top_p,
                    "min_p": w.min_p, "penalties": [w.rep, w.freq, w.pres],
                    "history_per_row": 0 if w.history is None else int(w.history.shape[1])},

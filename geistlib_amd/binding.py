@@ -89,6 +89,7 @@ def load_library():
     lib.geist_hip_sampler_set_whole_row_walk.argtypes = [vp, i32]
     lib.geist_hip_sampler_notify_ids.argtypes = [vp, i32]
     lib.geist_hip_sampler_wait_ids.argtypes = [vp]
+    lib.geist_hip_sampler_set_sums.argtypes = [vp, i32]
     lib.geist_hip_sampler_set_wait_spin.argtypes = [vp, C.c_uint32]
     lib.geist_hip_sample_rows.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, vp]
     lib.geist_hip_sample_rows_rng.argtypes = [vp, C.POINTER(Rows), C.POINTER(SampleParams), vp, i32,
@@ -254,6 +255,11 @@ class HipSampler:
     def wait_ids(self):
         """Returns when the ids of the last sampling call are written (see notify_ids)."""
         self._check(self.lib.geist_hip_sampler_wait_ids(self.h))
+
+    def set_sums(self, fast=False):
+        """The sums of exponentials bit-exact (default) or from the hardware's 2^z
+        (geist_hip_sampler_set_sums)."""
+        self._check(self.lib.geist_hip_sampler_set_sums(self.h, 1 if fast else 0))
 
     def set_wait_spin(self, microseconds):
         self._check(self.lib.geist_hip_sampler_set_wait_spin(self.h, microseconds))

@@ -58,6 +58,7 @@ struct geist_hip_sampler {
     bool       epoch_by_kernel = false; /* the call being enqueued reports from its own kernel */
     bool       tell = false;            /* the call being enqueued reports at all */
     uint32_t   wait_spin_us = 2000;  /* geist_hip_sampler_wait_ids: how long it watches the word */
+    bool       fast_sums = false;    /* geist_hip_sampler_set_sums */
     bool       handoff_far = false;  /* that kernel reads the hand-over with agent-scope loads
                                       * whatever the placement (geist_hip_sampler_handoff_scope) */
     bool       spec_one_launch = true; /* residual sums and draw of spec verification in one launch */
@@ -796,7 +797,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
         if (do_stream &&
             launch_scan_expsum(scan, rs.inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0,
                                nullptr, nullptr, 0, s->slab_sum,
-                               meet_space(s, scan, 1, (scan.rows & 7) == 0)))
+                               meet_space(s, scan, 1, (scan.rows & 7) == 0), s->fast_sums))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
         f.mode     = FINAL_TEMPERATURE;
         f.slab_sum = s->slab_sum;
@@ -832,7 +833,7 @@ int gs_host::sample_stages(geist_hip_sampler *s, const struct geist_hip_rows *ro
          * alone nobody reads them) */
         launch_scan_expsum(scan, rs.inv_t, f.minp_direct ? nullptr : s->tmax, s->chunk_best,
                            s->chunk_sum, nullptr, 0, nullptr, f.minp_listed ? &f.cand : nullptr,
-                           zb_m, nullptr, meet_space(s, scan, 1, (scan.rows & 7) == 0)))
+                           zb_m, nullptr, meet_space(s, scan, 1, (scan.rows & 7) == 0), s->fast_sums))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     if (!do_tail)
         return after_launch(s, "exp-sum scan");
@@ -975,6 +976,15 @@ int geist_hip_sampler_set_wait_spin(geist_hip_sampler *s, uint32_t microseconds)
     if (!s)
         return GEIST_HIP_E_INVALID_ARG;
     s->wait_spin_us = microseconds;
+    return GEIST_HIP_OK;
+}
+
+int geist_hip_sampler_set_sums(geist_hip_sampler *s, int mode) {
+    if (!s)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (mode != GEIST_HIP_SUMS_EXACT && mode != GEIST_HIP_SUMS_FAST)
+        return fail(s, GEIST_HIP_E_INVALID_ARG, "sums: GEIST_HIP_SUMS_EXACT or GEIST_HIP_SUMS_FAST");
+    s->fast_sums = mode == GEIST_HIP_SUMS_FAST;
     return GEIST_HIP_OK;
 }
 
@@ -1143,7 +1153,7 @@ int geist_hip_softmax_rows(geist_hip_sampler *s, const struct geist_hip_rows *ro
     const float inv_t = 1.0f / params->temperature;
     HIPCHK(s, hipSetDevice(s->device));
     if (launch_scan_expsum(L, inv_t, nullptr, s->chunk_best, s->chunk_sum, nullptr, 0, nullptr,
-                           nullptr, 0, nullptr, meet_space(s, L, 1, (L.rows & 7) == 0)))
+                           nullptr, 0, nullptr, meet_space(s, L, 1, (L.rows & 7) == 0), s->fast_sums))
         return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     launch_write_probs(L, inv_t, s->chunk_best, s->chunk_sum, d_probs, (long) ld_probs, nullptr);
     return after_launch(s, "softmax");
@@ -2104,7 +2114,7 @@ int geist_hip_spec_verify(geist_hip_sampler *s, const float *d_target, size_t ld
          * workgroup that walks the located chunk from its start */
         if (launch_scan_expsum(scan, inv_t, nullptr, s->chunk_best, s->chunk_sum, d_draft, (int) L,
                                s->probe_p, nullptr, 0, nullptr,
-                               meet_space(s, scan, 1, (scan.rows & 7) == 0)))
+                               meet_space(s, scan, 1, (scan.rows & 7) == 0), s->fast_sums))
             return fail(s, GEIST_HIP_E_BACKEND, "no launch geometry for the exp-sum pass");
     }
     SpecLaunch sp{};

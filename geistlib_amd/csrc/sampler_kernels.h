@@ -197,10 +197,13 @@ struct FinalLaunch {
  * list->count itself).
  * slab_sum != NULL (and no list): also the sums of the chunk's slabs of 1024 elements,
  * [rows][chunks][8], which the index-order walks locate their starting point with.
+ * fast: the weights of the sums from the hardware's 2^z (relative error about 1e-7) instead of
+ * the bit-exact expf; p at the probed token stays exact.
  * Returns 0 or a hipError_t value (the launch itself is checked by the caller as usual). */
 int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
                        double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
-                       const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet);
+                       const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet,
+                       bool fast = false);
 /* The temperature draw in one kernel (sampler_draw.h): out[row] = the id drawn with
  * uniforms[row]. For L.nv == 2. `meet.slots` holds 2 * rows * n_chunks zeroed words: the
  * workgroups of a row meet twice. */

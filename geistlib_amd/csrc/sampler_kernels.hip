@@ -299,11 +299,25 @@ __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, in
     return bb ? bb : pack_best(0u, 0u);
 }
 
+/* expf(x) for x <= 0 from the hardware's 2^z, for the sums of the tolerance mode
+ * (geist_hip_sampler_set_sums): x log2(e) as a binary32 product plus the product's rounding
+ * error and the low part of log2(e), 2^z of the high part, one correction term. Relative error
+ * about 1e-7 against the exact expf's half unit in the last place; -inf gives 0, NaN NaN. */
+__device__ __forceinline__ float fast_expf_le0(float x) {
+    const float L2E = 1.44269502f, L2E_LO = 1.92596299e-8f, LN2 = 0.693147182f;
+    x               = x < -200.0f ? -200.0f : x; /* (2^z is 0 long before; keeps -inf out of the fma) */
+    const float zh  = __fmul_rn(x, L2E);
+    float       zl  = fmaf(x, L2E, -zh);
+    zl              = fmaf(x, L2E_LO, zl);
+    const float e   = __builtin_amdgcn_exp2f(zh);
+    return fmaf(e, __fmul_rn(zl, LN2), e);
+}
+
 /* The work of one workgroup. PLAIN: a full, 16-byte aligned chunk without soft-cap or
  * allowed-token mask -- the common case, kept free of everything that would make the compiler
  * wait for all of the chunk's loads before the first group is looked at (a merge with the
  * element-wise loads of a ragged chunk, a branch around a mask load). */
-template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN>
+template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN, bool FAST>
 __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chunk, int n_rows,
                                              int base, int end, float inv_t,
                                              double *__restrict__ chunk_sum,
@@ -435,7 +449,8 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             args[c]        = softmax_arg(f4_get(v[j], c), mx, inv_t);
-            const double p = (double) geist_expf_glibc_le0(args[c], s_tab);
+            const double p = (double) (FAST ? fast_expf_le0(args[c])
+                                            : geist_expf_glibc_le0(args[c], s_tab));
             a4             = c == 0 ? p : a4 + p;
         }
         if (LISTM) {
@@ -559,7 +574,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
 /* The penalised list-making form needs 82 registers when left alone, two more than let a sixth
  * workgroup share a compute unit; held to 80 it spills nothing and a launch of 128 x 151936 is
  * about a microsecond shorter. (Held to 72 or 64 it spills and is slower.) */
-template <int NV, bool PEN, bool LISTM, bool SLABS>
+template <int NV, bool PEN, bool LISTM, bool SLABS, bool FAST = false>
 __global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan_expsum(RowView rv, float inv_t,
                                                      float *__restrict__ tmax,
                                                      uint64_t *__restrict__ chunk_best,
@@ -611,12 +626,12 @@ __global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan
     const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
                        rv.allowed == nullptr;
     if (plain)
-        expsum_chunk<NV, PEN, LISTM, SLABS, true>(
+        expsum_chunk<NV, PEN, LISTM, SLABS, true, FAST>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
             probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
             s_arrive + 3, fs);
     else
-        expsum_chunk<NV, PEN, LISTM, SLABS, false>(
+        expsum_chunk<NV, PEN, LISTM, SLABS, false, FAST>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
             probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
             s_arrive + 3, fs);
@@ -1828,28 +1843,28 @@ static void dispatch(int nv, bool pen, F &&f) {
 
 int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
                         double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
-                        const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet) {
+                        const CandSpace *list, int zb_list, double *slab_sum, const MeetSpace &meet,
+                        bool fast) {
     const dim3 grid(L.rv.n_chunks, L.rows), block(TPB);
+    auto go = [&](auto kernel) {
+        kernel<<<grid, block, 0, L.stream>>>(L.rv, inv_t, tmax, chunk_best, chunk_sum,
+                                             list ? nullptr : slab_sum, probe_token, probe_L, probe_p,
+                                             list ? *list : CandSpace{}, list ? zb_list : 0, meet);
+    };
     if (list && L.nv == 8) {
         if (L.pen)
-            k_scan_expsum<8, true, true, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
-                *list, zb_list, meet);
+            fast ? go(k_scan_expsum<8, true, true, false, true>) : go(k_scan_expsum<8, true, true, false>);
         else
-            k_scan_expsum<8, false, true, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
-                *list, zb_list, meet);
+            fast ? go(k_scan_expsum<8, false, true, false, true>) : go(k_scan_expsum<8, false, true, false>);
         return 0;
     }
     dispatch(L.nv, L.pen, [&](auto nv, auto pen) {
         if (slab_sum)
-            k_scan_expsum<GS_NV, GS_PEN, false, true><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, tmax, chunk_best, chunk_sum, slab_sum, probe_token, probe_L, probe_p,
-                CandSpace{}, 0, meet);
+            fast ? go(k_scan_expsum<GS_NV, GS_PEN, false, true, true>)
+                 : go(k_scan_expsum<GS_NV, GS_PEN, false, true>);
         else
-            k_scan_expsum<GS_NV, GS_PEN, false, false><<<grid, block, 0, L.stream>>>(
-                L.rv, inv_t, tmax, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p,
-                CandSpace{}, 0, meet);
+            fast ? go(k_scan_expsum<GS_NV, GS_PEN, false, false, true>)
+                 : go(k_scan_expsum<GS_NV, GS_PEN, false, false>);
     });
     return 0;
 }

@@ -213,6 +213,22 @@ int geist_hip_sampler_set_whole_row_walk(geist_hip_sampler *s, int mode);
  * slower, the same ids. always_agent = 1 makes these stores device-scope as well. */
 int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent);
 
+/* No counterpart in the reference. The modes that weigh every element (temperature, top-p /
+ * min-p over the whole vocabulary, normalised probabilities, speculative verification) form a
+ * row's sum of exponentials with the reference's own expf, bit for bit, so that every id is the
+ * reference's (GEIST_HIP_SUMS_EXACT, the default). GEIST_HIP_SUMS_FAST forms the SUMS from the
+ * hardware's 2^z instead (relative error of a sum about 1e-7); every weight that is compared
+ * with a share of a sum -- in the walks, the nucleus, the acceptance test -- stays exact. An id
+ * can then differ from the reference's only where the reference's own decision lies within that
+ * error of an edge (a draw within 1e-7 of a slot's edge, a nucleus that ends within 1e-7 of
+ * top_p): the tolerance the sampling contract states, used. The pass over the logits gets a
+ * tenth shorter. Which rows those are is not reported: a caller that has to know compares with
+ * the exact mode. The one-kernel temperature draw of a few rows and the top-k path form no such
+ * sums and are exact in both modes. */
+#define GEIST_HIP_SUMS_EXACT 0
+#define GEIST_HIP_SUMS_FAST 1
+int geist_hip_sampler_set_sums(geist_hip_sampler *s, int mode);
+
 /* No counterpart in the reference. Stochastic speculative verification sums the residual
  * max(0, p - q) and draws from it in one launch (the workgroups of a sequence wait for one
  * another's sums, the wait bounded by geist_hip_sampler_set_wait_limit) when sequences x chunks
