@@ -43,6 +43,7 @@ struct RowView {
  * slot per (row, chunk), zero until the chunk's workgroup stores its packed maximum there (never
  * zero). Two such arrays take turns from launch to launch: a launch finds its own array all
  * zero and zeroes the slots that the launch before it used in the other. */
+constexpr int ARRIVE_STRIDE_INTS = 32; /* a cache line of its own for every row's counter */
 struct MeetSpace {
     uint64_t *slots;       /* [rows * n_chunks] of this launch, zero on entry */
     uint64_t *stale;       /* the slots of the launch before, zeroed by this one */
@@ -198,7 +199,9 @@ struct FinalLaunch {
  * slab_sum != NULL (and no list): also the sums of the chunk's slabs of 1024 elements,
  * [rows][chunks][8], which the index-order walks locate their starting point with.
  * fast: the weights of the sums from the hardware's 2^z (relative error about 1e-7) instead of
- * the bit-exact expf; p at the probed token stays exact.
+ * the bit-exact expf; p at the probed token stays exact. Without penalties and without a list
+ * the workgroups of a row then do not meet: each sums against its chunk's maximum and a second,
+ * small launch scales the sums to the row's (k_rescale_sums).
  * Returns 0 or a hipError_t value (the launch itself is checked by the caller as usual). */
 int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chunk_best,
                        double *chunk_sum, const int32_t *probe_token, int probe_L, float *probe_p,
@@ -253,7 +256,7 @@ void launch_final_cand(const Launch &L, const FinalLaunch &f, const WaveCands &w
  * fall back to the slower paths. r_w / r_last: the rank of the bound of a full workgroup and of
  * the row's last one (cand_rank_for). far_always: read the hand-over with agent-scope loads whatever
  * the placement of the row's workgroups (for tests of that branch). */
-constexpr int ARRIVE_STRIDE_INTS = 32;
+
 /* *same_xcd: workgroups of a grid whose linear ids are equal modulo 8 run on one XCD (and so
  * share an L2): then launch_cand_scan_final hands a row over through that L2. Runs a small
  * kernel and waits for it. Returns a hipError_t value. */

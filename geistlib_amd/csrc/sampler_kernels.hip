@@ -317,7 +317,17 @@ __device__ __forceinline__ float fast_expf_le0(float x) {
  * allowed-token mask -- the common case, kept free of everything that would make the compiler
  * wait for all of the chunk's loads before the first group is looked at (a merge with the
  * element-wise loads of a ragged chunk, a branch around a mask load). */
-template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN, bool FAST>
+/* NOMEET (tolerance mode, no penalties, no list): the workgroups of a row do not wait for one
+ * another. Each sums its chunk against the chunk's own maximum, and a small launch behind the
+ * pass (k_rescale_sums) scales every chunk's sums by expf((chunk maximum - row maximum) * inv_t)
+ * -- exp((l - M) t) = exp((l - m) t) exp((m - M) t), which with arguments rounded to binary32
+ * holds to a few 1e-7 relative: the tolerance mode's accuracy -- and evaluates p at the probed
+ * token. What the two leave is what the meeting form leaves: chunk maxima, sums relative to the
+ * row's maximum. (The scaling by the workgroup that arrives last at a counter of the row's,
+ * inside the pass, was measured too: the acknowledged device-scope stores and the atomic it
+ * needs keep every workgroup longer than the launch costs; 50.6 against 48.6 us for the
+ * verification of 32 sequences, 53.3 with the meeting.) */
+template <int NV, bool PEN, bool LISTM, bool SLABS, bool PLAIN, bool FAST, bool NOMEET>
 __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chunk, int n_rows,
                                              int base, int end, float inv_t,
                                              double *__restrict__ chunk_sum,
@@ -413,13 +423,25 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
             if ((tid & (WAVE - 1)) == 0)
                 fs.chunk_best[(long) row * rv.n_chunks + chunk] = best;
         }
-        bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, last, fs, s_cnt16);
+        if (NOMEET) {
+            if (last && (tid & (WAVE - 1)) == 0)
+                *fs.s_bb = best; /* the chunk's own */
+            lds_barrier();
+            bb = *fs.s_bb;
+        } else {
+            bb = row_best_meet<NV, PEN>(rv, row, chunk, n_rows, best, last, fs, s_cnt16);
+        }
     }
     if (PEN)
         __builtin_amdgcn_s_setprio(0);
-    const float mx = key2f(best_key(bb));
+    float mx = key2f(best_key(bb));
+    /* (NOMEET: a chunk of nothing but -inf is summed against 0, so that it weighs 0 and not
+     * NaN; the scaling by the row's maximum makes the row's sums NaN where the meeting form's
+     * are, in a row of nothing but -inf) */
+    if (NOMEET && mx == -__builtin_inff())
+        mx = 0.0f;
 
-    if (tok >= base && tok < end) {
+    if (!NOMEET && tok >= base && tok < end) {
         /* the thread that holds the probed element evaluates it by itself (before the sums, so
          * that each group's registers are free once it has been added up) */
         const int off = tok - base, f = off >> 2;
@@ -574,7 +596,7 @@ __device__ __forceinline__ void expsum_chunk(const RowView &rv, int row, int chu
 /* The penalised list-making form needs 82 registers when left alone, two more than let a sixth
  * workgroup share a compute unit; held to 80 it spills nothing and a launch of 128 x 151936 is
  * about a microsecond shorter. (Held to 72 or 64 it spills and is slower.) */
-template <int NV, bool PEN, bool LISTM, bool SLABS, bool FAST = false>
+template <int NV, bool PEN, bool LISTM, bool SLABS, bool FAST = false, bool NOMEET = false>
 __global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan_expsum(RowView rv, float inv_t,
                                                      float *__restrict__ tmax,
                                                      uint64_t *__restrict__ chunk_best,
@@ -623,18 +645,67 @@ __global__ __launch_bounds__(TPB, (NV == 8 && PEN && LISTM) ? 6 : 1) void k_scan
     fs.s_red      = s_red;
     fs.s_bb       = &s_bb;
     fs.s_arrive   = s_arrive;
+    static_assert(!NOMEET || (FAST && !PEN && !LISTM), "the form without a meeting");
     const bool plain = rv.vec_ok && end - base == NV * TPB * 4 && !(rv.softcap > 0.0f) &&
                        rv.allowed == nullptr;
     if (plain)
-        expsum_chunk<NV, PEN, LISTM, SLABS, true, FAST>(
+        expsum_chunk<NV, PEN, LISTM, SLABS, true, FAST, NOMEET>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
             probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
             s_arrive + 3, fs);
     else
-        expsum_chunk<NV, PEN, LISTM, SLABS, false, FAST>(
+        expsum_chunk<NV, PEN, LISTM, SLABS, false, FAST, NOMEET>(
             rv, row, chunk, (int) gridDim.y, base, end, inv_t, chunk_sum, slab_sum,
             probe_token, probe_L, probe_p, list, zb_list, s_cnt16, s_sum, s_tab, tabv, s_tr, s_stage,
             s_arrive + 3, fs);
+}
+
+/* The scaling of the form without a meeting: a wavefront per row, a lane per chunk. */
+template <bool SLABS>
+__global__ __launch_bounds__(WAVE) void k_rescale_sums(RowView rv, float inv_t,
+                                                      const uint64_t *__restrict__ chunk_best,
+                                                      double *__restrict__ chunk_sum,
+                                                      double *__restrict__ slab_sum,
+                                                      const int32_t *__restrict__ probe_token,
+                                                      int probe_L, float *__restrict__ probe_p) {
+    __shared__ uint64_t s_tab[32];
+    const int row = blockIdx.x, lane = threadIdx.x, C = rv.n_chunks;
+    if (lane < 32)
+        s_tab[lane] = g_expf_tab[lane];
+    const long r0 = (long) row * C;
+    uint64_t   ba = lane < C ? chunk_best[r0 + lane] : 0, bb2 = lane + WAVE < C ? chunk_best[r0 + lane + WAVE] : 0;
+    int        tok = -1;
+    if (probe_token && lane == 0) {
+        const int j = row % (probe_L + 1);
+        if (j < probe_L)
+            tok = probe_token[(long) (row / (probe_L + 1)) * probe_L + j];
+    }
+    float x_tok = 0.0f;
+    if (tok >= 0)
+        x_tok = rv.logits[(long) row * rv.ld + tok];
+    __syncthreads();
+    const uint64_t rowb = wave_max_u64(ba > bb2 ? ba : bb2);
+    const float    M    = key2f(best_key(rowb));
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int c = lane + h * WAVE;
+        if (c >= C)
+            continue;
+        const float  mc = key2f(best_key(h ? bb2 : ba));
+        const double f  = (double) geist_expf_glibc_le0(softmax_arg(mc, M, inv_t), s_tab);
+        chunk_sum[r0 + c] *= f;
+        if (SLABS) {
+            double v8[SLABS_MAX];
+#pragma unroll
+            for (int j = 0; j < SLABS_MAX; ++j)
+                v8[j] = slab_sum[(r0 + c) * SLABS_MAX + j];
+#pragma unroll
+            for (int j = 0; j < SLABS_MAX; ++j)
+                slab_sum[(r0 + c) * SLABS_MAX + j] = v8[j] * f;
+        }
+    }
+    if (tok >= 0)
+        probe_p[row] = geist_expf_glibc_le0(softmax_arg(x_tok, M, inv_t), s_tab);
 }
 
 /* ============================================================================================
@@ -1851,6 +1922,21 @@ int launch_scan_expsum(const Launch &L, float inv_t, float *tmax, uint64_t *chun
                                              list ? nullptr : slab_sum, probe_token, probe_L, probe_p,
                                              list ? *list : CandSpace{}, list ? zb_list : 0, meet);
     };
+    if (fast && !list && !L.pen) { /* the tolerance mode's form without a meeting */
+        if (L.nv == 8)
+            slab_sum ? go(k_scan_expsum<8, false, false, true, true, true>)
+                     : go(k_scan_expsum<8, false, false, false, true, true>);
+        else
+            slab_sum ? go(k_scan_expsum<2, false, false, true, true, true>)
+                     : go(k_scan_expsum<2, false, false, false, true, true>);
+        if (slab_sum)
+            k_rescale_sums<true><<<dim3(L.rows), dim3(WAVE), 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, slab_sum, probe_token, probe_L, probe_p);
+        else
+            k_rescale_sums<false><<<dim3(L.rows), dim3(WAVE), 0, L.stream>>>(
+                L.rv, inv_t, chunk_best, chunk_sum, nullptr, probe_token, probe_L, probe_p);
+        return 0;
+    }
     if (list && L.nv == 8) {
         if (L.pen)
             fast ? go(k_scan_expsum<8, true, true, false, true>) : go(k_scan_expsum<8, true, true, false>);

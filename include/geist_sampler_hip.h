@@ -222,7 +222,9 @@ int geist_hip_sampler_handoff_scope(geist_hip_sampler *s, int always_agent);
  * can then differ from the reference's only where the reference's own decision lies within that
  * error of an edge (a draw within 1e-7 of a slot's edge, a nucleus that ends within 1e-7 of
  * top_p): the tolerance the sampling contract states, used. The pass over the logits gets a
- * tenth shorter. Which rows those are is not reported: a caller that has to know compares with
+ * fifth to a third shorter (without penalties and without a min-p list the workgroups of a row
+ * then do not wait for one another either: each sums against its chunk's maximum and a small
+ * launch scales the sums to the row's). Which rows those are is not reported: a caller that has to know compares with
  * the exact mode. The one-kernel temperature draw of a few rows and the top-k path form no such
  * sums and are exact in both modes. */
 #define GEIST_HIP_SUMS_EXACT 0

@@ -33,6 +33,9 @@ CASES = [
     (32, 151936, 2.0, dict(temperature=1.0, top_p=0.95, min_p=0.05), True),
     (32, 100000, 2.0, dict(temperature=1.0, top_p=0.9), False),
     (16, 128256, 0.5, dict(temperature=1.0, top_p=0.9), False),          # whole-row walks
+    (8, 128256, 2.0, dict(temperature=0.9), False),      # chunks of 2048, more than one kernel
+    (24, 50001, 2.0, dict(temperature=0.9), False),      # ragged rows: no float4 loads
+    (64, 60000, 2.5, dict(temperature=0.8), True),       # penalties: the workgroups meet
 ]
 
 
@@ -113,3 +116,24 @@ def test_sums_argument_errors(hs):
     from geistlib_amd.binding import GeistHipError
     with pytest.raises(GeistHipError):
         hs._check(hs.lib.geist_hip_sampler_set_sums(hs.h, 7))
+
+
+def test_rows_of_infinities_and_nan_with_fast_sums(hs, oracle):
+    """-inf regions (a chunk of nothing but -inf weighs nothing), +inf and NaN logits: the ids of
+    the exact mode."""
+    rows, n = 6, 70000
+    g = np.random.default_rng(5)
+    x = (g.standard_normal((rows, n)) * 2).astype(np.float32)
+    x[0, 8192:24576] = -np.inf        # two whole chunks
+    x[1, :60000] = -np.inf
+    x[2, 100] = np.inf
+    x[3, 200] = np.nan
+    x[4, :] = -np.inf
+    u = g.random(rows).astype(np.float32)
+    prm = P(temperature=0.9)
+    hs.set_sums(fast=False)
+    exact = run_rows(hs, torch, np.repeat(x, 16, axis=0), np.repeat(u, 16), prm)
+    hs.set_sums(fast=True)
+    fast = run_rows(hs, torch, np.repeat(x, 16, axis=0), np.repeat(u, 16), prm)
+    hs.set_sums(fast=False)
+    assert fast.tolist() == exact.tolist()
