@@ -266,7 +266,7 @@ __device__ __forceinline__ uint64_t row_best_meet(const RowView &rv, int row, in
             if (++polls > fs.wait_limit)
                 met = false;
             else
-                __builtin_amdgcn_s_sleep(8);
+                __builtin_amdgcn_s_sleep(2);
         }
         /* 1 is never a packed value: a row's first index is below 2^32 - 2 */
         const uint64_t got = met ? wave_max_u64(a > b ? a : b) : 1;
