@@ -404,6 +404,14 @@ int geist_hip_head_reserve_projection_q6k(struct geist_hip_head *h, size_t d_mod
     return GEIST_HIP_OK;
 }
 
+int geist_hip_head_set_sums(struct geist_hip_head *h, int mode) {
+    if (h == nullptr)
+        return GEIST_HIP_E_INVALID_ARG;
+    if (geist_hip_sampler_set_sums(h->hs, mode) != GEIST_HIP_OK)
+        return head_fail(h, GEIST_HIP_E_INVALID_ARG, "sums mode");
+    return GEIST_HIP_OK;
+}
+
 int geist_hip_head_set_projection(struct geist_hip_head *h, int mode) {
     if (h == nullptr)
         return GEIST_HIP_E_INVALID_ARG;

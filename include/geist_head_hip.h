@@ -95,6 +95,11 @@ int geist_hip_head_project_finalize(struct geist_hip_head *h, const float *d_hid
 /* GEIST_HIP_PROJECTION_X86 (default), _PORTABLE or _X86_AVX2 (include/geist_lm_head_hip.h): which
  * backend's arithmetic the project_finalize calls use. */
 int geist_hip_head_set_projection(struct geist_hip_head *h, int mode);
+/* GEIST_HIP_SUMS_EXACT (default) or GEIST_HIP_SUMS_FAST (include/geist_sampler_hip.h,
+ * geist_hip_sampler_set_sums): whether the head's sampling calls form the sums of exponentials
+ * with the reference's expf, bit for bit, or within the tolerance the sampling contract states.
+ * No counterpart in the reference. */
+int geist_hip_head_set_sums(struct geist_hip_head *h, int mode);
 /* The same over the int8 form of the table, which the reference's x86 backend substitutes for
  * the F16 table in a decode step (src/backends/cpu_x86/backend.c:332-372): d_embed_q8 [vocab,
  * d_model] int8 and d_scales [vocab] as geist_hip_f16_to_q8w produces them, d_model a multiple

@@ -217,6 +217,32 @@ def test_head_dispatch_precedence_and_rng(host, oracle):
         host.geist_hip_head_destroy(h)
 
 
+def test_head_sums_within_the_contracts_tolerance(host, oracle):
+    """geist_hip_head_set_sums(h, 1): the head's temperature and top-p rows with the sums of
+    exponentials from the hardware's 2^z. The tokens are the reference's on rows whose draws lie
+    away from slot edges (all of these: a draw within 1e-7 of an edge is a one-in-thousands
+    event), and the RNG is consumed as before."""
+    g = np.random.default_rng(77)
+    vocab = 50000
+    x = (g.standard_normal((24, vocab)) * 2).astype(np.float32)
+    d = torch.from_numpy(x).cuda()
+    host.geist_hip_head_set_sums.argtypes = [C.c_void_p, C.c_int]
+    for T, p, k in [(0.8, 1.0, 0), (0.9, 0.9, 0)]:
+        h = make_head(host, vocab)
+        opts = SessionOpts(0, T, p, k, 0xC0FFEE, None, 0, 0)
+        assert host.geist_hip_head_apply_opts(h, C.byref(opts)) == 0
+        assert host.geist_hip_head_set_sums(h, 7) != 0
+        assert host.geist_hip_head_set_sums(h, 1) == 0
+        sess = oracle.session(T, p, k, seed=0xC0FFEE)
+        out = (C.c_int32 * 24)()
+        assert host.geist_hip_head_finalize_batch(h, C.c_void_p(d.data_ptr()), 24, out) == 0
+        assert list(out) == oracle.finalize_batch(sess, x).tolist(), (T, p, k)
+        st = C.c_uint64(0)
+        assert host.geist_hip_head_rng_state(h, C.byref(st)) == 0
+        assert st.value == int(sess.rng.state)
+        host.geist_hip_head_destroy(h)
+
+
 def test_head_defaults_and_null_opts(host, oracle):
     vocab = 5000
     g = np.random.default_rng(2)
