@@ -137,3 +137,30 @@ def test_rows_of_infinities_and_nan_with_fast_sums(hs, oracle):
     fast = run_rows(hs, torch, np.repeat(x, 16, axis=0), np.repeat(u, 16), prm)
     hs.set_sums(fast=False)
     assert fast.tolist() == exact.tolist()
+
+
+@pytest.mark.parametrize("extra", ["softcap", "mask", "ragged"])
+def test_fast_sums_on_rows_that_are_not_plain(hs, oracle, extra):
+    """Soft-capped rows, rows under an allowed-token mask and rows that allow no float4 loads
+    take the pass's general form: the same ids as the exact mode (and the oracle's)."""
+    rows, n = 16, 70001 if extra == "ragged" else 70000
+    g = np.random.default_rng(len(extra))
+    x = (g.standard_normal((rows, n)) * 3).astype(np.float32)
+    u = g.random(rows).astype(np.float32)
+    cap = 6.0 if extra == "softcap" else 0.0
+    allowed = (g.random((rows, n)) < 0.4) if extra == "mask" else None
+    if allowed is not None:
+        allowed[:, 0] = True
+    prm = P(temperature=0.9, softcap=cap)
+    want = []
+    for r in range(rows):
+        row = oracle.softcap(x[r], cap) if cap else x[r]
+        if allowed is not None:
+            row = np.where(allowed[r], row, -np.inf).astype(np.float32)
+        want.append(oracle.chain_u(row, float(u[r]), temperature=0.9))
+    hs.set_sums(fast=True)
+    fast = run_rows(hs, torch, x, u, prm, allowed=allowed)
+    hs.set_sums(fast=False)
+    exact = run_rows(hs, torch, x, u, prm, allowed=allowed)
+    assert compare_ids(exact, [t for t, _ in want], [i for _, i in want], "exact") == 0
+    assert compare_ids(fast, [t for t, _ in want], [i for _, i in want], "fast") <= 1

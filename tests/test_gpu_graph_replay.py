@@ -20,17 +20,26 @@ def want_rows(oracle, x, u, **kw):
     return [t for t, _ in res], [i for _, i in res]
 
 
-@pytest.mark.parametrize("static", [False, True])
-@pytest.mark.parametrize("rows,n,kw", [
+MODES = [
     (4, 128256, dict(temperature=0.8)),                       # one-kernel temperature draw
     (32, 50000, dict(temperature=0.9)),                       # exp-sum pass + index-order walk
     (64, 128256, dict(temperature=0.7, top_k=40, top_p=0.9)), # top-k in one launch
-])
+]
+# the tolerance mode (a sampler object's: the entry point without one has no modes to set): the
+# pass without a meeting and the launch that scales its sums
+FAST = (32, 50000, dict(temperature=0.9, fast_sums=True))
+
+
+@pytest.mark.parametrize("static,rows,n,kw", [(st, *m) for st in (False, True) for m in MODES]
+                         + [(False, *FAST)])
 def test_recorded_call_replays(oracle, static, rows, n, kw):
     from geistlib_amd import HipSampler, SampleParams, sample_rows_static
+    kw = dict(kw)
+    fast = kw.pop("fast_sums", False)
     g = np.random.default_rng(rows + n + static)
     prm = SampleParams.make(**kw)
     hs = HipSampler(rows, n)
+    hs.set_sums(fast=fast)
     try:
         d_x = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
         d_u = torch.zeros(rows, dtype=torch.float32, device="cuda")
