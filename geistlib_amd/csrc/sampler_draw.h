@@ -130,8 +130,6 @@ __device__ __forceinline__ void row_sums_meet(uint64_t *row_slots, int chunk, in
                 break;
             if (++polls > wait_limit)
                 met = false;
-            else
-                __builtin_amdgcn_s_sleep(2);
         }
         if (met) {
             if (lane < C)
